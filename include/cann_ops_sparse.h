@@ -1,0 +1,317 @@
+/*
+ * Public C ABI of libops_sparse.so on AMD MI355X (gfx950): the generic CSR
+ * SpMV / SpMM path of the aclsparse API.
+ *
+ * This header is a drop-in for the subset of the reference's
+ * include/cann_ops_sparse.h that the CSR SpMV / SpMM path touches: the same
+ * type names, enumerators (same order, hence same values), function names and
+ * argument lists, so a caller written against the reference compiles and links
+ * unchanged.  Every declaration cites the reference declaration it replaces as
+ * [ref: file:line], relative to the reference tree.
+ *
+ * Conventions shared by every entry point
+ *   - returns aclsparseStatus_t, never throws, never aborts;
+ *   - "DEVICE" pointers are HIP device pointers that the library borrows and
+ *     never frees; "HOST" pointers are ordinary process memory;
+ *   - compute calls enqueue work on the handle's stream and return; the caller
+ *     synchronises the stream before reading results;
+ *   - a handle and the descriptors used with it must not be used from two
+ *     threads at once.
+ */
+#ifndef CANN_OPS_SPARSE_H_
+#define CANN_OPS_SPARSE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+#include <acl/acl_base_rt.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ enums */
+
+/* [ref: include/cann_ops_sparse.h:24-28] operation applied to an operand. */
+typedef enum aclsparseOperation_t {
+    ACL_SPARSE_OP_NON_TRANSPOSE = 0,
+    ACL_SPARSE_OP_TRANSPOSE,
+    ACL_SPARSE_OP_CONJUGATE_TRANSPOSE
+} aclsparseOperation_t;
+
+/* [ref: :50-53] storage order of a dense matrix (B and C of SpMM). */
+typedef enum aclsparseOrder_t {
+    ACL_SPARSE_ORDER_ROW = 0,
+    ACL_SPARSE_ORDER_COL = 1
+} aclsparseOrder_t;
+
+/* [ref: :56-70] algorithm selector of the SpMVOp API. */
+typedef enum aclsparseSpMVOpAlg_t {
+    ACL_SPARSE_SPMVOP_ALG_DEFAULT = 0,
+    ACL_SPARSE_SPMVOP_ALG1,
+    ACL_SPARSE_SPMVOP_ALG2
+} aclsparseSpMVOpAlg_t;
+
+/* [ref: :81-96] SpMM algorithm selector.  DEFAULT and CSR_ALG1 are the same
+ * kernels.  The reference's third value selects Kahan-compensated fp32
+ * accumulation; here every floating-point SpMM kernel already accumulates in
+ * fp64 and rounds once, so the three values give identical results. */
+typedef enum aclsparseSpMMAlg_t {
+    ACL_SPARSE_SPMM_ALG_DEFAULT = 0,
+    ACL_SPARSE_SPMM_CSR_ALG1,
+    ACL_SPARSE_SPMM_CSR_FP32_HIGH_PRECISION_ALG
+} aclsparseSpMMAlg_t;
+
+/* [ref: :98-148] status codes. */
+typedef enum aclsparseStatus_t {
+    ACL_SPARSE_STATUS_SUCCESS = 0,
+    ACL_SPARSE_STATUS_NOT_INITIALIZED,
+    ACL_SPARSE_STATUS_ALLOC_FAILED,
+    ACL_SPARSE_STATUS_INVALID_VALUE,
+    ACL_SPARSE_STATUS_ARCH_MISMATCH,
+    ACL_SPARSE_STATUS_EXECUTION_FAILED,
+    ACL_SPARSE_STATUS_INTERNAL_ERROR,
+    ACL_SPARSE_STATUS_MATRIX_TYPE_NOT_SUPPORTED,
+    ACL_SPARSE_STATUS_NOT_SUPPORTED,
+    ACL_SPARSE_STATUS_INSUFFICIENT_RESOURCES,
+    ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR
+} aclsparseStatus_t;
+
+/* [ref: :150-168] SpMV algorithm selector; only ALG_DEFAULT is accepted by
+ * aclsparseSpMV, as in the reference (sparse/spmv/arch22/spmv_host.cpp:144). */
+typedef enum aclsparseSpMVAlg_t {
+    ACL_SPARSE_SPMV_ALG_DEFAULT,
+    ACL_SPARSE_SPMV_COO_ALG1,
+    ACL_SPARSE_SPMV_COO_ALG2,
+    ACL_SPARSE_SPMV_CSR_ALG1,
+    ACL_SPARSE_SPMV_CSR_ALG2,
+    ACL_SPARSE_SPMV_SELL_ALG1
+} aclsparseSpMVAlg_t;
+
+/* [ref: :213-222] width of row offsets / column indices. */
+typedef enum aclsparseIndexType_t {
+    ACL_SPARSE_INDEX_32I = 0,
+    ACL_SPARSE_INDEX_64I
+} aclsparseIndexType_t;
+
+/* [ref: :229-232] */
+typedef enum aclsparseIndexBase_t {
+    ACL_SPARSE_INDEX_BASE_ZERO = 0,
+    ACL_SPARSE_INDEX_BASE_ONE
+} aclsparseIndexBase_t;
+
+/* [ref: :235-248] sparse storage format tag; only CSR descriptors can be
+ * created through this library, the other tags exist so that
+ * aclsparseSpMatGetFormat has the reference's value space. */
+typedef enum aclsparseFormat_t {
+    ACL_SPARSE_FORMAT_COO = 0,
+    ACL_SPARSE_FORMAT_CSR,
+    ACL_SPARSE_FORMAT_CSC,
+    ACL_SPARSE_FORMAT_BLOCKED_ELL,
+    ACL_SPARSE_FORMAT_SLICED_ELL,
+    ACL_SPARSE_FORMAT_BSR
+} aclsparseFormat_t;
+
+/* [ref: :898-901] where alpha / beta live. */
+typedef enum aclsparsePointerMode_t {
+    ACL_SPARSE_POINTER_MODE_HOST = 0,
+    ACL_SPARSE_POINTER_MODE_DEVICE = 1
+} aclsparsePointerMode_t;
+
+/* ---------------------------------------------------------- opaque types */
+
+/* [ref: :30-47, :73-78] */
+struct aclsparseContext;
+struct aclsparseSpMatDescr;
+struct aclsparseDnVecDescr;
+struct aclsparseDnMatDescr;
+struct aclsparseSpMVOpDescr;
+struct aclsparseSpMVOpPlan;
+
+typedef struct aclsparseContext *aclsparseHandle_t;
+typedef struct aclsparseSpMatDescr *aclsparseSpMatDescr_t;
+typedef struct aclsparseDnVecDescr *aclsparseDnVecDescr_t;
+typedef struct aclsparseDnMatDescr *aclsparseDnMatDescr_t;
+typedef struct aclsparseSpMatDescr const *aclsparseConstSpMatDescr_t;
+typedef struct aclsparseDnVecDescr const *aclsparseConstDnVecDescr_t;
+typedef struct aclsparseDnMatDescr const *aclsparseConstDnMatDescr_t;
+typedef struct aclsparseSpMVOpDescr *aclsparseSpMVOpDescr_t;
+typedef struct aclsparseSpMVOpDescr const *aclsparseConstSpMVOpDescr_t;
+typedef struct aclsparseSpMVOpPlan *aclsparseSpMVOpPlan_t;
+
+/* ----------------------------------------------------------------- handle */
+
+/* [ref: :817] Allocates a handle and its 4 MiB default device workspace.
+ * *handle must be NULL on entry (INVALID_VALUE otherwise); handle == NULL
+ * gives HANDLE_IS_NULLPTR. */
+aclsparseStatus_t aclsparseCreate(aclsparseHandle_t *handle);
+
+/* [ref: :828] Synchronises the handle's stream, frees the default workspace
+ * and the handle.  The stream and any user workspace stay with the caller. */
+aclsparseStatus_t aclsparseDestroy(aclsparseHandle_t handle);
+
+/* [ref: :837, :848] The stream all compute calls of this handle enqueue on. */
+aclsparseStatus_t aclsparseSetStream(aclsparseHandle_t handle, aclrtStream stream);
+aclsparseStatus_t aclsparseGetStream(aclsparseHandle_t handle, aclrtStream *stream);
+
+/* [ref: :867, :882] Borrow a caller-owned device workspace (grow-only: a
+ * request not larger than the current user workspace is ignored; NULL returns
+ * to the default workspace). */
+aclsparseStatus_t aclsparseSetWorkspace(aclsparseHandle_t handle, void *workspace, size_t workspaceSize);
+aclsparseStatus_t aclsparseGetWorkspace(aclsparseHandle_t handle, void **workspace, size_t *workspaceSize);
+
+/* [ref: :894] MAJOR*10000 + MINOR*100 + PATCH; handle may be NULL. */
+aclsparseStatus_t aclsparseGetVersion(aclsparseHandle_t handle, int *version);
+
+/* [ref: :903-904] HOST (default): alpha/beta are dereferenced on the host at
+ * call time.  DEVICE: they are device addresses read by the kernel, so no
+ * host synchronisation is needed to change them. */
+aclsparseStatus_t aclsparseSetPointerMode(aclsparseHandle_t handle, aclsparsePointerMode_t mode);
+aclsparseStatus_t aclsparseGetPointerMode(aclsparseHandle_t handle, aclsparsePointerMode_t *mode);
+
+/* ----------------------------------------------------------- dense vector */
+
+/* [ref: :259, :264, :273] size >= 0; values may be NULL only when size == 0. */
+aclsparseStatus_t aclsparseCreateDnVec(aclsparseDnVecDescr_t *dnVecDescr, int64_t size, void *values,
+                                       aclDataType valueType);
+aclsparseStatus_t aclsparseCreateConstDnVec(aclsparseConstDnVecDescr_t *dnVecDescr, int64_t size,
+                                            const void *values, aclDataType valueType);
+aclsparseStatus_t aclsparseDestroyDnVec(aclsparseConstDnVecDescr_t dnVecDescr);
+
+/* [ref: :335-373] accessors; NULL out-pointers of the Get* forms are skipped. */
+aclsparseStatus_t aclsparseDnVecGet(aclsparseDnVecDescr_t dnVecDescr, int64_t *size, void **values,
+                                    aclDataType *valueType);
+aclsparseStatus_t aclsparseConstDnVecGet(aclsparseConstDnVecDescr_t dnVecDescr, int64_t *size,
+                                         const void **values, aclDataType *valueType);
+aclsparseStatus_t aclsparseDnVecGetValues(aclsparseDnVecDescr_t dnVecDescr, void **values);
+aclsparseStatus_t aclsparseConstDnVecGetValues(aclsparseConstDnVecDescr_t dnVecDescr, const void **values);
+aclsparseStatus_t aclsparseDnVecSetValues(aclsparseDnVecDescr_t dnVecDescr, void *values);
+
+/* ---------------------------------------------------------- sparse matrix */
+
+/* [ref: :399-408] CSR descriptor over caller-owned device arrays:
+ * csrRowOffsets[rows+1], csrColInd[nnz], csrValues[nnz].  All four I32/I64
+ * combinations are accepted here; SpMV / SpMM accept (I32, I32) only. */
+aclsparseStatus_t aclsparseCreateCsr(aclsparseSpMatDescr_t *spMatDescr, int64_t rows, int64_t cols, int64_t nnz,
+                                     void *csrRowOffsets, void *csrColInd, void *csrValues,
+                                     aclsparseIndexType_t csrRowOffsetsType, aclsparseIndexType_t csrColIndType,
+                                     aclsparseIndexBase_t idxBase, aclDataType valueType);
+aclsparseStatus_t aclsparseCreateConstCsr(aclsparseConstSpMatDescr_t *spMatDescr, int64_t rows, int64_t cols,
+                                          int64_t nnz, const void *csrRowOffsets, const void *csrColInd,
+                                          const void *csrValues, aclsparseIndexType_t csrRowOffsetsType,
+                                          aclsparseIndexType_t csrColIndType, aclsparseIndexBase_t idxBase,
+                                          aclDataType valueType);
+
+/* [ref: :446] replace the three device arrays of a CSR descriptor; drops any
+ * preprocessing bound to the descriptor. */
+aclsparseStatus_t aclsparseCsrSetPointers(aclsparseSpMatDescr_t descr, void *rowOffsets, void *colIndices,
+                                          void *values);
+
+/* [ref: :459] NULL is accepted and returns SUCCESS. */
+aclsparseStatus_t aclsparseDestroySpMat(aclsparseConstSpMatDescr_t spMatDescr);
+
+/* [ref: :465-478] */
+aclsparseStatus_t aclsparseSpMatGetFormat(aclsparseConstSpMatDescr_t spMatDescr, aclsparseFormat_t *format);
+aclsparseStatus_t aclsparseSpMatGetValues(aclsparseSpMatDescr_t spMatDescr, void **values);
+aclsparseStatus_t aclsparseConstSpMatGetValues(aclsparseConstSpMatDescr_t spMatDescr, const void **values);
+aclsparseStatus_t aclsparseSpMatSetValues(aclsparseSpMatDescr_t spMatDescr, void *values);
+aclsparseStatus_t aclsparseSpMatGetSize(aclsparseConstSpMatDescr_t spMatDescr, int64_t *rows, int64_t *cols,
+                                        int64_t *nnz);
+
+/* ----------------------------------------------------------- dense matrix */
+
+/* [ref: :552-564] rows > 0, cols > 0, ld >= cols (row-major) or >= rows
+ * (column-major), values non-NULL. */
+aclsparseStatus_t aclsparseCreateDnMat(aclsparseDnMatDescr_t *dnMatDescr, int64_t rows, int64_t cols, int64_t ld,
+                                       void *values, aclDataType valueType, aclsparseOrder_t order);
+aclsparseStatus_t aclsparseCreateConstDnMat(aclsparseConstDnMatDescr_t *dnMatDescr, int64_t rows, int64_t cols,
+                                            int64_t ld, const void *values, aclDataType valueType,
+                                            aclsparseOrder_t order);
+aclsparseStatus_t aclsparseDestroyDnMat(aclsparseConstDnMatDescr_t dnMatDescr);
+
+/* [ref: :581-614] */
+aclsparseStatus_t aclsparseDnMatGet(aclsparseDnMatDescr_t dnMatDescr, int64_t *rows, int64_t *cols, int64_t *ld,
+                                    void **values, aclDataType *valueType, aclsparseOrder_t *order);
+aclsparseStatus_t aclsparseConstDnMatGet(aclsparseConstDnMatDescr_t dnMatDescr, int64_t *rows, int64_t *cols,
+                                         int64_t *ld, const void **values, aclDataType *valueType,
+                                         aclsparseOrder_t *order);
+aclsparseStatus_t aclsparseDnMatGetValues(aclsparseDnMatDescr_t dnMatDescr, void **values);
+aclsparseStatus_t aclsparseConstDnMatGetValues(aclsparseConstDnMatDescr_t dnMatDescr, const void **values);
+aclsparseStatus_t aclsparseDnMatSetValues(aclsparseDnMatDescr_t dnMatDescr, void *values);
+
+/* ------------------------------------------------------------------- SpMV */
+
+/*
+ * y = alpha * op(A) * x + beta * y, A in CSR with int32 zero-based indices.
+ *
+ * Type triples (A and x, y, computeType): (f32, f32, f32), (f16, f16, f32),
+ * (f16, f32, f32), (bf16, bf16, f32), (bf16, f32, f32), (i32, f32, f32),
+ * (i32, i32, i32) [ref: sparse/spmv/arch22/spmv.h:67-103].  Floating-point
+ * rows are accumulated in fp64 in stored order and rounded once to the type
+ * of y; y is not read when beta == 0.
+ *
+ * aclsparseSpMV [ref: include/cann_ops_sparse.h:531-533, implementation
+ * sparse/spmv/arch22/spmv_host.cpp:121-295] needs no buffer: with
+ * externalBuffer == NULL (or a buffer that was not preprocessed for matA) it
+ * uses a partition kept in the handle's workspace.  GetBufferSize /
+ * Preprocess [ref: :490-514, declared by the reference without a definition]
+ * analyse the row-length distribution once and store the kernel choice and the
+ * merge-path partition in the caller's buffer; later aclsparseSpMV calls that
+ * pass the same buffer skip that work.
+ *
+ * alpha / beta: typed by computeType; NULL means alpha = 1, beta = 0
+ * [ref: spmv_host.cpp:183-199]; read according to the handle's pointer mode.
+ */
+aclsparseStatus_t aclsparseSpMVGetBufferSize(aclsparseHandle_t handle, aclsparseOperation_t opA, const void *alpha,
+                                             aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX,
+                                             const void *beta, aclsparseDnVecDescr_t vecY, aclDataType computeType,
+                                             aclsparseSpMVAlg_t alg, size_t *bufferSize);
+aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOperation_t opA, const void *alpha,
+                                          aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX,
+                                          const void *beta, aclsparseDnVecDescr_t vecY, aclDataType computeType,
+                                          aclsparseSpMVAlg_t alg, void *externalBuffer);
+aclsparseStatus_t aclsparseSpMV(aclsparseHandle_t handle, aclsparseOperation_t opA, const void *alpha,
+                                aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX, const void *beta,
+                                aclsparseDnVecDescr_t vecY, aclDataType computeType, aclsparseSpMVAlg_t alg,
+                                void *externalBuffer);
+
+/* ------------------------------------------------------------------- SpMM */
+
+/*
+ * C = alpha * A * op(B) + beta * C, A in CSR (int32, zero-based), B and C
+ * dense in either order with leading dimensions honoured.
+ * [ref: include/cann_ops_sparse.h:682-704, implementation
+ * sparse/spmm/arch35/spmm_host.cpp:213-234, :335-362, :364-394]
+ *
+ * Type quadruples (A, B, C, computeType): (f32, f32, f32, f32),
+ * (f16, f16, f16, f32) with the result clamped to +-65504 before the fp16
+ * rounding, (i8, i8, i32, i32) saturating [ref: spmm_host.cpp:103-120], and
+ * the extension (f16, f16, f32, f32) which is the fp16 case without the final
+ * clamp and rounding.  C is not read when beta == 0.
+ *
+ * The three calls keep the reference's protocol: GetBufferSize reports the
+ * bytes Preprocess needs, Preprocess fills the buffer and binds it to matA,
+ * SpMM with the same buffer reuses it; SpMM with a different non-NULL buffer
+ * preprocesses into that buffer first.  buffer == NULL gives
+ * INSUFFICIENT_RESOURCES.  alpha / beta follow the handle's pointer mode;
+ * NULL is read as 0 [ref: spmm_host.cpp:62-74].
+ */
+aclsparseStatus_t aclsparseSpMMGetBufferSize(aclsparseHandle_t handle, aclsparseOperation_t opA,
+                                             aclsparseOperation_t opB, const void *alpha,
+                                             aclsparseConstSpMatDescr_t matA, aclsparseConstDnMatDescr_t matB,
+                                             const void *beta, aclsparseDnMatDescr_t matC, aclDataType computeType,
+                                             aclsparseSpMMAlg_t alg, size_t *size);
+aclsparseStatus_t aclsparseSpMMPreprocess(aclsparseHandle_t handle, aclsparseOperation_t opA,
+                                          aclsparseOperation_t opB, const void *alpha,
+                                          aclsparseConstSpMatDescr_t matA, aclsparseConstDnMatDescr_t matB,
+                                          const void *beta, aclsparseDnMatDescr_t matC, aclDataType computeType,
+                                          aclsparseSpMMAlg_t alg, void *buffer);
+aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t opA, aclsparseOperation_t opB,
+                                const void *alpha, aclsparseConstSpMatDescr_t matA,
+                                aclsparseConstDnMatDescr_t matB, const void *beta, aclsparseDnMatDescr_t matC,
+                                aclDataType computeType, aclsparseSpMMAlg_t alg, void *buffer);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CANN_OPS_SPARSE_H_ */

@@ -1,0 +1,164 @@
+/*
+ * Thin C-ABI launch layer between the aclsparse host code and the HIP kernels
+ * for gfx950.  Plain pointers and sizes only: this is the seam a foreign-
+ * language binding (ctypes, cgo, JNI) or another host library would call when
+ * it has its own descriptor handling and just wants the kernels.
+ *
+ * It plays the role the reference gives to its `extern "C"` kernel launchers:
+ *   spmv_kernel_do      [ref: sparse/spmv/arch22/spmv_host.cpp:29-34,
+ *                             sparse/spmv/arch22/kernels/spmv_kernel.cpp:21-55]
+ *   spmm_kernel_launch  [ref: sparse/spmm/arch35/spmm_host.cpp:29-33,
+ *                             sparse/spmm/arch35/spmm_kernel.cpp:447-477]
+ * i.e. raw device pointers + sizes + scalars + a workspace + a stream, no
+ * descriptor objects, no validation beyond what keeps a launch in bounds.
+ *
+ * All functions return 0 on success or a negative OPSPARSE_E_* code; nothing
+ * is printed.  `stream` is a hipStream_t passed as void*.  Unless stated
+ * otherwise a function only enqueues work and does not synchronise.
+ */
+#ifndef OPS_SPARSE_HIP_H_
+#define OPS_SPARSE_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OPSPARSE_OK 0
+#define OPSPARSE_E_INVALID (-1)     /* bad argument (null pointer, negative size, unknown enum) */
+#define OPSPARSE_E_UNSUPPORTED (-2) /* type / layout combination without a kernel */
+#define OPSPARSE_E_WORKSPACE (-3)   /* workspace missing or too small */
+#define OPSPARSE_E_LAUNCH (-4)      /* the HIP runtime reported an error */
+
+/* Element types of device arrays. */
+typedef enum OpsparseDtype {
+    OPSPARSE_F32 = 0,
+    OPSPARSE_F16 = 1,
+    OPSPARSE_BF16 = 2,
+    OPSPARSE_I32 = 3,
+    OPSPARSE_I8 = 4
+} OpsparseDtype;
+
+/* alpha or beta.  devicePtr == NULL: `value` is used.  Otherwise the kernel
+ * reads a float (isInt == 0) or an int32 (isInt != 0) from devicePtr. */
+typedef struct OpsparseScalar {
+    double value;
+    const void *devicePtr;
+    int32_t isInt;
+    int32_t reserved;
+} OpsparseScalar;
+
+/* ------------------------------------------------------------------ SpMV */
+
+/* Kernel families of the row-length-binned SpMV dispatcher. */
+typedef enum OpsparseSpmvKernel {
+    OPSPARSE_SPMV_AUTO = 0,        /* let the library pick from the statistics */
+    OPSPARSE_SPMV_SCALE_ONLY = 1,  /* nnz == 0: y = beta * y */
+    OPSPARSE_SPMV_STREAM_ROWS = 2, /* short rows: fixed row blocks, products staged in LDS,
+                                      one or a few lanes per row */
+    OPSPARSE_SPMV_VECTOR_ROWS = 3, /* medium rows: a 4..64-lane group per row, shuffle reduction */
+    OPSPARSE_SPMV_MERGE_PATH = 4   /* skewed rows: equal (rows + nnz) per workgroup, carry-out fix-up */
+} OpsparseSpmvKernel;
+
+/* Result of analysing one CSR matrix; plain data, safe to copy. */
+typedef struct OpsparseSpmvPlan {
+    int32_t kernel;        /* OpsparseSpmvKernel actually chosen */
+    int32_t lanesPerRow;   /* VECTOR_ROWS / STREAM_ROWS: lanes cooperating on one row */
+    int32_t rowsPerBlock;  /* STREAM_ROWS: rows owned by one workgroup */
+    int32_t mergeBlocks;   /* MERGE_PATH: number of workgroups == partition entries - 1 */
+    int32_t maxRowNnz;     /* longest row */
+    int32_t partitionReady;/* MERGE_PATH: partition table already in the workspace */
+    int64_t rows;
+    int64_t nnz;
+    int64_t partOff;       /* byte offsets into the workspace */
+    int64_t carryOff;
+    int64_t headOff;
+    int64_t bytes;         /* workspace bytes this plan uses */
+} OpsparseSpmvPlan;
+
+/* Bytes opsparse_spmv_csr_analyse / _launch may touch in `workspace`. */
+size_t opsparse_spmv_csr_workspace_bytes(int64_t rows, int64_t nnz);
+
+/*
+ * Row-length statistics -> kernel choice (+ merge-path partition written to
+ * `workspace`).  Synchronises `stream` once to read the statistics back.
+ * `forceKernel` != AUTO overrides the choice (tuning, tests).
+ */
+int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t cols, int64_t nnz,
+                              void *workspace, size_t workspaceBytes, int32_t forceKernel,
+                              OpsparseSpmvPlan *plan, void *stream);
+
+/*
+ * y = alpha * A * x + beta * y (transpose == 0) or y = alpha * A^T * x + beta * y.
+ * valType is the element type of csrValues and x, outType of y.
+ * plan == NULL: no prior analysis; the merge-path family is used with the
+ * partition rebuilt into `workspace` by a small kernel, or, when `workspace`
+ * is too small, a workspace-free VECTOR_ROWS launch sized from nnz / rows.
+ */
+int opsparse_spmv_csr_launch(const OpsparseSpmvPlan *plan, int32_t transpose, const int32_t *rowOffsets,
+                             const int32_t *colInd, const void *csrValues, const void *x, void *y, int64_t rows,
+                             int64_t cols, int64_t nnz, OpsparseScalar alpha, OpsparseScalar beta, int32_t valType,
+                             int32_t outType, int32_t computeIsInt, void *workspace, size_t workspaceBytes,
+                             void *stream);
+
+/* ------------------------------------------------------------------ SpMM */
+
+typedef enum OpsparseSpmmKernel {
+    OPSPARSE_SPMM_AUTO = 0,
+    OPSPARSE_SPMM_ROW_SPLIT = 1, /* every row by one lane group; B rows streamed coalesced */
+    OPSPARSE_SPMM_BINNED = 2     /* rows up to the long-row threshold as ROW_SPLIT, longer rows cut into
+                                    fixed nnz segments over several waves + a fix-up pass */
+} OpsparseSpmmKernel;
+
+typedef struct OpsparseSpmmPlan {
+    int32_t kernel;        /* OpsparseSpmmKernel */
+    int32_t maxRowNnz;
+    int32_t longRowNnz;    /* rows with more nnz than this are "long" */
+    int32_t numLongRows;
+    int32_t numSegments;   /* segments over all long rows */
+    int32_t segmentNnz;    /* nnz per segment */
+    int64_t rows;
+    int64_t nnz;
+    int64_t n;             /* columns of C the partial buffer was sized for */
+    int64_t longRowsOff;   /* int32 row ids of long rows */
+    int64_t segRowOff;     /* int32 [numSegments]: index into long rows */
+    int64_t segStartOff;   /* int32 [numSegments]: first nnz of the segment */
+    int64_t longFirstSegOff; /* int32 [numLongRows + 1]: first segment of each long row */
+    int64_t partialOff;    /* double [numSegments * n] */
+    int64_t bytes;
+} OpsparseSpmmPlan;
+
+size_t opsparse_spmm_csr_workspace_bytes(int64_t rows, int64_t nnz, int64_t n);
+
+/* Synchronises `stream` once (row statistics are read back). */
+int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t nnz, int64_t n, void *workspace,
+                              size_t workspaceBytes, int32_t forceKernel, OpsparseSpmmPlan *plan, void *stream);
+
+/*
+ * C[rows x n] = alpha * A * op(B) + beta * C.
+ * bColMajor / cColMajor select the storage order, ldb / ldc the leading
+ * dimensions in elements; transB != 0 reads B as its transpose, with the index
+ * formulas of the reference kernel [ref: sparse/spmm/arch35/spmm_kernel.cpp:155-168, :215-219].
+ * clampF16: when cType is F16, clamp to +-65504 before rounding [ref: :229-237].
+ * plan == NULL runs ROW_SPLIT without a workspace.
+ */
+int opsparse_spmm_csr_launch(const OpsparseSpmmPlan *plan, const int32_t *rowOffsets, const int32_t *colInd,
+                             const void *csrValues, const void *B, void *C, int64_t rows, int64_t k, int64_t n,
+                             int64_t nnz, int64_t ldb, int64_t ldc, int32_t bColMajor, int32_t cColMajor,
+                             int32_t transB, OpsparseScalar alpha, OpsparseScalar beta, int32_t valType,
+                             int32_t cType, void *workspace, size_t workspaceBytes, void *stream);
+
+/* ----------------------------------------------------------- measurement */
+
+/* Plain device-to-device copy kernel (dwordx4 per lane) used as the HBM
+ * bandwidth yard-stick and as the calibration kernel for the FETCH_SIZE /
+ * WRITE_SIZE counters.  bytes must be a multiple of 16. */
+int opsparse_copy_launch(const void *src, void *dst, size_t bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* OPS_SPARSE_HIP_H_ */

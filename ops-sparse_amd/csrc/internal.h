@@ -1,0 +1,113 @@
+// Internal object layouts of libops_sparse.so (handle, descriptors, SpMV / SpMM
+// plans).  Nothing here is visible through the public header: callers only see
+// opaque pointers.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+#include "cann_ops_sparse.h"
+#include "ops_sparse_hip.h"
+
+namespace opsparse {
+
+constexpr int kVersionMajor = 1;
+constexpr int kVersionMinor = 0;
+constexpr int kVersionPatch = 0;
+
+// Size of the device workspace every handle owns
+// (reference: sparse/common/aclsparse_handle_internal.h:44).
+constexpr size_t kDefaultWorkspaceBytes = 4u * 1024u * 1024u;
+
+// Tag stored in live dense-vector descriptors and checked by the accessors
+// (reference: sparse/common/aclsparse_descr.cpp:29).
+constexpr uint32_t kDnVecSignature = 0xD0D2D4D6u;
+
+inline size_t AlignUp(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace opsparse
+
+// What aclsparseSpMVPreprocess leaves behind for a matrix: the kernel family
+// picked from the row-length statistics and, for the merge-path family, where
+// in the caller's buffer the partition lives.
+struct OpsparseSpmvBinding {
+    const void *buffer = nullptr;  // buffer this plan was written into
+    OpsparseSpmvPlan plan{};
+};
+
+struct OpsparseSpmmBinding {
+    const void *buffer = nullptr;
+    OpsparseSpmmPlan plan{};
+};
+
+// reference: sparse/common/aclsparse_handle_internal.h:56-72
+struct aclsparseContext {
+    hipStream_t stream = nullptr;
+    aclsparsePointerMode_t pointerMode = ACL_SPARSE_POINTER_MODE_HOST;
+    void *defaultWorkspace = nullptr;
+    size_t defaultWorkspaceBytes = 0;
+    void *userWorkspace = nullptr;
+    size_t userWorkspaceBytes = 0;
+    bool useUserWorkspace = false;
+
+    void *workspace() const { return useUserWorkspace ? userWorkspace : defaultWorkspace; }
+    size_t workspaceBytes() const { return useUserWorkspace ? userWorkspaceBytes : defaultWorkspaceBytes; }
+};
+
+// reference: sparse/common/aclsparse_descr_internal.h:32-56 (the CSR part)
+struct aclsparseSpMatDescr {
+    aclsparseFormat_t format = ACL_SPARSE_FORMAT_CSR;
+    int64_t rows = 0;
+    int64_t cols = 0;
+    int64_t nnz = 0;
+    void *rowOffsets = nullptr;
+    void *colInd = nullptr;
+    void *values = nullptr;
+    aclsparseIndexType_t rowOffsetsType = ACL_SPARSE_INDEX_32I;
+    aclsparseIndexType_t colIndType = ACL_SPARSE_INDEX_32I;
+    aclsparseIndexBase_t idxBase = ACL_SPARSE_INDEX_BASE_ZERO;
+    aclDataType valueType = ACL_FLOAT;
+    // Preprocess results.  The public API hands the matrix in as a pointer to
+    // const, like the reference, and the reference's Preprocess records its
+    // active buffer in the descriptor all the same
+    // (sparse/spmm/arch35/spmm_host.cpp:360); `mutable` makes that explicit.
+    mutable OpsparseSpmvBinding spmv;
+    mutable OpsparseSpmmBinding spmm;
+};
+
+// reference: sparse/common/aclsparse_descr_internal.h:102-107
+struct aclsparseDnVecDescr {
+    uint32_t signature = 0;
+    int64_t size = 0;
+    void *values = nullptr;
+    aclDataType valueType = ACL_FLOAT;
+};
+
+// reference: sparse/common/aclsparse_descr_internal.h:121-128
+struct aclsparseDnMatDescr {
+    int64_t rows = 0;
+    int64_t cols = 0;
+    int64_t ld = 0;
+    aclsparseOrder_t order = ACL_SPARSE_ORDER_ROW;
+    void *values = nullptr;
+    aclDataType valueType = ACL_FLOAT;
+};
+
+namespace opsparse {
+
+// Error text goes to stderr only when OPS_SPARSE_LOG is set in the
+// environment; the success path never prints.
+void LogError(const char *fmt, ...);
+
+// Allocates the handle's default 4 MiB device workspace on first use (no-op when
+// a user workspace is active or the default one already exists).
+aclsparseStatus_t EnsureWorkspace(aclsparseContext *h);
+
+// Reads one scalar of `computeType` (ACL_FLOAT or ACL_INT32) for the launch
+// layer.  In HOST mode the value is dereferenced now (NULL gives `dflt`); in
+// DEVICE mode the address is passed on and the kernel reads it.
+OpsparseScalar MakeScalar(const void *p, aclDataType computeType, aclsparsePointerMode_t mode, double dflt);
+
+}  // namespace opsparse

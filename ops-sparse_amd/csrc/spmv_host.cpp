@@ -1,0 +1,213 @@
+// aclsparseSpMVGetBufferSize / aclsparseSpMVPreprocess / aclsparseSpMV.
+//
+// Argument checks, their order and their status codes follow the reference's
+// aclsparseSpMV (sparse/spmv/arch22/spmv_host.cpp:121-295).  Two things the
+// reference does on every call are deliberately absent: the device-to-host
+// copy of the whole row-offset array with a stream synchronisation (:86-112)
+// and the on-chip-buffer limit on the longest row (:244-252) — rows of any
+// length are handled by the merge-path kernels.
+#include "internal.h"
+
+namespace {
+
+struct SpmvCall {
+    const aclsparseSpMatDescr *A;
+    const aclsparseDnVecDescr *x;
+    const aclsparseDnVecDescr *y;
+    bool transpose;
+    int32_t valType, outType, computeIsInt;
+};
+
+int32_t DtypeOf(aclDataType t)
+{
+    switch (t) {
+        case ACL_FLOAT: return OPSPARSE_F32;
+        case ACL_FLOAT16: return OPSPARSE_F16;
+        case ACL_BF16: return OPSPARSE_BF16;
+        case ACL_INT32: return OPSPARSE_I32;
+        case ACL_INT8: return OPSPARSE_I8;
+        default: return -1;
+    }
+}
+
+// Checks shared by the three entry points, in the reference's order
+// (spmv_host.cpp:132-179, :225-240, :266-274).
+aclsparseStatus_t Validate(aclsparseHandle_t handle, aclsparseOperation_t opA, aclsparseConstSpMatDescr_t matA,
+                           aclsparseConstDnVecDescr_t vecX, aclsparseConstDnVecDescr_t vecY, aclDataType computeType,
+                           aclsparseSpMVAlg_t alg, SpmvCall *out)
+{
+    if (handle == nullptr) {
+        return ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR;
+    }
+    if (matA == nullptr || vecX == nullptr || vecY == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if (alg != ACL_SPARSE_SPMV_ALG_DEFAULT) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    if (computeType != ACL_FLOAT && computeType != ACL_INT32) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    if (matA->format != ACL_SPARSE_FORMAT_CSR || matA->idxBase != ACL_SPARSE_INDEX_BASE_ZERO) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    if (matA->rowOffsetsType != ACL_SPARSE_INDEX_32I || matA->colIndType != ACL_SPARSE_INDEX_32I) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    if (opA != ACL_SPARSE_OP_NON_TRANSPOSE && opA != ACL_SPARSE_OP_TRANSPOSE) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    out->A = matA;
+    out->x = vecX;
+    out->y = vecY;
+    out->transpose = (opA == ACL_SPARSE_OP_TRANSPOSE);
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t ValidateData(SpmvCall *c, aclDataType computeType)
+{
+    const aclsparseSpMatDescr *A = c->A;
+    // The reference insists on all five device pointers (spmv_host.cpp:225-230);
+    // arrays that hold no element (nnz == 0, an empty vector) may be NULL here.
+    if (A->rowOffsets == nullptr || (A->nnz > 0 && (A->colInd == nullptr || A->values == nullptr))) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    const int64_t needX = c->transpose ? A->rows : A->cols;
+    const int64_t needY = c->transpose ? A->cols : A->rows;
+    if ((needX > 0 && c->x->values == nullptr) || (needY > 0 && c->y->values == nullptr)) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if (c->x->size < needX || c->y->size < needY) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if (c->x->valueType != A->valueType) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    if (computeType == ACL_INT32 && (A->valueType != ACL_INT32 || c->y->valueType != ACL_INT32)) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    c->valType = DtypeOf(A->valueType);
+    c->outType = DtypeOf(c->y->valueType);
+    c->computeIsInt = (computeType == ACL_INT32) ? 1 : 0;
+    if (c->valType < 0 || c->outType < 0) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t FromLaunch(int rc)
+{
+    switch (rc) {
+        case OPSPARSE_OK: return ACL_SPARSE_STATUS_SUCCESS;
+        case OPSPARSE_E_INVALID: return ACL_SPARSE_STATUS_INVALID_VALUE;
+        case OPSPARSE_E_UNSUPPORTED: return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+        case OPSPARSE_E_WORKSPACE: return ACL_SPARSE_STATUS_INSUFFICIENT_RESOURCES;
+        default: return ACL_SPARSE_STATUS_EXECUTION_FAILED;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+aclsparseStatus_t aclsparseSpMVGetBufferSize(aclsparseHandle_t handle, aclsparseOperation_t opA, const void * /*alpha*/,
+                                             aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX,
+                                             const void * /*beta*/, aclsparseDnVecDescr_t vecY,
+                                             aclDataType computeType, aclsparseSpMVAlg_t alg, size_t *bufferSize)
+{
+    SpmvCall c{};
+    const aclsparseStatus_t st = Validate(handle, opA, matA, vecX, vecY, computeType, alg, &c);
+    if (st != ACL_SPARSE_STATUS_SUCCESS) {
+        return st;
+    }
+    if (bufferSize == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    *bufferSize = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOperation_t opA, const void * /*alpha*/,
+                                          aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX,
+                                          const void * /*beta*/, aclsparseDnVecDescr_t vecY, aclDataType computeType,
+                                          aclsparseSpMVAlg_t alg, void *externalBuffer)
+{
+    SpmvCall c{};
+    aclsparseStatus_t st = Validate(handle, opA, matA, vecX, vecY, computeType, alg, &c);
+    if (st != ACL_SPARSE_STATUS_SUCCESS) {
+        return st;
+    }
+    if (handle->stream == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    st = ValidateData(&c, computeType);
+    if (st != ACL_SPARSE_STATUS_SUCCESS) {
+        return st;
+    }
+    if (externalBuffer == nullptr) {
+        return ACL_SPARSE_STATUS_INSUFFICIENT_RESOURCES;
+    }
+    OpsparseSpmvPlan plan{};
+    const size_t bytes = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
+    const int rc = opsparse_spmv_csr_analyse(static_cast<const int32_t *>(matA->rowOffsets), matA->rows, matA->cols,
+                                             matA->nnz, externalBuffer, bytes, OPSPARSE_SPMV_AUTO, &plan,
+                                             handle->stream);
+    if (rc != OPSPARSE_OK) {
+        opsparse::LogError("aclsparseSpMVPreprocess: analysis failed (%d)", rc);
+        return FromLaunch(rc);
+    }
+    matA->spmv.buffer = externalBuffer;
+    matA->spmv.plan = plan;
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t aclsparseSpMV(aclsparseHandle_t handle, aclsparseOperation_t opA, const void *alpha,
+                                aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX, const void *beta,
+                                aclsparseDnVecDescr_t vecY, aclDataType computeType, aclsparseSpMVAlg_t alg,
+                                void *externalBuffer)
+{
+    SpmvCall c{};
+    aclsparseStatus_t st = Validate(handle, opA, matA, vecX, vecY, computeType, alg, &c);
+    if (st != ACL_SPARSE_STATUS_SUCCESS) {
+        return st;
+    }
+    // The reference refuses to run on the null stream (spmv_host.cpp:202-205).
+    if (handle->stream == nullptr) {
+        opsparse::LogError("aclsparseSpMV: no stream set, call aclsparseSetStream first");
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    st = ValidateData(&c, computeType);
+    if (st != ACL_SPARSE_STATUS_SUCCESS) {
+        return st;
+    }
+    const OpsparseScalar a = opsparse::MakeScalar(alpha, computeType, handle->pointerMode, 1.0);
+    const OpsparseScalar b = opsparse::MakeScalar(beta, computeType, handle->pointerMode, 0.0);
+
+    // A preprocessed buffer is only trusted when it is the one bound to matA.
+    const OpsparseSpmvPlan *plan = nullptr;
+    void *ws = nullptr;
+    size_t wsBytes = 0;
+    if (!c.transpose && externalBuffer != nullptr && matA->spmv.buffer == externalBuffer &&
+        matA->spmv.plan.rows == matA->rows && matA->spmv.plan.nnz == matA->nnz) {
+        plan = &matA->spmv.plan;
+        ws = externalBuffer;
+        wsBytes = static_cast<size_t>(plan->bytes);
+    } else if (!c.transpose && matA->nnz > 0) {
+        st = opsparse::EnsureWorkspace(handle);
+        if (st != ACL_SPARSE_STATUS_SUCCESS) {
+            return st;
+        }
+        ws = handle->workspace();
+        wsBytes = handle->workspaceBytes();
+    }
+    const int rc = opsparse_spmv_csr_launch(
+        plan, c.transpose ? 1 : 0, static_cast<const int32_t *>(matA->rowOffsets),
+        static_cast<const int32_t *>(matA->colInd), matA->values, vecX->values, vecY->values, matA->rows, matA->cols,
+        matA->nnz, a, b, c.valType, c.outType, c.computeIsInt, ws, wsBytes, handle->stream);
+    if (rc != OPSPARSE_OK) {
+        opsparse::LogError("aclsparseSpMV: launch failed (%d)", rc);
+    }
+    return FromLaunch(rc);
+}
+
+}  // extern "C"

@@ -1,0 +1,790 @@
+// CSR SpMV kernels for gfx950 and their C-ABI launcher.
+//
+// y = alpha * A * x + beta * y with A in CSR (int32 offsets and indices).
+// Replaces the device side of the reference's aclsparseSpMV
+// (sparse/spmv/arch22/kernels/spmv_kernel.h:27-310 for op = N, :321-640 for
+// op = T, dispatched by kernels/spmv_kernel.cpp:21-55).  The reference walks
+// one row at a time per core; here the rows are binned by length:
+//
+//   STREAM_ROWS  rows of at most a few dozen non-zeros.  A workgroup owns a
+//                fixed block of consecutive rows, loads their contiguous
+//                (colind, value) range with full-width coalesced non-temporal
+//                loads, gathers x, parks the products in LDS and then lets
+//                1..8 lanes per row add them up in stored order.
+//   VECTOR_ROWS  medium rows: a group of 4..64 lanes strides along one row and
+//                reduces with cross-lane shuffles.  Needs no workspace.
+//   MERGE_PATH   skewed (power-law) rows: the merge of "row ends" and "non-zero
+//                indices" is cut into equal pieces, so every workgroup gets the
+//                same rows + nnz whatever the row lengths are.  Products are
+//                staged in LDS as above; a row cut by a workgroup boundary
+//                leaves a carry-out, and a small fix-up kernel adds the pieces
+//                in ascending order, so the result is deterministic.
+//
+// Memory traffic per launch is the compulsory nnz*(sizeof(val)+4) +
+// (rows+1)*4 + rows*sizeof(y)*(1 + [beta != 0]) plus x: the kernels are
+// HBM-bound streaming kernels, there is no matrix-core work in them.
+#include <type_traits>
+
+#include "device_utils.h"
+
+namespace opsparse {
+
+// ------------------------------------------------------------- epilogue
+
+template <typename OutT, typename AccT>
+__device__ __forceinline__ void StoreRow(OutT *__restrict__ y, int64_t row, AccT sum, AccT alpha, AccT beta,
+                                         bool betaZero)
+{
+    AccT r = alpha * sum;
+    if (!betaZero) {
+        r += beta * ToAcc<AccT>(y[row]);
+    }
+    y[row] = FromAcc<OutT>(r);
+}
+
+// Loads 4 consecutive values and converts them to the accumulator type.
+template <typename AccT, typename ValT>
+__device__ __forceinline__ void LoadVals4(const ValT *p, AccT out[4])
+{
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        out[i] = ToAcc<AccT>(LoadStream(p + i));
+    }
+}
+template <>
+__device__ __forceinline__ void LoadVals4<double, float>(const float *p, double out[4])
+{
+    const Float4U v = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(p));
+    out[0] = v.x;
+    out[1] = v.y;
+    out[2] = v.z;
+    out[3] = v.w;
+}
+
+// Products val[k] * x[col[k]] for k in [0, count) of one contiguous nnz range,
+// written to LDS.  Each lane takes 4 consecutive non-zeros per step, so a
+// wavefront reads 1 KiB of indices and 1 KiB of fp32 values per instruction.
+template <typename ValT, typename AccT>
+__device__ __forceinline__ void StageProducts(const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+                                              const ValT *__restrict__ x, int32_t count, AccT *__restrict__ prod)
+{
+    const int32_t tid = threadIdx.x;
+    for (int32_t k = tid * 4; k < count; k += kBlockThreads * 4) {
+        if (k + 4 <= count) {
+            const Int4U c = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(colInd + k));
+            AccT v[4];
+            LoadVals4<AccT, ValT>(vals + k, v);
+            const AccT x0 = ToAcc<AccT>(x[c.x]);
+            const AccT x1 = ToAcc<AccT>(x[c.y]);
+            const AccT x2 = ToAcc<AccT>(x[c.z]);
+            const AccT x3 = ToAcc<AccT>(x[c.w]);
+            prod[k + 0] = v[0] * x0;
+            prod[k + 1] = v[1] * x1;
+            prod[k + 2] = v[2] * x2;
+            prod[k + 3] = v[3] * x3;
+        } else {
+            for (int32_t q = k; q < count; ++q) {
+                prod[q] = ToAcc<AccT>(LoadStream(vals + q)) * ToAcc<AccT>(x[LoadStream(colInd + q)]);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------- y = beta * y
+
+template <typename OutT, typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmvScaleKernel(OutT *__restrict__ y, int64_t len,
+                                                                 OpsparseScalar betaS)
+{
+    const AccT beta = ReadScalar<AccT>(betaS);
+    const bool betaZero = (beta == AccT(0));
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlockThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; i < len; i += stride) {
+        y[i] = betaZero ? FromAcc<OutT>(AccT(0)) : FromAcc<OutT>(beta * ToAcc<AccT>(y[i]));
+    }
+}
+
+// ------------------------------------------------------------- row statistics
+
+// stats[0] = max row length.  stats must be zeroed before the launch.
+__global__ __launch_bounds__(kBlockThreads) void RowStatsKernel(const int32_t *__restrict__ rowOffsets, int64_t rows,
+                                                                int32_t *__restrict__ stats)
+{
+    int32_t best = 0;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlockThreads;
+    for (int64_t r = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; r < rows; r += stride) {
+        const int32_t len = rowOffsets[r + 1] - rowOffsets[r];
+        best = len > best ? len : best;
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        const int32_t other = __shfl_xor(best, off, kWave);
+        best = other > best ? other : best;
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0 && best > 0) {
+        atomicMax(stats, best);
+    }
+}
+
+// ------------------------------------------------------------- STREAM_ROWS
+
+// One workgroup = `rowsPerBlock` consecutive rows; dynamic LDS holds
+// rowsPerBlock * maxRowNnz products.
+template <typename ValT, typename OutT, typename AccT, int G>
+__global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ x, OutT *__restrict__ y, int64_t rows, int32_t rowsPerBlock, OpsparseScalar alphaS,
+    OpsparseScalar betaS)
+{
+    extern __shared__ __align__(16) unsigned char ldsRaw[];
+    AccT *prod = reinterpret_cast<AccT *>(ldsRaw);
+
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    const AccT beta = ReadScalar<AccT>(betaS);
+    const bool betaZero = (beta == AccT(0));
+
+    const int64_t tile = XcdContiguousTile(blockIdx.x, gridDim.x);
+    const int64_t r0 = tile * rowsPerBlock;
+    const int64_t r1 = (r0 + rowsPerBlock < rows) ? r0 + rowsPerBlock : rows;
+    const int32_t first = rowOffsets[r0];
+    const int32_t count = rowOffsets[r1] - first;
+
+    // Issue this lane's first row bounds before the long-latency streaming phase.
+    constexpr int kGroups = kBlockThreads / G;
+    const int32_t lane = threadIdx.x % G;
+    int64_t r = r0 + threadIdx.x / G;
+    int32_t s = 0, e = 0;
+    if (r < r1) {
+        s = rowOffsets[r];
+        e = rowOffsets[r + 1];
+    }
+
+    StageProducts<ValT, AccT>(colInd + first, vals + first, x, count, prod);
+    __syncthreads();
+
+    while (r < r1) {
+        AccT sum = AccT(0);
+        for (int32_t k = s - first + lane; k < e - first; k += G) {
+            sum += prod[k];
+        }
+        sum = GroupSum<G>(sum);
+        if (lane == 0) {
+            StoreRow<OutT, AccT>(y, r, sum, alpha, beta, betaZero);
+        }
+        r += kGroups;
+        if (r < r1) {
+            s = rowOffsets[r];
+            e = rowOffsets[r + 1];
+        }
+    }
+}
+
+// ------------------------------------------------------------- VECTOR_ROWS
+
+template <typename ValT, typename OutT, typename AccT, int G>
+__global__ __launch_bounds__(kBlockThreads) void SpmvVectorRowsKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ x, OutT *__restrict__ y, int64_t rows, OpsparseScalar alphaS, OpsparseScalar betaS)
+{
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    const AccT beta = ReadScalar<AccT>(betaS);
+    const bool betaZero = (beta == AccT(0));
+
+    constexpr int kGroups = kBlockThreads / G;
+    const int64_t tile = XcdContiguousTile(blockIdx.x, gridDim.x);
+    const int64_t r = tile * kGroups + threadIdx.x / G;
+    const int32_t lane = threadIdx.x % G;
+    if (r >= rows) {
+        return;  // whole groups leave together: G divides the wavefront
+    }
+    const int32_t s = rowOffsets[r];
+    const int32_t e = rowOffsets[r + 1];
+    AccT sum0 = AccT(0), sum1 = AccT(0);
+    int32_t k = s + lane;
+    for (; k + G < e; k += 2 * G) {  // two independent gathers in flight per lane
+        const int32_t c0 = LoadStream(colInd + k);
+        const int32_t c1 = LoadStream(colInd + k + G);
+        const AccT v0 = ToAcc<AccT>(LoadStream(vals + k));
+        const AccT v1 = ToAcc<AccT>(LoadStream(vals + k + G));
+        sum0 += v0 * ToAcc<AccT>(x[c0]);
+        sum1 += v1 * ToAcc<AccT>(x[c1]);
+    }
+    if (k < e) {
+        sum0 += ToAcc<AccT>(LoadStream(vals + k)) * ToAcc<AccT>(x[LoadStream(colInd + k)]);
+    }
+    const AccT sum = GroupSum<G>(sum0 + sum1);
+    if (lane == 0) {
+        StoreRow<OutT, AccT>(y, r, sum, alpha, beta, betaZero);
+    }
+}
+
+// ------------------------------------------------------------- MERGE_PATH
+
+constexpr int kMergeItems = 2048;  // rows + non-zeros consumed by one workgroup
+
+__device__ __forceinline__ int64_t MergeDiagonal(int64_t block, int64_t rows, int64_t nnz)
+{
+    const int64_t d = block * kMergeItems;
+    return d < rows + nnz ? d : rows + nnz;
+}
+
+// part[b] = number of rows completed before diagonal b * kMergeItems of the
+// merge of (row end offsets, non-zero indices): the smallest i with
+// rowOffsets[i + 1] > d - i - 1.
+__global__ __launch_bounds__(kBlockThreads) void MergePartitionKernel(const int32_t *__restrict__ rowOffsets,
+                                                                      int64_t rows, int64_t nnz, int32_t numBlocks,
+                                                                      int32_t *__restrict__ part)
+{
+    const int64_t b = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
+    if (b > numBlocks) {
+        return;
+    }
+    const int64_t d = MergeDiagonal(b, rows, nnz);
+    int64_t lo = d > nnz ? d - nnz : 0;
+    int64_t hi = d < rows ? d : rows;
+    while (lo < hi) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (static_cast<int64_t>(rowOffsets[mid + 1]) <= d - mid - 1) {
+            lo = mid + 1;
+        } else {
+            hi = mid;
+        }
+    }
+    part[b] = static_cast<int32_t>(lo);
+}
+
+// Workgroup b consumes non-zeros [j0, j1) and completes rows [i0, i1), where
+// (i0, j0) and (i1, j1) are the merge-path coordinates of its two diagonals.
+//   - a completed row that started before j0 ("spanning" row, only i0 can be
+//     one) is not written here: its last piece goes to head[b];
+//   - the non-zeros after the last completed row belong to row i1, which ends
+//     in a later workgroup: their sum goes to carry[b];
+//   - every other completed row gets its final y value here.
+template <typename ValT, typename OutT, typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmvMergeKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ x, OutT *__restrict__ y, int64_t rows, int64_t nnz,
+    const int32_t *__restrict__ part, AccT *__restrict__ carry, AccT *__restrict__ head, OpsparseScalar alphaS,
+    OpsparseScalar betaS)
+{
+    __shared__ AccT prod[kMergeItems];
+
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    const AccT beta = ReadScalar<AccT>(betaS);
+    const bool betaZero = (beta == AccT(0));
+
+    const int64_t b = XcdContiguousTile(blockIdx.x, gridDim.x);
+    const int64_t i0 = part[b];
+    const int64_t i1 = part[b + 1];
+    const int64_t j0 = MergeDiagonal(b, rows, nnz) - i0;
+    const int64_t j1 = MergeDiagonal(b + 1, rows, nnz) - i1;
+    const int32_t count = static_cast<int32_t>(j1 - j0);
+
+    StageProducts<ValT, AccT>(colInd + j0, vals + j0, x, count, prod);
+    __syncthreads();
+
+    // Rows i0 .. i1-1 complete here; row i1 (if it exists) collects the tail.
+    const int32_t numRows = static_cast<int32_t>(i1 - i0) + (i1 < rows ? 1 : 0);
+    if (numRows == 0) {
+        return;
+    }
+    // Lanes per row from the average row length of this workgroup.
+    int g = 1;
+    while (g < kWave && count > 8 * g * numRows) {
+        g <<= 1;
+    }
+    const int32_t groups = kBlockThreads / g;
+    const int32_t lane = threadIdx.x & (g - 1);
+    for (int32_t q = threadIdx.x / g; q < numRows; q += groups) {
+        const int64_t row = i0 + q;
+        const bool completes = row < i1;
+        const int64_t begin = rowOffsets[row];
+        const int32_t s = begin > j0 ? static_cast<int32_t>(begin - j0) : 0;
+        const int32_t e = completes ? static_cast<int32_t>(rowOffsets[row + 1] - j0) : count;
+        AccT sum = AccT(0);
+        for (int32_t k = s + lane; k < e; k += g) {
+            sum += prod[k];
+        }
+        sum = GroupSumDyn(sum, g);
+        if (lane == 0) {
+            if (!completes) {
+                carry[b] = sum;
+            } else if (begin < j0) {
+                head[b] = sum;
+            } else {
+                StoreRow<OutT, AccT>(y, row, sum, alpha, beta, betaZero);
+            }
+        }
+    }
+}
+
+// One lane per workgroup of the merge kernel: if that workgroup completed a
+// spanning row, add the carries of the workgroups the row passed through (in
+// ascending order) to its head piece and write the row's final value.
+template <typename OutT, typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmvMergeFixupKernel(
+    const int32_t *__restrict__ rowOffsets, OutT *__restrict__ y, int64_t rows, int64_t nnz, int32_t numBlocks,
+    const int32_t *__restrict__ part, const AccT *__restrict__ carry, const AccT *__restrict__ head,
+    OpsparseScalar alphaS, OpsparseScalar betaS)
+{
+    const int64_t b = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
+    if (b >= numBlocks) {
+        return;
+    }
+    const int64_t i0 = part[b];
+    const int64_t i1 = part[b + 1];
+    if (i1 <= i0) {
+        return;  // no row ends in this workgroup
+    }
+    const int64_t begin = rowOffsets[i0];
+    if (begin >= MergeDiagonal(b, rows, nnz) - i0) {
+        return;  // first completed row also starts here
+    }
+    // Walk back to the workgroup in which row i0 starts.
+    int64_t p = b - 1;
+    while (p > 0 && MergeDiagonal(p, rows, nnz) - part[p] > begin) {
+        --p;
+    }
+    AccT sum = AccT(0);
+    for (; p < b; ++p) {
+        sum += carry[p];
+    }
+    sum += head[b];
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    const AccT beta = ReadScalar<AccT>(betaS);
+    StoreRow<OutT, AccT>(y, i0, sum, alpha, beta, beta == AccT(0));
+}
+
+// ------------------------------------------------------------- op(A) = A^T
+
+// y[col] += alpha * x[row] * val for every stored element; y was scaled by
+// beta beforehand.  Floating point only (hardware fp32 atomic add); the order
+// of the additions is not fixed, as in the reference's transpose path
+// (sparse/spmv/arch22/kernels/spmv_kernel.h:584-624).
+template <typename ValT, typename AccT, int G>
+__global__ __launch_bounds__(kBlockThreads) void SpmvTransposeScatterKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ x, float *__restrict__ y, int64_t rows, OpsparseScalar alphaS)
+{
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    constexpr int kGroups = kBlockThreads / G;
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * kGroups + threadIdx.x / G;
+    if (r >= rows) {
+        return;
+    }
+    const AccT ax = alpha * ToAcc<AccT>(x[r]);
+    if (ax == AccT(0)) {
+        return;
+    }
+    const int32_t e = rowOffsets[r + 1];
+    for (int32_t k = rowOffsets[r] + threadIdx.x % G; k < e; k += G) {
+        atomicAdd(y + LoadStream(colInd + k), static_cast<float>(ax * ToAcc<AccT>(LoadStream(vals + k))));
+    }
+}
+
+// ------------------------------------------------------------- copy yard-stick
+
+typedef uint32_t Uint4V __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(kBlockThreads) void CopyKernel(const Uint4V *__restrict__ src, Uint4V *__restrict__ dst,
+                                                            size_t n16)
+{
+    const size_t stride = static_cast<size_t>(gridDim.x) * kBlockThreads;
+    for (size_t i = static_cast<size_t>(blockIdx.x) * kBlockThreads + threadIdx.x; i < n16; i += stride) {
+        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+    }
+}
+
+// =============================================================== host side
+
+namespace {
+
+struct SpmvArgs {
+    const int32_t *rowOffsets;
+    const int32_t *colInd;
+    const void *vals;
+    const void *x;
+    void *y;
+    int64_t rows, cols, nnz;
+    OpsparseScalar alpha, beta;
+    void *ws;
+    size_t wsBytes;
+    hipStream_t stream;
+};
+
+inline int CheckLaunch()
+{
+    return hipGetLastError() == hipSuccess ? OPSPARSE_OK : OPSPARSE_E_LAUNCH;
+}
+
+inline uint32_t GridFor(int64_t items, int64_t perBlock)
+{
+    return static_cast<uint32_t>((items + perBlock - 1) / perBlock);
+}
+
+struct MergeLayout {
+    int32_t blocks;
+    int64_t partOff, carryOff, headOff, bytes;
+};
+
+// Workspace layout of the merge-path family: 256-byte header (row statistics),
+// partition table, carries, heads.  Carries are sized for the widest
+// accumulator (8 bytes).
+MergeLayout MakeMergeLayout(int64_t rows, int64_t nnz)
+{
+    MergeLayout l{};
+    l.blocks = static_cast<int32_t>((rows + nnz + kMergeItems - 1) / kMergeItems);
+    l.partOff = 256;
+    l.carryOff = l.partOff + static_cast<int64_t>((static_cast<size_t>(l.blocks) + 1) * 4 + 255) / 256 * 256;
+    l.headOff = l.carryOff + static_cast<int64_t>((static_cast<size_t>(l.blocks)) * 8 + 255) / 256 * 256;
+    l.bytes = l.headOff + static_cast<int64_t>((static_cast<size_t>(l.blocks)) * 8 + 255) / 256 * 256;
+    return l;
+}
+
+template <typename ValT, typename OutT, typename AccT, int G>
+int LaunchStream(const SpmvArgs &a, int32_t rowsPerBlock, int32_t maxRowNnz)
+{
+    const size_t lds = static_cast<size_t>(rowsPerBlock) * static_cast<size_t>(maxRowNnz) * sizeof(AccT);
+    const uint32_t grid = GridFor(a.rows, rowsPerBlock);
+    hipLaunchKernelGGL((SpmvStreamRowsKernel<ValT, OutT, AccT, G>), dim3(grid), dim3(kBlockThreads), lds, a.stream,
+                       a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
+                       static_cast<OutT *>(a.y), a.rows, rowsPerBlock, a.alpha, a.beta);
+    return CheckLaunch();
+}
+
+template <typename ValT, typename OutT, typename AccT, int G>
+int LaunchVector(const SpmvArgs &a)
+{
+    const uint32_t grid = GridFor(a.rows, kBlockThreads / G);
+    hipLaunchKernelGGL((SpmvVectorRowsKernel<ValT, OutT, AccT, G>), dim3(grid), dim3(kBlockThreads), 0, a.stream,
+                       a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
+                       static_cast<OutT *>(a.y), a.rows, a.alpha, a.beta);
+    return CheckLaunch();
+}
+
+template <typename ValT, typename OutT, typename AccT>
+int LaunchMerge(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
+{
+    auto *base = static_cast<unsigned char *>(a.ws);
+    auto *part = reinterpret_cast<int32_t *>(base + plan.partOff);
+    auto *carry = reinterpret_cast<AccT *>(base + plan.carryOff);
+    auto *head = reinterpret_cast<AccT *>(base + plan.headOff);
+    const int32_t nb = plan.mergeBlocks;
+    if (!plan.partitionReady) {
+        hipLaunchKernelGGL(MergePartitionKernel, dim3(GridFor(nb + 1, kBlockThreads)), dim3(kBlockThreads), 0,
+                           a.stream, a.rowOffsets, a.rows, a.nnz, nb, part);
+    }
+    hipLaunchKernelGGL((SpmvMergeKernel<ValT, OutT, AccT>), dim3(nb), dim3(kBlockThreads), 0, a.stream, a.rowOffsets,
+                       a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
+                       static_cast<OutT *>(a.y), a.rows, a.nnz, part, carry, head, a.alpha, a.beta);
+    hipLaunchKernelGGL((SpmvMergeFixupKernel<OutT, AccT>), dim3(GridFor(nb, kBlockThreads)), dim3(kBlockThreads), 0,
+                       a.stream, a.rowOffsets, static_cast<OutT *>(a.y), a.rows, a.nnz, nb, part, carry, head,
+                       a.alpha, a.beta);
+    return CheckLaunch();
+}
+
+template <typename OutT, typename AccT>
+int LaunchScale(OutT *y, int64_t len, OpsparseScalar beta, hipStream_t stream)
+{
+    if (len <= 0) {
+        return OPSPARSE_OK;
+    }
+    int64_t grid = (len + kBlockThreads - 1) / kBlockThreads;
+    grid = grid > 65536 ? 65536 : grid;
+    hipLaunchKernelGGL((SpmvScaleKernel<OutT, AccT>), dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0,
+                       stream, y, len, beta);
+    return CheckLaunch();
+}
+
+template <typename ValT, typename OutT, typename AccT>
+int RunPlanned(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
+{
+    switch (plan.kernel) {
+        case OPSPARSE_SPMV_SCALE_ONLY:
+            return LaunchScale<OutT, AccT>(static_cast<OutT *>(a.y), a.rows, a.beta, a.stream);
+        case OPSPARSE_SPMV_STREAM_ROWS:
+            switch (plan.lanesPerRow) {
+                case 1: return LaunchStream<ValT, OutT, AccT, 1>(a, plan.rowsPerBlock, plan.maxRowNnz);
+                case 2: return LaunchStream<ValT, OutT, AccT, 2>(a, plan.rowsPerBlock, plan.maxRowNnz);
+                case 4: return LaunchStream<ValT, OutT, AccT, 4>(a, plan.rowsPerBlock, plan.maxRowNnz);
+                case 8: return LaunchStream<ValT, OutT, AccT, 8>(a, plan.rowsPerBlock, plan.maxRowNnz);
+                default: return OPSPARSE_E_INVALID;
+            }
+        case OPSPARSE_SPMV_VECTOR_ROWS:
+            switch (plan.lanesPerRow) {
+                case 4: return LaunchVector<ValT, OutT, AccT, 4>(a);
+                case 8: return LaunchVector<ValT, OutT, AccT, 8>(a);
+                case 16: return LaunchVector<ValT, OutT, AccT, 16>(a);
+                case 32: return LaunchVector<ValT, OutT, AccT, 32>(a);
+                case 64: return LaunchVector<ValT, OutT, AccT, 64>(a);
+                default: return OPSPARSE_E_INVALID;
+            }
+        case OPSPARSE_SPMV_MERGE_PATH:
+            if (a.ws == nullptr || static_cast<int64_t>(a.wsBytes) < plan.bytes) {
+                return OPSPARSE_E_WORKSPACE;
+            }
+            return LaunchMerge<ValT, OutT, AccT>(a, plan);
+        default:
+            return OPSPARSE_E_INVALID;
+    }
+}
+
+int32_t VectorLanesFor(int64_t rows, int64_t nnz)
+{
+    const int64_t mean = rows > 0 ? nnz / rows : 0;
+    int32_t g = 4;
+    while (g < kWave && mean > 4 * g) {
+        g <<= 1;
+    }
+    return g;
+}
+
+// No plan: merge-path with the partition rebuilt into the workspace, or the
+// workspace-free vector kernel when the workspace is too small.
+OpsparseSpmvPlan AdHocPlan(int64_t rows, int64_t nnz, size_t wsBytes, const void *ws)
+{
+    OpsparseSpmvPlan p{};
+    p.rows = rows;
+    p.nnz = nnz;
+    if (nnz == 0) {
+        p.kernel = OPSPARSE_SPMV_SCALE_ONLY;
+        return p;
+    }
+    const MergeLayout l = MakeMergeLayout(rows, nnz);
+    if (ws != nullptr && static_cast<int64_t>(wsBytes) >= l.bytes) {
+        p.kernel = OPSPARSE_SPMV_MERGE_PATH;
+        p.mergeBlocks = l.blocks;
+        p.partOff = l.partOff;
+        p.carryOff = l.carryOff;
+        p.headOff = l.headOff;
+        p.bytes = l.bytes;
+        p.partitionReady = 0;
+    } else {
+        p.kernel = OPSPARSE_SPMV_VECTOR_ROWS;
+        p.lanesPerRow = VectorLanesFor(rows, nnz);
+    }
+    return p;
+}
+
+template <typename ValT, typename AccT>
+int RunTranspose(const SpmvArgs &a, int32_t outType)
+{
+    if (outType != OPSPARSE_F32) {
+        return OPSPARSE_E_UNSUPPORTED;
+    }
+    // y has `cols` elements for the transposed product.
+    int rc = LaunchScale<float, AccT>(static_cast<float *>(a.y), a.cols, a.beta, a.stream);
+    if (rc != OPSPARSE_OK || a.nnz == 0 || a.rows == 0) {
+        return rc;
+    }
+    const int32_t g = VectorLanesFor(a.rows, a.nnz);
+    auto launch = [&](auto tag) {
+        constexpr int G = decltype(tag)::value;
+        hipLaunchKernelGGL((SpmvTransposeScatterKernel<ValT, AccT, G>), dim3(GridFor(a.rows, kBlockThreads / G)),
+                           dim3(kBlockThreads), 0, a.stream, a.rowOffsets, a.colInd,
+                           static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
+                           static_cast<float *>(a.y), a.rows, a.alpha);
+    };
+    switch (g) {
+        case 4: launch(std::integral_constant<int, 4>{}); break;
+        case 8: launch(std::integral_constant<int, 8>{}); break;
+        case 16: launch(std::integral_constant<int, 16>{}); break;
+        case 32: launch(std::integral_constant<int, 32>{}); break;
+        default: launch(std::integral_constant<int, 64>{}); break;
+    }
+    return CheckLaunch();
+}
+
+template <typename ValT, typename OutT, typename AccT>
+int RunTyped(const OpsparseSpmvPlan *plan, const SpmvArgs &a)
+{
+    if (plan != nullptr) {
+        return RunPlanned<ValT, OutT, AccT>(a, *plan);
+    }
+    const OpsparseSpmvPlan adhoc = AdHocPlan(a.rows, a.nnz, a.wsBytes, a.ws);
+    return RunPlanned<ValT, OutT, AccT>(a, adhoc);
+}
+
+}  // namespace
+}  // namespace opsparse
+
+// ================================================================== C ABI
+
+using namespace opsparse;
+
+extern "C" {
+
+size_t opsparse_spmv_csr_workspace_bytes(int64_t rows, int64_t nnz)
+{
+    if (rows < 0 || nnz < 0) {
+        return 0;
+    }
+    return static_cast<size_t>(MakeMergeLayout(rows, nnz).bytes);
+}
+
+int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t cols, int64_t nnz, void *workspace,
+                              size_t workspaceBytes, int32_t forceKernel, OpsparseSpmvPlan *plan, void *stream)
+{
+    (void)cols;
+    if (plan == nullptr || rows < 0 || nnz < 0 || (rows > 0 && rowOffsets == nullptr)) {
+        return OPSPARSE_E_INVALID;
+    }
+    auto s = static_cast<hipStream_t>(stream);
+    OpsparseSpmvPlan p{};
+    p.rows = rows;
+    p.nnz = nnz;
+    if (rows == 0 || nnz == 0) {
+        p.kernel = OPSPARSE_SPMV_SCALE_ONLY;
+        *plan = p;
+        return OPSPARSE_OK;
+    }
+    const MergeLayout l = MakeMergeLayout(rows, nnz);
+    if (workspace == nullptr || static_cast<int64_t>(workspaceBytes) < l.bytes) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    // Longest row, reduced on the device into the workspace header.
+    auto *stats = static_cast<int32_t *>(workspace);
+    if (hipMemsetAsync(stats, 0, 256, s) != hipSuccess) {
+        return OPSPARSE_E_LAUNCH;
+    }
+    int64_t grid = (rows + kBlockThreads - 1) / kBlockThreads;
+    grid = grid > 4096 ? 4096 : grid;
+    hipLaunchKernelGGL(RowStatsKernel, dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0, s, rowOffsets, rows,
+                       stats);
+    int32_t maxRow = 0;
+    if (hipMemcpyAsync(&maxRow, stats, sizeof(int32_t), hipMemcpyDeviceToHost, s) != hipSuccess ||
+        hipStreamSynchronize(s) != hipSuccess) {
+        return OPSPARSE_E_LAUNCH;
+    }
+    p.maxRowNnz = maxRow;
+
+    const double mean = static_cast<double>(nnz) / static_cast<double>(rows);
+    int32_t kernel = forceKernel;
+    if (kernel == OPSPARSE_SPMV_AUTO) {
+        if (maxRow <= 48) {
+            kernel = OPSPARSE_SPMV_STREAM_ROWS;
+        } else if (mean >= 32.0 && static_cast<double>(maxRow) <= 16.0 * mean) {
+            kernel = OPSPARSE_SPMV_VECTOR_ROWS;
+        } else {
+            kernel = OPSPARSE_SPMV_MERGE_PATH;
+        }
+    }
+    p.kernel = kernel;
+    switch (kernel) {
+        case OPSPARSE_SPMV_STREAM_ROWS: {
+            if (maxRow > 48) {
+                return OPSPARSE_E_UNSUPPORTED;  // products of a row block would not fit LDS
+            }
+            const int32_t g = maxRow <= 12 ? 1 : (maxRow <= 24 ? 2 : 4);
+            p.lanesPerRow = g;
+            // One pass of the 256 / g lane groups over the block's rows.
+            p.rowsPerBlock = kBlockThreads / g;
+            break;
+        }
+        case OPSPARSE_SPMV_VECTOR_ROWS:
+            p.lanesPerRow = VectorLanesFor(rows, nnz);
+            break;
+        case OPSPARSE_SPMV_MERGE_PATH: {
+            p.mergeBlocks = l.blocks;
+            p.partOff = l.partOff;
+            p.carryOff = l.carryOff;
+            p.headOff = l.headOff;
+            p.bytes = l.bytes;
+            auto *part = reinterpret_cast<int32_t *>(static_cast<unsigned char *>(workspace) + l.partOff);
+            hipLaunchKernelGGL(MergePartitionKernel, dim3(GridFor(l.blocks + 1, kBlockThreads)), dim3(kBlockThreads),
+                               0, s, rowOffsets, rows, nnz, l.blocks, part);
+            if (CheckLaunch() != OPSPARSE_OK) {
+                return OPSPARSE_E_LAUNCH;
+            }
+            p.partitionReady = 1;
+            break;
+        }
+        default:
+            return OPSPARSE_E_INVALID;
+    }
+    *plan = p;
+    return OPSPARSE_OK;
+}
+
+int opsparse_spmv_csr_launch(const OpsparseSpmvPlan *plan, int32_t transpose, const int32_t *rowOffsets,
+                             const int32_t *colInd, const void *csrValues, const void *x, void *y, int64_t rows,
+                             int64_t cols, int64_t nnz, OpsparseScalar alpha, OpsparseScalar beta, int32_t valType,
+                             int32_t outType, int32_t computeIsInt, void *workspace, size_t workspaceBytes,
+                             void *stream)
+{
+    if (rows < 0 || cols < 0 || nnz < 0) {
+        return OPSPARSE_E_INVALID;
+    }
+    const int64_t outLen = transpose ? cols : rows;
+    if (outLen == 0) {
+        return OPSPARSE_OK;  // nothing to write
+    }
+    if (y == nullptr || (rows > 0 && rowOffsets == nullptr) ||
+        (nnz > 0 && (colInd == nullptr || csrValues == nullptr || x == nullptr))) {
+        return OPSPARSE_E_INVALID;
+    }
+    if (plan != nullptr && (plan->rows != rows || plan->nnz != nnz)) {
+        return OPSPARSE_E_INVALID;
+    }
+    SpmvArgs a{rowOffsets, colInd,         csrValues, x, y, rows, cols, nnz, alpha, beta, workspace,
+               workspaceBytes, static_cast<hipStream_t>(stream)};
+
+    if (transpose) {
+        if (computeIsInt) {
+            return OPSPARSE_E_UNSUPPORTED;
+        }
+        switch (valType) {
+            case OPSPARSE_F32: return RunTranspose<float, double>(a, outType);
+            case OPSPARSE_F16: return RunTranspose<Half, double>(a, outType);
+            case OPSPARSE_BF16: return RunTranspose<Bf16, double>(a, outType);
+            default: return OPSPARSE_E_UNSUPPORTED;
+        }
+    }
+    if (rows > 0 && nnz == 0) {
+        plan = nullptr;  // AdHocPlan turns this into the scale kernel
+    }
+    if (computeIsInt) {
+        if (valType == OPSPARSE_I32 && outType == OPSPARSE_I32) {
+            return RunTyped<int32_t, int32_t, int32_t>(plan, a);
+        }
+        return OPSPARSE_E_UNSUPPORTED;
+    }
+    switch (valType) {
+        case OPSPARSE_F32:
+            if (outType == OPSPARSE_F32) return RunTyped<float, float, double>(plan, a);
+            break;
+        case OPSPARSE_F16:
+            if (outType == OPSPARSE_F32) return RunTyped<Half, float, double>(plan, a);
+            if (outType == OPSPARSE_F16) return RunTyped<Half, Half, double>(plan, a);
+            break;
+        case OPSPARSE_BF16:
+            if (outType == OPSPARSE_F32) return RunTyped<Bf16, float, double>(plan, a);
+            if (outType == OPSPARSE_BF16) return RunTyped<Bf16, Bf16, double>(plan, a);
+            break;
+        case OPSPARSE_I32:
+            if (outType == OPSPARSE_F32) return RunTyped<int32_t, float, double>(plan, a);
+            break;
+        default:
+            break;
+    }
+    return OPSPARSE_E_UNSUPPORTED;
+}
+
+int opsparse_copy_launch(const void *src, void *dst, size_t bytes, void *stream)
+{
+    if (src == nullptr || dst == nullptr || bytes % 16 != 0) {
+        return OPSPARSE_E_INVALID;
+    }
+    if (bytes == 0) {
+        return OPSPARSE_OK;
+    }
+    const size_t n16 = bytes / 16;
+    size_t grid = (n16 + kBlockThreads - 1) / kBlockThreads;
+    grid = grid > 8192 ? 8192 : grid;
+    hipLaunchKernelGGL(CopyKernel, dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const Uint4V *>(src), static_cast<Uint4V *>(dst),
+                       n16);
+    return CheckLaunch();
+}
+
+}  // extern "C"

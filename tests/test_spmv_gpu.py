@@ -1,0 +1,138 @@
+"""GPU parity tests for aclsparseSpMV: the HIP path against the CPU oracle,
+called through the C ABI.
+
+Tolerance (fp32 output): per element |d| <= 1e-5 * max(|oracle|, 1e-30) against
+the fp64-accumulated oracle — the library accumulates in fp64 and rounds once,
+so the result is within an ulp of the oracle's.  The reference's own looser
+checks (fp32 golden, 2^-16 + 2^-10 |g|; MERE/MARE with the 2^-14 floor) are
+asserted as well where the reference test uses them.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import csr_from_lengths, random_csr, run_spmv
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-5
+
+
+def check_fp32(y, rows, cols, rowptr, colind, val, x, y0, alpha, beta):
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, alpha, beta)
+    err = oracle.max_rel_err(y[:rows], gold)
+    assert err <= RTOL, "max rel err %.3e" % err
+    # the reference's own acceptance rule against its fp32 golden (spmv_test.cpp:208-220, 271-307)
+    g32 = oracle.spmv_f32(rows, rowptr, colind, val, x, y0 if y0 is not None else np.zeros(rows, np.float32),
+                          alpha, beta)
+    d = np.abs(y[:rows] - g32)
+    ok = d <= 2.0 ** -16 + 2.0 ** -10 * np.abs(g32)
+    assert rows == 0 or abs(alpha) > 100 or (ok.mean() >= 0.99 and d.max() <= 1e-2)
+    mere, mare, mism, _ = oracle.mere_mare(y[:rows], gold)
+    assert mism == 0 and mere < 1e-6 and mare < 5e-6
+
+
+def test_c1_reference_config(osa, gpu_ctx):
+    """m = n = 4096, 16 nnz/row from the reference generator (seed 42), alpha 1, beta 0."""
+    rowptr, colind, val = oracle.fill_csr(42, 4096, 4096, 65536, -1.0, 1.0)
+    x = oracle.fill_dense(43, 4096, -1.0, 1.0)
+    y0 = np.full(4096, np.nan, np.float32)      # beta == 0: y must not be read
+    for pre in (True, False):
+        y = run_spmv(osa, gpu_ctx, 4096, 4096, rowptr, colind, val, x, y0, 1.0, 0.0, preprocess=pre)
+        check_fp32(y, 4096, 4096, rowptr, colind, val, x, None, 1.0, 0.0)
+
+
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (1.0, 1.0), (2.0, 0.5), (0.0, 1.0), (-1.0, 1.0), (0.0, 0.0),
+                                        (0.5, -1.0), (1e6, 1.0)])
+@pytest.mark.parametrize("preprocess", [True, False])
+def test_alpha_beta(osa, gpu_ctx, alpha, beta, preprocess):
+    rows, cols = 777, 1234
+    rowptr, colind, val = random_csr(rows, cols, 0.02, seed=11)
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-5, 5, cols).astype(np.float32)
+    y0 = rng.uniform(-5, 5, rows).astype(np.float32)
+    y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, alpha, beta, preprocess=preprocess)
+    check_fp32(y, rows, cols, rowptr, colind, val, x, y0, alpha, beta)
+
+
+SHAPES = [(1, 1, 1.0), (1, 1, 0.0), (4, 4, 0.5), (8, 8, 0.5), (32, 32, 0.9), (1, 100000, 0.3), (100000, 1, 0.5),
+          (1, 100000, 1.0), (1023, 17, 0.3), (17, 1023, 0.3), (2048, 2048, 0.05), (5000, 5000, 0.001),
+          (4096, 4096, 0.01), (300, 300, 0.0), (64, 70000, 0.2)]
+
+
+@pytest.mark.parametrize("rows,cols,density", SHAPES)
+def test_shapes(osa, gpu_ctx, rows, cols, density):
+    rowptr, colind, val = random_csr(rows, cols, density, seed=rows * 31 + cols)
+    rng = np.random.default_rng(rows + cols)
+    x = rng.uniform(-5, 5, cols).astype(np.float32)
+    y0 = rng.uniform(-5, 5, rows).astype(np.float32)
+    for pre in (True, False):
+        y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 1.5, -0.5, preprocess=pre)
+        check_fp32(y, rows, cols, rowptr, colind, val, x, y0, 1.5, -0.5)
+
+
+def test_empty_rows_unsorted_duplicates(osa, gpu_ctx):
+    rows, cols = 3000, 500
+    rowptr, colind, val = random_csr(rows, cols, 0.05, seed=3, empty_row_prob=0.5, unsorted=True, duplicates=True)
+    rng = np.random.default_rng(9)
+    x = rng.uniform(-3, 3, cols).astype(np.float32)
+    y0 = rng.uniform(-3, 3, rows).astype(np.float32)
+    y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 1.0, 1.0)
+    check_fp32(y, rows, cols, rowptr, colind, val, x, y0, 1.0, 1.0)
+
+
+def test_diagonal_closed_form(osa, gpu_ctx):
+    n = 10000
+    rowptr = np.arange(n + 1, dtype=np.int32)
+    colind = np.arange(n, dtype=np.int32)
+    val = np.full(n, 3.0, np.float32)
+    x = np.arange(n, dtype=np.float32)
+    y0 = np.ones(n, np.float32)
+    y = run_spmv(osa, gpu_ctx, n, n, rowptr, colind, val, x, y0, 2.0, -1.0)
+    assert np.array_equal(y, 6.0 * x - 1.0)
+
+
+def test_longer_vectors_untouched(osa, gpu_ctx):
+    """x longer than cols and y longer than rows are accepted; the extra y elements stay as they were."""
+    rows, cols = 100, 80
+    rowptr, colind, val = random_csr(rows, cols, 0.2, seed=1)
+    x = np.random.default_rng(2).uniform(-1, 1, cols + 7).astype(np.float32)
+    y0 = np.random.default_rng(3).uniform(-1, 1, rows + 5).astype(np.float32)
+    y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 1.0, 2.0)
+    check_fp32(y, rows, cols, rowptr, colind, val, x[:cols], y0[:rows], 1.0, 2.0)
+    assert np.array_equal(y[rows:], y0[rows:])
+
+
+FAMILIES = ["STREAM_ROWS", "VECTOR_ROWS", "MERGE_PATH"]
+
+
+@pytest.mark.parametrize("family", FAMILIES)
+@pytest.mark.parametrize("case", ["short", "medium", "skewed", "one_long_row", "many_empty"])
+def test_every_kernel_family(osa, gpu_ctx, family, case):
+    """Each kernel family forced through the raw launch layer on each row-length profile."""
+    rng = np.random.default_rng(FAMILIES.index(family) * 100 + len(case))
+    if case == "short":
+        rows, cols = 20000, 20000
+        lengths = rng.integers(0, 9, rows)
+    elif case == "medium":
+        rows, cols = 3000, 8000
+        lengths = rng.integers(20, 49, rows)
+    elif case == "skewed":
+        rows, cols = 30000, 50000
+        lengths = np.minimum((1.0 / rng.random(rows)).astype(np.int64), 40000)
+        lengths[123] = 40000
+    elif case == "one_long_row":
+        rows, cols = 5, 300000
+        lengths = np.array([3, 0, 250000, 1, 7])
+    else:
+        rows, cols = 50000, 64
+        lengths = np.zeros(rows, np.int64)
+        lengths[::997] = 5
+    if family == "STREAM_ROWS" and lengths.max() > 48:
+        pytest.skip("STREAM_ROWS only takes matrices whose longest row fits its LDS tile")
+    rowptr, colind, val = csr_from_lengths(lengths, cols, seed=7)
+    x = rng.uniform(-1, 1, cols).astype(np.float32)
+    y0 = rng.uniform(-1, 1, rows).astype(np.float32)
+    fam = getattr(osa, "OPSPARSE_SPMV_" + family)
+    y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 1.25, 0.75, force_kernel=fam)
+    check_fp32(y, rows, cols, rowptr, colind, val, x, y0, 1.25, 0.75)
