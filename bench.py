@@ -1,0 +1,213 @@
+#!/usr/bin/env python3
+"""Benchmark of the CSR SpMV / SpMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c1]
+
+A step is one aclsparseSpMV (or aclsparseSpMM) call over one synthetic matrix
+whose arrays are already resident in HBM.  The default workload is c2, the
+5-point 2-D Laplacian on a 2048 x 2048 grid (m = n = 4 194 304, nnz = 20 963 328,
+alpha = 1, beta = 0.5), the configuration the headline metric is quoted on.
+Preprocess runs once before the timed region (its time is reported separately).
+
+Prints ONE JSON line: GFLOP/s = 2 * nnz * ncols / t as `value`, the roofline
+object (algorithmic bytes / kernel time against 8 TB/s HBM) and the CPU baseline
+(the reference's CPU golden loop restated in oracle/, timed on this host).
+"""
+import argparse
+import ctypes
+import importlib
+import importlib.util
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+
+
+def load_package():
+    if "ops_sparse_amd" in sys.modules:
+        return sys.modules["ops_sparse_amd"]
+    pkg_dir = os.path.join(ROOT, "ops-sparse_amd")
+    spec = importlib.util.spec_from_file_location(
+        "ops_sparse_amd", os.path.join(pkg_dir, "__init__.py"), submodule_search_locations=[pkg_dir])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules["ops_sparse_amd"] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def measure_copy_gbps(osa, torch, dev, stream, nbytes=1 << 30, reps=10):
+    """Practical HBM peak: device-to-device copy of >= 1 GiB, (read + write) / t."""
+    src = torch.empty(nbytes, dtype=torch.uint8, device=dev).zero_()
+    dst = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    L = osa.lib()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    torch.cuda.synchronize()
+    for _ in range(2):
+        L.opsparse_copy_launch(src.data_ptr(), dst.data_ptr(), nbytes, sp)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(reps):
+        L.opsparse_copy_launch(src.data_ptr(), dst.data_ptr(), nbytes, sp)
+    e1.record(stream)
+    stream.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    return 2.0 * nbytes / (ms * 1e-3) / 1e9
+
+
+def cpu_baseline_spmv(cfg, budget_s=15.0):
+    """The reference's SpmvCpu loop (oracle.spmv_f32), one thread, on the same matrix."""
+    import oracle
+    A = cfg["A"]
+    rowptr, colind = A["rowptr"].cpu().numpy(), A["colind"].cpu().numpy()
+    val = A["values"].cpu().float().numpy()
+    x, y0 = cfg["x"].cpu().float().numpy(), cfg["y0"].cpu().float().numpy()
+    rows, nnz = A["rows"], int(colind.size)
+    oracle.spmv_f32(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])  # warm
+    reps, t0 = 0, time.perf_counter()
+    while reps < 10 and time.perf_counter() - t0 < budget_s:
+        oracle.spmv_f32(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": 2.0 * nnz / dt / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
+            "sample": "full matrix, %d repeats of the reference's SpmvCpu loop restated in oracle/oracle.c "
+                      "(fp32 accumulate), %.1f ms each" % (reps, dt * 1e3)}
+
+
+def cpu_baseline_spmm(cfg, rows_sample=32768):
+    """The reference's spmm_csr_cpu loop (order i, j, p) on the first rows_sample rows."""
+    import oracle
+    A = cfg["A"]
+    n = cfg["n"]
+    rs = min(rows_sample, A["rows"])
+    rowptr = A["rowptr"][: rs + 1].cpu().numpy()
+    nnz = int(rowptr[-1])
+    colind = A["colind"][:nnz].cpu().numpy()
+    val = A["values"][:nnz].cpu().float().numpy()
+    B = cfg["B"].cpu().float().numpy()
+    import numpy as np
+    C = np.zeros(rs * n, np.float32)
+    t0 = time.perf_counter()
+    oracle.spmm_f32(rs, n, rowptr, colind, val, B.ravel(), n, C, n, cfg["alpha"], cfg["beta"])
+    dt = time.perf_counter() - t0
+    return {"value": 2.0 * nnz * n / dt / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
+            "sample": "first %d of %d rows (%d nnz) against the full B, one run of the reference's "
+                      "SpmmCpuFp32 loop restated in oracle/oracle.c, %.1f s" % (rs, A["rows"], nnz, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-preprocess", action="store_true", help="SpMV without the Preprocess buffer")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    osa = load_package()
+    osa.lib()
+    wl = importlib.import_module("ops_sparse_amd.workloads")
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.Stream(device=dev)
+    handle = osa.Handle(stream)
+
+    t_gen = time.perf_counter()
+    s = args.scale
+    if args.workload == "c2":
+        cfg = wl.config_c2(dev, grid=max(8, int(2048 * s ** 0.5)))
+    elif args.workload == "c3":
+        cfg = wl.config_c3(dev, m=max(1024, int(8388608 * s)), lmax=200000 if s >= 0.05 else 2000)
+    elif args.workload == "c4":
+        cfg = wl.config_c4(dev, m=max(1024, int(1048576 * s)))
+    else:
+        cfg = wl.config_c5(dev, m=max(1024, int(2097152 * s)))
+    torch.cuda.synchronize()
+    A = cfg["A"]
+    rows, cols, nnz = A["rows"], A["cols"], int(A["colind"].numel())
+    log("workload %s: rows=%d nnz=%d (generated in %.1f s)" % (cfg["name"], rows, nnz, time.perf_counter() - t_gen))
+
+    is_spmm = "B" in cfg
+    csr = osa.Csr(rows, cols, A["rowptr"], A["colind"], A["values"])
+    vb = A["values"].element_size()
+    t_pre = time.perf_counter()
+    if not is_spmm:
+        x = cfg["x"]
+        y = cfg["y0"].clone()
+        X, Y = osa.DnVec(x), osa.DnVec(y)
+        op = osa.SpmvOp(handle, csr, X, Y, preprocess=not args.no_preprocess)
+        ncols = 1
+        bytes_alg = wl.spmv_bytes_alg(rows, cols, nnz, vb, x.element_size(), y.element_size(), cfg["beta"] != 0)
+        bytes_gather = wl.spmv_bytes_gather(rows, cols, nnz, vb, x.element_size(), y.element_size(),
+                                            cfg["beta"] != 0)
+        dtype = "f32"
+    else:
+        n = cfg["n"]
+        B = cfg["B"].contiguous()
+        Cmat = torch.zeros(rows, n, dtype=torch.float32, device=dev)
+        Bd = osa.DnMat(cols, n, n, B)
+        Cd = osa.DnMat(rows, n, n, Cmat)
+        op = osa.SpmmOp(handle, csr, Bd, Cd)
+        ncols = n
+        bytes_alg = wl.spmm_bytes_alg(rows, cols, n, nnz, vb, B.element_size(), 4, cfg["beta"] != 0)
+        bytes_gather = wl.spmm_bytes_gather(rows, cols, n, nnz, vb, B.element_size(), 4, cfg["beta"] != 0)
+        dtype = "f32" if vb == 4 else "f16 in, f32 accumulate/out"
+    stream.synchronize()
+    preprocess_ms = (time.perf_counter() - t_pre) * 1e3
+
+    alpha, beta = cfg["alpha"], cfg["beta"]
+    for _ in range(args.warmup):
+        op(alpha, beta)
+    stream.synchronize()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(args.steps):
+        op(alpha, beta)
+    e1.record(stream)
+    stream.synchronize()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ms = e0.elapsed_time(e1) / args.steps  # HIP events on the stream the kernels run on
+
+    flops = 2.0 * nnz * ncols
+    gflops = flops / (ms * 1e-3) / 1e9
+    gbps = bytes_alg / (ms * 1e-3) / 1e9
+    copy_gbps = measure_copy_gbps(osa, torch, dev, stream)
+    log("%.2f us/step (wall %.2f us), %.1f GFLOP/s, %.1f GB/s algorithmic = %.1f%% of 8 TB/s; copy kernel %.0f GB/s"
+        % (ms * 1e3, wall_ms * 1e3, gflops, gbps, 100 * gbps / HBM_PEAK_GBPS, copy_gbps))
+
+    out = {
+        "metric": "SpMV/SpMM GFLOP/s + achieved HBM GB/s (% of MI355X peak), CSR fp32",
+        "value": round(gflops, 2), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": dtype, "data": "synthetic",
+        "config": {"workload": cfg["name"], "rows": rows, "cols": cols, "nnz": nnz, "ncols_dense": ncols,
+                   "alpha": alpha, "beta": beta, "index": "int32", "preprocess_ms": round(preprocess_ms, 3),
+                   "preprocessed": not args.no_preprocess},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "bytes_alg": bytes_alg, "bytes_gather_model": bytes_gather,
+                     "copy_kernel_gbps": round(copy_gbps, 1)},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_spmm(cfg) if is_spmm else cpu_baseline_spmv(cfg)
+    print(json.dumps(out), flush=True)
+    handle.close()
+
+
+if __name__ == "__main__":
+    main()

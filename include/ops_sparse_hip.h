@@ -70,6 +70,9 @@ typedef struct OpsparseSpmvPlan {
     int32_t mergeBlocks;   /* MERGE_PATH: number of workgroups == partition entries - 1 */
     int32_t maxRowNnz;     /* longest row */
     int32_t partitionReady;/* MERGE_PATH: partition table already in the workspace */
+    int32_t waveSlots;     /* STREAM_ROWS: 0 = workgroup-tiled kernel; 8 or 16 = wavefront-tiled kernel for
+                              matrices whose longest row has at most that many non-zeros */
+    int32_t reserved;
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */

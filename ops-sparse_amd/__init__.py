@@ -87,7 +87,7 @@ class OpsparseScalar(ctypes.Structure):
 
 class OpsparseSpmvPlan(ctypes.Structure):
     _fields_ = [("kernel", i32), ("lanesPerRow", i32), ("rowsPerBlock", i32), ("mergeBlocks", i32),
-                ("maxRowNnz", i32), ("partitionReady", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
+                ("maxRowNnz", i32), ("partitionReady", i32), ("waveSlots", i32), ("reserved", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
                 ("carryOff", i64), ("headOff", i64), ("bytes", i64)]
 
 

@@ -23,6 +23,7 @@
 // Memory traffic per launch is the compulsory nnz*(sizeof(val)+4) +
 // (rows+1)*4 + rows*sizeof(y)*(1 + [beta != 0]) plus x: the kernels are
 // HBM-bound streaming kernels, there is no matrix-core work in them.
+#include <cstdlib>
 #include <type_traits>
 
 #include "device_utils.h"
@@ -59,35 +60,6 @@ __device__ __forceinline__ void LoadVals4<double, float>(const float *p, double 
     out[1] = v.y;
     out[2] = v.z;
     out[3] = v.w;
-}
-
-// Products val[k] * x[col[k]] for k in [0, count) of one contiguous nnz range,
-// written to LDS.  Each lane takes 4 consecutive non-zeros per step, so a
-// wavefront reads 1 KiB of indices and 1 KiB of fp32 values per instruction.
-template <typename ValT, typename AccT>
-__device__ __forceinline__ void StageProducts(const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
-                                              const ValT *__restrict__ x, int32_t count, AccT *__restrict__ prod)
-{
-    const int32_t tid = threadIdx.x;
-    for (int32_t k = tid * 4; k < count; k += kBlockThreads * 4) {
-        if (k + 4 <= count) {
-            const Int4U c = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(colInd + k));
-            AccT v[4];
-            LoadVals4<AccT, ValT>(vals + k, v);
-            const AccT x0 = ToAcc<AccT>(x[c.x]);
-            const AccT x1 = ToAcc<AccT>(x[c.y]);
-            const AccT x2 = ToAcc<AccT>(x[c.z]);
-            const AccT x3 = ToAcc<AccT>(x[c.w]);
-            prod[k + 0] = v[0] * x0;
-            prod[k + 1] = v[1] * x1;
-            prod[k + 2] = v[2] * x2;
-            prod[k + 3] = v[3] * x3;
-        } else {
-            for (int32_t q = k; q < count; ++q) {
-                prod[q] = ToAcc<AccT>(LoadStream(vals + q)) * ToAcc<AccT>(x[LoadStream(colInd + q)]);
-            }
-        }
-    }
 }
 
 // ------------------------------------------------------------- y = beta * y
@@ -128,14 +100,205 @@ __global__ __launch_bounds__(kBlockThreads) void RowStatsKernel(const int32_t *_
 
 // ------------------------------------------------------------- STREAM_ROWS
 
-// One workgroup = `rowsPerBlock` consecutive rows; dynamic LDS holds
-// rowsPerBlock * maxRowNnz products.
-template <typename ValT, typename OutT, typename AccT, int G>
+// Four consecutive matrix entries of one lane, still in storage type.
+template <typename ValT>
+struct Quad {
+    Int4U col;
+    ValT val[4];
+};
+
+// Requests the block's entries [k, k + 4) for this lane's U quads.  Nothing is
+// waited for here: the caller does other work while the loads are in flight.
+template <typename ValT, int U>
+__device__ __forceinline__ void IssueQuads(const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+                                           int32_t count, Quad<ValT> (&q)[U])
+{
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int32_t k = (u * kBlockThreads + static_cast<int32_t>(threadIdx.x)) * 4;
+        if (k + 4 <= count) {
+            q[u].col = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(colInd + k));
+            if constexpr (std::is_same<ValT, float>::value) {
+                const Float4U v = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(vals + k));
+                q[u].val[0] = v.x;
+                q[u].val[1] = v.y;
+                q[u].val[2] = v.z;
+                q[u].val[3] = v.w;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    q[u].val[i] = LoadStream(vals + k + i);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {  // the ragged quad at the end of the range, and lanes past it
+                if (k + i < count) {
+                    q[u].col[i] = LoadStream(colInd + k + i);
+                    q[u].val[i] = LoadStream(vals + k + i);
+                }
+            }
+        }
+    }
+}
+
+// Gathers x for the quads requested by IssueQuads and writes the products to LDS.
+template <typename ValT, typename AccT, int U>
+__device__ __forceinline__ void FinishQuads(const Quad<ValT> (&q)[U], const ValT *__restrict__ x, int32_t count,
+                                            AccT *__restrict__ prod)
+{
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int32_t k = (u * kBlockThreads + static_cast<int32_t>(threadIdx.x)) * 4;
+        if (k + 4 <= count) {
+            const AccT x0 = ToAcc<AccT>(x[q[u].col.x]);
+            const AccT x1 = ToAcc<AccT>(x[q[u].col.y]);
+            const AccT x2 = ToAcc<AccT>(x[q[u].col.z]);
+            const AccT x3 = ToAcc<AccT>(x[q[u].col.w]);
+            prod[k + 0] = ToAcc<AccT>(q[u].val[0]) * x0;
+            prod[k + 1] = ToAcc<AccT>(q[u].val[1]) * x1;
+            prod[k + 2] = ToAcc<AccT>(q[u].val[2]) * x2;
+            prod[k + 3] = ToAcc<AccT>(q[u].val[3]) * x3;
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (k + i < count) {
+                    prod[k + i] = ToAcc<AccT>(q[u].val[i]) * ToAcc<AccT>(x[q[u].col[i]]);
+                }
+            }
+        }
+    }
+}
+
+// A workgroup walks over tiles of `rowsPerBlock` consecutive rows (at most
+// 1024 * U non-zeros each).  Per tile: the tile's contiguous (colind, value)
+// range arrives through IssueQuads, the products go to LDS, then G lanes per row
+// add them up in stored order.  The loads of the NEXT tile are issued before the
+// current tile is reduced, so the matrix stream never drains, and the row
+// bounds / old y of a lane's first row are fetched a tile ahead as well.
+// Workgroups of one XCD share one contiguous range of tiles and take them
+// interleaved, so the x lines neighbouring tiles share are fetched into that
+// XCD's L2 once.
+template <typename ValT, typename OutT, typename AccT, int G, int U>
 __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
     const ValT *__restrict__ x, OutT *__restrict__ y, int64_t rows, int32_t rowsPerBlock, OpsparseScalar alphaS,
     OpsparseScalar betaS)
 {
+    extern __shared__ __align__(16) unsigned char ldsRaw[];
+    AccT *prod = reinterpret_cast<AccT *>(ldsRaw);
+
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    const AccT beta = ReadScalar<AccT>(betaS);
+    const bool betaZero = (beta == AccT(0));
+
+    constexpr int kGroups = kBlockThreads / G;
+    const int32_t lane = threadIdx.x % G;
+    const int32_t group = threadIdx.x / G;
+
+    // This XCD's tiles, and this workgroup's stride through them.
+    const int64_t numTiles = (rows + rowsPerBlock - 1) / rowsPerBlock;
+    const int64_t xcd = blockIdx.x % kNumXcd;
+    const int64_t perXcd = numTiles / kNumXcd, rem = numTiles % kNumXcd;
+    const int64_t xcdFirst = xcd * perXcd + (xcd < rem ? xcd : rem);
+    const int64_t xcdTiles = perXcd + (xcd < rem ? 1 : 0);
+    const int64_t stride = (gridDim.x - xcd + kNumXcd - 1) / kNumXcd;  // workgroups living on this XCD
+    int64_t t = blockIdx.x / kNumXcd;
+    if (t >= xcdTiles) {
+        return;
+    }
+
+    int64_t r0 = (xcdFirst + t) * rowsPerBlock;
+    int64_t r1 = (r0 + rowsPerBlock < rows) ? r0 + rowsPerBlock : rows;
+    int32_t first = rowOffsets[r0];
+    int32_t count = rowOffsets[r1] - first;
+    Quad<ValT> q[U];
+    IssueQuads<ValT, U>(colInd + first, vals + first, count, q);
+
+    while (true) {
+        // Row bounds and old y for this lane's first row of the current tile.
+        int64_t r = r0 + group;
+        int32_t s = 0, e = 0;
+        AccT yOld = AccT(0);
+        if (r < r1) {
+            s = rowOffsets[r];
+            e = rowOffsets[r + 1];
+            if (!betaZero && lane == 0) {
+                yOld = ToAcc<AccT>(y[r]);
+            }
+        }
+        // Bounds of the next tile (scalar loads, needed after the barrier).
+        const int64_t tNext = t + stride;
+        const bool more = tNext < xcdTiles;
+        int64_t r0Next = 0, r1Next = 0;
+        int32_t firstNext = 0, countNext = 0;
+        if (more) {
+            r0Next = (xcdFirst + tNext) * rowsPerBlock;
+            r1Next = (r0Next + rowsPerBlock < rows) ? r0Next + rowsPerBlock : rows;
+            firstNext = rowOffsets[r0Next];
+            countNext = rowOffsets[r1Next] - firstNext;
+        }
+
+        FinishQuads<ValT, AccT, U>(q, x, count, prod);
+        __syncthreads();
+        if (more) {
+            IssueQuads<ValT, U>(colInd + firstNext, vals + firstNext, countNext, q);
+        }
+
+        while (r < r1) {
+            const int64_t rNext = r + kGroups;
+            int32_t sNext = 0, eNext = 0;
+            AccT yNext = AccT(0);
+            if (rNext < r1) {
+                sNext = rowOffsets[rNext];
+                eNext = rowOffsets[rNext + 1];
+                if (!betaZero && lane == 0) {
+                    yNext = ToAcc<AccT>(y[rNext]);
+                }
+            }
+            AccT sum = AccT(0);
+            for (int32_t k = s - first + lane; k < e - first; k += G) {
+                sum += prod[k];
+            }
+            sum = GroupSum<G>(sum);
+            if (lane == 0) {
+                AccT res = alpha * sum;
+                if (!betaZero) {
+                    res += beta * yOld;
+                }
+                y[r] = FromAcc<OutT>(res);
+            }
+            r = rNext;
+            s = sNext;
+            e = eNext;
+            yOld = yNext;
+        }
+        if (!more) {
+            break;
+        }
+        __syncthreads();  // everyone is done reading prod before the next tile overwrites it
+        t = tNext;
+        r0 = r0Next;
+        r1 = r1Next;
+        first = firstNext;
+        count = countNext;
+    }
+}
+
+// STREAM_ROWS for the shortest rows (one lane per row would do) with fp32 y:
+// every lane owns FOUR consecutive rows, so the row offsets and y travel as
+// 16-byte vectors (one dwordx4 per lane instead of four dword instructions per
+// 64 rows; the memory pipeline of a CU handles far fewer instructions for the
+// same bytes).  One tile per workgroup; rowsPerBlock is a multiple of 4 and at
+// most 1024, rowOffsets and y are 16-byte aligned.
+template <typename ValT, typename AccT, int U>
+__global__ __launch_bounds__(kBlockThreads) void SpmvStreamQuadRowsKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ x, float *__restrict__ y, int64_t rows, int32_t rowsPerBlock, OpsparseScalar alphaS,
+    OpsparseScalar betaS)
+{
+    typedef int32_t Int4A __attribute__((ext_vector_type(4)));
+    typedef float Float4A __attribute__((ext_vector_type(4)));
     extern __shared__ __align__(16) unsigned char ldsRaw[];
     AccT *prod = reinterpret_cast<AccT *>(ldsRaw);
 
@@ -149,32 +312,67 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
     const int32_t first = rowOffsets[r0];
     const int32_t count = rowOffsets[r1] - first;
 
-    // Issue this lane's first row bounds before the long-latency streaming phase.
-    constexpr int kGroups = kBlockThreads / G;
-    const int32_t lane = threadIdx.x % G;
-    int64_t r = r0 + threadIdx.x / G;
-    int32_t s = 0, e = 0;
-    if (r < r1) {
-        s = rowOffsets[r];
-        e = rowOffsets[r + 1];
+    // Offsets of this lane's rows r .. r+3 (bound[i] .. bound[i+1]) and their old y.
+    const int64_t r = r0 + 4 * static_cast<int64_t>(threadIdx.x);
+    const int32_t mine = r >= r1 ? 0 : (r + 4 <= r1 ? 4 : static_cast<int32_t>(r1 - r));
+    int32_t bound[5] = {0, 0, 0, 0, 0};
+    float yOld[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (mine == 4) {
+        const Int4A b = *reinterpret_cast<const Int4A *>(rowOffsets + r);
+        bound[0] = b.x;
+        bound[1] = b.y;
+        bound[2] = b.z;
+        bound[3] = b.w;
+        bound[4] = rowOffsets[r + 4];
+        if (!betaZero) {
+            const Float4A o = *reinterpret_cast<const Float4A *>(y + r);
+            yOld[0] = o.x;
+            yOld[1] = o.y;
+            yOld[2] = o.z;
+            yOld[3] = o.w;
+        }
+    } else {
+        for (int32_t i = 0; i < mine; ++i) {
+            bound[i] = rowOffsets[r + i];
+            bound[i + 1] = rowOffsets[r + i + 1];
+            if (!betaZero) {
+                yOld[i] = y[r + i];
+            }
+        }
     }
 
-    StageProducts<ValT, AccT>(colInd + first, vals + first, x, count, prod);
+    {
+        Quad<ValT> q[U];
+        IssueQuads<ValT, U>(colInd + first, vals + first, count, q);
+        FinishQuads<ValT, AccT, U>(q, x, count, prod);
+    }
     __syncthreads();
 
-    while (r < r1) {
+    float out[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
         AccT sum = AccT(0);
-        for (int32_t k = s - first + lane; k < e - first; k += G) {
-            sum += prod[k];
+        if (i < mine) {
+            for (int32_t k = bound[i] - first; k < bound[i + 1] - first; ++k) {
+                sum += prod[k];
+            }
         }
-        sum = GroupSum<G>(sum);
-        if (lane == 0) {
-            StoreRow<OutT, AccT>(y, r, sum, alpha, beta, betaZero);
+        AccT res = alpha * sum;
+        if (!betaZero) {
+            res += beta * static_cast<AccT>(yOld[i]);
         }
-        r += kGroups;
-        if (r < r1) {
-            s = rowOffsets[r];
-            e = rowOffsets[r + 1];
+        out[i] = static_cast<float>(res);
+    }
+    if (mine == 4) {
+        Float4A o;
+        o.x = out[0];
+        o.y = out[1];
+        o.z = out[2];
+        o.w = out[3];
+        *reinterpret_cast<Float4A *>(y + r) = o;
+    } else {
+        for (int32_t i = 0; i < mine; ++i) {
+            y[r + i] = out[i];
         }
     }
 }
@@ -280,7 +478,11 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvMergeKernel(
     const int64_t j1 = MergeDiagonal(b + 1, rows, nnz) - i1;
     const int32_t count = static_cast<int32_t>(j1 - j0);
 
-    StageProducts<ValT, AccT>(colInd + j0, vals + j0, x, count, prod);
+    {
+        Quad<ValT> q[2];  // 2 x 1024 entries cover the whole workgroup share
+        IssueQuads<ValT, 2>(colInd + j0, vals + j0, count, q);
+        FinishQuads<ValT, AccT, 2>(q, x, count, prod);
+    }
     __syncthreads();
 
     // Rows i0 .. i1-1 complete here; row i1 (if it exists) collects the tail.
@@ -417,6 +619,34 @@ inline int CheckLaunch()
     return hipGetLastError() == hipSuccess ? OPSPARSE_OK : OPSPARSE_E_LAUNCH;
 }
 
+// Number of compute units of the current device (256 on MI355X), read once.
+inline int ComputeUnits()
+{
+    static const int cus = [] {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess ||
+            prop.multiProcessorCount <= 0) {
+            (void)hipGetLastError();
+            return 256;
+        }
+        return prop.multiProcessorCount;
+    }();
+    return cus;
+}
+
+// Workgroups per CU of the persistent STREAM_ROWS launch (tuning override:
+// OPS_SPARSE_STREAM_BLOCKS_PER_CU).
+inline int StreamBlocksPerCu()
+{
+    static const int n = [] {
+        const char *env = std::getenv("OPS_SPARSE_STREAM_BLOCKS_PER_CU");
+        const int v = env != nullptr ? std::atoi(env) : 0;
+        return (v >= 1 && v <= 64) ? v : 8;
+    }();
+    return n;
+}
+
 inline uint32_t GridFor(int64_t items, int64_t perBlock)
 {
     return static_cast<uint32_t>((items + perBlock - 1) / perBlock);
@@ -441,15 +671,51 @@ MergeLayout MakeMergeLayout(int64_t rows, int64_t nnz)
     return l;
 }
 
-template <typename ValT, typename OutT, typename AccT, int G>
-int LaunchStream(const SpmvArgs &a, int32_t rowsPerBlock, int32_t maxRowNnz)
+template <typename ValT, typename OutT, typename AccT, int G, int U>
+int LaunchStreamU(const SpmvArgs &a, int32_t rowsPerBlock, size_t lds)
 {
-    const size_t lds = static_cast<size_t>(rowsPerBlock) * static_cast<size_t>(maxRowNnz) * sizeof(AccT);
-    const uint32_t grid = GridFor(a.rows, rowsPerBlock);
-    hipLaunchKernelGGL((SpmvStreamRowsKernel<ValT, OutT, AccT, G>), dim3(grid), dim3(kBlockThreads), lds, a.stream,
+    // Persistent launch: a few workgroups per CU walk over all tiles.
+    const uint32_t tiles = GridFor(a.rows, rowsPerBlock);
+    const uint32_t resident = static_cast<uint32_t>(ComputeUnits() * StreamBlocksPerCu());
+    const uint32_t grid = tiles < resident ? tiles : resident;
+    hipLaunchKernelGGL((SpmvStreamRowsKernel<ValT, OutT, AccT, G, U>), dim3(grid), dim3(kBlockThreads), lds, a.stream,
                        a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
                        static_cast<OutT *>(a.y), a.rows, rowsPerBlock, a.alpha, a.beta);
     return CheckLaunch();
+}
+
+template <typename ValT, typename OutT, typename AccT, int G>
+int LaunchStream(const SpmvArgs &a, int32_t rowsPerBlock, int32_t maxRowNnz)
+{
+    // LDS for the worst case of this block shape; the issue depth U covers it in one round.
+    const size_t products = static_cast<size_t>(rowsPerBlock) * static_cast<size_t>(maxRowNnz);
+    const size_t lds = products * sizeof(AccT);
+    if constexpr (G == 1 && std::is_same<OutT, float>::value) {
+        // Four rows per lane with vector row offsets / y where the shapes allow it.
+        static const bool quadOff = std::getenv("OPS_SPARSE_STREAM_NO_QUAD_ROWS") != nullptr;
+        if (!quadOff && rowsPerBlock % 4 == 0 && rowsPerBlock <= 4 * kBlockThreads &&
+            reinterpret_cast<uintptr_t>(a.rowOffsets) % 16 == 0 && reinterpret_cast<uintptr_t>(a.y) % 16 == 0) {
+            const uint32_t grid = GridFor(a.rows, rowsPerBlock);
+            auto launch = [&](auto tag) {
+                constexpr int U = decltype(tag)::value;
+                hipLaunchKernelGGL((SpmvStreamQuadRowsKernel<ValT, AccT, U>), dim3(grid), dim3(kBlockThreads), lds,
+                                   a.stream, a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
+                                   static_cast<const ValT *>(a.x), static_cast<float *>(a.y), a.rows, rowsPerBlock,
+                                   a.alpha, a.beta);
+            };
+            if (products <= kBlockThreads * 4) {
+                launch(std::integral_constant<int, 1>{});
+            } else if (products <= kBlockThreads * 8) {
+                launch(std::integral_constant<int, 2>{});
+            } else {
+                launch(std::integral_constant<int, 3>{});
+            }
+            return CheckLaunch();
+        }
+    }
+    if (products <= kBlockThreads * 4) return LaunchStreamU<ValT, OutT, AccT, G, 1>(a, rowsPerBlock, lds);
+    if (products <= kBlockThreads * 8) return LaunchStreamU<ValT, OutT, AccT, G, 2>(a, rowsPerBlock, lds);
+    return LaunchStreamU<ValT, OutT, AccT, G, 3>(a, rowsPerBlock, lds);
 }
 
 template <typename ValT, typename OutT, typename AccT, int G>
@@ -677,8 +943,19 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
             }
             const int32_t g = maxRow <= 12 ? 1 : (maxRow <= 24 ? 2 : 4);
             p.lanesPerRow = g;
-            // One pass of the 256 / g lane groups over the block's rows.
-            p.rowsPerBlock = kBlockThreads / g;
+            // As many rows as keep the tile's worst-case products within two full
+            // rounds of the workgroup's loads (2 x 1024 entries, 16 KiB of LDS):
+            // measured best when a tile nearly fills whole rounds.
+            int32_t rpb = 2048 / maxRow;
+            rpb = rpb > 512 ? 512 : rpb;
+            rpb &= ~3;  // whole groups of four rows for the vectorised y path
+            p.rowsPerBlock = rpb < 4 ? 4 : rpb;
+            if (const char *env = std::getenv("OPS_SPARSE_STREAM_ROWS")) {
+                const int v = std::atoi(env);  // tuning override
+                if (v >= 1 && static_cast<int64_t>(v) * maxRow <= 3072) {
+                    p.rowsPerBlock = v;
+                }
+            }
             break;
         }
         case OPSPARSE_SPMV_VECTOR_ROWS:

@@ -27,7 +27,9 @@ def check_fp32(y, rows, cols, rowptr, colind, val, x, y0, alpha, beta):
                           alpha, beta)
     d = np.abs(y[:rows] - g32)
     ok = d <= 2.0 ** -16 + 2.0 ** -10 * np.abs(g32)
-    assert rows == 0 or abs(alpha) > 100 or (ok.mean() >= 0.99 and d.max() <= 1e-2)
+    # (that golden accumulates in fp32: on very long rows or huge alpha its own error exceeds the 1e-2 cap)
+    longest = int(np.diff(rowptr).max()) if rows else 0
+    assert rows == 0 or abs(alpha) > 100 or longest > 2048 or (ok.mean() >= 0.99 and d.max() <= 1e-2)
     mere, mare, mism, _ = oracle.mere_mare(y[:rows], gold)
     assert mism == 0 and mere < 1e-6 and mare < 5e-6
 
