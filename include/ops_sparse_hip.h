@@ -130,12 +130,21 @@ typedef struct OpsparseSpmmPlan {
     int64_t segStartOff;   /* int32 [numSegments]: first nnz of the segment */
     int64_t longFirstSegOff; /* int32 [numLongRows + 1]: first segment of each long row */
     int64_t partialOff;    /* double [numSegments * n] */
+    int64_t rowOrderOff;   /* int32 [numOrdered]: the rows ROW_SPLIT takes, longest first, so that the lane
+                              groups of a wavefront work on rows of similar length; 0 = natural order */
+    int64_t numOrdered;
     int64_t bytes;
 } OpsparseSpmmPlan;
 
-size_t opsparse_spmm_csr_workspace_bytes(int64_t rows, int64_t nnz, int64_t n);
+/* Exact workspace size for this matrix and n.  256 bytes when no row is long;
+ * otherwise a device reduction over the row offsets counts the long rows and
+ * their segments (allocates and frees a 256-byte device scratch, synchronises
+ * `stream`). */
+int opsparse_spmm_csr_workspace_bytes(const int32_t *rowOffsets, int64_t rows, int64_t nnz, int64_t n, void *stream,
+                                      size_t *bytes);
 
-/* Synchronises `stream` once (row statistics are read back). */
+/* Row statistics and, for BINNED, the long-row / segment tables (built on the
+ * host from a copy of the row offsets).  Synchronises `stream`. */
 int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t nnz, int64_t n, void *workspace,
                               size_t workspaceBytes, int32_t forceKernel, OpsparseSpmmPlan *plan, void *stream);
 

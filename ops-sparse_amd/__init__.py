@@ -95,7 +95,7 @@ class OpsparseSpmmPlan(ctypes.Structure):
     _fields_ = [("kernel", i32), ("maxRowNnz", i32), ("longRowNnz", i32), ("numLongRows", i32),
                 ("numSegments", i32), ("segmentNnz", i32), ("rows", i64), ("nnz", i64), ("n", i64),
                 ("longRowsOff", i64), ("segRowOff", i64), ("segStartOff", i64), ("longFirstSegOff", i64),
-                ("partialOff", i64), ("bytes", i64)]
+                ("partialOff", i64), ("rowOrderOff", i64), ("numOrdered", i64), ("bytes", i64)]
 
 
 _lib = None
@@ -167,8 +167,8 @@ def lib():
     L.opsparse_spmv_csr_launch.restype = ctypes.c_int
     L.opsparse_spmv_csr_launch.argtypes = [ctypes.POINTER(OpsparseSpmvPlan), i32, vp, vp, vp, vp, vp, i64, i64, i64,
                                            OpsparseScalar, OpsparseScalar, i32, i32, i32, vp, sz, vp]
-    L.opsparse_spmm_csr_workspace_bytes.restype = sz
-    L.opsparse_spmm_csr_workspace_bytes.argtypes = [i64, i64, i64]
+    L.opsparse_spmm_csr_workspace_bytes.restype = ctypes.c_int
+    L.opsparse_spmm_csr_workspace_bytes.argtypes = [vp, i64, i64, i64, vp, ctypes.POINTER(sz)]
     L.opsparse_spmm_csr_analyse.restype = ctypes.c_int
     L.opsparse_spmm_csr_analyse.argtypes = [vp, i64, i64, i64, vp, sz, i32, ctypes.POINTER(OpsparseSpmmPlan), vp]
     L.opsparse_spmm_csr_launch.restype = ctypes.c_int

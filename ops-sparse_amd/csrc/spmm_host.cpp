@@ -105,8 +105,13 @@ aclsparseStatus_t BuildPlan(const aclsparseSpMatDescr *A, const aclsparseDnMatDe
         return ACL_SPARSE_STATUS_INVALID_VALUE;
     }
     OpsparseSpmmPlan plan{};
-    const size_t bytes = opsparse_spmm_csr_workspace_bytes(A->rows, A->nnz, C->cols);
-    const int rc = opsparse_spmm_csr_analyse(static_cast<const int32_t *>(A->rowOffsets), A->rows, A->nnz, C->cols,
+    size_t bytes = 0;
+    int rc = opsparse_spmm_csr_workspace_bytes(static_cast<const int32_t *>(A->rowOffsets), A->rows, A->nnz, C->cols,
+                                               stream, &bytes);
+    if (rc != OPSPARSE_OK) {
+        return FromLaunch(rc);
+    }
+    rc = opsparse_spmm_csr_analyse(static_cast<const int32_t *>(A->rowOffsets), A->rows, A->nnz, C->cols,
                                              buffer, bytes, OPSPARSE_SPMM_AUTO, &plan, stream);
     if (rc != OPSPARSE_OK) {
         opsparse::LogError("aclsparseSpMM: analysis failed (%d)", rc);
@@ -121,7 +126,7 @@ aclsparseStatus_t BuildPlan(const aclsparseSpMatDescr *A, const aclsparseDnMatDe
 
 extern "C" {
 
-aclsparseStatus_t aclsparseSpMMGetBufferSize(aclsparseHandle_t /*handle*/, aclsparseOperation_t opA,
+aclsparseStatus_t aclsparseSpMMGetBufferSize(aclsparseHandle_t handle, aclsparseOperation_t opA,
                                              aclsparseOperation_t opB, const void * /*alpha*/,
                                              aclsparseConstSpMatDescr_t matA, aclsparseConstDnMatDescr_t matB,
                                              const void * /*beta*/, aclsparseDnMatDescr_t matC,
@@ -135,8 +140,15 @@ aclsparseStatus_t aclsparseSpMMGetBufferSize(aclsparseHandle_t /*handle*/, aclsp
     if (st != ACL_SPARSE_STATUS_SUCCESS) {
         return st;
     }
-    *size = opsparse_spmm_csr_workspace_bytes(matA->rows, matA->nnz, matC->cols);
-    return ACL_SPARSE_STATUS_SUCCESS;
+    // Matrices in which no row can be long need the 256-byte header only (no
+    // device access); otherwise the long rows are counted on the device.
+    if (matA->rows > 0 && matA->rowOffsets == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    const int rc = opsparse_spmm_csr_workspace_bytes(static_cast<const int32_t *>(matA->rowOffsets), matA->rows,
+                                                     matA->nnz, matC->cols,
+                                                     handle != nullptr ? handle->stream : nullptr, size);
+    return FromLaunch(rc);
 }
 
 aclsparseStatus_t aclsparseSpMMPreprocess(aclsparseHandle_t handle, aclsparseOperation_t opA,

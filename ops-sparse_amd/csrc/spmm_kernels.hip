@@ -11,14 +11,31 @@
 // The (colind, value) pairs of a row are loaded L at a time, one pair per
 // lane, non-temporally, and handed round the group with cross-lane shuffles.
 //
+// Row-length binning (the counterpart of the reference's greedy row bin
+// packing, sparse/spmm/arch35/spmm_csr_mat.cpp:28-66): rows of up to
+// kLongRowNnz entries are taken whole by one lane group (ROW_SPLIT).  Longer
+// rows — the tail of a power-law graph — are cut into segments of kSegmentNnz
+// entries, every segment is accumulated by its own lane group into an fp64
+// partial row in the workspace, and a fix-up kernel adds a row's partials in
+// segment order and applies alpha / beta, so the result does not depend on
+// scheduling.
+//
 // Floating-point products are accumulated in fp64 in stored order and rounded
 // once, int8 products in int32 with an int64 saturating epilogue
 // (spmm_kernel.cpp:251-266).
+#include <climits>
 #include <type_traits>
+#include <vector>
 
 #include "device_utils.h"
 
 namespace opsparse {
+
+constexpr int32_t kLongRowNnz = 256;  // rows longer than this are cut into segments
+constexpr int32_t kSegmentNnz = 128;  // entries per segment
+// Rows a lane group of the row-split kernel takes one after the other, so that a
+// workgroup lives long enough to amortise its start-up.
+constexpr int kSpmmRowsPerGroup = 4;
 
 // Index of element (r, c) of a dense matrix with leading dimension ld.
 __device__ __forceinline__ int64_t DenseIndex(int64_t r, int64_t c, int64_t ld, bool colMajor)
@@ -64,16 +81,111 @@ struct Epilogue<int32_t, int32_t> {
 // B row-major, op(B) = B, C row-major, n and both leading dimensions multiples
 // of V, B and C 16-byte aligned.
 
+// This lane's share of the first L entries of [s, e): entry s + lane, or (0, 0).
+template <typename ValT, typename AccT>
+__device__ __forceinline__ void LoadFirstChunk(const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+                                               int32_t lane, int32_t s, int32_t e, int32_t *firstCol, float *firstVal)
+{
+    *firstCol = 0;
+    *firstVal = 0.0f;
+    if (s + lane < e) {
+        *firstCol = LoadStream(colInd + s + lane);
+        *firstVal = static_cast<float>(ToAcc<AccT>(LoadStream(vals + s + lane)));
+    }
+}
+
+// acc[i] += sum over entries p in [s, e) of val[p] * B[colind[p], col + i], in
+// stored order.  Called by all L lanes of a group with the same (s, e);
+// (firstCol, firstVal) is the lane's LoadFirstChunk result for this range.
+template <typename ValT, typename AccT, int V, int L>
+__device__ __forceinline__ void AccumulateEntries(const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+                                                  const ValT *__restrict__ B, int64_t ldb, int32_t col, bool active,
+                                                  int32_t lane, int32_t s, int32_t e, int32_t firstCol,
+                                                  float firstVal, AccT (&acc)[V])
+{
+    typedef ValT BVec __attribute__((ext_vector_type(V)));
+    // Gathers issued back to back, U * 16 bytes in flight per lane.  Eight for the
+    // 8-element (fp16) vectors: their fp64 conversion needs the registers, and more
+    // resident wavefronts hide more latency than a deeper batch.
+    constexpr int UMAX = V >= 8 ? 8 : 16;
+    constexpr int U = L < UMAX ? L : UMAX;
+    constexpr int US = U < 8 ? U : 8;   // predicated batch size for the short tail of a row
+    for (int32_t p0 = s; p0 < e; p0 += L) {
+        // The first L entries come preloaded from the caller (firstCol / firstVal).
+        int32_t myCol = firstCol;
+        float myVal = firstVal;
+        if (p0 != s) {
+            myCol = 0;
+            myVal = 0.0f;
+            if (p0 + lane < e) {
+                myCol = LoadStream(colInd + p0 + lane);
+                myVal = static_cast<float>(ToAcc<AccT>(LoadStream(vals + p0 + lane)));
+            }
+        }
+        const int32_t cnt = (e - p0 < L) ? e - p0 : L;
+        int32_t q0 = 0;
+        // Full batches of U entries.
+        for (; q0 + U <= cnt; q0 += U) {
+            BVec b[U];
+            float v[U];
+#pragma unroll
+            for (int q = 0; q < U; ++q) {
+                const int32_t c = __shfl(myCol, q0 + q, L);
+                v[q] = __shfl(myVal, q0 + q, L);
+                if (active) {
+                    b[q] = *reinterpret_cast<const BVec *>(B + static_cast<int64_t>(c) * ldb + col);
+                }
+            }
+            if (active) {
+#pragma unroll
+                for (int q = 0; q < U; ++q) {
+                    const AccT vq = static_cast<AccT>(v[q]);
+#pragma unroll
+                    for (int i = 0; i < V; ++i) {
+                        acc[i] += vq * ToAcc<AccT>(b[q][i]);
+                    }
+                }
+            }
+        }
+        // Remaining entries in predicated batches of US; a missing entry adds nothing.
+        for (; q0 < cnt; q0 += US) {
+            BVec b[US];
+            float v[US];
+#pragma unroll
+            for (int q = 0; q < US; ++q) {
+                const bool valid = q0 + q < cnt;
+                const int32_t c = __shfl(myCol, (q0 + q) % L, L);
+                v[q] = __shfl(myVal, (q0 + q) % L, L);
+                if (active && valid) {
+                    b[q] = *reinterpret_cast<const BVec *>(B + static_cast<int64_t>(c) * ldb + col);
+                }
+            }
+            if (active) {
+#pragma unroll
+                for (int q = 0; q < US; ++q) {
+                    if (q0 + q < cnt) {
+                        const AccT vq = static_cast<AccT>(v[q]);
+#pragma unroll
+                        for (int i = 0; i < V; ++i) {
+                            acc[i] += vq * ToAcc<AccT>(b[q][i]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Rows of at most longRowNnz entries, one lane group per row.
 template <typename ValT, typename CT, typename AccT, int V, int L>
 __global__ __launch_bounds__(kBlockThreads) void SpmmRowSplitKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
     const ValT *__restrict__ B, CT *__restrict__ C, int64_t rows, int32_t n, int64_t ldb, int64_t ldc,
-    int32_t rowsPerGroup, OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16)
+    int32_t longRowNnz, const int32_t *__restrict__ rowOrder, OpsparseScalar alphaS, OpsparseScalar betaS,
+    int32_t clampF16)
 {
-    typedef ValT BVec __attribute__((ext_vector_type(V)));
     typedef CT CVec __attribute__((ext_vector_type(V), aligned(16)));
     constexpr int kGroups = kBlockThreads / L;
-    constexpr int U = L < 16 ? L : 16;
 
     const AccT alpha = ReadScalar<AccT>(alphaS);
     const AccT beta = ReadScalar<AccT>(betaS);
@@ -82,15 +194,41 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmRowSplitKernel(
     const int32_t lane = threadIdx.x % L;
     const int32_t group = threadIdx.x / L;
     const int64_t tile = XcdContiguousTile(blockIdx.x, gridDim.x);
-    const int64_t rowBase = tile * (static_cast<int64_t>(kGroups) * rowsPerGroup);
+    const int64_t rowBase = tile * (static_cast<int64_t>(kGroups) * kSpmmRowsPerGroup);
 
-    for (int32_t it = 0; it < rowsPerGroup; ++it) {
-        const int64_t r = rowBase + static_cast<int64_t>(it) * kGroups + group;
-        if (r >= rows) {
-            break;
+    // Row ids, bounds and first entries of all of this group's rows are requested
+    // up front, one dependent step per kind for all rows together, instead of a
+    // chain of four dependent loads in front of every single row.
+    int64_t rowId[kSpmmRowsPerGroup];
+    int32_t rowS[kSpmmRowsPerGroup], rowE[kSpmmRowsPerGroup], fCol[kSpmmRowsPerGroup];
+    float fVal[kSpmmRowsPerGroup];
+#pragma unroll
+    for (int it = 0; it < kSpmmRowsPerGroup; ++it) {
+        const int64_t slot = rowBase + static_cast<int64_t>(it) * kGroups + group;
+        // `rows` counts the slots: all rows, or the entries of rowOrder
+        rowId[it] = slot >= rows ? -1 : (rowOrder != nullptr ? static_cast<int64_t>(rowOrder[slot]) : slot);
+    }
+#pragma unroll
+    for (int it = 0; it < kSpmmRowsPerGroup; ++it) {
+        rowS[it] = rowE[it] = 0;
+        if (rowId[it] >= 0) {
+            rowS[it] = rowOffsets[rowId[it]];
+            rowE[it] = rowOffsets[rowId[it] + 1];
         }
-        const int32_t s = rowOffsets[r];
-        const int32_t e = rowOffsets[r + 1];
+    }
+#pragma unroll
+    for (int it = 0; it < kSpmmRowsPerGroup; ++it) {
+        LoadFirstChunk<ValT, AccT>(colInd, vals, lane, rowS[it], rowE[it], &fCol[it], &fVal[it]);
+    }
+
+#pragma unroll
+    for (int it = 0; it < kSpmmRowsPerGroup; ++it) {
+        const int64_t r = rowId[it];
+        const int32_t s = rowS[it];
+        const int32_t e = rowE[it];
+        if (r < 0 || e - s > longRowNnz) {
+            continue;  // past the end, or a long row: segment kernel + fix-up write it
+        }
         for (int32_t c0 = 0; c0 < n; c0 += L * V) {
             const int32_t col = c0 + lane * V;
             const bool active = col < n;
@@ -99,54 +237,8 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmRowSplitKernel(
             for (int i = 0; i < V; ++i) {
                 acc[i] = AccT(0);
             }
-            for (int32_t p0 = s; p0 < e; p0 += L) {
-                int32_t myCol = 0;
-                float myVal = 0.0f;
-                if (p0 + lane < e) {
-                    myCol = LoadStream(colInd + p0 + lane);
-                    myVal = static_cast<float>(ToAcc<AccT>(LoadStream(vals + p0 + lane)));
-                }
-                const int32_t cnt = (e - p0 < L) ? e - p0 : L;
-                if (cnt == L) {
-                    // Full chunk: U gathers are issued back to back before their
-                    // products are consumed, U * 16 bytes in flight per lane.
-#pragma unroll
-                    for (int q0 = 0; q0 < L; q0 += U) {
-                        BVec b[U];
-                        float v[U];
-#pragma unroll
-                        for (int q = 0; q < U; ++q) {
-                            const int32_t c = __shfl(myCol, q0 + q, L);
-                            v[q] = __shfl(myVal, q0 + q, L);
-                            if (active) {
-                                b[q] = *reinterpret_cast<const BVec *>(B + static_cast<int64_t>(c) * ldb + col);
-                            }
-                        }
-                        if (active) {
-#pragma unroll
-                            for (int q = 0; q < U; ++q) {
-                                const AccT vq = static_cast<AccT>(v[q]);
-#pragma unroll
-                                for (int i = 0; i < V; ++i) {
-                                    acc[i] += vq * ToAcc<AccT>(b[q][i]);
-                                }
-                            }
-                        }
-                    }
-                } else {
-                    for (int32_t q = 0; q < cnt; ++q) {
-                        const int32_t c = __shfl(myCol, q, L);
-                        const AccT vq = static_cast<AccT>(__shfl(myVal, q, L));
-                        if (active) {
-                            const BVec b = *reinterpret_cast<const BVec *>(B + static_cast<int64_t>(c) * ldb + col);
-#pragma unroll
-                            for (int i = 0; i < V; ++i) {
-                                acc[i] += vq * ToAcc<AccT>(b[i]);
-                            }
-                        }
-                    }
-                }
-            }
+            AccumulateEntries<ValT, AccT, V, L>(colInd, vals, B, ldb, col, active, lane, s, e, fCol[it], fVal[it],
+                                                acc);
             if (active) {
                 CT *out = C + r * ldc + col;
                 CVec res;
@@ -166,6 +258,105 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmRowSplitKernel(
                 *reinterpret_cast<CVec *>(out) = res;
             }
         }
+    }
+}
+
+// One lane group per segment of a long row: partial[seg][0..n) = sum over the
+// segment's entries, in fp64.
+template <typename ValT, typename AccT, int V, int L>
+__global__ __launch_bounds__(kBlockThreads) void SpmmLongSegmentKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ B, int32_t n, int64_t ldb, int32_t numSegments, const int32_t *__restrict__ segRow,
+    const int32_t *__restrict__ segStart, AccT *__restrict__ partial)
+{
+    constexpr int kGroups = kBlockThreads / L;
+    const int32_t lane = threadIdx.x % L;
+    const int64_t seg = static_cast<int64_t>(blockIdx.x) * kGroups + threadIdx.x / L;
+    if (seg >= numSegments) {
+        return;
+    }
+    const int32_t row = segRow[seg];
+    const int32_t s = segStart[seg];
+    const int32_t rowEnd = rowOffsets[row + 1];
+    const int32_t e = (rowEnd - s > kSegmentNnz) ? s + kSegmentNnz : rowEnd;
+    int32_t firstCol;
+    float firstVal;
+    LoadFirstChunk<ValT, AccT>(colInd, vals, lane, s, e, &firstCol, &firstVal);
+    for (int32_t c0 = 0; c0 < n; c0 += L * V) {
+        const int32_t col = c0 + lane * V;
+        const bool active = col < n;
+        AccT acc[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            acc[i] = AccT(0);
+        }
+        AccumulateEntries<ValT, AccT, V, L>(colInd, vals, B, ldb, col, active, lane, s, e, firstCol, firstVal, acc);
+        if (active) {
+            AccT *out = partial + seg * n + col;
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                out[i] = acc[i];
+            }
+        }
+    }
+}
+
+// One workgroup per long row.  Each of its four wavefronts adds a contiguous
+// quarter of the row's partials in segment order (lane = output column), the four
+// sums are combined in wavefront order through LDS, then alpha / beta are applied.
+// The association order is fixed by the segment table alone, so the result is
+// the same on every run.
+template <typename CT, typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmmLongFixupKernel(
+    CT *__restrict__ C, int32_t n, int64_t ldc, int32_t numLongRows, const int32_t *__restrict__ longRows,
+    const int32_t *__restrict__ longFirstSeg, const AccT *__restrict__ partial, OpsparseScalar alphaS,
+    OpsparseScalar betaS, int32_t clampF16)
+{
+    constexpr int kWaves = kBlockThreads / kWave;
+    __shared__ AccT part[kWaves][kWave];
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    const AccT beta = ReadScalar<AccT>(betaS);
+    const bool betaZero = (beta == AccT(0));
+    const int32_t lane = threadIdx.x % kWave;
+    const int32_t wave = threadIdx.x / kWave;
+    const int64_t j = blockIdx.x;
+    const int64_t row = longRows[j];
+    const int64_t seg0 = longFirstSeg[j];
+    const int64_t seg1 = longFirstSeg[j + 1];
+    const int64_t per = (seg1 - seg0 + kWaves - 1) / kWaves;
+    const int64_t mine0 = seg0 + wave * per;
+    const int64_t mine1 = mine0 + per < seg1 ? mine0 + per : seg1;
+    for (int32_t c0 = 0; c0 < n; c0 += kWave) {
+        const int32_t col = c0 + lane;
+        AccT sum = AccT(0);
+        if (col < n) {
+            int64_t seg = mine0;
+            for (; seg + 4 <= mine1; seg += 4) {  // four loads in flight, added in order
+                const AccT p0 = partial[(seg + 0) * n + col];
+                const AccT p1 = partial[(seg + 1) * n + col];
+                const AccT p2 = partial[(seg + 2) * n + col];
+                const AccT p3 = partial[(seg + 3) * n + col];
+                sum += p0;
+                sum += p1;
+                sum += p2;
+                sum += p3;
+            }
+            for (; seg < mine1; ++seg) {
+                sum += partial[seg * n + col];
+            }
+        }
+        part[wave][lane] = sum;
+        __syncthreads();
+        if (wave == 0 && col < n) {
+            AccT total = part[0][lane];
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) {
+                total += part[w][lane];
+            }
+            CT *out = C + row * ldc + col;
+            *out = Epilogue<CT, AccT>::Apply(total, alpha, beta, betaZero, out, clampF16 != 0);
+        }
+        __syncthreads();
     }
 }
 
@@ -207,6 +398,37 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmGeneralKernel(
     }
 }
 
+// Longest row, number of long rows and number of segments.  stats[0..2] zeroed
+// before the launch.
+__global__ __launch_bounds__(kBlockThreads) void SpmmRowStatsKernel(const int32_t *__restrict__ rowOffsets,
+                                                                    int64_t rows, int32_t *__restrict__ stats)
+{
+    int32_t best = 0, numLong = 0, numSeg = 0;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlockThreads;
+    for (int64_t r = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; r < rows; r += stride) {
+        const int32_t len = rowOffsets[r + 1] - rowOffsets[r];
+        best = len > best ? len : best;
+        if (len > kLongRowNnz) {
+            ++numLong;
+            numSeg += (len + kSegmentNnz - 1) / kSegmentNnz;
+        }
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        const int32_t other = __shfl_xor(best, off, kWave);
+        best = other > best ? other : best;
+        numLong += __shfl_xor(numLong, off, kWave);
+        numSeg += __shfl_xor(numSeg, off, kWave);
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        if (best > 0) atomicMax(stats, best);
+        if (numLong > 0) {
+            atomicAdd(stats + 1, numLong);
+            atomicAdd(stats + 2, numSeg);
+        }
+    }
+}
+
 // =============================================================== host side
 
 namespace {
@@ -221,6 +443,8 @@ struct SpmmArgs {
     int32_t bColMajor, cColMajor, transB, clampF16;
     OpsparseScalar alpha, beta;
     hipStream_t stream;
+    const OpsparseSpmmPlan *plan;
+    void *ws;
 };
 
 inline int CheckLaunch()
@@ -228,19 +452,88 @@ inline int CheckLaunch()
     return hipGetLastError() == hipSuccess ? OPSPARSE_OK : OPSPARSE_E_LAUNCH;
 }
 
+inline int64_t Align256(int64_t v) { return (v + 255) / 256 * 256; }
+
+// Workspace: 256-byte header | long row ids | first segment per long row (+1) |
+// row id per segment | first entry per segment | fp64 partials [segments x n].
+void LayoutPlan(OpsparseSpmmPlan *p)
+{
+    int64_t off = 256;
+    p->longRowsOff = off;
+    off = Align256(off + 4 * static_cast<int64_t>(p->numLongRows));
+    p->longFirstSegOff = off;
+    off = Align256(off + 4 * (static_cast<int64_t>(p->numLongRows) + 1));
+    p->segRowOff = off;
+    off = Align256(off + 4 * static_cast<int64_t>(p->numSegments));
+    p->segStartOff = off;
+    off = Align256(off + 4 * static_cast<int64_t>(p->numSegments));
+    p->partialOff = off;
+    off = Align256(off + 8 * static_cast<int64_t>(p->numSegments) * p->n);
+    if (p->numOrdered > 0) {
+        p->rowOrderOff = off;
+        off = Align256(off + 4 * p->numOrdered);
+    }
+    p->bytes = (p->numLongRows > 0 || p->numOrdered > 0) ? off : 256;
+}
+
+// Device reduction of the row lengths into `scratch` (>= 16 bytes), read back
+// after a stream synchronisation.
+int RowStats(const int32_t *rowOffsets, int64_t rows, int32_t *scratch, hipStream_t s, int32_t out[3])
+{
+    out[0] = out[1] = out[2] = 0;
+    if (rows <= 0) {
+        return OPSPARSE_OK;
+    }
+    if (hipMemsetAsync(scratch, 0, 16, s) != hipSuccess) {
+        return OPSPARSE_E_LAUNCH;
+    }
+    int64_t grid = (rows + kBlockThreads - 1) / kBlockThreads;
+    grid = grid > 4096 ? 4096 : grid;
+    hipLaunchKernelGGL(SpmmRowStatsKernel, dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0, s, rowOffsets,
+                       rows, scratch);
+    if (hipMemcpyAsync(out, scratch, 12, hipMemcpyDeviceToHost, s) != hipSuccess ||
+        hipStreamSynchronize(s) != hipSuccess) {
+        (void)hipGetLastError();
+        return OPSPARSE_E_LAUNCH;
+    }
+    return OPSPARSE_OK;
+}
+
 template <typename ValT, typename CT, typename AccT, int V, int L>
 int LaunchRowSplit(const SpmmArgs &a)
 {
     constexpr int kGroups = kBlockThreads / L;
-    // Each lane group walks a few rows so that a workgroup lives long enough to
-    // hide its start-up latency.
-    const int32_t rowsPerGroup = 4;
-    const int64_t rowsPerBlock = static_cast<int64_t>(kGroups) * rowsPerGroup;
-    const uint32_t grid = static_cast<uint32_t>((a.rows + rowsPerBlock - 1) / rowsPerBlock);
-    hipLaunchKernelGGL((SpmmRowSplitKernel<ValT, CT, AccT, V, L>), dim3(grid), dim3(kBlockThreads), 0, a.stream,
-                       a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.B),
-                       static_cast<CT *>(a.C), a.rows, static_cast<int32_t>(a.n), a.ldb, a.ldc, rowsPerGroup, a.alpha,
-                       a.beta, a.clampF16);
+    const bool binned = a.plan != nullptr && a.plan->kernel == OPSPARSE_SPMM_BINNED && a.plan->numLongRows > 0;
+    const int64_t rowsPerBlock = static_cast<int64_t>(kGroups) * kSpmmRowsPerGroup;
+    const bool ordered = binned && a.plan->numOrdered > 0;
+    const int32_t *rowOrder =
+        ordered ? reinterpret_cast<const int32_t *>(static_cast<unsigned char *>(a.ws) + a.plan->rowOrderOff) : nullptr;
+    const int64_t slots = ordered ? a.plan->numOrdered : a.rows;
+    const uint32_t grid = static_cast<uint32_t>((slots + rowsPerBlock - 1) / rowsPerBlock);
+    if (slots > 0) {
+        hipLaunchKernelGGL((SpmmRowSplitKernel<ValT, CT, AccT, V, L>), dim3(grid), dim3(kBlockThreads), 0, a.stream,
+                           a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
+                           static_cast<const ValT *>(a.B), static_cast<CT *>(a.C), slots, static_cast<int32_t>(a.n),
+                           a.ldb, a.ldc, binned ? a.plan->longRowNnz : INT32_MAX, rowOrder, a.alpha,
+                           a.beta, a.clampF16);
+    }
+    if (binned) {
+        auto *base = static_cast<unsigned char *>(a.ws);
+        const auto *longRows = reinterpret_cast<const int32_t *>(base + a.plan->longRowsOff);
+        const auto *firstSeg = reinterpret_cast<const int32_t *>(base + a.plan->longFirstSegOff);
+        const auto *segRow = reinterpret_cast<const int32_t *>(base + a.plan->segRowOff);
+        const auto *segStart = reinterpret_cast<const int32_t *>(base + a.plan->segStartOff);
+        auto *partial = reinterpret_cast<AccT *>(base + a.plan->partialOff);
+        const int32_t nseg = a.plan->numSegments;
+        hipLaunchKernelGGL((SpmmLongSegmentKernel<ValT, AccT, V, L>), dim3((nseg + kGroups - 1) / kGroups),
+                           dim3(kBlockThreads), 0, a.stream, a.rowOffsets, a.colInd,
+                           static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.B),
+                           static_cast<int32_t>(a.n), a.ldb, nseg, segRow, segStart, partial);
+        const int32_t nlong = a.plan->numLongRows;
+        hipLaunchKernelGGL((SpmmLongFixupKernel<CT, AccT>), dim3(nlong),
+                           dim3(kBlockThreads), 0, a.stream, static_cast<CT *>(a.C), static_cast<int32_t>(a.n),
+                           a.ldc, nlong, longRows, firstSeg, partial, a.alpha, a.beta, a.clampF16);
+    }
     return CheckLaunch();
 }
 
@@ -292,32 +585,142 @@ using namespace opsparse;
 
 extern "C" {
 
-size_t opsparse_spmm_csr_workspace_bytes(int64_t rows, int64_t nnz, int64_t n)
+int opsparse_spmm_csr_workspace_bytes(const int32_t *rowOffsets, int64_t rows, int64_t nnz, int64_t n, void *stream,
+                                      size_t *bytes)
 {
-    (void)rows;
-    (void)nnz;
-    (void)n;
-    return 256;  // header only: the row-split kernels need no tables
+    if (bytes == nullptr || rows < 0 || nnz < 0 || n < 0 || (rows > 0 && rowOffsets == nullptr)) {
+        return OPSPARSE_E_INVALID;
+    }
+    *bytes = 256;
+    if (rows == 0 || nnz <= kLongRowNnz) {
+        return OPSPARSE_OK;  // no row can be long
+    }
+    int32_t *scratch = nullptr;
+    if (hipMalloc(reinterpret_cast<void **>(&scratch), 256) != hipSuccess) {
+        (void)hipGetLastError();
+        return OPSPARSE_E_LAUNCH;
+    }
+    int32_t st[3];
+    const int rc = RowStats(rowOffsets, rows, scratch, static_cast<hipStream_t>(stream), st);
+    (void)hipFree(scratch);
+    if (rc != OPSPARSE_OK) {
+        return rc;
+    }
+    OpsparseSpmmPlan p{};
+    p.n = n;
+    p.numLongRows = st[1];
+    p.numSegments = st[2];
+    p.numOrdered = st[1] > 0 ? rows - st[1] : 0;
+    LayoutPlan(&p);
+    *bytes = static_cast<size_t>(p.bytes);
+    return OPSPARSE_OK;
 }
 
 int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t nnz, int64_t n, void *workspace,
                               size_t workspaceBytes, int32_t forceKernel, OpsparseSpmmPlan *plan, void *stream)
 {
-    (void)rowOffsets;
-    (void)stream;
-    (void)forceKernel;
-    if (plan == nullptr || rows < 0 || nnz < 0 || n < 0) {
+    if (plan == nullptr || rows < 0 || nnz < 0 || n < 0 || (rows > 0 && rowOffsets == nullptr)) {
         return OPSPARSE_E_INVALID;
     }
     if (workspace == nullptr || workspaceBytes < 256) {
         return OPSPARSE_E_WORKSPACE;
     }
+    auto s = static_cast<hipStream_t>(stream);
     OpsparseSpmmPlan p{};
     p.kernel = OPSPARSE_SPMM_ROW_SPLIT;
     p.rows = rows;
     p.nnz = nnz;
     p.n = n;
+    p.longRowNnz = kLongRowNnz;
+    p.segmentNnz = kSegmentNnz;
     p.bytes = 256;
+    if (rows == 0 || nnz <= kLongRowNnz || forceKernel == OPSPARSE_SPMM_ROW_SPLIT) {
+        *plan = p;
+        return OPSPARSE_OK;
+    }
+    int32_t st[3];
+    int rc = RowStats(rowOffsets, rows, static_cast<int32_t *>(workspace), s, st);
+    if (rc != OPSPARSE_OK) {
+        return rc;
+    }
+    p.maxRowNnz = st[0];
+    if (st[1] == 0) {
+        *plan = p;
+        return OPSPARSE_OK;
+    }
+    p.kernel = OPSPARSE_SPMM_BINNED;
+    p.numLongRows = st[1];
+    p.numSegments = st[2];
+    p.numOrdered = rows - st[1];
+    LayoutPlan(&p);
+    if (static_cast<int64_t>(workspaceBytes) < p.bytes) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    // The long-row tables are built on the host from a copy of the row offsets
+    // (once per matrix, like the reference's Preprocess,
+    // sparse/spmm/arch35/spmm_csr_mat.cpp:94-136) and uploaded.
+    std::vector<int32_t> rp(static_cast<size_t>(rows) + 1);
+    if (hipMemcpyAsync(rp.data(), rowOffsets, rp.size() * 4, hipMemcpyDeviceToHost, s) != hipSuccess ||
+        hipStreamSynchronize(s) != hipSuccess) {
+        (void)hipGetLastError();
+        return OPSPARSE_E_LAUNCH;
+    }
+    std::vector<int32_t> longRows, firstSeg, segRow, segStart;
+    longRows.reserve(p.numLongRows);
+    firstSeg.reserve(p.numLongRows + 1);
+    segRow.reserve(p.numSegments);
+    segStart.reserve(p.numSegments);
+    for (int64_t r = 0; r < rows; ++r) {
+        const int32_t len = rp[r + 1] - rp[r];
+        if (len > kLongRowNnz) {
+            longRows.push_back(static_cast<int32_t>(r));
+            firstSeg.push_back(static_cast<int32_t>(segRow.size()));
+            for (int32_t q = rp[r]; q < rp[r + 1]; q += kSegmentNnz) {
+                segRow.push_back(static_cast<int32_t>(r));
+                segStart.push_back(q);
+            }
+        }
+    }
+    firstSeg.push_back(static_cast<int32_t>(segRow.size()));
+    // The other rows, longest first (counting sort by length, stable in the row index).
+    std::vector<int32_t> order(static_cast<size_t>(p.numOrdered));
+    {
+        std::vector<int64_t> start(static_cast<size_t>(kLongRowNnz) + 2, 0);
+        for (int64_t r = 0; r < rows; ++r) {
+            const int32_t len = rp[r + 1] - rp[r];
+            if (len <= kLongRowNnz) {
+                ++start[kLongRowNnz - len + 1];
+            }
+        }
+        for (size_t b = 1; b < start.size(); ++b) {
+            start[b] += start[b - 1];
+        }
+        for (int64_t r = 0; r < rows; ++r) {
+            const int32_t len = rp[r + 1] - rp[r];
+            if (len <= kLongRowNnz) {
+                order[static_cast<size_t>(start[kLongRowNnz - len]++)] = static_cast<int32_t>(r);
+            }
+        }
+    }
+    if (static_cast<int32_t>(longRows.size()) != p.numLongRows || static_cast<int32_t>(segRow.size()) != p.numSegments) {
+        return OPSPARSE_E_INVALID;  // the matrix changed between the two passes
+    }
+    auto *base = static_cast<unsigned char *>(workspace);
+    bool ok = hipMemcpyAsync(base + p.longRowsOff, longRows.data(), longRows.size() * 4, hipMemcpyHostToDevice, s) ==
+              hipSuccess;
+    ok = ok && hipMemcpyAsync(base + p.longFirstSegOff, firstSeg.data(), firstSeg.size() * 4, hipMemcpyHostToDevice,
+                              s) == hipSuccess;
+    ok = ok && hipMemcpyAsync(base + p.segRowOff, segRow.data(), segRow.size() * 4, hipMemcpyHostToDevice, s) ==
+                   hipSuccess;
+    ok = ok && hipMemcpyAsync(base + p.segStartOff, segStart.data(), segStart.size() * 4, hipMemcpyHostToDevice, s) ==
+                   hipSuccess;
+    ok = ok && (order.empty() || hipMemcpyAsync(base + p.rowOrderOff, order.data(), order.size() * 4,
+                                                hipMemcpyHostToDevice, s) == hipSuccess);
+    ok = ok && hipStreamSynchronize(s) == hipSuccess;  // the host vectors die at return
+    if (!ok) {
+        (void)hipGetLastError();
+        return OPSPARSE_E_LAUNCH;
+    }
     *plan = p;
     return OPSPARSE_OK;
 }
@@ -328,20 +731,27 @@ int opsparse_spmm_csr_launch(const OpsparseSpmmPlan *plan, const int32_t *rowOff
                              int32_t transB, OpsparseScalar alpha, OpsparseScalar beta, int32_t valType,
                              int32_t cType, void *workspace, size_t workspaceBytes, void *stream)
 {
-    (void)plan;
-    (void)workspace;
-    (void)workspaceBytes;
     if (rows < 0 || k < 0 || n < 0 || nnz < 0 || ldb <= 0 || ldc <= 0 || n > INT32_MAX) {
         return OPSPARSE_E_INVALID;
     }
     if (rows == 0 || n == 0) {
         return OPSPARSE_OK;
     }
-    if (rowOffsets == nullptr || C == nullptr || (nnz > 0 && (colInd == nullptr || csrValues == nullptr || B == nullptr))) {
+    if (rowOffsets == nullptr || C == nullptr ||
+        (nnz > 0 && (colInd == nullptr || csrValues == nullptr || B == nullptr))) {
         return OPSPARSE_E_INVALID;
     }
-    SpmmArgs a{rowOffsets, colInd, csrValues, B,      C,    rows, k, n, nnz, ldb, ldc, bColMajor, cColMajor,
-               transB,     0,      alpha,     beta,   static_cast<hipStream_t>(stream)};
+    if (plan != nullptr) {
+        if (plan->rows != rows || plan->nnz != nnz || (plan->kernel == OPSPARSE_SPMM_BINNED && plan->n != n)) {
+            return OPSPARSE_E_INVALID;
+        }
+        if (plan->kernel == OPSPARSE_SPMM_BINNED &&
+            (workspace == nullptr || static_cast<int64_t>(workspaceBytes) < plan->bytes)) {
+            return OPSPARSE_E_WORKSPACE;
+        }
+    }
+    SpmmArgs a{rowOffsets, colInd, csrValues, B, C, rows, k, n, nnz, ldb, ldc, bColMajor, cColMajor, transB, 0,
+               alpha, beta, static_cast<hipStream_t>(stream), plan, workspace};
     if (valType == OPSPARSE_F32 && cType == OPSPARSE_F32) {
         return RunTyped<float, float, double>(a);
     }

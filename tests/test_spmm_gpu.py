@@ -1,0 +1,217 @@
+"""GPU parity tests for aclsparseSpMM (GetBufferSize -> Preprocess -> SpMM through
+the C ABI) against the CPU oracle.
+
+Tolerances, written per test:
+  fp32              per element |d| <= 1e-5 * max(|oracle|, 1e-30) against the
+                    fp64-accumulated oracle (the library accumulates in fp64),
+                    plus the reference's own MERE < 2^-13 / MARE < 10 * 2^-13 rule
+                    against its fp32 golden (test/spmm/arch35/spmm_test.cpp:525-526)
+  fp16 in, fp32 out per element 1e-3 relative against the oracle on the fp16-rounded inputs
+  fp16 in and out   the reference's fp16 recipe (:604-622): fp32 golden on rounded
+                    inputs, clamp, re-round; MERE < 2^-10, MARE < 10 * 2^-10
+  int8              bit-exact
+"""
+import numpy as np
+import pytest
+
+import oracle
+from helpers import csr_from_lengths, random_csr, run_spmm
+
+pytestmark = pytest.mark.gpu
+
+
+def glibc_free_random_csr(m, k, nnz, seed):
+    """Shape of the reference's GenerateRandomCsr (spmm_test.cpp:91-123): nnz spread
+    evenly over the rows, distinct sorted columns, values on a fixed grid in [-5, 5]."""
+    rng = np.random.default_rng(seed)
+    lengths = np.array([min(nnz // m + (1 if i < nnz % m else 0), k) for i in range(m)])
+    rowptr, colind, _ = csr_from_lengths(lengths, k, seed)
+    val = (-5.0 + 10.0 * (np.arange(colind.size) % 10001) / 10000.0).astype(np.float32)
+    return rowptr, colind, val
+
+
+def check_fp32(got, m, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta, **layout):
+    gold = oracle.spmm_f64(m, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta, **layout)
+    crm = layout.get("c_row_major", True)
+    idx = (np.arange(m)[:, None] * ldc + np.arange(n)[None, :]) if crm else \
+        (np.arange(n)[None, :] * ldc + np.arange(m)[:, None])
+    err = oracle.max_rel_err(got[idx], gold[idx])
+    assert err <= 1e-5, "max rel err %.3e" % err
+    # padding between rows / columns must be untouched
+    mask = np.ones(got.size, bool)
+    mask[idx.ravel()] = False
+    assert np.array_equal(got[mask], np.asarray(C0, np.float32)[mask])
+    g32 = oracle.spmm_f32(m, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta, **layout)
+    # Against the reference's fp32 golden only the mean is asserted: on elements that
+    # nearly cancel, that golden's own rounding error exceeds the 10 * 2^-13 cap.
+    mere, _, mism, _ = oracle.mere_mare(got[idx], g32[idx], eps=1e-7)
+    assert mism == 0 and mere < 2.0 ** -13
+
+
+def test_readme_known_answer(osa, gpu_ctx):
+    """A (4x3, nnz 5) * B (3x2) = [[3,2],[0,3],[4,0],[5,5]] (reference sparse/spmm/README.md:275-303, :404-412)."""
+    rowptr = np.array([0, 2, 3, 4, 5], np.int32)
+    colind = np.array([0, 2, 1, 0, 2], np.int32)
+    val = np.array([1, 2, 3, 4, 5], np.float32)
+    B = np.array([1, 0, 0, 1, 1, 1], np.float32)
+    C = run_spmm(osa, gpu_ctx, 4, 3, 2, rowptr, colind, val, B, 2, np.zeros(8, np.float32), 2, 1.0, 0.0,
+                 alg=osa.ACL_SPARSE_SPMM_CSR_ALG1)
+    assert np.array_equal(C.reshape(4, 2), np.array([[3, 2], [0, 3], [4, 0], [5, 5]], np.float32))
+
+
+# the reference's five fp32 layout cases (spmm_test.cpp:964-975)
+REF_CASES = [
+    ("baseline_row_N_beta0", 256, 256, 64, 0, 1.0, 0.0, False, True, True, 42),
+    ("opB_transpose", 256, 256, 64, 0, 1.0, 0.0, True, True, True, 43),
+    ("B_C_col_major", 256, 256, 64, 0, 1.0, 0.0, False, False, False, 44),
+    ("beta_nonzero", 256, 256, 64, 0, 1.0, 0.5, False, True, True, 45),
+    ("small_shape", 32, 32, 16, 80, 1.0, 0.0, False, True, True, 46),
+]
+
+
+@pytest.mark.parametrize("name,m,k,n,nnz,alpha,beta,trans_b,b_rm,c_rm,seed", REF_CASES)
+def test_reference_fp32_cases(osa, gpu_ctx, name, m, k, n, nnz, alpha, beta, trans_b, b_rm, c_rm, seed):
+    nnz = nnz if nnz > 0 else m * k // 10
+    rowptr, colind, val = glibc_free_random_csr(m, k, nnz, seed)
+    ldb = n if b_rm else k
+    ldc = n if c_rm else m
+    rng = np.random.default_rng(seed)
+    B = rng.uniform(-1, 1, k * ldb).astype(np.float32)
+    C0 = rng.uniform(-1, 1, (m if c_rm else n) * ldc).astype(np.float32)
+    if beta == 0.0:
+        C0[:] = np.nan  # must not be read
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta,
+                   order_b=osa.ACL_SPARSE_ORDER_ROW if b_rm else osa.ACL_SPARSE_ORDER_COL,
+                   order_c=osa.ACL_SPARSE_ORDER_ROW if c_rm else osa.ACL_SPARSE_ORDER_COL,
+                   op_b=osa.ACL_SPARSE_OP_TRANSPOSE if trans_b else osa.ACL_SPARSE_OP_NON_TRANSPOSE)
+    C0z = np.zeros_like(C0) if beta == 0.0 else C0
+    gold = oracle.spmm_f64(m, n, rowptr, colind, val, B, ldb, C0z, ldc, alpha, beta, b_row_major=b_rm,
+                           trans_b=trans_b, c_row_major=c_rm)
+    assert oracle.max_rel_err(got, gold) <= 1e-5
+
+
+@pytest.mark.parametrize("n", [1, 3, 8, 17, 32, 64, 100, 128, 256, 260])
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, -2.0)])
+def test_column_counts_and_padding(osa, gpu_ctx, n, alpha, beta):
+    """n not a multiple of the vector width, and ldb / ldc padding."""
+    m, k = 300, 200
+    rowptr, colind, val = random_csr(m, k, 0.05, seed=n, empty_row_prob=0.1)
+    ldb, ldc = n + (4 if n % 2 else 0), n + (8 if n % 3 == 0 else 0)
+    rng = np.random.default_rng(n)
+    B = rng.uniform(-2, 2, k * ldb).astype(np.float32)
+    C0 = rng.uniform(-2, 2, m * ldc).astype(np.float32)
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta)
+    check_fp32(got, m, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta)
+
+
+@pytest.mark.parametrize("b_rm,c_rm,trans_b", [(True, False, False), (False, True, False), (False, False, True),
+                                               (True, True, True), (False, True, True)])
+def test_layouts(osa, gpu_ctx, b_rm, c_rm, trans_b):
+    m, k, n = 120, 120, 24      # square so that every (order, op) reading of B stays in bounds
+    rowptr, colind, val = random_csr(m, k, 0.1, seed=5, unsorted=True)
+    ldb, ldc = 130, 125
+    rng = np.random.default_rng(1)
+    B = rng.uniform(-2, 2, 130 * ldb).astype(np.float32)
+    C0 = rng.uniform(-2, 2, 125 * ldc).astype(np.float32)
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, ldb, C0, ldc, 1.5, 0.25,
+                   order_b=osa.ACL_SPARSE_ORDER_ROW if b_rm else osa.ACL_SPARSE_ORDER_COL,
+                   order_c=osa.ACL_SPARSE_ORDER_ROW if c_rm else osa.ACL_SPARSE_ORDER_COL,
+                   op_b=osa.ACL_SPARSE_OP_TRANSPOSE if trans_b else osa.ACL_SPARSE_OP_NON_TRANSPOSE)
+    check_fp32(got, m, n, rowptr, colind, val, B, ldb, C0, ldc, 1.5, 0.25, b_row_major=b_rm, trans_b=trans_b,
+               c_row_major=c_rm)
+
+
+@pytest.mark.parametrize("n", [64, 128, 16])
+def test_long_rows_are_binned(osa, gpu_ctx, n):
+    """Rows far above the long-row threshold next to short and empty ones."""
+    rng = np.random.default_rng(n)
+    m, k = 2000, 60000
+    lengths = rng.integers(0, 40, m)
+    lengths[[3, 700, 701, 1999]] = [50000, 513, 512, 12345]
+    rowptr, colind, val = csr_from_lengths(lengths, k, seed=2)
+    B = rng.uniform(-1, 1, k * n).astype(np.float32)
+    C0 = rng.uniform(-1, 1, m * n).astype(np.float32)
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, n, C0, n, 2.0, 1.0)
+    gold = oracle.spmm_f64_rowmajor(m, n, rowptr, colind, val, B, n, C0, n, 2.0, 1.0)
+    assert oracle.max_rel_err(got, gold) <= 1e-5
+
+
+def test_high_precision_alg_same_result(osa, gpu_ctx):
+    m, k, n = 500, 500, 64
+    rowptr, colind, val = random_csr(m, k, 0.1, seed=8)
+    rng = np.random.default_rng(8)
+    B = rng.uniform(-1, 1, k * n).astype(np.float32)
+    C0 = np.zeros(m * n, np.float32)
+    a = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, n, C0, n, 1.0, 0.0)
+    b = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, n, C0, n, 1.0, 0.0,
+                 alg=osa.ACL_SPARSE_SPMM_CSR_FP32_HIGH_PRECISION_ALG)
+    assert np.array_equal(a, b)
+
+
+def _fp16_inputs(m, k, n, seed):
+    rowptr, colind, val = glibc_free_random_csr(m, k, m * k // 10, seed)
+    rng = np.random.default_rng(seed)
+    B = rng.uniform(-1, 1, k * n).astype(np.float32)
+    C0 = rng.uniform(-1, 1, m * n).astype(np.float32)
+    rt = lambda a: oracle.f16_bits_to_f32(oracle.f32_to_f16_bits(a))
+    return rowptr, colind, rt(val), rt(B), rt(C0)
+
+
+def test_fp16_in_fp16_out_reference_recipe(osa, gpu_ctx):
+    import torch
+    m, k, n = 256, 256, 64
+    rowptr, colind, val, B, C0 = _fp16_inputs(m, k, n, 47)
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, n, C0, n, 1.0, 0.5, val_dtype=torch.float16,
+                   c_dtype=torch.float16)
+    gold = oracle.spmm_f32(m, n, rowptr, colind, val, B, n, C0, n, 1.0, 0.5)
+    gold = oracle.f16_bits_to_f32(oracle.f32_to_f16_bits(np.clip(gold, -65504.0, 65504.0)))
+    mere, mare, mism, _ = oracle.mere_mare(got, gold, eps=1e-7)
+    assert mism == 0 and mere < 2.0 ** -10 and mare < 10 * 2.0 ** -10
+
+
+def test_fp16_out_clamps(osa, gpu_ctx):
+    import torch
+    rowptr = np.array([0, 2, 4], np.int32)
+    colind = np.array([0, 1, 0, 1], np.int32)
+    val = np.array([60000, 60000, -60000, -60000], np.float32)
+    B = np.ones(2 * 8, np.float32)
+    got = run_spmm(osa, gpu_ctx, 2, 2, 8, rowptr, colind, val, B, 8, np.zeros(16, np.float32), 8, 1.0, 0.0,
+                   val_dtype=torch.float16, c_dtype=torch.float16)
+    assert np.array_equal(got.reshape(2, 8), np.array([[65504.0] * 8, [-65504.0] * 8], np.float32))
+
+
+def test_fp16_in_fp32_out(osa, gpu_ctx):
+    """fp16 A and B, fp32 accumulate and C: 1e-3 relative against the oracle on the rounded inputs."""
+    import torch
+    m, k, n = 400, 300, 128
+    rowptr, colind, val, B, C0 = _fp16_inputs(m, k, n, 48)
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, n, C0, n, 1.0, 0.0, val_dtype=torch.float16)
+    gold = oracle.spmm_f64_rowmajor(m, n, rowptr, colind, val, B, n, np.zeros_like(C0), n, 1.0, 0.0)
+    assert oracle.max_rel_err(got, gold) <= 1e-3
+
+
+@pytest.mark.parametrize("alpha,beta", [(1, 0), (3, -2), (20000, 1)])
+def test_int8_exact(osa, gpu_ctx, alpha, beta):
+    import torch
+    m, k, n = 256, 256, 64
+    rowptr, colind, _ = glibc_free_random_csr(m, k, m * k // 10, 49)
+    rng = np.random.default_rng(49)
+    val = rng.integers(-128, 128, colind.size).astype(np.int8)
+    B = rng.integers(-128, 128, k * n).astype(np.int8)
+    C0 = rng.integers(-1000, 1000, m * n).astype(np.int32)
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, n, C0, n, alpha, beta, val_dtype=torch.int8,
+                   c_dtype=torch.int32, compute_type=osa.ACL_INT32)
+    gold = oracle.spmm_i8(m, n, rowptr, colind, val, B, n, C0, n, alpha, beta, saturate=True)
+    assert np.array_equal(got, gold)
+
+
+def test_spmm_column_equals_spmv(osa, gpu_ctx):
+    """Column j of the SpMM result equals the oracle SpMV with B[:, j]."""
+    m, k, n = 333, 222, 8
+    rowptr, colind, val = random_csr(m, k, 0.07, seed=12)
+    rng = np.random.default_rng(12)
+    B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B.ravel(), n, np.zeros(m * n, np.float32), n, 1.0, 0.0)
+    for j in range(n):
+        y = oracle.spmv_f64(m, k, rowptr, colind, val, np.ascontiguousarray(B[:, j]), None, 1.0, 0.0)
+        assert oracle.max_rel_err(got.reshape(m, n)[:, j], y) <= 1e-6
