@@ -1,0 +1,294 @@
+"""Host-only tests of the C ABI: every symbol the public headers declare is exported,
+and every argument check returns the status the reference returns for it, before any
+device work.  Device pointers are fake (never dereferenced on these paths)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+FAKE = ctypes.c_void_p(0x1000)
+NULL = ctypes.c_void_p(None)
+
+
+@pytest.fixture(scope="module")
+def L(osa):
+    return osa.lib()
+
+
+def declared(header, prefix):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(%s\w+)\s*\(" % prefix, text)))
+
+
+def test_every_declared_symbol_is_exported(osa, L):
+    acl = declared("cann_ops_sparse.h", "aclsparse")
+    raw = declared("ops_sparse_hip.h", "opsparse_")
+    assert len(acl) >= 40 and len(raw) >= 7
+    for name in acl + raw:
+        assert hasattr(L, name), name + " is declared but not exported"
+    # and the binding's own lists name exactly the declared functions
+    assert sorted(osa.ACLSPARSE_SYMBOLS) == acl
+    assert sorted(osa.OPSPARSE_SYMBOLS) == raw
+
+
+def test_enum_values_match_header(osa):
+    text = open(os.path.join(ROOT, "include", "cann_ops_sparse.h")).read()
+    m = re.search(r"typedef enum aclsparseStatus_t \{(.*?)\}", text, re.S)
+    names = re.findall(r"ACL_SPARSE_STATUS_(\w+)", m.group(1))
+    assert names == osa.STATUS_NAMES
+    assert osa.ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR == 10 and osa.ACL_SPARSE_STATUS_NOT_SUPPORTED == 8
+
+
+def st(osa, name):
+    return getattr(osa, "ACL_SPARSE_STATUS_" + name)
+
+
+# ------------------------------------------------------------------ handle
+
+def test_handle_lifecycle(osa, L):
+    assert L.aclsparseCreate(None) == st(osa, "HANDLE_IS_NULLPTR")
+    h = ctypes.c_void_p(None)
+    assert L.aclsparseCreate(ctypes.byref(h)) == 0 and h.value
+    assert L.aclsparseCreate(ctypes.byref(h)) == st(osa, "INVALID_VALUE")      # would overwrite a live handle
+    v = ctypes.c_int(0)
+    assert L.aclsparseGetVersion(None, ctypes.byref(v)) == 0 and v.value == 10000
+    assert L.aclsparseGetVersion(h, None) == st(osa, "INVALID_VALUE")
+    s = ctypes.c_void_p(123)
+    assert L.aclsparseGetStream(h, ctypes.byref(s)) == 0 and s.value is None
+    assert L.aclsparseSetStream(h, ctypes.c_void_p(0x55)) == 0
+    assert L.aclsparseGetStream(h, ctypes.byref(s)) == 0 and s.value == 0x55
+    assert L.aclsparseGetStream(h, None) == st(osa, "INVALID_VALUE")
+    assert L.aclsparseSetStream(None, s) == st(osa, "HANDLE_IS_NULLPTR")
+    mode = ctypes.c_int(-1)
+    assert L.aclsparseGetPointerMode(h, ctypes.byref(mode)) == 0 and mode.value == osa.ACL_SPARSE_POINTER_MODE_HOST
+    assert L.aclsparseSetPointerMode(h, 1) == 0
+    assert L.aclsparseGetPointerMode(h, ctypes.byref(mode)) == 0 and mode.value == 1
+    assert L.aclsparseSetPointerMode(h, 7) == st(osa, "INVALID_VALUE")
+    assert L.aclsparseSetPointerMode(None, 0) == st(osa, "HANDLE_IS_NULLPTR")
+    # workspace: grow-only user workspace, NULL switches back
+    assert L.aclsparseSetWorkspace(h, FAKE, 0) == st(osa, "INVALID_VALUE")
+    assert L.aclsparseSetWorkspace(h, FAKE, 1024) == 0
+    ws, n = ctypes.c_void_p(None), ctypes.c_size_t(0)
+    assert L.aclsparseGetWorkspace(h, ctypes.byref(ws), ctypes.byref(n)) == 0 and (ws.value, n.value) == (0x1000, 1024)
+    assert L.aclsparseSetWorkspace(h, ctypes.c_void_p(0x2000), 512) == 0        # not larger: ignored
+    assert L.aclsparseGetWorkspace(h, ctypes.byref(ws), ctypes.byref(n)) == 0 and (ws.value, n.value) == (0x1000, 1024)
+    assert L.aclsparseSetWorkspace(h, ctypes.c_void_p(0x2000), 4096) == 0
+    assert L.aclsparseGetWorkspace(h, ctypes.byref(ws), ctypes.byref(n)) == 0 and (ws.value, n.value) == (0x2000, 4096)
+    assert L.aclsparseGetWorkspace(h, None, ctypes.byref(n)) == st(osa, "INVALID_VALUE")
+    assert L.aclsparseGetWorkspace(None, ctypes.byref(ws), ctypes.byref(n)) == st(osa, "HANDLE_IS_NULLPTR")
+    # stream back to null before destroy: no device work was ever queued
+    assert L.aclsparseSetStream(h, NULL) == 0
+    assert L.aclsparseDestroy(h) == 0
+    assert L.aclsparseDestroy(None) == st(osa, "HANDLE_IS_NULLPTR")
+
+
+# -------------------------------------------------------------- descriptors
+
+def make_csr(osa, L, rows=4, cols=4, nnz=5, ptr=0, idx=0, base=0, vt=None, rp=FAKE, ci=FAKE, va=FAKE):
+    d = ctypes.c_void_p(None)
+    rc = L.aclsparseCreateCsr(ctypes.byref(d), rows, cols, nnz, rp, ci, va, ptr, idx, base,
+                              osa.ACL_FLOAT if vt is None else vt)
+    return rc, d
+
+
+def make_vec(osa, L, n=4, vt=None, p=FAKE):
+    d = ctypes.c_void_p(None)
+    return L.aclsparseCreateDnVec(ctypes.byref(d), n, p, osa.ACL_FLOAT if vt is None else vt), d
+
+
+def make_mat(osa, L, rows=4, cols=2, ld=2, vt=None, order=0, p=FAKE):
+    d = ctypes.c_void_p(None)
+    return L.aclsparseCreateDnMat(ctypes.byref(d), rows, cols, ld, p, osa.ACL_FLOAT if vt is None else vt, order), d
+
+
+def test_descriptor_creators(osa, L):
+    INV, NS = st(osa, "INVALID_VALUE"), st(osa, "NOT_SUPPORTED")
+    assert L.aclsparseCreateCsr(None, 1, 1, 1, FAKE, FAKE, FAKE, 0, 0, 0, 0) == INV
+    assert make_csr(osa, L, rows=-1)[0] == INV and make_csr(osa, L, nnz=-1)[0] == INV
+    assert make_csr(osa, L, ptr=5)[0] == NS and make_csr(osa, L, idx=9)[0] == NS
+    for ptr, idx in [(0, 0), (1, 0), (0, 1), (1, 1)]:          # every I32 / I64 mix can be described
+        rc, d = make_csr(osa, L, ptr=ptr, idx=idx)
+        assert rc == 0
+        assert L.aclsparseDestroySpMat(d) == 0
+    assert L.aclsparseDestroySpMat(None) == 0
+    rc, d = make_csr(osa, L, rows=3, cols=7, nnz=5)
+    r, c, z = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
+    assert L.aclsparseSpMatGetSize(d, ctypes.byref(r), ctypes.byref(c), ctypes.byref(z)) == 0
+    assert (r.value, c.value, z.value) == (3, 7, 5)
+    f = ctypes.c_int(-1)
+    assert L.aclsparseSpMatGetFormat(d, ctypes.byref(f)) == 0 and f.value == osa.ACL_SPARSE_FORMAT_CSR
+    v = ctypes.c_void_p(None)
+    assert L.aclsparseSpMatSetValues(d, ctypes.c_void_p(0x77)) == 0
+    assert L.aclsparseSpMatGetValues(d, ctypes.byref(v)) == 0 and v.value == 0x77
+    assert L.aclsparseConstSpMatGetValues(d, ctypes.byref(v)) == 0 and v.value == 0x77
+    assert L.aclsparseCsrSetPointers(d, FAKE, NULL, FAKE) == INV            # nnz > 0 needs indices
+    assert L.aclsparseCsrSetPointers(d, FAKE, FAKE, ctypes.c_void_p(0x88)) == 0
+    assert L.aclsparseSpMatGetValues(d, ctypes.byref(v)) == 0 and v.value == 0x88
+    assert L.aclsparseSpMatGetSize(None, None, None, None) == INV
+    L.aclsparseDestroySpMat(d)
+
+    assert make_vec(osa, L, n=-1)[0] == INV and make_vec(osa, L, n=3, p=NULL)[0] == INV
+    assert make_vec(osa, L, vt=12345)[0] == INV
+    rc, d = make_vec(osa, L, n=0, p=NULL)
+    assert rc == 0
+    n, t = ctypes.c_int64(-1), ctypes.c_int(-1)
+    assert L.aclsparseDnVecGet(d, ctypes.byref(n), ctypes.byref(v), ctypes.byref(t)) == 0 and n.value == 0
+    assert L.aclsparseDnVecSetValues(d, ctypes.c_void_p(0x99)) == 0
+    assert L.aclsparseDnVecGetValues(d, ctypes.byref(v)) == 0 and v.value == 0x99
+    assert L.aclsparseConstDnVecGetValues(d, ctypes.byref(v)) == 0
+    assert L.aclsparseDnVecGetValues(d, None) == INV
+    assert L.aclsparseDestroyDnVec(d) == 0
+    assert L.aclsparseDestroyDnVec(None) == INV
+    assert L.aclsparseDnVecGet(None, None, None, None) == INV
+
+    for kw in (dict(rows=0), dict(cols=0), dict(ld=0), dict(p=NULL), dict(vt=999), dict(order=5),
+               dict(cols=8, ld=7), dict(rows=9, ld=8, order=1)):
+        assert make_mat(osa, L, **kw)[0] == INV, kw
+    rc, d = make_mat(osa, L, rows=6, cols=3, ld=5)
+    a, b, c2, o = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int(-1)
+    assert L.aclsparseDnMatGet(d, ctypes.byref(a), ctypes.byref(b), ctypes.byref(c2), ctypes.byref(v), ctypes.byref(t),
+                               ctypes.byref(o)) == 0
+    assert (a.value, b.value, c2.value, o.value, v.value) == (6, 3, 5, 0, 0x1000)
+    assert L.aclsparseDnMatSetValues(d, ctypes.c_void_p(0x66)) == 0
+    assert L.aclsparseDnMatGetValues(d, ctypes.byref(v)) == 0 and v.value == 0x66
+    assert L.aclsparseDestroyDnMat(d) == 0
+    assert L.aclsparseDestroyDnMat(None) == INV
+
+
+# --------------------------------------------------------------------- SpMV
+
+@pytest.fixture()
+def handle(osa, L):
+    h = ctypes.c_void_p(None)
+    assert L.aclsparseCreate(ctypes.byref(h)) == 0
+    assert L.aclsparseSetStream(h, ctypes.c_void_p(0x55)) == 0     # fake stream: never used on failing paths
+    yield h
+    L.aclsparseSetStream(h, NULL)
+    L.aclsparseDestroy(h)
+
+
+def spmv(osa, L, h, A, x, y, op=0, ct=None, alg=0, buf=NULL):
+    return L.aclsparseSpMV(h, op, None, A, x, None, y, osa.ACL_FLOAT if ct is None else ct, alg, buf)
+
+
+def test_spmv_status_table(osa, L, handle):
+    """reference sparse/spmv/arch22/spmv_host.cpp:132-274, in its order."""
+    INV, NS = st(osa, "INVALID_VALUE"), st(osa, "NOT_SUPPORTED")
+    _, A = make_csr(osa, L)
+    _, x = make_vec(osa, L, 4)
+    _, y = make_vec(osa, L, 4)
+    assert spmv(osa, L, None, A, x, y) == st(osa, "HANDLE_IS_NULLPTR")
+    assert spmv(osa, L, handle, None, x, y) == INV
+    assert spmv(osa, L, handle, A, None, y) == INV
+    assert spmv(osa, L, handle, A, x, None) == INV
+    assert spmv(osa, L, handle, A, x, y, alg=osa.ACL_SPARSE_SPMV_CSR_ALG1) == NS
+    assert spmv(osa, L, handle, A, x, y, ct=osa.ACL_FLOAT16) == NS
+    assert spmv(osa, L, handle, A, x, y, op=osa.ACL_SPARSE_OP_CONJUGATE_TRANSPOSE) == NS
+    for kw in (dict(base=1), dict(ptr=1, idx=1), dict(ptr=1), dict(idx=1)):
+        _, bad = make_csr(osa, L, **kw)
+        assert spmv(osa, L, handle, bad, x, y) == NS, kw
+        L.aclsparseDestroySpMat(bad)
+    # no stream set
+    L.aclsparseSetStream(handle, NULL)
+    assert spmv(osa, L, handle, A, x, y) == INV
+    L.aclsparseSetStream(handle, ctypes.c_void_p(0x55))
+    # null device arrays
+    _, bad = make_csr(osa, L, va=NULL)
+    assert spmv(osa, L, handle, bad, x, y) == INV
+    L.aclsparseDestroySpMat(bad)
+    # vectors too short (x needs cols, y needs rows; swapped for the transpose)
+    _, xs = make_vec(osa, L, 3)
+    assert spmv(osa, L, handle, A, xs, y) == INV and spmv(osa, L, handle, A, x, xs) == INV
+    _, R = make_csr(osa, L, rows=3, cols=4, nnz=2)
+    assert spmv(osa, L, handle, R, x, xs, op=1) == INV           # transpose: y needs cols = 4
+    _, x2 = make_vec(osa, L, 2)
+    assert spmv(osa, L, handle, R, x2, y, op=1) == INV           # transpose: x needs rows = 3
+    L.aclsparseDestroyDnVec(x2)
+    # x type must equal A type; INT32 compute needs all-int32
+    _, xh = make_vec(osa, L, 4, vt=osa.ACL_FLOAT16)
+    assert spmv(osa, L, handle, A, xh, y) == NS
+    assert spmv(osa, L, handle, A, x, y, ct=osa.ACL_INT32) == NS
+    # GetBufferSize / Preprocess share the checks
+    n = ctypes.c_size_t(0)
+    assert L.aclsparseSpMVGetBufferSize(handle, 0, None, A, x, None, y, osa.ACL_FLOAT, 0, None) == INV
+    assert L.aclsparseSpMVGetBufferSize(None, 0, None, A, x, None, y, osa.ACL_FLOAT, 0, ctypes.byref(n)) == \
+        st(osa, "HANDLE_IS_NULLPTR")
+    assert L.aclsparseSpMVGetBufferSize(handle, 0, None, A, x, None, y, osa.ACL_FLOAT, 0, ctypes.byref(n)) == 0
+    assert n.value >= 256 and n.value == L.opsparse_spmv_csr_workspace_bytes(4, 5)
+    assert L.aclsparseSpMVPreprocess(handle, 0, None, A, x, None, y, osa.ACL_FLOAT, 0, None) == \
+        st(osa, "INSUFFICIENT_RESOURCES")
+    for d in (x, y, xs, xh):
+        L.aclsparseDestroyDnVec(d)
+    L.aclsparseDestroySpMat(A)
+    L.aclsparseDestroySpMat(R)
+
+
+# --------------------------------------------------------------------- SpMM
+
+def spmm_args(osa, h, A, B, C, opa=0, opb=0, ct=None, alg=0):
+    return (h, opa, opb, None, A, B, None, C, osa.ACL_FLOAT if ct is None else ct, alg)
+
+
+def test_spmm_status_table(osa, L, handle):
+    """reference sparse/spmm/arch35/spmm_host.cpp:152-191, :213-234, :335-362, :364-394."""
+    INV, NS, HN = st(osa, "INVALID_VALUE"), st(osa, "NOT_SUPPORTED"), st(osa, "HANDLE_IS_NULLPTR")
+    _, A = make_csr(osa, L, rows=4, cols=3, nnz=5)
+    _, B = make_mat(osa, L, rows=3, cols=2, ld=2)
+    _, C = make_mat(osa, L, rows=4, cols=2, ld=2)
+    n = ctypes.c_size_t(0)
+    run = lambda *a, **k: L.aclsparseSpMM(*spmm_args(osa, *a, **k), FAKE)
+    assert L.aclsparseSpMMGetBufferSize(*spmm_args(osa, handle, A, B, C), None) == INV
+    assert run(handle, None, B, C) == HN and run(handle, A, None, C) == HN and run(handle, A, B, None) == HN
+    assert run(handle, A, B, C, opa=1) == NS and run(handle, A, B, C, opb=2) == NS
+    assert run(handle, A, B, C, alg=7) == NS
+    assert run(handle, A, B, C, ct=osa.ACL_INT32) == NS                     # no (f32, f32, f32, i32) kernel
+    for kw in (dict(base=1), dict(ptr=1, idx=1), dict(idx=1)):
+        _, bad = make_csr(osa, L, rows=4, cols=3, nnz=5, **kw)
+        assert run(handle, bad, B, C) == NS, kw
+        L.aclsparseDestroySpMat(bad)
+    _, Bh = make_mat(osa, L, rows=3, cols=2, ld=2, vt=osa.ACL_FLOAT16)
+    assert run(handle, A, Bh, C) == NS                                       # mixed types
+    _, B4 = make_mat(osa, L, rows=4, cols=2, ld=2)
+    _, C3 = make_mat(osa, L, rows=4, cols=3, ld=3)
+    _, C5 = make_mat(osa, L, rows=5, cols=2, ld=2)
+    assert run(handle, A, B4, C) == INV and run(handle, A, B, C3) == INV and run(handle, A, B, C5) == INV
+    # buffer and handle are checked after the descriptors, in this order
+    assert L.aclsparseSpMM(*spmm_args(osa, handle, A, B, C), None) == st(osa, "INSUFFICIENT_RESOURCES")
+    assert L.aclsparseSpMM(*spmm_args(osa, None, A, B, C), None) == st(osa, "INSUFFICIENT_RESOURCES")
+    assert L.aclsparseSpMM(*spmm_args(osa, None, A, B, C), FAKE) == HN
+    assert L.aclsparseSpMMPreprocess(*spmm_args(osa, handle, A, B, C), None) == st(osa, "INSUFFICIENT_RESOURCES")
+    # a matrix this small cannot have a long row: 256-byte header, no device access
+    assert L.aclsparseSpMMGetBufferSize(*spmm_args(osa, None, A, B, C), ctypes.byref(n)) == 0 and n.value == 256
+    # Preprocess of an empty matrix is refused (reference spmm_csr_mat.cpp:148-150)
+    _, E = make_csr(osa, L, rows=0, cols=3, nnz=0)
+    _, C0 = make_mat(osa, L, rows=1, cols=2, ld=2)
+    assert L.aclsparseSpMMPreprocess(*spmm_args(osa, handle, E, B, C0), FAKE) == INV  # rows mismatch first
+    for d in (B, C, Bh, B4, C3, C5, C0):
+        L.aclsparseDestroyDnMat(d)
+    L.aclsparseDestroySpMat(A)
+    L.aclsparseDestroySpMat(E)
+
+
+def test_raw_layer_argument_checks(osa, L):
+    plan = osa.OpsparseSpmvPlan()
+    assert L.opsparse_spmv_csr_analyse(FAKE, -1, 1, 1, FAKE, 1 << 20, 0, ctypes.byref(plan), None) == -1
+    assert L.opsparse_spmv_csr_analyse(FAKE, 10, 10, 20, None, 0, 0, ctypes.byref(plan), None) == -3
+    assert L.opsparse_spmv_csr_analyse(FAKE, 10, 10, 0, None, 0, 0, ctypes.byref(plan), None) == 0
+    assert plan.kernel == osa.OPSPARSE_SPMV_SCALE_ONLY
+    s = osa.OpsparseScalar(1.0, None, 0, 0)
+    assert L.opsparse_spmv_csr_launch(None, 0, FAKE, FAKE, FAKE, FAKE, FAKE, 0, 5, 0, s, s, 0, 0, 0, None, 0, None) == 0
+    assert L.opsparse_spmv_csr_launch(None, 0, FAKE, FAKE, FAKE, FAKE, None, 3, 5, 2, s, s, 0, 0, 0, None, 0, None) == -1
+    assert L.opsparse_spmv_csr_workspace_bytes(-1, 0) == 0
+    n = ctypes.c_size_t(0)
+    assert L.opsparse_spmm_csr_workspace_bytes(FAKE, 10, 20, 4, None, None) == -1
+    assert L.opsparse_spmm_csr_workspace_bytes(FAKE, 10, 20, 4, None, ctypes.byref(n)) == 0 and n.value == 256
+    mp = osa.OpsparseSpmmPlan()
+    assert L.opsparse_spmm_csr_analyse(FAKE, 10, 20, 4, None, 0, 0, ctypes.byref(mp), None) == -3
+    assert L.opsparse_spmm_csr_launch(None, FAKE, FAKE, FAKE, FAKE, FAKE, 0, 3, 4, 0, 4, 4, 0, 0, 0, s, s, 0, 0, None,
+                                      0, None) == 0
+    assert L.opsparse_spmm_csr_launch(None, FAKE, FAKE, FAKE, FAKE, FAKE, 2, 3, 4, 5, 0, 4, 0, 0, 0, s, s, 0, 0, None,
+                                      0, None) == -1
+    assert L.opsparse_copy_launch(FAKE, FAKE, 17, None) == -1 and L.opsparse_copy_launch(FAKE, FAKE, 0, None) == 0
