@@ -42,23 +42,59 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def measure_copy_gbps(osa, torch, dev, stream, nbytes=1 << 30, reps=10):
-    """Practical HBM peak: device-to-device copy of >= 1 GiB, (read + write) / t."""
+def _time_launches(torch, stream, launch, reps):
+    for _ in range(2):
+        launch()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(reps):
+        launch()
+    e1.record(stream)
+    stream.synchronize()
+    return e0.elapsed_time(e1) / reps * 1e-3
+
+
+def measure_yardsticks(osa, torch, dev, stream, nbytes=1 << 30, reps=10):
+    """Practical HBM peaks of this GPU: a >= 1 GiB device-to-device copy, (read + write) / t,
+    and a read-only pass over the same buffer."""
     src = torch.empty(nbytes, dtype=torch.uint8, device=dev).zero_()
     dst = torch.empty(nbytes, dtype=torch.uint8, device=dev)
     L = osa.lib()
     sp = ctypes.c_void_p(stream.cuda_stream)
     torch.cuda.synchronize()
-    for _ in range(2):
-        L.opsparse_copy_launch(src.data_ptr(), dst.data_ptr(), nbytes, sp)
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record(stream)
-    for _ in range(reps):
-        L.opsparse_copy_launch(src.data_ptr(), dst.data_ptr(), nbytes, sp)
-    e1.record(stream)
-    stream.synchronize()
-    ms = e0.elapsed_time(e1) / reps
-    return 2.0 * nbytes / (ms * 1e-3) / 1e9
+    t_copy = _time_launches(torch, stream, lambda: L.opsparse_copy_launch(src.data_ptr(), dst.data_ptr(), nbytes, sp),
+                            reps)
+    t_read = _time_launches(torch, stream, lambda: L.opsparse_read_launch(src.data_ptr(), nbytes, None, sp), reps)
+    return 2.0 * nbytes / t_copy / 1e9, nbytes / t_read / 1e9
+
+
+def measure_gather(osa, torch, wl, dev, stream, count=1 << 26):
+    """Random 4-byte gathers per second from vectors of 4 MiB, 32 MiB and 256 MiB."""
+    L = osa.lib()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    out = {}
+    for mib in (4, 32, 256):
+        nx = mib << 18
+        x = torch.zeros(nx, dtype=torch.float32, device=dev)
+        idx = (wl._lsr(wl.hash64(77, torch.arange(count, dtype=torch.int64, device=dev)), 11) % nx).to(torch.int32)
+        torch.cuda.synchronize()
+        t = _time_launches(torch, stream, lambda: L.opsparse_gather_launch(idx.data_ptr(), x.data_ptr(), count, None,
+                                                                           sp), 5)
+        out["x_%dMiB" % mib] = round(count / t / 1e9, 2)
+    return out
+
+
+def load_traffic(name):
+    """Measured HBM traffic per launch for a workload, from the committed rocprof summary."""
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        table = json.load(f)
+    entry = table.get("workloads", {}).get(name)
+    if entry is None:
+        return None
+    return int(entry["fetch_kib"] * 1024 * table["fetch_scale"] + entry["write_kib"] * 1024 * table["write_scale"])
 
 
 def cpu_baseline_spmv(cfg, budget_s=15.0):
@@ -110,6 +146,7 @@ def main():
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-preprocess", action="store_true", help="SpMV without the Preprocess buffer")
+    ap.add_argument("--gather-probe", action="store_true", help="also measure random-gather rates (stderr)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -186,9 +223,12 @@ def main():
     flops = 2.0 * nnz * ncols
     gflops = flops / (ms * 1e-3) / 1e9
     gbps = bytes_alg / (ms * 1e-3) / 1e9
-    copy_gbps = measure_copy_gbps(osa, torch, dev, stream)
-    log("%.2f us/step (wall %.2f us), %.1f GFLOP/s, %.1f GB/s algorithmic = %.1f%% of 8 TB/s; copy kernel %.0f GB/s"
-        % (ms * 1e3, wall_ms * 1e3, gflops, gbps, 100 * gbps / HBM_PEAK_GBPS, copy_gbps))
+    copy_gbps, read_gbps = measure_yardsticks(osa, torch, dev, stream)
+    log("%.2f us/step (wall %.2f us), %.1f GFLOP/s, %.1f GB/s algorithmic = %.1f%% of 8 TB/s; "
+        "copy kernel %.0f GB/s, read kernel %.0f GB/s"
+        % (ms * 1e3, wall_ms * 1e3, gflops, gbps, 100 * gbps / HBM_PEAK_GBPS, copy_gbps, read_gbps))
+    if args.gather_probe:
+        log("random gathers, G/s: %s" % json.dumps(measure_gather(osa, torch, wl, dev, stream)))
 
     out = {
         "metric": "SpMV/SpMM GFLOP/s + achieved HBM GB/s (% of MI355X peak), CSR fp32",
@@ -199,9 +239,10 @@ def main():
                    "alpha": alpha, "beta": beta, "index": "int32", "preprocess_ms": round(preprocess_ms, 3),
                    "preprocessed": not args.no_preprocess},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                     "traffic": load_traffic(cfg["name"]) if args.scale == 1.0 else None,
                      "bytes_alg": bytes_alg, "bytes_gather_model": bytes_gather,
-                     "copy_kernel_gbps": round(copy_gbps, 1)},
+                     "copy_kernel_gbps": round(copy_gbps, 1), "read_kernel_gbps": round(read_gbps, 1)},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_spmm(cfg) if is_spmm else cpu_baseline_spmv(cfg)

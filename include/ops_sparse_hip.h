@@ -70,9 +70,8 @@ typedef struct OpsparseSpmvPlan {
     int32_t mergeBlocks;   /* MERGE_PATH: number of workgroups == partition entries - 1 */
     int32_t maxRowNnz;     /* longest row */
     int32_t partitionReady;/* MERGE_PATH: partition table already in the workspace */
-    int32_t waveSlots;     /* STREAM_ROWS: 0 = workgroup-tiled kernel; 8 or 16 = wavefront-tiled kernel for
-                              matrices whose longest row has at most that many non-zeros */
-    int32_t reserved;
+    int32_t reserved0;     /* unused, zero */
+    int32_t reserved1;
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */
@@ -168,6 +167,17 @@ int opsparse_spmm_csr_launch(const OpsparseSpmmPlan *plan, const int32_t *rowOff
  * bandwidth yard-stick and as the calibration kernel for the FETCH_SIZE /
  * WRITE_SIZE counters.  bytes must be a multiple of 16. */
 int opsparse_copy_launch(const void *src, void *dst, size_t bytes, void *stream);
+
+/* Reads `bytes` (a multiple of 16) once with non-temporal dwordx4 loads and
+ * writes nothing: the read-bandwidth ceiling of a streaming kernel.  `sink`
+ * (4 bytes, may be NULL) only keeps the loads alive. */
+int opsparse_read_launch(const void *src, size_t bytes, void *sink, void *stream);
+
+/* One independent 4-byte gather x[indices[i]] per index (indices streamed,
+ * results summed in registers): the rate at which this GPU serves random
+ * gathers from a vector of a given size, which bounds SpMV on matrices with
+ * scattered columns.  Indices must be valid positions in x or negative. */
+int opsparse_gather_launch(const int32_t *indices, const float *x, size_t count, void *sink, void *stream);
 
 #ifdef __cplusplus
 }

@@ -72,7 +72,7 @@ ACLSPARSE_SYMBOLS = [
 OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_workspace_bytes", "opsparse_spmv_csr_analyse", "opsparse_spmv_csr_launch",
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
-    "opsparse_copy_launch",
+    "opsparse_copy_launch", "opsparse_read_launch", "opsparse_gather_launch",
 ]
 
 vp = ctypes.c_void_p
@@ -87,7 +87,8 @@ class OpsparseScalar(ctypes.Structure):
 
 class OpsparseSpmvPlan(ctypes.Structure):
     _fields_ = [("kernel", i32), ("lanesPerRow", i32), ("rowsPerBlock", i32), ("mergeBlocks", i32),
-                ("maxRowNnz", i32), ("partitionReady", i32), ("waveSlots", i32), ("reserved", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
+                ("maxRowNnz", i32), ("partitionReady", i32), ("reserved0", i32),
+                ("reserved1", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
                 ("carryOff", i64), ("headOff", i64), ("bytes", i64)]
 
 
@@ -177,6 +178,10 @@ def lib():
                                            vp]
     L.opsparse_copy_launch.restype = ctypes.c_int
     L.opsparse_copy_launch.argtypes = [vp, vp, sz, vp]
+    L.opsparse_read_launch.restype = ctypes.c_int
+    L.opsparse_read_launch.argtypes = [vp, sz, vp, vp]
+    L.opsparse_gather_launch.restype = ctypes.c_int
+    L.opsparse_gather_launch.argtypes = [vp, vp, sz, vp, vp]
     _lib = L
     return L
 

@@ -29,6 +29,7 @@ SOURCES = [
     "spmm_host.cpp",
     "spmv_kernels.hip",
     "spmm_kernels.hip",
+    "measure_kernels.hip",
 ]
 
 # Packed fp32 VALU forms (v_pk_*_f32) are switched off for all device code.

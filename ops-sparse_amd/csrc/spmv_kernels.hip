@@ -584,19 +584,6 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvTransposeScatterKernel(
     }
 }
 
-// ------------------------------------------------------------- copy yard-stick
-
-typedef uint32_t Uint4V __attribute__((ext_vector_type(4)));
-
-__global__ __launch_bounds__(kBlockThreads) void CopyKernel(const Uint4V *__restrict__ src, Uint4V *__restrict__ dst,
-                                                            size_t n16)
-{
-    const size_t stride = static_cast<size_t>(gridDim.x) * kBlockThreads;
-    for (size_t i = static_cast<size_t>(blockIdx.x) * kBlockThreads + threadIdx.x; i < n16; i += stride) {
-        __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
-    }
-}
-
 // =============================================================== host side
 
 namespace {
@@ -1045,23 +1032,6 @@ int opsparse_spmv_csr_launch(const OpsparseSpmvPlan *plan, int32_t transpose, co
             break;
     }
     return OPSPARSE_E_UNSUPPORTED;
-}
-
-int opsparse_copy_launch(const void *src, void *dst, size_t bytes, void *stream)
-{
-    if (src == nullptr || dst == nullptr || bytes % 16 != 0) {
-        return OPSPARSE_E_INVALID;
-    }
-    if (bytes == 0) {
-        return OPSPARSE_OK;
-    }
-    const size_t n16 = bytes / 16;
-    size_t grid = (n16 + kBlockThreads - 1) / kBlockThreads;
-    grid = grid > 8192 ? 8192 : grid;
-    hipLaunchKernelGGL(CopyKernel, dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0,
-                       static_cast<hipStream_t>(stream), static_cast<const Uint4V *>(src), static_cast<Uint4V *>(dst),
-                       n16);
-    return CheckLaunch();
 }
 
 }  // extern "C"
