@@ -1,0 +1,152 @@
+"""GPU parity of the remaining aclsparseSpMV operand modes: element types, op(A) = A^T,
+device pointer mode.
+
+Tolerances: outputs in fp16 / bf16 are compared after rounding the oracle to the
+output type, allowing one unit in the last place of that type (2^-10 / 2^-7
+relative) — the reference's own bars are 2^-9 and 2^-6 (spmv_test.cpp:212-215);
+int32 is exact; the transposed product adds in fp32 with hardware atomics in
+unspecified order, like the reference, and is held to the reference's fp32 rule
+(|d| <= 2^-16 + 2^-10 |g| on >= 99 %, max |d| <= 1e-2)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import random_csr, run_spmv, to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _problem(rows, cols, density, seed, lo=-2.0, hi=2.0):
+    rowptr, colind, val = random_csr(rows, cols, density, seed, lo=lo, hi=hi, empty_row_prob=0.05)
+    rng = np.random.default_rng(seed + 1)
+    return rowptr, colind, val, rng.uniform(lo, hi, cols).astype(np.float32), rng.uniform(lo, hi, rows).astype(
+        np.float32)
+
+
+def _round(a, dtype):
+    return torch.from_numpy(a).to(dtype).float().numpy()
+
+
+@pytest.mark.parametrize("val_dtype,out_dtype,ulp", [(torch.float16, torch.float32, None),
+                                                     (torch.float16, torch.float16, 2.0 ** -10),
+                                                     (torch.bfloat16, torch.float32, None),
+                                                     (torch.bfloat16, torch.bfloat16, 2.0 ** -7)])
+@pytest.mark.parametrize("shape", [(600, 400, 0.02), (50, 3000, 0.3), (5000, 5000, 0.001)])
+def test_half_precision_inputs(osa, gpu_ctx, val_dtype, out_dtype, ulp, shape):
+    rows, cols, density = shape
+    rowptr, colind, val, x, y0 = _problem(rows, cols, density, 31)
+    val, x = _round(val, val_dtype), _round(x, val_dtype)          # the values the device really sees
+    y0 = _round(y0, out_dtype)
+    for pre in (True, False):
+        y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 1.5, 0.5, preprocess=pre,
+                     val_dtype=val_dtype, out_dtype=out_dtype)
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.5, 0.5)
+        if ulp is None:
+            assert oracle.max_rel_err(y, gold) <= 1e-5            # fp32 output: same bar as the fp32 path
+        else:
+            want = _round(gold, out_dtype)
+            assert np.all(np.abs(y - want) <= ulp * np.maximum(np.abs(want), 2.0 ** -14))
+
+
+def test_int32_exact(osa, gpu_ctx):
+    rows, cols = 700, 900
+    rowptr, colind, _ = random_csr(rows, cols, 0.03, 5)
+    rng = np.random.default_rng(6)
+    val = rng.integers(-50000, 50000, colind.size).astype(np.int32)
+    x = rng.integers(-50000, 50000, cols).astype(np.int32)
+    y0 = rng.integers(-1000, 1000, rows).astype(np.int32)
+    for pre in (True, False):
+        y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 3, -2, preprocess=pre,
+                     compute_type=osa.ACL_INT32)
+        assert np.array_equal(y, oracle.spmv_i32(rows, rowptr, colind, val, x, y0, 3, -2))   # wrap-around included
+
+
+def test_int32_values_float_output(osa, gpu_ctx):
+    rows, cols = 300, 300
+    rowptr, colind, _ = random_csr(rows, cols, 0.05, 8)
+    rng = np.random.default_rng(9)
+    val = rng.integers(-1000, 1000, colind.size).astype(np.int32)
+    x = rng.integers(-1000, 1000, cols).astype(np.int32)
+    y0 = rng.uniform(-1, 1, rows).astype(np.float32)
+    y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 0.5, 1.0)
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val.astype(np.float32), x.astype(np.float32), y0, 0.5, 1.0)
+    assert oracle.max_rel_err(y, gold) <= 1e-5
+
+
+@pytest.mark.parametrize("rows,cols,density", [(500, 300, 0.05), (64, 5000, 0.1), (3000, 40, 0.3), (1, 1, 1.0)])
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (2.0, 0.5), (1.0, 1.0), (0.0, 3.0)])
+def test_transpose(osa, gpu_ctx, rows, cols, density, alpha, beta):
+    rowptr, colind, val = random_csr(rows, cols, density, rows + cols)
+    rng = np.random.default_rng(4)
+    x = rng.uniform(-2, 2, rows).astype(np.float32)
+    y0 = rng.uniform(-2, 2, cols).astype(np.float32)
+    y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, alpha, beta,
+                 op=osa.ACL_SPARSE_OP_TRANSPOSE)
+    gold = oracle.spmv_trans_f64(rows, cols, rowptr, colind, val, x, y0, alpha, beta)
+    d = np.abs(y - gold)
+    assert (d <= 2.0 ** -16 + 2.0 ** -10 * np.abs(gold)).mean() >= 0.99 and d.max() <= 1e-2
+    g32 = oracle.spmv_trans_f32(rows, cols, rowptr, colind, val, x, y0, alpha, beta)
+    assert np.abs(y - g32).max() <= 1e-2
+
+
+def test_device_pointer_mode(osa, gpu_ctx):
+    """alpha / beta read by the kernel from device memory; changing them needs no new Preprocess."""
+    dev, stream, handle = gpu_ctx
+    rows, cols = 2000, 1500
+    rowptr, colind, val, x, y0 = _problem(rows, cols, 0.01, 77)
+    d_rowptr, d_colind, d_val = to_dev(rowptr, dev), to_dev(colind, dev), to_dev(val, dev)
+    d_x = to_dev(x, dev)
+    A = osa.Csr(rows, cols, d_rowptr, d_colind, d_val)
+    scal = torch.tensor([1.25, -0.75], dtype=torch.float32, device=dev)
+    L = osa.lib()
+    handle.set_pointer_mode(osa.ACL_SPARSE_POINTER_MODE_DEVICE)
+    try:
+        for buffered in (True, False):
+            d_y = to_dev(y0, dev)
+            X, Y = osa.DnVec(d_x), osa.DnVec(d_y)
+            op = osa.SpmvOp(handle, A, X, Y, preprocess=buffered)
+            buf = ctypes.c_void_p(op.buffer.data_ptr()) if buffered else None
+            for a, b in ((1.25, -0.75), (-2.0, 0.5)):
+                scal.copy_(torch.tensor([a, b]))
+                d_y.copy_(torch.from_numpy(y0))
+                torch.cuda.synchronize()
+                rc = L.aclsparseSpMV(handle.h, 0, ctypes.c_void_p(scal.data_ptr()), A.d, X.d,
+                                     ctypes.c_void_p(scal.data_ptr() + 4), Y.d, osa.ACL_FLOAT, 0, buf)
+                assert rc == 0
+                stream.synchronize()
+                gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, a, b)
+                assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+    finally:
+        handle.set_pointer_mode(osa.ACL_SPARSE_POINTER_MODE_HOST)
+
+
+def test_preprocessed_buffer_reused_and_rebound(osa, gpu_ctx):
+    """Same buffer for many calls and new values behind the same pattern; a foreign buffer is not trusted."""
+    dev, stream, handle = gpu_ctx
+    rows, cols = 4000, 4000
+    rowptr, colind, val, x, y0 = _problem(rows, cols, 0.002, 90)
+    d_val = to_dev(val, dev)
+    A = osa.Csr(rows, cols, to_dev(rowptr, dev), to_dev(colind, dev), d_val)
+    d_y = to_dev(y0, dev)
+    X, Y = osa.DnVec(to_dev(x, dev)), osa.DnVec(d_y)
+    op = osa.SpmvOp(handle, A, X, Y)
+    for scale in (1.0, 3.0):
+        d_val.copy_(torch.from_numpy(val * scale))             # aclsparseSpMatSetValues-style update in place
+        d_y.copy_(torch.from_numpy(y0))
+        torch.cuda.synchronize()
+        op(1.0, 1.0)
+        stream.synchronize()
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, (val * scale).astype(np.float32), x, y0, 1.0, 1.0)
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+    other = torch.zeros(op.buffer.numel(), dtype=torch.uint8, device=dev)   # never preprocessed
+    d_y.copy_(torch.from_numpy(y0))
+    torch.cuda.synchronize()
+    rc = osa.lib().aclsparseSpMV(handle.h, 0, None, A.d, X.d, None, Y.d, osa.ACL_FLOAT, 0,
+                                 ctypes.c_void_p(other.data_ptr()))
+    assert rc == 0
+    stream.synchronize()
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, (val * 3.0).astype(np.float32), x, y0, 1.0, 0.0)
+    assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
