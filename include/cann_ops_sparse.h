@@ -310,6 +310,49 @@ aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t o
                                 aclsparseConstDnMatDescr_t matB, const void *beta, aclsparseDnMatDescr_t matC,
                                 aclDataType computeType, aclsparseSpMMAlg_t alg, void *buffer);
 
+/* ------------------------------------------------------------------ SpMVOp
+ * [ref: include/cann_ops_sparse.h:1564-1637; host: sparse/spmv_op/arch35/spmv_op_host.cpp]
+ *
+ * Z = alpha * A * X + beta * Y with a descriptor / plan pair, fp32 only:
+ * opA = NON_TRANSPOSE, computeType ACL_FLOAT, CSR with fp32 values, 32-bit
+ * column indices, 32- or 64-bit row offsets, index base 0 or 1.  Z may be Y.
+ * Results are deterministic (fixed summation order, fp64 accumulator) for every
+ * algorithm value.
+ *
+ *   bufferSize    0 for ALG_DEFAULT / ALG1; for ALG2 the bytes of the
+ *                 nnz-balanced partition createDescr writes.
+ *   createDescr   snapshots matA's pointers and sizes (not its values: they may
+ *                 change between executions); ALG2 needs `buffer`, which must
+ *                 stay valid until destroyDescr.
+ *   createPlan    only the identity epilogue: a non-NULL LTO buffer or a
+ *                 non-zero size gives NOT_SUPPORTED.
+ *   destroy*      NULL is accepted and gives SUCCESS.
+ *   setGlobalUserData   checked and otherwise ignored (identity epilogue).
+ *   aclsparseSpMVOp     X, Y, Z must be fp32 vectors of exactly cols / rows /
+ *                 rows elements; Y's data may be NULL when beta is 0 (host
+ *                 pointer mode) or in device pointer mode.
+ */
+aclsparseStatus_t aclsparseSpMVOp_bufferSize(aclsparseHandle_t handle, aclsparseOperation_t opA,
+                                             aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX,
+                                             aclsparseConstDnVecDescr_t vecY, aclsparseDnVecDescr_t vecZ,
+                                             aclDataType computeType, aclsparseSpMVOpAlg_t alg, size_t *bufferSize);
+aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclsparseSpMVOpDescr_t *descr,
+                                              aclsparseOperation_t opA, aclsparseConstSpMatDescr_t matA,
+                                              aclsparseConstDnVecDescr_t vecX, aclsparseConstDnVecDescr_t vecY,
+                                              aclsparseDnVecDescr_t vecZ, aclDataType computeType,
+                                              aclsparseSpMVOpAlg_t alg, void *buffer);
+aclsparseStatus_t aclsparseSpMVOp_destroyDescr(aclsparseSpMVOpDescr_t descr);
+aclsparseStatus_t aclsparseSpMVOp_createPlan(aclsparseHandle_t handle, aclsparseSpMVOpDescr_t descr,
+                                             aclsparseSpMVOpPlan_t *plan, const void *epilogueLTOBuffer,
+                                             size_t epilogueLTOBufferSize);
+aclsparseStatus_t aclsparseSpMVOp_destroyPlan(aclsparseSpMVOpPlan_t plan);
+aclsparseStatus_t aclsparseSpMVOp_setGlobalUserData(aclsparseHandle_t handle, aclsparseSpMVOpPlan_t plan,
+                                                    const char *epilogueDataName, void *epilogueData,
+                                                    size_t epilogueDataSize);
+aclsparseStatus_t aclsparseSpMVOp(aclsparseHandle_t handle, aclsparseSpMVOpPlan_t plan, const void *alpha,
+                                  const void *beta, aclsparseConstDnVecDescr_t vecX, aclsparseConstDnVecDescr_t vecY,
+                                  aclsparseDnVecDescr_t vecZ);
+
 #ifdef __cplusplus
 }
 #endif

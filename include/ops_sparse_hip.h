@@ -105,6 +105,24 @@ int opsparse_spmv_csr_launch(const OpsparseSpmvPlan *plan, int32_t transpose, co
                              int32_t outType, int32_t computeIsInt, void *workspace, size_t workspaceBytes,
                              void *stream);
 
+/* Same as opsparse_spmv_csr_launch with separate input and output vectors:
+ * z = alpha * op(A) * x + beta * yIn.  z may be yIn (in place); yIn is only read
+ * when beta != 0 and may then be NULL otherwise. */
+int opsparse_spmv_csr_launch_zy(const OpsparseSpmvPlan *plan, int32_t transpose, const int32_t *rowOffsets,
+                                const int32_t *colInd, const void *csrValues, const void *x, const void *yIn, void *z,
+                                int64_t rows, int64_t cols, int64_t nnz, OpsparseScalar alpha, OpsparseScalar beta,
+                                int32_t valType, int32_t outType, int32_t computeIsInt, void *workspace,
+                                size_t workspaceBytes, void *stream);
+
+/* fp32 z = alpha * A * x + beta * yIn for the index variants of the SpMVOp API:
+ * int32 or int64 row offsets (rowOffsetsAre64), int32 column indices, index
+ * base 0 or 1 [ref: sparse/spmv_op/arch35/spmv_op_kernel.cpp:139-181].  One lane
+ * group per row, no workspace. */
+int opsparse_spmv_csr_indexed_launch(const void *rowOffsets, int32_t rowOffsetsAre64, int32_t indexBase,
+                                     const int32_t *colInd, const float *csrValues, const float *x,
+                                     const float *yIn, float *z, int64_t rows, int64_t cols, int64_t nnz,
+                                     OpsparseScalar alpha, OpsparseScalar beta, void *stream);
+
 /* ------------------------------------------------------------------ SpMM */
 
 typedef enum OpsparseSpmmKernel {

@@ -34,6 +34,8 @@ ACL_SPARSE_ORDER_ROW, ACL_SPARSE_ORDER_COL = 0, 1
 ACL_SPARSE_SPMM_ALG_DEFAULT, ACL_SPARSE_SPMM_CSR_ALG1, ACL_SPARSE_SPMM_CSR_FP32_HIGH_PRECISION_ALG = 0, 1, 2
 # ---- aclsparseSpMVAlg_t
 ACL_SPARSE_SPMV_ALG_DEFAULT, ACL_SPARSE_SPMV_COO_ALG1, ACL_SPARSE_SPMV_CSR_ALG1 = 0, 1, 3
+# ---- aclsparseSpMVOpAlg_t
+ACL_SPARSE_SPMVOP_ALG_DEFAULT, ACL_SPARSE_SPMVOP_ALG1, ACL_SPARSE_SPMVOP_ALG2 = 0, 1, 2
 # ---- aclsparseIndexType_t / aclsparseIndexBase_t / aclsparseFormat_t
 ACL_SPARSE_INDEX_32I, ACL_SPARSE_INDEX_64I = 0, 1
 ACL_SPARSE_INDEX_BASE_ZERO, ACL_SPARSE_INDEX_BASE_ONE = 0, 1
@@ -68,9 +70,13 @@ ACLSPARSE_SYMBOLS = [
     "aclsparseDnMatGet", "aclsparseConstDnMatGet", "aclsparseDnMatGetValues", "aclsparseConstDnMatGetValues",
     "aclsparseDnMatSetValues", "aclsparseSpMVGetBufferSize", "aclsparseSpMVPreprocess", "aclsparseSpMV",
     "aclsparseSpMMGetBufferSize", "aclsparseSpMMPreprocess", "aclsparseSpMM",
+    "aclsparseSpMVOp_bufferSize", "aclsparseSpMVOp_createDescr", "aclsparseSpMVOp_destroyDescr",
+    "aclsparseSpMVOp_createPlan", "aclsparseSpMVOp_destroyPlan", "aclsparseSpMVOp_setGlobalUserData",
+    "aclsparseSpMVOp",
 ]
 OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_workspace_bytes", "opsparse_spmv_csr_analyse", "opsparse_spmv_csr_launch",
+    "opsparse_spmv_csr_launch_zy", "opsparse_spmv_csr_indexed_launch",
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
     "opsparse_copy_launch", "opsparse_read_launch", "opsparse_gather_launch",
 ]
@@ -160,6 +166,14 @@ def lib():
     L.aclsparseSpMMGetBufferSize.argtypes = spmm_common + [ctypes.POINTER(sz)]
     L.aclsparseSpMMPreprocess.argtypes = spmm_common + [vp]
     L.aclsparseSpMM.argtypes = spmm_common + [vp]
+    spmvop_common = [vp, ctypes.c_int, vp, vp, vp, vp, ctypes.c_int, ctypes.c_int]
+    L.aclsparseSpMVOp_bufferSize.argtypes = spmvop_common + [ctypes.POINTER(sz)]
+    L.aclsparseSpMVOp_createDescr.argtypes = [vp, PV, ctypes.c_int, vp, vp, vp, vp, ctypes.c_int, ctypes.c_int, vp]
+    L.aclsparseSpMVOp_destroyDescr.argtypes = [vp]
+    L.aclsparseSpMVOp_createPlan.argtypes = [vp, vp, PV, vp, sz]
+    L.aclsparseSpMVOp_destroyPlan.argtypes = [vp]
+    L.aclsparseSpMVOp_setGlobalUserData.argtypes = [vp, vp, ctypes.c_char_p, vp, sz]
+    L.aclsparseSpMVOp.argtypes = [vp, vp, vp, vp, vp, vp, vp]
 
     L.opsparse_spmv_csr_workspace_bytes.restype = sz
     L.opsparse_spmv_csr_workspace_bytes.argtypes = [i64, i64]
@@ -168,6 +182,12 @@ def lib():
     L.opsparse_spmv_csr_launch.restype = ctypes.c_int
     L.opsparse_spmv_csr_launch.argtypes = [ctypes.POINTER(OpsparseSpmvPlan), i32, vp, vp, vp, vp, vp, i64, i64, i64,
                                            OpsparseScalar, OpsparseScalar, i32, i32, i32, vp, sz, vp]
+    L.opsparse_spmv_csr_launch_zy.restype = ctypes.c_int
+    L.opsparse_spmv_csr_launch_zy.argtypes = [ctypes.POINTER(OpsparseSpmvPlan), i32, vp, vp, vp, vp, vp, vp, i64, i64,
+                                              i64, OpsparseScalar, OpsparseScalar, i32, i32, i32, vp, sz, vp]
+    L.opsparse_spmv_csr_indexed_launch.restype = ctypes.c_int
+    L.opsparse_spmv_csr_indexed_launch.argtypes = [vp, i32, i32, vp, vp, vp, vp, vp, i64, i64, i64, OpsparseScalar,
+                                                   OpsparseScalar, vp]
     L.opsparse_spmm_csr_workspace_bytes.restype = ctypes.c_int
     L.opsparse_spmm_csr_workspace_bytes.argtypes = [vp, i64, i64, i64, vp, ctypes.POINTER(sz)]
     L.opsparse_spmm_csr_analyse.restype = ctypes.c_int
@@ -333,6 +353,57 @@ class SpmvOp:
         st = lib().aclsparseSpMV(self.handle.h, self.op, pa, self.A.d, self.x.d, pb, self.y.d, self.compute_type,
                                  self.alg, _ptr(self.buffer) if self.buffer is not None else vp(None))
         check(st, "aclsparseSpMV")
+
+
+class SpmvOpPlan:
+    """aclsparseSpMVOp_bufferSize -> createDescr -> createPlan, then z = alpha*A*x + beta*y per call.
+
+    x, y, z are DnVec objects; z may be y.  The descriptor, the plan and (ALG2) the
+    buffer live as long as this object.
+    """
+
+    def __init__(self, handle, A, x, y, z, alg=ACL_SPARSE_SPMVOP_ALG_DEFAULT):
+        import torch
+        self.handle, self.A, self.x, self.y, self.z, self.alg = handle, A, x, y, z, alg
+        self.descr, self.plan = vp(None), vp(None)
+        n = sz(0)
+        common = (ACL_SPARSE_OP_NON_TRANSPOSE, A.d, x.d, y.d, z.d, ACL_FLOAT, alg)
+        check(lib().aclsparseSpMVOp_bufferSize(handle.h, *common, ctypes.byref(n)), "aclsparseSpMVOp_bufferSize")
+        self.buffer_bytes = int(n.value)
+        self.buffer = None
+        if alg == ACL_SPARSE_SPMVOP_ALG2:
+            self.buffer = torch.empty(max(self.buffer_bytes, 16), dtype=torch.uint8, device=z.t.device)
+        check(lib().aclsparseSpMVOp_createDescr(handle.h, ctypes.byref(self.descr), *common,
+                                                _ptr(self.buffer) if self.buffer is not None else vp(None)),
+              "aclsparseSpMVOp_createDescr")
+        check(lib().aclsparseSpMVOp_createPlan(handle.h, self.descr, ctypes.byref(self.plan), None, 0),
+              "aclsparseSpMVOp_createPlan")
+
+    def __call__(self, alpha=1.0, beta=0.0, x=None, y=None, z=None):
+        """alpha / beta: Python numbers (HOST pointer mode) or one-element fp32 device tensors (DEVICE mode)."""
+        if hasattr(alpha, "data_ptr"):
+            pa, pb = vp(alpha.data_ptr()), vp(beta.data_ptr())
+        else:
+            ka, pa = _scalar_ref(alpha, ACL_FLOAT)
+            kb, pb = _scalar_ref(beta, ACL_FLOAT)
+        st = lib().aclsparseSpMVOp(self.handle.h, self.plan, pa, pb, (x or self.x).d, (y or self.y).d,
+                                   (z or self.z).d)
+        check(st, "aclsparseSpMVOp")
+
+    def close(self):
+        # plan first: it only borrows the descriptor
+        if self.plan:
+            lib().aclsparseSpMVOp_destroyPlan(self.plan)
+            self.plan = vp(None)
+        if self.descr:
+            lib().aclsparseSpMVOp_destroyDescr(self.descr)
+            self.descr = vp(None)
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
 
 
 class SpmmOp:

@@ -26,6 +26,7 @@ SOURCES = [
     "handle.cpp",
     "descr.cpp",
     "spmv_host.cpp",
+    "spmv_op_host.cpp",
     "spmm_host.cpp",
     "spmv_kernels.hip",
     "spmm_kernels.hip",

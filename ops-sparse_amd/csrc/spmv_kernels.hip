@@ -33,12 +33,12 @@ namespace opsparse {
 // ------------------------------------------------------------- epilogue
 
 template <typename OutT, typename AccT>
-__device__ __forceinline__ void StoreRow(OutT *__restrict__ y, int64_t row, AccT sum, AccT alpha, AccT beta,
+__device__ __forceinline__ void StoreRow(OutT *y, const OutT *yIn, int64_t row, AccT sum, AccT alpha, AccT beta,
                                          bool betaZero)
 {
     AccT r = alpha * sum;
     if (!betaZero) {
-        r += beta * ToAcc<AccT>(y[row]);
+        r += beta * ToAcc<AccT>(yIn[row]);
     }
     y[row] = FromAcc<OutT>(r);
 }
@@ -65,14 +65,14 @@ __device__ __forceinline__ void LoadVals4<double, float>(const float *p, double 
 // ------------------------------------------------------------- y = beta * y
 
 template <typename OutT, typename AccT>
-__global__ __launch_bounds__(kBlockThreads) void SpmvScaleKernel(OutT *__restrict__ y, int64_t len,
+__global__ __launch_bounds__(kBlockThreads) void SpmvScaleKernel(OutT *y, const OutT *yIn, int64_t len,
                                                                  OpsparseScalar betaS)
 {
     const AccT beta = ReadScalar<AccT>(betaS);
     const bool betaZero = (beta == AccT(0));
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlockThreads;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; i < len; i += stride) {
-        y[i] = betaZero ? FromAcc<OutT>(AccT(0)) : FromAcc<OutT>(beta * ToAcc<AccT>(y[i]));
+        y[i] = betaZero ? FromAcc<OutT>(AccT(0)) : FromAcc<OutT>(beta * ToAcc<AccT>(yIn[i]));
     }
 }
 
@@ -182,7 +182,7 @@ __device__ __forceinline__ void FinishQuads(const Quad<ValT> (&q)[U], const ValT
 template <typename ValT, typename OutT, typename AccT, int G, int U>
 __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
-    const ValT *__restrict__ x, OutT *__restrict__ y, int64_t rows, int32_t rowsPerBlock, OpsparseScalar alphaS,
+    const ValT *__restrict__ x, OutT *y, const OutT *yIn, int64_t rows, int32_t rowsPerBlock, OpsparseScalar alphaS,
     OpsparseScalar betaS)
 {
     extern __shared__ __align__(16) unsigned char ldsRaw[];
@@ -224,7 +224,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
             s = rowOffsets[r];
             e = rowOffsets[r + 1];
             if (!betaZero && lane == 0) {
-                yOld = ToAcc<AccT>(y[r]);
+                yOld = ToAcc<AccT>(yIn[r]);
             }
         }
         // Bounds of the next tile (scalar loads, needed after the barrier).
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
                 sNext = rowOffsets[rNext];
                 eNext = rowOffsets[rNext + 1];
                 if (!betaZero && lane == 0) {
-                    yNext = ToAcc<AccT>(y[rNext]);
+                    yNext = ToAcc<AccT>(yIn[rNext]);
                 }
             }
             AccT sum = AccT(0);
@@ -294,7 +294,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
 template <typename ValT, typename AccT, int U>
 __global__ __launch_bounds__(kBlockThreads) void SpmvStreamQuadRowsKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
-    const ValT *__restrict__ x, float *__restrict__ y, int64_t rows, int32_t rowsPerBlock, OpsparseScalar alphaS,
+    const ValT *__restrict__ x, float *y, const float *yIn, int64_t rows, int32_t rowsPerBlock, OpsparseScalar alphaS,
     OpsparseScalar betaS)
 {
     typedef int32_t Int4A __attribute__((ext_vector_type(4)));
@@ -325,7 +325,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamQuadRowsKernel(
         bound[3] = b.w;
         bound[4] = rowOffsets[r + 4];
         if (!betaZero) {
-            const Float4A o = *reinterpret_cast<const Float4A *>(y + r);
+            const Float4A o = *reinterpret_cast<const Float4A *>(yIn + r);
             yOld[0] = o.x;
             yOld[1] = o.y;
             yOld[2] = o.z;
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamQuadRowsKernel(
             bound[i] = rowOffsets[r + i];
             bound[i + 1] = rowOffsets[r + i + 1];
             if (!betaZero) {
-                yOld[i] = y[r + i];
+                yOld[i] = yIn[r + i];
             }
         }
     }
@@ -382,7 +382,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamQuadRowsKernel(
 template <typename ValT, typename OutT, typename AccT, int G>
 __global__ __launch_bounds__(kBlockThreads) void SpmvVectorRowsKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
-    const ValT *__restrict__ x, OutT *__restrict__ y, int64_t rows, OpsparseScalar alphaS, OpsparseScalar betaS)
+    const ValT *__restrict__ x, OutT *y, const OutT *yIn, int64_t rows, OpsparseScalar alphaS, OpsparseScalar betaS)
 {
     const AccT alpha = ReadScalar<AccT>(alphaS);
     const AccT beta = ReadScalar<AccT>(betaS);
@@ -412,7 +412,38 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvVectorRowsKernel(
     }
     const AccT sum = GroupSum<G>(sum0 + sum1);
     if (lane == 0) {
-        StoreRow<OutT, AccT>(y, r, sum, alpha, beta, betaZero);
+        StoreRow<OutT, AccT>(y, yIn, r, sum, alpha, beta, betaZero);
+    }
+}
+
+// The same lane-group-per-row scheme for the index variants the SpMVOp API
+// admits and the kernels above do not: 64-bit row offsets and / or index base 1
+// (reference sparse/spmv_op/arch35/spmv_op_kernel.cpp:139-181 handles them in its
+// one thread-per-row kernel).
+template <typename RowT, typename ValT, typename OutT, typename AccT, int G>
+__global__ __launch_bounds__(kBlockThreads) void SpmvIndexedRowsKernel(
+    const RowT *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ x, OutT *y, const OutT *yIn, int64_t rows, int32_t indexBase, OpsparseScalar alphaS,
+    OpsparseScalar betaS)
+{
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    const AccT beta = ReadScalar<AccT>(betaS);
+    const bool betaZero = (beta == AccT(0));
+    constexpr int kGroups = kBlockThreads / G;
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * kGroups + threadIdx.x / G;
+    const int32_t lane = threadIdx.x % G;
+    if (r >= rows) {
+        return;
+    }
+    const int64_t s = static_cast<int64_t>(rowOffsets[r]) - indexBase;
+    const int64_t e = static_cast<int64_t>(rowOffsets[r + 1]) - indexBase;
+    AccT sum = AccT(0);
+    for (int64_t k = s + lane; k < e; k += G) {
+        sum += ToAcc<AccT>(LoadStream(vals + k)) * ToAcc<AccT>(x[LoadStream(colInd + k) - indexBase]);
+    }
+    sum = GroupSum<G>(sum);
+    if (lane == 0) {
+        StoreRow<OutT, AccT>(y, yIn, r, sum, alpha, beta, betaZero);
     }
 }
 
@@ -461,7 +492,7 @@ __global__ __launch_bounds__(kBlockThreads) void MergePartitionKernel(const int3
 template <typename ValT, typename OutT, typename AccT>
 __global__ __launch_bounds__(kBlockThreads) void SpmvMergeKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
-    const ValT *__restrict__ x, OutT *__restrict__ y, int64_t rows, int64_t nnz,
+    const ValT *__restrict__ x, OutT *y, const OutT *yIn, int64_t rows, int64_t nnz,
     const int32_t *__restrict__ part, AccT *__restrict__ carry, AccT *__restrict__ head, OpsparseScalar alphaS,
     OpsparseScalar betaS)
 {
@@ -514,7 +545,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvMergeKernel(
             } else if (begin < j0) {
                 head[b] = sum;
             } else {
-                StoreRow<OutT, AccT>(y, row, sum, alpha, beta, betaZero);
+                StoreRow<OutT, AccT>(y, yIn, row, sum, alpha, beta, betaZero);
             }
         }
     }
@@ -525,7 +556,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvMergeKernel(
 // ascending order) to its head piece and write the row's final value.
 template <typename OutT, typename AccT>
 __global__ __launch_bounds__(kBlockThreads) void SpmvMergeFixupKernel(
-    const int32_t *__restrict__ rowOffsets, OutT *__restrict__ y, int64_t rows, int64_t nnz, int32_t numBlocks,
+    const int32_t *__restrict__ rowOffsets, OutT *y, const OutT *yIn, int64_t rows, int64_t nnz, int32_t numBlocks,
     const int32_t *__restrict__ part, const AccT *__restrict__ carry, const AccT *__restrict__ head,
     OpsparseScalar alphaS, OpsparseScalar betaS)
 {
@@ -554,7 +585,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvMergeFixupKernel(
     sum += head[b];
     const AccT alpha = ReadScalar<AccT>(alphaS);
     const AccT beta = ReadScalar<AccT>(betaS);
-    StoreRow<OutT, AccT>(y, i0, sum, alpha, beta, beta == AccT(0));
+    StoreRow<OutT, AccT>(y, yIn, i0, sum, alpha, beta, beta == AccT(0));
 }
 
 // ------------------------------------------------------------- op(A) = A^T
@@ -594,6 +625,7 @@ struct SpmvArgs {
     const void *vals;
     const void *x;
     void *y;
+    const void *yIn;  // old y (may be y itself)
     int64_t rows, cols, nnz;
     OpsparseScalar alpha, beta;
     void *ws;
@@ -667,7 +699,7 @@ int LaunchStreamU(const SpmvArgs &a, int32_t rowsPerBlock, size_t lds)
     const uint32_t grid = tiles < resident ? tiles : resident;
     hipLaunchKernelGGL((SpmvStreamRowsKernel<ValT, OutT, AccT, G, U>), dim3(grid), dim3(kBlockThreads), lds, a.stream,
                        a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
-                       static_cast<OutT *>(a.y), a.rows, rowsPerBlock, a.alpha, a.beta);
+                       static_cast<OutT *>(a.y), static_cast<const OutT *>(a.yIn), a.rows, rowsPerBlock, a.alpha, a.beta);
     return CheckLaunch();
 }
 
@@ -681,13 +713,15 @@ int LaunchStream(const SpmvArgs &a, int32_t rowsPerBlock, int32_t maxRowNnz)
         // Four rows per lane with vector row offsets / y where the shapes allow it.
         static const bool quadOff = std::getenv("OPS_SPARSE_STREAM_NO_QUAD_ROWS") != nullptr;
         if (!quadOff && rowsPerBlock % 4 == 0 && rowsPerBlock <= 4 * kBlockThreads &&
-            reinterpret_cast<uintptr_t>(a.rowOffsets) % 16 == 0 && reinterpret_cast<uintptr_t>(a.y) % 16 == 0) {
+            reinterpret_cast<uintptr_t>(a.rowOffsets) % 16 == 0 && reinterpret_cast<uintptr_t>(a.y) % 16 == 0 &&
+            reinterpret_cast<uintptr_t>(a.yIn) % 16 == 0) {
             const uint32_t grid = GridFor(a.rows, rowsPerBlock);
             auto launch = [&](auto tag) {
                 constexpr int U = decltype(tag)::value;
                 hipLaunchKernelGGL((SpmvStreamQuadRowsKernel<ValT, AccT, U>), dim3(grid), dim3(kBlockThreads), lds,
                                    a.stream, a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
-                                   static_cast<const ValT *>(a.x), static_cast<float *>(a.y), a.rows, rowsPerBlock,
+                                   static_cast<const ValT *>(a.x), static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.rows,
+                                   rowsPerBlock,
                                    a.alpha, a.beta);
             };
             if (products <= kBlockThreads * 4) {
@@ -711,7 +745,7 @@ int LaunchVector(const SpmvArgs &a)
     const uint32_t grid = GridFor(a.rows, kBlockThreads / G);
     hipLaunchKernelGGL((SpmvVectorRowsKernel<ValT, OutT, AccT, G>), dim3(grid), dim3(kBlockThreads), 0, a.stream,
                        a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
-                       static_cast<OutT *>(a.y), a.rows, a.alpha, a.beta);
+                       static_cast<OutT *>(a.y), static_cast<const OutT *>(a.yIn), a.rows, a.alpha, a.beta);
     return CheckLaunch();
 }
 
@@ -729,15 +763,15 @@ int LaunchMerge(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
     }
     hipLaunchKernelGGL((SpmvMergeKernel<ValT, OutT, AccT>), dim3(nb), dim3(kBlockThreads), 0, a.stream, a.rowOffsets,
                        a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
-                       static_cast<OutT *>(a.y), a.rows, a.nnz, part, carry, head, a.alpha, a.beta);
+                       static_cast<OutT *>(a.y), static_cast<const OutT *>(a.yIn), a.rows, a.nnz, part, carry, head, a.alpha, a.beta);
     hipLaunchKernelGGL((SpmvMergeFixupKernel<OutT, AccT>), dim3(GridFor(nb, kBlockThreads)), dim3(kBlockThreads), 0,
-                       a.stream, a.rowOffsets, static_cast<OutT *>(a.y), a.rows, a.nnz, nb, part, carry, head,
+                       a.stream, a.rowOffsets, static_cast<OutT *>(a.y), static_cast<const OutT *>(a.yIn), a.rows, a.nnz, nb, part, carry, head,
                        a.alpha, a.beta);
     return CheckLaunch();
 }
 
 template <typename OutT, typename AccT>
-int LaunchScale(OutT *y, int64_t len, OpsparseScalar beta, hipStream_t stream)
+int LaunchScale(OutT *y, const OutT *yIn, int64_t len, OpsparseScalar beta, hipStream_t stream)
 {
     if (len <= 0) {
         return OPSPARSE_OK;
@@ -745,7 +779,7 @@ int LaunchScale(OutT *y, int64_t len, OpsparseScalar beta, hipStream_t stream)
     int64_t grid = (len + kBlockThreads - 1) / kBlockThreads;
     grid = grid > 65536 ? 65536 : grid;
     hipLaunchKernelGGL((SpmvScaleKernel<OutT, AccT>), dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0,
-                       stream, y, len, beta);
+                       stream, y, yIn, len, beta);
     return CheckLaunch();
 }
 
@@ -754,7 +788,8 @@ int RunPlanned(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
 {
     switch (plan.kernel) {
         case OPSPARSE_SPMV_SCALE_ONLY:
-            return LaunchScale<OutT, AccT>(static_cast<OutT *>(a.y), a.rows, a.beta, a.stream);
+            return LaunchScale<OutT, AccT>(static_cast<OutT *>(a.y), static_cast<const OutT *>(a.yIn), a.rows, a.beta,
+                                           a.stream);
         case OPSPARSE_SPMV_STREAM_ROWS:
             switch (plan.lanesPerRow) {
                 case 1: return LaunchStream<ValT, OutT, AccT, 1>(a, plan.rowsPerBlock, plan.maxRowNnz);
@@ -826,7 +861,8 @@ int RunTranspose(const SpmvArgs &a, int32_t outType)
         return OPSPARSE_E_UNSUPPORTED;
     }
     // y has `cols` elements for the transposed product.
-    int rc = LaunchScale<float, AccT>(static_cast<float *>(a.y), a.cols, a.beta, a.stream);
+    int rc = LaunchScale<float, AccT>(static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.cols, a.beta,
+                                      a.stream);
     if (rc != OPSPARSE_OK || a.nnz == 0 || a.rows == 0) {
         return rc;
     }
@@ -976,6 +1012,16 @@ int opsparse_spmv_csr_launch(const OpsparseSpmvPlan *plan, int32_t transpose, co
                              int32_t outType, int32_t computeIsInt, void *workspace, size_t workspaceBytes,
                              void *stream)
 {
+    return opsparse_spmv_csr_launch_zy(plan, transpose, rowOffsets, colInd, csrValues, x, y, y, rows, cols, nnz, alpha,
+                                       beta, valType, outType, computeIsInt, workspace, workspaceBytes, stream);
+}
+
+int opsparse_spmv_csr_launch_zy(const OpsparseSpmvPlan *plan, int32_t transpose, const int32_t *rowOffsets,
+                                const int32_t *colInd, const void *csrValues, const void *x, const void *yIn, void *y,
+                                int64_t rows, int64_t cols, int64_t nnz, OpsparseScalar alpha, OpsparseScalar beta,
+                                int32_t valType, int32_t outType, int32_t computeIsInt, void *workspace,
+                                size_t workspaceBytes, void *stream)
+{
     if (rows < 0 || cols < 0 || nnz < 0) {
         return OPSPARSE_E_INVALID;
     }
@@ -983,15 +1029,18 @@ int opsparse_spmv_csr_launch(const OpsparseSpmvPlan *plan, int32_t transpose, co
     if (outLen == 0) {
         return OPSPARSE_OK;  // nothing to write
     }
-    if (y == nullptr || (rows > 0 && rowOffsets == nullptr) ||
-        (nnz > 0 && (colInd == nullptr || csrValues == nullptr || x == nullptr))) {
+    if (y == nullptr ||
+        (nnz > 0 && (rowOffsets == nullptr || colInd == nullptr || csrValues == nullptr || x == nullptr))) {
         return OPSPARSE_E_INVALID;
     }
     if (plan != nullptr && (plan->rows != rows || plan->nnz != nnz)) {
         return OPSPARSE_E_INVALID;
     }
-    SpmvArgs a{rowOffsets, colInd,         csrValues, x, y, rows, cols, nnz, alpha, beta, workspace,
-               workspaceBytes, static_cast<hipStream_t>(stream)};
+    if (yIn == nullptr) {
+        yIn = y;  // only read when beta != 0
+    }
+    SpmvArgs a{rowOffsets, colInd, csrValues, x,         y,     yIn, rows, cols, nnz, alpha, beta,
+               workspace,  workspaceBytes, static_cast<hipStream_t>(stream)};
 
     if (transpose) {
         if (computeIsInt) {
@@ -1032,6 +1081,50 @@ int opsparse_spmv_csr_launch(const OpsparseSpmvPlan *plan, int32_t transpose, co
             break;
     }
     return OPSPARSE_E_UNSUPPORTED;
+}
+
+int opsparse_spmv_csr_indexed_launch(const void *rowOffsets, int32_t rowOffsetsAre64, int32_t indexBase,
+                                     const int32_t *colInd, const float *csrValues, const float *x,
+                                     const float *yIn, float *z, int64_t rows, int64_t cols, int64_t nnz,
+                                     OpsparseScalar alpha, OpsparseScalar beta, void *stream)
+{
+    if (rows < 0 || cols < 0 || nnz < 0 || (indexBase != 0 && indexBase != 1)) {
+        return OPSPARSE_E_INVALID;
+    }
+    if (rows == 0) {
+        return OPSPARSE_OK;
+    }
+    if (z == nullptr || rowOffsets == nullptr || (nnz > 0 && (colInd == nullptr || csrValues == nullptr || x == nullptr))) {
+        return OPSPARSE_E_INVALID;
+    }
+    if (yIn == nullptr) {
+        yIn = z;
+    }
+    auto s = static_cast<hipStream_t>(stream);
+    const int32_t g = VectorLanesFor(rows, nnz);
+    auto launch = [&](auto rowTag, auto gTag) {
+        using RowT = typename decltype(rowTag)::type;
+        constexpr int G = decltype(gTag)::value;
+        hipLaunchKernelGGL((SpmvIndexedRowsKernel<RowT, float, float, double, G>),
+                           dim3(GridFor(rows, kBlockThreads / G)), dim3(kBlockThreads), 0, s,
+                           static_cast<const RowT *>(rowOffsets), colInd, csrValues, x, z, yIn, rows, indexBase, alpha,
+                           beta);
+    };
+    auto byLanes = [&](auto rowTag) {
+        switch (g) {
+            case 4: launch(rowTag, std::integral_constant<int, 4>{}); break;
+            case 8: launch(rowTag, std::integral_constant<int, 8>{}); break;
+            case 16: launch(rowTag, std::integral_constant<int, 16>{}); break;
+            case 32: launch(rowTag, std::integral_constant<int, 32>{}); break;
+            default: launch(rowTag, std::integral_constant<int, 64>{}); break;
+        }
+    };
+    if (rowOffsetsAre64) {
+        byLanes(std::enable_if<true, int64_t>{});
+    } else {
+        byLanes(std::enable_if<true, int32_t>{});
+    }
+    return CheckLaunch();
 }
 
 }  // extern "C"

@@ -1,0 +1,311 @@
+// The aclsparseSpMVOp_* API: Z = alpha * A * X + beta * Y through a descriptor
+// and a plan object.
+//
+// Argument checks, their order and status codes follow the reference
+// (sparse/spmv_op/arch35/spmv_op_host.cpp: validation :64-297, bufferSize
+// :496-541, createDescr :603-647, createPlan :660-686, execute :726-746 with the
+// m == 0 / nnz == 0 short cuts of :465-486).  What differs is underneath: the
+// reference runs one thread per row with a compensated dot product and, for
+// ALG2, a device-side sort of the rows; here every algorithm value runs the
+// fp64-accumulating SpMV kernels, which are deterministic, and ALG2's buffer
+// holds the merge-path partition (the nnz-balanced split that ALG2 asks for).
+#include <climits>
+#include <new>
+
+#include "internal.h"
+
+// reference: sparse/common/aclsparse_descr_internal.h:139-158
+struct aclsparseSpMVOpDescr {
+    int64_t rows = 0;
+    int64_t cols = 0;
+    int64_t nnz = 0;
+    aclsparseIndexBase_t indexBase = ACL_SPARSE_INDEX_BASE_ZERO;
+    aclsparseIndexType_t rowOffsetsType = ACL_SPARSE_INDEX_32I;
+    void *rowOffsets = nullptr;  // borrowed, like the matrix descriptor's
+    void *colInd = nullptr;
+    void *values = nullptr;
+    aclsparseSpMVOpAlg_t alg = ACL_SPARSE_SPMVOP_ALG1;
+    void *userBuffer = nullptr;  // ALG2: caller's buffer holding the partition
+    bool planned = false;        // userBuffer was analysed successfully
+    OpsparseSpmvPlan plan{};
+};
+
+struct aclsparseSpMVOpPlan {
+    aclsparseSpMVOpDescr *descr = nullptr;
+};
+
+namespace {
+
+aclsparseStatus_t ValidateMatrix(aclsparseConstSpMatDescr_t matA)
+{
+    if (matA == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if (matA->format != ACL_SPARSE_FORMAT_CSR || matA->valueType != ACL_FLOAT) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    // row offsets may be 32 or 64 bit, column indices must be 32 bit
+    if (matA->colIndType != ACL_SPARSE_INDEX_32I) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    if (matA->rowOffsetsType != ACL_SPARSE_INDEX_32I && matA->rowOffsetsType != ACL_SPARSE_INDEX_64I) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t ValidateCommon(aclsparseOperation_t opA, aclDataType computeType)
+{
+    if (opA != ACL_SPARSE_OP_NON_TRANSPOSE || computeType != ACL_FLOAT) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t ValidateAlg(aclsparseSpMVOpAlg_t alg)
+{
+    if (alg != ACL_SPARSE_SPMVOP_ALG_DEFAULT && alg != ACL_SPARSE_SPMVOP_ALG1 && alg != ACL_SPARSE_SPMVOP_ALG2) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+// The optimised kernels take 32-bit zero-based offsets; anything else goes to
+// the indexed-rows kernel.
+bool Plain(const aclsparseSpMVOpDescr *d)
+{
+    return d->rowOffsetsType == ACL_SPARSE_INDEX_32I && d->indexBase == ACL_SPARSE_INDEX_BASE_ZERO;
+}
+
+aclsparseStatus_t FromLaunch(int rc)
+{
+    switch (rc) {
+        case OPSPARSE_OK: return ACL_SPARSE_STATUS_SUCCESS;
+        case OPSPARSE_E_INVALID: return ACL_SPARSE_STATUS_INVALID_VALUE;
+        case OPSPARSE_E_UNSUPPORTED: return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+        case OPSPARSE_E_WORKSPACE: return ACL_SPARSE_STATUS_INSUFFICIENT_RESOURCES;
+        default: return ACL_SPARSE_STATUS_EXECUTION_FAILED;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+aclsparseStatus_t aclsparseSpMVOp_bufferSize(aclsparseHandle_t handle, aclsparseOperation_t opA,
+                                             aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t /*vecX*/,
+                                             aclsparseConstDnVecDescr_t /*vecY*/, aclsparseDnVecDescr_t /*vecZ*/,
+                                             aclDataType computeType, aclsparseSpMVOpAlg_t alg, size_t *bufferSize)
+{
+    if (handle == nullptr) {
+        return ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR;
+    }
+    aclsparseStatus_t st = ValidateCommon(opA, computeType);
+    if (st == ACL_SPARSE_STATUS_SUCCESS) {
+        st = ValidateMatrix(matA);
+    }
+    if (st == ACL_SPARSE_STATUS_SUCCESS) {
+        st = ValidateAlg(alg);
+    }
+    if (st != ACL_SPARSE_STATUS_SUCCESS) {
+        return st;
+    }
+    if (bufferSize == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if (matA->rows > INT32_MAX) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    // ALG1 / DEFAULT need no buffer; ALG2 keeps its partition in one.
+    *bufferSize = (alg == ACL_SPARSE_SPMVOP_ALG2) ? opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz) : 0;
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclsparseSpMVOpDescr_t *descr,
+                                              aclsparseOperation_t opA, aclsparseConstSpMatDescr_t matA,
+                                              aclsparseConstDnVecDescr_t /*vecX*/, aclsparseConstDnVecDescr_t /*vecY*/,
+                                              aclsparseDnVecDescr_t /*vecZ*/, aclDataType computeType,
+                                              aclsparseSpMVOpAlg_t alg, void *buffer)
+{
+    if (handle == nullptr) {
+        return ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR;
+    }
+    if (descr == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    aclsparseStatus_t st = ValidateMatrix(matA);
+    if (st == ACL_SPARSE_STATUS_SUCCESS) {
+        st = ValidateAlg(alg);
+    }
+    if (st != ACL_SPARSE_STATUS_SUCCESS) {
+        return st;
+    }
+    if (alg == ACL_SPARSE_SPMVOP_ALG2 && buffer == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    st = ValidateCommon(opA, computeType);
+    if (st != ACL_SPARSE_STATUS_SUCCESS) {
+        return st;
+    }
+    if (matA->rows > INT32_MAX) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    if (matA->idxBase != ACL_SPARSE_INDEX_BASE_ZERO && matA->idxBase != ACL_SPARSE_INDEX_BASE_ONE) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    auto *d = new (std::nothrow) aclsparseSpMVOpDescr();
+    if (d == nullptr) {
+        return ACL_SPARSE_STATUS_ALLOC_FAILED;
+    }
+    d->rows = matA->rows;
+    d->cols = matA->cols;
+    d->nnz = matA->nnz;
+    d->indexBase = matA->idxBase;
+    d->rowOffsetsType = matA->rowOffsetsType;
+    d->rowOffsets = matA->rowOffsets;
+    d->colInd = matA->colInd;
+    d->values = matA->values;
+    d->alg = (alg == ACL_SPARSE_SPMVOP_ALG_DEFAULT) ? ACL_SPARSE_SPMVOP_ALG1 : alg;
+    if (d->alg == ACL_SPARSE_SPMVOP_ALG2) {
+        d->userBuffer = buffer;
+        // The nnz-balanced split of ALG2: analyse the rows into the caller's buffer.
+        if (Plain(d) && d->rows > 0 && d->nnz > 0 && d->rowOffsets != nullptr) {
+            const int rc = opsparse_spmv_csr_analyse(static_cast<const int32_t *>(d->rowOffsets), d->rows, d->cols,
+                                                     d->nnz, buffer,
+                                                     opsparse_spmv_csr_workspace_bytes(d->rows, d->nnz),
+                                                     OPSPARSE_SPMV_AUTO, &d->plan, handle->stream);
+            if (rc != OPSPARSE_OK) {
+                delete d;
+                return FromLaunch(rc);
+            }
+            d->planned = true;
+        }
+    }
+    *descr = d;
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t aclsparseSpMVOp_destroyDescr(aclsparseSpMVOpDescr_t descr)
+{
+    delete descr;  // NULL is fine
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t aclsparseSpMVOp_createPlan(aclsparseHandle_t handle, aclsparseSpMVOpDescr_t descr,
+                                             aclsparseSpMVOpPlan_t *plan, const void *epilogueLTOBuffer,
+                                             size_t epilogueLTOBufferSize)
+{
+    if (handle == nullptr) {
+        return ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR;
+    }
+    if (descr == nullptr || plan == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    // Only the identity epilogue exists: a link-time-optimised one is refused.
+    if (epilogueLTOBuffer != nullptr || epilogueLTOBufferSize > 0) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    auto *p = new (std::nothrow) aclsparseSpMVOpPlan();
+    if (p == nullptr) {
+        return ACL_SPARSE_STATUS_ALLOC_FAILED;
+    }
+    p->descr = descr;
+    *plan = p;
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t aclsparseSpMVOp_destroyPlan(aclsparseSpMVOpPlan_t plan)
+{
+    delete plan;  // NULL is fine
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t aclsparseSpMVOp_setGlobalUserData(aclsparseHandle_t handle, aclsparseSpMVOpPlan_t plan,
+                                                    const char * /*epilogueDataName*/, void *epilogueData,
+                                                    size_t epilogueDataSize)
+{
+    if (handle == nullptr) {
+        return ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR;
+    }
+    if (plan == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if ((epilogueData == nullptr) != (epilogueDataSize == 0)) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    return ACL_SPARSE_STATUS_SUCCESS;  // the identity epilogue uses no data
+}
+
+aclsparseStatus_t aclsparseSpMVOp(aclsparseHandle_t handle, aclsparseSpMVOpPlan_t plan, const void *alpha,
+                                  const void *beta, aclsparseConstDnVecDescr_t vecX,
+                                  aclsparseConstDnVecDescr_t vecY, aclsparseDnVecDescr_t vecZ)
+{
+    if (handle == nullptr) {
+        return ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR;
+    }
+    if (plan == nullptr || plan->descr == nullptr || alpha == nullptr || beta == nullptr || vecX == nullptr ||
+        vecY == nullptr || vecZ == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    const aclsparseSpMVOpDescr *d = plan->descr;
+    if (vecX->valueType != ACL_FLOAT || vecY->valueType != ACL_FLOAT || vecZ->valueType != ACL_FLOAT) {
+        return ACL_SPARSE_STATUS_NOT_SUPPORTED;
+    }
+    if (d->cols > 0 && vecX->values == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    // Y may be absent when beta is known to be 0 on the host; in DEVICE mode the
+    // kernel's own beta == 0 short cut is trusted (spmv_op_host.cpp:256-268).
+    bool yMayBeNull = handle->pointerMode == ACL_SPARSE_POINTER_MODE_DEVICE;
+    if (handle->pointerMode == ACL_SPARSE_POINTER_MODE_HOST) {
+        yMayBeNull = (*static_cast<const float *>(beta) == 0.0f);
+    }
+    if (!yMayBeNull && d->rows > 0 && vecY->values == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if (d->rows > 0 && vecZ->values == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if (vecX->size != d->cols || vecY->size != d->rows || vecZ->size != d->rows) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if (d->rows == 0) {
+        return ACL_SPARSE_STATUS_SUCCESS;
+    }
+    const OpsparseScalar a = opsparse::MakeScalar(alpha, ACL_FLOAT, handle->pointerMode, 0.0);
+    const OpsparseScalar b = opsparse::MakeScalar(beta, ACL_FLOAT, handle->pointerMode, 0.0);
+    int rc;
+    if (Plain(d) || d->nnz == 0) {
+        const OpsparseSpmvPlan *p = d->planned ? &d->plan : nullptr;
+        void *ws = d->planned ? d->userBuffer : nullptr;
+        size_t wsBytes = d->planned ? static_cast<size_t>(d->plan.bytes) : 0;
+        if (p == nullptr && d->nnz > 0) {
+            const aclsparseStatus_t st = opsparse::EnsureWorkspace(handle);
+            if (st != ACL_SPARSE_STATUS_SUCCESS) {
+                return st;
+            }
+            ws = handle->workspace();
+            wsBytes = handle->workspaceBytes();
+        }
+        // nnz == 0 needs no offsets at all: Z = beta * Y whatever their width.
+        rc = opsparse_spmv_csr_launch_zy(p, 0, static_cast<const int32_t *>(d->nnz > 0 ? d->rowOffsets : nullptr),
+                                         static_cast<const int32_t *>(d->colInd), d->values, vecX->values,
+                                         vecY->values, vecZ->values, d->rows, d->cols, d->nnz, a, b, OPSPARSE_F32,
+                                         OPSPARSE_F32, 0, ws, wsBytes, handle->stream);
+    } else {
+        rc = opsparse_spmv_csr_indexed_launch(d->rowOffsets, d->rowOffsetsType == ACL_SPARSE_INDEX_64I ? 1 : 0,
+                                              d->indexBase == ACL_SPARSE_INDEX_BASE_ONE ? 1 : 0,
+                                              static_cast<const int32_t *>(d->colInd),
+                                              static_cast<const float *>(d->values),
+                                              static_cast<const float *>(vecX->values),
+                                              static_cast<const float *>(vecY->values),
+                                              static_cast<float *>(vecZ->values), d->rows, d->cols, d->nnz, a, b,
+                                              handle->stream);
+    }
+    if (rc != OPSPARSE_OK) {
+        opsparse::LogError("aclsparseSpMVOp: launch failed (%d)", rc);
+    }
+    return FromLaunch(rc);
+}
+
+}  // extern "C"

@@ -292,3 +292,108 @@ def test_raw_layer_argument_checks(osa, L):
     assert L.opsparse_spmm_csr_launch(None, FAKE, FAKE, FAKE, FAKE, FAKE, 2, 3, 4, 5, 0, 4, 0, 0, 0, s, s, 0, 0, None,
                                       0, None) == -1
     assert L.opsparse_copy_launch(FAKE, FAKE, 17, None) == -1 and L.opsparse_copy_launch(FAKE, FAKE, 0, None) == 0
+
+
+# ------------------------------------------------------------------- SpMVOp
+
+def test_spmvop_status_table(osa, L, handle):
+    """reference sparse/spmv_op/arch35/spmv_op_host.cpp:64-297 (checks), :496-541, :603-746 (entry points)."""
+    INV, NS, HN = st(osa, "INVALID_VALUE"), st(osa, "NOT_SUPPORTED"), st(osa, "HANDLE_IS_NULLPTR")
+    ALG1, ALG2 = osa.ACL_SPARSE_SPMVOP_ALG1, osa.ACL_SPARSE_SPMVOP_ALG2
+    F = osa.ACL_FLOAT
+    _, A = make_csr(osa, L)
+    _, x = make_vec(osa, L, 4)
+    _, y = make_vec(osa, L, 4)
+    _, z = make_vec(osa, L, 4)
+    n = ctypes.c_size_t(77)
+
+    # bufferSize: handle, (opA, computeType), matrix, alg, output pointer, in this order
+    size = lambda h, A_, op=0, ct=F, alg=0, out=ctypes.byref(n): L.aclsparseSpMVOp_bufferSize(h, op, A_, x, y, z, ct, alg, out)
+    assert size(None, A) == HN
+    assert size(handle, A, op=1) == NS and size(handle, A, ct=osa.ACL_FLOAT16) == NS
+    assert size(handle, None) == INV
+    assert size(handle, A, alg=3) == NS
+    assert size(handle, A, out=None) == INV
+    assert size(handle, None, op=1) == NS                       # opA is looked at before the matrix
+    assert size(handle, A) == 0 and n.value == 0
+    assert size(handle, A, alg=ALG1) == 0 and n.value == 0
+    assert size(handle, A, alg=ALG2) == 0 and n.value == L.opsparse_spmv_csr_workspace_bytes(4, 5)
+    _, big = make_csr(osa, L, rows=(1 << 31), cols=4, nnz=5)
+    assert size(handle, big) == NS
+    bad_mats = [dict(vt=osa.ACL_FLOAT16), dict(idx=1), dict(ptr=1, idx=1)]
+    for kw in bad_mats:
+        _, bad = make_csr(osa, L, **kw)
+        assert size(handle, bad) == NS, kw
+        L.aclsparseDestroySpMat(bad)
+    for kw in (dict(ptr=1), dict(base=1), dict(ptr=1, base=1)):       # 64-bit row offsets and base 1 are supported
+        _, ok = make_csr(osa, L, **kw)
+        assert size(handle, ok) == 0, kw
+        L.aclsparseDestroySpMat(ok)
+
+    # createDescr: handle, output pointer, matrix, alg, ALG2 buffer, (opA, computeType), rows
+    d = ctypes.c_void_p(None)
+    mk = lambda h, A_, op=0, ct=F, alg=0, buf=None, out=ctypes.byref(d): \
+        L.aclsparseSpMVOp_createDescr(h, out, op, A_, x, y, z, ct, alg, buf)
+    assert mk(None, A) == HN
+    assert mk(handle, A, out=None) == INV
+    assert mk(handle, None) == INV
+    assert mk(handle, A, alg=9) == NS
+    assert mk(handle, A, alg=ALG2, buf=None) == INV
+    assert mk(handle, A, alg=ALG2, buf=None, op=1) == INV        # the buffer check comes before opA
+    assert mk(handle, A, op=1) == NS and mk(handle, A, ct=osa.ACL_INT32) == NS
+    assert mk(handle, big) == NS
+    for kw in bad_mats:
+        _, bad = make_csr(osa, L, **kw)
+        assert mk(handle, bad) == NS, kw
+        L.aclsparseDestroySpMat(bad)
+    assert d.value is None                                          # nothing was created on the failing paths
+    assert mk(handle, A) == 0 and d.value
+
+    # createPlan
+    p = ctypes.c_void_p(None)
+    assert L.aclsparseSpMVOp_createPlan(None, d, ctypes.byref(p), None, 0) == HN
+    assert L.aclsparseSpMVOp_createPlan(handle, None, ctypes.byref(p), None, 0) == INV
+    assert L.aclsparseSpMVOp_createPlan(handle, d, None, None, 0) == INV
+    assert L.aclsparseSpMVOp_createPlan(handle, d, ctypes.byref(p), FAKE, 0) == NS
+    assert L.aclsparseSpMVOp_createPlan(handle, d, ctypes.byref(p), None, 8) == NS
+    assert p.value is None
+    assert L.aclsparseSpMVOp_createPlan(handle, d, ctypes.byref(p), None, 0) == 0 and p.value
+
+    # setGlobalUserData: accepted and ignored when consistent
+    sg = L.aclsparseSpMVOp_setGlobalUserData
+    assert sg(None, p, b"e", None, 0) == HN and sg(handle, None, b"e", None, 0) == INV
+    assert sg(handle, p, b"e", FAKE, 0) == INV and sg(handle, p, b"e", None, 4) == INV
+    assert sg(handle, p, b"e", None, 0) == 0 and sg(handle, p, None, FAKE, 4) == 0
+
+    # execute: handle, plan, alpha, beta, vectors, types, sizes
+    one, zero = ctypes.c_float(1.0), ctypes.c_float(0.0)
+    pa, pb = ctypes.cast(ctypes.pointer(one), ctypes.c_void_p), ctypes.cast(ctypes.pointer(zero), ctypes.c_void_p)
+    run = lambda h=handle, pl=p, a=pa, b=pb, X=x, Y=y, Z=z: L.aclsparseSpMVOp(h, pl, a, b, X, Y, Z)
+    assert run(h=None) == HN
+    assert run(pl=None) == INV and run(a=None) == INV and run(b=None) == INV
+    assert run(X=None) == INV and run(Y=None) == INV and run(Z=None) == INV
+    _, xh = make_vec(osa, L, 4, vt=osa.ACL_FLOAT16)
+    assert run(X=xh) == NS and run(Y=xh) == NS and run(Z=xh) == NS
+    _, v3 = make_vec(osa, L, 3)
+    _, v5 = make_vec(osa, L, 5)
+    for bad in (v3, v5):                                            # sizes must match exactly, longer is wrong too
+        assert run(X=bad) == INV and run(Y=bad) == INV and run(Z=bad) == INV
+    assert run(X=xh, Y=v3) == NS                                    # types are checked before sizes
+
+    # a matrix without rows executes to SUCCESS without touching the device
+    _, E = make_csr(osa, L, rows=0, cols=4, nnz=0, rp=NULL, ci=NULL, va=NULL)
+    de, pe = ctypes.c_void_p(None), ctypes.c_void_p(None)
+    _, v0 = make_vec(osa, L, 0, p=NULL)
+    assert L.aclsparseSpMVOp_createDescr(handle, ctypes.byref(de), 0, E, x, v0, v0, F, ALG2, FAKE) == 0
+    assert L.aclsparseSpMVOp_createPlan(handle, de, ctypes.byref(pe), None, 0) == 0
+    assert run(pl=pe, Y=v0, Z=v0) == 0
+    assert run(pl=pe, Y=y, Z=v0) == INV
+
+    # destroy: plan before descriptor; NULL is accepted
+    assert L.aclsparseSpMVOp_destroyPlan(pe) == 0 and L.aclsparseSpMVOp_destroyDescr(de) == 0
+    assert L.aclsparseSpMVOp_destroyPlan(p) == 0 and L.aclsparseSpMVOp_destroyDescr(d) == 0
+    assert L.aclsparseSpMVOp_destroyPlan(None) == 0 and L.aclsparseSpMVOp_destroyDescr(None) == 0
+    for v in (x, y, z, xh, v3, v5, v0):
+        L.aclsparseDestroyDnVec(v)
+    for m in (A, big, E):
+        L.aclsparseDestroySpMat(m)
