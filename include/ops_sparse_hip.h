@@ -127,7 +127,7 @@ int opsparse_spmv_csr_indexed_launch(const void *rowOffsets, int32_t rowOffsetsA
 
 typedef enum OpsparseSpmmKernel {
     OPSPARSE_SPMM_AUTO = 0,
-    OPSPARSE_SPMM_ROW_SPLIT = 1, /* every row by one lane group; B rows streamed coalesced */
+    OPSPARSE_SPMM_ROW_SPLIT = 1, /* no row above the long-row threshold: every row whole by one lane group */
     OPSPARSE_SPMM_BINNED = 2     /* rows up to the long-row threshold as ROW_SPLIT, longer rows cut into
                                     fixed nnz segments over several waves + a fix-up pass */
 } OpsparseSpmmKernel;
@@ -147,9 +147,8 @@ typedef struct OpsparseSpmmPlan {
     int64_t segStartOff;   /* int32 [numSegments]: first nnz of the segment */
     int64_t longFirstSegOff; /* int32 [numLongRows + 1]: first segment of each long row */
     int64_t partialOff;    /* double [numSegments * n] */
-    int64_t rowOrderOff;   /* int32 [numOrdered]: the rows ROW_SPLIT takes, longest first, so that the lane
-                              groups of a wavefront work on rows of similar length; 0 = natural order */
-    int64_t numOrdered;
+    int64_t reserved0;     /* unused, zero */
+    int64_t reserved1;
     int64_t bytes;
 } OpsparseSpmmPlan;
 
@@ -171,7 +170,9 @@ int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t n
  * dimensions in elements; transB != 0 reads B as its transpose, with the index
  * formulas of the reference kernel [ref: sparse/spmm/arch35/spmm_kernel.cpp:155-168, :215-219].
  * clampF16: when cType is F16, clamp to +-65504 before rounding [ref: :229-237].
- * plan == NULL runs ROW_SPLIT without a workspace.
+ * With a plan and row-major operands the rows are worked in slabs of consecutive
+ * rows staged through LDS (short rows share gather batches); plan == NULL runs
+ * one lane group per row without a workspace.
  */
 int opsparse_spmm_csr_launch(const OpsparseSpmmPlan *plan, const int32_t *rowOffsets, const int32_t *colInd,
                              const void *csrValues, const void *B, void *C, int64_t rows, int64_t k, int64_t n,

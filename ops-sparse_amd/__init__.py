@@ -21,7 +21,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "libops_sparse.so")
+# OPS_SPARSE_LIB points at another build of the library (kernel tuning experiments).
+LIB_PATH = os.environ.get("OPS_SPARSE_LIB") or os.path.join(_HERE, "lib", "libops_sparse.so")
 
 # ---- aclDataType (include/acl/acl_base_rt.h)
 ACL_FLOAT, ACL_FLOAT16, ACL_INT8, ACL_INT32 = 0, 1, 2, 3
@@ -102,7 +103,7 @@ class OpsparseSpmmPlan(ctypes.Structure):
     _fields_ = [("kernel", i32), ("maxRowNnz", i32), ("longRowNnz", i32), ("numLongRows", i32),
                 ("numSegments", i32), ("segmentNnz", i32), ("rows", i64), ("nnz", i64), ("n", i64),
                 ("longRowsOff", i64), ("segRowOff", i64), ("segStartOff", i64), ("longFirstSegOff", i64),
-                ("partialOff", i64), ("rowOrderOff", i64), ("numOrdered", i64), ("bytes", i64)]
+                ("partialOff", i64), ("reserved0", i64), ("reserved1", i64), ("bytes", i64)]
 
 
 _lib = None

@@ -13,7 +13,10 @@
 //
 // Row-length binning (the counterpart of the reference's greedy row bin
 // packing, sparse/spmm/arch35/spmm_csr_mat.cpp:28-66): rows of up to
-// kLongRowNnz entries are taken whole by one lane group (ROW_SPLIT).  Longer
+// kLongRowNnz entries are taken whole by one lane group — after Preprocess in
+// slabs of consecutive rows staged through LDS, where every lane group walks an
+// equal share of the slab's entries (SpmmSlabKernel), without Preprocess one
+// row after the other straight from global memory (SpmmRowSplitKernel).  Longer
 // rows — the tail of a power-law graph — are cut into segments of kSegmentNnz
 // entries, every segment is accumulated by its own lane group into an fp64
 // partial row in the workspace, and a fix-up kernel adds a row's partials in
@@ -24,6 +27,7 @@
 // once, int8 products in int32 with an int64 saturating epilogue
 // (spmm_kernel.cpp:251-266).
 #include <climits>
+#include <cstdlib>
 #include <type_traits>
 #include <vector>
 
@@ -181,8 +185,7 @@ template <typename ValT, typename CT, typename AccT, int V, int L>
 __global__ __launch_bounds__(kBlockThreads) void SpmmRowSplitKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
     const ValT *__restrict__ B, CT *__restrict__ C, int64_t rows, int32_t n, int64_t ldb, int64_t ldc,
-    int32_t longRowNnz, const int32_t *__restrict__ rowOrder, OpsparseScalar alphaS, OpsparseScalar betaS,
-    int32_t clampF16)
+    int32_t longRowNnz, OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16)
 {
     typedef CT CVec __attribute__((ext_vector_type(V), aligned(16)));
     constexpr int kGroups = kBlockThreads / L;
@@ -205,8 +208,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmRowSplitKernel(
 #pragma unroll
     for (int it = 0; it < kSpmmRowsPerGroup; ++it) {
         const int64_t slot = rowBase + static_cast<int64_t>(it) * kGroups + group;
-        // `rows` counts the slots: all rows, or the entries of rowOrder
-        rowId[it] = slot >= rows ? -1 : (rowOrder != nullptr ? static_cast<int64_t>(rowOrder[slot]) : slot);
+        rowId[it] = slot >= rows ? -1 : slot;
     }
 #pragma unroll
     for (int it = 0; it < kSpmmRowsPerGroup; ++it) {
@@ -258,6 +260,213 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmRowSplitKernel(
                 *reinterpret_cast<CVec *>(out) = res;
             }
         }
+    }
+}
+
+// ---------------------------------------------------------------- slab path
+// The same fast-path operands, rows of at most longRowNnz entries, worked on a
+// slab of consecutive rows at a time.  A workgroup copies the slab's (column,
+// value) pairs — one contiguous piece of the CSR arrays — and its row bounds
+// into LDS, cuts the slab's rows into one run of consecutive rows per lane group
+// with about the same number of entries each, and every lane group then walks
+// its run as one flat sequence of entries: batches of four or eight gathers of B
+// rows, two batches in flight, a row's sum written out whenever the sequence
+// crosses a row end.  Short rows therefore cost no more than their share of a
+// long one: no predicated partial batches, no chain of dependent loads in front
+// of every row.  Rows longer than longRowNnz are left out (the segment kernels
+// write them); a slab with more entries than the LDS holds is worked in several
+// pieces.
+
+constexpr int kSlabCap = 3072;      // entries a workgroup stages in LDS at a time
+constexpr int kSlabRowsMax = 255;   // rows whose bounds it stages at a time
+// Gathers a lane group issues back to back, two such batches in flight.  Four for
+// the 8-element (fp16) vectors, whose widening to fp64 needs the registers: with
+// eight the kernel drops to two resident wavefronts per SIMD and runs slower.
+template <int V>
+struct SlabTuning {
+    static constexpr int kBatch = V >= 8 ? 4 : 8;
+    static constexpr int kWavesPerSimd = V >= 8 ? 3 : 2;
+};
+constexpr int kSlabTarget = 2048;   // entries per slab the launcher aims for
+
+// Small32: B spans less than 4 GiB, so a gather address is the (uniform) base of
+// B plus a 32-bit byte offset — one register and one multiply per gather
+// instead of a 64-bit multiply-add and a register pair.
+template <typename ValT, typename CT, typename AccT, int V, int L, bool Small32>
+__global__ __launch_bounds__(kBlockThreads, SlabTuning<V>::kWavesPerSimd) void SpmmSlabKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ B, CT *__restrict__ C, int64_t rows, int32_t n, int64_t ldb, int64_t ldc,
+    int32_t rowsPerSlab, int32_t longRowNnz, OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16)
+{
+    typedef ValT BVec __attribute__((ext_vector_type(V)));
+    typedef CT CVec __attribute__((ext_vector_type(V), aligned(16)));
+    constexpr int kGroups = kBlockThreads / L;
+    constexpr int NB = SlabTuning<V>::kBatch;
+
+    __shared__ int32_t entCol[kSlabCap];
+    __shared__ float entVal[kSlabCap];
+    __shared__ int32_t rowAbs[kSlabRowsMax + 1];  // row offsets of the window, as stored
+    __shared__ int32_t runBound[kGroups + 1];     // first row (window-relative) of every lane group's run
+    __shared__ int32_t pieceRows;                 // rows of the window that go into this piece
+
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    const AccT beta = ReadScalar<AccT>(betaS);
+    const bool betaZero = (beta == AccT(0));
+    const int32_t tid = threadIdx.x;
+    const int32_t lane = tid % L;
+    const int32_t group = tid / L;
+    const int32_t col = lane * V;
+    const bool active = col < n;
+    const ValT *Bcol = B + col;
+    const uint32_t colBytes = static_cast<uint32_t>(col) * static_cast<uint32_t>(sizeof(ValT));
+    const uint32_t ldbBytes = static_cast<uint32_t>(ldb) * static_cast<uint32_t>(sizeof(ValT));
+
+    const int64_t slab = XcdContiguousTile(blockIdx.x, gridDim.x);
+    int64_t rowCur = slab * rowsPerSlab;
+    const int64_t rowEnd = (rowCur + rowsPerSlab < rows) ? rowCur + rowsPerSlab : rows;
+
+    while (rowCur < rowEnd) {  // uniform over the workgroup
+        const int32_t win = (rowEnd - rowCur < kSlabRowsMax) ? static_cast<int32_t>(rowEnd - rowCur) : kSlabRowsMax;
+        if (tid <= win) {
+            rowAbs[tid] = rowOffsets[rowCur + tid];
+        }
+        if (tid == 0) {
+            pieceRows = win;
+        }
+        __syncthreads();
+        const int32_t base = rowAbs[0];
+        // The piece ends in front of the first row that is long or no longer fits.
+        if (tid < win) {
+            const int32_t hi = rowAbs[tid + 1];
+            if (hi - rowAbs[tid] > longRowNnz || hi - base > kSlabCap) {
+                atomicMin(&pieceRows, tid);
+            }
+        }
+        __syncthreads();
+        const int32_t J = pieceRows;
+        if (J == 0) {
+            rowCur += 1;  // a long row: not this kernel's (longRowNnz <= kSlabCap, so a short row always fits)
+            __syncthreads();
+            continue;
+        }
+        const int32_t E = rowAbs[J] - base;
+        for (int32_t i = tid; i < E; i += kBlockThreads) {
+            entCol[i] = LoadStream(colInd + base + i);
+            entVal[i] = static_cast<float>(ToAcc<AccT>(LoadStream(vals + base + i)));
+        }
+        // Run g starts at the first row whose first entry is at or after g * share.
+        if (tid <= kGroups) {
+            const int32_t share = (E + kGroups - 1) / kGroups;
+            int32_t lo = 0, hi = J;
+            if (tid == kGroups) {
+                lo = J;
+            } else {
+                const int32_t want = base + tid * share;
+                while (lo < hi) {
+                    const int32_t mid = (lo + hi) >> 1;
+                    if (rowAbs[mid] < want) {
+                        lo = mid + 1;
+                    } else {
+                        hi = mid;
+                    }
+                }
+            }
+            runBound[tid] = lo;
+        }
+        __syncthreads();
+
+        int32_t cur = runBound[group];           // next row to finish
+        const int32_t last = runBound[group + 1];
+        int32_t f = rowAbs[cur] - base;          // next entry to consume
+        const int32_t fEnd = rowAbs[last] - base;
+        int32_t nextEnd = (cur < last) ? rowAbs[cur + 1] - base : INT32_MAX;
+
+        AccT acc[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            acc[i] = AccT(0);
+        }
+        // Writes every row of the run that ends at entry position `pos`.
+        auto finishRows = [&](int32_t pos) {
+            while (nextEnd <= pos) {
+                if (active) {
+                    CT *out = C + (rowCur + cur) * ldc + col;
+                    CVec res;
+                    if (betaZero) {
+#pragma unroll
+                        for (int i = 0; i < V; ++i) {
+                            res[i] = Epilogue<CT, AccT>::Apply(acc[i], alpha, beta, true, nullptr, clampF16 != 0);
+                        }
+                    } else {
+                        const CVec old = *reinterpret_cast<const CVec *>(out);
+#pragma unroll
+                        for (int i = 0; i < V; ++i) {
+                            const CT o = old[i];
+                            res[i] = Epilogue<CT, AccT>::Apply(acc[i], alpha, beta, false, &o, clampF16 != 0);
+                        }
+                    }
+                    *reinterpret_cast<CVec *>(out) = res;
+                }
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    acc[i] = AccT(0);
+                }
+                ++cur;
+                nextEnd = (cur < last) ? rowAbs[cur + 1] - base : INT32_MAX;
+            }
+        };
+        finishRows(f);  // empty rows at the head of the run
+
+        // Gathers are issued unconditionally (a position past the end of the run
+        // re-reads the run's last entry with a zero value, a lane past column n reads
+        // column 0), so that the compiler can count the loads in flight and wait for
+        // one batch while the next stays outstanding.
+        BVec bufA[NB], bufB[NB];
+        float valA[NB], valB[NB];
+        const uint32_t laneBytes = active ? colBytes : 0u;
+        const ValT *Blane = active ? Bcol : B;
+        auto fetch = [&](int32_t f0, BVec(&buf)[NB], float(&v)[NB]) {
+#pragma unroll
+            for (int q = 0; q < NB; ++q) {
+                const int32_t p = f0 + q;
+                const int32_t pc = p < fEnd ? p : fEnd - 1;
+                const int32_t c = entCol[pc];
+                v[q] = p < fEnd ? entVal[pc] : 0.0f;
+                if (Small32) {
+                    const uint32_t off = static_cast<uint32_t>(c) * ldbBytes + laneBytes;
+                    buf[q] = *reinterpret_cast<const BVec *>(reinterpret_cast<const char *>(B) + off);
+                } else {
+                    buf[q] = *reinterpret_cast<const BVec *>(Blane + static_cast<int64_t>(c) * ldb);
+                }
+            }
+        };
+        auto consume = [&](int32_t f0, BVec(&buf)[NB], float(&v)[NB]) {
+#pragma unroll
+            for (int q = 0; q < NB; ++q) {
+                const AccT vq = static_cast<AccT>(v[q]);
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    acc[i] += vq * ToAcc<AccT>(buf[q][i]);
+                }
+                finishRows(f0 + q + 1);  // positions past the end finish nothing: every row is done by then
+            }
+        };
+        if (f < fEnd) {
+            fetch(f, bufA, valA);
+        }
+        while (f < fEnd) {
+            fetch(f + NB, bufB, valB);  // also when nothing is left: a branch here would hide the load count
+            consume(f, bufA, valA);
+            f += NB;
+            if (f < fEnd) {
+                fetch(f + NB, bufA, valA);
+                consume(f, bufB, valB);
+                f += NB;
+            }
+        }
+        finishRows(fEnd);  // nothing left unless the run has no entry at all
+        rowCur += J;
+        __syncthreads();   // the next piece overwrites the LDS arrays
     }
 }
 
@@ -469,11 +678,7 @@ void LayoutPlan(OpsparseSpmmPlan *p)
     off = Align256(off + 4 * static_cast<int64_t>(p->numSegments));
     p->partialOff = off;
     off = Align256(off + 8 * static_cast<int64_t>(p->numSegments) * p->n);
-    if (p->numOrdered > 0) {
-        p->rowOrderOff = off;
-        off = Align256(off + 4 * p->numOrdered);
-    }
-    p->bytes = (p->numLongRows > 0 || p->numOrdered > 0) ? off : 256;
+    p->bytes = p->numLongRows > 0 ? off : 256;
 }
 
 // Device reduction of the row lengths into `scratch` (>= 16 bytes), read back
@@ -500,39 +705,88 @@ int RowStats(const int32_t *rowOffsets, int64_t rows, int32_t *scratch, hipStrea
 }
 
 template <typename ValT, typename CT, typename AccT, int V, int L>
+void LaunchLongRows(const SpmmArgs &a);
+
+template <typename ValT, typename CT, typename AccT, int V, int L>
 int LaunchRowSplit(const SpmmArgs &a)
 {
     constexpr int kGroups = kBlockThreads / L;
     const bool binned = a.plan != nullptr && a.plan->kernel == OPSPARSE_SPMM_BINNED && a.plan->numLongRows > 0;
     const int64_t rowsPerBlock = static_cast<int64_t>(kGroups) * kSpmmRowsPerGroup;
-    const bool ordered = binned && a.plan->numOrdered > 0;
-    const int32_t *rowOrder =
-        ordered ? reinterpret_cast<const int32_t *>(static_cast<unsigned char *>(a.ws) + a.plan->rowOrderOff) : nullptr;
-    const int64_t slots = ordered ? a.plan->numOrdered : a.rows;
+    const int64_t slots = a.rows;
     const uint32_t grid = static_cast<uint32_t>((slots + rowsPerBlock - 1) / rowsPerBlock);
     if (slots > 0) {
         hipLaunchKernelGGL((SpmmRowSplitKernel<ValT, CT, AccT, V, L>), dim3(grid), dim3(kBlockThreads), 0, a.stream,
                            a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
                            static_cast<const ValT *>(a.B), static_cast<CT *>(a.C), slots, static_cast<int32_t>(a.n),
-                           a.ldb, a.ldc, binned ? a.plan->longRowNnz : INT32_MAX, rowOrder, a.alpha,
-                           a.beta, a.clampF16);
+                           a.ldb, a.ldc, binned ? a.plan->longRowNnz : INT32_MAX, a.alpha, a.beta, a.clampF16);
     }
     if (binned) {
-        auto *base = static_cast<unsigned char *>(a.ws);
-        const auto *longRows = reinterpret_cast<const int32_t *>(base + a.plan->longRowsOff);
-        const auto *firstSeg = reinterpret_cast<const int32_t *>(base + a.plan->longFirstSegOff);
-        const auto *segRow = reinterpret_cast<const int32_t *>(base + a.plan->segRowOff);
-        const auto *segStart = reinterpret_cast<const int32_t *>(base + a.plan->segStartOff);
-        auto *partial = reinterpret_cast<AccT *>(base + a.plan->partialOff);
-        const int32_t nseg = a.plan->numSegments;
-        hipLaunchKernelGGL((SpmmLongSegmentKernel<ValT, AccT, V, L>), dim3((nseg + kGroups - 1) / kGroups),
-                           dim3(kBlockThreads), 0, a.stream, a.rowOffsets, a.colInd,
-                           static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.B),
-                           static_cast<int32_t>(a.n), a.ldb, nseg, segRow, segStart, partial);
-        const int32_t nlong = a.plan->numLongRows;
-        hipLaunchKernelGGL((SpmmLongFixupKernel<CT, AccT>), dim3(nlong),
-                           dim3(kBlockThreads), 0, a.stream, static_cast<CT *>(a.C), static_cast<int32_t>(a.n),
-                           a.ldc, nlong, longRows, firstSeg, partial, a.alpha, a.beta, a.clampF16);
+        LaunchLongRows<ValT, CT, AccT, V, L>(a);
+    }
+    return CheckLaunch();
+}
+
+// Segment + fix-up kernels for the long rows of a BINNED plan.
+template <typename ValT, typename CT, typename AccT, int V, int L>
+void LaunchLongRows(const SpmmArgs &a)
+{
+    constexpr int kGroups = kBlockThreads / L;
+    auto *base = static_cast<unsigned char *>(a.ws);
+    const auto *longRows = reinterpret_cast<const int32_t *>(base + a.plan->longRowsOff);
+    const auto *firstSeg = reinterpret_cast<const int32_t *>(base + a.plan->longFirstSegOff);
+    const auto *segRow = reinterpret_cast<const int32_t *>(base + a.plan->segRowOff);
+    const auto *segStart = reinterpret_cast<const int32_t *>(base + a.plan->segStartOff);
+    auto *partial = reinterpret_cast<AccT *>(base + a.plan->partialOff);
+    const int32_t nseg = a.plan->numSegments;
+    hipLaunchKernelGGL((SpmmLongSegmentKernel<ValT, AccT, V, L>), dim3((nseg + kGroups - 1) / kGroups),
+                       dim3(kBlockThreads), 0, a.stream, a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
+                       static_cast<const ValT *>(a.B), static_cast<int32_t>(a.n), a.ldb, nseg, segRow, segStart,
+                       partial);
+    const int32_t nlong = a.plan->numLongRows;
+    hipLaunchKernelGGL((SpmmLongFixupKernel<CT, AccT>), dim3(nlong), dim3(kBlockThreads), 0, a.stream,
+                       static_cast<CT *>(a.C), static_cast<int32_t>(a.n), a.ldc, nlong, longRows, firstSeg, partial,
+                       a.alpha, a.beta, a.clampF16);
+}
+
+// The slab kernel needs an analysed matrix (it must know that no row it is given
+// exceeds its LDS) and one column tile per lane group.
+bool UseSlabKernel(const SpmmArgs &a, int64_t lanesNeeded)
+{
+    static const bool off = std::getenv("OPS_SPARSE_SPMM_NO_SLAB") != nullptr;
+    if (off || a.plan == nullptr || lanesNeeded > 64) {
+        return false;
+    }
+    const bool binned = a.plan->kernel == OPSPARSE_SPMM_BINNED && a.plan->numLongRows > 0;
+    return binned || (a.plan->maxRowNnz > 0 && a.plan->maxRowNnz <= kSlabCap);
+}
+
+template <typename ValT, typename CT, typename AccT, int V, int L>
+int LaunchSlab(const SpmmArgs &a)
+{
+    const bool binned = a.plan->kernel == OPSPARSE_SPMM_BINNED && a.plan->numLongRows > 0;
+    // Slabs of about kSlabTarget entries on average.
+    static const int64_t target = std::getenv("OPS_SPARSE_SPMM_SLAB_ENTRIES") != nullptr
+                                      ? std::atoll(std::getenv("OPS_SPARSE_SPMM_SLAB_ENTRIES"))
+                                      : kSlabTarget;
+    int64_t rps = a.nnz > 0 ? target * a.rows / a.nnz : 4096;
+    rps = rps < 16 ? 16 : (rps > 4096 ? 4096 : rps);
+    const uint32_t grid = static_cast<uint32_t>((a.rows + rps - 1) / rps);
+    const int32_t longRowNnz = binned ? a.plan->longRowNnz : kSlabCap;
+    const bool small32 = static_cast<uint64_t>(a.k) * static_cast<uint64_t>(a.ldb) * sizeof(ValT) < (1ull << 32);
+    if (small32) {
+        hipLaunchKernelGGL((SpmmSlabKernel<ValT, CT, AccT, V, L, true>), dim3(grid), dim3(kBlockThreads), 0, a.stream,
+                           a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.B),
+                           static_cast<CT *>(a.C), a.rows, static_cast<int32_t>(a.n), a.ldb, a.ldc,
+                           static_cast<int32_t>(rps), longRowNnz, a.alpha, a.beta, a.clampF16);
+    } else {
+        hipLaunchKernelGGL((SpmmSlabKernel<ValT, CT, AccT, V, L, false>), dim3(grid), dim3(kBlockThreads), 0, a.stream,
+                           a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.B),
+                           static_cast<CT *>(a.C), a.rows, static_cast<int32_t>(a.n), a.ldb, a.ldc,
+                           static_cast<int32_t>(rps), longRowNnz, a.alpha, a.beta, a.clampF16);
+    }
+    if (binned) {
+        LaunchLongRows<ValT, CT, AccT, V, L>(a);
     }
     return CheckLaunch();
 }
@@ -570,6 +824,14 @@ int RunTyped(const SpmmArgs &a)
         return RunGeneral<ValT, CT, AccT>(a);
     }
     const int64_t lanesNeeded = a.n / V;
+    if (UseSlabKernel(a, lanesNeeded)) {
+        if (lanesNeeded <= 2) return LaunchSlab<ValT, CT, AccT, V, 2>(a);
+        if (lanesNeeded <= 4) return LaunchSlab<ValT, CT, AccT, V, 4>(a);
+        if (lanesNeeded <= 8) return LaunchSlab<ValT, CT, AccT, V, 8>(a);
+        if (lanesNeeded <= 16) return LaunchSlab<ValT, CT, AccT, V, 16>(a);
+        if (lanesNeeded <= 32) return LaunchSlab<ValT, CT, AccT, V, 32>(a);
+        return LaunchSlab<ValT, CT, AccT, V, 64>(a);
+    }
     if (lanesNeeded <= 2) return LaunchRowSplit<ValT, CT, AccT, V, 2>(a);
     if (lanesNeeded <= 4) return LaunchRowSplit<ValT, CT, AccT, V, 4>(a);
     if (lanesNeeded <= 8) return LaunchRowSplit<ValT, CT, AccT, V, 8>(a);
@@ -610,7 +872,6 @@ int opsparse_spmm_csr_workspace_bytes(const int32_t *rowOffsets, int64_t rows, i
     p.n = n;
     p.numLongRows = st[1];
     p.numSegments = st[2];
-    p.numOrdered = st[1] > 0 ? rows - st[1] : 0;
     LayoutPlan(&p);
     *bytes = static_cast<size_t>(p.bytes);
     return OPSPARSE_OK;
@@ -651,7 +912,6 @@ int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t n
     p.kernel = OPSPARSE_SPMM_BINNED;
     p.numLongRows = st[1];
     p.numSegments = st[2];
-    p.numOrdered = rows - st[1];
     LayoutPlan(&p);
     if (static_cast<int64_t>(workspaceBytes) < p.bytes) {
         return OPSPARSE_E_WORKSPACE;
@@ -682,26 +942,6 @@ int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t n
         }
     }
     firstSeg.push_back(static_cast<int32_t>(segRow.size()));
-    // The other rows, longest first (counting sort by length, stable in the row index).
-    std::vector<int32_t> order(static_cast<size_t>(p.numOrdered));
-    {
-        std::vector<int64_t> start(static_cast<size_t>(kLongRowNnz) + 2, 0);
-        for (int64_t r = 0; r < rows; ++r) {
-            const int32_t len = rp[r + 1] - rp[r];
-            if (len <= kLongRowNnz) {
-                ++start[kLongRowNnz - len + 1];
-            }
-        }
-        for (size_t b = 1; b < start.size(); ++b) {
-            start[b] += start[b - 1];
-        }
-        for (int64_t r = 0; r < rows; ++r) {
-            const int32_t len = rp[r + 1] - rp[r];
-            if (len <= kLongRowNnz) {
-                order[static_cast<size_t>(start[kLongRowNnz - len]++)] = static_cast<int32_t>(r);
-            }
-        }
-    }
     if (static_cast<int32_t>(longRows.size()) != p.numLongRows || static_cast<int32_t>(segRow.size()) != p.numSegments) {
         return OPSPARSE_E_INVALID;  // the matrix changed between the two passes
     }
@@ -714,8 +954,6 @@ int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t n
                    hipSuccess;
     ok = ok && hipMemcpyAsync(base + p.segStartOff, segStart.data(), segStart.size() * 4, hipMemcpyHostToDevice, s) ==
                    hipSuccess;
-    ok = ok && (order.empty() || hipMemcpyAsync(base + p.rowOrderOff, order.data(), order.size() * 4,
-                                                hipMemcpyHostToDevice, s) == hipSuccess);
     ok = ok && hipStreamSynchronize(s) == hipSuccess;  // the host vectors die at return
     if (!ok) {
         (void)hipGetLastError();

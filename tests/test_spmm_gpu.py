@@ -215,3 +215,80 @@ def test_spmm_column_equals_spmv(osa, gpu_ctx):
     for j in range(n):
         y = oracle.spmv_f64(m, k, rowptr, colind, val, np.ascontiguousarray(B[:, j]), None, 1.0, 0.0)
         assert oracle.max_rel_err(got.reshape(m, n)[:, j], y) <= 1e-6
+
+
+def _lengths(shape, m, rng):
+    if shape == "mostly_empty":                 # windows of more than 255 empty rows
+        lengths = np.zeros(m, np.int64)
+        lengths[rng.choice(m, m // 100, replace=False)] = rng.integers(1, 30, m // 100)
+    elif shape == "threshold":                  # 256 is still a short row, 257 is a long one
+        lengths = rng.integers(0, 12, m)
+        lengths[rng.choice(m, 40, replace=False)] = rng.choice([255, 256, 257, 300], 40)
+    elif shape == "dense_slabs":                # a slab holds more entries than one LDS piece takes
+        lengths = rng.integers(150, 257, m)
+    elif shape == "alternating":
+        lengths = np.arange(m) % 2
+    elif shape == "power_law":
+        lengths = np.minimum((1.0 / rng.uniform(1e-4, 1.0, m)).astype(np.int64), 4000)
+    else:
+        raise ValueError(shape)
+    return lengths
+
+
+@pytest.mark.parametrize("shape", ["mostly_empty", "threshold", "dense_slabs", "alternating", "power_law"])
+@pytest.mark.parametrize("n,beta", [(8, 0.0), (24, 0.5), (64, -1.0), (256, 0.0)])
+def test_row_length_mixes(osa, gpu_ctx, shape, n, beta):
+    """Preprocessed fast path (rows worked in LDS-staged slabs, long rows in segments) on row-length mixes that
+    hit its corner cases; n = 24 leaves lanes of a lane group without a column."""
+    rng = np.random.default_rng(len(shape) * 1000 + n)
+    m = 1 if shape == "single" else (700 if shape == "dense_slabs" else 6000)
+    k = 5000
+    rowptr, colind, val = csr_from_lengths(_lengths(shape, m, rng), k, seed=n)
+    B = rng.uniform(-1, 1, k * n).astype(np.float32)
+    C0 = rng.uniform(-1, 1, m * n).astype(np.float32)
+    if beta == 0.0:
+        C0[::7] = np.nan                         # C must not be read
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, n, C0, n, 1.25, beta)
+    gold = oracle.spmm_f64_rowmajor(m, n, rowptr, colind, val, B, n, np.nan_to_num(C0), n, 1.25, beta)
+    assert oracle.max_rel_err(got, gold) <= 1e-5
+
+
+@pytest.mark.parametrize("shape", ["threshold", "power_law"])
+def test_row_length_mixes_fp16(osa, gpu_ctx, shape):
+    import torch
+    rng = np.random.default_rng(77)
+    m, k, n = 5000, 4000, 128
+    rowptr, colind, val = csr_from_lengths(_lengths(shape, m, rng), k, seed=5)
+    val = val.astype(np.float16).astype(np.float32)
+    B = rng.uniform(-1, 1, k * n).astype(np.float16).astype(np.float32)
+    C0 = rng.uniform(-1, 1, m * n).astype(np.float32)
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, n, C0, n, 1.0, 0.5, val_dtype=torch.float16)
+    gold = oracle.spmm_f64_rowmajor(m, n, rowptr, colind, val, B, n, C0, n, 1.0, 0.5)
+    assert oracle.max_rel_err(got, gold) <= 1e-3
+
+
+@pytest.mark.parametrize("n", [4, 64, 512])
+def test_raw_launch_without_plan(osa, gpu_ctx, n):
+    """opsparse_spmm_csr_launch with plan == NULL: one lane group per row of any length, no workspace."""
+    import ctypes
+    import torch
+    from helpers import to_dev
+    dev, stream, handle = gpu_ctx
+    rng = np.random.default_rng(n)
+    m, k = 3000, 9000
+    lengths = rng.integers(0, 20, m)
+    lengths[[5, 2000]] = [7000, 300]
+    rowptr, colind, val = csr_from_lengths(lengths, k, seed=9)
+    B = rng.uniform(-1, 1, k * n).astype(np.float32)
+    C0 = rng.uniform(-1, 1, m * n).astype(np.float32)
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, B, C0)]
+    s = lambda v: osa.OpsparseScalar(v, None, 0, 0)
+    torch.cuda.synchronize()
+    rc = osa.lib().opsparse_spmm_csr_launch(None, d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(),
+                                            d[4].data_ptr(), m, k, n, colind.size, n, n, 0, 0, 0, s(0.5), s(2.0),
+                                            osa.OPSPARSE_F32, osa.OPSPARSE_F32, None, 0,
+                                            ctypes.c_void_p(stream.cuda_stream))
+    assert rc == 0
+    stream.synchronize()
+    gold = oracle.spmm_f64_rowmajor(m, n, rowptr, colind, val, B, n, C0, n, 0.5, 2.0)
+    assert oracle.max_rel_err(d[4].cpu().numpy(), gold) <= 1e-5
