@@ -117,6 +117,35 @@ typedef enum aclsparsePointerMode_t {
     ACL_SPARSE_POINTER_MODE_DEVICE = 1
 } aclsparsePointerMode_t;
 
+/* [ref: :192-210] attributes of the legacy matrix descriptor. */
+typedef enum aclsparseMatrixType_t {
+    ACL_SPARSE_MATRIX_TYPE_GENERAL = 0,
+    ACL_SPARSE_MATRIX_TYPE_SYMMETRIC,
+    ACL_SPARSE_MATRIX_TYPE_HERMITIAN,
+    ACL_SPARSE_MATRIX_TYPE_TRIANGULAR
+} aclsparseMatrixType_t;
+
+typedef enum aclsparseDiagType_t {
+    ACL_SPARSE_DIAG_TYPE_NON_UNIT = 0,
+    ACL_SPARSE_DIAG_TYPE_UNIT
+} aclsparseDiagType_t;
+
+typedef enum aclsparseFillMode_t {
+    ACL_SPARSE_FILL_MODE_LOWER = 0,
+    ACL_SPARSE_FILL_MODE_UPPER
+} aclsparseFillMode_t;
+
+/* [ref: :1369-1379] CSR -> CSC: structure only, or structure and values; algorithm tag. */
+typedef enum aclsparseAction_t {
+    ACL_SPARSE_ACTION_SYMBOLIC = 0,
+    ACL_SPARSE_ACTION_NUMERIC
+} aclsparseAction_t;
+
+typedef enum aclsparseCsr2CscAlg_t {
+    ACL_SPARSE_CSR2CSC_ALG_DEFAULT = 0,
+    ACL_SPARSE_CSR2CSC_ALG1
+} aclsparseCsr2CscAlg_t;
+
 /* ---------------------------------------------------------- opaque types */
 
 /* [ref: :30-47, :73-78] */
@@ -126,7 +155,9 @@ struct aclsparseDnVecDescr;
 struct aclsparseDnMatDescr;
 struct aclsparseSpMVOpDescr;
 struct aclsparseSpMVOpPlan;
+struct aclsparseMatDescr; /* [ref: :189-190] legacy descriptor: type, index base, diag, fill */
 
+typedef struct aclsparseMatDescr *aclsparseMatDescr_t;
 typedef struct aclsparseContext *aclsparseHandle_t;
 typedef struct aclsparseSpMatDescr *aclsparseSpMatDescr_t;
 typedef struct aclsparseDnVecDescr *aclsparseDnVecDescr_t;
@@ -352,6 +383,63 @@ aclsparseStatus_t aclsparseSpMVOp_setGlobalUserData(aclsparseHandle_t handle, ac
 aclsparseStatus_t aclsparseSpMVOp(aclsparseHandle_t handle, aclsparseSpMVOpPlan_t plan, const void *alpha,
                                   const void *beta, aclsparseConstDnVecDescr_t vecX, aclsparseConstDnVecDescr_t vecY,
                                   aclsparseDnVecDescr_t vecZ);
+
+/* ---------------------------------------------------------- CSR producers
+ * Integer / byte operations; every output is bit-exact against the reference's
+ * CPU goldens.  All enqueue on the handle's stream and return.
+ */
+
+/* Legacy matrix descriptor [ref: :910-919; sparse/common/aclsparse_matdescr.cpp:25-110].
+ * Create gives GENERAL / base 0 / NON_UNIT / LOWER; Destroy(NULL) is SUCCESS;
+ * setters ignore a NULL descriptor, getters return the default for it. */
+aclsparseStatus_t aclsparseCreateMatDescr(aclsparseMatDescr_t *descr);
+aclsparseStatus_t aclsparseDestroyMatDescr(aclsparseMatDescr_t descr);
+void aclsparseSetMatType(aclsparseMatDescr_t descr, aclsparseMatrixType_t type);
+void aclsparseSetMatIndexBase(aclsparseMatDescr_t descr, aclsparseIndexBase_t base);
+void aclsparseSetMatDiagType(aclsparseMatDescr_t descr, aclsparseDiagType_t diagType);
+void aclsparseSetMatFillMode(aclsparseMatDescr_t descr, aclsparseFillMode_t fillMode);
+aclsparseMatrixType_t aclsparseGetMatType(aclsparseMatDescr_t descr);
+aclsparseIndexBase_t aclsparseGetMatIndexBase(aclsparseMatDescr_t descr);
+aclsparseDiagType_t aclsparseGetMatDiagType(aclsparseMatDescr_t descr);
+aclsparseFillMode_t aclsparseGetMatFillMode(aclsparseMatDescr_t descr);
+
+/* [ref: :1816-1822; host sparse/coo2csr/arch35/coo2csr_host.cpp:38-80]
+ * csrRowPtr[0..m] from COO row indices (non-decreasing): per-row counts + prefix
+ * sum, + idxBase.  Row indices outside [0, m) are not counted.  Uses the
+ * handle's workspace (4 bytes per 2048 rows). */
+aclsparseStatus_t aclsparseXcoo2csr(aclsparseHandle_t handle, const int *cooRowInd, int nnz, int m, int *csrRowPtr,
+                                    aclsparseIndexBase_t idxBase);
+
+/* [ref: :1886-1891; host sparse/csr2coo/arch35/csr2coo_host.cpp:66-115]
+ * cooRowInd[j] = i + idxBase for j in [csrRowPtr[i], csrRowPtr[i+1]) - idxBase.
+ * A NULL handle gives NOT_INITIALIZED (this entry point's own code). */
+aclsparseStatus_t aclsparseXcsr2coo(aclsparseHandle_t handle, const int32_t *csrRowPtr, int64_t nnz, int64_t m,
+                                    int32_t *cooRowInd, aclsparseIndexBase_t idxBase);
+
+/* [ref: :1679-1711; host sparse/csrsort/arch35/csrsort_host.cpp:146-221]
+ * Stable ascending sort of the column indices inside every row, in place; P
+ * (any initial content, usually 0..nnz-1) is permuted the same way.  The index
+ * base comes from descrA.  pBuffer needs 4-byte alignment only. */
+aclsparseStatus_t aclsparseXcsrsort_bufferSizeExt(aclsparseHandle_t handle, int m, int n, int nnz,
+                                                  const int *csrRowPtr, const int *csrColInd,
+                                                  size_t *pBufferSizeInBytes);
+aclsparseStatus_t aclsparseXcsrsort(aclsparseHandle_t handle, int m, int n, int nnz, const aclsparseMatDescr_t descrA,
+                                    const int *csrRowPtr, int *csrColInd, int *P, void *pBuffer);
+
+/* [ref: :1401-1440; host sparse/csr2csc_ex2/arch35/csr2csc_ex2_host.cpp:109-232, :535-618]
+ * CSR (m x n) -> CSC: cscColPtr[0..n], cscRowInd and, for NUMERIC, cscVal; the
+ * entries of a column keep their CSR order (ascending rows).  Values are moved
+ * as raw 1 / 2 / 4-byte items (ACL_INT8, ACL_FLOAT16, ACL_BF16, ACL_FLOAT).
+ * buffer == NULL uses the handle's workspace when that is large enough. */
+aclsparseStatus_t aclsparseCsr2cscEx2_bufferSize(aclsparseHandle_t handle, int m, int n, int nnz, const void *csrVal,
+                                                 const int *csrRowPtr, const int *csrColInd, void *cscVal,
+                                                 int *cscColPtr, int *cscRowInd, aclDataType valType,
+                                                 aclsparseAction_t copyValues, aclsparseIndexBase_t idxBase,
+                                                 aclsparseCsr2CscAlg_t alg, size_t *bufferSize);
+aclsparseStatus_t aclsparseCsr2cscEx2(aclsparseHandle_t handle, int m, int n, int nnz, const void *csrVal,
+                                      const int *csrRowPtr, const int *csrColInd, void *cscVal, int *cscColPtr,
+                                      int *cscRowInd, aclDataType valType, aclsparseAction_t copyValues,
+                                      aclsparseIndexBase_t idxBase, aclsparseCsr2CscAlg_t alg, void *buffer);
 
 #ifdef __cplusplus
 }

@@ -180,6 +180,36 @@ int opsparse_spmm_csr_launch(const OpsparseSpmmPlan *plan, const int32_t *rowOff
                              int32_t transB, OpsparseScalar alpha, OpsparseScalar beta, int32_t valType,
                              int32_t cType, void *workspace, size_t workspaceBytes, void *stream);
 
+/* --------------------------------------------------------- CSR producers
+ * Raw launchers of the format conversions; they play the role of the reference's
+ * coo2csr_*_kernel_do / csr2coo_kernel_do / csrsort_kernel_do / csr2csc_ex2_*_kernel_do
+ * launchers [ref: sparse/coo2csr/arch35/coo2csr_kernel.h, sparse/csr2coo/arch35/csr2coo_kernel.h,
+ * sparse/csrsort/arch35/csrsort_kernel.h, sparse/csr2csc_ex2/arch35/csr2csc_ex2_kernel.h].
+ * indexBase is 0 or 1.  Workspaces need 4-byte alignment. */
+
+/* Scratch of the int32 prefix sum over `count` elements (the tile sums). */
+size_t opsparse_scan_workspace_bytes(int64_t count);
+
+/* csrRowPtr[0..m] from row indices; workspace >= opsparse_scan_workspace_bytes(m + 1). */
+int opsparse_coo2csr_launch(const int32_t *cooRowInd, int64_t nnz, int64_t m, int32_t *csrRowPtr, int32_t indexBase,
+                            void *workspace, size_t workspaceBytes, void *stream);
+
+/* cooRowInd[0..nnz) from csrRowPtr[0..m]. */
+int opsparse_csr2coo_launch(const int32_t *csrRowPtr, int64_t nnz, int64_t m, int32_t *cooRowInd, int32_t indexBase,
+                            void *stream);
+
+/* Per-row stable sort of csrColInd with perm carried along. */
+size_t opsparse_csrsort_workspace_bytes(int64_t m, int64_t nnz);
+int opsparse_csrsort_launch(int64_t m, int64_t n, int64_t nnz, int32_t indexBase, const int32_t *csrRowPtr,
+                            int32_t *csrColInd, int32_t *perm, void *workspace, size_t workspaceBytes, void *stream);
+
+/* CSR -> CSC.  valueBytes: 0 (structure only), 1, 2 or 4. */
+size_t opsparse_csr2csc_workspace_bytes(int64_t m, int64_t n, int64_t nnz);
+int opsparse_csr2csc_launch(int64_t m, int64_t n, int64_t nnz, const void *csrVal, const int32_t *csrRowPtr,
+                            const int32_t *csrColInd, void *cscVal, int32_t *cscColPtr, int32_t *cscRowInd,
+                            int32_t valueBytes, int32_t indexBase, void *workspace, size_t workspaceBytes,
+                            void *stream);
+
 /* ----------------------------------------------------------- measurement */
 
 /* Plain device-to-device copy kernel (dwordx4 per lane) used as the HBM

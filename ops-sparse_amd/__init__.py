@@ -74,11 +74,21 @@ ACLSPARSE_SYMBOLS = [
     "aclsparseSpMVOp_bufferSize", "aclsparseSpMVOp_createDescr", "aclsparseSpMVOp_destroyDescr",
     "aclsparseSpMVOp_createPlan", "aclsparseSpMVOp_destroyPlan", "aclsparseSpMVOp_setGlobalUserData",
     "aclsparseSpMVOp",
+    "aclsparseCreateMatDescr", "aclsparseDestroyMatDescr", "aclsparseSetMatType", "aclsparseSetMatIndexBase",
+    "aclsparseSetMatDiagType", "aclsparseSetMatFillMode", "aclsparseGetMatType", "aclsparseGetMatIndexBase",
+    "aclsparseGetMatDiagType", "aclsparseGetMatFillMode",
+    "aclsparseXcoo2csr", "aclsparseXcsr2coo", "aclsparseXcsrsort_bufferSizeExt", "aclsparseXcsrsort",
+    "aclsparseCsr2cscEx2_bufferSize", "aclsparseCsr2cscEx2",
 ]
+ACL_SPARSE_ACTION_SYMBOLIC, ACL_SPARSE_ACTION_NUMERIC = 0, 1
+ACL_SPARSE_CSR2CSC_ALG_DEFAULT, ACL_SPARSE_CSR2CSC_ALG1 = 0, 1
 OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_workspace_bytes", "opsparse_spmv_csr_analyse", "opsparse_spmv_csr_launch",
     "opsparse_spmv_csr_launch_zy", "opsparse_spmv_csr_indexed_launch",
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
+    "opsparse_scan_workspace_bytes", "opsparse_coo2csr_launch", "opsparse_csr2coo_launch",
+    "opsparse_csrsort_workspace_bytes", "opsparse_csrsort_launch", "opsparse_csr2csc_workspace_bytes",
+    "opsparse_csr2csc_launch",
     "opsparse_copy_launch", "opsparse_read_launch", "opsparse_gather_launch",
 ]
 
@@ -119,7 +129,7 @@ def lib():
             "libops_sparse.so is not built (%s missing); run `python ops-sparse_amd/build.py`" % LIB_PATH)
     L = ctypes.CDLL(LIB_PATH)
     for name in ACLSPARSE_SYMBOLS:
-        getattr(L, name).restype = ctypes.c_int
+        getattr(L, name).restype = None if name.startswith("aclsparseSetMat") else ctypes.c_int
     PV = ctypes.POINTER(vp)
     L.aclsparseCreate.argtypes = [PV]
     L.aclsparseDestroy.argtypes = [vp]
@@ -175,6 +185,33 @@ def lib():
     L.aclsparseSpMVOp_destroyPlan.argtypes = [vp]
     L.aclsparseSpMVOp_setGlobalUserData.argtypes = [vp, vp, ctypes.c_char_p, vp, sz]
     L.aclsparseSpMVOp.argtypes = [vp, vp, vp, vp, vp, vp, vp]
+    ci = ctypes.c_int
+    L.aclsparseCreateMatDescr.argtypes = [PV]
+    L.aclsparseDestroyMatDescr.argtypes = [vp]
+    for name in ("Type", "IndexBase", "DiagType", "FillMode"):
+        getattr(L, "aclsparseSetMat" + name).argtypes = [vp, ci]
+        getattr(L, "aclsparseGetMat" + name).argtypes = [vp]
+    L.aclsparseXcoo2csr.argtypes = [vp, vp, ci, ci, vp, ci]
+    L.aclsparseXcsr2coo.argtypes = [vp, vp, i64, i64, vp, ci]
+    L.aclsparseXcsrsort_bufferSizeExt.argtypes = [vp, ci, ci, ci, vp, vp, ctypes.POINTER(sz)]
+    L.aclsparseXcsrsort.argtypes = [vp, ci, ci, ci, vp, vp, vp, vp, vp]
+    csc_common = [vp, ci, ci, ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci]
+    L.aclsparseCsr2cscEx2_bufferSize.argtypes = csc_common + [ctypes.POINTER(sz)]
+    L.aclsparseCsr2cscEx2.argtypes = csc_common + [vp]
+    L.opsparse_scan_workspace_bytes.restype = sz
+    L.opsparse_scan_workspace_bytes.argtypes = [i64]
+    L.opsparse_coo2csr_launch.restype = ci
+    L.opsparse_coo2csr_launch.argtypes = [vp, i64, i64, vp, i32, vp, sz, vp]
+    L.opsparse_csr2coo_launch.restype = ci
+    L.opsparse_csr2coo_launch.argtypes = [vp, i64, i64, vp, i32, vp]
+    L.opsparse_csrsort_workspace_bytes.restype = sz
+    L.opsparse_csrsort_workspace_bytes.argtypes = [i64, i64]
+    L.opsparse_csrsort_launch.restype = ci
+    L.opsparse_csrsort_launch.argtypes = [i64, i64, i64, i32, vp, vp, vp, vp, sz, vp]
+    L.opsparse_csr2csc_workspace_bytes.restype = sz
+    L.opsparse_csr2csc_workspace_bytes.argtypes = [i64, i64, i64]
+    L.opsparse_csr2csc_launch.restype = ci
+    L.opsparse_csr2csc_launch.argtypes = [i64, i64, i64, vp, vp, vp, vp, vp, vp, i32, i32, vp, sz, vp]
 
     L.opsparse_spmv_csr_workspace_bytes.restype = sz
     L.opsparse_spmv_csr_workspace_bytes.argtypes = [i64, i64]

@@ -28,8 +28,10 @@ SOURCES = [
     "spmv_host.cpp",
     "spmv_op_host.cpp",
     "spmm_host.cpp",
+    "convert_host.cpp",
     "spmv_kernels.hip",
     "spmm_kernels.hip",
+    "convert_kernels.hip",
     "measure_kernels.hip",
 ]
 

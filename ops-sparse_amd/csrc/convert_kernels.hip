@@ -1,0 +1,786 @@
+// CSR producers for gfx950: COO rows -> CSR row offsets, CSR row offsets -> COO
+// rows, per-row stable sort of CSR column indices with a permutation, and CSR ->
+// CSC.  All of it is integer / byte work whose results must be bit-exact, and
+// all of it is bound by memory traffic, so the kernels stream their operands
+// with coalesced accesses and keep the shuffling in LDS.
+//
+// They replace the device side of
+//   aclsparseXcoo2csr     sparse/coo2csr/arch35/coo2csr_kernel.cpp   (count + prefix sum)
+//   aclsparseXcsr2coo     sparse/csr2coo/arch35/csr2coo_kernel.cpp   (row expansion)
+//   aclsparseXcsrsort     sparse/csrsort/arch35/csrsort_kernel.cpp   (runs + serial merge)
+//   aclsparseCsr2cscEx2   sparse/csr2csc_ex2/arch35/csr2csc_ex2_kernel.cpp (striped counting sort)
+// and produce what the reference's CPU goldens produce
+// (test/coo2csr/coo2csr_golden.h:44-77, test/csr2coo/csr2coo_golden.h:37-61,
+// test/csrsort/arch35/csrsort_golden.h:38-70, test/csr2csc_ex2/csr2csc_ex2_golden.h:50-110).
+//
+// Building blocks:
+//   * a three-kernel inclusive scan of int32 (tile sums, one-workgroup scan of the
+//     sums, tile rescan), in place if wanted;
+//   * a least-significant-digit radix sort of (key, payload) pairs, four bits a
+//     pass.  A thread owns consecutive items of its tile, counts them per digit,
+//     the workgroup scans the 16 x 256 counters digit-major, and every item goes to
+//     digit base + number of earlier items with its digit: stable by construction;
+//   * bitonic sorts of 64-bit (column, position) keys in registers (a wavefront per
+//     row of up to 64 entries) and in LDS (a workgroup per row of up to 2048); the
+//     position in the low half makes every key distinct, so any correct sort is
+//     the stable sort.
+#include <climits>
+
+#include "device_utils.h"
+
+namespace opsparse {
+
+constexpr int kScanItems = 8;                             // consecutive elements a thread scans
+constexpr int kScanTile = kBlockThreads * kScanItems;     // elements per workgroup
+constexpr int kRadixBits = 4;
+constexpr int kRadixDigits = 1 << kRadixBits;
+constexpr int kRadixItems = 4;                            // consecutive items a thread ranks
+constexpr int kRadixTile = kBlockThreads * kRadixItems;
+constexpr int kSortWaveRow = 64;                          // rows up to this length: one wavefront, registers
+constexpr int kSortLdsRow = 2048;                         // rows up to this length: one workgroup, LDS
+constexpr int kSortListBlocks = 2048;                     // workgroups walking the list of longer rows
+
+// ------------------------------------------------------------------- fill
+
+__global__ __launch_bounds__(kBlockThreads) void FillI32Kernel(int32_t *__restrict__ p, int64_t n, int32_t v)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlockThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; i < n; i += stride) {
+        p[i] = v;
+    }
+}
+
+// ------------------------------------------------------------------- scan
+
+// Exclusive scan of one value per thread over the workgroup; *total gets the sum.
+__device__ __forceinline__ int32_t BlockExclusiveScan(int32_t v, int32_t *waveSums /* [4] in LDS */, int32_t *total)
+{
+    const int32_t lane = threadIdx.x % kWave;
+    const int32_t wave = threadIdx.x / kWave;
+    int32_t incl = v;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const int32_t up = __shfl_up(incl, off, kWave);
+        if (lane >= off) {
+            incl += up;
+        }
+    }
+    if (lane == kWave - 1) {
+        waveSums[wave] = incl;
+    }
+    __syncthreads();
+    int32_t base = 0, all = 0;
+#pragma unroll
+    for (int w = 0; w < kBlockThreads / kWave; ++w) {
+        const int32_t s = waveSums[w];
+        base += (w < wave) ? s : 0;
+        all += s;
+    }
+    __syncthreads();  // waveSums may be reused by the caller's next call
+    *total = all;
+    return base + incl - v;
+}
+
+__global__ __launch_bounds__(kBlockThreads) void ScanTileSumsKernel(const int32_t *__restrict__ in, int64_t n,
+                                                                   int32_t *__restrict__ tileSums)
+{
+    __shared__ int32_t waveSums[kBlockThreads / kWave];
+    const int64_t base = static_cast<int64_t>(blockIdx.x) * kScanTile;
+    int32_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < kScanItems; ++i) {
+        const int64_t p = base + i * kBlockThreads + threadIdx.x;
+        sum += p < n ? in[p] : 0;
+    }
+    int32_t total;
+    (void)BlockExclusiveScan(sum, waveSums, &total);
+    if (threadIdx.x == 0) {
+        tileSums[blockIdx.x] = total;
+    }
+}
+
+// One workgroup: tileSums[i] <- sum of tileSums[0..i).
+__global__ __launch_bounds__(kBlockThreads) void ScanTileOffsetsKernel(int32_t *__restrict__ tileSums, int64_t numTiles)
+{
+    __shared__ int32_t waveSums[kBlockThreads / kWave];
+    int32_t carry = 0;
+    for (int64_t c0 = 0; c0 < numTiles; c0 += kBlockThreads) {
+        const int64_t p = c0 + threadIdx.x;
+        const int32_t v = p < numTiles ? tileSums[p] : 0;
+        int32_t total;
+        const int32_t excl = BlockExclusiveScan(v, waveSums, &total);
+        if (p < numTiles) {
+            tileSums[p] = carry + excl;
+        }
+        carry += total;
+    }
+}
+
+// out[i] = add + in[0] + ... + in[i]; out may be in.
+__global__ __launch_bounds__(kBlockThreads) void ScanApplyKernel(const int32_t *in, int32_t *out, int64_t n,
+                                                                const int32_t *__restrict__ tileOffsets, int32_t add)
+{
+    __shared__ int32_t waveSums[kBlockThreads / kWave];
+    const int64_t first = static_cast<int64_t>(blockIdx.x) * kScanTile + static_cast<int64_t>(threadIdx.x) * kScanItems;
+    int32_t v[kScanItems];
+    int32_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < kScanItems; ++i) {
+        v[i] = first + i < n ? in[first + i] : 0;
+        sum += v[i];
+        v[i] = sum;  // inclusive within the thread
+    }
+    int32_t total;
+    const int32_t before = BlockExclusiveScan(sum, waveSums, &total) + tileOffsets[blockIdx.x] + add;
+#pragma unroll
+    for (int i = 0; i < kScanItems; ++i) {
+        if (first + i < n) {
+            out[first + i] = before + v[i];
+        }
+    }
+}
+
+// ---------------------------------------------------------------- coo2csr
+
+// counts[r + 1] += number of entries with row r (rows outside [0, m) are
+// skipped, as the golden does).  A thread reads consecutive entries and adds a
+// whole run of equal rows with one atomic, so sorted input costs about one
+// atomic per distinct row and thread.
+__global__ __launch_bounds__(kBlockThreads) void CountRunsKernel(const int32_t *__restrict__ ind, int64_t nnz,
+                                                                int64_t m, int32_t base, int32_t *counts)
+{
+    constexpr int kItems = 8;
+    const int64_t first = (static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x) * kItems;
+    int32_t runRow = -1, runLen = 0;
+#pragma unroll
+    for (int i = 0; i < kItems; ++i) {
+        if (first + i < nnz) {
+            // unsigned subtraction, like the reference kernel: no signed overflow on hostile input
+            const int32_t r = static_cast<int32_t>(static_cast<uint32_t>(LoadStream(ind + first + i)) -
+                                                   static_cast<uint32_t>(base));
+            if (r == runRow) {
+                ++runLen;
+            } else {
+                if (runLen > 0 && runRow >= 0 && runRow < m) {
+                    atomicAdd(counts + runRow + 1, runLen);
+                }
+                runRow = r;
+                runLen = 1;
+            }
+        }
+    }
+    if (runLen > 0 && runRow >= 0 && runRow < m) {
+        atomicAdd(counts + runRow + 1, runLen);
+    }
+}
+
+// ---------------------------------------------------------------- csr2coo
+
+// A wavefront takes 64 consecutive rows.  Rows of up to 16 entries are written
+// by their own lane; a longer row is written by the whole wavefront, 64
+// consecutive entries per store.  A row whose bounds do not describe a range
+// inside [0, nnz) is skipped (csr2coo_golden.h:51-53).
+__global__ __launch_bounds__(kBlockThreads) void ExpandRowsKernel(const int32_t *__restrict__ rowPtr, int64_t m,
+                                                                 int64_t nnz, int32_t base,
+                                                                 int32_t *__restrict__ rowInd)
+{
+    const int32_t lane = threadIdx.x % kWave;
+    const int64_t row = (static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x);
+    int64_t lo = 0, hi = 0;
+    if (row < m) {
+        lo = static_cast<int64_t>(rowPtr[row]) - base;
+        hi = static_cast<int64_t>(rowPtr[row + 1]) - base;
+        if (lo < 0 || hi > nnz || lo > hi) {
+            lo = hi = 0;
+        }
+    }
+    const int32_t value = static_cast<int32_t>(row) + base;
+    const int64_t len = hi - lo;
+    if (len <= 16) {
+        for (int64_t j = 0; j < len; ++j) {
+            rowInd[lo + j] = value;
+        }
+    }
+    uint64_t longRows = __ballot(len > 16);
+    while (longRows != 0) {
+        const int32_t src = __ffsll(static_cast<long long>(longRows)) - 1;
+        longRows &= longRows - 1;
+        const int64_t l = __shfl(lo, src, kWave);
+        const int64_t h = __shfl(hi, src, kWave);
+        const int32_t v = __shfl(value, src, kWave);
+        for (int64_t p = l + lane; p < h; p += kWave) {
+            rowInd[p] = v;
+        }
+    }
+}
+
+// ------------------------------------------------------------- radix sort
+
+// Digit of a key for the pass at `shift`.
+__device__ __forceinline__ int32_t RadixDigit(int32_t key, int32_t shift)
+{
+    return static_cast<int32_t>((static_cast<uint32_t>(key) >> shift) & (kRadixDigits - 1));
+}
+
+// table[1 + digit * numTiles + tile] = items of that digit in the tile
+// (table[0] stays 0: an inclusive scan of the table then leaves, at the same
+// place shifted down by one, the first output position of every (digit, tile)).
+__global__ __launch_bounds__(kBlockThreads) void RadixCountKernel(const int32_t *__restrict__ keys, int64_t n,
+                                                                 int32_t keyBase, int32_t shift,
+                                                                 int32_t *__restrict__ table, int64_t numTiles)
+{
+    __shared__ int32_t hist[kRadixDigits];
+    if (threadIdx.x < kRadixDigits) {
+        hist[threadIdx.x] = 0;
+    }
+    __syncthreads();
+    const int64_t first = static_cast<int64_t>(blockIdx.x) * kRadixTile + static_cast<int64_t>(threadIdx.x) * kRadixItems;
+#pragma unroll
+    for (int i = 0; i < kRadixItems; ++i) {
+        if (first + i < n) {
+            atomicAdd(&hist[RadixDigit(keys[first + i] - keyBase, shift)], 1);
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < kRadixDigits) {
+        table[1 + static_cast<int64_t>(threadIdx.x) * numTiles + blockIdx.x] = hist[threadIdx.x];
+    }
+}
+
+// Exclusive scan, digit-major, of the 16 x 256 per-thread digit counters of a
+// workgroup.  counters[d * 256 + t] holds thread t's count of digit d on entry
+// and the number of items that sort before thread t's first item of digit d on
+// exit.
+__device__ __forceinline__ void ScanDigitCounters(int32_t *counters, int32_t *waveSums)
+{
+    constexpr int kPer = kRadixDigits;  // 4096 counters / 256 threads
+    int32_t v[kPer];
+    int32_t sum = 0;
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+        v[i] = counters[threadIdx.x * kPer + i];
+        sum += v[i];
+    }
+    int32_t total;
+    int32_t run = BlockExclusiveScan(sum, waveSums, &total);
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+        counters[threadIdx.x * kPer + i] = run;
+        run += v[i];
+    }
+    __syncthreads();
+}
+
+// One pass: items of tile `blockIdx.x` go to prefix[digit][tile] + their rank
+// among the tile's items of the same digit.  payloadIn == NULL means "the
+// payload of item i is i" (first pass).  keyBase is subtracted from the keys
+// read (first pass: the index base of the column indices) and the keys are
+// written without it.
+__global__ __launch_bounds__(kBlockThreads) void RadixScatterKernel(
+    const int32_t *__restrict__ keysIn, const int32_t *__restrict__ payloadIn, int32_t *__restrict__ keysOut,
+    int32_t *__restrict__ payloadOut, int64_t n, int32_t keyBase, int32_t shift, const int32_t *__restrict__ prefix,
+    int64_t numTiles)
+{
+    __shared__ int32_t counters[kRadixDigits * kBlockThreads];
+    __shared__ int32_t waveSums[kBlockThreads / kWave];
+    const int64_t first = static_cast<int64_t>(blockIdx.x) * kRadixTile + static_cast<int64_t>(threadIdx.x) * kRadixItems;
+    int32_t key[kRadixItems], pay[kRadixItems], dig[kRadixItems];
+    int32_t cnt[kRadixDigits];
+#pragma unroll
+    for (int d = 0; d < kRadixDigits; ++d) {
+        cnt[d] = 0;
+    }
+#pragma unroll
+    for (int i = 0; i < kRadixItems; ++i) {
+        dig[i] = -1;
+        if (first + i < n) {
+            key[i] = keysIn[first + i] - keyBase;
+            pay[i] = payloadIn != nullptr ? payloadIn[first + i] : static_cast<int32_t>(first + i);
+            dig[i] = RadixDigit(key[i], shift);
+#pragma unroll
+            for (int d = 0; d < kRadixDigits; ++d) {
+                cnt[d] += (dig[i] == d) ? 1 : 0;
+            }
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < kRadixDigits; ++d) {
+        counters[d * kBlockThreads + threadIdx.x] = cnt[d];
+    }
+    __syncthreads();
+    ScanDigitCounters(counters, waveSums);
+#pragma unroll
+    for (int i = 0; i < kRadixItems; ++i) {
+        if (dig[i] >= 0) {
+            // rank inside the tile among items of this digit: the thread's base for the digit, less the
+            // digit's own start, plus the thread's earlier items of the digit
+            int32_t earlier = 0;
+#pragma unroll
+            for (int j = 0; j < kRadixItems; ++j) {
+                earlier += (j < i && dig[j] == dig[i]) ? 1 : 0;
+            }
+            const int32_t inTile = counters[dig[i] * kBlockThreads + threadIdx.x] - counters[dig[i] * kBlockThreads] + earlier;
+            const int64_t dst = static_cast<int64_t>(prefix[static_cast<int64_t>(dig[i]) * numTiles + blockIdx.x]) + inTile;
+            keysOut[dst] = key[i];
+            payloadOut[dst] = pay[i];
+        }
+    }
+}
+
+// ---------------------------------------------------------------- csr2csc
+
+// cscRowInd[d] = row of source position pos[d] (+ base); cscVal[d] = csrVal[pos[d]].
+template <typename T>
+__global__ __launch_bounds__(kBlockThreads) void GatherByPositionKernel(const int32_t *__restrict__ pos,
+                                                                       const int32_t *__restrict__ rowOfPos,
+                                                                       const T *__restrict__ srcVal, int64_t nnz,
+                                                                       int32_t *__restrict__ rowOut,
+                                                                       T *__restrict__ valOut)
+{
+    const int64_t d = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
+    if (d >= nnz) {
+        return;
+    }
+    const int32_t p = LoadStream(pos + d);
+    rowOut[d] = rowOfPos[p];
+    if (valOut != nullptr) {
+        valOut[d] = srcVal[p];
+    }
+}
+
+// ---------------------------------------------------------------- csrsort
+
+// Orders by signed column first, position in the row second.
+__device__ __forceinline__ uint64_t SortKey(int32_t col, uint32_t idx)
+{
+    return (static_cast<uint64_t>(static_cast<uint32_t>(col) ^ 0x80000000u) << 32) | idx;
+}
+__device__ __forceinline__ int32_t SortKeyColumn(uint64_t key)
+{
+    return static_cast<int32_t>(static_cast<uint32_t>(key >> 32) ^ 0x80000000u);
+}
+
+// One wavefront per row: rows of 2..64 entries are sorted in registers (bitonic
+// network over the 64 lanes); longer rows are appended to `list`.
+__global__ __launch_bounds__(kBlockThreads) void SortShortRowsKernel(const int32_t *__restrict__ rowPtr, int64_t m,
+                                                                    int64_t nnz, int32_t base, int32_t *colInd,
+                                                                    int32_t *perm, int32_t *listCount,
+                                                                    int32_t *__restrict__ list)
+{
+    const int32_t lane = threadIdx.x % kWave;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * (kBlockThreads / kWave) + threadIdx.x / kWave;
+    if (row >= m) {
+        return;
+    }
+    const int64_t begin = static_cast<int64_t>(rowPtr[row]) - base;
+    const int64_t end = static_cast<int64_t>(rowPtr[row + 1]) - base;
+    const int64_t len = end - begin;
+    if (len <= 1 || begin < 0 || end > nnz) {
+        return;
+    }
+    if (len > kSortWaveRow) {
+        if (lane == 0) {
+            list[atomicAdd(listCount, 1)] = static_cast<int32_t>(row);
+        }
+        return;
+    }
+    const bool valid = lane < len;
+    uint64_t key = ~0ull;  // padding sorts last
+    int32_t pay = 0;
+    if (valid) {
+        key = SortKey(colInd[begin + lane], static_cast<uint32_t>(lane));
+        pay = perm[begin + lane];
+    }
+#pragma unroll
+    for (int k = 2; k <= kWave; k <<= 1) {
+#pragma unroll
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            const uint64_t other = __shfl_xor(key, j, kWave);
+            const bool ascending = (lane & k) == 0;
+            const bool lower = (lane & j) == 0;
+            const bool takeMin = ascending == lower;
+            const uint64_t mn = key < other ? key : other;
+            const uint64_t mx = key < other ? other : key;
+            key = takeMin ? mn : mx;
+        }
+    }
+    const int32_t from = static_cast<int32_t>(key & 0xffffffffu) & (kWave - 1);
+    const int32_t movedPay = __shfl(pay, from, kWave);
+    if (valid) {
+        colInd[begin + lane] = SortKeyColumn(key);
+        perm[begin + lane] = movedPay;
+    }
+}
+
+// Workgroups walk the list of rows longer than 64 entries.  Up to 2048 entries:
+// bitonic sort of the keys in LDS.  Longer: a workgroup-local radix sort, four
+// bits a pass, between the row and its place in the scratch arrays; thread t
+// owns the t-th contiguous part of the row, so the same counter scan as in
+// RadixScatterKernel keeps it stable.
+__global__ __launch_bounds__(kBlockThreads) void SortListedRowsKernel(const int32_t *__restrict__ rowPtr, int32_t base,
+                                                                     int32_t keyBits, int32_t *colInd, int32_t *perm,
+                                                                     int32_t *tmpCol, int32_t *tmpPerm,
+                                                                     const int32_t *__restrict__ listCount,
+                                                                     const int32_t *__restrict__ list)
+{
+    __shared__ uint64_t keys[kSortLdsRow];                          // 16 KB, doubles as the radix counters
+    __shared__ int32_t pays[kSortLdsRow];
+    __shared__ int32_t waveSums[kBlockThreads / kWave];
+    static_assert(sizeof(uint64_t) * kSortLdsRow >= sizeof(int32_t) * kRadixDigits * kBlockThreads, "counter space");
+    int32_t *counters = reinterpret_cast<int32_t *>(keys);
+
+    const int32_t count = *listCount;
+    for (int32_t item = blockIdx.x; item < count; item += gridDim.x) {
+        const int32_t row = list[item];
+        const int64_t begin = static_cast<int64_t>(rowPtr[row]) - base;
+        const int64_t len = static_cast<int64_t>(rowPtr[row + 1]) - base - begin;
+        if (len <= kSortLdsRow) {
+            int32_t npad = 128;
+            while (npad < len) {
+                npad <<= 1;
+            }
+            for (int32_t i = threadIdx.x; i < npad; i += kBlockThreads) {
+                keys[i] = i < len ? SortKey(colInd[begin + i], static_cast<uint32_t>(i)) : ~0ull;
+                pays[i] = i < len ? perm[begin + i] : 0;
+            }
+            __syncthreads();
+            for (int32_t k = 2; k <= npad; k <<= 1) {
+                for (int32_t j = k >> 1; j > 0; j >>= 1) {
+                    for (int32_t i = threadIdx.x; i < npad; i += kBlockThreads) {
+                        const int32_t partner = i ^ j;
+                        if (partner > i) {
+                            const uint64_t a = keys[i], b = keys[partner];
+                            const bool ascending = (i & k) == 0;
+                            if ((a > b) == ascending) {
+                                keys[i] = b;
+                                keys[partner] = a;
+                            }
+                        }
+                    }
+                    __syncthreads();
+                }
+            }
+            for (int32_t i = threadIdx.x; i < len; i += kBlockThreads) {
+                const uint64_t key = keys[i];
+                colInd[begin + i] = SortKeyColumn(key);
+                perm[begin + i] = pays[static_cast<uint32_t>(key & 0xffffffffu)];
+            }
+            __syncthreads();
+            continue;
+        }
+        // Radix passes over [begin, begin + len), thread t on entries [t * part, (t + 1) * part).
+        const int64_t part = (len + kBlockThreads - 1) / kBlockThreads;
+        const int64_t lo = begin + threadIdx.x * part < begin + len ? begin + threadIdx.x * part : begin + len;
+        const int64_t hi = lo + part < begin + len ? lo + part : begin + len;
+        int32_t *srcCol = colInd, *srcPerm = perm, *dstCol = tmpCol, *dstPerm = tmpPerm;
+        for (int32_t shift = 0; shift < keyBits; shift += kRadixBits) {
+            int32_t cnt[kRadixDigits];
+#pragma unroll
+            for (int d = 0; d < kRadixDigits; ++d) {
+                cnt[d] = 0;
+            }
+            for (int64_t p = lo; p < hi; ++p) {
+                const int32_t dg = RadixDigit(srcCol[p] - base, shift);
+#pragma unroll
+                for (int d = 0; d < kRadixDigits; ++d) {
+                    cnt[d] += (dg == d) ? 1 : 0;
+                }
+            }
+#pragma unroll
+            for (int d = 0; d < kRadixDigits; ++d) {
+                counters[d * kBlockThreads + threadIdx.x] = cnt[d];
+            }
+            __syncthreads();
+            ScanDigitCounters(counters, waveSums);
+#pragma unroll
+            for (int d = 0; d < kRadixDigits; ++d) {
+                cnt[d] = counters[d * kBlockThreads + threadIdx.x];  // next output slot of digit d for this thread
+            }
+            for (int64_t p = lo; p < hi; ++p) {
+                const int32_t c = srcCol[p];
+                const int32_t dg = RadixDigit(c - base, shift);
+                int32_t slot = 0;
+#pragma unroll
+                for (int d = 0; d < kRadixDigits; ++d) {
+                    if (dg == d) {
+                        slot = cnt[d]++;
+                    }
+                }
+                dstCol[begin + slot] = c;
+                dstPerm[begin + slot] = srcPerm[p];
+            }
+            __threadfence_block();
+            __syncthreads();
+            int32_t *t = srcCol;
+            srcCol = dstCol;
+            dstCol = t;
+            t = srcPerm;
+            srcPerm = dstPerm;
+            dstPerm = t;
+        }
+        if (srcCol != colInd) {  // an odd number of passes left the result in the scratch arrays
+            for (int64_t p = begin + threadIdx.x; p < begin + len; p += kBlockThreads) {
+                colInd[p] = srcCol[p];
+                perm[p] = srcPerm[p];
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// =============================================================== host side
+
+namespace {
+
+inline int CheckLaunch()
+{
+    return hipGetLastError() == hipSuccess ? OPSPARSE_OK : OPSPARSE_E_LAUNCH;
+}
+
+inline int64_t Align256(int64_t v) { return (v + 255) / 256 * 256; }
+
+inline uint32_t GridFor(int64_t items, int64_t perBlock, int64_t cap = INT32_MAX)
+{
+    int64_t g = (items + perBlock - 1) / perBlock;
+    g = g < 1 ? 1 : g;
+    return static_cast<uint32_t>(g > cap ? cap : g);
+}
+
+inline int64_t ScanTiles(int64_t count) { return (count + kScanTile - 1) / kScanTile; }
+
+// out[i] = add + in[0..i]; `tiles` holds ScanTiles(count) ints.
+void LaunchInclusiveScan(const int32_t *in, int32_t *out, int64_t count, int32_t add, int32_t *tiles, hipStream_t s)
+{
+    if (count <= 0) {
+        return;
+    }
+    const int64_t numTiles = ScanTiles(count);
+    hipLaunchKernelGGL(ScanTileSumsKernel, dim3(static_cast<uint32_t>(numTiles)), dim3(kBlockThreads), 0, s, in, count,
+                       tiles);
+    hipLaunchKernelGGL(ScanTileOffsetsKernel, dim3(1), dim3(kBlockThreads), 0, s, tiles, numTiles);
+    hipLaunchKernelGGL(ScanApplyKernel, dim3(static_cast<uint32_t>(numTiles)), dim3(kBlockThreads), 0, s, in, out,
+                       count, tiles, add);
+}
+
+void LaunchFill(int32_t *p, int64_t n, int32_t v, hipStream_t s)
+{
+    if (n > 0) {
+        hipLaunchKernelGGL(FillI32Kernel, dim3(GridFor(n, kBlockThreads, 8192)), dim3(kBlockThreads), 0, s, p, n, v);
+    }
+}
+
+// ptr[0..m] from sorted (or unsorted) indices: zero, count runs, scan.
+void LaunchIndicesToOffsets(const int32_t *ind, int64_t nnz, int64_t m, int32_t base, int32_t *ptr, int32_t *tiles,
+                            hipStream_t s)
+{
+    LaunchFill(ptr, m + 1, 0, s);
+    if (nnz > 0 && m > 0) {
+        hipLaunchKernelGGL(CountRunsKernel, dim3(GridFor(nnz, kBlockThreads * 8)), dim3(kBlockThreads), 0, s, ind, nnz,
+                           m, base, ptr);
+    }
+    LaunchInclusiveScan(ptr, ptr, m + 1, base, tiles, s);
+}
+
+int32_t KeyBits(int64_t n)
+{
+    int32_t bits = 1;
+    while (bits < 31 && (int64_t{1} << bits) < n) {
+        ++bits;
+    }
+    return bits;
+}
+
+struct Csr2CscLayout {
+    int64_t keysA, keysB, payA, payB, rowOfPos, table, tiles, bytes;
+    int64_t numTiles, tableCount;
+};
+
+Csr2CscLayout LayoutCsr2Csc(int64_t n, int64_t nnz)
+{
+    Csr2CscLayout l{};
+    l.numTiles = (nnz + kRadixTile - 1) / kRadixTile;
+    l.tableCount = static_cast<int64_t>(kRadixDigits) * l.numTiles + 1;
+    int64_t off = 0;
+    const int64_t arr = Align256(4 * nnz);
+    l.keysA = off; off += arr;
+    l.keysB = off; off += arr;
+    l.payA = off; off += arr;
+    l.payB = off; off += arr;
+    l.rowOfPos = off; off += arr;
+    l.table = off; off += Align256(4 * l.tableCount);
+    const int64_t scanCount = l.tableCount > n + 1 ? l.tableCount : n + 1;
+    l.tiles = off; off += Align256(4 * ScanTiles(scanCount));
+    l.bytes = off;
+    return l;
+}
+
+}  // namespace
+}  // namespace opsparse
+
+using namespace opsparse;
+
+extern "C" {
+
+size_t opsparse_scan_workspace_bytes(int64_t count)
+{
+    return count <= 0 ? 0 : static_cast<size_t>(Align256(4 * ScanTiles(count)));
+}
+
+int opsparse_coo2csr_launch(const int32_t *cooRowInd, int64_t nnz, int64_t m, int32_t *csrRowPtr, int32_t indexBase,
+                            void *workspace, size_t workspaceBytes, void *stream)
+{
+    if (nnz < 0 || m < 0 || nnz > INT32_MAX || m >= INT32_MAX || (indexBase != 0 && indexBase != 1) ||
+        csrRowPtr == nullptr || (nnz > 0 && (cooRowInd == nullptr || m == 0))) {
+        return OPSPARSE_E_INVALID;
+    }
+    if (workspace == nullptr || workspaceBytes < opsparse_scan_workspace_bytes(m + 1)) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    LaunchIndicesToOffsets(cooRowInd, nnz, m, indexBase, csrRowPtr, static_cast<int32_t *>(workspace),
+                           static_cast<hipStream_t>(stream));
+    return CheckLaunch();
+}
+
+int opsparse_csr2coo_launch(const int32_t *csrRowPtr, int64_t nnz, int64_t m, int32_t *cooRowInd, int32_t indexBase,
+                            void *stream)
+{
+    if (nnz < 0 || m < 0 || nnz > INT32_MAX || m > INT32_MAX || (indexBase != 0 && indexBase != 1) ||
+        (m == 0 && nnz != 0) || (m > 0 && csrRowPtr == nullptr) || (nnz > 0 && cooRowInd == nullptr)) {
+        return OPSPARSE_E_INVALID;
+    }
+    if (nnz == 0 || m == 0) {
+        return OPSPARSE_OK;
+    }
+    hipLaunchKernelGGL(ExpandRowsKernel, dim3(GridFor(m, kBlockThreads)), dim3(kBlockThreads), 0,
+                       static_cast<hipStream_t>(stream), csrRowPtr, m, nnz, indexBase, cooRowInd);
+    return CheckLaunch();
+}
+
+size_t opsparse_csrsort_workspace_bytes(int64_t m, int64_t nnz)
+{
+    if (m <= 0 || nnz <= 0) {
+        return 0;
+    }
+    return static_cast<size_t>(2 * Align256(4 * nnz) + 256 + Align256(4 * m));
+}
+
+int opsparse_csrsort_launch(int64_t m, int64_t n, int64_t nnz, int32_t indexBase, const int32_t *csrRowPtr,
+                            int32_t *csrColInd, int32_t *perm, void *workspace, size_t workspaceBytes, void *stream)
+{
+    if (m < 0 || n < 0 || nnz < 0 || m > INT32_MAX || nnz > INT32_MAX || (indexBase != 0 && indexBase != 1) ||
+        ((m == 0 || n == 0) && nnz != 0)) {
+        return OPSPARSE_E_INVALID;
+    }
+    if (nnz == 0) {
+        return OPSPARSE_OK;
+    }
+    if (csrRowPtr == nullptr || csrColInd == nullptr || perm == nullptr) {
+        return OPSPARSE_E_INVALID;
+    }
+    if (workspace == nullptr || workspaceBytes < opsparse_csrsort_workspace_bytes(m, nnz)) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    auto s = static_cast<hipStream_t>(stream);
+    auto *base = static_cast<unsigned char *>(workspace);
+    const int64_t arr = Align256(4 * nnz);
+    auto *tmpCol = reinterpret_cast<int32_t *>(base);
+    auto *tmpPerm = reinterpret_cast<int32_t *>(base + arr);
+    auto *listCount = reinterpret_cast<int32_t *>(base + 2 * arr);
+    auto *list = reinterpret_cast<int32_t *>(base + 2 * arr + 256);
+    LaunchFill(listCount, 1, 0, s);
+    hipLaunchKernelGGL(SortShortRowsKernel, dim3(GridFor(m, kBlockThreads / kWave)), dim3(kBlockThreads), 0, s,
+                       csrRowPtr, m, nnz, indexBase, csrColInd, perm, listCount, list);
+    hipLaunchKernelGGL(SortListedRowsKernel, dim3(kSortListBlocks), dim3(kBlockThreads), 0, s, csrRowPtr, indexBase,
+                       KeyBits(n), csrColInd, perm, tmpCol, tmpPerm, listCount, list);
+    return CheckLaunch();
+}
+
+size_t opsparse_csr2csc_workspace_bytes(int64_t m, int64_t n, int64_t nnz)
+{
+    if (m <= 0 || n <= 0 || nnz <= 0) {
+        return 0;
+    }
+    return static_cast<size_t>(LayoutCsr2Csc(n, nnz).bytes);
+}
+
+int opsparse_csr2csc_launch(int64_t m, int64_t n, int64_t nnz, const void *csrVal, const int32_t *csrRowPtr,
+                            const int32_t *csrColInd, void *cscVal, int32_t *cscColPtr, int32_t *cscRowInd,
+                            int32_t valueBytes, int32_t indexBase, void *workspace, size_t workspaceBytes,
+                            void *stream)
+{
+    if (m < 0 || n < 0 || nnz < 0 || m > INT32_MAX || n >= INT32_MAX || nnz > INT32_MAX - indexBase ||
+        (indexBase != 0 && indexBase != 1) || ((m == 0 || n == 0) && nnz != 0) || cscColPtr == nullptr ||
+        (valueBytes != 0 && valueBytes != 1 && valueBytes != 2 && valueBytes != 4)) {
+        return OPSPARSE_E_INVALID;
+    }
+    auto s = static_cast<hipStream_t>(stream);
+    if (nnz == 0) {
+        LaunchFill(cscColPtr, n + 1, indexBase, s);
+        return CheckLaunch();
+    }
+    if (csrRowPtr == nullptr || csrColInd == nullptr || cscRowInd == nullptr ||
+        (valueBytes != 0 && (csrVal == nullptr || cscVal == nullptr))) {
+        return OPSPARSE_E_INVALID;
+    }
+    const Csr2CscLayout l = LayoutCsr2Csc(n, nnz);
+    if (workspace == nullptr || static_cast<int64_t>(workspaceBytes) < l.bytes) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    auto *base = static_cast<unsigned char *>(workspace);
+    auto at = [&](int64_t off) { return reinterpret_cast<int32_t *>(base + off); };
+    int32_t *keys[2] = {at(l.keysA), at(l.keysB)};
+    int32_t *pays[2] = {at(l.payA), at(l.payB)};
+    int32_t *rowOfPos = at(l.rowOfPos), *table = at(l.table), *tiles = at(l.tiles);
+    const auto tileGrid = dim3(static_cast<uint32_t>(l.numTiles));
+
+    // Row index of every source position, with the output's index base.
+    hipLaunchKernelGGL(ExpandRowsKernel, dim3(GridFor(m, kBlockThreads)), dim3(kBlockThreads), 0, s, csrRowPtr, m, nnz,
+                       indexBase, rowOfPos);
+
+    // Stable sort of (column, source position) by column.
+    const int32_t keyBits = KeyBits(n);
+    const int32_t *keysIn = csrColInd;
+    const int32_t *paysIn = nullptr;
+    int32_t keyBase = indexBase;
+    int cur = 0;
+    for (int32_t shift = 0; shift < keyBits; shift += kRadixBits) {
+        LaunchFill(table, 1, 0, s);
+        hipLaunchKernelGGL(RadixCountKernel, tileGrid, dim3(kBlockThreads), 0, s, keysIn, nnz, keyBase, shift, table,
+                           l.numTiles);
+        LaunchInclusiveScan(table, table, l.tableCount, 0, tiles, s);
+        hipLaunchKernelGGL(RadixScatterKernel, tileGrid, dim3(kBlockThreads), 0, s, keysIn, paysIn, keys[cur],
+                           pays[cur], nnz, keyBase, shift, table, l.numTiles);
+        keysIn = keys[cur];
+        paysIn = pays[cur];
+        keyBase = 0;
+        cur ^= 1;
+    }
+
+    // Column offsets from the sorted (zero-based) columns, then rows and values by source position.
+    LaunchFill(cscColPtr, n + 1, 0, s);
+    hipLaunchKernelGGL(CountRunsKernel, dim3(GridFor(nnz, kBlockThreads * 8)), dim3(kBlockThreads), 0, s, keysIn, nnz,
+                       n, 0, cscColPtr);
+    LaunchInclusiveScan(cscColPtr, cscColPtr, n + 1, indexBase, tiles, s);
+    const auto grid = dim3(GridFor(nnz, kBlockThreads));
+    switch (valueBytes) {
+        case 0:
+            hipLaunchKernelGGL(GatherByPositionKernel<uint8_t>, grid, dim3(kBlockThreads), 0, s, paysIn, rowOfPos,
+                               static_cast<const uint8_t *>(nullptr), nnz, cscRowInd, static_cast<uint8_t *>(nullptr));
+            break;
+        case 1:
+            hipLaunchKernelGGL(GatherByPositionKernel<uint8_t>, grid, dim3(kBlockThreads), 0, s, paysIn, rowOfPos,
+                               static_cast<const uint8_t *>(csrVal), nnz, cscRowInd, static_cast<uint8_t *>(cscVal));
+            break;
+        case 2:
+            hipLaunchKernelGGL(GatherByPositionKernel<uint16_t>, grid, dim3(kBlockThreads), 0, s, paysIn, rowOfPos,
+                               static_cast<const uint16_t *>(csrVal), nnz, cscRowInd, static_cast<uint16_t *>(cscVal));
+            break;
+        default:
+            hipLaunchKernelGGL(GatherByPositionKernel<uint32_t>, grid, dim3(kBlockThreads), 0, s, paysIn, rowOfPos,
+                               static_cast<const uint32_t *>(csrVal), nnz, cscRowInd, static_cast<uint32_t *>(cscVal));
+            break;
+    }
+    return CheckLaunch();
+}
+
+}  // extern "C"

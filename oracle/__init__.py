@@ -250,3 +250,54 @@ def ref_fill_dense(seed, n, lo=-2.0, hi=2.0):
 def fnv1a(a):
     a = np.ascontiguousarray(a)
     return int(lib().oracle_fnv1a(_p(a), c_i64(a.nbytes)))
+
+
+# --------------------------------------------------------- CSR producers
+
+def coo2csr(row_ind, m, base=0):
+    row_ind = _c(row_ind, np.int32)
+    out = np.empty(m + 1, np.int32)
+    lib().oracle_coo2csr(_p(row_ind), c_i64(row_ind.size), c_i64(m), c_i32(base), _p(out))
+    return out
+
+
+def csr2coo(rowptr, nnz, base=0):
+    rowptr = _c(rowptr, np.int32)
+    out = np.empty(max(nnz, 0), np.int32)
+    lib().oracle_csr2coo(_p(rowptr), c_i64(rowptr.size - 1), c_i64(nnz), c_i32(base), _p(out))
+    return out
+
+
+def csrsort(rowptr, colind, perm, base=0):
+    rowptr = _c(rowptr, np.int32)
+    c, p = _c(colind, np.int32).copy(), _c(perm, np.int32).copy()
+    lib().oracle_csrsort(_p(rowptr), c_i64(rowptr.size - 1), c_i32(base), _p(c), _p(p))
+    return c, p
+
+
+def csr2csc(m, n, rowptr, colind, val=None, base=0):
+    """(colptr, rowind, cscval); val of any 1 / 2 / 4-byte dtype or None (structure only)."""
+    rowptr, colind = _c(rowptr, np.int32), _c(colind, np.int32)
+    nnz = colind.size
+    colptr, rowind = np.empty(n + 1, np.int32), np.empty(nnz, np.int32)
+    if val is None:
+        lib().oracle_csr2csc(c_i64(m), c_i64(n), c_i64(nnz), c_i32(base), _p(rowptr), _p(colind), None, c_i32(0),
+                             _p(colptr), _p(rowind), None)
+        return colptr, rowind, None
+    val = np.ascontiguousarray(val)
+    out = np.empty_like(val)
+    lib().oracle_csr2csc(c_i64(m), c_i64(n), c_i64(nnz), c_i32(base), _p(rowptr), _p(colind), _p(val),
+                         c_i32(val.dtype.itemsize), _p(colptr), _p(rowind), _p(out))
+    return colptr, rowind, out
+
+
+_ref_conv = None
+
+
+def ref_convert():
+    """The reference's own goldens of the CSR producers (oracle/_ref), or None when not built."""
+    global _ref_conv
+    path = os.path.join(_HERE, "_ref", "libref_convert.so")
+    if _ref_conv is None and os.path.exists(path):
+        _ref_conv = ctypes.CDLL(path)
+    return _ref_conv

@@ -518,3 +518,125 @@ uint64_t oracle_fnv1a(const void *data, int64_t bytes)
     }
     return h;
 }
+
+/* ---------------------------------------------------------- CSR producers
+ * Bit-exact integer / byte operations.  Pinned by: the reference's own goldens
+ * compiled in place (oracle/_ref/libref_convert.so) where present; numpy
+ * (bincount + cumsum, repeat, stable argsort) and scipy's CSR -> CSC on
+ * random inputs; hand-written small cases (tests/test_oracle.py).
+ */
+
+/* Coo2CsrGolden, test/coo2csr/coo2csr_golden.h:44-77: count per row (rows
+ * outside [0, m) ignored, unsigned subtraction of the base), prefix sum + base. */
+void oracle_coo2csr(const int32_t *rowInd, int64_t nnz, int64_t m, int32_t base, int32_t *rowPtr)
+{
+    for (int64_t i = 0; i <= m; ++i) {
+        rowPtr[i] = base;
+    }
+    if (nnz <= 0 || m <= 0) {
+        return;
+    }
+    int32_t *count = (int32_t *)calloc((size_t)m, sizeof(int32_t));
+    for (int64_t k = 0; k < nnz; ++k) {
+        const int32_t row = (int32_t)((uint32_t)rowInd[k] - (uint32_t)base);
+        if (row >= 0 && row < m) {
+            ++count[row];
+        }
+    }
+    int64_t run = 0;
+    for (int64_t i = 0; i < m; ++i) {
+        run += count[i];
+        rowPtr[i + 1] = (int32_t)(run + base);
+    }
+    free(count);
+}
+
+/* Csr2CooGolden, test/csr2coo/csr2coo_golden.h:37-61: rowInd zero-filled, row i
+ * written over [rowPtr[i], rowPtr[i+1]) - base; a row whose bounds leave
+ * [0, nnz] or run backwards is skipped. */
+void oracle_csr2coo(const int32_t *rowPtr, int64_t m, int64_t nnz, int32_t base, int32_t *rowInd)
+{
+    memset(rowInd, 0, sizeof(int32_t) * (size_t)(nnz > 0 ? nnz : 0));
+    for (int64_t i = 0; i < m; ++i) {
+        const int64_t s = (int64_t)rowPtr[i] - base, e = (int64_t)rowPtr[i + 1] - base;
+        if (s < 0 || e > nnz || s > e) {
+            continue;
+        }
+        for (int64_t j = s; j < e; ++j) {
+            rowInd[j] = (int32_t)i + base;
+        }
+    }
+}
+
+/* csrsortGolden, test/csrsort/arch35/csrsort_golden.h:38-70: per row a stable
+ * ascending sort of the (signed) column indices, perm moved the same way.
+ * Stable insertion into a merge: plain bottom-up merge sort on index pairs. */
+void oracle_csrsort(const int32_t *rowPtr, int64_t m, int32_t base, int32_t *colInd, int32_t *perm)
+{
+    for (int64_t r = 0; r < m; ++r) {
+        const int64_t b = (int64_t)rowPtr[r] - base, len = (int64_t)rowPtr[r + 1] - base - b;
+        if (len <= 1) {
+            continue;
+        }
+        int32_t *block = (int32_t *)malloc(sizeof(int32_t) * (size_t)len * 4);
+        int32_t *c0 = block, *p0 = c0 + len, *c1 = p0 + len, *p1 = c1 + len;
+        memcpy(c0, colInd + b, sizeof(int32_t) * (size_t)len);
+        memcpy(p0, perm + b, sizeof(int32_t) * (size_t)len);
+        for (int64_t w = 1; w < len; w *= 2) {
+            for (int64_t lo = 0; lo < len; lo += 2 * w) {
+                const int64_t mid = lo + w < len ? lo + w : len, hi = lo + 2 * w < len ? lo + 2 * w : len;
+                int64_t i = lo, j = mid, k = lo;
+                while (i < mid && j < hi) {
+                    if (c0[j] < c0[i]) {          /* strict: equal keys keep the left one first */
+                        c1[k] = c0[j]; p1[k++] = p0[j++];
+                    } else {
+                        c1[k] = c0[i]; p1[k++] = p0[i++];
+                    }
+                }
+                while (i < mid) { c1[k] = c0[i]; p1[k++] = p0[i++]; }
+                while (j < hi) { c1[k] = c0[j]; p1[k++] = p0[j++]; }
+            }
+            int32_t *t = c0; c0 = c1; c1 = t;
+            t = p0; p0 = p1; p1 = t;
+        }
+        memcpy(colInd + b, c0, sizeof(int32_t) * (size_t)len);
+        memcpy(perm + b, p0, sizeof(int32_t) * (size_t)len);
+        free(block);
+    }
+}
+
+/* Csr2CscGolden, test/csr2csc_ex2/csr2csc_ex2_golden.h:50-110: column counts,
+ * exclusive prefix sum + base, then a row-major walk that drops every entry at
+ * its column's next free slot (so rows ascend inside a column).  Values move
+ * as raw items of valBytes bytes (0: structure only). */
+void oracle_csr2csc(int64_t m, int64_t n, int64_t nnz, int32_t base, const int32_t *rowPtr, const int32_t *colInd,
+                    const void *val, int32_t valBytes, int32_t *colPtr, int32_t *rowInd, void *cscVal)
+{
+    for (int64_t j = 0; j <= n; ++j) {
+        colPtr[j] = base;
+    }
+    if (nnz <= 0) {
+        return;
+    }
+    int32_t *next = (int32_t *)calloc((size_t)n + 1, sizeof(int32_t));
+    for (int64_t k = 0; k < nnz; ++k) {
+        ++next[colInd[k] - base];
+    }
+    for (int64_t j = 0; j < n; ++j) {
+        colPtr[j + 1] = colPtr[j] + next[j];
+    }
+    for (int64_t j = 0; j < n; ++j) {
+        next[j] = colPtr[j] - base;
+    }
+    for (int64_t i = 0; i < m; ++i) {
+        for (int64_t k = (int64_t)rowPtr[i] - base; k < (int64_t)rowPtr[i + 1] - base; ++k) {
+            const int32_t dest = next[colInd[k] - base]++;
+            rowInd[dest] = (int32_t)i + base;
+            if (valBytes > 0) {
+                memcpy((unsigned char *)cscVal + (size_t)dest * valBytes, (const unsigned char *)val + (size_t)k * valBytes,
+                       (size_t)valBytes);
+            }
+        }
+    }
+    free(next);
+}

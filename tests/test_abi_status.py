@@ -397,3 +397,94 @@ def test_spmvop_status_table(osa, L, handle):
         L.aclsparseDestroyDnVec(v)
     for m in (A, big, E):
         L.aclsparseDestroySpMat(m)
+
+
+# ------------------------------------------------------------ CSR producers
+
+def test_matdescr(osa, L):
+    """reference sparse/common/aclsparse_matdescr.cpp:25-110."""
+    assert L.aclsparseCreateMatDescr(None) == st(osa, "INVALID_VALUE")
+    d = ctypes.c_void_p(None)
+    assert L.aclsparseCreateMatDescr(ctypes.byref(d)) == 0 and d.value
+    assert (L.aclsparseGetMatType(d), L.aclsparseGetMatIndexBase(d), L.aclsparseGetMatDiagType(d),
+            L.aclsparseGetMatFillMode(d)) == (0, 0, 0, 0)
+    L.aclsparseSetMatType(d, 3)
+    L.aclsparseSetMatIndexBase(d, 1)
+    L.aclsparseSetMatDiagType(d, 1)
+    L.aclsparseSetMatFillMode(d, 1)
+    assert (L.aclsparseGetMatType(d), L.aclsparseGetMatIndexBase(d), L.aclsparseGetMatDiagType(d),
+            L.aclsparseGetMatFillMode(d)) == (3, 1, 1, 1)
+    L.aclsparseSetMatIndexBase(None, 1)                       # ignored
+    assert L.aclsparseGetMatIndexBase(None) == 0
+    assert L.aclsparseDestroyMatDescr(d) == 0 and L.aclsparseDestroyMatDescr(None) == 0
+
+
+def test_conversion_status_table(osa, L, handle):
+    """reference coo2csr_host.cpp:38-80, csr2coo_host.cpp:66-115, csrsort_host.cpp:53-74 / :146-221,
+    csr2csc_ex2_host.cpp:109-232 / :535-618."""
+    INV, NS, HN = st(osa, "INVALID_VALUE"), st(osa, "NOT_SUPPORTED"), st(osa, "HANDLE_IS_NULLPTR")
+    IMAX = 2 ** 31 - 1
+    # coo2csr
+    c = L.aclsparseXcoo2csr
+    assert c(None, FAKE, 4, 4, FAKE, 0) == HN
+    assert c(handle, FAKE, -1, 4, FAKE, 0) == INV and c(handle, FAKE, IMAX, 4, FAKE, 1) == INV
+    assert c(handle, FAKE, 4, -1, FAKE, 0) == INV and c(handle, FAKE, 4, 0, FAKE, 0) == INV
+    assert c(handle, FAKE, 4, 4, FAKE, 2) == INV
+    assert c(handle, None, 4, 4, FAKE, 0) == INV and c(handle, FAKE, 4, 4, None, 0) == INV
+    # csr2coo: its null-handle code is NOT_INITIALIZED
+    r = L.aclsparseXcsr2coo
+    assert r(None, FAKE, 4, 4, FAKE, 0) == st(osa, "NOT_INITIALIZED")
+    assert r(handle, FAKE, -1, 4, FAKE, 0) == INV and r(handle, FAKE, 4, -1, FAKE, 0) == INV
+    assert r(handle, FAKE, 4, 0, FAKE, 0) == INV and r(handle, FAKE, 4, 4, FAKE, 7) == INV
+    assert r(handle, None, 4, 4, FAKE, 0) == INV and r(handle, FAKE, 4, 4, None, 0) == INV
+    assert r(handle, FAKE, 2 ** 31, 4, FAKE, 0) == INV and r(handle, FAKE, 4, 2 ** 31, FAKE, 0) == INV
+    assert r(handle, FAKE, 0, 4, None, 0) == 0 and r(handle, None, 0, 0, None, 1) == 0
+    # csrsort
+    n = ctypes.c_size_t(99)
+    bs = L.aclsparseXcsrsort_bufferSizeExt
+    assert bs(None, 4, 4, 5, FAKE, FAKE, ctypes.byref(n)) == HN
+    assert bs(handle, 4, 4, 5, FAKE, FAKE, None) == INV
+    for bad in ((-1, 4, 5), (4, -1, 5), (4, 4, -1), (0, 4, 5), (4, 0, 5)):
+        assert bs(handle, *bad, FAKE, FAKE, ctypes.byref(n)) == INV, bad
+    assert bs(handle, 4, 4, 5, None, FAKE, ctypes.byref(n)) == INV
+    assert bs(handle, 4, 4, 5, FAKE, None, ctypes.byref(n)) == INV
+    assert bs(handle, 4, 4, 0, FAKE, None, ctypes.byref(n)) == 0 and n.value == 0
+    assert bs(handle, 4, 4, 5, FAKE, FAKE, ctypes.byref(n)) == 0 and n.value == L.opsparse_csrsort_workspace_bytes(4, 5)
+    assert n.value >= 2 * 5 * 4                                   # at least the reference's 2 * nnz ints
+    d = ctypes.c_void_p(None)
+    L.aclsparseCreateMatDescr(ctypes.byref(d))
+    so = L.aclsparseXcsrsort
+    assert so(None, 4, 4, 5, d, FAKE, FAKE, FAKE, FAKE) == HN
+    assert so(handle, 4, 4, -5, d, FAKE, FAKE, FAKE, FAKE) == INV and so(handle, 0, 4, 5, d, FAKE, FAKE, FAKE, FAKE) == INV
+    assert so(handle, 4, 4, 5, d, None, FAKE, FAKE, FAKE) == INV and so(handle, 4, 4, 5, d, FAKE, None, FAKE, FAKE) == INV
+    assert so(handle, 4, 4, 5, None, FAKE, FAKE, FAKE, FAKE) == INV
+    L.aclsparseSetMatIndexBase(d, 5)
+    assert so(handle, 4, 4, 5, d, FAKE, FAKE, FAKE, FAKE) == INV
+    L.aclsparseSetMatIndexBase(d, 1)
+    assert so(handle, 4, 4, 0, d, FAKE, None, None, None) == 0       # nothing to sort
+    assert so(handle, 4, 4, 5, d, FAKE, FAKE, None, FAKE) == INV and so(handle, 4, 4, 5, d, FAKE, FAKE, FAKE, None) == INV
+    L.aclsparseDestroyMatDescr(d)
+    # csr2csc
+    F, NUM, SYM = osa.ACL_FLOAT, osa.ACL_SPARSE_ACTION_NUMERIC, osa.ACL_SPARSE_ACTION_SYMBOLIC
+    ptrs = (FAKE, FAKE, FAKE, FAKE, FAKE, FAKE)
+    cb = lambda h=handle, m=4, n_=4, nnz=5, p=ptrs, vt=F, cv=NUM, base=0, alg=0, out=ctypes.byref(n): \
+        L.aclsparseCsr2cscEx2_bufferSize(h, m, n_, nnz, *p, vt, cv, base, alg, out)
+    assert cb(h=None) == HN
+    assert cb(m=-1) == INV and cb(n_=-1) == INV and cb(n_=IMAX) == INV and cb(nnz=-1) == INV
+    assert cb(vt=osa.ACL_DOUBLE) == NS and cb(vt=osa.ACL_INT32) == NS
+    assert cb(cv=2) == INV and cb(base=2) == INV and cb(alg=2) == INV and cb(out=None) == INV
+    assert cb(m=-1, vt=osa.ACL_DOUBLE) == INV                       # sizes are checked before the value type
+    for vt in (F, osa.ACL_FLOAT16, osa.ACL_BF16, osa.ACL_INT8):
+        assert cb(vt=vt) == 0 and n.value == L.opsparse_csr2csc_workspace_bytes(4, 4, 5)
+    assert cb(nnz=0) == 0 and n.value == 0 and cb(m=0, nnz=0) == 0 and n.value == 0
+    cc = lambda h=handle, m=4, n_=4, nnz=5, p=ptrs, vt=F, cv=NUM, base=0, alg=1, buf=FAKE: \
+        L.aclsparseCsr2cscEx2(h, m, n_, nnz, *p, vt, cv, base, alg, buf)
+    assert cc(h=None) == HN and cc(vt=osa.ACL_INT64) == NS and cc(alg=5) == INV
+    for i in range(6):
+        p = list(ptrs)
+        p[i] = None
+        assert cc(p=tuple(p)) == INV, i
+    sym = (None, FAKE, FAKE, None, FAKE, FAKE)                      # SYMBOLIC needs no value arrays ...
+    assert cc(p=sym, cv=NUM) == INV
+    assert cc(m=0, nnz=5) == INV and cc(n_=0, nnz=5) == INV
+    assert cc(nnz=IMAX, base=1) == INV

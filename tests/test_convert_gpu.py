@@ -1,0 +1,306 @@
+"""GPU parity tests of the CSR producers (aclsparseXcoo2csr, aclsparseXcsr2coo, aclsparseXcsrsort,
+aclsparseCsr2cscEx2) through the C ABI.  Every output is compared bit for bit with the CPU oracle.
+
+The coo2csr / csr2coo / csr2csc case tables are the reference's own
+(test/<op>/arch35/<op>_test.csv, kept as data fixtures under tests/golden/); matrices come
+from the reference's fill generator through oracle/_ref where that is built and from a
+numpy generator of the same distribution otherwise.  The csrsort cases restate the inputs of
+test/csrsort/arch35/csrsort_test.cpp:239-650 (that test has no table).
+"""
+import csv
+import ctypes
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import random_csr, to_dev
+
+pytestmark = pytest.mark.gpu
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def load_cases(name):
+    with open(os.path.join(HERE, "golden", name)) as f:
+        return list(csv.DictReader(line for line in f if line.strip() and not line.startswith("#")))
+
+
+def matrix(c, lo=-5.0, hi=5.0):
+    """Zero-based CSR of a case row (test/frame/fill.h generator, or its numpy twin)."""
+    m, n, seed = int(c["m"]), int(c["n"]), int(c["seed"])
+    sparsity = float(c["sparsity"])
+    if c["pattern"] == "diag":
+        return np.arange(m + 1, dtype=np.int32), np.arange(m, dtype=np.int32), np.ones(m, np.float32)
+    if m <= 0 or n <= 0 or sparsity >= 1.0:
+        return np.zeros(max(m, 0) + 1, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32)
+    got = oracle.ref_fill_csr(seed, m, n, -1, sparsity, float(c["empty_row_prob"]), lo, hi)
+    if got is None:
+        got = random_csr(m, n, 1.0 - sparsity, seed, lo, hi, empty_row_prob=float(c["empty_row_prob"]))
+    return got
+
+
+def dev_i32(a, dev):
+    return to_dev(np.ascontiguousarray(a, np.int32), dev)
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() > 0 else None
+
+
+# ------------------------------------------------------------------ coo2csr
+
+COO2CSR = load_cases("coo2csr_cases.csv")
+
+
+@pytest.mark.parametrize("c", COO2CSR, ids=[c["case_name"] for c in COO2CSR])
+def test_coo2csr_reference_table(osa, gpu_ctx, c):
+    dev, stream, handle = gpu_ctx
+    m, base = int(c["m"]), int(c["idx_base"])
+    if c["pattern"] == "allsame":
+        nnz = max(int(m * int(c["n"]) * (1.0 - float(c["sparsity"]))), 1)
+        rows = np.zeros(nnz, np.int32)
+    else:
+        rowptr, colind, _ = matrix(c)
+        rows = oracle.csr2coo(rowptr, colind.size)
+    rows = rows + base
+    d_rows = dev_i32(rows, dev)
+    d_ptr = torch.full((m + 1,), -7, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    rc = osa.lib().aclsparseXcoo2csr(handle.h, ptr(d_rows), rows.size, m, ctypes.c_void_p(d_ptr.data_ptr()), base)
+    assert rc == 0
+    stream.synchronize()
+    assert np.array_equal(d_ptr.cpu().numpy(), oracle.coo2csr(rows, m, base))
+    assert np.array_equal(d_rows.cpu().numpy(), rows)
+
+
+@pytest.mark.parametrize("m,nnz,base", [(1, 1, 0), (5_000_000, 3_000_000, 1), (1000, 4_000_000, 0), (2049, 0, 1),
+                                        (4_194_304, 20_000_000, 0)])
+def test_coo2csr_large_and_unsorted(osa, gpu_ctx, m, nnz, base):
+    """Sizes around the scan tile and far above it; a second run on shuffled input must still equal the
+    count-based golden (coo2csr_golden.h:57-66 counts, it does not search)."""
+    dev, stream, handle = gpu_ctx
+    rng = np.random.default_rng(m + nnz)
+    rows = np.sort(rng.integers(0, m, nnz)).astype(np.int32) + base
+    for shuffled in (False, True):
+        if shuffled:
+            rng.shuffle(rows)
+            rows[: min(5, nnz)] = m + base + 3          # out of range: not counted
+        d_rows = dev_i32(rows, dev)
+        d_ptr = torch.empty(m + 1, dtype=torch.int32, device=dev)
+        torch.cuda.synchronize()
+        assert osa.lib().aclsparseXcoo2csr(handle.h, ptr(d_rows), nnz, m, ctypes.c_void_p(d_ptr.data_ptr()), base) == 0
+        stream.synchronize()
+        assert np.array_equal(d_ptr.cpu().numpy(), oracle.coo2csr(rows, m, base))
+
+
+# ------------------------------------------------------------------ csr2coo
+
+CSR2COO = load_cases("csr2coo_cases.csv")
+
+
+@pytest.mark.parametrize("c", CSR2COO, ids=[c["case_name"] for c in CSR2COO])
+def test_csr2coo_reference_table(osa, gpu_ctx, c):
+    dev, stream, handle = gpu_ctx
+    m, n, base = int(c["m"]), int(c["n"]), int(c["idx_base"])
+    rowptr, colind, val = matrix(c) if c["pattern"] != "csc" else matrix(dict(c, pattern="random"))
+    if c["pattern"] == "csc":                       # the column offsets of the same matrix, expanded to column indices
+        rowptr, _, _ = oracle.csr2csc(m, n, rowptr, colind, val)
+        m = n
+    nnz = int(rowptr[-1])
+    rowptr = rowptr + base
+    d_ptr = dev_i32(rowptr, dev)
+    d_rows = torch.full((nnz,), -7, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    assert osa.lib().aclsparseXcsr2coo(handle.h, ptr(d_ptr), nnz, m, ptr(d_rows), base) == 0
+    stream.synchronize()
+    assert np.array_equal(d_rows.cpu().numpy(), oracle.csr2coo(rowptr, nnz, base))
+
+
+def test_csr2coo_row_length_mix(osa, gpu_ctx):
+    """Rows on both sides of the 16-entry switch, very long rows, runs of empty rows, m not a multiple of 64."""
+    dev, stream, handle = gpu_ctx
+    rng = np.random.default_rng(4)
+    lengths = rng.integers(0, 40, 100_003)
+    lengths[rng.integers(0, lengths.size, 2000)] = 0
+    lengths[[7, 50_000, 100_002]] = [300_000, 17, 65_000]
+    lengths[1000:3000] = 0
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    nnz = int(rowptr[-1])
+    for base in (0, 1):
+        d_ptr = dev_i32(rowptr + base, dev)
+        d_rows = torch.full((nnz,), -7, dtype=torch.int32, device=dev)
+        torch.cuda.synchronize()
+        assert osa.lib().aclsparseXcsr2coo(handle.h, ptr(d_ptr), nnz, lengths.size, ptr(d_rows), base) == 0
+        stream.synchronize()
+        assert np.array_equal(d_rows.cpu().numpy(), oracle.csr2coo(rowptr + base, nnz, base))
+
+
+# ------------------------------------------------------------------ csrsort
+
+def run_csrsort(osa, gpu_ctx, m, n, rowptr, colind, base=0, perm=None, misalign=0):
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    nnz = int(colind.size)
+    perm = np.arange(nnz, dtype=np.int32) if perm is None else perm
+    d_ptr, d_col, d_perm = dev_i32(rowptr, dev), dev_i32(colind, dev), dev_i32(perm, dev)
+    size = ctypes.c_size_t(0)
+    assert L.aclsparseXcsrsort_bufferSizeExt(handle.h, m, n, nnz, ptr(d_ptr), ptr(d_col), ctypes.byref(size)) == 0
+    buf = torch.empty(size.value + 64, dtype=torch.uint8, device=dev)
+    descr = ctypes.c_void_p(None)
+    assert L.aclsparseCreateMatDescr(ctypes.byref(descr)) == 0
+    L.aclsparseSetMatIndexBase(descr, base)
+    torch.cuda.synchronize()
+    rc = L.aclsparseXcsrsort(handle.h, m, n, nnz, descr, ptr(d_ptr), ptr(d_col), ptr(d_perm),
+                             ctypes.c_void_p(buf.data_ptr() + misalign) if nnz else None)
+    assert rc == 0
+    stream.synchronize()
+    L.aclsparseDestroyMatDescr(descr)
+    want_c, want_p = oracle.csrsort(rowptr, colind, perm, base)
+    assert np.array_equal(d_ptr.cpu().numpy(), rowptr)
+    assert np.array_equal(d_col.cpu().numpy(), want_c) and np.array_equal(d_perm.cpu().numpy(), want_p)
+
+
+def _rows(lengths, colfn):
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    col = np.concatenate([np.asarray(colfn(r, int(l)), np.int64) for r, l in enumerate(lengths)] + [np.zeros(0, np.int64)])
+    return rowptr, col.astype(np.int32)
+
+
+def _skewed(row):
+    return 10000 if row % 64 == 0 else 2048 if row % 8 == 0 else (row % 7 if row % 5 != 0 else 0)
+
+
+SORT_CASES = {
+    "Basic": lambda: (3, 3, np.array([0, 3, 6, 9], np.int32), np.array([2, 1, 0, 0, 2, 1, 1, 2, 0], np.int32)),
+    "EmptyRows": lambda: (4, 5, np.array([0, 0, 2, 2, 4], np.int32), np.array([3, 1, 4, 2], np.int32)),
+    "AlreadySorted": lambda: (3, 5, np.array([0, 2, 4, 6], np.int32), np.array([0, 1, 2, 3, 0, 4], np.int32)),
+    "Reverse": lambda: (1, 64, np.array([0, 64], np.int32), np.arange(63, -1, -1, dtype=np.int32)),
+    "DuplicateCols": lambda: (2, 4, np.array([0, 6, 9], np.int32), np.array([3, 1, 3, 1, 0, 3, 2, 2, 2], np.int32)),
+    "EmptyMatrix": lambda: (5, 5, np.zeros(6, np.int32), np.zeros(0, np.int32)),
+    "SingleElemRows": lambda: (4, 9, np.arange(5, dtype=np.int32), np.array([8, 0, 3, 3], np.int32)),
+    "ManySmallRows": lambda: (200, 10) + _rows(np.random.default_rng(99).integers(0, 4, 200),
+                                               lambda r, l: np.random.default_rng(r).integers(0, 10, l)),
+    "MultiCoreSkewedRows": lambda: (257, 4096) + _rows([_skewed(r) for r in range(257)],
+                                                        lambda r, l: (r * 131 + l - np.arange(l)) % 4096),
+    "LongRow": lambda: (1, 1000, np.array([0, 1000], np.int32), np.random.default_rng(123).permutation(1000).astype(np.int32)),
+    "LongRowMultiRun": lambda: (1, 4096, np.array([0, 32768], np.int32),
+                                np.random.default_rng(2026).permutation(np.arange(32768) % 4096).astype(np.int32)),
+    "SingleHugeRow": lambda: (1, 65536, np.array([0, 1 << 20], np.int32),
+                              ((np.arange(1 << 20, dtype=np.uint64) * 65521 + 7919) % 4096).astype(np.int32)),
+    "LargeNnzMultiCoreRows": lambda: (64, 4096) + _rows([16384] * 64, lambda r, l: (r * 131 + l - np.arange(l)) % 4096),
+    "RunBoundaries": lambda: (12, 5000) + _rows([63, 64, 65, 127, 128, 129, 2047, 2048, 2049, 4095, 4096, 4097],
+                                                lambda r, l: np.random.default_rng(r).integers(0, 5000, l)),
+    "AlternatingTinyAndLarge": lambda: (400, 3000) + _rows([1 if r % 2 else 1500 for r in range(400)],
+                                                            lambda r, l: (np.arange(l) * 7919 + r) % 3000),
+}
+
+
+@pytest.mark.parametrize("name", list(SORT_CASES))
+def test_csrsort_reference_cases(osa, gpu_ctx, name):
+    m, n, rowptr, colind = SORT_CASES[name]()
+    run_csrsort(osa, gpu_ctx, m, n, rowptr, colind)
+
+
+def test_csrsort_base1_custom_perm_unaligned_buffer(osa, gpu_ctx):
+    """Base1 / NonIdentityP / NonAlignedBuffer of the reference test in one matrix."""
+    rng = np.random.default_rng(8)
+    m, n = 3000, 70000
+    lengths = rng.integers(0, 100, m)
+    lengths[[5, 2999]] = [5000, 20000]
+    rowptr, colind = _rows(lengths, lambda r, l: rng.integers(0, n, l))
+    perm = rng.integers(-1000, 1000, colind.size).astype(np.int32)
+    run_csrsort(osa, gpu_ctx, m, n, rowptr + 1, colind + 1, base=1, perm=perm, misalign=4)
+
+
+def test_csrsort_many_rows(osa, gpu_ctx):
+    """A million short rows (one wavefront each) with a power-law tail."""
+    rng = np.random.default_rng(9)
+    m, n = 1_000_000, 1_000_000
+    lengths = np.minimum((1.0 / rng.uniform(2e-5, 1.0, m)).astype(np.int64), 50000)
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, n, int(rowptr[-1])).astype(np.int32)
+    run_csrsort(osa, gpu_ctx, m, n, rowptr, colind)
+
+
+# ------------------------------------------------------------------ csr2csc
+
+CSR2CSC = load_cases("csr2csc_cases.csv")
+NP_TYPE = {"FP32": np.float32, "FP16": np.float16, "BF16": np.uint16, "INT8": np.int8}
+
+
+def run_csr2csc(osa, gpu_ctx, m, n, rowptr, colind, val, vt, numeric, base, use_buffer=True):
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    nnz = int(colind.size)
+    acl = {np.dtype(np.float32): osa.ACL_FLOAT, np.dtype(np.float16): osa.ACL_FLOAT16, np.dtype(np.uint16): osa.ACL_BF16,
+           np.dtype(np.int8): osa.ACL_INT8}[np.dtype(vt)]
+    d_ptr, d_col = dev_i32(rowptr, dev), dev_i32(colind, dev)
+    d_val = to_dev(np.ascontiguousarray(val).view(np.int16 if np.dtype(vt).itemsize == 2 else vt), dev)
+    sentinel = 0x55
+    o_val = torch.full((max(nnz, 1) * np.dtype(vt).itemsize,), sentinel, dtype=torch.uint8, device=dev)
+    o_ptr = torch.full((n + 1,), -7, dtype=torch.int32, device=dev)
+    o_row = torch.full((max(nnz, 1),), -7, dtype=torch.int32, device=dev)
+    action = osa.ACL_SPARSE_ACTION_NUMERIC if numeric else osa.ACL_SPARSE_ACTION_SYMBOLIC
+    args = (handle.h, m, n, nnz, ptr(d_val), ptr(d_ptr), ptr(d_col), ctypes.c_void_p(o_val.data_ptr()),
+            ctypes.c_void_p(o_ptr.data_ptr()), ctypes.c_void_p(o_row.data_ptr()), acl, action, base, 0)
+    size = ctypes.c_size_t(0)
+    assert L.aclsparseCsr2cscEx2_bufferSize(*args, ctypes.byref(size)) == 0
+    buf = torch.empty(max(size.value, 16), dtype=torch.uint8, device=dev) if use_buffer else None
+    torch.cuda.synchronize()
+    rc = L.aclsparseCsr2cscEx2(*args, ptr(buf))
+    if not use_buffer and size.value > 4 * 1024 * 1024:
+        assert rc == osa.ACL_SPARSE_STATUS_INSUFFICIENT_RESOURCES   # the handle's 4 MiB workspace cannot hold it
+        return
+    assert rc == 0
+    stream.synchronize()
+    want_ptr, want_row, want_val = oracle.csr2csc(m, n, rowptr, colind, val if numeric else None, base)
+    assert np.array_equal(o_ptr.cpu().numpy(), want_ptr)
+    assert np.array_equal(o_row.cpu().numpy()[:nnz], want_row)
+    got_val = o_val.cpu().numpy()[: nnz * np.dtype(vt).itemsize]
+    if numeric:
+        assert np.array_equal(got_val, np.ascontiguousarray(want_val).view(np.uint8))
+    else:
+        assert np.all(got_val == sentinel)                           # SYMBOLIC leaves cscVal alone
+    assert np.array_equal(d_ptr.cpu().numpy(), rowptr) and np.array_equal(d_col.cpu().numpy(), colind)
+
+
+def _typed(val, name):
+    if name == "INT8":
+        return np.clip(np.rint(val * 20), -128, 127).astype(np.int8)
+    if name == "BF16":
+        return (val.view(np.uint32) >> 16).astype(np.uint16)
+    return val.astype(NP_TYPE[name])
+
+
+@pytest.mark.parametrize("c", CSR2CSC, ids=[c["case_name"] for c in CSR2CSC])
+def test_csr2csc_reference_table(osa, gpu_ctx, c):
+    m, n, base = int(c["m"]), int(c["n"]), int(c["idx_base"])
+    rowptr, colind, val = matrix(c)
+    run_csr2csc(osa, gpu_ctx, m, n, rowptr + base, colind + base, _typed(val, c["val_type"]), NP_TYPE[c["val_type"]],
+                c["copy_values"] == "NUMERIC", base)
+
+
+@pytest.mark.parametrize("m,n,density", [(1, 1, 1.0), (3, 100_000, 0.001), (100_000, 3, 0.5), (20000, 20000, 0.002),
+                                         (1000, 1 << 20, 0.00002), (300, 17, 0.0)])
+def test_csr2csc_shapes_unsorted_duplicates(osa, gpu_ctx, m, n, density):
+    rowptr, colind, val = random_csr(m, n, density, m + n, unsorted=True, duplicates=True, empty_row_prob=0.1)
+    for base in (0, 1):
+        run_csr2csc(osa, gpu_ctx, m, n, rowptr + base, colind + base, val, np.float32, True, base)
+    run_csr2csc(osa, gpu_ctx, m, n, rowptr, colind, val, np.float32, True, 0, use_buffer=False)
+
+
+def test_csr2csc_twice_is_sorted_csr(osa, gpu_ctx):
+    """Size-independent property at a large size: CSR -> CSC -> CSR equals the row-sorted matrix (checked against
+    csrsort on the GPU and the oracle on the host)."""
+    m, n = 400_000, 300_000
+    rng = np.random.default_rng(12)
+    lengths = rng.integers(0, 30, m)
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, n, int(rowptr[-1])).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    run_csr2csc(osa, gpu_ctx, m, n, rowptr, colind, val, np.float32, True, 0)
+    colptr, rowind, cval = oracle.csr2csc(m, n, rowptr, colind, val)
+    run_csr2csc(osa, gpu_ctx, n, m, colptr, rowind, cval, np.float32, True, 0)
+    run_csrsort(osa, gpu_ctx, m, n, rowptr, colind)
