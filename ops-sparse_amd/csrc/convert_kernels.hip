@@ -143,34 +143,35 @@ __global__ __launch_bounds__(kBlockThreads) void ScanApplyKernel(const int32_t *
 // ---------------------------------------------------------------- coo2csr
 
 // counts[r + 1] += number of entries with row r (rows outside [0, m) are
-// skipped, as the golden does).  A thread reads consecutive entries and adds a
-// whole run of equal rows with one atomic, so sorted input costs about one
-// atomic per distinct row and thread.
+// skipped, as the golden does).  A wavefront reads 64 consecutive entries at a
+// time; the first lane of every run of equal rows adds the run's length with
+// one atomic, so sorted input costs about one atomic per distinct row and
+// unsorted input still counts correctly.
 __global__ __launch_bounds__(kBlockThreads) void CountRunsKernel(const int32_t *__restrict__ ind, int64_t nnz,
                                                                 int64_t m, int32_t base, int32_t *counts)
 {
-    constexpr int kItems = 8;
-    const int64_t first = (static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x) * kItems;
-    int32_t runRow = -1, runLen = 0;
+    constexpr int kRounds = 8;
+    const int32_t lane = threadIdx.x % kWave;
+    const int64_t wave = static_cast<int64_t>(blockIdx.x) * (kBlockThreads / kWave) + threadIdx.x / kWave;
+    const int64_t first = wave * (kWave * kRounds);
 #pragma unroll
-    for (int i = 0; i < kItems; ++i) {
-        if (first + i < nnz) {
-            // unsigned subtraction, like the reference kernel: no signed overflow on hostile input
-            const int32_t r = static_cast<int32_t>(static_cast<uint32_t>(LoadStream(ind + first + i)) -
-                                                   static_cast<uint32_t>(base));
-            if (r == runRow) {
-                ++runLen;
-            } else {
-                if (runLen > 0 && runRow >= 0 && runRow < m) {
-                    atomicAdd(counts + runRow + 1, runLen);
-                }
-                runRow = r;
-                runLen = 1;
-            }
+    for (int r = 0; r < kRounds; ++r) {
+        const int64_t p = first + r * kWave + lane;
+        const bool valid = p < nnz;
+        // unsigned subtraction, like the reference kernel: no signed overflow on hostile input
+        const int32_t row = valid ? static_cast<int32_t>(static_cast<uint32_t>(LoadStream(ind + p)) -
+                                                         static_cast<uint32_t>(base))
+                                  : -1;
+        const int32_t prev = __shfl_up(row, 1, kWave);
+        const bool head = valid && (lane == 0 || prev != row);
+        const uint64_t heads = __ballot(head);
+        const uint64_t valids = __ballot(valid);
+        if (head && row >= 0 && row < m) {
+            // the run ends in front of the next head, or with the last valid lane
+            const uint64_t later = lane == kWave - 1 ? 0 : (heads >> (lane + 1)) << (lane + 1);
+            const int32_t end = later != 0 ? __ffsll(static_cast<long long>(later)) - 1 : __popcll(valids);
+            atomicAdd(counts + row + 1, end - lane);
         }
-    }
-    if (runLen > 0 && runRow >= 0 && runRow < m) {
-        atomicAdd(counts + runRow + 1, runLen);
     }
 }
 
@@ -360,55 +361,96 @@ __device__ __forceinline__ int32_t SortKeyColumn(uint64_t key)
     return static_cast<int32_t>(static_cast<uint32_t>(key >> 32) ^ 0x80000000u);
 }
 
-// One wavefront per row: rows of 2..64 entries are sorted in registers (bitonic
-// network over the 64 lanes); longer rows are appended to `list`.
-__global__ __launch_bounds__(kBlockThreads) void SortShortRowsKernel(const int32_t *__restrict__ rowPtr, int64_t m,
-                                                                    int64_t nnz, int32_t base, int32_t *colInd,
-                                                                    int32_t *perm, int32_t *listCount,
-                                                                    int32_t *__restrict__ list)
+// Bitonic sort of one (key, payload) per lane over the G lanes of a group; `g` is
+// the lane's index in its group.  Returns the sorted key; *pay follows its key.
+template <int G>
+__device__ __forceinline__ uint64_t GroupBitonicSort(uint64_t key, int32_t *pay, int32_t g)
 {
     const int32_t lane = threadIdx.x % kWave;
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * (kBlockThreads / kWave) + threadIdx.x / kWave;
-    if (row >= m) {
-        return;
-    }
-    const int64_t begin = static_cast<int64_t>(rowPtr[row]) - base;
-    const int64_t end = static_cast<int64_t>(rowPtr[row + 1]) - base;
-    const int64_t len = end - begin;
-    if (len <= 1 || begin < 0 || end > nnz) {
-        return;
-    }
-    if (len > kSortWaveRow) {
-        if (lane == 0) {
-            list[atomicAdd(listCount, 1)] = static_cast<int32_t>(row);
-        }
-        return;
-    }
-    const bool valid = lane < len;
-    uint64_t key = ~0ull;  // padding sorts last
-    int32_t pay = 0;
-    if (valid) {
-        key = SortKey(colInd[begin + lane], static_cast<uint32_t>(lane));
-        pay = perm[begin + lane];
-    }
 #pragma unroll
-    for (int k = 2; k <= kWave; k <<= 1) {
+    for (int k = 2; k <= G; k <<= 1) {
 #pragma unroll
         for (int j = k >> 1; j > 0; j >>= 1) {
             const uint64_t other = __shfl_xor(key, j, kWave);
-            const bool ascending = (lane & k) == 0;
-            const bool lower = (lane & j) == 0;
-            const bool takeMin = ascending == lower;
+            const bool ascending = (g & k) == 0;
+            const bool lower = (g & j) == 0;
             const uint64_t mn = key < other ? key : other;
             const uint64_t mx = key < other ? other : key;
-            key = takeMin ? mn : mx;
+            key = (ascending == lower) ? mn : mx;
         }
     }
-    const int32_t from = static_cast<int32_t>(key & 0xffffffffu) & (kWave - 1);
-    const int32_t movedPay = __shfl(pay, from, kWave);
+    // the low half of a key is the lane (in the group) its entry came from
+    const int32_t from = (lane - g) + (static_cast<int32_t>(key & 0xffffffffu) & (G - 1));
+    *pay = __shfl(*pay, from, kWave);
+    return key;
+}
+
+template <int G>
+__device__ __forceinline__ void SortRowInGroup(int64_t begin, int64_t len, int32_t g, int32_t *colInd, int32_t *perm)
+{
+    const bool valid = g < len;
+    uint64_t key = ~0ull;  // padding sorts last
+    int32_t pay = 0;
     if (valid) {
-        colInd[begin + lane] = SortKeyColumn(key);
-        perm[begin + lane] = movedPay;
+        key = SortKey(colInd[begin + g], static_cast<uint32_t>(g));
+        pay = perm[begin + g];
+    }
+    key = GroupBitonicSort<G>(key, &pay, g);
+    if (valid) {
+        colInd[begin + g] = SortKeyColumn(key);
+        perm[begin + g] = pay;
+    }
+}
+
+// A group of G lanes per row: rows of 2..G entries are sorted in registers (bitonic
+// network over the group's lanes); rows of up to 64 entries that do not fit the
+// group go to midList (one wavefront each, next kernel), longer rows to longList.
+// counters[0] / counters[1] are the two list lengths.
+template <int G>
+__global__ __launch_bounds__(kBlockThreads) void SortShortRowsKernel(const int32_t *__restrict__ rowPtr, int64_t m,
+                                                                    int64_t nnz, int32_t base, int32_t *colInd,
+                                                                    int32_t *perm, int32_t *counters,
+                                                                    int32_t *__restrict__ midList,
+                                                                    int32_t *__restrict__ longList)
+{
+    const int32_t g = threadIdx.x % G;
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * (kBlockThreads / G) + threadIdx.x / G;
+    int64_t begin = 0, len = 0;
+    if (row < m) {
+        begin = static_cast<int64_t>(rowPtr[row]) - base;
+        len = static_cast<int64_t>(rowPtr[row + 1]) - base - begin;
+        if (len <= 1 || begin < 0 || begin + len > nnz) {
+            len = 0;  // nothing to sort, or bounds that do not describe a range of the arrays
+        }
+    }
+    if (len > G) {
+        if (g == 0) {
+            if (len <= kSortWaveRow) {
+                midList[atomicAdd(counters, 1)] = static_cast<int32_t>(row);
+            } else {
+                longList[atomicAdd(counters + 1, 1)] = static_cast<int32_t>(row);
+            }
+        }
+        len = 0;
+    }
+    // every lane takes part in the shuffles; groups without a row sort padding
+    SortRowInGroup<G>(begin, len, g, colInd, perm);
+}
+
+// Wavefronts walk midList: rows of up to 64 entries, one wavefront each.
+__global__ __launch_bounds__(kBlockThreads) void SortMidRowsKernel(const int32_t *__restrict__ rowPtr, int32_t base,
+                                                                  int32_t *colInd, int32_t *perm,
+                                                                  const int32_t *__restrict__ counters,
+                                                                  const int32_t *__restrict__ midList)
+{
+    const int32_t lane = threadIdx.x % kWave;
+    const int32_t count = counters[0];
+    const int32_t wavesInGrid = gridDim.x * (kBlockThreads / kWave);
+    for (int32_t item = blockIdx.x * (kBlockThreads / kWave) + threadIdx.x / kWave; item < count; item += wavesInGrid) {
+        const int32_t row = midList[item];
+        const int64_t begin = static_cast<int64_t>(rowPtr[row]) - base;
+        const int64_t len = static_cast<int64_t>(rowPtr[row + 1]) - base - begin;
+        SortRowInGroup<kWave>(begin, len, lane, colInd, perm);
     }
 }
 
@@ -420,7 +462,7 @@ __global__ __launch_bounds__(kBlockThreads) void SortShortRowsKernel(const int32
 __global__ __launch_bounds__(kBlockThreads) void SortListedRowsKernel(const int32_t *__restrict__ rowPtr, int32_t base,
                                                                      int32_t keyBits, int32_t *colInd, int32_t *perm,
                                                                      int32_t *tmpCol, int32_t *tmpPerm,
-                                                                     const int32_t *__restrict__ listCount,
+                                                                     const int32_t *__restrict__ listCounts,
                                                                      const int32_t *__restrict__ list)
 {
     __shared__ uint64_t keys[kSortLdsRow];                          // 16 KB, doubles as the radix counters
@@ -429,7 +471,7 @@ __global__ __launch_bounds__(kBlockThreads) void SortListedRowsKernel(const int3
     static_assert(sizeof(uint64_t) * kSortLdsRow >= sizeof(int32_t) * kRadixDigits * kBlockThreads, "counter space");
     int32_t *counters = reinterpret_cast<int32_t *>(keys);
 
-    const int32_t count = *listCount;
+    const int32_t count = listCounts[1];
     for (int32_t item = blockIdx.x; item < count; item += gridDim.x) {
         const int32_t row = list[item];
         const int64_t begin = static_cast<int64_t>(rowPtr[row]) - base;
@@ -661,7 +703,7 @@ size_t opsparse_csrsort_workspace_bytes(int64_t m, int64_t nnz)
     if (m <= 0 || nnz <= 0) {
         return 0;
     }
-    return static_cast<size_t>(2 * Align256(4 * nnz) + 256 + Align256(4 * m));
+    return static_cast<size_t>(2 * Align256(4 * nnz) + 256 + 2 * Align256(4 * m));
 }
 
 int opsparse_csrsort_launch(int64_t m, int64_t n, int64_t nnz, int32_t indexBase, const int32_t *csrRowPtr,
@@ -685,13 +727,38 @@ int opsparse_csrsort_launch(int64_t m, int64_t n, int64_t nnz, int32_t indexBase
     const int64_t arr = Align256(4 * nnz);
     auto *tmpCol = reinterpret_cast<int32_t *>(base);
     auto *tmpPerm = reinterpret_cast<int32_t *>(base + arr);
-    auto *listCount = reinterpret_cast<int32_t *>(base + 2 * arr);
-    auto *list = reinterpret_cast<int32_t *>(base + 2 * arr + 256);
-    LaunchFill(listCount, 1, 0, s);
-    hipLaunchKernelGGL(SortShortRowsKernel, dim3(GridFor(m, kBlockThreads / kWave)), dim3(kBlockThreads), 0, s,
-                       csrRowPtr, m, nnz, indexBase, csrColInd, perm, listCount, list);
+    auto *counters = reinterpret_cast<int32_t *>(base + 2 * arr);
+    auto *midList = reinterpret_cast<int32_t *>(base + 2 * arr + 256);
+    auto *longList = reinterpret_cast<int32_t *>(base + 2 * arr + 256 + Align256(4 * m));
+    LaunchFill(counters, 2, 0, s);
+    // Lanes per row from the mean row length: twice the mean, a power of two in [8, 64].
+    const int64_t mean2 = 2 * nnz / m;
+    const int g = mean2 <= 8 ? 8 : mean2 <= 16 ? 16 : mean2 <= 32 ? 32 : 64;
+    const auto shortGrid = dim3(GridFor(m, kBlockThreads / g));
+    switch (g) {
+        case 8:
+            hipLaunchKernelGGL(SortShortRowsKernel<8>, shortGrid, dim3(kBlockThreads), 0, s, csrRowPtr, m, nnz,
+                               indexBase, csrColInd, perm, counters, midList, longList);
+            break;
+        case 16:
+            hipLaunchKernelGGL(SortShortRowsKernel<16>, shortGrid, dim3(kBlockThreads), 0, s, csrRowPtr, m, nnz,
+                               indexBase, csrColInd, perm, counters, midList, longList);
+            break;
+        case 32:
+            hipLaunchKernelGGL(SortShortRowsKernel<32>, shortGrid, dim3(kBlockThreads), 0, s, csrRowPtr, m, nnz,
+                               indexBase, csrColInd, perm, counters, midList, longList);
+            break;
+        default:
+            hipLaunchKernelGGL(SortShortRowsKernel<64>, shortGrid, dim3(kBlockThreads), 0, s, csrRowPtr, m, nnz,
+                               indexBase, csrColInd, perm, counters, midList, longList);
+            break;
+    }
+    if (g < kSortWaveRow) {
+        hipLaunchKernelGGL(SortMidRowsKernel, dim3(kSortListBlocks), dim3(kBlockThreads), 0, s, csrRowPtr, indexBase,
+                           csrColInd, perm, counters, midList);
+    }
     hipLaunchKernelGGL(SortListedRowsKernel, dim3(kSortListBlocks), dim3(kBlockThreads), 0, s, csrRowPtr, indexBase,
-                       KeyBits(n), csrColInd, perm, tmpCol, tmpPerm, listCount, list);
+                       KeyBits(n), csrColInd, perm, tmpCol, tmpPerm, counters, longList);
     return CheckLaunch();
 }
 
