@@ -146,6 +146,8 @@ def main():
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-preprocess", action="store_true", help="SpMV without the Preprocess buffer")
+    ap.add_argument("--panels", action="store_true",
+                    help="SpMV with ACL_SPARSE_SPMV_CSR_ALG2: column-panel layout built by Preprocess (c3)")
     ap.add_argument("--gather-probe", action="store_true", help="also measure random-gather rates (stderr)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -159,6 +161,7 @@ def main():
     wl = importlib.import_module("ops_sparse_amd.workloads")
     dev = torch.device("cuda:0")
     stream = torch.cuda.Stream(device=dev)
+    torch.cuda.set_stream(stream)  # torch's fills / uploads and the library's kernels on one stream, in order
     handle = osa.Handle(stream)
 
     t_gen = time.perf_counter()
@@ -184,7 +187,8 @@ def main():
         x = cfg["x"]
         y = cfg["y0"].clone()
         X, Y = osa.DnVec(x), osa.DnVec(y)
-        op = osa.SpmvOp(handle, csr, X, Y, preprocess=not args.no_preprocess)
+        op = osa.SpmvOp(handle, csr, X, Y, preprocess=not args.no_preprocess,
+                        alg=osa.ACL_SPARSE_SPMV_CSR_ALG2 if args.panels else osa.ACL_SPARSE_SPMV_ALG_DEFAULT)
         ncols = 1
         bytes_alg = wl.spmv_bytes_alg(rows, cols, nnz, vb, x.element_size(), y.element_size(), cfg["beta"] != 0)
         bytes_gather = wl.spmv_bytes_gather(rows, cols, nnz, vb, x.element_size(), y.element_size(),
@@ -237,7 +241,7 @@ def main():
         "dtype": dtype, "data": "synthetic",
         "config": {"workload": cfg["name"], "rows": rows, "cols": cols, "nnz": nnz, "ncols_dense": ncols,
                    "alpha": alpha, "beta": beta, "index": "int32", "preprocess_ms": round(preprocess_ms, 3),
-                   "preprocessed": not args.no_preprocess},
+                   "preprocessed": not args.no_preprocess, "column_panels": bool(args.panels)},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
                      "traffic": load_traffic(cfg["name"]) if args.scale == 1.0 else None,

@@ -59,8 +59,13 @@ typedef enum OpsparseSpmvKernel {
     OPSPARSE_SPMV_STREAM_ROWS = 2, /* short rows: fixed row blocks, products staged in LDS,
                                       one or a few lanes per row */
     OPSPARSE_SPMV_VECTOR_ROWS = 3, /* medium rows: a 4..64-lane group per row, shuffle reduction */
-    OPSPARSE_SPMV_MERGE_PATH = 4   /* skewed rows: equal (rows + nnz) per workgroup, carry-out fix-up */
+    OPSPARSE_SPMV_MERGE_PATH = 4,  /* skewed rows: equal (rows + nnz) per workgroup, carry-out fix-up */
+    OPSPARSE_SPMV_COLUMN_PANELS = 5 /* x larger than an L2: the matrix re-stored as panels of 2^20 columns, each
+                                      worked on one XCD so that its slice of x stays in that L2; fp32 only; holds a
+                                      copy of the VALUES as they were at analysis time */
 } OpsparseSpmvKernel;
+
+#define OPSPARSE_SPMV_MAX_PANELS 16
 
 /* Result of analysing one CSR matrix; plain data, safe to copy. */
 typedef struct OpsparseSpmvPlan {
@@ -70,14 +75,15 @@ typedef struct OpsparseSpmvPlan {
     int32_t mergeBlocks;   /* MERGE_PATH: number of workgroups == partition entries - 1 */
     int32_t maxRowNnz;     /* longest row */
     int32_t partitionReady;/* MERGE_PATH: partition table already in the workspace */
-    int32_t reserved0;     /* unused, zero */
-    int32_t reserved1;
+    int32_t numPanels;     /* COLUMN_PANELS: number of column panels */
+    int32_t panelShift;    /* COLUMN_PANELS: log2 of the panel width */
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */
     int64_t carryOff;
     int64_t headOff;
     int64_t bytes;         /* workspace bytes this plan uses */
+    int64_t panelStart[OPSPARSE_SPMV_MAX_PANELS + 1]; /* COLUMN_PANELS: first entry of every panel */
 } OpsparseSpmvPlan;
 
 /* Bytes opsparse_spmv_csr_analyse / _launch may touch in `workspace`. */
@@ -104,6 +110,19 @@ int opsparse_spmv_csr_launch(const OpsparseSpmvPlan *plan, int32_t transpose, co
                              int64_t cols, int64_t nnz, OpsparseScalar alpha, OpsparseScalar beta, int32_t valType,
                              int32_t outType, int32_t computeIsInt, void *workspace, size_t workspaceBytes,
                              void *stream);
+
+/*
+ * COLUMN_PANELS analysis (fp32, op(A) = A): bytes of the workspace, or 0 when the
+ * family does not apply (it needs 2..16 panels of 2^20 columns, i.e. 1 M < cols <= 16 M).
+ * The analysis re-stores the matrix — column indices AND values — in the
+ * workspace, panel by panel; launches with the resulting plan read that copy and
+ * ignore the rowOffsets / colInd / csrValues arguments, so the analysis must be
+ * repeated after the values change.  Synchronises `stream` once.
+ */
+size_t opsparse_spmv_csr_panels_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz);
+int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
+                                     int64_t rows, int64_t cols, int64_t nnz, void *workspace, size_t workspaceBytes,
+                                     OpsparseSpmvPlan *plan, void *stream);
 
 /* Same as opsparse_spmv_csr_launch with separate input and output vectors:
  * z = alpha * op(A) * x + beta * yIn.  z may be yIn (in place); yIn is only read

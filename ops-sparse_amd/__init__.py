@@ -35,6 +35,7 @@ ACL_SPARSE_ORDER_ROW, ACL_SPARSE_ORDER_COL = 0, 1
 ACL_SPARSE_SPMM_ALG_DEFAULT, ACL_SPARSE_SPMM_CSR_ALG1, ACL_SPARSE_SPMM_CSR_FP32_HIGH_PRECISION_ALG = 0, 1, 2
 # ---- aclsparseSpMVAlg_t
 ACL_SPARSE_SPMV_ALG_DEFAULT, ACL_SPARSE_SPMV_COO_ALG1, ACL_SPARSE_SPMV_CSR_ALG1 = 0, 1, 3
+ACL_SPARSE_SPMV_CSR_ALG2 = 4
 # ---- aclsparseSpMVOpAlg_t
 ACL_SPARSE_SPMVOP_ALG_DEFAULT, ACL_SPARSE_SPMVOP_ALG1, ACL_SPARSE_SPMVOP_ALG2 = 0, 1, 2
 # ---- aclsparseIndexType_t / aclsparseIndexBase_t / aclsparseFormat_t
@@ -57,6 +58,7 @@ STATUS_NAMES = ["SUCCESS", "NOT_INITIALIZED", "ALLOC_FAILED", "INVALID_VALUE", "
 OPSPARSE_F32, OPSPARSE_F16, OPSPARSE_BF16, OPSPARSE_I32, OPSPARSE_I8 = range(5)
 (OPSPARSE_SPMV_AUTO, OPSPARSE_SPMV_SCALE_ONLY, OPSPARSE_SPMV_STREAM_ROWS, OPSPARSE_SPMV_VECTOR_ROWS,
  OPSPARSE_SPMV_MERGE_PATH) = range(5)
+OPSPARSE_SPMV_COLUMN_PANELS = 5
 OPSPARSE_SPMM_AUTO, OPSPARSE_SPMM_ROW_SPLIT, OPSPARSE_SPMM_BINNED = range(3)
 
 # Every symbol the two public headers declare; tests check that the library exports all of them.
@@ -85,6 +87,7 @@ ACL_SPARSE_CSR2CSC_ALG_DEFAULT, ACL_SPARSE_CSR2CSC_ALG1 = 0, 1
 OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_workspace_bytes", "opsparse_spmv_csr_analyse", "opsparse_spmv_csr_launch",
     "opsparse_spmv_csr_launch_zy", "opsparse_spmv_csr_indexed_launch",
+    "opsparse_spmv_csr_panels_workspace_bytes", "opsparse_spmv_csr_panels_analyse",
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
     "opsparse_scan_workspace_bytes", "opsparse_coo2csr_launch", "opsparse_csr2coo_launch",
     "opsparse_csrsort_workspace_bytes", "opsparse_csrsort_launch", "opsparse_csr2csc_workspace_bytes",
@@ -104,9 +107,9 @@ class OpsparseScalar(ctypes.Structure):
 
 class OpsparseSpmvPlan(ctypes.Structure):
     _fields_ = [("kernel", i32), ("lanesPerRow", i32), ("rowsPerBlock", i32), ("mergeBlocks", i32),
-                ("maxRowNnz", i32), ("partitionReady", i32), ("reserved0", i32),
-                ("reserved1", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
-                ("carryOff", i64), ("headOff", i64), ("bytes", i64)]
+                ("maxRowNnz", i32), ("partitionReady", i32), ("numPanels", i32),
+                ("panelShift", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
+                ("carryOff", i64), ("headOff", i64), ("bytes", i64), ("panelStart", i64 * 17)]
 
 
 class OpsparseSpmmPlan(ctypes.Structure):
@@ -223,6 +226,11 @@ def lib():
     L.opsparse_spmv_csr_launch_zy.restype = ctypes.c_int
     L.opsparse_spmv_csr_launch_zy.argtypes = [ctypes.POINTER(OpsparseSpmvPlan), i32, vp, vp, vp, vp, vp, vp, i64, i64,
                                               i64, OpsparseScalar, OpsparseScalar, i32, i32, i32, vp, sz, vp]
+    L.opsparse_spmv_csr_panels_workspace_bytes.restype = sz
+    L.opsparse_spmv_csr_panels_workspace_bytes.argtypes = [i64, i64, i64]
+    L.opsparse_spmv_csr_panels_analyse.restype = ctypes.c_int
+    L.opsparse_spmv_csr_panels_analyse.argtypes = [vp, vp, vp, i64, i64, i64, vp, sz, ctypes.POINTER(OpsparseSpmvPlan),
+                                                   vp]
     L.opsparse_spmv_csr_indexed_launch.restype = ctypes.c_int
     L.opsparse_spmv_csr_indexed_launch.argtypes = [vp, i32, i32, vp, vp, vp, vp, vp, i64, i64, i64, OpsparseScalar,
                                                    OpsparseScalar, vp]

@@ -26,6 +26,7 @@
 //     the stable sort.
 #include <climits>
 
+#include "convert_internal.h"
 #include "device_utils.h"
 
 namespace opsparse {
@@ -611,6 +612,45 @@ void LaunchFill(int32_t *p, int64_t n, int32_t v, hipStream_t s)
     }
 }
 
+}  // namespace
+
+int64_t ScanScratchInts(int64_t count) { return count <= 0 ? 0 : ScanTiles(count); }
+
+void LaunchExpandRows(const int32_t *rowPtr, int64_t m, int64_t nnz, int32_t base, int32_t *rowInd, hipStream_t s)
+{
+    if (m > 0 && nnz > 0) {
+        hipLaunchKernelGGL(ExpandRowsKernel, dim3(GridFor(m, kBlockThreads)), dim3(kBlockThreads), 0, s, rowPtr, m, nnz,
+                           base, rowInd);
+    }
+}
+
+int64_t RadixTiles(int64_t n) { return (n + kRadixTile - 1) / kRadixTile; }
+int64_t RadixTableInts(int64_t n) { return static_cast<int64_t>(kRadixDigits) * RadixTiles(n) + 1; }
+
+void LaunchRadixPass(const int32_t *keysIn, const int32_t *payIn, int32_t *keysOut, int32_t *payOut, int64_t n,
+                     int32_t keyBase, int32_t shift, int32_t *table, int32_t *scratch, hipStream_t s)
+{
+    if (n <= 0) {
+        return;
+    }
+    const int64_t numTiles = RadixTiles(n);
+    const auto grid = dim3(static_cast<uint32_t>(numTiles));
+    LaunchFill(table, 1, 0, s);
+    hipLaunchKernelGGL(RadixCountKernel, grid, dim3(kBlockThreads), 0, s, keysIn, n, keyBase, shift, table, numTiles);
+    LaunchInclusiveScan(table, table, RadixTableInts(n), 0, scratch, s);
+    hipLaunchKernelGGL(RadixScatterKernel, grid, dim3(kBlockThreads), 0, s, keysIn, payIn, keysOut, payOut, n, keyBase,
+                       shift, table, numTiles);
+}
+
+void LaunchGatherByPosition(const int32_t *pos, const int32_t *rowOfPos, const uint32_t *srcVal, int64_t nnz,
+                            int32_t *rowOut, uint32_t *valOut, hipStream_t s)
+{
+    if (nnz > 0) {
+        hipLaunchKernelGGL(GatherByPositionKernel<uint32_t>, dim3(GridFor(nnz, kBlockThreads)), dim3(kBlockThreads), 0,
+                           s, pos, rowOfPos, srcVal, nnz, rowOut, valOut);
+    }
+}
+
 // ptr[0..m] from sorted (or unsorted) indices: zero, count runs, scan.
 void LaunchIndicesToOffsets(const int32_t *ind, int64_t nnz, int64_t m, int32_t base, int32_t *ptr, int32_t *tiles,
                             hipStream_t s)
@@ -622,6 +662,8 @@ void LaunchIndicesToOffsets(const int32_t *ind, int64_t nnz, int64_t m, int32_t 
     }
     LaunchInclusiveScan(ptr, ptr, m + 1, base, tiles, s);
 }
+
+namespace {
 
 int32_t KeyBits(int64_t n)
 {
@@ -798,7 +840,6 @@ int opsparse_csr2csc_launch(int64_t m, int64_t n, int64_t nnz, const void *csrVa
     int32_t *keys[2] = {at(l.keysA), at(l.keysB)};
     int32_t *pays[2] = {at(l.payA), at(l.payB)};
     int32_t *rowOfPos = at(l.rowOfPos), *table = at(l.table), *tiles = at(l.tiles);
-    const auto tileGrid = dim3(static_cast<uint32_t>(l.numTiles));
 
     // Row index of every source position, with the output's index base.
     hipLaunchKernelGGL(ExpandRowsKernel, dim3(GridFor(m, kBlockThreads)), dim3(kBlockThreads), 0, s, csrRowPtr, m, nnz,
@@ -811,12 +852,7 @@ int opsparse_csr2csc_launch(int64_t m, int64_t n, int64_t nnz, const void *csrVa
     int32_t keyBase = indexBase;
     int cur = 0;
     for (int32_t shift = 0; shift < keyBits; shift += kRadixBits) {
-        LaunchFill(table, 1, 0, s);
-        hipLaunchKernelGGL(RadixCountKernel, tileGrid, dim3(kBlockThreads), 0, s, keysIn, nnz, keyBase, shift, table,
-                           l.numTiles);
-        LaunchInclusiveScan(table, table, l.tableCount, 0, tiles, s);
-        hipLaunchKernelGGL(RadixScatterKernel, tileGrid, dim3(kBlockThreads), 0, s, keysIn, paysIn, keys[cur],
-                           pays[cur], nnz, keyBase, shift, table, l.numTiles);
+        LaunchRadixPass(keysIn, paysIn, keys[cur], pays[cur], nnz, keyBase, shift, table, tiles, s);
         keysIn = keys[cur];
         paysIn = pays[cur];
         keyBase = 0;

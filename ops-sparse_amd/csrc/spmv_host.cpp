@@ -42,7 +42,9 @@ aclsparseStatus_t Validate(aclsparseHandle_t handle, aclsparseOperation_t opA, a
     if (matA == nullptr || vecX == nullptr || vecY == nullptr) {
         return ACL_SPARSE_STATUS_INVALID_VALUE;
     }
-    if (alg != ACL_SPARSE_SPMV_ALG_DEFAULT) {
+    // ALG_DEFAULT is the only value the reference accepts (spmv_host.cpp:144-146).  CSR_ALG2 is accepted here
+    // as well: it asks Preprocess for the column-panel layout, which copies the VALUES into the buffer.
+    if (alg != ACL_SPARSE_SPMV_ALG_DEFAULT && alg != ACL_SPARSE_SPMV_CSR_ALG2) {
         return ACL_SPARSE_STATUS_NOT_SUPPORTED;
     }
     if (computeType != ACL_FLOAT && computeType != ACL_INT32) {
@@ -95,6 +97,17 @@ aclsparseStatus_t ValidateData(SpmvCall *c, aclDataType computeType)
     return ACL_SPARSE_STATUS_SUCCESS;
 }
 
+// Bytes of the column-panel layout when CSR_ALG2 asks for it and it applies (fp32, op(A) = A, 2..16 panels).
+size_t PanelBytes(aclsparseOperation_t opA, aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX,
+                  aclsparseConstDnVecDescr_t vecY, aclDataType computeType, aclsparseSpMVAlg_t alg)
+{
+    if (alg != ACL_SPARSE_SPMV_CSR_ALG2 || opA != ACL_SPARSE_OP_NON_TRANSPOSE || computeType != ACL_FLOAT ||
+        matA->valueType != ACL_FLOAT || vecX->valueType != ACL_FLOAT || vecY->valueType != ACL_FLOAT) {
+        return 0;
+    }
+    return opsparse_spmv_csr_panels_workspace_bytes(matA->rows, matA->cols, matA->nnz);
+}
+
 aclsparseStatus_t FromLaunch(int rc)
 {
     switch (rc) {
@@ -123,7 +136,9 @@ aclsparseStatus_t aclsparseSpMVGetBufferSize(aclsparseHandle_t handle, aclsparse
     if (bufferSize == nullptr) {
         return ACL_SPARSE_STATUS_INVALID_VALUE;
     }
-    *bufferSize = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
+    const size_t plain = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
+    const size_t panels = PanelBytes(opA, matA, vecX, vecY, computeType, alg);
+    *bufferSize = panels > plain ? panels : plain;
     return ACL_SPARSE_STATUS_SUCCESS;
 }
 
@@ -148,10 +163,18 @@ aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOpe
         return ACL_SPARSE_STATUS_INSUFFICIENT_RESOURCES;
     }
     OpsparseSpmvPlan plan{};
-    const size_t bytes = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
-    const int rc = opsparse_spmv_csr_analyse(static_cast<const int32_t *>(matA->rowOffsets), matA->rows, matA->cols,
-                                             matA->nnz, externalBuffer, bytes, OPSPARSE_SPMV_AUTO, &plan,
-                                             handle->stream);
+    const size_t panels = PanelBytes(opA, matA, vecX, vecY, computeType, alg);
+    int rc;
+    if (panels > 0) {
+        rc = opsparse_spmv_csr_panels_analyse(static_cast<const int32_t *>(matA->rowOffsets),
+                                              static_cast<const int32_t *>(matA->colInd),
+                                              static_cast<const float *>(matA->values), matA->rows, matA->cols,
+                                              matA->nnz, externalBuffer, panels, &plan, handle->stream);
+    } else {
+        const size_t bytes = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
+        rc = opsparse_spmv_csr_analyse(static_cast<const int32_t *>(matA->rowOffsets), matA->rows, matA->cols,
+                                       matA->nnz, externalBuffer, bytes, OPSPARSE_SPMV_AUTO, &plan, handle->stream);
+    }
     if (rc != OPSPARSE_OK) {
         opsparse::LogError("aclsparseSpMVPreprocess: analysis failed (%d)", rc);
         return FromLaunch(rc);

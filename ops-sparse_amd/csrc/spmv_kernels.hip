@@ -26,6 +26,7 @@
 #include <cstdlib>
 #include <type_traits>
 
+#include "convert_internal.h"
 #include "device_utils.h"
 
 namespace opsparse {
@@ -40,7 +41,13 @@ __device__ __forceinline__ void StoreRow(OutT *y, const OutT *yIn, int64_t row, 
     if (!betaZero) {
         r += beta * ToAcc<AccT>(yIn[row]);
     }
-    y[row] = FromAcc<OutT>(r);
+    if constexpr (std::is_same<OutT, double>::value) {
+        // fp64 outputs are the column panels' partial vectors: written once, read once by the combine
+        // kernel, and they must not push the panel's slice of x out of the L2
+        __builtin_nontemporal_store(r, y + row);
+    } else {
+        y[row] = FromAcc<OutT>(r);
+    }
 }
 
 // Loads 4 consecutive values and converts them to the accumulator type.
@@ -482,6 +489,12 @@ __global__ __launch_bounds__(kBlockThreads) void MergePartitionKernel(const int3
     part[b] = static_cast<int32_t>(lo);
 }
 
+template <typename OutT, typename AccT>
+__device__ __forceinline__ void MergeTileRows(int64_t b, int64_t i0, int64_t i1, int64_t j0, int32_t count,
+                                              const int32_t *__restrict__ rowOffsets, OutT *y, const OutT *yIn,
+                                              int64_t rows, AccT *__restrict__ carry, AccT *__restrict__ head,
+                                              AccT alpha, AccT beta, bool betaZero, const AccT *prod);
+
 // Workgroup b consumes non-zeros [j0, j1) and completes rows [i0, i1), where
 // (i0, j0) and (i1, j1) are the merge-path coordinates of its two diagonals.
 //   - a completed row that started before j0 ("spanning" row, only i0 can be
@@ -490,19 +503,13 @@ __global__ __launch_bounds__(kBlockThreads) void MergePartitionKernel(const int3
 //     in a later workgroup: their sum goes to carry[b];
 //   - every other completed row gets its final y value here.
 template <typename ValT, typename OutT, typename AccT>
-__global__ __launch_bounds__(kBlockThreads) void SpmvMergeKernel(
-    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
-    const ValT *__restrict__ x, OutT *y, const OutT *yIn, int64_t rows, int64_t nnz,
-    const int32_t *__restrict__ part, AccT *__restrict__ carry, AccT *__restrict__ head, OpsparseScalar alphaS,
-    OpsparseScalar betaS)
+__device__ __forceinline__ void MergeTile(int64_t b, const int32_t *__restrict__ rowOffsets,
+                                          const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+                                          const ValT *__restrict__ x, OutT *y, const OutT *yIn, int64_t rows,
+                                          int64_t nnz, const int32_t *__restrict__ part, AccT *__restrict__ carry,
+                                          AccT *__restrict__ head, AccT alpha, AccT beta, bool betaZero,
+                                          AccT *prod /* [kMergeItems] in LDS */)
 {
-    __shared__ AccT prod[kMergeItems];
-
-    const AccT alpha = ReadScalar<AccT>(alphaS);
-    const AccT beta = ReadScalar<AccT>(betaS);
-    const bool betaZero = (beta == AccT(0));
-
-    const int64_t b = XcdContiguousTile(blockIdx.x, gridDim.x);
     const int64_t i0 = part[b];
     const int64_t i1 = part[b + 1];
     const int64_t j0 = MergeDiagonal(b, rows, nnz) - i0;
@@ -515,7 +522,17 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvMergeKernel(
         FinishQuads<ValT, AccT, 2>(q, x, count, prod);
     }
     __syncthreads();
+    MergeTileRows<OutT, AccT>(b, i0, i1, j0, count, rowOffsets, y, yIn, rows, carry, head, alpha, beta, betaZero, prod);
+}
 
+// The row phase of a merge tile: prod[0..count) holds the products of non-zeros
+// j0 .. j0+count-1.
+template <typename OutT, typename AccT>
+__device__ __forceinline__ void MergeTileRows(int64_t b, int64_t i0, int64_t i1, int64_t j0, int32_t count,
+                                              const int32_t *__restrict__ rowOffsets, OutT *y, const OutT *yIn,
+                                              int64_t rows, AccT *__restrict__ carry, AccT *__restrict__ head,
+                                              AccT alpha, AccT beta, bool betaZero, const AccT *prod)
+{
     // Rows i0 .. i1-1 complete here; row i1 (if it exists) collects the tail.
     const int32_t numRows = static_cast<int32_t>(i1 - i0) + (i1 < rows ? 1 : 0);
     if (numRows == 0) {
@@ -531,9 +548,9 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvMergeKernel(
     for (int32_t q = threadIdx.x / g; q < numRows; q += groups) {
         const int64_t row = i0 + q;
         const bool completes = row < i1;
-        const int64_t begin = rowOffsets[row];
+        const int64_t begin = LoadStream(rowOffsets + row);
         const int32_t s = begin > j0 ? static_cast<int32_t>(begin - j0) : 0;
-        const int32_t e = completes ? static_cast<int32_t>(rowOffsets[row + 1] - j0) : count;
+        const int32_t e = completes ? static_cast<int32_t>(LoadStream(rowOffsets + row + 1) - j0) : count;
         AccT sum = AccT(0);
         for (int32_t k = s + lane; k < e; k += g) {
             sum += prod[k];
@@ -551,19 +568,29 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvMergeKernel(
     }
 }
 
-// One lane per workgroup of the merge kernel: if that workgroup completed a
-// spanning row, add the carries of the workgroups the row passed through (in
-// ascending order) to its head piece and write the row's final value.
-template <typename OutT, typename AccT>
-__global__ __launch_bounds__(kBlockThreads) void SpmvMergeFixupKernel(
-    const int32_t *__restrict__ rowOffsets, OutT *y, const OutT *yIn, int64_t rows, int64_t nnz, int32_t numBlocks,
-    const int32_t *__restrict__ part, const AccT *__restrict__ carry, const AccT *__restrict__ head,
-    OpsparseScalar alphaS, OpsparseScalar betaS)
+template <typename ValT, typename OutT, typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmvMergeKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ x, OutT *y, const OutT *yIn, int64_t rows, int64_t nnz,
+    const int32_t *__restrict__ part, AccT *__restrict__ carry, AccT *__restrict__ head, OpsparseScalar alphaS,
+    OpsparseScalar betaS)
 {
-    const int64_t b = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
-    if (b >= numBlocks) {
-        return;
-    }
+    __shared__ AccT prod[kMergeItems];
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    const AccT beta = ReadScalar<AccT>(betaS);
+    MergeTile<ValT, OutT, AccT>(XcdContiguousTile(blockIdx.x, gridDim.x), rowOffsets, colInd, vals, x, y, yIn, rows, nnz,
+                                part, carry, head, alpha, beta, beta == AccT(0), prod);
+}
+
+// Workgroup b of the merge kernel: if it completed a spanning row, add the
+// carries of the workgroups the row passed through (in ascending order) to its
+// head piece and write the row's final value.
+template <typename OutT, typename AccT>
+__device__ __forceinline__ void MergeFixupTile(int64_t b, const int32_t *__restrict__ rowOffsets, OutT *y,
+                                               const OutT *yIn, int64_t rows, int64_t nnz,
+                                               const int32_t *__restrict__ part, const AccT *__restrict__ carry,
+                                               const AccT *__restrict__ head, AccT alpha, AccT beta)
+{
     const int64_t i0 = part[b];
     const int64_t i1 = part[b + 1];
     if (i1 <= i0) {
@@ -583,9 +610,112 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvMergeFixupKernel(
         sum += carry[p];
     }
     sum += head[b];
+    StoreRow<OutT, AccT>(y, yIn, i0, sum, alpha, beta, beta == AccT(0));
+}
+
+// One lane per workgroup of the merge kernel.
+template <typename OutT, typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmvMergeFixupKernel(
+    const int32_t *__restrict__ rowOffsets, OutT *y, const OutT *yIn, int64_t rows, int64_t nnz, int32_t numBlocks,
+    const int32_t *__restrict__ part, const AccT *__restrict__ carry, const AccT *__restrict__ head,
+    OpsparseScalar alphaS, OpsparseScalar betaS)
+{
+    const int64_t b = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
+    if (b >= numBlocks) {
+        return;
+    }
+    MergeFixupTile<OutT, AccT>(b, rowOffsets, y, yIn, rows, nnz, part, carry, head, ReadScalar<AccT>(alphaS),
+                               ReadScalar<AccT>(betaS));
+}
+
+// --------------------------------------------------------- COLUMN_PANELS
+// For matrices whose x does not fit an L2 (4 MB per XCD): the matrix is split at
+// Preprocess into panels of 2^20 columns, each a CSR matrix of its own over all
+// rows, and panel p is worked only by workgroups whose id is p modulo 8 — the
+// hardware deals workgroup ids round-robin to the 8 XCDs, so the 4 MiB slice of
+// x a panel gathers from stays in that XCD's L2 (measured: 181 G gathers/s
+// against 64 G/s for gathers over all of x).  Every panel is a merge-path SpMV
+// into its own fp64 partial vector; a last kernel adds a row's partials in panel
+// order and applies alpha / beta.  Deterministic, no atomics.
+
+struct PanelTable {
+    int64_t start[OPSPARSE_SPMV_MAX_PANELS + 1];  // first entry of every panel in the panel-ordered arrays
+};
+
+__device__ __forceinline__ int64_t PanelTiles(int64_t rows, int64_t nnzP)
+{
+    return (rows + nnzP + kMergeItems - 1) / kMergeItems;
+}
+
+// Workgroup b: panel panelBase + b % 8, merge tile b / 8 of that panel.  (A
+// persistent variant that requested the next tile's entries ahead of the row
+// phase measured slower than letting the hardware schedule one short workgroup
+// per tile: 986 against 859 us on an 8 M x 8 M power-law matrix.)
+template <typename ValT, typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmvPanelMergeKernel(
+    const int32_t *__restrict__ rowPtrP, const int32_t *__restrict__ colIndP, const ValT *__restrict__ valsP,
+    const ValT *__restrict__ x, AccT *__restrict__ ypart, int64_t rows, PanelTable pt, int32_t panelBase,
+    int32_t numPanels, const int32_t *__restrict__ partAll, AccT *__restrict__ carryAll, AccT *__restrict__ headAll,
+    int64_t tileBound)
+{
+    __shared__ AccT prod[kMergeItems];
+    const int32_t p = panelBase + static_cast<int32_t>(blockIdx.x % kNumXcd);
+    const int64_t tile = blockIdx.x / kNumXcd;
+    if (p >= numPanels) {
+        return;
+    }
+    const int64_t nnzP = pt.start[p + 1] - pt.start[p];
+    if (tile >= PanelTiles(rows, nnzP)) {
+        return;
+    }
+    AccT *yp = ypart + static_cast<int64_t>(p) * rows;
+    MergeTile<ValT, AccT, AccT>(tile, rowPtrP + static_cast<int64_t>(p) * (rows + 1), colIndP + pt.start[p],
+                                valsP + pt.start[p], x, yp, yp, rows, nnzP, partAll + static_cast<int64_t>(p) * (tileBound + 1),
+                                carryAll + static_cast<int64_t>(p) * tileBound, headAll + static_cast<int64_t>(p) * tileBound,
+                                AccT(1), AccT(0), true, prod);
+}
+
+// blockIdx.y = panel.
+template <typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmvPanelFixupKernel(const int32_t *__restrict__ rowPtrP,
+                                                                     AccT *__restrict__ ypart, int64_t rows,
+                                                                     PanelTable pt,
+                                                                     const int32_t *__restrict__ partAll,
+                                                                     const AccT *__restrict__ carryAll,
+                                                                     const AccT *__restrict__ headAll,
+                                                                     int64_t tileBound)
+{
+    const int32_t p = blockIdx.y;
+    const int64_t b = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
+    const int64_t nnzP = pt.start[p + 1] - pt.start[p];
+    if (b >= PanelTiles(rows, nnzP)) {
+        return;
+    }
+    AccT *yp = ypart + static_cast<int64_t>(p) * rows;
+    MergeFixupTile<AccT, AccT>(b, rowPtrP + static_cast<int64_t>(p) * (rows + 1), yp, yp, rows, nnzP,
+                               partAll + static_cast<int64_t>(p) * (tileBound + 1),
+                               carryAll + static_cast<int64_t>(p) * tileBound,
+                               headAll + static_cast<int64_t>(p) * tileBound, AccT(1), AccT(0));
+}
+
+// y[r] = alpha * (ypart[0][r] + ... + ypart[P-1][r]) + beta * yIn[r], partials added in panel order.
+template <typename OutT, typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmvPanelCombineKernel(const AccT *__restrict__ ypart,
+                                                                       int32_t numPanels, int64_t rows, OutT *y,
+                                                                       const OutT *yIn, OpsparseScalar alphaS,
+                                                                       OpsparseScalar betaS)
+{
     const AccT alpha = ReadScalar<AccT>(alphaS);
     const AccT beta = ReadScalar<AccT>(betaS);
-    StoreRow<OutT, AccT>(y, yIn, i0, sum, alpha, beta, beta == AccT(0));
+    const bool betaZero = (beta == AccT(0));
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlockThreads;
+    for (int64_t r = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; r < rows; r += stride) {
+        AccT sum = AccT(0);
+        for (int32_t p = 0; p < numPanels; ++p) {
+            sum += LoadStream(ypart + static_cast<int64_t>(p) * rows + r);
+        }
+        StoreRow<OutT, AccT>(y, yIn, r, sum, alpha, beta, betaZero);
+    }
 }
 
 // ------------------------------------------------------------- op(A) = A^T
@@ -783,6 +913,9 @@ int LaunchScale(OutT *y, const OutT *yIn, int64_t len, OpsparseScalar beta, hipS
     return CheckLaunch();
 }
 
+template <typename OutT>
+int LaunchPanels(const SpmvArgs &a, const OpsparseSpmvPlan &plan);
+
 template <typename ValT, typename OutT, typename AccT>
 int RunPlanned(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
 {
@@ -812,9 +945,99 @@ int RunPlanned(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
                 return OPSPARSE_E_WORKSPACE;
             }
             return LaunchMerge<ValT, OutT, AccT>(a, plan);
+        case OPSPARSE_SPMV_COLUMN_PANELS:
+            if constexpr (std::is_same<ValT, float>::value && std::is_same<AccT, double>::value) {
+                return LaunchPanels<OutT>(a, plan);
+            } else {
+                return OPSPARSE_E_UNSUPPORTED;  // the panel copy holds fp32 values
+            }
         default:
             return OPSPARSE_E_INVALID;
     }
+}
+
+// ---- COLUMN_PANELS: workspace layout, preprocessing, launch
+
+constexpr int32_t kPanelShift = 20;  // 2^20 columns = 4 MiB of fp32 x per panel: one XCD's L2
+
+int32_t PanelCount(int64_t cols)
+{
+    return static_cast<int32_t>((cols + (int64_t{1} << kPanelShift) - 1) >> kPanelShift);
+}
+
+struct PanelLayout {
+    int64_t tileBound;  // upper bound of the merge tiles of one panel
+    int64_t rowPtrOff, colIndOff, valsOff, partOff, carryOff, headOff, ypartOff;   // used by every launch
+    int64_t posOff, rowOfPosOff, rowSortedOff, tableOff, scratchOff;               // preprocessing only
+    int64_t bytes;
+};
+
+PanelLayout MakePanelLayout(int64_t rows, int64_t nnz, int32_t numPanels)
+{
+    auto align = [](int64_t v) { return (v + 255) / 256 * 256; };
+    PanelLayout l{};
+    const int64_t P = numPanels;
+    l.tileBound = (rows + nnz + kMergeItems - 1) / kMergeItems + 1;
+    int64_t off = 256;
+    l.rowPtrOff = off; off += align(4 * P * (rows + 1));
+    l.colIndOff = off; off += align(4 * nnz);
+    l.valsOff = off; off += align(4 * nnz);
+    l.partOff = off; off += align(4 * P * (l.tileBound + 1));
+    l.carryOff = off; off += align(8 * P * l.tileBound);
+    l.headOff = off; off += align(8 * P * l.tileBound);
+    l.ypartOff = off; off += align(8 * P * rows);
+    l.posOff = off; off += align(4 * nnz);
+    l.rowOfPosOff = off; off += align(4 * nnz);
+    l.rowSortedOff = off; off += align(4 * nnz);
+    l.tableOff = off; off += align(4 * RadixTableInts(nnz));
+    const int64_t scanA = ScanScratchInts(RadixTableInts(nnz)), scanB = ScanScratchInts(rows + 1);
+    l.scratchOff = off; off += align(4 * (scanA > scanB ? scanA : scanB));
+    l.bytes = off;
+    return l;
+}
+
+template <typename OutT>
+int LaunchPanels(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
+{
+    using AccT = double;
+    const int32_t P = plan.numPanels;
+    const PanelLayout l = MakePanelLayout(a.rows, a.nnz, P);
+    if (a.ws == nullptr || static_cast<int64_t>(a.wsBytes) < l.bytes || plan.bytes != l.bytes) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    auto *base = static_cast<unsigned char *>(a.ws);
+    const auto *rowPtrP = reinterpret_cast<const int32_t *>(base + l.rowPtrOff);
+    const auto *colIndP = reinterpret_cast<const int32_t *>(base + l.colIndOff);
+    const auto *valsP = reinterpret_cast<const float *>(base + l.valsOff);
+    const auto *part = reinterpret_cast<const int32_t *>(base + l.partOff);
+    auto *carry = reinterpret_cast<AccT *>(base + l.carryOff);
+    auto *head = reinterpret_cast<AccT *>(base + l.headOff);
+    auto *ypart = reinterpret_cast<AccT *>(base + l.ypartOff);
+    PanelTable pt{};
+    int64_t maxTiles = 0;
+    for (int32_t p = 0; p <= P; ++p) {
+        pt.start[p] = plan.panelStart[p];
+    }
+    // Panels in groups of 8, one per XCD.
+    for (int32_t panelBase = 0; panelBase < P; panelBase += kNumXcd) {
+        int64_t tiles = 0;
+        for (int32_t p = panelBase; p < P && p < panelBase + kNumXcd; ++p) {
+            const int64_t t = (a.rows + (pt.start[p + 1] - pt.start[p]) + kMergeItems - 1) / kMergeItems;
+            tiles = t > tiles ? t : tiles;
+        }
+        maxTiles = tiles > maxTiles ? tiles : maxTiles;
+        hipLaunchKernelGGL((SpmvPanelMergeKernel<float, AccT>), dim3(static_cast<uint32_t>(tiles * kNumXcd)),
+                           dim3(kBlockThreads), 0, a.stream, rowPtrP, colIndP, valsP, static_cast<const float *>(a.x),
+                           ypart, a.rows, pt, panelBase, P, part, carry, head, l.tileBound);
+    }
+    hipLaunchKernelGGL((SpmvPanelFixupKernel<AccT>), dim3(GridFor(maxTiles, kBlockThreads), static_cast<uint32_t>(P)),
+                       dim3(kBlockThreads), 0, a.stream, rowPtrP, ypart, a.rows, pt, part, carry, head, l.tileBound);
+    int64_t grid = (a.rows + kBlockThreads - 1) / kBlockThreads;
+    grid = grid > 16384 ? 16384 : grid;
+    hipLaunchKernelGGL((SpmvPanelCombineKernel<OutT, AccT>), dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0,
+                       a.stream, ypart, P, a.rows, static_cast<OutT *>(a.y), static_cast<const OutT *>(a.yIn), a.alpha,
+                       a.beta);
+    return CheckLaunch();
 }
 
 int32_t VectorLanesFor(int64_t rows, int64_t nnz)
@@ -1002,6 +1225,87 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
         default:
             return OPSPARSE_E_INVALID;
     }
+    *plan = p;
+    return OPSPARSE_OK;
+}
+
+size_t opsparse_spmv_csr_panels_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz)
+{
+    const int32_t P = PanelCount(cols);
+    if (rows <= 0 || nnz <= 0 || nnz > INT32_MAX || rows >= INT32_MAX || P < 2 || P > OPSPARSE_SPMV_MAX_PANELS) {
+        return 0;
+    }
+    return static_cast<size_t>(MakePanelLayout(rows, nnz, P).bytes);
+}
+
+int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
+                                     int64_t rows, int64_t cols, int64_t nnz, void *workspace, size_t workspaceBytes,
+                                     OpsparseSpmvPlan *plan, void *stream)
+{
+    if (plan == nullptr || rowOffsets == nullptr || colInd == nullptr || csrValues == nullptr) {
+        return OPSPARSE_E_INVALID;
+    }
+    const size_t need = opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz);
+    if (need == 0) {
+        return OPSPARSE_E_UNSUPPORTED;
+    }
+    if (workspace == nullptr || workspaceBytes < need) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    auto s = static_cast<hipStream_t>(stream);
+    const int32_t P = PanelCount(cols);
+    const PanelLayout l = MakePanelLayout(rows, nnz, P);
+    auto *base = static_cast<unsigned char *>(workspace);
+    auto at = [&](int64_t off) { return reinterpret_cast<int32_t *>(base + off); };
+    int32_t *rowPtrP = at(l.rowPtrOff), *colIndP = at(l.colIndOff), *pos = at(l.posOff);
+    int32_t *rowOfPos = at(l.rowOfPosOff), *rowSorted = at(l.rowSortedOff), *table = at(l.tableOff);
+    int32_t *scratch = at(l.scratchOff), *part = at(l.partOff);
+    auto *valsP = reinterpret_cast<uint32_t *>(base + l.valsOff);
+
+    // Entries in (panel, original position) order: one stable radix pass on the panel number.
+    LaunchExpandRows(rowOffsets, rows, nnz, 0, rowOfPos, s);
+    LaunchRadixPass(colInd, nullptr, colIndP, pos, nnz, 0, kPanelShift, table, scratch, s);
+    LaunchGatherByPosition(pos, rowOfPos, reinterpret_cast<const uint32_t *>(csrValues), nnz, rowSorted, valsP, s);
+    // First entry of every panel = first output position of its digit.
+    const int64_t radixTiles = RadixTiles(nnz);
+    OpsparseSpmvPlan p{};
+    int32_t starts[OPSPARSE_SPMV_MAX_PANELS];
+    for (int32_t d = 0; d < P; ++d) {
+        if (hipMemcpyAsync(&starts[d], table + static_cast<int64_t>(d) * radixTiles, sizeof(int32_t),
+                           hipMemcpyDeviceToHost, s) != hipSuccess) {
+            (void)hipGetLastError();
+            return OPSPARSE_E_LAUNCH;
+        }
+    }
+    if (hipStreamSynchronize(s) != hipSuccess) {
+        (void)hipGetLastError();
+        return OPSPARSE_E_LAUNCH;
+    }
+    for (int32_t d = 0; d < P; ++d) {
+        p.panelStart[d] = starts[d];
+    }
+    p.panelStart[P] = nnz;
+    // Row offsets (relative to the panel's first entry) and merge partition of every panel.
+    for (int32_t d = 0; d < P; ++d) {
+        const int64_t nnzP = p.panelStart[d + 1] - p.panelStart[d];
+        if (nnzP < 0) {
+            return OPSPARSE_E_INVALID;  // a column index outside [0, cols)
+        }
+        int32_t *rp = rowPtrP + static_cast<int64_t>(d) * (rows + 1);
+        LaunchIndicesToOffsets(rowSorted + p.panelStart[d], nnzP, rows, 0, rp, scratch, s);
+        const int32_t tiles = static_cast<int32_t>((rows + nnzP + kMergeItems - 1) / kMergeItems);
+        hipLaunchKernelGGL(MergePartitionKernel, dim3(GridFor(tiles + 1, kBlockThreads)), dim3(kBlockThreads), 0, s, rp,
+                           rows, nnzP, tiles, part + static_cast<int64_t>(d) * (l.tileBound + 1));
+    }
+    if (CheckLaunch() != OPSPARSE_OK) {
+        return OPSPARSE_E_LAUNCH;
+    }
+    p.kernel = OPSPARSE_SPMV_COLUMN_PANELS;
+    p.numPanels = P;
+    p.panelShift = kPanelShift;
+    p.rows = rows;
+    p.nnz = nnz;
+    p.bytes = l.bytes;
     *plan = p;
     return OPSPARSE_OK;
 }

@@ -48,6 +48,8 @@ def gpu_ctx(osa):
     osa.lib()  # raises if libops_sparse.so is missing: there is no fallback to test
     dev = torch.device("cuda:0")
     stream = torch.cuda.Stream(device=dev)
+    # torch's own kernels (fills, clones, uploads) go on the same stream as the library's, so the two are ordered
+    torch.cuda.set_stream(stream)
     handle = osa.Handle(stream)
     yield dev, stream, handle
     handle.close()

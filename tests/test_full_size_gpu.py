@@ -13,12 +13,12 @@ import oracle
 pytestmark = pytest.mark.gpu
 
 
-def _spmv(osa, gpu_ctx, cfg, preprocess=True):
+def _spmv(osa, gpu_ctx, cfg, preprocess=True, alg=0):
     dev, stream, handle = gpu_ctx
     A = cfg["A"]
     csr = osa.Csr(A["rows"], A["cols"], A["rowptr"], A["colind"], A["values"])
     y = cfg["y0"].clone()
-    op = osa.SpmvOp(handle, csr, osa.DnVec(cfg["x"]), osa.DnVec(y), preprocess=preprocess)
+    op = osa.SpmvOp(handle, csr, osa.DnVec(cfg["x"]), osa.DnVec(y), preprocess=preprocess, alg=alg)
     op(cfg["alpha"], cfg["beta"])
     stream.synchronize()
     return y
@@ -67,6 +67,9 @@ def test_c3_power_law_full(osa, workloads, gpu_ctx):
     # without Preprocess (partition rebuilt per call in the handle workspace, or the vector kernel)
     y2 = _spmv(osa, gpu_ctx, cfg, preprocess=False)
     assert oracle.max_rel_err(y2.cpu().numpy(), gold) <= 1e-5
+    # the column-panel layout (CSR_ALG2): eight panels of 2^20 columns
+    y5 = _spmv(osa, gpu_ctx, cfg, alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
+    assert oracle.max_rel_err(y5.cpu().numpy(), gold) <= 1e-5
     # linearity: scaling x by 2 is exact in binary floating point
     cfg["x"] = cfg["x"] * 2.0
     y3 = _spmv(osa, gpu_ctx, cfg)

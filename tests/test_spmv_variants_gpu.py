@@ -150,3 +150,63 @@ def test_preprocessed_buffer_reused_and_rebound(osa, gpu_ctx):
     stream.synchronize()
     gold = oracle.spmv_f64(rows, cols, rowptr, colind, (val * 3.0).astype(np.float32), x, y0, 1.0, 0.0)
     assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+
+def _wide_problem(rows, cols, seed, long_rows=()):
+    rng = np.random.default_rng(seed)
+    lengths = rng.integers(0, 12, rows)
+    for r, l in long_rows:
+        lengths[r] = l
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = np.concatenate([np.sort(rng.choice(cols, int(l), replace=False)) for l in lengths] +
+                            [np.zeros(0, np.int64)]).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    return rowptr, colind, val, rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+
+
+@pytest.mark.parametrize("cols,panels", [(3_000_000, 3), (1_048_577, 2), (9_000_000, 9), (1_000_000, 0), (17_000_000, 0)])
+def test_column_panels_csr_alg2(osa, gpu_ctx, cols, panels):
+    """ACL_SPARSE_SPMV_CSR_ALG2: Preprocess re-stores the matrix as panels of 2^20 columns (x wider than an L2);
+    matrices with fewer than 2 or more than 16 panels silently take the ordinary families.  Same 1e-5 bar, and
+    bit-equal from run to run (partials are added in panel order)."""
+    dev, stream, handle = gpu_ctx
+    rows = 60_000
+    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, cols % 1000, long_rows=((7, 90_000), (59_999, 30_000)))
+    L = osa.lib()
+    assert (L.opsparse_spmv_csr_panels_workspace_bytes(rows, cols, colind.size) > 0) == (panels > 0)
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    A = osa.Csr(rows, cols, d[0], d[1], d[2])
+    d_y = to_dev(y0, dev)
+    op = osa.SpmvOp(handle, A, osa.DnVec(d[3]), osa.DnVec(d_y), alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
+    assert op.buffer.numel() >= L.opsparse_spmv_csr_panels_workspace_bytes(rows, cols, colind.size)
+    outs = []
+    for alpha, beta in ((1.0, 0.0), (-2.0, 0.75), (-2.0, 0.75)):
+        d_y.copy_(torch.from_numpy(y0))
+        op(alpha, beta)
+        stream.synchronize()
+        outs.append(d_y.cpu().numpy())
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, alpha, beta)
+        assert oracle.max_rel_err(outs[-1], gold) <= 1e-5
+    assert np.array_equal(outs[1], outs[2])
+    assert np.array_equal(d[1].cpu().numpy(), colind) and np.array_equal(d[2].cpu().numpy(), val)
+
+
+def test_column_panels_through_spmvop_alg2(osa, gpu_ctx):
+    """aclsparseSpMVOp ALG2 on a wide matrix uses the same layout; Z separate from Y and aliased."""
+    dev, stream, handle = gpu_ctx
+    rows, cols = 40_000, 2_500_000
+    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 5, long_rows=((3, 50_000),))
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    A = osa.Csr(rows, cols, d[0], d[1], d[2])
+    for alias in (False, True):
+        d_y = to_dev(y0, dev)
+        d_z = d_y if alias else torch.zeros(rows, dtype=torch.float32, device=dev)
+        Y = osa.DnVec(d_y)
+        Z = Y if alias else osa.DnVec(d_z)
+        op = osa.SpmvOpPlan(handle, A, osa.DnVec(d[3]), Y, Z, alg=osa.ACL_SPARSE_SPMVOP_ALG2)
+        assert op.buffer_bytes == osa.lib().opsparse_spmv_csr_panels_workspace_bytes(rows, cols, colind.size) > 0
+        op(1.25, -0.5)
+        stream.synchronize()
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.25, -0.5)
+        assert oracle.max_rel_err(d_z.cpu().numpy(), gold) <= 1e-5
+        op.close()
