@@ -244,7 +244,8 @@ def main():
                    "preprocessed": not args.no_preprocess, "column_panels": bool(args.panels)},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": load_traffic(cfg["name"]) if args.scale == 1.0 else None,
+                     "traffic": load_traffic(cfg["name"] + ("+column_panels" if args.panels else ""))
+                     if args.scale == 1.0 else None,
                      "bytes_alg": bytes_alg, "bytes_gather_model": bytes_gather,
                      "copy_kernel_gbps": round(copy_gbps, 1), "read_kernel_gbps": round(read_gbps, 1)},
     }
