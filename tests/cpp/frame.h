@@ -1,0 +1,241 @@
+// Small C++ test frame over HIP for callers written against cann_ops_sparse.h:
+// RAII owners for the stream, the aclsparse handle, device arrays and
+// descriptors, a CSV case-table loader and a seeded CSR generator.  It plays the
+// role of the reference's test/frame (descriptor_manager.h, sparse_test.h,
+// csv_loader.h, fill.h) for the case tables kept under tests/golden/, without
+// GoogleTest: a test program is a plain main() that prints one line per case.
+// Test infrastructure only; links libops_sparse.so and (as the checker)
+// oracle/liboracle.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <fstream>
+#include <map>
+#include <random>
+#include <sstream>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "cann_ops_sparse.h"
+
+// The CPU checker (oracle/oracle.c).
+extern "C" {
+void oracle_spmv_f64(int64_t rows, int64_t cols, const int32_t *rowptr, const int32_t *colind, const float *val,
+                     const float *x, const float *y, float alpha, float beta, float *z);
+void oracle_mere_mare(const float *out, const float *gold, int64_t n, double eps, double *result);
+void oracle_coo2csr(const int32_t *rowInd, int64_t nnz, int64_t m, int32_t base, int32_t *rowPtr);
+void oracle_csr2coo(const int32_t *rowPtr, int64_t m, int64_t nnz, int32_t base, int32_t *rowInd);
+void oracle_csr2csc(int64_t m, int64_t n, int64_t nnz, int32_t base, const int32_t *rowPtr, const int32_t *colInd,
+                    const void *val, int32_t valBytes, int32_t *colPtr, int32_t *rowInd, void *cscVal);
+}
+
+namespace frame {
+
+inline void Check(hipError_t e, const char *what)
+{
+    if (e != hipSuccess) {
+        throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
+    }
+}
+inline void Check(aclsparseStatus_t s, const char *what)
+{
+    if (s != ACL_SPARSE_STATUS_SUCCESS) {
+        throw std::runtime_error(std::string(what) + ": aclsparse status " + std::to_string(static_cast<int>(s)));
+    }
+}
+
+class Stream {
+public:
+    Stream() { Check(hipStreamCreate(&s_), "hipStreamCreate"); }
+    ~Stream() { (void)hipStreamDestroy(s_); }
+    Stream(const Stream &) = delete;
+    Stream &operator=(const Stream &) = delete;
+    hipStream_t get() const { return s_; }
+    void sync() const { Check(hipStreamSynchronize(s_), "hipStreamSynchronize"); }
+
+private:
+    hipStream_t s_ = nullptr;
+};
+
+class Handle {
+public:
+    explicit Handle(const Stream &s)
+    {
+        Check(aclsparseCreate(&h_), "aclsparseCreate");
+        Check(aclsparseSetStream(h_, s.get()), "aclsparseSetStream");
+    }
+    ~Handle() { (void)aclsparseDestroy(h_); }
+    Handle(const Handle &) = delete;
+    Handle &operator=(const Handle &) = delete;
+    aclsparseHandle_t get() const { return h_; }
+
+private:
+    aclsparseHandle_t h_ = nullptr;
+};
+
+// Device array with upload / download; an empty array has a NULL pointer.
+template <typename T>
+class DeviceArray {
+public:
+    DeviceArray() = default;
+    explicit DeviceArray(size_t n) { Allocate(n); }
+    explicit DeviceArray(const std::vector<T> &host)
+    {
+        Allocate(host.size());
+        if (n_ > 0) {
+            Check(hipMemcpy(p_, host.data(), n_ * sizeof(T), hipMemcpyHostToDevice), "hipMemcpy H2D");
+        }
+    }
+    ~DeviceArray() { (void)hipFree(p_); }
+    DeviceArray(const DeviceArray &) = delete;
+    DeviceArray &operator=(const DeviceArray &) = delete;
+    DeviceArray(DeviceArray &&o) noexcept : p_(o.p_), n_(o.n_) { o.p_ = nullptr; o.n_ = 0; }
+    T *get() const { return p_; }
+    size_t size() const { return n_; }
+    std::vector<T> download() const
+    {
+        std::vector<T> out(n_);
+        if (n_ > 0) {
+            Check(hipMemcpy(out.data(), p_, n_ * sizeof(T), hipMemcpyDeviceToHost), "hipMemcpy D2H");
+        }
+        return out;
+    }
+
+private:
+    void Allocate(size_t n)
+    {
+        n_ = n;
+        if (n_ > 0) {
+            Check(hipMalloc(reinterpret_cast<void **>(&p_), n_ * sizeof(T)), "hipMalloc");
+        }
+    }
+    T *p_ = nullptr;
+    size_t n_ = 0;
+};
+
+struct CsrHost {
+    int64_t rows = 0, cols = 0;
+    std::vector<int32_t> rowptr{0}, colind;
+    std::vector<float> val;
+    int64_t nnz() const { return static_cast<int64_t>(colind.size()); }
+};
+
+// Seeded CSR: Binomial(cols, 1 - sparsity) entries per row (0 with probability emptyRowProb), distinct
+// sorted columns, values uniform in [lo, hi).  Same distribution as the reference generator, own stream.
+inline CsrHost RandomCsr(int64_t rows, int64_t cols, double sparsity, double emptyRowProb, uint32_t seed, float lo,
+                         float hi)
+{
+    CsrHost a;
+    a.rows = rows;
+    a.cols = cols;
+    a.rowptr.assign(static_cast<size_t>(rows) + 1, 0);
+    std::mt19937 rng(seed);
+    std::binomial_distribution<int64_t> len(cols, 1.0 - sparsity);
+    std::uniform_real_distribution<double> u01(0.0, 1.0);
+    std::uniform_real_distribution<float> uv(lo, hi);
+    std::vector<int32_t> stamp(static_cast<size_t>(cols), -1);
+    for (int64_t r = 0; r < rows; ++r) {
+        int64_t l = (cols > 0 && sparsity < 1.0) ? len(rng) : 0;
+        if (emptyRowProb > 0.0 && u01(rng) < emptyRowProb) {
+            l = 0;
+        }
+        std::vector<int32_t> picked;
+        if (l * 2 > cols) {  // dense row: keep each column with probability l / cols, then trim / top up
+            for (int32_t c = 0; c < cols && static_cast<int64_t>(picked.size()) < l; ++c) {
+                if (cols - c <= l - static_cast<int64_t>(picked.size()) || u01(rng) * cols < l) {
+                    picked.push_back(c);
+                }
+            }
+        } else {
+            std::uniform_int_distribution<int32_t> uc(0, static_cast<int32_t>(cols) - 1);
+            while (static_cast<int64_t>(picked.size()) < l) {
+                const int32_t c = uc(rng);
+                if (stamp[c] != r) {
+                    stamp[c] = static_cast<int32_t>(r);
+                    picked.push_back(c);
+                }
+            }
+            std::sort(picked.begin(), picked.end());
+        }
+        for (int32_t c : picked) {
+            a.colind.push_back(c);
+            a.val.push_back(uv(rng));
+        }
+        a.rowptr[r + 1] = static_cast<int32_t>(a.colind.size());
+    }
+    return a;
+}
+
+inline CsrHost DiagCsr(int64_t m)
+{
+    CsrHost a;
+    a.rows = a.cols = m;
+    a.rowptr.resize(static_cast<size_t>(m) + 1);
+    for (int64_t i = 0; i <= m; ++i) {
+        a.rowptr[i] = static_cast<int32_t>(i);
+    }
+    for (int64_t i = 0; i < m; ++i) {
+        a.colind.push_back(static_cast<int32_t>(i));
+        a.val.push_back(1.0f);
+    }
+    return a;
+}
+
+inline std::vector<float> RandomVector(int64_t n, float lo, float hi, uint32_t seed)
+{
+    std::mt19937 rng(seed);
+    std::uniform_real_distribution<float> u(lo, hi);
+    std::vector<float> v(static_cast<size_t>(n > 0 ? n : 0));
+    for (auto &e : v) {
+        e = u(rng);
+    }
+    return v;
+}
+
+// Rows of a CSV case table keyed by the header names; lines starting with '#' are comments.
+inline std::vector<std::map<std::string, std::string>> LoadCsv(const std::string &path)
+{
+    std::ifstream in(path);
+    if (!in) {
+        throw std::runtime_error("cannot open " + path);
+    }
+    auto split = [](const std::string &line) {
+        std::vector<std::string> out;
+        std::stringstream ss(line);
+        std::string cell;
+        while (std::getline(ss, cell, ',')) {
+            while (!cell.empty() && (cell.back() == '\r' || cell.back() == ' ')) {
+                cell.pop_back();
+            }
+            out.push_back(cell);
+        }
+        return out;
+    };
+    std::string line;
+    std::vector<std::string> header;
+    std::vector<std::map<std::string, std::string>> rows;
+    while (std::getline(in, line)) {
+        if (line.empty() || line[0] == '#') {
+            continue;
+        }
+        const auto cells = split(line);
+        if (header.empty()) {
+            header = cells;
+            continue;
+        }
+        std::map<std::string, std::string> row;
+        for (size_t i = 0; i < header.size() && i < cells.size(); ++i) {
+            row[header[i]] = cells[i];
+        }
+        rows.push_back(row);
+    }
+    return rows;
+}
+
+}  // namespace frame
