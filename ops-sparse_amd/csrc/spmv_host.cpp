@@ -215,7 +215,9 @@ aclsparseStatus_t aclsparseSpMV(aclsparseHandle_t handle, aclsparseOperation_t o
         plan = &matA->spmv.plan;
         ws = externalBuffer;
         wsBytes = static_cast<size_t>(plan->bytes);
-    } else if (!c.transpose && matA->nnz > 0) {
+    } else if (matA->nnz > 0 || (c.transpose && c.outType != OPSPARSE_F32)) {
+        // the merge-path partition of an unprepared call, or the fp32 staging vector of a transposed
+        // product with fp16 / bf16 y (cols * 4 bytes: enlarge it with aclsparseSetWorkspace if need be)
         st = opsparse::EnsureWorkspace(handle);
         if (st != ACL_SPARSE_STATUS_SUCCESS) {
             return st;

@@ -83,6 +83,29 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvScaleKernel(OutT *y, const 
     }
 }
 
+// dst = beta * src widened to fp32 (0 when beta == 0: src is not read), and the way back: the transposed
+// product adds into an fp32 vector, which for fp16 / bf16 y is a staging vector in the workspace.
+template <typename InT>
+__global__ __launch_bounds__(kBlockThreads) void ScaleIntoFloatKernel(float *__restrict__ dst, const InT *src,
+                                                                      int64_t len, OpsparseScalar betaS)
+{
+    const double beta = ReadScalar<double>(betaS);
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlockThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; i < len; i += stride) {
+        dst[i] = beta == 0.0 ? 0.0f : static_cast<float>(beta * ToAcc<double>(src[i]));
+    }
+}
+
+template <typename OutT>
+__global__ __launch_bounds__(kBlockThreads) void ConvertFromFloatKernel(OutT *__restrict__ dst,
+                                                                        const float *__restrict__ src, int64_t len)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlockThreads;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; i < len; i += stride) {
+        dst[i] = FromAcc<OutT>(static_cast<double>(src[i]));
+    }
+}
+
 // ------------------------------------------------------------- row statistics
 
 // stats[0] = max row length.  stats must be zeroed before the launch.
@@ -1080,14 +1103,49 @@ OpsparseSpmvPlan AdHocPlan(int64_t rows, int64_t nnz, size_t wsBytes, const void
 template <typename ValT, typename AccT>
 int RunTranspose(const SpmvArgs &a, int32_t outType)
 {
-    if (outType != OPSPARSE_F32) {
+    if (outType != OPSPARSE_F32 && outType != OPSPARSE_F16 && outType != OPSPARSE_BF16) {
         return OPSPARSE_E_UNSUPPORTED;
     }
-    // y has `cols` elements for the transposed product.
-    int rc = LaunchScale<float, AccT>(static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.cols, a.beta,
-                                      a.stream);
-    if (rc != OPSPARSE_OK || a.nnz == 0 || a.rows == 0) {
+    // y has `cols` elements for the transposed product.  fp16 / bf16 y: the sums are formed in an fp32
+    // staging vector in the workspace and rounded once at the end.
+    const bool staged = outType != OPSPARSE_F32;
+    float *acc = static_cast<float *>(a.y);
+    int64_t grid = (a.cols + kBlockThreads - 1) / kBlockThreads;
+    grid = grid > 65536 ? 65536 : (grid < 1 ? 1 : grid);
+    int rc = OPSPARSE_OK;
+    if (!staged) {
+        rc = LaunchScale<float, AccT>(acc, static_cast<const float *>(a.yIn), a.cols, a.beta, a.stream);
+    } else if (a.cols > 0) {
+        if (a.ws == nullptr || a.wsBytes < static_cast<size_t>(a.cols) * sizeof(float)) {
+            return OPSPARSE_E_WORKSPACE;
+        }
+        acc = static_cast<float *>(a.ws);
+        if (outType == OPSPARSE_F16) {
+            hipLaunchKernelGGL(ScaleIntoFloatKernel<Half>, dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0,
+                               a.stream, acc, static_cast<const Half *>(a.yIn), a.cols, a.beta);
+        } else {
+            hipLaunchKernelGGL(ScaleIntoFloatKernel<Bf16>, dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0,
+                               a.stream, acc, static_cast<const Bf16 *>(a.yIn), a.cols, a.beta);
+        }
+        rc = CheckLaunch();
+    }
+    auto finish = [&]() {
+        if (staged && a.cols > 0) {
+            if (outType == OPSPARSE_F16) {
+                hipLaunchKernelGGL(ConvertFromFloatKernel<Half>, dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads),
+                                   0, a.stream, static_cast<Half *>(a.y), acc, a.cols);
+            } else {
+                hipLaunchKernelGGL(ConvertFromFloatKernel<Bf16>, dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads),
+                                   0, a.stream, static_cast<Bf16 *>(a.y), acc, a.cols);
+            }
+        }
+        return CheckLaunch();
+    };
+    if (rc != OPSPARSE_OK) {
         return rc;
+    }
+    if (a.nnz == 0 || a.rows == 0) {
+        return finish();
     }
     const int32_t g = VectorLanesFor(a.rows, a.nnz);
     auto launch = [&](auto tag) {
@@ -1095,7 +1153,7 @@ int RunTranspose(const SpmvArgs &a, int32_t outType)
         hipLaunchKernelGGL((SpmvTransposeScatterKernel<ValT, AccT, G>), dim3(GridFor(a.rows, kBlockThreads / G)),
                            dim3(kBlockThreads), 0, a.stream, a.rowOffsets, a.colInd,
                            static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
-                           static_cast<float *>(a.y), a.rows, a.alpha);
+                           acc, a.rows, a.alpha);
     };
     switch (g) {
         case 4: launch(std::integral_constant<int, 4>{}); break;
@@ -1104,7 +1162,7 @@ int RunTranspose(const SpmvArgs &a, int32_t outType)
         case 32: launch(std::integral_constant<int, 32>{}); break;
         default: launch(std::integral_constant<int, 64>{}); break;
     }
-    return CheckLaunch();
+    return finish();
 }
 
 template <typename ValT, typename OutT, typename AccT>

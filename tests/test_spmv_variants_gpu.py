@@ -210,3 +210,19 @@ def test_column_panels_through_spmvop_alg2(osa, gpu_ctx):
         gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.25, -0.5)
         assert oracle.max_rel_err(d_z.cpu().numpy(), gold) <= 1e-5
         op.close()
+
+
+@pytest.mark.parametrize("dtype,rel", [(torch.float16, 2.0 ** -10), (torch.bfloat16, 2.0 ** -7)])
+@pytest.mark.parametrize("beta", [0.0, 0.5])
+def test_transpose_half_precision_output(osa, gpu_ctx, dtype, rel, beta):
+    """y = alpha * A^T x + beta * y with fp16 / bf16 A, x and y: sums formed in an fp32 staging vector (handle
+    workspace), rounded once.  Bar: one rounding of the output type (+ the fp32 atomics' 1e-4 absolute slack)."""
+    rows, cols = 3000, 900
+    rowptr, colind, val = random_csr(rows, cols, 0.02, 21, lo=-1.0, hi=1.0)
+    rng = np.random.default_rng(6)
+    rt = lambda a: torch.from_numpy(a).to(dtype).float().numpy()          # values as the kernel sees them
+    val, x, y0 = rt(val), rt(rng.uniform(-1, 1, rows).astype(np.float32)), rt(rng.uniform(-1, 1, cols).astype(np.float32))
+    y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 1.5, beta, op=osa.ACL_SPARSE_OP_TRANSPOSE,
+                 val_dtype=dtype, out_dtype=dtype)
+    gold = oracle.spmv_trans_f64(rows, cols, rowptr, colind, val, x, y0, 1.5, beta)
+    assert np.all(np.abs(y - gold) <= rel * np.abs(gold) + 1e-4)
