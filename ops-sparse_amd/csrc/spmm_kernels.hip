@@ -293,10 +293,10 @@ constexpr int kSlabTarget = 2048;   // entries per slab the launcher aims for
 // B plus a 32-bit byte offset — one register and one multiply per gather
 // instead of a 64-bit multiply-add and a register pair.
 template <typename ValT, typename CT, typename AccT, int V, int L, bool Small32>
-__global__ __launch_bounds__(kBlockThreads, SlabTuning<V>::kWavesPerSimd) void SpmmSlabKernel(
-    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
-    const ValT *__restrict__ B, CT *__restrict__ C, int64_t rows, int32_t n, int64_t ldb, int64_t ldc,
-    int32_t rowsPerSlab, int32_t longRowNnz, OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16)
+__device__ __forceinline__ void SlabBody(
+    int64_t slab, const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd,
+    const ValT *__restrict__ vals, const ValT *__restrict__ B, CT *__restrict__ C, int64_t rows, int32_t n, int64_t ldb,
+    int64_t ldc, int32_t rowsPerSlab, int32_t longRowNnz, OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16)
 {
     typedef ValT BVec __attribute__((ext_vector_type(V)));
     typedef CT CVec __attribute__((ext_vector_type(V), aligned(16)));
@@ -321,7 +321,6 @@ __global__ __launch_bounds__(kBlockThreads, SlabTuning<V>::kWavesPerSimd) void S
     const uint32_t colBytes = static_cast<uint32_t>(col) * static_cast<uint32_t>(sizeof(ValT));
     const uint32_t ldbBytes = static_cast<uint32_t>(ldb) * static_cast<uint32_t>(sizeof(ValT));
 
-    const int64_t slab = XcdContiguousTile(blockIdx.x, gridDim.x);
     int64_t rowCur = slab * rowsPerSlab;
     const int64_t rowEnd = (rowCur + rowsPerSlab < rows) ? rowCur + rowsPerSlab : rows;
 
@@ -473,14 +472,15 @@ __global__ __launch_bounds__(kBlockThreads, SlabTuning<V>::kWavesPerSimd) void S
 // One lane group per segment of a long row: partial[seg][0..n) = sum over the
 // segment's entries, in fp64.
 template <typename ValT, typename AccT, int V, int L>
-__global__ __launch_bounds__(kBlockThreads) void SpmmLongSegmentKernel(
-    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
-    const ValT *__restrict__ B, int32_t n, int64_t ldb, int32_t numSegments, const int32_t *__restrict__ segRow,
-    const int32_t *__restrict__ segStart, AccT *__restrict__ partial)
+__device__ __forceinline__ void SegmentBody(int64_t block, const int32_t *__restrict__ rowOffsets,
+                                            const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+                                            const ValT *__restrict__ B, int32_t n, int64_t ldb, int32_t numSegments,
+                                            const int32_t *__restrict__ segRow, const int32_t *__restrict__ segStart,
+                                            AccT *__restrict__ partial)
 {
     constexpr int kGroups = kBlockThreads / L;
     const int32_t lane = threadIdx.x % L;
-    const int64_t seg = static_cast<int64_t>(blockIdx.x) * kGroups + threadIdx.x / L;
+    const int64_t seg = block * kGroups + threadIdx.x / L;
     if (seg >= numSegments) {
         return;
     }
@@ -508,6 +508,45 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmLongSegmentKernel(
             }
         }
     }
+}
+
+template <typename ValT, typename AccT, int V, int L>
+__global__ __launch_bounds__(kBlockThreads) void SpmmLongSegmentKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ B, int32_t n, int64_t ldb, int32_t numSegments, const int32_t *__restrict__ segRow,
+    const int32_t *__restrict__ segStart, AccT *__restrict__ partial)
+{
+    SegmentBody<ValT, AccT, V, L>(blockIdx.x, rowOffsets, colInd, vals, B, n, ldb, numSegments, segRow, segStart, partial);
+}
+
+// The slab kernel proper.  With long rows (segBlocks > 0) the workgroups of their
+// segments are spread evenly among the slab workgroups of the same launch: the
+// segment workgroups stream at the gather ceiling and fill the moments in which a
+// slab workgroup is between slabs and has no gather in flight.
+template <typename ValT, typename CT, typename AccT, int V, int L, bool Small32>
+__global__ __launch_bounds__(kBlockThreads, SlabTuning<V>::kWavesPerSimd) void SpmmSlabKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ B, CT *__restrict__ C, int64_t rows, int32_t n, int64_t ldb, int64_t ldc,
+    int32_t rowsPerSlab, int32_t longRowNnz, OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16,
+    uint32_t segBlocks, int32_t numSegments, const int32_t *__restrict__ segRow,
+    const int32_t *__restrict__ segStart, AccT *__restrict__ partial)
+{
+    int64_t slab;
+    if (segBlocks > 0) {
+        // workgroup b is a segment workgroup iff floor((b + 1) * segBlocks / total) > floor(b * segBlocks / total)
+        const uint64_t before = static_cast<uint64_t>(blockIdx.x) * segBlocks / gridDim.x;
+        const uint64_t after = (static_cast<uint64_t>(blockIdx.x) + 1) * segBlocks / gridDim.x;
+        if (after > before) {
+            SegmentBody<ValT, AccT, V, L>(static_cast<int64_t>(before), rowOffsets, colInd, vals, B, n, ldb, numSegments,
+                                          segRow, segStart, partial);
+            return;
+        }
+        slab = static_cast<int64_t>(blockIdx.x) - static_cast<int64_t>(before);
+    } else {
+        slab = XcdContiguousTile(blockIdx.x, gridDim.x);
+    }
+    SlabBody<ValT, CT, AccT, V, L, Small32>(slab, rowOffsets, colInd, vals, B, C, rows, n, ldb, ldc, rowsPerSlab,
+                                            longRowNnz, alphaS, betaS, clampF16);
 }
 
 // One workgroup per long row.  Each of its four wavefronts adds a contiguous
@@ -774,19 +813,34 @@ int LaunchSlab(const SpmmArgs &a)
     const uint32_t grid = static_cast<uint32_t>((a.rows + rps - 1) / rps);
     const int32_t longRowNnz = binned ? a.plan->longRowNnz : kSlabCap;
     const bool small32 = static_cast<uint64_t>(a.k) * static_cast<uint64_t>(a.ldb) * sizeof(ValT) < (1ull << 32);
+    // Long rows: their segment workgroups ride in the same launch, the fix-up follows.
+    constexpr int kGroups = kBlockThreads / L;
+    auto *base = static_cast<unsigned char *>(a.ws);
+    const int32_t nseg = binned ? a.plan->numSegments : 0;
+    const uint32_t segBlocks = static_cast<uint32_t>((nseg + kGroups - 1) / kGroups);
+    const int32_t *segRow = binned ? reinterpret_cast<const int32_t *>(base + a.plan->segRowOff) : nullptr;
+    const int32_t *segStart = binned ? reinterpret_cast<const int32_t *>(base + a.plan->segStartOff) : nullptr;
+    AccT *partial = binned ? reinterpret_cast<AccT *>(base + a.plan->partialOff) : nullptr;
+    auto launch = [&](auto tag) {
+        constexpr bool kSmall = decltype(tag)::value;
+        hipLaunchKernelGGL((SpmmSlabKernel<ValT, CT, AccT, V, L, kSmall>), dim3(grid + segBlocks), dim3(kBlockThreads),
+                           0, a.stream, a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
+                           static_cast<const ValT *>(a.B), static_cast<CT *>(a.C), a.rows, static_cast<int32_t>(a.n),
+                           a.ldb, a.ldc, static_cast<int32_t>(rps), longRowNnz, a.alpha, a.beta, a.clampF16, segBlocks,
+                           nseg, segRow, segStart, partial);
+    };
     if (small32) {
-        hipLaunchKernelGGL((SpmmSlabKernel<ValT, CT, AccT, V, L, true>), dim3(grid), dim3(kBlockThreads), 0, a.stream,
-                           a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.B),
-                           static_cast<CT *>(a.C), a.rows, static_cast<int32_t>(a.n), a.ldb, a.ldc,
-                           static_cast<int32_t>(rps), longRowNnz, a.alpha, a.beta, a.clampF16);
+        launch(std::true_type{});
     } else {
-        hipLaunchKernelGGL((SpmmSlabKernel<ValT, CT, AccT, V, L, false>), dim3(grid), dim3(kBlockThreads), 0, a.stream,
-                           a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.B),
-                           static_cast<CT *>(a.C), a.rows, static_cast<int32_t>(a.n), a.ldb, a.ldc,
-                           static_cast<int32_t>(rps), longRowNnz, a.alpha, a.beta, a.clampF16);
+        launch(std::false_type{});
     }
     if (binned) {
-        LaunchLongRows<ValT, CT, AccT, V, L>(a);
+        const auto *longRows = reinterpret_cast<const int32_t *>(base + a.plan->longRowsOff);
+        const auto *firstSeg = reinterpret_cast<const int32_t *>(base + a.plan->longFirstSegOff);
+        const int32_t nlong = a.plan->numLongRows;
+        hipLaunchKernelGGL((SpmmLongFixupKernel<CT, AccT>), dim3(nlong), dim3(kBlockThreads), 0, a.stream,
+                           static_cast<CT *>(a.C), static_cast<int32_t>(a.n), a.ldc, nlong, longRows, firstSeg, partial,
+                           a.alpha, a.beta, a.clampF16);
     }
     return CheckLaunch();
 }
