@@ -146,13 +146,18 @@ def main():
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-preprocess", action="store_true", help="SpMV without the Preprocess buffer")
+    ap.add_argument("--alg2", action="store_true",
+                    help="SpMV with ACL_SPARSE_SPMV_CSR_ALG2: Preprocess re-stores the matrix (c3: blocked gather)")
     ap.add_argument("--panels", action="store_true",
-                    help="SpMV with ACL_SPARSE_SPMV_CSR_ALG2: column-panel layout built by Preprocess (c3)")
+                    help="like --alg2 with the blocked-gather layout switched off: column panels (c3)")
     ap.add_argument("--gather-probe", action="store_true", help="also measure random-gather rates (stderr)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
 
+    if args.panels:
+        os.environ["OPS_SPARSE_SPMV_NO_BLOCKED"] = "1"
+    layout = "column_panels" if args.panels else "blocked_gather" if args.alg2 else "csr"
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
@@ -188,7 +193,9 @@ def main():
         y = cfg["y0"].clone()
         X, Y = osa.DnVec(x), osa.DnVec(y)
         op = osa.SpmvOp(handle, csr, X, Y, preprocess=not args.no_preprocess,
-                        alg=osa.ACL_SPARSE_SPMV_CSR_ALG2 if args.panels else osa.ACL_SPARSE_SPMV_ALG_DEFAULT)
+                        alg=osa.ACL_SPARSE_SPMV_CSR_ALG2 if layout != "csr" else osa.ACL_SPARSE_SPMV_ALG_DEFAULT)
+        if layout == "blocked_gather" and not osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz):
+            layout = "column_panels" if osa.lib().opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz) else "csr"
         ncols = 1
         bytes_alg = wl.spmv_bytes_alg(rows, cols, nnz, vb, x.element_size(), y.element_size(), cfg["beta"] != 0)
         bytes_gather = wl.spmv_bytes_gather(rows, cols, nnz, vb, x.element_size(), y.element_size(),
@@ -241,10 +248,10 @@ def main():
         "dtype": dtype, "data": "synthetic",
         "config": {"workload": cfg["name"], "rows": rows, "cols": cols, "nnz": nnz, "ncols_dense": ncols,
                    "alpha": alpha, "beta": beta, "index": "int32", "preprocess_ms": round(preprocess_ms, 3),
-                   "preprocessed": not args.no_preprocess, "column_panels": bool(args.panels)},
+                   "preprocessed": not args.no_preprocess, "layout": layout},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": load_traffic(cfg["name"] + ("+column_panels" if args.panels else ""))
+                     "traffic": load_traffic(cfg["name"] + ("+" + layout if layout != "csr" else ""))
                      if args.scale == 1.0 else None,
                      "bytes_alg": bytes_alg, "bytes_gather_model": bytes_gather,
                      "copy_kernel_gbps": round(copy_gbps, 1), "read_kernel_gbps": round(read_gbps, 1)},

@@ -60,9 +60,13 @@ typedef enum OpsparseSpmvKernel {
                                       one or a few lanes per row */
     OPSPARSE_SPMV_VECTOR_ROWS = 3, /* medium rows: a 4..64-lane group per row, shuffle reduction */
     OPSPARSE_SPMV_MERGE_PATH = 4,  /* skewed rows: equal (rows + nnz) per workgroup, carry-out fix-up */
-    OPSPARSE_SPMV_COLUMN_PANELS = 5 /* x larger than an L2: the matrix re-stored as panels of 2^20 columns, each
+    OPSPARSE_SPMV_COLUMN_PANELS = 5,/* x larger than an L2: the matrix re-stored as panels of 2^20 columns, each
                                       worked on one XCD so that its slice of x stays in that L2; fp32 only; holds a
                                       copy of the VALUES as they were at analysis time */
+    OPSPARSE_SPMV_BLOCKED_GATHER = 6 /* x larger than an L2: two passes.  Entries re-stored by panels of 2^15 columns,
+                                      x gathered from LDS into a linear stream; then row blocks of up to 2^14 rows
+                                      summed in LDS.  16 bytes of traffic per entry and no line-sized gathers;
+                                      fp32 only; holds a copy of the VALUES as they were at analysis time */
 } OpsparseSpmvKernel;
 
 #define OPSPARSE_SPMV_MAX_PANELS 16
@@ -75,8 +79,10 @@ typedef struct OpsparseSpmvPlan {
     int32_t mergeBlocks;   /* MERGE_PATH: number of workgroups == partition entries - 1 */
     int32_t maxRowNnz;     /* longest row */
     int32_t partitionReady;/* MERGE_PATH: partition table already in the workspace */
-    int32_t numPanels;     /* COLUMN_PANELS: number of column panels */
-    int32_t panelShift;    /* COLUMN_PANELS: log2 of the panel width */
+    int32_t numPanels;     /* COLUMN_PANELS / BLOCKED_GATHER: number of column panels */
+    int32_t panelShift;    /* COLUMN_PANELS / BLOCKED_GATHER: log2 of the panel width */
+    int32_t numRowBlocks;  /* BLOCKED_GATHER: number of row blocks */
+    int32_t entryWindow;   /* BLOCKED_GATHER: a row block also ends where the entry count passes a multiple of this */
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */
@@ -123,6 +129,19 @@ size_t opsparse_spmv_csr_panels_workspace_bytes(int64_t rows, int64_t cols, int6
 int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
                                      int64_t rows, int64_t cols, int64_t nnz, void *workspace, size_t workspaceBytes,
                                      OpsparseSpmvPlan *plan, void *stream);
+
+/*
+ * BLOCKED_GATHER analysis (fp32, op(A) = A): bytes of the workspace, or 0 when the
+ * family does not apply (it needs more than 2^20 and at most 2^26 columns, and at
+ * least 32 entries per (panel, row block) chunk on average).  Like the panel
+ * analysis it re-stores indices AND values in the workspace; launches with the
+ * resulting plan ignore the rowOffsets / colInd / csrValues arguments.  Returns
+ * OPSPARSE_E_INVALID for a column index outside [0, cols).  Synchronises `stream` once.
+ */
+size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz);
+int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
+                                      int64_t rows, int64_t cols, int64_t nnz, void *workspace, size_t workspaceBytes,
+                                      OpsparseSpmvPlan *plan, void *stream);
 
 /* Same as opsparse_spmv_csr_launch with separate input and output vectors:
  * z = alpha * op(A) * x + beta * yIn.  z may be yIn (in place); yIn is only read

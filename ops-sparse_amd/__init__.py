@@ -58,7 +58,9 @@ STATUS_NAMES = ["SUCCESS", "NOT_INITIALIZED", "ALLOC_FAILED", "INVALID_VALUE", "
 OPSPARSE_F32, OPSPARSE_F16, OPSPARSE_BF16, OPSPARSE_I32, OPSPARSE_I8 = range(5)
 (OPSPARSE_SPMV_AUTO, OPSPARSE_SPMV_SCALE_ONLY, OPSPARSE_SPMV_STREAM_ROWS, OPSPARSE_SPMV_VECTOR_ROWS,
  OPSPARSE_SPMV_MERGE_PATH) = range(5)
+OPSPARSE_OK, OPSPARSE_E_INVALID, OPSPARSE_E_UNSUPPORTED, OPSPARSE_E_WORKSPACE, OPSPARSE_E_LAUNCH = 0, -1, -2, -3, -4
 OPSPARSE_SPMV_COLUMN_PANELS = 5
+OPSPARSE_SPMV_BLOCKED_GATHER = 6
 OPSPARSE_SPMM_AUTO, OPSPARSE_SPMM_ROW_SPLIT, OPSPARSE_SPMM_BINNED = range(3)
 
 # Every symbol the two public headers declare; tests check that the library exports all of them.
@@ -88,6 +90,7 @@ OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_workspace_bytes", "opsparse_spmv_csr_analyse", "opsparse_spmv_csr_launch",
     "opsparse_spmv_csr_launch_zy", "opsparse_spmv_csr_indexed_launch",
     "opsparse_spmv_csr_panels_workspace_bytes", "opsparse_spmv_csr_panels_analyse",
+    "opsparse_spmv_csr_blocked_workspace_bytes", "opsparse_spmv_csr_blocked_analyse",
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
     "opsparse_scan_workspace_bytes", "opsparse_coo2csr_launch", "opsparse_csr2coo_launch",
     "opsparse_csrsort_workspace_bytes", "opsparse_csrsort_launch", "opsparse_csr2csc_workspace_bytes",
@@ -108,7 +111,7 @@ class OpsparseScalar(ctypes.Structure):
 class OpsparseSpmvPlan(ctypes.Structure):
     _fields_ = [("kernel", i32), ("lanesPerRow", i32), ("rowsPerBlock", i32), ("mergeBlocks", i32),
                 ("maxRowNnz", i32), ("partitionReady", i32), ("numPanels", i32),
-                ("panelShift", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
+                ("panelShift", i32), ("numRowBlocks", i32), ("entryWindow", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
                 ("carryOff", i64), ("headOff", i64), ("bytes", i64), ("panelStart", i64 * 17)]
 
 
@@ -228,6 +231,11 @@ def lib():
                                               i64, OpsparseScalar, OpsparseScalar, i32, i32, i32, vp, sz, vp]
     L.opsparse_spmv_csr_panels_workspace_bytes.restype = sz
     L.opsparse_spmv_csr_panels_workspace_bytes.argtypes = [i64, i64, i64]
+    L.opsparse_spmv_csr_blocked_workspace_bytes.restype = sz
+    L.opsparse_spmv_csr_blocked_workspace_bytes.argtypes = [i64, i64, i64]
+    L.opsparse_spmv_csr_blocked_analyse.restype = ctypes.c_int
+    L.opsparse_spmv_csr_blocked_analyse.argtypes = [vp, vp, vp, i64, i64, i64, vp, sz, ctypes.POINTER(OpsparseSpmvPlan),
+                                                    vp]
     L.opsparse_spmv_csr_panels_analyse.restype = ctypes.c_int
     L.opsparse_spmv_csr_panels_analyse.argtypes = [vp, vp, vp, i64, i64, i64, vp, sz, ctypes.POINTER(OpsparseSpmvPlan),
                                                    vp]

@@ -30,6 +30,7 @@ SOURCES = [
     "spmm_host.cpp",
     "convert_host.cpp",
     "spmv_kernels.hip",
+    "spmv_blocked.hip",
     "spmm_kernels.hip",
     "convert_kernels.hip",
     "measure_kernels.hip",

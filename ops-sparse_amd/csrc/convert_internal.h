@@ -1,6 +1,6 @@
 // Launchers of the conversion building blocks (convert_kernels.hip) that other
-// parts of the library use: the SpMV column-panel preprocessing splits a CSR
-// matrix with them.  Everything only enqueues work on `s`.
+// parts of the library use: the SpMV column-panel and blocked-gather
+// preprocessing re-store a CSR matrix with them.  Everything only enqueues work on `s`.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -11,6 +11,12 @@ namespace opsparse {
 
 // Number of int32 the prefix sum over `count` elements needs as scratch.
 int64_t ScanScratchInts(int64_t count);
+
+// out[i] = add + in[0] + ... + in[i] (in place allowed).  scratch: ScanScratchInts(count) ints.
+void LaunchInclusiveScanI32(const int32_t *in, int32_t *out, int64_t count, int32_t add, int32_t *scratch, hipStream_t s);
+
+// p[0..n) = v.
+void LaunchFillI32(int32_t *p, int64_t n, int32_t v, hipStream_t s);
 
 // rowInd[j] = i + base for j in [rowPtr[i], rowPtr[i+1]) - base.
 void LaunchExpandRows(const int32_t *rowPtr, int64_t m, int64_t nnz, int32_t base, int32_t *rowInd, hipStream_t s);

@@ -616,6 +616,16 @@ void LaunchFill(int32_t *p, int64_t n, int32_t v, hipStream_t s)
 
 int64_t ScanScratchInts(int64_t count) { return count <= 0 ? 0 : ScanTiles(count); }
 
+void LaunchInclusiveScanI32(const int32_t *in, int32_t *out, int64_t count, int32_t add, int32_t *scratch, hipStream_t s)
+{
+    LaunchInclusiveScan(in, out, count, add, scratch, s);
+}
+
+void LaunchFillI32(int32_t *p, int64_t n, int32_t v, hipStream_t s)
+{
+    LaunchFill(p, n, v, s);
+}
+
 void LaunchExpandRows(const int32_t *rowPtr, int64_t m, int64_t nnz, int32_t base, int32_t *rowInd, hipStream_t s)
 {
     if (m > 0 && nnz > 0) {

@@ -1,0 +1,577 @@
+// BLOCKED_GATHER: CSR SpMV for a matrix whose x does not fit a cache, fp32.
+//
+// Replaces the device side of the reference's aclsparseSpMV / SpMVOp with the
+// ALG2 preprocessing (sparse/spmv/arch35/spmv_kernel.cpp, launched by
+// sparse/spmv/spmv_host.cpp:196-260) for that case.  A row-wise kernel gathers
+// x[col] straight from memory, and with random columns every gather moves a
+// whole 128-byte line for 4 useful bytes: the gather rate, not the matrix
+// stream, sets the time.  Here x is gathered from LDS instead.
+//
+//   phase 1  the entries are stored a second time sorted by column panel
+//            (2^15 columns = 128 KiB of x).  A workgroup copies its panel's
+//            slice of x into LDS and writes xg[i] = x[col[i]] for the panel's
+//            entries: 2 bytes of local column index read, 4 bytes written per
+//            entry, both as linear streams.
+//   phase 2  rows are grouped into row blocks (at most 2^14 rows, cut also
+//            wherever the entry count passes a multiple of the entry window,
+//            so that blocks of short rows hold similar numbers of entries).  A
+//            workgroup owns one block, keeps an fp64 accumulator per row in
+//            LDS and streams the block's entries in (block, panel) order:
+//            value and local row index linearly, the gathered xg in one
+//            contiguous piece per (panel, block) chunk.  val * xg is exact in
+//            fp64; a row's result is rounded once when the block is written.
+//
+// Every entry costs 16 bytes of HBM traffic (2 + 4 in phase 1, 4 + 2 + 4 in
+// phase 2) against 8 algorithmic bytes plus a 128-byte line per gather in the
+// row-wise kernels.  The order of the fp64 additions into a row's accumulator
+// depends on scheduling; the sum is rounded to fp32 afterwards.
+//
+// Preprocessing (once per matrix, all on the device): a stable radix sort of
+// the entries on the panel number keeps rows, hence row blocks, ascending inside
+// a panel, so it yields the (panel, block) order directly; the position of a
+// chunk in (block, panel) order follows from the chunk sizes by a prefix sum.
+// The VALUES are copied in (block, panel) order: the analysis must be repeated
+// after they change.
+#include <climits>
+
+#include "convert_internal.h"
+#include "device_utils.h"
+#include "spmv_internal.h"
+
+namespace opsparse {
+
+constexpr int kBlkThreads = 1024;                 // one workgroup per CU: it owns 128 KiB of LDS
+constexpr int kBlkWaves = kBlkThreads / kWave;
+constexpr int kPanelLog = 15;                     // columns per panel: 128 KiB of fp32 x
+constexpr int kPanelCols = 1 << kPanelLog;
+constexpr int kRowBlockLog = 14;                  // rows per row block: 128 KiB of fp64 accumulators
+constexpr int kRowBlockRows = 1 << kRowBlockLog;
+constexpr int kMaxPanels = 2048;                  // chunk tables of one row block in LDS: 16 KiB
+constexpr int kGatherBatch = 8;                   // groups of 4 entries in flight per lane, phase 1
+constexpr int kReduceBatch = 8;                   // entries in flight per lane, phase 2
+constexpr int64_t kMinEntryWindow = 16384;
+constexpr int64_t kMinChunkEntries = 32;          // below this mean chunk size the layout does not pay
+
+typedef float Float4 __attribute__((ext_vector_type(4)));
+typedef unsigned short Ushort4 __attribute__((ext_vector_type(4)));
+
+// Row block of a row: 2^14-row blocks, cut again wherever the row's first entry
+// passes a multiple of the entry window.  Monotone in the row number.
+__device__ __forceinline__ int32_t RowBlockOf(const int32_t *__restrict__ rowOffsets, int32_t row, int32_t window,
+                                              int32_t numBlocks)
+{
+    const int32_t b = (row >> kRowBlockLog) + rowOffsets[row] / window;
+    return b < 0 ? 0 : (b < numBlocks ? b : numBlocks - 1);  // in range whatever rowOffsets holds
+}
+
+// ------------------------------------------------------------ preprocessing
+
+// For the entries in (panel, original position) order: local column index, chunk
+// key panel * B + block, and the row.  A column outside [0, cols) sets *status.
+__global__ __launch_bounds__(kBlockThreads) void BlockedChunkKeysKernel(
+    const int32_t *__restrict__ colSorted, const int32_t *__restrict__ pos, const int32_t *__restrict__ rowOfPos,
+    const int32_t *__restrict__ rowOffsets, int64_t nnz, int64_t cols, int32_t numBlocks, int32_t window,
+    uint16_t *__restrict__ colLocal, int32_t *__restrict__ chunkKey, int32_t *__restrict__ rowOfSrc,
+    int32_t *__restrict__ status)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
+        const int32_t col = colSorted[i];
+        const int32_t row = rowOfPos[pos[i]];
+        rowOfSrc[i] = row;
+        colLocal[i] = static_cast<uint16_t>(col & (kPanelCols - 1));
+        if (col < 0 || col >= cols) {
+            atomicOr(status, 1);
+            chunkKey[i] = -1;
+        } else {
+            chunkKey[i] = (col >> kPanelLog) * numBlocks + RowBlockOf(rowOffsets, row, window, numBlocks);
+        }
+    }
+}
+
+// From srcStart (first entry of chunk (panel, block) in panel order, P * B + 1 values):
+// dstStart[1 + block * P + panel] = size of the chunk (prefix-summed afterwards) and
+// srcStartT[block * P + panel] = srcStart[panel * B + block].
+__global__ __launch_bounds__(kBlockThreads) void BlockedTablesKernel(const int32_t *__restrict__ srcStart, int32_t P,
+                                                                     int32_t B, int32_t *__restrict__ dstStart,
+                                                                     int32_t *__restrict__ srcStartT)
+{
+    const int64_t total = static_cast<int64_t>(P) * B;
+    const int64_t j = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (j == 0) {
+        dstStart[0] = 0;
+    }
+    if (j < total) {
+        const int64_t b = j / P, p = j % P;
+        const int32_t s = srcStart[p * B + b];
+        dstStart[1 + j] = srcStart[p * B + b + 1] - s;
+        srcStartT[j] = s;
+    }
+}
+
+// blockRow[b] = first row of row block b (blockRow pre-filled with `rows`).
+__global__ __launch_bounds__(kBlockThreads) void BlockedRowBlocksKernel(const int32_t *__restrict__ rowOffsets,
+                                                                        int32_t rows, int32_t window, int32_t B,
+                                                                        int32_t *__restrict__ blockRow)
+{
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (r >= rows) {
+        return;
+    }
+    const int32_t row = static_cast<int32_t>(r);
+    const int32_t cur = RowBlockOf(rowOffsets, row, window, B);
+    const int32_t prev = row > 0 ? RowBlockOf(rowOffsets, row - 1, window, B) : -1;
+    for (int32_t b = prev + 1; b <= cur; ++b) {
+        blockRow[b] = row;
+    }
+}
+
+// Values and local row indices into (block, panel) order.
+__global__ __launch_bounds__(kBlockThreads) void BlockedScatterKernel(
+    const int32_t *__restrict__ pos, const int32_t *__restrict__ rowOfSrc, const int32_t *__restrict__ chunkKey,
+    const float *__restrict__ vals, const int32_t *__restrict__ srcStart,
+    const int32_t *__restrict__ dstStart, const int32_t *__restrict__ blockRow, int64_t nnz, int32_t P, int32_t B,
+    float *__restrict__ valD, uint16_t *__restrict__ rowLocal)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
+        const int32_t key = chunkKey[i];
+        if (key < 0) {
+            continue;
+        }
+        const int32_t p = key / B, b = key % B;
+        const int64_t dst = i - srcStart[key] + dstStart[static_cast<int64_t>(b) * P + p];
+        valD[dst] = vals[pos[i]];
+        rowLocal[dst] = static_cast<uint16_t>((rowOfSrc[i] - blockRow[b]) & (kRowBlockRows - 1));
+    }
+}
+
+// blockOrder: row blocks by falling entry count (ties by block number), so that the
+// heaviest blocks start first and the short ones fill in behind them.
+__global__ __launch_bounds__(kBlockThreads) void BlockedOrderKernel(const int32_t *__restrict__ dstStart, int32_t P,
+                                                                    int32_t B, int32_t *__restrict__ blockOrder)
+{
+    const int32_t i = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
+    if (i >= B) {
+        return;
+    }
+    const int32_t mine = dstStart[static_cast<int64_t>(i + 1) * P] - dstStart[static_cast<int64_t>(i) * P];
+    int32_t rank = 0;
+    for (int32_t j = 0; j < B; ++j) {
+        const int32_t other = dstStart[static_cast<int64_t>(j + 1) * P] - dstStart[static_cast<int64_t>(j) * P];
+        rank += (other > mine || (other == mine && j < i)) ? 1 : 0;
+    }
+    blockOrder[rank] = i;
+}
+
+// ------------------------------------------------------------------ phase 1
+
+// xg[i] = x[panel * 2^15 + colLocal[i]] for the entries of one panel (a part of them when
+// `splits` > 1), the panel's slice of x held in LDS.
+__global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint16_t *__restrict__ colLocal,
+                                                                     const float *__restrict__ x,
+                                                                     float *__restrict__ xg,
+                                                                     const int32_t *__restrict__ srcStart,
+                                                                     int64_t cols, int32_t B, int32_t splits)
+{
+    __shared__ float xs[kPanelCols];
+    const int tid = threadIdx.x;
+    const int64_t p = blockIdx.x / splits, part = blockIdx.x % splits;
+    const int64_t c0 = p << kPanelLog;
+    const int64_t cn = cols - c0 < kPanelCols ? cols - c0 : kPanelCols;
+    const int64_t a = srcStart[p * B], e = srcStart[(p + 1) * B];
+    const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    for (int64_t i = tid * 4; i < cn; i += kBlkThreads * 4) {
+        if (vec && i + 4 <= cn) {
+            *reinterpret_cast<Float4 *>(xs + i) = *reinterpret_cast<const Float4 *>(x + c0 + i);
+        } else {
+            for (int64_t k = i; k < cn && k < i + 4; ++k) {
+                xs[k] = x[c0 + k];
+            }
+        }
+    }
+    __syncthreads();
+    const int64_t len = e - a;
+    const int64_t lo = a + len * part / splits, hi = a + len * (part + 1) / splits;
+    if (lo >= hi) {
+        return;
+    }
+    // Whole aligned groups of 4 entries go as 8-byte loads and 16-byte stores; what is left at
+    // either end of [lo, hi) is done one by one.
+    const int64_t g0 = (lo + 3) >> 2, g1 = hi >> 2;
+    if (g0 > g1) {
+        if (tid < 4 && lo + tid < hi) {
+            xg[lo + tid] = xs[colLocal[lo + tid]];
+        }
+        return;
+    }
+    if (tid < 4) {
+        const int64_t i = lo + tid;
+        if (i < g0 * 4) {
+            xg[i] = xs[colLocal[i]];
+        }
+    } else if (tid < 8) {
+        const int64_t i = g1 * 4 + (tid - 4);
+        if (i < hi) {
+            xg[i] = xs[colLocal[i]];
+        }
+    }
+    for (int64_t g = g0; g < g1; g += kGatherBatch * kBlkThreads) {
+        Ushort4 c[kGatherBatch];
+        // Unconditional loads (clamped to the last group): the compiler keeps all of them in flight.
+#pragma unroll
+        for (int u = 0; u < kGatherBatch; ++u) {
+            int64_t gg = g + u * kBlkThreads + tid;
+            gg = gg < g1 ? gg : g1 - 1;
+            c[u] = __builtin_nontemporal_load(reinterpret_cast<const Ushort4 *>(colLocal) + gg);
+        }
+#pragma unroll
+        for (int u = 0; u < kGatherBatch; ++u) {
+            const int64_t gg = g + u * kBlkThreads + tid;
+            Float4 r;
+            r.x = xs[c[u].x];
+            r.y = xs[c[u].y];
+            r.z = xs[c[u].z];
+            r.w = xs[c[u].w];
+            if (gg < g1) {
+                *(reinterpret_cast<Float4 *>(xg) + gg) = r;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ phase 2
+
+template <int CTRL>
+__device__ __forceinline__ int DppMove(int v)
+{
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
+}
+
+template <int CTRL>
+__device__ __forceinline__ double DppMoveF64(double v)
+{
+    const long long bits = __double_as_longlong(v);
+    const int lo = DppMove<CTRL>(static_cast<int>(bits));
+    const int hi = DppMove<CTRL>(static_cast<int>(bits >> 32));
+    return __longlong_as_double((static_cast<long long>(hi) << 32) | static_cast<unsigned int>(lo));
+}
+
+constexpr int kDppRowShr = 0x110;  // row_shr:n is kDppRowShr + n: lane i of a row of 16 reads lane i - n
+constexpr int kDppRowShl = 0x100;  // row_shl:n is kDppRowShl + n
+
+// One step of the segmented sum inside rows of 16 lanes: a lane whose sum does not yet reach
+// back to the head of its run takes over the sum of the lane OFF to its left.
+template <int OFF>
+__device__ __forceinline__ void RunSumStep(double &t, int &closed)
+{
+    const double o = DppMoveF64<kDppRowShr + OFF>(t);
+    const int c = DppMove<kDppRowShr + OFF>(closed);
+    if (!closed) {
+        t += o;
+        closed = c;
+    }
+}
+
+// Positions in xg (panel order) of the kReduceBatch * 64 entries of a wavefront's batch that
+// starts at `start` in block order.  tabD[p] is the first block-order position of the block's
+// chunk from panel p, tabDelta[p] the distance from there to the chunk in panel order.
+__device__ __forceinline__ void BatchSources(const int32_t *tabD, const int32_t *tabDelta, int32_t P, int32_t start,
+                                             int32_t end, int lane, int32_t (&src)[kReduceBatch])
+{
+    int lo = 0, hi = P;  // largest p with tabD[p] <= start
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (tabD[mid] <= start) {
+            lo = mid;
+        } else {
+            hi = mid;
+        }
+    }
+    int cur = lo;
+#pragma unroll
+    for (int u = 0; u < kReduceBatch; ++u) {
+        int32_t i = start + u * kWave + lane;
+        i = i < end ? i : end - 1;
+        int p = cur;
+        while (p + 1 < P && tabD[p + 1] <= i) {
+            ++p;
+        }
+        src[u] = i + tabDelta[p];
+        cur = __shfl(p, kWave - 1);
+    }
+}
+
+// One workgroup per row block: y[row] = alpha * sum(val * xg) + beta * yIn[row].
+__global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
+    const float *__restrict__ valD, const float *__restrict__ xg, const uint16_t *__restrict__ rowLocal,
+    const int32_t *__restrict__ dstStart, const int32_t *__restrict__ srcStartT, int32_t P,
+    const int32_t *__restrict__ blockOrder, const int32_t *__restrict__ blockRow, float *__restrict__ y,
+    const float *__restrict__ yIn, OpsparseScalar alphaS, OpsparseScalar betaS)
+{
+    __shared__ double acc[kRowBlockRows];
+    __shared__ int32_t tabD[kMaxPanels + 1];
+    __shared__ int32_t tabDelta[kMaxPanels];
+    const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+    const int64_t blk = blockOrder[blockIdx.x];
+    const int32_t row0 = blockRow[blk], row1 = blockRow[blk + 1];
+    if (row0 >= row1) {
+        return;  // a block number no row maps to
+    }
+    for (int i = tid; i < row1 - row0; i += kBlkThreads) {
+        acc[i] = 0.0;
+    }
+    for (int i = tid; i <= P; i += kBlkThreads) {
+        tabD[i] = dstStart[blk * P + i];
+    }
+    for (int i = tid; i < P; i += kBlkThreads) {
+        tabDelta[i] = srcStartT[blk * P + i] - dstStart[blk * P + i];
+    }
+    __syncthreads();
+    const int32_t d0 = tabD[0], d1 = tabD[P];
+    constexpr int kBatch = kWave * kReduceBatch;
+    int32_t src[kReduceBatch];
+    int32_t start = d0 + wave * kBatch;
+    if (start < d1) {
+        BatchSources(tabD, tabDelta, P, start, d1, lane, src);
+    }
+    for (; start < d1; start += kBlkWaves * kBatch) {
+        int32_t r[kReduceBatch];
+        float v[kReduceBatch], a[kReduceBatch];
+        // Unconditional loads, positions past the end clamped: one wait covers the whole batch.
+#pragma unroll
+        for (int u = 0; u < kReduceBatch; ++u) {
+            const int32_t d = start + u * kWave + lane;
+            const int32_t dc = d < d1 ? d : d1 - 1;
+            const int32_t rr = static_cast<int32_t>(__builtin_nontemporal_load(rowLocal + dc)) & (kRowBlockRows - 1);
+            a[u] = __builtin_nontemporal_load(valD + dc);
+            v[u] = __builtin_nontemporal_load(xg + src[u]);
+            r[u] = d < d1 ? rr : -1 - lane;  // distinct negative keys: padding lanes form no runs
+        }
+        // The next batch's positions come from LDS only: computed while this batch's loads are in flight.
+        const int32_t next = start + kBlkWaves * kBatch;
+        if (next < d1) {
+            BatchSources(tabD, tabDelta, P, next, d1, lane, src);
+        }
+#pragma unroll
+        for (int u = 0; u < kReduceBatch; ++u) {
+            double t = static_cast<double>(a[u]) * static_cast<double>(v[u]);
+            const int32_t key = r[u];
+            // Entries of one row are neighbours inside a chunk.  Where a row has three or more in a
+            // row of 16 lanes, add them up there and let the last lane of each run add to LDS:
+            // atomics on one address are carried out one after the other.
+            const int32_t prev2 = DppMove<kDppRowShr + 2>(key);
+            if (__any((lane & 15) >= 2 && prev2 == key)) {
+                const int32_t prev = DppMove<kDppRowShr + 1>(key);
+                int closed = ((lane & 15) == 0 || prev != key) ? 1 : 0;
+                RunSumStep<1>(t, closed);
+                RunSumStep<2>(t, closed);
+                RunSumStep<4>(t, closed);
+                RunSumStep<8>(t, closed);
+                const int32_t nxt = DppMove<kDppRowShl + 1>(key);
+                if (key >= 0 && ((lane & 15) == 15 || nxt != key)) {
+                    atomicAdd(&acc[key], t);
+                }
+            } else if (key >= 0) {
+                atomicAdd(&acc[key], t);
+            }
+        }
+    }
+    __syncthreads();
+    const double alpha = ReadScalar<double>(alphaS), beta = ReadScalar<double>(betaS);
+    for (int i = tid; i < row1 - row0; i += kBlkThreads) {
+        const int64_t row = row0 + i;
+        double o = alpha * acc[i];
+        if (beta != 0.0) {
+            o += beta * static_cast<double>(yIn[row]);
+        }
+        y[row] = static_cast<float>(o);
+    }
+}
+
+// ------------------------------------------------------------------- host
+
+namespace {
+
+struct BlockedLayout {
+    int32_t P, B, window, passes;
+    // used by every launch
+    int64_t colLocalOff, xgOff, valOff, rowLocalOff, srcStartOff, dstStartOff, srcStartTOff, orderOff, blockRowOff;
+    // preprocessing only
+    int64_t keys0Off, keys1Off, pos0Off, pos1Off, rowOfPosOff, tableOff, scratchOff;
+    int64_t bytes;
+};
+
+// 0 panels: the layout does not apply.
+BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz)
+{
+    BlockedLayout l{};
+    if (rows <= 0 || cols <= 0 || nnz <= 0 || nnz > INT32_MAX || rows >= INT32_MAX || cols > INT32_MAX) {
+        return l;
+    }
+    const int64_t P = (cols + kPanelCols - 1) >> kPanelLog;
+    const int64_t fullBlocks = rows >> kRowBlockLog;
+    int64_t window = nnz / (fullBlocks > 0 ? fullBlocks : 1);
+    window = window < kMinEntryWindow ? kMinEntryWindow : window;
+    const int64_t B = ((rows + kRowBlockRows - 1) >> kRowBlockLog) + nnz / window + 1;
+    // x must be larger than an L2 (2^20 columns) for the two passes to pay, and the chunks long enough to stream.
+    if (cols <= (int64_t{1} << 20) || P > kMaxPanels || P * B + 1 > INT32_MAX || nnz / (P * B) < kMinChunkEntries) {
+        return l;
+    }
+    l.P = static_cast<int32_t>(P);
+    l.B = static_cast<int32_t>(B);
+    l.window = static_cast<int32_t>(window);
+    int bits = 0;
+    while ((int64_t{1} << bits) < P) {
+        ++bits;
+    }
+    l.passes = (bits + 3) / 4;
+    auto align = [](int64_t v) { return (v + 255) / 256 * 256; };
+    int64_t off = 256;  // header: status word of the analysis
+    l.colLocalOff = off; off += align(2 * nnz + 8);
+    l.xgOff = off; off += align(4 * nnz + 16);
+    l.valOff = off; off += align(4 * nnz);
+    l.rowLocalOff = off; off += align(2 * nnz);
+    l.srcStartOff = off; off += align(4 * (P * B + 1));
+    l.dstStartOff = off; off += align(4 * (P * B + 1));
+    l.srcStartTOff = off; off += align(4 * P * B);
+    l.orderOff = off; off += align(4 * B);
+    l.blockRowOff = off; off += align(4 * (B + 1));
+    l.keys0Off = off; off += align(4 * nnz);
+    l.keys1Off = off; off += align(4 * nnz);
+    l.pos0Off = off; off += align(4 * nnz);
+    l.pos1Off = off; off += align(4 * nnz);
+    l.rowOfPosOff = off; off += align(4 * nnz);
+    l.tableOff = off; off += align(4 * RadixTableInts(nnz));
+    const int64_t scanA = ScanScratchInts(RadixTableInts(nnz)), scanB = ScanScratchInts(P * B + 1);
+    l.scratchOff = off; off += align(4 * (scanA > scanB ? scanA : scanB));
+    l.bytes = off;
+    return l;
+}
+
+uint32_t GridOf(int64_t items, int64_t perBlock, int64_t cap)
+{
+    int64_t g = (items + perBlock - 1) / perBlock;
+    g = g < 1 ? 1 : g;
+    return static_cast<uint32_t>(g > cap ? cap : g);
+}
+
+}  // namespace
+
+int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
+{
+    const BlockedLayout l = MakeBlockedLayout(a.rows, a.cols, a.nnz);
+    if (l.P == 0 || plan.numPanels != l.P || plan.numRowBlocks != l.B) {
+        return OPSPARSE_E_INVALID;
+    }
+    if (a.ws == nullptr || static_cast<int64_t>(a.wsBytes) < l.bytes || plan.bytes != l.bytes) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    auto *base = static_cast<unsigned char *>(a.ws);
+    auto ints = [&](int64_t off) { return reinterpret_cast<const int32_t *>(base + off); };
+    const auto *colLocal = reinterpret_cast<const uint16_t *>(base + l.colLocalOff);
+    const auto *rowLocal = reinterpret_cast<const uint16_t *>(base + l.rowLocalOff);
+    auto *xg = reinterpret_cast<float *>(base + l.xgOff);
+    const auto *valD = reinterpret_cast<const float *>(base + l.valOff);
+    // Few panels: several workgroups per panel, so that every CU has one.
+    const int32_t splits = l.P >= 192 ? 1 : (256 + l.P - 1) / l.P;
+    hipLaunchKernelGGL(SpmvBlockGatherKernel, dim3(static_cast<uint32_t>(l.P) * splits), dim3(kBlkThreads), 0, a.stream,
+                       colLocal, static_cast<const float *>(a.x), xg, ints(l.srcStartOff), a.cols, l.B, splits);
+    hipLaunchKernelGGL(SpmvBlockReduceKernel, dim3(static_cast<uint32_t>(l.B)), dim3(kBlkThreads), 0, a.stream, valD, xg,
+                       rowLocal, ints(l.dstStartOff), ints(l.srcStartTOff), l.P, ints(l.orderOff), ints(l.blockRowOff),
+                       static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha, a.beta);
+    return CheckLaunch();
+}
+
+}  // namespace opsparse
+
+using namespace opsparse;
+
+extern "C" {
+
+size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz)
+{
+    return static_cast<size_t>(MakeBlockedLayout(rows, cols, nnz).bytes);
+}
+
+int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
+                                      int64_t rows, int64_t cols, int64_t nnz, void *workspace, size_t workspaceBytes,
+                                      OpsparseSpmvPlan *plan, void *stream)
+{
+    if (plan == nullptr || rowOffsets == nullptr || colInd == nullptr || csrValues == nullptr) {
+        return OPSPARSE_E_INVALID;
+    }
+    const BlockedLayout l = MakeBlockedLayout(rows, cols, nnz);
+    if (l.P == 0) {
+        return OPSPARSE_E_UNSUPPORTED;
+    }
+    if (workspace == nullptr || static_cast<int64_t>(workspaceBytes) < l.bytes) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    auto s = static_cast<hipStream_t>(stream);
+    auto *base = static_cast<unsigned char *>(workspace);
+    auto ints = [&](int64_t off) { return reinterpret_cast<int32_t *>(base + off); };
+    int32_t *status = ints(0);
+    int32_t *keys[2] = {ints(l.keys0Off), ints(l.keys1Off)};
+    int32_t *poss[2] = {ints(l.pos0Off), ints(l.pos1Off)};
+    int32_t *rowOfPos = ints(l.rowOfPosOff), *table = ints(l.tableOff), *scratch = ints(l.scratchOff);
+    int32_t *srcStart = ints(l.srcStartOff), *dstStart = ints(l.dstStartOff), *srcStartT = ints(l.srcStartTOff);
+    int32_t *blockOrder = ints(l.orderOff), *blockRow = ints(l.blockRowOff);
+    auto *colLocal = reinterpret_cast<uint16_t *>(base + l.colLocalOff);
+    auto *rowLocal = reinterpret_cast<uint16_t *>(base + l.rowLocalOff);
+    auto *valD = reinterpret_cast<float *>(base + l.valOff);
+
+    LaunchFillI32(status, 1, 0, s);
+    LaunchExpandRows(rowOffsets, rows, nnz, 0, rowOfPos, s);
+    // Entries in (panel, original position) order: stable 4-bit radix passes over the panel number.
+    int cur = 0;
+    for (int32_t pass = 0; pass < l.passes; ++pass) {
+        const int32_t *keysIn = pass == 0 ? colInd : keys[cur];
+        const int32_t *posIn = pass == 0 ? nullptr : poss[cur];
+        const int out = pass == 0 ? 0 : 1 - cur;
+        LaunchRadixPass(keysIn, posIn, keys[out], poss[out], nnz, 0, kPanelLog + 4 * pass, table, scratch, s);
+        cur = out;
+    }
+    const int32_t *colSorted = keys[cur], *pos = poss[cur];
+    int32_t *chunkKey = keys[1 - cur], *rowOfSrc = poss[1 - cur];
+    hipLaunchKernelGGL(BlockedChunkKeysKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
+                       colSorted, pos, rowOfPos, rowOffsets, nnz, cols, l.B, l.window, colLocal, chunkKey, rowOfSrc,
+                       status);
+    int32_t bad = 0;
+    if (hipMemcpyAsync(&bad, status, sizeof(bad), hipMemcpyDeviceToHost, s) != hipSuccess ||
+        hipStreamSynchronize(s) != hipSuccess) {
+        (void)hipGetLastError();
+        return OPSPARSE_E_LAUNCH;
+    }
+    if (bad != 0) {
+        return OPSPARSE_E_INVALID;  // a column index outside [0, cols)
+    }
+    const int64_t chunks = static_cast<int64_t>(l.P) * l.B;
+    LaunchIndicesToOffsets(chunkKey, nnz, chunks, 0, srcStart, scratch, s);
+    hipLaunchKernelGGL(BlockedTablesKernel, dim3(GridOf(chunks, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
+                       srcStart, l.P, l.B, dstStart, srcStartT);
+    LaunchInclusiveScanI32(dstStart + 1, dstStart + 1, chunks, 0, scratch, s);
+    LaunchFillI32(blockRow, l.B + 1, static_cast<int32_t>(rows), s);
+    hipLaunchKernelGGL(BlockedRowBlocksKernel, dim3(GridOf(rows, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
+                       rowOffsets, static_cast<int32_t>(rows), l.window, l.B, blockRow);
+    hipLaunchKernelGGL(BlockedScatterKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
+                       pos, rowOfSrc, chunkKey, csrValues, srcStart, dstStart, blockRow, nnz, l.P, l.B, valD, rowLocal);
+    hipLaunchKernelGGL(BlockedOrderKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
+                       dstStart, l.P, l.B, blockOrder);
+    if (CheckLaunch() != OPSPARSE_OK) {
+        return OPSPARSE_E_LAUNCH;
+    }
+    OpsparseSpmvPlan p{};
+    p.kernel = OPSPARSE_SPMV_BLOCKED_GATHER;
+    p.numPanels = l.P;
+    p.panelShift = kPanelLog;
+    p.numRowBlocks = l.B;
+    p.entryWindow = l.window;
+    p.rows = rows;
+    p.nnz = nnz;
+    p.bytes = l.bytes;
+    *plan = p;
+    return OPSPARSE_OK;
+}
+
+}  // extern "C"

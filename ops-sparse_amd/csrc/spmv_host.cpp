@@ -6,6 +6,8 @@
 // copy of the whole row-offset array with a stream synchronisation (:86-112)
 // and the on-chip-buffer limit on the longest row (:244-252) — rows of any
 // length are handled by the merge-path kernels.
+#include <cstdlib>
+
 #include "internal.h"
 
 namespace {
@@ -97,15 +99,18 @@ aclsparseStatus_t ValidateData(SpmvCall *c, aclDataType computeType)
     return ACL_SPARSE_STATUS_SUCCESS;
 }
 
-// Bytes of the column-panel layout when CSR_ALG2 asks for it and it applies (fp32, op(A) = A, 2..16 panels).
-size_t PanelBytes(aclsparseOperation_t opA, aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX,
-                  aclsparseConstDnVecDescr_t vecY, aclDataType computeType, aclsparseSpMVAlg_t alg)
+// The re-stored layouts CSR_ALG2 asks for, where they apply (fp32, op(A) = A, x larger than an L2): the
+// blocked-gather layout first, the column panels where that one does not fit the matrix.
+using Restored = opsparse::RestoredChoice;
+
+Restored RestoredLayout(aclsparseOperation_t opA, aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX,
+                        aclsparseConstDnVecDescr_t vecY, aclDataType computeType, aclsparseSpMVAlg_t alg)
 {
     if (alg != ACL_SPARSE_SPMV_CSR_ALG2 || opA != ACL_SPARSE_OP_NON_TRANSPOSE || computeType != ACL_FLOAT ||
         matA->valueType != ACL_FLOAT || vecX->valueType != ACL_FLOAT || vecY->valueType != ACL_FLOAT) {
-        return 0;
+        return {0, 0};
     }
-    return opsparse_spmv_csr_panels_workspace_bytes(matA->rows, matA->cols, matA->nnz);
+    return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz);
 }
 
 aclsparseStatus_t FromLaunch(int rc)
@@ -120,6 +125,35 @@ aclsparseStatus_t FromLaunch(int rc)
 }
 
 }  // namespace
+
+namespace opsparse {
+
+RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz)
+{
+    if (std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") == nullptr) {
+        const size_t blocked = opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz);
+        if (blocked > 0) {
+            return {OPSPARSE_SPMV_BLOCKED_GATHER, blocked};
+        }
+    }
+    const size_t panels = opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz);
+    if (panels > 0) {
+        return {OPSPARSE_SPMV_COLUMN_PANELS, panels};
+    }
+    return {0, 0};
+}
+
+int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const float *values, int64_t rows,
+                    int64_t cols, int64_t nnz, void *buffer, size_t bytes, OpsparseSpmvPlan *plan, void *stream)
+{
+    if (kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {
+        return opsparse_spmv_csr_blocked_analyse(rowOffsets, colInd, values, rows, cols, nnz, buffer, bytes, plan,
+                                                 stream);
+    }
+    return opsparse_spmv_csr_panels_analyse(rowOffsets, colInd, values, rows, cols, nnz, buffer, bytes, plan, stream);
+}
+
+}  // namespace opsparse
 
 extern "C" {
 
@@ -137,8 +171,8 @@ aclsparseStatus_t aclsparseSpMVGetBufferSize(aclsparseHandle_t handle, aclsparse
         return ACL_SPARSE_STATUS_INVALID_VALUE;
     }
     const size_t plain = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
-    const size_t panels = PanelBytes(opA, matA, vecX, vecY, computeType, alg);
-    *bufferSize = panels > plain ? panels : plain;
+    const Restored restored = RestoredLayout(opA, matA, vecX, vecY, computeType, alg);
+    *bufferSize = restored.bytes > plain ? restored.bytes : plain;
     return ACL_SPARSE_STATUS_SUCCESS;
 }
 
@@ -163,13 +197,13 @@ aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOpe
         return ACL_SPARSE_STATUS_INSUFFICIENT_RESOURCES;
     }
     OpsparseSpmvPlan plan{};
-    const size_t panels = PanelBytes(opA, matA, vecX, vecY, computeType, alg);
+    const Restored restored = RestoredLayout(opA, matA, vecX, vecY, computeType, alg);
     int rc;
-    if (panels > 0) {
-        rc = opsparse_spmv_csr_panels_analyse(static_cast<const int32_t *>(matA->rowOffsets),
-                                              static_cast<const int32_t *>(matA->colInd),
-                                              static_cast<const float *>(matA->values), matA->rows, matA->cols,
-                                              matA->nnz, externalBuffer, panels, &plan, handle->stream);
+    if (restored.kernel != 0) {
+        rc = opsparse::AnalyseRestored(restored.kernel, static_cast<const int32_t *>(matA->rowOffsets),
+                                       static_cast<const int32_t *>(matA->colInd),
+                                       static_cast<const float *>(matA->values), matA->rows, matA->cols, matA->nnz,
+                                       externalBuffer, restored.bytes, &plan, handle->stream);
     } else {
         const size_t bytes = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
         rc = opsparse_spmv_csr_analyse(static_cast<const int32_t *>(matA->rowOffsets), matA->rows, matA->cols,

@@ -27,6 +27,7 @@
 #include <type_traits>
 
 #include "convert_internal.h"
+#include "spmv_internal.h"
 #include "device_utils.h"
 
 namespace opsparse {
@@ -772,25 +773,6 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvTransposeScatterKernel(
 
 namespace {
 
-struct SpmvArgs {
-    const int32_t *rowOffsets;
-    const int32_t *colInd;
-    const void *vals;
-    const void *x;
-    void *y;
-    const void *yIn;  // old y (may be y itself)
-    int64_t rows, cols, nnz;
-    OpsparseScalar alpha, beta;
-    void *ws;
-    size_t wsBytes;
-    hipStream_t stream;
-};
-
-inline int CheckLaunch()
-{
-    return hipGetLastError() == hipSuccess ? OPSPARSE_OK : OPSPARSE_E_LAUNCH;
-}
-
 // Number of compute units of the current device (256 on MI355X), read once.
 inline int ComputeUnits()
 {
@@ -973,6 +955,12 @@ int RunPlanned(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
                 return LaunchPanels<OutT>(a, plan);
             } else {
                 return OPSPARSE_E_UNSUPPORTED;  // the panel copy holds fp32 values
+            }
+        case OPSPARSE_SPMV_BLOCKED_GATHER:
+            if constexpr (std::is_same<ValT, float>::value && std::is_same<OutT, float>::value) {
+                return LaunchBlockedF32(a, plan);
+            } else {
+                return OPSPARSE_E_UNSUPPORTED;  // the re-stored copy holds fp32 values
             }
         default:
             return OPSPARSE_E_INVALID;

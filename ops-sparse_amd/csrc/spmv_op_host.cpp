@@ -77,15 +77,16 @@ bool Plain(const aclsparseSpMVOpDescr *d)
     return d->rowOffsetsType == ACL_SPARSE_INDEX_32I && d->indexBase == ACL_SPARSE_INDEX_BASE_ZERO;
 }
 
-// ALG2's device-side reorder is, for a matrix whose x does not fit an L2, the column-panel layout: the
-// buffer then holds a copy of the matrix (indices and values), which is why csrValues must not change under
-// an ALG2 descriptor (reference include/cann_ops_sparse.h:64-69 says the same of its own ALG2).
-size_t PanelBytes(aclsparseConstSpMatDescr_t matA)
+// ALG2's device-side reorder is, for a matrix whose x does not fit an L2, a re-stored layout (blocked gather,
+// else column panels): the buffer then holds a copy of the matrix (indices and values), which is why csrValues
+// must not change under an ALG2 descriptor (reference include/cann_ops_sparse.h:64-69 says the same of its
+// own ALG2).
+opsparse::RestoredChoice RestoredLayout(aclsparseConstSpMatDescr_t matA)
 {
     if (matA->rowOffsetsType != ACL_SPARSE_INDEX_32I || matA->idxBase != ACL_SPARSE_INDEX_BASE_ZERO) {
-        return 0;
+        return {0, 0};
     }
-    return opsparse_spmv_csr_panels_workspace_bytes(matA->rows, matA->cols, matA->nnz);
+    return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz);
 }
 
 aclsparseStatus_t FromLaunch(int rc)
@@ -131,8 +132,8 @@ aclsparseStatus_t aclsparseSpMVOp_bufferSize(aclsparseHandle_t handle, aclsparse
     *bufferSize = 0;
     if (alg == ACL_SPARSE_SPMVOP_ALG2) {
         const size_t plain = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
-        const size_t panels = PanelBytes(matA);
-        *bufferSize = panels > plain ? panels : plain;
+        const size_t restored = RestoredLayout(matA).bytes;
+        *bufferSize = restored > plain ? restored : plain;
     }
     return ACL_SPARSE_STATUS_SUCCESS;
 }
@@ -186,13 +187,13 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
         d->userBuffer = buffer;
         // The nnz-balanced split of ALG2: analyse the rows into the caller's buffer.
         if (Plain(d) && d->rows > 0 && d->nnz > 0 && d->rowOffsets != nullptr) {
-            const size_t panels = PanelBytes(matA);
+            const opsparse::RestoredChoice restored = RestoredLayout(matA);
             const int rc =
-                panels > 0 && d->colInd != nullptr && d->values != nullptr
-                    ? opsparse_spmv_csr_panels_analyse(static_cast<const int32_t *>(d->rowOffsets),
-                                                       static_cast<const int32_t *>(d->colInd),
-                                                       static_cast<const float *>(d->values), d->rows, d->cols, d->nnz,
-                                                       buffer, panels, &d->plan, handle->stream)
+                restored.kernel != 0 && d->colInd != nullptr && d->values != nullptr
+                    ? opsparse::AnalyseRestored(restored.kernel, static_cast<const int32_t *>(d->rowOffsets),
+                                                static_cast<const int32_t *>(d->colInd),
+                                                static_cast<const float *>(d->values), d->rows, d->cols, d->nnz, buffer,
+                                                restored.bytes, &d->plan, handle->stream)
                     : opsparse_spmv_csr_analyse(static_cast<const int32_t *>(d->rowOffsets), d->rows, d->cols, d->nnz,
                                                 buffer, opsparse_spmv_csr_workspace_bytes(d->rows, d->nnz),
                                                 OPSPARSE_SPMV_AUTO, &d->plan, handle->stream);

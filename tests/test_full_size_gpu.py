@@ -54,7 +54,7 @@ def test_c2_laplacian_full(osa, workloads, gpu_ctx, preprocess):
     assert float(ones.sum()) == 4 * 2048
 
 
-def test_c3_power_law_full(osa, workloads, gpu_ctx):
+def test_c3_power_law_full(osa, workloads, gpu_ctx, monkeypatch):
     dev = gpu_ctx[0]
     cfg = workloads.config_c3(dev)
     A = cfg["A"]
@@ -67,9 +67,15 @@ def test_c3_power_law_full(osa, workloads, gpu_ctx):
     # without Preprocess (partition rebuilt per call in the handle workspace, or the vector kernel)
     y2 = _spmv(osa, gpu_ctx, cfg, preprocess=False)
     assert oracle.max_rel_err(y2.cpu().numpy(), gold) <= 1e-5
-    # the column-panel layout (CSR_ALG2): eight panels of 2^20 columns
+    # CSR_ALG2: the blocked-gather layout (256 panels of 2^15 columns, about a thousand row blocks) ...
+    assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(A["rows"], A["cols"], colind.size) > 0
     y5 = _spmv(osa, gpu_ctx, cfg, alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
     assert oracle.max_rel_err(y5.cpu().numpy(), gold) <= 1e-5
+    # ... and, with that one switched off, the column-panel layout (eight panels of 2^20 columns)
+    monkeypatch.setenv("OPS_SPARSE_SPMV_NO_BLOCKED", "1")
+    y6 = _spmv(osa, gpu_ctx, cfg, alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
+    monkeypatch.delenv("OPS_SPARSE_SPMV_NO_BLOCKED")
+    assert oracle.max_rel_err(y6.cpu().numpy(), gold) <= 1e-5
     # linearity: scaling x by 2 is exact in binary floating point
     cfg["x"] = cfg["x"] * 2.0
     y3 = _spmv(osa, gpu_ctx, cfg)

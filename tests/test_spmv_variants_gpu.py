@@ -165,10 +165,11 @@ def _wide_problem(rows, cols, seed, long_rows=()):
 
 
 @pytest.mark.parametrize("cols,panels", [(3_000_000, 3), (1_048_577, 2), (9_000_000, 9), (1_000_000, 0), (17_000_000, 0)])
-def test_column_panels_csr_alg2(osa, gpu_ctx, cols, panels):
-    """ACL_SPARSE_SPMV_CSR_ALG2: Preprocess re-stores the matrix as panels of 2^20 columns (x wider than an L2);
-    matrices with fewer than 2 or more than 16 panels silently take the ordinary families.  Same 1e-5 bar, and
-    bit-equal from run to run (partials are added in panel order)."""
+def test_column_panels_csr_alg2(osa, gpu_ctx, cols, panels, monkeypatch):
+    """ACL_SPARSE_SPMV_CSR_ALG2 with the blocked-gather layout switched off: Preprocess re-stores the matrix as
+    panels of 2^20 columns (x wider than an L2); matrices with fewer than 2 or more than 16 panels silently take
+    the ordinary families.  Same 1e-5 bar, and bit-equal from run to run (partials are added in panel order)."""
+    monkeypatch.setenv("OPS_SPARSE_SPMV_NO_BLOCKED", "1")
     dev, stream, handle = gpu_ctx
     rows = 60_000
     rowptr, colind, val, x, y0 = _wide_problem(rows, cols, cols % 1000, long_rows=((7, 90_000), (59_999, 30_000)))
@@ -191,8 +192,10 @@ def test_column_panels_csr_alg2(osa, gpu_ctx, cols, panels):
     assert np.array_equal(d[1].cpu().numpy(), colind) and np.array_equal(d[2].cpu().numpy(), val)
 
 
-def test_column_panels_through_spmvop_alg2(osa, gpu_ctx):
-    """aclsparseSpMVOp ALG2 on a wide matrix uses the same layout; Z separate from Y and aliased."""
+def test_column_panels_through_spmvop_alg2(osa, gpu_ctx, monkeypatch):
+    """aclsparseSpMVOp ALG2 on a wide matrix (blocked gather switched off) uses the panel layout; Z separate from Y
+    and aliased."""
+    monkeypatch.setenv("OPS_SPARSE_SPMV_NO_BLOCKED", "1")
     dev, stream, handle = gpu_ctx
     rows, cols = 40_000, 2_500_000
     rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 5, long_rows=((3, 50_000),))
@@ -210,6 +213,110 @@ def test_column_panels_through_spmvop_alg2(osa, gpu_ctx):
         gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.25, -0.5)
         assert oracle.max_rel_err(d_z.cpu().numpy(), gold) <= 1e-5
         op.close()
+
+
+@pytest.mark.parametrize("rows,cols,applies", [(60_000, 3_000_000, True), (60_000, 1_048_577, True),
+                                               (20_000, 17_000_000, True), (60_000, 1_000_000, False),
+                                               (300_000, 2_000_000, True)])
+def test_blocked_gather_csr_alg2(osa, gpu_ctx, rows, cols, applies):
+    """ACL_SPARSE_SPMV_CSR_ALG2 on a matrix whose x is wider than an L2: Preprocess re-stores the entries by
+    panels of 2^15 columns and row blocks, SpMV gathers x from LDS in one pass and sums row blocks in LDS in a
+    second.  Products are exact in fp64 and rounded once: the 1e-5 bar of every other family.  Rows longer than a
+    row block's entry window, empty rows and a last partial panel / row block are all in."""
+    dev, stream, handle = gpu_ctx
+    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, cols % 1000 + rows,
+                                               long_rows=((7, 90_000), (rows // 2, 1), (rows - 1, 30_000)))
+    L = osa.lib()
+    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size)
+    assert (need > 0) == applies
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    A = osa.Csr(rows, cols, d[0], d[1], d[2])
+    d_y = to_dev(y0, dev)
+    op = osa.SpmvOp(handle, A, osa.DnVec(d[3]), osa.DnVec(d_y), alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
+    assert op.buffer.numel() >= need
+    for alpha, beta in ((1.0, 0.0), (-2.0, 0.75), (0.5, 1.0)):
+        d_y.copy_(torch.from_numpy(y0))
+        op(alpha, beta)
+        stream.synchronize()
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, alpha, beta)
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+    assert np.array_equal(d[1].cpu().numpy(), colind) and np.array_equal(d[2].cpu().numpy(), val)
+
+
+def test_blocked_gather_hot_rows_and_unaligned_x(osa, gpu_ctx):
+    """Rows that put dozens of entries into one (panel, row block) chunk — the in-register run sums before the LDS
+    atomics — next to one- and two-entry rows, and an x that is only 4-byte aligned."""
+    dev, stream, handle = gpu_ctx
+    rows, cols = 50_000, 1_500_000
+    rng = np.random.default_rng(11)
+    lengths = rng.integers(0, 3, rows)
+    hot = rng.choice(rows, 40, replace=False)
+    lengths[hot] = rng.integers(2_000, 60_000, hot.size)
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = np.concatenate([np.sort(rng.choice(cols, int(l), replace=False)) for l in lengths]).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    x = rng.uniform(-1, 1, cols).astype(np.float32)
+    y0 = rng.uniform(-1, 1, rows).astype(np.float32)
+    assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size) > 0
+    d = [to_dev(a, dev) for a in (rowptr, colind, val)]
+    xbuf = torch.zeros(cols + 1, dtype=torch.float32, device=dev)
+    xbuf[1:].copy_(torch.from_numpy(x))
+    d_x = xbuf[1:]
+    assert d_x.data_ptr() % 16 == 4
+    d_y = to_dev(y0, dev)
+    op = osa.SpmvOp(handle, osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d_x), osa.DnVec(d_y),
+                    alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
+    op(1.5, -0.25)
+    stream.synchronize()
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.5, -0.25)
+    assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+
+def test_blocked_gather_through_spmvop_alg2(osa, gpu_ctx):
+    """aclsparseSpMVOp ALG2 on a wide matrix uses the blocked-gather layout; Z separate from Y and aliased."""
+    dev, stream, handle = gpu_ctx
+    rows, cols = 40_000, 2_500_000
+    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 5, long_rows=((3, 50_000),))
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    A = osa.Csr(rows, cols, d[0], d[1], d[2])
+    for alias in (False, True):
+        d_y = to_dev(y0, dev)
+        d_z = d_y if alias else torch.zeros(rows, dtype=torch.float32, device=dev)
+        Y = osa.DnVec(d_y)
+        Z = Y if alias else osa.DnVec(d_z)
+        op = osa.SpmvOpPlan(handle, A, osa.DnVec(d[3]), Y, Z, alg=osa.ACL_SPARSE_SPMVOP_ALG2)
+        assert op.buffer_bytes == osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size) > 0
+        op(1.25, -0.5)
+        stream.synchronize()
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.25, -0.5)
+        assert oracle.max_rel_err(d_z.cpu().numpy(), gold) <= 1e-5
+        op.close()
+
+
+def test_blocked_gather_rejects_column_out_of_range(osa, gpu_ctx):
+    """The analysis checks every column index against cols (the kernels index LDS with it) and returns
+    OPSPARSE_E_INVALID; aclsparseSpMVPreprocess turns that into INVALID_VALUE."""
+    dev, stream, handle = gpu_ctx
+    rows, cols = 30_000, 1_200_000
+    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 9)
+    colind = colind.copy()
+    colind[colind.size // 2] = cols + 5
+    L = osa.lib()
+    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size)
+    assert need > 0
+    d = [to_dev(a, dev) for a in (rowptr, colind, val)]
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    plan = osa.OpsparseSpmvPlan()
+    torch.cuda.synchronize()
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    rc = L.opsparse_spmv_csr_blocked_analyse(p(d[0]), p(d[1]), p(d[2]), rows, cols, colind.size, p(ws), need,
+                                             ctypes.byref(plan), ctypes.c_void_p(stream.cuda_stream))
+    assert rc == osa.OPSPARSE_E_INVALID
+    d_x, d_y = to_dev(x, dev), to_dev(y0, dev)
+    A, X, Y = osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d_x), osa.DnVec(d_y)
+    st = L.aclsparseSpMVPreprocess(handle.h, 0, None, A.d, X.d, None, Y.d, osa.ACL_FLOAT,
+                                   osa.ACL_SPARSE_SPMV_CSR_ALG2, p(ws))
+    assert st == osa.ACL_SPARSE_STATUS_INVALID_VALUE
 
 
 @pytest.mark.parametrize("dtype,rel", [(torch.float16, 2.0 ** -10), (torch.bfloat16, 2.0 ** -7)])
