@@ -46,9 +46,11 @@ constexpr int kPanelLog = 15;                     // columns per panel: 128 KiB 
 constexpr int kPanelCols = 1 << kPanelLog;
 constexpr int kRowBlockLog = 14;                  // rows per row block: 128 KiB of fp64 accumulators
 constexpr int kRowBlockRows = 1 << kRowBlockLog;
-constexpr int kMaxPanels = 2048;                  // chunk tables of one row block in LDS: 16 KiB
+constexpr int kMaxPanels = 1024;                  // chunk tables of one row block in LDS: 8 KiB
+constexpr int kMaxGroups = 11776;                 // chunk of every 64th entry of a row block in LDS: 23 KiB
 constexpr int kGatherBatch = 8;                   // groups of 4 entries in flight per lane, phase 1
-constexpr int kReduceBatch = 8;                   // entries in flight per lane, phase 2
+constexpr int kReduceBatch = 8;                   // entries per lane and batch, phase 2
+constexpr int kRunTrigger = 4;                    // run length inside 16 lanes from which runs are summed in registers
 constexpr int64_t kMinEntryWindow = 16384;
 constexpr int64_t kMinChunkEntries = 32;          // below this mean chunk size the layout does not pay
 
@@ -273,32 +275,92 @@ __device__ __forceinline__ void RunSumStep(double &t, int &closed)
     }
 }
 
-// Positions in xg (panel order) of the kReduceBatch * 64 entries of a wavefront's batch that
-// starts at `start` in block order.  tabD[p] is the first block-order position of the block's
-// chunk from panel p, tabDelta[p] the distance from there to the chunk in panel order.
-__device__ __forceinline__ void BatchSources(const int32_t *tabD, const int32_t *tabDelta, int32_t P, int32_t start,
-                                             int32_t end, int lane, int32_t (&src)[kReduceBatch])
+// Adds the per-lane sums of a wavefront to acc[key] (key < 0: nothing pending).
+__device__ __forceinline__ void FlushPending(double *acc, int32_t key, double pending)
 {
-    int lo = 0, hi = P;  // largest p with tabD[p] <= start
+    if (key < 0) {
+        return;
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        pending += __shfl_xor(pending, off);
+    }
+    if (threadIdx.x % kWave == 0) {
+        atomicAdd(&acc[key], pending);
+    }
+}
+
+// Chunk (panel) of block-order position `pos`: the largest p with tabD[p] <= pos.
+__device__ __forceinline__ int ChunkOf(const int32_t *tabD, int32_t P, int32_t pos)
+{
+    int lo = 0, hi = P;
     while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
-        if (tabD[mid] <= start) {
+        if (tabD[mid] <= pos) {
             lo = mid;
         } else {
             hi = mid;
         }
     }
-    int cur = lo;
+    return lo;
+}
+
+// Positions in xg (panel order) of the kReduceBatch * 64 entries of a wavefront's batch that starts at
+// `start` in block order (start - d0 a multiple of 64).  tabD[p] is the first block-order position of the
+// block's chunk from panel p, tabDelta[p] the distance from there to the chunk in panel order, and
+// groupChunk[g] the chunk of the block's entry 64 * g for g < groups (the rest of that table is not
+// written: padding positions past `end` use the last group).  Straight-line code: the LDS reads of all entries
+// are issued together and waited for four times per batch; only where two chunk bounds fall inside 64
+// entries does a lane search the table.
+__device__ __forceinline__ void BatchSources(const int32_t *tabD, const int32_t *tabDelta,
+                                             const uint16_t *groupChunk, int32_t groups, int32_t P, int32_t d0,
+                                             int32_t start, int32_t end, int lane, int32_t (&src)[kReduceBatch])
+{
+    start = start < end ? start : d0 + (end - 1 - d0) / kWave * kWave;  // past the end: the last group again
+    const int32_t g0 = (start - d0) / kWave;
+    int32_t i[kReduceBatch];
+    int p[kReduceBatch];
+    int beyond = 0;
+    if (g0 + kReduceBatch > kMaxGroups) {  // a block with more entries than the table covers
+        beyond = ChunkOf(tabD, P, start < end ? start : end - 1);
+    }
 #pragma unroll
     for (int u = 0; u < kReduceBatch; ++u) {
-        int32_t i = start + u * kWave + lane;
-        i = i < end ? i : end - 1;
-        int p = cur;
-        while (p + 1 < P && tabD[p + 1] <= i) {
-            ++p;
+        const int32_t pos = start + u * kWave + lane;
+        i[u] = pos < end ? pos : end - 1;
+        const int32_t g = g0 + u;
+        const int listed = groupChunk[g < groups ? g : groups - 1];
+        p[u] = g < kMaxGroups ? listed : beyond;
+    }
+    int32_t bound[kReduceBatch];
+#pragma unroll
+    for (int u = 0; u < kReduceBatch; ++u) {
+        bound[u] = tabD[p[u] + 1];  // p < P, tabD has P + 1 values
+    }
+#pragma unroll
+    for (int u = 0; u < kReduceBatch; ++u) {
+        p[u] += (p[u] + 1 < P && bound[u] <= i[u]) ? 1 : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < kReduceBatch; ++u) {
+        bound[u] = tabD[p[u] + 1];
+    }
+    bool more = false;
+#pragma unroll
+    for (int u = 0; u < kReduceBatch; ++u) {
+        more |= p[u] + 1 < P && bound[u] <= i[u];
+    }
+    if (__any(more)) {  // chunks of a few entries (a row block with hardly any): search instead of walking on
+#pragma unroll
+        for (int u = 0; u < kReduceBatch; ++u) {
+            if (p[u] + 1 < P && bound[u] <= i[u]) {
+                p[u] = ChunkOf(tabD, P, i[u]);
+            }
         }
-        src[u] = i + tabDelta[p];
-        cur = __shfl(p, kWave - 1);
+    }
+#pragma unroll
+    for (int u = 0; u < kReduceBatch; ++u) {
+        src[u] = i[u] + tabDelta[p[u]];
     }
 }
 
@@ -312,6 +374,7 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
     __shared__ double acc[kRowBlockRows];
     __shared__ int32_t tabD[kMaxPanels + 1];
     __shared__ int32_t tabDelta[kMaxPanels];
+    __shared__ uint16_t groupChunk[kMaxGroups];
     const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const int64_t blk = blockOrder[blockIdx.x];
     const int32_t row0 = blockRow[blk], row1 = blockRow[blk + 1];
@@ -329,39 +392,59 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
     }
     __syncthreads();
     const int32_t d0 = tabD[0], d1 = tabD[P];
-    constexpr int kBatch = kWave * kReduceBatch;
-    int32_t src[kReduceBatch];
-    int32_t start = d0 + wave * kBatch;
-    if (start < d1) {
-        BatchSources(tabD, tabDelta, P, start, d1, lane, src);
+    int32_t groups = (d1 - d0 + kWave - 1) / kWave;
+    groups = groups < kMaxGroups ? groups : kMaxGroups;
+    for (int32_t g = tid; g < groups; g += kBlkThreads) {
+        groupChunk[g] = static_cast<uint16_t>(ChunkOf(tabD, P, d0 + g * kWave));
     }
-    for (; start < d1; start += kBlkWaves * kBatch) {
+    __syncthreads();
+    constexpr int kBatch = kWave * kReduceBatch;
+    constexpr int kStride = kBlkWaves * kBatch;
+    // A long row fills whole wavefronts with its entries: those are summed per lane in `pending` and
+    // reach the row's accumulator once, when the row (pendingKey) changes.
+    double pending = 0.0;
+    int32_t pendingKey = -1;
+    int32_t start = d0 + wave * kBatch;
+    int32_t src[kReduceBatch];
+    if (start < d1) {
+        BatchSources(tabD, tabDelta, groupChunk, groups, P, d0, start, d1, lane, src);
+    }
+    for (; start < d1; start += kStride) {
         int32_t r[kReduceBatch];
         float v[kReduceBatch], a[kReduceBatch];
-        // Unconditional loads, positions past the end clamped: one wait covers the whole batch.
+        // Unconditional loads, positions past the end clamped to the last entry: one wait covers the batch.
 #pragma unroll
         for (int u = 0; u < kReduceBatch; ++u) {
             const int32_t d = start + u * kWave + lane;
             const int32_t dc = d < d1 ? d : d1 - 1;
-            const int32_t rr = static_cast<int32_t>(__builtin_nontemporal_load(rowLocal + dc)) & (kRowBlockRows - 1);
+            r[u] = static_cast<int32_t>(__builtin_nontemporal_load(rowLocal + dc));
             a[u] = __builtin_nontemporal_load(valD + dc);
             v[u] = __builtin_nontemporal_load(xg + src[u]);
-            r[u] = d < d1 ? rr : -1 - lane;  // distinct negative keys: padding lanes form no runs
         }
         // The next batch's positions come from LDS only: computed while this batch's loads are in flight.
-        const int32_t next = start + kBlkWaves * kBatch;
-        if (next < d1) {
-            BatchSources(tabD, tabDelta, P, next, d1, lane, src);
+        if (start + kStride < d1) {
+            BatchSources(tabD, tabDelta, groupChunk, groups, P, d0, start + kStride, d1, lane, src);
         }
 #pragma unroll
         for (int u = 0; u < kReduceBatch; ++u) {
             double t = static_cast<double>(a[u]) * static_cast<double>(v[u]);
-            const int32_t key = r[u];
-            // Entries of one row are neighbours inside a chunk.  Where a row has three or more in a
-            // row of 16 lanes, add them up there and let the last lane of each run add to LDS:
-            // atomics on one address are carried out one after the other.
-            const int32_t prev2 = DppMove<kDppRowShr + 2>(key);
-            if (__any((lane & 15) >= 2 && prev2 == key)) {
+            // padding lanes get distinct negative keys: they form no runs and add nothing
+            const int32_t key = start + u * kWave + lane < d1 ? (r[u] & (kRowBlockRows - 1)) : -1 - lane;
+            const int32_t first = __builtin_amdgcn_readfirstlane(key);
+            if (__all(key == first)) {
+                if (first != pendingKey) {
+                    FlushPending(acc, pendingKey, pending);
+                    pendingKey = first;
+                    pending = 0.0;
+                }
+                pending += t;
+                continue;
+            }
+            // Entries of one row are neighbours inside a chunk.  Where a row has several in a row of 16
+            // lanes, add them up there and let the last lane of each run add to LDS: atomics on one
+            // address are carried out one after the other.
+            const int32_t prevK = DppMove<kDppRowShr + kRunTrigger>(key);
+            if (__any((lane & 15) >= kRunTrigger && prevK == key)) {
                 const int32_t prev = DppMove<kDppRowShr + 1>(key);
                 int closed = ((lane & 15) == 0 || prev != key) ? 1 : 0;
                 RunSumStep<1>(t, closed);
@@ -377,6 +460,7 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
             }
         }
     }
+    FlushPending(acc, pendingKey, pending);
     __syncthreads();
     const double alpha = ReadScalar<double>(alphaS), beta = ReadScalar<double>(betaS);
     for (int i = tid; i < row1 - row0; i += kBlkThreads) {
