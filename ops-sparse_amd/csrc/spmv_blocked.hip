@@ -18,13 +18,18 @@
 //            workgroup owns one block, keeps an fp64 accumulator per row in
 //            LDS and streams the block's entries in (block, panel) order:
 //            value and local row index linearly, the gathered xg in one
-//            contiguous piece per (panel, block) chunk.  val * xg is exact in
-//            fp64; a row's result is rounded once when the block is written.
+//            contiguous piece per (panel, block) chunk.  Chunks are padded to
+//            multiples of 8 positions in that order, so that a lane's 8
+//            consecutive positions share a chunk and all three streams come
+//            as 16-byte loads.  val * xg is exact in fp64; a row's result is
+//            rounded once when the block is written.  The blocks are started
+//            heaviest first.
 //
 // Every entry costs 16 bytes of HBM traffic (2 + 4 in phase 1, 4 + 2 + 4 in
-// phase 2) against 8 algorithmic bytes plus a 128-byte line per gather in the
-// row-wise kernels.  The order of the fp64 additions into a row's accumulator
-// depends on scheduling; the sum is rounded to fp32 afterwards.
+// phase 2, plus the padding) against 8 algorithmic bytes plus a 128-byte line
+// per gather in the row-wise kernels.  The order of the fp64 additions into a
+// row's accumulator depends on scheduling; the sum is rounded to fp32
+// afterwards.
 //
 // Preprocessing (once per matrix, all on the device): a stable radix sort of
 // the entries on the panel number keeps rows, hence row blocks, ascending inside
@@ -40,17 +45,17 @@
 
 namespace opsparse {
 
-constexpr int kBlkThreads = 1024;                 // one workgroup per CU: it owns 128 KiB of LDS
+constexpr int kBlkThreads = 1024;                 // one workgroup per CU: it owns 128 KiB of LDS and more
 constexpr int kBlkWaves = kBlkThreads / kWave;
 constexpr int kPanelLog = 15;                     // columns per panel: 128 KiB of fp32 x
 constexpr int kPanelCols = 1 << kPanelLog;
 constexpr int kRowBlockLog = 14;                  // rows per row block: 128 KiB of fp64 accumulators
 constexpr int kRowBlockRows = 1 << kRowBlockLog;
 constexpr int kMaxPanels = 1024;                  // chunk tables of one row block in LDS: 8 KiB
-constexpr int kMaxGroups = 11776;                 // chunk of every 64th entry of a row block in LDS: 23 KiB
+constexpr int kMaxGroups = 11776;                 // chunk of every 64th position of a row block in LDS: 23 KiB
 constexpr int kGatherBatch = 8;                   // groups of 4 entries in flight per lane, phase 1
-constexpr int kReduceBatch = 8;                   // entries per lane and batch, phase 2
-constexpr int kRunTrigger = 4;                    // run length inside 16 lanes from which runs are summed in registers
+constexpr int kLaneEntries = 8;                   // consecutive entries a lane takes per batch, phase 2
+constexpr uint32_t kPadRow = 0x8000;              // local row of a padding position in block order
 constexpr int64_t kMinEntryWindow = 16384;
 constexpr int64_t kMinChunkEntries = 32;          // below this mean chunk size the layout does not pay
 
@@ -92,7 +97,8 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedChunkKeysKernel(
 }
 
 // From srcStart (first entry of chunk (panel, block) in panel order, P * B + 1 values):
-// dstStart[1 + block * P + panel] = size of the chunk (prefix-summed afterwards) and
+// dstStart[1 + block * P + panel] = size of the chunk, rounded up to a multiple of kLaneEntries (prefix-summed
+// afterwards: in block order every chunk starts on such a multiple, the gap behind it is padding), and
 // srcStartT[block * P + panel] = srcStart[panel * B + block].
 __global__ __launch_bounds__(kBlockThreads) void BlockedTablesKernel(const int32_t *__restrict__ srcStart, int32_t P,
                                                                      int32_t B, int32_t *__restrict__ dstStart,
@@ -106,7 +112,8 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedTablesKernel(const int32
     if (j < total) {
         const int64_t b = j / P, p = j % P;
         const int32_t s = srcStart[p * B + b];
-        dstStart[1 + j] = srcStart[p * B + b + 1] - s;
+        const int32_t count = srcStart[p * B + b + 1] - s;
+        dstStart[1 + j] = (count + kLaneEntries - 1) / kLaneEntries * kLaneEntries;
         srcStartT[j] = s;
     }
 }
@@ -144,7 +151,7 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedScatterKernel(
         const int32_t p = key / B, b = key % B;
         const int64_t dst = i - srcStart[key] + dstStart[static_cast<int64_t>(b) * P + p];
         valD[dst] = vals[pos[i]];
-        rowLocal[dst] = static_cast<uint16_t>((rowOfSrc[i] - blockRow[b]) & (kRowBlockRows - 1));
+        rowLocal[dst] = static_cast<uint16_t>((rowOfSrc[i] - blockRow[b]) & (kRowBlockRows - 1));  // < kPadRow
     }
 }
 
@@ -244,36 +251,8 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint1
 
 // ------------------------------------------------------------------ phase 2
 
-template <int CTRL>
-__device__ __forceinline__ int DppMove(int v)
-{
-    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, false);
-}
-
-template <int CTRL>
-__device__ __forceinline__ double DppMoveF64(double v)
-{
-    const long long bits = __double_as_longlong(v);
-    const int lo = DppMove<CTRL>(static_cast<int>(bits));
-    const int hi = DppMove<CTRL>(static_cast<int>(bits >> 32));
-    return __longlong_as_double((static_cast<long long>(hi) << 32) | static_cast<unsigned int>(lo));
-}
-
-constexpr int kDppRowShr = 0x110;  // row_shr:n is kDppRowShr + n: lane i of a row of 16 reads lane i - n
-constexpr int kDppRowShl = 0x100;  // row_shl:n is kDppRowShl + n
-
-// One step of the segmented sum inside rows of 16 lanes: a lane whose sum does not yet reach
-// back to the head of its run takes over the sum of the lane OFF to its left.
-template <int OFF>
-__device__ __forceinline__ void RunSumStep(double &t, int &closed)
-{
-    const double o = DppMoveF64<kDppRowShr + OFF>(t);
-    const int c = DppMove<kDppRowShr + OFF>(closed);
-    if (!closed) {
-        t += o;
-        closed = c;
-    }
-}
+typedef float Float4U1 __attribute__((ext_vector_type(4), aligned(4)));   // dword-aligned 16-byte load
+typedef uint32_t Uint4 __attribute__((ext_vector_type(4)));
 
 // Adds the per-lane sums of a wavefront to acc[key] (key < 0: nothing pending).
 __device__ __forceinline__ void FlushPending(double *acc, int32_t key, double pending)
@@ -305,66 +284,23 @@ __device__ __forceinline__ int ChunkOf(const int32_t *tabD, int32_t P, int32_t p
     return lo;
 }
 
-// Positions in xg (panel order) of the kReduceBatch * 64 entries of a wavefront's batch that starts at
-// `start` in block order (start - d0 a multiple of 64).  tabD[p] is the first block-order position of the
-// block's chunk from panel p, tabDelta[p] the distance from there to the chunk in panel order, and
-// groupChunk[g] the chunk of the block's entry 64 * g for g < groups (the rest of that table is not
-// written: padding positions past `end` use the last group).  Straight-line code: the LDS reads of all entries
-// are issued together and waited for four times per batch; only where two chunk bounds fall inside 64
-// entries does a lane search the table.
-__device__ __forceinline__ void BatchSources(const int32_t *tabD, const int32_t *tabDelta,
-                                             const uint16_t *groupChunk, int32_t groups, int32_t P, int32_t d0,
-                                             int32_t start, int32_t end, int lane, int32_t (&src)[kReduceBatch])
-{
-    start = start < end ? start : d0 + (end - 1 - d0) / kWave * kWave;  // past the end: the last group again
-    const int32_t g0 = (start - d0) / kWave;
-    int32_t i[kReduceBatch];
-    int p[kReduceBatch];
-    int beyond = 0;
-    if (g0 + kReduceBatch > kMaxGroups) {  // a block with more entries than the table covers
-        beyond = ChunkOf(tabD, P, start < end ? start : end - 1);
-    }
-#pragma unroll
-    for (int u = 0; u < kReduceBatch; ++u) {
-        const int32_t pos = start + u * kWave + lane;
-        i[u] = pos < end ? pos : end - 1;
-        const int32_t g = g0 + u;
-        const int listed = groupChunk[g < groups ? g : groups - 1];
-        p[u] = g < kMaxGroups ? listed : beyond;
-    }
-    int32_t bound[kReduceBatch];
-#pragma unroll
-    for (int u = 0; u < kReduceBatch; ++u) {
-        bound[u] = tabD[p[u] + 1];  // p < P, tabD has P + 1 values
-    }
-#pragma unroll
-    for (int u = 0; u < kReduceBatch; ++u) {
-        p[u] += (p[u] + 1 < P && bound[u] <= i[u]) ? 1 : 0;
-    }
-#pragma unroll
-    for (int u = 0; u < kReduceBatch; ++u) {
-        bound[u] = tabD[p[u] + 1];
-    }
-    bool more = false;
-#pragma unroll
-    for (int u = 0; u < kReduceBatch; ++u) {
-        more |= p[u] + 1 < P && bound[u] <= i[u];
-    }
-    if (__any(more)) {  // chunks of a few entries (a row block with hardly any): search instead of walking on
-#pragma unroll
-        for (int u = 0; u < kReduceBatch; ++u) {
-            if (p[u] + 1 < P && bound[u] <= i[u]) {
-                p[u] = ChunkOf(tabD, P, i[u]);
-            }
-        }
-    }
-#pragma unroll
-    for (int u = 0; u < kReduceBatch; ++u) {
-        src[u] = i[u] + tabDelta[p[u]];
-    }
-}
+// What a lane loads for one batch: kLaneEntries consecutive positions of the block.
+struct LanePiece {
+    Float4U1 a0, a1, x0, x1;
+    Uint4 rows;
+    bool live;  // false: a lane past the block's end, which re-read the last piece
+};
 
 // One workgroup per row block: y[row] = alpha * sum(val * xg) + beta * yIn[row].
+//
+// In block order every (panel, block) chunk starts on a multiple of kLaneEntries and is padded to one
+// (padding carries the local row kPadRow and the value 0).  A lane takes kLaneEntries consecutive positions
+// per batch, which therefore lie in one chunk: values, local rows and the gathered x all come as 16-byte
+// loads.  tabD[p] is the first block-order position of the block's chunk from panel p, tabDelta[p] the
+// distance from there to the chunk in panel order, groupChunk[g] the chunk of the block's position 64 * g.
+// Two batches are in flight: the next one's loads are issued, unconditionally, before this one is added up.
+// Entries of one row are neighbours: a lane adds its runs up in registers and touches the row's accumulator
+// in LDS once per run; a row that fills whole wavefronts is summed per lane in `pending` and reaches LDS once.
 __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
     const float *__restrict__ valD, const float *__restrict__ xg, const uint16_t *__restrict__ rowLocal,
     const int32_t *__restrict__ dstStart, const int32_t *__restrict__ srcStartT, int32_t P,
@@ -391,73 +327,98 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
         tabDelta[i] = srcStartT[blk * P + i] - dstStart[blk * P + i];
     }
     __syncthreads();
-    const int32_t d0 = tabD[0], d1 = tabD[P];
+    const int32_t d0 = tabD[0], d1 = tabD[P];  // both multiples of kLaneEntries
     int32_t groups = (d1 - d0 + kWave - 1) / kWave;
     groups = groups < kMaxGroups ? groups : kMaxGroups;
-    for (int32_t g = tid; g < groups; g += kBlkThreads) {
-        groupChunk[g] = static_cast<uint16_t>(ChunkOf(tabD, P, d0 + g * kWave));
+    // groupChunk[g] = chunk that holds position d0 + 64 g: every chunk writes the groups that start inside it
+    for (int32_t p = tid; p < P; p += kBlkThreads) {
+        int32_t g = (tabD[p] - d0 + kWave - 1) / kWave;
+        int32_t gEnd = (tabD[p + 1] - d0 + kWave - 1) / kWave;
+        gEnd = gEnd < groups ? gEnd : groups;
+        for (; g < gEnd; ++g) {
+            groupChunk[g] = static_cast<uint16_t>(p);
+        }
     }
     __syncthreads();
-    constexpr int kBatch = kWave * kReduceBatch;
+    constexpr int kBatch = kWave * kLaneEntries;
     constexpr int kStride = kBlkWaves * kBatch;
-    // A long row fills whole wavefronts with its entries: those are summed per lane in `pending` and
-    // reach the row's accumulator once, when the row (pendingKey) changes.
+
+    auto fetch = [&](int32_t start) {
+        LanePiece piece;
+        const int32_t mine = start + lane * kLaneEntries;
+        piece.live = mine < d1;
+        const int32_t i0 = piece.live ? mine : d1 - kLaneEntries;
+        // chunk of i0: from the table of every 64th position, at most two bounds further on
+        const int32_t g = (i0 - d0) / kWave;
+        int p = g < groups ? static_cast<int>(groupChunk[g]) : ChunkOf(tabD, P, i0);
+        p += (p + 1 < P && tabD[p + 1] <= i0) ? 1 : 0;
+        p += (p + 1 < P && tabD[p + 1] <= i0) ? 1 : 0;
+        if (__any(p + 1 < P && tabD[p + 1] <= i0)) {  // chunks of a few entries
+            p = ChunkOf(tabD, P, i0);
+        }
+        const Float4U1 *vp = reinterpret_cast<const Float4U1 *>(valD + i0);
+        const Float4U1 *xp = reinterpret_cast<const Float4U1 *>(xg + (i0 + tabDelta[p]));  // 4-byte aligned only
+        piece.a0 = __builtin_nontemporal_load(vp);
+        piece.a1 = __builtin_nontemporal_load(vp + 1);
+        piece.rows = __builtin_nontemporal_load(reinterpret_cast<const Uint4 *>(rowLocal + i0));
+        piece.x0 = __builtin_nontemporal_load(xp);
+        piece.x1 = __builtin_nontemporal_load(xp + 1);
+        return piece;
+    };
+
     double pending = 0.0;
     int32_t pendingKey = -1;
     int32_t start = d0 + wave * kBatch;
-    int32_t src[kReduceBatch];
     if (start < d1) {
-        BatchSources(tabD, tabDelta, groupChunk, groups, P, d0, start, d1, lane, src);
-    }
-    for (; start < d1; start += kStride) {
-        int32_t r[kReduceBatch];
-        float v[kReduceBatch], a[kReduceBatch];
-        // Unconditional loads, positions past the end clamped to the last entry: one wait covers the batch.
+        LanePiece cur = fetch(start);
+        while (true) {
+            const LanePiece next = fetch(start + kStride);  // past the end: every lane re-reads the last piece
+            const float av[kLaneEntries] = {cur.a0.x, cur.a0.y, cur.a0.z, cur.a0.w,
+                                            cur.a1.x, cur.a1.y, cur.a1.z, cur.a1.w};
+            const float xv[kLaneEntries] = {cur.x0.x, cur.x0.y, cur.x0.z, cur.x0.w,
+                                            cur.x1.x, cur.x1.y, cur.x1.z, cur.x1.w};
+            const uint32_t rws[4] = {cur.rows.x, cur.rows.y, cur.rows.z, cur.rows.w};
+            int32_t key[kLaneEntries];
+            double t[kLaneEntries];
+            bool same = true;
 #pragma unroll
-        for (int u = 0; u < kReduceBatch; ++u) {
-            const int32_t d = start + u * kWave + lane;
-            const int32_t dc = d < d1 ? d : d1 - 1;
-            r[u] = static_cast<int32_t>(__builtin_nontemporal_load(rowLocal + dc));
-            a[u] = __builtin_nontemporal_load(valD + dc);
-            v[u] = __builtin_nontemporal_load(xg + src[u]);
-        }
-        // The next batch's positions come from LDS only: computed while this batch's loads are in flight.
-        if (start + kStride < d1) {
-            BatchSources(tabD, tabDelta, groupChunk, groups, P, d0, start + kStride, d1, lane, src);
-        }
-#pragma unroll
-        for (int u = 0; u < kReduceBatch; ++u) {
-            double t = static_cast<double>(a[u]) * static_cast<double>(v[u]);
-            // padding lanes get distinct negative keys: they form no runs and add nothing
-            const int32_t key = start + u * kWave + lane < d1 ? (r[u] & (kRowBlockRows - 1)) : -1 - lane;
-            const int32_t first = __builtin_amdgcn_readfirstlane(key);
-            if (__all(key == first)) {
+            for (int j = 0; j < kLaneEntries; ++j) {
+                const uint32_t k = (j & 1) ? rws[j / 2] >> 16 : rws[j / 2] & 0xffffu;
+                // padding and lanes past the end carry key -1 and add nothing
+                key[j] = (cur.live && k < kPadRow) ? static_cast<int32_t>(k & (kRowBlockRows - 1)) : -1;
+                t[j] = static_cast<double>(av[j]) * static_cast<double>(xv[j]);
+                same = same && key[j] == key[0];
+            }
+            const int32_t first = __builtin_amdgcn_readfirstlane(key[0]);
+            if (first >= 0 && __all(same && key[0] == first)) {
+                // one row fills the wavefront's batch
                 if (first != pendingKey) {
                     FlushPending(acc, pendingKey, pending);
                     pendingKey = first;
                     pending = 0.0;
                 }
-                pending += t;
-                continue;
-            }
-            // Entries of one row are neighbours inside a chunk.  Where a row has several in a row of 16
-            // lanes, add them up there and let the last lane of each run add to LDS: atomics on one
-            // address are carried out one after the other.
-            const int32_t prevK = DppMove<kDppRowShr + kRunTrigger>(key);
-            if (__any((lane & 15) >= kRunTrigger && prevK == key)) {
-                const int32_t prev = DppMove<kDppRowShr + 1>(key);
-                int closed = ((lane & 15) == 0 || prev != key) ? 1 : 0;
-                RunSumStep<1>(t, closed);
-                RunSumStep<2>(t, closed);
-                RunSumStep<4>(t, closed);
-                RunSumStep<8>(t, closed);
-                const int32_t nxt = DppMove<kDppRowShl + 1>(key);
-                if (key >= 0 && ((lane & 15) == 15 || nxt != key)) {
-                    atomicAdd(&acc[key], t);
+                pending += ((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]));
+            } else {
+                double run = t[0];
+#pragma unroll
+                for (int j = 1; j < kLaneEntries; ++j) {
+                    if (key[j] != key[j - 1]) {
+                        if (key[j - 1] >= 0) {
+                            atomicAdd(&acc[key[j - 1]], run);
+                        }
+                        run = 0.0;
+                    }
+                    run += t[j];
                 }
-            } else if (key >= 0) {
-                atomicAdd(&acc[key], t);
+                if (key[kLaneEntries - 1] >= 0) {
+                    atomicAdd(&acc[key[kLaneEntries - 1]], run);
+                }
             }
+            start += kStride;
+            if (start >= d1) {
+                break;
+            }
+            cur = next;
         }
     }
     FlushPending(acc, pendingKey, pending);
@@ -479,6 +440,7 @@ namespace {
 
 struct BlockedLayout {
     int32_t P, B, window, passes;
+    int64_t padded;  // upper bound of the positions in block order
     // used by every launch
     int64_t colLocalOff, xgOff, valOff, rowLocalOff, srcStartOff, dstStartOff, srcStartTOff, orderOff, blockRowOff;
     // preprocessing only
@@ -499,7 +461,7 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz)
     window = window < kMinEntryWindow ? kMinEntryWindow : window;
     const int64_t B = ((rows + kRowBlockRows - 1) >> kRowBlockLog) + nnz / window + 1;
     // x must be larger than an L2 (2^20 columns) for the two passes to pay, and the chunks long enough to stream.
-    if (cols <= (int64_t{1} << 20) || P > kMaxPanels || P * B + 1 > INT32_MAX || nnz / (P * B) < kMinChunkEntries) {
+    if (cols <= (int64_t{1} << 20) || P > kMaxPanels || P * B + 1 > INT32_MAX || nnz + kLaneEntries * P * B > INT32_MAX || nnz / (P * B) < kMinChunkEntries) {
         return l;
     }
     l.P = static_cast<int32_t>(P);
@@ -512,10 +474,12 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz)
     l.passes = (bits + 3) / 4;
     auto align = [](int64_t v) { return (v + 255) / 256 * 256; };
     int64_t off = 256;  // header: status word of the analysis
+    const int64_t padded = nnz + kLaneEntries * P * B;  // every chunk padded to a multiple of kLaneEntries
+    l.padded = padded;
     l.colLocalOff = off; off += align(2 * nnz + 8);
-    l.xgOff = off; off += align(4 * nnz + 16);
-    l.valOff = off; off += align(4 * nnz);
-    l.rowLocalOff = off; off += align(2 * nnz);
+    l.xgOff = off; off += align(4 * nnz) + 256;  // a lane's 16-byte loads of xg may run 7 entries past a chunk
+    l.valOff = off; off += align(4 * padded);
+    l.rowLocalOff = off; off += align(2 * padded);
     l.srcStartOff = off; off += align(4 * (P * B + 1));
     l.dstStartOff = off; off += align(4 * (P * B + 1));
     l.srcStartTOff = off; off += align(4 * P * B);
@@ -635,6 +599,9 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     hipLaunchKernelGGL(BlockedTablesKernel, dim3(GridOf(chunks, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
                        srcStart, l.P, l.B, dstStart, srcStartT);
     LaunchInclusiveScanI32(dstStart + 1, dstStart + 1, chunks, 0, scratch, s);
+    // padding positions: local row kPadRow, value 0
+    LaunchFillI32(reinterpret_cast<int32_t *>(rowLocal), (l.padded + 1) / 2, static_cast<int32_t>(kPadRow * 0x10001u), s);
+    LaunchFillI32(reinterpret_cast<int32_t *>(valD), l.padded, 0, s);
     LaunchFillI32(blockRow, l.B + 1, static_cast<int32_t>(rows), s);
     hipLaunchKernelGGL(BlockedRowBlocksKernel, dim3(GridOf(rows, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
                        rowOffsets, static_cast<int32_t>(rows), l.window, l.B, blockRow);
