@@ -132,7 +132,7 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
 
 /*
  * BLOCKED_GATHER analysis (fp32, op(A) = A): bytes of the workspace, or 0 when the
- * family does not apply (it needs more than 2^20 and at most 2^26 columns, and at
+ * family does not apply (it needs more than 2^20 and at most 2^25 columns, and at
  * least 32 entries per (panel, row block) chunk on average).  Like the panel
  * analysis it re-stores indices AND values in the workspace; launches with the
  * resulting plan ignore the rowOffsets / colInd / csrValues arguments.  Returns
