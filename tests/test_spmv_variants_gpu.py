@@ -272,6 +272,38 @@ def test_blocked_gather_hot_rows_and_unaligned_x(osa, gpu_ctx):
     assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
 
 
+def test_blocked_gather_giant_row_and_device_scalars(osa, gpu_ctx):
+    """One row of a million entries — a row block with more 64-entry groups than its chunk table in LDS
+    covers, and whole wavefronts of a single row — and alpha / beta read from device memory."""
+    dev, stream, handle = gpu_ctx
+    rows, cols = 20_000, 2_200_000
+    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 3, long_rows=((11_111, 1_000_000), (11_112, 70_000)))
+    assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size) > 0
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    A, X = osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3])
+    d_y = to_dev(y0, dev)
+    Y = osa.DnVec(d_y)
+    op = osa.SpmvOp(handle, A, X, Y, alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
+    op(1.0, 0.0)
+    stream.synchronize()
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.0, 0.0)
+    assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+    scal = torch.tensor([-0.5, 2.0], dtype=torch.float32, device=dev)
+    d_y.copy_(torch.from_numpy(y0))
+    torch.cuda.synchronize()
+    handle.set_pointer_mode(osa.ACL_SPARSE_POINTER_MODE_DEVICE)
+    try:
+        rc = osa.lib().aclsparseSpMV(handle.h, 0, ctypes.c_void_p(scal.data_ptr()), A.d, X.d,
+                                     ctypes.c_void_p(scal.data_ptr() + 4), Y.d, osa.ACL_FLOAT,
+                                     osa.ACL_SPARSE_SPMV_CSR_ALG2, ctypes.c_void_p(op.buffer.data_ptr()))
+        assert rc == 0
+        stream.synchronize()
+    finally:
+        handle.set_pointer_mode(osa.ACL_SPARSE_POINTER_MODE_HOST)
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, -0.5, 2.0)
+    assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+
 def test_blocked_gather_through_spmvop_alg2(osa, gpu_ctx):
     """aclsparseSpMVOp ALG2 on a wide matrix uses the blocked-gather layout; Z separate from Y and aliased."""
     dev, stream, handle = gpu_ctx
