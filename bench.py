@@ -97,14 +97,19 @@ def load_traffic(name):
     return int(entry["fetch_kib"] * 1024 * table["fetch_scale"] + entry["write_kib"] * 1024 * table["write_scale"])
 
 
-def cpu_baseline_spmv(cfg, budget_s=15.0):
-    """The reference's SpmvCpu loop (oracle.spmv_f32), one thread, on the same matrix."""
+def cpu_baseline_spmv(cfg, y_gpu, budget_s=15.0):
+    """The reference's SpmvCpu loop (oracle.spmv_f32), one thread, on the same matrix; the GPU result of one
+    launch (y_gpu) is checked against the fp64-accumulated oracle on the way."""
     import oracle
     A = cfg["A"]
     rowptr, colind = A["rowptr"].cpu().numpy(), A["colind"].cpu().numpy()
     val = A["values"].cpu().float().numpy()
     x, y0 = cfg["x"].cpu().float().numpy(), cfg["y0"].cpu().float().numpy()
     rows, nnz = A["rows"], int(colind.size)
+    gold = oracle.spmv_f64(rows, A["cols"], rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])
+    err = oracle.max_rel_err(y_gpu.cpu().numpy(), gold)
+    if err > 1e-5:
+        sys.exit("bench.py: the GPU result differs from the fp64 oracle (max relative error %.3g > 1e-5)" % err)
     oracle.spmv_f32(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])  # warm
     reps, t0 = 0, time.perf_counter()
     while reps < 10 and time.perf_counter() - t0 < budget_s:
@@ -113,11 +118,13 @@ def cpu_baseline_spmv(cfg, budget_s=15.0):
     dt = (time.perf_counter() - t0) / reps
     return {"value": 2.0 * nnz / dt / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
             "sample": "full matrix, %d repeats of the reference's SpmvCpu loop restated in oracle/oracle.c "
-                      "(fp32 accumulate), %.1f ms each" % (reps, dt * 1e3)}
+                      "(fp32 accumulate), %.1f ms each" % (reps, dt * 1e3),
+            "gpu_vs_fp64_oracle_max_rel_err": err}
 
 
-def cpu_baseline_spmm(cfg, rows_sample=32768):
-    """The reference's spmm_csr_cpu loop (order i, j, p) on the first rows_sample rows."""
+def cpu_baseline_spmm(cfg, c_gpu, rows_sample=32768):
+    """The reference's spmm_csr_cpu loop (order i, j, p) on the first rows_sample rows; the same rows of the GPU
+    result of one launch (c_gpu) are checked against the fp64-accumulated oracle on the way."""
     import oracle
     A = cfg["A"]
     n = cfg["n"]
@@ -132,9 +139,16 @@ def cpu_baseline_spmm(cfg, rows_sample=32768):
     t0 = time.perf_counter()
     oracle.spmm_f32(rs, n, rowptr, colind, val, B.ravel(), n, C, n, cfg["alpha"], cfg["beta"])
     dt = time.perf_counter() - t0
+    gold = oracle.spmm_f64_rowmajor(rs, n, rowptr, colind, val, B, n, np.zeros((rs, n), np.float32), n, cfg["alpha"],
+                                    cfg["beta"])
+    err = oracle.max_rel_err(c_gpu[:rs].cpu().numpy(), np.asarray(gold))
+    tol = 1e-5 if A["values"].element_size() == 4 else 1e-3
+    if err > tol:
+        sys.exit("bench.py: the GPU result differs from the fp64 oracle (max relative error %.3g > %g)" % (err, tol))
     return {"value": 2.0 * nnz * n / dt / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
             "sample": "first %d of %d rows (%d nnz) against the full B, one run of the reference's "
-                      "SpmmCpuFp32 loop restated in oracle/oracle.c, %.1f s" % (rs, A["rows"], nnz, dt)}
+                      "SpmmCpuFp32 loop restated in oracle/oracle.c, %.1f s" % (rs, A["rows"], nnz, dt),
+            "gpu_vs_fp64_oracle_max_rel_err": err}
 
 
 def main():
@@ -216,6 +230,11 @@ def main():
     preprocess_ms = (time.perf_counter() - t_pre) * 1e3
 
     alpha, beta = cfg["alpha"], cfg["beta"]
+    first_result = None
+    if not args.no_cpu:  # one launch from the initial y / C, kept for the check in the CPU leg
+        op(alpha, beta)
+        stream.synchronize()
+        first_result = (y if not is_spmm else Cmat).clone()
     for _ in range(args.warmup):
         op(alpha, beta)
     stream.synchronize()
@@ -257,7 +276,7 @@ def main():
                      "copy_kernel_gbps": round(copy_gbps, 1), "read_kernel_gbps": round(read_gbps, 1)},
     }
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline_spmm(cfg) if is_spmm else cpu_baseline_spmv(cfg)
+        out["cpu_baseline"] = cpu_baseline_spmm(cfg, first_result) if is_spmm else cpu_baseline_spmv(cfg, first_result)
     print(json.dumps(out), flush=True)
     handle.close()
 
