@@ -56,6 +56,7 @@ constexpr int kMaxGroups = 11776;                 // chunk of every 64th positio
 constexpr int kGatherBatch = 8;                   // groups of 4 entries in flight per lane, phase 1
 constexpr int kLaneEntries = 8;                   // consecutive entries a lane takes per batch, phase 2
 constexpr uint32_t kPadRow = 0x8000;              // local row of a padding position in block order
+constexpr int32_t kRankedBlocks = 8192;           // up to here the block order is found by counting ranks
 constexpr int64_t kMinEntryWindow = 16384;
 constexpr int64_t kMinChunkEntries = 32;          // below this mean chunk size the layout does not pay
 
@@ -171,6 +172,16 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedOrderKernel(const int32_
         rank += (other > mine || (other == mine && j < i)) ? 1 : 0;
     }
     blockOrder[rank] = i;
+}
+
+// keys[b] = INT32_MAX - entries of block b: ascending keys are falling entry counts.
+__global__ __launch_bounds__(kBlockThreads) void BlockedOrderKeysKernel(const int32_t *__restrict__ dstStart, int32_t P,
+                                                                        int32_t B, int32_t *__restrict__ keys)
+{
+    const int32_t i = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
+    if (i < B) {
+        keys[i] = INT32_MAX - (dstStart[static_cast<int64_t>(i + 1) * P] - dstStart[static_cast<int64_t>(i) * P]);
+    }
 }
 
 // ------------------------------------------------------------------ phase 1
@@ -607,8 +618,20 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
                        rowOffsets, static_cast<int32_t>(rows), l.window, l.B, blockRow);
     hipLaunchKernelGGL(BlockedScatterKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
                        pos, rowOfSrc, chunkKey, csrValues, srcStart, dstStart, blockRow, nnz, l.P, l.B, valD, rowLocal);
-    hipLaunchKernelGGL(BlockedOrderKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
-                       dstStart, l.P, l.B, blockOrder);
+    if (l.B <= kRankedBlocks) {
+        hipLaunchKernelGGL(BlockedOrderKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
+                           dstStart, l.P, l.B, blockOrder);
+    } else {
+        // many blocks: a stable radix sort of the counts instead of B * B comparisons (the key / position
+        // arrays of the entry sort are free again)
+        hipLaunchKernelGGL(BlockedOrderKeysKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
+                           s, dstStart, l.P, l.B, keys[0]);
+        for (int32_t pass = 0; pass < 8; ++pass) {
+            const int in = pass % 2, out = 1 - in;
+            LaunchRadixPass(keys[in], pass == 0 ? nullptr : poss[in], keys[out], pass == 7 ? blockOrder : poss[out], l.B, 0,
+                            4 * pass, table, scratch, s);
+        }
+    }
     if (CheckLaunch() != OPSPARSE_OK) {
         return OPSPARSE_E_LAUNCH;
     }
