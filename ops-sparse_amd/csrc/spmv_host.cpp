@@ -250,6 +250,10 @@ aclsparseStatus_t aclsparseSpMV(aclsparseHandle_t handle, aclsparseOperation_t o
         ws = externalBuffer;
         wsBytes = static_cast<size_t>(plan->bytes);
     } else if (matA->nnz > 0 || (c.transpose && c.outType != OPSPARSE_F32)) {
+        if (c.transpose && externalBuffer != nullptr && matA->spmv.buffer == externalBuffer &&
+            matA->spmv.plan.rows == matA->rows && matA->spmv.plan.nnz == matA->nnz) {
+            plan = &matA->spmv.plan;  // op(A) = A^T only takes the row-length statistics from it
+        }
         // the merge-path partition of an unprepared call, or the fp32 staging vector of a transposed
         // product with fp16 / bf16 y (cols * 4 bytes: enlarge it with aclsparseSetWorkspace if need be)
         st = opsparse::EnsureWorkspace(handle);

@@ -769,6 +769,60 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvTransposeScatterKernel(
     }
 }
 
+// Row that holds entry k: the largest r in [lo, hi] with offsets[r] <= k.
+__device__ __forceinline__ int64_t RowOfEntry(const int32_t *offsets, int64_t lo, int64_t hi, int32_t k)
+{
+    while (lo < hi) {
+        const int64_t mid = (lo + hi + 1) >> 1;
+        if (offsets[mid] <= k) {
+            lo = mid;
+        } else {
+            hi = mid - 1;
+        }
+    }
+    return lo;
+}
+
+constexpr int kTransposeTile = 2048;      // entries per workgroup
+constexpr int kTransposeRowSlots = 2304;  // row offsets of one tile staged in LDS
+
+// The same product with equal numbers of ENTRIES per workgroup, whatever the row lengths: a tile of
+// kTransposeTile consecutive entries, the offsets of the rows it touches staged in LDS, every lane finds the
+// row of its entries there.  A row of 200 000 entries is spread over a hundred workgroups instead of being
+// walked by one lane group.
+template <typename ValT, typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmvTransposeFlatKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ x, float *__restrict__ y, int64_t rows, int64_t nnz, OpsparseScalar alphaS)
+{
+    __shared__ int32_t slice[kTransposeRowSlots];
+    __shared__ int64_t bounds[2];
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    const int64_t k0 = static_cast<int64_t>(blockIdx.x) * kTransposeTile;
+    const int64_t k1 = k0 + kTransposeTile < nnz ? k0 + kTransposeTile : nnz;
+    if (threadIdx.x < 2) {
+        const int32_t k = static_cast<int32_t>(threadIdx.x == 0 ? k0 : k1 - 1);
+        bounds[threadIdx.x] = RowOfEntry(rowOffsets, 0, rows - 1, k);
+    }
+    __syncthreads();
+    const int64_t rLo = bounds[0], rHi = bounds[1];
+    const bool staged = rHi - rLo + 2 <= kTransposeRowSlots;
+    if (staged) {
+        for (int64_t i = threadIdx.x; i <= rHi - rLo + 1; i += kBlockThreads) {
+            slice[i] = rowOffsets[rLo + i];
+        }
+    }
+    __syncthreads();
+    for (int64_t k = k0 + threadIdx.x; k < k1; k += kBlockThreads) {
+        const int32_t kk = static_cast<int32_t>(k);
+        const int64_t r = staged ? rLo + RowOfEntry(slice, 0, rHi - rLo, kk) : RowOfEntry(rowOffsets, rLo, rHi, kk);
+        const AccT ax = alpha * ToAcc<AccT>(x[r]);
+        if (ax != AccT(0)) {
+            atomicAdd(y + LoadStream(colInd + k), static_cast<float>(ax * ToAcc<AccT>(LoadStream(vals + k))));
+        }
+    }
+}
+
 // =============================================================== host side
 
 namespace {
@@ -1089,7 +1143,7 @@ OpsparseSpmvPlan AdHocPlan(int64_t rows, int64_t nnz, size_t wsBytes, const void
 }
 
 template <typename ValT, typename AccT>
-int RunTranspose(const SpmvArgs &a, int32_t outType)
+int RunTranspose(const SpmvArgs &a, int32_t outType, bool skewedRows)
 {
     if (outType != OPSPARSE_F32 && outType != OPSPARSE_F16 && outType != OPSPARSE_BF16) {
         return OPSPARSE_E_UNSUPPORTED;
@@ -1133,6 +1187,13 @@ int RunTranspose(const SpmvArgs &a, int32_t outType)
         return rc;
     }
     if (a.nnz == 0 || a.rows == 0) {
+        return finish();
+    }
+    if (skewedRows && a.nnz >= 8 * kTransposeTile) {
+        // equal entries per workgroup: no lane group is left walking a long row on its own
+        hipLaunchKernelGGL((SpmvTransposeFlatKernel<ValT, AccT>), dim3(GridFor(a.nnz, kTransposeTile)),
+                           dim3(kBlockThreads), 0, a.stream, a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
+                           static_cast<const ValT *>(a.x), acc, a.rows, a.nnz, a.alpha);
         return finish();
     }
     const int32_t g = VectorLanesFor(a.rows, a.nnz);
@@ -1396,10 +1457,14 @@ int opsparse_spmv_csr_launch_zy(const OpsparseSpmvPlan *plan, int32_t transpose,
         if (computeIsInt) {
             return OPSPARSE_E_UNSUPPORTED;
         }
+        // The analysis found a row far longer than the mean: the transposed product then splits the work by
+        // entries rather than by rows.
+        const bool skewedRows = plan != nullptr && rows > 0 &&
+                                static_cast<int64_t>(plan->maxRowNnz) > 16 * (nnz / rows) + 64;
         switch (valType) {
-            case OPSPARSE_F32: return RunTranspose<float, double>(a, outType);
-            case OPSPARSE_F16: return RunTranspose<Half, double>(a, outType);
-            case OPSPARSE_BF16: return RunTranspose<Bf16, double>(a, outType);
+            case OPSPARSE_F32: return RunTranspose<float, double>(a, outType, skewedRows);
+            case OPSPARSE_F16: return RunTranspose<Half, double>(a, outType, skewedRows);
+            case OPSPARSE_BF16: return RunTranspose<Bf16, double>(a, outType, skewedRows);
             default: return OPSPARSE_E_UNSUPPORTED;
         }
     }

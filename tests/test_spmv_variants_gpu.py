@@ -92,6 +92,29 @@ def test_transpose(osa, gpu_ctx, rows, cols, density, alpha, beta):
     assert np.abs(y - g32).max() <= 1e-2
 
 
+@pytest.mark.parametrize("val_dtype", [None, torch.float16])
+def test_transpose_skewed_rows_split_by_entries(osa, gpu_ctx, val_dtype):
+    """op(A) = A^T on rows of very different lengths after Preprocess: the work is cut into tiles of 2048 entries
+    (a row of 60 000 entries is shared by thirty workgroups), the rows of a tile found through their offsets in
+    LDS; long runs of empty rows in between make one tile span more rows than LDS holds.  The reference's fp32
+    rule for the transposed product (atomics in unspecified order)."""
+    rng = np.random.default_rng(31)
+    lengths = rng.integers(0, 6, 40_000)
+    lengths[5_000:12_000] = 0                       # thousands of empty rows inside one tile
+    lengths[[3, 20_000, 39_999]] = [60_000, 9_000, 25_000]
+    rows, cols = lengths.size, 70_000
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = np.concatenate([np.sort(rng.choice(cols, int(l), replace=False)) for l in lengths]).astype(np.int32)
+    rt = (lambda a: a) if val_dtype is None else (lambda a: torch.from_numpy(a).to(val_dtype).float().numpy())
+    val = rt(rng.uniform(-1, 1, colind.size).astype(np.float32))
+    x, y0 = rt(rng.uniform(-1, 1, rows).astype(np.float32)), rng.uniform(-1, 1, cols).astype(np.float32)
+    y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 1.5, 0.5, op=osa.ACL_SPARSE_OP_TRANSPOSE,
+                 val_dtype=val_dtype, out_dtype=torch.float32 if val_dtype is not None else None)
+    gold = oracle.spmv_trans_f64(rows, cols, rowptr, colind, val, x, y0, 1.5, 0.5)
+    d = np.abs(y - gold)
+    assert (d <= 2.0 ** -16 + 2.0 ** -10 * np.abs(gold)).mean() >= 0.99 and d.max() <= 1e-2
+
+
 def test_device_pointer_mode(osa, gpu_ctx):
     """alpha / beta read by the kernel from device memory; changing them needs no new Preprocess."""
     dev, stream, handle = gpu_ctx
