@@ -208,7 +208,7 @@ def main():
         X, Y = osa.DnVec(x), osa.DnVec(y)
         op = osa.SpmvOp(handle, csr, X, Y, preprocess=not args.no_preprocess,
                         alg=osa.ACL_SPARSE_SPMV_CSR_ALG2 if layout != "csr" else osa.ACL_SPARSE_SPMV_ALG_DEFAULT)
-        if layout == "blocked_gather" and not osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz):
+        if layout == "blocked_gather" and not osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, 0):
             layout = "column_panels" if osa.lib().opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz) else "csr"
         ncols = 1
         bytes_alg = wl.spmv_bytes_alg(rows, cols, nnz, vb, x.element_size(), y.element_size(), cfg["beta"] != 0)

@@ -83,6 +83,8 @@ typedef struct OpsparseSpmvPlan {
     int32_t panelShift;    /* COLUMN_PANELS / BLOCKED_GATHER: log2 of the panel width */
     int32_t numRowBlocks;  /* BLOCKED_GATHER: number of row blocks */
     int32_t entryWindow;   /* BLOCKED_GATHER: a row block also ends where the entry count passes a multiple of this */
+    int32_t transposed;    /* BLOCKED_GATHER: the layout was built for op(A) = A^T and serves only that */
+    int32_t reserved0;
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */
@@ -131,17 +133,19 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
                                      OpsparseSpmvPlan *plan, void *stream);
 
 /*
- * BLOCKED_GATHER analysis (fp32, op(A) = A): bytes of the workspace, or 0 when the
- * family does not apply (it needs more than 2^20 and at most 2^25 columns, and at
- * least 32 entries per (panel, row block) chunk on average).  Like the panel
+ * BLOCKED_GATHER analysis (fp32): bytes of the workspace, or 0 when the family does
+ * not apply (x must have more than 2^20 and at most 2^25 elements, and a (panel, row
+ * block) chunk at least 32 entries on average).  transpose != 0 builds the layout of
+ * y = alpha * A^T * x + beta * y instead: panels over the rows of A, blocks over its
+ * columns, with no atomics on y; a plan serves the op(A) it was built for.  Like the panel
  * analysis it re-stores indices AND values in the workspace; launches with the
  * resulting plan ignore the rowOffsets / colInd / csrValues arguments.  Returns
  * OPSPARSE_E_INVALID for a column index outside [0, cols).  Synchronises `stream` once.
  */
-size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz);
+size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t transpose);
 int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
-                                      int64_t rows, int64_t cols, int64_t nnz, void *workspace, size_t workspaceBytes,
-                                      OpsparseSpmvPlan *plan, void *stream);
+                                      int64_t rows, int64_t cols, int64_t nnz, int32_t transpose, void *workspace,
+                                      size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream);
 
 /* Same as opsparse_spmv_csr_launch with separate input and output vectors:
  * z = alpha * op(A) * x + beta * yIn.  z may be yIn (in place); yIn is only read

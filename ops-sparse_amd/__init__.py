@@ -111,7 +111,8 @@ class OpsparseScalar(ctypes.Structure):
 class OpsparseSpmvPlan(ctypes.Structure):
     _fields_ = [("kernel", i32), ("lanesPerRow", i32), ("rowsPerBlock", i32), ("mergeBlocks", i32),
                 ("maxRowNnz", i32), ("partitionReady", i32), ("numPanels", i32),
-                ("panelShift", i32), ("numRowBlocks", i32), ("entryWindow", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
+                ("panelShift", i32), ("numRowBlocks", i32), ("entryWindow", i32), ("transposed", i32),
+                ("reserved0", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
                 ("carryOff", i64), ("headOff", i64), ("bytes", i64), ("panelStart", i64 * 17)]
 
 
@@ -232,10 +233,10 @@ def lib():
     L.opsparse_spmv_csr_panels_workspace_bytes.restype = sz
     L.opsparse_spmv_csr_panels_workspace_bytes.argtypes = [i64, i64, i64]
     L.opsparse_spmv_csr_blocked_workspace_bytes.restype = sz
-    L.opsparse_spmv_csr_blocked_workspace_bytes.argtypes = [i64, i64, i64]
+    L.opsparse_spmv_csr_blocked_workspace_bytes.argtypes = [i64, i64, i64, i32]
     L.opsparse_spmv_csr_blocked_analyse.restype = ctypes.c_int
-    L.opsparse_spmv_csr_blocked_analyse.argtypes = [vp, vp, vp, i64, i64, i64, vp, sz, ctypes.POINTER(OpsparseSpmvPlan),
-                                                    vp]
+    L.opsparse_spmv_csr_blocked_analyse.argtypes = [vp, vp, vp, i64, i64, i64, i32, vp, sz,
+                                                    ctypes.POINTER(OpsparseSpmvPlan), vp]
     L.opsparse_spmv_csr_panels_analyse.restype = ctypes.c_int
     L.opsparse_spmv_csr_panels_analyse.argtypes = [vp, vp, vp, i64, i64, i64, vp, sz, ctypes.POINTER(OpsparseSpmvPlan),
                                                    vp]

@@ -111,14 +111,15 @@ aclsparseStatus_t EnsureWorkspace(aclsparseContext *h);
 OpsparseScalar MakeScalar(const void *p, aclDataType computeType, aclsparsePointerMode_t mode, double dflt);
 
 // The re-stored SpMV layout an ALG2 request gets for a plain fp32 CSR matrix: BLOCKED_GATHER where it
-// applies, else COLUMN_PANELS, else none (kernel 0, 0 bytes).  OPS_SPARSE_SPMV_NO_BLOCKED in the
+// applies, else (op(A) = A only) COLUMN_PANELS, else none (kernel 0, 0 bytes).  OPS_SPARSE_SPMV_NO_BLOCKED in the
 // environment skips the first (tuning, tests of the panel path).
 struct RestoredChoice {
     int32_t kernel;
     size_t bytes;
 };
-RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz);
+RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose);
 int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const float *values, int64_t rows,
-                    int64_t cols, int64_t nnz, void *buffer, size_t bytes, OpsparseSpmvPlan *plan, void *stream);
+                    int64_t cols, int64_t nnz, bool transpose, void *buffer, size_t bytes, OpsparseSpmvPlan *plan,
+                    void *stream);
 
 }  // namespace opsparse

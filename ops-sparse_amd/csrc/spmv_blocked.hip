@@ -97,6 +97,38 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedChunkKeysKernel(
     }
 }
 
+// op(A) = A^T, entries in CSR order: chunk key (row panel) * B + (block of the column), -1 and *status for a
+// column outside [0, cols).  outPtr[c] = number of entries in columns below c.
+__global__ __launch_bounds__(kBlockThreads) void BlockedTransposedKeysKernel(
+    const int32_t *__restrict__ colInd, const int32_t *__restrict__ rowOfPos, const int32_t *__restrict__ outPtr,
+    int64_t nnz, int64_t cols, int32_t numBlocks, int32_t window, int32_t *__restrict__ chunkKey,
+    int32_t *__restrict__ status)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
+        const int32_t col = colInd[i];
+        if (col < 0 || col >= cols) {
+            atomicOr(status, 1);
+            chunkKey[i] = -1;
+        } else {
+            chunkKey[i] = (rowOfPos[i] >> kPanelLog) * numBlocks + RowBlockOf(outPtr, col, window, numBlocks);
+        }
+    }
+}
+
+// op(A) = A^T, entries sorted by chunk key: local input index (row of A) and output index (column of A).
+__global__ __launch_bounds__(kBlockThreads) void BlockedTransposedFieldsKernel(
+    const int32_t *__restrict__ colInd, const int32_t *__restrict__ rowOfPos, const int32_t *__restrict__ pos,
+    int64_t nnz, uint16_t *__restrict__ colLocal, int32_t *__restrict__ rowOfSrc)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
+        const int32_t at = pos[i];
+        colLocal[i] = static_cast<uint16_t>(rowOfPos[at] & (kPanelCols - 1));
+        rowOfSrc[i] = colInd[at];
+    }
+}
+
 // From srcStart (first entry of chunk (panel, block) in panel order, P * B + 1 values):
 // dstStart[1 + block * P + panel] = size of the chunk, rounded up to a multiple of kLaneEntries (prefix-summed
 // afterwards: in block order every chunk starts on such a multiple, the gap behind it is padding), and
@@ -455,12 +487,13 @@ struct BlockedLayout {
     // used by every launch
     int64_t colLocalOff, xgOff, valOff, rowLocalOff, srcStartOff, dstStartOff, srcStartTOff, orderOff, blockRowOff;
     // preprocessing only
-    int64_t keys0Off, keys1Off, pos0Off, pos1Off, rowOfPosOff, tableOff, scratchOff;
+    int64_t keys0Off, keys1Off, pos0Off, pos1Off, rowOfPosOff, outPtrOff, tableOff, scratchOff;
     int64_t bytes;
 };
 
+// Layout for a product with `rows` outputs and `cols` inputs (op(A) = A^T: the columns of A are the outputs).
 // 0 panels: the layout does not apply.
-BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz)
+BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool transposed)
 {
     BlockedLayout l{};
     if (rows <= 0 || cols <= 0 || nnz <= 0 || nnz > INT32_MAX || rows >= INT32_MAX || cols > INT32_MAX) {
@@ -483,6 +516,14 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz)
         ++bits;
     }
     l.passes = (bits + 3) / 4;
+    if (transposed) {
+        // CSR order is ascending in the input index but not in the output block: sort on the whole chunk key
+        bits = 0;
+        while ((int64_t{1} << bits) < P * B) {
+            ++bits;
+        }
+        l.passes = (bits + 3) / 4;
+    }
     auto align = [](int64_t v) { return (v + 255) / 256 * 256; };
     int64_t off = 256;  // header: status word of the analysis
     const int64_t padded = nnz + kLaneEntries * P * B;  // every chunk padded to a multiple of kLaneEntries
@@ -501,9 +542,12 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz)
     l.pos0Off = off; off += align(4 * nnz);
     l.pos1Off = off; off += align(4 * nnz);
     l.rowOfPosOff = off; off += align(4 * nnz);
+    l.outPtrOff = off; off += transposed ? align(4 * (rows + 1)) : 0;  // entries per output (column of A), prefix-summed
     l.tableOff = off; off += align(4 * RadixTableInts(nnz));
-    const int64_t scanA = ScanScratchInts(RadixTableInts(nnz)), scanB = ScanScratchInts(P * B + 1);
-    l.scratchOff = off; off += align(4 * (scanA > scanB ? scanA : scanB));
+    int64_t scan = ScanScratchInts(RadixTableInts(nnz));
+    scan = ScanScratchInts(P * B + 1) > scan ? ScanScratchInts(P * B + 1) : scan;
+    scan = transposed && ScanScratchInts(rows + 1) > scan ? ScanScratchInts(rows + 1) : scan;
+    l.scratchOff = off; off += align(4 * scan);
     l.bytes = off;
     return l;
 }
@@ -519,7 +563,8 @@ uint32_t GridOf(int64_t items, int64_t perBlock, int64_t cap)
 
 int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
 {
-    const BlockedLayout l = MakeBlockedLayout(a.rows, a.cols, a.nnz);
+    // a.rows outputs, a.cols inputs: the caller has exchanged them for op(A) = A^T
+    const BlockedLayout l = MakeBlockedLayout(a.rows, a.cols, a.nnz, plan.transposed != 0);
     if (l.P == 0 || plan.numPanels != l.P || plan.numRowBlocks != l.B) {
         return OPSPARSE_E_INVALID;
     }
@@ -548,19 +593,22 @@ using namespace opsparse;
 
 extern "C" {
 
-size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz)
+size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t transpose)
 {
-    return static_cast<size_t>(MakeBlockedLayout(rows, cols, nnz).bytes);
+    return static_cast<size_t>(
+        (transpose ? MakeBlockedLayout(cols, rows, nnz, true) : MakeBlockedLayout(rows, cols, nnz, false)).bytes);
 }
 
 int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
-                                      int64_t rows, int64_t cols, int64_t nnz, void *workspace, size_t workspaceBytes,
-                                      OpsparseSpmvPlan *plan, void *stream)
+                                      int64_t rows, int64_t cols, int64_t nnz, int32_t transpose, void *workspace,
+                                      size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream)
 {
     if (plan == nullptr || rowOffsets == nullptr || colInd == nullptr || csrValues == nullptr) {
         return OPSPARSE_E_INVALID;
     }
-    const BlockedLayout l = MakeBlockedLayout(rows, cols, nnz);
+    const bool transposed = transpose != 0;
+    const int64_t outputs = transposed ? cols : rows;
+    const BlockedLayout l = transposed ? MakeBlockedLayout(cols, rows, nnz, true) : MakeBlockedLayout(rows, cols, nnz, false);
     if (l.P == 0) {
         return OPSPARSE_E_UNSUPPORTED;
     }
@@ -582,20 +630,45 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
 
     LaunchFillI32(status, 1, 0, s);
     LaunchExpandRows(rowOffsets, rows, nnz, 0, rowOfPos, s);
-    // Entries in (panel, original position) order: stable 4-bit radix passes over the panel number.
-    int cur = 0;
-    for (int32_t pass = 0; pass < l.passes; ++pass) {
-        const int32_t *keysIn = pass == 0 ? colInd : keys[cur];
-        const int32_t *posIn = pass == 0 ? nullptr : poss[cur];
-        const int out = pass == 0 ? 0 : 1 - cur;
-        LaunchRadixPass(keysIn, posIn, keys[out], poss[out], nnz, 0, kPanelLog + 4 * pass, table, scratch, s);
-        cur = out;
+    const int32_t *pos = nullptr, *outOffsets = rowOffsets;
+    int32_t *chunkKey = nullptr, *rowOfSrc = nullptr;
+    if (!transposed) {
+        // Entries in (panel, original position) order: stable 4-bit radix passes over the panel number.
+        int cur = 0;
+        for (int32_t pass = 0; pass < l.passes; ++pass) {
+            const int32_t *keysIn = pass == 0 ? colInd : keys[cur];
+            const int32_t *posIn = pass == 0 ? nullptr : poss[cur];
+            const int out = pass == 0 ? 0 : 1 - cur;
+            LaunchRadixPass(keysIn, posIn, keys[out], poss[out], nnz, 0, kPanelLog + 4 * pass, table, scratch, s);
+            cur = out;
+        }
+        pos = poss[cur];
+        chunkKey = keys[1 - cur];
+        rowOfSrc = poss[1 - cur];
+        hipLaunchKernelGGL(BlockedChunkKeysKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
+                           keys[cur], pos, rowOfPos, rowOffsets, nnz, cols, l.B, l.window, colLocal, chunkKey, rowOfSrc,
+                           status);
+    } else {
+        // The outputs are the columns of A: entries per column, then chunk keys in CSR order and a stable
+        // sort on the whole key.
+        int32_t *outPtr = ints(l.outPtrOff);
+        LaunchIndicesToOffsets(colInd, nnz, cols, 0, outPtr, scratch, s);
+        outOffsets = outPtr;
+        hipLaunchKernelGGL(BlockedTransposedKeysKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0,
+                           s, colInd, rowOfPos, outPtr, nnz, cols, l.B, l.window, keys[1], status);
+        int cur = 1;
+        for (int32_t pass = 0; pass < l.passes; ++pass) {
+            const int out = 1 - cur;
+            LaunchRadixPass(keys[cur], pass == 0 ? nullptr : poss[cur], keys[out], poss[out], nnz, 0, 4 * pass, table,
+                            scratch, s);
+            cur = out;
+        }
+        pos = poss[cur];
+        chunkKey = keys[cur];
+        rowOfSrc = poss[1 - cur];
+        hipLaunchKernelGGL(BlockedTransposedFieldsKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads),
+                           0, s, colInd, rowOfPos, pos, nnz, colLocal, rowOfSrc);
     }
-    const int32_t *colSorted = keys[cur], *pos = poss[cur];
-    int32_t *chunkKey = keys[1 - cur], *rowOfSrc = poss[1 - cur];
-    hipLaunchKernelGGL(BlockedChunkKeysKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
-                       colSorted, pos, rowOfPos, rowOffsets, nnz, cols, l.B, l.window, colLocal, chunkKey, rowOfSrc,
-                       status);
     int32_t bad = 0;
     if (hipMemcpyAsync(&bad, status, sizeof(bad), hipMemcpyDeviceToHost, s) != hipSuccess ||
         hipStreamSynchronize(s) != hipSuccess) {
@@ -613,9 +686,9 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     // padding positions: local row kPadRow, value 0
     LaunchFillI32(reinterpret_cast<int32_t *>(rowLocal), (l.padded + 1) / 2, static_cast<int32_t>(kPadRow * 0x10001u), s);
     LaunchFillI32(reinterpret_cast<int32_t *>(valD), l.padded, 0, s);
-    LaunchFillI32(blockRow, l.B + 1, static_cast<int32_t>(rows), s);
-    hipLaunchKernelGGL(BlockedRowBlocksKernel, dim3(GridOf(rows, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
-                       rowOffsets, static_cast<int32_t>(rows), l.window, l.B, blockRow);
+    LaunchFillI32(blockRow, l.B + 1, static_cast<int32_t>(outputs), s);
+    hipLaunchKernelGGL(BlockedRowBlocksKernel, dim3(GridOf(outputs, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
+                       s, outOffsets, static_cast<int32_t>(outputs), l.window, l.B, blockRow);
     hipLaunchKernelGGL(BlockedScatterKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
                        pos, rowOfSrc, chunkKey, csrValues, srcStart, dstStart, blockRow, nnz, l.P, l.B, valD, rowLocal);
     if (l.B <= kRankedBlocks) {
@@ -641,6 +714,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     p.panelShift = kPanelLog;
     p.numRowBlocks = l.B;
     p.entryWindow = l.window;
+    p.transposed = transposed ? 1 : 0;
     p.rows = rows;
     p.nnz = nnz;
     p.bytes = l.bytes;

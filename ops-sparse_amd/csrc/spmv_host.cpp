@@ -106,11 +106,11 @@ using Restored = opsparse::RestoredChoice;
 Restored RestoredLayout(aclsparseOperation_t opA, aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX,
                         aclsparseConstDnVecDescr_t vecY, aclDataType computeType, aclsparseSpMVAlg_t alg)
 {
-    if (alg != ACL_SPARSE_SPMV_CSR_ALG2 || opA != ACL_SPARSE_OP_NON_TRANSPOSE || computeType != ACL_FLOAT ||
-        matA->valueType != ACL_FLOAT || vecX->valueType != ACL_FLOAT || vecY->valueType != ACL_FLOAT) {
+    if (alg != ACL_SPARSE_SPMV_CSR_ALG2 || computeType != ACL_FLOAT || matA->valueType != ACL_FLOAT ||
+        vecX->valueType != ACL_FLOAT || vecY->valueType != ACL_FLOAT) {
         return {0, 0};
     }
-    return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz);
+    return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz, opA != ACL_SPARSE_OP_NON_TRANSPOSE);
 }
 
 aclsparseStatus_t FromLaunch(int rc)
@@ -128,15 +128,15 @@ aclsparseStatus_t FromLaunch(int rc)
 
 namespace opsparse {
 
-RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz)
+RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose)
 {
     if (std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") == nullptr) {
-        const size_t blocked = opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz);
+        const size_t blocked = opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, transpose ? 1 : 0);
         if (blocked > 0) {
             return {OPSPARSE_SPMV_BLOCKED_GATHER, blocked};
         }
     }
-    const size_t panels = opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz);
+    const size_t panels = transpose ? 0 : opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz);
     if (panels > 0) {
         return {OPSPARSE_SPMV_COLUMN_PANELS, panels};
     }
@@ -144,11 +144,12 @@ RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz)
 }
 
 int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const float *values, int64_t rows,
-                    int64_t cols, int64_t nnz, void *buffer, size_t bytes, OpsparseSpmvPlan *plan, void *stream)
+                    int64_t cols, int64_t nnz, bool transpose, void *buffer, size_t bytes, OpsparseSpmvPlan *plan,
+                    void *stream)
 {
     if (kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {
-        return opsparse_spmv_csr_blocked_analyse(rowOffsets, colInd, values, rows, cols, nnz, buffer, bytes, plan,
-                                                 stream);
+        return opsparse_spmv_csr_blocked_analyse(rowOffsets, colInd, values, rows, cols, nnz, transpose ? 1 : 0, buffer,
+                                                 bytes, plan, stream);
     }
     return opsparse_spmv_csr_panels_analyse(rowOffsets, colInd, values, rows, cols, nnz, buffer, bytes, plan, stream);
 }
@@ -203,7 +204,8 @@ aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOpe
         rc = opsparse::AnalyseRestored(restored.kernel, static_cast<const int32_t *>(matA->rowOffsets),
                                        static_cast<const int32_t *>(matA->colInd),
                                        static_cast<const float *>(matA->values), matA->rows, matA->cols, matA->nnz,
-                                       externalBuffer, restored.bytes, &plan, handle->stream);
+                                       opA != ACL_SPARSE_OP_NON_TRANSPOSE, externalBuffer, restored.bytes, &plan,
+                                       handle->stream);
     } else {
         const size_t bytes = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
         rc = opsparse_spmv_csr_analyse(static_cast<const int32_t *>(matA->rowOffsets), matA->rows, matA->cols,
@@ -244,14 +246,25 @@ aclsparseStatus_t aclsparseSpMV(aclsparseHandle_t handle, aclsparseOperation_t o
     const OpsparseSpmvPlan *plan = nullptr;
     void *ws = nullptr;
     size_t wsBytes = 0;
-    if (!c.transpose && externalBuffer != nullptr && matA->spmv.buffer == externalBuffer &&
-        matA->spmv.plan.rows == matA->rows && matA->spmv.plan.nnz == matA->nnz) {
+    const bool bound = externalBuffer != nullptr && matA->spmv.buffer == externalBuffer &&
+                       matA->spmv.plan.rows == matA->rows && matA->spmv.plan.nnz == matA->nnz;
+    const bool blockedPlan = bound && matA->spmv.plan.kernel == OPSPARSE_SPMV_BLOCKED_GATHER;
+    if (blockedPlan && (matA->spmv.plan.transposed != 0) != c.transpose) {
+        // Preprocess built the re-stored layout for the other op(A): this call runs without it
+        if (matA->nnz > 0 || (c.transpose && c.outType != OPSPARSE_F32)) {
+            st = opsparse::EnsureWorkspace(handle);
+            if (st != ACL_SPARSE_STATUS_SUCCESS) {
+                return st;
+            }
+            ws = handle->workspace();
+            wsBytes = handle->workspaceBytes();
+        }
+    } else if (bound && (!c.transpose || blockedPlan)) {
         plan = &matA->spmv.plan;
         ws = externalBuffer;
         wsBytes = static_cast<size_t>(plan->bytes);
     } else if (matA->nnz > 0 || (c.transpose && c.outType != OPSPARSE_F32)) {
-        if (c.transpose && externalBuffer != nullptr && matA->spmv.buffer == externalBuffer &&
-            matA->spmv.plan.rows == matA->rows && matA->spmv.plan.nnz == matA->nnz) {
+        if (c.transpose && bound) {
             plan = &matA->spmv.plan;  // op(A) = A^T only takes the row-length statistics from it
         }
         // the merge-path partition of an unprepared call, or the fp32 staging vector of a transposed

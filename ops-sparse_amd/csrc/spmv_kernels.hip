@@ -1453,6 +1453,18 @@ int opsparse_spmv_csr_launch_zy(const OpsparseSpmvPlan *plan, int32_t transpose,
     SpmvArgs a{rowOffsets, colInd, csrValues, x,         y,     yIn, rows, cols, nnz, alpha, beta,
                workspace,  workspaceBytes, static_cast<hipStream_t>(stream)};
 
+    if (plan != nullptr && plan->kernel == OPSPARSE_SPMV_BLOCKED_GATHER && (plan->transposed != 0) != (transpose != 0)) {
+        return OPSPARSE_E_INVALID;  // the re-stored layout serves the op(A) it was built for
+    }
+    if (transpose && plan != nullptr && plan->kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {
+        if (computeIsInt || valType != OPSPARSE_F32 || outType != OPSPARSE_F32) {
+            return OPSPARSE_E_UNSUPPORTED;
+        }
+        SpmvArgs t = a;  // the columns of A are the outputs, its rows the inputs
+        t.rows = cols;
+        t.cols = rows;
+        return LaunchBlockedF32(t, *plan);
+    }
     if (transpose) {
         if (computeIsInt) {
             return OPSPARSE_E_UNSUPPORTED;

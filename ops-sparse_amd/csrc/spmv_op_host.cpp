@@ -86,7 +86,7 @@ opsparse::RestoredChoice RestoredLayout(aclsparseConstSpMatDescr_t matA)
     if (matA->rowOffsetsType != ACL_SPARSE_INDEX_32I || matA->idxBase != ACL_SPARSE_INDEX_BASE_ZERO) {
         return {0, 0};
     }
-    return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz);
+    return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz, false);
 }
 
 aclsparseStatus_t FromLaunch(int rc)
@@ -192,8 +192,8 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
                 restored.kernel != 0 && d->colInd != nullptr && d->values != nullptr
                     ? opsparse::AnalyseRestored(restored.kernel, static_cast<const int32_t *>(d->rowOffsets),
                                                 static_cast<const int32_t *>(d->colInd),
-                                                static_cast<const float *>(d->values), d->rows, d->cols, d->nnz, buffer,
-                                                restored.bytes, &d->plan, handle->stream)
+                                                static_cast<const float *>(d->values), d->rows, d->cols, d->nnz, false,
+                                                buffer, restored.bytes, &d->plan, handle->stream)
                     : opsparse_spmv_csr_analyse(static_cast<const int32_t *>(d->rowOffsets), d->rows, d->cols, d->nnz,
                                                 buffer, opsparse_spmv_csr_workspace_bytes(d->rows, d->nnz),
                                                 OPSPARSE_SPMV_AUTO, &d->plan, handle->stream);

@@ -68,7 +68,7 @@ def test_c3_power_law_full(osa, workloads, gpu_ctx, monkeypatch):
     y2 = _spmv(osa, gpu_ctx, cfg, preprocess=False)
     assert oracle.max_rel_err(y2.cpu().numpy(), gold) <= 1e-5
     # CSR_ALG2: the blocked-gather layout (256 panels of 2^15 columns, about a thousand row blocks) ...
-    assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(A["rows"], A["cols"], colind.size) > 0
+    assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(A["rows"], A["cols"], colind.size, 0) > 0
     y5 = _spmv(osa, gpu_ctx, cfg, alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
     assert oracle.max_rel_err(y5.cpu().numpy(), gold) <= 1e-5
     # ... and, with that one switched off, the column-panel layout (eight panels of 2^20 columns)

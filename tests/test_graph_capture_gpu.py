@@ -50,7 +50,7 @@ def test_spmv_replays(osa, gpu_ctx, kind):
         rows, cols = 30_000, 1_300_000
         rowptr, colind, val = _power_law(rows, cols, 3, 60_000)
         alg = osa.ACL_SPARSE_SPMV_CSR_ALG2
-        assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size) > 0
+        assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 0) > 0
     rng = np.random.default_rng(7)
     y0 = rng.uniform(-1, 1, rows).astype(np.float32)
     d = [to_dev(a, dev) for a in (rowptr, colind, val)]

@@ -250,7 +250,7 @@ def test_blocked_gather_csr_alg2(osa, gpu_ctx, rows, cols, applies):
     rowptr, colind, val, x, y0 = _wide_problem(rows, cols, cols % 1000 + rows,
                                                long_rows=((7, 90_000), (rows // 2, 1), (rows - 1, 30_000)))
     L = osa.lib()
-    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size)
+    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 0)
     assert (need > 0) == applies
     d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
     A = osa.Csr(rows, cols, d[0], d[1], d[2])
@@ -280,7 +280,7 @@ def test_blocked_gather_hot_rows_and_unaligned_x(osa, gpu_ctx):
     val = rng.uniform(-1, 1, colind.size).astype(np.float32)
     x = rng.uniform(-1, 1, cols).astype(np.float32)
     y0 = rng.uniform(-1, 1, rows).astype(np.float32)
-    assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size) > 0
+    assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 0) > 0
     d = [to_dev(a, dev) for a in (rowptr, colind, val)]
     xbuf = torch.zeros(cols + 1, dtype=torch.float32, device=dev)
     xbuf[1:].copy_(torch.from_numpy(x))
@@ -301,7 +301,7 @@ def test_blocked_gather_giant_row_and_device_scalars(osa, gpu_ctx):
     dev, stream, handle = gpu_ctx
     rows, cols = 20_000, 2_200_000
     rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 3, long_rows=((11_111, 1_000_000), (11_112, 70_000)))
-    assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size) > 0
+    assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 0) > 0
     d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
     A, X = osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3])
     d_y = to_dev(y0, dev)
@@ -327,6 +327,50 @@ def test_blocked_gather_giant_row_and_device_scalars(osa, gpu_ctx):
     assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
 
 
+@pytest.mark.parametrize("rows,cols", [(1_400_000, 50_000), (2_000_000, 2_000_000), (1_100_000, 300)])
+def test_blocked_gather_transposed(osa, gpu_ctx, rows, cols):
+    """ACL_SPARSE_SPMV_CSR_ALG2 with op(A) = A^T and more than 2^20 rows: the layout is built over the rows of A
+    (panels, x) and its columns (row blocks, y), and the product has no atomics on y: the 1e-5 bar of op(A) = A,
+    not the reference's loose rule for its atomic transpose path.  A plan built for A^T does not serve A: the
+    same descriptor and buffer then run op(A) = A through the ordinary kernels."""
+    dev, stream, handle = gpu_ctx
+    rng = np.random.default_rng(rows % 1000 + cols)
+    lengths = rng.integers(0, 4, rows)
+    lengths[[5, rows // 3]] = [min(cols, 40_000), min(cols, 9_000)]
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)     # unsorted, repeated columns
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    x = rng.uniform(-1, 1, rows).astype(np.float32)
+    y0 = rng.uniform(-1, 1, cols).astype(np.float32)
+    L = osa.lib()
+    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 1)
+    assert need > 0
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    A = osa.Csr(rows, cols, d[0], d[1], d[2])
+    d_y = to_dev(y0, dev)
+    op = osa.SpmvOp(handle, A, osa.DnVec(d[3]), osa.DnVec(d_y), op=osa.ACL_SPARSE_OP_TRANSPOSE,
+                    alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
+    assert op.buffer.numel() >= need
+    for alpha, beta in ((1.0, 0.0), (-1.5, 0.5)):
+        d_y.copy_(torch.from_numpy(y0))
+        op(alpha, beta)
+        stream.synchronize()
+        gold = oracle.spmv_trans_f64(rows, cols, rowptr, colind, val, x, y0, alpha, beta)
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+    # the same buffer handed to an op(A) = A call: ignored, result still right
+    xn = rng.uniform(-1, 1, cols).astype(np.float32)
+    yn0 = rng.uniform(-1, 1, rows).astype(np.float32)
+    d_xn, d_yn = to_dev(xn, dev), to_dev(yn0, dev)
+    Xn, Yn = osa.DnVec(d_xn), osa.DnVec(d_yn)
+    one, half = ctypes.c_float(1.0), ctypes.c_float(0.5)
+    rc = L.aclsparseSpMV(handle.h, 0, ctypes.byref(one), A.d, Xn.d, ctypes.byref(half), Yn.d, osa.ACL_FLOAT,
+                         osa.ACL_SPARSE_SPMV_CSR_ALG2, ctypes.c_void_p(op.buffer.data_ptr()))
+    assert rc == 0
+    stream.synchronize()
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, xn, yn0, 1.0, 0.5)
+    assert oracle.max_rel_err(d_yn.cpu().numpy(), gold) <= 1e-5
+
+
 def test_blocked_gather_through_spmvop_alg2(osa, gpu_ctx):
     """aclsparseSpMVOp ALG2 on a wide matrix uses the blocked-gather layout; Z separate from Y and aliased."""
     dev, stream, handle = gpu_ctx
@@ -340,7 +384,7 @@ def test_blocked_gather_through_spmvop_alg2(osa, gpu_ctx):
         Y = osa.DnVec(d_y)
         Z = Y if alias else osa.DnVec(d_z)
         op = osa.SpmvOpPlan(handle, A, osa.DnVec(d[3]), Y, Z, alg=osa.ACL_SPARSE_SPMVOP_ALG2)
-        assert op.buffer_bytes == osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size) > 0
+        assert op.buffer_bytes == osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 0) > 0
         op(1.25, -0.5)
         stream.synchronize()
         gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.25, -0.5)
@@ -357,14 +401,14 @@ def test_blocked_gather_rejects_column_out_of_range(osa, gpu_ctx):
     colind = colind.copy()
     colind[colind.size // 2] = cols + 5
     L = osa.lib()
-    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size)
+    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 0)
     assert need > 0
     d = [to_dev(a, dev) for a in (rowptr, colind, val)]
     ws = torch.empty(need, dtype=torch.uint8, device=dev)
     plan = osa.OpsparseSpmvPlan()
     torch.cuda.synchronize()
     p = lambda t: ctypes.c_void_p(t.data_ptr())
-    rc = L.opsparse_spmv_csr_blocked_analyse(p(d[0]), p(d[1]), p(d[2]), rows, cols, colind.size, p(ws), need,
+    rc = L.opsparse_spmv_csr_blocked_analyse(p(d[0]), p(d[1]), p(d[2]), rows, cols, colind.size, 0, p(ws), need,
                                              ctypes.byref(plan), ctypes.c_void_p(stream.cuda_stream))
     assert rc == osa.OPSPARSE_E_INVALID
     d_x, d_y = to_dev(x, dev), to_dev(y0, dev)
