@@ -294,6 +294,43 @@ def test_raw_layer_argument_checks(osa, L):
     assert L.opsparse_copy_launch(FAKE, FAKE, 17, None) == -1 and L.opsparse_copy_launch(FAKE, FAKE, 0, None) == 0
 
 
+def test_restored_layout_applicability(osa, L, handle):
+    """When ACL_SPARSE_SPMV_CSR_ALG2 gets a re-stored layout, decided on the host from the sizes alone: blocked
+    gather needs an x of more than 2^20 and at most 2^25 elements and 32 entries per (panel, row block) chunk;
+    column panels (op(A) = A only) need 2 .. 16 panels of 2^20 columns.  GetBufferSize reports the larger of
+    that layout and the ordinary buffer, and the ordinary one for anything else."""
+    blocked, panels = L.opsparse_spmv_csr_blocked_workspace_bytes, L.opsparse_spmv_csr_panels_workspace_bytes
+    m = 1 << 23
+    assert blocked(m, m, 8 * m, 0) > 12 * 8 * m and blocked(m, m, 8 * m, 1) > blocked(m, m, 8 * m, 0)
+    assert blocked(m, 1 << 20, 8 * m, 0) == 0 and blocked(m, (1 << 20) + 1, 8 * m, 0) > 0     # x must exceed an L2
+    assert blocked(m, (1 << 25) + 1, 64 * m, 0) == 0                                         # too many panels
+    assert blocked(m, m, m // 64, 0) == 0                                                    # chunks too short
+    assert blocked(1 << 20, m, 8 * m, 1) == 0 and blocked(m, 1000, 8 * m, 1) > 0             # op(A) = A^T: x has m rows
+    assert blocked(0, m, 0, 0) == 0 and blocked(m, m, (1 << 31), 0) == 0
+    assert panels(m, m, 8 * m) > 0 and panels(m, 1 << 20, 8 * m) == 0 and panels(m, (1 << 24) + 1, 8 * m) == 0
+    n = ctypes.c_size_t(0)
+    A, X, Y = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+    assert L.aclsparseCreateCsr(ctypes.byref(A), m, m, 8 * m, FAKE, FAKE, FAKE, 0, 0, 0, osa.ACL_FLOAT) == 0
+    assert L.aclsparseCreateDnVec(ctypes.byref(X), m, FAKE, osa.ACL_FLOAT) == 0
+    assert L.aclsparseCreateDnVec(ctypes.byref(Y), m, FAKE, osa.ACL_FLOAT) == 0
+    plain = L.opsparse_spmv_csr_workspace_bytes(m, 8 * m)
+    for op, alg, want in ((0, osa.ACL_SPARSE_SPMV_CSR_ALG2, blocked(m, m, 8 * m, 0)),
+                          (1, osa.ACL_SPARSE_SPMV_CSR_ALG2, blocked(m, m, 8 * m, 1)),
+                          (0, osa.ACL_SPARSE_SPMV_ALG_DEFAULT, plain)):
+        assert L.aclsparseSpMVGetBufferSize(handle, op, None, A, X, None, Y, osa.ACL_FLOAT, alg, ctypes.byref(n)) == 0
+        assert n.value == max(want, plain)
+    os.environ["OPS_SPARSE_SPMV_NO_BLOCKED"] = "1"
+    try:
+        assert L.aclsparseSpMVGetBufferSize(handle, 0, None, A, X, None, Y, osa.ACL_FLOAT,
+                                            osa.ACL_SPARSE_SPMV_CSR_ALG2, ctypes.byref(n)) == 0
+        assert n.value == max(panels(m, m, 8 * m), plain)
+    finally:
+        del os.environ["OPS_SPARSE_SPMV_NO_BLOCKED"]
+    for d in (X, Y):
+        assert L.aclsparseDestroyDnVec(d) == 0
+    assert L.aclsparseDestroySpMat(A) == 0
+
+
 # ------------------------------------------------------------------- SpMVOp
 
 def test_spmvop_status_table(osa, L, handle):
