@@ -116,13 +116,23 @@ def cpu_baseline_spmv(cfg, y_gpu, budget_s=15.0):
         oracle.spmv_f32(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])
         reps += 1
     dt = (time.perf_counter() - t0) / reps
+    # the same loop with its rows shared out among all host threads (second baseline, reported beside the first)
+    threads = oracle.host_threads()
+    oracle.spmv_f32_threads(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"], threads)
+    t0 = time.perf_counter()
+    for _ in range(5):
+        oracle.spmv_f32_threads(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"], threads)
+    dt_all = (time.perf_counter() - t0) / 5
     return {"value": 2.0 * nnz / dt / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
             "sample": "full matrix, %d repeats of the reference's SpmvCpu loop restated in oracle/oracle.c "
                       "(fp32 accumulate), %.1f ms each" % (reps, dt * 1e3),
+            "all_cores": {"value": 2.0 * nnz / dt_all / 1e9, "unit": "GFLOP/s", "cores": threads,
+                          "sample": "the same loop, rows shared out among %d OpenMP threads, %.1f ms each"
+                                    % (threads, dt_all * 1e3)},
             "gpu_vs_fp64_oracle_max_rel_err": err}
 
 
-def cpu_baseline_spmm(cfg, c_gpu, rows_sample=32768):
+def cpu_baseline_spmm(cfg, c_gpu, rows_sample=262144):
     """The reference's spmm_csr_cpu loop (order i, j, p) on the first rows_sample rows; the same rows of the GPU
     result of one launch (c_gpu) are checked against the fp64-accumulated oracle on the way."""
     import oracle
@@ -145,9 +155,16 @@ def cpu_baseline_spmm(cfg, c_gpu, rows_sample=32768):
     tol = 1e-5 if A["values"].element_size() == 4 else 1e-3
     if err > tol:
         sys.exit("bench.py: the GPU result differs from the fp64 oracle (max relative error %.3g > %g)" % (err, tol))
+    threads = oracle.host_threads()
+    t0 = time.perf_counter()
+    oracle.spmm_f32_threads(rs, n, rowptr, colind, val, B.ravel(), n, C, n, cfg["alpha"], cfg["beta"], threads)
+    dt_all = time.perf_counter() - t0
     return {"value": 2.0 * nnz * n / dt / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
             "sample": "first %d of %d rows (%d nnz) against the full B, one run of the reference's "
                       "SpmmCpuFp32 loop restated in oracle/oracle.c, %.1f s" % (rs, A["rows"], nnz, dt),
+            "all_cores": {"value": 2.0 * nnz * n / dt_all / 1e9, "unit": "GFLOP/s", "cores": threads,
+                          "sample": "the same rows and loop shared out among %d OpenMP threads, %.2f s"
+                                    % (threads, dt_all)},
             "gpu_vs_fp64_oracle_max_rel_err": err}
 
 

@@ -90,6 +90,16 @@ def spmv_f32(rows, rowptr, colind, val, x, y, alpha, beta):
     return z
 
 
+def spmv_f32_threads(rows, rowptr, colind, val, x, y, alpha, beta, threads):
+    """spmv_f32 with the rows shared out among `threads` OpenMP threads (identical results)."""
+    rowptr, colind = _c(rowptr, np.int32), _c(colind, np.int32)
+    val, x, y = _c(val, np.float32), _c(x, np.float32), _c(y, np.float32)
+    z = np.empty(rows, np.float32)
+    lib().oracle_spmv_f32_threads(c_i64(rows), _p(rowptr), _p(colind), _p(val), _p(x), _p(y), c_f32(alpha),
+                                  c_f32(beta), _p(z), ctypes.c_int(threads))
+    return z
+
+
 def spmv_trans_f32(rows, cols, rowptr, colind, val, x, y, alpha, beta):
     rowptr, colind = _c(rowptr, np.int32), _c(colind, np.int32)
     val, x, y = _c(val, np.float32), _c(x, np.float32), _c(y, np.float32)
@@ -136,6 +146,22 @@ def spmm_f32(m, n, rowptr, colind, val, B, ldb, C, ldc, alpha, beta, b_row_major
     are flat buffers in their storage layout; a copy of C is returned."""
     return _spmm(lib().oracle_spmm_f32, m, n, rowptr, colind, val, B, ldb, b_row_major, trans_b, C, ldc,
                  c_row_major, alpha, beta)
+
+
+def spmm_f32_threads(m, n, rowptr, colind, val, B, ldb, C, ldc, alpha, beta, threads, b_row_major=True,
+                     trans_b=False, c_row_major=True):
+    """spmm_f32 with the rows shared out among `threads` OpenMP threads (identical results)."""
+    fn = lib().oracle_spmm_f32_threads
+    return _spmm(lambda *a: fn(*a, ctypes.c_int(threads)), m, n, rowptr, colind, val, B, ldb, b_row_major, trans_b,
+                 C, ldc, c_row_major, alpha, beta)
+
+
+def host_threads():
+    """Threads the all-cores CPU baseline uses: OMP_NUM_THREADS when set, else the CPUs this process may run on."""
+    env = os.environ.get("OMP_NUM_THREADS", "")
+    if env.isdigit() and int(env) > 0:
+        return int(env)
+    return len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
 
 
 def spmm_f64(m, n, rowptr, colind, val, B, ldb, C, ldc, alpha, beta, b_row_major=True, trans_b=False,

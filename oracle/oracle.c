@@ -72,6 +72,21 @@ void oracle_spmv_f32(int64_t rows, const int32_t *rowptr, const int32_t *colind,
     }
 }
 
+/* The same loop with its rows shared out among `threads` OpenMP threads (rows are independent: the results
+ * are those of oracle_spmv_f32 bit for bit).  The all-cores CPU baseline of the benchmark. */
+void oracle_spmv_f32_threads(int64_t rows, const int32_t *rowptr, const int32_t *colind, const float *val,
+                             const float *x, const float *y, float alpha, float beta, float *z, int threads)
+{
+#pragma omp parallel for schedule(static, 4096) num_threads(threads)
+    for (int64_t i = 0; i < rows; ++i) {
+        float sum = 0.0f;
+        for (int32_t p = rowptr[i]; p < rowptr[i + 1]; ++p) {
+            sum += val[p] * x[colind[p]];
+        }
+        z[i] = alpha * sum + beta * y[i];
+    }
+}
+
 /*
  * Transposed fp32 golden: z = beta * y, then z[col] += (alpha * x[row]) * val
  * row by row.  SpmvTransCpu, test/spmv/arch22/spmv_test.cpp:177-197.
@@ -157,6 +172,24 @@ void oracle_spmm_f32(int64_t m, int64_t n, const int32_t *rowptr, const int32_t 
                      const float *B, int64_t ldb, int b_row_major, int trans_b, float *C, int64_t ldc,
                      int c_row_major, float alpha, float beta)
 {
+    for (int64_t r = 0; r < m; ++r) {
+        for (int64_t j = 0; j < n; ++j) {
+            float acc = 0.0f;
+            for (int32_t p = rowptr[r]; p < rowptr[r + 1]; ++p) {
+                acc += val[p] * B[b_index(colind[p], j, ldb, b_row_major, trans_b)];
+            }
+            const int64_t ci = c_index(r, j, ldc, c_row_major);
+            C[ci] = alpha * acc + beta * C[ci];
+        }
+    }
+}
+
+/* oracle_spmm_f32 with its rows shared out among `threads` OpenMP threads (same results bit for bit). */
+void oracle_spmm_f32_threads(int64_t m, int64_t n, const int32_t *rowptr, const int32_t *colind, const float *val,
+                             const float *B, int64_t ldb, int b_row_major, int trans_b, float *C, int64_t ldc,
+                             int c_row_major, float alpha, float beta, int threads)
+{
+#pragma omp parallel for schedule(dynamic, 64) num_threads(threads)
     for (int64_t r = 0; r < m; ++r) {
         for (int64_t j = 0; j < n; ++j) {
             float acc = 0.0f;

@@ -99,6 +99,24 @@ def test_spmv_f32_golden_close_to_f64_oracle():
     assert not np.array_equal(g32, g64)  # they are different computations
 
 
+def test_threaded_goldens_equal_the_single_thread_loops():
+    """The all-cores CPU baselines of the benchmark are the reference loops with rows shared out among threads:
+    bit-identical to the single-thread loops, whatever the number of threads."""
+    rows, cols, n = 3000, 700, 9
+    rowptr, colind, val = random_csr(rows, cols, 0.02, 5, empty_row_prob=0.1)
+    rng = np.random.default_rng(6)
+    x, y = rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+    B = rng.uniform(-1, 1, (cols, n)).astype(np.float32)
+    C = rng.uniform(-1, 1, (rows, n)).astype(np.float32)
+    one = oracle.spmv_f32(rows, rowptr, colind, val, x, y, 1.5, -0.5)
+    mm = oracle.spmm_f32(rows, n, rowptr, colind, val, B.ravel(), n, C.ravel(), n, 1.5, -0.5)
+    for threads in (1, 3, 8):
+        assert np.array_equal(oracle.spmv_f32_threads(rows, rowptr, colind, val, x, y, 1.5, -0.5, threads), one)
+        assert np.array_equal(oracle.spmm_f32_threads(rows, n, rowptr, colind, val, B.ravel(), n, C.ravel(), n, 1.5,
+                                                      -0.5, threads), mm)
+    assert oracle.host_threads() >= 1
+
+
 def test_spmv_int32_wraps():
     rowptr = np.array([0, 2, 3], np.int32)
     colind = np.array([0, 1, 1], np.int32)
