@@ -134,8 +134,8 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
 
 /*
  * BLOCKED_GATHER analysis (fp32): bytes of the workspace, or 0 when the family does
- * not apply (x must have more than 2^20 and at most 2^25 elements, and a (panel, row
- * block) chunk at least 32 entries on average).  transpose != 0 builds the layout of
+ * not apply (x must have more than 2^20 and at most 2^25 elements, the matrix at least
+ * two million entries, and a (panel, row block) chunk at least 32 entries on average).  transpose != 0 builds the layout of
  * y = alpha * A^T * x + beta * y instead: panels over the rows of A, blocks over its
  * columns, with no atomics on y; a plan serves the op(A) it was built for.  Like the panel
  * analysis it re-stores indices AND values in the workspace; launches with the

@@ -58,6 +58,8 @@ constexpr int kLaneEntries = 8;                   // consecutive entries a lane 
 constexpr uint32_t kPadRow = 0x8000;              // local row of a padding position in block order
 constexpr int32_t kRankedBlocks = 8192;           // up to here the block order is found by counting ranks
 constexpr int64_t kMinEntryWindow = 16384;
+constexpr int64_t kMinEntryBlocks = 512;          // entry windows a matrix is cut into at least (if it has the entries)
+constexpr int64_t kMinEntries = 2000000;          // below this the ordinary kernels are as fast or faster
 constexpr int64_t kMinChunkEntries = 32;          // below this mean chunk size the layout does not pay
 
 typedef float Float4 __attribute__((ext_vector_type(4)));
@@ -500,12 +502,14 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
         return l;
     }
     const int64_t P = (cols + kPanelCols - 1) >> kPanelLog;
+    // Entry window: blocks of short rows get about nnz / (full row blocks) entries; a matrix of few, long rows is
+    // still cut into kMinEntryBlocks pieces, or phase 2 would run on a handful of workgroups.
     const int64_t fullBlocks = rows >> kRowBlockLog;
-    int64_t window = nnz / (fullBlocks > 0 ? fullBlocks : 1);
+    int64_t window = nnz / (fullBlocks > kMinEntryBlocks ? fullBlocks : kMinEntryBlocks);
     window = window < kMinEntryWindow ? kMinEntryWindow : window;
     const int64_t B = ((rows + kRowBlockRows - 1) >> kRowBlockLog) + nnz / window + 1;
     // x must be larger than an L2 (2^20 columns) for the two passes to pay, and the chunks long enough to stream.
-    if (cols <= (int64_t{1} << 20) || P > kMaxPanels || P * B + 1 > INT32_MAX || nnz + kLaneEntries * P * B > INT32_MAX || nnz / (P * B) < kMinChunkEntries) {
+    if (cols <= (int64_t{1} << 20) || nnz < kMinEntries || P > kMaxPanels || P * B + 1 > INT32_MAX || nnz + kLaneEntries * P * B > INT32_MAX || nnz / (P * B) < kMinChunkEntries) {
         return l;
     }
     l.P = static_cast<int32_t>(P);

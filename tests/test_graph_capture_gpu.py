@@ -29,9 +29,9 @@ def _capture(stream, launch):
     return graph
 
 
-def _power_law(rows, cols, seed, longest):
+def _power_law(rows, cols, seed, longest, at_least=1):
     rng = np.random.default_rng(seed)
-    lengths = np.minimum((rng.pareto(1.2, rows) + 1).astype(np.int64), longest)
+    lengths = np.minimum((rng.pareto(1.2, rows) + at_least).astype(np.int64), longest)
     lengths[rng.integers(0, rows, 3)] = longest
     return csr_from_lengths(lengths, cols, seed + 1)
 
@@ -48,7 +48,7 @@ def test_spmv_replays(osa, gpu_ctx, kind):
         rowptr, colind, val = _power_law(rows, cols, 2, 9_000)
     else:
         rows, cols = 30_000, 1_300_000
-        rowptr, colind, val = _power_law(rows, cols, 3, 60_000)
+        rowptr, colind, val = _power_law(rows, cols, 3, 60_000, at_least=80)
         alg = osa.ACL_SPARSE_SPMV_CSR_ALG2
         assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 0) > 0
     rng = np.random.default_rng(7)

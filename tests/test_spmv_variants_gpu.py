@@ -175,9 +175,9 @@ def test_preprocessed_buffer_reused_and_rebound(osa, gpu_ctx):
     assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
 
 
-def _wide_problem(rows, cols, seed, long_rows=()):
+def _wide_problem(rows, cols, seed, long_rows=(), per_row=12):
     rng = np.random.default_rng(seed)
-    lengths = rng.integers(0, 12, rows)
+    lengths = rng.integers(0, per_row, rows)
     for r, l in long_rows:
         lengths[r] = l
     rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
@@ -239,7 +239,8 @@ def test_column_panels_through_spmvop_alg2(osa, gpu_ctx, monkeypatch):
 
 
 @pytest.mark.parametrize("rows,cols,applies", [(60_000, 3_000_000, True), (60_000, 1_048_577, True),
-                                               (20_000, 17_000_000, True), (60_000, 1_000_000, False),
+                                               (60_000, 9_000_000, True), (60_000, 1_000_000, False),
+                                               (20_000, 17_000_000, False),     # 519 panels: chunks of < 32 entries
                                                (300_000, 2_000_000, True)])
 def test_blocked_gather_csr_alg2(osa, gpu_ctx, rows, cols, applies):
     """ACL_SPARSE_SPMV_CSR_ALG2 on a matrix whose x is wider than an L2: Preprocess re-stores the entries by
@@ -247,8 +248,9 @@ def test_blocked_gather_csr_alg2(osa, gpu_ctx, rows, cols, applies):
     second.  Products are exact in fp64 and rounded once: the 1e-5 bar of every other family.  Rows longer than a
     row block's entry window, empty rows and a last partial panel / row block are all in."""
     dev, stream, handle = gpu_ctx
-    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, cols % 1000 + rows,
+    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, cols % 1000 + rows, per_row=max(12, 4_800_000 // rows),
                                                long_rows=((7, 90_000), (rows // 2, 1), (rows - 1, 30_000)))
+    assert colind.size > 2_000_000      # smaller matrices keep the ordinary kernels
     L = osa.lib()
     need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 0)
     assert (need > 0) == applies
@@ -273,7 +275,7 @@ def test_blocked_gather_hot_rows_and_unaligned_x(osa, gpu_ctx):
     rows, cols = 50_000, 1_500_000
     rng = np.random.default_rng(11)
     lengths = rng.integers(0, 3, rows)
-    hot = rng.choice(rows, 40, replace=False)
+    hot = rng.choice(rows, 90, replace=False)
     lengths[hot] = rng.integers(2_000, 60_000, hot.size)
     rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
     colind = np.concatenate([np.sort(rng.choice(cols, int(l), replace=False)) for l in lengths]).astype(np.int32)
@@ -300,7 +302,8 @@ def test_blocked_gather_giant_row_and_device_scalars(osa, gpu_ctx):
     covers, and whole wavefronts of a single row — and alpha / beta read from device memory."""
     dev, stream, handle = gpu_ctx
     rows, cols = 20_000, 2_200_000
-    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 3, long_rows=((11_111, 1_000_000), (11_112, 70_000)))
+    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 3, per_row=120,
+                                               long_rows=((11_111, 1_000_000), (11_112, 70_000)))
     assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 0) > 0
     d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
     A, X = osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3])
@@ -335,7 +338,7 @@ def test_blocked_gather_transposed(osa, gpu_ctx, rows, cols):
     same descriptor and buffer then run op(A) = A through the ordinary kernels."""
     dev, stream, handle = gpu_ctx
     rng = np.random.default_rng(rows % 1000 + cols)
-    lengths = rng.integers(0, 4, rows)
+    lengths = rng.integers(0, 6, rows)
     lengths[[5, rows // 3]] = [min(cols, 40_000), min(cols, 9_000)]
     rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
     colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)     # unsorted, repeated columns
@@ -375,7 +378,7 @@ def test_blocked_gather_through_spmvop_alg2(osa, gpu_ctx):
     """aclsparseSpMVOp ALG2 on a wide matrix uses the blocked-gather layout; Z separate from Y and aliased."""
     dev, stream, handle = gpu_ctx
     rows, cols = 40_000, 2_500_000
-    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 5, long_rows=((3, 50_000),))
+    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 5, long_rows=((3, 50_000),), per_row=120)
     d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
     A = osa.Csr(rows, cols, d[0], d[1], d[2])
     for alias in (False, True):
@@ -397,7 +400,7 @@ def test_blocked_gather_rejects_column_out_of_range(osa, gpu_ctx):
     OPSPARSE_E_INVALID; aclsparseSpMVPreprocess turns that into INVALID_VALUE."""
     dev, stream, handle = gpu_ctx
     rows, cols = 30_000, 1_200_000
-    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 9)
+    rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 9, per_row=160)
     colind = colind.copy()
     colind[colind.size // 2] = cols + 5
     L = osa.lib()
