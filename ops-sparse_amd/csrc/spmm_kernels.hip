@@ -29,7 +29,6 @@
 #include <climits>
 #include <cstdlib>
 #include <type_traits>
-#include <vector>
 
 #include "device_utils.h"
 
@@ -720,6 +719,40 @@ void LayoutPlan(OpsparseSpmmPlan *p)
     p->bytes = p->numLongRows > 0 ? off : 256;
 }
 
+// Tables of the long rows: longRows[i] = row, firstSeg[i] = its first segment (firstSeg[numLongRows] = all
+// segments), and for every segment its row and first entry.  `counter` starts at zero.
+__global__ __launch_bounds__(kBlockThreads) void SpmmLongTablesKernel(
+    const int32_t *__restrict__ rowOffsets, int64_t rows, int32_t numLongRows, int32_t numSegments,
+    unsigned long long *__restrict__ counter, int32_t *__restrict__ longRows, int32_t *__restrict__ firstSeg,
+    int32_t *__restrict__ segRow, int32_t *__restrict__ segStart)
+{
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (r >= rows) {
+        return;
+    }
+    const int32_t first = rowOffsets[r];
+    const int32_t len = rowOffsets[r + 1] - first;
+    if (len <= kLongRowNnz) {
+        return;
+    }
+    const int32_t segments = (len + kSegmentNnz - 1) / kSegmentNnz;
+    const unsigned long long old = atomicAdd(counter, (1ull << 32) | static_cast<unsigned int>(segments));
+    const int64_t index = static_cast<int64_t>(old >> 32);
+    const int64_t seg0 = static_cast<int64_t>(old & 0xffffffffull);
+    if (index >= numLongRows || seg0 + segments > numSegments) {
+        return;  // more long rows than were counted: the host sees it in the counter
+    }
+    longRows[index] = static_cast<int32_t>(r);
+    firstSeg[index] = static_cast<int32_t>(seg0);
+    if (index == numLongRows - 1) {
+        firstSeg[numLongRows] = static_cast<int32_t>(seg0 + segments);
+    }
+    for (int32_t j = 0; j < segments; ++j) {
+        segRow[seg0 + j] = static_cast<int32_t>(r);
+        segStart[seg0 + j] = first + j * kSegmentNnz;
+    }
+}
+
 // Device reduction of the row lengths into `scratch` (>= 16 bytes), read back
 // after a stream synchronisation.
 int RowStats(const int32_t *rowOffsets, int64_t rows, int32_t *scratch, hipStream_t s, int32_t out[3])
@@ -970,48 +1003,31 @@ int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t n
     if (static_cast<int64_t>(workspaceBytes) < p.bytes) {
         return OPSPARSE_E_WORKSPACE;
     }
-    // The long-row tables are built on the host from a copy of the row offsets
-    // (once per matrix, like the reference's Preprocess,
-    // sparse/spmm/arch35/spmm_csr_mat.cpp:94-136) and uploaded.
-    std::vector<int32_t> rp(static_cast<size_t>(rows) + 1);
-    if (hipMemcpyAsync(rp.data(), rowOffsets, rp.size() * 4, hipMemcpyDeviceToHost, s) != hipSuccess ||
+    // The long-row tables are written by one kernel: a long row takes its number among the long rows and its
+    // first segment from ONE 64-bit counter (rows in the upper half, segments in the lower), so the two
+    // numberings agree and firstSeg is a prefix sum whatever order the rows arrive in.  Nothing but the counter
+    // comes back to the host (the reference copies the row offsets to the host and builds its tables there,
+    // sparse/spmm/arch35/spmm_csr_mat.cpp:94-136).
+    auto *base = static_cast<unsigned char *>(workspace);
+    auto *counter = reinterpret_cast<unsigned long long *>(base + 16);
+    if (hipMemsetAsync(counter, 0, sizeof(unsigned long long), s) != hipSuccess) {
+        (void)hipGetLastError();
+        return OPSPARSE_E_LAUNCH;
+    }
+    hipLaunchKernelGGL(SpmmLongTablesKernel, dim3(static_cast<uint32_t>((rows + kBlockThreads - 1) / kBlockThreads)),
+                       dim3(kBlockThreads), 0, s, rowOffsets, rows, p.numLongRows, p.numSegments, counter,
+                       reinterpret_cast<int32_t *>(base + p.longRowsOff),
+                       reinterpret_cast<int32_t *>(base + p.longFirstSegOff),
+                       reinterpret_cast<int32_t *>(base + p.segRowOff),
+                       reinterpret_cast<int32_t *>(base + p.segStartOff));
+    unsigned long long counted = 0;
+    if (hipMemcpyAsync(&counted, counter, sizeof(counted), hipMemcpyDeviceToHost, s) != hipSuccess ||
         hipStreamSynchronize(s) != hipSuccess) {
         (void)hipGetLastError();
         return OPSPARSE_E_LAUNCH;
     }
-    std::vector<int32_t> longRows, firstSeg, segRow, segStart;
-    longRows.reserve(p.numLongRows);
-    firstSeg.reserve(p.numLongRows + 1);
-    segRow.reserve(p.numSegments);
-    segStart.reserve(p.numSegments);
-    for (int64_t r = 0; r < rows; ++r) {
-        const int32_t len = rp[r + 1] - rp[r];
-        if (len > kLongRowNnz) {
-            longRows.push_back(static_cast<int32_t>(r));
-            firstSeg.push_back(static_cast<int32_t>(segRow.size()));
-            for (int32_t q = rp[r]; q < rp[r + 1]; q += kSegmentNnz) {
-                segRow.push_back(static_cast<int32_t>(r));
-                segStart.push_back(q);
-            }
-        }
-    }
-    firstSeg.push_back(static_cast<int32_t>(segRow.size()));
-    if (static_cast<int32_t>(longRows.size()) != p.numLongRows || static_cast<int32_t>(segRow.size()) != p.numSegments) {
+    if (counted != ((static_cast<unsigned long long>(p.numLongRows) << 32) | static_cast<unsigned int>(p.numSegments))) {
         return OPSPARSE_E_INVALID;  // the matrix changed between the two passes
-    }
-    auto *base = static_cast<unsigned char *>(workspace);
-    bool ok = hipMemcpyAsync(base + p.longRowsOff, longRows.data(), longRows.size() * 4, hipMemcpyHostToDevice, s) ==
-              hipSuccess;
-    ok = ok && hipMemcpyAsync(base + p.longFirstSegOff, firstSeg.data(), firstSeg.size() * 4, hipMemcpyHostToDevice,
-                              s) == hipSuccess;
-    ok = ok && hipMemcpyAsync(base + p.segRowOff, segRow.data(), segRow.size() * 4, hipMemcpyHostToDevice, s) ==
-                   hipSuccess;
-    ok = ok && hipMemcpyAsync(base + p.segStartOff, segStart.data(), segStart.size() * 4, hipMemcpyHostToDevice, s) ==
-                   hipSuccess;
-    ok = ok && hipStreamSynchronize(s) == hipSuccess;  // the host vectors die at return
-    if (!ok) {
-        (void)hipGetLastError();
-        return OPSPARSE_E_LAUNCH;
     }
     *plan = p;
     return OPSPARSE_OK;
