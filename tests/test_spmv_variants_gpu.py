@@ -374,6 +374,45 @@ def test_blocked_gather_transposed(osa, gpu_ctx, rows, cols):
     assert oracle.max_rel_err(d_yn.cpu().numpy(), gold) <= 1e-5
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
+def test_blocked_gather_random_shapes(osa, gpu_ctx, seed):
+    """Seeded random shapes, both op(A): uniform short rows, power-law rows with a few of several hundred thousand
+    entries, or dense stretches between long runs of empty rows; unsorted columns with repeats.  The products are
+    exact in fp64 and rounded once, the same 1e-5 bar."""
+    dev, stream, handle = gpu_ctx
+    rng = np.random.default_rng(seed)
+    transpose = seed % 2 == 0
+    big, small = int(rng.integers(1_050_000, 4_000_000)), int(rng.integers(3_000, 400_000))
+    rows, cols = (big, small) if transpose else (small, big)
+    kind = ("uniform", "power", "clustered")[seed % 3]
+    if kind == "uniform":
+        lengths = rng.integers(0, 8, rows)
+    elif kind == "power":
+        lengths = np.minimum((rng.pareto(1.1, rows) * 3).astype(np.int64), 300_000)
+        lengths[rng.integers(0, rows, 3)] = rng.integers(50_000, 300_000, 3)
+    else:
+        lengths = np.zeros(rows, np.int64)
+        for _ in range(12):
+            a, w = int(rng.integers(0, rows)), int(rng.integers(1, max(2, rows // 40)))
+            lengths[a:a + w] = rng.integers(1, 60, min(w, rows - a))
+    lengths = np.minimum(lengths + max(0, (2_300_000 - int(lengths.sum())) // rows + 1), cols)
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    nin, nout = (rows, cols) if transpose else (cols, rows)
+    x, y0 = rng.uniform(-1, 1, nin).astype(np.float32), rng.uniform(-1, 1, nout).astype(np.float32)
+    assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, int(transpose)) > 0
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    d_y = to_dev(y0, dev)
+    op = osa.SpmvOp(handle, osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3]), osa.DnVec(d_y),
+                    op=osa.ACL_SPARSE_OP_TRANSPOSE if transpose else osa.ACL_SPARSE_OP_NON_TRANSPOSE,
+                    alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
+    op(-1.25, 0.5)
+    stream.synchronize()
+    gold = (oracle.spmv_trans_f64 if transpose else oracle.spmv_f64)(rows, cols, rowptr, colind, val, x, y0, -1.25, 0.5)
+    assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+
 def test_blocked_gather_through_spmvop_alg2(osa, gpu_ctx):
     """aclsparseSpMVOp ALG2 on a wide matrix uses the blocked-gather layout; Z separate from Y and aliased."""
     dev, stream, handle = gpu_ctx
