@@ -1,9 +1,12 @@
 // BLOCKED_GATHER: CSR SpMV for a matrix whose x does not fit a cache, fp32.
 //
-// Replaces the device side of the reference's aclsparseSpMV / SpMVOp with the
-// ALG2 preprocessing (sparse/spmv/arch35/spmv_kernel.cpp, launched by
-// sparse/spmv/spmv_host.cpp:196-260) for that case.  A row-wise kernel gathers
-// x[col] straight from memory, and with random columns every gather moves a
+// Takes the place of the reference's aclsparseSpMVOp with ALG2 — a device-side
+// preprocessing pass that re-orders the rows into the caller's buffer, then a
+// thread-per-row kernel (sparse/spmv_op/arch35/spmv_op_host.cpp:543-573 and
+// :423-457, spmv_op_kernel.cpp:413-535) — and of aclsparseSpMV's kernel
+// (sparse/spmv/arch22/kernels/spmv_kernel.h:27-310) for that case.  A
+// row-wise kernel gathers x[col] straight from memory, and with random columns
+// every gather moves a
 // whole 128-byte line for 4 useful bytes: the gather rate, not the matrix
 // stream, sets the time.  Here x is gathered from LDS instead.
 //
