@@ -120,6 +120,16 @@ int opsparse_spmv_csr_launch(const OpsparseSpmvPlan *plan, int32_t transpose, co
                              void *stream);
 
 /*
+ * Are the gathers of x scattered?  Samples up to 65 536 rows (32 entries each) and sets *scattered when more
+ * than one sampled column in twenty lies further than 2^17 columns from where its row sits on the diagonal.
+ * A banded or mesh-like matrix (not scattered) keeps x in cache under the row-wise kernels and gains nothing
+ * from a re-stored layout.  `workspace` needs 256 bytes.  Synchronises `stream` once.
+ */
+int opsparse_spmv_csr_gathers_scattered(const int32_t *rowOffsets, const int32_t *colInd, int64_t rows, int64_t cols,
+                                        int64_t nnz, void *workspace, size_t workspaceBytes, int32_t *scattered,
+                                        void *stream);
+
+/*
  * COLUMN_PANELS analysis (fp32, op(A) = A): bytes of the workspace, or 0 when the
  * family does not apply (it needs 2..16 panels of 2^20 columns, i.e. 1 M < cols <= 16 M).
  * The analysis re-stores the matrix — column indices AND values — in the

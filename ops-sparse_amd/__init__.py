@@ -91,6 +91,7 @@ OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_launch_zy", "opsparse_spmv_csr_indexed_launch",
     "opsparse_spmv_csr_panels_workspace_bytes", "opsparse_spmv_csr_panels_analyse",
     "opsparse_spmv_csr_blocked_workspace_bytes", "opsparse_spmv_csr_blocked_analyse",
+    "opsparse_spmv_csr_gathers_scattered",
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
     "opsparse_scan_workspace_bytes", "opsparse_coo2csr_launch", "opsparse_csr2coo_launch",
     "opsparse_csrsort_workspace_bytes", "opsparse_csrsort_launch", "opsparse_csr2csc_workspace_bytes",
@@ -232,6 +233,8 @@ def lib():
                                               i64, OpsparseScalar, OpsparseScalar, i32, i32, i32, vp, sz, vp]
     L.opsparse_spmv_csr_panels_workspace_bytes.restype = sz
     L.opsparse_spmv_csr_panels_workspace_bytes.argtypes = [i64, i64, i64]
+    L.opsparse_spmv_csr_gathers_scattered.restype = ctypes.c_int
+    L.opsparse_spmv_csr_gathers_scattered.argtypes = [vp, vp, i64, i64, i64, vp, sz, ctypes.POINTER(i32), vp]
     L.opsparse_spmv_csr_blocked_workspace_bytes.restype = sz
     L.opsparse_spmv_csr_blocked_workspace_bytes.argtypes = [i64, i64, i64, i32]
     L.opsparse_spmv_csr_blocked_analyse.restype = ctypes.c_int

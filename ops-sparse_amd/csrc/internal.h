@@ -110,7 +110,8 @@ aclsparseStatus_t EnsureWorkspace(aclsparseContext *h);
 // DEVICE mode the address is passed on and the kernel reads it.
 OpsparseScalar MakeScalar(const void *p, aclDataType computeType, aclsparsePointerMode_t mode, double dflt);
 
-// The re-stored SpMV layout an ALG2 request gets for a plain fp32 CSR matrix: BLOCKED_GATHER where it
+// The re-stored SpMV layout an ALG2 request gets for a plain fp32 CSR matrix (AnalyseRestored falls back to
+// the ordinary analysis in the same buffer when a sample of the columns shows the gathers are local): BLOCKED_GATHER where it
 // applies, else (op(A) = A only) COLUMN_PANELS, else none (kernel 0, 0 bytes).  OPS_SPARSE_SPMV_NO_BLOCKED in the
 // environment skips the first (tuning, tests of the panel path).
 struct RestoredChoice {

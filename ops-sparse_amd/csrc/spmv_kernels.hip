@@ -129,6 +129,40 @@ __global__ __launch_bounds__(kBlockThreads) void RowStatsKernel(const int32_t *_
     }
 }
 
+// How local are the gathers of x?  Every `rowStride`-th row is sampled, up to 32 of its entries each:
+// counts[0] = sampled entries, counts[1] = those whose column lies more than `band` away from where the
+// row sits on the diagonal (row * cols / rows).  counts must be zeroed before the launch.
+__global__ __launch_bounds__(kBlockThreads) void GatherLocalityKernel(const int32_t *__restrict__ rowOffsets,
+                                                                      const int32_t *__restrict__ colInd, int64_t rows,
+                                                                      int64_t cols, int64_t rowStride, int64_t band,
+                                                                      int32_t *__restrict__ counts)
+{
+    int32_t seen = 0, far = 0;
+    const int64_t sample = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
+    const int64_t r = sample * rowStride;
+    if (r < rows) {
+        const int64_t centre = static_cast<int64_t>(static_cast<double>(r) * static_cast<double>(cols) /
+                                                    static_cast<double>(rows));
+        const int32_t first = rowOffsets[r];
+        int32_t last = rowOffsets[r + 1];
+        last = last - first > 32 ? first + 32 : last;
+        for (int32_t k = first; k < last; ++k) {
+            const int64_t d = static_cast<int64_t>(colInd[k]) - centre;
+            ++seen;
+            far += (d > band || d < -band) ? 1 : 0;
+        }
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        seen += __shfl_xor(seen, off, kWave);
+        far += __shfl_xor(far, off, kWave);
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0 && seen > 0) {
+        atomicAdd(counts, seen);
+        atomicAdd(counts + 1, far);
+    }
+}
+
 // ------------------------------------------------------------- STREAM_ROWS
 
 // Four consecutive matrix entries of one lane, still in storage type.
@@ -1333,6 +1367,41 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
             return OPSPARSE_E_INVALID;
     }
     *plan = p;
+    return OPSPARSE_OK;
+}
+
+int opsparse_spmv_csr_gathers_scattered(const int32_t *rowOffsets, const int32_t *colInd, int64_t rows, int64_t cols,
+                                        int64_t nnz, void *workspace, size_t workspaceBytes, int32_t *scattered,
+                                        void *stream)
+{
+    if (scattered == nullptr || rows < 0 || cols < 0 || nnz < 0 ||
+        (rows > 0 && nnz > 0 && (rowOffsets == nullptr || colInd == nullptr))) {
+        return OPSPARSE_E_INVALID;
+    }
+    *scattered = 0;
+    if (rows == 0 || nnz == 0 || cols == 0) {
+        return OPSPARSE_OK;
+    }
+    if (workspace == nullptr || workspaceBytes < 256) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    auto s = static_cast<hipStream_t>(stream);
+    auto *counts = static_cast<int32_t *>(workspace) + 8;  // header words 8 and 9
+    LaunchFillI32(counts, 2, 0, s);
+    constexpr int64_t kSamples = 65536;
+    constexpr int64_t kBand = 131072;  // 2 * band * 4 bytes = 1 MiB of x around the diagonal: a quarter of an L2
+    const int64_t rowStride = (rows + kSamples - 1) / kSamples;
+    const int64_t samples = (rows + rowStride - 1) / rowStride;
+    hipLaunchKernelGGL(GatherLocalityKernel, dim3(static_cast<uint32_t>((samples + kBlockThreads - 1) / kBlockThreads)),
+                       dim3(kBlockThreads), 0, s, rowOffsets, colInd, rows, cols, rowStride, kBand, counts);
+    int32_t host[2] = {0, 0};
+    if (hipMemcpyAsync(host, counts, sizeof(host), hipMemcpyDeviceToHost, s) != hipSuccess ||
+        hipStreamSynchronize(s) != hipSuccess) {
+        (void)hipGetLastError();
+        return OPSPARSE_E_LAUNCH;
+    }
+    // scattered: more than one sampled gather in twenty lands outside the band
+    *scattered = (host[0] > 0 && static_cast<int64_t>(host[1]) * 20 > host[0]) ? 1 : 0;
     return OPSPARSE_OK;
 }
 

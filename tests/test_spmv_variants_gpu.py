@@ -330,7 +330,7 @@ def test_blocked_gather_giant_row_and_device_scalars(osa, gpu_ctx):
     assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
 
 
-@pytest.mark.parametrize("rows,cols", [(1_400_000, 50_000), (2_000_000, 2_000_000), (1_100_000, 300)])
+@pytest.mark.parametrize("rows,cols", [(1_400_000, 50_000), (2_000_000, 2_000_000), (1_200_000, 900_000), (1_100_000, 300)])
 def test_blocked_gather_transposed(osa, gpu_ctx, rows, cols):
     """ACL_SPARSE_SPMV_CSR_ALG2 with op(A) = A^T and more than 2^20 rows: the layout is built over the rows of A
     (panels, x) and its columns (row blocks, y), and the product has no atomics on y: the 1e-5 bar of op(A) = A,
@@ -410,6 +410,46 @@ def test_blocked_gather_random_shapes(osa, gpu_ctx, seed):
     op(-1.25, 0.5)
     stream.synchronize()
     gold = (oracle.spmv_trans_f64 if transpose else oracle.spmv_f64)(rows, cols, rowptr, colind, val, x, y0, -1.25, 0.5)
+    assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+
+def test_alg2_keeps_row_kernels_for_local_gathers(osa, workloads, gpu_ctx):
+    """A mesh matrix wide enough for the re-stored layouts (1.2 M columns, 6 M entries): its gathers stay within
+    1100 columns of the diagonal, x stays in cache under the row-wise kernels, and Preprocess with CSR_ALG2 keeps
+    those (the sampled-locality probe says "not scattered"); the same shape with random columns is scattered."""
+    dev, stream, handle = gpu_ctx
+    A = workloads.laplacian_2d(1100, dev)
+    rows, cols, nnz = A["rows"], A["cols"], int(A["colind"].numel())
+    L = osa.lib()
+    assert L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, 0) > 0
+    ws = torch.zeros(256, dtype=torch.uint8, device=dev)
+    flag = ctypes.c_int32(-1)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    torch.cuda.synchronize()
+    assert L.opsparse_spmv_csr_gathers_scattered(p(A["rowptr"]), p(A["colind"]), rows, cols, nnz, p(ws), 256,
+                                                 ctypes.byref(flag), sp) == 0 and flag.value == 0
+    shuffled = torch.randint(0, cols, (nnz,), dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    assert L.opsparse_spmv_csr_gathers_scattered(p(A["rowptr"]), p(shuffled), rows, cols, nnz, p(ws), 256,
+                                                 ctypes.byref(flag), sp) == 0 and flag.value == 1
+    rng = np.random.default_rng(3)
+    x, y0 = rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+    d_x, d_y = to_dev(x, dev), to_dev(y0, dev)
+    op = osa.SpmvOp(handle, osa.Csr(rows, cols, A["rowptr"], A["colind"], A["values"]), osa.DnVec(d_x), osa.DnVec(d_y),
+                    alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
+    op(1.0, 0.5)
+    stream.synchronize()
+    gold = oracle.spmv_f64(rows, cols, A["rowptr"].cpu().numpy(), A["colind"].cpu().numpy(),
+                           A["values"].cpu().numpy(), x, y0, 1.0, 0.5)
+    assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+    # the buffer holds an ordinary plan: changing the values needs no new Preprocess
+    A["values"].mul_(2.0)
+    d_y.copy_(torch.from_numpy(y0))
+    op(1.0, 0.5)
+    stream.synchronize()
+    gold = oracle.spmv_f64(rows, cols, A["rowptr"].cpu().numpy(), A["colind"].cpu().numpy(),
+                           A["values"].cpu().numpy(), x, y0, 1.0, 0.5)
     assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
 
 
