@@ -26,12 +26,17 @@ struct aclsparseSpMVOpDescr {
     void *values = nullptr;
     aclsparseSpMVOpAlg_t alg = ACL_SPARSE_SPMVOP_ALG1;
     void *userBuffer = nullptr;  // ALG2: caller's buffer holding the partition
-    bool planned = false;        // userBuffer was analysed successfully
+    bool planned = false;        // plan is valid (ALG2: userBuffer was analysed; ALG1: a row-wise kernel, no buffer)
     OpsparseSpmvPlan plan{};
 };
 
 struct aclsparseSpMVOpPlan {
     aclsparseSpMVOpDescr *descr = nullptr;
+    // ALG1 has no buffer, but the row-wise kernels keep nothing in one: the first execution looks at the row
+    // lengths once (one short kernel and a synchronisation) and later ones run the kernel they select.
+    bool rowsLooked = false;
+    bool rowsPlanned = false;
+    OpsparseSpmvPlan rowsPlan{};
 };
 
 namespace {
@@ -75,6 +80,32 @@ aclsparseStatus_t ValidateAlg(aclsparseSpMVOpAlg_t alg)
 bool Plain(const aclsparseSpMVOpDescr *d)
 {
     return d->rowOffsetsType == ACL_SPARSE_INDEX_32I && d->indexBase == ACL_SPARSE_INDEX_BASE_ZERO;
+}
+
+// First execution of an unplanned descriptor (ALG1): the row statistics into the handle's workspace.  A plan for
+// the stream-rows or vector-rows kernel is kept (the 2048 x 2048 Laplacian: 41 us a call against 71 us for the
+// merge path); a merge-path plan would live in that workspace, which other calls overwrite, and is dropped.
+// Not under stream capture: the analysis synchronises.
+void LookAtRows(aclsparseHandle_t handle, aclsparseSpMVOpPlan *plan)
+{
+    const aclsparseSpMVOpDescr *d = plan->descr;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(handle->stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return;  // looked at again by the next execution outside a capture
+    }
+    plan->rowsLooked = true;
+    if (handle->workspaceBytes() < opsparse_spmv_csr_workspace_bytes(d->rows, d->nnz)) {
+        return;
+    }
+    OpsparseSpmvPlan p{};
+    const int rc = opsparse_spmv_csr_analyse(static_cast<const int32_t *>(d->rowOffsets), d->rows, d->cols, d->nnz,
+                                             handle->workspace(), handle->workspaceBytes(), OPSPARSE_SPMV_AUTO, &p,
+                                             handle->stream);
+    if (rc == OPSPARSE_OK && (p.kernel == OPSPARSE_SPMV_STREAM_ROWS || p.kernel == OPSPARSE_SPMV_VECTOR_ROWS)) {
+        plan->rowsPlan = p;
+        plan->rowsPlanned = true;
+    }
 }
 
 // ALG2's device-side reorder is, for a matrix whose x does not fit an L2, a re-stored layout (blocked gather,
@@ -309,6 +340,12 @@ aclsparseStatus_t aclsparseSpMVOp(aclsparseHandle_t handle, aclsparseSpMVOpPlan_
             }
             ws = handle->workspace();
             wsBytes = handle->workspaceBytes();
+            if (!plan->rowsLooked) {
+                LookAtRows(handle, plan);
+            }
+            if (plan->rowsPlanned) {
+                p = &plan->rowsPlan;
+            }
         }
         // nnz == 0 needs no offsets at all: Z = beta * Y whatever their width.
         rc = opsparse_spmv_csr_launch_zy(p, 0, static_cast<const int32_t *>(d->nnz > 0 ? d->rowOffsets : nullptr),

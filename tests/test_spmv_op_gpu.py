@@ -20,7 +20,7 @@ import pytest
 import torch
 
 import oracle
-from helpers import random_csr, to_dev
+from helpers import csr_from_lengths, random_csr, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -212,3 +212,48 @@ def test_raw_indexed_launch_matches_plain(osa, gpu_ctx):
     assert L.opsparse_spmv_csr_indexed_launch(d_rp64.data_ptr(), 1, 2, d_ci1.data_ptr(), d_val.data_ptr(),
                                               d_x.data_ptr(), d_y.data_ptr(), d_z.data_ptr(), m, k, nnz, sa, sb,
                                               sp) == -1
+
+
+@pytest.mark.parametrize("shape", ["short_rows", "even_rows", "skewed_rows"])
+def test_alg1_repeated_executions_and_value_updates(osa, gpu_ctx, shape):
+    """ALG1 supports changing csrValues under a live descriptor (reference include/cann_ops_sparse.h:58-63).  The
+    first execution looks at the row lengths and later ones run the kernel they select (short rows: stream rows,
+    even long rows: vector rows, skewed: the merge path every time); every execution must match the oracle on the
+    values of that moment, with other calls using the handle's workspace in between."""
+    dev, stream, handle = gpu_ctx
+    rng = np.random.default_rng(17)
+    m, k = 50_000, 60_000
+    if shape == "short_rows":
+        lengths = rng.integers(0, 9, m)
+    elif shape == "even_rows":
+        lengths = rng.integers(60, 90, m)
+    else:
+        lengths = np.minimum((rng.pareto(1.1, m) * 2).astype(np.int64), 20_000)
+        lengths[7] = 20_000
+    rowptr, colind, val = csr_from_lengths(lengths, k, 23)
+    x, y = rng.uniform(-1, 1, k).astype(np.float32), rng.uniform(-1, 1, m).astype(np.float32)
+    d_rp, d_ci, d_val, d_x, d_y = (to_dev(a, dev) for a in (rowptr, colind, val, x, y))
+    d_z = torch.zeros(m, dtype=torch.float32, device=dev)
+    A = osa.Csr(m, k, d_rp, d_ci, d_val)
+    op = osa.SpmvOpPlan(handle, A, osa.DnVec(d_x), osa.DnVec(d_y), osa.DnVec(d_z), alg=osa.ACL_SPARSE_SPMVOP_ALG1)
+    # another user of the handle's workspace between the executions
+    o_rp, o_ci, o_val = csr_from_lengths(np.minimum((rng.pareto(1.0, 3000) * 3).astype(np.int64), 2500), 4000, 29)
+    o_x = rng.uniform(-1, 1, 4000).astype(np.float32)
+    d_o = [to_dev(a, dev) for a in (o_rp, o_ci, o_val, o_x)]
+    d_oy = torch.zeros(3000, dtype=torch.float32, device=dev)
+    other = osa.SpmvOp(handle, osa.Csr(3000, 4000, d_o[0], d_o[1], d_o[2]), osa.DnVec(d_o[3]), osa.DnVec(d_oy),
+                       preprocess=False)
+    for step in range(4):
+        if step:
+            val = (val * np.float32(-0.5) + np.float32(0.125 * step)).astype(np.float32)
+            d_val.copy_(torch.from_numpy(val))
+        d_z.zero_()
+        op(1.5, -0.25)
+        stream.synchronize()
+        check(d_z.cpu().numpy(), m, k, rowptr, colind, val, x, y, 1.5, -0.25)
+        other(1.0, 0.0)
+        stream.synchronize()
+        assert oracle.max_rel_err(d_oy.cpu().numpy(),
+                                  oracle.spmv_f64(3000, 4000, o_rp, o_ci, o_val, o_x, np.zeros(3000, np.float32),
+                                                  1.0, 0.0)) <= 1e-5
+    op.close()
