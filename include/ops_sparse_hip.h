@@ -84,7 +84,9 @@ typedef struct OpsparseSpmvPlan {
     int32_t numRowBlocks;  /* BLOCKED_GATHER: number of row blocks */
     int32_t entryWindow;   /* BLOCKED_GATHER: a row block also ends where the entry count passes a multiple of this */
     int32_t transposed;    /* BLOCKED_GATHER: the layout was built for op(A) = A^T and serves only that */
-    int32_t reserved0;
+    int32_t guardTiles;    /* STREAM_ROWS: the row offsets may have changed since the analysis: a tile with more
+                              entries than its LDS was sized for is summed from memory instead (set by callers
+                              that keep a plan without the user having asked for one; 0 after analyse) */
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */

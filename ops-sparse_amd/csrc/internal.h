@@ -37,6 +37,15 @@ struct OpsparseSpmvBinding {
     OpsparseSpmvPlan plan{};
 };
 
+// What the first aclsparseSpMV call without a preprocessed buffer learns about the rows of a matrix: the row-wise
+// kernels keep nothing in a buffer, so later calls on the same row offsets run the one these statistics select.
+struct OpsparseSpmvRowsSeen {
+    const void *rowOffsets = nullptr;  // the statistics are of these offsets, this many rows and entries
+    int64_t rows = -1;
+    int64_t nnz = -1;
+    OpsparseSpmvPlan plan{};
+};
+
 struct OpsparseSpmmBinding {
     const void *buffer = nullptr;
     OpsparseSpmmPlan plan{};
@@ -74,6 +83,7 @@ struct aclsparseSpMatDescr {
     // active buffer in the descriptor all the same
     // (sparse/spmm/arch35/spmm_host.cpp:360); `mutable` makes that explicit.
     mutable OpsparseSpmvBinding spmv;
+    mutable OpsparseSpmvRowsSeen rowsSeen;
     mutable OpsparseSpmmBinding spmm;
 };
 

@@ -124,6 +124,44 @@ aclsparseStatus_t FromLaunch(int rc)
     }
 }
 
+// An unprepared call (no preprocessed buffer bound to matA): the row statistics of matA, taken once per set of row
+// offsets into the handle's workspace (one short kernel and a stream synchronisation; the reference copies all
+// row offsets to the host at every call, spmv_host.cpp:86-112).  Returns the plan to run with, or NULL for the
+// merge path, whose partition is rebuilt by every call because the workspace is shared.  The row-wise kernels read
+// no buffer and stay correct, only slower, on row offsets that changed in place since the statistics were taken.
+// Not under stream capture, where nothing may synchronise: such a call takes the merge path.
+const OpsparseSpmvPlan *RowsSeen(aclsparseHandle_t handle, aclsparseConstSpMatDescr_t matA, bool transpose)
+{
+    OpsparseSpmvRowsSeen &seen = matA->rowsSeen;
+    if (seen.rowOffsets != matA->rowOffsets || seen.rows != matA->rows || seen.nnz != matA->nnz) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(handle->stream, &capturing) != hipSuccess ||
+            capturing != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        if (handle->workspaceBytes() < opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz)) {
+            return nullptr;
+        }
+        OpsparseSpmvPlan plan{};
+        if (opsparse_spmv_csr_analyse(static_cast<const int32_t *>(matA->rowOffsets), matA->rows, matA->cols,
+                                      matA->nnz, handle->workspace(), handle->workspaceBytes(), OPSPARSE_SPMV_AUTO,
+                                      &plan, handle->stream) != OPSPARSE_OK) {
+            return nullptr;
+        }
+        seen.rowOffsets = matA->rowOffsets;
+        seen.rows = matA->rows;
+        seen.nnz = matA->nnz;
+        seen.plan = plan;
+        seen.plan.guardTiles = 1;  // nobody promised that these row offsets stay as they are
+    }
+    // op(A) = A^T only takes the longest row from the plan, whatever its kernel
+    if (transpose || seen.plan.kernel == OPSPARSE_SPMV_STREAM_ROWS || seen.plan.kernel == OPSPARSE_SPMV_VECTOR_ROWS) {
+        return &seen.plan;
+    }
+    return nullptr;
+}
+
 }  // namespace
 
 namespace opsparse {
@@ -290,6 +328,9 @@ aclsparseStatus_t aclsparseSpMV(aclsparseHandle_t handle, aclsparseOperation_t o
         }
         ws = handle->workspace();
         wsBytes = handle->workspaceBytes();
+        if (plan == nullptr && matA->nnz > 0 && matA->rows > 0) {
+            plan = RowsSeen(handle, matA, c.transpose);
+        }
     }
     const int rc = opsparse_spmv_csr_launch(
         plan, c.transpose ? 1 : 0, static_cast<const int32_t *>(matA->rowOffsets),

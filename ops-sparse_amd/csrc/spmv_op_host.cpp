@@ -104,6 +104,7 @@ void LookAtRows(aclsparseHandle_t handle, aclsparseSpMVOpPlan *plan)
                                              handle->stream);
     if (rc == OPSPARSE_OK && (p.kernel == OPSPARSE_SPMV_STREAM_ROWS || p.kernel == OPSPARSE_SPMV_VECTOR_ROWS)) {
         plan->rowsPlan = p;
+        plan->rowsPlan.guardTiles = 1;
         plan->rowsPlanned = true;
     }
 }

@@ -514,3 +514,59 @@ def test_transpose_half_precision_output(osa, gpu_ctx, dtype, rel, beta):
                  val_dtype=dtype, out_dtype=dtype)
     gold = oracle.spmv_trans_f64(rows, cols, rowptr, colind, val, x, y0, 1.5, beta)
     assert np.all(np.abs(y - gold) <= rel * np.abs(gold) + 1e-4)
+
+
+@pytest.mark.parametrize("per_row,out_dtype", [(4, None), (20, None), (6, torch.float16), (40, None)])
+def test_unprepared_calls_survive_row_offsets_changed_in_place(osa, gpu_ctx, per_row, out_dtype):
+    """The first call without a preprocessed buffer takes the row statistics of the matrix, and later ones run the
+    stream-rows kernel they select, whose LDS is sized for the longest row seen.  Nobody promised those calls
+    that the row offsets stay: rewritten in place afterwards — same array, same entry count, one row now thousands
+    of entries long, others empty, one row twice as long inside an unchanged tile — they must still give the
+    right product (such tiles are summed from memory).  After Preprocess the structure is the caller's promise."""
+    dev, stream, handle = gpu_ctx
+    rng = np.random.default_rng(per_row)
+    rows, cols = 60_000, 50_000
+    lengths = np.full(rows, per_row, np.int64)
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    x, y0 = rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+    if out_dtype is not None:
+        val, x = (torch.from_numpy(a).to(out_dtype).float().numpy() for a in (val, x))
+    vt = out_dtype or torch.float32
+    d_rp, d_ci = to_dev(rowptr, dev), to_dev(colind, dev)
+    d_val, d_x = torch.from_numpy(val).to(vt).to(dev), torch.from_numpy(x).to(vt).to(dev)
+    d_y = torch.from_numpy(y0).to(vt).to(dev)
+    A = osa.Csr(rows, cols, d_rp, d_ci, d_val)
+    op = osa.SpmvOp(handle, A, osa.DnVec(d_x), osa.DnVec(d_y), preprocess=False)
+    y0r = d_y.float().cpu().numpy()
+
+    def check_against(rp):
+        d_y.copy_(torch.from_numpy(y0r).to(vt))
+        op(1.5, 0.5)
+        stream.synchronize()
+        gold = oracle.spmv_f64(rows, cols, rp, colind, val, x, y0r, 1.5, 0.5)
+        got = d_y.float().cpu().numpy()
+        if out_dtype is None:
+            assert oracle.max_rel_err(got, gold) <= 1e-5
+        else:                                          # y rounded once to fp16: within an ulp of the rounded oracle
+            want = _round(gold, out_dtype)
+            assert np.all(np.abs(got - want) <= 2.0 ** -10 * np.maximum(np.abs(want), 2.0 ** -14))
+
+    check_against(rowptr)
+    moved = lengths.copy()
+    moved[5] += 3000                                   # far beyond what a tile's LDS was sized for
+    taken, r = 0, 30_000
+    while taken < 3000:                                # taken from rows that become empty / shorter
+        t = min(per_row, 3000 - taken)
+        moved[r] -= t
+        taken += t
+        r += 1
+    moved[50_001] += moved[50_000]                     # a row twice as long, its tile's entry count unchanged
+    moved[50_000] = 0
+    assert moved.sum() == lengths.sum()
+    rowptr2 = np.concatenate([[0], np.cumsum(moved)]).astype(np.int32)
+    d_rp.copy_(torch.from_numpy(rowptr2))
+    check_against(rowptr2)
+    d_rp.copy_(torch.from_numpy(rowptr))
+    check_against(rowptr)
