@@ -126,6 +126,8 @@ int opsparse_spmv_csr_launch(const OpsparseSpmvPlan *plan, int32_t transpose, co
  * than one sampled column in twenty lies further than 2^17 columns from where its row sits on the diagonal.
  * A banded or mesh-like matrix (not scattered) keeps x in cache under the row-wise kernels and gains nothing
  * from a re-stored layout.  `workspace` needs 256 bytes.  Synchronises `stream` once.
+ * No counterpart in the reference, whose ALG2 preprocessing (sparse/spmv_op/arch35/spmv_op_host.cpp:543-573)
+ * reorders every matrix alike; here it is one of the questions that preprocessing asks.
  */
 int opsparse_spmv_csr_gathers_scattered(const int32_t *rowOffsets, const int32_t *colInd, int64_t rows, int64_t cols,
                                         int64_t nnz, void *workspace, size_t workspaceBytes, int32_t *scattered,
