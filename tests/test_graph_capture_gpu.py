@@ -124,3 +124,39 @@ def test_spmm_replays(osa, gpu_ctx):
         stream.synchronize()
         gold = oracle.spmm_f64_rowmajor(m, n, rowptr, colind, val, b, n, c0, n, 1.25, 0.5)
         assert oracle.max_rel_err(d_c.cpu().numpy(), np.asarray(gold).ravel()) <= 1e-5, replay
+
+
+def test_first_unprepared_call_inside_a_capture(osa, gpu_ctx):
+    """The first aclsparseSpMV on a matrix without a preprocessed buffer normally synchronises once to read the row
+    statistics.  Inside a capture nothing may synchronise: the call must notice, take the merge path, leave the
+    capture intact, and the statistics are then taken by the next eager call."""
+    dev, stream, handle = gpu_ctx
+    rng = np.random.default_rng(41)
+    warm = csr_from_lengths(np.full(100, 3), 100, 1)                 # the handle's workspace exists after this
+    d_w = [to_dev(a, dev) for a in warm]
+    wx, wy = torch.ones(100, device=dev), torch.zeros(100, device=dev)
+    osa.SpmvOp(handle, osa.Csr(100, 100, *d_w), osa.DnVec(wx), osa.DnVec(wy), preprocess=False)(1.0, 0.0)
+    stream.synchronize()
+
+    rows = cols = 30_000
+    rowptr, colind, val = csr_from_lengths(np.full(rows, 6), cols, 43)  # short even rows: stream rows once seen
+    x, y0 = rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    d_y = to_dev(y0, dev)
+    op = osa.SpmvOp(handle, osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3]), osa.DnVec(d_y), preprocess=False)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        op(2.0, 0.5)                                                 # never ran eagerly before
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 2.0, 0.5)
+    for replay in range(2):
+        d_y.copy_(torch.from_numpy(y0))
+        stream.synchronize()
+        graph.replay()
+        stream.synchronize()
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5, replay
+    d_y.copy_(torch.from_numpy(y0))
+    op(2.0, 0.5)                                                     # eager: statistics now, row-wise kernel
+    op(1.0, 0.0)
+    stream.synchronize()
+    gold2 = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, gold.astype(np.float32), 1.0, 0.0)
+    assert oracle.max_rel_err(d_y.cpu().numpy(), gold2) <= 1e-5
