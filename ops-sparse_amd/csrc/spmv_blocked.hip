@@ -512,7 +512,9 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     window = window < kMinEntryWindow ? kMinEntryWindow : window;
     const int64_t B = ((rows + kRowBlockRows - 1) >> kRowBlockLog) + nnz / window + 1;
     // x must be larger than an L2 (2^20 columns) for the two passes to pay, and the chunks long enough to stream.
-    if (cols <= (int64_t{1} << 20) || nnz < kMinEntries || P > kMaxPanels || P * B + 1 > INT32_MAX || nnz + kLaneEntries * P * B > INT32_MAX || nnz / (P * B) < kMinChunkEntries) {
+    // Positions are 32-bit, and phase 2 looks two batches past a block's end before it clamps.
+    if (cols <= (int64_t{1} << 20) || nnz < kMinEntries || P > kMaxPanels || P * B + 1 > INT32_MAX ||
+        nnz + kLaneEntries * P * B > INT32_MAX - 65536 || nnz / (P * B) < kMinChunkEntries) {
         return l;
     }
     l.P = static_cast<int32_t>(P);

@@ -331,7 +331,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
                     sum += prod[k];
                 }
             } else {
-                for (int32_t k = s + lane; k < e; k += G) {
+                for (int64_t k = static_cast<int64_t>(s) + lane; k < e; k += G) {
                     sum += ToAcc<AccT>(vals[k]) * ToAcc<AccT>(x[colInd[k]]);
                 }
             }
@@ -491,7 +491,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvVectorRowsKernel(
     const int32_t s = rowOffsets[r];
     const int32_t e = rowOffsets[r + 1];
     AccT sum0 = AccT(0), sum1 = AccT(0);
-    int32_t k = s + lane;
+    int64_t k = static_cast<int64_t>(s) + lane;  // 64 bits: k + 2 G may pass 2^31 when nnz is close to it
     for (; k + G < e; k += 2 * G) {  // two independent gathers in flight per lane
         const int32_t c0 = LoadStream(colInd + k);
         const int32_t c1 = LoadStream(colInd + k + G);
@@ -826,7 +826,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvTransposeScatterKernel(
         return;
     }
     const int32_t e = rowOffsets[r + 1];
-    for (int32_t k = rowOffsets[r] + threadIdx.x % G; k < e; k += G) {
+    for (int64_t k = static_cast<int64_t>(rowOffsets[r]) + threadIdx.x % G; k < e; k += G) {
         atomicAdd(y + LoadStream(colInd + k), static_cast<float>(ax * ToAcc<AccT>(LoadStream(vals + k))));
     }
 }
@@ -1344,9 +1344,15 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
     const double mean = static_cast<double>(nnz) / static_cast<double>(rows);
     int32_t kernel = forceKernel;
     if (kernel == OPSPARSE_SPMV_AUTO) {
-        if (maxRow <= 48) {
+        // Measured on 64 M entries, even rows and rows of 0.5 - 1.5 times the mean, banded and random columns:
+        // stream rows sizes its tiles for the longest row and wins while they are mostly full or the rows very
+        // short (mean 16 - 48 even: 160 - 173 us against 195 - 200 us for the merge path; varied: 217 - 222 us
+        // against 194 - 199 us); a lane group per row only pays for long rows of nearly equal length (mean 128 -
+        // 256: 180 us against 195 us; varied rows 250 - 350 us against 189 us); the merge path does not care.
+        if (maxRow <= 48 && (maxRow <= 12 || static_cast<double>(maxRow) * static_cast<double>(rows) <=
+                                                 1.25 * static_cast<double>(nnz))) {
             kernel = OPSPARSE_SPMV_STREAM_ROWS;
-        } else if (mean >= 32.0 && static_cast<double>(maxRow) <= 16.0 * mean) {
+        } else if (mean >= 96.0 && mean <= 400.0 && static_cast<double>(maxRow) <= 1.125 * mean) {
             kernel = OPSPARSE_SPMV_VECTOR_ROWS;
         } else {
             kernel = OPSPARSE_SPMV_MERGE_PATH;
