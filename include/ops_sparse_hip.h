@@ -216,7 +216,7 @@ int opsparse_spmm_csr_workspace_bytes(const int32_t *rowOffsets, int64_t rows, i
                                       size_t *bytes);
 
 /* Row statistics and, for BINNED, the long-row / segment tables (built on the
- * host from a copy of the row offsets).  Synchronises `stream`. */
+ * device; 12 bytes of statistics and one counter travel to the host).  Synchronises `stream`. */
 int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t nnz, int64_t n, void *workspace,
                               size_t workspaceBytes, int32_t forceKernel, OpsparseSpmmPlan *plan, void *stream);
 
@@ -235,6 +235,16 @@ int opsparse_spmm_csr_launch(const OpsparseSpmmPlan *plan, const int32_t *rowOff
                              int64_t nnz, int64_t ldb, int64_t ldc, int32_t bColMajor, int32_t cColMajor,
                              int32_t transB, OpsparseScalar alpha, OpsparseScalar beta, int32_t valType,
                              int32_t cType, void *workspace, size_t workspaceBytes, void *stream);
+
+/*
+ * Dense rows x cols matrix copied from one storage order / leading dimension to another (elements of 1, 2 or
+ * 4 bytes); columns cols .. colsDst-1 of the destination are written as zero.  aclsparseSpMM uses it to hand
+ * column-major or transposed B / C to the row-major kernels through a staging area of the SpMM buffer: the
+ * index formulas are the reference kernel's [ref: sparse/spmm/arch35/spmm_kernel.cpp:155-168, :215-219], which
+ * reads such operands in place, one element per line.
+ */
+int opsparse_dense_restage(const void *src, void *dst, int64_t rows, int64_t cols, int64_t colsDst, int64_t ldSrc,
+                           int32_t srcColMajor, int64_t ldDst, int32_t dstColMajor, int32_t elemBytes, void *stream);
 
 /* --------------------------------------------------------- CSR producers
  * Raw launchers of the format conversions; they play the role of the reference's

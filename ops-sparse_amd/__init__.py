@@ -93,6 +93,7 @@ OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_blocked_workspace_bytes", "opsparse_spmv_csr_blocked_analyse",
     "opsparse_spmv_csr_gathers_scattered",
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
+    "opsparse_dense_restage",
     "opsparse_scan_workspace_bytes", "opsparse_coo2csr_launch", "opsparse_csr2coo_launch",
     "opsparse_csrsort_workspace_bytes", "opsparse_csrsort_launch", "opsparse_csr2csc_workspace_bytes",
     "opsparse_csr2csc_launch",
@@ -254,6 +255,8 @@ def lib():
     L.opsparse_spmm_csr_launch.argtypes = [ctypes.POINTER(OpsparseSpmmPlan), vp, vp, vp, vp, vp, i64, i64, i64, i64,
                                            i64, i64, i32, i32, i32, OpsparseScalar, OpsparseScalar, i32, i32, vp, sz,
                                            vp]
+    L.opsparse_dense_restage.restype = ctypes.c_int
+    L.opsparse_dense_restage.argtypes = [vp, vp, i64, i64, i64, i64, i32, i64, i32, i32, vp]
     L.opsparse_copy_launch.restype = ctypes.c_int
     L.opsparse_copy_launch.argtypes = [vp, vp, sz, vp]
     L.opsparse_read_launch.restype = ctypes.c_int

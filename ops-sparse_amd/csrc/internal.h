@@ -49,6 +49,7 @@ struct OpsparseSpmvRowsSeen {
 struct OpsparseSpmmBinding {
     const void *buffer = nullptr;
     OpsparseSpmmPlan plan{};
+    int64_t stagingBytes = 0;  // room behind the plan's tables for row-major copies of B / C (0: none)
 };
 
 // reference: sparse/common/aclsparse_handle_internal.h:56-72

@@ -93,9 +93,57 @@ aclsparseStatus_t FromLaunch(int rc)
     }
 }
 
-// Row statistics and long-row tables into `buffer`; binds the buffer to A.
-aclsparseStatus_t BuildPlan(const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *C, void *buffer,
-                            hipStream_t stream)
+int64_t ElementBytes(int32_t type)
+{
+    return type == OPSPARSE_F32 || type == OPSPARSE_I32 ? 4 : (type == OPSPARSE_I8 ? 1 : 2);
+}
+
+// Column-major or transposed B, column-major C: the reference kernel reads them in place through its index
+// formulas (spmm_kernel.cpp:155-168, :215-219), which here would mean one cache line per element (32/row, n = 64,
+// column-major B: 37.8 ms against 1.2 ms row-major).  Instead the SpMM buffer carries, behind the plan's tables,
+// room for compact row-major copies of such operands: B is copied in, the row-major kernels run, C is copied
+// in (unless beta is known to be 0) and out.  n is padded to whole 16-byte vectors in the copies, so that a
+// width the vector kernels do not take (n = 12) goes the same way.  Not for int8, which has no vector kernel.
+struct Staging {
+    bool b = false, c = false;
+    int64_t nPadded = 0, bOff = 0, cOff = 0;
+    int64_t bytes = 0;  // beyond the plan's own bytes, 0: the operands are used where they are
+};
+
+Staging MakeStaging(const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *B, const aclsparseDnMatDescr *C,
+                    aclsparseOperation_t opB, const SpmmTypes &t, int64_t planBytes)
+{
+    Staging g{};
+    const bool bColMajor = (B->order == ACL_SPARSE_ORDER_COL) != (opB == ACL_SPARSE_OP_TRANSPOSE);
+    const bool cColMajor = C->order == ACL_SPARSE_ORDER_COL;
+    if (t.valType == OPSPARSE_I8 || (!bColMajor && !cColMajor) || A->rows <= 0 || A->cols <= 0 || C->cols <= 0) {
+        return g;
+    }
+    const int64_t vec = 16 / ElementBytes(t.valType);
+    g.nPadded = (C->cols + vec - 1) / vec * vec;
+    // a width that is not whole vectors needs both copies: the kernels then run on the padded width
+    g.b = bColMajor || g.nPadded != C->cols;
+    g.c = cColMajor || g.nPadded != C->cols;
+    auto align = [](int64_t v) { return (v + 255) / 256 * 256; };
+    int64_t off = align(planBytes);
+    g.bOff = off;
+    off += g.b ? align(A->cols * g.nPadded * ElementBytes(t.valType)) : 0;
+    g.cOff = off;
+    off += g.c ? align(A->rows * g.nPadded * ElementBytes(t.cType)) : 0;
+    g.bytes = off - planBytes;
+    return g;
+}
+
+// The width the plan is made for: the padded one when the product runs on staged copies.
+int64_t PlanWidth(const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *B, const aclsparseDnMatDescr *C,
+                  aclsparseOperation_t opB, const SpmmTypes &t)
+{
+    const Staging g = MakeStaging(A, B, C, opB, t, 0);
+    return g.bytes > 0 ? g.nPadded : C->cols;
+}
+
+// Row statistics and long-row tables for width n into `buffer`; binds the buffer to A.
+aclsparseStatus_t BuildPlan(const aclsparseSpMatDescr *A, int64_t n, void *buffer, hipStream_t stream)
 {
     // An empty matrix has nothing to preprocess (spmm_csr_mat.cpp:148-150).
     if (A->rows <= 0) {
@@ -106,20 +154,71 @@ aclsparseStatus_t BuildPlan(const aclsparseSpMatDescr *A, const aclsparseDnMatDe
     }
     OpsparseSpmmPlan plan{};
     size_t bytes = 0;
-    int rc = opsparse_spmm_csr_workspace_bytes(static_cast<const int32_t *>(A->rowOffsets), A->rows, A->nnz, C->cols,
+    int rc = opsparse_spmm_csr_workspace_bytes(static_cast<const int32_t *>(A->rowOffsets), A->rows, A->nnz, n,
                                                stream, &bytes);
     if (rc != OPSPARSE_OK) {
         return FromLaunch(rc);
     }
-    rc = opsparse_spmm_csr_analyse(static_cast<const int32_t *>(A->rowOffsets), A->rows, A->nnz, C->cols,
-                                             buffer, bytes, OPSPARSE_SPMM_AUTO, &plan, stream);
+    rc = opsparse_spmm_csr_analyse(static_cast<const int32_t *>(A->rowOffsets), A->rows, A->nnz, n, buffer, bytes,
+                                   OPSPARSE_SPMM_AUTO, &plan, stream);
     if (rc != OPSPARSE_OK) {
         opsparse::LogError("aclsparseSpMM: analysis failed (%d)", rc);
         return FromLaunch(rc);
     }
     A->spmm.buffer = buffer;
     A->spmm.plan = plan;
+    A->spmm.stagingBytes = 0;
     return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+bool ScalarIsZero(const void *host, aclDataType computeType)
+{
+    return computeType == ACL_INT32 ? *static_cast<const int32_t *>(host) == 0
+                                    : *static_cast<const float *>(host) == 0.0f;
+}
+
+// The product through the staging area: B copied to compact row-major (padded width), the row-major kernels,
+// C copied in (unless beta is 0 for certain) and out.  Kernels only, all on `stream`.
+int RunStaged(const Staging &g, const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *B,
+              const aclsparseDnMatDescr *C, aclsparseOperation_t opB, OpsparseScalar alpha, OpsparseScalar beta,
+              const SpmmTypes &t, bool betaIsZero, void *buffer, hipStream_t stream)
+{
+    auto *base = static_cast<unsigned char *>(buffer);
+    const int64_t k = A->cols, m = A->rows, n = C->cols;
+    const bool bColMajor = (B->order == ACL_SPARSE_ORDER_COL) != (opB == ACL_SPARSE_OP_TRANSPOSE);
+    const bool cColMajor = C->order == ACL_SPARSE_ORDER_COL;
+    const void *bUse = B->values;
+    void *cUse = C->values;
+    int64_t ldb = B->ld, ldc = C->ld;
+    int rc = OPSPARSE_OK;
+    if (g.b) {
+        rc = opsparse_dense_restage(B->values, base + g.bOff, k, n, g.nPadded, B->ld, bColMajor ? 1 : 0, g.nPadded, 0,
+                                    static_cast<int32_t>(ElementBytes(t.valType)), stream);
+        bUse = base + g.bOff;
+        ldb = g.nPadded;
+    }
+    if (rc == OPSPARSE_OK && g.c) {
+        cUse = base + g.cOff;
+        ldc = g.nPadded;
+        if (!betaIsZero) {
+            rc = opsparse_dense_restage(C->values, cUse, m, n, g.nPadded, C->ld, cColMajor ? 1 : 0, g.nPadded, 0,
+                                        static_cast<int32_t>(ElementBytes(t.cType)), stream);
+        }
+    }
+    if (rc != OPSPARSE_OK) {
+        return rc;
+    }
+    // both copies exist whenever the width was padded, so the kernels may take the padded width as theirs
+    const int64_t nRun = A->spmm.plan.n;  // the padded width, which the plan was made for
+    rc = opsparse_spmm_csr_launch(&A->spmm.plan, static_cast<const int32_t *>(A->rowOffsets),
+                                  static_cast<const int32_t *>(A->colInd), A->values, bUse, cUse, m, k, nRun, A->nnz,
+                                  ldb, ldc, 0, g.c ? 0 : (cColMajor ? 1 : 0), 0, alpha, beta, t.valType, t.cType,
+                                  buffer, static_cast<size_t>(A->spmm.plan.bytes), stream);
+    if (rc == OPSPARSE_OK && g.c) {
+        rc = opsparse_dense_restage(cUse, C->values, m, n, n, g.nPadded, 0, C->ld, cColMajor ? 1 : 0,
+                                    static_cast<int32_t>(ElementBytes(t.cType)), stream);
+    }
+    return rc;
 }
 
 }  // namespace
@@ -146,8 +245,11 @@ aclsparseStatus_t aclsparseSpMMGetBufferSize(aclsparseHandle_t handle, aclsparse
         return ACL_SPARSE_STATUS_INVALID_VALUE;
     }
     const int rc = opsparse_spmm_csr_workspace_bytes(static_cast<const int32_t *>(matA->rowOffsets), matA->rows,
-                                                     matA->nnz, matC->cols,
+                                                     matA->nnz, PlanWidth(matA, matB, matC, opB, t),
                                                      handle != nullptr ? handle->stream : nullptr, size);
+    if (rc == OPSPARSE_OK) {
+        *size += static_cast<size_t>(MakeStaging(matA, matB, matC, opB, t, static_cast<int64_t>(*size)).bytes);
+    }
     return FromLaunch(rc);
 }
 
@@ -166,7 +268,13 @@ aclsparseStatus_t aclsparseSpMMPreprocess(aclsparseHandle_t handle, aclsparseOpe
         return ACL_SPARSE_STATUS_INSUFFICIENT_RESOURCES;
     }
     // The reference ignores the handle here; its stream is used when there is one.
-    return BuildPlan(matA, matC, buffer, handle != nullptr ? handle->stream : nullptr);
+    const aclsparseStatus_t built = BuildPlan(matA, PlanWidth(matA, matB, matC, opB, t), buffer,
+                                              handle != nullptr ? handle->stream : nullptr);
+    if (built == ACL_SPARSE_STATUS_SUCCESS) {
+        // the buffer was sized by GetBufferSize for these operands: their staging area exists
+        matA->spmm.stagingBytes = MakeStaging(matA, matB, matC, opB, t, matA->spmm.plan.bytes).bytes;
+    }
+    return built;
 }
 
 aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t opA, aclsparseOperation_t opB,
@@ -185,11 +293,16 @@ aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t o
     if (handle == nullptr) {
         return ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR;
     }
-    // A buffer that is not the one bound to matA is preprocessed first
-    // (spmm_host.cpp:310-321).
-    if (matA->spmm.buffer != buffer || matA->spmm.plan.rows != matA->rows || matA->spmm.plan.nnz != matA->nnz ||
-        matA->spmm.plan.n != matC->cols) {
-        st = BuildPlan(matA, matC, buffer, handle->stream);
+    // Staged copies of B / C only in a buffer that Preprocess was given for operands needing at least as much:
+    // nothing else says how large the buffer is.  A buffer that is not the one bound to matA is preprocessed first
+    // (spmm_host.cpp:310-321), without a staging area.
+    const Staging g = MakeStaging(matA, matB, matC, opB, t, matA->spmm.plan.bytes);
+    const bool bound = matA->spmm.buffer == buffer && matA->spmm.plan.rows == matA->rows &&
+                       matA->spmm.plan.nnz == matA->nnz;
+    bool staged = bound && g.bytes > 0 && g.bytes <= matA->spmm.stagingBytes && matA->spmm.plan.n == g.nPadded &&
+                  matA->nnz > 0;
+    if (!staged && (!bound || matA->spmm.plan.n != matC->cols)) {
+        st = BuildPlan(matA, matC->cols, buffer, handle->stream);
         if (st != ACL_SPARSE_STATUS_SUCCESS) {
             return st;
         }
@@ -197,12 +310,19 @@ aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t o
     // NULL scalars read as 0 (spmm_host.cpp:62-74).
     const OpsparseScalar a = opsparse::MakeScalar(alpha, computeType, handle->pointerMode, 0.0);
     const OpsparseScalar b = opsparse::MakeScalar(beta, computeType, handle->pointerMode, 0.0);
-    const int rc = opsparse_spmm_csr_launch(
-        &matA->spmm.plan, static_cast<const int32_t *>(matA->rowOffsets), static_cast<const int32_t *>(matA->colInd),
-        matA->values, matB->values, matC->values, matA->rows, matA->cols, matC->cols, matA->nnz, matB->ld, matC->ld,
-        matB->order == ACL_SPARSE_ORDER_COL ? 1 : 0, matC->order == ACL_SPARSE_ORDER_COL ? 1 : 0,
-        opB == ACL_SPARSE_OP_TRANSPOSE ? 1 : 0, a, b, t.valType, t.cType, buffer,
-        static_cast<size_t>(matA->spmm.plan.bytes), handle->stream);
+    int rc;
+    if (staged) {
+        rc = RunStaged(g, matA, matB, matC, opB, a, b, t, handle->pointerMode == ACL_SPARSE_POINTER_MODE_HOST &&
+                                                              beta != nullptr && ScalarIsZero(beta, computeType),
+                       buffer, handle->stream);
+    } else {
+        rc = opsparse_spmm_csr_launch(
+            &matA->spmm.plan, static_cast<const int32_t *>(matA->rowOffsets),
+            static_cast<const int32_t *>(matA->colInd), matA->values, matB->values, matC->values, matA->rows,
+            matA->cols, matC->cols, matA->nnz, matB->ld, matC->ld, matB->order == ACL_SPARSE_ORDER_COL ? 1 : 0,
+            matC->order == ACL_SPARSE_ORDER_COL ? 1 : 0, opB == ACL_SPARSE_OP_TRANSPOSE ? 1 : 0, a, b, t.valType,
+            t.cType, buffer, static_cast<size_t>(matA->spmm.plan.bytes), handle->stream);
+    }
     if (rc != OPSPARSE_OK) {
         opsparse::LogError("aclsparseSpMM: launch failed (%d)", rc);
     }

@@ -645,6 +645,40 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmGeneralKernel(
     }
 }
 
+// A dense rows x cols matrix copied from one storage order / leading dimension to another, a 32 x 32 tile per
+// workgroup through LDS: the tile is read along the source's contiguous direction and written along the
+// destination's.  Columns cols .. colsDst-1 of the destination (padding) are written as zero.
+template <typename T>
+__global__ __launch_bounds__(kBlockThreads) void DenseRestageKernel(const T *__restrict__ src, T *__restrict__ dst,
+                                                                    int64_t rows, int64_t cols, int64_t colsDst,
+                                                                    int64_t ldSrc, int32_t srcColMajor, int64_t ldDst,
+                                                                    int32_t dstColMajor, int64_t tilesAcross)
+{
+    constexpr int kTile = 32;
+    __shared__ T tile[kTile][kTile + 1];  // [row][column]
+    const int64_t r0 = static_cast<int64_t>(blockIdx.x) / tilesAcross * kTile;
+    const int64_t c0 = static_cast<int64_t>(blockIdx.x) % tilesAcross * kTile;
+    const int tx = threadIdx.x % kTile, ty = threadIdx.x / kTile;
+    constexpr int kStep = kBlockThreads / kTile;
+    for (int i = ty; i < kTile; i += kStep) {
+        const int rr = srcColMajor ? tx : i, cc = srcColMajor ? i : tx;
+        const int64_t r = r0 + rr, c = c0 + cc;
+        T v = T(0);
+        if (r < rows && c < cols) {
+            v = src[srcColMajor ? r + c * ldSrc : r * ldSrc + c];
+        }
+        tile[rr][cc] = v;
+    }
+    __syncthreads();
+    for (int i = ty; i < kTile; i += kStep) {
+        const int rr = dstColMajor ? tx : i, cc = dstColMajor ? i : tx;
+        const int64_t r = r0 + rr, c = c0 + cc;
+        if (r < rows && c < colsDst) {
+            dst[dstColMajor ? r + c * ldDst : r * ldDst + c] = tile[rr][cc];
+        }
+    }
+}
+
 // Longest row, number of long rows and number of segments.  stats[0..2] zeroed
 // before the launch.
 __global__ __launch_bounds__(kBlockThreads) void SpmmRowStatsKernel(const int32_t *__restrict__ rowOffsets,
@@ -1074,6 +1108,50 @@ int opsparse_spmm_csr_launch(const OpsparseSpmmPlan *plan, const int32_t *rowOff
         return RunGeneral<int8_t, int32_t, int32_t>(a);
     }
     return OPSPARSE_E_UNSUPPORTED;
+}
+
+int opsparse_dense_restage(const void *src, void *dst, int64_t rows, int64_t cols, int64_t colsDst, int64_t ldSrc,
+                           int32_t srcColMajor, int64_t ldDst, int32_t dstColMajor, int32_t elemBytes, void *stream)
+{
+    if (rows < 0 || cols < 0 || colsDst < cols || ldSrc <= 0 || ldDst <= 0 ||
+        (elemBytes != 1 && elemBytes != 2 && elemBytes != 4)) {
+        return OPSPARSE_E_INVALID;
+    }
+    // the source is read through the index formula whatever its ld (a transposed reading of B may overlap);
+    // the destination's rows / columns must not
+    if (ldDst < (dstColMajor ? rows : colsDst)) {
+        return OPSPARSE_E_INVALID;
+    }
+    if (rows == 0 || colsDst == 0) {
+        return OPSPARSE_OK;
+    }
+    if (src == nullptr || dst == nullptr) {
+        return OPSPARSE_E_INVALID;
+    }
+    const int64_t across = (colsDst + 31) / 32, down = (rows + 31) / 32;
+    if (across * down > INT32_MAX) {
+        return OPSPARSE_E_UNSUPPORTED;
+    }
+    const dim3 grid(static_cast<uint32_t>(across * down));
+    auto s = static_cast<hipStream_t>(stream);
+    switch (elemBytes) {
+        case 4:
+            hipLaunchKernelGGL(DenseRestageKernel<uint32_t>, grid, dim3(kBlockThreads), 0, s,
+                               static_cast<const uint32_t *>(src), static_cast<uint32_t *>(dst), rows, cols, colsDst,
+                               ldSrc, srcColMajor, ldDst, dstColMajor, across);
+            break;
+        case 2:
+            hipLaunchKernelGGL(DenseRestageKernel<uint16_t>, grid, dim3(kBlockThreads), 0, s,
+                               static_cast<const uint16_t *>(src), static_cast<uint16_t *>(dst), rows, cols, colsDst,
+                               ldSrc, srcColMajor, ldDst, dstColMajor, across);
+            break;
+        default:
+            hipLaunchKernelGGL(DenseRestageKernel<uint8_t>, grid, dim3(kBlockThreads), 0, s,
+                               static_cast<const uint8_t *>(src), static_cast<uint8_t *>(dst), rows, cols, colsDst,
+                               ldSrc, srcColMajor, ldDst, dstColMajor, across);
+            break;
+    }
+    return CheckLaunch();
 }
 
 }  // extern "C"

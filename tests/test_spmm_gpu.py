@@ -11,11 +11,14 @@ Tolerances, written per test:
                     inputs, clamp, re-round; MERE < 2^-10, MARE < 10 * 2^-10
   int8              bit-exact
 """
+import ctypes
+
 import numpy as np
 import pytest
+import torch
 
 import oracle
-from helpers import csr_from_lengths, random_csr, run_spmm
+from helpers import csr_from_lengths, random_csr, run_spmm, to_dev
 
 pytestmark = pytest.mark.gpu
 
@@ -292,3 +295,76 @@ def test_raw_launch_without_plan(osa, gpu_ctx, n):
     stream.synchronize()
     gold = oracle.spmm_f64_rowmajor(m, n, rowptr, colind, val, B, n, C0, n, 0.5, 2.0)
     assert oracle.max_rel_err(d[4].cpu().numpy(), gold) <= 1e-5
+
+
+@pytest.mark.parametrize("b_rm,c_rm,trans_b", [(False, True, False), (True, False, False), (False, False, False),
+                                               (True, True, True), (False, False, True)])
+@pytest.mark.parametrize("n,half", [(64, False), (10, False), (44, True)])
+def test_layouts_through_the_staging_area(osa, gpu_ctx, b_rm, c_rm, trans_b, n, half):
+    """Column-major / transposed operands at a size with many tiles, long rows (the binned path) and a width that
+    is not whole 16-byte vectors: Preprocess reserves row-major copies behind the plan, the product runs on them
+    and C comes back in its own layout, padding of ldb / ldc untouched.  beta = 0 must not read C (NaN)."""
+    rng = np.random.default_rng(n + 7 * b_rm + 3 * c_rm + trans_b)
+    m = k = 3000
+    lengths = rng.integers(0, 30, m)
+    lengths[[5, 1500]] = [2800, 700]
+    rowptr, colind, val = csr_from_lengths(lengths, k, seed=9)
+    eff_col = (not b_rm) != trans_b                 # op(B) = B^T flips which index of B is contiguous
+    ldb = k + 3 if (eff_col or not b_rm) else n + 4  # a column-major descriptor needs ld >= rows in any case
+    ldc = n + 8 if c_rm else m + 5
+    B = rng.uniform(-1, 1, (n if eff_col else k) * ldb).astype(np.float32)
+    C_len = (m * ldc) if c_rm else (n * ldc)
+    vd, cd, tol = (torch.float16, torch.float32, 1e-5) if half else (None, None, 1e-5)
+    if half:
+        val, B = (torch.from_numpy(a).to(torch.float16).float().numpy() for a in (val, B))
+    for alpha, beta in ((1.5, 0.25), (2.0, 0.0)):
+        C0 = rng.uniform(-1, 1, C_len).astype(np.float32)
+        C_in = C0.copy()
+        if beta == 0.0:
+            logical = np.zeros(C_len, bool)
+            idx = (np.arange(m)[:, None] * ldc + np.arange(n)[None, :]) if c_rm else \
+                  (np.arange(m)[:, None] + np.arange(n)[None, :] * ldc)
+            logical[idx.ravel()] = True
+            C_in[logical] = np.nan               # must not be read; the padding keeps its values
+        got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, ldb, C_in, ldc, alpha, beta,
+                       order_b=osa.ACL_SPARSE_ORDER_ROW if b_rm else osa.ACL_SPARSE_ORDER_COL,
+                       order_c=osa.ACL_SPARSE_ORDER_ROW if c_rm else osa.ACL_SPARSE_ORDER_COL,
+                       op_b=osa.ACL_SPARSE_OP_TRANSPOSE if trans_b else osa.ACL_SPARSE_OP_NON_TRANSPOSE,
+                       val_dtype=vd, c_dtype=cd)
+        gold = oracle.spmm_f64(m, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta, b_row_major=b_rm,
+                               trans_b=trans_b, c_row_major=c_rm)
+        assert oracle.max_rel_err(got, gold) <= tol
+
+
+def test_staging_needs_a_buffer_preprocessed_for_it(osa, gpu_ctx):
+    """A buffer sized and preprocessed for row-major operands (256 bytes here) and then used with a column-major B:
+    no staging area was promised, the product must run in place (slowly) and stay inside the buffer — the guard
+    bytes behind it keep their pattern."""
+    dev, stream, handle = gpu_ctx
+    rng = np.random.default_rng(3)
+    m, k, n = 500, 400, 12
+    rowptr, colind, val = random_csr(m, k, 0.05, seed=4)
+    B = rng.uniform(-1, 1, k * n).astype(np.float32)
+    C0 = rng.uniform(-1, 1, m * n).astype(np.float32)
+    d = [to_dev(a, dev) for a in (rowptr, colind, val)]
+    d_B, d_C = to_dev(B, dev), to_dev(C0, dev)
+    A = osa.Csr(m, k, d[0], d[1], d[2])
+    B_row, B_col = osa.DnMat(k, n, n, d_B), osa.DnMat(k, n, k, d_B, osa.ACL_SPARSE_ORDER_COL)
+    Cd = osa.DnMat(m, n, n, d_C)
+    L = osa.lib()
+    size = ctypes.c_size_t(0)
+    args = lambda Bd: (handle.h, 0, 0, None, A.d, Bd.d, None, Cd.d, osa.ACL_FLOAT, osa.ACL_SPARSE_SPMM_ALG_DEFAULT)
+    assert L.aclsparseSpMMGetBufferSize(*args(B_row), ctypes.byref(size)) == 0
+    small = int(size.value)
+    assert L.aclsparseSpMMGetBufferSize(*args(B_col), ctypes.byref(size)) == 0 and int(size.value) >= small + k * n * 4
+    buf = torch.full((small + 4096,), 0x5A, dtype=torch.uint8, device=dev)
+    bp = ctypes.c_void_p(buf.data_ptr())
+    assert L.aclsparseSpMMPreprocess(*args(B_row), bp) == 0
+    one, half_ = ctypes.c_float(1.0), ctypes.c_float(0.5)
+    assert L.aclsparseSpMM(handle.h, 0, 0, ctypes.byref(one), A.d, B_col.d, ctypes.byref(half_), Cd.d, osa.ACL_FLOAT,
+                           osa.ACL_SPARSE_SPMM_ALG_DEFAULT, bp) == 0
+    stream.synchronize()
+    assert bool((buf[small:] == 0x5A).all())
+    gold = oracle.spmm_f64(m, n, rowptr, colind, val, B, k, C0, n, 1.0, 0.5, b_row_major=False, trans_b=False,
+                           c_row_major=True)
+    assert oracle.max_rel_err(d_C.cpu().numpy(), gold) <= 1e-5
