@@ -102,8 +102,9 @@ int64_t ElementBytes(int32_t type)
 // formulas (spmm_kernel.cpp:155-168, :215-219), which here would mean one cache line per element (32/row, n = 64,
 // column-major B: 37.8 ms against 1.2 ms row-major).  Instead the SpMM buffer carries, behind the plan's tables,
 // room for compact row-major copies of such operands: B is copied in, the row-major kernels run, C is copied
-// in (unless beta is known to be 0) and out.  n is padded to whole 16-byte vectors in the copies, so that a
-// width the vector kernels do not take (n = 12) goes the same way.  Not for int8, which has no vector kernel.
+// in (unless beta is known to be 0) and out.  n is padded to whole 16-byte vectors in the copies, so row-major
+// operands of a width or leading dimension the vector kernels do not take go the same way (n = 62: 3.2 ms in
+// place, n = 64: 1.2 ms).  Not for int8, which has no vector kernel.
 struct Staging {
     bool b = false, c = false;
     int64_t nPadded = 0, bOff = 0, cOff = 0;
@@ -116,14 +117,18 @@ Staging MakeStaging(const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *B, 
     Staging g{};
     const bool bColMajor = (B->order == ACL_SPARSE_ORDER_COL) != (opB == ACL_SPARSE_OP_TRANSPOSE);
     const bool cColMajor = C->order == ACL_SPARSE_ORDER_COL;
-    if (t.valType == OPSPARSE_I8 || (!bColMajor && !cColMajor) || A->rows <= 0 || A->cols <= 0 || C->cols <= 0) {
+    if (t.valType == OPSPARSE_I8 || A->rows <= 0 || A->cols <= 0 || C->cols <= 0) {
         return g;
     }
     const int64_t vec = 16 / ElementBytes(t.valType);
     g.nPadded = (C->cols + vec - 1) / vec * vec;
-    // a width that is not whole vectors needs both copies: the kernels then run on the padded width
-    g.b = bColMajor || g.nPadded != C->cols;
-    g.c = cColMajor || g.nPadded != C->cols;
+    // a width that is not whole vectors needs both copies: the kernels then run on the padded width; a row-major
+    // operand whose leading dimension is not whole vectors needs its own
+    g.b = bColMajor || g.nPadded != C->cols || B->ld % vec != 0;
+    g.c = cColMajor || g.nPadded != C->cols || C->ld % vec != 0;
+    if (!g.b && !g.c) {
+        return g;
+    }
     auto align = [](int64_t v) { return (v + 255) / 256 * 256; };
     int64_t off = align(planBytes);
     g.bOff = off;
