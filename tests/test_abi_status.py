@@ -260,8 +260,14 @@ def test_spmm_status_table(osa, L, handle):
     assert L.aclsparseSpMM(*spmm_args(osa, None, A, B, C), None) == st(osa, "INSUFFICIENT_RESOURCES")
     assert L.aclsparseSpMM(*spmm_args(osa, None, A, B, C), FAKE) == HN
     assert L.aclsparseSpMMPreprocess(*spmm_args(osa, handle, A, B, C), None) == st(osa, "INSUFFICIENT_RESOURCES")
-    # a matrix this small cannot have a long row: 256-byte header, no device access
-    assert L.aclsparseSpMMGetBufferSize(*spmm_args(osa, None, A, B, C), ctypes.byref(n)) == 0 and n.value == 256
+    # a matrix this small cannot have a long row: 256-byte header, no device access; n = 2 is not a whole 16-byte
+    # vector of fp32, so the buffer also holds padded copies of B (3 x 4) and C (4 x 4), 256 bytes each
+    assert L.aclsparseSpMMGetBufferSize(*spmm_args(osa, None, A, B, C), ctypes.byref(n)) == 0 and n.value == 768
+    _, B4w = make_mat(osa, L, rows=3, cols=4, ld=4)
+    _, C4w = make_mat(osa, L, rows=4, cols=4, ld=4)
+    assert L.aclsparseSpMMGetBufferSize(*spmm_args(osa, None, A, B4w, C4w), ctypes.byref(n)) == 0 and n.value == 256
+    L.aclsparseDestroyDnMat(B4w)
+    L.aclsparseDestroyDnMat(C4w)
     # Preprocess of an empty matrix is refused (reference spmm_csr_mat.cpp:148-150)
     _, E = make_csr(osa, L, rows=0, cols=3, nnz=0)
     _, C0 = make_mat(osa, L, rows=1, cols=2, ld=2)
