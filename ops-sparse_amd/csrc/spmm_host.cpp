@@ -104,7 +104,7 @@ int64_t ElementBytes(int32_t type)
 // room for compact row-major copies of such operands: B is copied in, the row-major kernels run, C is copied
 // in (unless beta is known to be 0) and out.  n is padded to whole 16-byte vectors in the copies, so row-major
 // operands of a width or leading dimension the vector kernels do not take go the same way (n = 62: 3.2 ms in
-// place, n = 64: 1.2 ms).  Not for int8, which has no vector kernel.
+// place, n = 64: 1.2 ms).
 struct Staging {
     bool b = false, c = false;
     int64_t nPadded = 0, bOff = 0, cOff = 0;
@@ -117,7 +117,7 @@ Staging MakeStaging(const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *B, 
     Staging g{};
     const bool bColMajor = (B->order == ACL_SPARSE_ORDER_COL) != (opB == ACL_SPARSE_OP_TRANSPOSE);
     const bool cColMajor = C->order == ACL_SPARSE_ORDER_COL;
-    if (t.valType == OPSPARSE_I8 || A->rows <= 0 || A->cols <= 0 || C->cols <= 0) {
+    if (A->rows <= 0 || A->cols <= 0 || C->cols <= 0) {
         return g;
     }
     const int64_t vec = 16 / ElementBytes(t.valType);

@@ -208,6 +208,34 @@ def test_int8_exact(osa, gpu_ctx, alpha, beta):
     assert np.array_equal(got, gold)
 
 
+@pytest.mark.parametrize("n,b_rm,c_rm", [(64, True, True), (128, True, True), (50, True, True), (48, False, True),
+                                         (16, True, False)])
+def test_int8_vector_kernels_long_rows_and_layouts(osa, gpu_ctx, n, b_rm, c_rm):
+    """int8 x int8 -> int32 on the 16-bytes-per-lane kernels (16 columns a lane): long rows through the segment
+    path, a width that is not whole vectors and column-major operands through the staged copies; bit-exact,
+    saturating epilogue."""
+    import torch
+    rng = np.random.default_rng(n)
+    m, k = 2500, 4000
+    lengths = rng.integers(0, 25, m)
+    lengths[[7, 1200]] = [3000, 600]
+    rowptr, colind, _ = csr_from_lengths(lengths, k, seed=n)
+    val = rng.integers(-128, 128, colind.size).astype(np.int8)
+    ldb, ldc = (n if b_rm else k), (n if c_rm else m)
+    B = rng.integers(-128, 128, (k if b_rm else n) * ldb).astype(np.int8)
+    C0 = rng.integers(-1000, 1000, (m if c_rm else n) * ldc).astype(np.int32)
+    for alpha, beta in ((1, 0), (3, -2), (70000, 1)):
+        got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta,
+                       order_b=osa.ACL_SPARSE_ORDER_ROW if b_rm else osa.ACL_SPARSE_ORDER_COL,
+                       order_c=osa.ACL_SPARSE_ORDER_ROW if c_rm else osa.ACL_SPARSE_ORDER_COL,
+                       val_dtype=torch.int8, c_dtype=torch.int32, compute_type=osa.ACL_INT32)
+        Bl = B.reshape(k, n) if b_rm else B.reshape(n, k).T          # logical k x n
+        gold = oracle.spmm_i8(m, n, rowptr, colind, val, np.ascontiguousarray(Bl).ravel(), n,
+                              (C0.reshape(m, n) if c_rm else C0.reshape(n, m).T).ravel().copy(), n, alpha, beta,
+                              saturate=True).reshape(m, n)
+        assert np.array_equal(got.reshape(m, n) if c_rm else got.reshape(n, m).T, gold)
+
+
 def test_spmm_column_equals_spmv(osa, gpu_ctx):
     """Column j of the SpMM result equals the oracle SpMV with B[:, j]."""
     m, k, n = 333, 222, 8
