@@ -885,6 +885,64 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvTransposeFlatKernel(
     }
 }
 
+constexpr int kNarrowCols = 8192;        // y of op(A) = A^T kept per workgroup in LDS up to this many columns
+constexpr int kNarrowMaxBlocks = 1024;
+
+// op(A) = A^T with few columns: millions of atomic updates would fall on a handful of addresses (40 000 rows of 120
+// entries over 9 columns: half a million fp32 adds per element of y, one after the other in the L2).  Every
+// workgroup instead takes a contiguous run of entry tiles, adds its products up in an fp64 copy of y in LDS, and
+// at the end adds each non-zero element of that copy to y once: at most kNarrowMaxBlocks fp32 updates per element.
+template <typename ValT, typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmvTransposeNarrowKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ x, float *__restrict__ y, int64_t rows, int64_t cols, int64_t nnz, int64_t tilesPerBlock,
+    OpsparseScalar alphaS)
+{
+    __shared__ AccT sums[kNarrowCols];
+    __shared__ int32_t slice[kTransposeRowSlots];
+    __shared__ int64_t bounds[2];
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    for (int64_t c = threadIdx.x; c < cols; c += kBlockThreads) {
+        sums[c] = AccT(0);
+    }
+    const int64_t numTiles = (nnz + kTransposeTile - 1) / kTransposeTile;
+    const int64_t t0 = static_cast<int64_t>(blockIdx.x) * tilesPerBlock;
+    const int64_t t1 = t0 + tilesPerBlock < numTiles ? t0 + tilesPerBlock : numTiles;
+    for (int64_t t = t0; t < t1; ++t) {
+        const int64_t k0 = t * kTransposeTile;
+        const int64_t k1 = k0 + kTransposeTile < nnz ? k0 + kTransposeTile : nnz;
+        __syncthreads();  // the previous tile's slice is no longer read; the first time: sums are zero
+        if (threadIdx.x < 2) {
+            const int32_t k = static_cast<int32_t>(threadIdx.x == 0 ? k0 : k1 - 1);
+            bounds[threadIdx.x] = RowOfEntry(rowOffsets, 0, rows - 1, k);
+        }
+        __syncthreads();
+        const int64_t rLo = bounds[0], rHi = bounds[1];
+        const bool staged = rHi - rLo + 2 <= kTransposeRowSlots;
+        if (staged) {
+            for (int64_t i = threadIdx.x; i <= rHi - rLo + 1; i += kBlockThreads) {
+                slice[i] = rowOffsets[rLo + i];
+            }
+        }
+        __syncthreads();
+        for (int64_t k = k0 + threadIdx.x; k < k1; k += kBlockThreads) {
+            const int32_t kk = static_cast<int32_t>(k);
+            const int64_t r = staged ? rLo + RowOfEntry(slice, 0, rHi - rLo, kk) : RowOfEntry(rowOffsets, rLo, rHi, kk);
+            const int32_t c = LoadStream(colInd + k);
+            if (c >= 0 && c < cols) {  // an index outside y must not reach LDS
+                atomicAdd(&sums[c], alpha * ToAcc<AccT>(x[r]) * ToAcc<AccT>(LoadStream(vals + k)));
+            }
+        }
+    }
+    __syncthreads();
+    for (int64_t c = threadIdx.x; c < cols; c += kBlockThreads) {
+        const AccT v = sums[c];
+        if (v != AccT(0)) {
+            atomicAdd(y + c, static_cast<float>(v));
+        }
+    }
+}
+
 // =============================================================== host side
 
 namespace {
@@ -1251,6 +1309,15 @@ int RunTranspose(const SpmvArgs &a, int32_t outType, bool skewedRows)
         return rc;
     }
     if (a.nnz == 0 || a.rows == 0) {
+        return finish();
+    }
+    if (a.cols <= kNarrowCols && a.nnz >= 16 * kTransposeTile && a.nnz >= 8 * a.cols) {
+        // few columns: y per workgroup in LDS, one global update per workgroup and element
+        const int64_t numTiles = (a.nnz + kTransposeTile - 1) / kTransposeTile;
+        const int64_t tilesPerBlock = (numTiles + kNarrowMaxBlocks - 1) / kNarrowMaxBlocks;
+        hipLaunchKernelGGL((SpmvTransposeNarrowKernel<ValT, AccT>), dim3(GridFor(numTiles, tilesPerBlock)),
+                           dim3(kBlockThreads), 0, a.stream, a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
+                           static_cast<const ValT *>(a.x), acc, a.rows, a.cols, a.nnz, tilesPerBlock, a.alpha);
         return finish();
     }
     if (skewedRows && a.nnz >= 8 * kTransposeTile) {

@@ -570,3 +570,28 @@ def test_unprepared_calls_survive_row_offsets_changed_in_place(osa, gpu_ctx, per
     check_against(rowptr2)
     d_rp.copy_(torch.from_numpy(rowptr))
     check_against(rowptr)
+
+
+@pytest.mark.parametrize("rows,cols,per_row,half", [(40_000, 9, 120, True), (200_000, 300, 20, False),
+                                                    (60_000, 8192, 40, False), (30_000, 8193, 40, False)])
+def test_transpose_few_columns_accumulates_per_workgroup(osa, gpu_ctx, rows, cols, per_row, half):
+    """op(A) = A^T onto a short y: hundreds of thousands of contributions per element.  With one fp32 atomic each
+    (the reference's scheme) the rounding errors add up past 1e-2 in absolute terms; summed per workgroup in fp64
+    and added to y once per workgroup they stay at fp32 round-off of the result.  8193 columns are one too many
+    for that kernel and take the atomic one, under the loose rule only."""
+    rng = np.random.default_rng(rows + cols)
+    rowptr = (np.arange(rows + 1, dtype=np.int64) * per_row).astype(np.int32)
+    colind = rng.integers(0, cols, rows * per_row).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    x, y0 = rng.uniform(-1, 1, rows).astype(np.float32), rng.uniform(-1, 1, cols).astype(np.float32)
+    if half:
+        val, x = _round(val, torch.float16), _round(x, torch.float16)
+    for prep in (False, True):
+        y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 2.25, 0.5, preprocess=prep,
+                     op=osa.ACL_SPARSE_OP_TRANSPOSE, val_dtype=torch.float16 if half else None,
+                     out_dtype=torch.float32 if half else None)
+        gold = oracle.spmv_trans_f64(rows, cols, rowptr, colind, val, x, y0, 2.25, 0.5)
+        d = np.abs(y - gold)
+        assert (d <= 2.0 ** -16 + 2.0 ** -10 * np.abs(gold)).mean() >= 0.99 and d.max() <= 1e-2
+        if cols <= 8192:
+            assert d.max() <= 1e-4 * max(1.0, float(np.abs(gold).max()))
