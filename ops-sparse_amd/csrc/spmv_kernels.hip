@@ -885,20 +885,20 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvTransposeFlatKernel(
     }
 }
 
-constexpr int kNarrowCols = 8192;        // y of op(A) = A^T kept per workgroup in LDS up to this many columns
+constexpr int kNarrowCols = 16384;       // y of op(A) = A^T kept per workgroup in LDS up to this many columns
 constexpr int kNarrowMaxBlocks = 1024;
 
 // op(A) = A^T with few columns: millions of atomic updates would fall on a handful of addresses (40 000 rows of 120
 // entries over 9 columns: half a million fp32 adds per element of y, one after the other in the L2).  Every
 // workgroup instead takes a contiguous run of entry tiles, adds its products up in an fp64 copy of y in LDS, and
 // at the end adds each non-zero element of that copy to y once: at most kNarrowMaxBlocks fp32 updates per element.
-template <typename ValT, typename AccT>
+template <typename ValT, typename AccT, int Capacity>
 __global__ __launch_bounds__(kBlockThreads) void SpmvTransposeNarrowKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
     const ValT *__restrict__ x, float *__restrict__ y, int64_t rows, int64_t cols, int64_t nnz, int64_t tilesPerBlock,
     OpsparseScalar alphaS)
 {
-    __shared__ AccT sums[kNarrowCols];
+    __shared__ AccT sums[Capacity];  // 64 KiB (two workgroups per CU) or 128 KiB
     __shared__ int32_t slice[kTransposeRowSlots];
     __shared__ int64_t bounds[2];
     const AccT alpha = ReadScalar<AccT>(alphaS);
@@ -1315,9 +1315,11 @@ int RunTranspose(const SpmvArgs &a, int32_t outType, bool skewedRows)
         // few columns: y per workgroup in LDS, one global update per workgroup and element
         const int64_t numTiles = (a.nnz + kTransposeTile - 1) / kTransposeTile;
         const int64_t tilesPerBlock = (numTiles + kNarrowMaxBlocks - 1) / kNarrowMaxBlocks;
-        hipLaunchKernelGGL((SpmvTransposeNarrowKernel<ValT, AccT>), dim3(GridFor(numTiles, tilesPerBlock)),
-                           dim3(kBlockThreads), 0, a.stream, a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
-                           static_cast<const ValT *>(a.x), acc, a.rows, a.cols, a.nnz, tilesPerBlock, a.alpha);
+        auto narrow = a.cols <= kNarrowCols / 2 ? SpmvTransposeNarrowKernel<ValT, AccT, kNarrowCols / 2>
+                                                : SpmvTransposeNarrowKernel<ValT, AccT, kNarrowCols>;
+        hipLaunchKernelGGL(narrow, dim3(GridFor(numTiles, tilesPerBlock)), dim3(kBlockThreads), 0, a.stream,
+                           a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
+                           acc, a.rows, a.cols, a.nnz, tilesPerBlock, a.alpha);
         return finish();
     }
     if (skewedRows && a.nnz >= 8 * kTransposeTile) {
