@@ -596,3 +596,20 @@ def test_transpose_few_columns_accumulates_per_workgroup(osa, gpu_ctx, rows, col
         assert (d <= 2.0 ** -16 + 2.0 ** -10 * np.abs(gold)).mean() >= 0.99 and d.max() <= 1e-2
         if cols <= 16384:
             assert d.max() <= 1e-4 * max(1.0, float(np.abs(gold).max()))
+
+
+@pytest.mark.parametrize("prepared", [True, False])
+def test_rows_through_hundreds_of_merge_workgroups(osa, gpu_ctx, prepared):
+    """Rows of 1.2 M, 140 000 and 131 entries between short ones: the long ones pass through 590 and 69 merge
+    workgroups, whose carries the fix-up adds with a whole wavefront; the third through one or two (one lane)."""
+    rng = np.random.default_rng(77)
+    rows, cols = 30_000, 2_000_000
+    lengths = rng.integers(0, 7, rows)
+    lengths[[0, 12_345, 29_999]] = [140_000, 1_200_000, 131]
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    x, y0 = rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+    y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, -1.5, 0.25, preprocess=prepared)
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, -1.5, 0.25)
+    assert oracle.max_rel_err(y, gold) <= 1e-5
