@@ -865,7 +865,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvPanelCombineKernel(const Ac
 template <typename ValT, typename AccT, int G>
 __global__ __launch_bounds__(kBlockThreads) void SpmvTransposeScatterKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
-    const ValT *__restrict__ x, float *__restrict__ y, int64_t rows, OpsparseScalar alphaS)
+    const ValT *__restrict__ x, float *__restrict__ y, int64_t rows, int32_t maxLen, OpsparseScalar alphaS)
 {
     const AccT alpha = ReadScalar<AccT>(alphaS);
     constexpr int kGroups = kBlockThreads / G;
@@ -878,8 +878,49 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvTransposeScatterKernel(
         return;
     }
     const int32_t e = rowOffsets[r + 1];
+    if (e - rowOffsets[r] > maxLen) {
+        return;  // left to SpmvTransposeLongRowsKernel
+    }
     for (int64_t k = static_cast<int64_t>(rowOffsets[r]) + threadIdx.x % G; k < e; k += G) {
         atomicAdd(y + LoadStream(colInd + k), static_cast<float>(ax * ToAcc<AccT>(LoadStream(vals + k))));
+    }
+}
+
+// The rows the scatter kernel skipped (longer than minLen): a workgroup looks at 256 consecutive rows, lists the
+// long ones among them in LDS and walks each of them with all its lanes.  With it a lane group is never left alone
+// with a row of thousands of entries, and nothing has to be searched for: a matrix of short rows with a few long
+// ones costs one more pass over the row offsets.
+template <typename ValT, typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmvTransposeLongRowsKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ x, float *__restrict__ y, int64_t rows, int32_t minLen, OpsparseScalar alphaS)
+{
+    __shared__ int32_t listed[kBlockThreads];
+    __shared__ int32_t numListed;
+    if (threadIdx.x == 0) {
+        numListed = 0;
+    }
+    __syncthreads();
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
+    if (r < rows && rowOffsets[r + 1] - rowOffsets[r] > minLen) {
+        listed[atomicAdd(&numListed, 1)] = static_cast<int32_t>(threadIdx.x);
+    }
+    __syncthreads();
+    const int32_t count = numListed;
+    if (count == 0) {
+        return;
+    }
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    for (int32_t i = 0; i < count; ++i) {
+        const int64_t row = static_cast<int64_t>(blockIdx.x) * kBlockThreads + listed[i];
+        const AccT ax = alpha * ToAcc<AccT>(x[row]);
+        if (ax == AccT(0)) {
+            continue;
+        }
+        const int64_t e = rowOffsets[row + 1];
+        for (int64_t k = static_cast<int64_t>(rowOffsets[row]) + threadIdx.x; k < e; k += kBlockThreads) {
+            atomicAdd(y + LoadStream(colInd + k), static_cast<float>(ax * ToAcc<AccT>(LoadStream(vals + k))));
+        }
     }
 }
 
@@ -898,6 +939,8 @@ __device__ __forceinline__ int64_t RowOfEntry(const int32_t *offsets, int64_t lo
 }
 
 constexpr int kTransposeTile = 2048;      // entries per workgroup
+constexpr int kTransposeFewRows = 8192;   // fewer rows than this: split by entries instead of by rows
+constexpr int kTransposeLongRow = 512;    // a row longer than this is walked by a whole workgroup
 constexpr int kTransposeRowSlots = 2304;  // row offsets of one tile staged in LDS
 
 // The same product with equal numbers of ENTRIES per workgroup, whatever the row lengths: a tile of
@@ -1374,20 +1417,30 @@ int RunTranspose(const SpmvArgs &a, int32_t outType, bool skewedRows)
                            acc, a.rows, a.cols, a.nnz, tilesPerBlock, a.alpha);
         return finish();
     }
-    if (skewedRows && a.nnz >= 8 * kTransposeTile) {
-        // equal entries per workgroup: no lane group is left walking a long row on its own
+    if (a.rows < kTransposeFewRows && a.nnz >= 8 * kTransposeTile) {
+        // too few rows to occupy the GPU with a lane group each (ten rows of 2 M entries: 17 ms that way, 0.3 ms
+        // here): equal entries per workgroup, the row of an entry looked up in the few offsets there are
         hipLaunchKernelGGL((SpmvTransposeFlatKernel<ValT, AccT>), dim3(GridFor(a.nnz, kTransposeTile)),
                            dim3(kBlockThreads), 0, a.stream, a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
                            static_cast<const ValT *>(a.x), acc, a.rows, a.nnz, a.alpha);
         return finish();
     }
+    // Rows far longer than the mean: the lane groups take the rows up to kTransposeLongRow entries, whole
+    // workgroups the others.
+    const int32_t maxLen = skewedRows ? kTransposeLongRow : INT32_MAX;
     const int32_t g = VectorLanesFor(a.rows, a.nnz);
     auto launch = [&](auto tag) {
         constexpr int G = decltype(tag)::value;
         hipLaunchKernelGGL((SpmvTransposeScatterKernel<ValT, AccT, G>), dim3(GridFor(a.rows, kBlockThreads / G)),
                            dim3(kBlockThreads), 0, a.stream, a.rowOffsets, a.colInd,
                            static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
-                           acc, a.rows, a.alpha);
+                           acc, a.rows, maxLen, a.alpha);
+        if (skewedRows) {
+            hipLaunchKernelGGL((SpmvTransposeLongRowsKernel<ValT, AccT>), dim3(GridFor(a.rows, kBlockThreads)),
+                               dim3(kBlockThreads), 0, a.stream, a.rowOffsets, a.colInd,
+                               static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x), acc, a.rows, maxLen,
+                               a.alpha);
+        }
     };
     switch (g) {
         case 4: launch(std::integral_constant<int, 4>{}); break;
