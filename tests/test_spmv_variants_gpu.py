@@ -613,3 +613,22 @@ def test_rows_through_hundreds_of_merge_workgroups(osa, gpu_ctx, prepared):
     y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, -1.5, 0.25, preprocess=prepared)
     gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, -1.5, 0.25)
     assert oracle.max_rel_err(y, gold) <= 1e-5
+
+
+def test_transpose_few_long_rows_split_by_entries(osa, gpu_ctx):
+    """Fifty rows of thousands of entries onto 200 000 columns: too few rows for a lane group each, the entries are
+    dealt out 2048 to a workgroup and the row of an entry is looked up in the offsets (some rows empty)."""
+    rng = np.random.default_rng(5)
+    rows, cols = 50, 200_000
+    lengths = rng.integers(2_000, 9_000, rows)
+    lengths[[0, 17, 49]] = 0
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    x, y0 = rng.uniform(-1, 1, rows).astype(np.float32), rng.uniform(-1, 1, cols).astype(np.float32)
+    for prep in (True, False):
+        y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 1.5, -0.5, preprocess=prep,
+                     op=osa.ACL_SPARSE_OP_TRANSPOSE)
+        gold = oracle.spmv_trans_f64(rows, cols, rowptr, colind, val, x, y0, 1.5, -0.5)
+        d = np.abs(y - gold)
+        assert (d <= 2.0 ** -16 + 2.0 ** -10 * np.abs(gold)).mean() >= 0.99 and d.max() <= 1e-2
