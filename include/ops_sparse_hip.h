@@ -87,6 +87,9 @@ typedef struct OpsparseSpmvPlan {
     int32_t guardTiles;    /* STREAM_ROWS: the row offsets may have changed since the analysis: a tile with more
                               entries than its LDS was sized for is summed from memory instead (set by callers
                               that keep a plan without the user having asked for one; 0 after analyse) */
+    int32_t tileRowNnz;    /* STREAM_ROWS: the row length the tiles are sized for (0: maxRowNnz) */
+    int32_t longRowsBeside;/* STREAM_ROWS: a few rows are longer than that: the tiles skip rows of more than 64
+                              entries and a second kernel sums those, a workgroup per row */
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */

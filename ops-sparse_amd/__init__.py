@@ -114,7 +114,7 @@ class OpsparseSpmvPlan(ctypes.Structure):
     _fields_ = [("kernel", i32), ("lanesPerRow", i32), ("rowsPerBlock", i32), ("mergeBlocks", i32),
                 ("maxRowNnz", i32), ("partitionReady", i32), ("numPanels", i32),
                 ("panelShift", i32), ("numRowBlocks", i32), ("entryWindow", i32), ("transposed", i32),
-                ("guardTiles", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
+                ("guardTiles", i32), ("tileRowNnz", i32), ("longRowsBeside", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
                 ("carryOff", i64), ("headOff", i64), ("bytes", i64), ("panelStart", i64 * 17)]
 
 

@@ -109,23 +109,44 @@ __global__ __launch_bounds__(kBlockThreads) void ConvertFromFloatKernel(OutT *__
 
 // ------------------------------------------------------------- row statistics
 
-// stats[0] = max row length.  stats must be zeroed before the launch.
+constexpr int kStreamMaxRow = 48;   // the stream-rows tiles are sized for rows up to this long
+constexpr int kBesideRow = 64;      // with SpmvLongRowsKernel beside them, the stream-rows kernels skip longer rows
+constexpr int kBesideMaxRow = 8192; // ... which one workgroup sums: beyond this length the merge path is the better answer
+
+// stats[0] = longest row, stats[1] = longest row of at most kStreamMaxRow entries, stats[2] = number of longer
+// rows, stats[3] = their entries.  stats must be zeroed before the launch.
 __global__ __launch_bounds__(kBlockThreads) void RowStatsKernel(const int32_t *__restrict__ rowOffsets, int64_t rows,
                                                                 int32_t *__restrict__ stats)
 {
-    int32_t best = 0;
+    int32_t best = 0, bestShort = 0, numLong = 0;
+    uint32_t nnzLong = 0;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kBlockThreads;
     for (int64_t r = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; r < rows; r += stride) {
         const int32_t len = rowOffsets[r + 1] - rowOffsets[r];
         best = len > best ? len : best;
+        if (len <= kStreamMaxRow) {
+            bestShort = len > bestShort ? len : bestShort;
+        } else {
+            ++numLong;
+            nnzLong += static_cast<uint32_t>(len);
+        }
     }
 #pragma unroll
     for (int off = kWave / 2; off > 0; off >>= 1) {
         const int32_t other = __shfl_xor(best, off, kWave);
         best = other > best ? other : best;
+        const int32_t otherShort = __shfl_xor(bestShort, off, kWave);
+        bestShort = otherShort > bestShort ? otherShort : bestShort;
+        numLong += __shfl_xor(numLong, off, kWave);
+        nnzLong += __shfl_xor(nnzLong, off, kWave);
     }
     if ((threadIdx.x & (kWave - 1)) == 0 && best > 0) {
         atomicMax(stats, best);
+        atomicMax(stats + 1, bestShort);
+        if (numLong > 0) {
+            atomicAdd(stats + 2, numLong);
+            atomicAdd(reinterpret_cast<uint32_t *>(stats) + 3, nnzLong);
+        }
     }
 }
 
@@ -248,7 +269,7 @@ template <typename ValT, typename OutT, typename AccT, int G, int U>
 __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
     const ValT *__restrict__ x, OutT *y, const OutT *yIn, int64_t rows, int32_t rowsPerBlock, int32_t capacity,
-    OpsparseScalar alphaS, OpsparseScalar betaS)
+    int32_t skipLonger, OpsparseScalar alphaS, OpsparseScalar betaS)
 {
     extern __shared__ __align__(16) unsigned char ldsRaw[];
     AccT *prod = reinterpret_cast<AccT *>(ldsRaw);
@@ -326,7 +347,10 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
                 }
             }
             AccT sum = AccT(0);
-            if (staged) {
+            // skipLonger > 0: rows longer than that are SpmvLongRowsKernel's, which runs after this kernel
+            const bool skip = skipLonger > 0 && e - s > skipLonger;
+            if (skip) {
+            } else if (staged) {
                 for (int32_t k = s - first + lane; k < e - first; k += G) {
                     sum += prod[k];
                 }
@@ -336,7 +360,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
                 }
             }
             sum = GroupSum<G>(sum);
-            if (lane == 0) {
+            if (lane == 0 && !skip) {
                 AccT res = alpha * sum;
                 if (!betaZero) {
                     res += beta * yOld;
@@ -370,9 +394,12 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
 template <typename ValT, typename AccT, int U, bool GuardTiles>
 __global__ __launch_bounds__(kBlockThreads) void SpmvStreamQuadRowsKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
-    const ValT *__restrict__ x, float *y, const float *yIn, int64_t rows, int32_t rowsPerBlock, int32_t capacity,
+    const ValT *__restrict__ x, float *y, const float *yIn, int64_t rows, int32_t rowsPerBlock, int32_t guard,
     OpsparseScalar alphaS, OpsparseScalar betaS)
 {
+    // guard (read by the GuardTiles instantiation only): the products the LDS of this launch holds in its low 16
+    // bits, above them the row length beyond which rows are left to SpmvLongRowsKernel (0: none)
+    const int32_t capacity = guard & 0xffff, skipLonger = guard >> 16;
     typedef int32_t Int4A __attribute__((ext_vector_type(4)));
     typedef float Float4A __attribute__((ext_vector_type(4)));
     extern __shared__ __align__(16) unsigned char ldsRaw[];
@@ -422,6 +449,9 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamQuadRowsKernel(
         // the row offsets changed since.  The tile is summed straight from memory.  (A flag of the instantiation:
         // the test alone costs the 2048 x 2048 Laplacian 0.5 us of 41.)
         for (int32_t i = 0; i < mine; ++i) {
+            if (skipLonger > 0 && bound[i + 1] - bound[i] > skipLonger) {
+                continue;  // SpmvLongRowsKernel's, which runs after this kernel
+            }
             AccT sum = AccT(0);
             for (int32_t k = bound[i]; k < bound[i + 1]; ++k) {
                 sum += ToAcc<AccT>(vals[k]) * ToAcc<AccT>(x[colInd[k]]);
@@ -455,6 +485,10 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamQuadRowsKernel(
             res += beta * static_cast<AccT>(yOld[i]);
         }
         out[i] = static_cast<float>(res);
+        if (GuardTiles && skipLonger > 0 && i < mine && bound[i + 1] - bound[i] > skipLonger) {
+            // a long row inside a tile that fitted: SpmvLongRowsKernel's; y keeps what it held (beta == 0: anything)
+            out[i] = betaZero ? 0.0f : yOld[i];
+        }
     }
     if (mine == 4) {
         Float4A o;
@@ -466,6 +500,109 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamQuadRowsKernel(
     } else {
         for (int32_t i = 0; i < mine; ++i) {
             y[r + i] = out[i];
+        }
+    }
+}
+
+// The rows the stream-rows kernels skipped (longer than minLen), for matrices of short rows with a few long ones
+// among them — a mesh with some dense constraint rows, a graph with a few hubs: a workgroup looks at 256
+// consecutive rows, lists the long ones in LDS and sums each of them with all its lanes, in fp64, in a fixed order.
+constexpr int kLongScanRows = 16;   // rows a lane looks at in SpmvLongRowsKernel's first pass (at most 32: a bit each)
+
+template <typename ValT, typename OutT, typename AccT>
+__global__ __launch_bounds__(kBlockThreads) void SpmvLongRowsKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ x, OutT *y, const OutT *yIn, int64_t rows, int32_t minLen, OpsparseScalar alphaS,
+    OpsparseScalar betaS)
+{
+    constexpr int kWaves = kBlockThreads / kWave;
+    constexpr int64_t kSpan = static_cast<int64_t>(kBlockThreads) * kLongScanRows;  // rows of one workgroup
+    __shared__ int32_t listed[kBlockThreads];
+    __shared__ int32_t numListed;
+    __shared__ AccT waveSum[kWaves];
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const int64_t span0 = static_cast<int64_t>(blockIdx.x) * kSpan;
+    // Coarse pass: is any of this workgroup's rows long?  Nearly always not, and the workgroup is done after
+    // reading its offsets once.
+    __shared__ uint32_t groupsWithLong;  // bit i: a long row among rows span0 + 256 i ... + 255
+    if (threadIdx.x == 0) {
+        groupsWithLong = 0;
+    }
+    __syncthreads();
+    uint32_t mine = 0;  // bit i: row span0 + 256 i + threadIdx.x is long (neighbouring rows in neighbouring lanes)
+#pragma unroll
+    for (int i = 0; i < kLongScanRows; ++i) {
+        const int64_t r = span0 + static_cast<int64_t>(i) * kBlockThreads + threadIdx.x;
+        if (r < rows && rowOffsets[r + 1] - rowOffsets[r] > minLen) {
+            mine |= 1u << i;
+        }
+    }
+    if (mine != 0) {
+        atomicOr(&groupsWithLong, mine);
+    }
+    __syncthreads();
+    const AccT alpha = ReadScalar<AccT>(alphaS), beta = ReadScalar<AccT>(betaS);
+    for (uint32_t todo = groupsWithLong; todo != 0; todo &= todo - 1) {
+        const int g = __ffs(static_cast<int>(todo)) - 1;
+        const int64_t base = span0 + static_cast<int64_t>(g) * kBlockThreads;
+        const bool isLong = (mine >> g) & 1u;
+        if (threadIdx.x == 0) {
+            numListed = 0;
+        }
+        __syncthreads();
+        // listed in row order (a ballot per wavefront, the wavefronts one after the other), so that nothing about
+        // the result depends on the order in which lanes arrive
+        const uint64_t votes = __ballot(isLong);
+        for (int w = 0; w < kWaves; ++w) {
+            if (w == wave && isLong) {
+                listed[numListed + __popcll(votes & ((uint64_t{1} << lane) - 1))] = static_cast<int32_t>(threadIdx.x);
+            }
+            __syncthreads();
+            if (w == wave && lane == 0) {
+                numListed += __popcll(votes);
+            }
+            __syncthreads();
+        }
+        const int32_t count = numListed;
+        for (int32_t i = 0; i < count; ++i) {
+            const int64_t row = base + listed[i];
+            const int64_t e = rowOffsets[row + 1];
+            // four entries per lane and round, loaded unconditionally (past the end: the last entry again, counted
+            // as zero), so that four gathers are in flight: one workgroup is alone with this row
+            AccT part[4] = {AccT(0), AccT(0), AccT(0), AccT(0)};
+            for (int64_t k = static_cast<int64_t>(rowOffsets[row]) + threadIdx.x; k < e; k += 4 * kBlockThreads) {
+                int32_t c[4];
+                AccT v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int64_t ku = k + static_cast<int64_t>(u) * kBlockThreads;
+                    const int64_t at = ku < e ? ku : e - 1;
+                    c[u] = LoadStream(colInd + at);
+                    v[u] = ku < e ? ToAcc<AccT>(LoadStream(vals + at)) : AccT(0);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    part[u] += v[u] * ToAcc<AccT>(x[c[u]]);
+                }
+            }
+            AccT sum = (part[0] + part[1]) + (part[2] + part[3]);
+#pragma unroll
+            for (int off = kWave / 2; off > 0; off >>= 1) {
+                sum += __shfl_xor(sum, off, kWave);
+            }
+            if (lane == 0) {
+                waveSum[wave] = sum;
+            }
+            __syncthreads();
+            if (threadIdx.x == 0) {
+                AccT total = waveSum[0];
+#pragma unroll
+                for (int w = 1; w < kWaves; ++w) {
+                    total += waveSum[w];
+                }
+                StoreRow<OutT, AccT>(y, yIn, row, total, alpha, beta, beta == AccT(0));
+            }
+            __syncthreads();
         }
     }
 }
@@ -1095,7 +1232,7 @@ MergeLayout MakeMergeLayout(int64_t rows, int64_t nnz)
 }
 
 template <typename ValT, typename OutT, typename AccT, int G, int U>
-int LaunchStreamU(const SpmvArgs &a, int32_t rowsPerBlock, size_t lds)
+int LaunchStreamU(const SpmvArgs &a, int32_t rowsPerBlock, size_t lds, int32_t skipLonger)
 {
     // Persistent launch: a few workgroups per CU walk over all tiles.
     const uint32_t tiles = GridFor(a.rows, rowsPerBlock);
@@ -1104,15 +1241,15 @@ int LaunchStreamU(const SpmvArgs &a, int32_t rowsPerBlock, size_t lds)
     hipLaunchKernelGGL((SpmvStreamRowsKernel<ValT, OutT, AccT, G, U>), dim3(grid), dim3(kBlockThreads), lds, a.stream,
                        a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
                        static_cast<OutT *>(a.y), static_cast<const OutT *>(a.yIn), a.rows, rowsPerBlock,
-                       static_cast<int32_t>(lds / sizeof(AccT)), a.alpha, a.beta);
+                       static_cast<int32_t>(lds / sizeof(AccT)), skipLonger, a.alpha, a.beta);
     return CheckLaunch();
 }
 
 template <typename ValT, typename OutT, typename AccT, int G>
-int LaunchStream(const SpmvArgs &a, int32_t rowsPerBlock, int32_t maxRowNnz, bool guardTiles)
+int LaunchStreamTiles(const SpmvArgs &a, int32_t rowsPerBlock, int32_t tileRowNnz, bool guardTiles, int32_t skipLonger)
 {
     // LDS for the worst case of this block shape; the issue depth U covers it in one round.
-    const size_t products = static_cast<size_t>(rowsPerBlock) * static_cast<size_t>(maxRowNnz);
+    const size_t products = static_cast<size_t>(rowsPerBlock) * static_cast<size_t>(tileRowNnz);
     const size_t lds = products * sizeof(AccT);
     if constexpr (G == 1 && std::is_same<OutT, float>::value) {
         // Four rows per lane with vector row offsets / y where the shapes allow it.
@@ -1128,7 +1265,7 @@ int LaunchStream(const SpmvArgs &a, int32_t rowsPerBlock, int32_t maxRowNnz, boo
                 hipLaunchKernelGGL(kernel, dim3(grid), dim3(kBlockThreads), lds, a.stream, a.rowOffsets, a.colInd,
                                    static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
                                    static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.rows, rowsPerBlock,
-                                   static_cast<int32_t>(products), a.alpha, a.beta);
+                                   static_cast<int32_t>(products) | (skipLonger << 16), a.alpha, a.beta);
             };
             if (products <= kBlockThreads * 4) {
                 launch(std::integral_constant<int, 1>{});
@@ -1140,9 +1277,29 @@ int LaunchStream(const SpmvArgs &a, int32_t rowsPerBlock, int32_t maxRowNnz, boo
             return CheckLaunch();
         }
     }
-    if (products <= kBlockThreads * 4) return LaunchStreamU<ValT, OutT, AccT, G, 1>(a, rowsPerBlock, lds);
-    if (products <= kBlockThreads * 8) return LaunchStreamU<ValT, OutT, AccT, G, 2>(a, rowsPerBlock, lds);
-    return LaunchStreamU<ValT, OutT, AccT, G, 3>(a, rowsPerBlock, lds);
+    if (products <= kBlockThreads * 4) return LaunchStreamU<ValT, OutT, AccT, G, 1>(a, rowsPerBlock, lds, skipLonger);
+    if (products <= kBlockThreads * 8) return LaunchStreamU<ValT, OutT, AccT, G, 2>(a, rowsPerBlock, lds, skipLonger);
+    return LaunchStreamU<ValT, OutT, AccT, G, 3>(a, rowsPerBlock, lds, skipLonger);
+}
+
+// The stream-rows family for a plan: the tiles, and the long rows beside them where the plan says so.
+template <typename ValT, typename OutT, typename AccT, int G>
+int LaunchStream(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
+{
+    const bool beside = plan.longRowsBeside != 0;
+    const int32_t tileRowNnz = plan.tileRowNnz > 0 ? plan.tileRowNnz : plan.maxRowNnz;
+    // with long rows beside, the tiles must be guarded: a tile that holds one does not fit its LDS
+    int rc = LaunchStreamTiles<ValT, OutT, AccT, G>(a, plan.rowsPerBlock, tileRowNnz, plan.guardTiles != 0 || beside,
+                                                    beside ? kBesideRow : 0);
+    if (rc == OPSPARSE_OK && beside) {
+        hipLaunchKernelGGL((SpmvLongRowsKernel<ValT, OutT, AccT>),
+                           dim3(GridFor(a.rows, static_cast<int64_t>(kBlockThreads) * kLongScanRows)),
+                           dim3(kBlockThreads), 0, a.stream, a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
+                           static_cast<const ValT *>(a.x), static_cast<OutT *>(a.y), static_cast<const OutT *>(a.yIn),
+                           a.rows, kBesideRow, a.alpha, a.beta);
+        rc = CheckLaunch();
+    }
+    return rc;
 }
 
 template <typename ValT, typename OutT, typename AccT, int G>
@@ -1201,10 +1358,10 @@ int RunPlanned(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
                                            a.stream);
         case OPSPARSE_SPMV_STREAM_ROWS:
             switch (plan.lanesPerRow) {
-                case 1: return LaunchStream<ValT, OutT, AccT, 1>(a, plan.rowsPerBlock, plan.maxRowNnz, plan.guardTiles != 0);
-                case 2: return LaunchStream<ValT, OutT, AccT, 2>(a, plan.rowsPerBlock, plan.maxRowNnz, plan.guardTiles != 0);
-                case 4: return LaunchStream<ValT, OutT, AccT, 4>(a, plan.rowsPerBlock, plan.maxRowNnz, plan.guardTiles != 0);
-                case 8: return LaunchStream<ValT, OutT, AccT, 8>(a, plan.rowsPerBlock, plan.maxRowNnz, plan.guardTiles != 0);
+                case 1: return LaunchStream<ValT, OutT, AccT, 1>(a, plan);
+                case 2: return LaunchStream<ValT, OutT, AccT, 2>(a, plan);
+                case 4: return LaunchStream<ValT, OutT, AccT, 4>(a, plan);
+                case 8: return LaunchStream<ValT, OutT, AccT, 8>(a, plan);
                 default: return OPSPARSE_E_INVALID;
             }
         case OPSPARSE_SPMV_VECTOR_ROWS:
@@ -1508,11 +1665,13 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
     grid = grid > 4096 ? 4096 : grid;
     hipLaunchKernelGGL(RowStatsKernel, dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0, s, rowOffsets, rows,
                        stats);
-    int32_t maxRow = 0;
-    if (hipMemcpyAsync(&maxRow, stats, sizeof(int32_t), hipMemcpyDeviceToHost, s) != hipSuccess ||
+    int32_t seen[4] = {0, 0, 0, 0};  // longest row, longest of the short rows, rows longer than those, their entries
+    if (hipMemcpyAsync(seen, stats, sizeof(seen), hipMemcpyDeviceToHost, s) != hipSuccess ||
         hipStreamSynchronize(s) != hipSuccess) {
         return OPSPARSE_E_LAUNCH;
     }
+    const int32_t maxRow = seen[0], maxShort = seen[1], numLong = seen[2];
+    const int64_t nnzShort = nnz - static_cast<int64_t>(static_cast<uint32_t>(seen[3]));
     p.maxRowNnz = maxRow;
 
     const double mean = static_cast<double>(nnz) / static_cast<double>(rows);
@@ -1523,9 +1682,20 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
         // short (mean 16 - 48 even: 160 - 173 us against 195 - 200 us for the merge path; varied: 217 - 222 us
         // against 194 - 199 us); a lane group per row only pays for long rows of nearly equal length (mean 128 -
         // 256: 180 us against 195 us; varied rows 250 - 350 us against 189 us); the merge path does not care.
-        if (maxRow <= 48 && (maxRow <= 12 || static_cast<double>(maxRow) * static_cast<double>(rows) <=
-                                                 1.25 * static_cast<double>(nnz))) {
+        if (maxRow <= kStreamMaxRow && (maxRow <= 12 || static_cast<double>(maxRow) * static_cast<double>(rows) <=
+                                                            1.25 * static_cast<double>(nnz))) {
             kernel = OPSPARSE_SPMV_STREAM_ROWS;
+        } else if (maxRow > kStreamMaxRow && maxRow <= kBesideMaxRow && maxShort >= 1 && numLong <= 4096 &&
+                   static_cast<int64_t>(numLong) * 1024 <= rows &&
+                   (maxShort <= 12 || static_cast<double>(maxShort) * static_cast<double>(rows) <=
+                                          1.25 * static_cast<double>(nnzShort))) {
+            // Short rows with a few long ones among them (at most one row in a thousand, 4096 in all: a mesh with
+            // dense constraint rows, a graph with a few hubs): the stream-rows tiles sized for the short rows, the
+            // long rows summed beside them by a workgroup each (2048 x 2048 mesh with 11 rows of 3000 entries:
+            // 47 us, against 91 us for the merge path the longest row would otherwise call for).
+            kernel = OPSPARSE_SPMV_STREAM_ROWS;
+            p.longRowsBeside = 1;
+            p.tileRowNnz = maxShort;
         } else if (mean >= 96.0 && mean <= 400.0 && static_cast<double>(maxRow) <= 1.125 * mean) {
             kernel = OPSPARSE_SPMV_VECTOR_ROWS;
         } else {
@@ -1535,21 +1705,24 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
     p.kernel = kernel;
     switch (kernel) {
         case OPSPARSE_SPMV_STREAM_ROWS: {
-            if (maxRow > 48) {
+            // the row length the tiles are sized for: the longest row, or the longest short one with the rest beside
+            const int32_t tileRow = p.longRowsBeside ? p.tileRowNnz : maxRow;
+            if (tileRow > kStreamMaxRow) {
                 return OPSPARSE_E_UNSUPPORTED;  // products of a row block would not fit LDS
             }
-            const int32_t g = maxRow <= 12 ? 1 : (maxRow <= 24 ? 2 : 4);
+            p.tileRowNnz = tileRow;
+            const int32_t g = tileRow <= 12 ? 1 : (tileRow <= 24 ? 2 : 4);
             p.lanesPerRow = g;
             // As many rows as keep the tile's worst-case products within two full
             // rounds of the workgroup's loads (2 x 1024 entries, 16 KiB of LDS):
             // measured best when a tile nearly fills whole rounds.
-            int32_t rpb = 2048 / maxRow;
+            int32_t rpb = 2048 / tileRow;
             rpb = rpb > 512 ? 512 : rpb;
             rpb &= ~3;  // whole groups of four rows for the vectorised y path
             p.rowsPerBlock = rpb < 4 ? 4 : rpb;
             if (const char *env = std::getenv("OPS_SPARSE_STREAM_ROWS")) {
                 const int v = std::atoi(env);  // tuning override
-                if (v >= 1 && static_cast<int64_t>(v) * maxRow <= 3072) {
+                if (v >= 1 && static_cast<int64_t>(v) * tileRow <= 3072) {
                     p.rowsPerBlock = v;
                 }
             }

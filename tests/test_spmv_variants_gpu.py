@@ -632,3 +632,47 @@ def test_transpose_few_long_rows_split_by_entries(osa, gpu_ctx):
         gold = oracle.spmv_trans_f64(rows, cols, rowptr, colind, val, x, y0, 1.5, -0.5)
         d = np.abs(y - gold)
         assert (d <= 2.0 ** -16 + 2.0 ** -10 * np.abs(gold)).mean() >= 0.99 and d.max() <= 1e-2
+
+
+@pytest.mark.parametrize("short,out_dtype,prepared", [(5, None, True), (5, None, False), (20, None, True),
+                                                      (7, torch.float16, True), (40, None, False)])
+def test_short_rows_with_a_few_long_ones_beside(osa, gpu_ctx, short, out_dtype, prepared):
+    """A banded matrix of short rows with a handful of long ones (65 - 8192 entries, some next to each other, one
+    the first row, one the last): the stream-rows tiles are sized for the short rows and skip the long ones,
+    which a second kernel sums with a workgroup each.  Every row must be written exactly once — in place with
+    beta != 0 a second write would show.  Rows of 49 - 64 entries are too long for the tiles' sizing but not
+    skipped: their tiles are summed from memory."""
+    rng = np.random.default_rng(short)
+    rows = cols = 300_000
+    lengths = rng.integers(max(1, short - 3), short + 1, rows)
+    lengths[rng.choice(rows, 40, replace=False)] = 0
+    long_rows = np.array([0, 1, 2, 77_000, 150_000, 150_001, 299_999])
+    lengths[long_rows] = [65, 3000, 8192, 512, 513, 8_000, 700]
+    lengths[[5_000, 5_001, 250_000]] = [49, 64, 60]
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    centre = np.repeat(np.arange(rows), lengths)
+    colind = np.clip(centre + rng.integers(-3000, 3001, centre.size), 0, cols - 1).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    x, y0 = rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+    if out_dtype is not None:
+        val, x, y0 = _round(val, out_dtype), _round(x, out_dtype), _round(y0, out_dtype)
+    if prepared:
+        plan = osa.OpsparseSpmvPlan()
+        dev, stream, handle = gpu_ctx
+        d_rp = to_dev(rowptr, dev)
+        L = osa.lib()
+        ws = torch.empty(max(L.opsparse_spmv_csr_workspace_bytes(rows, colind.size), 256), dtype=torch.uint8, device=dev)
+        assert L.opsparse_spmv_csr_analyse(d_rp.data_ptr(), rows, cols, colind.size, ws.data_ptr(), ws.numel(),
+                                           osa.OPSPARSE_SPMV_AUTO, ctypes.byref(plan),
+                                           ctypes.c_void_p(stream.cuda_stream)) == 0
+        assert plan.kernel == osa.OPSPARSE_SPMV_STREAM_ROWS and plan.longRowsBeside == 1
+        assert plan.tileRowNnz == short and plan.maxRowNnz == 8192
+    for alpha, beta in ((1.5, 0.5), (2.0, 0.0)):
+        y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, alpha, beta, preprocess=prepared,
+                     val_dtype=out_dtype, out_dtype=out_dtype)
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, alpha, beta)
+        if out_dtype is None:
+            assert oracle.max_rel_err(y, gold) <= 1e-5
+        else:
+            want = _round(gold, out_dtype)
+            assert np.all(np.abs(y - want) <= 2.0 ** -10 * np.maximum(np.abs(want), 2.0 ** -14))
