@@ -581,6 +581,17 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmLongFixupKernel(
         AccT sum = AccT(0);
         if (col < n) {
             int64_t seg = mine0;
+            for (; seg + 16 <= mine1; seg += 16) {  // a row of thousands of segments: sixteen loads in flight
+                AccT p[16];
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    p[u] = partial[(seg + u) * n + col];
+                }
+#pragma unroll
+                for (int u = 0; u < 16; ++u) {
+                    sum += p[u];  // added in segment order
+                }
+            }
             for (; seg + 4 <= mine1; seg += 4) {  // four loads in flight, added in order
                 const AccT p0 = partial[(seg + 0) * n + col];
                 const AccT p1 = partial[(seg + 1) * n + col];
