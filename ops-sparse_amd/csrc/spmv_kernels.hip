@@ -10,15 +10,25 @@
 //                fixed block of consecutive rows, loads their contiguous
 //                (colind, value) range with full-width coalesced non-temporal
 //                loads, gathers x, parks the products in LDS and then lets
-//                1..8 lanes per row add them up in stored order.
-//   VECTOR_ROWS  medium rows: a group of 4..64 lanes strides along one row and
-//                reduces with cross-lane shuffles.  Needs no workspace.
-//   MERGE_PATH   skewed (power-law) rows: the merge of "row ends" and "non-zero
-//                indices" is cut into equal pieces, so every workgroup gets the
-//                same rows + nnz whatever the row lengths are.  Products are
-//                staged in LDS as above; a row cut by a workgroup boundary
-//                leaves a carry-out, and a small fix-up kernel adds the pieces
-//                in ascending order, so the result is deterministic.
+//                1..8 lanes per row add them up in stored order.  A few long
+//                rows among short ones are left out by the tiles and summed
+//                beside them, a workgroup per row (SpmvLongRowsKernel).
+//   VECTOR_ROWS  long rows of nearly equal length: a group of 4..64 lanes
+//                strides along one row and reduces with cross-lane shuffles.
+//                Needs no workspace.
+//   MERGE_PATH   everything else (power-law rows, rows of varying length): the
+//                merge of "row ends" and "non-zero indices" is cut into equal
+//                pieces, so every workgroup gets the same rows + nnz whatever
+//                the row lengths are.  Products are staged in LDS as above; a
+//                row cut by a workgroup boundary leaves a carry-out, and a
+//                small fix-up kernel adds the pieces in a fixed order, so the
+//                result is deterministic.
+//
+// The family is chosen per matrix from row statistics (opsparse_spmv_csr_analyse,
+// where the measurements behind the rule are quoted).  op(A) = A^T has its own
+// kernels further down: fp32 atomics per entry like the reference, per-workgroup
+// sums in LDS when y is short, whole workgroups for long rows, an entry-split
+// kernel when the rows are few.
 //
 // Memory traffic per launch is the compulsory nnz*(sizeof(val)+4) +
 // (rows+1)*4 + rows*sizeof(y)*(1 + [beta != 0]) plus x: the kernels are
