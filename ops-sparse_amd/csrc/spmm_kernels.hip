@@ -25,7 +25,11 @@
 //
 // Floating-point products are accumulated in fp64 in stored order and rounded
 // once, int8 products in int32 with an int64 saturating epilogue
-// (spmm_kernel.cpp:251-266).
+// (spmm_kernel.cpp:251-266); int8 runs the same kernels with 8 (narrow B: 4)
+// bytes of B per lane.  Operands in other layouts — column-major, op(B) = B^T,
+// widths or leading dimensions that are not whole vectors — reach these kernels
+// as row-major copies staged in the SpMM buffer (DenseRestageKernel, driven by
+// spmm_host.cpp); what cannot be staged runs SpmmGeneralKernel in place.
 #include <climits>
 #include <cstdlib>
 #include <type_traits>

@@ -7,8 +7,12 @@
 // m == 0 / nnz == 0 short cuts of :465-486).  What differs is underneath: the
 // reference runs one thread per row with a compensated dot product and, for
 // ALG2, a device-side sort of the rows; here every algorithm value runs the
-// fp64-accumulating SpMV kernels, which are deterministic, and ALG2's buffer
-// holds the merge-path partition (the nnz-balanced split that ALG2 asks for).
+// fp64-accumulating SpMV kernels, which are deterministic.  ALG2's buffer holds
+// what its analysis leaves: the merge-path partition (the nnz-balanced split
+// that ALG2 asks for) or, for a wide matrix with scattered columns, the
+// re-stored blocked-gather / column-panel layout.  ALG1 has no buffer: its
+// first execution reads the row lengths once and later ones run the row-wise
+// kernel they select.
 #include <climits>
 #include <new>
 
