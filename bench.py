@@ -244,6 +244,15 @@ def main():
         bytes_gather = wl.spmm_bytes_gather(rows, cols, n, nnz, vb, B.element_size(), 4, cfg["beta"] != 0)
         dtype = "f32" if vb == 4 else "f16 in, f32 accumulate/out"
     stream.synchronize()
+    first_use_ms = (time.perf_counter() - t_pre) * 1e3  # includes loading the library's kernels onto the device
+    # the same GetBufferSize + buffer allocation + Preprocess once more, now that the kernels are loaded: what a
+    # second matrix would cost
+    t_pre = time.perf_counter()
+    if not is_spmm:
+        op = osa.SpmvOp(handle, csr, X, Y, preprocess=not args.no_preprocess, alg=op.alg)
+    else:
+        op = osa.SpmmOp(handle, csr, Bd, Cd)
+    stream.synchronize()
     preprocess_ms = (time.perf_counter() - t_pre) * 1e3
 
     alpha, beta = cfg["alpha"], cfg["beta"]
@@ -283,7 +292,7 @@ def main():
         "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": dtype, "data": "synthetic",
         "config": {"workload": cfg["name"], "rows": rows, "cols": cols, "nnz": nnz, "ncols_dense": ncols,
-                   "alpha": alpha, "beta": beta, "index": "int32", "preprocess_ms": round(preprocess_ms, 3),
+                   "alpha": alpha, "beta": beta, "index": "int32", "preprocess_ms": round(preprocess_ms, 3), "first_use_ms": round(first_use_ms, 3),
                    "preprocessed": not args.no_preprocess, "layout": layout},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),

@@ -150,12 +150,33 @@ __global__ __launch_bounds__(kBlockThreads) void RowStatsKernel(const int32_t *_
         numLong += __shfl_xor(numLong, off, kWave);
         nnzLong += __shfl_xor(nnzLong, off, kWave);
     }
-    if ((threadIdx.x & (kWave - 1)) == 0 && best > 0) {
-        atomicMax(stats, best);
-        atomicMax(stats + 1, bestShort);
-        if (numLong > 0) {
-            atomicAdd(stats + 2, numLong);
-            atomicAdd(reinterpret_cast<uint32_t *>(stats) + 3, nnzLong);
+    // one set of atomics per workgroup: thousands of wavefronts updating the same four words take longer than
+    // reading the offsets does
+    constexpr int kWaves = kBlockThreads / kWave;
+    __shared__ int32_t waveBest[kWaves], waveShort[kWaves], waveLong[kWaves];
+    __shared__ uint32_t waveNnz[kWaves];
+    const int wave = threadIdx.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        waveBest[wave] = best;
+        waveShort[wave] = bestShort;
+        waveLong[wave] = numLong;
+        waveNnz[wave] = nnzLong;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kWaves; ++w) {
+            best = waveBest[w] > best ? waveBest[w] : best;
+            bestShort = waveShort[w] > bestShort ? waveShort[w] : bestShort;
+            numLong += waveLong[w];
+            nnzLong += waveNnz[w];
+        }
+        if (best > 0) {
+            atomicMax(stats, best);
+            atomicMax(stats + 1, bestShort);
+            if (numLong > 0) {
+                atomicAdd(stats + 2, numLong);
+                atomicAdd(reinterpret_cast<uint32_t *>(stats) + 3, nnzLong);
+            }
         }
     }
 }
@@ -1672,7 +1693,7 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
         return OPSPARSE_E_LAUNCH;
     }
     int64_t grid = (rows + kBlockThreads - 1) / kBlockThreads;
-    grid = grid > 4096 ? 4096 : grid;
+    grid = grid > 2048 ? 2048 : grid;
     hipLaunchKernelGGL(RowStatsKernel, dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0, s, rowOffsets, rows,
                        stats);
     int32_t seen[4] = {0, 0, 0, 0};  // longest row, longest of the short rows, rows longer than those, their entries
