@@ -377,6 +377,21 @@ __global__ __launch_bounds__(kBlockThreads) void RadixScatterKernel(
     }
 }
 
+// csrsort of a matrix of long rows, between its two sorts: the entries are sorted by column and carry (row,
+// permutation value); the second sort is by row and carries (column, permutation value).
+__global__ __launch_bounds__(kBlockThreads) void RegroupByRowKernel(const int32_t *__restrict__ colKeys,
+                                                                   const RadixPair *__restrict__ rowAndPerm, int64_t n,
+                                                                   int32_t colBase, int32_t *__restrict__ rowKeys,
+                                                                   RadixPair *__restrict__ colAndPerm)
+{
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
+    if (i < n) {
+        const RadixPair in = rowAndPerm[i];
+        rowKeys[i] = in.row;
+        colAndPerm[i] = RadixPair{colKeys[i] + colBase, in.val};
+    }
+}
+
 // ---------------------------------------------------------------- csr2csc
 
 // cscRowInd[d] = row of source position pos[d] (+ base); cscVal[d] = csrVal[pos[d]].
@@ -828,10 +843,40 @@ int opsparse_csr2coo_launch(const int32_t *csrRowPtr, int64_t nnz, int64_t m, in
     return CheckLaunch();
 }
 
+// Rows of thousands of entries on average: too few rows to occupy the GPU with a workgroup each (one row of 4 M
+// entries: 128 ms that way).  The whole matrix is then sorted with the device-wide radix passes, by column and
+// after that, stably, by row, 0.1 - 0.2 ms a pass for such sizes.  The mean is known on the host; a matrix of short
+// rows with single very long ones among them still takes the per-row kernels.
+constexpr int64_t kSortWholeMeanRow = 4096;
+
+static bool SortWhole(int64_t m, int64_t nnz) { return nnz / m >= kSortWholeMeanRow; }
+
+struct SortWholeLayout {
+    int64_t keysA, keysB, pairsA, pairsB, rowOfPos, table, tiles, bytes;
+};
+
+static SortWholeLayout LayoutSortWhole(int64_t nnz)
+{
+    SortWholeLayout l{};
+    int64_t off = 0;
+    l.keysA = off; off += Align256(4 * nnz);
+    l.keysB = off; off += Align256(4 * nnz);
+    l.pairsA = off; off += Align256(8 * nnz);
+    l.pairsB = off; off += Align256(8 * nnz);
+    l.rowOfPos = off; off += Align256(4 * nnz);
+    l.table = off; off += Align256(4 * RadixTableInts(nnz));
+    l.tiles = off; off += Align256(4 * ScanTiles(RadixTableInts(nnz)));
+    l.bytes = off;
+    return l;
+}
+
 size_t opsparse_csrsort_workspace_bytes(int64_t m, int64_t nnz)
 {
     if (m <= 0 || nnz <= 0) {
         return 0;
+    }
+    if (SortWhole(m, nnz)) {
+        return static_cast<size_t>(LayoutSortWhole(nnz).bytes);
     }
     return static_cast<size_t>(2 * Align256(4 * nnz) + 256 + 2 * Align256(4 * m));
 }
@@ -854,6 +899,45 @@ int opsparse_csrsort_launch(int64_t m, int64_t n, int64_t nnz, int32_t indexBase
     }
     auto s = static_cast<hipStream_t>(stream);
     auto *base = static_cast<unsigned char *>(workspace);
+    if (SortWhole(m, nnz)) {
+        const SortWholeLayout l = LayoutSortWhole(nnz);
+        auto at = [&](int64_t off) { return reinterpret_cast<int32_t *>(base + off); };
+        int32_t *keys[2] = {at(l.keysA), at(l.keysB)};
+        void *pairs[2] = {base + l.pairsA, base + l.pairsB};
+        int32_t *rowOfPos = at(l.rowOfPos), *table = at(l.table), *tiles = at(l.tiles);
+        hipLaunchKernelGGL(ExpandRowsKernel, dim3(GridFor(m, kBlockThreads)), dim3(kBlockThreads), 0, s, csrRowPtr, m,
+                           nnz, indexBase, rowOfPos);  // rows numbered from indexBase: the order is what matters
+        // by column, carrying (row, permutation value) ...
+        const RadixPairIo in{rowOfPos, perm, nullptr, nullptr, 4};
+        const int32_t colPasses = (KeyBits(n) + kRadixBits - 1) / kRadixBits;
+        const int32_t *keysIn = csrColInd;
+        const void *pairsIn = nullptr;
+        int cur = 0;
+        for (int32_t pass = 0; pass < colPasses; ++pass) {
+            LaunchRadixPairPass(pass == 0 ? kPayPairFirst : kPayPair, keysIn, pairsIn, keys[cur], pairs[cur], nnz,
+                                pass == 0 ? indexBase : 0, pass * kRadixBits, table, tiles, in, s);
+            keysIn = keys[cur];
+            pairsIn = pairs[cur];
+            cur ^= 1;
+        }
+        // ... then, stably, by row, carrying (column, permutation value); the last pass writes both in place
+        hipLaunchKernelGGL(RegroupByRowKernel, dim3(GridFor(nnz, kBlockThreads)), dim3(kBlockThreads), 0, s, keysIn,
+                           static_cast<const RadixPair *>(pairsIn), nnz, indexBase, keys[cur],
+                           static_cast<RadixPair *>(pairs[cur]));
+        keysIn = keys[cur];
+        pairsIn = pairs[cur];
+        cur ^= 1;
+        const RadixPairIo out{nullptr, nullptr, csrColInd, perm, 4};
+        const int32_t rowPasses = (KeyBits(m + indexBase) + kRadixBits - 1) / kRadixBits;
+        for (int32_t pass = 0; pass < rowPasses; ++pass) {
+            LaunchRadixPairPass(pass == rowPasses - 1 ? kPayPairLast : kPayPair, keysIn, pairsIn, keys[cur], pairs[cur],
+                                nnz, 0, pass * kRadixBits, table, tiles, out, s);
+            keysIn = keys[cur];
+            pairsIn = pairs[cur];
+            cur ^= 1;
+        }
+        return CheckLaunch();
+    }
     const int64_t arr = Align256(4 * nnz);
     auto *tmpCol = reinterpret_cast<int32_t *>(base);
     auto *tmpPerm = reinterpret_cast<int32_t *>(base + arr);

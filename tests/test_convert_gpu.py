@@ -224,6 +224,19 @@ def test_csrsort_many_rows(osa, gpu_ctx):
     run_csrsort(osa, gpu_ctx, m, n, rowptr, colind)
 
 
+@pytest.mark.parametrize("lengths,n,base", [([300_000], 2_000_000, 0), ([0, 40_000, 0, 9_000, 70_000, 1, 0], 50_000, 1),
+                                            ([4096] * 33, 17, 0), ([5000, 4000, 3500], 1, 0)])
+def test_csrsort_long_rows_on_average(osa, gpu_ctx, lengths, n, base):
+    """Thousands of entries per row on average: the whole matrix is sorted by the device-wide radix passes (by
+    column, then stably by row) instead of a workgroup per row.  Repeated columns keep their order (P tells), empty
+    rows, one row only, one column only, index base 1, P not the identity."""
+    rng = np.random.default_rng(len(lengths) + n)
+    assert sum(lengths) // len(lengths) >= 4096
+    rowptr, colind = _rows(lengths, lambda r, l: rng.integers(0, n, l))
+    perm = rng.integers(-1000, 1000, colind.size).astype(np.int32) if base else None
+    run_csrsort(osa, gpu_ctx, len(lengths), n, rowptr + base, colind + base, base=base, perm=perm, misalign=4 * base)
+
+
 # ------------------------------------------------------------------ csr2csc
 
 CSR2CSC = load_cases("csr2csc_cases.csv")
