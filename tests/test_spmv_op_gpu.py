@@ -257,3 +257,30 @@ def test_alg1_repeated_executions_and_value_updates(osa, gpu_ctx, shape):
                                   oracle.spmv_f64(3000, 4000, o_rp, o_ci, o_val, o_x, np.zeros(3000, np.float32),
                                                   1.0, 0.0)) <= 1e-5
     op.close()
+
+
+@pytest.mark.parametrize("alias", [False, True])
+def test_alg1_short_rows_with_long_ones_beside(osa, gpu_ctx, alias):
+    """ALG1 on short rows with a few long ones: after the first execution the stream-rows tiles run with the long
+    rows summed beside them by a second kernel; Z separate from Y and Z aliasing Y must both see every row written
+    exactly once (beta != 0)."""
+    dev, stream, handle = gpu_ctx
+    rng = np.random.default_rng(31)
+    m = k = 120_000
+    lengths = rng.integers(2, 7, m)
+    lengths[[0, 500, 60_000, 119_999]] = [2_000, 65, 7_000, 300]
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = np.clip(np.repeat(np.arange(m), lengths) + rng.integers(-900, 901, int(rowptr[-1])), 0, k - 1).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    x, y = rng.uniform(-1, 1, k).astype(np.float32), rng.uniform(-1, 1, m).astype(np.float32)
+    d_rp, d_ci, d_val, d_x, d_y = (to_dev(a, dev) for a in (rowptr, colind, val, x, y))
+    d_z = d_y if alias else torch.zeros(m, dtype=torch.float32, device=dev)
+    Y = osa.DnVec(d_y)
+    Z = Y if alias else osa.DnVec(d_z)
+    op = osa.SpmvOpPlan(handle, osa.Csr(m, k, d_rp, d_ci, d_val), osa.DnVec(d_x), Y, Z, alg=osa.ACL_SPARSE_SPMVOP_ALG1)
+    for step in range(3):                       # the first execution takes the statistics, the others use them
+        d_y.copy_(torch.from_numpy(y))
+        op(1.25, -0.5)
+        stream.synchronize()
+        check(d_z.cpu().numpy(), m, k, rowptr, colind, val, x, y, 1.25, -0.5)
+    op.close()
