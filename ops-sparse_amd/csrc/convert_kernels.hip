@@ -574,10 +574,21 @@ __global__ __launch_bounds__(kBlockThreads) void SortListedRowsKernel(const int3
             __syncthreads();
             continue;
         }
-        // Radix passes over [begin, begin + len), thread t on entries [t * part, (t + 1) * part).
-        const int64_t part = (len + kBlockThreads - 1) / kBlockThreads;
-        const int64_t lo = begin + threadIdx.x * part < begin + len ? begin + threadIdx.x * part : begin + len;
-        const int64_t hi = lo + part < begin + len ? lo + part : begin + len;
+        // Stable 4-bit radix passes over [begin, begin + len) between the row and the scratch arrays.  Wavefront w
+        // owns the w-th quarter of the row and walks it 64 consecutive entries at a time, so every load is
+        // coalesced.  Counting pass: per-lane digit counts, added up over the wavefront.  Then the first output
+        // slot of every (digit, wavefront), digit-major, so that equal digits keep their order.  Scatter pass: the
+        // lanes of a round that hold the same digit are found with four ballots, the rank among them is a population
+        // count, and a running count per digit carries on from round to round.
+        constexpr int kWaves = kBlockThreads / kWave;
+        constexpr int kRounds = 8;  // rounds whose loads are issued together
+        int32_t *waveDigit = counters;                        // [kWaves][kRadixDigits] counts, then first slots
+        int32_t *running = counters + kWaves * kRadixDigits;  // [kWaves][kRadixDigits] entries placed so far
+        const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+        const uint64_t below = (uint64_t{1} << lane) - 1;
+        const int64_t quarter = (len + kWaves - 1) / kWaves;
+        const int64_t lo = begin + wave * quarter < begin + len ? begin + wave * quarter : begin + len;
+        const int64_t hi = lo + quarter < begin + len ? lo + quarter : begin + len;
         int32_t *srcCol = colInd, *srcPerm = perm, *dstCol = tmpCol, *dstPerm = tmpPerm;
         for (int32_t shift = 0; shift < keyBits; shift += kRadixBits) {
             int32_t cnt[kRadixDigits];
@@ -585,35 +596,76 @@ __global__ __launch_bounds__(kBlockThreads) void SortListedRowsKernel(const int3
             for (int d = 0; d < kRadixDigits; ++d) {
                 cnt[d] = 0;
             }
-            for (int64_t p = lo; p < hi; ++p) {
-                const int32_t dg = RadixDigit(srcCol[p] - base, shift);
+            for (int64_t p0 = lo + lane; p0 < hi; p0 += kRounds * kWave) {
+                int32_t c[kRounds];
 #pragma unroll
-                for (int d = 0; d < kRadixDigits; ++d) {
-                    cnt[d] += (dg == d) ? 1 : 0;
+                for (int u = 0; u < kRounds; ++u) {  // the loads of kRounds rounds issued together
+                    const int64_t p = p0 + u * kWave;
+                    c[u] = p < hi ? srcCol[p] : -1;
                 }
-            }
 #pragma unroll
-            for (int d = 0; d < kRadixDigits; ++d) {
-                counters[d * kBlockThreads + threadIdx.x] = cnt[d];
-            }
-            __syncthreads();
-            ScanDigitCounters(counters, waveSums);
+                for (int u = 0; u < kRounds; ++u) {
+                    const int32_t dg = p0 + u * kWave < hi ? RadixDigit(c[u] - base, shift) : -1;
 #pragma unroll
-            for (int d = 0; d < kRadixDigits; ++d) {
-                cnt[d] = counters[d * kBlockThreads + threadIdx.x];  // next output slot of digit d for this thread
-            }
-            for (int64_t p = lo; p < hi; ++p) {
-                const int32_t c = srcCol[p];
-                const int32_t dg = RadixDigit(c - base, shift);
-                int32_t slot = 0;
-#pragma unroll
-                for (int d = 0; d < kRadixDigits; ++d) {
-                    if (dg == d) {
-                        slot = cnt[d]++;
+                    for (int d = 0; d < kRadixDigits; ++d) {
+                        cnt[d] += (dg == d) ? 1 : 0;
                     }
                 }
-                dstCol[begin + slot] = c;
-                dstPerm[begin + slot] = srcPerm[p];
+            }
+#pragma unroll
+            for (int d = 0; d < kRadixDigits; ++d) {
+                int32_t c = cnt[d];
+#pragma unroll
+                for (int off = kWave / 2; off > 0; off >>= 1) {
+                    c += __shfl_xor(c, off, kWave);
+                }
+                if (lane == 0) {
+                    waveDigit[wave * kRadixDigits + d] = c;
+                    running[wave * kRadixDigits + d] = 0;
+                }
+            }
+            __syncthreads();
+            if (threadIdx.x == 0) {  // 64 numbers: first slot of (digit, wavefront), digit-major
+                int32_t run = 0;
+                for (int d = 0; d < kRadixDigits; ++d) {
+                    for (int w = 0; w < kWaves; ++w) {
+                        const int32_t c = waveDigit[w * kRadixDigits + d];
+                        waveDigit[w * kRadixDigits + d] = run;
+                        run += c;
+                    }
+                }
+            }
+            __syncthreads();
+            for (int64_t p0 = lo; p0 < hi; p0 += kRounds * kWave) {
+                int32_t c[kRounds], pv[kRounds];
+                bool valid[kRounds];
+#pragma unroll
+                for (int u = 0; u < kRounds; ++u) {
+                    const int64_t p = p0 + u * kWave + lane;
+                    valid[u] = p < hi;
+                    c[u] = valid[u] ? srcCol[p] : 0;
+                    pv[u] = valid[u] ? srcPerm[p] : 0;
+                }
+#pragma unroll
+                for (int u = 0; u < kRounds; ++u) {
+                    const int32_t dg = RadixDigit(c[u] - base, shift);
+                    uint64_t same = __ballot(valid[u]);
+#pragma unroll
+                    for (int b = 0; b < kRadixBits; ++b) {
+                        const bool bit = (dg >> b) & 1;
+                        const uint64_t votes = __ballot(valid[u] && bit);
+                        same &= bit ? votes : ~votes;
+                    }
+                    const int32_t before = running[wave * kRadixDigits + dg];
+                    if (valid[u]) {
+                        const int64_t slot = begin + waveDigit[wave * kRadixDigits + dg] + before + __popcll(same & below);
+                        dstCol[slot] = c[u];
+                        dstPerm[slot] = pv[u];
+                        if ((same & below) == 0) {  // the lowest lane of every digit present in this round
+                            running[wave * kRadixDigits + dg] = before + __popcll(same);
+                        }
+                    }
+                }
             }
             __threadfence_block();
             __syncthreads();
