@@ -40,6 +40,7 @@ constexpr int kRadixTile = kBlockThreads * kRadixItems;
 constexpr int kSortWaveRow = 64;                          // rows up to this length: one wavefront, registers
 constexpr int kSortLdsRow = 2048;                         // rows up to this length: one workgroup, LDS
 constexpr int kSortListBlocks = 2048;                     // workgroups walking the list of longer rows
+constexpr int kSortWideRow = 16384;                       // listed rows longer than this get 1024 lanes instead of 256
 
 // ------------------------------------------------------------------- fill
 
@@ -523,36 +524,45 @@ __global__ __launch_bounds__(kBlockThreads) void SortMidRowsKernel(const int32_t
 // bits a pass, between the row and its place in the scratch arrays; thread t
 // owns the t-th contiguous part of the row, so the same counter scan as in
 // RadixScatterKernel keeps it stable.
-__global__ __launch_bounds__(kBlockThreads) void SortListedRowsKernel(const int32_t *__restrict__ rowPtr, int32_t base,
+template <int kThreads>
+__global__ __launch_bounds__(kThreads) void SortListedRowsKernel(const int32_t *__restrict__ rowPtr, int32_t base,
                                                                      int32_t keyBits, int32_t *colInd, int32_t *perm,
                                                                      int32_t *tmpCol, int32_t *tmpPerm,
-                                                                     const int32_t *__restrict__ listCounts,
-                                                                     const int32_t *__restrict__ list)
+                                                                     int32_t *listCounts, const int32_t *__restrict__ list,
+                                                                     int32_t countSlot, int64_t lenTo,
+                                                                     int32_t *__restrict__ longerList)
 {
     __shared__ uint64_t keys[kSortLdsRow];                          // 16 KB, doubles as the radix counters
     __shared__ int32_t pays[kSortLdsRow];
-    __shared__ int32_t waveSums[kBlockThreads / kWave];
-    static_assert(sizeof(uint64_t) * kSortLdsRow >= sizeof(int32_t) * kRadixDigits * kBlockThreads, "counter space");
+    __shared__ int32_t waveSums[kThreads / kWave];
+    static_assert(sizeof(uint64_t) * kSortLdsRow >= sizeof(int32_t) * 2 * (kThreads / kWave) * kRadixDigits, "counter space");
     int32_t *counters = reinterpret_cast<int32_t *>(keys);
 
-    const int32_t count = listCounts[1];
+    const int32_t count = listCounts[countSlot];
     for (int32_t item = blockIdx.x; item < count; item += gridDim.x) {
         const int32_t row = list[item];
         const int64_t begin = static_cast<int64_t>(rowPtr[row]) - base;
         const int64_t len = static_cast<int64_t>(rowPtr[row + 1]) - base - begin;
+        if (len > lenTo) {
+            // too long for this launch: listed for the next one, which runs with more lanes per row
+            if (threadIdx.x == 0) {
+                longerList[atomicAdd(&listCounts[2], 1)] = row;
+            }
+            continue;
+        }
         if (len <= kSortLdsRow) {
             int32_t npad = 128;
             while (npad < len) {
                 npad <<= 1;
             }
-            for (int32_t i = threadIdx.x; i < npad; i += kBlockThreads) {
+            for (int32_t i = threadIdx.x; i < npad; i += kThreads) {
                 keys[i] = i < len ? SortKey(colInd[begin + i], static_cast<uint32_t>(i)) : ~0ull;
                 pays[i] = i < len ? perm[begin + i] : 0;
             }
             __syncthreads();
             for (int32_t k = 2; k <= npad; k <<= 1) {
                 for (int32_t j = k >> 1; j > 0; j >>= 1) {
-                    for (int32_t i = threadIdx.x; i < npad; i += kBlockThreads) {
+                    for (int32_t i = threadIdx.x; i < npad; i += kThreads) {
                         const int32_t partner = i ^ j;
                         if (partner > i) {
                             const uint64_t a = keys[i], b = keys[partner];
@@ -566,7 +576,7 @@ __global__ __launch_bounds__(kBlockThreads) void SortListedRowsKernel(const int3
                     __syncthreads();
                 }
             }
-            for (int32_t i = threadIdx.x; i < len; i += kBlockThreads) {
+            for (int32_t i = threadIdx.x; i < len; i += kThreads) {
                 const uint64_t key = keys[i];
                 colInd[begin + i] = SortKeyColumn(key);
                 perm[begin + i] = pays[static_cast<uint32_t>(key & 0xffffffffu)];
@@ -580,7 +590,7 @@ __global__ __launch_bounds__(kBlockThreads) void SortListedRowsKernel(const int3
         // slot of every (digit, wavefront), digit-major, so that equal digits keep their order.  Scatter pass: the
         // lanes of a round that hold the same digit are found with four ballots, the rank among them is a population
         // count, and a running count per digit carries on from round to round.
-        constexpr int kWaves = kBlockThreads / kWave;
+        constexpr int kWaves = kThreads / kWave;
         constexpr int kRounds = 8;  // rounds whose loads are issued together
         int32_t *waveDigit = counters;                        // [kWaves][kRadixDigits] counts, then first slots
         int32_t *running = counters + kWaves * kRadixDigits;  // [kWaves][kRadixDigits] entries placed so far
@@ -677,7 +687,7 @@ __global__ __launch_bounds__(kBlockThreads) void SortListedRowsKernel(const int3
             dstPerm = t;
         }
         if (srcCol != colInd) {  // an odd number of passes left the result in the scratch arrays
-            for (int64_t p = begin + threadIdx.x; p < begin + len; p += kBlockThreads) {
+            for (int64_t p = begin + threadIdx.x; p < begin + len; p += kThreads) {
                 colInd[p] = srcCol[p];
                 perm[p] = srcPerm[p];
             }
@@ -996,7 +1006,7 @@ int opsparse_csrsort_launch(int64_t m, int64_t n, int64_t nnz, int32_t indexBase
     auto *counters = reinterpret_cast<int32_t *>(base + 2 * arr);
     auto *midList = reinterpret_cast<int32_t *>(base + 2 * arr + 256);
     auto *longList = reinterpret_cast<int32_t *>(base + 2 * arr + 256 + Align256(4 * m));
-    LaunchFill(counters, 2, 0, s);
+    LaunchFill(counters, 3, 0, s);
     // Lanes per row from the mean row length: twice the mean, a power of two in [8, 64].
     const int64_t mean2 = 2 * nnz / m;
     const int g = mean2 <= 8 ? 8 : mean2 <= 16 ? 16 : mean2 <= 32 ? 32 : 64;
@@ -1023,8 +1033,15 @@ int opsparse_csrsort_launch(int64_t m, int64_t n, int64_t nnz, int32_t indexBase
         hipLaunchKernelGGL(SortMidRowsKernel, dim3(kSortListBlocks), dim3(kBlockThreads), 0, s, csrRowPtr, indexBase,
                            csrColInd, perm, counters, midList);
     }
-    hipLaunchKernelGGL(SortListedRowsKernel, dim3(kSortListBlocks), dim3(kBlockThreads), 0, s, csrRowPtr, indexBase,
-                       KeyBits(n), csrColInd, perm, tmpCol, tmpPerm, counters, longList);
+    // Listed rows of up to kSortWideRow entries: 256 lanes each, many rows at a time.  The few beyond: 1024 lanes
+    // each, because the longest of them is what the call waits for (a row of 1 M entries 12.5 -> 6 ms).
+    // (the list of the mid rows has been used up by then: its space takes the rows handed on)
+    hipLaunchKernelGGL(SortListedRowsKernel<kBlockThreads>, dim3(kSortListBlocks), dim3(kBlockThreads), 0, s, csrRowPtr,
+                       indexBase, KeyBits(n), csrColInd, perm, tmpCol, tmpPerm, counters, longList, 1,
+                       int64_t{kSortWideRow}, midList);
+    hipLaunchKernelGGL(SortListedRowsKernel<1024>, dim3(kSortListBlocks / 4), dim3(1024), 0, s, csrRowPtr, indexBase,
+                       KeyBits(n), csrColInd, perm, tmpCol, tmpPerm, counters, midList, 2, int64_t{INT32_MAX},
+                       static_cast<int32_t *>(nullptr));
     return CheckLaunch();
 }
 
