@@ -168,6 +168,89 @@ def cpu_baseline_spmm(cfg, c_gpu, rows_sample=262144):
             "gpu_vs_fp64_oracle_max_rel_err": err}
 
 
+def vendor_yardstick(torch, cfg, is_spmm, flops, bytes_alg, steps, stream, ours):
+    """The same product through rocSPARSE's generic API (rocsparse_spmv / rocsparse_spmm: buffer size and
+    preprocess once, then `steps` compute calls between two events on `stream`), for each of its CSR
+    algorithms.  A yard-stick beside the figures, not an oracle; `ours` is this library's result for beta = 0,
+    and one more call with beta = 0 is compared with it so that an algorithm that did nothing is not quoted."""
+    import ctypes
+    try:
+        rs = ctypes.CDLL("librocsparse.so.1")
+    except OSError as exc:
+        return {"error": str(exc)}
+    vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    I32, F16, F32, NONE, ROW = 2, 150, 151, 111, 0  # rocsparse_indextype / datatype / operation / order values
+    rs.rocsparse_create_csr_descr.argtypes = [ctypes.POINTER(vp), i64, i64, i64, vp, vp, vp, ci, ci, ci, ci]
+    rs.rocsparse_create_dnvec_descr.argtypes = [ctypes.POINTER(vp), i64, vp, ci]
+    rs.rocsparse_create_dnmat_descr.argtypes = [ctypes.POINTER(vp), i64, i64, i64, vp, ci, ci]
+    rs.rocsparse_set_stream.argtypes = [vp, vp]
+    rs.rocsparse_spmv.argtypes = [vp, ci, vp, vp, vp, vp, vp, ci, ci, ci, ctypes.POINTER(ctypes.c_size_t), vp]
+    rs.rocsparse_spmm.argtypes = [vp, ci, ci, vp, vp, vp, vp, vp, ci, ci, ci, ctypes.POINTER(ctypes.c_size_t), vp]
+    A = cfg["A"]
+    rows, cols, nnz = A["rows"], A["cols"], int(A["colind"].numel())
+    vt = F32 if A["values"].element_size() == 4 else F16
+    handle, mat, dx, dy = vp(), vp(), vp(), vp()
+    if rs.rocsparse_create_handle(ctypes.byref(handle)):
+        return {"error": "rocsparse_create_handle failed"}
+    rs.rocsparse_set_stream(handle, vp(stream.cuda_stream))
+    rs.rocsparse_create_csr_descr(ctypes.byref(mat), rows, cols, nnz, A["rowptr"].data_ptr(), A["colind"].data_ptr(),
+                                  A["values"].data_ptr(), I32, I32, 0, vt)
+    if is_spmm:
+        n = cfg["n"]
+        dense = cfg["B"].contiguous()
+        out = torch.zeros(rows, n, dtype=torch.float32, device=dense.device)
+        rs.rocsparse_create_dnmat_descr(ctypes.byref(dx), cols, n, n, dense.data_ptr(), vt, ROW)
+        rs.rocsparse_create_dnmat_descr(ctypes.byref(dy), rows, n, n, out.data_ptr(), F32, ROW)
+        algs = {"default": 0, "csr": 1, "csr_row_split": 4, "csr_nnz_split": 5, "csr_merge_path": 9}
+    else:
+        dense = cfg["x"]
+        out = cfg["y0"].clone()
+        rs.rocsparse_create_dnvec_descr(ctypes.byref(dx), cols, dense.data_ptr(), vt)
+        rs.rocsparse_create_dnvec_descr(ctypes.byref(dy), rows, out.data_ptr(), F32)
+        algs = {"default": 0, "csr_adaptive": 2, "csr_rowsplit": 3, "csr_lrb": 7, "csr_nnzsplit": 8}
+    alpha, beta, zero = ctypes.c_float(cfg["alpha"]), ctypes.c_float(cfg["beta"]), ctypes.c_float(0.0)
+    scale = float(ours.abs().max().item()) or 1.0
+
+    def call(alg, stage, size, buf, b=beta):
+        if is_spmm:
+            return rs.rocsparse_spmm(handle, NONE, NONE, ctypes.byref(alpha), mat, dx, ctypes.byref(b), dy, F32,
+                                     alg, stage, ctypes.byref(size), buf)
+        return rs.rocsparse_spmv(handle, NONE, ctypes.byref(alpha), mat, dx, ctypes.byref(b), dy, F32, alg, stage,
+                                 ctypes.byref(size), buf)
+
+    res = {"what": "rocsparse_%s, buffer size and preprocess once, %d compute calls per algorithm"
+                   % ("spmm" if is_spmm else "spmv", steps)}
+    for name, alg in algs.items():
+        size = ctypes.c_size_t(0)
+        st = call(alg, 1, size, None)
+        buf = torch.empty(max(int(size.value), 256), dtype=torch.uint8, device=dense.device)
+        st = st or call(alg, 2, size, vp(buf.data_ptr()))
+        st = st or call(alg, 3, size, vp(buf.data_ptr()))
+        stream.synchronize()
+        if st:
+            res[name] = {"status": st}
+            continue
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(steps):
+            call(alg, 3, size, vp(buf.data_ptr()))
+        e1.record(stream)
+        stream.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        out.zero_()  # not NaN: some of the vendor's kernels scale y by beta = 0 before they add to it
+        call(alg, 3, size, vp(buf.data_ptr()), zero)
+        stream.synchronize()
+        diff = float(((out - ours).abs().max() / scale).item())
+        if not diff <= 1e-3:
+            res[name] = {"error": "result differs from this library's (max |d| / max |ours| = %g): not quoted" % diff,
+                         "ms_per_step": round(ms, 6)}
+            continue
+        res[name] = {"ms_per_step": round(ms, 6), "value": round(flops / (ms * 1e-3) / 1e9, 2), "unit": "GFLOP/s",
+                     "frac_of_8TBs": round(bytes_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "buffer_bytes": int(size.value), "max_diff_vs_ours": diff}
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -182,6 +265,8 @@ def main():
     ap.add_argument("--panels", action="store_true",
                     help="like --alg2 with the blocked-gather layout switched off: column panels (c3)")
     ap.add_argument("--gather-probe", action="store_true", help="also measure random-gather rates (stderr)")
+    ap.add_argument("--vendor", action="store_true",
+                    help="also time the same product through rocSPARSE's generic API, as a yard-stick beside the figures")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -301,6 +386,11 @@ def main():
                      "bytes_alg": bytes_alg, "bytes_gather_model": bytes_gather,
                      "copy_kernel_gbps": round(copy_gbps, 1), "read_kernel_gbps": round(read_gbps, 1)},
     }
+    if args.vendor:
+        op(alpha, 0.0)
+        stream.synchronize()
+        out["vendor_yardstick"] = vendor_yardstick(torch, cfg, is_spmm, flops, bytes_alg, max(5, args.steps // 4),
+                                                   stream, (y if not is_spmm else Cmat).clone())
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline_spmm(cfg, first_result) if is_spmm else cpu_baseline_spmv(cfg, first_result)
     print(json.dumps(out), flush=True)
