@@ -224,6 +224,18 @@ def test_csrsort_many_rows(osa, gpu_ctx):
     run_csrsort(osa, gpu_ctx, m, n, rowptr, colind)
 
 
+@pytest.mark.parametrize("n", [7, 3_000_000])
+def test_csrsort_rows_either_side_of_the_wide_launch(osa, gpu_ctx, n):
+    """Rows of 16 383 - 16 385 entries and a few far longer ones among 3000 short rows: the listed rows are sorted by
+    two launches, 256 lanes a row up to 16 384 entries and 1024 beyond; few distinct columns (long runs of equal
+    keys, whose order P shows) and many (all key bits in use)."""
+    rng = np.random.default_rng(n)
+    lengths = rng.integers(0, 40, 3000)
+    lengths[[0, 17, 18, 1500, 2998, 2999]] = [16385, 16384, 16383, 131_073, 40_000, 16_400]
+    rowptr, colind = _rows(lengths, lambda r, l: rng.integers(0, n, l))
+    run_csrsort(osa, gpu_ctx, 3000, n, rowptr, colind)
+
+
 @pytest.mark.parametrize("lengths,n,base", [([300_000], 2_000_000, 0), ([0, 40_000, 0, 9_000, 70_000, 1, 0], 50_000, 1),
                                             ([4096] * 33, 17, 0), ([5000, 4000, 3500], 1, 0)])
 def test_csrsort_long_rows_on_average(osa, gpu_ctx, lengths, n, base):
