@@ -371,6 +371,7 @@ def main():
     if args.gather_probe:
         log("random gathers, G/s: %s" % json.dumps(measure_gather(osa, torch, wl, dev, stream)))
 
+    traffic = load_traffic(cfg["name"] + ("+" + layout if layout != "csr" else "")) if args.scale == 1.0 else None
     out = {
         "metric": "SpMV/SpMM GFLOP/s + achieved HBM GB/s (% of MI355X peak), CSR fp32",
         "value": round(gflops, 2), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -381,9 +382,12 @@ def main():
                    "preprocessed": not args.no_preprocess, "layout": layout},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": load_traffic(cfg["name"] + ("+" + layout if layout != "csr" else ""))
-                     if args.scale == 1.0 else None,
+                     "traffic": traffic,
+                     "traffic_gbps": round(traffic / (ms * 1e-3) / 1e9, 1) if traffic else None,
                      "bytes_alg": bytes_alg, "bytes_gather_model": bytes_gather,
+                     # the dense operand counted once per use instead of once: what a row-wise kernel has to move
+                     # when none of its gathers hits a cache (never the headline figure: it credits cache hits)
+                     "gather_model_gbps": round(bytes_gather / (ms * 1e-3) / 1e9, 1),
                      "copy_kernel_gbps": round(copy_gbps, 1), "read_kernel_gbps": round(read_gbps, 1)},
     }
     if args.vendor:
