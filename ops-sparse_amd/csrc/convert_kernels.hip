@@ -534,7 +534,6 @@ __global__ __launch_bounds__(kThreads) void SortListedRowsKernel(const int32_t *
 {
     __shared__ uint64_t keys[kSortLdsRow];                          // 16 KB, doubles as the radix counters
     __shared__ int32_t pays[kSortLdsRow];
-    __shared__ int32_t waveSums[kThreads / kWave];
     static_assert(sizeof(uint64_t) * kSortLdsRow >= sizeof(int32_t) * 2 * (kThreads / kWave) * kRadixDigits, "counter space");
     int32_t *counters = reinterpret_cast<int32_t *>(keys);
 

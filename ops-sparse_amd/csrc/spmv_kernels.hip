@@ -1027,13 +1027,14 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvPanelCombineKernel(const Ac
 // ------------------------------------------------------------- op(A) = A^T
 
 // y[col] += alpha * x[row] * val for every stored element; y was scaled by
-// beta beforehand.  Floating point only (hardware fp32 atomic add); the order
-// of the additions is not fixed, as in the reference's transpose path
-// (sparse/spmv/arch22/kernels/spmv_kernel.h:584-624).
-template <typename ValT, typename AccT, int G>
+// beta beforehand.  Hardware atomic add on fp32 y: the order of the additions
+// is not fixed, as in the reference's transpose path
+// (sparse/spmv/arch22/kernels/spmv_kernel.h:584-624).  On int32 y (int32
+// compute type) the additions wrap around, so their order does not show.
+template <typename ValT, typename AccT, int G, typename YT = float>
 __global__ __launch_bounds__(kBlockThreads) void SpmvTransposeScatterKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
-    const ValT *__restrict__ x, float *__restrict__ y, int64_t rows, int32_t maxLen, OpsparseScalar alphaS)
+    const ValT *__restrict__ x, YT *__restrict__ y, int64_t rows, int32_t maxLen, OpsparseScalar alphaS)
 {
     const AccT alpha = ReadScalar<AccT>(alphaS);
     constexpr int kGroups = kBlockThreads / G;
@@ -1050,7 +1051,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvTransposeScatterKernel(
         return;  // left to SpmvTransposeLongRowsKernel
     }
     for (int64_t k = static_cast<int64_t>(rowOffsets[r]) + threadIdx.x % G; k < e; k += G) {
-        atomicAdd(y + LoadStream(colInd + k), static_cast<float>(ax * ToAcc<AccT>(LoadStream(vals + k))));
+        atomicAdd(y + LoadStream(colInd + k), static_cast<YT>(ax * ToAcc<AccT>(LoadStream(vals + k))));
     }
 }
 
@@ -1640,6 +1641,34 @@ int RunTranspose(const SpmvArgs &a, int32_t outType, bool skewedRows)
     return finish();
 }
 
+// op(A) = A^T in int32 arithmetic (the reference's SpmvKernelTrans<int32_t, int32_t, int32_t>,
+// sparse/spmv/arch22/kernels/spmv_kernel.cpp:21-55): y = beta * y, then an integer atomic add per entry, a lane
+// group per row.  Products and sums wrap around like the reference's int32 arithmetic, so the result does not
+// depend on the order of the additions.
+int RunTransposeInt(const SpmvArgs &a)
+{
+    int32_t *y = static_cast<int32_t *>(a.y);
+    const int rc = LaunchScale<int32_t, int32_t>(y, static_cast<const int32_t *>(a.yIn), a.cols, a.beta, a.stream);
+    if (rc != OPSPARSE_OK || a.nnz == 0 || a.rows == 0) {
+        return rc;
+    }
+    auto launch = [&](auto tag) {
+        constexpr int G = decltype(tag)::value;
+        hipLaunchKernelGGL((SpmvTransposeScatterKernel<int32_t, int32_t, G, int32_t>),
+                           dim3(GridFor(a.rows, kBlockThreads / G)), dim3(kBlockThreads), 0, a.stream, a.rowOffsets,
+                           a.colInd, static_cast<const int32_t *>(a.vals), static_cast<const int32_t *>(a.x), y, a.rows,
+                           INT32_MAX, a.alpha);
+    };
+    switch (VectorLanesFor(a.rows, a.nnz)) {
+        case 4: launch(std::integral_constant<int, 4>{}); break;
+        case 8: launch(std::integral_constant<int, 8>{}); break;
+        case 16: launch(std::integral_constant<int, 16>{}); break;
+        case 32: launch(std::integral_constant<int, 32>{}); break;
+        default: launch(std::integral_constant<int, 64>{}); break;
+    }
+    return CheckLaunch();
+}
+
 template <typename ValT, typename OutT, typename AccT>
 int RunTyped(const OpsparseSpmvPlan *plan, const SpmvArgs &a)
 {
@@ -1950,7 +1979,7 @@ int opsparse_spmv_csr_launch_zy(const OpsparseSpmvPlan *plan, int32_t transpose,
     }
     if (transpose) {
         if (computeIsInt) {
-            return OPSPARSE_E_UNSUPPORTED;
+            return valType == OPSPARSE_I32 && outType == OPSPARSE_I32 ? RunTransposeInt(a) : OPSPARSE_E_UNSUPPORTED;
         }
         // The analysis found a row far longer than the mean: the transposed product then splits the work by
         // entries rather than by rows.
@@ -1960,6 +1989,7 @@ int opsparse_spmv_csr_launch_zy(const OpsparseSpmvPlan *plan, int32_t transpose,
             case OPSPARSE_F32: return RunTranspose<float, double>(a, outType, skewedRows);
             case OPSPARSE_F16: return RunTranspose<Half, double>(a, outType, skewedRows);
             case OPSPARSE_BF16: return RunTranspose<Bf16, double>(a, outType, skewedRows);
+            case OPSPARSE_I32: return RunTranspose<int32_t, double>(a, outType, skewedRows);  // int32 values, fp32 y
             default: return OPSPARSE_E_UNSUPPORTED;
         }
     }
