@@ -137,6 +137,31 @@ def test_csr2coo_row_length_mix(osa, gpu_ctx):
         assert np.array_equal(d_rows.cpu().numpy(), oracle.csr2coo(rowptr + base, nnz, base))
 
 
+@pytest.mark.parametrize("name,rowptr,nnz,base,compare", [
+    ("non_monotonic", [0, 3, 1, 4], 4, 0, False),          # rows 0 and 2 overlap: which one wins is not defined
+    ("nnz_mismatch", [0, 1, 2, 3], 5, 0, True),
+    ("idxbase_mismatch", [0, 1, 2, 3, 4], 4, 1, True),
+    ("simd_row_exceeds_nnz", [0, 5], 3, 0, True),
+    ("simd_non_monotonic", [0, 250, 100], 300, 0, True),
+    ("simd_idxbase_mismatch", [0, 3], 3, 1, True)])
+def test_csr2coo_malformed_offsets_are_skipped(osa, gpu_ctx, name, rowptr, nnz, base, compare):
+    """The abnormal-input cases of the reference test (csr2coo_test.cpp, ABN_*): offsets that do not describe a
+    range inside [0, nnz) are not an error; such rows are skipped and nothing outside cooRowInd[0, nnz) is written
+    (csr2coo_golden.h:51-53).  The output starts as zeros, as in that test, with a guard element behind it."""
+    dev, stream, handle = gpu_ctx
+    rowptr = np.asarray(rowptr, np.int32)
+    d_ptr = dev_i32(rowptr, dev)
+    d_rows = torch.zeros(nnz + 1, dtype=torch.int32, device=dev)
+    d_rows[nnz] = -99
+    torch.cuda.synchronize()
+    assert osa.lib().aclsparseXcsr2coo(handle.h, ptr(d_ptr), nnz, rowptr.size - 1, ptr(d_rows), base) == 0
+    stream.synchronize()
+    got = d_rows.cpu().numpy()
+    assert got[nnz] == -99
+    if compare:
+        assert np.array_equal(got[:nnz], oracle.csr2coo(rowptr, nnz, base))
+
+
 # ------------------------------------------------------------------ csrsort
 
 def run_csrsort(osa, gpu_ctx, m, n, rowptr, colind, base=0, perm=None, misalign=0):
@@ -195,6 +220,45 @@ SORT_CASES = {
     "AlternatingTinyAndLarge": lambda: (400, 3000) + _rows([1 if r % 2 else 1500 for r in range(400)],
                                                             lambda r, l: (np.arange(l) * 7919 + r) % 3000),
 }
+
+
+def _mixed_stress(run):
+    """MixedShortAndMultiRunStress of the reference test (csrsort_test.cpp:604-656) with `run` for its run size."""
+    lengths = [[0, 1, 17, run, run + 1, run + 37, 63, min(run, 2047)][row % 8] for row in range(193)]
+    return (193, 16384) + _rows(lengths, lambda r, l: (r * 131 + (l - np.arange(l)) * 29 + np.arange(l) % 11) % 16384)
+
+
+def _run_boundaries(run):
+    """RunSizeBoundaries (csrsort_test.cpp:501-519): rows of run - 1, run and run + 1 entries, columns descending."""
+    nnz = 3 * run
+    return 3, 4096, np.array([0, run - 1, 2 * run - 1, nnz], np.int32), ((nnz - np.arange(nnz)) % 4096).astype(np.int32)
+
+
+# The reference sizes these cases by the run its on-chip buffer holds (CsrsortTiling::FindMaxRunSize); here they are
+# sized by the row lengths at which this library changes kernels: 64 (registers), 2048 (LDS), 16 384 (1024 lanes).
+SORT_CASES.update({
+    "RandomMedium": lambda: (50, 50) + _rows(np.random.default_rng(77).binomial(50, 0.15, 50),
+                                             lambda r, l: np.random.default_rng(77 + r).permutation(50)[:l]),
+    "Non64ElementCounts": lambda: (5, 257) + _rows([7, 63, 64, 65, 127], lambda r, l: (r * 37 + l - np.arange(l)) % 257),
+    "LargeAlignmentBoundaryMatrix": lambda: (640, 4096) + _rows(
+        [[31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 513, 1025][r % 15] for r in range(640)],
+        lambda r, l: (r * 193 + np.arange(l) * 61 + l - np.arange(l)) % 4096),
+    "RunSizeBoundaries64": lambda: _run_boundaries(64),
+    "RunSizeBoundaries2048": lambda: _run_boundaries(2048),
+    "RunSizeBoundaries16384": lambda: _run_boundaries(16384),
+    "MixedShortAndMultiRunStress64": lambda: _mixed_stress(64),
+    "MixedShortAndMultiRunStress2048": lambda: _mixed_stress(2048),
+    "MixedShortAndMultiRunStress16384": lambda: _mixed_stress(16384),
+})
+
+
+def test_csrsort_alternating_rows_with_custom_perm(osa, gpu_ctx):
+    """AlternatingTinyAndLargeShortRows as the reference runs it (csrsort_test.cpp:544-572): rows of 7 and of 4093
+    entries in turn, 257 distinct columns (long runs of equal keys) and P = row * 100000 + position."""
+    lengths = [7 if r % 2 == 0 else 4093 for r in range(512)]
+    rowptr, colind = _rows(lengths, lambda r, l: (r * 17 + l - np.arange(l)) % 257)
+    perm = np.concatenate([r * 100000 + np.arange(l) for r, l in enumerate(lengths)]).astype(np.int32)
+    run_csrsort(osa, gpu_ctx, 512, 8192, rowptr, colind, perm=perm)
 
 
 @pytest.mark.parametrize("name", list(SORT_CASES))
