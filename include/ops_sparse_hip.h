@@ -173,6 +173,24 @@ int opsparse_spmv_csr_launch_zy(const OpsparseSpmvPlan *plan, int32_t transpose,
                                 int32_t valType, int32_t outType, int32_t computeIsInt, void *workspace,
                                 size_t workspaceBytes, void *stream);
 
+/*
+ * opsparse_spmv_csr_launch with plan == NULL for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): y = alpha * A * x + beta * y by the merge-path
+ * kernels, whose partition, carries and heads live in a 4 MiB array that is part of the library's device image
+ * (one copy per GPU, held until the process ends) instead of a caller's workspace.  No counterpart in the
+ * reference.  Calls no hipMalloc / hipFree and no allocating library routine; the first call on a device looks
+ * the array's address up (hipGetSymbolAddress), so make that call outside a capture.
+ * Limit: opsparse_spmv_csr_workspace_bytes(rows, nnz) <= opsparse_spmv_csr_noalloc_max_bytes() (4 MiB: rows + nnz
+ * up to about 4.2e8); beyond it the call returns OPSPARSE_E_WORKSPACE and launches nothing.
+ * All calls on one GPU share the array: calls that overlap there (two streams, two threads) race; calls on one
+ * stream are ordered and safe.  Same types, scalars and result as opsparse_spmv_csr_launch.
+ */
+size_t opsparse_spmv_csr_noalloc_max_bytes(void);
+int opsparse_spmv_csr_launch_noalloc(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
+                                     const void *x, void *y, int64_t rows, int64_t cols, int64_t nnz,
+                                     OpsparseScalar alpha, OpsparseScalar beta, int32_t valType, int32_t outType,
+                                     int32_t computeIsInt, void *stream);
+
 /* fp32 z = alpha * A * x + beta * yIn for the index variants of the SpMVOp API:
  * int32 or int64 row offsets (rowOffsetsAre64), int32 column indices, index
  * base 0 or 1 [ref: sparse/spmv_op/arch35/spmv_op_kernel.cpp:139-181].  One lane

@@ -89,6 +89,7 @@ ACL_SPARSE_CSR2CSC_ALG_DEFAULT, ACL_SPARSE_CSR2CSC_ALG1 = 0, 1
 OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_workspace_bytes", "opsparse_spmv_csr_analyse", "opsparse_spmv_csr_launch",
     "opsparse_spmv_csr_launch_zy", "opsparse_spmv_csr_indexed_launch",
+    "opsparse_spmv_csr_launch_noalloc", "opsparse_spmv_csr_noalloc_max_bytes",
     "opsparse_spmv_csr_panels_workspace_bytes", "opsparse_spmv_csr_panels_analyse",
     "opsparse_spmv_csr_blocked_workspace_bytes", "opsparse_spmv_csr_blocked_analyse",
     "opsparse_spmv_csr_gathers_scattered",
@@ -232,6 +233,11 @@ def lib():
     L.opsparse_spmv_csr_launch_zy.restype = ctypes.c_int
     L.opsparse_spmv_csr_launch_zy.argtypes = [ctypes.POINTER(OpsparseSpmvPlan), i32, vp, vp, vp, vp, vp, vp, i64, i64,
                                               i64, OpsparseScalar, OpsparseScalar, i32, i32, i32, vp, sz, vp]
+    L.opsparse_spmv_csr_noalloc_max_bytes.restype = sz
+    L.opsparse_spmv_csr_noalloc_max_bytes.argtypes = []
+    L.opsparse_spmv_csr_launch_noalloc.restype = ctypes.c_int
+    L.opsparse_spmv_csr_launch_noalloc.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, OpsparseScalar, OpsparseScalar,
+                                                   i32, i32, i32, vp]
     L.opsparse_spmv_csr_panels_workspace_bytes.restype = sz
     L.opsparse_spmv_csr_panels_workspace_bytes.argtypes = [i64, i64, i64]
     L.opsparse_spmv_csr_gathers_scattered.restype = ctypes.c_int

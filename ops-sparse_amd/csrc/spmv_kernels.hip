@@ -34,6 +34,7 @@
 // (rows+1)*4 + rows*sizeof(y)*(1 + [beta != 0]) plus x: the kernels are
 // HBM-bound streaming kernels, there is no matrix-core work in them.
 #include <cstdlib>
+#include <mutex>
 #include <type_traits>
 
 #include "convert_internal.h"
@@ -1686,6 +1687,40 @@ int RunTyped(const OpsparseSpmvPlan *plan, const SpmvArgs &a)
 
 using namespace opsparse;
 
+// Scratch of opsparse_spmv_csr_launch_noalloc: the merge-path partition, carries and heads of one launch.  Every
+// GPU the library runs on holds its own 4 MiB copy until the process ends.  In host code the array's name is only
+// a stand-in for the symbol; the device address comes from hipGetSymbolAddress, once per device (StaticScratch).
+#define OPSPARSE_NOALLOC_SCRATCH_BYTES (4u << 20)
+static __device__ __align__(256) unsigned char scratch[OPSPARSE_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+
+// Device address of `scratch` on the current device, resolved on the first call there; nullptr on failure.
+void *StaticScratch()
+{
+    static std::mutex lock;
+    static void *ptrOf[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    std::lock_guard<std::mutex> guard(lock);
+    if (ptrOf[dev] == nullptr) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || ptr == nullptr) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        ptrOf[dev] = ptr;
+    }
+    return ptrOf[dev];
+}
+
+}  // namespace
+
 extern "C" {
 
 size_t opsparse_spmv_csr_workspace_bytes(int64_t rows, int64_t nnz)
@@ -2021,6 +2056,34 @@ int opsparse_spmv_csr_launch_zy(const OpsparseSpmvPlan *plan, int32_t transpose,
             break;
     }
     return OPSPARSE_E_UNSUPPORTED;
+}
+
+size_t opsparse_spmv_csr_noalloc_max_bytes(void)
+{
+    return OPSPARSE_NOALLOC_SCRATCH_BYTES;
+}
+
+int opsparse_spmv_csr_launch_noalloc(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
+                                     const void *x, void *y, int64_t rows, int64_t cols, int64_t nnz,
+                                     OpsparseScalar alpha, OpsparseScalar beta, int32_t valType, int32_t outType,
+                                     int32_t computeIsInt, void *stream)
+{
+    if (rows < 0 || cols < 0 || nnz < 0) {
+        return OPSPARSE_E_INVALID;
+    }
+    // The merge-path tables of this matrix must fit the static array: no other kernel family is substituted, so
+    // that a caller learns at once that the matrix is beyond this entry point.
+    if (opsparse_spmv_csr_workspace_bytes(rows, nnz) > OPSPARSE_NOALLOC_SCRATCH_BYTES) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    void *ws = StaticScratch();
+    if (ws == nullptr) {
+        return OPSPARSE_E_LAUNCH;
+    }
+    // Nothing in the tables has to start at zero: the partition kernel writes every partition entry, and the
+    // fix-up kernel reads only carries and heads that the merge kernel of the same launch has written.
+    return opsparse_spmv_csr_launch_zy(nullptr, 0, rowOffsets, colInd, csrValues, x, y, y, rows, cols, nnz, alpha, beta,
+                                       valType, outType, computeIsInt, ws, OPSPARSE_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 int opsparse_spmv_csr_indexed_launch(const void *rowOffsets, int32_t rowOffsetsAre64, int32_t indexBase,
