@@ -1,17 +1,25 @@
 #!/usr/bin/env python3
 """Benchmark of the CSR SpMV / SpMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5|c1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|c2|c3|c4|c5|convert]
 
 A step is one aclsparseSpMV (or aclsparseSpMM) call over one synthetic matrix
-whose arrays are already resident in HBM.  The default workload is c2, the
+whose arrays are already resident in HBM.  The headline workload is c2, the
 5-point 2-D Laplacian on a 2048 x 2048 grid (m = n = 4 194 304, nnz = 20 963 328,
-alpha = 1, beta = 0.5), the configuration the headline metric is quoted on.
-Preprocess runs once before the timed region (its time is reported separately).
+alpha = 1, beta = 0.5), the configuration the headline metric is quoted on; its
+238 MB fit the 256 MB Infinity Cache, so its launches go round three independent
+copies of the operands (the figure on one copy is kept as roofline.warm).  With
+the default --workload all the other measured configurations follow in the same
+run and land in the `workloads` object: c3 (power-law SpMV; default plan and the
+ALG2 layout), c4 (fp32 SpMM) and c5 (fp16 SpMM), each with its own roofline and
+CPU baseline.  Preprocess runs once before the timed region (its time is
+reported separately).  Timing: rounds of K launches between two HIP events on
+the handle's stream, repeated until 50 ms of GPU time; the median round counts.
 
 Prints ONE JSON line: GFLOP/s = 2 * nnz * ncols / t as `value`, the roofline
 object (algorithmic bytes / kernel time against 8 TB/s HBM) and the CPU baseline
 (the reference's CPU golden loop restated in oracle/, timed on this host).
+--workload convert times the CSR producers instead (its own JSON line).
 """
 import argparse
 import ctypes
@@ -97,9 +105,10 @@ def load_traffic(name):
     return int(entry["fetch_kib"] * 1024 * table["fetch_scale"] + entry["write_kib"] * 1024 * table["write_scale"])
 
 
-def cpu_baseline_spmv(cfg, y_gpu, budget_s=15.0):
+def cpu_baseline_spmv(cfg, y_gpu, base=None, budget_s=15.0):
     """The reference's SpmvCpu loop (oracle.spmv_f32), one thread, on the same matrix; the GPU result of one
-    launch (y_gpu) is checked against the fp64-accumulated oracle on the way."""
+    launch (y_gpu) is checked against the fp64-accumulated oracle on the way.  `base` is the result of an earlier
+    call on the same matrix: the CPU timing is taken from it and only the check is repeated."""
     import oracle
     A = cfg["A"]
     rowptr, colind = A["rowptr"].cpu().numpy(), A["colind"].cpu().numpy()
@@ -110,6 +119,8 @@ def cpu_baseline_spmv(cfg, y_gpu, budget_s=15.0):
     err = oracle.max_rel_err(y_gpu.cpu().numpy(), gold)
     if err > 1e-5:
         sys.exit("bench.py: the GPU result differs from the fp64 oracle (max relative error %.3g > 1e-5)" % err)
+    if base is not None:
+        return dict(base, gpu_vs_fp64_oracle_max_rel_err=err)
     oracle.spmv_f32(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])  # warm
     reps, t0 = 0, time.perf_counter()
     while reps < 10 and time.perf_counter() - t0 < budget_s:
@@ -132,7 +143,7 @@ def cpu_baseline_spmv(cfg, y_gpu, budget_s=15.0):
             "gpu_vs_fp64_oracle_max_rel_err": err}
 
 
-def cpu_baseline_spmm(cfg, c_gpu, rows_sample=262144):
+def cpu_baseline_spmm(cfg, c_gpu, base=None, rows_sample=262144):
     """The reference's spmm_csr_cpu loop (order i, j, p) on the first rows_sample rows; the same rows of the GPU
     result of one launch (c_gpu) are checked against the fp64-accumulated oracle on the way."""
     import oracle
@@ -251,13 +262,273 @@ def vendor_yardstick(torch, cfg, is_spmm, flops, bytes_alg, steps, stream, ours)
     return res
 
 
+def time_rounds(torch, stream, launch, steps, restore=None, min_gpu_ms=50.0, min_rounds=5, max_rounds=2000):
+    """Rounds of `steps` back-to-back launches, each between two HIP events recorded on `stream` (the stream the
+    kernels run on), repeated until `min_gpu_ms` of GPU time has been timed.  `launch(i)` gets the running launch
+    number; `restore()` runs before every round, outside the timed region (y back to y0 when beta != 0).
+    Returns per-step milliseconds: (median round, fastest round, mean, number of rounds)."""
+    per_step, total, i = [], 0.0, 0
+    while (total < min_gpu_ms or len(per_step) < min_rounds) and len(per_step) < max_rounds:
+        if restore is not None:
+            restore()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(steps):
+            launch(i)
+            i += 1
+        e1.record(stream)
+        stream.synchronize()
+        ms = e0.elapsed_time(e1)
+        per_step.append(ms / steps)
+        total += ms
+    if os.environ.get("BENCH_LOG_ROUNDS"):
+        log("rounds (ms per step, in order): " + " ".join("%.4f" % v for v in per_step))
+    s = sorted(per_step)
+    return s[len(s) // 2], s[0], sum(s) / len(s), len(s)
+
+
+WORKLOADS = {
+    # key: (generator config, layout)
+    "c2": ("c2", "csr"),
+    "c3": ("c3", "csr"),
+    "c3_alg2": ("c3", "blocked_gather"),
+    "c3_panels": ("c3", "column_panels"),
+    "c4": ("c4", "csr"),
+    "c5": ("c5", "csr"),
+}
+_cfg_cache = {}
+
+
+def make_config(wl, torch, dev, which, scale):
+    """The synthetic operands of one configuration, kept until another configuration is asked for (the two c3
+    entries share one matrix)."""
+    key = (which, scale)
+    if key in _cfg_cache:
+        return _cfg_cache[key]
+    _cfg_cache.clear()
+    torch.cuda.empty_cache()
+    s = scale
+    t_gen = time.perf_counter()
+    if which == "c2":
+        cfg = wl.config_c2(dev, grid=max(8, int(2048 * s ** 0.5)))
+    elif which == "c3":
+        cfg = wl.config_c3(dev, m=max(1024, int(8388608 * s)), lmax=200000 if s >= 0.05 else 2000)
+    elif which == "c4":
+        cfg = wl.config_c4(dev, m=max(1024, int(1048576 * s)))
+    else:
+        cfg = wl.config_c5(dev, m=max(1024, int(2097152 * s)))
+    torch.cuda.synchronize()
+    log("workload %s: rows=%d nnz=%d (generated in %.1f s)"
+        % (cfg["name"], cfg["A"]["rows"], int(cfg["A"]["colind"].numel()), time.perf_counter() - t_gen))
+    _cfg_cache[key] = cfg
+    return cfg
+
+
+def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
+    """One workload: Preprocess once, then rounds of `--steps` calls; returns the fields of its JSON object."""
+    which, layout = WORKLOADS[key]
+    os.environ.pop("OPS_SPARSE_SPMV_NO_BLOCKED", None)
+    if layout == "column_panels":
+        os.environ["OPS_SPARSE_SPMV_NO_BLOCKED"] = "1"
+    cfg = make_config(wl, torch, dev, which, args.scale)
+    A = cfg["A"]
+    rows, cols, nnz = A["rows"], A["cols"], int(A["colind"].numel())
+    is_spmm = "B" in cfg
+    vb = A["values"].element_size()
+    alpha, beta = cfg["alpha"], cfg["beta"]
+    # Operand sets.  A timed loop over ONE set re-reads the same bytes every launch; when they fit the 256 MB
+    # Infinity Cache (c2: 238 MB) part of them never comes from HBM.  The headline of such a workload is therefore
+    # timed over `nsets` independent copies of (A, x, y) used in turn, 3 x 238 MB, and the figure on one set is
+    # kept beside it as `warm`.
+    footprint = sum(t.numel() * t.element_size() for t in (A["rowptr"], A["colind"], A["values"]))
+    footprint += sum(cfg[k].numel() * cfg[k].element_size() for k in ("x", "y0", "B") if k in cfg)
+    nsets = 1 if (footprint > 400e6 or args.warm_only) else 3
+    sets = []
+    t_pre = time.perf_counter()
+    first_use_ms = preprocess_ms = None
+    for s in range(nsets + 1):  # set 0 is built twice: the first build also loads the kernels onto the device
+        if s <= 1:
+            arrs = (A["rowptr"], A["colind"], A["values"])
+        else:
+            arrs = tuple(t.clone() for t in (A["rowptr"], A["colind"], A["values"]))
+        csr = osa.Csr(rows, cols, *arrs)
+        stream.synchronize()
+        t_pre = time.perf_counter()
+        if not is_spmm:
+            x = cfg["x"] if s <= 1 else cfg["x"].clone()
+            y = cfg["y0"].clone()
+            X, Y = osa.DnVec(x), osa.DnVec(y)
+            op = osa.SpmvOp(handle, csr, X, Y, preprocess=not args.no_preprocess,
+                            alg=osa.ACL_SPARSE_SPMV_CSR_ALG2 if layout != "csr" else osa.ACL_SPARSE_SPMV_ALG_DEFAULT)
+            out_t = y
+        else:
+            n = cfg["n"]
+            B = cfg["B"].contiguous() if s <= 1 else cfg["B"].clone()
+            Cmat = torch.zeros(rows, n, dtype=torch.float32, device=dev)
+            op = osa.SpmmOp(handle, csr, osa.DnMat(cols, n, n, B), osa.DnMat(rows, n, n, Cmat))
+            out_t = Cmat
+        stream.synchronize()
+        dt = (time.perf_counter() - t_pre) * 1e3
+        if s == 0:
+            first_use_ms = dt       # includes loading the library's kernels onto the device
+            continue
+        if s == 1:
+            preprocess_ms = dt      # GetBufferSize + buffer allocation + Preprocess: what a second matrix costs
+        sets.append((op, out_t))
+    if not is_spmm:
+        if layout == "blocked_gather" and not osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, 0):
+            layout = "column_panels" if osa.lib().opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz) else "csr"
+        ncols = 1
+        bytes_alg = wl.spmv_bytes_alg(rows, cols, nnz, vb, 4, 4, beta != 0)
+        bytes_gather = wl.spmv_bytes_gather(rows, cols, nnz, vb, 4, 4, beta != 0)
+        dtype = "f32"
+    else:
+        ncols = cfg["n"]
+        eb = cfg["B"].element_size()
+        bytes_alg = wl.spmm_bytes_alg(rows, cols, ncols, nnz, vb, eb, 4, beta != 0)
+        bytes_gather = wl.spmm_bytes_gather(rows, cols, ncols, nnz, vb, eb, 4, beta != 0)
+        dtype = "f32" if vb == 4 else "f16 in, f32 accumulate/out"
+
+    def restore():
+        if beta != 0:  # y back to y0 before every round, outside the timed region
+            for _, t in sets:
+                t.copy_(cfg["y0"])
+
+    restore()
+    sets[0][0](alpha, beta)  # one launch from the initial y / C, kept for the check against the fp64 oracle
+    stream.synchronize()
+    first_result = sets[0][1].clone()
+    for i in range(args.warmup):
+        sets[i % len(sets)][0](alpha, beta)
+    stream.synchronize()
+    ms, ms_min, ms_mean, nrounds = time_rounds(torch, stream, lambda i: sets[i % len(sets)][0](alpha, beta),
+                                               args.steps, restore, args.min_gpu_ms)
+    warm = None
+    if len(sets) > 1:
+        w_ms, w_min, _, _ = time_rounds(torch, stream, lambda i: sets[0][0](alpha, beta), args.steps, restore,
+                                        args.min_gpu_ms)
+        warm = {"ms_per_step": round(w_ms, 6), "ms_per_step_min": round(w_min, 6),
+                "achieved": round(bytes_alg / (w_ms * 1e-3) / 1e9, 1),
+                "frac": round(bytes_alg / (w_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                "what": "every launch on the same operand set (%.0f MB, inside the 256 MB Infinity Cache)"
+                        % (footprint / 1e6)}
+    flops = 2.0 * nnz * ncols
+    gflops = flops / (ms * 1e-3) / 1e9
+    gbps = bytes_alg / (ms * 1e-3) / 1e9
+    log("%-9s %.2f us/step (median of %d rounds of %d; fastest %.2f, mean %.2f), %.1f GFLOP/s, %.1f GB/s algorithmic "
+        "= %.1f%% of 8 TB/s%s"
+        % (key, ms * 1e3, nrounds, args.steps, ms_min * 1e3, ms_mean * 1e3, gflops, gbps, 100 * gbps / HBM_PEAK_GBPS,
+           "; same operands every launch %.2f us = %.1f%%" % (warm["ms_per_step"] * 1e3, 100 * warm["frac"])
+           if warm else ""))
+    traffic = load_traffic(cfg["name"] + ("+" + layout if layout != "csr" else "")) if args.scale == 1.0 else None
+    out = {
+        "value": round(gflops, 2), "unit": "GFLOP/s", "ms_per_step": round(ms, 6),
+        "ms_per_step_min": round(ms_min, 6), "ms_per_step_mean": round(ms_mean, 6), "rounds": nrounds,
+        "dtype": dtype,
+        "config": {"workload": cfg["name"], "rows": rows, "cols": cols, "nnz": nnz, "ncols_dense": ncols,
+                   "alpha": alpha, "beta": beta, "index": "int32", "preprocess_ms": round(preprocess_ms, 3),
+                   "first_use_ms": round(first_use_ms, 3), "preprocessed": not args.no_preprocess, "layout": layout,
+                   "operand_sets": len(sets),
+                   "timing": "median over rounds of `steps` launches between HIP events on the handle's stream, "
+                             "rounds repeated until %.0f ms of GPU time%s" % (
+                                 args.min_gpu_ms, "; y restored to y0 before every round" if beta != 0 else "")},
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                     "traffic": traffic,
+                     "traffic_gbps": round(traffic / (ms * 1e-3) / 1e9, 1) if traffic else None,
+                     "bytes_alg": bytes_alg, "bytes_gather_model": bytes_gather,
+                     # the dense operand counted once per use instead of once: what a row-wise kernel has to move
+                     # when none of its gathers hits a cache (never the headline figure: it credits cache hits)
+                     "gather_model_gbps": round(bytes_gather / (ms * 1e-3) / 1e9, 1)},
+    }
+    if warm:
+        out["roofline"]["warm"] = warm
+    if args.vendor:
+        sets[0][0](alpha, 0.0)
+        stream.synchronize()
+        out["vendor_yardstick"] = vendor_yardstick(torch, cfg, is_spmm, flops, bytes_alg, max(5, args.steps // 4),
+                                                   stream, sets[0][1].clone())
+    if not args.no_cpu:
+        base = cpu_cache.get(which)
+        res = (cpu_baseline_spmm if is_spmm else cpu_baseline_spmv)(cfg, first_result, base)
+        cpu_cache[which] = res
+        out["cpu_baseline"] = res
+        out["gpu_vs_fp64_oracle_max_rel_err"] = res["gpu_vs_fp64_oracle_max_rel_err"]
+    del sets
+    return out
+
+
+def run_convert(args, osa, torch, dev, stream, handle):
+    """The CSR producers (coo2csr, csr2coo, csrsort, csr2csc) on 33.5 M and 21 M entries through the aclsparse
+    entry points; one JSON line with a time and an algorithmic GB/s per operation."""
+    L = osa.lib()
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    res = {}
+    for name, m, n, per in (("uniform32", 1 << 20, 1 << 20, 32), ("lap", 1 << 22, 1 << 22, 5)):
+        m, n = max(1024, int(m * args.scale)), max(1024, int(n * args.scale))
+        g = torch.Generator(device=dev)
+        g.manual_seed(1)
+        nnz = m * per
+        rowptr = (torch.arange(m + 1, device=dev, dtype=torch.int64) * per).to(torch.int32)
+        col = torch.randint(0, n, (nnz,), device=dev, dtype=torch.int32, generator=g)
+        val = torch.rand(nnz, device=dev, generator=g)
+        rowsOut = torch.empty(nnz, dtype=torch.int32, device=dev)
+        ptr2 = torch.empty(m + 1, dtype=torch.int32, device=dev)
+        size = ctypes.c_size_t(0)
+
+        def timed(fn):
+            fn()
+            stream.synchronize()
+            ms, ms_min, _, _ = time_rounds(torch, stream, lambda i: fn(), 3, None, 20.0)
+            return ms
+
+        t = timed(lambda: L.aclsparseXcsr2coo(handle.h, P(rowptr), nnz, m, P(rowsOut), 0))
+        res[name + "_csr2coo"] = {"ms": round(t, 4), "gbps": round(4 * (nnz + m) / t / 1e6, 1)}
+        t = timed(lambda: L.aclsparseXcoo2csr(handle.h, P(rowsOut), nnz, m, P(ptr2), 0))
+        if not torch.equal(ptr2, rowptr):
+            sys.exit("bench.py: coo2csr(csr2coo(rowptr)) != rowptr")
+        res[name + "_coo2csr"] = {"ms": round(t, 4), "gbps": round(4 * (nnz + m) / t / 1e6, 1)}
+        L.aclsparseXcsrsort_bufferSizeExt(handle.h, m, n, nnz, P(rowptr), P(col), ctypes.byref(size))
+        buf = torch.empty(max(16, size.value), dtype=torch.uint8, device=dev)
+        d = ctypes.c_void_p(None)
+        L.aclsparseCreateMatDescr(ctypes.byref(d))
+        perm = torch.arange(nnz, dtype=torch.int32, device=dev)
+        c2 = col.clone()
+        t = timed(lambda: L.aclsparseXcsrsort(handle.h, m, n, nnz, d, P(rowptr), P(c2), P(perm), P(buf)))
+        L.aclsparseDestroyMatDescr(d)
+        res[name + "_csrsort"] = {"ms": round(t, 4), "gbps": round((16 * nnz + 4 * m) / t / 1e6, 1)}
+        cp = torch.empty(n + 1, dtype=torch.int32, device=dev)
+        ri = torch.empty(nnz, dtype=torch.int32, device=dev)
+        cv = torch.empty(nnz, device=dev)
+        a = (handle.h, m, n, nnz, P(val), P(rowptr), P(col), P(cv), P(cp), P(ri), osa.ACL_FLOAT, 1, 0, 0)
+        L.aclsparseCsr2cscEx2_bufferSize(*a, ctypes.byref(size))
+        buf = torch.empty(max(16, size.value), dtype=torch.uint8, device=dev)
+        t = timed(lambda: L.aclsparseCsr2cscEx2(*a, P(buf)))
+        # a checksum of the permutation: the transposed matrix holds the same (row, col, value) triples
+        chk_in = (torch.repeat_interleave(torch.arange(m, device=dev), per).double() * 3 + col.double() * 5).sum()
+        colOf = torch.repeat_interleave(torch.arange(n, device=dev), (cp[1:] - cp[:-1]).long())
+        chk_out = (ri.double() * 3 + colOf.double() * 5).sum()
+        if chk_in.item() != chk_out.item() or not torch.all(ri[1:][colOf[1:] == colOf[:-1]] >= ri[:-1][colOf[1:] == colOf[:-1]]):
+            sys.exit("bench.py: csr2csc result fails its checksum / order check")
+        res[name + "_csr2csc"] = {"ms": round(t, 4), "gbps": round((16 * nnz + 4 * (m + n)) / t / 1e6, 1),
+                                  "workspace_mib": size.value >> 20}
+        log(name, json.dumps({k: v for k, v in res.items() if k.startswith(name)}))
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="all",
+                    choices=["all", "c2", "c3", "c4", "c5", "convert"],
+                    help="all: c2 as the headline plus c3 (default plan and ALG2), c4 and c5 in `workloads`")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
+    ap.add_argument("--min-gpu-ms", type=float, default=50.0,
+                    help="rounds of --steps launches are repeated until this much GPU time has been timed")
+    ap.add_argument("--warm-only", action="store_true",
+                    help="time every launch on one operand set also where that fits the Infinity Cache")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-preprocess", action="store_true", help="SpMV without the Preprocess buffer")
     ap.add_argument("--alg2", action="store_true",
@@ -271,9 +542,6 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
 
-    if args.panels:
-        os.environ["OPS_SPARSE_SPMV_NO_BLOCKED"] = "1"
-    layout = "column_panels" if args.panels else "blocked_gather" if args.alg2 else "csr"
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
@@ -285,118 +553,32 @@ def main():
     torch.cuda.set_stream(stream)  # torch's fills / uploads and the library's kernels on one stream, in order
     handle = osa.Handle(stream)
 
-    t_gen = time.perf_counter()
-    s = args.scale
-    if args.workload == "c2":
-        cfg = wl.config_c2(dev, grid=max(8, int(2048 * s ** 0.5)))
-    elif args.workload == "c3":
-        cfg = wl.config_c3(dev, m=max(1024, int(8388608 * s)), lmax=200000 if s >= 0.05 else 2000)
-    elif args.workload == "c4":
-        cfg = wl.config_c4(dev, m=max(1024, int(1048576 * s)))
-    else:
-        cfg = wl.config_c5(dev, m=max(1024, int(2097152 * s)))
-    torch.cuda.synchronize()
-    A = cfg["A"]
-    rows, cols, nnz = A["rows"], A["cols"], int(A["colind"].numel())
-    log("workload %s: rows=%d nnz=%d (generated in %.1f s)" % (cfg["name"], rows, nnz, time.perf_counter() - t_gen))
+    if args.workload == "convert":
+        print(json.dumps({"metric": "CSR producers, time per call", "unit": "ms", "data": "synthetic",
+                          "operations": run_convert(args, osa, torch, dev, stream, handle)}), flush=True)
+        handle.close()
+        return
 
-    is_spmm = "B" in cfg
-    csr = osa.Csr(rows, cols, A["rowptr"], A["colind"], A["values"])
-    vb = A["values"].element_size()
-    t_pre = time.perf_counter()
-    if not is_spmm:
-        x = cfg["x"]
-        y = cfg["y0"].clone()
-        X, Y = osa.DnVec(x), osa.DnVec(y)
-        op = osa.SpmvOp(handle, csr, X, Y, preprocess=not args.no_preprocess,
-                        alg=osa.ACL_SPARSE_SPMV_CSR_ALG2 if layout != "csr" else osa.ACL_SPARSE_SPMV_ALG_DEFAULT)
-        if layout == "blocked_gather" and not osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, 0):
-            layout = "column_panels" if osa.lib().opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz) else "csr"
-        ncols = 1
-        bytes_alg = wl.spmv_bytes_alg(rows, cols, nnz, vb, x.element_size(), y.element_size(), cfg["beta"] != 0)
-        bytes_gather = wl.spmv_bytes_gather(rows, cols, nnz, vb, x.element_size(), y.element_size(),
-                                            cfg["beta"] != 0)
-        dtype = "f32"
-    else:
-        n = cfg["n"]
-        B = cfg["B"].contiguous()
-        Cmat = torch.zeros(rows, n, dtype=torch.float32, device=dev)
-        Bd = osa.DnMat(cols, n, n, B)
-        Cd = osa.DnMat(rows, n, n, Cmat)
-        op = osa.SpmmOp(handle, csr, Bd, Cd)
-        ncols = n
-        bytes_alg = wl.spmm_bytes_alg(rows, cols, n, nnz, vb, B.element_size(), 4, cfg["beta"] != 0)
-        bytes_gather = wl.spmm_bytes_gather(rows, cols, n, nnz, vb, B.element_size(), 4, cfg["beta"] != 0)
-        dtype = "f32" if vb == 4 else "f16 in, f32 accumulate/out"
-    stream.synchronize()
-    first_use_ms = (time.perf_counter() - t_pre) * 1e3  # includes loading the library's kernels onto the device
-    # the same GetBufferSize + buffer allocation + Preprocess once more, now that the kernels are loaded: what a
-    # second matrix would cost
-    t_pre = time.perf_counter()
-    if not is_spmm:
-        op = osa.SpmvOp(handle, csr, X, Y, preprocess=not args.no_preprocess, alg=op.alg)
-    else:
-        op = osa.SpmmOp(handle, csr, Bd, Cd)
-    stream.synchronize()
-    preprocess_ms = (time.perf_counter() - t_pre) * 1e3
-
-    alpha, beta = cfg["alpha"], cfg["beta"]
-    first_result = None
-    if not args.no_cpu:  # one launch from the initial y / C, kept for the check in the CPU leg
-        op(alpha, beta)
-        stream.synchronize()
-        first_result = (y if not is_spmm else Cmat).clone()
-    for _ in range(args.warmup):
-        op(alpha, beta)
-    stream.synchronize()
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record(stream)
-    for _ in range(args.steps):
-        op(alpha, beta)
-    e1.record(stream)
-    stream.synchronize()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    ms = e0.elapsed_time(e1) / args.steps  # HIP events on the stream the kernels run on
-
-    flops = 2.0 * nnz * ncols
-    gflops = flops / (ms * 1e-3) / 1e9
-    gbps = bytes_alg / (ms * 1e-3) / 1e9
+    head_key = "c2" if args.workload == "all" else args.workload
+    if head_key == "c3" and (args.alg2 or args.panels):
+        head_key = "c3_panels" if args.panels else "c3_alg2"
+    cpu_cache = {}
+    head = run_workload(args, osa, wl, torch, dev, stream, handle, head_key, cpu_cache)
     copy_gbps, read_gbps = measure_yardsticks(osa, torch, dev, stream)
-    log("%.2f us/step (wall %.2f us), %.1f GFLOP/s, %.1f GB/s algorithmic = %.1f%% of 8 TB/s; "
-        "copy kernel %.0f GB/s, read kernel %.0f GB/s"
-        % (ms * 1e3, wall_ms * 1e3, gflops, gbps, 100 * gbps / HBM_PEAK_GBPS, copy_gbps, read_gbps))
+    log("copy kernel %.0f GB/s, read kernel %.0f GB/s" % (copy_gbps, read_gbps))
     if args.gather_probe:
         log("random gathers, G/s: %s" % json.dumps(measure_gather(osa, torch, wl, dev, stream)))
-
-    traffic = load_traffic(cfg["name"] + ("+" + layout if layout != "csr" else "")) if args.scale == 1.0 else None
-    out = {
-        "metric": "SpMV/SpMM GFLOP/s + achieved HBM GB/s (% of MI355X peak), CSR fp32",
-        "value": round(gflops, 2), "unit": "GFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": dtype, "data": "synthetic",
-        "config": {"workload": cfg["name"], "rows": rows, "cols": cols, "nnz": nnz, "ncols_dense": ncols,
-                   "alpha": alpha, "beta": beta, "index": "int32", "preprocess_ms": round(preprocess_ms, 3), "first_use_ms": round(first_use_ms, 3),
-                   "preprocessed": not args.no_preprocess, "layout": layout},
-        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": traffic,
-                     "traffic_gbps": round(traffic / (ms * 1e-3) / 1e9, 1) if traffic else None,
-                     "bytes_alg": bytes_alg, "bytes_gather_model": bytes_gather,
-                     # the dense operand counted once per use instead of once: what a row-wise kernel has to move
-                     # when none of its gathers hits a cache (never the headline figure: it credits cache hits)
-                     "gather_model_gbps": round(bytes_gather / (ms * 1e-3) / 1e9, 1),
-                     "copy_kernel_gbps": round(copy_gbps, 1), "read_kernel_gbps": round(read_gbps, 1)},
-    }
-    if args.vendor:
-        op(alpha, 0.0)
-        stream.synchronize()
-        out["vendor_yardstick"] = vendor_yardstick(torch, cfg, is_spmm, flops, bytes_alg, max(5, args.steps // 4),
-                                                   stream, (y if not is_spmm else Cmat).clone())
-    if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline_spmm(cfg, first_result) if is_spmm else cpu_baseline_spmv(cfg, first_result)
+    head["roofline"]["copy_kernel_gbps"] = round(copy_gbps, 1)
+    head["roofline"]["read_kernel_gbps"] = round(read_gbps, 1)
+    out = {"metric": "SpMV/SpMM GFLOP/s + achieved HBM GB/s (% of MI355X peak), CSR fp32",
+           "value": head.pop("value"), "unit": head.pop("unit"), "n_gpus": 1, "steps": args.steps,
+           "warmup": args.warmup, "ms_per_step": head.pop("ms_per_step"), "higher_is_better": True,
+           "scaling": "weak", "vs_baseline": None, "dtype": head.pop("dtype"), "data": "synthetic"}
+    out.update(head)
+    if args.workload == "all":
+        out["workloads"] = {}
+        for key in ("c3", "c3_alg2", "c4", "c5"):
+            out["workloads"][key] = run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache)
     print(json.dumps(out), flush=True)
     handle.close()
 
