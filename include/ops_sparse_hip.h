@@ -158,8 +158,11 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
  * analysis it re-stores indices AND values in the workspace; launches with the
  * resulting plan ignore the rowOffsets / colInd / csrValues arguments.  Returns
  * OPSPARSE_E_INVALID for a column index outside [0, cols).  Synchronises `stream` once.
+ * Launches touch only the first opsparse_spmv_csr_blocked_resident_bytes() of the workspace; the rest serves the
+ * analysis and may be handed back afterwards (a launch accepts a workspace of at least the resident size).
  */
 size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t transpose);
+size_t opsparse_spmv_csr_blocked_resident_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t transpose);
 int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
                                       int64_t rows, int64_t cols, int64_t nnz, int32_t transpose, void *workspace,
                                       size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream);

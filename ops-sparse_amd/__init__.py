@@ -91,7 +91,8 @@ OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_launch_zy", "opsparse_spmv_csr_indexed_launch",
     "opsparse_spmv_csr_launch_noalloc", "opsparse_spmv_csr_noalloc_max_bytes",
     "opsparse_spmv_csr_panels_workspace_bytes", "opsparse_spmv_csr_panels_analyse",
-    "opsparse_spmv_csr_blocked_workspace_bytes", "opsparse_spmv_csr_blocked_analyse",
+    "opsparse_spmv_csr_blocked_workspace_bytes", "opsparse_spmv_csr_blocked_resident_bytes",
+    "opsparse_spmv_csr_blocked_analyse",
     "opsparse_spmv_csr_gathers_scattered",
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
     "opsparse_dense_restage",
@@ -244,6 +245,8 @@ def lib():
     L.opsparse_spmv_csr_gathers_scattered.argtypes = [vp, vp, i64, i64, i64, vp, sz, ctypes.POINTER(i32), vp]
     L.opsparse_spmv_csr_blocked_workspace_bytes.restype = sz
     L.opsparse_spmv_csr_blocked_workspace_bytes.argtypes = [i64, i64, i64, i32]
+    L.opsparse_spmv_csr_blocked_resident_bytes.restype = sz
+    L.opsparse_spmv_csr_blocked_resident_bytes.argtypes = [i64, i64, i64, i32]
     L.opsparse_spmv_csr_blocked_analyse.restype = ctypes.c_int
     L.opsparse_spmv_csr_blocked_analyse.argtypes = [vp, vp, vp, i64, i64, i64, i32, vp, sz,
                                                     ctypes.POINTER(OpsparseSpmvPlan), vp]

@@ -22,9 +22,10 @@
 //            LDS and streams the block's entries in (block, panel) order:
 //            value and local row index linearly, the gathered xg in one
 //            contiguous piece per (panel, block) chunk.  Chunks are padded to
-//            multiples of 8 positions in that order, so that a lane's 8
-//            consecutive positions share a chunk and all three streams come
-//            as 16-byte loads.  val * xg is exact in fp64; a row's result is
+//            multiples of 8 positions in that order, so that a lane's run of 4
+//            consecutive positions shares a chunk, the streams come as 16- and
+//            8-byte loads and the lanes of a wavefront read neighbouring
+//            pieces.  val * xg is exact in fp64; a row's result is
 //            rounded once when the block is written.  The blocks are started
 //            heaviest first.
 //
@@ -301,6 +302,7 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint1
 
 typedef float Float4U1 __attribute__((ext_vector_type(4), aligned(4)));   // dword-aligned 16-byte load
 typedef uint32_t Uint4 __attribute__((ext_vector_type(4)));
+typedef uint32_t Uint2 __attribute__((ext_vector_type(2)));
 
 // Adds the per-lane sums of a wavefront to acc[key] (key < 0: nothing pending).
 __device__ __forceinline__ void FlushPending(double *acc, int32_t key, double pending)
@@ -332,23 +334,29 @@ __device__ __forceinline__ int ChunkOf(const int32_t *tabD, int32_t P, int32_t p
     return lo;
 }
 
-// What a lane loads for one batch: kLaneEntries consecutive positions of the block.
+// What a lane loads for one batch: kSubBatches runs of kSubEntries consecutive positions of the block, run s
+// at start + s * (64 * kSubEntries) + lane * kSubEntries, so that every load instruction of a wavefront covers
+// one contiguous kilobyte (values, gathered x) or half of one (local rows).
+constexpr int kSubEntries = 4;
+constexpr int kSubBatches = kLaneEntries / kSubEntries;
+constexpr int kSubSpan = kWave * kSubEntries;  // positions one load instruction of a wavefront covers
+
 struct LanePiece {
-    Float4U1 a0, a1, x0, x1;
-    Uint4 rows;
-    bool live;  // false: a lane past the block's end, which re-read the last piece
+    Float4U1 a[kSubBatches], x[kSubBatches];
+    Uint2 rows[kSubBatches];
+    bool live[kSubBatches];  // false: a run past the block's end, which re-read the last run
 };
 
 // One workgroup per row block: y[row] = alpha * sum(val * xg) + beta * yIn[row].
 //
 // In block order every (panel, block) chunk starts on a multiple of kLaneEntries and is padded to one
-// (padding carries the local row kPadRow and the value 0).  A lane takes kLaneEntries consecutive positions
-// per batch, which therefore lie in one chunk: values, local rows and the gathered x all come as 16-byte
-// loads.  tabD[p] is the first block-order position of the block's chunk from panel p, tabDelta[p] the
-// distance from there to the chunk in panel order, groupChunk[g] the chunk of the block's position 64 * g.
-// Two batches are in flight: the next one's loads are issued, unconditionally, before this one is added up.
-// Entries of one row are neighbours: a lane adds its runs up in registers and touches the row's accumulator
-// in LDS once per run; a row that fills whole wavefronts is summed per lane in `pending` and reaches LDS once.
+// (padding carries the local row kPadRow and the value 0).  A lane takes runs of kSubEntries consecutive
+// positions, which therefore lie in one chunk.  tabD[p] is the first block-order position of the block's chunk
+// from panel p, tabDelta[p] the distance from there to the chunk in panel order, groupChunk[g] the chunk of
+// the block's position 64 * g.  Two batches are in flight: the next one's loads are issued, unconditionally,
+// before this one is added up.  Entries of one row are neighbours: a lane adds its runs up in registers and
+// touches the row's accumulator in LDS once per run; a row that fills whole wavefronts is summed per lane in
+// `pending` and reaches LDS once.
 __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
     const float *__restrict__ valD, const float *__restrict__ xg, const uint16_t *__restrict__ rowLocal,
     const int32_t *__restrict__ dstStart, const int32_t *__restrict__ srcStartT, int32_t P,
@@ -378,7 +386,6 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
     const int32_t d0 = tabD[0], d1 = tabD[P];  // both multiples of kLaneEntries
     int32_t groups = (d1 - d0 + kWave - 1) / kWave;
     groups = groups < kMaxGroups ? groups : kMaxGroups;
-    // groupChunk[g] = chunk that holds position d0 + 64 g: every chunk writes the groups that start inside it
     for (int32_t p = tid; p < P; p += kBlkThreads) {
         int32_t g = (tabD[p] - d0 + kWave - 1) / kWave;
         int32_t gEnd = (tabD[p + 1] - d0 + kWave - 1) / kWave;
@@ -393,73 +400,75 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
 
     auto fetch = [&](int32_t start) {
         LanePiece piece;
-        const int32_t mine = start + lane * kLaneEntries;
-        piece.live = mine < d1;
-        const int32_t i0 = piece.live ? mine : d1 - kLaneEntries;
-        // chunk of i0: from the table of every 64th position, at most two bounds further on
-        const int32_t g = (i0 - d0) / kWave;
-        int p = g < groups ? static_cast<int>(groupChunk[g]) : ChunkOf(tabD, P, i0);
-        p += (p + 1 < P && tabD[p + 1] <= i0) ? 1 : 0;
-        p += (p + 1 < P && tabD[p + 1] <= i0) ? 1 : 0;
-        if (__any(p + 1 < P && tabD[p + 1] <= i0)) {  // chunks of a few entries
-            p = ChunkOf(tabD, P, i0);
+#pragma unroll
+        for (int s = 0; s < kSubBatches; ++s) {
+            const int32_t mine = start + s * kSubSpan + lane * kSubEntries;
+            piece.live[s] = mine < d1;
+            const int32_t i0 = piece.live[s] ? mine : d1 - kSubEntries;
+            const int32_t g = (i0 - d0) / kWave;
+            int p = g < groups ? static_cast<int>(groupChunk[g]) : ChunkOf(tabD, P, i0);
+            p += (p + 1 < P && tabD[p + 1] <= i0) ? 1 : 0;
+            p += (p + 1 < P && tabD[p + 1] <= i0) ? 1 : 0;
+            if (__any(p + 1 < P && tabD[p + 1] <= i0)) {
+                p = ChunkOf(tabD, P, i0);
+            }
+            piece.a[s] = __builtin_nontemporal_load(reinterpret_cast<const Float4U1 *>(valD + i0));
+            piece.rows[s] = __builtin_nontemporal_load(reinterpret_cast<const Uint2 *>(rowLocal + i0));
+            piece.x[s] = __builtin_nontemporal_load(reinterpret_cast<const Float4U1 *>(xg + (i0 + tabDelta[p])));
         }
-        const Float4U1 *vp = reinterpret_cast<const Float4U1 *>(valD + i0);
-        const Float4U1 *xp = reinterpret_cast<const Float4U1 *>(xg + (i0 + tabDelta[p]));  // 4-byte aligned only
-        piece.a0 = __builtin_nontemporal_load(vp);
-        piece.a1 = __builtin_nontemporal_load(vp + 1);
-        piece.rows = __builtin_nontemporal_load(reinterpret_cast<const Uint4 *>(rowLocal + i0));
-        piece.x0 = __builtin_nontemporal_load(xp);
-        piece.x1 = __builtin_nontemporal_load(xp + 1);
         return piece;
     };
 
+    int32_t start = d0 + wave * kBatch;
+    LanePiece cur;
+    if (start < d1) {
+        cur = fetch(start);
+    }
     double pending = 0.0;
     int32_t pendingKey = -1;
-    int32_t start = d0 + wave * kBatch;
     if (start < d1) {
-        LanePiece cur = fetch(start);
         while (true) {
-            const LanePiece next = fetch(start + kStride);  // past the end: every lane re-reads the last piece
-            const float av[kLaneEntries] = {cur.a0.x, cur.a0.y, cur.a0.z, cur.a0.w,
-                                            cur.a1.x, cur.a1.y, cur.a1.z, cur.a1.w};
-            const float xv[kLaneEntries] = {cur.x0.x, cur.x0.y, cur.x0.z, cur.x0.w,
-                                            cur.x1.x, cur.x1.y, cur.x1.z, cur.x1.w};
-            const uint32_t rws[4] = {cur.rows.x, cur.rows.y, cur.rows.z, cur.rows.w};
-            int32_t key[kLaneEntries];
-            double t[kLaneEntries];
-            bool same = true;
+            const LanePiece next = fetch(start + kStride);  // past the end: every lane re-reads the last run
 #pragma unroll
-            for (int j = 0; j < kLaneEntries; ++j) {
-                const uint32_t k = (j & 1) ? rws[j / 2] >> 16 : rws[j / 2] & 0xffffu;
-                // padding and lanes past the end carry key -1 and add nothing
-                key[j] = (cur.live && k < kPadRow) ? static_cast<int32_t>(k & (kRowBlockRows - 1)) : -1;
-                t[j] = static_cast<double>(av[j]) * static_cast<double>(xv[j]);
-                same = same && key[j] == key[0];
-            }
-            const int32_t first = __builtin_amdgcn_readfirstlane(key[0]);
-            if (first >= 0 && __all(same && key[0] == first)) {
-                // one row fills the wavefront's batch
-                if (first != pendingKey) {
-                    FlushPending(acc, pendingKey, pending);
-                    pendingKey = first;
-                    pending = 0.0;
+            for (int s = 0; s < kSubBatches; ++s) {
+                const float av[kSubEntries] = {cur.a[s].x, cur.a[s].y, cur.a[s].z, cur.a[s].w};
+                const float xv[kSubEntries] = {cur.x[s].x, cur.x[s].y, cur.x[s].z, cur.x[s].w};
+                const uint32_t rws[2] = {cur.rows[s].x, cur.rows[s].y};
+                int32_t key[kSubEntries];
+                double t[kSubEntries];
+                bool same = true;
+#pragma unroll
+                for (int j = 0; j < kSubEntries; ++j) {
+                    const uint32_t k = (j & 1) ? rws[j / 2] >> 16 : rws[j / 2] & 0xffffu;
+                    // padding and runs past the end carry key -1 and add nothing
+                    key[j] = (cur.live[s] && k < kPadRow) ? static_cast<int32_t>(k & (kRowBlockRows - 1)) : -1;
+                    t[j] = static_cast<double>(av[j]) * static_cast<double>(xv[j]);
+                    same = same && key[j] == key[0];
                 }
-                pending += ((t[0] + t[1]) + (t[2] + t[3])) + ((t[4] + t[5]) + (t[6] + t[7]));
-            } else {
-                double run = t[0];
-#pragma unroll
-                for (int j = 1; j < kLaneEntries; ++j) {
-                    if (key[j] != key[j - 1]) {
-                        if (key[j - 1] >= 0) {
-                            atomicAdd(&acc[key[j - 1]], run);
-                        }
-                        run = 0.0;
+                const int32_t first = __builtin_amdgcn_readfirstlane(key[0]);
+                if (first >= 0 && __all(same && key[0] == first)) {
+                    // one row fills the wavefront's 256 positions
+                    if (first != pendingKey) {
+                        FlushPending(acc, pendingKey, pending);
+                        pendingKey = first;
+                        pending = 0.0;
                     }
-                    run += t[j];
-                }
-                if (key[kLaneEntries - 1] >= 0) {
-                    atomicAdd(&acc[key[kLaneEntries - 1]], run);
+                    pending += (t[0] + t[1]) + (t[2] + t[3]);
+                } else {
+                    double run = t[0];
+#pragma unroll
+                    for (int j = 1; j < kSubEntries; ++j) {
+                        if (key[j] != key[j - 1]) {
+                            if (key[j - 1] >= 0) {
+                                atomicAdd(&acc[key[j - 1]], run);
+                            }
+                            run = 0.0;
+                        }
+                        run += t[j];
+                    }
+                    if (key[kSubEntries - 1] >= 0) {
+                        atomicAdd(&acc[key[kSubEntries - 1]], run);
+                    }
                 }
             }
             start += kStride;
@@ -489,8 +498,9 @@ namespace {
 struct BlockedLayout {
     int32_t P, B, window, passes;
     int64_t padded;  // upper bound of the positions in block order
-    // used by every launch
+    // used by every launch (the first `resident` bytes)
     int64_t colLocalOff, xgOff, valOff, rowLocalOff, srcStartOff, dstStartOff, srcStartTOff, orderOff, blockRowOff;
+    int64_t resident;
     // preprocessing only
     int64_t keys0Off, keys1Off, pos0Off, pos1Off, rowOfPosOff, outPtrOff, tableOff, scratchOff;
     int64_t bytes;
@@ -546,6 +556,7 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     l.srcStartTOff = off; off += align(4 * P * B);
     l.orderOff = off; off += align(4 * B);
     l.blockRowOff = off; off += align(4 * (B + 1));
+    l.resident = off;
     l.keys0Off = off; off += align(4 * nnz);
     l.keys1Off = off; off += align(4 * nnz);
     l.pos0Off = off; off += align(4 * nnz);
@@ -577,7 +588,8 @@ int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
     if (l.P == 0 || plan.numPanels != l.P || plan.numRowBlocks != l.B) {
         return OPSPARSE_E_INVALID;
     }
-    if (a.ws == nullptr || static_cast<int64_t>(a.wsBytes) < l.bytes || plan.bytes != l.bytes) {
+    // a launch touches the first `resident` bytes only: the tail served the analysis and may have been handed back
+    if (a.ws == nullptr || static_cast<int64_t>(a.wsBytes) < l.resident || plan.bytes != l.bytes) {
         return OPSPARSE_E_WORKSPACE;
     }
     auto *base = static_cast<unsigned char *>(a.ws);
@@ -606,6 +618,12 @@ size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int
 {
     return static_cast<size_t>(
         (transpose ? MakeBlockedLayout(cols, rows, nnz, true) : MakeBlockedLayout(rows, cols, nnz, false)).bytes);
+}
+
+size_t opsparse_spmv_csr_blocked_resident_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t transpose)
+{
+    return static_cast<size_t>(
+        (transpose ? MakeBlockedLayout(cols, rows, nnz, true) : MakeBlockedLayout(rows, cols, nnz, false)).resident);
 }
 
 int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
