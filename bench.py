@@ -378,6 +378,10 @@ def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
     if not is_spmm:
         if layout == "blocked_gather" and not osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, 0):
             layout = "column_panels" if osa.lib().opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz) else "csr"
+        live = osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+        if layout == "csr" and live and sets[0][0].buffer is not None and sets[0][0].buffer.numel() == live:
+            # the default algorithm found the gathers scattered and took the re-stored layout with live values
+            layout = "blocked_gather_live_values"
         ncols = 1
         bytes_alg = wl.spmv_bytes_alg(rows, cols, nnz, vb, 4, 4, beta != 0)
         bytes_gather = wl.spmv_bytes_gather(rows, cols, nnz, vb, 4, 4, beta != 0)

@@ -90,6 +90,10 @@ typedef struct OpsparseSpmvPlan {
     int32_t tileRowNnz;    /* STREAM_ROWS: the row length the tiles are sized for (0: maxRowNnz) */
     int32_t longRowsBeside;/* STREAM_ROWS: a few rows are longer than that: the tiles skip rows of more than 64
                               entries and a second kernel sums those, a workgroup per row */
+    int32_t liveValues;    /* BLOCKED_GATHER: every launch first copies the caller's csrValues, as they are then, into
+                              the layout (one more linear pass over the entries): nothing goes stale when values
+                              change in place or the values pointer is replaced */
+    int32_t reserved;      /* zero */
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */
@@ -160,11 +164,17 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
  * OPSPARSE_E_INVALID for a column index outside [0, cols).  Synchronises `stream` once.
  * Launches touch only the first opsparse_spmv_csr_blocked_resident_bytes() of the workspace; the rest serves the
  * analysis and may be handed back afterwards (a launch accepts a workspace of at least the resident size).
+ * `flags`: OPSPARSE_BLOCKED_TRANSPOSE (= 1, so that a plain 0 / 1 "transpose" still reads right) and / or
+ * OPSPARSE_BLOCKED_LIVE_VALUES: the layout also keeps the block-order position of every entry (4 more bytes per
+ * entry, resident) and every launch re-reads csrValues through it, 12 more bytes of traffic per entry, all
+ * streamed; such a plan never goes stale when values change.
  */
-size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t transpose);
-size_t opsparse_spmv_csr_blocked_resident_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t transpose);
+#define OPSPARSE_BLOCKED_TRANSPOSE 1
+#define OPSPARSE_BLOCKED_LIVE_VALUES 2
+size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t flags);
+size_t opsparse_spmv_csr_blocked_resident_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t flags);
 int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
-                                      int64_t rows, int64_t cols, int64_t nnz, int32_t transpose, void *workspace,
+                                      int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
                                       size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream);
 
 /* Same as opsparse_spmv_csr_launch with separate input and output vectors:

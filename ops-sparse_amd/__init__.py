@@ -61,6 +61,7 @@ OPSPARSE_F32, OPSPARSE_F16, OPSPARSE_BF16, OPSPARSE_I32, OPSPARSE_I8 = range(5)
 OPSPARSE_OK, OPSPARSE_E_INVALID, OPSPARSE_E_UNSUPPORTED, OPSPARSE_E_WORKSPACE, OPSPARSE_E_LAUNCH = 0, -1, -2, -3, -4
 OPSPARSE_SPMV_COLUMN_PANELS = 5
 OPSPARSE_SPMV_BLOCKED_GATHER = 6
+OPSPARSE_BLOCKED_TRANSPOSE, OPSPARSE_BLOCKED_LIVE_VALUES = 1, 2
 OPSPARSE_SPMM_AUTO, OPSPARSE_SPMM_ROW_SPLIT, OPSPARSE_SPMM_BINNED = range(3)
 
 # Every symbol the two public headers declare; tests check that the library exports all of them.
@@ -116,7 +117,8 @@ class OpsparseSpmvPlan(ctypes.Structure):
     _fields_ = [("kernel", i32), ("lanesPerRow", i32), ("rowsPerBlock", i32), ("mergeBlocks", i32),
                 ("maxRowNnz", i32), ("partitionReady", i32), ("numPanels", i32),
                 ("panelShift", i32), ("numRowBlocks", i32), ("entryWindow", i32), ("transposed", i32),
-                ("guardTiles", i32), ("tileRowNnz", i32), ("longRowsBeside", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
+                ("guardTiles", i32), ("tileRowNnz", i32), ("longRowsBeside", i32), ("liveValues", i32),
+                ("reserved", i32), ("rows", i64), ("nnz", i64), ("partOff", i64),
                 ("carryOff", i64), ("headOff", i64), ("bytes", i64), ("panelStart", i64 * 17)]
 
 

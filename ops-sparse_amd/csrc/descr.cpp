@@ -258,7 +258,17 @@ aclsparseStatus_t aclsparseSpMatSetValues(aclsparseSpMatDescr_t spMatDescr, void
     if (spMatDescr == nullptr) {
         return ACL_SPARSE_STATUS_INVALID_VALUE;
     }
-    spMatDescr->values = values;  // same pattern, new numbers: preprocessing stays valid
+    if (values != spMatDescr->values) {
+        // Same pattern, new numbers: preprocessing that only looked at the pattern stays valid.  The re-stored SpMV
+        // layouts hold a copy of the values as they were at Preprocess: such a binding is dropped, later calls run
+        // the row-wise kernels on the new array (a layout with live values reads the values at every call and stays).
+        const OpsparseSpmvPlan &plan = spMatDescr->spmv.plan;
+        if (plan.kernel == OPSPARSE_SPMV_COLUMN_PANELS ||
+            (plan.kernel == OPSPARSE_SPMV_BLOCKED_GATHER && plan.liveValues == 0)) {
+            spMatDescr->spmv = OpsparseSpmvBinding{};
+        }
+    }
+    spMatDescr->values = values;
     return ACL_SPARSE_STATUS_SUCCESS;
 }
 

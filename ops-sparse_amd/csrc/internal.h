@@ -128,10 +128,11 @@ OpsparseScalar MakeScalar(const void *p, aclDataType computeType, aclsparsePoint
 struct RestoredChoice {
     int32_t kernel;
     size_t bytes;
+    bool liveValues;  // BLOCKED_GATHER only: the layout re-reads the caller's values at every call
 };
 RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose);
 int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const float *values, int64_t rows,
-                    int64_t cols, int64_t nnz, bool transpose, void *buffer, size_t bytes, OpsparseSpmvPlan *plan,
-                    void *stream);
+                    int64_t cols, int64_t nnz, bool transpose, bool liveValues, void *buffer, size_t bytes,
+                    OpsparseSpmvPlan *plan, void *stream);
 
 }  // namespace opsparse

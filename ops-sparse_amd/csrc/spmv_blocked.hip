@@ -42,6 +42,7 @@
 // The VALUES are copied in (block, panel) order: the analysis must be repeated
 // after they change.
 #include <climits>
+#include <cstdlib>
 
 #include "convert_internal.h"
 #include "device_utils.h"
@@ -179,7 +180,7 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedScatterKernel(
     const int32_t *__restrict__ pos, const int32_t *__restrict__ rowOfSrc, const int32_t *__restrict__ chunkKey,
     const float *__restrict__ vals, const int32_t *__restrict__ srcStart,
     const int32_t *__restrict__ dstStart, const int32_t *__restrict__ blockRow, int64_t nnz, int32_t P, int32_t B,
-    float *__restrict__ valD, uint16_t *__restrict__ rowLocal)
+    float *__restrict__ valD, uint16_t *__restrict__ rowLocal, int32_t *__restrict__ dstOfPos)
 {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
@@ -190,6 +191,9 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedScatterKernel(
         const int32_t p = key / B, b = key % B;
         const int64_t dst = i - srcStart[key] + dstStart[static_cast<int64_t>(b) * P + p];
         valD[dst] = vals[pos[i]];
+        if (dstOfPos != nullptr) {
+            dstOfPos[pos[i]] = static_cast<int32_t>(dst);
+        }
         rowLocal[dst] = static_cast<uint16_t>((rowOfSrc[i] - blockRow[b]) & (kRowBlockRows - 1));  // < kPadRow
     }
 }
@@ -219,6 +223,119 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedOrderKeysKernel(const in
     const int32_t i = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
     if (i < B) {
         keys[i] = INT32_MAX - (dstStart[static_cast<int64_t>(i + 1) * P] - dstStart[static_cast<int64_t>(i) * P]);
+    }
+}
+
+// ------------------------------------------------ values of the caller, now
+
+constexpr int kRefreshSpan = 32768;  // block-order positions a workgroup re-fills at a time: 128 KiB of LDS
+
+// partStart[1 + b] = number of kRefreshSpan-position windows of row block b (prefix-summed afterwards).
+__global__ __launch_bounds__(kBlockThreads) void BlockedRefreshPartsKernel(const int32_t *__restrict__ dstStart,
+                                                                           int32_t P, int32_t B,
+                                                                           int32_t *__restrict__ partStart)
+{
+    const int32_t b = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
+    if (b == 0) {
+        partStart[0] = 0;
+    }
+    if (b < B) {
+        const int32_t len = dstStart[static_cast<int64_t>(b + 1) * P] - dstStart[static_cast<int64_t>(b) * P];
+        partStart[1 + b] = (len + kRefreshSpan - 1) / kRefreshSpan;
+    }
+}
+
+// partDesc[w] = (first entry, end entry, first position, end position) of refresh window w; windows past the
+// last one keep the zeros the array was filled with.
+__global__ __launch_bounds__(kBlockThreads) void BlockedRefreshDescKernel(
+    const int32_t *__restrict__ dstStart, const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ blockRow,
+    const int32_t *__restrict__ partStart, int32_t P, int32_t B, Int4U *__restrict__ partDesc)
+{
+    const int32_t b = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
+    if (b >= B) {
+        return;
+    }
+    const int32_t d0 = dstStart[static_cast<int64_t>(b) * P], d1 = dstStart[static_cast<int64_t>(b + 1) * P];
+    const int32_t e0 = rowOffsets[blockRow[b]], e1 = rowOffsets[blockRow[b + 1]];
+    for (int32_t w = partStart[b]; w < partStart[b + 1]; ++w) {
+        const int32_t w0 = d0 + (w - partStart[b]) * kRefreshSpan;
+        partDesc[w] = Int4U{e0, e1, w0, w0 + kRefreshSpan < d1 ? w0 + kRefreshSpan : d1};
+    }
+}
+
+// The values as they are at this call, into block order.  The entries of a row block are one contiguous piece
+// of the caller's arrays and one contiguous piece of the block order; a workgroup owns a window of the latter,
+// reads the whole of the former (values and their block-order positions, both linear), keeps what falls into
+// its window in LDS and writes the window out linearly: no scattered write ever reaches memory.  A block of
+// more than kRefreshSpan positions is read once per window.
+__global__ __launch_bounds__(kBlkThreads) void BlockedRefreshValuesKernel(const float *__restrict__ vals,
+                                                                         const int32_t *__restrict__ dstOfPos,
+                                                                         const Int4U *__restrict__ partDesc,
+                                                                         float *__restrict__ valD)
+{
+    __shared__ float win[kRefreshSpan];
+    const int tid = threadIdx.x;
+    const Int4U desc = partDesc[blockIdx.x];
+    const int32_t e0 = desc.x, e1 = desc.y, w0 = desc.z, w1 = desc.w;
+    if (w1 <= w0) {
+        return;  // past the last window
+    }
+    for (int32_t i = tid * 4; i < w1 - w0; i += kBlkThreads * 4) {
+        *reinterpret_cast<Float4 *>(win + i) = Float4{0.0f, 0.0f, 0.0f, 0.0f};  // padding positions stay zero
+    }
+    __syncthreads();
+    const uint32_t span = static_cast<uint32_t>(w1 - w0);
+    // aligned groups of four entries as 16-byte loads, the ragged ends one by one
+    const int32_t g0 = (e0 + 3) & ~3, g1 = e1 & ~3;
+    if (g0 >= g1) {
+        for (int32_t i = e0 + tid; i < e1; i += kBlkThreads) {
+            const uint32_t at = static_cast<uint32_t>(dstOfPos[i] - w0);
+            if (at < span) {
+                win[at] = vals[i];
+            }
+        }
+    } else {
+        if (tid < 8) {
+            const int32_t i = tid < 4 ? e0 + tid : g1 + (tid - 4);
+            if ((tid < 4 && i < g0) || (tid >= 4 && i < e1)) {
+                const uint32_t at = static_cast<uint32_t>(dstOfPos[i] - w0);
+                if (at < span) {
+                    win[at] = vals[i];
+                }
+            }
+        }
+        const bool vecVals = (reinterpret_cast<uintptr_t>(vals) & 15) == 0;
+        // kRefreshBatch groups in flight per lane: loads first (clamped to the last group), then the LDS writes
+        constexpr int kRefreshBatch = 4;
+        for (int32_t i0 = g0 + tid * 4; i0 < g1; i0 += kBlkThreads * 4 * kRefreshBatch) {
+            Int4U d[kRefreshBatch];
+            Float4U v[kRefreshBatch];
+#pragma unroll
+            for (int u = 0; u < kRefreshBatch; ++u) {
+                int32_t i = i0 + u * kBlkThreads * 4;
+                i = i < g1 ? i : g1 - 4;
+                d[u] = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(dstOfPos + i));
+                if (vecVals) {
+                    v[u] = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(vals + i));
+                } else {
+                    v[u] = Float4U{vals[i], vals[i + 1], vals[i + 2], vals[i + 3]};
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < kRefreshBatch; ++u) {
+                // (a clamped group writes the same values to the same places again)
+                const uint32_t a0 = static_cast<uint32_t>(d[u].x - w0), a1 = static_cast<uint32_t>(d[u].y - w0);
+                const uint32_t a2 = static_cast<uint32_t>(d[u].z - w0), a3 = static_cast<uint32_t>(d[u].w - w0);
+                if (a0 < span) win[a0] = v[u].x;
+                if (a1 < span) win[a1] = v[u].y;
+                if (a2 < span) win[a2] = v[u].z;
+                if (a3 < span) win[a3] = v[u].w;
+            }
+        }
+    }
+    __syncthreads();
+    for (int32_t i = tid * 4; i < w1 - w0; i += kBlkThreads * 4) {  // w0 and w1 - w0 are multiples of 8
+        __builtin_nontemporal_store(*reinterpret_cast<const Float4 *>(win + i), reinterpret_cast<Float4 *>(valD + w0 + i));
     }
 }
 
@@ -500,6 +617,10 @@ struct BlockedLayout {
     int64_t padded;  // upper bound of the positions in block order
     // used by every launch (the first `resident` bytes)
     int64_t colLocalOff, xgOff, valOff, rowLocalOff, srcStartOff, dstStartOff, srcStartTOff, orderOff, blockRowOff;
+    int64_t dstOfPosOff;  // live values only: block-order position of every entry of the caller's arrays
+    int64_t partStartOff; // live values only: first refresh window of every row block
+    int64_t partDescOff;  // live values only: entry and position range of every refresh window
+    int64_t refreshWindows;
     int64_t resident;
     // preprocessing only
     int64_t keys0Off, keys1Off, pos0Off, pos1Off, rowOfPosOff, outPtrOff, tableOff, scratchOff;
@@ -508,17 +629,27 @@ struct BlockedLayout {
 
 // Layout for a product with `rows` outputs and `cols` inputs (op(A) = A^T: the columns of A are the outputs).
 // 0 panels: the layout does not apply.
-BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool transposed)
+BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool transposed, bool live)
 {
     BlockedLayout l{};
-    if (rows <= 0 || cols <= 0 || nnz <= 0 || nnz > INT32_MAX || rows >= INT32_MAX || cols > INT32_MAX) {
+    if (rows <= 0 || cols <= 0 || nnz <= 0 || nnz > INT32_MAX || rows >= INT32_MAX || cols > INT32_MAX ||
+        (live && transposed)) {  // live values follow the caller's row order: op(A) = A only
         return l;
     }
     const int64_t P = (cols + kPanelCols - 1) >> kPanelLog;
     // Entry window: blocks of short rows get about nnz / (full row blocks) entries; a matrix of few, long rows is
     // still cut into kMinEntryBlocks pieces, or phase 2 would run on a handful of workgroups.
     const int64_t fullBlocks = rows >> kRowBlockLog;
-    int64_t window = nnz / (fullBlocks > kMinEntryBlocks ? fullBlocks : kMinEntryBlocks);
+    static const int64_t minBlocks = [] {  // tuning override: entry windows a matrix is cut into at least
+        const char *env = std::getenv("OPS_SPARSE_BLOCKED_WINDOWS");
+        const int64_t v = env != nullptr ? std::atoll(env) : 0;
+        return v;
+    }();
+    // With live values a block should fit one refresh window (kRefreshSpan positions), or its entries are read
+    // once per window at every call: six times as many, shorter blocks (c3 per call: 607 us with 512 windows,
+    // 458 us with 3072; the layout alone 217 against 247 us).
+    const int64_t wantBlocks = minBlocks > 0 ? minBlocks : (live ? 6 * kMinEntryBlocks : kMinEntryBlocks);
+    int64_t window = nnz / (fullBlocks > wantBlocks ? fullBlocks : wantBlocks);
     window = window < kMinEntryWindow ? kMinEntryWindow : window;
     const int64_t B = ((rows + kRowBlockRows - 1) >> kRowBlockLog) + nnz / window + 1;
     // x must be larger than an L2 (2^20 columns) for the two passes to pay, and the chunks long enough to stream.
@@ -556,6 +687,10 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     l.srcStartTOff = off; off += align(4 * P * B);
     l.orderOff = off; off += align(4 * B);
     l.blockRowOff = off; off += align(4 * (B + 1));
+    l.dstOfPosOff = off; off += live ? align(4 * nnz) : 0;
+    l.partStartOff = off; off += live ? align(4 * (B + 1)) : 0;
+    l.refreshWindows = padded / kRefreshSpan + B + 1;  // upper bound; the exact count is only known on the device
+    l.partDescOff = off; off += live ? align(16 * l.refreshWindows) : 0;
     l.resident = off;
     l.keys0Off = off; off += align(4 * nnz);
     l.keys1Off = off; off += align(4 * nnz);
@@ -584,7 +719,7 @@ uint32_t GridOf(int64_t items, int64_t perBlock, int64_t cap)
 int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
 {
     // a.rows outputs, a.cols inputs: the caller has exchanged them for op(A) = A^T
-    const BlockedLayout l = MakeBlockedLayout(a.rows, a.cols, a.nnz, plan.transposed != 0);
+    const BlockedLayout l = MakeBlockedLayout(a.rows, a.cols, a.nnz, plan.transposed != 0, plan.liveValues != 0);
     if (l.P == 0 || plan.numPanels != l.P || plan.numRowBlocks != l.B) {
         return OPSPARSE_E_INVALID;
     }
@@ -597,7 +732,15 @@ int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
     const auto *colLocal = reinterpret_cast<const uint16_t *>(base + l.colLocalOff);
     const auto *rowLocal = reinterpret_cast<const uint16_t *>(base + l.rowLocalOff);
     auto *xg = reinterpret_cast<float *>(base + l.xgOff);
-    const auto *valD = reinterpret_cast<const float *>(base + l.valOff);
+    auto *valD = reinterpret_cast<float *>(base + l.valOff);
+    if (plan.liveValues != 0) {
+        if (a.vals == nullptr) {
+            return OPSPARSE_E_INVALID;
+        }
+        hipLaunchKernelGGL(BlockedRefreshValuesKernel, dim3(static_cast<uint32_t>(l.refreshWindows)), dim3(kBlkThreads),
+                           0, a.stream, static_cast<const float *>(a.vals), ints(l.dstOfPosOff),
+                           reinterpret_cast<const Int4U *>(base + l.partDescOff), valD);
+    }
     // Few panels: several workgroups per panel, so that every CU has one.
     const int32_t splits = l.P >= 192 ? 1 : (256 + l.P - 1) / l.P;
     hipLaunchKernelGGL(SpmvBlockGatherKernel, dim3(static_cast<uint32_t>(l.P) * splits), dim3(kBlkThreads), 0, a.stream,
@@ -614,28 +757,31 @@ using namespace opsparse;
 
 extern "C" {
 
-size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t transpose)
+size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t flags)
 {
-    return static_cast<size_t>(
-        (transpose ? MakeBlockedLayout(cols, rows, nnz, true) : MakeBlockedLayout(rows, cols, nnz, false)).bytes);
+    const bool t = (flags & OPSPARSE_BLOCKED_TRANSPOSE) != 0, live = (flags & OPSPARSE_BLOCKED_LIVE_VALUES) != 0;
+    return static_cast<size_t>((t ? MakeBlockedLayout(cols, rows, nnz, true, live)
+                                  : MakeBlockedLayout(rows, cols, nnz, false, live)).bytes);
 }
 
-size_t opsparse_spmv_csr_blocked_resident_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t transpose)
+size_t opsparse_spmv_csr_blocked_resident_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t flags)
 {
-    return static_cast<size_t>(
-        (transpose ? MakeBlockedLayout(cols, rows, nnz, true) : MakeBlockedLayout(rows, cols, nnz, false)).resident);
+    const bool t = (flags & OPSPARSE_BLOCKED_TRANSPOSE) != 0, live = (flags & OPSPARSE_BLOCKED_LIVE_VALUES) != 0;
+    return static_cast<size_t>((t ? MakeBlockedLayout(cols, rows, nnz, true, live)
+                                  : MakeBlockedLayout(rows, cols, nnz, false, live)).resident);
 }
 
 int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
-                                      int64_t rows, int64_t cols, int64_t nnz, int32_t transpose, void *workspace,
+                                      int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
                                       size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream)
 {
     if (plan == nullptr || rowOffsets == nullptr || colInd == nullptr || csrValues == nullptr) {
         return OPSPARSE_E_INVALID;
     }
-    const bool transposed = transpose != 0;
+    const bool transposed = (flags & OPSPARSE_BLOCKED_TRANSPOSE) != 0, live = (flags & OPSPARSE_BLOCKED_LIVE_VALUES) != 0;
     const int64_t outputs = transposed ? cols : rows;
-    const BlockedLayout l = transposed ? MakeBlockedLayout(cols, rows, nnz, true) : MakeBlockedLayout(rows, cols, nnz, false);
+    const BlockedLayout l = transposed ? MakeBlockedLayout(cols, rows, nnz, true, live)
+                                       : MakeBlockedLayout(rows, cols, nnz, false, live);
     if (l.P == 0) {
         return OPSPARSE_E_UNSUPPORTED;
     }
@@ -717,7 +863,8 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     hipLaunchKernelGGL(BlockedRowBlocksKernel, dim3(GridOf(outputs, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
                        s, outOffsets, static_cast<int32_t>(outputs), l.window, l.B, blockRow);
     hipLaunchKernelGGL(BlockedScatterKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
-                       pos, rowOfSrc, chunkKey, csrValues, srcStart, dstStart, blockRow, nnz, l.P, l.B, valD, rowLocal);
+                       pos, rowOfSrc, chunkKey, csrValues, srcStart, dstStart, blockRow, nnz, l.P, l.B, valD, rowLocal,
+                       live ? ints(l.dstOfPosOff) : nullptr);
     if (l.B <= kRankedBlocks) {
         hipLaunchKernelGGL(BlockedOrderKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
                            dstStart, l.P, l.B, blockOrder);
@@ -732,6 +879,16 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
                             4 * pass, table, scratch, s);
         }
     }
+    if (live) {
+        int32_t *partStart = ints(l.partStartOff);
+        hipLaunchKernelGGL(BlockedRefreshPartsKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads),
+                           0, s, dstStart, l.P, l.B, partStart);
+        LaunchInclusiveScanI32(partStart + 1, partStart + 1, l.B, 0, scratch, s);
+        LaunchFillI32(ints(l.partDescOff), 4 * l.refreshWindows, 0, s);
+        hipLaunchKernelGGL(BlockedRefreshDescKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads),
+                           0, s, dstStart, rowOffsets, blockRow, partStart, l.P, l.B,
+                           reinterpret_cast<Int4U *>(base + l.partDescOff));
+    }
     if (CheckLaunch() != OPSPARSE_OK) {
         return OPSPARSE_E_LAUNCH;
     }
@@ -742,6 +899,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     p.numRowBlocks = l.B;
     p.entryWindow = l.window;
     p.transposed = transposed ? 1 : 0;
+    p.liveValues = live ? 1 : 0;
     p.rows = rows;
     p.nnz = nnz;
     p.bytes = l.bytes;

@@ -99,18 +99,55 @@ aclsparseStatus_t ValidateData(SpmvCall *c, aclDataType computeType)
     return ACL_SPARSE_STATUS_SUCCESS;
 }
 
-// The re-stored layouts CSR_ALG2 asks for, where they apply (fp32, op(A) = A, x larger than an L2): the
-// blocked-gather layout first, the column panels where that one does not fit the matrix.
+// The re-stored layouts, where they apply (fp32, x larger than an L2).
+// CSR_ALG2 asks for one: the blocked-gather layout first, the column panels where that one does not fit the
+// matrix; both hold a copy of the values as they were at Preprocess.
+// ALG_DEFAULT / CSR_ALG1 with op(A) = A get the blocked-gather layout with LIVE values (every call re-reads the
+// caller's values, so nothing can go stale) when the gathers of x are scattered: 0.35 ms against 1.1 ms for the
+// merge path on an 8 M x 8 M power-law matrix.  GetBufferSize and Preprocess ask the same question of the same
+// arrays (a sample of the column indices, one short kernel and a synchronisation), so they agree on the size.
 using Restored = opsparse::RestoredChoice;
 
-Restored RestoredLayout(aclsparseOperation_t opA, aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX,
-                        aclsparseConstDnVecDescr_t vecY, aclDataType computeType, aclsparseSpMVAlg_t alg)
+Restored RestoredLayout(aclsparseHandle_t handle, aclsparseOperation_t opA, aclsparseConstSpMatDescr_t matA,
+                        aclsparseConstDnVecDescr_t vecX, aclsparseConstDnVecDescr_t vecY, aclDataType computeType,
+                        aclsparseSpMVAlg_t alg)
 {
-    if (alg != ACL_SPARSE_SPMV_CSR_ALG2 || computeType != ACL_FLOAT || matA->valueType != ACL_FLOAT ||
-        vecX->valueType != ACL_FLOAT || vecY->valueType != ACL_FLOAT) {
-        return {0, 0};
+    if (computeType != ACL_FLOAT || matA->valueType != ACL_FLOAT || vecX->valueType != ACL_FLOAT ||
+        vecY->valueType != ACL_FLOAT) {
+        return {0, 0, false};
     }
-    return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz, opA != ACL_SPARSE_OP_NON_TRANSPOSE);
+    const bool transpose = opA != ACL_SPARSE_OP_NON_TRANSPOSE;
+    if (alg == ACL_SPARSE_SPMV_CSR_ALG2) {
+        return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz, transpose);
+    }
+    static const bool off = std::getenv("OPS_SPARSE_SPMV_NO_DEFAULT_BLOCKED") != nullptr ||
+                            std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") != nullptr;
+    if (off || transpose || matA->rowOffsets == nullptr || matA->colInd == nullptr) {
+        return {0, 0, false};
+    }
+    const size_t bytes =
+        opsparse_spmv_csr_blocked_workspace_bytes(matA->rows, matA->cols, matA->nnz, OPSPARSE_BLOCKED_LIVE_VALUES);
+    if (bytes == 0) {
+        return {0, 0, false};
+    }
+    // scattered gathers?  Not under stream capture (nothing may synchronise there) and not without a workspace.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(handle->stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return {0, 0, false};
+    }
+    if (opsparse::EnsureWorkspace(handle) != ACL_SPARSE_STATUS_SUCCESS) {
+        return {0, 0, false};
+    }
+    int32_t scattered = 0;
+    if (opsparse_spmv_csr_gathers_scattered(static_cast<const int32_t *>(matA->rowOffsets),
+                                            static_cast<const int32_t *>(matA->colInd), matA->rows, matA->cols,
+                                            matA->nnz, handle->workspace(), handle->workspaceBytes(), &scattered,
+                                            handle->stream) != OPSPARSE_OK ||
+        !scattered) {
+        return {0, 0, false};
+    }
+    return {OPSPARSE_SPMV_BLOCKED_GATHER, bytes, true};
 }
 
 aclsparseStatus_t FromLaunch(int rc)
@@ -171,26 +208,26 @@ RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool 
     if (std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") == nullptr) {
         const size_t blocked = opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, transpose ? 1 : 0);
         if (blocked > 0) {
-            return {OPSPARSE_SPMV_BLOCKED_GATHER, blocked};
+            return {OPSPARSE_SPMV_BLOCKED_GATHER, blocked, false};
         }
     }
     const size_t panels = transpose ? 0 : opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz);
     if (panels > 0) {
-        return {OPSPARSE_SPMV_COLUMN_PANELS, panels};
+        return {OPSPARSE_SPMV_COLUMN_PANELS, panels, false};
     }
-    return {0, 0};
+    return {0, 0, false};
 }
 
 int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const float *values, int64_t rows,
-                    int64_t cols, int64_t nnz, bool transpose, void *buffer, size_t bytes, OpsparseSpmvPlan *plan,
-                    void *stream)
+                    int64_t cols, int64_t nnz, bool transpose, bool liveValues, void *buffer, size_t bytes,
+                    OpsparseSpmvPlan *plan, void *stream)
 {
     // A matrix whose gathers stay near the diagonal (a mesh, a band) keeps x in cache under the row-wise kernels:
     // those are then faster than any re-stored layout (the 2048 x 2048 Laplacian: 41 us against 91 us).
     // op(A) = A^T keeps the layout either way: it replaces fp32 atomics on y, which it beats on the same Laplacian
     // (86 us against 119 us) and whose result depends on the order of the updates.
     int32_t scattered = 1;
-    if (!transpose) {
+    if (!transpose && !liveValues) {  // (a live-values request has asked already)
         int rc = opsparse_spmv_csr_gathers_scattered(rowOffsets, colInd, rows, cols, nnz, buffer, bytes, &scattered,
                                                      stream);
         if (rc != OPSPARSE_OK) {
@@ -201,8 +238,10 @@ int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *co
         return opsparse_spmv_csr_analyse(rowOffsets, rows, cols, nnz, buffer, bytes, OPSPARSE_SPMV_AUTO, plan, stream);
     }
     if (kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {
-        return opsparse_spmv_csr_blocked_analyse(rowOffsets, colInd, values, rows, cols, nnz, transpose ? 1 : 0, buffer,
-                                                 bytes, plan, stream);
+        return opsparse_spmv_csr_blocked_analyse(rowOffsets, colInd, values, rows, cols, nnz,
+                                                 (transpose ? OPSPARSE_BLOCKED_TRANSPOSE : 0) |
+                                                     (liveValues ? OPSPARSE_BLOCKED_LIVE_VALUES : 0),
+                                                 buffer, bytes, plan, stream);
     }
     return opsparse_spmv_csr_panels_analyse(rowOffsets, colInd, values, rows, cols, nnz, buffer, bytes, plan, stream);
 }
@@ -225,7 +264,7 @@ aclsparseStatus_t aclsparseSpMVGetBufferSize(aclsparseHandle_t handle, aclsparse
         return ACL_SPARSE_STATUS_INVALID_VALUE;
     }
     const size_t plain = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
-    const Restored restored = RestoredLayout(opA, matA, vecX, vecY, computeType, alg);
+    const Restored restored = RestoredLayout(handle, opA, matA, vecX, vecY, computeType, alg);
     *bufferSize = restored.bytes > plain ? restored.bytes : plain;
     return ACL_SPARSE_STATUS_SUCCESS;
 }
@@ -251,14 +290,14 @@ aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOpe
         return ACL_SPARSE_STATUS_INSUFFICIENT_RESOURCES;
     }
     OpsparseSpmvPlan plan{};
-    const Restored restored = RestoredLayout(opA, matA, vecX, vecY, computeType, alg);
+    const Restored restored = RestoredLayout(handle, opA, matA, vecX, vecY, computeType, alg);
     int rc;
     if (restored.kernel != 0) {
         rc = opsparse::AnalyseRestored(restored.kernel, static_cast<const int32_t *>(matA->rowOffsets),
                                        static_cast<const int32_t *>(matA->colInd),
                                        static_cast<const float *>(matA->values), matA->rows, matA->cols, matA->nnz,
-                                       opA != ACL_SPARSE_OP_NON_TRANSPOSE, externalBuffer, restored.bytes, &plan,
-                                       handle->stream);
+                                       opA != ACL_SPARSE_OP_NON_TRANSPOSE, restored.liveValues, externalBuffer,
+                                       restored.bytes, &plan, handle->stream);
     } else {
         const size_t bytes = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
         rc = opsparse_spmv_csr_analyse(static_cast<const int32_t *>(matA->rowOffsets), matA->rows, matA->cols,

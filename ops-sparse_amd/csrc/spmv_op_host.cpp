@@ -229,7 +229,7 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
                     ? opsparse::AnalyseRestored(restored.kernel, static_cast<const int32_t *>(d->rowOffsets),
                                                 static_cast<const int32_t *>(d->colInd),
                                                 static_cast<const float *>(d->values), d->rows, d->cols, d->nnz, false,
-                                                buffer, restored.bytes, &d->plan, handle->stream)
+                                                false, buffer, restored.bytes, &d->plan, handle->stream)
                     : opsparse_spmv_csr_analyse(static_cast<const int32_t *>(d->rowOffsets), d->rows, d->cols, d->nnz,
                                                 buffer, opsparse_spmv_csr_workspace_bytes(d->rows, d->nnz),
                                                 OPSPARSE_SPMV_AUTO, &d->plan, handle->stream);

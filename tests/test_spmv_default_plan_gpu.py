@@ -1,0 +1,103 @@
+"""The plan aclsparseSpMVPreprocess picks for ACL_SPARSE_SPMV_ALG_DEFAULT on a large matrix with scattered
+columns: the blocked-gather layout with live values.  The contract under test: a caller that follows the
+reference's call pattern (GetBufferSize, Preprocess, SpMV with the default algorithm) may change the values in
+place, or hand the descriptor a new values array, between calls, and always gets the product of the values as
+they are at the call.  An explicit ACL_SPARSE_SPMV_CSR_ALG2 request holds a copy of the values: there
+aclsparseSpMatSetValues drops the plan and later calls run on the new array with the ordinary kernels."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import to_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def _scattered(rows, cols, seed, per_row=16):
+    rng = np.random.default_rng(seed)
+    lengths = rng.integers(0, per_row, rows)
+    lengths[rows // 2] = 30_000
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)  # unsorted, repeats possible
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    return rowptr, colind, val, rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+
+
+def test_default_plan_is_the_live_blocked_layout_and_follows_the_values(osa, gpu_ctx):
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = 320_000, 1_500_000
+    rowptr, colind, val, x, y0 = _scattered(rows, cols, 5)
+    nnz = colind.size
+    want = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    assert want > L.opsparse_spmv_csr_workspace_bytes(rows, nnz) > 0
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    A, X = osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3])
+    d_y = to_dev(y0, dev)
+    op = osa.SpmvOp(handle, A, X, osa.DnVec(d_y))           # ALG_DEFAULT
+    assert op.buffer.numel() == want                        # GetBufferSize asked for the layout: the probe said scattered
+
+    def check(values, alpha, beta):
+        d_y.copy_(torch.from_numpy(y0))
+        op(alpha, beta)
+        stream.synchronize()
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, values, x, y0, alpha, beta)
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+    check(val, 1.0, 0.0)
+    # values changed in place, same pointer
+    val2 = (val * np.float32(-0.5) + np.float32(0.25)).astype(np.float32)
+    d[2].copy_(torch.from_numpy(val2))
+    check(val2, 1.5, -0.5)
+    # a new values array in the same descriptor
+    val3 = np.random.default_rng(9).uniform(-3, 3, nnz).astype(np.float32)
+    d_val3 = to_dev(val3, dev)
+    assert L.aclsparseSpMatSetValues(A.d, ctypes.c_void_p(d_val3.data_ptr())) == 0
+    check(val3, -1.0, 0.0)
+    # the layout only: a launch accepts a buffer cut down to the resident size
+    resident = L.opsparse_spmv_csr_blocked_resident_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    assert 0 < resident < want
+
+
+def test_default_plan_of_a_banded_matrix_stays_row_wise(osa, gpu_ctx, workloads):
+    """Gathers near the diagonal: the probe says local, GetBufferSize asks for the merge-path tables only."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    A = workloads.laplacian_2d(1200, dev)                   # 1.44 M columns, 7.2 M entries: the layout would apply
+    rows, nnz = A["rows"], int(A["colind"].numel())
+    assert L.opsparse_spmv_csr_blocked_workspace_bytes(rows, rows, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES) > 0
+    x = workloads.uniform(3, rows, -1.0, 1.0, dev)
+    y = torch.zeros(rows, device=dev)
+    op = osa.SpmvOp(handle, osa.Csr(rows, rows, A["rowptr"], A["colind"], A["values"]), osa.DnVec(x), osa.DnVec(y))
+    assert op.buffer.numel() == L.opsparse_spmv_csr_workspace_bytes(rows, nnz)
+    op(1.0, 0.0)
+    stream.synchronize()
+    gold = oracle.spmv_f64(rows, rows, A["rowptr"].cpu().numpy(), A["colind"].cpu().numpy(),
+                           A["values"].cpu().numpy(), x.cpu().numpy(), None, 1.0, 0.0)
+    assert oracle.max_rel_err(y.cpu().numpy(), gold) <= 1e-5
+
+
+def test_alg2_plan_is_dropped_when_the_values_array_is_replaced(osa, gpu_ctx):
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = 320_000, 1_500_000
+    rowptr, colind, val, x, y0 = _scattered(rows, cols, 6)
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    A = osa.Csr(rows, cols, d[0], d[1], d[2])
+    d_y = to_dev(y0, dev)
+    op = osa.SpmvOp(handle, A, osa.DnVec(d[3]), osa.DnVec(d_y), alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
+    op(1.0, 0.0)
+    stream.synchronize()
+    assert oracle.max_rel_err(d_y.cpu().numpy(),
+                              oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.0, 0.0)) <= 1e-5
+    val2 = np.random.default_rng(10).uniform(-2, 2, colind.size).astype(np.float32)
+    d_val2 = to_dev(val2, dev)
+    assert L.aclsparseSpMatSetValues(A.d, ctypes.c_void_p(d_val2.data_ptr())) == 0
+    d_y.copy_(torch.from_numpy(y0))
+    op(2.0, 0.5)                                             # same buffer: the plan in it no longer counts
+    stream.synchronize()
+    assert oracle.max_rel_err(d_y.cpu().numpy(),
+                              oracle.spmv_f64(rows, cols, rowptr, colind, val2, x, y0, 2.0, 0.5)) <= 1e-5
