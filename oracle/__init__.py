@@ -327,3 +327,55 @@ def ref_convert():
     if _ref_conv is None and os.path.exists(path):
         _ref_conv = ctypes.CDLL(path)
     return _ref_conv
+
+
+# ------------------------------------- the SpMM test programs' seeded generators
+
+def spmm22_seek(outputs=0):
+    """Put the arch22 test program's thread_local std::mt19937(42) where it is after `outputs` engine outputs."""
+    lib().oracle_spmm22_seek(ctypes.c_uint64(int(outputs)))
+
+
+def spmm22_outputs_used():
+    lib().oracle_spmm22_outputs_used.restype = ctypes.c_uint64
+    return int(lib().oracle_spmm22_outputs_used())
+
+
+def spmm22_csr(dist, rows, cols, nnz, store=True):
+    """generate_random_csr (dist 'uniform') / generate_powerlaw_csr ('powerlaw') of test/spmm/arch22/spmm_test.cpp,
+    continuing the engine where the last call (or spmm22_seek) left it.  store=False only moves the engine on and
+    returns the number of entries."""
+    L = lib()
+    L.oracle_spmm22_csr.restype = c_i64
+    power = 1 if dist == "powerlaw" else 0
+    if not store:
+        return int(L.oracle_spmm22_csr(power, ctypes.c_uint64(rows), ctypes.c_uint64(cols), ctypes.c_uint64(nnz), None,
+                                       None, None))
+    cap = max(min(nnz, rows * cols) + rows, 1)  # the power-law recipe may hand out a few entries more than nnz
+    rowptr = np.zeros(rows + 1, np.int32)
+    colind = np.zeros(cap, np.int32)
+    val = np.zeros(cap, np.float32)
+    total = int(L.oracle_spmm22_csr(power, ctypes.c_uint64(rows), ctypes.c_uint64(cols), ctypes.c_uint64(nnz),
+                                    _p(rowptr), _p(colind), _p(val)))
+    if total < 0:
+        raise MemoryError("oracle_spmm22_csr")
+    return rowptr, colind[:total].copy(), val[:total].copy()
+
+
+def glibc_rand_stream(seed, count):
+    out = np.zeros(count, np.int32)
+    lib().oracle_glibc_rand_stream(ctypes.c_uint32(seed), c_i64(count), _p(out))
+    return out
+
+
+def spmm35_random_csr(seed, m, k, nnz):
+    """GenerateRandomCsr of test/spmm/arch35/spmm_test.cpp after std::srand(seed) (glibc's rand())."""
+    L = lib()
+    L.oracle_spmm35_random_csr.restype = c_i64
+    cap = max(min(nnz, m * k), 1)
+    rowptr = np.zeros(max(m, 0) + 1, np.int32)
+    colind = np.zeros(cap, np.int32)
+    val = np.zeros(cap, np.float32)
+    total = int(L.oracle_spmm35_random_csr(ctypes.c_uint32(seed), c_i32(m), c_i32(k), c_i32(nnz), _p(rowptr), _p(colind),
+                                           _p(val)))
+    return rowptr, colind[:total].copy(), val[:total].copy()

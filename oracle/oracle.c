@@ -20,6 +20,13 @@
  *   oracle_mere_mare   hand-computed 3-element vectors
  *   oracle_fill_*      the reference generator itself (oracle/_ref, built
  *        from test/frame/fill.h) where present, and committed fixture hashes
+ *   oracle_spmm22_*    (the arch22 SpMM program's random_col / generate_*_csr)
+ *        a second statement of the same recipe in Python over numpy's MT19937
+ *        stream; row lengths, value formula, Zipf shares and distinctness as
+ *        closed forms; the engine itself is the one pinned by oracle_fill_*
+ *   oracle_glibc_rand_stream / oracle_spmm35_random_csr   the host's own
+ *        libc (srand / rand through ctypes) on eight seeds; row lengths,
+ *        ascending distinct columns, value grid, the first row by hand
  */
 #include <math.h>
 #include <stdint.h>
@@ -672,4 +679,230 @@ void oracle_csr2csc(int64_t m, int64_t n, int64_t nnz, int32_t base, const int32
         }
     }
     free(next);
+}
+
+/* ------------------------------ the SpMM test programs' seeded generators
+ *
+ * arch22 (test/spmm/arch22/spmm_test.cpp:42-131): random_col() draws from ONE
+ * thread_local std::mt19937(42) through a fresh uniform_int_distribution<int>(0,
+ * cols - 1) per call; the engine is never re-seeded, so the inputs of a case depend
+ * on how many engine outputs the cases before it consumed.  The engine lives here
+ * as a process-wide state with a counter of consumed outputs: oracle_spmm22_seek(n)
+ * puts it where the reference's engine is after n outputs (seed 42, discard n).
+ * fill_row_random_cols (:56-74) keeps a row's columns in the order drawn, rejects a
+ * repeat by drawing again (an unordered_set there, a stamp array here: only
+ * membership matters), and sets values[cur] = 0.1f + 0.0001f * cur. */
+static mt19937_t g_spmm22;
+static uint64_t g_spmm22_used = 0;
+static int g_spmm22_ready = 0;
+
+void oracle_spmm22_seek(uint64_t outputs)
+{
+    mt_seed(&g_spmm22, 42u);
+    for (uint64_t i = 0; i < outputs; ++i) {
+        (void)mt_next(&g_spmm22);
+    }
+    g_spmm22_used = outputs;
+    g_spmm22_ready = 1;
+}
+
+uint64_t oracle_spmm22_outputs_used(void)
+{
+    return g_spmm22_used;
+}
+
+/* random_col (:42-51) */
+static int32_t spmm22_random_col(uint64_t cols)
+{
+    if (!g_spmm22_ready) {
+        oracle_spmm22_seek(0);
+    }
+    if (cols == 0) {
+        return 0;
+    }
+    const uint32_t range = (uint32_t)cols;
+    uint64_t product = (uint64_t)mt_next(&g_spmm22) * (uint64_t)range;
+    g_spmm22_used++;
+    uint32_t low = (uint32_t)product;
+    if (low < range) {
+        const uint32_t threshold = (0u - range) % range;
+        while (low < threshold) {
+            product = (uint64_t)mt_next(&g_spmm22) * (uint64_t)range;
+            g_spmm22_used++;
+            low = (uint32_t)product;
+        }
+    }
+    return (int32_t)(product >> 32);
+}
+
+/* fill_row_random_cols (:56-74); stamp[c] == tag marks column c as used in this row */
+static uint64_t spmm22_fill_row(uint64_t row_nnz, uint64_t cols, int32_t *indices, float *values, uint64_t cur,
+                                int64_t *stamp, int64_t tag)
+{
+    for (uint64_t j = 0; j < row_nnz; ++j) {
+        int32_t col;
+        do {
+            col = spmm22_random_col(cols);
+        } while (stamp[col] == tag);
+        stamp[col] = tag;
+        if (indices != NULL) {
+            indices[cur] = col;
+            values[cur] = 0.1f + 0.0001f * (float)cur; /* 0.0001f * cur: cur converts to float first */
+        }
+        cur++;
+    }
+    return cur;
+}
+
+/* generate_random_csr (:76-93) when powerlaw == 0, generate_powerlaw_csr (:98-131) otherwise.  indices ==
+ * NULL: nothing is stored, the engine is only moved on (offsets are still written when given).  Returns the
+ * number of entries, or -1 when memory for the stamp array is short. */
+int64_t oracle_spmm22_csr(int powerlaw, uint64_t rows, uint64_t cols, uint64_t nnz, int32_t *offsets, int32_t *indices,
+                          float *values)
+{
+    if (offsets != NULL) {
+        offsets[0] = 0;
+    }
+    if (rows == 0 || cols == 0) {
+        return 0;
+    }
+    int64_t *stamp = (int64_t *)malloc(sizeof(int64_t) * cols);
+    uint64_t *row_nnz = (uint64_t *)malloc(sizeof(uint64_t) * rows);
+    if (stamp == NULL || row_nnz == NULL) {
+        free(stamp);
+        free(row_nnz);
+        return -1;
+    }
+    for (uint64_t c = 0; c < cols; ++c) {
+        stamp[c] = -1;
+    }
+    if (!powerlaw) {
+        for (uint64_t i = 0; i < rows; ++i) {
+            row_nnz[i] = nnz / rows + (i < nnz % rows ? 1 : 0);
+        }
+    } else {
+        /* Zipf weights 1 / (i + 1), shares truncated, the remainder to the top rows, each capped at cols */
+        double total = 0.0;
+        for (uint64_t i = 0; i < rows; ++i) {
+            total += 1.0 / (double)(i + 1);
+        }
+        uint64_t assigned = 0;
+        for (uint64_t i = 0; i < rows; ++i) {
+            row_nnz[i] = (uint64_t)((double)nnz * (1.0 / (double)(i + 1)) / total);
+            assigned += row_nnz[i];
+        }
+        for (uint64_t i = 0; assigned < nnz && i < rows; ++i) {
+            row_nnz[i]++;
+            assigned++;
+        }
+        for (uint64_t i = 0; i < rows; ++i) {
+            if (row_nnz[i] > cols) {
+                row_nnz[i] = cols;
+            }
+        }
+    }
+    uint64_t cur = 0;
+    for (uint64_t i = 0; i < rows; ++i) {
+        cur = spmm22_fill_row(row_nnz[i], cols, indices, values, cur, stamp, (int64_t)i);
+        if (offsets != NULL) {
+            offsets[i + 1] = (int32_t)cur;
+        }
+    }
+    free(stamp);
+    free(row_nnz);
+    return (int64_t)cur;
+}
+
+/* arch35 (test/spmm/arch35/spmm_test.cpp:91-123, seeds :964-975): std::srand(seed), then per row nnz / m
+ * (+ 1 for the first nnz % m rows, capped at k) distinct columns std::rand() % k collected in a std::set
+ * (so stored ascending), values -5 + 10 * (produced % 10001) / 10000.  std::rand() is glibc's here: the
+ * TYPE_3 additive feedback generator r[i] = r[i-3] + r[i-31] over 32-bit words, seeded by the Lehmer
+ * generator 16807 mod 2^31 - 1, the first 310 outputs dropped, each output shifted right by one. */
+typedef struct {
+    uint32_t r[34];
+    int f, b; /* front and rear positions in the circular table of 31 words */
+    uint32_t t[31];
+} glibc_rand_t;
+
+static void glibc_srand(glibc_rand_t *g, uint32_t seed)
+{
+    int32_t word = (int32_t)(seed == 0 ? 1 : seed);
+    g->t[0] = (uint32_t)word;
+    for (int i = 1; i < 31; ++i) {
+        const int32_t hi = word / 127773, lo = word % 127773;
+        word = 16807 * lo - 2836 * hi;
+        if (word < 0) {
+            word += 2147483647;
+        }
+        g->t[i] = (uint32_t)word;
+    }
+    g->f = 3;
+    g->b = 0;
+    for (int i = 0; i < 310; ++i) {
+        g->t[g->f] += g->t[g->b];
+        g->f = (g->f + 1) % 31;
+        g->b = (g->b + 1) % 31;
+    }
+}
+
+static int32_t glibc_rand(glibc_rand_t *g)
+{
+    g->t[g->f] += g->t[g->b];
+    const int32_t out = (int32_t)(g->t[g->f] >> 1);
+    g->f = (g->f + 1) % 31;
+    g->b = (g->b + 1) % 31;
+    return out;
+}
+
+/* The first `count` outputs of std::rand() after std::srand(seed) (glibc). */
+void oracle_glibc_rand_stream(uint32_t seed, int64_t count, int32_t *out)
+{
+    glibc_rand_t g;
+    glibc_srand(&g, seed);
+    for (int64_t i = 0; i < count; ++i) {
+        out[i] = glibc_rand(&g);
+    }
+}
+
+int64_t oracle_spmm35_random_csr(uint32_t seed, int32_t m, int32_t k, int32_t nnz, int32_t *row_off, int32_t *col_ind,
+                                 float *vals)
+{
+    for (int32_t i = 0; i <= (m > 0 ? m : 0); ++i) {
+        row_off[i] = 0;
+    }
+    if (m <= 0 || k <= 0) {
+        return 0;
+    }
+    glibc_rand_t g;
+    glibc_srand(&g, seed);
+    unsigned char *picked = (unsigned char *)calloc((size_t)k, 1);
+    if (picked == NULL) {
+        return -1;
+    }
+    int32_t produced = 0;
+    for (int32_t i = 0; i < m; ++i) {
+        int32_t row_nnz = nnz / m + (i < (nnz % m) ? 1 : 0);
+        if (row_nnz > k) {
+            row_nnz = k;
+        }
+        int32_t have = 0;
+        while (have < row_nnz) {
+            const int32_t c = glibc_rand(&g) % k;
+            if (!picked[c]) {
+                picked[c] = 1;
+                have++;
+            }
+        }
+        for (int32_t c = 0; c < k; ++c) { /* a std::set iterates in ascending order */
+            if (picked[c]) {
+                picked[c] = 0;
+                col_ind[produced] = c;
+                vals[produced] = -5.0f + 10.0f * (float)(produced % 10001) / 10000.0f;
+                produced++;
+            }
+        }
+        row_off[i + 1] = produced;
+    }
+    free(picked);
+    return produced;
 }

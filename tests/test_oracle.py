@@ -306,3 +306,101 @@ def test_c1_structure():
     c = colind.reshape(4096, 16)
     assert np.all(np.diff(c, axis=1) > 0) and c.min() >= 0 and c.max() < 4096
     assert np.all(np.abs(val) <= 1.0)
+
+
+# ------------------------------------------- the SpMM test programs' seeded generators
+
+def _lemire(raw, rng_range):
+    """libstdc++'s uniform_int_distribution on a 32-bit engine, from an iterator of raw engine outputs."""
+    while True:
+        product = int(next(raw)) * rng_range
+        low = product & 0xFFFFFFFF
+        if low >= rng_range or low >= ((1 << 32) - rng_range) % rng_range:
+            return product >> 32
+
+
+def _python_spmm22(rows, cols, nnz, raw):
+    """generate_random_csr of the arch22 SpMM test program, written again in Python over numpy's MT19937 stream
+    (RandomState(42) seeds like std::mt19937(42)): an independent second statement for small cases."""
+    offsets, indices = [0], []
+    for i in range(rows):
+        used = set()
+        for _ in range(nnz // rows + (1 if i < nnz % rows else 0)):
+            col = _lemire(raw, cols)
+            while col in used:
+                col = _lemire(raw, cols)
+            used.add(col)
+            indices.append(col)
+        offsets.append(len(indices))
+    return np.array(offsets, np.int32), np.array(indices, np.int32)
+
+
+def test_spmm22_generator_against_a_second_statement_and_its_invariants():
+    raw = iter(np.random.RandomState(42).randint(0, 2 ** 32, size=200000, dtype=np.uint64))
+    oracle.spmm22_seek(0)
+    for rows, cols, nnz in ((16, 16, 128), (7, 300, 100), (40, 40, 1000), (3, 5, 15)):  # one engine, never re-seeded
+        want_ptr, want_col = _python_spmm22(rows, cols, nnz, raw)
+        ptr, col, val = oracle.spmm22_csr("uniform", rows, cols, nnz)
+        assert np.array_equal(ptr, want_ptr) and np.array_equal(col, want_col)
+        assert np.array_equal(np.diff(ptr), [nnz // rows + (i < nnz % rows) for i in range(rows)])
+        assert np.array_equal(val, np.float32(0.1) + np.float32(0.0001) * np.arange(nnz, dtype=np.float32))
+    used = oracle.spmm22_outputs_used()
+    # the engine position is what seek() reproduces: the same case again from that position gives the same matrix
+    a = oracle.spmm22_csr("powerlaw", 50, 64, 900)
+    oracle.spmm22_seek(used)
+    b = oracle.spmm22_csr("powerlaw", 50, 64, 900)
+    assert all(np.array_equal(x, y) for x, y in zip(a, b))
+    # store=False moves the engine exactly as far
+    after = oracle.spmm22_outputs_used()
+    oracle.spmm22_seek(used)
+    assert oracle.spmm22_csr("powerlaw", 50, 64, 900, store=False) == a[1].size and oracle.spmm22_outputs_used() == after
+    # Zipf shares: truncated nnz * (1 / (i + 1)) / H, the remainder one each to the top rows, capped at the columns
+    ptr, col, _ = a
+    w = 1.0 / np.arange(1, 51)
+    share = (900 * w / w.sum()).astype(np.int64)
+    share[: 900 - share.sum()] += 1
+    assert np.array_equal(np.diff(ptr), np.minimum(share, 64))
+    assert all(np.unique(col[ptr[r]:ptr[r + 1]]).size == ptr[r + 1] - ptr[r] for r in range(50))
+
+
+def test_spmm22_case_table_positions_are_those_of_the_generators():
+    """The engine_outputs_before column of the committed case table, recomputed for the leading cases."""
+    import csv
+    import os
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "spmm_arch22_cases.csv")) as f:
+        cases = list(csv.DictReader(f))
+    assert len(cases) == 200 and cases[0]["engine_outputs_before"] == "0"
+    oracle.spmm22_seek(0)
+    for c in cases[:25]:
+        assert oracle.spmm22_outputs_used() == int(c["engine_outputs_before"])
+        oracle.spmm22_csr(c["dist"], int(c["m"]), int(c["k"]), int(c["nnz"]), store=False)
+
+
+def test_glibc_rand_restated_against_this_hosts_libc():
+    """std::rand() of the arch35 SpMM test program is glibc's: the restatement against the C library itself."""
+    import ctypes
+    libc = ctypes.CDLL("libc.so.6")
+    for seed in (42, 43, 44, 45, 46, 1, 0, 2 ** 31 + 5):
+        libc.srand(ctypes.c_uint(seed))
+        assert [libc.rand() for _ in range(2000)] == list(oracle.glibc_rand_stream(seed, 2000))
+
+
+def test_spmm35_generator_invariants():
+    for seed, m, k, nnz in ((42, 256, 256, 6553), (46, 32, 32, 80), (7, 5, 3, 100)):
+        ptr, col, val = oracle.spmm35_random_csr(seed, m, k, nnz)
+        lengths = np.minimum([nnz // m + (i < nnz % m) for i in range(m)], k)
+        assert np.array_equal(np.diff(ptr), lengths)
+        assert all(np.all(np.diff(col[ptr[r]:ptr[r + 1]]) > 0) for r in range(m))     # a std::set: ascending, distinct
+        assert col.min() >= 0 and col.max() < k
+        want = np.float32(-5.0) + np.float32(10.0) * (np.arange(col.size) % 10001).astype(np.float32) / np.float32(1e4)
+        assert np.array_equal(val, want)
+    # first row of seed 42: the first distinct values of rand() % 256, sorted
+    stream = oracle.glibc_rand_stream(42, 400) % 256
+    first = []
+    for c in stream:
+        if c not in first:
+            first.append(int(c))
+        if len(first) == 6553 // 256 + 1:
+            break
+    ptr, col, _ = oracle.spmm35_random_csr(42, 256, 256, 6553)
+    assert list(col[: ptr[1]]) == sorted(first)

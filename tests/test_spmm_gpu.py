@@ -23,14 +23,16 @@ from helpers import csr_from_lengths, random_csr, run_spmm, to_dev
 pytestmark = pytest.mark.gpu
 
 
-def glibc_free_random_csr(m, k, nnz, seed):
-    """Shape of the reference's GenerateRandomCsr (spmm_test.cpp:91-123): nnz spread
-    evenly over the rows, distinct sorted columns, values on a fixed grid in [-5, 5]."""
-    rng = np.random.default_rng(seed)
-    lengths = np.array([min(nnz // m + (1 if i < nnz % m else 0), k) for i in range(m)])
-    rowptr, colind, _ = csr_from_lengths(lengths, k, seed)
-    val = (-5.0 + 10.0 * (np.arange(colind.size) % 10001) / 10000.0).astype(np.float32)
-    return rowptr, colind, val
+def reference_random_csr(m, k, nnz, seed):
+    """The reference's GenerateRandomCsr after std::srand(seed) (spmm_test.cpp:91-123, seeds :964-975 and :995),
+    restated in oracle/: the same matrix the reference's program multiplies."""
+    return oracle.spmm35_random_csr(seed, m, k, nnz)
+
+
+def reference_dense(count):
+    """The fill of B (and of C when beta != 0) in that program: -5 + 10 * (i % 10001) / 10000 (:406-415)."""
+    i = (np.arange(count) % 10001).astype(np.float32)
+    return (np.float32(-5.0) + np.float32(10.0) * i / np.float32(10000.0)).astype(np.float32)
 
 
 def check_fp32(got, m, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta, **layout):
@@ -75,14 +77,15 @@ REF_CASES = [
 @pytest.mark.parametrize("name,m,k,n,nnz,alpha,beta,trans_b,b_rm,c_rm,seed", REF_CASES)
 def test_reference_fp32_cases(osa, gpu_ctx, name, m, k, n, nnz, alpha, beta, trans_b, b_rm, c_rm, seed):
     nnz = nnz if nnz > 0 else m * k // 10
-    rowptr, colind, val = glibc_free_random_csr(m, k, nnz, seed)
+    rowptr, colind, val = reference_random_csr(m, k, nnz, seed)
     ldb = n if b_rm else k
     ldc = n if c_rm else m
-    rng = np.random.default_rng(seed)
-    B = rng.uniform(-1, 1, k * ldb).astype(np.float32)
-    C0 = rng.uniform(-1, 1, (m if c_rm else n) * ldc).astype(np.float32)
+    # B has k * ldb elements and C m * ldc, as that program sizes them (:406, :410): with op(B) = B^T or
+    # column-major storage that is more than the product touches
+    B = reference_dense(k * ldb)
+    C0 = reference_dense(m * ldc)
     if beta == 0.0:
-        C0[:] = np.nan  # must not be read
+        C0[:] = np.nan  # the program zero-fills C then; here: must not be read
     got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta,
                    order_b=osa.ACL_SPARSE_ORDER_ROW if b_rm else osa.ACL_SPARSE_ORDER_COL,
                    order_c=osa.ACL_SPARSE_ORDER_ROW if c_rm else osa.ACL_SPARSE_ORDER_COL,
@@ -90,7 +93,12 @@ def test_reference_fp32_cases(osa, gpu_ctx, name, m, k, n, nnz, alpha, beta, tra
     C0z = np.zeros_like(C0) if beta == 0.0 else C0
     gold = oracle.spmm_f64(m, n, rowptr, colind, val, B, ldb, C0z, ldc, alpha, beta, b_row_major=b_rm,
                            trans_b=trans_b, c_row_major=c_rm)
-    assert oracle.max_rel_err(got, gold) <= 1e-5
+    used = (np.arange(m)[:, None] * ldc + np.arange(n)[None, :]) if c_rm else \
+        (np.arange(n)[None, :] * ldc + np.arange(m)[:, None])
+    assert oracle.max_rel_err(got[used], gold[used]) <= 1e-5
+    rest = np.ones(got.size, bool)
+    rest[used.ravel()] = False
+    assert np.array_equal(got[rest].view(np.uint32), C0[rest].view(np.uint32))  # what lies beyond C stays as it was
 
 
 @pytest.mark.parametrize("n", [1, 3, 8, 17, 32, 64, 100, 128, 256, 260])
@@ -152,7 +160,7 @@ def test_high_precision_alg_same_result(osa, gpu_ctx):
 
 
 def _fp16_inputs(m, k, n, seed):
-    rowptr, colind, val = glibc_free_random_csr(m, k, m * k // 10, seed)
+    rowptr, colind, val = reference_random_csr(m, k, m * k // 10, seed)
     rng = np.random.default_rng(seed)
     B = rng.uniform(-1, 1, k * n).astype(np.float32)
     C0 = rng.uniform(-1, 1, m * n).astype(np.float32)
@@ -197,7 +205,7 @@ def test_fp16_in_fp32_out(osa, gpu_ctx):
 def test_int8_exact(osa, gpu_ctx, alpha, beta):
     import torch
     m, k, n = 256, 256, 64
-    rowptr, colind, _ = glibc_free_random_csr(m, k, m * k // 10, 49)
+    rowptr, colind, _ = reference_random_csr(m, k, m * k // 10, 49)
     rng = np.random.default_rng(49)
     val = rng.integers(-128, 128, colind.size).astype(np.int8)
     B = rng.integers(-128, 128, k * n).astype(np.int8)

@@ -1,11 +1,12 @@
 """The case table of the reference's arch22 SpMM test program, row by row, through the three-step aclsparseSpMM API.
 
 tests/golden/spmm_arch22_cases.csv holds kTestCases of test/spmm/arch22/spmm_test.cpp:446- (M, K, N, nnz, alpha,
-beta, row distribution: 200 rows from 16 x 16 to 65 536 x 65 536 with 16.7 M entries).  Every case is built the way
-that program builds it (:42-131, :376-383): `uniform` gives every row nnz / M entries (the first nnz % M one more),
-`powerlaw` shares nnz out by Zipf weights 1 / (row + 1), capped at K; distinct random columns in the order drawn
-(not sorted); values 0.1 + 0.0001 * position; B[i] = 0.5 + 0.0001 * (i % 1000), C[i] = 0.01 * (i % 100), both
-compact row-major.  Judged by that program's rule (verify_result, :149-170, called with 1e-3 / 1e-3: an element fails
+beta, row distribution: 200 rows from 16 x 16 to 65 536 x 65 536 with 16.7 M entries, and the number of engine
+outputs the program has used when it reaches the row).  Every case is built by that program's own generators
+(:42-131, :376-383), restated in oracle/ with their seeded engine, so the inputs are the reference's: `uniform` gives
+every row nnz / M entries (the first nnz % M one more), `powerlaw` shares nnz out by Zipf weights 1 / (row + 1),
+capped at K; distinct random columns in the order drawn (not sorted); values 0.1 + 0.0001 * position;
+B[i] = 0.5 + 0.0001 * (i % 1000), C[i] = 0.01 * (i % 100), both compact row-major.  Judged by that program's rule (verify_result, :149-170, called with 1e-3 / 1e-3: an element fails
 when it is off by more than 1e-3 absolutely AND relatively) against its fp32 golden (spmm_csr_cpu, :132-147), and by
 this build's bar, 1e-5 per element against the fp64-accumulated oracle, on the leading rows (all of them unless the
 case is large: the oracle is a CPU loop).
@@ -26,41 +27,14 @@ with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "sp
     CASES = list(csv.DictReader(f))
 
 
-def _matrix(m, k, nnz, dist, dev, seed):
-    """Row lengths by the reference's two recipes; distinct uniformly random columns per row in the order drawn.
-    Drawn with torch on `dev` (the largest case has 16.7 M entries): every entry gets a random column, entries that
-    repeat an earlier column of their row are drawn again until none is left; rows that fill more than a sixteenth
-    of the columns take the head of a random permutation instead."""
-    if dist == "uniform":
-        lengths = np.full(m, nnz // m, np.int64)
-        lengths[: nnz % m] += 1
-    else:
-        weight = 1.0 / np.arange(1, m + 1, dtype=np.float64)
-        lengths = (nnz * weight / weight.sum()).astype(np.int64)
-        lengths[: max(0, min(m, nnz - int(lengths.sum())))] += 1
-    lengths = np.minimum(lengths, k)
-    rowptr = np.concatenate([[0], np.cumsum(lengths)])
-    total = int(rowptr[-1])
-    gen = torch.Generator(device=dev)
-    gen.manual_seed(seed)
-    row_of = torch.repeat_interleave(torch.arange(m, device=dev), torch.from_numpy(lengths).to(dev))
-    col = torch.randint(0, k, (total,), generator=gen, device=dev)
-    crowded = 16 * lengths > k
-    for r in np.nonzero(crowded)[0]:
-        col[rowptr[r]:rowptr[r + 1]] = torch.randperm(k, generator=gen, device=dev)[: int(lengths[r])]
-    redraw = ~torch.from_numpy(crowded).to(dev)[row_of]
-    while True:
-        keys, order = torch.sort(row_of * k + col, stable=True)
-        later = torch.zeros(total, dtype=torch.bool, device=dev)
-        later[1:] = keys[1:] == keys[:-1]
-        again = order[later]
-        again = again[redraw[again]]
-        if again.numel() == 0:
-            break
-        col[again] = torch.randint(0, k, (again.numel(),), generator=gen, device=dev)
-    colind = col.to(torch.int32).cpu().numpy()
-    val = np.float32(0.1) + np.float32(0.0001) * np.arange(total, dtype=np.float32)
-    return rowptr.astype(np.int32), colind, val
+def _matrix(c):
+    """The matrix the reference's program builds for this row of its table: its generators restated in oracle/
+    (generate_random_csr / generate_powerlaw_csr over random_col's engine), the engine put where the program's is
+    when it reaches the case — cases that run in table order continue it, any other order seeks."""
+    before = int(c["engine_outputs_before"])
+    if oracle.spmm22_outputs_used() != before:
+        oracle.spmm22_seek(before)
+    return oracle.spmm22_csr(c["dist"], int(c["m"]), int(c["k"]), int(c["nnz"]))
 
 
 def _rows_within(rowptr, n, budget, from_end=False):
@@ -77,7 +51,7 @@ def test_reference_arch22_case(osa, gpu_ctx, c):
     m, k, n, nnz = int(c["m"]), int(c["k"]), int(c["n"]), int(c["nnz"])
     alpha, beta = float(c["alpha"]), float(c["beta"])
     dev = gpu_ctx[0]
-    rowptr, colind, val = _matrix(m, k, nnz, c["dist"], dev, m * 7 + k * 3 + n + nnz)
+    rowptr, colind, val = _matrix(c)
     lengths = np.diff(rowptr)
     assert all(np.unique(colind[rowptr[r]:rowptr[r + 1]]).size == lengths[r] for r in (0, m // 2, m - 1))
     B = (np.float32(0.5) + np.float32(0.0001) * (np.arange(k * n) % 1000).astype(np.float32)).astype(np.float32)
