@@ -1,8 +1,10 @@
 // Small C++ test frame over HIP for callers written against cann_ops_sparse.h:
 // RAII owners for the stream, the aclsparse handle, device arrays and
-// descriptors, a CSV case-table loader and a seeded CSR generator.  It plays the
-// role of the reference's test/frame (descriptor_manager.h, sparse_test.h,
-// csv_loader.h, fill.h) for the case tables kept under tests/golden/, without
+// descriptors, a CSV case-table loader with typed case parameters, the
+// verification rules (absolute, relative, MERE / MARE, exact, integer) and a
+// seeded CSR generator.  It plays the role of the reference's test/frame
+// (descriptor_manager.h, sparse_test.h, csv_loader.h:125-136, verify.h:28-196,
+// types.h:18-60, fill.h) for the case tables kept under tests/golden/, without
 // GoogleTest: a test program is a plain main() that prints one line per case.
 // Test infrastructure only; links libops_sparse.so and (as the checker)
 // oracle/liboracle.so.
@@ -11,6 +13,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -33,6 +36,7 @@ void oracle_coo2csr(const int32_t *rowInd, int64_t nnz, int64_t m, int32_t base,
 void oracle_csr2coo(const int32_t *rowPtr, int64_t m, int64_t nnz, int32_t base, int32_t *rowInd);
 void oracle_csr2csc(int64_t m, int64_t n, int64_t nnz, int32_t base, const int32_t *rowPtr, const int32_t *colInd,
                     const void *val, int32_t valBytes, int32_t *colPtr, int32_t *rowInd, void *cscVal);
+void oracle_csrsort(const int32_t *rowPtr, int64_t m, int32_t base, int32_t *colInd, int32_t *perm);
 }
 
 namespace frame {
@@ -119,6 +123,146 @@ private:
     size_t n_ = 0;
 };
 
+// Owners of the API's descriptors, in the shape of the reference's SpMatManager / DnVecManager
+// (test/frame/descriptor_manager.h:22-60, :190-): a static creator per format, get(), destroyed with the owner.
+class SpMat {
+public:
+    SpMat() = default;
+    static SpMat createCsr(int64_t rows, int64_t cols, int64_t nnz, void *rowOffsets, void *colIndices, void *values,
+                           aclsparseIndexType_t rowOffsetType = ACL_SPARSE_INDEX_32I,
+                           aclsparseIndexType_t colIdxType = ACL_SPARSE_INDEX_32I,
+                           aclsparseIndexBase_t idxBase = ACL_SPARSE_INDEX_BASE_ZERO, aclDataType valueType = ACL_FLOAT)
+    {
+        SpMat m;
+        Check(aclsparseCreateCsr(&m.d_, rows, cols, nnz, rowOffsets, colIndices, values, rowOffsetType, colIdxType,
+                                 idxBase, valueType), "aclsparseCreateCsr");
+        return m;
+    }
+    ~SpMat() { if (d_ != nullptr) { (void)aclsparseDestroySpMat(d_); } }
+    SpMat(const SpMat &) = delete;
+    SpMat &operator=(const SpMat &) = delete;
+    SpMat(SpMat &&o) noexcept : d_(o.d_) { o.d_ = nullptr; }
+    aclsparseSpMatDescr_t get() const { return d_; }
+
+private:
+    aclsparseSpMatDescr_t d_ = nullptr;
+};
+
+class DnVec {
+public:
+    DnVec() = default;
+    static DnVec create(int64_t size, void *values, aclDataType valueType = ACL_FLOAT)
+    {
+        DnVec v;
+        Check(aclsparseCreateDnVec(&v.d_, size, values, valueType), "aclsparseCreateDnVec");
+        return v;
+    }
+    ~DnVec() { if (d_ != nullptr) { (void)aclsparseDestroyDnVec(d_); } }
+    DnVec(const DnVec &) = delete;
+    DnVec &operator=(const DnVec &) = delete;
+    DnVec(DnVec &&o) noexcept : d_(o.d_) { o.d_ = nullptr; }
+    aclsparseDnVecDescr_t get() const { return d_; }
+
+private:
+    aclsparseDnVecDescr_t d_ = nullptr;
+};
+
+// ------------------------------------------------------------ verification
+// The reference's rules (test/frame/types.h:18-60, verify.h:28-196), one function instead of a strategy
+// class per rule.  Elements are read with a stride, as there.  Defaults are the reference's: MERE / MARE with
+// threshold 2^-13 and multiplier 10, relative errors over |golden| + 2^-14.
+enum class PrecisionMode { ABS, REL, COMBINED, MERE_MARE, EXACT, INTEGER };
+
+struct VerifyConfig {
+    PrecisionMode mode = PrecisionMode::MERE_MARE;
+    double absTol = 1e-5;
+    double relTol = 1e-5;
+    double mereThreshold = 0.0001220703125;  // 2^-13
+    double mareMultiplier = 10.0;
+    double epsilonForRel = 1e-7;
+    VerifyConfig &SetMode(PrecisionMode m) { mode = m; return *this; }
+    VerifyConfig &SetAbsTol(double t) { absTol = t; return *this; }
+    VerifyConfig &SetRelTol(double t) { relTol = t; return *this; }
+    VerifyConfig &SetMERE(double t) { mereThreshold = t; return *this; }
+    VerifyConfig &SetMARE(double m) { mareMultiplier = m; return *this; }
+    VerifyConfig &SetEpsilon(double e) { epsilonForRel = e; return *this; }
+};
+
+struct VerifyReport {
+    bool pass = false;
+    size_t count = 0, skipped = 0, failures = 0, mismatches = 0, outliers = 0;
+    double mere = 0.0, mare = 0.0;  // mean and maximum relative error over the elements that were compared
+};
+
+inline VerifyReport Verify(const float *output, const float *golden, size_t count, int64_t stride,
+                           const VerifyConfig &cfg = VerifyConfig())
+{
+    constexpr double kMereEpsilon = 0.00006103515625;  // 2^-14 (verify.h:153)
+    VerifyReport r;
+    r.count = count;
+    double sumRel = 0.0;
+    const double outlierLimit = cfg.mareMultiplier * cfg.mereThreshold;
+    for (size_t i = 0; i < count; ++i) {
+        const float o = output[static_cast<int64_t>(i) * stride], g = golden[static_cast<int64_t>(i) * stride];
+        const bool oBad = std::isnan(o) || std::isinf(o), gBad = std::isnan(g) || std::isinf(g);
+        if (cfg.mode == PrecisionMode::INTEGER) {  // never skips (verify.h:178)
+            r.failures += static_cast<int64_t>(o) != static_cast<int64_t>(g) ? 1 : 0;
+            continue;
+        }
+        // equal values and a NaN on both sides are not looked at (verify.h:51-55); MERE / MARE also passes over
+        // an infinity or NaN on both sides (:117-123)
+        if (o == g || (std::isnan(o) && std::isnan(g)) || (cfg.mode == PrecisionMode::MERE_MARE && oBad && gBad)) {
+            r.skipped++;
+            continue;
+        }
+        const double d = std::abs(o - g);  // in float, like the reference
+        switch (cfg.mode) {
+            case PrecisionMode::ABS:
+                r.failures += d > cfg.absTol ? 1 : 0;
+                break;
+            case PrecisionMode::REL: {
+                const double rel = d / (std::abs(g) + cfg.epsilonForRel);
+                r.mare = rel > r.mare ? rel : r.mare;
+                break;
+            }
+            case PrecisionMode::COMBINED:
+                r.failures += d > cfg.absTol + cfg.relTol * std::abs(g) ? 1 : 0;
+                break;
+            case PrecisionMode::MERE_MARE: {
+                if (oBad || gBad) {
+                    r.mismatches++;
+                    break;
+                }
+                const double rel = d / (std::abs(g) + kMereEpsilon);
+                sumRel += rel;
+                r.mare = rel > r.mare ? rel : r.mare;
+                r.outliers += rel > outlierLimit ? 1 : 0;
+                break;
+            }
+            case PrecisionMode::EXACT:
+                r.failures++;  // anything that was not skipped as equal
+                break;
+            default:
+                break;
+        }
+    }
+    switch (cfg.mode) {
+        case PrecisionMode::REL:
+            r.pass = r.mare < cfg.relTol;
+            break;
+        case PrecisionMode::MERE_MARE: {
+            const size_t effective = count - r.skipped - r.mismatches;
+            r.mere = effective > 0 ? sumRel / static_cast<double>(effective) : 0.0;
+            r.pass = r.mismatches == 0 && r.mere < cfg.mereThreshold && r.mare < outlierLimit;
+            break;
+        }
+        default:
+            r.pass = r.failures == 0;
+            break;
+    }
+    return r;
+}
+
 struct CsrHost {
     int64_t rows = 0, cols = 0;
     std::vector<int32_t> rowptr{0}, colind;
@@ -199,7 +343,31 @@ inline std::vector<float> RandomVector(int64_t n, float lo, float hi, uint32_t s
 }
 
 // Rows of a CSV case table keyed by the header names; lines starting with '#' are comments.
-inline std::vector<std::map<std::string, std::string>> LoadCsv(const std::string &path)
+using CsvRow = std::map<std::string, std::string>;
+inline std::vector<CsvRow> LoadCsv(const std::string &path);
+
+// A test's parameter type fills itself from a row and names its case (the reference's SparseTestParamBase,
+// csv_loader.h:112-122); GetCasesFromCsv<ParamType> turns a table into a vector of them (:125-136).
+class CaseParamBase {
+public:
+    virtual ~CaseParamBase() = default;
+    virtual void fillCustom(const CsvRow &row) = 0;
+    virtual std::string caseId() const = 0;
+};
+
+template <typename ParamType>
+std::vector<ParamType> GetCasesFromCsv(const std::string &csvPath)
+{
+    std::vector<ParamType> cases;
+    for (const CsvRow &row : LoadCsv(csvPath)) {
+        ParamType p;
+        p.fillCustom(row);
+        cases.push_back(std::move(p));
+    }
+    return cases;
+}
+
+inline std::vector<CsvRow> LoadCsv(const std::string &path)
 {
     std::ifstream in(path);
     if (!in) {

@@ -4,10 +4,12 @@
 //
 //   run_case_tables <directory with the csv files> [table ...]
 //
-// Tables: spmv_op, coo2csr, csr2coo, csr2csc (default: all).  Mirrors
+// Tables: spmv_op, coo2csr, csr2coo, csr2csc, csrsort (default: all).  Mirrors
 // test/spmv_op/arch35/spmv_op_test.cpp:73-142, test/coo2csr/arch35/coo2csr_test.cpp,
 // test/csr2coo/arch35/csr2coo_test.cpp and test/csr2csc_ex2/arch35/csr2csc_ex2_test.cpp of the
-// reference, with the frame of tests/cpp/frame.h and the CPU oracle as golden.
+// reference, with the frame of tests/cpp/frame.h and the CPU oracle as golden.  csrsort has no
+// csv in the reference: its named success cases (test/csrsort/arch35/csrsort_test.cpp:239-420) are
+// built here as that program builds them.
 #include <cmath>
 #include <cstring>
 
@@ -68,16 +70,12 @@ bool SpmvOpCase(const frame::Stream &stream, const frame::Handle &handle, const 
     frame::DeviceArray<float> dScal(std::vector<float>{alpha, beta});
     void *rowPtr = i64 ? static_cast<void *>(dPtr64.get()) : static_cast<void *>(dPtr32.get());
 
-    aclsparseSpMatDescr_t matA = nullptr;
-    aclsparseDnVecDescr_t vx = nullptr, vy = nullptr, vz = nullptr;
-    Check(aclsparseCreateCsr(&matA, m, k, nnz, rowPtr, dCol.get(), dVal.get(),
-                             i64 ? ACL_SPARSE_INDEX_64I : ACL_SPARSE_INDEX_32I, ACL_SPARSE_INDEX_32I,
-                             ACL_SPARSE_INDEX_BASE_ZERO, ACL_FLOAT), "aclsparseCreateCsr");
-    Check(aclsparseCreateDnVec(&vx, k, dX.get(), ACL_FLOAT), "aclsparseCreateDnVec x");
-    Check(aclsparseCreateDnVec(&vy, m, dY.get(), ACL_FLOAT), "aclsparseCreateDnVec y");
-    if (!alias) {
-        Check(aclsparseCreateDnVec(&vz, m, dZ.get(), ACL_FLOAT), "aclsparseCreateDnVec z");
-    }
+    const frame::SpMat ownA = frame::SpMat::createCsr(m, k, nnz, rowPtr, dCol.get(), dVal.get(),
+                                                      i64 ? ACL_SPARSE_INDEX_64I : ACL_SPARSE_INDEX_32I);
+    const frame::DnVec ownX = frame::DnVec::create(k, dX.get()), ownY = frame::DnVec::create(m, dY.get());
+    const frame::DnVec ownZ = alias ? frame::DnVec() : frame::DnVec::create(m, dZ.get());
+    const aclsparseSpMatDescr_t matA = ownA.get();
+    const aclsparseDnVecDescr_t vx = ownX.get(), vy = ownY.get(), vz = ownZ.get();
     aclsparseDnVecDescr_t out = alias ? vy : vz;
     const std::string algName = r.at("alg");
     const aclsparseSpMVOpAlg_t alg = algName == "ALG2"   ? ACL_SPARSE_SPMVOP_ALG2
@@ -103,12 +101,6 @@ bool SpmvOpCase(const frame::Stream &stream, const frame::Handle &handle, const 
     const std::vector<float> got = alias ? dY.download() : dZ.download();
     (void)aclsparseSpMVOp_destroyPlan(plan);
     (void)aclsparseSpMVOp_destroyDescr(descr);
-    (void)aclsparseDestroyDnVec(vx);
-    (void)aclsparseDestroyDnVec(vy);
-    if (vz != nullptr) {
-        (void)aclsparseDestroyDnVec(vz);
-    }
-    (void)aclsparseDestroySpMat(matA);
 
     // |d| <= 1e-5 |gold| per element, and the table's own MERE / MARE limits
     for (int64_t i = 0; i < m; ++i) {
@@ -118,12 +110,124 @@ bool SpmvOpCase(const frame::Stream &stream, const frame::Handle &handle, const 
             return false;
         }
     }
-    double res[4] = {0, 0, 0, 0};
-    if (m > 0) {
-        oracle_mere_mare(got.data(), gold.data(), m, std::ldexp(1.0, -14), res);
+    const frame::VerifyReport rep = frame::Verify(
+        got.data(), gold.data(), static_cast<size_t>(m), 1,
+        frame::VerifyConfig().SetMERE(D(r, "mere_threshold")).SetMARE(D(r, "mare_multiplier")));
+    return rep.pass;
+}
+
+// ---- csrsort: the named cases of the reference's test program
+
+struct SortCase {
+    std::string name;
+    int m = 0, n = 0;
+    int32_t base = 0;
+    std::vector<int32_t> rowPtr, colInd, perm;  // perm empty: the identity
+};
+
+std::vector<SortCase> SortCases()
+{
+    std::vector<SortCase> c;
+    c.push_back({"Basic", 3, 3, 0, {0, 3, 6, 9}, {2, 1, 0, 0, 2, 1, 1, 2, 0}, {}});
+    c.push_back({"EmptyRows", 4, 5, 0, {0, 0, 2, 2, 4}, {3, 1, 4, 2}, {}});
+    c.push_back({"AlreadySorted", 3, 5, 0, {0, 2, 4, 6}, {0, 1, 2, 3, 0, 4}, {}});
+    c.push_back({"Reverse", 3, 5, 0, {0, 2, 4, 6}, {4, 0, 3, 2, 4, 1}, {}});
+    c.push_back({"DuplicateCols", 1, 5, 0, {0, 5}, {2, 1, 2, 1, 0}, {10, 20, 30, 40, 50}});
+    c.push_back({"NonIdentityP", 2, 4, 0, {0, 2, 4}, {3, 1, 0, 2}, {100, 200, 300, 400}});
+    c.push_back({"Base1", 2, 4, 1, {1, 3, 5}, {4, 2, 1, 3}, {}});
+    c.push_back({"EmptyMatrix", 3, 3, 0, {0, 0, 0, 0}, {}, {}});
+    c.push_back({"SingleElemRows", 4, 4, 0, {0, 0, 1, 1, 2}, {3, 1}, {}});
+    {  // ManySmallRows: 200 rows of rng() % 4 entries, columns rng() % 10, std::mt19937(99)
+        SortCase s{"ManySmallRows", 200, 10, 0, std::vector<int32_t>(201, 0), {}, {}};
+        std::mt19937 rng(99);
+        for (int i = 0; i < s.m; ++i) {
+            const int len = static_cast<int>(rng() % 4);
+            for (int j = 0; j < len; ++j) {
+                s.colInd.push_back(static_cast<int32_t>(rng() % static_cast<uint32_t>(s.n)));
+            }
+            s.rowPtr[i + 1] = static_cast<int32_t>(s.colInd.size());
+        }
+        c.push_back(s);
     }
-    const double mere = D(r, "mere_threshold");
-    return res[2] == 0 && res[0] < mere && res[1] < mere * D(r, "mare_multiplier");
+    {  // MultiCoreSkewedRows: rows of 10000, 2048, 0 and row % 7 entries
+        SortCase s{"MultiCoreSkewedRows", 257, 4096, 0, std::vector<int32_t>(258, 0), {}, {}};
+        for (int row = 0; row < s.m; ++row) {
+            const int len = row % 64 == 0 ? 10000 : (row % 8 == 0 ? 2048 : (row % 5 != 0 ? row % 7 : 0));
+            for (int j = 0; j < len; ++j) {
+                s.colInd.push_back((row * 131 + len - j) % s.n);
+            }
+            s.rowPtr[row + 1] = static_cast<int32_t>(s.colInd.size());
+        }
+        c.push_back(s);
+    }
+    {  // LongRow: one row, a shuffle of 0 .. 999
+        SortCase s{"LongRow", 1, 1000, 0, {0, 1000}, std::vector<int32_t>(1000), {}};
+        for (int i = 0; i < 1000; ++i) {
+            s.colInd[i] = i;
+        }
+        std::mt19937 rng(123);
+        std::shuffle(s.colInd.begin(), s.colInd.end(), rng);
+        c.push_back(s);
+    }
+    {  // LongRowMultiRun: one row of 32768 entries over 4096 columns, every key eight times
+        SortCase s{"LongRowMultiRun", 1, 4096, 0, {0, 32768}, std::vector<int32_t>(32768), {}};
+        for (int i = 0; i < 32768; ++i) {
+            s.colInd[i] = i % s.n;
+        }
+        std::mt19937 rng(2026);
+        std::shuffle(s.colInd.begin(), s.colInd.end(), rng);
+        c.push_back(s);
+    }
+    {  // SingleHugeRow: a million entries in one row, 4096 distinct keys
+        constexpr int nnz = 1024 * 1024;
+        SortCase s{"SingleHugeRow", 1, 65536, 0, {0, nnz}, std::vector<int32_t>(nnz), std::vector<int32_t>(nnz)};
+        for (int i = 0; i < nnz; ++i) {
+            s.colInd[i] = static_cast<int32_t>((static_cast<uint64_t>(i) * 65521U + 7919U) % 4096U);
+            s.perm[i] = i;
+        }
+        c.push_back(s);
+    }
+    return c;
+}
+
+// RunSortAndVerify of the reference (csrsort_test.cpp:118-232): an empty matrix needs no buffer and no arrays;
+// otherwise bufferSizeExt must ask for a buffer, and row offsets, sorted columns and P are compared exactly.
+bool CsrsortCase(const frame::Stream &stream, const frame::Handle &handle, const SortCase &c)
+{
+    const int nnz = static_cast<int>(c.colInd.size());
+    aclsparseMatDescr_t descr = nullptr;
+    Check(aclsparseCreateMatDescr(&descr), "aclsparseCreateMatDescr");
+    aclsparseSetMatIndexBase(descr, static_cast<aclsparseIndexBase_t>(c.base));
+    bool ok = false;
+    if (nnz == 0) {
+        size_t bytes = 42;
+        Check(aclsparseXcsrsort_bufferSizeExt(handle.get(), c.m, c.n, 0, c.rowPtr.data(), nullptr, &bytes),
+              "aclsparseXcsrsort_bufferSizeExt");
+        Check(aclsparseXcsrsort(handle.get(), c.m, c.n, 0, descr, c.rowPtr.data(), nullptr, nullptr, nullptr),
+              "aclsparseXcsrsort");
+        ok = bytes == 0;
+    } else {
+        std::vector<int32_t> perm = c.perm;
+        if (perm.empty()) {
+            perm.resize(static_cast<size_t>(nnz));
+            for (int i = 0; i < nnz; ++i) {
+                perm[i] = i;
+            }
+        }
+        std::vector<int32_t> goldCol = c.colInd, goldPerm = perm;
+        oracle_csrsort(c.rowPtr.data(), c.m, c.base, goldCol.data(), goldPerm.data());
+        frame::DeviceArray<int32_t> dPtr(c.rowPtr), dCol(c.colInd), dPerm(perm);
+        size_t bytes = 0;
+        Check(aclsparseXcsrsort_bufferSizeExt(handle.get(), c.m, c.n, nnz, dPtr.get(), dCol.get(), &bytes),
+              "aclsparseXcsrsort_bufferSizeExt");
+        frame::DeviceArray<unsigned char> buffer(bytes);
+        Check(aclsparseXcsrsort(handle.get(), c.m, c.n, nnz, descr, dPtr.get(), dCol.get(), dPerm.get(), buffer.get()),
+              "aclsparseXcsrsort");
+        stream.sync();
+        ok = bytes > 0 && dPtr.download() == c.rowPtr && dCol.download() == goldCol && dPerm.download() == goldPerm;
+    }
+    (void)aclsparseDestroyMatDescr(descr);
+    return ok;
 }
 
 bool Coo2CsrCase(const frame::Stream &stream, const frame::Handle &handle, const Row &r)
@@ -213,7 +317,8 @@ bool Csr2CscCase(const frame::Stream &stream, const frame::Handle &handle, const
 int main(int argc, char **argv)
 {
     if (argc < 2) {
-        std::fprintf(stderr, "usage: %s <directory with the csv case tables> [spmv_op|coo2csr|csr2coo|csr2csc ...]\n", argv[0]);
+        std::fprintf(stderr, "usage: %s <directory with the csv case tables> [spmv_op|coo2csr|csr2coo|csr2csc|csrsort ...]\n",
+                     argv[0]);
         return 2;
     }
     const std::string dir = argv[1];
@@ -222,13 +327,29 @@ int main(int argc, char **argv)
         tables.push_back(argv[i]);
     }
     if (tables.empty()) {
-        tables = {"spmv_op", "coo2csr", "csr2coo", "csr2csc"};
+        tables = {"spmv_op", "coo2csr", "csr2coo", "csr2csc", "csrsort"};
     }
     int failed = 0, total = 0;
     try {
         frame::Stream stream;
         frame::Handle handle(stream);
         for (const std::string &t : tables) {
+            if (t == "csrsort") {
+                for (const SortCase &c : SortCases()) {
+                    bool ok = false;
+                    std::string error;
+                    try {
+                        ok = CsrsortCase(stream, handle, c);
+                    } catch (const std::exception &e) {
+                        error = e.what();
+                    }
+                    ++total;
+                    failed += ok ? 0 : 1;
+                    std::printf("[%s] %-32s %s %s\n", t.c_str(), c.name.c_str(), ok ? "PASS" : "FAIL", error.c_str());
+                    std::fflush(stdout);
+                }
+                continue;
+            }
             const auto rows = frame::LoadCsv(dir + "/" + t + "_cases.csv");
             for (const Row &r : rows) {
                 bool ok = false;
