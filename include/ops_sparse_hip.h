@@ -204,10 +204,18 @@ int opsparse_spmv_csr_launch_noalloc(const int32_t *rowOffsets, const int32_t *c
                                      OpsparseScalar alpha, OpsparseScalar beta, int32_t valType, int32_t outType,
                                      int32_t computeIsInt, void *stream);
 
+/* out[i] = offsets[i] - indexBase as int32, i < count: 64-bit and / or one-based row offsets turned into what the
+ * kernels above take.  With one-based column indices left as they are, a caller then passes x - 1 for x and
+ * cols + 1 for cols: x[col - 1] is (x - 1)[col], and the row-wise kernels only touch x at the indices present
+ * [ref: the index variants of sparse/spmv_op/arch35/spmv_op_kernel.cpp:139-181]. */
+int opsparse_rebase_offsets_launch(const void *offsets, int32_t offsetsAre64, int32_t indexBase, int64_t count,
+                                   int32_t *out, void *stream);
+
 /* fp32 z = alpha * A * x + beta * yIn for the index variants of the SpMVOp API:
  * int32 or int64 row offsets (rowOffsetsAre64), int32 column indices, index
  * base 0 or 1 [ref: sparse/spmv_op/arch35/spmv_op_kernel.cpp:139-181].  One lane
- * group per row, no workspace. */
+ * group per row, no workspace: the route for matrices of more than 2^31 - 1 entries, which the 32-bit kernels
+ * cannot index (aclsparseSpMVOp rebases smaller ones and runs the binned kernels). */
 int opsparse_spmv_csr_indexed_launch(const void *rowOffsets, int32_t rowOffsetsAre64, int32_t indexBase,
                                      const int32_t *colInd, const float *csrValues, const float *x,
                                      const float *yIn, float *z, int64_t rows, int64_t cols, int64_t nnz,

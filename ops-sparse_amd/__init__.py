@@ -90,7 +90,7 @@ ACL_SPARSE_CSR2CSC_ALG_DEFAULT, ACL_SPARSE_CSR2CSC_ALG1 = 0, 1
 OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_workspace_bytes", "opsparse_spmv_csr_analyse", "opsparse_spmv_csr_launch",
     "opsparse_spmv_csr_launch_zy", "opsparse_spmv_csr_indexed_launch",
-    "opsparse_spmv_csr_launch_noalloc", "opsparse_spmv_csr_noalloc_max_bytes",
+    "opsparse_spmv_csr_launch_noalloc", "opsparse_spmv_csr_noalloc_max_bytes", "opsparse_rebase_offsets_launch",
     "opsparse_spmv_csr_panels_workspace_bytes", "opsparse_spmv_csr_panels_analyse",
     "opsparse_spmv_csr_blocked_workspace_bytes", "opsparse_spmv_csr_blocked_resident_bytes",
     "opsparse_spmv_csr_blocked_analyse",
@@ -255,6 +255,8 @@ def lib():
     L.opsparse_spmv_csr_panels_analyse.restype = ctypes.c_int
     L.opsparse_spmv_csr_panels_analyse.argtypes = [vp, vp, vp, i64, i64, i64, vp, sz, ctypes.POINTER(OpsparseSpmvPlan),
                                                    vp]
+    L.opsparse_rebase_offsets_launch.restype = ctypes.c_int
+    L.opsparse_rebase_offsets_launch.argtypes = [vp, i32, i32, i64, vp, vp]
     L.opsparse_spmv_csr_indexed_launch.restype = ctypes.c_int
     L.opsparse_spmv_csr_indexed_launch.argtypes = [vp, i32, i32, vp, vp, vp, vp, vp, i64, i64, i64, OpsparseScalar,
                                                    OpsparseScalar, vp]

@@ -719,6 +719,17 @@ __device__ __forceinline__ int64_t MergeDiagonal(int64_t block, int64_t rows, in
     return d < rows + nnz ? d : rows + nnz;
 }
 
+// out[i] = in[i] - base as int32: row offsets of either width and index base for the kernels below.
+template <typename RowT>
+__global__ __launch_bounds__(kBlockThreads) void RebaseOffsetsKernel(const RowT *__restrict__ in, int64_t count,
+                                                                     int32_t base, int32_t *__restrict__ out)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < count; i += stride) {
+        out[i] = static_cast<int32_t>(static_cast<int64_t>(in[i]) - base);
+    }
+}
+
 // part[b] = number of rows completed before diagonal b * kMergeItems of the
 // merge of (row end offsets, non-zero indices): the smallest i with
 // rowOffsets[i + 1] > d - i - 1.
@@ -2084,6 +2095,28 @@ int opsparse_spmv_csr_launch_noalloc(const int32_t *rowOffsets, const int32_t *c
     // fix-up kernel reads only carries and heads that the merge kernel of the same launch has written.
     return opsparse_spmv_csr_launch_zy(nullptr, 0, rowOffsets, colInd, csrValues, x, y, y, rows, cols, nnz, alpha, beta,
                                        valType, outType, computeIsInt, ws, OPSPARSE_NOALLOC_SCRATCH_BYTES, stream);
+}
+
+int opsparse_rebase_offsets_launch(const void *offsets, int32_t offsetsAre64, int32_t indexBase, int64_t count,
+                                   int32_t *out, void *stream)
+{
+    if (count < 0 || (indexBase != 0 && indexBase != 1) || (count > 0 && (offsets == nullptr || out == nullptr))) {
+        return OPSPARSE_E_INVALID;
+    }
+    if (count == 0) {
+        return OPSPARSE_OK;
+    }
+    int64_t grid = (count + kBlockThreads - 1) / kBlockThreads;
+    grid = grid > 4096 ? 4096 : grid;
+    auto s = static_cast<hipStream_t>(stream);
+    if (offsetsAre64) {
+        hipLaunchKernelGGL(RebaseOffsetsKernel<int64_t>, dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0, s,
+                           static_cast<const int64_t *>(offsets), count, indexBase, out);
+    } else {
+        hipLaunchKernelGGL(RebaseOffsetsKernel<int32_t>, dim3(static_cast<uint32_t>(grid)), dim3(kBlockThreads), 0, s,
+                           static_cast<const int32_t *>(offsets), count, indexBase, out);
+    }
+    return CheckLaunch();
 }
 
 int opsparse_spmv_csr_indexed_launch(const void *rowOffsets, int32_t rowOffsetsAre64, int32_t indexBase,

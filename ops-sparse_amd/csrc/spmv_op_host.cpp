@@ -7,7 +7,11 @@
 // m == 0 / nnz == 0 short cuts of :465-486).  What differs is underneath: the
 // reference runs one thread per row with a compensated dot product and, for
 // ALG2, a device-side sort of the rows; here every algorithm value runs the
-// fp64-accumulating SpMV kernels, which are deterministic.  ALG2's buffer holds
+// fp64-accumulating SpMV kernels, which are deterministic.  64-bit row offsets
+// and index base 1 reach the same kernels: the descriptor owns a 32-bit
+// zero-based copy of the row offsets (rewritten from the caller's at every
+// ALG1 execution, once for ALG2), and one-based column indices are used as they
+// are with x - 1 in place of x.  ALG2's buffer holds
 // what its analysis leaves: the merge-path partition (the nnz-balanced split
 // that ALG2 asks for) or, for a wide matrix with scattered columns, the
 // re-stored blocked-gather / column-panel layout.  ALG1 has no buffer: its
@@ -32,6 +36,7 @@ struct aclsparseSpMVOpDescr {
     void *userBuffer = nullptr;  // ALG2: caller's buffer holding the partition
     bool planned = false;        // plan is valid (ALG2: userBuffer was analysed; ALG1: a row-wise kernel, no buffer)
     OpsparseSpmvPlan plan{};
+    int32_t *offsets32 = nullptr;  // owned: the row offsets as int32, zero-based (64-bit offsets or index base 1 only)
 };
 
 struct aclsparseSpMVOpPlan {
@@ -79,11 +84,23 @@ aclsparseStatus_t ValidateAlg(aclsparseSpMVOpAlg_t alg)
     return ACL_SPARSE_STATUS_SUCCESS;
 }
 
-// The optimised kernels take 32-bit zero-based offsets; anything else goes to
-// the indexed-rows kernel.
+// The optimised kernels take 32-bit zero-based offsets.
 bool Plain(const aclsparseSpMVOpDescr *d)
 {
     return d->rowOffsetsType == ACL_SPARSE_INDEX_32I && d->indexBase == ACL_SPARSE_INDEX_BASE_ZERO;
+}
+
+// What they are given: the caller's offsets, or the descriptor's rebased copy of them.
+const int32_t *Offsets32(const aclsparseSpMVOpDescr *d)
+{
+    return d->offsets32 != nullptr ? d->offsets32 : static_cast<const int32_t *>(d->rowOffsets);
+}
+
+int Rebase(const aclsparseSpMVOpDescr *d, hipStream_t stream)
+{
+    return opsparse_rebase_offsets_launch(d->rowOffsets, d->rowOffsetsType == ACL_SPARSE_INDEX_64I ? 1 : 0,
+                                          d->indexBase == ACL_SPARSE_INDEX_BASE_ONE ? 1 : 0, d->rows + 1, d->offsets32,
+                                          stream);
 }
 
 // First execution of an unplanned descriptor (ALG1): the row statistics into the handle's workspace.  A plan for
@@ -103,9 +120,8 @@ void LookAtRows(aclsparseHandle_t handle, aclsparseSpMVOpPlan *plan)
         return;
     }
     OpsparseSpmvPlan p{};
-    const int rc = opsparse_spmv_csr_analyse(static_cast<const int32_t *>(d->rowOffsets), d->rows, d->cols, d->nnz,
-                                             handle->workspace(), handle->workspaceBytes(), OPSPARSE_SPMV_AUTO, &p,
-                                             handle->stream);
+    const int rc = opsparse_spmv_csr_analyse(Offsets32(d), d->rows, d->cols, d->nnz, handle->workspace(),
+                                             handle->workspaceBytes(), OPSPARSE_SPMV_AUTO, &p, handle->stream);
     if (rc == OPSPARSE_OK && (p.kernel == OPSPARSE_SPMV_STREAM_ROWS || p.kernel == OPSPARSE_SPMV_VECTOR_ROWS)) {
         plan->rowsPlan = p;
         plan->rowsPlan.guardTiles = 1;
@@ -219,10 +235,24 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
     d->colInd = matA->colInd;
     d->values = matA->values;
     d->alg = (alg == ACL_SPARSE_SPMVOP_ALG_DEFAULT) ? ACL_SPARSE_SPMVOP_ALG1 : alg;
+    if (!Plain(d) && d->rows > 0 && d->nnz > 0 && d->nnz <= INT32_MAX && d->rowOffsets != nullptr) {
+        // 64-bit offsets and / or index base 1: a 32-bit zero-based copy for the binned kernels
+        if (hipMalloc(reinterpret_cast<void **>(&d->offsets32), sizeof(int32_t) * static_cast<size_t>(d->rows + 1)) !=
+            hipSuccess) {
+            (void)hipGetLastError();
+            delete d;
+            return ACL_SPARSE_STATUS_ALLOC_FAILED;
+        }
+        if (Rebase(d, handle->stream) != OPSPARSE_OK) {
+            (void)hipFree(d->offsets32);
+            delete d;
+            return ACL_SPARSE_STATUS_EXECUTION_FAILED;
+        }
+    }
     if (d->alg == ACL_SPARSE_SPMVOP_ALG2) {
         d->userBuffer = buffer;
         // The nnz-balanced split of ALG2: analyse the rows into the caller's buffer.
-        if (Plain(d) && d->rows > 0 && d->nnz > 0 && d->rowOffsets != nullptr) {
+        if ((Plain(d) || d->offsets32 != nullptr) && d->rows > 0 && d->nnz > 0 && d->rowOffsets != nullptr) {
             const opsparse::RestoredChoice restored = RestoredLayout(matA);
             const int rc =
                 restored.kernel != 0 && d->colInd != nullptr && d->values != nullptr
@@ -230,10 +260,11 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
                                                 static_cast<const int32_t *>(d->colInd),
                                                 static_cast<const float *>(d->values), d->rows, d->cols, d->nnz, false,
                                                 false, buffer, restored.bytes, &d->plan, handle->stream)
-                    : opsparse_spmv_csr_analyse(static_cast<const int32_t *>(d->rowOffsets), d->rows, d->cols, d->nnz,
-                                                buffer, opsparse_spmv_csr_workspace_bytes(d->rows, d->nnz),
-                                                OPSPARSE_SPMV_AUTO, &d->plan, handle->stream);
+                    : opsparse_spmv_csr_analyse(Offsets32(d), d->rows, d->cols, d->nnz, buffer,
+                                                opsparse_spmv_csr_workspace_bytes(d->rows, d->nnz), OPSPARSE_SPMV_AUTO,
+                                                &d->plan, handle->stream);
             if (rc != OPSPARSE_OK) {
+                (void)hipFree(d->offsets32);
                 delete d;
                 return FromLaunch(rc);
             }
@@ -246,6 +277,9 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
 
 aclsparseStatus_t aclsparseSpMVOp_destroyDescr(aclsparseSpMVOpDescr_t descr)
 {
+    if (descr != nullptr && descr->offsets32 != nullptr) {
+        (void)hipFree(descr->offsets32);  // waits for the work that still reads it
+    }
     delete descr;  // NULL is fine
     return ACL_SPARSE_STATUS_SUCCESS;
 }
@@ -334,7 +368,16 @@ aclsparseStatus_t aclsparseSpMVOp(aclsparseHandle_t handle, aclsparseSpMVOpPlan_
     const OpsparseScalar a = opsparse::MakeScalar(alpha, ACL_FLOAT, handle->pointerMode, 0.0);
     const OpsparseScalar b = opsparse::MakeScalar(beta, ACL_FLOAT, handle->pointerMode, 0.0);
     int rc;
-    if (Plain(d) || d->nnz == 0) {
+    if (Plain(d) || d->nnz == 0 || d->offsets32 != nullptr) {
+        // index base 1: the column indices stay one-based, x - 1 stands for x (only indices that occur are read)
+        const int64_t shift = (d->nnz > 0 && d->indexBase == ACL_SPARSE_INDEX_BASE_ONE) ? 1 : 0;
+        const float *x = static_cast<const float *>(vecX->values) - shift;
+        if (d->offsets32 != nullptr && d->nnz > 0 && d->alg != ACL_SPARSE_SPMVOP_ALG2) {
+            rc = Rebase(d, handle->stream);  // ALG1 promises nothing about the offsets between executions
+            if (rc != OPSPARSE_OK) {
+                return FromLaunch(rc);
+            }
+        }
         const OpsparseSpmvPlan *p = d->planned ? &d->plan : nullptr;
         void *ws = d->planned ? d->userBuffer : nullptr;
         size_t wsBytes = d->planned ? static_cast<size_t>(d->plan.bytes) : 0;
@@ -353,9 +396,9 @@ aclsparseStatus_t aclsparseSpMVOp(aclsparseHandle_t handle, aclsparseSpMVOpPlan_
             }
         }
         // nnz == 0 needs no offsets at all: Z = beta * Y whatever their width.
-        rc = opsparse_spmv_csr_launch_zy(p, 0, static_cast<const int32_t *>(d->nnz > 0 ? d->rowOffsets : nullptr),
-                                         static_cast<const int32_t *>(d->colInd), d->values, vecX->values,
-                                         vecY->values, vecZ->values, d->rows, d->cols, d->nnz, a, b, OPSPARSE_F32,
+        rc = opsparse_spmv_csr_launch_zy(p, 0, d->nnz > 0 ? Offsets32(d) : nullptr,
+                                         static_cast<const int32_t *>(d->colInd), d->values, x, vecY->values,
+                                         vecZ->values, d->rows, d->cols + shift, d->nnz, a, b, OPSPARSE_F32,
                                          OPSPARSE_F32, 0, ws, wsBytes, handle->stream);
     } else {
         rc = opsparse_spmv_csr_indexed_launch(d->rowOffsets, d->rowOffsetsType == ACL_SPARSE_INDEX_64I ? 1 : 0,

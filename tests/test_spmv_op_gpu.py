@@ -284,3 +284,39 @@ def test_alg1_short_rows_with_long_ones_beside(osa, gpu_ctx, alias):
         stream.synchronize()
         check(d_z.cpu().numpy(), m, k, rowptr, colind, val, x, y, 1.25, -0.5)
     op.close()
+
+
+def test_index_variants_run_the_binned_kernels(osa, gpu_ctx, workloads):
+    """64-bit row offsets and index base 1 on a power-law matrix (rows up to 20 000 entries): same result as the
+    32-bit zero-based descriptor to 1e-5 against the oracle, and no load-imbalance penalty — the calls take about
+    as long (a lane group per row, the kernel these variants used to get, is several times slower here)."""
+    import torch
+    dev, stream, handle = gpu_ctx
+    m = 400_000
+    A = workloads.power_law_csr(m, m, 2.0, 1, 20_000, 77, dev)
+    nnz = int(A["colind"].numel())
+    x = workloads.uniform(78, m, -1.0, 1.0, dev)
+    y0 = workloads.uniform(79, m, -1.0, 1.0, dev)
+    gold = oracle.spmv_f64(m, m, A["rowptr"].cpu().numpy(), A["colind"].cpu().numpy(), A["values"].cpu().numpy(),
+                           x.cpu().numpy(), y0.cpu().numpy(), 1.5, -0.5)
+    X, Y = osa.DnVec(x), osa.DnVec(y0)
+    times = {}
+    for name, rowptr, colind, base in (
+            ("i32", A["rowptr"], A["colind"], osa.ACL_SPARSE_INDEX_BASE_ZERO),
+            ("i64", A["rowptr"].to(torch.int64), A["colind"], osa.ACL_SPARSE_INDEX_BASE_ZERO),
+            ("i64 base 1", A["rowptr"].to(torch.int64) + 1, A["colind"] + 1, osa.ACL_SPARSE_INDEX_BASE_ONE)):
+        z = torch.zeros(m, device=dev)
+        op = osa.SpmvOpPlan(handle, osa.Csr(m, m, rowptr, colind, A["values"], index_base=base), X, Y, osa.DnVec(z))
+        op(1.5, -0.5)
+        stream.synchronize()
+        assert oracle.max_rel_err(z.cpu().numpy(), gold) <= 1e-5, name
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(20):
+            op(1.5, -0.5)
+        e1.record(stream)
+        stream.synchronize()
+        times[name] = e0.elapsed_time(e1) / 20
+        op.close()
+    print("SpMVOp per call, ms:", {k: round(v, 4) for k, v in times.items()})
+    assert times["i64"] <= 1.5 * times["i32"] and times["i64 base 1"] <= 1.5 * times["i32"], times
