@@ -7,6 +7,8 @@
 // (:281-308); alpha / beta travel as kernel arguments instead.
 #include <climits>
 
+#include <cstdint>
+
 #include "internal.h"
 
 namespace {
@@ -158,14 +160,11 @@ aclsparseStatus_t BuildPlan(const aclsparseSpMatDescr *A, int64_t n, void *buffe
         return ACL_SPARSE_STATUS_INVALID_VALUE;
     }
     OpsparseSpmmPlan plan{};
-    size_t bytes = 0;
-    int rc = opsparse_spmm_csr_workspace_bytes(static_cast<const int32_t *>(A->rowOffsets), A->rows, A->nnz, n,
-                                               stream, &bytes);
-    if (rc != OPSPARSE_OK) {
-        return FromLaunch(rc);
-    }
-    rc = opsparse_spmm_csr_analyse(static_cast<const int32_t *>(A->rowOffsets), A->rows, A->nnz, n, buffer, bytes,
-                                   OPSPARSE_SPMM_AUTO, &plan, stream);
+    // Nothing says how large the caller's buffer is: it was sized by GetBufferSize for this matrix and width, and the
+    // analysis lays out exactly what GetBufferSize counted (one reduction over the row offsets, no allocation).
+    const size_t bytes = static_cast<size_t>(INT64_MAX);
+    const int rc = opsparse_spmm_csr_analyse(static_cast<const int32_t *>(A->rowOffsets), A->rows, A->nnz, n, buffer,
+                                             bytes, OPSPARSE_SPMM_AUTO, &plan, stream);
     if (rc != OPSPARSE_OK) {
         opsparse::LogError("aclsparseSpMM: analysis failed (%d)", rc);
         return FromLaunch(rc);
@@ -306,10 +305,20 @@ aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t o
                        matA->spmm.plan.nnz == matA->nnz;
     bool staged = bound && g.bytes > 0 && g.bytes <= matA->spmm.stagingBytes && matA->spmm.plan.n == g.nPadded &&
                   matA->nnz > 0;
+    const OpsparseSpmmPlan *plan = &matA->spmm.plan;
     if (!staged && (!bound || matA->spmm.plan.n != matC->cols)) {
-        st = BuildPlan(matA, matC->cols, buffer, handle->stream);
-        if (st != ACL_SPARSE_STATUS_SUCCESS) {
-            return st;
+        // The analysis reads two numbers back and synchronises, which a stream under capture must not: such a call
+        // runs without a plan (a lane group per row, no tables), like the raw launch layer with plan == NULL.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(handle->stream, &capturing) != hipSuccess ||
+            capturing != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            plan = nullptr;
+        } else {
+            st = BuildPlan(matA, matC->cols, buffer, handle->stream);
+            if (st != ACL_SPARSE_STATUS_SUCCESS) {
+                return st;
+            }
         }
     }
     // NULL scalars read as 0 (spmm_host.cpp:62-74).
@@ -322,11 +331,11 @@ aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t o
                        buffer, handle->stream);
     } else {
         rc = opsparse_spmm_csr_launch(
-            &matA->spmm.plan, static_cast<const int32_t *>(matA->rowOffsets),
+            plan, static_cast<const int32_t *>(matA->rowOffsets),
             static_cast<const int32_t *>(matA->colInd), matA->values, matB->values, matC->values, matA->rows,
             matA->cols, matC->cols, matA->nnz, matB->ld, matC->ld, matB->order == ACL_SPARSE_ORDER_COL ? 1 : 0,
             matC->order == ACL_SPARSE_ORDER_COL ? 1 : 0, opB == ACL_SPARSE_OP_TRANSPOSE ? 1 : 0, a, b, t.valType,
-            t.cType, buffer, static_cast<size_t>(matA->spmm.plan.bytes), handle->stream);
+            t.cType, buffer, plan != nullptr ? static_cast<size_t>(plan->bytes) : 0, handle->stream);
     }
     if (rc != OPSPARSE_OK) {
         opsparse::LogError("aclsparseSpMM: launch failed (%d)", rc);

@@ -730,6 +730,11 @@ __global__ __launch_bounds__(kBlockThreads) void RebaseOffsetsKernel(const RowT 
     }
 }
 
+__device__ __forceinline__ int64_t ClampTo(int64_t v, int64_t lo, int64_t hi)
+{
+    return v < lo ? lo : (v > hi ? hi : v);
+}
+
 // part[b] = number of rows completed before diagonal b * kMergeItems of the
 // merge of (row end offsets, non-zero indices): the smallest i with
 // rowOffsets[i + 1] > d - i - 1.
@@ -776,10 +781,13 @@ __device__ __forceinline__ void MergeTile(int64_t b, const int32_t *__restrict__
                                           AccT *__restrict__ head, AccT alpha, AccT beta, bool betaZero,
                                           AccT *prod /* [kMergeItems] in LDS */)
 {
-    const int64_t i0 = part[b];
-    const int64_t i1 = part[b + 1];
-    const int64_t j0 = MergeDiagonal(b, rows, nnz) - i0;
-    const int64_t j1 = MergeDiagonal(b + 1, rows, nnz) - i1;
+    // The partition comes from a buffer the caller owns: whatever it holds, rows stay inside [0, rows] and the
+    // entries of a tile inside [0, nnz] and inside the tile's LDS (a stale buffer gives wrong numbers, never an
+    // access out of range).
+    const int64_t i0 = ClampTo(part[b], 0, rows);
+    const int64_t i1 = ClampTo(part[b + 1], i0, rows);
+    const int64_t j0 = ClampTo(MergeDiagonal(b, rows, nnz) - i0, 0, nnz);
+    const int64_t j1 = ClampTo(MergeDiagonal(b + 1, rows, nnz) - i1, j0, j0 + kMergeItems < nnz ? j0 + kMergeItems : nnz);
     const int32_t count = static_cast<int32_t>(j1 - j0);
 
     {
@@ -815,8 +823,9 @@ __device__ __forceinline__ void MergeTileRows(int64_t b, int64_t i0, int64_t i1,
         const int64_t row = i0 + q;
         const bool completes = row < i1;
         const int64_t begin = LoadStream(rowOffsets + row);
-        const int32_t s = begin > j0 ? static_cast<int32_t>(begin - j0) : 0;
-        const int32_t e = completes ? static_cast<int32_t>(LoadStream(rowOffsets + row + 1) - j0) : count;
+        const int32_t s = begin > j0 ? static_cast<int32_t>(begin - j0 < count ? begin - j0 : count) : 0;
+        const int64_t rowEnd = completes ? static_cast<int64_t>(LoadStream(rowOffsets + row + 1)) - j0 : count;
+        const int32_t e = static_cast<int32_t>(rowEnd < count ? rowEnd : count);  // inside the staged products
         AccT sum = AccT(0);
         for (int32_t k = s + lane; k < e; k += g) {
             sum += prod[k];
@@ -907,8 +916,8 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvMergeFixupKernel(
     int64_t i0 = 0, first = b;  // first: the workgroup in which the spanning row starts
     bool spanning = false;
     if (b < numBlocks) {
-        i0 = part[b];
-        const int64_t i1 = part[b + 1];
+        i0 = ClampTo(part[b], 0, rows);
+        const int64_t i1 = ClampTo(part[b + 1], i0, rows);
         if (i1 > i0) {  // a row ends in this workgroup
             const int64_t begin = rowOffsets[i0];
             if (begin < MergeDiagonal(b, rows, nnz) - i0) {  // and it started before it

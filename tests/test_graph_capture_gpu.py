@@ -160,3 +160,43 @@ def test_first_unprepared_call_inside_a_capture(osa, gpu_ctx):
     stream.synchronize()
     gold2 = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, gold.astype(np.float32), 1.0, 0.0)
     assert oracle.max_rel_err(d_y.cpu().numpy(), gold2) <= 1e-5
+
+
+def test_unprepared_spmm_inside_a_capture(osa, gpu_ctx):
+    """aclsparseSpMM on a buffer that was never preprocessed for the matrix would analyse the rows first, which
+    synchronises; inside a capture it runs without a plan instead and leaves the capture intact.  The same call made
+    eagerly afterwards analyses and binds the buffer as usual."""
+    import ctypes
+    dev, stream, handle = gpu_ctx
+    m, k, n = 5_000, 7_000, 64
+    rowptr, colind, val = _power_law(m, k, 17, 2_500)               # rows long enough for the binned plan
+    rng = np.random.default_rng(19)
+    b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    c0 = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    d = [to_dev(a, dev) for a in (rowptr, colind, val)]
+    d_b, d_c = to_dev(b.ravel(), dev), to_dev(c0.ravel(), dev)
+    A, B, C = osa.Csr(m, k, d[0], d[1], d[2]), osa.DnMat(k, n, n, d_b), osa.DnMat(m, n, n, d_c)
+    L = osa.lib()
+    size = ctypes.c_size_t(0)
+    args = (handle.h, 0, 0, None, A.d, B.d, None, C.d, osa.ACL_FLOAT, osa.ACL_SPARSE_SPMM_ALG_DEFAULT)
+    assert L.aclsparseSpMMGetBufferSize(*args, ctypes.byref(size)) == 0
+    buf = torch.empty(max(size.value, 16), dtype=torch.uint8, device=dev)   # sized, but never preprocessed
+    alpha, beta = ctypes.c_float(1.5), ctypes.c_float(-0.25)
+
+    def call():
+        rc = L.aclsparseSpMM(handle.h, 0, 0, ctypes.byref(alpha), A.d, B.d, ctypes.byref(beta), C.d, osa.ACL_FLOAT,
+                             osa.ACL_SPARSE_SPMM_ALG_DEFAULT, ctypes.c_void_p(buf.data_ptr()))
+        assert rc == 0
+
+    graph = _capture(stream, call)
+    gold = np.asarray(oracle.spmm_f64_rowmajor(m, n, rowptr, colind, val, b, n, c0, n, 1.5, -0.25)).ravel()
+    for replay in range(2):
+        d_c.copy_(torch.from_numpy(c0.ravel()))
+        stream.synchronize()
+        graph.replay()
+        stream.synchronize()
+        assert oracle.max_rel_err(d_c.cpu().numpy(), gold) <= 1e-5, replay
+    d_c.copy_(torch.from_numpy(c0.ravel()))
+    call()                                                          # eager: analyses, binds, runs the binned kernels
+    stream.synchronize()
+    assert oracle.max_rel_err(d_c.cpu().numpy(), gold) <= 1e-5
