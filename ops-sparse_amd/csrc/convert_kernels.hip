@@ -250,6 +250,14 @@ __global__ __launch_bounds__(kBlockThreads) void RadixCountKernel(const int32_t 
     }
 }
 
+// LDS arrays that one phase reads with lane t at t * 16 + i and another with lane t at d * 256 + t: one unused
+// word after every 32 keeps both patterns free of bank conflicts (unpadded, the first puts all lanes on two banks).
+__device__ __forceinline__ int32_t Padded(int32_t i)
+{
+    return i + (i >> 5);
+}
+constexpr int kCounterSlots = kRadixDigits * kBlockThreads + kRadixDigits * kBlockThreads / 32;
+
 // Exclusive scan, digit-major, of the 16 x 256 per-thread digit counters of a
 // workgroup.  counters[d * 256 + t] holds thread t's count of digit d on entry
 // and the number of items that sort before thread t's first item of digit d on
@@ -261,14 +269,14 @@ __device__ __forceinline__ void ScanDigitCounters(int32_t *counters, int32_t *wa
     int32_t sum = 0;
 #pragma unroll
     for (int i = 0; i < kPer; ++i) {
-        v[i] = counters[threadIdx.x * kPer + i];
+        v[i] = counters[Padded(threadIdx.x * kPer + i)];
         sum += v[i];
     }
     int32_t total;
     int32_t run = BlockExclusiveScan(sum, waveSums, &total);
 #pragma unroll
     for (int i = 0; i < kPer; ++i) {
-        counters[threadIdx.x * kPer + i] = run;
+        counters[Padded(threadIdx.x * kPer + i)] = run;
         run += v[i];
     }
     __syncthreads();
@@ -303,7 +311,7 @@ __global__ __launch_bounds__(kBlockThreads) void RadixScatterKernel(
     void *__restrict__ payloadOut, int64_t n, int32_t keyBase, int32_t shift, const int32_t *__restrict__ prefix,
     int64_t numTiles, RadixPairIo io)
 {
-    __shared__ int32_t counters[kRadixDigits * kBlockThreads];
+    __shared__ int32_t counters[kCounterSlots];
     __shared__ int32_t waveSums[kBlockThreads / kWave];
     const int64_t first = static_cast<int64_t>(blockIdx.x) * kRadixTile + static_cast<int64_t>(threadIdx.x) * kRadixItems;
     int32_t key[kRadixItems], dig[kRadixItems];
@@ -343,7 +351,7 @@ __global__ __launch_bounds__(kBlockThreads) void RadixScatterKernel(
     }
 #pragma unroll
     for (int d = 0; d < kRadixDigits; ++d) {
-        counters[d * kBlockThreads + threadIdx.x] = cnt[d];
+        counters[Padded(d * kBlockThreads + threadIdx.x)] = cnt[d];
     }
     __syncthreads();
     ScanDigitCounters(counters, waveSums);
@@ -357,7 +365,8 @@ __global__ __launch_bounds__(kBlockThreads) void RadixScatterKernel(
             for (int j = 0; j < kRadixItems; ++j) {
                 earlier += (j < i && dig[j] == dig[i]) ? 1 : 0;
             }
-            const int32_t inTile = counters[dig[i] * kBlockThreads + threadIdx.x] - counters[dig[i] * kBlockThreads] + earlier;
+            const int32_t inTile = counters[Padded(dig[i] * kBlockThreads + threadIdx.x)] -
+                                   counters[Padded(dig[i] * kBlockThreads)] + earlier;
             const int64_t dst = static_cast<int64_t>(prefix[static_cast<int64_t>(dig[i]) * numTiles + blockIdx.x]) + inTile;
             keysOut[dst] = key[i];
             if (Mode == kPayPairLast) {
@@ -373,6 +382,163 @@ __global__ __launch_bounds__(kBlockThreads) void RadixScatterKernel(
                 static_cast<int32_t *>(payloadOut)[dst] = pay[i].row;
             } else {
                 static_cast<RadixPair *>(payloadOut)[dst] = pay[i];
+            }
+        }
+    }
+}
+
+// ----------------------------------------------- radix sort, 8 bits a pass
+// csr2csc's passes.  Sixteen times as many buckets as the 4-bit pass, so a tile's items for one bucket are few:
+// written straight from the lanes that hold them they would leave as scattered 12-byte pieces.  The tile is
+// therefore ordered by its 8-bit digit inside LDS first and written out in that order: neighbouring lanes then
+// write neighbouring addresses of one bucket's run.  What is ordered is one word an item, (digit, slot in the
+// tile), by two stable 4-bit splits; the items themselves stay where the loads put them and are fetched by slot at
+// the end.  A thread counts its items' digits in one 64-bit register, four bits a digit: the instruction count,
+// not the memory system, bounds this kernel, and a counter per digit selected by comparisons costs ten times more.
+
+constexpr int kWideBits = 8;
+constexpr int kWideDigits = 1 << kWideBits;
+constexpr int kWideItems = 15;                              // items a thread ranks: a 4-bit counter holds them,
+                                                            // and an odd stride over LDS has no bank conflicts
+constexpr int kWideTile = kBlockThreads * kWideItems;      // 3840
+constexpr int kWideSlotBits = 12;
+static_assert(kWideTile <= (1 << kWideSlotBits), "a slot number fits its field");
+static_assert(kWideDigits == kBlockThreads, "one thread per digit");
+
+__device__ __forceinline__ int32_t WideDigit(int32_t key, int32_t shift)
+{
+    return static_cast<int32_t>((static_cast<uint32_t>(key) >> shift) & (kWideDigits - 1));
+}
+
+// table[1 + digit * numTiles + tile] = items of that digit in the tile (see RadixCountKernel).
+__global__ __launch_bounds__(kBlockThreads) void WideCountKernel(const int32_t *__restrict__ keys, int64_t n,
+                                                                int32_t keyBase, int32_t shift,
+                                                                int32_t *__restrict__ table, int64_t numTiles)
+{
+    __shared__ int32_t hist[kWideDigits];
+    hist[threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kWideTile;
+#pragma unroll
+    for (int i = 0; i < kWideItems; ++i) {
+        const int64_t at = tile0 + i * kBlockThreads + threadIdx.x;
+        if (at < n) {
+            atomicAdd(&hist[WideDigit(keys[at] - keyBase, shift)], 1);
+        }
+    }
+    __syncthreads();
+    table[1 + static_cast<int64_t>(threadIdx.x) * numTiles + blockIdx.x] = hist[threadIdx.x];
+}
+
+// One pass over tile `blockIdx.x`; the payload modes are those of RadixScatterKernel (pairs only).  prefix is the
+// scanned table: prefix[digit * numTiles + tile] is the first output position of the tile's items of that digit,
+// and the entry after it, in that same flat order, ends them.
+template <int Mode>
+__global__ __launch_bounds__(kBlockThreads) void WideScatterKernel(
+    const int32_t *__restrict__ keysIn, const RadixPair *__restrict__ pairsIn, int32_t *__restrict__ keysOut,
+    RadixPair *__restrict__ pairsOut, int64_t n, int32_t keyBase, int32_t shift, const int32_t *__restrict__ prefix,
+    int64_t numTiles, RadixPairIo io)
+{
+    __shared__ int32_t sKey[kWideTile];
+    __shared__ __align__(8) RadixPair sPay[kWideTile];
+    __shared__ uint32_t sWord[kWideTile];
+    __shared__ int32_t counters[kCounterSlots];
+    __shared__ int32_t waveSums[kBlockThreads / kWave];
+    __shared__ int32_t outOf[kWideDigits];  // output position less slot, for the items of a digit
+    const int tid = threadIdx.x;
+    const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kWideTile;
+    const int32_t valid = static_cast<int32_t>(n - tile0 < kWideTile ? n - tile0 : kWideTile);
+    // the tile into LDS in its own order, neighbouring lanes reading neighbouring items; a slot past the end gets
+    // the largest digit, so that it sorts behind every real item
+#pragma unroll
+    for (int i = 0; i < kWideItems; ++i) {
+        const int32_t p = i * kBlockThreads + tid;
+        int32_t key = static_cast<int32_t>((kWideDigits - 1) << shift);
+        RadixPair pay{0, 0u};
+        if (p < valid) {
+            const int64_t at = tile0 + p;
+            key = keysIn[at] - keyBase;
+            if (Mode == kPayPairFirst) {
+                pay.row = io.rowSrc[at];
+                if (io.valueBytes == 4) {
+                    pay.val = static_cast<const uint32_t *>(io.valSrc)[at];
+                } else if (io.valueBytes == 2) {
+                    pay.val = static_cast<const uint16_t *>(io.valSrc)[at];
+                } else if (io.valueBytes == 1) {
+                    pay.val = static_cast<const uint8_t *>(io.valSrc)[at];
+                }
+            } else {
+                pay = pairsIn[at];
+            }
+        }
+        sKey[p] = key;
+        sPay[p] = pay;
+    }
+    {
+        // where the tile's run of digit `tid` starts in the ordered tile, from the lengths of the runs before it
+        const int64_t flat = static_cast<int64_t>(tid) * numTiles + blockIdx.x;
+        const int32_t first = prefix[flat];
+        int32_t total;
+        const int32_t start = BlockExclusiveScan(prefix[flat + 1] - first, waveSums, &total);  // has barriers
+        outOf[tid] = first - start;
+    }
+    // a thread takes kWideItems consecutive slots of the current order
+    uint32_t word[kWideItems];
+#pragma unroll
+    for (int i = 0; i < kWideItems; ++i) {
+        const int32_t p = tid * kWideItems + i;
+        word[i] = (static_cast<uint32_t>(WideDigit(sKey[p], shift)) << kWideSlotBits) | static_cast<uint32_t>(p);
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const int32_t at = kWideSlotBits + half * kRadixBits;
+        uint64_t packed = 0;  // the thread's count of digit d in bits [4 d, 4 d + 4)
+        int32_t earlier[kWideItems];
+#pragma unroll
+        for (int i = 0; i < kWideItems; ++i) {
+            const uint32_t sh = ((word[i] >> at) & (kRadixDigits - 1)) * 4;
+            earlier[i] = static_cast<int32_t>((packed >> sh) & 15);
+            packed += uint64_t{1} << sh;
+        }
+#pragma unroll
+        for (int d = 0; d < kRadixDigits; ++d) {
+            counters[Padded(d * kBlockThreads + tid)] = static_cast<int32_t>((packed >> (4 * d)) & 15);
+        }
+        __syncthreads();
+        ScanDigitCounters(counters, waveSums);  // counters[d][t]: slots that sort before thread t's first item of d
+#pragma unroll
+        for (int i = 0; i < kWideItems; ++i) {
+            const int32_t d = static_cast<int32_t>((word[i] >> at) & (kRadixDigits - 1));
+            sWord[counters[Padded(d * kBlockThreads + tid)] + earlier[i]] = word[i];
+        }
+        __syncthreads();
+        if (half == 0) {
+#pragma unroll
+            for (int i = 0; i < kWideItems; ++i) {
+                word[i] = sWord[tid * kWideItems + i];
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kWideItems; ++i) {
+        const int32_t p = i * kBlockThreads + tid;
+        if (p < valid) {  // the real items are the first `valid` slots of the ordered tile
+            const uint32_t w = sWord[p];
+            const int32_t slot = static_cast<int32_t>(w & ((1u << kWideSlotBits) - 1));
+            const int64_t dst = static_cast<int64_t>(outOf[w >> kWideSlotBits] + p);
+            const RadixPair out = sPay[slot];
+            keysOut[dst] = sKey[slot];
+            if (Mode == kPayPairLast) {
+                io.rowOut[dst] = out.row;
+                if (io.valueBytes == 4) {
+                    static_cast<uint32_t *>(io.valOut)[dst] = out.val;
+                } else if (io.valueBytes == 2) {
+                    static_cast<uint16_t *>(io.valOut)[dst] = static_cast<uint16_t>(out.val);
+                } else if (io.valueBytes == 1) {
+                    static_cast<uint8_t *>(io.valOut)[dst] = static_cast<uint8_t>(out.val);
+                }
+            } else {
+                pairsOut[dst] = out;
             }
         }
     }
@@ -806,6 +972,40 @@ void LaunchRadixPairPass(int mode, const int32_t *keysIn, const void *pairsIn, i
     }
 }
 
+int64_t WideTiles(int64_t n) { return (n + kWideTile - 1) / kWideTile; }
+int64_t WideTableInts(int64_t n) { return static_cast<int64_t>(kWideDigits) * WideTiles(n) + 1; }
+
+// One 8-bit pass carrying csr2csc's (row, value) pairs; table: WideTableInts(n) ints.
+void LaunchWidePairPass(int mode, const int32_t *keysIn, const void *pairsIn, int32_t *keysOut, void *pairsOut,
+                        int64_t n, int32_t keyBase, int32_t shift, int32_t *table, int32_t *scratch,
+                        const RadixPairIo &io, hipStream_t s)
+{
+    if (n <= 0) {
+        return;
+    }
+    const int64_t numTiles = WideTiles(n);
+    const auto grid = dim3(static_cast<uint32_t>(numTiles));
+    const auto *pin = static_cast<const RadixPair *>(pairsIn);
+    auto *pout = static_cast<RadixPair *>(pairsOut);
+    LaunchFill(table, 1, 0, s);
+    hipLaunchKernelGGL(WideCountKernel, grid, dim3(kBlockThreads), 0, s, keysIn, n, keyBase, shift, table, numTiles);
+    LaunchInclusiveScan(table, table, WideTableInts(n), 0, scratch, s);
+    switch (mode) {
+        case kPayPairFirst:
+            hipLaunchKernelGGL(WideScatterKernel<kPayPairFirst>, grid, dim3(kBlockThreads), 0, s, keysIn, pin, keysOut,
+                               pout, n, keyBase, shift, table, numTiles, io);
+            break;
+        case kPayPairLast:
+            hipLaunchKernelGGL(WideScatterKernel<kPayPairLast>, grid, dim3(kBlockThreads), 0, s, keysIn, pin, keysOut,
+                               pout, n, keyBase, shift, table, numTiles, io);
+            break;
+        default:
+            hipLaunchKernelGGL(WideScatterKernel<kPayPair>, grid, dim3(kBlockThreads), 0, s, keysIn, pin, keysOut, pout,
+                               n, keyBase, shift, table, numTiles, io);
+            break;
+    }
+}
+
 void LaunchGatherByPosition(const int32_t *pos, const int32_t *rowOfPos, const uint32_t *srcVal, int64_t nnz,
                             int32_t *rowOut, uint32_t *valOut, hipStream_t s)
 {
@@ -846,8 +1046,8 @@ struct Csr2CscLayout {
 Csr2CscLayout LayoutCsr2Csc(int64_t n, int64_t nnz)
 {
     Csr2CscLayout l{};
-    l.numTiles = (nnz + kRadixTile - 1) / kRadixTile;
-    l.tableCount = static_cast<int64_t>(kRadixDigits) * l.numTiles + 1;
+    l.numTiles = (nnz + kWideTile - 1) / kWideTile;
+    l.tableCount = static_cast<int64_t>(kWideDigits) * l.numTiles + 1;
     int64_t off = 0;
     const int64_t arr = Align256(4 * nnz);
     l.keysA = off; off += arr;
@@ -1088,7 +1288,9 @@ int opsparse_csr2csc_launch(int64_t m, int64_t n, int64_t nnz, const void *csrVa
     // Stable sort by column of (column; row, value): the pair travels with its key, 8 bytes a pass and entry more
     // than a source position would, and the last pass writes rows and values where they belong — no gather by
     // position at the end, which cost two cache-line fills per entry (33.5 M entries: 2.9 -> 1.9 ms).
-    int32_t passes = (KeyBits(n) + kRadixBits - 1) / kRadixBits;
+    // Eight bits a pass, the tile sorted through LDS before it leaves (33.5 M entries over 2^20 columns: three
+    // passes instead of five).
+    int32_t passes = (KeyBits(n) + kWideBits - 1) / kWideBits;
     passes = passes < 2 ? 2 : passes;  // a first pass that reads the sources and a last one that writes the outputs
     const RadixPairIo io{rowOfPos, csrVal, cscRowInd, cscVal, valueBytes};
     const int32_t *keysIn = csrColInd;
@@ -1096,8 +1298,8 @@ int opsparse_csr2csc_launch(int64_t m, int64_t n, int64_t nnz, const void *csrVa
     int cur = 0;
     for (int32_t pass = 0; pass < passes; ++pass) {
         const int mode = pass == 0 ? kPayPairFirst : (pass == passes - 1 ? kPayPairLast : kPayPair);
-        LaunchRadixPairPass(mode, keysIn, pairsIn, keys[cur], pairs[cur], nnz, pass == 0 ? indexBase : 0,
-                            pass * kRadixBits, table, tiles, io, s);
+        LaunchWidePairPass(mode, keysIn, pairsIn, keys[cur], pairs[cur], nnz, pass == 0 ? indexBase : 0,
+                           pass * kWideBits, table, tiles, io, s);
         keysIn = keys[cur];
         pairsIn = pairs[cur];
         cur ^= 1;
