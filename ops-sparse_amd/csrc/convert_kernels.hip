@@ -25,6 +25,8 @@
 //     position in the low half makes every key distinct, so any correct sort is
 //     the stable sort.
 #include <climits>
+#include <type_traits>
+#include <cstdlib>
 
 #include "convert_internal.h"
 #include "device_utils.h"
@@ -54,7 +56,16 @@ __global__ __launch_bounds__(kBlockThreads) void FillI32Kernel(int32_t *__restri
 
 // ------------------------------------------------------------------- scan
 
-// Exclusive scan of one value per thread over the workgroup; *total gets the sum.
+// A workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global load and store
+// the wavefront has in flight; this one leaves them outstanding (a tile's loads issued ahead of their use).
+__device__ __forceinline__ void LdsBarrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// Exclusive scan of one value per thread over the workgroup; *total gets the sum.  Its barriers order LDS only.
 __device__ __forceinline__ int32_t BlockExclusiveScan(int32_t v, int32_t *waveSums /* [4] in LDS */, int32_t *total)
 {
     const int32_t lane = threadIdx.x % kWave;
@@ -70,7 +81,7 @@ __device__ __forceinline__ int32_t BlockExclusiveScan(int32_t v, int32_t *waveSu
     if (lane == kWave - 1) {
         waveSums[wave] = incl;
     }
-    __syncthreads();
+    LdsBarrier();
     int32_t base = 0, all = 0;
 #pragma unroll
     for (int w = 0; w < kBlockThreads / kWave; ++w) {
@@ -78,7 +89,7 @@ __device__ __forceinline__ int32_t BlockExclusiveScan(int32_t v, int32_t *waveSu
         base += (w < wave) ? s : 0;
         all += s;
     }
-    __syncthreads();  // waveSums may be reused by the caller's next call
+    LdsBarrier();  // waveSums may be reused by the caller's next call
     *total = all;
     return base + incl - v;
 }
@@ -279,7 +290,7 @@ __device__ __forceinline__ void ScanDigitCounters(int32_t *counters, int32_t *wa
         counters[Padded(threadIdx.x * kPer + i)] = run;
         run += v[i];
     }
-    __syncthreads();
+    LdsBarrier();
 }
 
 // What travels with the keys through a pass.  kPayIndex: one int32 per item (a source position; payloadIn ==
@@ -405,89 +416,149 @@ constexpr int kWideSlotBits = 12;
 static_assert(kWideTile <= (1 << kWideSlotBits), "a slot number fits its field");
 static_assert(kWideDigits == kBlockThreads, "one thread per digit");
 
-__device__ __forceinline__ int32_t WideDigit(int32_t key, int32_t shift)
+// A pass's digit: `mask` = 2^bits - 1 with bits <= kWideBits (the passes of a sort share its key bits evenly).
+__device__ __forceinline__ int32_t WideDigit(int32_t key, int32_t shift, int32_t mask)
 {
-    return static_cast<int32_t>((static_cast<uint32_t>(key) >> shift) & (kWideDigits - 1));
+    return static_cast<int32_t>((static_cast<uint32_t>(key) >> shift) & static_cast<uint32_t>(mask));
 }
 
-// table[1 + digit * numTiles + tile] = items of that digit in the tile (see RadixCountKernel).
+// table[1 + digit * numTiles + tile] = items of that digit in the tile (see RadixCountKernel).  A workgroup counts
+// kWideCountTiles consecutive tiles and writes their counts of one digit side by side: a tile a workgroup leaves
+// the table written four bytes at a time, a cache line for each.
+constexpr int kWideCountTiles = 8;
+
 __global__ __launch_bounds__(kBlockThreads) void WideCountKernel(const int32_t *__restrict__ keys, int64_t n,
-                                                                int32_t keyBase, int32_t shift,
+                                                                int32_t keyBase, int32_t shift, int32_t mask,
                                                                 int32_t *__restrict__ table, int64_t numTiles)
 {
-    __shared__ int32_t hist[kWideDigits];
-    hist[threadIdx.x] = 0;
-    __syncthreads();
-    const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kWideTile;
+    __shared__ int32_t hist[kWideCountTiles][kWideDigits];
 #pragma unroll
-    for (int i = 0; i < kWideItems; ++i) {
-        const int64_t at = tile0 + i * kBlockThreads + threadIdx.x;
-        if (at < n) {
-            atomicAdd(&hist[WideDigit(keys[at] - keyBase, shift)], 1);
+    for (int j = 0; j < kWideCountTiles; ++j) {
+        hist[j][threadIdx.x] = 0;
+    }
+    __syncthreads();
+    const int64_t firstTile = static_cast<int64_t>(blockIdx.x) * kWideCountTiles;
+    // The keys of a tile are loaded, all of them, a tile ahead of their counting: the compiler keeps a load and the
+    // LDS atomic after it in program order, and an atomic straight behind its load is a round trip to memory for
+    // every item.  No branch around a load: an item past the end reads the last key and counts for nothing.
+    int32_t key[2][kWideItems];
+    auto fetch = [&](int j) {
+#pragma unroll
+        for (int i = 0; i < kWideItems; ++i) {
+            const int64_t at = (firstTile + j) * kWideTile + i * kBlockThreads + threadIdx.x;
+            key[j & 1][i] = keys[at < n ? at : n - 1];
+        }
+    };
+    fetch(0);
+#pragma unroll
+    for (int j = 0; j < kWideCountTiles; ++j) {
+        if (j + 1 < kWideCountTiles) {
+            fetch(j + 1);
+        }
+#pragma unroll
+        for (int i = 0; i < kWideItems; ++i) {
+            const int64_t at = (firstTile + j) * kWideTile + i * kBlockThreads + threadIdx.x;
+            atomicAdd(&hist[j][WideDigit(key[j & 1][i] - keyBase, shift, mask)], at < n ? 1 : 0);
         }
     }
     __syncthreads();
-    table[1 + static_cast<int64_t>(threadIdx.x) * numTiles + blockIdx.x] = hist[threadIdx.x];
+    // lanes j = 0 .. kWideCountTiles - 1 of a group write neighbouring tiles of one digit
+    constexpr int kDigitsAtOnce = kBlockThreads / kWideCountTiles;
+    const int32_t j = threadIdx.x % kWideCountTiles;
+#pragma unroll
+    for (int d0 = 0; d0 < kWideDigits; d0 += kDigitsAtOnce) {
+        const int32_t d = d0 + threadIdx.x / kWideCountTiles;
+        if (firstTile + j < numTiles) {
+            table[1 + static_cast<int64_t>(d) * numTiles + firstTile + j] = hist[j][d];
+        }
+    }
 }
 
-// One pass over tile `blockIdx.x`; the payload modes are those of RadixScatterKernel (pairs only).  prefix is the
-// scanned table: prefix[digit * numTiles + tile] is the first output position of the tile's items of that digit,
-// and the entry after it, in that same flat order, ends them.
-template <int Mode>
-__global__ __launch_bounds__(kBlockThreads) void WideScatterKernel(
-    const int32_t *__restrict__ keysIn, const RadixPair *__restrict__ pairsIn, int32_t *__restrict__ keysOut,
-    RadixPair *__restrict__ pairsOut, int64_t n, int32_t keyBase, int32_t shift, const int32_t *__restrict__ prefix,
-    int64_t numTiles, RadixPairIo io)
+// Between two passes the n (row, value) pairs lie as n rows followed by n values in the 8 n bytes of their buffer:
+// 4-byte stores to a bucket's run, as for the keys (8-byte stores of whole pairs to such short runs took half as
+// long again).
+template <typename P>
+__device__ __forceinline__ auto WideRows(P *pairs)
 {
-    __shared__ int32_t sKey[kWideTile];
-    __shared__ __align__(8) RadixPair sPay[kWideTile];
-    __shared__ uint32_t sWord[kWideTile];
-    __shared__ int32_t counters[kCounterSlots];
-    __shared__ int32_t waveSums[kBlockThreads / kWave];
-    __shared__ int32_t outOf[kWideDigits];  // output position less slot, for the items of a digit
+    return reinterpret_cast<std::conditional_t<std::is_const<P>::value, const int32_t, int32_t> *>(pairs);
+}
+template <typename P>
+__device__ __forceinline__ auto WideVals(P *pairs, int64_t n)
+{
+    return reinterpret_cast<std::conditional_t<std::is_const<P>::value, const uint32_t, uint32_t> *>(pairs) + n;
+}
+
+// A tile's items as the loads deliver them, lane t holding slots t, t + 256, ...
+struct WideTileRegs {
+    int32_t key[kWideItems];
+    RadixPair pay[kWideItems];
+    int32_t first, next;  // prefix[digit tid][tile] and the entry after it
+};
+
+template <int Mode, int VB, bool Full>
+__device__ __forceinline__ void WideFetch(WideTileRegs &r, int64_t tile, const int32_t *__restrict__ keysIn,
+                                          const RadixPair *__restrict__ pairsIn, int64_t n, int32_t keyBase,
+                                          int32_t shift, int32_t mask, const int32_t *__restrict__ prefix,
+                                          int64_t numTiles, const RadixPairIo &io)
+{
     const int tid = threadIdx.x;
-    const int64_t tile0 = static_cast<int64_t>(blockIdx.x) * kWideTile;
-    const int32_t valid = static_cast<int32_t>(n - tile0 < kWideTile ? n - tile0 : kWideTile);
-    // the tile into LDS in its own order, neighbouring lanes reading neighbouring items; a slot past the end gets
-    // the largest digit, so that it sorts behind every real item
+    const int64_t tile0 = tile * kWideTile;
+    const int64_t flat = static_cast<int64_t>(tid) * numTiles + tile;
+    r.first = prefix[flat];
+    r.next = prefix[flat + 1];
 #pragma unroll
     for (int i = 0; i < kWideItems; ++i) {
-        const int32_t p = i * kBlockThreads + tid;
-        int32_t key = static_cast<int32_t>((kWideDigits - 1) << shift);
-        RadixPair pay{0, 0u};
-        if (p < valid) {
-            const int64_t at = tile0 + p;
-            key = keysIn[at] - keyBase;
+        const int64_t at = tile0 + i * kBlockThreads + tid;
+        // a slot past the end gets the largest digit, so that it sorts behind every real item
+        r.key[i] = static_cast<int32_t>(static_cast<uint32_t>(mask) << shift);
+        r.pay[i] = RadixPair{0, 0u};
+        if (Full || at < n) {
+            r.key[i] = keysIn[at] - keyBase;
             if (Mode == kPayPairFirst) {
-                pay.row = io.rowSrc[at];
-                if (io.valueBytes == 4) {
-                    pay.val = static_cast<const uint32_t *>(io.valSrc)[at];
-                } else if (io.valueBytes == 2) {
-                    pay.val = static_cast<const uint16_t *>(io.valSrc)[at];
-                } else if (io.valueBytes == 1) {
-                    pay.val = static_cast<const uint8_t *>(io.valSrc)[at];
+                r.pay[i].row = io.rowSrc[at];
+                if (VB == 4) {
+                    r.pay[i].val = static_cast<const uint32_t *>(io.valSrc)[at];
+                } else if (VB == 2) {
+                    r.pay[i].val = static_cast<const uint16_t *>(io.valSrc)[at];
+                } else if (VB == 1) {
+                    r.pay[i].val = static_cast<const uint8_t *>(io.valSrc)[at];
                 }
             } else {
-                pay = pairsIn[at];
+                r.pay[i] = RadixPair{WideRows(pairsIn)[at], WideVals(pairsIn, n)[at]};
             }
         }
-        sKey[p] = key;
-        sPay[p] = pay;
     }
+}
+
+struct WideLds {
+    int32_t key[kWideTile];
+    __align__(8) RadixPair pay[kWideTile];
+    uint32_t word[kWideTile];
+    int32_t counters[kCounterSlots];
+    int32_t waveSums[kBlockThreads / kWave];
+    int32_t outOf[kWideDigits];  // output position less slot in the ordered tile, for the items of a digit
+};
+
+// Orders the tile held in LDS (key, pay filled, barrier not yet passed) and writes it out.  Ends with the stores
+// issued and no barrier behind them.
+template <int Mode, int VB, bool Full>
+__device__ __forceinline__ void WideOrderAndWrite(WideLds &lds, int32_t first, int32_t next, int64_t tile, int64_t n,
+                                                  int32_t shift, int32_t mask, int32_t *__restrict__ keysOut,
+                                                  RadixPair *__restrict__ pairsOut, const RadixPairIo &io)
+{
+    const int tid = threadIdx.x;
     {
         // where the tile's run of digit `tid` starts in the ordered tile, from the lengths of the runs before it
-        const int64_t flat = static_cast<int64_t>(tid) * numTiles + blockIdx.x;
-        const int32_t first = prefix[flat];
         int32_t total;
-        const int32_t start = BlockExclusiveScan(prefix[flat + 1] - first, waveSums, &total);  // has barriers
-        outOf[tid] = first - start;
+        const int32_t start = BlockExclusiveScan(next - first, lds.waveSums, &total);  // has barriers
+        lds.outOf[tid] = first - start;
     }
     // a thread takes kWideItems consecutive slots of the current order
     uint32_t word[kWideItems];
 #pragma unroll
     for (int i = 0; i < kWideItems; ++i) {
         const int32_t p = tid * kWideItems + i;
-        word[i] = (static_cast<uint32_t>(WideDigit(sKey[p], shift)) << kWideSlotBits) | static_cast<uint32_t>(p);
+        word[i] = (static_cast<uint32_t>(WideDigit(lds.key[p], shift, mask)) << kWideSlotBits) | static_cast<uint32_t>(p);
     }
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
@@ -502,45 +573,110 @@ __global__ __launch_bounds__(kBlockThreads) void WideScatterKernel(
         }
 #pragma unroll
         for (int d = 0; d < kRadixDigits; ++d) {
-            counters[Padded(d * kBlockThreads + tid)] = static_cast<int32_t>((packed >> (4 * d)) & 15);
+            lds.counters[Padded(d * kBlockThreads + tid)] = static_cast<int32_t>((packed >> (4 * d)) & 15);
         }
-        __syncthreads();
-        ScanDigitCounters(counters, waveSums);  // counters[d][t]: slots that sort before thread t's first item of d
+        LdsBarrier();
+        ScanDigitCounters(lds.counters, lds.waveSums);  // counters[d][t]: slots before thread t's first item of d
 #pragma unroll
         for (int i = 0; i < kWideItems; ++i) {
             const int32_t d = static_cast<int32_t>((word[i] >> at) & (kRadixDigits - 1));
-            sWord[counters[Padded(d * kBlockThreads + tid)] + earlier[i]] = word[i];
+            lds.word[lds.counters[Padded(d * kBlockThreads + tid)] + earlier[i]] = word[i];
         }
-        __syncthreads();
+        LdsBarrier();
         if (half == 0) {
 #pragma unroll
             for (int i = 0; i < kWideItems; ++i) {
-                word[i] = sWord[tid * kWideItems + i];
+                word[i] = lds.word[tid * kWideItems + i];
             }
         }
     }
+    const int64_t tile0 = tile * kWideTile;
+    const int32_t valid = Full ? kWideTile : static_cast<int32_t>(n - tile0);
 #pragma unroll
     for (int i = 0; i < kWideItems; ++i) {
         const int32_t p = i * kBlockThreads + tid;
-        if (p < valid) {  // the real items are the first `valid` slots of the ordered tile
-            const uint32_t w = sWord[p];
+        if (Full || p < valid) {  // the real items are the first `valid` slots of the ordered tile
+            const uint32_t w = lds.word[p];
             const int32_t slot = static_cast<int32_t>(w & ((1u << kWideSlotBits) - 1));
-            const int64_t dst = static_cast<int64_t>(outOf[w >> kWideSlotBits] + p);
-            const RadixPair out = sPay[slot];
-            keysOut[dst] = sKey[slot];
+            const int64_t dst = static_cast<int64_t>(lds.outOf[w >> kWideSlotBits] + p);
+            const RadixPair out = lds.pay[slot];
+            keysOut[dst] = lds.key[slot];
             if (Mode == kPayPairLast) {
                 io.rowOut[dst] = out.row;
-                if (io.valueBytes == 4) {
+                if (VB == 4) {
                     static_cast<uint32_t *>(io.valOut)[dst] = out.val;
-                } else if (io.valueBytes == 2) {
+                } else if (VB == 2) {
                     static_cast<uint16_t *>(io.valOut)[dst] = static_cast<uint16_t>(out.val);
-                } else if (io.valueBytes == 1) {
+                } else if (VB == 1) {
                     static_cast<uint8_t *>(io.valOut)[dst] = static_cast<uint8_t>(out.val);
                 }
             } else {
-                pairsOut[dst] = out;
+                WideRows(pairsOut)[dst] = out.row;
+                WideVals(pairsOut, n)[dst] = out.val;
             }
         }
+    }
+}
+
+template <bool Full>
+__device__ __forceinline__ void WideStage(WideLds &lds, const WideTileRegs &r)
+{
+#pragma unroll
+    for (int i = 0; i < kWideItems; ++i) {
+        const int32_t p = i * kBlockThreads + threadIdx.x;
+        lds.key[p] = r.key[i];
+        lds.pay[p] = r.pay[i];
+    }
+}
+
+// One pass; the payload modes are those of RadixScatterKernel (pairs only), VB the bytes of a value in the arrays
+// that the first pass reads and the last one writes (a template parameter: a branch on it among the loads would
+// leave the compiler unable to count what is in flight).  prefix is the scanned table:
+// prefix[digit * numTiles + tile] is the first output position of the tile's items of that digit, and the entry
+// after it, in that same flat order, ends them.  A workgroup takes the full tiles blockIdx.x, blockIdx.x +
+// gridDim.x, ... and has the loads of its next tile in flight while it orders and writes the current one (with
+// two workgroups on a compute unit and a tile's phases one after another, a tile fetched only when its turn comes
+// leaves the memory system idle most of the time: 3.2 TB/s for a pass that does nothing but copy).  The tile that
+// the end of the array cuts short is done last, by workgroup 0, with bounds checks.
+template <int Mode, int VB>
+__global__ __launch_bounds__(kBlockThreads) void WideScatterKernel(
+    const int32_t *__restrict__ keysIn, const RadixPair *__restrict__ pairsIn, int32_t *__restrict__ keysOut,
+    RadixPair *__restrict__ pairsOut, int64_t n, int32_t keyBase, int32_t shift, int32_t mask,
+    const int32_t *__restrict__ prefix, int64_t numTiles, RadixPairIo io)
+{
+    __shared__ WideLds lds;
+    const int64_t fullTiles = n / kWideTile;
+    WideTileRegs r;
+    // a workgroup's tiles are consecutive: the runs it writes into a bucket follow one another, and the cache line
+    // that one run leaves half written is completed by the next from the same compute unit
+    const int64_t perBlock = (fullTiles + gridDim.x - 1) / gridDim.x;
+    int64_t tile = blockIdx.x * perBlock;
+    const int64_t tileEnd = tile + perBlock < fullTiles ? tile + perBlock : fullTiles;
+    auto turn = [&]() {
+        WideStage<true>(lds, r);
+        const int32_t first = r.first, next = r.next;
+        // the next tile's loads (the last turn fetches its own tile again rather than branch around the loads:
+        // a wait for "all but the stores issued since" needs one straight path)
+        const int64_t ahead = tile + 1 < tileEnd ? tile + 1 : tile;
+        WideFetch<Mode, VB, true>(r, ahead, keysIn, pairsIn, n, keyBase, shift, mask, prefix, numTiles, io);
+        __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, not where the scheduler finds room later
+        WideOrderAndWrite<Mode, VB, true>(lds, first, next, tile, n, shift, mask, keysOut, pairsOut, io);
+        LdsBarrier();  // the tile's LDS is free again
+        ++tile;
+    };
+    if (tile < tileEnd) {
+        WideFetch<Mode, VB, true>(r, tile, keysIn, pairsIn, n, keyBase, shift, mask, prefix, numTiles, io);
+        // the first turn stands outside the loop: entered from here, with no stores behind the loads, the loop's
+        // wait for the loads would be a wait for everything, the stores of the turn before included
+        turn();
+        while (tile < tileEnd) {
+            turn();
+        }
+    }
+    if (blockIdx.x == 0 && fullTiles < numTiles) {
+        WideFetch<Mode, VB, false>(r, fullTiles, keysIn, pairsIn, n, keyBase, shift, mask, prefix, numTiles, io);
+        WideStage<false>(lds, r);
+        WideOrderAndWrite<Mode, VB, false>(lds, r.first, r.next, fullTiles, n, shift, mask, keysOut, pairsOut, io);
     }
 }
 
@@ -975,35 +1111,67 @@ void LaunchRadixPairPass(int mode, const int32_t *keysIn, const void *pairsIn, i
 int64_t WideTiles(int64_t n) { return (n + kWideTile - 1) / kWideTile; }
 int64_t WideTableInts(int64_t n) { return static_cast<int64_t>(kWideDigits) * WideTiles(n) + 1; }
 
+// Workgroups of the 8-bit scatter pass: two a compute unit, which is what their LDS allows to be resident.
+static uint32_t WideScatterBlocks(int64_t n)
+{
+    static const int64_t resident = [] {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        int64_t cus = 256;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+            prop.multiProcessorCount > 0) {
+            cus = prop.multiProcessorCount;
+        } else {
+            (void)hipGetLastError();
+        }
+        const char *env = std::getenv("OPS_SPARSE_WIDE_BLOCKS_PER_CU");  // tuning override
+        const int64_t perCu = env != nullptr && std::atoi(env) > 0 ? std::atoi(env) : 2;
+        return cus * perCu;
+    }();
+    const int64_t fullTiles = n / kWideTile;
+    return static_cast<uint32_t>(fullTiles < 1 ? 1 : (fullTiles < resident ? fullTiles : resident));
+}
+
 // One 8-bit pass carrying csr2csc's (row, value) pairs; table: WideTableInts(n) ints.
 void LaunchWidePairPass(int mode, const int32_t *keysIn, const void *pairsIn, int32_t *keysOut, void *pairsOut,
-                        int64_t n, int32_t keyBase, int32_t shift, int32_t *table, int32_t *scratch,
+                        int64_t n, int32_t keyBase, int32_t shift, int32_t bits, int32_t *table, int32_t *scratch,
                         const RadixPairIo &io, hipStream_t s)
 {
     if (n <= 0) {
         return;
     }
+    const int32_t mask = (1 << bits) - 1;
     const int64_t numTiles = WideTiles(n);
-    const auto grid = dim3(static_cast<uint32_t>(numTiles));
     const auto *pin = static_cast<const RadixPair *>(pairsIn);
     auto *pout = static_cast<RadixPair *>(pairsOut);
     LaunchFill(table, 1, 0, s);
-    hipLaunchKernelGGL(WideCountKernel, grid, dim3(kBlockThreads), 0, s, keysIn, n, keyBase, shift, table, numTiles);
+    hipLaunchKernelGGL(WideCountKernel, dim3(static_cast<uint32_t>((numTiles + kWideCountTiles - 1) / kWideCountTiles)),
+                       dim3(kBlockThreads), 0, s, keysIn, n, keyBase, shift, mask, table, numTiles);
     LaunchInclusiveScan(table, table, WideTableInts(n), 0, scratch, s);
+    const auto grid = dim3(WideScatterBlocks(n));
+#define OPSPARSE_WIDE_SCATTER(MODE, VB)                                                                              \
+    hipLaunchKernelGGL((WideScatterKernel<MODE, VB>), grid, dim3(kBlockThreads), 0, s, keysIn, pin, keysOut, pout, n, \
+                       keyBase, shift, mask, table, numTiles, io)
+#define OPSPARSE_WIDE_SCATTER_BY_VALUE(MODE)                                                                         \
+    switch (io.valueBytes) {                                                                                         \
+        case 4: OPSPARSE_WIDE_SCATTER(MODE, 4); break;                                                               \
+        case 2: OPSPARSE_WIDE_SCATTER(MODE, 2); break;                                                               \
+        case 1: OPSPARSE_WIDE_SCATTER(MODE, 1); break;                                                               \
+        default: OPSPARSE_WIDE_SCATTER(MODE, 0); break;                                                              \
+    }
     switch (mode) {
         case kPayPairFirst:
-            hipLaunchKernelGGL(WideScatterKernel<kPayPairFirst>, grid, dim3(kBlockThreads), 0, s, keysIn, pin, keysOut,
-                               pout, n, keyBase, shift, table, numTiles, io);
+            OPSPARSE_WIDE_SCATTER_BY_VALUE(kPayPairFirst);
             break;
         case kPayPairLast:
-            hipLaunchKernelGGL(WideScatterKernel<kPayPairLast>, grid, dim3(kBlockThreads), 0, s, keysIn, pin, keysOut,
-                               pout, n, keyBase, shift, table, numTiles, io);
+            OPSPARSE_WIDE_SCATTER_BY_VALUE(kPayPairLast);
             break;
         default:
-            hipLaunchKernelGGL(WideScatterKernel<kPayPair>, grid, dim3(kBlockThreads), 0, s, keysIn, pin, keysOut, pout,
-                               n, keyBase, shift, table, numTiles, io);
+            OPSPARSE_WIDE_SCATTER(kPayPair, 4);
             break;
     }
+#undef OPSPARSE_WIDE_SCATTER_BY_VALUE
+#undef OPSPARSE_WIDE_SCATTER
 }
 
 void LaunchGatherByPosition(const int32_t *pos, const int32_t *rowOfPos, const uint32_t *srcVal, int64_t nnz,
@@ -1288,10 +1456,14 @@ int opsparse_csr2csc_launch(int64_t m, int64_t n, int64_t nnz, const void *csrVa
     // Stable sort by column of (column; row, value): the pair travels with its key, 8 bytes a pass and entry more
     // than a source position would, and the last pass writes rows and values where they belong — no gather by
     // position at the end, which cost two cache-line fills per entry (33.5 M entries: 2.9 -> 1.9 ms).
-    // Eight bits a pass, the tile sorted through LDS before it leaves (33.5 M entries over 2^20 columns: three
-    // passes instead of five).
-    int32_t passes = (KeyBits(n) + kWideBits - 1) / kWideBits;
+    // Up to eight bits a pass, the tile ordered through LDS before it leaves (33.5 M entries over 2^20 columns:
+    // three passes instead of five, 1.2 ms).
+    const int32_t keyBits = KeyBits(n);
+    int32_t passes = (keyBits + kWideBits - 1) / kWideBits;
     passes = passes < 2 ? 2 : passes;  // a first pass that reads the sources and a last one that writes the outputs
+    // the passes share the key's bits evenly (20 bits: 7, 7, 6 rather than 8, 8, 4): the fewer buckets a pass has,
+    // the longer the runs its tiles write, and short runs are what the memory side is slow at
+    const int32_t perPass = (keyBits + passes - 1) / passes;
     const RadixPairIo io{rowOfPos, csrVal, cscRowInd, cscVal, valueBytes};
     const int32_t *keysIn = csrColInd;
     const void *pairsIn = nullptr;
@@ -1299,7 +1471,7 @@ int opsparse_csr2csc_launch(int64_t m, int64_t n, int64_t nnz, const void *csrVa
     for (int32_t pass = 0; pass < passes; ++pass) {
         const int mode = pass == 0 ? kPayPairFirst : (pass == passes - 1 ? kPayPairLast : kPayPair);
         LaunchWidePairPass(mode, keysIn, pairsIn, keys[cur], pairs[cur], nnz, pass == 0 ? indexBase : 0,
-                           pass * kWideBits, table, tiles, io, s);
+                           pass * perPass, perPass, table, tiles, io, s);
         keysIn = keys[cur];
         pairsIn = pairs[cur];
         cur ^= 1;
