@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the CSR SpMV / SpMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|c2|c3|c4|c5|convert]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|c2|c3|c4|c5|convert|cache]
 
 A step is one aclsparseSpMV (or aclsparseSpMM) call over one synthetic matrix
 whose arrays are already resident in HBM.  The headline workload is c2, the
@@ -19,7 +19,9 @@ the handle's stream, repeated until 50 ms of GPU time; the median round counts.
 Prints ONE JSON line: GFLOP/s = 2 * nnz * ncols / t as `value`, the roofline
 object (algorithmic bytes / kernel time against 8 TB/s HBM) and the CPU baseline
 (the reference's CPU golden loop restated in oracle/, timed on this host).
---workload convert times the CSR producers instead (its own JSON line).
+--workload convert times the CSR producers instead (its own JSON line); --workload cache is the Infinity-Cache
+probe: the copy / read yard-sticks by buffer size, and the c4 product with the rows of B it gathers confined to a
+window of B.
 """
 import argparse
 import ctypes
@@ -462,6 +464,44 @@ def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
     return out
 
 
+def run_cache_probe(args, osa, wl, torch, dev, stream, handle):
+    """What the 256 MB Infinity Cache is worth on this path.  (1) The copy and read kernels on buffers from 8 MiB
+    to 1 GiB, launched back to back on the same buffer.  (2) The c4 product (1 M rows of 32 entries, n = 64,
+    fp32) with the column indices drawn from the first `w` rows of B only, w x 256 bytes from 4 MiB to the whole
+    256 MiB: same entries, same bytes gathered, only the footprint of the gathered rows changes."""
+    L = osa.lib()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    res = {"yardsticks": {}, "c4_b_window": {}}
+    for mib in (8, 16, 32, 64, 128, 512, 1024):
+        nb = mib << 20
+        src = torch.zeros(nb, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        tc = time_rounds(torch, stream, lambda i: L.opsparse_copy_launch(src.data_ptr(), dst.data_ptr(), nb, sp), 20,
+                         None, 30.0)
+        tr = time_rounds(torch, stream, lambda i: L.opsparse_read_launch(src.data_ptr(), nb, None, sp), 20, None, 30.0)
+        res["yardsticks"]["%d_MiB" % mib] = {"copy_gbps": round(2 * nb / tc[0] / 1e6, 0),
+                                             "read_gbps": round(nb / tr[0] / 1e6, 0)}
+        log("buffer %4d MiB: copy %7.0f GB/s, read %7.0f GB/s" % (mib, 2 * nb / tc[0] / 1e6, nb / tr[0] / 1e6))
+        del src, dst
+    m, n = 1 << 20, 64
+    B = wl.uniform(3002, m * n, -1.0, 1.0, dev).view(m, n)
+    for wrows in (1 << 14, 1 << 15, 1 << 17, 1 << 18, 1 << 19, 1 << 20):
+        A = wl.uniform_rows_csr(m, wrows, 32, 3001, dev)
+        csr = osa.Csr(m, m, A["rowptr"], A["colind"], A["values"])
+        C = torch.zeros(m, n, device=dev)
+        op = osa.SpmmOp(handle, csr, osa.DnMat(m, n, n, B), osa.DnMat(m, n, n, C))
+        op(1.0, 0.0)
+        stream.synchronize()
+        t = time_rounds(torch, stream, lambda i: op(1.0, 0.0), 5, None, args.min_gpu_ms)
+        gathered = m * 32 * (8 + 256) + m * 256
+        res["c4_b_window"]["%d_MiB" % (wrows * 256 >> 20)] = {"ms": round(t[0], 4),
+                                                             "gather_model_gbps": round(gathered / t[0] / 1e6, 0)}
+        log("c4 shape, columns within the first %8d rows of B (%3d MiB): %.3f ms, gather model %.2f TB/s"
+            % (wrows, wrows * 256 >> 20, t[0], gathered / t[0] / 1e9))
+        del op, csr, A, C
+    return res
+
+
 def run_convert(args, osa, torch, dev, stream, handle):
     """The CSR producers (coo2csr, csr2coo, csrsort, csr2csc) on 33.5 M and 21 M entries through the aclsparse
     entry points; one JSON line with a time and an algorithmic GB/s per operation."""
@@ -526,7 +566,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all",
-                    choices=["all", "c2", "c3", "c4", "c5", "convert"],
+                    choices=["all", "c2", "c3", "c4", "c5", "convert", "cache"],
                     help="all: c2 as the headline plus c3 (default plan and ALG2), c4 and c5 in `workloads`")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
     ap.add_argument("--min-gpu-ms", type=float, default=50.0,
@@ -557,6 +597,11 @@ def main():
     torch.cuda.set_stream(stream)  # torch's fills / uploads and the library's kernels on one stream, in order
     handle = osa.Handle(stream)
 
+    if args.workload == "cache":
+        print(json.dumps({"metric": "Infinity-Cache probe", "data": "synthetic",
+                          "probe": run_cache_probe(args, osa, wl, torch, dev, stream, handle)}), flush=True)
+        handle.close()
+        return
     if args.workload == "convert":
         print(json.dumps({"metric": "CSR producers, time per call", "unit": "ms", "data": "synthetic",
                           "operations": run_convert(args, osa, torch, dev, stream, handle)}), flush=True)
