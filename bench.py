@@ -395,6 +395,14 @@ def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
         bytes_gather = wl.spmm_bytes_gather(rows, cols, ncols, nnz, vb, eb, 4, beta != 0)
         dtype = "f32" if vb == 4 else "f16 in, f32 accumulate/out"
 
+    # the buffer Preprocess was given and, for the blocked-gather layouts, the part of it the launches need
+    buf = getattr(sets[0][0], "buffer", None)
+    buffer_mib = round(buf.numel() / 2.0 ** 20, 1) if buf is not None else 0.0
+    resident_mib = buffer_mib
+    if layout.startswith("blocked_gather"):
+        flags = osa.OPSPARSE_BLOCKED_LIVE_VALUES if layout.endswith("live_values") else 0
+        resident_mib = round(osa.lib().opsparse_spmv_csr_blocked_resident_bytes(rows, cols, nnz, flags) / 2.0 ** 20, 1)
+
     def restore():
         if beta != 0:  # y back to y0 before every round, outside the timed region
             for _, t in sets:
@@ -434,7 +442,7 @@ def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
         "config": {"workload": cfg["name"], "rows": rows, "cols": cols, "nnz": nnz, "ncols_dense": ncols,
                    "alpha": alpha, "beta": beta, "index": "int32", "preprocess_ms": round(preprocess_ms, 3),
                    "first_use_ms": round(first_use_ms, 3), "preprocessed": not args.no_preprocess, "layout": layout,
-                   "operand_sets": len(sets),
+                   "operand_sets": len(sets), "buffer_mib": buffer_mib, "buffer_resident_mib": resident_mib,
                    "timing": "median over rounds of `steps` launches between HIP events on the handle's stream, "
                              "rounds repeated until %.0f ms of GPU time%s" % (
                                  args.min_gpu_ms, "; y restored to y0 before every round" if beta != 0 else "")},
@@ -626,7 +634,7 @@ def main():
     out.update(head)
     if args.workload == "all":
         out["workloads"] = {}
-        for key in ("c3", "c3_alg2", "c4", "c5"):
+        for key in ("c4", "c5", "c3", "c3_alg2"):
             out["workloads"][key] = run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache)
     print(json.dumps(out), flush=True)
     handle.close()
