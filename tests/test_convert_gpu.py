@@ -380,6 +380,24 @@ def test_csr2csc_shapes_unsorted_duplicates(osa, gpu_ctx, m, n, density):
     run_csr2csc(osa, gpu_ctx, m, n, rowptr, colind, val, np.float32, True, 0, use_buffer=False)
 
 
+@pytest.mark.parametrize("val_type,numeric", [("FP16", True), ("BF16", True), ("INT8", True), ("FP32", False)])
+@pytest.mark.parametrize("m,n,nnz", [(700, 5000, 3840 * 6), (50, 3, 3840 * 2 + 17), (9000, 40_000_000, 61_003),
+                                     (1, 70_000, 3839)])
+def test_csr2csc_value_sizes_and_key_widths_over_whole_tiles(osa, gpu_ctx, m, n, nnz, val_type, numeric):
+    """The sort passes work on tiles of 3 840 entries, whole tiles in a loop and the last, partial one apart; the
+    value size is compiled into the first and last pass.  Every value size (and none: SYMBOLIC) on entry counts
+    that are a multiple of the tile, a multiple plus a few, and just under one tile, over 2, 13, 17 and 26 column
+    bits (two to four passes), unsorted columns with repeats, both index bases."""
+    rng = np.random.default_rng(nnz + n)
+    cuts = np.sort(rng.integers(0, nnz + 1, m - 1)) if m > 1 else np.zeros(0, np.int64)
+    rowptr = np.concatenate([[0], cuts, [nnz]]).astype(np.int32)
+    colind = rng.integers(0, n, nnz).astype(np.int32)
+    val = rng.uniform(-1, 1, nnz).astype(np.float32)
+    for base in (0, 1):
+        run_csr2csc(osa, gpu_ctx, m, n, rowptr + base, colind + base, _typed(val, val_type), NP_TYPE[val_type], numeric,
+                    base)
+
+
 def test_csr2csc_twice_is_sorted_csr(osa, gpu_ctx):
     """Size-independent property at a large size: CSR -> CSC -> CSR equals the row-sorted matrix (checked against
     csrsort on the GPU and the oracle on the host)."""
