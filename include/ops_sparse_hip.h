@@ -245,8 +245,8 @@ typedef struct OpsparseSpmmPlan {
     int64_t segStartOff;   /* int32 [numSegments]: first nnz of the segment */
     int64_t longFirstSegOff; /* int32 [numLongRows + 1]: first segment of each long row */
     int64_t partialOff;    /* double [numSegments * n] */
-    int64_t reserved0;     /* unused, zero */
-    int64_t reserved1;
+    int64_t slabStartOff;  /* int32 [numSlabs + 1]: first row of every slab of the slab kernel (0: no table) */
+    int64_t numSlabs;
     int64_t bytes;
 } OpsparseSpmmPlan;
 

@@ -126,7 +126,7 @@ class OpsparseSpmmPlan(ctypes.Structure):
     _fields_ = [("kernel", i32), ("maxRowNnz", i32), ("longRowNnz", i32), ("numLongRows", i32),
                 ("numSegments", i32), ("segmentNnz", i32), ("rows", i64), ("nnz", i64), ("n", i64),
                 ("longRowsOff", i64), ("segRowOff", i64), ("segStartOff", i64), ("longFirstSegOff", i64),
-                ("partialOff", i64), ("reserved0", i64), ("reserved1", i64), ("bytes", i64)]
+                ("partialOff", i64), ("slabStartOff", i64), ("numSlabs", i64), ("bytes", i64)]
 
 
 _lib = None

@@ -299,7 +299,8 @@ template <typename ValT, typename CT, typename AccT, int V, int L, bool Small32>
 __device__ __forceinline__ void SlabBody(
     int64_t slab, const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd,
     const ValT *__restrict__ vals, const ValT *__restrict__ B, CT *__restrict__ C, int64_t rows, int32_t n, int64_t ldb,
-    int64_t ldc, int32_t rowsPerSlab, int32_t longRowNnz, OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16)
+    int64_t ldc, int32_t rowsPerSlab, const int32_t *__restrict__ slabStart, int32_t longRowNnz,
+    OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16)
 {
     typedef ValT BVec __attribute__((ext_vector_type(V)));
     typedef CT CVec __attribute__((ext_vector_type(V), aligned(16)));
@@ -324,8 +325,17 @@ __device__ __forceinline__ void SlabBody(
     const uint32_t colBytes = static_cast<uint32_t>(col) * static_cast<uint32_t>(sizeof(ValT));
     const uint32_t ldbBytes = static_cast<uint32_t>(ldb) * static_cast<uint32_t>(sizeof(ValT));
 
-    int64_t rowCur = slab * rowsPerSlab;
-    const int64_t rowEnd = (rowCur + rowsPerSlab < rows) ? rowCur + rowsPerSlab : rows;
+    // Slabs of equal work (entries + rows) from the plan's table where there is one, else of equal numbers of rows.
+    int64_t rowCur, rowEnd;
+    if (slabStart != nullptr) {
+        rowCur = slabStart[slab];
+        rowEnd = slabStart[slab + 1];
+        rowEnd = rowEnd < rows ? rowEnd : rows;  // (the table is the caller's buffer: never past the matrix)
+        rowCur = rowCur < 0 ? 0 : rowCur;
+    } else {
+        rowCur = slab * rowsPerSlab;
+        rowEnd = (rowCur + rowsPerSlab < rows) ? rowCur + rowsPerSlab : rows;
+    }
 
     while (rowCur < rowEnd) {  // uniform over the workgroup
         const int32_t win = (rowEnd - rowCur < kSlabRowsMax) ? static_cast<int32_t>(rowEnd - rowCur) : kSlabRowsMax;
@@ -533,8 +543,8 @@ template <typename ValT, typename CT, typename AccT, int V, int L, bool Small32>
 __global__ __launch_bounds__(kBlockThreads, SlabTuning<V>::kWavesPerSimd) void SpmmSlabKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
     const ValT *__restrict__ B, CT *__restrict__ C, int64_t rows, int32_t n, int64_t ldb, int64_t ldc,
-    int32_t rowsPerSlab, int32_t longRowNnz, OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16,
-    uint32_t segBlocks, int32_t numSegments, const int32_t *__restrict__ segRow,
+    int32_t rowsPerSlab, const int32_t *__restrict__ slabStart, int32_t longRowNnz, OpsparseScalar alphaS,
+    OpsparseScalar betaS, int32_t clampF16, uint32_t segBlocks, int32_t numSegments, const int32_t *__restrict__ segRow,
     const int32_t *__restrict__ segStart, AccT *__restrict__ partial)
 {
     int64_t slab;
@@ -552,7 +562,7 @@ __global__ __launch_bounds__(kBlockThreads, SlabTuning<V>::kWavesPerSimd) void S
         slab = XcdContiguousTile(blockIdx.x, gridDim.x);
     }
     SlabBody<ValT, CT, AccT, V, L, Small32>(slab, rowOffsets, colInd, vals, B, C, rows, n, ldb, ldc, rowsPerSlab,
-                                            longRowNnz, alphaS, betaS, clampF16);
+                                            slabStart, longRowNnz, alphaS, betaS, clampF16);
 }
 
 // One workgroup per long row.  Each of its four wavefronts adds a contiguous
@@ -753,11 +763,35 @@ inline int CheckLaunch()
 
 inline int64_t Align256(int64_t v) { return (v + 255) / 256 * 256; }
 
-// Workspace: 256-byte header | long row ids | first segment per long row (+1) |
+// Slabs of the slab kernel: about kSlabTarget entries each, cut where the running count of entries + rows passes
+// a multiple of `share` (a row costs its entries and one row of C), so that a matrix whose rows are sorted by
+// length is cut as evenly as one whose rows are mixed.
+int64_t SlabShare(int64_t rows, int64_t nnz)
+{
+    static const int64_t target = std::getenv("OPS_SPARSE_SPMM_SLAB_ENTRIES") != nullptr
+                                      ? std::atoll(std::getenv("OPS_SPARSE_SPMM_SLAB_ENTRIES"))
+                                      : kSlabTarget;
+    const int64_t t = target < 64 ? 64 : target;
+    int64_t rps = nnz > 0 ? t * rows / nnz : 4096;
+    rps = rps < 16 ? 16 : (rps > 4096 ? 4096 : rps);
+    return t + rps;
+}
+
+int64_t SlabCount(int64_t rows, int64_t nnz)
+{
+    const int64_t share = SlabShare(rows, nnz);
+    return (rows + nnz + share - 1) / share;
+}
+
+// Workspace: 256-byte header | first row per slab (+1) | long row ids | first segment per long row (+1) |
 // row id per segment | first entry per segment | fp64 partials [segments x n].
 void LayoutPlan(OpsparseSpmmPlan *p)
 {
     int64_t off = 256;
+    p->numSlabs = SlabCount(p->rows, p->nnz);
+    p->slabStartOff = off;
+    off = Align256(off + 4 * (p->numSlabs + 1));
+    const int64_t slabEnd = off;
     p->longRowsOff = off;
     off = Align256(off + 4 * static_cast<int64_t>(p->numLongRows));
     p->longFirstSegOff = off;
@@ -768,7 +802,33 @@ void LayoutPlan(OpsparseSpmmPlan *p)
     off = Align256(off + 4 * static_cast<int64_t>(p->numSegments));
     p->partialOff = off;
     off = Align256(off + 8 * static_cast<int64_t>(p->numSegments) * p->n);
-    p->bytes = p->numLongRows > 0 ? off : 256;
+    p->bytes = p->numLongRows > 0 ? off : slabEnd;
+}
+
+// slabStart[s] = first row r with rowOffsets[r] + r >= s * share (slabStart[numSlabs] = rows).
+__global__ __launch_bounds__(kBlockThreads) void SpmmSlabTableKernel(const int32_t *__restrict__ rowOffsets,
+                                                                    int64_t rows, int64_t numSlabs, int64_t share,
+                                                                    int32_t *__restrict__ slabStart)
+{
+    const int64_t s = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (s > numSlabs) {
+        return;
+    }
+    int64_t lo = 0, hi = rows;
+    if (s == numSlabs) {
+        lo = rows;
+    } else {
+        const int64_t want = s * share;
+        while (lo < hi) {
+            const int64_t mid = (lo + hi) >> 1;
+            if (static_cast<int64_t>(rowOffsets[mid]) - rowOffsets[0] + mid < want) {
+                lo = mid + 1;
+            } else {
+                hi = mid;
+            }
+        }
+    }
+    slabStart[s] = static_cast<int32_t>(lo);
 }
 
 // Tables of the long rows: longRows[i] = row, firstSeg[i] = its first segment (firstSeg[numLongRows] = all
@@ -889,13 +949,17 @@ template <typename ValT, typename CT, typename AccT, int V, int L>
 int LaunchSlab(const SpmmArgs &a)
 {
     const bool binned = a.plan->kernel == OPSPARSE_SPMM_BINNED && a.plan->numLongRows > 0;
-    // Slabs of about kSlabTarget entries on average.
+    // Slabs of about kSlabTarget entries: of equal work from the plan's table, of equal numbers of rows without it.
     static const int64_t target = std::getenv("OPS_SPARSE_SPMM_SLAB_ENTRIES") != nullptr
                                       ? std::atoll(std::getenv("OPS_SPARSE_SPMM_SLAB_ENTRIES"))
                                       : kSlabTarget;
     int64_t rps = a.nnz > 0 ? target * a.rows / a.nnz : 4096;
     rps = rps < 16 ? 16 : (rps > 4096 ? 4096 : rps);
-    const uint32_t grid = static_cast<uint32_t>((a.rows + rps - 1) / rps);
+    static const bool noTable = std::getenv("OPS_SPARSE_SPMM_NO_SLAB_TABLE") != nullptr;
+    const bool table = !noTable && a.plan->slabStartOff > 0 && a.plan->numSlabs > 0;
+    const int32_t *slabStart =
+        table ? reinterpret_cast<const int32_t *>(static_cast<unsigned char *>(a.ws) + a.plan->slabStartOff) : nullptr;
+    const uint32_t grid = table ? static_cast<uint32_t>(a.plan->numSlabs) : static_cast<uint32_t>((a.rows + rps - 1) / rps);
     const int32_t longRowNnz = binned ? a.plan->longRowNnz : kSlabCap;
     const bool small32 = static_cast<uint64_t>(a.k) * static_cast<uint64_t>(a.ldb) * sizeof(ValT) < (1ull << 32);
     // Long rows: their segment workgroups ride in the same launch, the fix-up follows.
@@ -911,8 +975,8 @@ int LaunchSlab(const SpmmArgs &a)
         hipLaunchKernelGGL((SpmmSlabKernel<ValT, CT, AccT, V, L, kSmall>), dim3(grid + segBlocks), dim3(kBlockThreads),
                            0, a.stream, a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
                            static_cast<const ValT *>(a.B), static_cast<CT *>(a.C), a.rows, static_cast<int32_t>(a.n),
-                           a.ldb, a.ldc, static_cast<int32_t>(rps), longRowNnz, a.alpha, a.beta, a.clampF16, segBlocks,
-                           nseg, segRow, segStart, partial);
+                           a.ldb, a.ldc, static_cast<int32_t>(rps), slabStart, longRowNnz, a.alpha, a.beta, a.clampF16,
+                           segBlocks, nseg, segRow, segStart, partial);
     };
     if (small32) {
         launch(std::true_type{});
@@ -1014,6 +1078,8 @@ int opsparse_spmm_csr_workspace_bytes(const int32_t *rowOffsets, int64_t rows, i
         return rc;
     }
     OpsparseSpmmPlan p{};
+    p.rows = rows;
+    p.nnz = nnz;
     p.n = n;
     p.numLongRows = st[1];
     p.numSegments = st[2];
@@ -1050,14 +1116,26 @@ int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t n
         return rc;
     }
     p.maxRowNnz = st[0];
-    if (st[1] == 0) {
-        *plan = p;
-        return OPSPARSE_OK;
-    }
-    p.kernel = OPSPARSE_SPMM_BINNED;
     p.numLongRows = st[1];
     p.numSegments = st[2];
     LayoutPlan(&p);
+    auto *base = static_cast<unsigned char *>(workspace);
+    if (static_cast<int64_t>(workspaceBytes) >= p.slabStartOff + 4 * (p.numSlabs + 1)) {
+        hipLaunchKernelGGL(SpmmSlabTableKernel, dim3(static_cast<uint32_t>((p.numSlabs + kBlockThreads) / kBlockThreads)),
+                           dim3(kBlockThreads), 0, s, rowOffsets, rows, p.numSlabs, SlabShare(rows, nnz),
+                           reinterpret_cast<int32_t *>(base + p.slabStartOff));
+    } else if (st[1] == 0) {
+        p.slabStartOff = 0;  // a 256-byte workspace, which is all a matrix without long rows used to need:
+        p.numSlabs = 0;      // slabs of equal numbers of rows then
+        p.bytes = 256;
+    }
+    if (st[1] == 0) {
+        p.numLongRows = 0;
+        p.numSegments = 0;
+        *plan = p;
+        return CheckLaunch();
+    }
+    p.kernel = OPSPARSE_SPMM_BINNED;
     if (static_cast<int64_t>(workspaceBytes) < p.bytes) {
         return OPSPARSE_E_WORKSPACE;
     }
@@ -1066,7 +1144,6 @@ int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t n
     // numberings agree and firstSeg is a prefix sum whatever order the rows arrive in.  Nothing but the counter
     // comes back to the host (the reference copies the row offsets to the host and builds its tables there,
     // sparse/spmm/arch35/spmm_csr_mat.cpp:94-136).
-    auto *base = static_cast<unsigned char *>(workspace);
     auto *counter = reinterpret_cast<unsigned long long *>(base + 16);
     if (hipMemsetAsync(counter, 0, sizeof(unsigned long long), s) != hipSuccess) {
         (void)hipGetLastError();

@@ -269,12 +269,16 @@ def _lengths(shape, m, rng):
         lengths = np.arange(m) % 2
     elif shape == "power_law":
         lengths = np.minimum((1.0 / rng.uniform(1e-4, 1.0, m)).astype(np.int64), 4000)
+    elif shape in ("sorted_up", "sorted_down"):  # a graph ordered by degree: slabs are cut by work, not by rows
+        lengths = np.sort(np.minimum((1.0 / rng.uniform(1e-4, 1.0, m)).astype(np.int64), 4000))
+        lengths = lengths[::-1].copy() if shape == "sorted_down" else lengths
     else:
         raise ValueError(shape)
     return lengths
 
 
-@pytest.mark.parametrize("shape", ["mostly_empty", "threshold", "dense_slabs", "alternating", "power_law"])
+@pytest.mark.parametrize("shape", ["mostly_empty", "threshold", "dense_slabs", "alternating", "power_law",
+                                   "sorted_up", "sorted_down"])
 @pytest.mark.parametrize("n,beta", [(8, 0.0), (24, 0.5), (64, -1.0), (256, 0.0)])
 def test_row_length_mixes(osa, gpu_ctx, shape, n, beta):
     """Preprocessed fast path (rows worked in LDS-staged slabs, long rows in segments) on row-length mixes that
@@ -290,6 +294,38 @@ def test_row_length_mixes(osa, gpu_ctx, shape, n, beta):
     got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, n, C0, n, 1.25, beta)
     gold = oracle.spmm_f64_rowmajor(m, n, rowptr, colind, val, B, n, np.nan_to_num(C0), n, 1.25, beta)
     assert oracle.max_rel_err(got, gold) <= 1e-5
+
+
+def test_slab_table_cuts_by_work(osa, gpu_ctx):
+    """The analysis leaves, for the slab kernel, the first row of every slab: slab s starts at the first row with
+    s * share entries + rows in front of it, whatever the order of the rows (checked against numpy on rows sorted
+    by length, where slabs of equal numbers of rows would differ in work a hundredfold)."""
+    import torch
+    dev, stream, handle = gpu_ctx
+    rng = np.random.default_rng(3)
+    m = 300_000
+    lengths = np.sort(np.minimum((1.0 / rng.uniform(1e-4, 1.0, m)).astype(np.int64), 256))[::-1].copy()
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    nnz = int(rowptr[-1])
+    L = osa.lib()
+    d_rp = to_dev(rowptr, dev)
+    size = ctypes.c_size_t(0)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    assert L.opsparse_spmm_csr_workspace_bytes(d_rp.data_ptr(), m, nnz, 64, sp, ctypes.byref(size)) == 0
+    ws = torch.zeros(size.value, dtype=torch.uint8, device=dev)
+    plan = osa.OpsparseSpmmPlan()
+    assert L.opsparse_spmm_csr_analyse(d_rp.data_ptr(), m, nnz, 64, ws.data_ptr(), size.value, 0, ctypes.byref(plan),
+                                       sp) == 0
+    stream.synchronize()
+    assert plan.numSlabs > 0 and plan.slabStartOff >= 256 and plan.bytes <= size.value
+    table = ws[plan.slabStartOff: plan.slabStartOff + 4 * (plan.numSlabs + 1)].view(torch.int32).cpu().numpy()
+    work = rowptr[:-1].astype(np.int64) + np.arange(m)            # entries + rows in front of row r
+    share = 2048 + min(max(2048 * m // nnz, 16), 4096)            # about 2048 entries and their rows a slab
+    assert plan.numSlabs == -(-(m + nnz) // share)
+    want = np.concatenate([np.searchsorted(work, np.arange(plan.numSlabs) * share, side="left"), [m]])
+    assert np.array_equal(table, want)
+    per_slab = np.diff(np.concatenate([work, [m + nnz]])[table])
+    assert per_slab.max() <= share + 257                           # a slab overshoots its share by at most a row
 
 
 @pytest.mark.parametrize("shape", ["threshold", "power_law"])
