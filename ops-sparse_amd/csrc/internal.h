@@ -35,6 +35,10 @@ inline size_t AlignUp(size_t v, size_t a) { return (v + a - 1) / a * a; }
 struct OpsparseSpmvBinding {
     const void *buffer = nullptr;  // buffer this plan was written into
     OpsparseSpmvPlan plan{};
+    // op(A) = A^T with fp16 / bf16 y sums into an fp32 vector of `cols` elements: room for it behind the plan's
+    // own part of the buffer (0 bytes: the buffer was preprocessed for a call that needs none)
+    int64_t stagingOffset = 0;
+    int64_t stagingBytes = 0;
 };
 
 // What the first aclsparseSpMV call without a preprocessed buffer learns about the rows of a matrix: the row-wise

@@ -248,6 +248,18 @@ int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *co
 
 }  // namespace opsparse
 
+namespace {
+
+// op(A) = A^T with fp16 / bf16 y: the sums are formed in an fp32 vector of `cols` elements and rounded once.
+bool StagedTranspose(const SpmvCall &c)
+{
+    const int32_t yType = DtypeOf(c.y->valueType);  // (outType is only filled in by ValidateData)
+    return c.transpose && (yType == OPSPARSE_F16 || yType == OPSPARSE_BF16);
+}
+size_t StagingBytes(aclsparseConstSpMatDescr_t matA) { return static_cast<size_t>(matA->cols) * sizeof(float); }
+
+}  // namespace
+
 extern "C" {
 
 aclsparseStatus_t aclsparseSpMVGetBufferSize(aclsparseHandle_t handle, aclsparseOperation_t opA, const void * /*alpha*/,
@@ -265,7 +277,8 @@ aclsparseStatus_t aclsparseSpMVGetBufferSize(aclsparseHandle_t handle, aclsparse
     }
     const size_t plain = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
     const Restored restored = RestoredLayout(handle, opA, matA, vecX, vecY, computeType, alg);
-    *bufferSize = restored.bytes > plain ? restored.bytes : plain;
+    const size_t own = restored.bytes > plain ? restored.bytes : plain;
+    *bufferSize = StagedTranspose(c) ? opsparse::AlignUp(own, 256) + StagingBytes(matA) : own;
     return ACL_SPARSE_STATUS_SUCCESS;
 }
 
@@ -309,6 +322,15 @@ aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOpe
     }
     matA->spmv.buffer = externalBuffer;
     matA->spmv.plan = plan;
+    matA->spmv.stagingOffset = 0;
+    matA->spmv.stagingBytes = 0;
+    if (StagedTranspose(c)) {
+        // behind everything GetBufferSize counted for the plan (the same sum as there)
+        const size_t plain = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
+        const size_t own = restored.bytes > plain ? restored.bytes : plain;
+        matA->spmv.stagingOffset = static_cast<int64_t>(opsparse::AlignUp(own, 256));
+        matA->spmv.stagingBytes = static_cast<int64_t>(StagingBytes(matA));
+    }
     return ACL_SPARSE_STATUS_SUCCESS;
 }
 
@@ -369,6 +391,13 @@ aclsparseStatus_t aclsparseSpMV(aclsparseHandle_t handle, aclsparseOperation_t o
         wsBytes = handle->workspaceBytes();
         if (plan == nullptr && matA->nnz > 0 && matA->rows > 0) {
             plan = RowsSeen(handle, matA, c.transpose);
+        }
+        if (StagedTranspose(c) && bound && wsBytes < StagingBytes(matA) &&
+            matA->spmv.stagingBytes >= static_cast<int64_t>(StagingBytes(matA))) {
+            // y too long for the handle's workspace: the buffer was preprocessed for this kind of call and has
+            // the room (a transposed product uses the workspace for nothing else)
+            ws = static_cast<unsigned char *>(externalBuffer) + matA->spmv.stagingOffset;
+            wsBytes = static_cast<size_t>(matA->spmv.stagingBytes);
         }
     }
     const int rc = opsparse_spmv_csr_launch(

@@ -516,6 +516,54 @@ def test_transpose_half_precision_output(osa, gpu_ctx, dtype, rel, beta):
     assert np.all(np.abs(y - gold) <= rel * np.abs(gold) + 1e-4)
 
 
+def test_transpose_half_precision_output_longer_than_the_workspace(osa, gpu_ctx):
+    """fp16 y of 1.5 M elements under op(A) = A^T: its fp32 staging vector (6 MB) does not fit the handle's 4 MiB
+    workspace.  aclsparseSpMVGetBufferSize counts it in, and the call sums in the preprocessed buffer; without
+    Preprocess the call reports INSUFFICIENT_RESOURCES (aclsparseSetWorkspace is the way then) and leaves y."""
+    dev, stream, handle = gpu_ctx
+    rows, cols, per_row = 4000, 1_500_000, 25
+    rng = np.random.default_rng(77)
+    rowptr = (np.arange(rows + 1) * per_row).astype(np.int32)
+    colind = rng.integers(0, cols, rows * per_row).astype(np.int32)
+    rt = lambda a: torch.from_numpy(a.astype(np.float32)).to(torch.float16).float().numpy()
+    val, x, y0 = rt(rng.uniform(-1, 1, colind.size)), rt(rng.uniform(-1, 1, rows)), rt(rng.uniform(-1, 1, cols))
+    gold = oracle.spmv_trans_f64(rows, cols, rowptr, colind, val, x, y0, 1.5, 0.5)
+    d_rp, d_ci = to_dev(rowptr, dev), to_dev(colind, dev)
+    d_val, d_x = to_dev(val, dev, torch.float16), to_dev(x, dev, torch.float16)
+    A, X = osa.Csr(rows, cols, d_rp, d_ci, d_val), osa.DnVec(d_x)
+    # unprepared: the default workspace is too small
+    d_y = to_dev(y0, dev, torch.float16)
+    bare = osa.SpmvOp(handle, A, X, osa.DnVec(d_y), op=osa.ACL_SPARSE_OP_TRANSPOSE, preprocess=False)
+    with pytest.raises(osa.AclsparseError) as err:
+        bare(1.5, 0.5)
+    assert err.value.status == osa.ACL_SPARSE_STATUS_INSUFFICIENT_RESOURCES
+    stream.synchronize()
+    assert np.array_equal(d_y.cpu().float().numpy(), y0)
+    # preprocessed: the buffer holds the staging vector behind the plan
+    Y = osa.DnVec(d_y)
+    n = ctypes.c_size_t(0)
+    L = osa.lib()
+    assert L.aclsparseSpMVGetBufferSize(handle.h, osa.ACL_SPARSE_OP_TRANSPOSE, None, A.d, X.d, None, Y.d, osa.ACL_FLOAT,
+                                        0, ctypes.byref(n)) == 0
+    assert n.value >= cols * 4
+    op = osa.SpmvOp(handle, A, X, Y, op=osa.ACL_SPARSE_OP_TRANSPOSE)
+    for _ in range(2):                                                     # the buffer serves every call
+        d_y.copy_(torch.from_numpy(y0).to(torch.float16))
+        op(1.5, 0.5)
+        stream.synchronize()
+        y = d_y.cpu().float().numpy()
+        assert np.all(np.abs(y - gold) <= 2.0 ** -10 * np.abs(gold) + 1e-4)
+    # the same buffer still serves op(A) = A (its own part is in front of the staging vector)
+    d_x2, d_y2 = to_dev(rt(rng.uniform(-1, 1, cols)), dev, torch.float16), torch.zeros(rows, dtype=torch.float16, device=dev)
+    (ka, pa), (kb, pb) = osa._scalar_ref(1.0, osa.ACL_FLOAT), osa._scalar_ref(0.0, osa.ACL_FLOAT)
+    X2, Y2 = osa.DnVec(d_x2), osa.DnVec(d_y2)
+    st = L.aclsparseSpMV(handle.h, 0, pa, A.d, X2.d, pb, Y2.d, osa.ACL_FLOAT, 0, ctypes.c_void_p(op.buffer.data_ptr()))
+    assert st == 0
+    stream.synchronize()
+    gold2 = oracle.spmv_f64(rows, cols, rowptr, colind, val, d_x2.cpu().float().numpy(), np.zeros(rows, np.float32), 1.0, 0.0)
+    assert np.all(np.abs(d_y2.cpu().float().numpy() - gold2) <= 2.0 ** -10 * np.abs(gold2) + 1e-4)
+
+
 @pytest.mark.parametrize("per_row,out_dtype", [(4, None), (20, None), (6, torch.float16), (40, None)])
 def test_unprepared_calls_survive_row_offsets_changed_in_place(osa, gpu_ctx, per_row, out_dtype):
     """The first call without a preprocessed buffer takes the row statistics of the matrix, and later ones run the
