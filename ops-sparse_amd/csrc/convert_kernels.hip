@@ -728,43 +728,123 @@ __device__ __forceinline__ int32_t SortKeyColumn(uint64_t key)
     return static_cast<int32_t>(static_cast<uint32_t>(key >> 32) ^ 0x80000000u);
 }
 
-// Bitonic sort of one (key, payload) per lane over the G lanes of a group; `g` is
-// the lane's index in its group.  Returns the sorted key; *pay follows its key.
-template <int G>
-__device__ __forceinline__ uint64_t GroupBitonicSort(uint64_t key, int32_t *pay, int32_t g)
+// The value of lane (l ^ J) for every lane l of a wavefront, all of whose lanes are active.  Distances 1, 2, 4
+// and 8 stay inside a row of 16 lanes and are data-parallel-primitive moves in the vector ALU (quad permutes,
+// rotations of a row); only 16 and 32 go through the LDS crossbar, where every distance went before (the sort of
+// a 64-lane group issued 42 such operations and spent its time waiting for them).  `ror4` says whether the
+// rotation by 4 or the one by 12 brings lane l the value of lane l ^ 4: found once per thread by sending the
+// lane numbers through both, which leaves the direction of the rotation out of the argument.
+__device__ __forceinline__ uint32_t DppMove(uint32_t v, int ctrl)
 {
-    const int32_t lane = threadIdx.x % kWave;
-#pragma unroll
-    for (int k = 2; k <= G; k <<= 1) {
-#pragma unroll
-        for (int j = k >> 1; j > 0; j >>= 1) {
-            const uint64_t other = __shfl_xor(key, j, kWave);
-            const bool ascending = (g & k) == 0;
-            const bool lower = (g & j) == 0;
-            const uint64_t mn = key < other ? key : other;
-            const uint64_t mx = key < other ? other : key;
-            key = (ascending == lower) ? mn : mx;
-        }
+    switch (ctrl) {  // the control word is an immediate of the instruction
+        case 0xB1: return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0xB1, 0xF, 0xF, false));
+        case 0x4E: return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x4E, 0xF, 0xF, false));
+        case 0x124: return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x124, 0xF, 0xF, false));
+        case 0x128: return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x128, 0xF, 0xF, false));
+        default: return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x12C, 0xF, 0xF, false));
     }
-    // the low half of a key is the lane (in the group) its entry came from
-    const int32_t from = (lane - g) + (static_cast<int32_t>(key & 0xffffffffu) & (G - 1));
-    *pay = __shfl(*pay, from, kWave);
+}
+
+__device__ __forceinline__ bool Ror4IsXor4()
+{
+    const uint32_t lane = threadIdx.x % kWave;
+    return DppMove(lane, 0x124) == (lane ^ 4u);
+}
+
+template <int J>
+__device__ __forceinline__ uint32_t XorLanes(uint32_t v, bool ror4)
+{
+    if (J == 1) {
+        return DppMove(v, 0xB1);  // quad_perm [1, 0, 3, 2]
+    } else if (J == 2) {
+        return DppMove(v, 0x4E);  // quad_perm [2, 3, 0, 1]
+    } else if (J == 4) {
+        const uint32_t a = DppMove(v, 0x124), b = DppMove(v, 0x12C);  // row_ror 4 and 12
+        return ror4 ? a : b;
+    } else if (J == 8) {
+        return DppMove(v, 0x128);  // row_ror 8: the same in either direction
+    } else {
+        return static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), J, kWave));
+    }
+}
+
+template <int J>
+__device__ __forceinline__ uint64_t XorLanes(uint64_t v, bool ror4)
+{
+    const uint32_t lo = XorLanes<J>(static_cast<uint32_t>(v), ror4);
+    const uint32_t hi = XorLanes<J>(static_cast<uint32_t>(v >> 32), ror4);
+    return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+
+template <int K, int J, typename KeyT>
+__device__ __forceinline__ void BitonicStep(KeyT &key, int32_t g, bool ror4)
+{
+    const KeyT other = XorLanes<J>(key, ror4);
+    const bool ascending = (g & K) == 0;
+    const bool lower = (g & J) == 0;
+    const KeyT mn = key < other ? key : other;
+    const KeyT mx = key < other ? other : key;
+    key = (ascending == lower) ? mn : mx;
+}
+
+template <int K, int J, typename KeyT>
+__device__ __forceinline__ void BitonicMerge(KeyT &key, int32_t g, bool ror4)
+{
+    BitonicStep<K, J>(key, g, ror4);
+    if constexpr (J > 1) {
+        BitonicMerge<K, J / 2>(key, g, ror4);
+    }
+}
+
+template <int G, int K, typename KeyT>
+__device__ __forceinline__ void BitonicStages(KeyT &key, int32_t g, bool ror4)
+{
+    BitonicMerge<K, K / 2>(key, g, ror4);
+    if constexpr (K < G) {
+        BitonicStages<G, K * 2>(key, g, ror4);
+    }
+}
+
+// Bitonic sort of one key per lane over the G lanes of a group (all 64 lanes of the wavefront take part); `g` is
+// the lane's index in its group.  The low bits of a key hold the group lane its entry came from, so all keys
+// differ and the sort is the stable one.  Returns the sorted key.
+template <int G, typename KeyT>
+__device__ __forceinline__ KeyT GroupBitonicSort(KeyT key, int32_t g)
+{
+    const bool ror4 = Ror4IsXor4();
+    BitonicStages<G, 2>(key, g, ror4);
     return key;
 }
 
-template <int G>
+// Packed: the key is (column << log2 G | lane) in 32 bits, half the moves of the 64-bit key; the launcher takes
+// it when every column index of a valid matrix fits (columns outside [0, n) then only lose their order: the
+// entries themselves travel by source lane, not inside the key).
+template <int G, bool Packed>
 __device__ __forceinline__ void SortRowInGroup(int64_t begin, int64_t len, int32_t g, int32_t *colInd, int32_t *perm)
 {
+    constexpr int kLog = G == 64 ? 6 : G == 32 ? 5 : G == 16 ? 4 : 3;
+    static_assert((1 << kLog) == G, "8, 16, 32 or 64 lanes a row");
+    const int32_t lane = threadIdx.x % kWave;
     const bool valid = g < len;
-    uint64_t key = ~0ull;  // padding sorts last
-    int32_t pay = 0;
+    int32_t col = 0, pay = 0;
     if (valid) {
-        key = SortKey(colInd[begin + g], static_cast<uint32_t>(g));
+        col = colInd[begin + g];
         pay = perm[begin + g];
     }
-    key = GroupBitonicSort<G>(key, &pay, g);
+    int32_t from;
+    if (Packed) {
+        uint32_t key = valid ? (static_cast<uint32_t>(col) << kLog) | static_cast<uint32_t>(g) : ~0u;  // padding last
+        key = GroupBitonicSort<G>(key, g);
+        from = (lane - g) + static_cast<int32_t>(key & (G - 1));
+    } else {
+        uint64_t key = valid ? SortKey(col, static_cast<uint32_t>(g)) : ~0ull;
+        key = GroupBitonicSort<G>(key, g);
+        from = (lane - g) + (static_cast<int32_t>(key & 0xffffffffu) & (G - 1));
+    }
+    col = __shfl(col, from, kWave);
+    pay = __shfl(pay, from, kWave);
     if (valid) {
-        colInd[begin + g] = SortKeyColumn(key);
+        colInd[begin + g] = col;
         perm[begin + g] = pay;
     }
 }
@@ -773,7 +853,7 @@ __device__ __forceinline__ void SortRowInGroup(int64_t begin, int64_t len, int32
 // network over the group's lanes); rows of up to 64 entries that do not fit the
 // group go to midList (one wavefront each, next kernel), longer rows to longList.
 // counters[0] / counters[1] are the two list lengths.
-template <int G>
+template <int G, bool Packed>
 __global__ __launch_bounds__(kBlockThreads) void SortShortRowsKernel(const int32_t *__restrict__ rowPtr, int64_t m,
                                                                     int64_t nnz, int32_t base, int32_t *colInd,
                                                                     int32_t *perm, int32_t *counters,
@@ -801,10 +881,11 @@ __global__ __launch_bounds__(kBlockThreads) void SortShortRowsKernel(const int32
         len = 0;
     }
     // every lane takes part in the shuffles; groups without a row sort padding
-    SortRowInGroup<G>(begin, len, g, colInd, perm);
+    SortRowInGroup<G, Packed>(begin, len, g, colInd, perm);
 }
 
 // Wavefronts walk midList: rows of up to 64 entries, one wavefront each.
+template <bool Packed>
 __global__ __launch_bounds__(kBlockThreads) void SortMidRowsKernel(const int32_t *__restrict__ rowPtr, int32_t base,
                                                                   int32_t *colInd, int32_t *perm,
                                                                   const int32_t *__restrict__ counters,
@@ -817,7 +898,7 @@ __global__ __launch_bounds__(kBlockThreads) void SortMidRowsKernel(const int32_t
         const int32_t row = midList[item];
         const int64_t begin = static_cast<int64_t>(rowPtr[row]) - base;
         const int64_t len = static_cast<int64_t>(rowPtr[row + 1]) - base - begin;
-        SortRowInGroup<kWave>(begin, len, lane, colInd, perm);
+        SortRowInGroup<kWave, Packed>(begin, len, lane, colInd, perm);
     }
 }
 
@@ -1378,27 +1459,39 @@ int opsparse_csrsort_launch(int64_t m, int64_t n, int64_t nnz, int32_t indexBase
     const int64_t mean2 = 2 * nnz / m;
     const int g = mean2 <= 8 ? 8 : mean2 <= 16 ? 16 : mean2 <= 32 ? 32 : 64;
     const auto shortGrid = dim3(GridFor(m, kBlockThreads / g));
-    switch (g) {
-        case 8:
-            hipLaunchKernelGGL(SortShortRowsKernel<8>, shortGrid, dim3(kBlockThreads), 0, s, csrRowPtr, m, nnz,
-                               indexBase, csrColInd, perm, counters, midList, longList);
-            break;
-        case 16:
-            hipLaunchKernelGGL(SortShortRowsKernel<16>, shortGrid, dim3(kBlockThreads), 0, s, csrRowPtr, m, nnz,
-                               indexBase, csrColInd, perm, counters, midList, longList);
-            break;
-        case 32:
-            hipLaunchKernelGGL(SortShortRowsKernel<32>, shortGrid, dim3(kBlockThreads), 0, s, csrRowPtr, m, nnz,
-                               indexBase, csrColInd, perm, counters, midList, longList);
-            break;
-        default:
-            hipLaunchKernelGGL(SortShortRowsKernel<64>, shortGrid, dim3(kBlockThreads), 0, s, csrRowPtr, m, nnz,
-                               indexBase, csrColInd, perm, counters, midList, longList);
-            break;
+    // 32-bit keys (column and lane packed) where the columns of a valid matrix leave room for the lane number
+    auto packedFor = [&](int lanes) {
+        int log = 0;
+        while ((1 << log) < lanes) {
+            ++log;
+        }
+        return static_cast<int64_t>(n) + indexBase < (int64_t{1} << (32 - log)) - 1;
+    };
+#define OPSPARSE_SORT_SHORT(G, PACKED)                                                                              \
+    hipLaunchKernelGGL((SortShortRowsKernel<G, PACKED>), shortGrid, dim3(kBlockThreads), 0, s, csrRowPtr, m, nnz,    \
+                       indexBase, csrColInd, perm, counters, midList, longList)
+#define OPSPARSE_SORT_SHORT_G(G)            \
+    if (packedFor(G)) {                     \
+        OPSPARSE_SORT_SHORT(G, true);       \
+    } else {                                \
+        OPSPARSE_SORT_SHORT(G, false);      \
     }
+    switch (g) {
+        case 8: OPSPARSE_SORT_SHORT_G(8); break;
+        case 16: OPSPARSE_SORT_SHORT_G(16); break;
+        case 32: OPSPARSE_SORT_SHORT_G(32); break;
+        default: OPSPARSE_SORT_SHORT_G(64); break;
+    }
+#undef OPSPARSE_SORT_SHORT_G
+#undef OPSPARSE_SORT_SHORT
     if (g < kSortWaveRow) {
-        hipLaunchKernelGGL(SortMidRowsKernel, dim3(kSortListBlocks), dim3(kBlockThreads), 0, s, csrRowPtr, indexBase,
-                           csrColInd, perm, counters, midList);
+        if (packedFor(kWave)) {
+            hipLaunchKernelGGL(SortMidRowsKernel<true>, dim3(kSortListBlocks), dim3(kBlockThreads), 0, s, csrRowPtr,
+                               indexBase, csrColInd, perm, counters, midList);
+        } else {
+            hipLaunchKernelGGL(SortMidRowsKernel<false>, dim3(kSortListBlocks), dim3(kBlockThreads), 0, s, csrRowPtr,
+                               indexBase, csrColInd, perm, counters, midList);
+        }
     }
     // Listed rows of up to kSortWideRow entries: 256 lanes each, many rows at a time.  The few beyond: 1024 lanes
     // each, because the longest of them is what the call waits for (a row of 1 M entries 12.5 -> 6 ms).

@@ -278,6 +278,23 @@ def test_csrsort_base1_custom_perm_unaligned_buffer(osa, gpu_ctx):
     run_csrsort(osa, gpu_ctx, m, n, rowptr + 1, colind + 1, base=1, perm=perm, misalign=4)
 
 
+@pytest.mark.parametrize("mean", [3, 7, 14, 40])
+@pytest.mark.parametrize("n,base", [(1000, 0), ((1 << 26) - 70, 1), ((1 << 29) + 5, 0), (2 ** 31 - 2, 1)])
+def test_csrsort_short_rows_every_group_size_and_key_width(osa, gpu_ctx, mean, n, base):
+    """Rows sorted in registers by groups of 8, 16, 32 or 64 lanes (chosen from the mean row length), the keys
+    column-and-lane packed into 32 bits where the column range leaves room and 64-bit otherwise: few and many
+    distinct columns, the largest column indices an int32 holds, both index bases, rows of every length up to the
+    group size and a few beyond it."""
+    rng = np.random.default_rng(mean * 1000 + n % 997)
+    m = 5000
+    lengths = rng.integers(0, 2 * mean + 1, m)
+    lengths[rng.choice(m, 20, replace=False)] = rng.integers(2 * mean, 2 * mean + 70, 20)
+    hi = min(n, 2 ** 31 - 1 - base)
+    rowptr, colind = _rows(lengths, lambda r, l: np.concatenate([rng.integers(0, hi, l - l // 3),
+                                                                 hi - 1 - rng.integers(0, min(hi, 50), l // 3)]))
+    run_csrsort(osa, gpu_ctx, m, n, rowptr + base, colind + base, base=base)
+
+
 def test_csrsort_many_rows(osa, gpu_ctx):
     """A million short rows (one wavefront each) with a power-law tail."""
     rng = np.random.default_rng(9)
