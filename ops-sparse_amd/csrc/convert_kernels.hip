@@ -167,13 +167,20 @@ __global__ __launch_bounds__(kBlockThreads) void CountRunsKernel(const int32_t *
     const int32_t lane = threadIdx.x % kWave;
     const int64_t wave = static_cast<int64_t>(blockIdx.x) * (kBlockThreads / kWave) + threadIdx.x / kWave;
     const int64_t first = wave * (kWave * kRounds);
+    // all loads first, unconditionally (a position past the end re-reads the last entry and is not counted): behind
+    // the branch around the atomic the compiler would wait for each load before issuing the next
+    int32_t raw[kRounds];
+#pragma unroll
+    for (int r = 0; r < kRounds; ++r) {
+        const int64_t p = first + r * kWave + lane;
+        raw[r] = LoadStream(ind + (p < nnz ? p : nnz - 1));
+    }
 #pragma unroll
     for (int r = 0; r < kRounds; ++r) {
         const int64_t p = first + r * kWave + lane;
         const bool valid = p < nnz;
         // unsigned subtraction, like the reference kernel: no signed overflow on hostile input
-        const int32_t row = valid ? static_cast<int32_t>(static_cast<uint32_t>(LoadStream(ind + p)) -
-                                                         static_cast<uint32_t>(base))
+        const int32_t row = valid ? static_cast<int32_t>(static_cast<uint32_t>(raw[r]) - static_cast<uint32_t>(base))
                                   : -1;
         const int32_t prev = __shfl_up(row, 1, kWave);
         const bool head = valid && (lane == 0 || prev != row);
@@ -190,25 +197,74 @@ __global__ __launch_bounds__(kBlockThreads) void CountRunsKernel(const int32_t *
 
 // ---------------------------------------------------------------- csr2coo
 
-// A wavefront takes 64 consecutive rows.  Rows of up to 16 entries are written
-// by their own lane; a longer row is written by the whole wavefront, 64
-// consecutive entries per store.  A row whose bounds do not describe a range
-// inside [0, nnz) is skipped (csr2coo_golden.h:51-53).
+// A wavefront takes 64 consecutive rows.  Where their bounds chain (every row ends where the next begins, as in
+// any well-formed CSR matrix) the 64 rows are one contiguous piece of the output: lane l writes positions
+// first + l, first + l + 64, ..., a whole 256-byte line per store instruction, and finds the row of a position
+// by walking the wavefront's 65 offsets, kept in LDS, forwards.  Otherwise (a row whose bounds do not describe
+// a range inside [0, nnz) is skipped, csr2coo_golden.h:51-53, and rows may overlap or leave gaps) rows of up to
+// 16 entries are written by their own lane and a longer row by the whole wavefront, 64 entries per store.
 __global__ __launch_bounds__(kBlockThreads) void ExpandRowsKernel(const int32_t *__restrict__ rowPtr, int64_t m,
                                                                  int64_t nnz, int32_t base,
                                                                  int32_t *__restrict__ rowInd)
 {
-    const int32_t lane = threadIdx.x % kWave;
+    __shared__ int32_t offs[kBlockThreads / kWave][kWave + 1];
+    const int32_t lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
     const int64_t row = (static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x);
     int64_t lo = 0, hi = 0;
+    bool bad = false;
     if (row < m) {
         lo = static_cast<int64_t>(rowPtr[row]) - base;
         hi = static_cast<int64_t>(rowPtr[row + 1]) - base;
         if (lo < 0 || hi > nnz || lo > hi) {
             lo = hi = 0;
+            bad = true;
         }
     }
     const int32_t value = static_cast<int32_t>(row) + base;
+    const int32_t live = __popcll(__ballot(row < m));  // rows of this wavefront: the first `live` lanes
+    if (live == 0) {
+        return;
+    }
+    const int64_t nextLo = __shfl_down(lo, 1, kWave);
+    const bool chained = !bad && (lane + 1 >= live || hi == nextLo);
+    if (__all(chained || lane >= live)) {
+        int32_t *mine = offs[wave];
+        if (lane < live) {
+            mine[lane] = static_cast<int32_t>(lo);
+        }
+        if (lane == live - 1) {
+            mine[live] = static_cast<int32_t>(hi);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int32_t first = mine[0], last = mine[live];
+        const int32_t row0 = static_cast<int32_t>(row) - lane + base;
+        if (static_cast<int64_t>(last - first) >= 11 * static_cast<int64_t>(live)) {
+            // rows of 11 entries and more on average: from one position of a lane to its next (64 further) at most
+            // six row ends are passed, and walking past them is cheaper than searching
+            int32_t cur = 0;
+            for (int32_t p = first + lane; p < last; p += kWave) {
+                while (mine[cur + 1] <= p) {  // ends at the latest at cur + 1 == live, whose offset is `last` > p
+                    ++cur;
+                }
+                rowInd[p] = row0 + cur;
+            }
+        } else {
+            for (int32_t p = first + lane; p < last; p += kWave) {
+                int32_t a = 0, b = live - 1;  // the last row with mine[row] <= p (mine[0] <= p < mine[live]): 64 candidates
+#pragma unroll
+                for (int step = 0; step < 6; ++step) {
+                    const int32_t mid = (a + b + 1) >> 1;
+                    const bool right = mine[mid] <= p;
+                    a = right ? mid : a;
+                    b = right ? b : mid - 1;
+                }
+                rowInd[p] = row0 + a;
+            }
+        }
+        return;
+    }
     const int64_t len = hi - lo;
     if (len <= 16) {
         for (int64_t j = 0; j < len; ++j) {
