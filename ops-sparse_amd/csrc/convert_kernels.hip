@@ -875,30 +875,38 @@ __device__ __forceinline__ KeyT GroupBitonicSort(KeyT key, int32_t g)
 // Packed: the key is (column << log2 G | lane) in 32 bits, half the moves of the 64-bit key; the launcher takes
 // it when every column index of a valid matrix fits (columns outside [0, n) then only lose their order: the
 // entries themselves travel by source lane, not inside the key).
+// The entry a lane holds of its group's row, sorted within the group: (col, pay) of lane g become those of the
+// g-th entry of the sorted row.
 template <int G, bool Packed>
-__device__ __forceinline__ void SortRowInGroup(int64_t begin, int64_t len, int32_t g, int32_t *colInd, int32_t *perm)
+__device__ __forceinline__ void SortHeldRow(bool valid, int32_t g, int32_t *col, int32_t *pay)
 {
     constexpr int kLog = G == 64 ? 6 : G == 32 ? 5 : G == 16 ? 4 : 3;
     static_assert((1 << kLog) == G, "8, 16, 32 or 64 lanes a row");
     const int32_t lane = threadIdx.x % kWave;
+    int32_t from;
+    if (Packed) {
+        uint32_t key = valid ? (static_cast<uint32_t>(*col) << kLog) | static_cast<uint32_t>(g) : ~0u;  // padding last
+        key = GroupBitonicSort<G>(key, g);
+        from = (lane - g) + static_cast<int32_t>(key & (G - 1));
+    } else {
+        uint64_t key = valid ? SortKey(*col, static_cast<uint32_t>(g)) : ~0ull;
+        key = GroupBitonicSort<G>(key, g);
+        from = (lane - g) + (static_cast<int32_t>(key & 0xffffffffu) & (G - 1));
+    }
+    *col = __shfl(*col, from, kWave);
+    *pay = __shfl(*pay, from, kWave);
+}
+
+template <int G, bool Packed>
+__device__ __forceinline__ void SortRowInGroup(int64_t begin, int64_t len, int32_t g, int32_t *colInd, int32_t *perm)
+{
     const bool valid = g < len;
     int32_t col = 0, pay = 0;
     if (valid) {
         col = colInd[begin + g];
         pay = perm[begin + g];
     }
-    int32_t from;
-    if (Packed) {
-        uint32_t key = valid ? (static_cast<uint32_t>(col) << kLog) | static_cast<uint32_t>(g) : ~0u;  // padding last
-        key = GroupBitonicSort<G>(key, g);
-        from = (lane - g) + static_cast<int32_t>(key & (G - 1));
-    } else {
-        uint64_t key = valid ? SortKey(col, static_cast<uint32_t>(g)) : ~0ull;
-        key = GroupBitonicSort<G>(key, g);
-        from = (lane - g) + (static_cast<int32_t>(key & 0xffffffffu) & (G - 1));
-    }
-    col = __shfl(col, from, kWave);
-    pay = __shfl(pay, from, kWave);
+    SortHeldRow<G, Packed>(valid, g, &col, &pay);
     if (valid) {
         colInd[begin + g] = col;
         perm[begin + g] = pay;
@@ -908,7 +916,11 @@ __device__ __forceinline__ void SortRowInGroup(int64_t begin, int64_t len, int32
 // A group of G lanes per row: rows of 2..G entries are sorted in registers (bitonic
 // network over the group's lanes); rows of up to 64 entries that do not fit the
 // group go to midList (one wavefront each, next kernel), longer rows to longList.
-// counters[0] / counters[1] are the two list lengths.
+// counters[0] / counters[1] are the two list lengths.  A group takes kSortRowsPerGroup consecutive rows and loads
+// all of them before it sorts the first: with a row a group, a wavefront's life was one round trip to memory for
+// the offsets, one for the entries and a store, and a million such wavefronts waited more than they moved.
+constexpr int kSortRowsPerGroup = 8;
+
 template <int G, bool Packed>
 __global__ __launch_bounds__(kBlockThreads) void SortShortRowsKernel(const int32_t *__restrict__ rowPtr, int64_t m,
                                                                     int64_t nnz, int32_t base, int32_t *colInd,
@@ -916,28 +928,54 @@ __global__ __launch_bounds__(kBlockThreads) void SortShortRowsKernel(const int32
                                                                     int32_t *__restrict__ midList,
                                                                     int32_t *__restrict__ longList)
 {
+    constexpr int R = kSortRowsPerGroup;
     const int32_t g = threadIdx.x % G;
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * (kBlockThreads / G) + threadIdx.x / G;
-    int64_t begin = 0, len = 0;
-    if (row < m) {
-        begin = static_cast<int64_t>(rowPtr[row]) - base;
-        len = static_cast<int64_t>(rowPtr[row + 1]) - base - begin;
-        if (len <= 1 || begin < 0 || begin + len > nnz) {
-            len = 0;  // nothing to sort, or bounds that do not describe a range of the arrays
-        }
+    const int64_t row0 = (static_cast<int64_t>(blockIdx.x) * (kBlockThreads / G) + threadIdx.x / G) * R;
+    int32_t off[R + 1];
+#pragma unroll
+    for (int r = 0; r <= R; ++r) {
+        off[r] = rowPtr[row0 + r <= m ? row0 + r : m];  // (rowPtr has m + 1 entries)
     }
-    if (len > G) {
-        if (g == 0) {
-            if (len <= kSortWaveRow) {
-                midList[atomicAdd(counters, 1)] = static_cast<int32_t>(row);
-            } else {
-                longList[atomicAdd(counters + 1, 1)] = static_cast<int32_t>(row);
+    int64_t begin[R], len[R];
+    int32_t col[R], pay[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int64_t row = row0 + r;
+        begin[r] = 0;
+        len[r] = 0;
+        if (row < m) {
+            begin[r] = static_cast<int64_t>(off[r]) - base;
+            len[r] = static_cast<int64_t>(off[r + 1]) - base - begin[r];
+            if (len[r] <= 1 || begin[r] < 0 || begin[r] + len[r] > nnz) {
+                len[r] = 0;  // nothing to sort, or bounds that do not describe a range of the arrays
             }
         }
-        len = 0;
+        if (len[r] > G) {
+            if (g == 0) {
+                if (len[r] <= kSortWaveRow) {
+                    midList[atomicAdd(counters, 1)] = static_cast<int32_t>(row);
+                } else {
+                    longList[atomicAdd(counters + 1, 1)] = static_cast<int32_t>(row);
+                }
+            }
+            len[r] = 0;
+        }
+        col[r] = 0;
+        pay[r] = 0;
+        if (g < len[r]) {
+            col[r] = colInd[begin[r] + g];
+            pay[r] = perm[begin[r] + g];
+        }
     }
     // every lane takes part in the shuffles; groups without a row sort padding
-    SortRowInGroup<G, Packed>(begin, len, g, colInd, perm);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        SortHeldRow<G, Packed>(g < len[r], g, &col[r], &pay[r]);
+        if (g < len[r]) {
+            colInd[begin[r] + g] = col[r];
+            perm[begin[r] + g] = pay[r];
+        }
+    }
 }
 
 // Wavefronts walk midList: rows of up to 64 entries, one wavefront each.
@@ -1514,7 +1552,7 @@ int opsparse_csrsort_launch(int64_t m, int64_t n, int64_t nnz, int32_t indexBase
     // Lanes per row from the mean row length: twice the mean, a power of two in [8, 64].
     const int64_t mean2 = 2 * nnz / m;
     const int g = mean2 <= 8 ? 8 : mean2 <= 16 ? 16 : mean2 <= 32 ? 32 : 64;
-    const auto shortGrid = dim3(GridFor(m, kBlockThreads / g));
+    const auto shortGrid = dim3(GridFor(m, static_cast<int64_t>(kBlockThreads / g) * kSortRowsPerGroup));
     // 32-bit keys (column and lane packed) where the columns of a valid matrix leave room for the lane number
     auto packedFor = [&](int lanes) {
         int log = 0;
