@@ -93,7 +93,8 @@ typedef struct OpsparseSpmvPlan {
     int32_t liveValues;    /* BLOCKED_GATHER: every launch first copies the caller's csrValues, as they are then, into
                               the layout (one more linear pass over the entries): nothing goes stale when values
                               change in place or the values pointer is replaced */
-    int32_t reserved;      /* zero */
+    int32_t numLongRows;   /* BLOCKED_GATHER: rows kept out of the re-stored layout: phase 1 sums them from the caller's
+                              colInd / csrValues, panel by panel, with the panel's x in LDS */
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */

@@ -41,6 +41,14 @@
 // chunk in (block, panel) order follows from the chunk sizes by a prefix sum.
 // The VALUES are copied in (block, panel) order: the analysis must be repeated
 // after they change.
+//
+// Long rows (op(A) = A only).  A row with 16 entries per panel on average (and 4096 in all) whose columns ascend
+// is kept out of all that.  Its entries in one panel are a contiguous piece of the caller's own arrays, found by
+// a search in the sorted columns, so the phase-1 workgroup of the panel, which has the panel's x in LDS anyway,
+// sums val * x over that piece straight from colInd / csrValues: 8 bytes an entry instead of 16, nothing stored
+// a second time, and the values read are the caller's as they are at the call.  The fp64 sum of every
+// (long row, panel) piece goes to a small table, and the phase-2 workgroup that owns the row adds the row's
+// pieces up, in panel order, before it writes the row.
 #include <climits>
 #include <cstdlib>
 
@@ -66,6 +74,13 @@ constexpr int64_t kMinEntryWindow = 16384;
 constexpr int64_t kMinEntryBlocks = 512;          // entry windows a matrix is cut into at least (if it has the entries)
 constexpr int64_t kMinEntries = 2000000;          // below this the ordinary kernels are as fast or faster
 constexpr int64_t kMinChunkEntries = 32;          // below this mean chunk size the layout does not pay
+constexpr int64_t kLongChunkMean = 64;            // a row is "long" with this many entries per panel on average
+constexpr int64_t kLongMinRow = 4096;             // and at least this many in all
+#ifndef VAR_LONG_LANES
+#define VAR_LONG_LANES 16
+#endif
+constexpr int kLongLanes = VAR_LONG_LANES;        // lanes that sum one (long row, panel) piece in phase 1
+constexpr int kLongTile = 3072;                   // long rows whose piece bounds a phase-1 workgroup stages in LDS at a time
 
 typedef float Float4 __attribute__((ext_vector_type(4)));
 typedef unsigned short Ushort4 __attribute__((ext_vector_type(4)));
@@ -79,6 +94,12 @@ __device__ __forceinline__ int32_t RowBlockOf(const int32_t *__restrict__ rowOff
     return b < 0 ? 0 : (b < numBlocks ? b : numBlocks - 1);  // in range whatever rowOffsets holds
 }
 
+// longBefore[r] = number of long rows among rows 0 .. r (an inclusive prefix sum of the flags).
+__device__ __forceinline__ bool IsLongRow(const int32_t *__restrict__ longBefore, int32_t row)
+{
+    return longBefore[row] != (row > 0 ? longBefore[row - 1] : 0);
+}
+
 // ------------------------------------------------------------ preprocessing
 
 // For the entries in (panel, original position) order: local column index, chunk
@@ -86,8 +107,8 @@ __device__ __forceinline__ int32_t RowBlockOf(const int32_t *__restrict__ rowOff
 __global__ __launch_bounds__(kBlockThreads) void BlockedChunkKeysKernel(
     const int32_t *__restrict__ colSorted, const int32_t *__restrict__ pos, const int32_t *__restrict__ rowOfPos,
     const int32_t *__restrict__ rowOffsets, int64_t nnz, int64_t cols, int32_t numBlocks, int32_t window,
-    uint16_t *__restrict__ colLocal, int32_t *__restrict__ chunkKey, int32_t *__restrict__ rowOfSrc,
-    int32_t *__restrict__ status)
+    const int32_t *__restrict__ longBefore, uint16_t *__restrict__ colLocal, int32_t *__restrict__ chunkKey,
+    int32_t *__restrict__ rowOfSrc, int32_t *__restrict__ status)
 {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
@@ -95,12 +116,141 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedChunkKeysKernel(
         const int32_t row = rowOfPos[pos[i]];
         rowOfSrc[i] = row;
         colLocal[i] = static_cast<uint16_t>(col & (kPanelCols - 1));
-        if (col < 0 || col >= cols) {
+        if (longBefore != nullptr && IsLongRow(longBefore, row)) {
+            chunkKey[i] = -1;  // an entry of a long row (sorted behind every panel): phase 1 takes it from the CSR arrays
+        } else if (col < 0 || col >= cols) {
             atomicOr(status, 1);
             chunkKey[i] = -1;
         } else {
             chunkKey[i] = (col >> kPanelLog) * numBlocks + RowBlockOf(rowOffsets, row, window, numBlocks);
         }
+    }
+}
+
+// flags[r] = 1 for a row of at least `minLen` entries.
+__global__ __launch_bounds__(kBlockThreads) void LongRowFlagsKernel(const int32_t *__restrict__ rowOffsets,
+                                                                    int64_t rows, int32_t minLen,
+                                                                    int32_t *__restrict__ flags)
+{
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (r < rows) {
+        flags[r] = (rowOffsets[r + 1] - rowOffsets[r] >= minLen) ? 1 : 0;
+    }
+}
+
+// Clears the flag of a row with a column outside [0, cols) or columns that do not ascend: such a row takes the
+// ordinary way (which reports the bad column).
+__global__ __launch_bounds__(kBlockThreads) void LongRowCheckKernel(const int32_t *__restrict__ rowOffsets,
+                                                                    const int32_t *__restrict__ colInd,
+                                                                    const int32_t *__restrict__ rowOfPos, int64_t nnz,
+                                                                    int64_t cols, int32_t *flags)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
+        const int32_t row = rowOfPos[i];
+        if (flags[row] == 0) {
+            continue;
+        }
+        const int32_t c = colInd[i];
+        bool bad = c < 0 || c >= cols;
+        if (i + 1 < rowOffsets[row + 1] && colInd[i + 1] < c) {
+            bad = true;
+        }
+        if (bad) {
+            flags[row] = 0;
+        }
+    }
+}
+
+// From the prefix-summed flags: the list of long rows, their number (header[1]) and entries (header[2], zero
+// before).
+__global__ __launch_bounds__(kBlockThreads) void LongRowListKernel(const int32_t *__restrict__ rowOffsets,
+                                                                   const int32_t *__restrict__ longBefore,
+                                                                   int64_t rows, int32_t maxLong,
+                                                                   int32_t *__restrict__ longRows,
+                                                                   int32_t *__restrict__ header)
+{
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (r >= rows) {
+        return;
+    }
+    const int32_t row = static_cast<int32_t>(r);
+    if (r == rows - 1) {
+        header[1] = longBefore[row] < maxLong ? longBefore[row] : maxLong;
+    }
+    if (IsLongRow(longBefore, row) && longBefore[row] <= maxLong) {
+        longRows[longBefore[row] - 1] = row;
+        atomicAdd(header + 2, rowOffsets[row + 1] - rowOffsets[row]);
+    }
+}
+
+// Row offsets with the entries of the long rows taken out, which is what the row blocks are cut by (a block is to
+// hold a share of the entries that phase 2 streams).  First out[r + 1] = entries of row r if it is long (out[0] =
+// 0), then, after an inclusive prefix sum, out[r] = rowOffsets[r] - out[r].
+__global__ __launch_bounds__(kBlockThreads) void LongRowEntriesKernel(const int32_t *__restrict__ rowOffsets,
+                                                                      const int32_t *__restrict__ longBefore,
+                                                                      int64_t rows, int32_t *__restrict__ out)
+{
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (r == 0) {
+        out[0] = 0;
+    }
+    if (r < rows) {
+        const int32_t row = static_cast<int32_t>(r);
+        out[r + 1] = IsLongRow(longBefore, row) ? rowOffsets[row + 1] - rowOffsets[row] : 0;
+    }
+}
+
+__global__ __launch_bounds__(kBlockThreads) void ShortOffsetsKernel(const int32_t *__restrict__ rowOffsets,
+                                                                    int64_t rows, int32_t *__restrict__ inOut)
+{
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (r <= rows) {
+        inOut[r] = rowOffsets[r] - inOut[r];
+    }
+}
+
+// Sort keys of the entries in CSR order: the column, or for an entry of a long row `longKey`, the first column
+// past the last panel, which sorts it behind every panel.
+__global__ __launch_bounds__(kBlockThreads) void LongRowKeysKernel(const int32_t *__restrict__ colInd,
+                                                                   const int32_t *__restrict__ rowOfPos,
+                                                                   const int32_t *__restrict__ longBefore, int64_t nnz,
+                                                                   int32_t longKey, int32_t *__restrict__ keys)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
+        keys[i] = IsLongRow(longBefore, rowOfPos[i]) ? longKey : colInd[i];
+    }
+}
+
+// longChunk[p * maxLong + l] = first entry of long row l with a column in panel p or later (p == P: the row's end).
+// Panel-major: the workgroup of a panel reads the bounds of all rows as two linear pieces.
+__global__ __launch_bounds__(kBlockThreads) void LongRowChunksKernel(const int32_t *__restrict__ rowOffsets,
+                                                                     const int32_t *__restrict__ colInd,
+                                                                     const int32_t *__restrict__ longRows,
+                                                                     const int32_t *__restrict__ header, int32_t P,
+                                                                     int32_t maxLong, int32_t *__restrict__ longChunk)
+{
+    const int64_t total = static_cast<int64_t>(header[1]) * (P + 1);
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t j = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; j < total; j += stride) {
+        const int32_t l = static_cast<int32_t>(j / (P + 1)), p = static_cast<int32_t>(j % (P + 1));
+        const int32_t row = longRows[l];
+        int32_t lo = rowOffsets[row], hi = rowOffsets[row + 1];
+        if (p == P) {
+            lo = hi;
+        } else {
+            const int32_t want = p << kPanelLog;
+            while (lo < hi) {
+                const int32_t mid = lo + ((hi - lo) >> 1);
+                if (colInd[mid] < want) {
+                    lo = mid + 1;
+                } else {
+                    hi = mid;
+                }
+            }
+        }
+        longChunk[static_cast<int64_t>(p) * maxLong + l] = lo;
     }
 }
 
@@ -343,15 +493,29 @@ __global__ __launch_bounds__(kBlkThreads) void BlockedRefreshValuesKernel(const 
 
 // xg[i] = x[panel * 2^15 + colLocal[i]] for the entries of one panel (a part of them when
 // `splits` > 1), the panel's slice of x held in LDS.
+//
+// Long rows: `header[1]` of them; long row l has the entries longChunk[l * (P + 1) + p] .. [.. + p + 1) of the
+// caller's colInd / vals in this panel.  Groups of kLongLanes lanes take the rows in turn and leave the fp64 sum
+// of val * x over the piece in longPartial[l * P + p].
 __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint16_t *__restrict__ colLocal,
                                                                      const float *__restrict__ x,
                                                                      float *__restrict__ xg,
                                                                      const int32_t *__restrict__ srcStart,
-                                                                     int64_t cols, int32_t B, int32_t splits)
+                                                                     int64_t cols, int32_t B, int32_t splits,
+                                                                     const int32_t *__restrict__ header,
+                                                                     const int32_t *__restrict__ longChunk,
+                                                                     const int32_t *__restrict__ colInd,
+                                                                     const float *__restrict__ vals, int64_t nnz,
+                                                                     int32_t P, int32_t maxLong,
+                                                                     double *__restrict__ longPartial)
 {
     __shared__ float xs[kPanelCols];
+    __shared__ int32_t pieceLo[kLongTile], pieceHi[kLongTile];
     const int tid = threadIdx.x;
-    const int64_t p = blockIdx.x / splits, part = blockIdx.x % splits;
+    // Neighbouring panels on one XCD: the pieces of a long row in panels p and p + 1 are neighbours in memory, and
+    // the cache line they share is then fetched once, by the L2 both workgroups sit behind.
+    const int64_t p = splits == 1 ? XcdContiguousTile(blockIdx.x, gridDim.x) : blockIdx.x / splits;
+    const int64_t part = splits == 1 ? 0 : blockIdx.x % splits;
     const int64_t c0 = p << kPanelLog;
     const int64_t cn = cols - c0 < kPanelCols ? cols - c0 : kPanelCols;
     const int64_t a = srcStart[p * B], e = srcStart[(p + 1) * B];
@@ -368,48 +532,135 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint1
     __syncthreads();
     const int64_t len = e - a;
     const int64_t lo = a + len * part / splits, hi = a + len * (part + 1) / splits;
-    if (lo >= hi) {
-        return;
-    }
     // Whole aligned groups of 4 entries go as 8-byte loads and 16-byte stores; what is left at
     // either end of [lo, hi) is done one by one.
     const int64_t g0 = (lo + 3) >> 2, g1 = hi >> 2;
-    if (g0 > g1) {
+    if (lo < hi && g0 > g1) {
         if (tid < 4 && lo + tid < hi) {
             xg[lo + tid] = xs[colLocal[lo + tid]];
         }
+    } else if (lo < hi) {
+        if (tid < 4) {
+            const int64_t i = lo + tid;
+            if (i < g0 * 4) {
+                xg[i] = xs[colLocal[i]];
+            }
+        } else if (tid < 8) {
+            const int64_t i = g1 * 4 + (tid - 4);
+            if (i < hi) {
+                xg[i] = xs[colLocal[i]];
+            }
+        }
+        for (int64_t g = g0; g < g1; g += kGatherBatch * kBlkThreads) {
+            Ushort4 c[kGatherBatch];
+            // Unconditional loads (clamped to the last group): the compiler keeps all of them in flight.
+#pragma unroll
+            for (int u = 0; u < kGatherBatch; ++u) {
+                int64_t gg = g + u * kBlkThreads + tid;
+                gg = gg < g1 ? gg : g1 - 1;
+                c[u] = __builtin_nontemporal_load(reinterpret_cast<const Ushort4 *>(colLocal) + gg);
+            }
+#pragma unroll
+            for (int u = 0; u < kGatherBatch; ++u) {
+                const int64_t gg = g + u * kBlkThreads + tid;
+                Float4 r;
+                r.x = xs[c[u].x];
+                r.y = xs[c[u].y];
+                r.z = xs[c[u].z];
+                r.w = xs[c[u].w];
+                if (gg < g1) {
+                    *(reinterpret_cast<Float4 *>(xg) + gg) = r;
+                }
+            }
+        }
+    }
+    // ---- long rows: this panel's piece of each, summed from the caller's arrays
+    const int32_t numLong = header != nullptr ? header[1] : 0;
+    if (numLong == 0) {
         return;
     }
-    if (tid < 4) {
-        const int64_t i = lo + tid;
-        if (i < g0 * 4) {
-            xg[i] = xs[colLocal[i]];
+    constexpr int kGroups = kBlkThreads / kLongLanes;
+    const int32_t gl = tid / kLongLanes, gt = tid % kLongLanes;
+    const int32_t base = static_cast<int32_t>(c0);
+    const int32_t *loTab = longChunk + p * maxLong, *hiTab = longChunk + (p + 1) * maxLong;
+    for (int32_t t0 = 0; t0 < numLong; t0 += kLongTile) {
+        const int32_t tn = numLong - t0 < kLongTile ? numLong - t0 : kLongTile;
+        __syncthreads();  // (the tile before is done with)
+        for (int32_t i = tid; i < tn; i += kBlkThreads) {
+            pieceLo[i] = loTab[t0 + i];
+            pieceHi[i] = hiTab[t0 + i];
         }
-    } else if (tid < 8) {
-        const int64_t i = g1 * 4 + (tid - 4);
-        if (i < hi) {
-            xg[i] = xs[colLocal[i]];
-        }
-    }
-    for (int64_t g = g0; g < g1; g += kGatherBatch * kBlkThreads) {
-        Ushort4 c[kGatherBatch];
-        // Unconditional loads (clamped to the last group): the compiler keeps all of them in flight.
+        __syncthreads();
+        // Groups of kLongLanes lanes take the rows of the tile in turn (a part of them when a panel has several
+        // workgroups), each lane 16 bytes of either array per request.  Most pieces are a request or two long, so
+        // what a group waits for is the round trip of each piece: the first request of the group's next piece is
+        // made before this piece is added up (for the last piece the same one again: no branch around the loads).
+        const int32_t stride = static_cast<int32_t>(splits) * kGroups;
+        int32_t k = static_cast<int32_t>(part) + static_cast<int32_t>(splits) * gl;
+        if (k < tn) {
+            // Group q of a piece [i0, i1) holds its entries 4 q .. 4 q + 3; the last group may be short.  A request
+            // is always four whole entries: it starts at most at i1 - 4 (never below 0), so the last group reads a
+            // few entries in front of its own, and a group past the end re-reads the last one; `add` takes only the
+            // entries that are the group's own.  No entry is ever fetched one by one.
+            auto request = [&](int32_t i0, int32_t i1, int32_t q, Int4U *c, Float4U *v) {
+                int64_t at = i0 + 4 * static_cast<int64_t>(q);
+                at = at + 4 <= i1 ? at : static_cast<int64_t>(i1) - 4;
+                at = at < 0 ? 0 : at;
+                *c = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(colInd + at));
+                *v = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(vals + at));
+            };
+            auto add = [&](int32_t i0, int32_t i1, int32_t q, const Int4U &c, const Float4U &v, double *sum) {
+                const int64_t own = i0 + 4 * static_cast<int64_t>(q);  // first entry of the group
+                int64_t at = own + 4 <= i1 ? own : static_cast<int64_t>(i1) - 4;
+                at = at < 0 ? 0 : at;
+                const uint32_t mask = kPanelCols - 1;  // an entry of the group is in the panel by construction
+                const int32_t cs[4] = {c.x, c.y, c.z, c.w};
+                const float vs[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-        for (int u = 0; u < kGatherBatch; ++u) {
-            int64_t gg = g + u * kBlkThreads + tid;
-            gg = gg < g1 ? gg : g1 - 1;
-            c[u] = __builtin_nontemporal_load(reinterpret_cast<const Ushort4 *>(colLocal) + gg);
-        }
+                for (int j = 0; j < 4; ++j) {
+                    const double t = static_cast<double>(vs[j]) *
+                                     static_cast<double>(xs[static_cast<uint32_t>(cs[j] - base) & mask]);
+                    *sum += (at + j >= own && at + j < i1) ? t : 0.0;
+                }
+            };
+            int32_t i0 = pieceLo[k], i1 = pieceHi[k];
+            Int4U cFirst;
+            Float4U vFirst;
+            request(i0, i1, gt, &cFirst, &vFirst);
+            while (true) {
+                const int32_t kn = k + stride;
+                const int32_t kk = kn < tn ? kn : k;
+                const int32_t j0 = pieceLo[kk], j1 = pieceHi[kk];
+                Int4U cAhead;
+                Float4U vAhead;
+                request(j0, j1, gt, &cAhead, &vAhead);
+                const int32_t n4 = (i1 - i0 + 3) >> 2;  // groups of the piece, the last one maybe short
+                double sum = 0.0;
+                Int4U c = cFirst;
+                Float4U v = vFirst;
+                for (int32_t q = gt; q < n4; q += kLongLanes) {
+                    Int4U cNext;
+                    Float4U vNext;
+                    request(i0, i1, q + kLongLanes, &cNext, &vNext);
+                    add(i0, i1, q, c, v, &sum);
+                    c = cNext;
+                    v = vNext;
+                }
 #pragma unroll
-        for (int u = 0; u < kGatherBatch; ++u) {
-            const int64_t gg = g + u * kBlkThreads + tid;
-            Float4 r;
-            r.x = xs[c[u].x];
-            r.y = xs[c[u].y];
-            r.z = xs[c[u].z];
-            r.w = xs[c[u].w];
-            if (gg < g1) {
-                *(reinterpret_cast<Float4 *>(xg) + gg) = r;
+                for (int off = kLongLanes / 2; off > 0; off >>= 1) {
+                    sum += __shfl_xor(sum, off, kLongLanes);
+                }
+                if (gt == 0) {
+                    longPartial[static_cast<int64_t>(t0 + k) * P + p] = sum;
+                }
+                if (kn >= tn) {
+                    break;
+                }
+                k = kn;
+                i0 = j0;
+                i1 = j1;
+                cFirst = cAhead;
+                vFirst = vAhead;
             }
         }
     }
@@ -478,7 +729,8 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
     const float *__restrict__ valD, const float *__restrict__ xg, const uint16_t *__restrict__ rowLocal,
     const int32_t *__restrict__ dstStart, const int32_t *__restrict__ srcStartT, int32_t P,
     const int32_t *__restrict__ blockOrder, const int32_t *__restrict__ blockRow, float *__restrict__ y,
-    const float *__restrict__ yIn, OpsparseScalar alphaS, OpsparseScalar betaS)
+    const float *__restrict__ yIn, OpsparseScalar alphaS, OpsparseScalar betaS, const int32_t *__restrict__ header,
+    const int32_t *__restrict__ longRows, const double *__restrict__ longPartial)
 {
     __shared__ double acc[kRowBlockRows];
     __shared__ int32_t tabD[kMaxPanels + 1];
@@ -597,6 +849,34 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
     }
     FlushPending(acc, pendingKey, pending);
     __syncthreads();
+    // Long rows of this block: phase 1 left the fp64 sum of each of their panels; a wavefront adds a row's up, lane
+    // by lane in panel order and then across the lanes, the same way at every call.
+    const int32_t numLong = header != nullptr ? header[1] : 0;
+    if (numLong > 0) {
+        int32_t lo = 0, hi = numLong;  // first long row at or behind row0
+        while (lo < hi) {
+            const int32_t mid = (lo + hi) >> 1;
+            if (longRows[mid] < row0) {
+                lo = mid + 1;
+            } else {
+                hi = mid;
+            }
+        }
+        for (int32_t l = lo + wave; l < numLong && longRows[l] < row1; l += kBlkWaves) {
+            double sum = 0.0;
+            for (int32_t p = lane; p < P; p += kWave) {
+                sum += longPartial[static_cast<int64_t>(l) * P + p];
+            }
+#pragma unroll
+            for (int off = kWave / 2; off > 0; off >>= 1) {
+                sum += __shfl_xor(sum, off);
+            }
+            if (lane == 0) {
+                acc[longRows[l] - row0] += sum;
+            }
+        }
+        __syncthreads();
+    }
     const double alpha = ReadScalar<double>(alphaS), beta = ReadScalar<double>(betaS);
     for (int i = tid; i < row1 - row0; i += kBlkThreads) {
         const int64_t row = row0 + i;
@@ -621,9 +901,13 @@ struct BlockedLayout {
     int64_t partStartOff; // live values only: first refresh window of every row block
     int64_t partDescOff;  // live values only: entry and position range of every refresh window
     int64_t refreshWindows;
+    // long rows (op(A) = A): row ids, first entry of every (long row, panel) piece, fp64 sum of every piece
+    int32_t longMinRow;   // rows of at least this many entries are candidates (0: no long-row path)
+    int32_t maxLong;      // room for this many
+    int64_t longRowsOff, longChunkOff, longPartialOff;
     int64_t resident;
     // preprocessing only
-    int64_t keys0Off, keys1Off, pos0Off, pos1Off, rowOfPosOff, outPtrOff, tableOff, scratchOff;
+    int64_t keys0Off, keys1Off, pos0Off, pos1Off, rowOfPosOff, outPtrOff, longBeforeOff, shortOffsetsOff, tableOff, scratchOff;
     int64_t bytes;
 };
 
@@ -666,6 +950,25 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
         ++bits;
     }
     l.passes = (bits + 3) / 4;
+    static const bool noLong = std::getenv("OPS_SPARSE_BLOCKED_NO_LONG_ROWS") != nullptr;
+    // (only with live values for now: with the values frozen the re-stored layout is as fast for these rows)
+    if (!transposed && !noLong && live) {
+        static const int64_t chunkMean = [] {  // tuning override: entries a long row has per panel at least, on average
+            const char *env = std::getenv("OPS_SPARSE_BLOCKED_LONG_MEAN");
+            const int64_t v = env != nullptr ? std::atoll(env) : 0;
+            return v > 0 ? v : kLongChunkMean;
+        }();
+        const int64_t minRow = chunkMean * P > kLongMinRow ? chunkMean * P : kLongMinRow;
+        if (minRow <= INT32_MAX && nnz / minRow > 0) {
+            l.longMinRow = static_cast<int32_t>(minRow);
+            l.maxLong = static_cast<int32_t>(nnz / minRow);
+            bits = 0;
+            while ((int64_t{1} << bits) < P + 1) {  // their entries sort as one more panel behind the others
+                ++bits;
+            }
+            l.passes = (bits + 3) / 4;
+        }
+    }
     if (transposed) {
         // CSR order is ascending in the input index but not in the output block: sort on the whole chunk key
         bits = 0;
@@ -691,6 +994,9 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     l.partStartOff = off; off += live ? align(4 * (B + 1)) : 0;
     l.refreshWindows = padded / kRefreshSpan + B + 1;  // upper bound; the exact count is only known on the device
     l.partDescOff = off; off += live ? align(16 * l.refreshWindows) : 0;
+    l.longRowsOff = off; off += align(4 * static_cast<int64_t>(l.maxLong));
+    l.longChunkOff = off; off += align(4 * static_cast<int64_t>(l.maxLong) * (P + 1));
+    l.longPartialOff = off; off += align(8 * static_cast<int64_t>(l.maxLong) * P);
     l.resident = off;
     l.keys0Off = off; off += align(4 * nnz);
     l.keys1Off = off; off += align(4 * nnz);
@@ -698,10 +1004,13 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     l.pos1Off = off; off += align(4 * nnz);
     l.rowOfPosOff = off; off += align(4 * nnz);
     l.outPtrOff = off; off += transposed ? align(4 * (rows + 1)) : 0;  // entries per output (column of A), prefix-summed
+    l.longBeforeOff = off; off += l.maxLong > 0 ? align(4 * rows) : 0;  // long rows among rows 0 .. r
+    l.shortOffsetsOff = off; off += l.maxLong > 0 ? align(4 * (rows + 1)) : 0;  // row offsets without their entries
     l.tableOff = off; off += align(4 * RadixTableInts(nnz));
     int64_t scan = ScanScratchInts(RadixTableInts(nnz));
     scan = ScanScratchInts(P * B + 1) > scan ? ScanScratchInts(P * B + 1) : scan;
     scan = transposed && ScanScratchInts(rows + 1) > scan ? ScanScratchInts(rows + 1) : scan;
+    scan = l.maxLong > 0 && ScanScratchInts(rows + 1) > scan ? ScanScratchInts(rows + 1) : scan;
     l.scratchOff = off; off += align(4 * scan);
     l.bytes = off;
     return l;
@@ -743,11 +1052,21 @@ int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
     }
     // Few panels: several workgroups per panel, so that every CU has one.
     const int32_t splits = l.P >= 192 ? 1 : (256 + l.P - 1) / l.P;
+    // long rows: summed from the caller's own arrays (header[1] of them, counted by the analysis)
+    const bool longRows = plan.numLongRows > 0;
+    if (longRows && (a.vals == nullptr || a.colInd == nullptr)) {
+        return OPSPARSE_E_INVALID;
+    }
+    const int32_t *header = longRows ? ints(0) : nullptr;
+    auto *longPartial = reinterpret_cast<double *>(base + l.longPartialOff);
     hipLaunchKernelGGL(SpmvBlockGatherKernel, dim3(static_cast<uint32_t>(l.P) * splits), dim3(kBlkThreads), 0, a.stream,
-                       colLocal, static_cast<const float *>(a.x), xg, ints(l.srcStartOff), a.cols, l.B, splits);
+                       colLocal, static_cast<const float *>(a.x), xg, ints(l.srcStartOff), a.cols, l.B, splits, header,
+                       ints(l.longChunkOff), a.colInd, static_cast<const float *>(a.vals), a.nnz, l.P, l.maxLong,
+                       longPartial);
     hipLaunchKernelGGL(SpmvBlockReduceKernel, dim3(static_cast<uint32_t>(l.B)), dim3(kBlkThreads), 0, a.stream, valD, xg,
                        rowLocal, ints(l.dstStartOff), ints(l.srcStartTOff), l.P, ints(l.orderOff), ints(l.blockRowOff),
-                       static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha, a.beta);
+                       static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha, a.beta, header,
+                       ints(l.longRowsOff), longPartial);
     return CheckLaunch();
 }
 
@@ -801,15 +1120,43 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     auto *rowLocal = reinterpret_cast<uint16_t *>(base + l.rowLocalOff);
     auto *valD = reinterpret_cast<float *>(base + l.valOff);
 
-    LaunchFillI32(status, 1, 0, s);
+    LaunchFillI32(status, 3, 0, s);  // status, number of long rows, their entries
     LaunchExpandRows(rowOffsets, rows, nnz, 0, rowOfPos, s);
     const int32_t *pos = nullptr, *outOffsets = rowOffsets;
     int32_t *chunkKey = nullptr, *rowOfSrc = nullptr;
+    int32_t *longBefore = nullptr;
+    if (l.maxLong > 0) {
+        // Long rows: candidates by length, checked for ascending columns inside [0, cols), numbered, listed.
+        longBefore = ints(l.longBeforeOff);
+        hipLaunchKernelGGL(LongRowFlagsKernel, dim3(GridOf(rows, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
+                           rowOffsets, rows, l.longMinRow, longBefore);
+        hipLaunchKernelGGL(LongRowCheckKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
+                           rowOffsets, colInd, rowOfPos, nnz, cols, longBefore);
+        LaunchInclusiveScanI32(longBefore, longBefore, rows, 0, scratch, s);
+        hipLaunchKernelGGL(LongRowListKernel, dim3(GridOf(rows, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
+                           rowOffsets, longBefore, rows, l.maxLong, ints(l.longRowsOff), status);
+        hipLaunchKernelGGL(LongRowChunksKernel, dim3(GridOf(static_cast<int64_t>(l.maxLong) * (l.P + 1), kBlockThreads, 4096)),
+                           dim3(kBlockThreads), 0, s, rowOffsets, colInd, ints(l.longRowsOff), status, l.P, l.maxLong,
+                           ints(l.longChunkOff));
+        int32_t *shortOffsets = ints(l.shortOffsetsOff);
+        hipLaunchKernelGGL(LongRowEntriesKernel, dim3(GridOf(rows, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
+                           rowOffsets, longBefore, rows, shortOffsets);
+        LaunchInclusiveScanI32(shortOffsets, shortOffsets, rows + 1, 0, scratch, s);
+        hipLaunchKernelGGL(ShortOffsetsKernel, dim3(GridOf(rows + 1, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
+                           rowOffsets, rows, shortOffsets);
+        outOffsets = shortOffsets;  // the row blocks are cut by the entries that stay
+    }
     if (!transposed) {
         // Entries in (panel, original position) order: stable 4-bit radix passes over the panel number.
+        const int32_t *firstKeys = colInd;
+        if (longBefore != nullptr) {
+            hipLaunchKernelGGL(LongRowKeysKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
+                               colInd, rowOfPos, longBefore, nnz, static_cast<int32_t>(l.P) << kPanelLog, keys[1]);
+            firstKeys = keys[1];
+        }
         int cur = 0;
         for (int32_t pass = 0; pass < l.passes; ++pass) {
-            const int32_t *keysIn = pass == 0 ? colInd : keys[cur];
+            const int32_t *keysIn = pass == 0 ? firstKeys : keys[cur];
             const int32_t *posIn = pass == 0 ? nullptr : poss[cur];
             const int out = pass == 0 ? 0 : 1 - cur;
             LaunchRadixPass(keysIn, posIn, keys[out], poss[out], nnz, 0, kPanelLog + 4 * pass, table, scratch, s);
@@ -819,8 +1166,8 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
         chunkKey = keys[1 - cur];
         rowOfSrc = poss[1 - cur];
         hipLaunchKernelGGL(BlockedChunkKeysKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
-                           keys[cur], pos, rowOfPos, rowOffsets, nnz, cols, l.B, l.window, colLocal, chunkKey, rowOfSrc,
-                           status);
+                           keys[cur], pos, rowOfPos, outOffsets, nnz, cols, l.B, l.window, longBefore, colLocal, chunkKey,
+                           rowOfSrc, status);
     } else {
         // The outputs are the columns of A: entries per column, then chunk keys in CSR order and a stable
         // sort on the whole key.
@@ -842,12 +1189,13 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
         hipLaunchKernelGGL(BlockedTransposedFieldsKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads),
                            0, s, colInd, rowOfPos, pos, nnz, colLocal, rowOfSrc);
     }
-    int32_t bad = 0;
-    if (hipMemcpyAsync(&bad, status, sizeof(bad), hipMemcpyDeviceToHost, s) != hipSuccess ||
+    int32_t head[3] = {0, 0, 0};  // status, long rows, their entries
+    if (hipMemcpyAsync(head, status, sizeof(head), hipMemcpyDeviceToHost, s) != hipSuccess ||
         hipStreamSynchronize(s) != hipSuccess) {
         (void)hipGetLastError();
         return OPSPARSE_E_LAUNCH;
     }
+    const int32_t bad = head[0];
     if (bad != 0) {
         return OPSPARSE_E_INVALID;  // a column index outside [0, cols)
     }
@@ -859,6 +1207,9 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     // padding positions: local row kPadRow, value 0
     LaunchFillI32(reinterpret_cast<int32_t *>(rowLocal), (l.padded + 1) / 2, static_cast<int32_t>(kPadRow * 0x10001u), s);
     LaunchFillI32(reinterpret_cast<int32_t *>(valD), l.padded, 0, s);
+    if (live) {
+        LaunchFillI32(ints(l.dstOfPosOff), nnz, -1, s);  // entries of long rows have no place in block order
+    }
     LaunchFillI32(blockRow, l.B + 1, static_cast<int32_t>(outputs), s);
     hipLaunchKernelGGL(BlockedRowBlocksKernel, dim3(GridOf(outputs, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
                        s, outOffsets, static_cast<int32_t>(outputs), l.window, l.B, blockRow);
@@ -900,6 +1251,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     p.entryWindow = l.window;
     p.transposed = transposed ? 1 : 0;
     p.liveValues = live ? 1 : 0;
+    p.numLongRows = head[1];
     p.rows = rows;
     p.nnz = nnz;
     p.bytes = l.bytes;

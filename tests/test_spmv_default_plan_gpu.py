@@ -62,6 +62,70 @@ def test_default_plan_is_the_live_blocked_layout_and_follows_the_values(osa, gpu
     assert 0 < resident < want
 
 
+def _with_long_rows(rows, cols, seed):
+    """Short scattered rows and, among them, long ones: first row, last row, two neighbours, one with repeated
+    columns (ascending all the same), one whose columns do not ascend, lengths either side of the threshold."""
+    rng = np.random.default_rng(seed)
+    lengths = rng.integers(0, 20, rows)
+    long_rows = {0: 9000, 7: 4096, 8: 4095, 1000: 40_000, 1001: 20_000, 150_000: 120_000, 200_000: 6000,
+                 rows - 1: 5000}
+    for r, l in long_rows.items():
+        lengths[r] = l
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)
+    for r in long_rows:
+        a, b = rowptr[r], rowptr[r + 1]
+        if r == 200_000:
+            continue                                         # stays unsorted: not a long row to the library
+        seg = np.sort(rng.integers(0, cols, b - a)) if r == 1001 else np.sort(rng.choice(cols, b - a, replace=False))
+        colind[a:b] = seg.astype(np.int32)                   # row 1001 keeps its repeated columns
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    return rowptr, colind, val, rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+
+
+def test_default_plan_sums_long_rows_from_the_callers_arrays(osa, gpu_ctx):
+    """Rows of 64 entries per column panel and more (4096 at least) with ascending columns are kept out of the
+    re-stored layout: the workgroup that has a panel's x in LDS sums their entries of that panel straight from
+    colInd / csrValues.  The analysis must find exactly those rows; the product must follow values changed in
+    place, a new x, beta != 0 and y read and written in place."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = 300_000, 1_400_000                          # 43 panels: the threshold is the 4096 entries
+    rowptr, colind, val, x, y0 = _with_long_rows(rows, cols, 11)
+    nnz = colind.size
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    # the analysis through the raw layer: which rows it took
+    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    plan = osa.OpsparseSpmvPlan()
+    pv = lambda t: ctypes.c_void_p(t.data_ptr())
+    assert L.opsparse_spmv_csr_blocked_analyse(pv(d[0]), pv(d[1]), pv(d[2]), rows, cols, nnz,
+                                               osa.OPSPARSE_BLOCKED_LIVE_VALUES, pv(ws), need, ctypes.byref(plan),
+                                               ctypes.c_void_p(stream.cuda_stream)) == 0
+    assert plan.liveValues == 1 and plan.numLongRows == 6    # 9000, 4096, 40 000, 20 000, 120 000, 5000
+    del ws
+    A, X = osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3])
+    d_y = to_dev(y0, dev)
+    op = osa.SpmvOp(handle, A, X, osa.DnVec(d_y))            # ALG_DEFAULT
+    assert op.buffer.numel() == need
+
+    def check(values, xv, alpha, beta):
+        d_y.copy_(torch.from_numpy(y0))
+        op(alpha, beta)
+        stream.synchronize()
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, values, xv, y0, alpha, beta)
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+    check(val, x, 1.0, 0.0)
+    check(val, x, -0.75, 2.0)
+    val2 = (val * np.float32(3.0) - np.float32(0.125)).astype(np.float32)
+    d[2].copy_(torch.from_numpy(val2))                       # in place: long and short rows alike follow
+    check(val2, x, 1.0, 0.5)
+    x2 = np.random.default_rng(12).uniform(-2, 2, cols).astype(np.float32)
+    d[3].copy_(torch.from_numpy(x2))
+    check(val2, x2, 2.0, 0.0)
+
+
 def test_default_plan_of_a_banded_matrix_stays_row_wise(osa, gpu_ctx, workloads):
     """Gathers near the diagonal: the probe says local, GetBufferSize asks for the merge-path tables only."""
     dev, stream, handle = gpu_ctx
