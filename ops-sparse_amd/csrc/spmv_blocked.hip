@@ -76,10 +76,11 @@ constexpr int64_t kMinEntries = 2000000;          // below this the ordinary ker
 constexpr int64_t kMinChunkEntries = 32;          // below this mean chunk size the layout does not pay
 constexpr int64_t kLongChunkMean = 64;            // a row is "long" with this many entries per panel on average
 constexpr int64_t kLongMinRow = 4096;             // and at least this many in all
-#ifndef VAR_LONG_LANES
-#define VAR_LONG_LANES 16
-#endif
-constexpr int kLongLanes = VAR_LONG_LANES;        // lanes that sum one (long row, panel) piece in phase 1
+// (frozen values: the long entries are stored again, a panel's in one piece, and stream whatever the rows' lengths;
+// c3 per call: 218.8 us without long rows, 200.5 with the thresholds above, 194.5 with these)
+constexpr int64_t kLongChunkMeanFrozen = 4;
+constexpr int64_t kLongMinRowFrozen = 1024;
+constexpr int kLongLanes = 16;        // lanes that sum one (long row, panel) piece in phase 1
 constexpr int kLongTile = 3072;                   // long rows whose piece bounds a phase-1 workgroup stages in LDS at a time
 
 typedef float Float4 __attribute__((ext_vector_type(4)));
@@ -210,17 +211,57 @@ __global__ __launch_bounds__(kBlockThreads) void ShortOffsetsKernel(const int32_
     }
 }
 
-// Sort keys of the entries in CSR order: the column, or for an entry of a long row `longKey`, the first column
-// past the last panel, which sorts it behind every panel.
+// Sort keys of the entries in CSR order: the column, or for an entry of a long row a column past the last panel,
+// which sorts it behind every panel: `longKey` itself (live values: the entries are then read where the caller
+// has them), or longKey + column (frozen values: behind the short entries the long ones follow panel by panel,
+// in row order inside a panel, and are stored there a second time like the short ones).
 __global__ __launch_bounds__(kBlockThreads) void LongRowKeysKernel(const int32_t *__restrict__ colInd,
                                                                    const int32_t *__restrict__ rowOfPos,
                                                                    const int32_t *__restrict__ longBefore, int64_t nnz,
-                                                                   int32_t longKey, int32_t *__restrict__ keys)
+                                                                   int32_t longKey, int32_t byPanel,
+                                                                   int32_t *__restrict__ keys)
 {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
-        keys[i] = IsLongRow(longBefore, rowOfPos[i]) ? longKey : colInd[i];
+        const int32_t col = colInd[i];
+        keys[i] = IsLongRow(longBefore, rowOfPos[i]) ? longKey + (byPanel != 0 ? col : 0) : col;
     }
+}
+
+// Frozen values.  pieceStart[p * (maxLong + 1) + l] = position, in the sorted order, of the first entry of long
+// row l in panel p; the entry after the last row of a panel ends it.  One thread a panel: the panel's part of the
+// sorted order starts where the keys reach longKey + (p << 15) (a search), the pieces follow each other in row
+// order, and their lengths are those of the rows' pieces in the CSR arrays (csrChunk, panel-major).
+__global__ __launch_bounds__(kBlockThreads) void LongRowPiecesKernel(const int32_t *__restrict__ sortedKeys, int64_t nnz,
+                                                                     const int32_t *__restrict__ csrChunk,
+                                                                     const int32_t *__restrict__ header, int32_t P,
+                                                                     int32_t maxLong, int32_t longKey,
+                                                                     int32_t *__restrict__ pieceStart)
+{
+    const int32_t p = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
+    if (p >= P) {
+        return;
+    }
+    // (the order is by the panel field of the keys only: inside a panel the entries keep their CSR order)
+    const int32_t want = (longKey >> kPanelLog) + p;
+    int64_t lo = 0, hi = nnz;
+    while (lo < hi) {
+        const int64_t mid = lo + ((hi - lo) >> 1);
+        if ((sortedKeys[mid] >> kPanelLog) < want) {
+            lo = mid + 1;
+        } else {
+            hi = mid;
+        }
+    }
+    const int32_t numLong = header[1];
+    int32_t at = static_cast<int32_t>(lo);
+    int32_t *out = pieceStart + static_cast<int64_t>(p) * (maxLong + 1);
+    const int32_t *from = csrChunk + static_cast<int64_t>(p) * maxLong, *to = from + maxLong;
+    for (int32_t l = 0; l < numLong; ++l) {
+        out[l] = at;
+        at += to[l] - from[l];
+    }
+    out[numLong] = at;
 }
 
 // longChunk[p * maxLong + l] = first entry of long row l with a column in panel p or later (p == P: the row's end).
@@ -325,17 +366,37 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedRowBlocksKernel(const in
     }
 }
 
+// longFirst[b] = number of long rows in front of row block b (b = B: of all rows): block b has the long rows
+// longFirst[b] .. longFirst[b + 1] - 1.
+__global__ __launch_bounds__(kBlockThreads) void BlockedLongFirstKernel(const int32_t *__restrict__ blockRow,
+                                                                        const int32_t *__restrict__ longBefore, int32_t B,
+                                                                        int32_t *__restrict__ longFirst)
+{
+    const int32_t b = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
+    if (b <= B) {
+        const int32_t row = blockRow[b];
+        longFirst[b] = row > 0 ? longBefore[row - 1] : 0;
+    }
+}
+
 // Values and local row indices into (block, panel) order.
 __global__ __launch_bounds__(kBlockThreads) void BlockedScatterKernel(
     const int32_t *__restrict__ pos, const int32_t *__restrict__ rowOfSrc, const int32_t *__restrict__ chunkKey,
     const float *__restrict__ vals, const int32_t *__restrict__ srcStart,
     const int32_t *__restrict__ dstStart, const int32_t *__restrict__ blockRow, int64_t nnz, int32_t P, int32_t B,
-    float *__restrict__ valD, uint16_t *__restrict__ rowLocal, int32_t *__restrict__ dstOfPos)
+    float *__restrict__ valD, uint16_t *__restrict__ rowLocal, int32_t *__restrict__ dstOfPos,
+    float *__restrict__ longVals, uint16_t *__restrict__ longRowOf, const int32_t *__restrict__ longBefore)
 {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
         const int32_t key = chunkKey[i];
         if (key < 0) {
+            if (longVals != nullptr) {
+                // an entry of a long row, frozen values: its value and the number of its row among the long rows
+                // beside its local column, all three at its place in the sorted order
+                longVals[i] = vals[pos[i]];
+                longRowOf[i] = static_cast<uint16_t>(longBefore[rowOfSrc[i]] - 1);
+            }
             continue;
         }
         const int32_t p = key / B, b = key % B;
@@ -494,9 +555,16 @@ __global__ __launch_bounds__(kBlkThreads) void BlockedRefreshValuesKernel(const 
 // xg[i] = x[panel * 2^15 + colLocal[i]] for the entries of one panel (a part of them when
 // `splits` > 1), the panel's slice of x held in LDS.
 //
-// Long rows: `header[1]` of them; long row l has the entries longChunk[l * (P + 1) + p] .. [.. + p + 1) of the
-// caller's colInd / vals in this panel.  Groups of kLongLanes lanes take the rows in turn and leave the fp64 sum
-// of val * x over the piece in longPartial[l * P + p].
+// Long rows: `header[1]` of them; longPartial[l * P + p] receives the fp64 sum of val * x over the entries of long
+// row l in panel p.  Live values: these are the entries longChunk[p * maxLong + l] .. longChunk[(p + 1) * maxLong +
+// l] of the caller's colInd / vals, and groups of kLongLanes lanes take the rows in turn.  Frozen values
+// (LongSorted): the panel's long entries follow each other, in row order, at the positions longChunk[p * (maxLong
+// + 1)] .. longChunk[p * (maxLong + 1) + header[1]] of colLocal, of xg (which there holds their values) and of
+// longRowOf (the number l of each one's row); the workgroup streams them like phase 2 streams a row block, with an
+// fp64 accumulator a row in LDS, kLongTile rows at a time ([.. + l] is where row l starts).
+constexpr int kLongBatch = 4;  // groups of 4 long entries a lane has in flight (frozen values)
+
+template <bool LongSorted>
 __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint16_t *__restrict__ colLocal,
                                                                      const float *__restrict__ x,
                                                                      float *__restrict__ xg,
@@ -507,10 +575,12 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint1
                                                                      const int32_t *__restrict__ colInd,
                                                                      const float *__restrict__ vals, int64_t nnz,
                                                                      int32_t P, int32_t maxLong,
+                                                                     const uint16_t *__restrict__ longRowOf,
                                                                      double *__restrict__ longPartial)
 {
     __shared__ float xs[kPanelCols];
-    __shared__ int32_t pieceLo[kLongTile], pieceHi[kLongTile];
+    __shared__ __align__(16) int32_t tileBuf[2 * kLongTile];  // piece bounds (live) or fp64 accumulators (frozen)
+    int32_t *pieceLo = tileBuf, *pieceHi = tileBuf + kLongTile;
     const int tid = threadIdx.x;
     // Neighbouring panels on one XCD: the pieces of a long row in panels p and p + 1 are neighbours in memory, and
     // the cache line they share is then fetched once, by the L2 both workgroups sit behind.
@@ -577,6 +647,79 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint1
     // ---- long rows: this panel's piece of each, summed from the caller's arrays
     const int32_t numLong = header != nullptr ? header[1] : 0;
     if (numLong == 0) {
+        return;
+    }
+    if constexpr (LongSorted) {
+        if (part != 0) {
+            return;  // (a partial sum has one writer: the panel's first workgroup)
+        }
+        double *accL = reinterpret_cast<double *>(tileBuf);
+        const int32_t *tab = longChunk + p * (maxLong + 1);
+        for (int32_t t0 = 0; t0 < numLong; t0 += kLongTile) {
+            const int32_t tn = numLong - t0 < kLongTile ? numLong - t0 : kLongTile;
+            const int64_t from = tab[t0], to = tab[t0 + tn];
+            __syncthreads();  // (the tile before is written out)
+            for (int32_t i = tid; i < tn; i += kBlkThreads) {
+                accL[i] = 0.0;
+            }
+            __syncthreads();
+            auto one = [&](int64_t i) {
+                atomicAdd(&accL[longRowOf[i] - t0], static_cast<double>(xg[i]) * static_cast<double>(xs[colLocal[i]]));
+            };
+            const int64_t h0 = (from + 3) >> 2, h1 = to >> 2;  // whole aligned groups of 4 entries, as above
+            if (from < to && h0 > h1) {
+                if (tid < 4 && from + tid < to) {
+                    one(from + tid);
+                }
+            } else if (from < to) {
+                if (tid < 4) {
+                    if (from + tid < h0 * 4) {
+                        one(from + tid);
+                    }
+                } else if (tid < 8) {
+                    if (h1 * 4 + (tid - 4) < to) {
+                        one(h1 * 4 + (tid - 4));
+                    }
+                }
+                for (int64_t g = h0; g < h1; g += kLongBatch * kBlkThreads) {
+                    Ushort4 c[kLongBatch], r[kLongBatch];
+                    Float4 v[kLongBatch];
+#pragma unroll
+                    for (int u = 0; u < kLongBatch; ++u) {
+                        int64_t gg = g + u * kBlkThreads + tid;
+                        gg = gg < h1 ? gg : h1 - 1;
+                        c[u] = __builtin_nontemporal_load(reinterpret_cast<const Ushort4 *>(colLocal) + gg);
+                        r[u] = __builtin_nontemporal_load(reinterpret_cast<const Ushort4 *>(longRowOf) + gg);
+                        v[u] = __builtin_nontemporal_load(reinterpret_cast<const Float4 *>(xg) + gg);
+                    }
+#pragma unroll
+                    for (int u = 0; u < kLongBatch; ++u) {
+                        if (g + u * kBlkThreads + tid >= h1) {
+                            continue;
+                        }
+                        const int32_t key[4] = {r[u].x - t0, r[u].y - t0, r[u].z - t0, r[u].w - t0};
+                        const double t[4] = {static_cast<double>(v[u].x) * static_cast<double>(xs[c[u].x]),
+                                             static_cast<double>(v[u].y) * static_cast<double>(xs[c[u].y]),
+                                             static_cast<double>(v[u].z) * static_cast<double>(xs[c[u].z]),
+                                             static_cast<double>(v[u].w) * static_cast<double>(xs[c[u].w])};
+                        double run = t[0];  // entries of one row are neighbours: one addition in LDS a run
+#pragma unroll
+                        for (int j = 1; j < 4; ++j) {
+                            if (key[j] != key[j - 1]) {
+                                atomicAdd(&accL[key[j - 1]], run);
+                                run = 0.0;
+                            }
+                            run += t[j];
+                        }
+                        atomicAdd(&accL[key[3]], run);
+                    }
+                }
+            }
+            __syncthreads();
+            for (int32_t i = tid; i < tn; i += kBlkThreads) {
+                longPartial[static_cast<int64_t>(t0 + i) * P + p] = accL[i];
+            }
+        }
         return;
     }
     constexpr int kGroups = kBlkThreads / kLongLanes;
@@ -729,7 +872,7 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
     const float *__restrict__ valD, const float *__restrict__ xg, const uint16_t *__restrict__ rowLocal,
     const int32_t *__restrict__ dstStart, const int32_t *__restrict__ srcStartT, int32_t P,
     const int32_t *__restrict__ blockOrder, const int32_t *__restrict__ blockRow, float *__restrict__ y,
-    const float *__restrict__ yIn, OpsparseScalar alphaS, OpsparseScalar betaS, const int32_t *__restrict__ header,
+    const float *__restrict__ yIn, OpsparseScalar alphaS, OpsparseScalar betaS, const int32_t *__restrict__ longFirst,
     const int32_t *__restrict__ longRows, const double *__restrict__ longPartial)
 {
     __shared__ double acc[kRowBlockRows];
@@ -851,18 +994,9 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
     __syncthreads();
     // Long rows of this block: phase 1 left the fp64 sum of each of their panels; a wavefront adds a row's up, lane
     // by lane in panel order and then across the lanes, the same way at every call.
-    const int32_t numLong = header != nullptr ? header[1] : 0;
-    if (numLong > 0) {
-        int32_t lo = 0, hi = numLong;  // first long row at or behind row0
-        while (lo < hi) {
-            const int32_t mid = (lo + hi) >> 1;
-            if (longRows[mid] < row0) {
-                lo = mid + 1;
-            } else {
-                hi = mid;
-            }
-        }
-        for (int32_t l = lo + wave; l < numLong && longRows[l] < row1; l += kBlkWaves) {
+    const int32_t l0 = longFirst != nullptr ? longFirst[blk] : 0, l1 = longFirst != nullptr ? longFirst[blk + 1] : 0;
+    if (l0 < l1) {
+        for (int32_t l = l0 + wave; l < l1; l += kBlkWaves) {
             double sum = 0.0;
             for (int32_t p = lane; p < P; p += kWave) {
                 sum += longPartial[static_cast<int64_t>(l) * P + p];
@@ -904,10 +1038,11 @@ struct BlockedLayout {
     // long rows (op(A) = A): row ids, first entry of every (long row, panel) piece, fp64 sum of every piece
     int32_t longMinRow;   // rows of at least this many entries are candidates (0: no long-row path)
     int32_t maxLong;      // room for this many
-    int64_t longRowsOff, longChunkOff, longPartialOff;
+    int64_t longRowsOff, longChunkOff, longPartialOff, longFirstOff;
     int64_t resident;
     // preprocessing only
-    int64_t keys0Off, keys1Off, pos0Off, pos1Off, rowOfPosOff, outPtrOff, longBeforeOff, shortOffsetsOff, tableOff, scratchOff;
+    int64_t keys0Off, keys1Off, pos0Off, pos1Off, rowOfPosOff, outPtrOff, longBeforeOff, shortOffsetsOff, longCsrOff, tableOff,
+        scratchOff;
     int64_t bytes;
 };
 
@@ -951,19 +1086,25 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     }
     l.passes = (bits + 3) / 4;
     static const bool noLong = std::getenv("OPS_SPARSE_BLOCKED_NO_LONG_ROWS") != nullptr;
-    // (only with live values for now: with the values frozen the re-stored layout is as fast for these rows)
-    if (!transposed && !noLong && live) {
+    if (!transposed && !noLong) {
         static const int64_t chunkMean = [] {  // tuning override: entries a long row has per panel at least, on average
             const char *env = std::getenv("OPS_SPARSE_BLOCKED_LONG_MEAN");
             const int64_t v = env != nullptr ? std::atoll(env) : 0;
-            return v > 0 ? v : kLongChunkMean;
+            return v;
         }();
-        const int64_t minRow = chunkMean * P > kLongMinRow ? chunkMean * P : kLongMinRow;
+        // live values: the pieces are read where the caller has them, scattered over the arrays, and pay from 64
+        // entries (256 bytes of either array); frozen: they are stored again panel by panel and stream
+        const int64_t mean = chunkMean > 0 ? chunkMean : (live ? kLongChunkMean : kLongChunkMeanFrozen);
+        const int64_t floor = live ? kLongMinRow : kLongMinRowFrozen;
+        int64_t minRow = mean * P > floor ? mean * P : floor;
+        if (!live && nnz / minRow > 65535) {
+            minRow = nnz / 65535 + 1;  // frozen values keep a long row's number, below nnz / minRow, in 16 bits
+        }
         if (minRow <= INT32_MAX && nnz / minRow > 0) {
             l.longMinRow = static_cast<int32_t>(minRow);
             l.maxLong = static_cast<int32_t>(nnz / minRow);
-            bits = 0;
-            while ((int64_t{1} << bits) < P + 1) {  // their entries sort as one more panel behind the others
+            bits = 0;  // their entries sort as one more panel behind the others, or (frozen values) as P more
+            while ((int64_t{1} << bits) < (live ? P + 1 : 2 * P)) {
                 ++bits;
             }
             l.passes = (bits + 3) / 4;
@@ -995,8 +1136,11 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     l.refreshWindows = padded / kRefreshSpan + B + 1;  // upper bound; the exact count is only known on the device
     l.partDescOff = off; off += live ? align(16 * l.refreshWindows) : 0;
     l.longRowsOff = off; off += align(4 * static_cast<int64_t>(l.maxLong));
-    l.longChunkOff = off; off += align(4 * static_cast<int64_t>(l.maxLong) * (P + 1));
+    // live: first entry of piece (p, l) in the CSR arrays at [p * maxLong + l], p = 0 .. P; frozen: in the sorted
+    // order at [p * (maxLong + 1) + l], l = 0 .. L
+    l.longChunkOff = off; off += align(4 * (static_cast<int64_t>(l.maxLong) + 1) * (P + 1));
     l.longPartialOff = off; off += align(8 * static_cast<int64_t>(l.maxLong) * P);
+    l.longFirstOff = off; off += l.maxLong > 0 ? align(4 * (B + 1)) : 0;
     l.resident = off;
     l.keys0Off = off; off += align(4 * nnz);
     l.keys1Off = off; off += align(4 * nnz);
@@ -1006,6 +1150,7 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     l.outPtrOff = off; off += transposed ? align(4 * (rows + 1)) : 0;  // entries per output (column of A), prefix-summed
     l.longBeforeOff = off; off += l.maxLong > 0 ? align(4 * rows) : 0;  // long rows among rows 0 .. r
     l.shortOffsetsOff = off; off += l.maxLong > 0 ? align(4 * (rows + 1)) : 0;  // row offsets without their entries
+    l.longCsrOff = off; off += l.maxLong > 0 && !live ? align(4 * static_cast<int64_t>(l.maxLong) * (P + 1)) : 0;
     l.tableOff = off; off += align(4 * RadixTableInts(nnz));
     int64_t scan = ScanScratchInts(RadixTableInts(nnz));
     scan = ScanScratchInts(P * B + 1) > scan ? ScanScratchInts(P * B + 1) : scan;
@@ -1015,6 +1160,11 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     l.bytes = off;
     return l;
 }
+
+// Frozen values: the number of its long row, for a long entry at position i of the sorted order, is kept at
+// rowLocal[i + LongRowOfShift]: the block order, which that array serves, ends in front of it (it holds the short
+// entries and at most 8 positions of padding for each of the P x B chunks).
+int64_t LongRowOfShift(const BlockedLayout &l) { return static_cast<int64_t>(kLaneEntries) * l.P * l.B; }
 
 uint32_t GridOf(int64_t items, int64_t perBlock, int64_t cap)
 {
@@ -1054,19 +1204,26 @@ int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
     const int32_t splits = l.P >= 192 ? 1 : (256 + l.P - 1) / l.P;
     // long rows: summed from the caller's own arrays (header[1] of them, counted by the analysis)
     const bool longRows = plan.numLongRows > 0;
-    if (longRows && (a.vals == nullptr || a.colInd == nullptr)) {
+    if (longRows && plan.liveValues != 0 && (a.vals == nullptr || a.colInd == nullptr)) {
         return OPSPARSE_E_INVALID;
     }
     const int32_t *header = longRows ? ints(0) : nullptr;
     auto *longPartial = reinterpret_cast<double *>(base + l.longPartialOff);
-    hipLaunchKernelGGL(SpmvBlockGatherKernel, dim3(static_cast<uint32_t>(l.P) * splits), dim3(kBlkThreads), 0, a.stream,
-                       colLocal, static_cast<const float *>(a.x), xg, ints(l.srcStartOff), a.cols, l.B, splits, header,
-                       ints(l.longChunkOff), a.colInd, static_cast<const float *>(a.vals), a.nnz, l.P, l.maxLong,
-                       longPartial);
+    if (plan.liveValues != 0 || !longRows) {
+        hipLaunchKernelGGL(SpmvBlockGatherKernel<false>, dim3(static_cast<uint32_t>(l.P) * splits), dim3(kBlkThreads), 0,
+                           a.stream, colLocal, static_cast<const float *>(a.x), xg, ints(l.srcStartOff), a.cols, l.B, splits,
+                           header, ints(l.longChunkOff), a.colInd, static_cast<const float *>(a.vals), a.nnz, l.P,
+                           l.maxLong, static_cast<const uint16_t *>(nullptr), longPartial);
+    } else {
+        hipLaunchKernelGGL(SpmvBlockGatherKernel<true>, dim3(static_cast<uint32_t>(l.P) * splits), dim3(kBlkThreads), 0,
+                           a.stream, colLocal, static_cast<const float *>(a.x), xg, ints(l.srcStartOff), a.cols, l.B, splits,
+                           header, ints(l.longChunkOff), a.colInd, static_cast<const float *>(a.vals), a.nnz, l.P,
+                           l.maxLong, rowLocal + LongRowOfShift(l), longPartial);
+    }
     hipLaunchKernelGGL(SpmvBlockReduceKernel, dim3(static_cast<uint32_t>(l.B)), dim3(kBlkThreads), 0, a.stream, valD, xg,
                        rowLocal, ints(l.dstStartOff), ints(l.srcStartTOff), l.P, ints(l.orderOff), ints(l.blockRowOff),
-                       static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha, a.beta, header,
-                       ints(l.longRowsOff), longPartial);
+                       static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha, a.beta,
+                       longRows ? ints(l.longFirstOff) : nullptr, ints(l.longRowsOff), longPartial);
     return CheckLaunch();
 }
 
@@ -1137,7 +1294,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
                            rowOffsets, longBefore, rows, l.maxLong, ints(l.longRowsOff), status);
         hipLaunchKernelGGL(LongRowChunksKernel, dim3(GridOf(static_cast<int64_t>(l.maxLong) * (l.P + 1), kBlockThreads, 4096)),
                            dim3(kBlockThreads), 0, s, rowOffsets, colInd, ints(l.longRowsOff), status, l.P, l.maxLong,
-                           ints(l.longChunkOff));
+                           ints(live ? l.longChunkOff : l.longCsrOff));
         int32_t *shortOffsets = ints(l.shortOffsetsOff);
         hipLaunchKernelGGL(LongRowEntriesKernel, dim3(GridOf(rows, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
                            rowOffsets, longBefore, rows, shortOffsets);
@@ -1151,7 +1308,8 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
         const int32_t *firstKeys = colInd;
         if (longBefore != nullptr) {
             hipLaunchKernelGGL(LongRowKeysKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
-                               colInd, rowOfPos, longBefore, nnz, static_cast<int32_t>(l.P) << kPanelLog, keys[1]);
+                               colInd, rowOfPos, longBefore, nnz, static_cast<int32_t>(l.P) << kPanelLog, live ? 0 : 1,
+                               keys[1]);
             firstKeys = keys[1];
         }
         int cur = 0;
@@ -1168,6 +1326,11 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
         hipLaunchKernelGGL(BlockedChunkKeysKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
                            keys[cur], pos, rowOfPos, outOffsets, nnz, cols, l.B, l.window, longBefore, colLocal, chunkKey,
                            rowOfSrc, status);
+        if (longBefore != nullptr && !live) {
+            hipLaunchKernelGGL(LongRowPiecesKernel, dim3(GridOf(l.P, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
+                               keys[cur], nnz, ints(l.longCsrOff), status, l.P, l.maxLong,
+                               static_cast<int32_t>(l.P) << kPanelLog, ints(l.longChunkOff));
+        }
     } else {
         // The outputs are the columns of A: entries per column, then chunk keys in CSR order and a stable
         // sort on the whole key.
@@ -1213,9 +1376,15 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     LaunchFillI32(blockRow, l.B + 1, static_cast<int32_t>(outputs), s);
     hipLaunchKernelGGL(BlockedRowBlocksKernel, dim3(GridOf(outputs, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
                        s, outOffsets, static_cast<int32_t>(outputs), l.window, l.B, blockRow);
+    if (longBefore != nullptr) {
+        hipLaunchKernelGGL(BlockedLongFirstKernel, dim3(GridOf(l.B + 1, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
+                           s, blockRow, longBefore, l.B, ints(l.longFirstOff));
+    }
     hipLaunchKernelGGL(BlockedScatterKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
                        pos, rowOfSrc, chunkKey, csrValues, srcStart, dstStart, blockRow, nnz, l.P, l.B, valD, rowLocal,
-                       live ? ints(l.dstOfPosOff) : nullptr);
+                       live ? ints(l.dstOfPosOff) : nullptr,
+                       longBefore != nullptr && !live ? reinterpret_cast<float *>(base + l.xgOff) : nullptr,
+                       rowLocal + LongRowOfShift(l), longBefore);
     if (l.B <= kRankedBlocks) {
         hipLaunchKernelGGL(BlockedOrderKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
                            dstStart, l.P, l.B, blockOrder);

@@ -165,3 +165,55 @@ def test_alg2_plan_is_dropped_when_the_values_array_is_replaced(osa, gpu_ctx):
     stream.synchronize()
     assert oracle.max_rel_err(d_y.cpu().numpy(),
                               oracle.spmv_f64(rows, cols, rowptr, colind, val2, x, y0, 2.0, 0.5)) <= 1e-5
+
+
+def test_alg2_layout_streams_long_rows_panel_by_panel(osa, gpu_ctx):
+    """ACL_SPARSE_SPMV_CSR_ALG2 (values frozen at Preprocess): rows of 1024 entries and more with ascending
+    columns leave the row-block order; a panel's workgroup streams their entries of that panel, stored a second
+    time in one piece, into one fp64 accumulator a row in LDS.  Cases: the mixed matrix of the test above (rows
+    either side of the threshold, first and last row, neighbours, repeated columns, an unsorted long row), and a
+    matrix with more long rows than the 3072 accumulators of a tile, short rows between them."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    pv = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def run(rows, cols, rowptr, colind, val, x, y0, want_long):
+        nnz = colind.size
+        d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+        need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, 0)
+        assert need > 0
+        ws = torch.empty(need, dtype=torch.uint8, device=dev)
+        plan = osa.OpsparseSpmvPlan()
+        assert L.opsparse_spmv_csr_blocked_analyse(pv(d[0]), pv(d[1]), pv(d[2]), rows, cols, nnz, 0, pv(ws), need,
+                                                   ctypes.byref(plan), ctypes.c_void_p(stream.cuda_stream)) == 0
+        assert plan.liveValues == 0 and plan.numLongRows == want_long
+        del ws
+        d_y = to_dev(y0, dev)
+        op = osa.SpmvOp(handle, osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3]), osa.DnVec(d_y),
+                        alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
+        for alpha, beta, xv in ((1.0, 0.0, x), (-0.75, 2.0, x),
+                                (2.0, 0.5, np.random.default_rng(5).uniform(-2, 2, cols).astype(np.float32))):
+            d[3].copy_(torch.from_numpy(xv))
+            d_y.copy_(torch.from_numpy(y0))
+            op(alpha, beta)
+            stream.synchronize()
+            gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, xv, y0, alpha, beta)
+            assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+    rows, cols = 300_000, 1_400_000
+    # 9000, 4096, 4095, 40 000, 20 000, 120 000, 5000 (the 6000 of row 200 000 do not ascend)
+    run(rows, cols, *_with_long_rows(rows, cols, 11), want_long=7)
+
+    rng = np.random.default_rng(21)
+    rows, cols = 120_000, 1_200_000
+    lengths = rng.integers(0, 12, rows)
+    long_at = rng.choice(rows, 3500, replace=False)
+    lengths[long_at] = rng.integers(1024, 1400, long_at.size)
+    lengths[long_at[:40]] = 1023                             # one short of the threshold
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)
+    for r in long_at:
+        colind[rowptr[r]:rowptr[r + 1]].sort()
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    run(rows, cols, rowptr, colind, val, rng.uniform(-1, 1, cols).astype(np.float32),
+        rng.uniform(-1, 1, rows).astype(np.float32), want_long=3460)
