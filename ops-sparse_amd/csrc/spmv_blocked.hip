@@ -59,11 +59,15 @@
 namespace opsparse {
 
 constexpr int kBlkThreads = 1024;                 // one workgroup per CU: it owns 128 KiB of LDS and more
-constexpr int kBlkWaves = kBlkThreads / kWave;
 constexpr int kPanelLog = 15;                     // columns per panel: 128 KiB of fp32 x
 constexpr int kPanelCols = 1 << kPanelLog;
 constexpr int kRowBlockLog = 14;                  // rows per row block: 128 KiB of fp64 accumulators
 constexpr int kRowBlockRows = 1 << kRowBlockLog;
+// Live values: the workgroup of a row block also holds the block's values, as they are at the call, in LDS
+constexpr int kLiveRowBlockLog = 12;              // 32 KiB of accumulators
+constexpr int kLiveRowBlockRows = 1 << kLiveRowBlockLog;
+constexpr int kRefreshSpan = 24576;               // block-order positions whose values it holds at a time: 96 KiB
+constexpr int64_t kLiveWindow = 20000;            // entries of a row block that is to fit that, padding included
 constexpr int kMaxPanels = 1024;                  // chunk tables of one row block in LDS: 8 KiB
 constexpr int kMaxGroups = 11776;                 // chunk of every 64th position of a row block in LDS: 23 KiB
 constexpr int kGatherBatch = 8;                   // groups of 4 entries in flight per lane, phase 1
@@ -88,10 +92,10 @@ typedef unsigned short Ushort4 __attribute__((ext_vector_type(4)));
 
 // Row block of a row: 2^14-row blocks, cut again wherever the row's first entry
 // passes a multiple of the entry window.  Monotone in the row number.
-__device__ __forceinline__ int32_t RowBlockOf(const int32_t *__restrict__ rowOffsets, int32_t row, int32_t window,
+__device__ __forceinline__ int32_t RowBlockOf(const int32_t *__restrict__ rowOffsets, int32_t row, int32_t rowLog, int32_t window,
                                               int32_t numBlocks)
 {
-    const int32_t b = (row >> kRowBlockLog) + rowOffsets[row] / window;
+    const int32_t b = (row >> rowLog) + rowOffsets[row] / window;
     return b < 0 ? 0 : (b < numBlocks ? b : numBlocks - 1);  // in range whatever rowOffsets holds
 }
 
@@ -107,7 +111,7 @@ __device__ __forceinline__ bool IsLongRow(const int32_t *__restrict__ longBefore
 // key panel * B + block, and the row.  A column outside [0, cols) sets *status.
 __global__ __launch_bounds__(kBlockThreads) void BlockedChunkKeysKernel(
     const int32_t *__restrict__ colSorted, const int32_t *__restrict__ pos, const int32_t *__restrict__ rowOfPos,
-    const int32_t *__restrict__ rowOffsets, int64_t nnz, int64_t cols, int32_t numBlocks, int32_t window,
+    const int32_t *__restrict__ rowOffsets, int64_t nnz, int64_t cols, int32_t numBlocks, int32_t rowLog, int32_t window,
     const int32_t *__restrict__ longBefore, uint16_t *__restrict__ colLocal, int32_t *__restrict__ chunkKey,
     int32_t *__restrict__ rowOfSrc, int32_t *__restrict__ status)
 {
@@ -123,7 +127,7 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedChunkKeysKernel(
             atomicOr(status, 1);
             chunkKey[i] = -1;
         } else {
-            chunkKey[i] = (col >> kPanelLog) * numBlocks + RowBlockOf(rowOffsets, row, window, numBlocks);
+            chunkKey[i] = (col >> kPanelLog) * numBlocks + RowBlockOf(rowOffsets, row, rowLog, window, numBlocks);
         }
     }
 }
@@ -299,7 +303,7 @@ __global__ __launch_bounds__(kBlockThreads) void LongRowChunksKernel(const int32
 // column outside [0, cols).  outPtr[c] = number of entries in columns below c.
 __global__ __launch_bounds__(kBlockThreads) void BlockedTransposedKeysKernel(
     const int32_t *__restrict__ colInd, const int32_t *__restrict__ rowOfPos, const int32_t *__restrict__ outPtr,
-    int64_t nnz, int64_t cols, int32_t numBlocks, int32_t window, int32_t *__restrict__ chunkKey,
+    int64_t nnz, int64_t cols, int32_t numBlocks, int32_t rowLog, int32_t window, int32_t *__restrict__ chunkKey,
     int32_t *__restrict__ status)
 {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
@@ -309,7 +313,7 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedTransposedKeysKernel(
             atomicOr(status, 1);
             chunkKey[i] = -1;
         } else {
-            chunkKey[i] = (rowOfPos[i] >> kPanelLog) * numBlocks + RowBlockOf(outPtr, col, window, numBlocks);
+            chunkKey[i] = (rowOfPos[i] >> kPanelLog) * numBlocks + RowBlockOf(outPtr, col, rowLog, window, numBlocks);
         }
     }
 }
@@ -351,16 +355,16 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedTablesKernel(const int32
 
 // blockRow[b] = first row of row block b (blockRow pre-filled with `rows`).
 __global__ __launch_bounds__(kBlockThreads) void BlockedRowBlocksKernel(const int32_t *__restrict__ rowOffsets,
-                                                                        int32_t rows, int32_t window, int32_t B,
-                                                                        int32_t *__restrict__ blockRow)
+                                                                        int32_t rows, int32_t rowLog, int32_t window,
+                                                                        int32_t B, int32_t *__restrict__ blockRow)
 {
     const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (r >= rows) {
         return;
     }
     const int32_t row = static_cast<int32_t>(r);
-    const int32_t cur = RowBlockOf(rowOffsets, row, window, B);
-    const int32_t prev = row > 0 ? RowBlockOf(rowOffsets, row - 1, window, B) : -1;
+    const int32_t cur = RowBlockOf(rowOffsets, row, rowLog, window, B);
+    const int32_t prev = row > 0 ? RowBlockOf(rowOffsets, row - 1, rowLog, window, B) : -1;
     for (int32_t b = prev + 1; b <= cur; ++b) {
         blockRow[b] = row;
     }
@@ -401,7 +405,9 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedScatterKernel(
         }
         const int32_t p = key / B, b = key % B;
         const int64_t dst = i - srcStart[key] + dstStart[static_cast<int64_t>(b) * P + p];
-        valD[dst] = vals[pos[i]];
+        if (valD != nullptr) {
+            valD[dst] = vals[pos[i]];
+        }
         if (dstOfPos != nullptr) {
             dstOfPos[pos[i]] = static_cast<int32_t>(dst);
         }
@@ -439,7 +445,6 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedOrderKeysKernel(const in
 
 // ------------------------------------------------ values of the caller, now
 
-constexpr int kRefreshSpan = 32768;  // block-order positions a workgroup re-fills at a time: 128 KiB of LDS
 
 // partStart[1 + b] = number of kRefreshSpan-position windows of row block b (prefix-summed afterwards).
 __global__ __launch_bounds__(kBlockThreads) void BlockedRefreshPartsKernel(const int32_t *__restrict__ dstStart,
@@ -474,28 +479,14 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedRefreshDescKernel(
     }
 }
 
-// The values as they are at this call, into block order.  The entries of a row block are one contiguous piece
-// of the caller's arrays and one contiguous piece of the block order; a workgroup owns a window of the latter,
-// reads the whole of the former (values and their block-order positions, both linear), keeps what falls into
-// its window in LDS and writes the window out linearly: no scattered write ever reaches memory.  A block of
-// more than kRefreshSpan positions is read once per window.
-__global__ __launch_bounds__(kBlkThreads) void BlockedRefreshValuesKernel(const float *__restrict__ vals,
-                                                                         const int32_t *__restrict__ dstOfPos,
-                                                                         const Int4U *__restrict__ partDesc,
-                                                                         float *__restrict__ valD)
+// Live values.  The entries of a row block are one contiguous piece [e0, e1) of the caller's arrays and one
+// contiguous piece of the block order.  The workgroup that owns the block reads the former (values and their
+// block-order positions, both linear) and keeps what falls into the window [w0, w0 + span) of the latter in LDS:
+// win[position - w0] = value as it is at this call.  Entries of long rows carry position -1.  A block of more than
+// kRefreshSpan positions reads its entries once per window.
+__device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, const int32_t *__restrict__ dstOfPos,
+                                               int32_t e0, int32_t e1, int32_t w0, uint32_t span, float *win, int tid)
 {
-    __shared__ float win[kRefreshSpan];
-    const int tid = threadIdx.x;
-    const Int4U desc = partDesc[blockIdx.x];
-    const int32_t e0 = desc.x, e1 = desc.y, w0 = desc.z, w1 = desc.w;
-    if (w1 <= w0) {
-        return;  // past the last window
-    }
-    for (int32_t i = tid * 4; i < w1 - w0; i += kBlkThreads * 4) {
-        *reinterpret_cast<Float4 *>(win + i) = Float4{0.0f, 0.0f, 0.0f, 0.0f};  // padding positions stay zero
-    }
-    __syncthreads();
-    const uint32_t span = static_cast<uint32_t>(w1 - w0);
     // aligned groups of four entries as 16-byte loads, the ragged ends one by one
     const int32_t g0 = (e0 + 3) & ~3, g1 = e1 & ~3;
     if (g0 >= g1) {
@@ -505,48 +496,44 @@ __global__ __launch_bounds__(kBlkThreads) void BlockedRefreshValuesKernel(const 
                 win[at] = vals[i];
             }
         }
-    } else {
-        if (tid < 8) {
-            const int32_t i = tid < 4 ? e0 + tid : g1 + (tid - 4);
-            if ((tid < 4 && i < g0) || (tid >= 4 && i < e1)) {
-                const uint32_t at = static_cast<uint32_t>(dstOfPos[i] - w0);
-                if (at < span) {
-                    win[at] = vals[i];
-                }
-            }
-        }
-        const bool vecVals = (reinterpret_cast<uintptr_t>(vals) & 15) == 0;
-        // kRefreshBatch groups in flight per lane: loads first (clamped to the last group), then the LDS writes
-        constexpr int kRefreshBatch = 4;
-        for (int32_t i0 = g0 + tid * 4; i0 < g1; i0 += kBlkThreads * 4 * kRefreshBatch) {
-            Int4U d[kRefreshBatch];
-            Float4U v[kRefreshBatch];
-#pragma unroll
-            for (int u = 0; u < kRefreshBatch; ++u) {
-                int32_t i = i0 + u * kBlkThreads * 4;
-                i = i < g1 ? i : g1 - 4;
-                d[u] = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(dstOfPos + i));
-                if (vecVals) {
-                    v[u] = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(vals + i));
-                } else {
-                    v[u] = Float4U{vals[i], vals[i + 1], vals[i + 2], vals[i + 3]};
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < kRefreshBatch; ++u) {
-                // (a clamped group writes the same values to the same places again)
-                const uint32_t a0 = static_cast<uint32_t>(d[u].x - w0), a1 = static_cast<uint32_t>(d[u].y - w0);
-                const uint32_t a2 = static_cast<uint32_t>(d[u].z - w0), a3 = static_cast<uint32_t>(d[u].w - w0);
-                if (a0 < span) win[a0] = v[u].x;
-                if (a1 < span) win[a1] = v[u].y;
-                if (a2 < span) win[a2] = v[u].z;
-                if (a3 < span) win[a3] = v[u].w;
+        return;
+    }
+    if (tid < 8) {
+        const int32_t i = tid < 4 ? e0 + tid : g1 + (tid - 4);
+        if ((tid < 4 && i < g0) || (tid >= 4 && i < e1)) {
+            const uint32_t at = static_cast<uint32_t>(dstOfPos[i] - w0);
+            if (at < span) {
+                win[at] = vals[i];
             }
         }
     }
-    __syncthreads();
-    for (int32_t i = tid * 4; i < w1 - w0; i += kBlkThreads * 4) {  // w0 and w1 - w0 are multiples of 8
-        __builtin_nontemporal_store(*reinterpret_cast<const Float4 *>(win + i), reinterpret_cast<Float4 *>(valD + w0 + i));
+    const bool vecVals = (reinterpret_cast<uintptr_t>(vals) & 15) == 0;
+    // kRefreshBatch groups in flight per lane: loads first (clamped to the last group), then the LDS writes
+    constexpr int kRefreshBatch = 4;
+    for (int32_t i0 = g0 + tid * 4; i0 < g1; i0 += kBlkThreads * 4 * kRefreshBatch) {
+        Int4U d[kRefreshBatch];
+        Float4U v[kRefreshBatch];
+#pragma unroll
+        for (int u = 0; u < kRefreshBatch; ++u) {
+            int32_t i = i0 + u * kBlkThreads * 4;
+            i = i < g1 ? i : g1 - 4;
+            d[u] = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(dstOfPos + i));
+            if (vecVals) {
+                v[u] = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(vals + i));
+            } else {
+                v[u] = Float4U{vals[i], vals[i + 1], vals[i + 2], vals[i + 3]};
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kRefreshBatch; ++u) {
+            // (a clamped group writes the same values to the same places again)
+            const uint32_t a0 = static_cast<uint32_t>(d[u].x - w0), a1 = static_cast<uint32_t>(d[u].y - w0);
+            const uint32_t a2 = static_cast<uint32_t>(d[u].z - w0), a3 = static_cast<uint32_t>(d[u].w - w0);
+            if (a0 < span) win[a0] = v[u].x;
+            if (a1 < span) win[a1] = v[u].y;
+            if (a2 < span) win[a2] = v[u].z;
+            if (a3 < span) win[a3] = v[u].w;
+        }
     }
 }
 
@@ -855,8 +842,13 @@ constexpr int kSubSpan = kWave * kSubEntries;  // positions one load instruction
 struct LanePiece {
     Float4U1 a[kSubBatches], x[kSubBatches];
     Uint2 rows[kSubBatches];
-    bool live[kSubBatches];  // false: a run past the block's end, which re-read the last run
+    bool live[kSubBatches];  // false: a run past the end, which re-read the last run
 };
+
+// (Row blocks of 2^13 or 2^12 rows, so that two or three workgroups of 512 or 1024 threads share a CU, were no
+// faster on c3 with frozen values: 193.7 .. 211 us a call against 191.4; the shorter chunks cost what the overlap
+// gains.)
+constexpr int kRedThreads = kBlkThreads, kRedWaves = kRedThreads / kWave;
 
 // One workgroup per row block: y[row] = alpha * sum(val * xg) + beta * yIn[row].
 //
@@ -864,130 +856,151 @@ struct LanePiece {
 // (padding carries the local row kPadRow and the value 0).  A lane takes runs of kSubEntries consecutive
 // positions, which therefore lie in one chunk.  tabD[p] is the first block-order position of the block's chunk
 // from panel p, tabDelta[p] the distance from there to the chunk in panel order, groupChunk[g] the chunk of
-// the block's position 64 * g.  Two batches are in flight: the next one's loads are issued, unconditionally,
-// before this one is added up.  Entries of one row are neighbours: a lane adds its runs up in registers and
-// touches the row's accumulator in LDS once per run; a row that fills whole wavefronts is summed per lane in
-// `pending` and reaches LDS once.
-__global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
+// position 64 * g of the piece being streamed.  Two batches are in flight: the next one's loads are issued,
+// unconditionally, before this one is added up.  Entries of one row are neighbours: a lane adds its runs up in
+// registers and touches the row's accumulator in LDS once per run; a row that fills whole wavefronts is summed
+// per lane in `pending` and reaches LDS once.
+//
+// Frozen values (Live == false): the block's positions are streamed in one piece, values from valD.  Live: window
+// by window of kRefreshSpan positions (partDesc[partStart[block]] ..: entries, positions); the values of a window
+// are first collected in LDS from the caller's array, and the stream takes them from there.  Padding positions of
+// a window hold whatever LDS held: their products are formed and dropped.
+template <bool Live>
+__global__ __launch_bounds__(kRedThreads) void SpmvBlockReduceKernel(
     const float *__restrict__ valD, const float *__restrict__ xg, const uint16_t *__restrict__ rowLocal,
     const int32_t *__restrict__ dstStart, const int32_t *__restrict__ srcStartT, int32_t P,
     const int32_t *__restrict__ blockOrder, const int32_t *__restrict__ blockRow, float *__restrict__ y,
     const float *__restrict__ yIn, OpsparseScalar alphaS, OpsparseScalar betaS, const int32_t *__restrict__ longFirst,
-    const int32_t *__restrict__ longRows, const double *__restrict__ longPartial)
+    const int32_t *__restrict__ longRows, const double *__restrict__ longPartial, const float *__restrict__ vals,
+    const int32_t *__restrict__ dstOfPos, const int32_t *__restrict__ partStart, const Int4U *__restrict__ partDesc)
 {
-    __shared__ double acc[kRowBlockRows];
+    constexpr int kGroupSlots = Live ? kRefreshSpan / kWave : kMaxGroups;
+    __shared__ double acc[Live ? kLiveRowBlockRows : kRowBlockRows];
     __shared__ int32_t tabD[kMaxPanels + 1];
     __shared__ int32_t tabDelta[kMaxPanels];
-    __shared__ uint16_t groupChunk[kMaxGroups];
+    __shared__ uint16_t groupChunk[kGroupSlots];
+    __shared__ __align__(16) float win[Live ? kRefreshSpan : 4];
     const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
     const int64_t blk = blockOrder[blockIdx.x];
     const int32_t row0 = blockRow[blk], row1 = blockRow[blk + 1];
     if (row0 >= row1) {
         return;  // a block number no row maps to
     }
-    for (int i = tid; i < row1 - row0; i += kBlkThreads) {
+    for (int i = tid; i < row1 - row0; i += kRedThreads) {
         acc[i] = 0.0;
     }
-    for (int i = tid; i <= P; i += kBlkThreads) {
+    for (int i = tid; i <= P; i += kRedThreads) {
         tabD[i] = dstStart[blk * P + i];
     }
-    for (int i = tid; i < P; i += kBlkThreads) {
+    for (int i = tid; i < P; i += kRedThreads) {
         tabDelta[i] = srcStartT[blk * P + i] - dstStart[blk * P + i];
     }
-    __syncthreads();
-    const int32_t d0 = tabD[0], d1 = tabD[P];  // both multiples of kLaneEntries
-    int32_t groups = (d1 - d0 + kWave - 1) / kWave;
-    groups = groups < kMaxGroups ? groups : kMaxGroups;
-    for (int32_t p = tid; p < P; p += kBlkThreads) {
-        int32_t g = (tabD[p] - d0 + kWave - 1) / kWave;
-        int32_t gEnd = (tabD[p + 1] - d0 + kWave - 1) / kWave;
-        gEnd = gEnd < groups ? gEnd : groups;
-        for (; g < gEnd; ++g) {
-            groupChunk[g] = static_cast<uint16_t>(p);
-        }
-    }
-    __syncthreads();
+    const int32_t part0 = Live ? partStart[blk] : 0, part1 = Live ? partStart[blk + 1] : 1;
     constexpr int kBatch = kWave * kLaneEntries;
-    constexpr int kStride = kBlkWaves * kBatch;
-
-    auto fetch = [&](int32_t start) {
-        LanePiece piece;
-#pragma unroll
-        for (int s = 0; s < kSubBatches; ++s) {
-            const int32_t mine = start + s * kSubSpan + lane * kSubEntries;
-            piece.live[s] = mine < d1;
-            const int32_t i0 = piece.live[s] ? mine : d1 - kSubEntries;
-            const int32_t g = (i0 - d0) / kWave;
-            int p = g < groups ? static_cast<int>(groupChunk[g]) : ChunkOf(tabD, P, i0);
-            p += (p + 1 < P && tabD[p + 1] <= i0) ? 1 : 0;
-            p += (p + 1 < P && tabD[p + 1] <= i0) ? 1 : 0;
-            if (__any(p + 1 < P && tabD[p + 1] <= i0)) {
-                p = ChunkOf(tabD, P, i0);
-            }
-            piece.a[s] = __builtin_nontemporal_load(reinterpret_cast<const Float4U1 *>(valD + i0));
-            piece.rows[s] = __builtin_nontemporal_load(reinterpret_cast<const Uint2 *>(rowLocal + i0));
-            piece.x[s] = __builtin_nontemporal_load(reinterpret_cast<const Float4U1 *>(xg + (i0 + tabDelta[p])));
-        }
-        return piece;
-    };
-
-    int32_t start = d0 + wave * kBatch;
-    LanePiece cur;
-    if (start < d1) {
-        cur = fetch(start);
-    }
+    constexpr int kStride = kRedWaves * kBatch;
     double pending = 0.0;
     int32_t pendingKey = -1;
-    if (start < d1) {
-        while (true) {
-            const LanePiece next = fetch(start + kStride);  // past the end: every lane re-reads the last run
+    for (int32_t part = part0; part < part1; ++part) {
+        __syncthreads();  // the tables are there; the window before is done with
+        // the piece [d0, d1) of the block order, both multiples of kLaneEntries
+        int32_t d0 = tabD[0], d1 = tabD[P];
+        if (Live) {
+            const Int4U desc = partDesc[part];
+            d0 = desc.z;
+            d1 = desc.w;
+            FillLiveWindow(vals, dstOfPos, desc.x, desc.y, d0, static_cast<uint32_t>(d1 - d0), win, tid);
+        }
+        int32_t groups = (d1 - d0 + kWave - 1) / kWave;
+        groups = groups < kGroupSlots ? groups : kGroupSlots;
+        for (int32_t p = tid; p < P; p += kRedThreads) {
+            int32_t g = (tabD[p] - d0 + kWave - 1) / kWave;
+            int32_t gEnd = (tabD[p + 1] - d0 + kWave - 1) / kWave;
+            g = g > 0 ? g : 0;
+            gEnd = gEnd < groups ? gEnd : groups;
+            for (; g < gEnd; ++g) {
+                groupChunk[g] = static_cast<uint16_t>(p);
+            }
+        }
+        __syncthreads();
+
+        auto fetch = [&](int32_t start) {
+            LanePiece piece;
 #pragma unroll
             for (int s = 0; s < kSubBatches; ++s) {
-                const float av[kSubEntries] = {cur.a[s].x, cur.a[s].y, cur.a[s].z, cur.a[s].w};
-                const float xv[kSubEntries] = {cur.x[s].x, cur.x[s].y, cur.x[s].z, cur.x[s].w};
-                const uint32_t rws[2] = {cur.rows[s].x, cur.rows[s].y};
-                int32_t key[kSubEntries];
-                double t[kSubEntries];
-                bool same = true;
-#pragma unroll
-                for (int j = 0; j < kSubEntries; ++j) {
-                    const uint32_t k = (j & 1) ? rws[j / 2] >> 16 : rws[j / 2] & 0xffffu;
-                    // padding and runs past the end carry key -1 and add nothing
-                    key[j] = (cur.live[s] && k < kPadRow) ? static_cast<int32_t>(k & (kRowBlockRows - 1)) : -1;
-                    t[j] = static_cast<double>(av[j]) * static_cast<double>(xv[j]);
-                    same = same && key[j] == key[0];
+                const int32_t mine = start + s * kSubSpan + lane * kSubEntries;
+                piece.live[s] = mine < d1;
+                const int32_t i0 = piece.live[s] ? mine : d1 - kSubEntries;
+                const int32_t g = (i0 - d0) / kWave;
+                int p = g < groups ? static_cast<int>(groupChunk[g]) : ChunkOf(tabD, P, i0);
+                p += (p + 1 < P && tabD[p + 1] <= i0) ? 1 : 0;
+                p += (p + 1 < P && tabD[p + 1] <= i0) ? 1 : 0;
+                if (__any(p + 1 < P && tabD[p + 1] <= i0)) {
+                    p = ChunkOf(tabD, P, i0);
                 }
-                const int32_t first = __builtin_amdgcn_readfirstlane(key[0]);
-                if (first >= 0 && __all(same && key[0] == first)) {
-                    // one row fills the wavefront's 256 positions
-                    if (first != pendingKey) {
-                        FlushPending(acc, pendingKey, pending);
-                        pendingKey = first;
-                        pending = 0.0;
-                    }
-                    pending += (t[0] + t[1]) + (t[2] + t[3]);
+                if (Live) {
+                    piece.a[s] = *reinterpret_cast<const Float4U1 *>(win + (i0 - d0));
                 } else {
-                    double run = t[0];
+                    piece.a[s] = __builtin_nontemporal_load(reinterpret_cast<const Float4U1 *>(valD + i0));
+                }
+                piece.rows[s] = __builtin_nontemporal_load(reinterpret_cast<const Uint2 *>(rowLocal + i0));
+                piece.x[s] = __builtin_nontemporal_load(reinterpret_cast<const Float4U1 *>(xg + (i0 + tabDelta[p])));
+            }
+            return piece;
+        };
+
+        int32_t start = d0 + wave * kBatch;
+        if (start < d1) {
+            LanePiece cur = fetch(start);
+            while (true) {
+                const LanePiece next = fetch(start + kStride);  // past the end: every lane re-reads the last run
 #pragma unroll
-                    for (int j = 1; j < kSubEntries; ++j) {
-                        if (key[j] != key[j - 1]) {
-                            if (key[j - 1] >= 0) {
-                                atomicAdd(&acc[key[j - 1]], run);
-                            }
-                            run = 0.0;
-                        }
-                        run += t[j];
+                for (int s = 0; s < kSubBatches; ++s) {
+                    const float av[kSubEntries] = {cur.a[s].x, cur.a[s].y, cur.a[s].z, cur.a[s].w};
+                    const float xv[kSubEntries] = {cur.x[s].x, cur.x[s].y, cur.x[s].z, cur.x[s].w};
+                    const uint32_t rws[2] = {cur.rows[s].x, cur.rows[s].y};
+                    int32_t key[kSubEntries];
+                    double t[kSubEntries];
+                    bool same = true;
+#pragma unroll
+                    for (int j = 0; j < kSubEntries; ++j) {
+                        const uint32_t k = (j & 1) ? rws[j / 2] >> 16 : rws[j / 2] & 0xffffu;
+                        // padding and runs past the end carry key -1 and add nothing
+                        key[j] = (cur.live[s] && k < kPadRow) ? static_cast<int32_t>(k & (kRowBlockRows - 1)) : -1;
+                        t[j] = static_cast<double>(av[j]) * static_cast<double>(xv[j]);
+                        same = same && key[j] == key[0];
                     }
-                    if (key[kSubEntries - 1] >= 0) {
-                        atomicAdd(&acc[key[kSubEntries - 1]], run);
+                    const int32_t first = __builtin_amdgcn_readfirstlane(key[0]);
+                    if (first >= 0 && __all(same && key[0] == first)) {
+                        // one row fills the wavefront's 256 positions
+                        if (first != pendingKey) {
+                            FlushPending(acc, pendingKey, pending);
+                            pendingKey = first;
+                            pending = 0.0;
+                        }
+                        pending += (t[0] + t[1]) + (t[2] + t[3]);
+                    } else {
+                        double run = t[0];
+#pragma unroll
+                        for (int j = 1; j < kSubEntries; ++j) {
+                            if (key[j] != key[j - 1]) {
+                                if (key[j - 1] >= 0) {
+                                    atomicAdd(&acc[key[j - 1]], run);
+                                }
+                                run = 0.0;
+                            }
+                            run += t[j];
+                        }
+                        if (key[kSubEntries - 1] >= 0) {
+                            atomicAdd(&acc[key[kSubEntries - 1]], run);
+                        }
                     }
                 }
+                start += kStride;
+                if (start >= d1) {
+                    break;
+                }
+                cur = next;
             }
-            start += kStride;
-            if (start >= d1) {
-                break;
-            }
-            cur = next;
         }
     }
     FlushPending(acc, pendingKey, pending);
@@ -996,7 +1009,7 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
     // by lane in panel order and then across the lanes, the same way at every call.
     const int32_t l0 = longFirst != nullptr ? longFirst[blk] : 0, l1 = longFirst != nullptr ? longFirst[blk + 1] : 0;
     if (l0 < l1) {
-        for (int32_t l = l0 + wave; l < l1; l += kBlkWaves) {
+        for (int32_t l = l0 + wave; l < l1; l += kRedWaves) {
             double sum = 0.0;
             for (int32_t p = lane; p < P; p += kWave) {
                 sum += longPartial[static_cast<int64_t>(l) * P + p];
@@ -1012,7 +1025,7 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockReduceKernel(
         __syncthreads();
     }
     const double alpha = ReadScalar<double>(alphaS), beta = ReadScalar<double>(betaS);
-    for (int i = tid; i < row1 - row0; i += kBlkThreads) {
+    for (int i = tid; i < row1 - row0; i += kRedThreads) {
         const int64_t row = row0 + i;
         double o = alpha * acc[i];
         if (beta != 0.0) {
@@ -1028,6 +1041,7 @@ namespace {
 
 struct BlockedLayout {
     int32_t P, B, window, passes;
+    int32_t rowLog;  // a row block has at most 2^rowLog rows
     int64_t padded;  // upper bound of the positions in block order
     // used by every launch (the first `resident` bytes)
     int64_t colLocalOff, xgOff, valOff, rowLocalOff, srcStartOff, dstStartOff, srcStartTOff, orderOff, blockRowOff;
@@ -1058,19 +1072,20 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     const int64_t P = (cols + kPanelCols - 1) >> kPanelLog;
     // Entry window: blocks of short rows get about nnz / (full row blocks) entries; a matrix of few, long rows is
     // still cut into kMinEntryBlocks pieces, or phase 2 would run on a handful of workgroups.
-    const int64_t fullBlocks = rows >> kRowBlockLog;
+    const int rowLog = live ? kLiveRowBlockLog : kRowBlockLog;
+    const int64_t fullBlocks = rows >> rowLog;
     static const int64_t minBlocks = [] {  // tuning override: entry windows a matrix is cut into at least
         const char *env = std::getenv("OPS_SPARSE_BLOCKED_WINDOWS");
         const int64_t v = env != nullptr ? std::atoll(env) : 0;
         return v;
     }();
-    // With live values a block should fit one refresh window (kRefreshSpan positions), or its entries are read
-    // once per window at every call: six times as many, shorter blocks (c3 per call: 607 us with 512 windows,
-    // 458 us with 3072; the layout alone 217 against 247 us).
-    const int64_t wantBlocks = minBlocks > 0 ? minBlocks : (live ? 6 * kMinEntryBlocks : kMinEntryBlocks);
+    // With live values a block should fit one window of kRefreshSpan positions, padding included, or its entries
+    // in the caller's arrays are read once per window at every call: blocks of about kLiveWindow entries.
+    const int64_t liveBlocks = nnz / kLiveWindow > 6 * kMinEntryBlocks ? nnz / kLiveWindow : 6 * kMinEntryBlocks;
+    const int64_t wantBlocks = minBlocks > 0 ? minBlocks : (live ? liveBlocks : kMinEntryBlocks);
     int64_t window = nnz / (fullBlocks > wantBlocks ? fullBlocks : wantBlocks);
     window = window < kMinEntryWindow ? kMinEntryWindow : window;
-    const int64_t B = ((rows + kRowBlockRows - 1) >> kRowBlockLog) + nnz / window + 1;
+    const int64_t B = ((rows + (int64_t{1} << rowLog) - 1) >> rowLog) + nnz / window + 1;
     // x must be larger than an L2 (2^20 columns) for the two passes to pay, and the chunks long enough to stream.
     // Positions are 32-bit, and phase 2 looks two batches past a block's end before it clamps.
     if (cols <= (int64_t{1} << 20) || nnz < kMinEntries || P > kMaxPanels || P * B + 1 > INT32_MAX ||
@@ -1079,6 +1094,7 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     }
     l.P = static_cast<int32_t>(P);
     l.B = static_cast<int32_t>(B);
+    l.rowLog = rowLog;
     l.window = static_cast<int32_t>(window);
     int bits = 0;
     while ((int64_t{1} << bits) < P) {
@@ -1124,7 +1140,7 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     l.padded = padded;
     l.colLocalOff = off; off += align(2 * nnz + 8);
     l.xgOff = off; off += align(4 * nnz) + 256;  // a lane's 16-byte loads of xg may run 7 entries past a chunk
-    l.valOff = off; off += align(4 * padded);
+    l.valOff = off; off += live ? 0 : align(4 * padded);  // (live values: none are kept)
     l.rowLocalOff = off; off += align(2 * padded);
     l.srcStartOff = off; off += align(4 * (P * B + 1));
     l.dstStartOff = off; off += align(4 * (P * B + 1));
@@ -1192,13 +1208,8 @@ int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
     const auto *rowLocal = reinterpret_cast<const uint16_t *>(base + l.rowLocalOff);
     auto *xg = reinterpret_cast<float *>(base + l.xgOff);
     auto *valD = reinterpret_cast<float *>(base + l.valOff);
-    if (plan.liveValues != 0) {
-        if (a.vals == nullptr) {
-            return OPSPARSE_E_INVALID;
-        }
-        hipLaunchKernelGGL(BlockedRefreshValuesKernel, dim3(static_cast<uint32_t>(l.refreshWindows)), dim3(kBlkThreads),
-                           0, a.stream, static_cast<const float *>(a.vals), ints(l.dstOfPosOff),
-                           reinterpret_cast<const Int4U *>(base + l.partDescOff), valD);
+    if (plan.liveValues != 0 && a.vals == nullptr) {
+        return OPSPARSE_E_INVALID;
     }
     // Few panels: several workgroups per panel, so that every CU has one.
     const int32_t splits = l.P >= 192 ? 1 : (256 + l.P - 1) / l.P;
@@ -1220,10 +1231,21 @@ int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
                            header, ints(l.longChunkOff), a.colInd, static_cast<const float *>(a.vals), a.nnz, l.P,
                            l.maxLong, rowLocal + LongRowOfShift(l), longPartial);
     }
-    hipLaunchKernelGGL(SpmvBlockReduceKernel, dim3(static_cast<uint32_t>(l.B)), dim3(kBlkThreads), 0, a.stream, valD, xg,
-                       rowLocal, ints(l.dstStartOff), ints(l.srcStartTOff), l.P, ints(l.orderOff), ints(l.blockRowOff),
-                       static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha, a.beta,
-                       longRows ? ints(l.longFirstOff) : nullptr, ints(l.longRowsOff), longPartial);
+    if (plan.liveValues != 0) {
+        hipLaunchKernelGGL(SpmvBlockReduceKernel<true>, dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads), 0, a.stream,
+                           static_cast<const float *>(nullptr), xg, rowLocal, ints(l.dstStartOff), ints(l.srcStartTOff), l.P,
+                           ints(l.orderOff), ints(l.blockRowOff), static_cast<float *>(a.y),
+                           static_cast<const float *>(a.yIn), a.alpha, a.beta, longRows ? ints(l.longFirstOff) : nullptr,
+                           ints(l.longRowsOff), longPartial, static_cast<const float *>(a.vals), ints(l.dstOfPosOff),
+                           ints(l.partStartOff), reinterpret_cast<const Int4U *>(base + l.partDescOff));
+    } else {
+        hipLaunchKernelGGL(SpmvBlockReduceKernel<false>, dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads), 0, a.stream,
+                           valD, xg, rowLocal, ints(l.dstStartOff), ints(l.srcStartTOff), l.P, ints(l.orderOff),
+                           ints(l.blockRowOff), static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha,
+                           a.beta, longRows ? ints(l.longFirstOff) : nullptr, ints(l.longRowsOff), longPartial,
+                           static_cast<const float *>(nullptr), static_cast<const int32_t *>(nullptr),
+                           static_cast<const int32_t *>(nullptr), static_cast<const Int4U *>(nullptr));
+    }
     return CheckLaunch();
 }
 
@@ -1324,7 +1346,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
         chunkKey = keys[1 - cur];
         rowOfSrc = poss[1 - cur];
         hipLaunchKernelGGL(BlockedChunkKeysKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
-                           keys[cur], pos, rowOfPos, outOffsets, nnz, cols, l.B, l.window, longBefore, colLocal, chunkKey,
+                           keys[cur], pos, rowOfPos, outOffsets, nnz, cols, l.B, l.rowLog, l.window, longBefore, colLocal, chunkKey,
                            rowOfSrc, status);
         if (longBefore != nullptr && !live) {
             hipLaunchKernelGGL(LongRowPiecesKernel, dim3(GridOf(l.P, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
@@ -1338,7 +1360,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
         LaunchIndicesToOffsets(colInd, nnz, cols, 0, outPtr, scratch, s);
         outOffsets = outPtr;
         hipLaunchKernelGGL(BlockedTransposedKeysKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0,
-                           s, colInd, rowOfPos, outPtr, nnz, cols, l.B, l.window, keys[1], status);
+                           s, colInd, rowOfPos, outPtr, nnz, cols, l.B, l.rowLog, l.window, keys[1], status);
         int cur = 1;
         for (int32_t pass = 0; pass < l.passes; ++pass) {
             const int out = 1 - cur;
@@ -1369,19 +1391,20 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     LaunchInclusiveScanI32(dstStart + 1, dstStart + 1, chunks, 0, scratch, s);
     // padding positions: local row kPadRow, value 0
     LaunchFillI32(reinterpret_cast<int32_t *>(rowLocal), (l.padded + 1) / 2, static_cast<int32_t>(kPadRow * 0x10001u), s);
-    LaunchFillI32(reinterpret_cast<int32_t *>(valD), l.padded, 0, s);
-    if (live) {
+    if (!live) {
+        LaunchFillI32(reinterpret_cast<int32_t *>(valD), l.padded, 0, s);
+    } else {
         LaunchFillI32(ints(l.dstOfPosOff), nnz, -1, s);  // entries of long rows have no place in block order
     }
     LaunchFillI32(blockRow, l.B + 1, static_cast<int32_t>(outputs), s);
     hipLaunchKernelGGL(BlockedRowBlocksKernel, dim3(GridOf(outputs, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
-                       s, outOffsets, static_cast<int32_t>(outputs), l.window, l.B, blockRow);
+                       s, outOffsets, static_cast<int32_t>(outputs), l.rowLog, l.window, l.B, blockRow);
     if (longBefore != nullptr) {
         hipLaunchKernelGGL(BlockedLongFirstKernel, dim3(GridOf(l.B + 1, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
                            s, blockRow, longBefore, l.B, ints(l.longFirstOff));
     }
     hipLaunchKernelGGL(BlockedScatterKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
-                       pos, rowOfSrc, chunkKey, csrValues, srcStart, dstStart, blockRow, nnz, l.P, l.B, valD, rowLocal,
+                       pos, rowOfSrc, chunkKey, csrValues, srcStart, dstStart, blockRow, nnz, l.P, l.B, live ? nullptr : valD, rowLocal,
                        live ? ints(l.dstOfPosOff) : nullptr,
                        longBefore != nullptr && !live ? reinterpret_cast<float *>(base + l.xgOff) : nullptr,
                        rowLocal + LongRowOfShift(l), longBefore);
