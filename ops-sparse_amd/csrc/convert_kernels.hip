@@ -56,15 +56,6 @@ __global__ __launch_bounds__(kBlockThreads) void FillI32Kernel(int32_t *__restri
 
 // ------------------------------------------------------------------- scan
 
-// A workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global load and store
-// the wavefront has in flight; this one leaves them outstanding (a tile's loads issued ahead of their use).
-__device__ __forceinline__ void LdsBarrier()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
 // Exclusive scan of one value per thread over the workgroup; *total gets the sum.  Its barriers order LDS only.
 __device__ __forceinline__ int32_t BlockExclusiveScan(int32_t v, int32_t *waveSums /* [4] in LDS */, int32_t *total)
 {

@@ -148,4 +148,13 @@ __device__ __forceinline__ T GroupSumDyn(T v, int g)
     return v;
 }
 
+// A workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global load and store
+// the wavefront has in flight; this one leaves them outstanding (a tile's loads issued ahead of their use).
+__device__ __forceinline__ void LdsBarrier()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 }  // namespace opsparse

@@ -446,36 +446,22 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedOrderKeysKernel(const in
 // ------------------------------------------------ values of the caller, now
 
 
-// partStart[1 + b] = number of kRefreshSpan-position windows of row block b (prefix-summed afterwards).
-__global__ __launch_bounds__(kBlockThreads) void BlockedRefreshPartsKernel(const int32_t *__restrict__ dstStart,
-                                                                           int32_t P, int32_t B,
-                                                                           int32_t *__restrict__ partStart)
+// Live values.  blockEntry[b] = first entry, in the caller's arrays, of row block b (b = B: the entry count);
+// longSpan[2 l], [2 l + 1] = first entry of long row l and of the row behind it.
+__global__ __launch_bounds__(kBlockThreads) void BlockedLiveTablesKernel(const int32_t *__restrict__ rowOffsets,
+                                                                         const int32_t *__restrict__ blockRow, int32_t B,
+                                                                         const int32_t *__restrict__ longRows,
+                                                                         const int32_t *__restrict__ header,
+                                                                         int32_t *__restrict__ blockEntry,
+                                                                         int32_t *__restrict__ longSpan)
 {
-    const int32_t b = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
-    if (b == 0) {
-        partStart[0] = 0;
+    const int32_t i = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
+    if (i <= B) {
+        blockEntry[i] = rowOffsets[blockRow[i]];
     }
-    if (b < B) {
-        const int32_t len = dstStart[static_cast<int64_t>(b + 1) * P] - dstStart[static_cast<int64_t>(b) * P];
-        partStart[1 + b] = (len + kRefreshSpan - 1) / kRefreshSpan;
-    }
-}
-
-// partDesc[w] = (first entry, end entry, first position, end position) of refresh window w; windows past the
-// last one keep the zeros the array was filled with.
-__global__ __launch_bounds__(kBlockThreads) void BlockedRefreshDescKernel(
-    const int32_t *__restrict__ dstStart, const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ blockRow,
-    const int32_t *__restrict__ partStart, int32_t P, int32_t B, Int4U *__restrict__ partDesc)
-{
-    const int32_t b = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
-    if (b >= B) {
-        return;
-    }
-    const int32_t d0 = dstStart[static_cast<int64_t>(b) * P], d1 = dstStart[static_cast<int64_t>(b + 1) * P];
-    const int32_t e0 = rowOffsets[blockRow[b]], e1 = rowOffsets[blockRow[b + 1]];
-    for (int32_t w = partStart[b]; w < partStart[b + 1]; ++w) {
-        const int32_t w0 = d0 + (w - partStart[b]) * kRefreshSpan;
-        partDesc[w] = Int4U{e0, e1, w0, w0 + kRefreshSpan < d1 ? w0 + kRefreshSpan : d1};
+    if (header != nullptr && i < header[1]) {
+        longSpan[2 * i] = rowOffsets[longRows[i]];
+        longSpan[2 * i + 1] = rowOffsets[longRows[i] + 1];
     }
 }
 
@@ -483,7 +469,8 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedRefreshDescKernel(
 // contiguous piece of the block order.  The workgroup that owns the block reads the former (values and their
 // block-order positions, both linear) and keeps what falls into the window [w0, w0 + span) of the latter in LDS:
 // win[position - w0] = value as it is at this call.  Entries of long rows carry position -1.  A block of more than
-// kRefreshSpan positions reads its entries once per window.
+// kRefreshSpan positions reads its entries once per window.  [e0, e1) here is a piece of the block's entries
+// between two long rows (whose own entries have no position and are skipped).
 __device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, const int32_t *__restrict__ dstOfPos,
                                                int32_t e0, int32_t e1, int32_t w0, uint32_t span, float *win, int tid)
 {
@@ -509,7 +496,7 @@ __device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, c
     }
     const bool vecVals = (reinterpret_cast<uintptr_t>(vals) & 15) == 0;
     // kRefreshBatch groups in flight per lane: loads first (clamped to the last group), then the LDS writes
-    constexpr int kRefreshBatch = 4;
+    constexpr int kRefreshBatch = 6;  // (a block of kLiveWindow entries in one turn)
     for (int32_t i0 = g0 + tid * 4; i0 < g1; i0 += kBlkThreads * 4 * kRefreshBatch) {
         Int4U d[kRefreshBatch];
         Float4U v[kRefreshBatch];
@@ -872,44 +859,95 @@ __global__ __launch_bounds__(kRedThreads) void SpmvBlockReduceKernel(
     const int32_t *__restrict__ blockOrder, const int32_t *__restrict__ blockRow, float *__restrict__ y,
     const float *__restrict__ yIn, OpsparseScalar alphaS, OpsparseScalar betaS, const int32_t *__restrict__ longFirst,
     const int32_t *__restrict__ longRows, const double *__restrict__ longPartial, const float *__restrict__ vals,
-    const int32_t *__restrict__ dstOfPos, const int32_t *__restrict__ partStart, const Int4U *__restrict__ partDesc)
+    const int32_t *__restrict__ dstOfPos, const int32_t *__restrict__ blockEntry, const int32_t *__restrict__ longSpan)
 {
     constexpr int kGroupSlots = Live ? kRefreshSpan / kWave : kMaxGroups;
-    __shared__ double acc[Live ? kLiveRowBlockRows : kRowBlockRows];
+    constexpr int kAccRows = Live ? kLiveRowBlockRows : kRowBlockRows;
+    __shared__ __align__(16) double acc[kAccRows];
     __shared__ int32_t tabD[kMaxPanels + 1];
     __shared__ int32_t tabDelta[kMaxPanels];
     __shared__ uint16_t groupChunk[kGroupSlots];
     __shared__ __align__(16) float win[Live ? kRefreshSpan : 4];
     const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-    const int64_t blk = blockOrder[blockIdx.x];
+    // What a workgroup waits for is a chain of round trips to memory, one workgroup a CU: everything that does not
+    // depend on an earlier load is asked for at the start.  (Live values: the blocks are alike in size by
+    // construction and are taken in row order; the frozen layout starts its heaviest blocks first.)
+    const int64_t blk = Live ? static_cast<int64_t>(blockIdx.x) : blockOrder[blockIdx.x];
     const int32_t row0 = blockRow[blk], row1 = blockRow[blk + 1];
+    const int32_t l0 = longFirst != nullptr ? longFirst[blk] : 0, l1 = longFirst != nullptr ? longFirst[blk + 1] : 0;
+    const int32_t dBeg = dstStart[blk * P], dEnd = dstStart[blk * P + P];  // the block's piece of the block order
+    const int32_t e0 = Live ? blockEntry[blk] : 0, e1 = Live ? blockEntry[blk + 1] : 0;
+    typedef double Double2 __attribute__((ext_vector_type(2)));
+    for (int i = tid * 2; i < kAccRows; i += kRedThreads * 2) {
+        *reinterpret_cast<Double2 *>(acc + i) = Double2{0.0, 0.0};
+    }
+    LdsBarrier();
     if (row0 >= row1) {
         return;  // a block number no row maps to
     }
-    for (int i = tid; i < row1 - row0; i += kRedThreads) {
-        acc[i] = 0.0;
+    // the chunk tables, into registers for now (P + 1 <= 1025 entries: one a thread, thread 0 the last as well)
+    const int32_t tabMine = tid <= P ? dstStart[blk * P + tid] : 0;
+    const int32_t tabSrc = tid < P ? srcStartT[blk * P + tid] : 0;
+    const int32_t tabLast = (tid == 0 && P >= kRedThreads) ? dstStart[blk * P + kRedThreads] : 0;
+    const int32_t spanMax = Live ? kRefreshSpan : INT32_MAX;
+    auto fillWindow = [&](int32_t w0, int32_t w1) {
+        // the block's entries without those of its long rows
+        int32_t cur = e0;
+        for (int32_t l = l0; l < l1; ++l) {
+            FillLiveWindow(vals, dstOfPos, cur, longSpan[2 * l], w0, static_cast<uint32_t>(w1 - w0), win, tid);
+            cur = longSpan[2 * l + 1];
+        }
+        FillLiveWindow(vals, dstOfPos, cur, e1, w0, static_cast<uint32_t>(w1 - w0), win, tid);
+    };
+    if (Live && dBeg < dEnd) {
+        fillWindow(dBeg, dEnd - dBeg > spanMax ? dBeg + spanMax : dEnd);
     }
-    for (int i = tid; i <= P; i += kRedThreads) {
-        tabD[i] = dstStart[blk * P + i];
+    if (tid <= P) {
+        tabD[tid] = tabMine;
     }
-    for (int i = tid; i < P; i += kRedThreads) {
-        tabDelta[i] = srcStartT[blk * P + i] - dstStart[blk * P + i];
+    if (tid < P) {
+        tabDelta[tid] = tabSrc - tabMine;
     }
-    const int32_t part0 = Live ? partStart[blk] : 0, part1 = Live ? partStart[blk + 1] : 1;
+    if (tid == 0 && P >= kRedThreads) {
+        tabD[kRedThreads] = tabLast;
+    }
+    // Long rows of this block: phase 1 left the fp64 sum of each of their panels; a wavefront adds a row's up, lane
+    // by lane in panel order and then across the lanes, the same way at every call.
+    for (int32_t l = l0 + wave; l < l1; l += kRedWaves) {
+        double sum = 0.0;
+        const double *from = longPartial + static_cast<int64_t>(l) * P;
+        for (int32_t p0 = 0; p0 < P; p0 += 4 * kWave) {
+            double v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int32_t p = p0 + u * kWave + lane;
+                v[u] = from[p < P ? p : P - 1];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                sum += p0 + u * kWave + lane < P ? v[u] : 0.0;
+            }
+        }
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) {
+            sum += __shfl_xor(sum, off);
+        }
+        if (lane == 0) {
+            atomicAdd(&acc[longRows[l] - row0], sum);
+        }
+    }
     constexpr int kBatch = kWave * kLaneEntries;
     constexpr int kStride = kRedWaves * kBatch;
     double pending = 0.0;
     int32_t pendingKey = -1;
-    for (int32_t part = part0; part < part1; ++part) {
-        __syncthreads();  // the tables are there; the window before is done with
-        // the piece [d0, d1) of the block order, both multiples of kLaneEntries
-        int32_t d0 = tabD[0], d1 = tabD[P];
-        if (Live) {
-            const Int4U desc = partDesc[part];
-            d0 = desc.z;
-            d1 = desc.w;
-            FillLiveWindow(vals, dstOfPos, desc.x, desc.y, d0, static_cast<uint32_t>(d1 - d0), win, tid);
+    // the piece [d0, d1) of the block order, both multiples of kLaneEntries: all of the block, or window by window
+    for (int32_t d0 = dBeg, d1; d0 < dEnd; d0 = d1) {
+        d1 = dEnd - d0 > spanMax ? d0 + spanMax : dEnd;
+        if (Live && d0 > dBeg) {
+            __syncthreads();  // the window before is done with
+            fillWindow(d0, d1);
         }
+        __syncthreads();
         int32_t groups = (d1 - d0 + kWave - 1) / kWave;
         groups = groups < kGroupSlots ? groups : kGroupSlots;
         for (int32_t p = tid; p < P; p += kRedThreads) {
@@ -1005,25 +1043,6 @@ __global__ __launch_bounds__(kRedThreads) void SpmvBlockReduceKernel(
     }
     FlushPending(acc, pendingKey, pending);
     __syncthreads();
-    // Long rows of this block: phase 1 left the fp64 sum of each of their panels; a wavefront adds a row's up, lane
-    // by lane in panel order and then across the lanes, the same way at every call.
-    const int32_t l0 = longFirst != nullptr ? longFirst[blk] : 0, l1 = longFirst != nullptr ? longFirst[blk + 1] : 0;
-    if (l0 < l1) {
-        for (int32_t l = l0 + wave; l < l1; l += kRedWaves) {
-            double sum = 0.0;
-            for (int32_t p = lane; p < P; p += kWave) {
-                sum += longPartial[static_cast<int64_t>(l) * P + p];
-            }
-#pragma unroll
-            for (int off = kWave / 2; off > 0; off >>= 1) {
-                sum += __shfl_xor(sum, off);
-            }
-            if (lane == 0) {
-                acc[longRows[l] - row0] += sum;
-            }
-        }
-        __syncthreads();
-    }
     const double alpha = ReadScalar<double>(alphaS), beta = ReadScalar<double>(betaS);
     for (int i = tid; i < row1 - row0; i += kRedThreads) {
         const int64_t row = row0 + i;
@@ -1046,9 +1065,8 @@ struct BlockedLayout {
     // used by every launch (the first `resident` bytes)
     int64_t colLocalOff, xgOff, valOff, rowLocalOff, srcStartOff, dstStartOff, srcStartTOff, orderOff, blockRowOff;
     int64_t dstOfPosOff;  // live values only: block-order position of every entry of the caller's arrays
-    int64_t partStartOff; // live values only: first refresh window of every row block
-    int64_t partDescOff;  // live values only: entry and position range of every refresh window
-    int64_t refreshWindows;
+    int64_t blockEntryOff;  // live values only: first entry of every row block in the caller's arrays
+    int64_t longSpanOff;    // live values only: first and end entry of every long row
     // long rows (op(A) = A): row ids, first entry of every (long row, panel) piece, fp64 sum of every piece
     int32_t longMinRow;   // rows of at least this many entries are candidates (0: no long-row path)
     int32_t maxLong;      // room for this many
@@ -1148,9 +1166,8 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     l.orderOff = off; off += align(4 * B);
     l.blockRowOff = off; off += align(4 * (B + 1));
     l.dstOfPosOff = off; off += live ? align(4 * nnz) : 0;
-    l.partStartOff = off; off += live ? align(4 * (B + 1)) : 0;
-    l.refreshWindows = padded / kRefreshSpan + B + 1;  // upper bound; the exact count is only known on the device
-    l.partDescOff = off; off += live ? align(16 * l.refreshWindows) : 0;
+    l.blockEntryOff = off; off += live ? align(4 * (B + 1)) : 0;
+    l.longSpanOff = off; off += live ? align(8 * static_cast<int64_t>(l.maxLong)) : 0;
     l.longRowsOff = off; off += align(4 * static_cast<int64_t>(l.maxLong));
     // live: first entry of piece (p, l) in the CSR arrays at [p * maxLong + l], p = 0 .. P; frozen: in the sorted
     // order at [p * (maxLong + 1) + l], l = 0 .. L
@@ -1237,14 +1254,14 @@ int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
                            ints(l.orderOff), ints(l.blockRowOff), static_cast<float *>(a.y),
                            static_cast<const float *>(a.yIn), a.alpha, a.beta, longRows ? ints(l.longFirstOff) : nullptr,
                            ints(l.longRowsOff), longPartial, static_cast<const float *>(a.vals), ints(l.dstOfPosOff),
-                           ints(l.partStartOff), reinterpret_cast<const Int4U *>(base + l.partDescOff));
+                           ints(l.blockEntryOff), ints(l.longSpanOff));
     } else {
         hipLaunchKernelGGL(SpmvBlockReduceKernel<false>, dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads), 0, a.stream,
                            valD, xg, rowLocal, ints(l.dstStartOff), ints(l.srcStartTOff), l.P, ints(l.orderOff),
                            ints(l.blockRowOff), static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha,
                            a.beta, longRows ? ints(l.longFirstOff) : nullptr, ints(l.longRowsOff), longPartial,
                            static_cast<const float *>(nullptr), static_cast<const int32_t *>(nullptr),
-                           static_cast<const int32_t *>(nullptr), static_cast<const Int4U *>(nullptr));
+                           static_cast<const int32_t *>(nullptr), static_cast<const int32_t *>(nullptr));
     }
     return CheckLaunch();
 }
@@ -1423,14 +1440,10 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
         }
     }
     if (live) {
-        int32_t *partStart = ints(l.partStartOff);
-        hipLaunchKernelGGL(BlockedRefreshPartsKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads),
-                           0, s, dstStart, l.P, l.B, partStart);
-        LaunchInclusiveScanI32(partStart + 1, partStart + 1, l.B, 0, scratch, s);
-        LaunchFillI32(ints(l.partDescOff), 4 * l.refreshWindows, 0, s);
-        hipLaunchKernelGGL(BlockedRefreshDescKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads),
-                           0, s, dstStart, rowOffsets, blockRow, partStart, l.P, l.B,
-                           reinterpret_cast<Int4U *>(base + l.partDescOff));
+        const int64_t items = l.B + 1 > l.maxLong ? l.B + 1 : l.maxLong;
+        hipLaunchKernelGGL(BlockedLiveTablesKernel, dim3(GridOf(items, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
+                           s, rowOffsets, blockRow, l.B, ints(l.longRowsOff), longBefore != nullptr ? status : nullptr,
+                           ints(l.blockEntryOff), ints(l.longSpanOff));
     }
     if (CheckLaunch() != OPSPARSE_OK) {
         return OPSPARSE_E_LAUNCH;
