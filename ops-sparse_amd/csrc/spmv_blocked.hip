@@ -233,13 +233,10 @@ __global__ __launch_bounds__(kBlockThreads) void LongRowKeysKernel(const int32_t
 }
 
 // Frozen values.  pieceStart[p * (maxLong + 1) + l] = position, in the sorted order, of the first entry of long
-// row l in panel p; the entry after the last row of a panel ends it.  One thread a panel: the panel's part of the
-// sorted order starts where the keys reach longKey + (p << 15) (a search), the pieces follow each other in row
-// order, and their lengths are those of the rows' pieces in the CSR arrays (csrChunk, panel-major).
-__global__ __launch_bounds__(kBlockThreads) void LongRowPiecesKernel(const int32_t *__restrict__ sortedKeys, int64_t nnz,
-                                                                     const int32_t *__restrict__ csrChunk,
-                                                                     const int32_t *__restrict__ header, int32_t P,
-                                                                     int32_t maxLong, int32_t longKey,
+// row l in panel p; the entry after the last row of a panel ends it.  First the panels' parts of the sorted order
+// (l = 0): a panel's starts where the keys reach longKey + (p << 15), a search by one thread a panel.
+__global__ __launch_bounds__(kBlockThreads) void LongRowPanelsKernel(const int32_t *__restrict__ sortedKeys, int64_t nnz,
+                                                                     int32_t P, int32_t maxLong, int32_t longKey,
                                                                      int32_t *__restrict__ pieceStart)
 {
     const int32_t p = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
@@ -257,15 +254,38 @@ __global__ __launch_bounds__(kBlockThreads) void LongRowPiecesKernel(const int32
             hi = mid;
         }
     }
+    pieceStart[static_cast<int64_t>(p) * (maxLong + 1)] = static_cast<int32_t>(lo);
+}
+
+// Then the rows l = 1 .. header[1] of every panel, a thread each.  Inside a panel's part the entries keep their CSR
+// order, so their positions in the caller's arrays (`pos`) ascend there, and row l starts where they reach the
+// row's first entry of this panel or a later one in the caller's arrays (csrChunk, panel-major).
+__global__ __launch_bounds__(kBlockThreads) void LongRowPiecesKernel(const int32_t *__restrict__ pos, int64_t nnz,
+                                                                     const int32_t *__restrict__ csrChunk,
+                                                                     const int32_t *__restrict__ header, int32_t P,
+                                                                     int32_t maxLong, int32_t *pieceStart)
+{
     const int32_t numLong = header[1];
-    int32_t at = static_cast<int32_t>(lo);
-    int32_t *out = pieceStart + static_cast<int64_t>(p) * (maxLong + 1);
-    const int32_t *from = csrChunk + static_cast<int64_t>(p) * maxLong, *to = from + maxLong;
-    for (int32_t l = 0; l < numLong; ++l) {
-        out[l] = at;
-        at += to[l] - from[l];
+    const int64_t total = static_cast<int64_t>(numLong) * P;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t j = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; j < total; j += stride) {
+        const int64_t p = j / numLong;
+        const int32_t l = static_cast<int32_t>(j % numLong) + 1;
+        int32_t lo = pieceStart[p * (maxLong + 1)];
+        int32_t hi = p + 1 < P ? pieceStart[(p + 1) * (maxLong + 1)] : static_cast<int32_t>(nnz);
+        if (l < numLong) {
+            const int32_t want = csrChunk[p * maxLong + l];
+            while (lo < hi) {
+                const int32_t mid = lo + ((hi - lo) >> 1);
+                if (pos[mid] < want) {
+                    lo = mid + 1;
+                } else {
+                    hi = mid;
+                }
+            }
+        }
+        pieceStart[p * (maxLong + 1) + l] = hi;
     }
-    out[numLong] = at;
 }
 
 // longChunk[p * maxLong + l] = first entry of long row l with a column in panel p or later (p == P: the row's end).
@@ -1366,9 +1386,13 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
                            keys[cur], pos, rowOfPos, outOffsets, nnz, cols, l.B, l.rowLog, l.window, longBefore, colLocal, chunkKey,
                            rowOfSrc, status);
         if (longBefore != nullptr && !live) {
-            hipLaunchKernelGGL(LongRowPiecesKernel, dim3(GridOf(l.P, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
-                               keys[cur], nnz, ints(l.longCsrOff), status, l.P, l.maxLong,
-                               static_cast<int32_t>(l.P) << kPanelLog, ints(l.longChunkOff));
+            hipLaunchKernelGGL(LongRowPanelsKernel, dim3(GridOf(l.P, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
+                               keys[cur], nnz, l.P, l.maxLong, static_cast<int32_t>(l.P) << kPanelLog,
+                               ints(l.longChunkOff));
+            hipLaunchKernelGGL(LongRowPiecesKernel,
+                               dim3(GridOf(static_cast<int64_t>(l.maxLong) * l.P, kBlockThreads, 8192)),
+                               dim3(kBlockThreads), 0, s, pos, nnz, ints(l.longCsrOff), status, l.P, l.maxLong,
+                               ints(l.longChunkOff));
         }
     } else {
         // The outputs are the columns of A: entries per column, then chunk keys in CSR order and a stable
@@ -1425,7 +1449,9 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
                        live ? ints(l.dstOfPosOff) : nullptr,
                        longBefore != nullptr && !live ? reinterpret_cast<float *>(base + l.xgOff) : nullptr,
                        rowLocal + LongRowOfShift(l), longBefore);
-    if (l.B <= kRankedBlocks) {
+    if (live) {
+        // (the blocks are alike in size by construction and are taken in row order)
+    } else if (l.B <= kRankedBlocks) {
         hipLaunchKernelGGL(BlockedOrderKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
                            dstStart, l.P, l.B, blockOrder);
     } else {
