@@ -163,12 +163,15 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
  * analysis it re-stores indices AND values in the workspace; launches with the
  * resulting plan ignore the rowOffsets / colInd / csrValues arguments.  Returns
  * OPSPARSE_E_INVALID for a column index outside [0, cols).  Synchronises `stream` once.
+ * Rows with many entries in every column panel and ascending columns ("long rows", plan->numLongRows of them)
+ * are summed by the first kernel instead of going through the row-block order.
  * Launches touch only the first opsparse_spmv_csr_blocked_resident_bytes() of the workspace; the rest serves the
  * analysis and may be handed back afterwards (a launch accepts a workspace of at least the resident size).
  * `flags`: OPSPARSE_BLOCKED_TRANSPOSE (= 1, so that a plain 0 / 1 "transpose" still reads right) and / or
- * OPSPARSE_BLOCKED_LIVE_VALUES: the layout also keeps the block-order position of every entry (4 more bytes per
- * entry, resident) and every launch re-reads csrValues through it, 12 more bytes of traffic per entry, all
- * streamed; such a plan never goes stale when values change.
+ * OPSPARSE_BLOCKED_LIVE_VALUES: the layout keeps the block-order position of every entry instead of the values
+ * and every launch takes the values from the csrValues argument (8 more bytes of traffic per entry, all
+ * streamed), and for the long rows the column indices from colInd as well: such a plan never goes stale when
+ * values change; rowOffsets / colInd must be the arrays of the analysis.
  */
 #define OPSPARSE_BLOCKED_TRANSPOSE 1
 #define OPSPARSE_BLOCKED_LIVE_VALUES 2

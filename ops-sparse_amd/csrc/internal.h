@@ -132,7 +132,7 @@ OpsparseScalar MakeScalar(const void *p, aclDataType computeType, aclsparsePoint
 struct RestoredChoice {
     int32_t kernel;
     size_t bytes;
-    bool liveValues;  // BLOCKED_GATHER only: the layout re-reads the caller's values at every call
+    bool liveValues;  // BLOCKED_GATHER only: the layout holds no values, every call takes the caller's
 };
 RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose);
 int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const float *values, int64_t rows,

@@ -40,15 +40,21 @@
 // a panel, so it yields the (panel, block) order directly; the position of a
 // chunk in (block, panel) order follows from the chunk sizes by a prefix sum.
 // The VALUES are copied in (block, panel) order: the analysis must be repeated
-// after they change.
+// after they change.  With "live values" none are copied: the phase-2 workgroup
+// of a row block reads the block's entries of the caller's array, linearly,
+// together with their positions in (block, panel) order, collects them in a
+// window of LDS and streams against that window.
 //
-// Long rows (op(A) = A only).  A row with 16 entries per panel on average (and 4096 in all) whose columns ascend
-// is kept out of all that.  Its entries in one panel are a contiguous piece of the caller's own arrays, found by
-// a search in the sorted columns, so the phase-1 workgroup of the panel, which has the panel's x in LDS anyway,
-// sums val * x over that piece straight from colInd / csrValues: 8 bytes an entry instead of 16, nothing stored
-// a second time, and the values read are the caller's as they are at the call.  The fp64 sum of every
-// (long row, panel) piece goes to a small table, and the phase-2 workgroup that owns the row adds the row's
-// pieces up, in panel order, before it writes the row.
+// Long rows (op(A) = A only).  A row with many entries in every panel, whose columns ascend, is kept out of the
+// (block, panel) order: the phase-1 workgroup of a panel, which has the panel's x in LDS anyway, sums val * x over
+// the row's entries of that panel and leaves the fp64 sum in a small table; the phase-2 workgroup that owns the
+// row adds the row's sums up, in panel order, before it writes the row.  8 bytes an entry instead of 16.  With
+// frozen values (rows of 1024 entries and 4 per panel or more) the long entries are stored a second time, a
+// panel's in one piece in row order as (local column, value, number of the row), and stream into one fp64
+// accumulator a long row in LDS.  With live values (4096 entries and 64 per panel) a row's entries of a panel
+// are a contiguous piece of the caller's own arrays, found by a search in the sorted columns, and lane groups
+// take the pieces in turn: nothing is stored a second time, and the values read are the caller's as they are at
+// the call.
 #include <climits>
 #include <cstdlib>
 
