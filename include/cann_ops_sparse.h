@@ -426,6 +426,30 @@ aclsparseStatus_t aclsparseXcsrsort_bufferSizeExt(aclsparseHandle_t handle, int 
 aclsparseStatus_t aclsparseXcsrsort(aclsparseHandle_t handle, int m, int n, int nnz, const aclsparseMatDescr_t descrA,
                                     const int *csrRowPtr, int *csrColInd, int *P, void *pBuffer);
 
+/* [ref: :1825-1864; host sparse/cscsort/arch35/cscsort_host.cpp:52-216; order test/cscsort/arch35/cscsort_golden.h:30-70]
+ * The column-wise twin of aclsparseXcsrsort: stable ascending sort of the row indices inside every column, in
+ * place; P is permuted the same way; cscColPtr is not modified.  The index base comes from descrA.  pBuffer must
+ * be 128-byte aligned (INVALID_VALUE otherwise, as in the reference). */
+aclsparseStatus_t aclsparseXcscsort_bufferSizeExt(aclsparseHandle_t handle, int m, int n, int nnz,
+                                                  const int *cscColPtr, const int *cscRowInd,
+                                                  size_t *pBufferSizeInBytes);
+aclsparseStatus_t aclsparseXcscsort(aclsparseHandle_t handle, int m, int n, int nnz, const aclsparseMatDescr_t descrA,
+                                    const int *cscColPtr, int *cscRowInd, int *P, void *pBuffer);
+
+/* [ref: :1516-1563; host sparse/coosort/arch35/coosort_host.cpp:48-78, :262-371; order
+ * test/coosort/arch35/coosort_golden.h:52-85]
+ * Stable sort of the COO triples (row, column, P) in place.  ByRow: ascending in the row and, among equal rows,
+ * in the column; ByColumn: ascending in the column and, among equal columns, in the row; equal (row, column)
+ * keep their input order.  Indices are compared as signed integers and need not lie inside [0, m) x [0, n): m
+ * and n are only checked to be positive.  P (usually preset to 0..nnz-1) travels with its entry, so that
+ * sortedVal[i] = origVal[P[i]].  The call synchronises the handle's stream once. */
+aclsparseStatus_t aclsparseXcoosort_bufferSizeExt(aclsparseHandle_t handle, int m, int n, int nnz, const int *cooRowsA,
+                                                  const int *cooColsA, size_t *pBufferSizeInBytes);
+aclsparseStatus_t aclsparseXcoosortByRow(aclsparseHandle_t handle, int m, int n, int nnz, int *cooRowsA, int *cooColsA,
+                                         int *P, void *pBuffer);
+aclsparseStatus_t aclsparseXcoosortByColumn(aclsparseHandle_t handle, int m, int n, int nnz, int *cooRowsA,
+                                            int *cooColsA, int *P, void *pBuffer);
+
 /* [ref: :1401-1440; host sparse/csr2csc_ex2/arch35/csr2csc_ex2_host.cpp:109-232, :535-618]
  * CSR (m x n) -> CSC: cscColPtr[0..n], cscRowInd and, for NUMERIC, cscVal; the
  * entries of a column keep their CSR order (ascending rows).  Values are moved

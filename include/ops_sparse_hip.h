@@ -315,6 +315,13 @@ size_t opsparse_csrsort_workspace_bytes(int64_t m, int64_t nnz);
 int opsparse_csrsort_launch(int64_t m, int64_t n, int64_t nnz, int32_t indexBase, const int32_t *csrRowPtr,
                             int32_t *csrColInd, int32_t *perm, void *workspace, size_t workspaceBytes, void *stream);
 
+/* Stable sort of (cooRows, cooCols, perm) triples in place: byRow != 0 ascending in the row and, among equal rows,
+ * in the column; byRow == 0 the other way round.  Signed indices of any value.  Synchronises `stream` once (the
+ * range the indices span is read back and sets the number of passes). */
+size_t opsparse_coosort_workspace_bytes(int64_t nnz);
+int opsparse_coosort_launch(int64_t nnz, int32_t byRow, int32_t *cooRows, int32_t *cooCols, int32_t *perm,
+                            void *workspace, size_t workspaceBytes, void *stream);
+
 /* CSR -> CSC.  valueBytes: 0 (structure only), 1, 2 or 4. */
 size_t opsparse_csr2csc_workspace_bytes(int64_t m, int64_t n, int64_t nnz);
 int opsparse_csr2csc_launch(int64_t m, int64_t n, int64_t nnz, const void *csrVal, const int32_t *csrRowPtr,

@@ -83,6 +83,8 @@ ACLSPARSE_SYMBOLS = [
     "aclsparseSetMatDiagType", "aclsparseSetMatFillMode", "aclsparseGetMatType", "aclsparseGetMatIndexBase",
     "aclsparseGetMatDiagType", "aclsparseGetMatFillMode",
     "aclsparseXcoo2csr", "aclsparseXcsr2coo", "aclsparseXcsrsort_bufferSizeExt", "aclsparseXcsrsort",
+    "aclsparseXcscsort_bufferSizeExt", "aclsparseXcscsort",
+    "aclsparseXcoosort_bufferSizeExt", "aclsparseXcoosortByRow", "aclsparseXcoosortByColumn",
     "aclsparseCsr2cscEx2_bufferSize", "aclsparseCsr2cscEx2",
 ]
 ACL_SPARSE_ACTION_SYMBOLIC, ACL_SPARSE_ACTION_NUMERIC = 0, 1
@@ -98,7 +100,8 @@ OPSPARSE_SYMBOLS = [
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
     "opsparse_dense_restage",
     "opsparse_scan_workspace_bytes", "opsparse_coo2csr_launch", "opsparse_csr2coo_launch",
-    "opsparse_csrsort_workspace_bytes", "opsparse_csrsort_launch", "opsparse_csr2csc_workspace_bytes",
+    "opsparse_csrsort_workspace_bytes", "opsparse_csrsort_launch", "opsparse_coosort_workspace_bytes",
+    "opsparse_coosort_launch", "opsparse_csr2csc_workspace_bytes",
     "opsparse_csr2csc_launch",
     "opsparse_copy_launch", "opsparse_read_launch", "opsparse_gather_launch",
 ]
@@ -208,6 +211,11 @@ def lib():
     L.aclsparseXcsr2coo.argtypes = [vp, vp, i64, i64, vp, ci]
     L.aclsparseXcsrsort_bufferSizeExt.argtypes = [vp, ci, ci, ci, vp, vp, ctypes.POINTER(sz)]
     L.aclsparseXcsrsort.argtypes = [vp, ci, ci, ci, vp, vp, vp, vp, vp]
+    L.aclsparseXcscsort_bufferSizeExt.argtypes = [vp, ci, ci, ci, vp, vp, ctypes.POINTER(sz)]
+    L.aclsparseXcscsort.argtypes = [vp, ci, ci, ci, vp, vp, vp, vp, vp]
+    L.aclsparseXcoosort_bufferSizeExt.argtypes = [vp, ci, ci, ci, vp, vp, ctypes.POINTER(sz)]
+    L.aclsparseXcoosortByRow.argtypes = [vp, ci, ci, ci, vp, vp, vp, vp]
+    L.aclsparseXcoosortByColumn.argtypes = [vp, ci, ci, ci, vp, vp, vp, vp]
     csc_common = [vp, ci, ci, ci, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci]
     L.aclsparseCsr2cscEx2_bufferSize.argtypes = csc_common + [ctypes.POINTER(sz)]
     L.aclsparseCsr2cscEx2.argtypes = csc_common + [vp]
@@ -221,6 +229,10 @@ def lib():
     L.opsparse_csrsort_workspace_bytes.argtypes = [i64, i64]
     L.opsparse_csrsort_launch.restype = ci
     L.opsparse_csrsort_launch.argtypes = [i64, i64, i64, i32, vp, vp, vp, vp, sz, vp]
+    L.opsparse_coosort_workspace_bytes.restype = sz
+    L.opsparse_coosort_workspace_bytes.argtypes = [i64]
+    L.opsparse_coosort_launch.restype = ci
+    L.opsparse_coosort_launch.argtypes = [i64, i32, vp, vp, vp, vp, sz, vp]
     L.opsparse_csr2csc_workspace_bytes.restype = sz
     L.opsparse_csr2csc_workspace_bytes.argtypes = [i64, i64, i64]
     L.opsparse_csr2csc_launch.restype = ci

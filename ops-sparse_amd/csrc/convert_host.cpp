@@ -1,5 +1,6 @@
 // CSR producers of the aclsparse API: aclsparseXcoo2csr, aclsparseXcsr2coo,
-// aclsparseXcsrsort(+_bufferSizeExt), aclsparseCsr2cscEx2(+_bufferSize) and the
+// aclsparseXcsrsort / Xcscsort (+_bufferSizeExt), aclsparseXcoosortByRow / ByColumn (+_bufferSizeExt),
+// aclsparseCsr2cscEx2(+_bufferSize) and the
 // legacy matrix descriptor that csrsort takes its index base from.
 //
 // Argument checks, their order and status codes follow the reference's host
@@ -246,6 +247,136 @@ aclsparseStatus_t aclsparseXcsrsort(aclsparseHandle_t handle, int m, int n, int 
         opsparse::LogError("aclsparseXcsrsort: launch failed (%d)", rc);
     }
     return FromLaunch(rc);
+}
+
+// ------------------------------------------------------------------ cscsort
+
+// reference: sparse/cscsort/arch35/cscsort_host.cpp:52-72
+static aclsparseStatus_t CscsortCommon(int m, int n, int nnz, const int *cscColPtr, const int *cscRowInd)
+{
+    if (m < 0 || n < 0 || nnz < 0) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if ((m == 0 || n == 0) && nnz != 0) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if ((n > 0 && cscColPtr == nullptr) || (nnz > 0 && cscRowInd == nullptr)) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t aclsparseXcscsort_bufferSizeExt(aclsparseHandle_t handle, int m, int n, int nnz,
+                                                  const int *cscColPtr, const int *cscRowInd,
+                                                  size_t *pBufferSizeInBytes)
+{
+    if (handle == nullptr) {
+        return ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR;
+    }
+    if (pBufferSizeInBytes == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    const aclsparseStatus_t st = CscsortCommon(m, n, nnz, cscColPtr, cscRowInd);
+    if (st != ACL_SPARSE_STATUS_SUCCESS) {
+        return st;
+    }
+    *pBufferSizeInBytes = opsparse_csrsort_workspace_bytes(n, nnz);  // the columns take the rows' part; 0 when nnz == 0
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t aclsparseXcscsort(aclsparseHandle_t handle, int m, int n, int nnz, const aclsparseMatDescr_t descrA,
+                                    const int *cscColPtr, int *cscRowInd, int *P, void *pBuffer)
+{
+    if (handle == nullptr) {
+        return ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR;
+    }
+    const aclsparseStatus_t st = CscsortCommon(m, n, nnz, cscColPtr, cscRowInd);
+    if (st != ACL_SPARSE_STATUS_SUCCESS) {
+        return st;
+    }
+    if (descrA == nullptr || !ValidBase(descrA->indexBase)) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if (nnz == 0) {
+        return ACL_SPARSE_STATUS_SUCCESS;
+    }
+    if (P == nullptr || pBuffer == nullptr || reinterpret_cast<uintptr_t>(pBuffer) % 128U != 0U) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    // a CSC matrix is the CSR form of its transpose: n "rows" whose "column" indices lie below m
+    const int rc = opsparse_csrsort_launch(n, m, nnz, static_cast<int32_t>(descrA->indexBase), cscColPtr, cscRowInd, P,
+                                           pBuffer, opsparse_csrsort_workspace_bytes(n, nnz), handle->stream);
+    if (rc != OPSPARSE_OK) {
+        opsparse::LogError("aclsparseXcscsort: launch failed (%d)", rc);
+    }
+    return FromLaunch(rc);
+}
+
+// ------------------------------------------------------------------ coosort
+
+// reference: sparse/coosort/arch35/coosort_host.cpp:48-78
+static aclsparseStatus_t CoosortCommon(int m, int n, int nnz, const int *cooRowsA, const int *cooColsA)
+{
+    if (m <= 0 || n <= 0 || nnz < 0) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    if (nnz > 0 && (cooRowsA == nullptr || cooColsA == nullptr)) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+aclsparseStatus_t aclsparseXcoosort_bufferSizeExt(aclsparseHandle_t handle, int m, int n, int nnz, const int *cooRowsA,
+                                                  const int *cooColsA, size_t *pBufferSizeInBytes)
+{
+    if (handle == nullptr) {
+        return ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR;
+    }
+    if (pBufferSizeInBytes == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    const aclsparseStatus_t st = CoosortCommon(m, n, nnz, cooRowsA, cooColsA);
+    if (st != ACL_SPARSE_STATUS_SUCCESS) {
+        return st;
+    }
+    *pBufferSizeInBytes = opsparse_coosort_workspace_bytes(nnz);  // 0 when nnz == 0
+    return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+static aclsparseStatus_t Coosort(const char *api, aclsparseHandle_t handle, int m, int n, int nnz, int byRow,
+                                 int *cooRowsA, int *cooColsA, int *P, void *pBuffer)
+{
+    if (handle == nullptr) {
+        return ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR;
+    }
+    const aclsparseStatus_t st = CoosortCommon(m, n, nnz, cooRowsA, cooColsA);
+    if (st != ACL_SPARSE_STATUS_SUCCESS) {
+        return st;
+    }
+    if (nnz == 0) {
+        return ACL_SPARSE_STATUS_SUCCESS;
+    }
+    if (P == nullptr || pBuffer == nullptr) {
+        return ACL_SPARSE_STATUS_INVALID_VALUE;
+    }
+    const int rc = opsparse_coosort_launch(nnz, byRow, cooRowsA, cooColsA, P, pBuffer,
+                                           opsparse_coosort_workspace_bytes(nnz), handle->stream);
+    if (rc != OPSPARSE_OK) {
+        opsparse::LogError("%s: launch failed (%d)", api, rc);
+    }
+    return FromLaunch(rc);
+}
+
+aclsparseStatus_t aclsparseXcoosortByRow(aclsparseHandle_t handle, int m, int n, int nnz, int *cooRowsA, int *cooColsA,
+                                         int *P, void *pBuffer)
+{
+    return Coosort("aclsparseXcoosortByRow", handle, m, n, nnz, 1, cooRowsA, cooColsA, P, pBuffer);
+}
+
+aclsparseStatus_t aclsparseXcoosortByColumn(aclsparseHandle_t handle, int m, int n, int nnz, int *cooRowsA,
+                                            int *cooColsA, int *P, void *pBuffer)
+{
+    return Coosort("aclsparseXcoosortByColumn", handle, m, n, nnz, 0, cooRowsA, cooColsA, P, pBuffer);
 }
 
 // ------------------------------------------------------------------ csr2csc

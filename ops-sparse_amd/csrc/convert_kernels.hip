@@ -463,6 +463,12 @@ constexpr int kWideSlotBits = 12;
 static_assert(kWideTile <= (1 << kWideSlotBits), "a slot number fits its field");
 static_assert(kWideDigits == kBlockThreads, "one thread per digit");
 
+// key - keyBase in wrap-around arithmetic (the keys of a COO sort may span the whole int32 range).
+__device__ __forceinline__ int32_t Rebased(int32_t key, int32_t keyBase)
+{
+    return static_cast<int32_t>(static_cast<uint32_t>(key) - static_cast<uint32_t>(keyBase));
+}
+
 // A pass's digit: `mask` = 2^bits - 1 with bits <= kWideBits (the passes of a sort share its key bits evenly).
 __device__ __forceinline__ int32_t WideDigit(int32_t key, int32_t shift, int32_t mask)
 {
@@ -505,7 +511,7 @@ __global__ __launch_bounds__(kBlockThreads) void WideCountKernel(const int32_t *
 #pragma unroll
         for (int i = 0; i < kWideItems; ++i) {
             const int64_t at = (firstTile + j) * kWideTile + i * kBlockThreads + threadIdx.x;
-            atomicAdd(&hist[j][WideDigit(key[j & 1][i] - keyBase, shift, mask)], at < n ? 1 : 0);
+            atomicAdd(&hist[j][WideDigit(Rebased(key[j & 1][i], keyBase), shift, mask)], at < n ? 1 : 0);
         }
     }
     __syncthreads();
@@ -560,7 +566,7 @@ __device__ __forceinline__ void WideFetch(WideTileRegs &r, int64_t tile, const i
         r.key[i] = static_cast<int32_t>(static_cast<uint32_t>(mask) << shift);
         r.pay[i] = RadixPair{0, 0u};
         if (Full || at < n) {
-            r.key[i] = keysIn[at] - keyBase;
+            r.key[i] = Rebased(keysIn[at], keyBase);
             if (Mode == kPayPairFirst) {
                 r.pay[i].row = io.rowSrc[at];
                 if (VB == 4) {
@@ -1660,6 +1666,186 @@ int opsparse_csr2csc_launch(int64_t m, int64_t n, int64_t nnz, const void *csrVa
     hipLaunchKernelGGL(CountRunsKernel, dim3(GridFor(nnz, kBlockThreads * 8)), dim3(kBlockThreads), 0, s, keysIn, nnz,
                        n, 0, cscColPtr);
     LaunchInclusiveScan(cscColPtr, cscColPtr, n + 1, indexBase, tiles, s);
+    return CheckLaunch();
+}
+
+
+// ------------------------------------------------------------------ coosort
+//
+// aclsparseXcoosortByRow / ByColumn (sparse/coosort/arch35/coosort_host.cpp:309-371; the order is the one of
+// test/coosort/arch35/coosort_golden.h:52-85): a stable sort of (primary, secondary, P) triples, signed keys,
+// ascending in the primary key and, among equal ones, in the secondary.  Least-significant-key first: the 8-bit
+// passes of csr2csc over the secondary key, the primary key and P travelling as the pair, then over the primary
+// key with the secondary key and P as the pair; the last pass writes the caller's three arrays.  The keys are
+// taken relative to their minimum, found on the device first, so that a pass count follows from the range the
+// indices really span (one read-back of four integers: the call synchronises its stream once).
+
+}  // extern "C"
+
+namespace opsparse {
+namespace {
+
+// range[0..3] = min / max of a[], min / max of b[] (pre-filled with INT32_MAX / INT32_MIN alternately).
+__global__ __launch_bounds__(kBlockThreads) void CooRangeKernel(const int32_t *__restrict__ a,
+                                                                const int32_t *__restrict__ b, int64_t n,
+                                                                int32_t *__restrict__ range)
+{
+    int32_t lo[2] = {INT32_MAX, INT32_MAX}, hi[2] = {INT32_MIN, INT32_MIN};
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
+        const int32_t v[2] = {a[i], b[i]};
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            lo[k] = v[k] < lo[k] ? v[k] : lo[k];
+            hi[k] = v[k] > hi[k] ? v[k] : hi[k];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+#pragma unroll
+        for (int off = kWave / 2; off > 0; off >>= 1) {
+            const int32_t l = __shfl_xor(lo[k], off), h = __shfl_xor(hi[k], off);
+            lo[k] = l < lo[k] ? l : lo[k];
+            hi[k] = h > hi[k] ? h : hi[k];
+        }
+    }
+    if (threadIdx.x % kWave == 0) {
+        atomicMin(range + 0, lo[0]);
+        atomicMax(range + 1, hi[0]);
+        atomicMin(range + 2, lo[1]);
+        atomicMax(range + 3, hi[1]);
+    }
+}
+
+__global__ __launch_bounds__(kBlockThreads) void CooRangeInitKernel(int32_t *range)
+{
+    if (threadIdx.x < 4) {
+        range[threadIdx.x] = (threadIdx.x & 1) ? INT32_MIN : INT32_MAX;
+    }
+}
+
+// a[i] += addA, b[i] += addB (wrap-around: the sorted keys come back relative to their minimum).
+__global__ __launch_bounds__(kBlockThreads) void CooRebaseKernel(int32_t *__restrict__ a, int32_t *__restrict__ b,
+                                                                 int64_t n, int32_t addA, int32_t addB)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
+        a[i] = static_cast<int32_t>(static_cast<uint32_t>(a[i]) + static_cast<uint32_t>(addA));
+        b[i] = static_cast<int32_t>(static_cast<uint32_t>(b[i]) + static_cast<uint32_t>(addB));
+    }
+}
+
+struct CoosortLayout {
+    int64_t range, keysA, keysB, pairsA, pairsB, table, tiles, bytes;
+};
+
+CoosortLayout LayoutCoosort(int64_t nnz)
+{
+    CoosortLayout l{};
+    int64_t off = 0;
+    l.range = off; off += 256;
+    l.keysA = off; off += Align256(4 * nnz);
+    l.keysB = off; off += Align256(4 * nnz);
+    l.pairsA = off; off += Align256(8 * nnz);
+    l.pairsB = off; off += Align256(8 * nnz);
+    l.table = off; off += Align256(4 * WideTableInts(nnz));
+    l.tiles = off; off += Align256(4 * ScanTiles(WideTableInts(nnz)));
+    l.bytes = off;
+    return l;
+}
+
+// Bits that hold hi - lo (both int32, hi >= lo), at least 1.
+int32_t RangeBits(int32_t lo, int32_t hi)
+{
+    const uint32_t span = static_cast<uint32_t>(hi) - static_cast<uint32_t>(lo);
+    int32_t bits = 1;
+    while (bits < 32 && (span >> bits) != 0) {
+        ++bits;
+    }
+    return bits;
+}
+
+}  // namespace
+}  // namespace opsparse
+
+extern "C" {
+
+size_t opsparse_coosort_workspace_bytes(int64_t nnz)
+{
+    return nnz <= 0 ? 0 : static_cast<size_t>(LayoutCoosort(nnz).bytes);
+}
+
+int opsparse_coosort_launch(int64_t nnz, int32_t byRow, int32_t *cooRows, int32_t *cooCols, int32_t *perm,
+                            void *workspace, size_t workspaceBytes, void *stream)
+{
+    if (nnz < 0 || nnz > INT32_MAX) {
+        return OPSPARSE_E_INVALID;
+    }
+    if (nnz == 0) {
+        return OPSPARSE_OK;
+    }
+    if (cooRows == nullptr || cooCols == nullptr || perm == nullptr) {
+        return OPSPARSE_E_INVALID;
+    }
+    const CoosortLayout l = LayoutCoosort(nnz);
+    if (workspace == nullptr || static_cast<int64_t>(workspaceBytes) < l.bytes) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    auto s = static_cast<hipStream_t>(stream);
+    auto *base = static_cast<unsigned char *>(workspace);
+    auto at = [&](int64_t off) { return reinterpret_cast<int32_t *>(base + off); };
+    int32_t *keys[2] = {at(l.keysA), at(l.keysB)};
+    void *pairs[2] = {base + l.pairsA, base + l.pairsB};
+    int32_t *table = at(l.table), *tiles = at(l.tiles), *range = at(l.range);
+    int32_t *primary = byRow != 0 ? cooRows : cooCols, *secondary = byRow != 0 ? cooCols : cooRows;
+
+    hipLaunchKernelGGL(CooRangeInitKernel, dim3(1), dim3(kBlockThreads), 0, s, range);
+    hipLaunchKernelGGL(CooRangeKernel, dim3(GridFor(nnz, kBlockThreads * 16)), dim3(kBlockThreads), 0, s, primary,
+                       secondary, nnz, range);
+    int32_t r[4] = {0, 0, 0, 0};  // min / max of the primary key, of the secondary key
+    if (hipMemcpyAsync(r, range, sizeof(r), hipMemcpyDeviceToHost, s) != hipSuccess ||
+        hipStreamSynchronize(s) != hipSuccess) {
+        (void)hipGetLastError();
+        return OPSPARSE_E_LAUNCH;
+    }
+
+    int cur = 0;
+    // One key's passes: the first reads (key, pair) from three arrays, the last writes three arrays.
+    auto sortBy = [&](const int32_t *keySrc, int32_t keyBase, int32_t bits, const int32_t *pairRowSrc,
+                      const void *pairValSrc, int32_t *keyDst, int32_t *pairRowDst, void *pairValDst) {
+        int32_t passes = (bits + kWideBits - 1) / kWideBits;
+        passes = passes < 2 ? 2 : passes;
+        const int32_t perPass = (bits + passes - 1) / passes;
+        const RadixPairIo io{pairRowSrc, pairValSrc, pairRowDst, pairValDst, 4};
+        const int32_t *keysIn = keySrc;
+        const void *pairsIn = nullptr;
+        for (int32_t pass = 0; pass < passes; ++pass) {
+            const bool last = pass == passes - 1;
+            const int mode = pass == 0 ? kPayPairFirst : (last ? kPayPairLast : kPayPair);
+            int32_t *keysOut = last ? keyDst : keys[cur];
+            LaunchWidePairPass(mode, keysIn, pairsIn, keysOut, pairs[cur], nnz, pass == 0 ? keyBase : 0, pass * perPass,
+                               perPass, table, tiles, io, s);
+            keysIn = keysOut;
+            pairsIn = pairs[cur];
+            cur ^= 1;
+        }
+    };
+    // by the secondary key, (primary key, P) as the pair: the result stays in the workspace ...
+    int32_t *midKeys = keys[1];                                   // (two or four passes: the last one writes buffer 1
+    auto *midRows = static_cast<int32_t *>(pairs[1]);             //  only when their number is even)
+    const int32_t bitsS = RangeBits(r[2], r[3]), bitsP = RangeBits(r[0], r[1]);
+    const int32_t passesS = (bitsS + kWideBits - 1) / kWideBits < 2 ? 2 : (bitsS + kWideBits - 1) / kWideBits;
+    const int lastBuf = (passesS - 1) & 1;                        // buffer the last pass of that stage writes
+    midKeys = keys[lastBuf];
+    midRows = static_cast<int32_t *>(pairs[lastBuf]);
+    uint32_t *midVals = reinterpret_cast<uint32_t *>(pairs[lastBuf]) + nnz;
+    sortBy(secondary, r[2], bitsS, primary, perm, midKeys, midRows, midVals);
+    // ... then, stably, by the primary key, (secondary key, P) as the pair, into the caller's arrays
+    sortBy(midRows, r[0], bitsP, midKeys, midVals, primary, secondary, perm);
+    if (r[0] != 0 || r[2] != 0) {
+        hipLaunchKernelGGL(CooRebaseKernel, dim3(GridFor(nnz, kBlockThreads * 8)), dim3(kBlockThreads), 0, s, primary,
+                           secondary, nnz, r[0], r[2]);
+    }
     return CheckLaunch();
 }
 

@@ -301,6 +301,20 @@ def csrsort(rowptr, colind, perm, base=0):
     return c, p
 
 
+def cscsort(colptr, rowind, perm, base=0):
+    colptr = _c(colptr, np.int32)
+    r, p = _c(rowind, np.int32).copy(), _c(perm, np.int32).copy()
+    lib().oracle_cscsort(_p(colptr), c_i64(colptr.size - 1), c_i32(base), _p(r), _p(p))
+    return r, p
+
+
+def coosort(rows, cols, perm, by_row=True):
+    """(rows, cols, perm) stably sorted by (row, col), or by (col, row) when by_row is false."""
+    r, c, p = _c(rows, np.int32).copy(), _c(cols, np.int32).copy(), _c(perm, np.int32).copy()
+    lib().oracle_coosort(c_i64(r.size), c_i32(1 if by_row else 0), _p(r), _p(c), _p(p))
+    return r, c, p
+
+
 def csr2csc(m, n, rowptr, colind, val=None, base=0):
     """(colptr, rowind, cscval); val of any 1 / 2 / 4-byte dtype or None (structure only)."""
     rowptr, colind = _c(rowptr, np.int32), _c(colind, np.int32)

@@ -645,6 +645,51 @@ void oracle_csrsort(const int32_t *rowPtr, int64_t m, int32_t base, int32_t *col
     }
 }
 
+/* cscsortGolden, test/cscsort/arch35/cscsort_golden.h:30-70: the column-wise twin of csrsortGolden; a CSC matrix is
+ * the CSR form of its transpose, so the same walk over colPtr does it. */
+void oracle_cscsort(const int32_t *colPtr, int64_t n, int32_t base, int32_t *rowInd, int32_t *perm)
+{
+    oracle_csrsort(colPtr, n, base, rowInd, perm);
+}
+
+/* coosortGolden, test/coosort/arch35/coosort_golden.h:52-85: a stable sort of the (row, col, P) triples, signed
+ * keys, by (row, col) when byRow != 0 and by (col, row) otherwise; P travels with its entry.  Bottom-up merge sort
+ * that takes from the right run only when its key is strictly smaller. */
+void oracle_coosort(int64_t nnz, int32_t byRow, int32_t *rows, int32_t *cols, int32_t *perm)
+{
+    if (nnz <= 1) {
+        return;
+    }
+    int32_t *block = (int32_t *)malloc(sizeof(int32_t) * (size_t)nnz * 6);
+    int32_t *a0 = block, *b0 = a0 + nnz, *p0 = b0 + nnz, *a1 = p0 + nnz, *b1 = a1 + nnz, *p1 = b1 + nnz;
+    memcpy(a0, byRow ? rows : cols, sizeof(int32_t) * (size_t)nnz);  /* a: primary key, b: secondary */
+    memcpy(b0, byRow ? cols : rows, sizeof(int32_t) * (size_t)nnz);
+    memcpy(p0, perm, sizeof(int32_t) * (size_t)nnz);
+    for (int64_t w = 1; w < nnz; w *= 2) {
+        for (int64_t lo = 0; lo < nnz; lo += 2 * w) {
+            const int64_t mid = lo + w < nnz ? lo + w : nnz, hi = lo + 2 * w < nnz ? lo + 2 * w : nnz;
+            int64_t i = lo, j = mid, k = lo;
+            while (i < mid && j < hi) {
+                const int less = a0[j] != a0[i] ? a0[j] < a0[i] : b0[j] < b0[i];
+                if (less) {
+                    a1[k] = a0[j]; b1[k] = b0[j]; p1[k++] = p0[j++];
+                } else {
+                    a1[k] = a0[i]; b1[k] = b0[i]; p1[k++] = p0[i++];
+                }
+            }
+            while (i < mid) { a1[k] = a0[i]; b1[k] = b0[i]; p1[k++] = p0[i++]; }
+            while (j < hi) { a1[k] = a0[j]; b1[k] = b0[j]; p1[k++] = p0[j++]; }
+        }
+        int32_t *t = a0; a0 = a1; a1 = t;
+        t = b0; b0 = b1; b1 = t;
+        t = p0; p0 = p1; p1 = t;
+    }
+    memcpy(byRow ? rows : cols, a0, sizeof(int32_t) * (size_t)nnz);
+    memcpy(byRow ? cols : rows, b0, sizeof(int32_t) * (size_t)nnz);
+    memcpy(perm, p0, sizeof(int32_t) * (size_t)nnz);
+    free(block);
+}
+
 /* Csr2CscGolden, test/csr2csc_ex2/csr2csc_ex2_golden.h:50-110: column counts,
  * exclusive prefix sum + base, then a row-major walk that drops every entry at
  * its column's next free slot (so rows ascend inside a column).  Values move

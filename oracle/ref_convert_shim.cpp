@@ -10,6 +10,8 @@
 #include REF_CSR2COO_H
 #include REF_CSRSORT_H
 #include REF_CSR2CSC_H
+#include REF_COOSORT_H
+#include REF_CSCSORT_H
 
 #include <cstdint>
 #include <cstring>
@@ -56,6 +58,29 @@ void ref_csr2csc(int32_t m, int32_t n, int32_t nnz, int32_t base, const int32_t 
     if (nnz > 0) {
         std::memcpy(rowInd, r.cscRowInd.data(), sizeof(int32_t) * nnz);
         std::memcpy(cscVal, r.cscVal.data(), sizeof(float) * nnz);
+    }
+}
+
+// P is taken to be 0 .. nnz-1 on entry, as the golden does.
+void ref_coosort(const int32_t *rows, const int32_t *cols, int32_t nnz, int32_t byRow, int32_t *outRows,
+                 int32_t *outCols, int32_t *outP)
+{
+    const std::vector<int32_t> r(rows, rows + nnz), c(cols, cols + nnz);
+    const sparse_test::CoosortGoldenResult g = sparse_test::coosortGolden(r, c, byRow != 0);
+    if (nnz > 0) {
+        std::memcpy(outRows, g.rows.data(), sizeof(int32_t) * nnz);
+        std::memcpy(outCols, g.cols.data(), sizeof(int32_t) * nnz);
+        std::memcpy(outP, g.P.data(), sizeof(int32_t) * nnz);
+    }
+}
+
+void ref_cscsort(const int32_t *colPtr, int32_t n, int32_t nnz, int32_t base, int32_t *rowInd, int32_t *perm)
+{
+    const std::vector<int32_t> cp(colPtr, colPtr + n + 1), ri(rowInd, rowInd + nnz), p(perm, perm + nnz);
+    const sparse_test::CscsortGoldenResult r = sparse_test::cscsortGolden(cp, ri, p, n, base);
+    if (nnz > 0) {
+        std::memcpy(rowInd, r.rowInd.data(), sizeof(int32_t) * nnz);
+        std::memcpy(perm, r.P.data(), sizeof(int32_t) * nnz);
     }
 }
 

@@ -513,6 +513,51 @@ def test_conversion_status_table(osa, L, handle):
     assert so(handle, 4, 4, 0, d, FAKE, None, None, None) == 0       # nothing to sort
     assert so(handle, 4, 4, 5, d, FAKE, FAKE, None, FAKE) == INV and so(handle, 4, 4, 5, d, FAKE, FAKE, FAKE, None) == INV
     L.aclsparseDestroyMatDescr(d)
+    # cscsort (sparse/cscsort/arch35/cscsort_host.cpp:52-216): csrsort's checks with the columns in the rows' part,
+    # and a buffer that must be 128-byte aligned
+    bs = L.aclsparseXcscsort_bufferSizeExt
+    assert bs(None, 4, 4, 5, FAKE, FAKE, ctypes.byref(n)) == HN
+    assert bs(handle, 4, 4, 5, FAKE, FAKE, None) == INV
+    for bad in ((-1, 4, 5), (4, -1, 5), (4, 4, -1), (0, 4, 5), (4, 0, 5)):
+        assert bs(handle, *bad, FAKE, FAKE, ctypes.byref(n)) == INV, bad
+    assert bs(handle, 4, 4, 5, None, FAKE, ctypes.byref(n)) == INV
+    assert bs(handle, 4, 4, 5, FAKE, None, ctypes.byref(n)) == INV
+    assert bs(handle, 4, 0, 0, None, None, ctypes.byref(n)) == 0 and n.value == 0   # no column: no colPtr needed
+    assert bs(handle, 4, 6, 5, FAKE, FAKE, ctypes.byref(n)) == 0 and n.value == L.opsparse_csrsort_workspace_bytes(6, 5)
+    assert n.value >= 2 * 5 * 4
+    d = ctypes.c_void_p(None)
+    L.aclsparseCreateMatDescr(ctypes.byref(d))
+    so = L.aclsparseXcscsort
+    ALIGNED, ODD = ctypes.c_void_p(0x7f0000001000), ctypes.c_void_p(0x7f0000001040)
+    assert so(None, 4, 4, 5, d, FAKE, FAKE, FAKE, ALIGNED) == HN
+    assert so(handle, 4, 4, -5, d, FAKE, FAKE, FAKE, ALIGNED) == INV and so(handle, 4, 0, 5, d, FAKE, FAKE, FAKE, ALIGNED) == INV
+    assert so(handle, 4, 4, 5, d, None, FAKE, FAKE, ALIGNED) == INV and so(handle, 4, 4, 5, d, FAKE, None, FAKE, ALIGNED) == INV
+    assert so(handle, 4, 4, 5, None, FAKE, FAKE, FAKE, ALIGNED) == INV
+    L.aclsparseSetMatIndexBase(d, 5)
+    assert so(handle, 4, 4, 5, d, FAKE, FAKE, FAKE, ALIGNED) == INV
+    L.aclsparseSetMatIndexBase(d, 1)
+    assert so(handle, 4, 4, 0, d, FAKE, None, None, None) == 0       # nothing to sort
+    assert so(handle, 4, 4, 5, d, FAKE, FAKE, None, ALIGNED) == INV and so(handle, 4, 4, 5, d, FAKE, FAKE, FAKE, None) == INV
+    assert so(handle, 4, 4, 5, d, FAKE, FAKE, FAKE, ODD) == INV      # 64-byte aligned only
+    L.aclsparseDestroyMatDescr(d)
+    # coosort (sparse/coosort/arch35/coosort_host.cpp:48-78, :262-371): m and n must be positive, whatever nnz
+    bs = L.aclsparseXcoosort_bufferSizeExt
+    assert bs(None, 4, 4, 5, FAKE, FAKE, ctypes.byref(n)) == HN
+    assert bs(handle, 4, 4, 5, FAKE, FAKE, None) == INV
+    for bad in ((0, 4, 5), (4, 0, 5), (-1, 4, 5), (4, -3, 5), (4, 4, -1), (0, 4, 0)):
+        assert bs(handle, *bad, FAKE, FAKE, ctypes.byref(n)) == INV, bad
+    assert bs(handle, 4, 4, 5, None, FAKE, ctypes.byref(n)) == INV and bs(handle, 4, 4, 5, FAKE, None, ctypes.byref(n)) == INV
+    assert bs(handle, 4, 4, 0, None, None, ctypes.byref(n)) == 0 and n.value == 0
+    assert bs(handle, 4, 4, 5, FAKE, FAKE, ctypes.byref(n)) == 0 and n.value == L.opsparse_coosort_workspace_bytes(5)
+    assert n.value >= 5 * 12                                         # at least the reference's 12 bytes an entry
+    assert bs(handle, 1, 1, IMAX, FAKE, FAKE, ctypes.byref(n)) == 0 and n.value >= 24 * IMAX
+    for so in (L.aclsparseXcoosortByRow, L.aclsparseXcoosortByColumn):
+        assert so(None, 4, 4, 5, FAKE, FAKE, FAKE, FAKE) == HN
+        assert so(handle, 0, 4, 5, FAKE, FAKE, FAKE, FAKE) == INV and so(handle, 4, 0, 5, FAKE, FAKE, FAKE, FAKE) == INV
+        assert so(handle, 4, 4, -1, FAKE, FAKE, FAKE, FAKE) == INV
+        assert so(handle, 4, 4, 5, None, FAKE, FAKE, FAKE) == INV and so(handle, 4, 4, 5, FAKE, None, FAKE, FAKE) == INV
+        assert so(handle, 4, 4, 0, None, None, None, None) == 0      # nothing to sort: P and the buffer may be NULL
+        assert so(handle, 4, 4, 5, FAKE, FAKE, None, FAKE) == INV and so(handle, 4, 4, 5, FAKE, FAKE, FAKE, None) == INV
     # csr2csc
     F, NUM, SYM = osa.ACL_FLOAT, osa.ACL_SPARSE_ACTION_NUMERIC, osa.ACL_SPARSE_ACTION_SYMBOLIC
     ptrs = (FAKE, FAKE, FAKE, FAKE, FAKE, FAKE)

@@ -1,5 +1,5 @@
 """GPU parity tests of the CSR producers (aclsparseXcoo2csr, aclsparseXcsr2coo, aclsparseXcsrsort,
-aclsparseCsr2cscEx2) through the C ABI.  Every output is compared bit for bit with the CPU oracle.
+aclsparseXcscsort, aclsparseXcoosortByRow / ByColumn, aclsparseCsr2cscEx2) through the C ABI.  Every output is compared bit for bit with the CPU oracle.
 
 The coo2csr / csr2coo / csr2csc case tables are the reference's own
 (test/<op>/arch35/<op>_test.csv, kept as data fixtures under tests/golden/); matrices come
@@ -328,6 +328,148 @@ def test_csrsort_long_rows_on_average(osa, gpu_ctx, lengths, n, base):
     rowptr, colind = _rows(lengths, lambda r, l: rng.integers(0, n, l))
     perm = rng.integers(-1000, 1000, colind.size).astype(np.int32) if base else None
     run_csrsort(osa, gpu_ctx, len(lengths), n, rowptr + base, colind + base, base=base, perm=perm, misalign=4 * base)
+
+
+# ------------------------------------------------------------------ cscsort
+
+def run_cscsort(osa, gpu_ctx, m, n, colptr, rowind, base=0, perm=None):
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    nnz = int(rowind.size)
+    perm = np.arange(nnz, dtype=np.int32) if perm is None else perm
+    d_ptr, d_row, d_perm = dev_i32(colptr, dev), dev_i32(rowind, dev), dev_i32(perm, dev)
+    size = ctypes.c_size_t(0)
+    assert L.aclsparseXcscsort_bufferSizeExt(handle.h, m, n, nnz, ptr(d_ptr), ptr(d_row), ctypes.byref(size)) == 0
+    buf = torch.empty(size.value + 256, dtype=torch.uint8, device=dev)
+    aligned = (buf.data_ptr() + 127) // 128 * 128                    # the reference asks for 128-byte alignment
+    descr = ctypes.c_void_p(None)
+    assert L.aclsparseCreateMatDescr(ctypes.byref(descr)) == 0
+    L.aclsparseSetMatIndexBase(descr, base)
+    torch.cuda.synchronize()
+    if nnz:
+        assert L.aclsparseXcscsort(handle.h, m, n, nnz, descr, ptr(d_ptr), ptr(d_row), ptr(d_perm),
+                                   ctypes.c_void_p(aligned + 4)) == osa.ACL_SPARSE_STATUS_INVALID_VALUE
+    assert L.aclsparseXcscsort(handle.h, m, n, nnz, descr, ptr(d_ptr), ptr(d_row), ptr(d_perm),
+                               ctypes.c_void_p(aligned) if nnz else None) == 0
+    stream.synchronize()
+    L.aclsparseDestroyMatDescr(descr)
+    want_r, want_p = oracle.cscsort(colptr, rowind, perm, base)
+    assert np.array_equal(d_ptr.cpu().numpy(), colptr)
+    assert np.array_equal(d_row.cpu().numpy(), want_r) and np.array_equal(d_perm.cpu().numpy(), want_p)
+
+
+@pytest.mark.parametrize("name", list(SORT_CASES))
+def test_cscsort_reference_cases(osa, gpu_ctx, name):
+    """test/cscsort/arch35/cscsort_test.cpp:245-530 builds the same shapes as the csrsort test with the roles of
+    rows and columns exchanged (Basic, EmptyCols, Reverse, DuplicateRows, ManySmallCols, MultiCoreSkewedCols,
+    LongCol, LongColMultiRun, RandomMedium, RunSizeBoundaries, LargeNnzMultiCore ...): the csrsort cases, read
+    as CSC matrices of n x m."""
+    cols_, rows_, colptr, rowind = SORT_CASES[name]()
+    run_cscsort(osa, gpu_ctx, rows_, cols_, colptr, rowind)
+
+
+def test_cscsort_base1_custom_perm_last_column_empty_single_row(osa, gpu_ctx):
+    """Base1 / NonIdentityP / LastColEmpty / SingleRow of the reference test."""
+    rng = np.random.default_rng(18)
+    m, n = 70000, 3000
+    lengths = rng.integers(0, 100, n)
+    lengths[[5, 2998]] = [5000, 20000]
+    lengths[-1] = 0
+    colptr, rowind = _rows(lengths, lambda c, l: rng.integers(0, m, l))
+    perm = rng.integers(-1000, 1000, rowind.size).astype(np.int32)
+    run_cscsort(osa, gpu_ctx, m, n, colptr + 1, rowind + 1, base=1, perm=perm)
+    # one row: every column holds the row 0 once or not at all, several times in one (a stable no-op)
+    colptr = np.array([0, 1, 1, 4, 5], np.int32)
+    run_cscsort(osa, gpu_ctx, 1, 4, colptr, np.zeros(5, np.int32), perm=np.array([9, 8, 7, 6, 5], np.int32))
+    run_cscsort(osa, gpu_ctx, 6, 6, np.zeros(7, np.int32), np.zeros(0, np.int32))       # EmptyMatrix
+
+
+# ------------------------------------------------------------------ coosort
+
+def run_coosort(osa, gpu_ctx, m, n, rows, cols, by_row, perm=None):
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = np.ascontiguousarray(rows, np.int32), np.ascontiguousarray(cols, np.int32)
+    nnz = int(rows.size)
+    perm = np.arange(nnz, dtype=np.int32) if perm is None else perm
+    d_r, d_c, d_p = dev_i32(rows, dev), dev_i32(cols, dev), dev_i32(perm, dev)
+    size = ctypes.c_size_t(0)
+    assert L.aclsparseXcoosort_bufferSizeExt(handle.h, m, n, nnz, ptr(d_r), ptr(d_c), ctypes.byref(size)) == 0
+    assert (size.value > 0) == (nnz > 0)
+    buf = torch.empty(size.value + 64, dtype=torch.uint8, device=dev)
+    torch.cuda.synchronize()
+    fn = L.aclsparseXcoosortByRow if by_row else L.aclsparseXcoosortByColumn
+    # (the reference asks for no alignment of the buffer: 4 bytes off the allocation)
+    assert fn(handle.h, m, n, nnz, ptr(d_r), ptr(d_c), ptr(d_p), ctypes.c_void_p(buf.data_ptr() + 4) if nnz else None) == 0
+    stream.synchronize()
+    want = oracle.coosort(rows, cols, perm, by_row)
+    for got, exp, what in zip((d_r, d_c, d_p), want, ("rows", "cols", "P")):
+        assert np.array_equal(got.cpu().numpy(), exp), what
+
+
+@pytest.mark.parametrize("by_row", [True, False])
+def test_coosort_reference_small_cases(osa, gpu_ctx, by_row):
+    """ByRowBasic, ByColumnBasic, ByRowStableDuplicateKey, NnzZero and one entry
+    (test/coosort/arch35/coosort_test.cpp:233-262, :531-546)."""
+    run_coosort(osa, gpu_ctx, 4, 4, [2, 0, 3, 0, 1, 2], [1, 3, 2, 1, 0, 3], by_row)
+    run_coosort(osa, gpu_ctx, 3, 5, [0, 0, 0, 1, 1, 2], [4, 1, 3, 2, 0, 9], by_row)
+    run_coosort(osa, gpu_ctx, 4, 4, [], [], by_row)
+    run_coosort(osa, gpu_ctx, 4, 4, [3], [2], by_row, perm=np.array([77], np.int32))
+
+
+@pytest.mark.parametrize("nnz,m,n", [(12, 8, 8), (49, 16, 16), (103, 32, 24), (215, 40, 64), (388, 64, 64),
+                                     (3839, 100, 100), (3840, 100, 100), (3841, 100, 100), (20000, 300, 200),
+                                     (100_000, 5000, 7000), (1_000_003, 65536, 65536), (3_000_000, 4, 3)])
+@pytest.mark.parametrize("by_row", [True, False])
+def test_coosort_random_matrices(osa, gpu_ctx, nnz, m, n, by_row):
+    """ByRowRandom_seed42..46 / ByColumnRandom (nnz 12 .. 388, coosort_test.cpp:266-352) and the multi-core cases
+    (:563-680, hundreds of thousands of entries), duplicates of whole (row, column) pairs included: with few
+    distinct pairs (4 x 3 over three million entries) the order inside a pair is what P shows.  Sizes either
+    side of the 3840-entry tile of a pass."""
+    rng = np.random.default_rng(nnz + (1 if by_row else 0))
+    run_coosort(osa, gpu_ctx, m, n, rng.integers(0, m, nnz), rng.integers(0, n, nnz), by_row)
+
+
+@pytest.mark.parametrize("by_row", [True, False])
+def test_coosort_signed_indices_custom_perm_and_sorted_input(osa, gpu_ctx, by_row):
+    """Indices are compared as signed integers and need not lie inside the matrix
+    (test/coosort/arch35/coosort_golden.h:29): negative ones, the whole int32 range, a range of one value; P not
+    the identity travels with its entry; input already sorted, and sorted the other way."""
+    rng = np.random.default_rng(5)
+    nnz = 50_000
+    run_coosort(osa, gpu_ctx, 10, 10, rng.integers(-700, 300, nnz), rng.integers(-5, 5, nnz), by_row,
+                perm=rng.integers(-10 ** 9, 10 ** 9, nnz).astype(np.int32))
+    run_coosort(osa, gpu_ctx, 10, 10, rng.integers(-2 ** 31, 2 ** 31 - 1, nnz), rng.integers(-2 ** 31, 2 ** 31 - 1, nnz),
+                by_row)
+    ends = np.array([-2 ** 31, 2 ** 31 - 1, 0, -1, 1, 2 ** 31 - 1, -2 ** 31], np.int64)
+    run_coosort(osa, gpu_ctx, 10, 10, ends, ends[::-1], by_row)
+    run_coosort(osa, gpu_ctx, 10, 10, np.full(nnz, 7), rng.integers(0, 1000, nnz), by_row)     # one row only
+    run_coosort(osa, gpu_ctx, 10, 10, np.full(5000, -3), np.full(5000, 12), by_row)           # one entry repeated
+    r, c = np.divmod(np.arange(nnz), 250)
+    run_coosort(osa, gpu_ctx, 200, 250, r, c, by_row)                                          # sorted by row
+    run_coosort(osa, gpu_ctx, 200, 250, r[::-1], c[::-1], by_row)                              # reversed
+
+
+def test_coosort_then_coo2csr_is_csr2csc(osa, gpu_ctx):
+    """Sorting a matrix's COO triples by column and compressing the column indices gives its CSC form: the same
+    row indices, values (through P) and column offsets as aclsparseCsr2cscEx2's oracle."""
+    m, n = 3000, 2000
+    rowptr, colind, val = random_csr(m, n, 0.01, 4, unsorted=True)
+    nnz = colind.size
+    rows = oracle.csr2coo(rowptr, nnz)
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    d_r, d_c, d_p = dev_i32(rows, dev), dev_i32(colind, dev), dev_i32(np.arange(nnz), dev)
+    size = ctypes.c_size_t(0)
+    assert L.aclsparseXcoosort_bufferSizeExt(handle.h, m, n, nnz, ptr(d_r), ptr(d_c), ctypes.byref(size)) == 0
+    buf = torch.empty(size.value, dtype=torch.uint8, device=dev)
+    assert L.aclsparseXcoosortByColumn(handle.h, m, n, nnz, ptr(d_r), ptr(d_c), ptr(d_p), ptr(buf)) == 0
+    d_ptr = torch.empty(n + 1, dtype=torch.int32, device=dev)
+    assert L.aclsparseXcoo2csr(handle.h, ptr(d_c), nnz, n, ptr(d_ptr), 0) == 0
+    stream.synchronize()
+    colptr, rowind, cval = oracle.csr2csc(m, n, rowptr, colind, val)
+    assert np.array_equal(d_ptr.cpu().numpy(), colptr) and np.array_equal(d_r.cpu().numpy(), rowind)
+    assert np.array_equal(val[d_p.cpu().numpy()].view(np.uint32), cval.view(np.uint32))
 
 
 # ------------------------------------------------------------------ csr2csc

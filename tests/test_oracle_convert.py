@@ -1,4 +1,4 @@
-"""Pins the CPU oracles of the CSR producers (oracle.coo2csr / csr2coo / csrsort / csr2csc):
+"""Pins the CPU oracles of the CSR producers (oracle.coo2csr / csr2coo / csrsort / cscsort / coosort / csr2csc):
 against the reference's own goldens compiled in place (oracle/_ref/libref_convert.so,
 skipped where that is not built), against numpy / scipy formulations of the same
 definitions, and against hand-written small cases.  Everything is bit-exact."""
@@ -99,3 +99,64 @@ def test_round_trips():
     rp2, ci2, v2 = oracle.csr2csc(n, m, colptr, rowind, cval)
     sc, sperm = oracle.csrsort(rowptr, colind, np.arange(colind.size, dtype=np.int32))
     assert np.array_equal(rp2, rowptr) and np.array_equal(ci2, sc) and np.array_equal(v2, val[sperm])
+
+
+# ------------------------------------------------------- cscsort / coosort
+
+def _coo(nnz, lo, hi, seed):
+    rng = np.random.default_rng(seed)
+    return rng.integers(lo, hi, nnz).astype(np.int32), rng.integers(lo, hi, nnz).astype(np.int32)
+
+
+def test_sort_hand_cases():
+    # ByRowBasic / ByColumnBasic of test/coosort/arch35/coosort_test.cpp:233-249
+    rows, cols = [2, 0, 3, 0, 1, 2], [1, 3, 2, 1, 0, 3]
+    r, c, p = oracle.coosort(rows, cols, np.arange(6), True)
+    assert (r.tolist(), c.tolist(), p.tolist()) == ([0, 0, 1, 2, 2, 3], [1, 3, 0, 1, 3, 2], [3, 1, 4, 0, 5, 2])
+    r, c, p = oracle.coosort(rows, cols, np.arange(6), False)
+    assert (r.tolist(), c.tolist(), p.tolist()) == ([1, 0, 2, 3, 0, 2], [0, 1, 1, 2, 3, 3], [4, 3, 0, 2, 1, 5])
+    # equal (row, col) pairs keep their input order; P travels whatever it holds; negative indices sort first
+    r, c, p = oracle.coosort([1, -2, 1, 1, -2], [5, 0, 5, -7, 0], [50, 40, 30, 20, 10], True)
+    assert (r.tolist(), c.tolist(), p.tolist()) == ([-2, -2, 1, 1, 1], [0, 0, -7, 5, 5], [40, 10, 20, 50, 30])
+    # a CSC matrix with columns of 3, 0 and 2 entries, base 1
+    r, p = oracle.cscsort([1, 4, 4, 6], [3, 1, 3, 9, 2], [10, 11, 12, 13, 14], base=1)
+    assert (r.tolist(), p.tolist()) == ([1, 3, 3, 2, 9], [11, 10, 12, 14, 13])
+
+
+@pytest.mark.parametrize("nnz,lo,hi", [(0, 0, 5), (1, 0, 5), (12, 0, 4), (388, 0, 50), (5000, -300, 300),
+                                        (20000, 0, 7), (3000, -2 ** 31, 2 ** 31 - 1)])
+@pytest.mark.parametrize("by_row", [True, False])
+def test_coosort_against_numpy_and_the_reference_golden(nnz, lo, hi, by_row):
+    rows, cols = _coo(nnz, lo, hi, nnz + 7)
+    perm0 = np.arange(nnz, dtype=np.int32)
+    r, c, p = oracle.coosort(rows, cols, perm0, by_row)
+    # numpy: lexsort is stable and takes the LAST key as the primary one
+    order = np.lexsort((cols, rows) if by_row else (rows, cols)).astype(np.int32)
+    assert np.array_equal(p, order) and np.array_equal(r, rows[order]) and np.array_equal(c, cols[order])
+    # P travels with its entry whatever it holds
+    other = (perm0 * 7 - 3).astype(np.int32)
+    assert np.array_equal(oracle.coosort(rows, cols, other, by_row)[2], other[order])
+    R = oracle.ref_convert()
+    if R is not None and hasattr(R, "ref_coosort"):
+        gr, gc, gp = np.zeros(nnz, np.int32), np.zeros(nnz, np.int32), np.zeros(nnz, np.int32)
+        R.ref_coosort(_p(rows), _p(cols), ctypes.c_int32(nnz), ctypes.c_int32(1 if by_row else 0), _p(gr), _p(gc),
+                      _p(gp))
+        assert np.array_equal(gr, r) and np.array_equal(gc, c) and np.array_equal(gp, p)
+
+
+@pytest.mark.parametrize("m,n,density,base", CASES)
+def test_cscsort_against_csrsort_of_the_transpose_and_the_reference_golden(m, n, density, base):
+    # a CSC matrix of m x n is stored exactly like a CSR matrix of n x m
+    colptr, rowind, _ = _csr(n, m, density, m * 7 + n, base, empty_row_prob=0.3, unsorted=True, duplicates=True)
+    nnz = rowind.size
+    perm0 = (np.arange(nnz, dtype=np.int32) * 5 + 1).astype(np.int32)
+    r, p = oracle.cscsort(colptr, rowind, perm0, base)
+    for j in range(n):                                       # every column by numpy's stable sort
+        a, b = colptr[j] - base, colptr[j + 1] - base
+        order = np.argsort(rowind[a:b], kind="stable")
+        assert np.array_equal(r[a:b], rowind[a:b][order]) and np.array_equal(p[a:b], perm0[a:b][order])
+    R = oracle.ref_convert()
+    if R is not None and hasattr(R, "ref_cscsort"):
+        gr, gp = rowind.copy(), perm0.copy()
+        R.ref_cscsort(_p(colptr), ctypes.c_int32(n), ctypes.c_int32(nnz), ctypes.c_int32(base), _p(gr), _p(gp))
+        assert np.array_equal(gr, r) and np.array_equal(gp, p)
