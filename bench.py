@@ -511,7 +511,7 @@ def run_cache_probe(args, osa, wl, torch, dev, stream, handle):
 
 
 def run_convert(args, osa, torch, dev, stream, handle):
-    """The CSR producers (coo2csr, csr2coo, csrsort, csr2csc) on 33.5 M and 21 M entries through the aclsparse
+    """The CSR producers (coo2csr, csr2coo, csrsort, csr2csc, coosort) on 33.5 M and 21 M entries through the aclsparse
     entry points; one JSON line with a time and an algorithmic GB/s per operation."""
     L = osa.lib()
     P = lambda t: ctypes.c_void_p(t.data_ptr())
@@ -564,6 +564,29 @@ def run_convert(args, osa, torch, dev, stream, handle):
             sys.exit("bench.py: csr2csc result fails its checksum / order check")
         res[name + "_csr2csc"] = {"ms": round(t, 4), "gbps": round((16 * nnz + 4 * (m + n)) / t / 1e6, 1),
                                   "workspace_mib": size.value >> 20}
+        # COO triples of the same matrix in a shuffled order, sorted by row (then column): rows, columns and P move,
+        # 12 bytes an entry in and out.  Each timed call sorts a fresh copy (the copy is part of the timed call).
+        shuffle = torch.randperm(nnz, device=dev, generator=g)
+        r0 = torch.repeat_interleave(torch.arange(m, device=dev, dtype=torch.int32), per)[shuffle].contiguous()
+        c0 = col[shuffle].contiguous()
+        p0 = torch.arange(nnz, dtype=torch.int32, device=dev)
+        r1, c1, p1 = torch.empty_like(r0), torch.empty_like(c0), torch.empty_like(p0)
+        L.aclsparseXcoosort_bufferSizeExt(handle.h, m, n, nnz, P(r0), P(c0), ctypes.byref(size))
+        buf = torch.empty(max(16, size.value), dtype=torch.uint8, device=dev)
+
+        def coosort():
+            r1.copy_(r0), c1.copy_(c0), p1.copy_(p0)
+            if L.aclsparseXcoosortByRow(handle.h, m, n, nnz, P(r1), P(c1), P(p1), P(buf)) != 0:
+                sys.exit("bench.py: aclsparseXcoosortByRow failed")
+
+        copies = timed(lambda: (r1.copy_(r0), c1.copy_(c0), p1.copy_(p0)))
+        t = timed(coosort) - copies
+        key = r1.long() * n + c1.long()
+        if not torch.all(key[1:] >= key[:-1]) or not torch.equal(r0[p1.long()], r1) or not torch.equal(c0[p1.long()], c1):
+            sys.exit("bench.py: coosort result is not sorted or P does not lead back to the input")
+        res[name + "_coosort_by_row"] = {"ms": round(t, 4), "gbps": round(24 * nnz / t / 1e6, 1),
+                                         "workspace_mib": size.value >> 20}
+        del shuffle, r0, c0, p0, r1, c1, p1, key, buf
         log(name, json.dumps({k: v for k, v in res.items() if k.startswith(name)}))
     return res
 
