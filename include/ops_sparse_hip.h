@@ -90,9 +90,10 @@ typedef struct OpsparseSpmvPlan {
     int32_t tileRowNnz;    /* STREAM_ROWS: the row length the tiles are sized for (0: maxRowNnz) */
     int32_t longRowsBeside;/* STREAM_ROWS: a few rows are longer than that: the tiles skip rows of more than 64
                               entries and a second kernel sums those, a workgroup per row */
-    int32_t liveValues;    /* BLOCKED_GATHER: every launch first copies the caller's csrValues, as they are then, into
-                              the layout (one more linear pass over the entries): nothing goes stale when values
-                              change in place or the values pointer is replaced */
+    int32_t liveValues;    /* BLOCKED_GATHER: the layout holds no values; every launch takes the caller's csrValues as
+                              they are then: nothing goes stale when values change in place or the values pointer
+                              is replaced (1: 32-bit positions of the entries, 2: 16-bit ones relative to their
+                              row block, which the analysis chooses where every block is shorter than 65535) */
     int32_t numLongRows;   /* BLOCKED_GATHER: rows kept out of the re-stored layout: phase 1 sums them from the caller's
                               colInd / csrValues, panel by panel, with the panel's x in LDS */
     int64_t rows;

@@ -491,20 +491,80 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedLiveTablesKernel(const i
     }
 }
 
-// Live values.  The entries of a row block are one contiguous piece [e0, e1) of the caller's arrays and one
-// contiguous piece of the block order.  The workgroup that owns the block reads the former (values and their
-// block-order positions, both linear) and keeps what falls into the window [w0, w0 + span) of the latter in LDS:
-// win[position - w0] = value as it is at this call.  Entries of long rows carry position -1.  A block of more than
-// kRefreshSpan positions reads its entries once per window.  [e0, e1) here is a piece of the block's entries
-// between two long rows (whose own entries have no position and are skipped).
-__device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, const int32_t *__restrict__ dstOfPos,
-                                               int32_t e0, int32_t e1, int32_t w0, uint32_t span, float *win, int tid)
+// header[3] = positions of the longest row block (zero before).
+__global__ __launch_bounds__(kBlockThreads) void BlockedMaxPositionsKernel(const int32_t *__restrict__ dstStart,
+                                                                           int32_t P, int32_t B,
+                                                                           int32_t *__restrict__ header)
 {
+    const int32_t b = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
+    if (b < B) {
+        atomicMax(header + 3, dstStart[static_cast<int64_t>(b + 1) * P] - dstStart[static_cast<int64_t>(b) * P]);
+    }
+}
+
+constexpr uint32_t kNoPosition16 = 0xffffu;  // short position of an entry that has none (a long row's)
+constexpr int32_t kLiveShortPositions = 2;   // plan.liveValues of a layout whose positions were re-stored that way
+
+// Live values, every row block shorter than 65535 positions.  The block-order position of entry i of block b is
+// re-stored as 16 bits relative to the block's first position, at ((uint16_t *)(dstOfPos + e0))[i - e0] with e0 the
+// block's first entry: the short positions of a block lie in the front half of the bytes its 32-bit ones had, so
+// a workgroup a block can convert in place, a piece at a time, reading a piece before it writes it (what it writes
+// lies below what it has not read yet).
+__global__ __launch_bounds__(kBlkThreads) void BlockedShortPositionsKernel(const int32_t *__restrict__ blockEntry,
+                                                                          const int32_t *__restrict__ dstStart,
+                                                                          int32_t P, int32_t *dstOfPos)
+{
+    constexpr int kPer = 8;
+    const int64_t b = blockIdx.x;
+    const int32_t e0 = blockEntry[b], e1 = blockEntry[b + 1], dBeg = dstStart[b * P];
+    auto *out = reinterpret_cast<uint16_t *>(dstOfPos + e0);
+    for (int32_t c0 = e0; c0 < e1; c0 += kBlkThreads * kPer) {
+        int32_t v[kPer];
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) {
+            const int32_t i = c0 + u * kBlkThreads + static_cast<int32_t>(threadIdx.x);
+            v[u] = i < e1 ? dstOfPos[i] : -1;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < kPer; ++u) {
+            const int32_t i = c0 + u * kBlkThreads + static_cast<int32_t>(threadIdx.x);
+            if (i < e1) {
+                out[i - e0] = static_cast<uint16_t>(v[u] < 0 ? kNoPosition16 : static_cast<uint32_t>(v[u] - dBeg));
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// Live values.  The entries of a row block are one contiguous piece of the caller's arrays and one contiguous
+// piece of the block order.  The workgroup that owns the block reads the former (values and their block-order
+// positions, both linear) and keeps what falls into the window [w0, w0 + span) of the latter in LDS:
+// win[position - w0] = value as it is at this call.  Entries of long rows have no position (-1, or kNoPosition16).
+// A block of more than kRefreshSpan positions reads its entries once per window.  [e0, e1) here is a piece of the
+// block's entries between two long rows (whose own entries are skipped); Short: the positions are the 16-bit ones
+// of BlockedShortPositionsKernel, blockE0 and dBeg the block's first entry and first position.
+template <bool Short>
+__device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, const int32_t *__restrict__ dstOfPos,
+                                               int32_t e0, int32_t e1, int32_t w0, uint32_t span, float *win, int tid,
+                                               int32_t blockE0, int32_t dBeg)
+{
+    typedef unsigned short Ushort4U __attribute__((ext_vector_type(4), aligned(2)));
+    const uint16_t *pos16 = reinterpret_cast<const uint16_t *>(dstOfPos + blockE0) - blockE0;  // indexed by entry
+    const uint32_t shift = static_cast<uint32_t>(dBeg - w0);
+    // window-relative position of entry i, or a value >= span
+    auto place = [&](int32_t i) {
+        if (Short) {
+            const uint32_t d = pos16[i];
+            return d == kNoPosition16 ? 0xffffffffu : d + shift;
+        }
+        return static_cast<uint32_t>(dstOfPos[i] - w0);
+    };
     // aligned groups of four entries as 16-byte loads, the ragged ends one by one
     const int32_t g0 = (e0 + 3) & ~3, g1 = e1 & ~3;
     if (g0 >= g1) {
         for (int32_t i = e0 + tid; i < e1; i += kBlkThreads) {
-            const uint32_t at = static_cast<uint32_t>(dstOfPos[i] - w0);
+            const uint32_t at = place(i);
             if (at < span) {
                 win[at] = vals[i];
             }
@@ -514,7 +574,7 @@ __device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, c
     if (tid < 8) {
         const int32_t i = tid < 4 ? e0 + tid : g1 + (tid - 4);
         if ((tid < 4 && i < g0) || (tid >= 4 && i < e1)) {
-            const uint32_t at = static_cast<uint32_t>(dstOfPos[i] - w0);
+            const uint32_t at = place(i);
             if (at < span) {
                 win[at] = vals[i];
             }
@@ -525,12 +585,17 @@ __device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, c
     constexpr int kRefreshBatch = 6;  // (a block of kLiveWindow entries in one turn)
     for (int32_t i0 = g0 + tid * 4; i0 < g1; i0 += kBlkThreads * 4 * kRefreshBatch) {
         Int4U d[kRefreshBatch];
+        Ushort4U d16[kRefreshBatch];
         Float4U v[kRefreshBatch];
 #pragma unroll
         for (int u = 0; u < kRefreshBatch; ++u) {
             int32_t i = i0 + u * kBlkThreads * 4;
             i = i < g1 ? i : g1 - 4;
-            d[u] = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(dstOfPos + i));
+            if (Short) {
+                d16[u] = __builtin_nontemporal_load(reinterpret_cast<const Ushort4U *>(pos16 + i));
+            } else {
+                d[u] = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(dstOfPos + i));
+            }
             if (vecVals) {
                 v[u] = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(vals + i));
             } else {
@@ -540,8 +605,19 @@ __device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, c
 #pragma unroll
         for (int u = 0; u < kRefreshBatch; ++u) {
             // (a clamped group writes the same values to the same places again)
-            const uint32_t a0 = static_cast<uint32_t>(d[u].x - w0), a1 = static_cast<uint32_t>(d[u].y - w0);
-            const uint32_t a2 = static_cast<uint32_t>(d[u].z - w0), a3 = static_cast<uint32_t>(d[u].w - w0);
+            uint32_t a0, a1, a2, a3;
+            if (Short) {
+                const uint32_t q[4] = {d16[u].x, d16[u].y, d16[u].z, d16[u].w};
+                a0 = q[0] == kNoPosition16 ? 0xffffffffu : q[0] + shift;
+                a1 = q[1] == kNoPosition16 ? 0xffffffffu : q[1] + shift;
+                a2 = q[2] == kNoPosition16 ? 0xffffffffu : q[2] + shift;
+                a3 = q[3] == kNoPosition16 ? 0xffffffffu : q[3] + shift;
+            } else {
+                a0 = static_cast<uint32_t>(d[u].x - w0);
+                a1 = static_cast<uint32_t>(d[u].y - w0);
+                a2 = static_cast<uint32_t>(d[u].z - w0);
+                a3 = static_cast<uint32_t>(d[u].w - w0);
+            }
             if (a0 < span) win[a0] = v[u].x;
             if (a1 < span) win[a1] = v[u].y;
             if (a2 < span) win[a2] = v[u].z;
@@ -878,7 +954,7 @@ constexpr int kRedThreads = kBlkThreads, kRedWaves = kRedThreads / kWave;
 // by window of kRefreshSpan positions (partDesc[partStart[block]] ..: entries, positions); the values of a window
 // are first collected in LDS from the caller's array, and the stream takes them from there.  Padding positions of
 // a window hold whatever LDS held: their products are formed and dropped.
-template <bool Live>
+template <bool Live, bool Short>
 __global__ __launch_bounds__(kRedThreads) void SpmvBlockReduceKernel(
     const float *__restrict__ valD, const float *__restrict__ xg, const uint16_t *__restrict__ rowLocal,
     const int32_t *__restrict__ dstStart, const int32_t *__restrict__ srcStartT, int32_t P,
@@ -920,10 +996,11 @@ __global__ __launch_bounds__(kRedThreads) void SpmvBlockReduceKernel(
         // the block's entries without those of its long rows
         int32_t cur = e0;
         for (int32_t l = l0; l < l1; ++l) {
-            FillLiveWindow(vals, dstOfPos, cur, longSpan[2 * l], w0, static_cast<uint32_t>(w1 - w0), win, tid);
+            FillLiveWindow<Short>(vals, dstOfPos, cur, longSpan[2 * l], w0, static_cast<uint32_t>(w1 - w0), win, tid, e0,
+                                  dBeg);
             cur = longSpan[2 * l + 1];
         }
-        FillLiveWindow(vals, dstOfPos, cur, e1, w0, static_cast<uint32_t>(w1 - w0), win, tid);
+        FillLiveWindow<Short>(vals, dstOfPos, cur, e1, w0, static_cast<uint32_t>(w1 - w0), win, tid, e0, dBeg);
     };
     if (Live && dBeg < dEnd) {
         fillWindow(dBeg, dEnd - dBeg > spanMax ? dBeg + spanMax : dEnd);
@@ -1274,21 +1351,26 @@ int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
                            header, ints(l.longChunkOff), a.colInd, static_cast<const float *>(a.vals), a.nnz, l.P,
                            l.maxLong, rowLocal + LongRowOfShift(l), longPartial);
     }
-    if (plan.liveValues != 0) {
-        hipLaunchKernelGGL(SpmvBlockReduceKernel<true>, dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads), 0, a.stream,
-                           static_cast<const float *>(nullptr), xg, rowLocal, ints(l.dstStartOff), ints(l.srcStartTOff), l.P,
-                           ints(l.orderOff), ints(l.blockRowOff), static_cast<float *>(a.y),
-                           static_cast<const float *>(a.yIn), a.alpha, a.beta, longRows ? ints(l.longFirstOff) : nullptr,
-                           ints(l.longRowsOff), longPartial, static_cast<const float *>(a.vals), ints(l.dstOfPosOff),
-                           ints(l.blockEntryOff), ints(l.longSpanOff));
+#define OPSPARSE_BLOCK_REDUCE_LIVE(SHORT)                                                                           \
+    hipLaunchKernelGGL((SpmvBlockReduceKernel<true, SHORT>), dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads), 0,    \
+                       a.stream, static_cast<const float *>(nullptr), xg, rowLocal, ints(l.dstStartOff),               \
+                       ints(l.srcStartTOff), l.P, ints(l.orderOff), ints(l.blockRowOff), static_cast<float *>(a.y),     \
+                       static_cast<const float *>(a.yIn), a.alpha, a.beta, longRows ? ints(l.longFirstOff) : nullptr,   \
+                       ints(l.longRowsOff), longPartial, static_cast<const float *>(a.vals), ints(l.dstOfPosOff),       \
+                       ints(l.blockEntryOff), ints(l.longSpanOff))
+    if (plan.liveValues == kLiveShortPositions) {
+        OPSPARSE_BLOCK_REDUCE_LIVE(true);
+    } else if (plan.liveValues != 0) {
+        OPSPARSE_BLOCK_REDUCE_LIVE(false);
     } else {
-        hipLaunchKernelGGL(SpmvBlockReduceKernel<false>, dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads), 0, a.stream,
-                           valD, xg, rowLocal, ints(l.dstStartOff), ints(l.srcStartTOff), l.P, ints(l.orderOff),
+        hipLaunchKernelGGL((SpmvBlockReduceKernel<false, false>), dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads), 0,
+                           a.stream, valD, xg, rowLocal, ints(l.dstStartOff), ints(l.srcStartTOff), l.P, ints(l.orderOff),
                            ints(l.blockRowOff), static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha,
                            a.beta, longRows ? ints(l.longFirstOff) : nullptr, ints(l.longRowsOff), longPartial,
                            static_cast<const float *>(nullptr), static_cast<const int32_t *>(nullptr),
                            static_cast<const int32_t *>(nullptr), static_cast<const int32_t *>(nullptr));
     }
+#undef OPSPARSE_BLOCK_REDUCE_LIVE
     return CheckLaunch();
 }
 
@@ -1342,7 +1424,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     auto *rowLocal = reinterpret_cast<uint16_t *>(base + l.rowLocalOff);
     auto *valD = reinterpret_cast<float *>(base + l.valOff);
 
-    LaunchFillI32(status, 3, 0, s);  // status, number of long rows, their entries
+    LaunchFillI32(status, 4, 0, s);  // status, number of long rows, their entries, positions of the longest block
     LaunchExpandRows(rowOffsets, rows, nnz, 0, rowOfPos, s);
     const int32_t *pos = nullptr, *outOffsets = rowOffsets;
     int32_t *chunkKey = nullptr, *rowOfSrc = nullptr;
@@ -1477,6 +1559,25 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
                            s, rowOffsets, blockRow, l.B, ints(l.longRowsOff), longBefore != nullptr ? status : nullptr,
                            ints(l.blockEntryOff), ints(l.longSpanOff));
     }
+    int32_t liveKind = live ? 1 : 0;
+    if (live) {
+        // Row blocks of fewer than 65535 positions, all of them (the rule unless a row that cannot go the long rows'
+        // way is longer than that): 16-bit positions relative to the block, 2 bytes an entry less at every call.
+        hipLaunchKernelGGL(BlockedMaxPositionsKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
+                           s, dstStart, l.P, l.B, status);
+        int32_t longest = 0;
+        if (hipMemcpyAsync(&longest, status + 3, sizeof(longest), hipMemcpyDeviceToHost, s) != hipSuccess ||
+            hipStreamSynchronize(s) != hipSuccess) {
+            (void)hipGetLastError();
+            return OPSPARSE_E_LAUNCH;
+        }
+        static const bool noShort = std::getenv("OPS_SPARSE_BLOCKED_NO_SHORT_POSITIONS") != nullptr;
+        if (!noShort && longest < static_cast<int32_t>(kNoPosition16)) {
+            hipLaunchKernelGGL(BlockedShortPositionsKernel, dim3(static_cast<uint32_t>(l.B)), dim3(kBlkThreads), 0, s,
+                               ints(l.blockEntryOff), dstStart, l.P, ints(l.dstOfPosOff));
+            liveKind = kLiveShortPositions;
+        }
+    }
     if (CheckLaunch() != OPSPARSE_OK) {
         return OPSPARSE_E_LAUNCH;
     }
@@ -1487,7 +1588,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     p.numRowBlocks = l.B;
     p.entryWindow = l.window;
     p.transposed = transposed ? 1 : 0;
-    p.liveValues = live ? 1 : 0;
+    p.liveValues = liveKind;
     p.numLongRows = head[1];
     p.rows = rows;
     p.nnz = nnz;

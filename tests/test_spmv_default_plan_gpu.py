@@ -102,7 +102,7 @@ def test_default_plan_sums_long_rows_from_the_callers_arrays(osa, gpu_ctx):
     assert L.opsparse_spmv_csr_blocked_analyse(pv(d[0]), pv(d[1]), pv(d[2]), rows, cols, nnz,
                                                osa.OPSPARSE_BLOCKED_LIVE_VALUES, pv(ws), need, ctypes.byref(plan),
                                                ctypes.c_void_p(stream.cuda_stream)) == 0
-    assert plan.liveValues == 1 and plan.numLongRows == 6    # 9000, 4096, 40 000, 20 000, 120 000, 5000
+    assert plan.liveValues == 2 and plan.numLongRows == 6     # 9000, 4096, 40 000, 20 000, 120 000, 5000; short positions
     del ws
     A, X = osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3])
     d_y = to_dev(y0, dev)
@@ -124,6 +124,42 @@ def test_default_plan_sums_long_rows_from_the_callers_arrays(osa, gpu_ctx):
     x2 = np.random.default_rng(12).uniform(-2, 2, cols).astype(np.float32)
     d[3].copy_(torch.from_numpy(x2))
     check(val2, x2, 2.0, 0.0)
+
+
+def test_default_plan_keeps_32_bit_positions_for_a_block_of_70000_entries(osa, gpu_ctx):
+    """The positions of the entries in their row block are kept in 16 bits where every block is shorter than 65535
+    positions.  A row of 70 000 entries whose columns do not ascend cannot go the long rows' way, makes a block of
+    several windows, and the layout keeps its 32-bit positions (plan.liveValues == 1); same product either way."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = 300_000, 1_400_000
+    rng = np.random.default_rng(31)
+    lengths = rng.integers(0, 20, rows)
+    lengths[123_456] = 70_000
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)      # unsorted everywhere
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    x, y0 = rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    nnz = colind.size
+    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    plan = osa.OpsparseSpmvPlan()
+    pv = lambda t: ctypes.c_void_p(t.data_ptr())
+    assert L.opsparse_spmv_csr_blocked_analyse(pv(d[0]), pv(d[1]), pv(d[2]), rows, cols, nnz,
+                                               osa.OPSPARSE_BLOCKED_LIVE_VALUES, pv(ws), need, ctypes.byref(plan),
+                                               ctypes.c_void_p(stream.cuda_stream)) == 0
+    assert plan.liveValues == 1 and plan.numLongRows == 0
+    del ws
+    d_y = to_dev(y0, dev)
+    op = osa.SpmvOp(handle, osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3]), osa.DnVec(d_y))
+    for values, alpha, beta in ((val, 1.0, 0.0), ((val * np.float32(-2.0)).astype(np.float32), 0.5, 1.5)):
+        d[2].copy_(torch.from_numpy(values))
+        d_y.copy_(torch.from_numpy(y0))
+        op(alpha, beta)
+        stream.synchronize()
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, values, x, y0, alpha, beta)
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
 
 
 def test_default_plan_of_a_banded_matrix_stays_row_wise(osa, gpu_ctx, workloads):
