@@ -115,3 +115,22 @@ def test_random_case(osa, gpu_ctx, seed):
             gold = oracle.spmm_f64(rows, n, rowptr, colind, vh, B, ldb, C0, ldc, alpha, beta, b_row_major=True,
                                    trans_b=False, c_row_major=True)
             assert oracle.max_rel_err(got, gold) <= 1e-5
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_conversion_case(osa, gpu_ctx, seed):
+    """The CSR producers on the same random matrices (columns unsorted, with repeats): csrsort, the same arrays read
+    as a CSC matrix through cscsort, the COO triples in a shuffled order through coosort by row and by column, and
+    csr2csc; every output bit for bit against the oracle."""
+    from test_convert_gpu import run_coosort, run_cscsort, run_csr2csc, run_csrsort
+    rng = np.random.default_rng(19_000 + seed)
+    rows, cols, rowptr, colind, val = _matrix(rng)
+    base = int(rng.integers(0, 2))
+    perm = rng.integers(-10 ** 6, 10 ** 6, colind.size).astype(np.int32) if seed % 2 else None
+    run_csrsort(osa, gpu_ctx, rows, cols, rowptr + base, colind + base, base=base, perm=perm)
+    run_cscsort(osa, gpu_ctx, cols, rows, rowptr + base, colind + base, base=base, perm=perm)
+    order = rng.permutation(colind.size)
+    coo_rows = oracle.csr2coo(rowptr, colind.size)[order]
+    run_coosort(osa, gpu_ctx, rows, cols, coo_rows, colind[order], bool(seed % 2), perm=perm)
+    run_coosort(osa, gpu_ctx, rows, cols, coo_rows - 3, colind[order] - 40_000, not bool(seed % 2))
+    run_csr2csc(osa, gpu_ctx, rows, cols, rowptr + base, colind + base, val, np.float32, True, base)
