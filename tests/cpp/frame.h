@@ -37,6 +37,8 @@ void oracle_csr2coo(const int32_t *rowPtr, int64_t m, int64_t nnz, int32_t base,
 void oracle_csr2csc(int64_t m, int64_t n, int64_t nnz, int32_t base, const int32_t *rowPtr, const int32_t *colInd,
                     const void *val, int32_t valBytes, int32_t *colPtr, int32_t *rowInd, void *cscVal);
 void oracle_csrsort(const int32_t *rowPtr, int64_t m, int32_t base, int32_t *colInd, int32_t *perm);
+void oracle_cscsort(const int32_t *colPtr, int64_t n, int32_t base, int32_t *rowInd, int32_t *perm);
+void oracle_coosort(int64_t nnz, int32_t byRow, int32_t *rows, int32_t *cols, int32_t *perm);
 }
 
 namespace frame {

@@ -230,6 +230,123 @@ bool CsrsortCase(const frame::Stream &stream, const frame::Handle &handle, const
     return ok;
 }
 
+// The csrsort cases read as CSC matrices (test/cscsort/arch35/cscsort_test.cpp:245-530 builds the same shapes with
+// rows and columns exchanged): c.m columns, row indices below c.n.  The buffer is aligned to 128 bytes, as the
+// reference demands of its callers; one that is not must be refused.
+bool CscsortCase(const frame::Stream &stream, const frame::Handle &handle, const SortCase &c)
+{
+    const int nnz = static_cast<int>(c.colInd.size());
+    const int rows = c.n, cols = c.m;
+    aclsparseMatDescr_t descr = nullptr;
+    Check(aclsparseCreateMatDescr(&descr), "aclsparseCreateMatDescr");
+    aclsparseSetMatIndexBase(descr, static_cast<aclsparseIndexBase_t>(c.base));
+    bool ok = false;
+    if (nnz == 0) {
+        size_t bytes = 42;
+        Check(aclsparseXcscsort_bufferSizeExt(handle.get(), rows, cols, 0, c.rowPtr.data(), nullptr, &bytes),
+              "aclsparseXcscsort_bufferSizeExt");
+        Check(aclsparseXcscsort(handle.get(), rows, cols, 0, descr, c.rowPtr.data(), nullptr, nullptr, nullptr),
+              "aclsparseXcscsort");
+        ok = bytes == 0;
+    } else {
+        std::vector<int32_t> perm = c.perm;
+        if (perm.empty()) {
+            perm.resize(static_cast<size_t>(nnz));
+            for (int i = 0; i < nnz; ++i) {
+                perm[i] = 3 * i + 1;  // NonIdentityP
+            }
+        }
+        std::vector<int32_t> goldRow = c.colInd, goldPerm = perm;
+        oracle_cscsort(c.rowPtr.data(), cols, c.base, goldRow.data(), goldPerm.data());
+        frame::DeviceArray<int32_t> dPtr(c.rowPtr), dRow(c.colInd), dPerm(perm);
+        size_t bytes = 0;
+        Check(aclsparseXcscsort_bufferSizeExt(handle.get(), rows, cols, nnz, dPtr.get(), dRow.get(), &bytes),
+              "aclsparseXcscsort_bufferSizeExt");
+        frame::DeviceArray<unsigned char> buffer(bytes + 256);
+        auto *aligned = reinterpret_cast<unsigned char *>((reinterpret_cast<uintptr_t>(buffer.get()) + 127) / 128 * 128);
+        const bool refused = aclsparseXcscsort(handle.get(), rows, cols, nnz, descr, dPtr.get(), dRow.get(), dPerm.get(),
+                                               aligned + 8) == ACL_SPARSE_STATUS_INVALID_VALUE;
+        Check(aclsparseXcscsort(handle.get(), rows, cols, nnz, descr, dPtr.get(), dRow.get(), dPerm.get(), aligned),
+              "aclsparseXcscsort");
+        stream.sync();
+        ok = refused && bytes > 0 && dPtr.download() == c.rowPtr && dRow.download() == goldRow &&
+             dPerm.download() == goldPerm;
+    }
+    (void)aclsparseDestroyMatDescr(descr);
+    return ok;
+}
+
+struct CooCase {
+    std::string name;
+    int m, n;
+    bool byRow;
+    std::vector<int32_t> rows, cols;
+};
+
+// Inputs of test/coosort/arch35/coosort_test.cpp: the hand-written cases (:233-262), random matrices of 12 .. 388
+// entries (:266-352), the sizes of its multi-core cases (:563-680), and indices outside the matrix, which the
+// sort compares as signed integers (coosort_golden.h:29).
+std::vector<CooCase> CooCases()
+{
+    std::vector<CooCase> c;
+    for (const bool byRow : {true, false}) {
+        c.push_back({byRow ? "ByRowBasic" : "ByColumnBasic", 4, 4, byRow, {2, 0, 3, 0, 1, 2}, {1, 3, 2, 1, 0, 3}});
+        c.push_back({byRow ? "ByRowStableDuplicateKey" : "ByColumnStableDuplicateKey", 3, 5, byRow, {0, 0, 0, 1, 1, 2},
+                     {4, 1, 3, 2, 0, 9}});
+        c.push_back({byRow ? "ByRowNnzZero" : "ByColumnNnzZero", 4, 4, byRow, {}, {}});
+        int seed = 42;
+        for (const int nnz : {12, 49, 103, 215, 388, 4097, 70000, 300001}) {
+            std::mt19937 rng(static_cast<uint32_t>(seed++));
+            const int m = nnz < 1000 ? 64 : 5000, n = nnz < 1000 ? 48 : 3000;
+            CooCase k{(byRow ? "ByRowRandom_" : "ByColumnRandom_") + std::to_string(nnz), m, n, byRow, {}, {}};
+            for (int i = 0; i < nnz; ++i) {
+                k.rows.push_back(static_cast<int32_t>(rng() % static_cast<uint32_t>(m)));
+                k.cols.push_back(static_cast<int32_t>(rng() % static_cast<uint32_t>(n)));
+            }
+            c.push_back(k);
+        }
+        CooCase k{byRow ? "ByRowSignedIndices" : "ByColumnSignedIndices", 10, 10, byRow, {}, {}};
+        std::mt19937 rng(7);
+        for (int i = 0; i < 20000; ++i) {
+            k.rows.push_back(static_cast<int32_t>(rng()));  // the whole int32 range
+            k.cols.push_back(static_cast<int32_t>(rng() % 9U) - 4);
+        }
+        c.push_back(k);
+    }
+    return c;
+}
+
+// RunSortAndVerify of the reference (coosort_test.cpp:141-228): P preset to 0 .. nnz-1, bufferSizeExt must ask for
+// a buffer when there is something to sort, rows, columns and P compared exactly.
+bool CoosortCase(const frame::Stream &stream, const frame::Handle &handle, const CooCase &c)
+{
+    const int nnz = static_cast<int>(c.rows.size());
+    size_t bytes = 42;
+    if (nnz == 0) {
+        Check(aclsparseXcoosort_bufferSizeExt(handle.get(), c.m, c.n, 0, nullptr, nullptr, &bytes),
+              "aclsparseXcoosort_bufferSizeExt");
+        Check((c.byRow ? aclsparseXcoosortByRow : aclsparseXcoosortByColumn)(handle.get(), c.m, c.n, 0, nullptr, nullptr,
+                                                                             nullptr, nullptr), "aclsparseXcoosort");
+        return bytes == 0;
+    }
+    std::vector<int32_t> perm(static_cast<size_t>(nnz));
+    for (int i = 0; i < nnz; ++i) {
+        perm[i] = i;
+    }
+    std::vector<int32_t> goldRows = c.rows, goldCols = c.cols, goldPerm = perm;
+    oracle_coosort(nnz, c.byRow ? 1 : 0, goldRows.data(), goldCols.data(), goldPerm.data());
+    frame::DeviceArray<int32_t> dRows(c.rows), dCols(c.cols), dPerm(perm);
+    Check(aclsparseXcoosort_bufferSizeExt(handle.get(), c.m, c.n, nnz, dRows.get(), dCols.get(), &bytes),
+          "aclsparseXcoosort_bufferSizeExt");
+    frame::DeviceArray<unsigned char> buffer(bytes);
+    Check((c.byRow ? aclsparseXcoosortByRow : aclsparseXcoosortByColumn)(handle.get(), c.m, c.n, nnz, dRows.get(),
+                                                                         dCols.get(), dPerm.get(), buffer.get()),
+          "aclsparseXcoosort");
+    stream.sync();
+    return bytes >= static_cast<size_t>(nnz) * 12 && dRows.download() == goldRows && dCols.download() == goldCols &&
+           dPerm.download() == goldPerm;
+}
+
 bool Coo2CsrCase(const frame::Stream &stream, const frame::Handle &handle, const Row &r)
 {
     const int32_t base = static_cast<int32_t>(I(r, "idx_base"));
@@ -317,7 +434,7 @@ bool Csr2CscCase(const frame::Stream &stream, const frame::Handle &handle, const
 int main(int argc, char **argv)
 {
     if (argc < 2) {
-        std::fprintf(stderr, "usage: %s <directory with the csv case tables> [spmv_op|coo2csr|csr2coo|csr2csc|csrsort ...]\n",
+        std::fprintf(stderr, "usage: %s <directory with the csv case tables> [spmv_op|coo2csr|csr2coo|csr2csc|csrsort|cscsort|coosort ...]\n",
                      argv[0]);
         return 2;
     }
@@ -327,19 +444,35 @@ int main(int argc, char **argv)
         tables.push_back(argv[i]);
     }
     if (tables.empty()) {
-        tables = {"spmv_op", "coo2csr", "csr2coo", "csr2csc", "csrsort"};
+        tables = {"spmv_op", "coo2csr", "csr2coo", "csr2csc", "csrsort", "cscsort", "coosort"};
     }
     int failed = 0, total = 0;
     try {
         frame::Stream stream;
         frame::Handle handle(stream);
         for (const std::string &t : tables) {
-            if (t == "csrsort") {
+            if (t == "coosort") {
+                for (const CooCase &c : CooCases()) {
+                    bool ok = false;
+                    std::string error;
+                    try {
+                        ok = CoosortCase(stream, handle, c);
+                    } catch (const std::exception &e) {
+                        error = e.what();
+                    }
+                    ++total;
+                    failed += ok ? 0 : 1;
+                    std::printf("[%s] %-32s %s %s\n", t.c_str(), c.name.c_str(), ok ? "PASS" : "FAIL", error.c_str());
+                    std::fflush(stdout);
+                }
+                continue;
+            }
+            if (t == "csrsort" || t == "cscsort") {
                 for (const SortCase &c : SortCases()) {
                     bool ok = false;
                     std::string error;
                     try {
-                        ok = CsrsortCase(stream, handle, c);
+                        ok = t == "csrsort" ? CsrsortCase(stream, handle, c) : CscsortCase(stream, handle, c);
                     } catch (const std::exception &e) {
                         error = e.what();
                     }

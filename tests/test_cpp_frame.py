@@ -30,7 +30,7 @@ def test_frame_rules_and_typed_loader_on_the_cpu():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("table", ["spmv_op", "coo2csr", "csr2coo", "csr2csc", "csrsort"])
+@pytest.mark.parametrize("table", ["spmv_op", "coo2csr", "csr2coo", "csr2csc", "csrsort", "cscsort", "coosort"])
 def test_case_tables_from_cpp(gpu_ctx, table):
     assert os.path.exists(RUNNER), "tests/cpp/bin/run_case_tables is not built: run `make -C tests/cpp`"
     proc = subprocess.run([RUNNER, os.path.join(ROOT, "tests", "golden"), table], capture_output=True, text=True,
