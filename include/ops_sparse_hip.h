@@ -96,6 +96,9 @@ typedef struct OpsparseSpmvPlan {
                               row block, which the analysis chooses where every block is shorter than 65535) */
     int32_t numLongRows;   /* BLOCKED_GATHER: rows kept out of the re-stored layout: phase 1 sums them from the caller's
                               colInd / csrValues, panel by panel, with the panel's x in LDS */
+    int32_t numDeferredLongRows; /* BLOCKED_GATHER: those of them that sit more than 64 to a row block: a third kernel,
+                              a wavefront a row, adds their partial sums up instead of the block's workgroup */
+    int32_t reserved;
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */

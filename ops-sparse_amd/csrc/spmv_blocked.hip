@@ -91,6 +91,9 @@ constexpr int64_t kLongMinRow = 4096;             // and at least this many in a
 constexpr int64_t kLongChunkMeanFrozen = 4;
 constexpr int64_t kLongMinRowFrozen = 1024;
 constexpr int kLongLanes = 16;        // lanes that sum one (long row, panel) piece in phase 1
+constexpr int32_t kInBlockLongRows = 64;          // long rows a row block's own workgroup adds up at most
+// acc[] of a long row whose sum is left to SpmvLongRowSumKernel: a NaN that no arithmetic on fp32 inputs yields
+constexpr long long kDeferredRowMark = 0x7ff8dead0000beefLL;
 constexpr int kLongTile = 3072;                   // long rows whose piece bounds a phase-1 workgroup stages in LDS at a time
 
 typedef float Float4 __attribute__((ext_vector_type(4)));
@@ -406,6 +409,26 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedLongFirstKernel(const in
     if (b <= B) {
         const int32_t row = blockRow[b];
         longFirst[b] = row > 0 ? longBefore[row - 1] : 0;
+    }
+}
+
+// longDeferred[l] = 1 for the long rows of a row block that holds more than kInBlockLongRows of them, else 0;
+// header[4] (zero before) = their number.
+__global__ __launch_bounds__(kBlockThreads) void BlockedLongDeferKernel(const int32_t *__restrict__ longFirst, int32_t B,
+                                                                        int32_t *__restrict__ longDeferred,
+                                                                        int32_t *__restrict__ header)
+{
+    const int32_t b = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
+    if (b >= B) {
+        return;
+    }
+    const int32_t l0 = longFirst[b], l1 = longFirst[b + 1];
+    const int32_t defer = l1 - l0 > kInBlockLongRows ? 1 : 0;
+    for (int32_t l = l0; l < l1; ++l) {
+        longDeferred[l] = defer;
+    }
+    if (defer != 0) {
+        atomicAdd(header + 4, l1 - l0);
     }
 }
 
@@ -726,13 +749,15 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint1
         return;
     }
     if constexpr (LongSorted) {
-        if (part != 0) {
-            return;  // (a partial sum has one writer: the panel's first workgroup)
-        }
+        // Tiles of long rows, shared out among the panel's workgroups where it has several (a partial sum has one
+        // writer); as many tiles as workgroups at least.
         double *accL = reinterpret_cast<double *>(tileBuf);
         const int32_t *tab = longChunk + p * (maxLong + 1);
-        for (int32_t t0 = 0; t0 < numLong; t0 += kLongTile) {
-            const int32_t tn = numLong - t0 < kLongTile ? numLong - t0 : kLongTile;
+        int32_t tile = (numLong + static_cast<int32_t>(splits) - 1) / static_cast<int32_t>(splits);
+        tile = (tile + kWave - 1) / kWave * kWave;
+        tile = tile < kLongTile ? tile : kLongTile;
+        for (int32_t t0 = static_cast<int32_t>(part) * tile; t0 < numLong; t0 += static_cast<int32_t>(splits) * tile) {
+            const int32_t tn = numLong - t0 < tile ? numLong - t0 : tile;
             const int64_t from = tab[t0], to = tab[t0 + tn];
             __syncthreads();  // (the tile before is written out)
             for (int32_t i = tid; i < tn; i += kBlkThreads) {
@@ -1015,8 +1040,16 @@ __global__ __launch_bounds__(kRedThreads) void SpmvBlockReduceKernel(
         tabD[kRedThreads] = tabLast;
     }
     // Long rows of this block: phase 1 left the fp64 sum of each of their panels; a wavefront adds a row's up, lane
-    // by lane in panel order and then across the lanes, the same way at every call.
-    for (int32_t l = l0 + wave; l < l1; l += kRedWaves) {
+    // by lane in panel order and then across the lanes, the same way at every call.  A block with more than
+    // kInBlockLongRows of them leaves that to SpmvLongRowSumKernel (a matrix of long rows only has few blocks) and
+    // marks the rows, which nothing else touches, so that they are not written here.
+    const bool deferLong = l1 - l0 > kInBlockLongRows;
+    if (deferLong) {
+        for (int32_t l = l0 + tid; l < l1; l += kRedThreads) {
+            acc[longRows[l] - row0] = __longlong_as_double(kDeferredRowMark);
+        }
+    }
+    for (int32_t l = l0 + wave; l < l1 && !deferLong; l += kRedWaves) {
         double sum = 0.0;
         const double *from = longPartial + static_cast<int64_t>(l) * P;
         for (int32_t p0 = 0; p0 < P; p0 += 4 * kWave) {
@@ -1149,7 +1182,51 @@ __global__ __launch_bounds__(kRedThreads) void SpmvBlockReduceKernel(
     const double alpha = ReadScalar<double>(alphaS), beta = ReadScalar<double>(betaS);
     for (int i = tid; i < row1 - row0; i += kRedThreads) {
         const int64_t row = row0 + i;
+        if (deferLong && __double_as_longlong(acc[i]) == kDeferredRowMark) {
+            continue;  // SpmvLongRowSumKernel's
+        }
         double o = alpha * acc[i];
+        if (beta != 0.0) {
+            o += beta * static_cast<double>(yIn[row]);
+        }
+        y[row] = static_cast<float>(o);
+    }
+}
+
+// The long rows of the row blocks that hold more than kInBlockLongRows of them (longDeferred[l] != 0), a wavefront a
+// row: y[row] = alpha * (the row's partial sums, added up as phase 2 does) + beta * yIn[row].
+__global__ __launch_bounds__(kBlockThreads) void SpmvLongRowSumKernel(
+    const int32_t *__restrict__ header, const int32_t *__restrict__ longRows, const int32_t *__restrict__ longDeferred,
+    const double *__restrict__ longPartial, int32_t P, float *__restrict__ y, const float *__restrict__ yIn,
+    OpsparseScalar alphaS, OpsparseScalar betaS)
+{
+    const int lane = threadIdx.x % kWave;
+    const int32_t l = static_cast<int32_t>(blockIdx.x) * (kBlockThreads / kWave) + threadIdx.x / kWave;
+    if (l >= header[1] || longDeferred[l] == 0) {
+        return;
+    }
+    double sum = 0.0;
+    const double *from = longPartial + static_cast<int64_t>(l) * P;
+    for (int32_t p0 = 0; p0 < P; p0 += 4 * kWave) {
+        double v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int32_t p = p0 + u * kWave + lane;
+            v[u] = from[p < P ? p : P - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            sum += p0 + u * kWave + lane < P ? v[u] : 0.0;
+        }
+    }
+#pragma unroll
+    for (int off = kWave / 2; off > 0; off >>= 1) {
+        sum += __shfl_xor(sum, off);
+    }
+    if (lane == 0) {
+        const int64_t row = longRows[l];
+        const double alpha = ReadScalar<double>(alphaS), beta = ReadScalar<double>(betaS);
+        double o = alpha * sum;
         if (beta != 0.0) {
             o += beta * static_cast<double>(yIn[row]);
         }
@@ -1173,7 +1250,7 @@ struct BlockedLayout {
     // long rows (op(A) = A): row ids, first entry of every (long row, panel) piece, fp64 sum of every piece
     int32_t longMinRow;   // rows of at least this many entries are candidates (0: no long-row path)
     int32_t maxLong;      // room for this many
-    int64_t longRowsOff, longChunkOff, longPartialOff, longFirstOff;
+    int64_t longRowsOff, longChunkOff, longPartialOff, longFirstOff, longDeferredOff;
     int64_t resident;
     // preprocessing only
     int64_t keys0Off, keys1Off, pos0Off, pos1Off, rowOfPosOff, outPtrOff, longBeforeOff, shortOffsetsOff, longCsrOff, tableOff,
@@ -1277,6 +1354,7 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     l.longChunkOff = off; off += align(4 * (static_cast<int64_t>(l.maxLong) + 1) * (P + 1));
     l.longPartialOff = off; off += align(8 * static_cast<int64_t>(l.maxLong) * P);
     l.longFirstOff = off; off += l.maxLong > 0 ? align(4 * (B + 1)) : 0;
+    l.longDeferredOff = off; off += align(4 * static_cast<int64_t>(l.maxLong));
     l.resident = off;
     l.keys0Off = off; off += align(4 * nnz);
     l.keys1Off = off; off += align(4 * nnz);
@@ -1371,6 +1449,12 @@ int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
                            static_cast<const int32_t *>(nullptr), static_cast<const int32_t *>(nullptr));
     }
 #undef OPSPARSE_BLOCK_REDUCE_LIVE
+    if (longRows && plan.numDeferredLongRows > 0) {
+        constexpr int kRowsPerBlock = kBlockThreads / kWave;
+        hipLaunchKernelGGL(SpmvLongRowSumKernel, dim3((plan.numLongRows + kRowsPerBlock - 1) / kRowsPerBlock),
+                           dim3(kBlockThreads), 0, a.stream, header, ints(l.longRowsOff), ints(l.longDeferredOff),
+                           longPartial, l.P, static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha, a.beta);
+    }
     return CheckLaunch();
 }
 
@@ -1424,7 +1508,8 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     auto *rowLocal = reinterpret_cast<uint16_t *>(base + l.rowLocalOff);
     auto *valD = reinterpret_cast<float *>(base + l.valOff);
 
-    LaunchFillI32(status, 4, 0, s);  // status, number of long rows, their entries, positions of the longest block
+    // status, number of long rows, their entries, positions of the longest block, long rows summed on their own
+    LaunchFillI32(status, 5, 0, s);
     LaunchExpandRows(rowOffsets, rows, nnz, 0, rowOfPos, s);
     const int32_t *pos = nullptr, *outOffsets = rowOffsets;
     int32_t *chunkKey = nullptr, *rowOfSrc = nullptr;
@@ -1531,6 +1616,8 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     if (longBefore != nullptr) {
         hipLaunchKernelGGL(BlockedLongFirstKernel, dim3(GridOf(l.B + 1, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
                            s, blockRow, longBefore, l.B, ints(l.longFirstOff));
+        hipLaunchKernelGGL(BlockedLongDeferKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
+                           ints(l.longFirstOff), l.B, ints(l.longDeferredOff), status);
     }
     hipLaunchKernelGGL(BlockedScatterKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
                        pos, rowOfSrc, chunkKey, csrValues, srcStart, dstStart, blockRow, nnz, l.P, l.B, live ? nullptr : valD, rowLocal,
@@ -1560,17 +1647,22 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
                            ints(l.blockEntryOff), ints(l.longSpanOff));
     }
     int32_t liveKind = live ? 1 : 0;
+    int32_t tail[2] = {0, 0};  // positions of the longest row block, long rows that are summed on their own
     if (live) {
-        // Row blocks of fewer than 65535 positions, all of them (the rule unless a row that cannot go the long rows'
-        // way is longer than that): 16-bit positions relative to the block, 2 bytes an entry less at every call.
         hipLaunchKernelGGL(BlockedMaxPositionsKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
                            s, dstStart, l.P, l.B, status);
-        int32_t longest = 0;
-        if (hipMemcpyAsync(&longest, status + 3, sizeof(longest), hipMemcpyDeviceToHost, s) != hipSuccess ||
+    }
+    if (live || longBefore != nullptr) {
+        if (hipMemcpyAsync(tail, status + 3, sizeof(tail), hipMemcpyDeviceToHost, s) != hipSuccess ||
             hipStreamSynchronize(s) != hipSuccess) {
             (void)hipGetLastError();
             return OPSPARSE_E_LAUNCH;
         }
+    }
+    if (live) {
+        // Row blocks of fewer than 65535 positions, all of them (the rule unless a row that cannot go the long rows'
+        // way is longer than that): 16-bit positions relative to the block, 2 bytes an entry less at every call.
+        const int32_t longest = tail[0];
         static const bool noShort = std::getenv("OPS_SPARSE_BLOCKED_NO_SHORT_POSITIONS") != nullptr;
         if (!noShort && longest < static_cast<int32_t>(kNoPosition16)) {
             hipLaunchKernelGGL(BlockedShortPositionsKernel, dim3(static_cast<uint32_t>(l.B)), dim3(kBlkThreads), 0, s,
@@ -1589,6 +1681,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     p.entryWindow = l.window;
     p.transposed = transposed ? 1 : 0;
     p.liveValues = liveKind;
+    p.numDeferredLongRows = tail[1];
     p.numLongRows = head[1];
     p.rows = rows;
     p.nnz = nnz;

@@ -126,6 +126,53 @@ def test_default_plan_sums_long_rows_from_the_callers_arrays(osa, gpu_ctx):
     check(val2, x2, 2.0, 0.0)
 
 
+@pytest.mark.parametrize("live", [True, False])
+def test_many_long_rows_in_one_row_block_are_summed_by_their_own_kernel(osa, gpu_ctx, live):
+    """A row block's workgroup adds up the partial sums of at most 64 long rows; a block with more of them (here
+    200 neighbouring rows of 4200 .. 5000 entries among short ones, and in a second matrix nothing but long rows)
+    marks them and leaves them to a kernel with a wavefront a row.  Default plan and ALG2; beta != 0 with y
+    read and written in place."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    pv = lambda t: ctypes.c_void_p(t.data_ptr())
+    flags = osa.OPSPARSE_BLOCKED_LIVE_VALUES if live else 0
+
+    def run(rows, cols, lengths, want_long, seed):
+        rng = np.random.default_rng(seed)
+        rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+        colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)
+        for r in np.nonzero(lengths >= 1024)[0]:
+            colind[rowptr[r]:rowptr[r + 1]].sort()
+        val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+        x, y0 = rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+        d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+        nnz = colind.size
+        need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, flags)
+        assert need > 0
+        ws = torch.empty(need, dtype=torch.uint8, device=dev)
+        plan = osa.OpsparseSpmvPlan()
+        assert L.opsparse_spmv_csr_blocked_analyse(pv(d[0]), pv(d[1]), pv(d[2]), rows, cols, nnz, flags, pv(ws), need,
+                                                   ctypes.byref(plan), ctypes.c_void_p(stream.cuda_stream)) == 0
+        assert plan.numLongRows == want_long and plan.numDeferredLongRows == want_long
+        del ws
+        d_y = to_dev(y0, dev)
+        op = osa.SpmvOp(handle, osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3]), osa.DnVec(d_y),
+                        alg=0 if live else osa.ACL_SPARSE_SPMV_CSR_ALG2)
+        for alpha, beta in ((1.0, 0.0), (-1.5, 0.75)):
+            d_y.copy_(torch.from_numpy(y0))
+            op(alpha, beta)
+            stream.synchronize()
+            gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, alpha, beta)
+            assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+    rows, cols = 300_000, 1_400_000                          # 43 panels: long from 4096 (live) / 1024 (frozen) entries
+    rng = np.random.default_rng(41)
+    lengths = rng.integers(0, 20, rows)
+    lengths[5000:5200] = rng.integers(4200, 5000, 200)
+    run(rows, cols, lengths, 200, 42)
+    run(700, 1_300_000, np.full(700, 4500), 700, 43)         # long rows only: no entry in the row-block order
+
+
 def test_default_plan_keeps_32_bit_positions_for_a_block_of_70000_entries(osa, gpu_ctx):
     """The positions of the entries in their row block are kept in 16 bits where every block is shorter than 65535
     positions.  A row of 70 000 entries whose columns do not ascend cannot go the long rows' way, makes a block of
