@@ -84,6 +84,11 @@ constexpr int64_t kMinEntryWindow = 16384;
 constexpr int64_t kMinEntryBlocks = 512;          // entry windows a matrix is cut into at least (if it has the entries)
 constexpr int64_t kMinEntries = 2000000;          // below this the ordinary kernels are as fast or faster
 constexpr int64_t kMinChunkEntries = 32;          // below this mean chunk size the layout does not pay
+// Live values (the default plan, which competes with the merge path on the caller's arrays rather than with a
+// re-stored matrix): the window of values in LDS makes the row blocks short and the chunks with them; it pays down
+// to 8 entries a chunk (2 M rows x 16 over 30 M columns, 17 a chunk: 212 us against 603 for the merge path; 6 M
+// rows x 2 over 20 M columns, 9.5 a chunk: 123 us against 230).
+constexpr int64_t kMinChunkEntriesLive = 8;
 constexpr int64_t kLongChunkMean = 64;            // a row is "long" with this many entries per panel on average
 constexpr int64_t kLongMinRow = 4096;             // and at least this many in all
 // (frozen values: the long entries are stored again, a panel's in one piece, and stream whatever the rows' lengths;
@@ -1286,8 +1291,9 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     const int64_t B = ((rows + (int64_t{1} << rowLog) - 1) >> rowLog) + nnz / window + 1;
     // x must be larger than an L2 (2^20 columns) for the two passes to pay, and the chunks long enough to stream.
     // Positions are 32-bit, and phase 2 looks two batches past a block's end before it clamps.
-    if (cols <= (int64_t{1} << 20) || nnz < kMinEntries || P > kMaxPanels || P * B + 1 > INT32_MAX ||
-        nnz + kLaneEntries * P * B > INT32_MAX - 65536 || nnz / (P * B) < kMinChunkEntries) {
+    if (cols <= (int64_t{1} << 20) || nnz < kMinEntries || P > kMaxPanels ||
+        P * B + 1 > INT32_MAX || nnz + kLaneEntries * P * B > INT32_MAX - 65536 ||
+        nnz / (P * B) < (live ? kMinChunkEntriesLive : kMinChunkEntries)) {
         return l;
     }
     l.P = static_cast<int32_t>(P);

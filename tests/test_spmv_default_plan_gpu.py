@@ -16,6 +16,13 @@ from helpers import to_dev
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _layout_for_small_matrices(monkeypatch):
+    """The default plan takes the layout from 7 M entries on; the matrices here have 2.5 - 4 M so that the fp64
+    oracle stays quick.  The override is read at every GetBufferSize / Preprocess."""
+    monkeypatch.setenv("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ", "0")
+
+
 def _scattered(rows, cols, seed, per_row=16):
     rng = np.random.default_rng(seed)
     lengths = rng.integers(0, per_row, rows)
@@ -207,6 +214,32 @@ def test_default_plan_keeps_32_bit_positions_for_a_block_of_70000_entries(osa, g
         stream.synchronize()
         gold = oracle.spmv_f64(rows, cols, rowptr, colind, values, x, y0, alpha, beta)
         assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+
+def test_default_plan_leaves_small_matrices_to_the_merge_path(osa, gpu_ctx, monkeypatch):
+    """Below 7 M entries GetBufferSize asks for the merge-path tables only, scattered gathers or not; from there on
+    (and with the tuning override at any size) for the layout."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = 320_000, 1_500_000
+    rowptr, colind, val, x, y0 = _scattered(rows, cols, 5)
+    nnz = colind.size
+    assert 2_000_000 < nnz < 7_000_000
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    A, X, Y = osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3]), osa.DnVec(to_dev(y0, dev))
+    layout = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    assert layout > 0
+    monkeypatch.delenv("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ")
+    assert osa.SpmvOp(handle, A, X, Y).buffer.numel() == L.opsparse_spmv_csr_workspace_bytes(rows, nnz)
+    monkeypatch.setenv("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ", str(nnz))
+    assert osa.SpmvOp(handle, A, X, Y).buffer.numel() == layout
+    monkeypatch.setenv("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ", str(nnz + 1))
+    op = osa.SpmvOp(handle, A, X, Y)
+    assert op.buffer.numel() == L.opsparse_spmv_csr_workspace_bytes(rows, nnz)
+    op(1.0, 0.0)
+    stream.synchronize()
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.0, 0.0)
+    assert oracle.max_rel_err(Y.t.cpu().numpy(), gold) <= 1e-5
 
 
 def test_default_plan_of_a_banded_matrix_stays_row_wise(osa, gpu_ctx, workloads):
