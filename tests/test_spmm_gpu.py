@@ -328,6 +328,42 @@ def test_slab_table_cuts_by_work(osa, gpu_ctx):
     assert per_slab.max() <= share + 257                           # a slab overshoots its share by at most a row
 
 
+@pytest.mark.parametrize("lengths,binned", [("even 300", False), ("even 512", False), ("even 513", True),
+                                            ("300 among 10", True), ("even 200", False)])
+def test_long_rows_alike_in_length_are_not_cut(osa, gpu_ctx, lengths, binned):
+    """Rows of more than 256 entries are cut into segments so that a power-law matrix balances; rows that are all
+    about as long (none beyond 512 entries or four times the mean) gain nothing from that and go to the row-split
+    kernel whole.  GetBufferSize and the analysis agree, and the product is the oracle's either way."""
+    import torch
+    dev, stream, handle = gpu_ctx
+    rng = np.random.default_rng(len(lengths))
+    m, k, n = 3000, 50_000, 64
+    if lengths.startswith("even"):
+        base_len = int(lengths.split()[1])
+        lens = rng.integers(base_len - 40, base_len + 1, m)
+        lens[7] = base_len
+    else:
+        lens = np.full(m, 10)
+        lens[[5, 2000]] = 300
+    rowptr, colind, val = csr_from_lengths(lens, k, seed=9)
+    L = osa.lib()
+    d_rp = to_dev(rowptr, dev)
+    size = ctypes.c_size_t(0)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    nnz = int(rowptr[-1])
+    assert L.opsparse_spmm_csr_workspace_bytes(d_rp.data_ptr(), m, nnz, n, sp, ctypes.byref(size)) == 0
+    ws = torch.zeros(size.value, dtype=torch.uint8, device=dev)
+    plan = osa.OpsparseSpmmPlan()
+    assert L.opsparse_spmm_csr_analyse(d_rp.data_ptr(), m, nnz, n, ws.data_ptr(), size.value, 0, ctypes.byref(plan),
+                                       sp) == 0
+    assert (plan.numLongRows > 0) == binned and plan.bytes <= size.value
+    B = rng.uniform(-1, 1, k * n).astype(np.float32)
+    C0 = rng.uniform(-1, 1, m * n).astype(np.float32)
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, n, C0, n, -0.5, 2.0)
+    gold = oracle.spmm_f64_rowmajor(m, n, rowptr, colind, val, B, n, C0, n, -0.5, 2.0)
+    assert oracle.max_rel_err(got, gold) <= 1e-5
+
+
 @pytest.mark.parametrize("shape", ["threshold", "power_law"])
 def test_row_length_mixes_fp16(osa, gpu_ctx, shape):
     import torch
