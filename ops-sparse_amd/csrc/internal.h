@@ -129,6 +129,11 @@ OpsparseScalar MakeScalar(const void *p, aclDataType computeType, aclsparsePoint
 // the ordinary analysis in the same buffer when a sample of the columns shows the gathers are local): BLOCKED_GATHER where it
 // applies, else (op(A) = A only) COLUMN_PANELS, else none (kernel 0, 0 bytes).  OPS_SPARSE_SPMV_NO_BLOCKED in the
 // environment skips the first (tuning, tests of the panel path).
+// Sampled gathers in a thousand that must land far from the diagonal (opsparse_spmv_csr_gathers_scattered) for a
+// re-stored layout to pay: with the values frozen, and with live values.
+constexpr int32_t kScatteredForFrozenLayout = 190;
+constexpr int32_t kScatteredForLiveLayout = 310;
+
 struct RestoredChoice {
     int32_t kernel;
     size_t bytes;

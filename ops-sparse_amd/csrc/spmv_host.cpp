@@ -151,7 +151,7 @@ Restored RestoredLayout(aclsparseHandle_t handle, aclsparseOperation_t opA, acls
                                             static_cast<const int32_t *>(matA->colInd), matA->rows, matA->cols,
                                             matA->nnz, handle->workspace(), handle->workspaceBytes(), &scattered,
                                             handle->stream) != OPSPARSE_OK ||
-        !scattered) {
+        scattered < opsparse::kScatteredForLiveLayout) {
         return {0, 0, false};
     }
     return {OPSPARSE_SPMV_BLOCKED_GATHER, bytes, true};
@@ -230,10 +230,13 @@ int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *co
                     OpsparseSpmvPlan *plan, void *stream)
 {
     // A matrix whose gathers stay near the diagonal (a mesh, a band) keeps x in cache under the row-wise kernels:
-    // those are then faster than any re-stored layout (the 2048 x 2048 Laplacian: 41 us against 91 us).
+    // those are then faster than any re-stored layout (the 2048 x 2048 Laplacian: 41 us against 91 us).  With some
+    // gathers far from the diagonal among them the row-wise kernels take about 1.2 us per million entries and 13 us
+    // per million far gathers (4 M rows of a band and 1 .. 6 random columns each); the layouts take 3.6 us (values
+    // frozen) and 5.2 us (live values) per million entries whatever the columns.
     // op(A) = A^T keeps the layout either way: it replaces fp32 atomics on y, which it beats on the same Laplacian
     // (86 us against 119 us) and whose result depends on the order of the updates.
-    int32_t scattered = 1;
+    int32_t scattered = 1000;
     if (!transpose && !liveValues) {  // (a live-values request has asked already)
         int rc = opsparse_spmv_csr_gathers_scattered(rowOffsets, colInd, rows, cols, nnz, buffer, bytes, &scattered,
                                                      stream);
@@ -241,7 +244,7 @@ int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *co
             return rc;
         }
     }
-    if (!scattered) {
+    if (scattered < kScatteredForFrozenLayout) {
         return opsparse_spmv_csr_analyse(rowOffsets, rows, cols, nnz, buffer, bytes, OPSPARSE_SPMV_AUTO, plan, stream);
     }
     if (kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {

@@ -1898,8 +1898,8 @@ int opsparse_spmv_csr_gathers_scattered(const int32_t *rowOffsets, const int32_t
         (void)hipGetLastError();
         return OPSPARSE_E_LAUNCH;
     }
-    // scattered: more than one sampled gather in twenty lands outside the band
-    *scattered = (host[0] > 0 && static_cast<int64_t>(host[1]) * 20 > host[0]) ? 1 : 0;
+    // how many sampled gathers in a thousand land outside the band
+    *scattered = host[0] > 0 ? static_cast<int32_t>(static_cast<int64_t>(host[1]) * 1000 / host[0]) : 0;
     return OPSPARSE_OK;
 }
 

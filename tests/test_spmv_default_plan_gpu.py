@@ -260,6 +260,47 @@ def test_default_plan_of_a_banded_matrix_stays_row_wise(osa, gpu_ctx, workloads)
     assert oracle.max_rel_err(y.cpu().numpy(), gold) <= 1e-5
 
 
+@pytest.mark.parametrize("far,layout_default,layout_alg2", [(1, False, False), (2, False, True), (4, True, True)])
+def test_a_band_with_some_random_columns_gets_the_layout_only_where_it_pays(osa, gpu_ctx, far, layout_default,
+                                                                             layout_alg2):
+    """Eight entries a row, `far` of them anywhere and the others within a few columns of the diagonal.  The row-wise
+    kernels pay for the far gathers only, the layouts for every entry: the default plan re-stores from 31 % far
+    gathers on, ALG2 (values frozen, a cheaper layout) from 19 %.  One in eight: neither; two: ALG2 only; four: both.
+    Which plan ran shows in the buffer the default plan asks for and, for ALG2, in the kernel of the plan bound."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows = 1_300_000
+    rng = np.random.default_rng(far)
+    near = (np.arange(rows)[:, None] + rng.integers(-40, 41, (rows, 8 - far))).clip(0, rows - 1)
+    cols = np.concatenate([near, rng.integers(0, rows, (rows, far))], axis=1)
+    colind = np.sort(cols, axis=1).astype(np.int32).reshape(-1)
+    rowptr = (np.arange(rows + 1) * 8).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    x, y0 = rng.uniform(-1, 1, rows).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    nnz = colind.size
+    A, X = osa.Csr(rows, rows, d[0], d[1], d[2]), osa.DnVec(d[3])
+    gold = oracle.spmv_f64(rows, rows, rowptr, colind, val, x, y0, 1.0, 0.5)
+    live_bytes = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, rows, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    assert live_bytes > 0
+    for alg, want_layout in ((osa.ACL_SPARSE_SPMV_ALG_DEFAULT, layout_default), (osa.ACL_SPARSE_SPMV_CSR_ALG2, layout_alg2)):
+        d_y = to_dev(y0, dev)
+        op = osa.SpmvOp(handle, A, X, osa.DnVec(d_y), alg=alg)
+        if alg == osa.ACL_SPARSE_SPMV_ALG_DEFAULT:
+            assert (op.buffer.numel() == live_bytes) == want_layout
+        op(1.0, 0.5)
+        stream.synchronize()
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+    # the analysis ALG2's Preprocess runs, through the raw layer: the probe's figure against its threshold
+    ws = torch.zeros(256, dtype=torch.uint8, device=dev)
+    flag = ctypes.c_int32(-1)
+    pv = lambda t: ctypes.c_void_p(t.data_ptr())
+    assert L.opsparse_spmv_csr_gathers_scattered(pv(d[0]), pv(d[1]), rows, rows, nnz, pv(ws), 256, ctypes.byref(flag),
+                                                 ctypes.c_void_p(stream.cuda_stream)) == 0
+    assert abs(flag.value - 125 * far * (1 - 262144 / rows)) <= 15       # (a random column is near by chance one time in five)
+    assert (flag.value >= 190) == layout_alg2 and (flag.value >= 310) == layout_default
+
+
 def test_alg2_plan_is_dropped_when_the_values_array_is_replaced(osa, gpu_ctx):
     dev, stream, handle = gpu_ctx
     L = osa.lib()

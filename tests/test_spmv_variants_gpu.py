@@ -432,7 +432,13 @@ def test_alg2_keeps_row_kernels_for_local_gathers(osa, workloads, gpu_ctx):
     shuffled = torch.randint(0, cols, (nnz,), dtype=torch.int32, device=dev)
     torch.cuda.synchronize()
     assert L.opsparse_spmv_csr_gathers_scattered(p(A["rowptr"]), p(shuffled), rows, cols, nnz, p(ws), 256,
-                                                 ctypes.byref(flag), sp) == 0 and flag.value == 1
+                                                 ctypes.byref(flag), sp) == 0 and flag.value > 700   # in a thousand
+    # one column in five sent anywhere: every fifth sampled gather, less the few that land near the diagonal by chance
+    some = A["colind"].clone()
+    some[::5] = shuffled[::5]
+    torch.cuda.synchronize()
+    assert L.opsparse_spmv_csr_gathers_scattered(p(A["rowptr"]), p(some), rows, cols, nnz, p(ws), 256,
+                                                 ctypes.byref(flag), sp) == 0 and 120 <= flag.value <= 200
     rng = np.random.default_rng(3)
     x, y0 = rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
     d_x, d_y = to_dev(x, dev), to_dev(y0, dev)
