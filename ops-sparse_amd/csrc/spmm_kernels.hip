@@ -303,7 +303,7 @@ __device__ __forceinline__ void SlabBody(
     int64_t slab, const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd,
     const ValT *__restrict__ vals, const ValT *__restrict__ B, CT *__restrict__ C, int64_t rows, int32_t n, int64_t ldb,
     int64_t ldc, int32_t rowsPerSlab, const int32_t *__restrict__ slabStart, int32_t longRowNnz,
-    OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16)
+    OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16, int32_t tileCol0, int32_t tileCols)
 {
     typedef ValT BVec __attribute__((ext_vector_type(V)));
     typedef CT CVec __attribute__((ext_vector_type(V), aligned(16)));
@@ -322,8 +322,8 @@ __device__ __forceinline__ void SlabBody(
     const int32_t tid = threadIdx.x;
     const int32_t lane = tid % L;
     const int32_t group = tid / L;
-    const int32_t col = lane * V;
-    const bool active = col < n;
+    const int32_t col = tileCol0 + lane * V;  // the workgroup's tile of at most L * V columns of B and C
+    const bool active = lane * V < tileCols && col < n;
     const ValT *Bcol = B + col;
     const uint32_t colBytes = static_cast<uint32_t>(col) * static_cast<uint32_t>(sizeof(ValT));
     const uint32_t ldbBytes = static_cast<uint32_t>(ldb) * static_cast<uint32_t>(sizeof(ValT));
@@ -495,7 +495,7 @@ __device__ __forceinline__ void SegmentBody(int64_t block, const int32_t *__rest
                                             const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
                                             const ValT *__restrict__ B, int32_t n, int64_t ldb, int32_t numSegments,
                                             const int32_t *__restrict__ segRow, const int32_t *__restrict__ segStart,
-                                            AccT *__restrict__ partial)
+                                            AccT *__restrict__ partial, int32_t colBegin, int32_t colEnd)
 {
     constexpr int kGroups = kBlockThreads / L;
     const int32_t lane = threadIdx.x % L;
@@ -510,9 +510,9 @@ __device__ __forceinline__ void SegmentBody(int64_t block, const int32_t *__rest
     int32_t firstCol;
     float firstVal;
     LoadFirstChunk<ValT, AccT>(colInd, vals, lane, s, e, &firstCol, &firstVal);
-    for (int32_t c0 = 0; c0 < n; c0 += L * V) {
+    for (int32_t c0 = colBegin; c0 < colEnd; c0 += L * V) {
         const int32_t col = c0 + lane * V;
-        const bool active = col < n;
+        const bool active = col < colEnd;
         AccT acc[V];
 #pragma unroll
         for (int i = 0; i < V; ++i) {
@@ -535,7 +535,8 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmLongSegmentKernel(
     const ValT *__restrict__ B, int32_t n, int64_t ldb, int32_t numSegments, const int32_t *__restrict__ segRow,
     const int32_t *__restrict__ segStart, AccT *__restrict__ partial)
 {
-    SegmentBody<ValT, AccT, V, L>(blockIdx.x, rowOffsets, colInd, vals, B, n, ldb, numSegments, segRow, segStart, partial);
+    SegmentBody<ValT, AccT, V, L>(blockIdx.x, rowOffsets, colInd, vals, B, n, ldb, numSegments, segRow, segStart, partial,
+                                  0, n);
 }
 
 // The slab kernel proper.  With long rows (segBlocks > 0) the workgroups of their
@@ -548,8 +549,10 @@ __global__ __launch_bounds__(kBlockThreads, SlabTuning<V>::kWavesPerSimd) void S
     const ValT *__restrict__ B, CT *__restrict__ C, int64_t rows, int32_t n, int64_t ldb, int64_t ldc,
     int32_t rowsPerSlab, const int32_t *__restrict__ slabStart, int32_t longRowNnz, OpsparseScalar alphaS,
     OpsparseScalar betaS, int32_t clampF16, uint32_t segBlocks, int32_t numSegments, const int32_t *__restrict__ segRow,
-    const int32_t *__restrict__ segStart, AccT *__restrict__ partial)
+    const int32_t *__restrict__ segStart, AccT *__restrict__ partial, int32_t tileCols)
 {
+    // blockIdx.y: which tile of tileCols (<= L * V) columns of B and C.
+    const int32_t tileCol0 = static_cast<int32_t>(blockIdx.y) * tileCols;
     int64_t slab;
     if (segBlocks > 0) {
         // workgroup b is a segment workgroup iff floor((b + 1) * segBlocks / total) > floor(b * segBlocks / total)
@@ -557,7 +560,8 @@ __global__ __launch_bounds__(kBlockThreads, SlabTuning<V>::kWavesPerSimd) void S
         const uint64_t after = (static_cast<uint64_t>(blockIdx.x) + 1) * segBlocks / gridDim.x;
         if (after > before) {
             SegmentBody<ValT, AccT, V, L>(static_cast<int64_t>(before), rowOffsets, colInd, vals, B, n, ldb, numSegments,
-                                          segRow, segStart, partial);
+                                          segRow, segStart, partial, tileCol0,
+                                          (n - tileCol0 < tileCols) ? n : tileCol0 + tileCols);
             return;
         }
         slab = static_cast<int64_t>(blockIdx.x) - static_cast<int64_t>(before);
@@ -565,7 +569,7 @@ __global__ __launch_bounds__(kBlockThreads, SlabTuning<V>::kWavesPerSimd) void S
         slab = XcdContiguousTile(blockIdx.x, gridDim.x);
     }
     SlabBody<ValT, CT, AccT, V, L, Small32>(slab, rowOffsets, colInd, vals, B, C, rows, n, ldb, ldc, rowsPerSlab,
-                                            slabStart, longRowNnz, alphaS, betaS, clampF16);
+                                            slabStart, longRowNnz, alphaS, betaS, clampF16, tileCol0, tileCols);
 }
 
 // One workgroup per long row.  Each of its four wavefronts adds a contiguous
@@ -956,7 +960,7 @@ void LaunchLongRows(const SpmmArgs &a)
 bool UseSlabKernel(const SpmmArgs &a, int64_t lanesNeeded)
 {
     static const bool off = std::getenv("OPS_SPARSE_SPMM_NO_SLAB") != nullptr;
-    if (off || a.plan == nullptr || lanesNeeded > 64) {
+    if (off || a.plan == nullptr || lanesNeeded > 64 * 65535) {
         return false;
     }
     const bool binned = a.plan->kernel == OPSPARSE_SPMM_BINNED && a.plan->numLongRows > 0;
@@ -985,6 +989,17 @@ int LaunchSlab(const SpmmArgs &a)
     const bool small32 = static_cast<uint64_t>(a.k) * static_cast<uint64_t>(a.ldb) * sizeof(ValT) < (1ull << 32);
     // Long rows: their segment workgroups ride in the same launch, the fix-up follows.
     constexpr int kGroups = kBlockThreads / L;
+    // More columns than a lane group spans: one workgroup a (slab, tile of columns), the tiles of equal width (a
+    // last tile of a few columns would cost a whole pass over the slab: n = 260, 8.2 ms against 5.0 ms).
+    // A tile is a whole number of 64-byte pieces of a row of B: four lanes' loads share one (n = 1000 in tiles of
+    // 252 columns 27.3 ms, in tiles of 256 25.1 ms).
+    const int64_t vecs = (a.n + V - 1) / V;
+    const uint32_t colTiles = static_cast<uint32_t>((vecs + L - 1) / L);
+    int64_t tileVecs = (vecs + colTiles - 1) / colTiles;
+    if (colTiles > 1) {
+        tileVecs = (tileVecs + 3) / 4 * 4;  // (L is 64 here)
+    }
+    const int32_t tileCols = static_cast<int32_t>(tileVecs) * V;
     auto *base = static_cast<unsigned char *>(a.ws);
     const int32_t nseg = binned ? a.plan->numSegments : 0;
     const uint32_t segBlocks = static_cast<uint32_t>((nseg + kGroups - 1) / kGroups);
@@ -993,11 +1008,12 @@ int LaunchSlab(const SpmmArgs &a)
     AccT *partial = binned ? reinterpret_cast<AccT *>(base + a.plan->partialOff) : nullptr;
     auto launch = [&](auto tag) {
         constexpr bool kSmall = decltype(tag)::value;
-        hipLaunchKernelGGL((SpmmSlabKernel<ValT, CT, AccT, V, L, kSmall>), dim3(grid + segBlocks), dim3(kBlockThreads),
+        hipLaunchKernelGGL((SpmmSlabKernel<ValT, CT, AccT, V, L, kSmall>), dim3(grid + segBlocks, colTiles),
+                           dim3(kBlockThreads),
                            0, a.stream, a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
                            static_cast<const ValT *>(a.B), static_cast<CT *>(a.C), a.rows, static_cast<int32_t>(a.n),
                            a.ldb, a.ldc, static_cast<int32_t>(rps), slabStart, longRowNnz, a.alpha, a.beta, a.clampF16,
-                           segBlocks, nseg, segRow, segStart, partial);
+                           segBlocks, nseg, segRow, segStart, partial, tileCols);
     };
     if (small32) {
         launch(std::true_type{});

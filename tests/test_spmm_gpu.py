@@ -101,7 +101,7 @@ def test_reference_fp32_cases(osa, gpu_ctx, name, m, k, n, nnz, alpha, beta, tra
     assert np.array_equal(got[rest].view(np.uint32), C0[rest].view(np.uint32))  # what lies beyond C stays as it was
 
 
-@pytest.mark.parametrize("n", [1, 3, 8, 17, 32, 64, 100, 128, 256, 260])
+@pytest.mark.parametrize("n", [1, 3, 8, 17, 32, 64, 100, 128, 256, 260, 516, 1000])
 @pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, -2.0)])
 def test_column_counts_and_padding(osa, gpu_ctx, n, alpha, beta):
     """n not a multiple of the vector width, and ldb / ldc padding."""
@@ -132,7 +132,7 @@ def test_layouts(osa, gpu_ctx, b_rm, c_rm, trans_b):
                c_row_major=c_rm)
 
 
-@pytest.mark.parametrize("n", [64, 128, 16])
+@pytest.mark.parametrize("n", [64, 128, 16, 300])
 def test_long_rows_are_binned(osa, gpu_ctx, n):
     """Rows far above the long-row threshold next to short and empty ones."""
     rng = np.random.default_rng(n)
@@ -279,10 +279,11 @@ def _lengths(shape, m, rng):
 
 @pytest.mark.parametrize("shape", ["mostly_empty", "threshold", "dense_slabs", "alternating", "power_law",
                                    "sorted_up", "sorted_down"])
-@pytest.mark.parametrize("n,beta", [(8, 0.0), (24, 0.5), (64, -1.0), (256, 0.0)])
+@pytest.mark.parametrize("n,beta", [(8, 0.0), (24, 0.5), (64, -1.0), (256, 0.0), (260, 0.5), (1000, 0.0)])
 def test_row_length_mixes(osa, gpu_ctx, shape, n, beta):
     """Preprocessed fast path (rows worked in LDS-staged slabs, long rows in segments) on row-length mixes that
-    hit its corner cases; n = 24 leaves lanes of a lane group without a column."""
+    hit its corner cases; n = 24 leaves lanes of a lane group without a column; n = 260 and 1000 are more columns
+    than a lane group spans: several workgroups a slab, one a tile of columns."""
     rng = np.random.default_rng(len(shape) * 1000 + n)
     m = 1 if shape == "single" else (700 if shape == "dense_slabs" else 6000)
     k = 5000
@@ -364,11 +365,12 @@ def test_long_rows_alike_in_length_are_not_cut(osa, gpu_ctx, lengths, binned):
     assert oracle.max_rel_err(got, gold) <= 1e-5
 
 
+@pytest.mark.parametrize("n", [128, 520])
 @pytest.mark.parametrize("shape", ["threshold", "power_law"])
-def test_row_length_mixes_fp16(osa, gpu_ctx, shape):
+def test_row_length_mixes_fp16(osa, gpu_ctx, shape, n):
     import torch
     rng = np.random.default_rng(77)
-    m, k, n = 5000, 4000, 128
+    m, k = 5000, 4000
     rowptr, colind, val = csr_from_lengths(_lengths(shape, m, rng), k, seed=5)
     val = val.astype(np.float16).astype(np.float32)
     B = rng.uniform(-1, 1, k * n).astype(np.float16).astype(np.float32)
