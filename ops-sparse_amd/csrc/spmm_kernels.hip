@@ -13,10 +13,11 @@
 //
 // Row-length binning (the counterpart of the reference's greedy row bin
 // packing, sparse/spmm/arch35/spmm_csr_mat.cpp:28-66): rows of up to
-// kLongRowNnz entries are taken whole by one lane group — after Preprocess in
-// slabs of consecutive rows staged through LDS, where every lane group walks an
-// equal share of the slab's entries (SpmmSlabKernel), without Preprocess one
-// row after the other straight from global memory (SpmmRowSplitKernel).  Longer
+// kLongRowNnz entries are worked — after Preprocess — in slabs of consecutive
+// rows staged through LDS, where every lane group walks an equal share of the
+// slab's entries and a row that lies across two shares is cut between them
+// (SpmmSlabKernel); without Preprocess a lane group takes one row after the
+// other straight from global memory (SpmmRowSplitKernel).  Longer
 // rows — the tail of a power-law graph — are cut into segments of kSegmentNnz
 // entries, every segment is accumulated by its own lane group into an fp64
 // partial row in the workspace, and a fix-up kernel adds a row's partials in
@@ -38,10 +39,7 @@
 
 namespace opsparse {
 
-#ifndef VAR_EVEN_MAX
-#define VAR_EVEN_MAX 512
-#endif
-constexpr int32_t kLongRowNnz = 256;  // rows longer than this are cut into segments
+constexpr int32_t kLongRowNnz = 2048;  // rows longer than this are cut into segments
 constexpr int32_t kSegmentNnz = 128;  // entries per segment
 // Rows a lane group of the row-split kernel takes one after the other, so that a
 // workgroup lives long enough to amortise its start-up.
@@ -273,15 +271,18 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmRowSplitKernel(
 // The same fast-path operands, rows of at most longRowNnz entries, worked on a
 // slab of consecutive rows at a time.  A workgroup copies the slab's (column,
 // value) pairs — one contiguous piece of the CSR arrays — and its row bounds
-// into LDS, cuts the slab's rows into one run of consecutive rows per lane group
-// with about the same number of entries each, and every lane group then walks
-// its run as one flat sequence of entries: batches of four or eight gathers of B
-// rows, two batches in flight, a row's sum written out whenever the sequence
-// crosses a row end.  Short rows therefore cost no more than their share of a
-// long one: no predicated partial batches, no chain of dependent loads in front
-// of every row.  Rows longer than longRowNnz are left out (the segment kernels
-// write them); a slab with more entries than the LDS holds is worked in several
-// pieces.
+// into LDS, cuts the slab's entries into one run per lane group with about the
+// same number of entries each (a run starts at a row's first entry, or inside a
+// row of kSplitRowMin entries or more), and every lane group then walks its run
+// as one flat sequence of entries: batches of four or eight gathers of B rows,
+// two batches in flight, a row's sum written out whenever the sequence crosses a
+// row end.  Short rows therefore cost no more than their share of a long one: no
+// predicated partial batches, no chain of dependent loads in front of every row.
+// The parts of a row cut between runs meet in LDS once the piece has been
+// streamed, and the lane group in which the row ends adds them up in the order
+// of the entries: the result does not depend on scheduling.  Rows longer than
+// longRowNnz are left out (the segment kernels write them); a slab with more
+// entries than the LDS holds is worked in several pieces.
 
 constexpr int kSlabCap = 3072;      // entries a workgroup stages in LDS at a time
 constexpr int kSlabRowsMax = 255;   // rows whose bounds it stages at a time
@@ -294,6 +295,14 @@ struct SlabTuning {
     static constexpr int kWavesPerSimd = V >= 8 ? 3 : 2;
 };
 constexpr int kSlabTarget = 2048;   // entries per slab the launcher aims for
+// A row of at least kSplitRowMin entries that lies across the boundary between two runs is cut there (neither part
+// shorter than kSplitPartMin): the lane group in which it ends adds up the parts.  Without this a row of 250 entries
+// makes its run twice as long as the others of its slab, which wait for it (a power-law graph of 2 M rows, mean 16,
+// fp16, n = 128: 1.57 -> 1.46 ms), and with it rows of up to 2048 entries are better left to the slabs than cut
+// into segments (1.46 -> 1.39 ms; rows of 300, 600 or 2000 entries each run like rows of 64).
+constexpr int kSplitRowMin = 16;
+constexpr int kSplitPartMin = 4;
+static_assert(kLongRowNnz <= kSlabCap, "a row that is not long fits the staging area");
 
 // Small32: B spans less than 4 GiB, so a gather address is the (uniform) base of
 // B plus a 32-bit byte offset — one register and one multiply per gather
@@ -310,11 +319,19 @@ __device__ __forceinline__ void SlabBody(
     constexpr int kGroups = kBlockThreads / L;
     constexpr int NB = SlabTuning<V>::kBatch;
 
-    __shared__ int32_t entCol[kSlabCap];
-    __shared__ float entVal[kSlabCap];
+    // The staged entries; once a piece has been streamed, the same memory takes what every lane group has left of
+    // a row that goes on in the next group.
+    __shared__ __align__(16) unsigned char stage[kSlabCap * 8];
+    int32_t *const entCol = reinterpret_cast<int32_t *>(stage);
+    float *const entVal = reinterpret_cast<float *>(stage + kSlabCap * 4);
+    AccT *const tailSum = reinterpret_cast<AccT *>(stage);
+    static_assert(sizeof(AccT) * kBlockThreads * V <= sizeof(stage), "the parts of cut rows share the staging area");
+    __shared__ AccT headSum[kBlockThreads * V];   // a group's sum of the rest of a row that began in an earlier group
     __shared__ int32_t rowAbs[kSlabRowsMax + 1];  // row offsets of the window, as stored
-    __shared__ int32_t runBound[kGroups + 1];     // first row (window-relative) of every lane group's run
+    __shared__ int32_t runRow[kGroups + 1];       // row (window-relative) in which every lane group's run starts,
+    __shared__ int32_t runEntry[kGroups + 1];     // and its first entry (piece-relative): past the row's first if cut
     __shared__ int32_t pieceRows;                 // rows of the window that go into this piece
+    __shared__ int32_t pieceSplit;                // whether any row of the piece is cut between lane groups
 
     const AccT alpha = ReadScalar<AccT>(alphaS);
     const AccT beta = ReadScalar<AccT>(betaS);
@@ -347,6 +364,7 @@ __device__ __forceinline__ void SlabBody(
         }
         if (tid == 0) {
             pieceRows = win;
+            pieceSplit = 0;
         }
         __syncthreads();
         const int32_t base = rowAbs[0];
@@ -375,11 +393,10 @@ __device__ __forceinline__ void SlabBody(
         // 2.55 ms.)
         if (tid <= kGroups) {
             const int32_t share = (E + J + kGroups - 1) / kGroups;
-            int32_t lo = 0, hi = J;
-            if (tid == kGroups) {
-                lo = J;
-            } else {
+            int32_t row = J, first = E;
+            if (tid < kGroups) {
                 const int32_t want = tid * share;
+                int32_t lo = 0, hi = J;
                 while (lo < hi) {
                     const int32_t mid = (lo + hi) >> 1;
                     if (rowAbs[mid] - base + mid < want) {
@@ -388,15 +405,34 @@ __device__ __forceinline__ void SlabBody(
                         hi = mid;
                     }
                 }
+                row = lo;
+                first = rowAbs[lo] - base;
+                if (lo > 0) {
+                    // Row lo - 1 lies across `want`: cut it where entries + rows in front come to `want`.
+                    const int32_t rowFirst = rowAbs[lo - 1] - base;
+                    const int32_t cut = want - (lo - 1);
+                    if (first - rowFirst >= kSplitRowMin && first - cut >= kSplitPartMin) {
+                        row = lo - 1;  // (a cut near the row's end goes to the end, one near its start to the start:
+                                       // the starts of the runs must not go backwards)
+                        if (cut - rowFirst >= kSplitPartMin) {
+                            first = cut;
+                            pieceSplit = 1;
+                        } else {
+                            first = rowFirst;
+                        }
+                    }
+                }
             }
-            runBound[tid] = lo;
+            runRow[tid] = row;
+            runEntry[tid] = first;
         }
         __syncthreads();
 
-        int32_t cur = runBound[group];           // next row to finish
-        const int32_t last = runBound[group + 1];
-        int32_t f = rowAbs[cur] - base;          // next entry to consume
-        const int32_t fEnd = rowAbs[last] - base;
+        int32_t cur = runRow[group];             // next row to finish
+        const int32_t last = runRow[group + 1];  // first row that this run does not finish
+        int32_t f = runEntry[group];             // next entry to consume
+        const int32_t fEnd = runEntry[group + 1];
+        bool headRow = f > rowAbs[cur] - base;   // the run starts inside row `cur`
         int32_t nextEnd = (cur < last) ? rowAbs[cur + 1] - base : INT32_MAX;
 
         AccT acc[V];
@@ -404,26 +440,36 @@ __device__ __forceinline__ void SlabBody(
         for (int i = 0; i < V; ++i) {
             acc[i] = AccT(0);
         }
-        // Writes every row of the run that ends at entry position `pos`.
+        auto writeRow = [&](int32_t row, const AccT(&sum)[V]) {
+            CT *out = C + (rowCur + row) * ldc + col;
+            CVec res;
+            if (betaZero) {
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    res[i] = Epilogue<CT, AccT>::Apply(sum[i], alpha, beta, true, nullptr, clampF16 != 0);
+                }
+            } else {
+                const CVec old = *reinterpret_cast<const CVec *>(out);
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    const CT o = old[i];
+                    res[i] = Epilogue<CT, AccT>::Apply(sum[i], alpha, beta, false, &o, clampF16 != 0);
+                }
+            }
+            *reinterpret_cast<CVec *>(out) = res;
+        };
+        // Writes every row of the run that ends at entry position `pos`; the rest of a row that began in an earlier
+        // run is kept for the addition of its parts.
         auto finishRows = [&](int32_t pos) {
             while (nextEnd <= pos) {
-                if (active) {
-                    CT *out = C + (rowCur + cur) * ldc + col;
-                    CVec res;
-                    if (betaZero) {
+                if (headRow) {
 #pragma unroll
-                        for (int i = 0; i < V; ++i) {
-                            res[i] = Epilogue<CT, AccT>::Apply(acc[i], alpha, beta, true, nullptr, clampF16 != 0);
-                        }
-                    } else {
-                        const CVec old = *reinterpret_cast<const CVec *>(out);
-#pragma unroll
-                        for (int i = 0; i < V; ++i) {
-                            const CT o = old[i];
-                            res[i] = Epilogue<CT, AccT>::Apply(acc[i], alpha, beta, false, &o, clampF16 != 0);
-                        }
+                    for (int i = 0; i < V; ++i) {
+                        headSum[tid * V + i] = acc[i];
                     }
-                    *reinterpret_cast<CVec *>(out) = res;
+                    headRow = false;
+                } else if (active) {
+                    writeRow(cur, acc);
                 }
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
@@ -483,6 +529,42 @@ __device__ __forceinline__ void SlabBody(
             }
         }
         finishRows(fEnd);  // nothing left unless the run has no entry at all
+        if (pieceSplit != 0) {  // uniform over the workgroup
+            // What a run holds at its end belongs to a row that goes on in the next run (zero if there is none).
+            __syncthreads();    // every run is done with the staged entries
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                tailSum[tid * V + i] = acc[i];
+            }
+            __syncthreads();
+            const int32_t row = runRow[group];
+            const int32_t rowFirst = rowAbs[row] - base;
+            if (runEntry[group] > rowFirst && last > row) {
+                // Row `row` ends in this run: its parts in the order of the entries, from the run in which it starts.
+                int32_t g0 = group - 1;
+                while (g0 > 0 && runRow[g0] == row && runEntry[g0] > rowFirst) {
+                    --g0;
+                }
+                AccT sum[V];
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    sum[i] = tailSum[(g0 * L + lane) * V + i];
+                }
+                for (int32_t g = g0 + 1; g < group; ++g) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) {
+                        sum[i] += tailSum[(g * L + lane) * V + i];
+                    }
+                }
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    sum[i] += headSum[tid * V + i];
+                }
+                if (active) {
+                    writeRow(row, sum);
+                }
+            }
+        }
         rowCur += J;
         __syncthreads();   // the next piece overwrites the LDS arrays
     }
@@ -895,19 +977,12 @@ int RowStats(const int32_t *rowOffsets, int64_t rows, int32_t *scratch, hipStrea
     return OPSPARSE_OK;
 }
 
-// Rows that are long but alike in length (no row beyond kEvenRowsMax entries or kEvenRowsSpread times the mean):
-// cutting them into segments buys no balance and costs the partial rows; a lane group a row does better
-// (200 000 rows x 300 entries, n = 64: 2.46 ms against 3.04 ms).  st: longest row, long rows, segments.
-constexpr int32_t kEvenRowsMax = VAR_EVEN_MAX;
-constexpr int64_t kEvenRowsSpread = 4;
-
-bool EvenLongRows(const int32_t st[3], int64_t rows, int64_t nnz)
+// OPS_SPARSE_SPMM_NO_BINNING: no row is cut into segments; a matrix with rows beyond kLongRowNnz entries then goes
+// to the kernel with a lane group a row (for measurements).
+bool NoBinning()
 {
     static const bool force = std::getenv("OPS_SPARSE_SPMM_NO_BINNING") != nullptr;
-    if (force) {
-        return true;
-    }
-    return st[1] > 0 && st[0] <= kEvenRowsMax && static_cast<int64_t>(st[0]) * rows <= kEvenRowsSpread * nnz;
+    return force;
 }
 
 template <typename ValT, typename CT, typename AccT, int V, int L>
@@ -965,7 +1040,7 @@ bool UseSlabKernel(const SpmmArgs &a, int64_t lanesNeeded)
     }
     const bool binned = a.plan->kernel == OPSPARSE_SPMM_BINNED && a.plan->numLongRows > 0;
     if (!binned && a.plan->maxRowNnz > kLongRowNnz) {
-        return false;  // rows that long and alike: a few to a slab, most of whose lane groups would idle
+        return false;  // (only with OPS_SPARSE_SPMM_NO_BINNING) rows that do not fit the staging area
     }
     return binned || (a.plan->maxRowNnz > 0 && a.plan->maxRowNnz <= kSlabCap);
 }
@@ -1114,7 +1189,7 @@ int opsparse_spmm_csr_workspace_bytes(const int32_t *rowOffsets, int64_t rows, i
     if (rc != OPSPARSE_OK) {
         return rc;
     }
-    if (EvenLongRows(st, rows, nnz)) {
+    if (NoBinning()) {
         st[1] = st[2] = 0;
     }
     OpsparseSpmmPlan p{};
@@ -1155,7 +1230,7 @@ int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t n
     if (rc != OPSPARSE_OK) {
         return rc;
     }
-    if (EvenLongRows(st, rows, nnz)) {
+    if (NoBinning()) {
         st[1] = st[2] = 0;
     }
     p.maxRowNnz = st[0];

@@ -260,9 +260,12 @@ def _lengths(shape, m, rng):
     if shape == "mostly_empty":                 # windows of more than 255 empty rows
         lengths = np.zeros(m, np.int64)
         lengths[rng.choice(m, m // 100, replace=False)] = rng.integers(1, 30, m // 100)
-    elif shape == "threshold":                  # 256 is still a short row, 257 is a long one
+    elif shape == "threshold":                  # 2048 is still a short row, 2049 is a long one
         lengths = rng.integers(0, 12, m)
-        lengths[rng.choice(m, 40, replace=False)] = rng.choice([255, 256, 257, 300], 40)
+        lengths[rng.choice(m, 40, replace=False)] = rng.choice([255, 300, 2047, 2048, 2049, 2100], 40)
+    elif shape == "cut_rows":                   # rows that lie across several lane groups' shares of a slab
+        lengths = rng.choice([0, 1, 2, 3, 15, 16, 17, 40, 100, 700, 1500, 2048], m,
+                             p=[.1, .2, .2, .2, .05, .05, .05, .05, .05, .02, .02, .01])
     elif shape == "dense_slabs":                # a slab holds more entries than one LDS piece takes
         lengths = rng.integers(150, 257, m)
     elif shape == "alternating":
@@ -277,7 +280,7 @@ def _lengths(shape, m, rng):
     return lengths
 
 
-@pytest.mark.parametrize("shape", ["mostly_empty", "threshold", "dense_slabs", "alternating", "power_law",
+@pytest.mark.parametrize("shape", ["mostly_empty", "threshold", "cut_rows", "dense_slabs", "alternating", "power_law",
                                    "sorted_up", "sorted_down"])
 @pytest.mark.parametrize("n,beta", [(8, 0.0), (24, 0.5), (64, -1.0), (256, 0.0), (260, 0.5), (1000, 0.0)])
 def test_row_length_mixes(osa, gpu_ctx, shape, n, beta):
@@ -329,23 +332,25 @@ def test_slab_table_cuts_by_work(osa, gpu_ctx):
     assert per_slab.max() <= share + 257                           # a slab overshoots its share by at most a row
 
 
-@pytest.mark.parametrize("lengths,binned", [("even 300", False), ("even 512", False), ("even 513", True),
-                                            ("300 among 10", True), ("even 200", False)])
-def test_long_rows_alike_in_length_are_not_cut(osa, gpu_ctx, lengths, binned):
-    """Rows of more than 256 entries are cut into segments so that a power-law matrix balances; rows that are all
-    about as long (none beyond 512 entries or four times the mean) gain nothing from that and go to the row-split
-    kernel whole.  GetBufferSize and the analysis agree, and the product is the oracle's either way."""
+@pytest.mark.parametrize("lengths,binned", [("even 300", False), ("even 2048", False), ("even 2049", True),
+                                            ("300 among 10", False), ("2100 among 10", True)])
+def test_only_rows_beyond_2048_entries_are_cut_into_segments(osa, gpu_ctx, lengths, binned):
+    """Rows of up to 2048 entries stay with the slabs, whose lane groups share them out; longer ones are cut into
+    segments so that a power-law matrix balances.  GetBufferSize and the analysis agree, and the product is the
+    oracle's either way."""
     import torch
     dev, stream, handle = gpu_ctx
     rng = np.random.default_rng(len(lengths))
-    m, k, n = 3000, 50_000, 64
+    k, n = 50_000, 64
     if lengths.startswith("even"):
         base_len = int(lengths.split()[1])
+        m = 3000 if base_len < 1000 else 500
         lens = rng.integers(base_len - 40, base_len + 1, m)
         lens[7] = base_len
     else:
+        m = 3000
         lens = np.full(m, 10)
-        lens[[5, 2000]] = 300
+        lens[[5, 2000]] = int(lengths.split()[0])
     rowptr, colind, val = csr_from_lengths(lens, k, seed=9)
     L = osa.lib()
     d_rp = to_dev(rowptr, dev)
@@ -366,7 +371,7 @@ def test_long_rows_alike_in_length_are_not_cut(osa, gpu_ctx, lengths, binned):
 
 
 @pytest.mark.parametrize("n", [128, 520])
-@pytest.mark.parametrize("shape", ["threshold", "power_law"])
+@pytest.mark.parametrize("shape", ["threshold", "cut_rows", "power_law"])
 def test_row_length_mixes_fp16(osa, gpu_ctx, shape, n):
     import torch
     rng = np.random.default_rng(77)
