@@ -98,6 +98,7 @@ __device__ __forceinline__ AccT ReadScalar(const OpsparseScalar &s)
 
 typedef int32_t Int4U __attribute__((ext_vector_type(4), aligned(4)));
 typedef float Float4U __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint16_t Short4U __attribute__((ext_vector_type(4), aligned(2)));  // four fp16 / bf16 values at any even address
 
 template <typename T>
 __device__ __forceinline__ T LoadStream(const T *p)

@@ -236,17 +236,15 @@ __device__ __forceinline__ void IssueQuads(const int32_t *__restrict__ colInd, c
         const int32_t k = (u * kBlockThreads + static_cast<int32_t>(threadIdx.x)) * 4;
         if (k + 4 <= count) {
             q[u].col = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(colInd + k));
-            if constexpr (std::is_same<ValT, float>::value) {
-                const Float4U v = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(vals + k));
-                q[u].val[0] = v.x;
-                q[u].val[1] = v.y;
-                q[u].val[2] = v.z;
-                q[u].val[3] = v.w;
+            // The four values as one load, whatever their type (four 2-byte loads a quad cost the fp16 Laplacian
+            // more than the bytes they save: 45.9 us against 41.3 us in fp32).
+            static_assert(sizeof(ValT) == 4 || sizeof(ValT) == 2, "values of 2 or 4 bytes");
+            if constexpr (sizeof(ValT) == 4) {
+                const Int4U v = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(vals + k));
+                __builtin_memcpy(q[u].val, &v, 16);
             } else {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    q[u].val[i] = LoadStream(vals + k + i);
-                }
+                const Short4U v = __builtin_nontemporal_load(reinterpret_cast<const Short4U *>(vals + k));
+                __builtin_memcpy(q[u].val, &v, 8);
             }
         } else {
 #pragma unroll
