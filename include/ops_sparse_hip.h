@@ -98,7 +98,8 @@ typedef struct OpsparseSpmvPlan {
                               colInd / csrValues, panel by panel, with the panel's x in LDS */
     int32_t numDeferredLongRows; /* BLOCKED_GATHER: those of them that sit more than 64 to a row block: a third kernel,
                               a wavefront a row, adds their partial sums up instead of the block's workgroup */
-    int32_t reserved;
+    int32_t valueType;     /* BLOCKED_GATHER: the OPSPARSE_F32 / F16 / BF16 the layout was built from; launches must
+                              bring values and x of that type (and an fp32 y) */
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */
@@ -161,7 +162,7 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
                                      OpsparseSpmvPlan *plan, void *stream);
 
 /*
- * BLOCKED_GATHER analysis (fp32): bytes of the workspace, or 0 when the family does
+ * BLOCKED_GATHER analysis (fp32; fp16 / bf16 values and x with frozen values): bytes of the workspace, or 0 when the family does
  * not apply (x must have more than 2^20 and at most 2^25 elements, the matrix at least
  * two million entries, and a (panel, row block) chunk at least 32 entries on average).  transpose != 0 builds the layout of
  * y = alpha * A^T * x + beta * y instead: panels over the rows of A, blocks over its
@@ -178,12 +179,17 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
  * and every launch takes the values from the csrValues argument (8 more bytes of traffic per entry, all
  * streamed), and for the long rows the column indices from colInd as well: such a plan never goes stale when
  * values change; rowOffsets / colInd must be the arrays of the analysis.
+ * OPSPARSE_BLOCKED_VALUES_F16 / _BF16: csrValues (and, at the launches, x) are fp16 / bf16 instead of fp32; the
+ * layout keeps the values as fp32, which holds them exactly, and the first kernel widens x while it loads a
+ * panel's slice.  Not together with OPSPARSE_BLOCKED_LIVE_VALUES (OPSPARSE_E_UNSUPPORTED); y stays fp32.
  */
 #define OPSPARSE_BLOCKED_TRANSPOSE 1
 #define OPSPARSE_BLOCKED_LIVE_VALUES 2
+#define OPSPARSE_BLOCKED_VALUES_F16 4
+#define OPSPARSE_BLOCKED_VALUES_BF16 8
 size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t flags);
 size_t opsparse_spmv_csr_blocked_resident_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t flags);
-int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
+int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
                                       int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
                                       size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream);
 

@@ -139,9 +139,10 @@ struct RestoredChoice {
     size_t bytes;
     bool liveValues;  // BLOCKED_GATHER only: the layout holds no values, every call takes the caller's
 };
-RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose);
-int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const float *values, int64_t rows,
-                    int64_t cols, int64_t nnz, bool transpose, bool liveValues, void *buffer, size_t bytes,
-                    OpsparseSpmvPlan *plan, void *stream);
+// valueType: the OPSPARSE_* type of the values and of x (fp16 and bf16: BLOCKED_GATHER with frozen values only).
+RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose, int32_t valueType);
+int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const void *values,
+                    int32_t valueType, int64_t rows, int64_t cols, int64_t nnz, bool transpose, bool liveValues,
+                    void *buffer, size_t bytes, OpsparseSpmvPlan *plan, void *stream);
 
 }  // namespace opsparse

@@ -437,10 +437,16 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedLongDeferKernel(const in
     }
 }
 
+// A value or an element of x as the layout keeps it: fp32 (exact for fp16 and bf16).
+__device__ __forceinline__ float AsFloat(float v) { return v; }
+__device__ __forceinline__ float AsFloat(Half v) { return static_cast<float>(v); }
+__device__ __forceinline__ float AsFloat(Bf16 v) { return Bf16ToFloat(v); }
+
 // Values and local row indices into (block, panel) order.
+template <typename ValT>
 __global__ __launch_bounds__(kBlockThreads) void BlockedScatterKernel(
     const int32_t *__restrict__ pos, const int32_t *__restrict__ rowOfSrc, const int32_t *__restrict__ chunkKey,
-    const float *__restrict__ vals, const int32_t *__restrict__ srcStart,
+    const ValT *__restrict__ vals, const int32_t *__restrict__ srcStart,
     const int32_t *__restrict__ dstStart, const int32_t *__restrict__ blockRow, int64_t nnz, int32_t P, int32_t B,
     float *__restrict__ valD, uint16_t *__restrict__ rowLocal, int32_t *__restrict__ dstOfPos,
     float *__restrict__ longVals, uint16_t *__restrict__ longRowOf, const int32_t *__restrict__ longBefore)
@@ -452,7 +458,7 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedScatterKernel(
             if (longVals != nullptr) {
                 // an entry of a long row, frozen values: its value and the number of its row among the long rows
                 // beside its local column, all three at its place in the sorted order
-                longVals[i] = vals[pos[i]];
+                longVals[i] = AsFloat(vals[pos[i]]);
                 longRowOf[i] = static_cast<uint16_t>(longBefore[rowOfSrc[i]] - 1);
             }
             continue;
@@ -460,7 +466,7 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedScatterKernel(
         const int32_t p = key / B, b = key % B;
         const int64_t dst = i - srcStart[key] + dstStart[static_cast<int64_t>(b) * P + p];
         if (valD != nullptr) {
-            valD[dst] = vals[pos[i]];
+            valD[dst] = AsFloat(vals[pos[i]]);
         }
         if (dstOfPos != nullptr) {
             dstOfPos[pos[i]] = static_cast<int32_t>(dst);
@@ -668,9 +674,9 @@ __device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, c
 // fp64 accumulator a row in LDS, kLongTile rows at a time ([.. + l] is where row l starts).
 constexpr int kLongBatch = 4;  // groups of 4 long entries a lane has in flight (frozen values)
 
-template <bool LongSorted>
+template <bool LongSorted, typename XT>
 __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint16_t *__restrict__ colLocal,
-                                                                     const float *__restrict__ x,
+                                                                     const XT *__restrict__ x,
                                                                      float *__restrict__ xg,
                                                                      const int32_t *__restrict__ srcStart,
                                                                      int64_t cols, int32_t B, int32_t splits,
@@ -693,13 +699,35 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint1
     const int64_t c0 = p << kPanelLog;
     const int64_t cn = cols - c0 < kPanelCols ? cols - c0 : kPanelCols;
     const int64_t a = srcStart[p * B], e = srcStart[(p + 1) * B];
-    const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
-    for (int64_t i = tid * 4; i < cn; i += kBlkThreads * 4) {
-        if (vec && i + 4 <= cn) {
-            *reinterpret_cast<Float4 *>(xs + i) = *reinterpret_cast<const Float4 *>(x + c0 + i);
-        } else {
-            for (int64_t k = i; k < cn && k < i + 4; ++k) {
-                xs[k] = x[c0 + k];
+    if constexpr (std::is_same<XT, float>::value) {
+        const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+        for (int64_t i = tid * 4; i < cn; i += kBlkThreads * 4) {
+            if (vec && i + 4 <= cn) {
+                *reinterpret_cast<Float4 *>(xs + i) = *reinterpret_cast<const Float4 *>(x + c0 + i);
+            } else {
+                for (int64_t k = i; k < cn && k < i + 4; ++k) {
+                    xs[k] = x[c0 + k];
+                }
+            }
+        }
+    } else {
+        // fp16 / bf16 x (frozen values only): widened once, here; the panel's slice starts at a multiple of 2^15
+        // elements, so 8-byte loads are aligned where x is
+        const bool vec = (reinterpret_cast<uintptr_t>(x) & 7) == 0;
+        for (int64_t i = tid * 4; i < cn; i += kBlkThreads * 4) {
+            if (vec && i + 4 <= cn) {
+                XT four[4];
+                *reinterpret_cast<uint2 *>(four) = *reinterpret_cast<const uint2 *>(x + c0 + i);
+                Float4 f;
+                f.x = AsFloat(four[0]);
+                f.y = AsFloat(four[1]);
+                f.z = AsFloat(four[2]);
+                f.w = AsFloat(four[3]);
+                *reinterpret_cast<Float4 *>(xs + i) = f;
+            } else {
+                for (int64_t k = i; k < cn && k < i + 4; ++k) {
+                    xs[k] = AsFloat(x[c0 + k]);
+                }
             }
         }
     }
@@ -1395,8 +1423,13 @@ uint32_t GridOf(int64_t items, int64_t perBlock, int64_t cap)
 
 }  // namespace
 
-int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
+// valType: the type of the caller's values and of x (OPSPARSE_F32 / F16 / BF16); y is fp32.  fp16 and bf16 are served
+// by a layout with frozen values only (they sit in the layout as fp32, and phase 1 widens x as it loads the slice).
+int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valType)
 {
+    if (plan.valueType != valType || (valType != OPSPARSE_F32 && plan.liveValues != 0)) {
+        return OPSPARSE_E_INVALID;  // the plan was made for values of another type
+    }
     // a.rows outputs, a.cols inputs: the caller has exchanged them for op(A) = A^T
     const BlockedLayout l = MakeBlockedLayout(a.rows, a.cols, a.nnz, plan.transposed != 0, plan.liveValues != 0);
     if (l.P == 0 || plan.numPanels != l.P || plan.numRowBlocks != l.B) {
@@ -1424,16 +1457,28 @@ int LaunchBlockedF32(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
     }
     const int32_t *header = longRows ? ints(0) : nullptr;
     auto *longPartial = reinterpret_cast<double *>(base + l.longPartialOff);
+    auto gather = [&](auto longSorted, auto xTag) {
+        constexpr bool kSorted = decltype(longSorted)::value;
+        using XT = decltype(xTag);
+        hipLaunchKernelGGL((SpmvBlockGatherKernel<kSorted, XT>), dim3(static_cast<uint32_t>(l.P) * splits),
+                           dim3(kBlkThreads), 0, a.stream, colLocal, static_cast<const XT *>(a.x), xg, ints(l.srcStartOff),
+                           a.cols, l.B, splits, header, ints(l.longChunkOff), a.colInd,
+                           static_cast<const float *>(kSorted ? nullptr : a.vals), a.nnz, l.P, l.maxLong,
+                           kSorted ? rowLocal + LongRowOfShift(l) : static_cast<const uint16_t *>(nullptr), longPartial);
+    };
+    auto gatherTyped = [&](auto longSorted) {
+        if (valType == OPSPARSE_F16) {
+            gather(longSorted, Half{});
+        } else if (valType == OPSPARSE_BF16) {
+            gather(longSorted, Bf16{});
+        } else {
+            gather(longSorted, float{});
+        }
+    };
     if (plan.liveValues != 0 || !longRows) {
-        hipLaunchKernelGGL(SpmvBlockGatherKernel<false>, dim3(static_cast<uint32_t>(l.P) * splits), dim3(kBlkThreads), 0,
-                           a.stream, colLocal, static_cast<const float *>(a.x), xg, ints(l.srcStartOff), a.cols, l.B, splits,
-                           header, ints(l.longChunkOff), a.colInd, static_cast<const float *>(a.vals), a.nnz, l.P,
-                           l.maxLong, static_cast<const uint16_t *>(nullptr), longPartial);
+        gatherTyped(std::false_type{});  // (frozen values without long rows: nothing of the caller's arrays is read)
     } else {
-        hipLaunchKernelGGL(SpmvBlockGatherKernel<true>, dim3(static_cast<uint32_t>(l.P) * splits), dim3(kBlkThreads), 0,
-                           a.stream, colLocal, static_cast<const float *>(a.x), xg, ints(l.srcStartOff), a.cols, l.B, splits,
-                           header, ints(l.longChunkOff), a.colInd, static_cast<const float *>(a.vals), a.nnz, l.P,
-                           l.maxLong, rowLocal + LongRowOfShift(l), longPartial);
+        gatherTyped(std::true_type{});
     }
 #define OPSPARSE_BLOCK_REDUCE_LIVE(SHORT)                                                                           \
     hipLaunchKernelGGL((SpmvBlockReduceKernel<true, SHORT>), dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads), 0,    \
@@ -1484,7 +1529,7 @@ size_t opsparse_spmv_csr_blocked_resident_bytes(int64_t rows, int64_t cols, int6
                                   : MakeBlockedLayout(rows, cols, nnz, false, live)).resident);
 }
 
-int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const float *csrValues,
+int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
                                       int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
                                       size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream)
 {
@@ -1492,6 +1537,12 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
         return OPSPARSE_E_INVALID;
     }
     const bool transposed = (flags & OPSPARSE_BLOCKED_TRANSPOSE) != 0, live = (flags & OPSPARSE_BLOCKED_LIVE_VALUES) != 0;
+    const int32_t valueType = (flags & OPSPARSE_BLOCKED_VALUES_F16) != 0    ? OPSPARSE_F16
+                              : (flags & OPSPARSE_BLOCKED_VALUES_BF16) != 0 ? OPSPARSE_BF16
+                                                                            : OPSPARSE_F32;
+    if (valueType != OPSPARSE_F32 && live) {
+        return OPSPARSE_E_UNSUPPORTED;  // live values are read as fp32 by the launches
+    }
     const int64_t outputs = transposed ? cols : rows;
     const BlockedLayout l = transposed ? MakeBlockedLayout(cols, rows, nnz, true, live)
                                        : MakeBlockedLayout(rows, cols, nnz, false, live);
@@ -1625,11 +1676,21 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
         hipLaunchKernelGGL(BlockedLongDeferKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
                            ints(l.longFirstOff), l.B, ints(l.longDeferredOff), status);
     }
-    hipLaunchKernelGGL(BlockedScatterKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
-                       pos, rowOfSrc, chunkKey, csrValues, srcStart, dstStart, blockRow, nnz, l.P, l.B, live ? nullptr : valD, rowLocal,
-                       live ? ints(l.dstOfPosOff) : nullptr,
-                       longBefore != nullptr && !live ? reinterpret_cast<float *>(base + l.xgOff) : nullptr,
-                       rowLocal + LongRowOfShift(l), longBefore);
+    auto scatter = [&](auto tag) {
+        using ValT = decltype(tag);
+        hipLaunchKernelGGL(BlockedScatterKernel<ValT>, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
+                           pos, rowOfSrc, chunkKey, static_cast<const ValT *>(csrValues), srcStart, dstStart, blockRow, nnz,
+                           l.P, l.B, live ? nullptr : valD, rowLocal, live ? ints(l.dstOfPosOff) : nullptr,
+                           longBefore != nullptr && !live ? reinterpret_cast<float *>(base + l.xgOff) : nullptr,
+                           rowLocal + LongRowOfShift(l), longBefore);
+    };
+    if (valueType == OPSPARSE_F16) {
+        scatter(Half{});
+    } else if (valueType == OPSPARSE_BF16) {
+        scatter(Bf16{});
+    } else {
+        scatter(float{});
+    }
     if (live) {
         // (the blocks are alike in size by construction and are taken in row order)
     } else if (l.B <= kRankedBlocks) {
@@ -1687,6 +1748,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     p.entryWindow = l.window;
     p.transposed = transposed ? 1 : 0;
     p.liveValues = liveKind;
+    p.valueType = valueType;
     p.numDeferredLongRows = tail[1];
     p.numLongRows = head[1];
     p.rows = rows;

@@ -108,17 +108,40 @@ aclsparseStatus_t ValidateData(SpmvCall *c, aclDataType computeType)
 // arrays (a sample of the column indices, one short kernel and a synchronisation), so they agree on the size.
 using Restored = opsparse::RestoredChoice;
 
+// The OPSPARSE_* type of values and x where a re-stored layout can hold them, else -1.
+int32_t RestoredValueType(aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDescr_t vecX)
+{
+    if (matA->valueType != vecX->valueType) {
+        return -1;
+    }
+    switch (matA->valueType) {
+        case ACL_FLOAT:
+            return OPSPARSE_F32;
+        case ACL_FLOAT16:
+            return OPSPARSE_F16;
+        case ACL_BF16:
+            return OPSPARSE_BF16;
+        default:
+            return -1;
+    }
+}
+
 Restored RestoredLayout(aclsparseHandle_t handle, aclsparseOperation_t opA, aclsparseConstSpMatDescr_t matA,
                         aclsparseConstDnVecDescr_t vecX, aclsparseConstDnVecDescr_t vecY, aclDataType computeType,
                         aclsparseSpMVAlg_t alg)
 {
-    if (computeType != ACL_FLOAT || matA->valueType != ACL_FLOAT || vecX->valueType != ACL_FLOAT ||
-        vecY->valueType != ACL_FLOAT) {
+    // fp32 throughout, or fp16 / bf16 values and x with an fp32 y (the frozen blocked-gather layout only: it keeps
+    // the values as fp32 and widens x as it loads it)
+    const int32_t valueType = RestoredValueType(matA, vecX);
+    if (computeType != ACL_FLOAT || vecY->valueType != ACL_FLOAT || valueType < 0) {
         return {0, 0, false};
     }
     const bool transpose = opA != ACL_SPARSE_OP_NON_TRANSPOSE;
     if (alg == ACL_SPARSE_SPMV_CSR_ALG2) {
-        return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz, transpose);
+        return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz, transpose, valueType);
+    }
+    if (valueType != OPSPARSE_F32) {
+        return {0, 0, false};
     }
     static const bool off = std::getenv("OPS_SPARSE_SPMV_NO_DEFAULT_BLOCKED") != nullptr ||
                             std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") != nullptr;
@@ -210,7 +233,7 @@ const OpsparseSpmvPlan *RowsSeen(aclsparseHandle_t handle, aclsparseConstSpMatDe
 
 namespace opsparse {
 
-RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose)
+RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose, int32_t valueType)
 {
     if (std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") == nullptr) {
         const size_t blocked = opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, transpose ? 1 : 0);
@@ -218,16 +241,18 @@ RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool 
             return {OPSPARSE_SPMV_BLOCKED_GATHER, blocked, false};
         }
     }
-    const size_t panels = transpose ? 0 : opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz);
+    // (the column panels hold and read fp32 only)
+    const size_t panels =
+        transpose || valueType != OPSPARSE_F32 ? 0 : opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz);
     if (panels > 0) {
         return {OPSPARSE_SPMV_COLUMN_PANELS, panels, false};
     }
     return {0, 0, false};
 }
 
-int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const float *values, int64_t rows,
-                    int64_t cols, int64_t nnz, bool transpose, bool liveValues, void *buffer, size_t bytes,
-                    OpsparseSpmvPlan *plan, void *stream)
+int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const void *values,
+                    int32_t valueType, int64_t rows, int64_t cols, int64_t nnz, bool transpose, bool liveValues,
+                    void *buffer, size_t bytes, OpsparseSpmvPlan *plan, void *stream)
 {
     // A matrix whose gathers stay near the diagonal (a mesh, a band) keeps x in cache under the row-wise kernels:
     // those are then faster than any re-stored layout (the 2048 x 2048 Laplacian: 41 us against 91 us).  With some
@@ -250,10 +275,17 @@ int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *co
     if (kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {
         return opsparse_spmv_csr_blocked_analyse(rowOffsets, colInd, values, rows, cols, nnz,
                                                  (transpose ? OPSPARSE_BLOCKED_TRANSPOSE : 0) |
-                                                     (liveValues ? OPSPARSE_BLOCKED_LIVE_VALUES : 0),
+                                                     (liveValues ? OPSPARSE_BLOCKED_LIVE_VALUES : 0) |
+                                                     (valueType == OPSPARSE_F16    ? OPSPARSE_BLOCKED_VALUES_F16
+                                                      : valueType == OPSPARSE_BF16 ? OPSPARSE_BLOCKED_VALUES_BF16
+                                                                                   : 0),
                                                  buffer, bytes, plan, stream);
     }
-    return opsparse_spmv_csr_panels_analyse(rowOffsets, colInd, values, rows, cols, nnz, buffer, bytes, plan, stream);
+    if (valueType != OPSPARSE_F32) {
+        return OPSPARSE_E_UNSUPPORTED;
+    }
+    return opsparse_spmv_csr_panels_analyse(rowOffsets, colInd, static_cast<const float *>(values), rows, cols, nnz,
+                                            buffer, bytes, plan, stream);
 }
 
 }  // namespace opsparse
@@ -317,8 +349,8 @@ aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOpe
     int rc;
     if (restored.kernel != 0) {
         rc = opsparse::AnalyseRestored(restored.kernel, static_cast<const int32_t *>(matA->rowOffsets),
-                                       static_cast<const int32_t *>(matA->colInd),
-                                       static_cast<const float *>(matA->values), matA->rows, matA->cols, matA->nnz,
+                                       static_cast<const int32_t *>(matA->colInd), matA->values,
+                                       RestoredValueType(matA, vecX), matA->rows, matA->cols, matA->nnz,
                                        opA != ACL_SPARSE_OP_NON_TRANSPOSE, restored.liveValues, externalBuffer,
                                        restored.bytes, &plan, handle->stream);
     } else {

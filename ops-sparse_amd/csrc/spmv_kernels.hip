@@ -1436,10 +1436,14 @@ int RunPlanned(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
                 return OPSPARSE_E_UNSUPPORTED;  // the panel copy holds fp32 values
             }
         case OPSPARSE_SPMV_BLOCKED_GATHER:
-            if constexpr (std::is_same<ValT, float>::value && std::is_same<OutT, float>::value) {
-                return LaunchBlockedF32(a, plan);
+            if constexpr (std::is_same<OutT, float>::value && std::is_same<AccT, double>::value &&
+                          (std::is_same<ValT, float>::value || std::is_same<ValT, Half>::value ||
+                           std::is_same<ValT, Bf16>::value)) {
+                return LaunchBlocked(a, plan, std::is_same<ValT, Half>::value   ? OPSPARSE_F16
+                                              : std::is_same<ValT, Bf16>::value ? OPSPARSE_BF16
+                                                                                : OPSPARSE_F32);
             } else {
-                return OPSPARSE_E_UNSUPPORTED;  // the re-stored copy holds fp32 values
+                return OPSPARSE_E_UNSUPPORTED;  // the re-stored copy holds fp32 values, y is written as fp32
             }
         default:
             return OPSPARSE_E_INVALID;
@@ -2022,13 +2026,14 @@ int opsparse_spmv_csr_launch_zy(const OpsparseSpmvPlan *plan, int32_t transpose,
         return OPSPARSE_E_INVALID;  // the re-stored layout serves the op(A) it was built for
     }
     if (transpose && plan != nullptr && plan->kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {
-        if (computeIsInt || valType != OPSPARSE_F32 || outType != OPSPARSE_F32) {
+        if (computeIsInt || (valType != OPSPARSE_F32 && valType != OPSPARSE_F16 && valType != OPSPARSE_BF16) ||
+            outType != OPSPARSE_F32) {
             return OPSPARSE_E_UNSUPPORTED;
         }
         SpmvArgs t = a;  // the columns of A are the outputs, its rows the inputs
         t.rows = cols;
         t.cols = rows;
-        return LaunchBlockedF32(t, *plan);
+        return LaunchBlocked(t, *plan, valType);
     }
     if (transpose) {
         if (computeIsInt) {

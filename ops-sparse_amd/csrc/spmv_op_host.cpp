@@ -138,7 +138,7 @@ opsparse::RestoredChoice RestoredLayout(aclsparseConstSpMatDescr_t matA)
     if (matA->rowOffsetsType != ACL_SPARSE_INDEX_32I || matA->idxBase != ACL_SPARSE_INDEX_BASE_ZERO) {
         return {0, 0};
     }
-    return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz, false);
+    return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz, false, OPSPARSE_F32);
 }
 
 aclsparseStatus_t FromLaunch(int rc)
@@ -257,9 +257,9 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
             const int rc =
                 restored.kernel != 0 && d->colInd != nullptr && d->values != nullptr
                     ? opsparse::AnalyseRestored(restored.kernel, static_cast<const int32_t *>(d->rowOffsets),
-                                                static_cast<const int32_t *>(d->colInd),
-                                                static_cast<const float *>(d->values), d->rows, d->cols, d->nnz, false,
-                                                false, buffer, restored.bytes, &d->plan, handle->stream)
+                                                static_cast<const int32_t *>(d->colInd), d->values, OPSPARSE_F32,
+                                                d->rows, d->cols, d->nnz, false, false, buffer, restored.bytes,
+                                                &d->plan, handle->stream)
                     : opsparse_spmv_csr_analyse(Offsets32(d), d->rows, d->cols, d->nnz, buffer,
                                                 opsparse_spmv_csr_workspace_bytes(d->rows, d->nnz), OPSPARSE_SPMV_AUTO,
                                                 &d->plan, handle->stream);

@@ -374,6 +374,68 @@ def test_blocked_gather_transposed(osa, gpu_ctx, rows, cols):
     assert oracle.max_rel_err(d_yn.cpu().numpy(), gold) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("transpose", [False, True])
+def test_blocked_gather_csr_alg2_half_precision_values(osa, gpu_ctx, dtype, transpose):
+    """fp16 / bf16 values and x with an fp32 y under ACL_SPARSE_SPMV_CSR_ALG2: the same re-stored layout (it keeps
+    the values as fp32, which holds them exactly, and widens x as it loads a panel's slice), long rows included;
+    against the fp64 oracle on the rounded inputs at the fp32 bar.  A launch with values of another type than the
+    layout was built from is refused by the raw layer."""
+    dev, stream, handle = gpu_ctx
+    rows, cols = (1_300_000, 60_000) if transpose else (60_000, 3_000_000)
+    rng = np.random.default_rng(rows % 977 + (1 if dtype == torch.float16 else 2))
+    if transpose:
+        lengths = rng.integers(0, 6, rows)
+        lengths[[5, rows // 3]] = [40_000, 9_000]
+        rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+        colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)
+        val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+        x, y0 = rng.uniform(-1, 1, rows).astype(np.float32), rng.uniform(-1, 1, cols).astype(np.float32)
+    else:
+        rowptr, colind, val, x, y0 = _wide_problem(rows, cols, 5, per_row=80,
+                                                   long_rows=((7, 90_000), (rows // 2, 1), (rows - 1, 30_000), (100, 1024)))
+    rnd = lambda a: torch.from_numpy(a).to(dtype).float().numpy()
+    val, x = rnd(val), rnd(x)
+    L = osa.lib()
+    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 1 if transpose else 0)
+    assert need > 0
+    d_rp, d_ci = to_dev(rowptr, dev), to_dev(colind, dev)
+    d_val, d_x, d_y = to_dev(val, dev, dtype), to_dev(x, dev, dtype), to_dev(y0, dev)
+    A = osa.Csr(rows, cols, d_rp, d_ci, d_val)
+    op = osa.SpmvOp(handle, A, osa.DnVec(d_x), osa.DnVec(d_y), alg=osa.ACL_SPARSE_SPMV_CSR_ALG2,
+                    op=osa.ACL_SPARSE_OP_TRANSPOSE if transpose else osa.ACL_SPARSE_OP_NON_TRANSPOSE)
+    assert op.buffer.numel() >= need                         # the layout, not the ordinary plan's few hundred KB
+    golden = oracle.spmv_trans_f64 if transpose else oracle.spmv_f64
+    for alpha, beta in ((1.0, 0.0), (-2.0, 0.75)):
+        d_y.copy_(torch.from_numpy(y0))
+        op(alpha, beta)
+        stream.synchronize()
+        gold = golden(rows, cols, rowptr, colind, val, x, y0, alpha, beta)
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+    # raw layer: the plan remembers the type it was built from
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    plan = osa.OpsparseSpmvPlan()
+    flag = (4 if dtype == torch.float16 else 8) | (1 if transpose else 0)
+    assert L.opsparse_spmv_csr_blocked_analyse(d_rp.data_ptr(), d_ci.data_ptr(), d_val.data_ptr(), rows, cols, colind.size,
+                                               flag, ws.data_ptr(), need, ctypes.byref(plan), sp) == 0
+    want = osa.OPSPARSE_F16 if dtype == torch.float16 else osa.OPSPARSE_BF16
+    assert plan.kernel == osa.OPSPARSE_SPMV_BLOCKED_GATHER and plan.valueType == want and plan.liveValues == 0
+    one, zero = osa.OpsparseScalar(1.0, None, 0, 0), osa.OpsparseScalar(0.0, None, 0, 0)
+    launch = lambda vt, v, xx: L.opsparse_spmv_csr_launch(ctypes.byref(plan), 1 if transpose else 0, d_rp.data_ptr(),
+                                                          d_ci.data_ptr(), v.data_ptr(), xx.data_ptr(), d_y.data_ptr(), rows,
+                                                          cols, colind.size, one, zero, vt, osa.OPSPARSE_F32, 0,
+                                                          ws.data_ptr(), need, sp)
+    assert launch(want, d_val, d_x) == 0
+    stream.synchronize()
+    assert oracle.max_rel_err(d_y.cpu().numpy(), golden(rows, cols, rowptr, colind, val, x, y0, 1.0, 0.0)) <= 1e-5
+    f_val, f_x = to_dev(val, dev), to_dev(x, dev)
+    assert launch(osa.OPSPARSE_F32, f_val, f_x) != 0         # fp32 operands with a plan built from 2-byte values
+    # and live values are fp32 only
+    assert L.opsparse_spmv_csr_blocked_analyse(d_rp.data_ptr(), d_ci.data_ptr(), d_val.data_ptr(), rows, cols, colind.size,
+                                               flag | 2, ws.data_ptr(), need, ctypes.byref(plan), sp) != 0
+
+
 @pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
 def test_blocked_gather_random_shapes(osa, gpu_ctx, seed):
     """Seeded random shapes, both op(A): uniform short rows, power-law rows with a few of several hundred thousand
