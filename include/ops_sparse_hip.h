@@ -162,7 +162,7 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
                                      OpsparseSpmvPlan *plan, void *stream);
 
 /*
- * BLOCKED_GATHER analysis (fp32; fp16 / bf16 values and x with frozen values): bytes of the workspace, or 0 when the family does
+ * BLOCKED_GATHER analysis (fp32, or fp16 / bf16 values and x with an fp32 y): bytes of the workspace, or 0 when the family does
  * not apply (x must have more than 2^20 and at most 2^25 elements, the matrix at least
  * two million entries, and a (panel, row block) chunk at least 32 entries on average).  transpose != 0 builds the layout of
  * y = alpha * A^T * x + beta * y instead: panels over the rows of A, blocks over its
@@ -180,8 +180,8 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
  * streamed), and for the long rows the column indices from colInd as well: such a plan never goes stale when
  * values change; rowOffsets / colInd must be the arrays of the analysis.
  * OPSPARSE_BLOCKED_VALUES_F16 / _BF16: csrValues (and, at the launches, x) are fp16 / bf16 instead of fp32; the
- * layout keeps the values as fp32, which holds them exactly, and the first kernel widens x while it loads a
- * panel's slice.  Not together with OPSPARSE_BLOCKED_LIVE_VALUES (OPSPARSE_E_UNSUPPORTED); y stays fp32.
+ * layout keeps frozen values as fp32, which holds them exactly, live ones are widened where the launches read
+ * them, and the first kernel widens x while it loads a panel's slice.  y stays fp32.
  */
 #define OPSPARSE_BLOCKED_TRANSPOSE 1
 #define OPSPARSE_BLOCKED_LIVE_VALUES 2

@@ -442,6 +442,21 @@ __device__ __forceinline__ float AsFloat(float v) { return v; }
 __device__ __forceinline__ float AsFloat(Half v) { return static_cast<float>(v); }
 __device__ __forceinline__ float AsFloat(Bf16 v) { return Bf16ToFloat(v); }
 
+// Four consecutive values of the caller's array as fp32, in one load (fp32: at any 4-byte-aligned address; fp16 /
+// bf16: at any 2-byte-aligned one).
+template <typename ValT>
+__device__ __forceinline__ Float4U LoadFourValues(const ValT *p)
+{
+    if constexpr (std::is_same<ValT, float>::value) {
+        return __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(p));
+    } else {
+        const Short4U raw = __builtin_nontemporal_load(reinterpret_cast<const Short4U *>(p));
+        ValT four[4];
+        __builtin_memcpy(four, &raw, 8);
+        return Float4U{AsFloat(four[0]), AsFloat(four[1]), AsFloat(four[2]), AsFloat(four[3])};
+    }
+}
+
 // Values and local row indices into (block, panel) order.
 template <typename ValT>
 __global__ __launch_bounds__(kBlockThreads) void BlockedScatterKernel(
@@ -578,8 +593,8 @@ __global__ __launch_bounds__(kBlkThreads) void BlockedShortPositionsKernel(const
 // A block of more than kRefreshSpan positions reads its entries once per window.  [e0, e1) here is a piece of the
 // block's entries between two long rows (whose own entries are skipped); Short: the positions are the 16-bit ones
 // of BlockedShortPositionsKernel, blockE0 and dBeg the block's first entry and first position.
-template <bool Short>
-__device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, const int32_t *__restrict__ dstOfPos,
+template <bool Short, typename ValT>
+__device__ __forceinline__ void FillLiveWindow(const ValT *__restrict__ vals, const int32_t *__restrict__ dstOfPos,
                                                int32_t e0, int32_t e1, int32_t w0, uint32_t span, float *win, int tid,
                                                int32_t blockE0, int32_t dBeg)
 {
@@ -600,7 +615,7 @@ __device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, c
         for (int32_t i = e0 + tid; i < e1; i += kBlkThreads) {
             const uint32_t at = place(i);
             if (at < span) {
-                win[at] = vals[i];
+                win[at] = AsFloat(vals[i]);
             }
         }
         return;
@@ -610,11 +625,11 @@ __device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, c
         if ((tid < 4 && i < g0) || (tid >= 4 && i < e1)) {
             const uint32_t at = place(i);
             if (at < span) {
-                win[at] = vals[i];
+                win[at] = AsFloat(vals[i]);
             }
         }
     }
-    const bool vecVals = (reinterpret_cast<uintptr_t>(vals) & 15) == 0;
+    const bool vecVals = (reinterpret_cast<uintptr_t>(vals) & (4 * sizeof(ValT) - 1)) == 0;
     // kRefreshBatch groups in flight per lane: loads first (clamped to the last group), then the LDS writes
     constexpr int kRefreshBatch = 6;  // (a block of kLiveWindow entries in one turn)
     for (int32_t i0 = g0 + tid * 4; i0 < g1; i0 += kBlkThreads * 4 * kRefreshBatch) {
@@ -631,9 +646,9 @@ __device__ __forceinline__ void FillLiveWindow(const float *__restrict__ vals, c
                 d[u] = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(dstOfPos + i));
             }
             if (vecVals) {
-                v[u] = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(vals + i));
+                v[u] = LoadFourValues(vals + i);
             } else {
-                v[u] = Float4U{vals[i], vals[i + 1], vals[i + 2], vals[i + 3]};
+                v[u] = Float4U{AsFloat(vals[i]), AsFloat(vals[i + 1]), AsFloat(vals[i + 2]), AsFloat(vals[i + 3])};
             }
         }
 #pragma unroll
@@ -683,7 +698,7 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint1
                                                                      const int32_t *__restrict__ header,
                                                                      const int32_t *__restrict__ longChunk,
                                                                      const int32_t *__restrict__ colInd,
-                                                                     const float *__restrict__ vals, int64_t nnz,
+                                                                     const XT *__restrict__ vals, int64_t nnz,
                                                                      int32_t P, int32_t maxLong,
                                                                      const uint16_t *__restrict__ longRowOf,
                                                                      double *__restrict__ longPartial)
@@ -711,7 +726,7 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint1
             }
         }
     } else {
-        // fp16 / bf16 x (frozen values only): widened once, here; the panel's slice starts at a multiple of 2^15
+        // fp16 / bf16 x: widened once, here; the panel's slice starts at a multiple of 2^15
         // elements, so 8-byte loads are aligned where x is
         const bool vec = (reinterpret_cast<uintptr_t>(x) & 7) == 0;
         for (int64_t i = tid * 4; i < cn; i += kBlkThreads * 4) {
@@ -884,7 +899,7 @@ __global__ __launch_bounds__(kBlkThreads) void SpmvBlockGatherKernel(const uint1
                 at = at + 4 <= i1 ? at : static_cast<int64_t>(i1) - 4;
                 at = at < 0 ? 0 : at;
                 *c = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(colInd + at));
-                *v = __builtin_nontemporal_load(reinterpret_cast<const Float4U *>(vals + at));
+                *v = LoadFourValues(vals + at);
             };
             auto add = [&](int32_t i0, int32_t i1, int32_t q, const Int4U &c, const Float4U &v, double *sum) {
                 const int64_t own = i0 + 4 * static_cast<int64_t>(q);  // first entry of the group
@@ -1012,13 +1027,13 @@ constexpr int kRedThreads = kBlkThreads, kRedWaves = kRedThreads / kWave;
 // by window of kRefreshSpan positions (partDesc[partStart[block]] ..: entries, positions); the values of a window
 // are first collected in LDS from the caller's array, and the stream takes them from there.  Padding positions of
 // a window hold whatever LDS held: their products are formed and dropped.
-template <bool Live, bool Short>
+template <bool Live, bool Short, typename ValT>
 __global__ __launch_bounds__(kRedThreads) void SpmvBlockReduceKernel(
     const float *__restrict__ valD, const float *__restrict__ xg, const uint16_t *__restrict__ rowLocal,
     const int32_t *__restrict__ dstStart, const int32_t *__restrict__ srcStartT, int32_t P,
     const int32_t *__restrict__ blockOrder, const int32_t *__restrict__ blockRow, float *__restrict__ y,
     const float *__restrict__ yIn, OpsparseScalar alphaS, OpsparseScalar betaS, const int32_t *__restrict__ longFirst,
-    const int32_t *__restrict__ longRows, const double *__restrict__ longPartial, const float *__restrict__ vals,
+    const int32_t *__restrict__ longRows, const double *__restrict__ longPartial, const ValT *__restrict__ vals,
     const int32_t *__restrict__ dstOfPos, const int32_t *__restrict__ blockEntry, const int32_t *__restrict__ longSpan)
 {
     constexpr int kGroupSlots = Live ? kRefreshSpan / kWave : kMaxGroups;
@@ -1054,11 +1069,11 @@ __global__ __launch_bounds__(kRedThreads) void SpmvBlockReduceKernel(
         // the block's entries without those of its long rows
         int32_t cur = e0;
         for (int32_t l = l0; l < l1; ++l) {
-            FillLiveWindow<Short>(vals, dstOfPos, cur, longSpan[2 * l], w0, static_cast<uint32_t>(w1 - w0), win, tid, e0,
+            FillLiveWindow<Short, ValT>(vals, dstOfPos, cur, longSpan[2 * l], w0, static_cast<uint32_t>(w1 - w0), win, tid, e0,
                                   dBeg);
             cur = longSpan[2 * l + 1];
         }
-        FillLiveWindow<Short>(vals, dstOfPos, cur, e1, w0, static_cast<uint32_t>(w1 - w0), win, tid, e0, dBeg);
+        FillLiveWindow<Short, ValT>(vals, dstOfPos, cur, e1, w0, static_cast<uint32_t>(w1 - w0), win, tid, e0, dBeg);
     };
     if (Live && dBeg < dEnd) {
         fillWindow(dBeg, dEnd - dBeg > spanMax ? dBeg + spanMax : dEnd);
@@ -1423,11 +1438,12 @@ uint32_t GridOf(int64_t items, int64_t perBlock, int64_t cap)
 
 }  // namespace
 
-// valType: the type of the caller's values and of x (OPSPARSE_F32 / F16 / BF16); y is fp32.  fp16 and bf16 are served
-// by a layout with frozen values only (they sit in the layout as fp32, and phase 1 widens x as it loads the slice).
+// valType: the type of the caller's values and of x (OPSPARSE_F32 / F16 / BF16); y is fp32.  Frozen fp16 and bf16
+// values sit in the layout as fp32, live ones are widened where they are read, and phase 1 widens x as it loads
+// the slice.
 int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valType)
 {
-    if (plan.valueType != valType || (valType != OPSPARSE_F32 && plan.liveValues != 0)) {
+    if (plan.valueType != valType) {
         return OPSPARSE_E_INVALID;  // the plan was made for values of another type
     }
     // a.rows outputs, a.cols inputs: the caller has exchanged them for op(A) = A^T
@@ -1463,7 +1479,7 @@ int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valTy
         hipLaunchKernelGGL((SpmvBlockGatherKernel<kSorted, XT>), dim3(static_cast<uint32_t>(l.P) * splits),
                            dim3(kBlkThreads), 0, a.stream, colLocal, static_cast<const XT *>(a.x), xg, ints(l.srcStartOff),
                            a.cols, l.B, splits, header, ints(l.longChunkOff), a.colInd,
-                           static_cast<const float *>(kSorted ? nullptr : a.vals), a.nnz, l.P, l.maxLong,
+                           static_cast<const XT *>(kSorted ? nullptr : a.vals), a.nnz, l.P, l.maxLong,
                            kSorted ? rowLocal + LongRowOfShift(l) : static_cast<const uint16_t *>(nullptr), longPartial);
     };
     auto gatherTyped = [&](auto longSorted) {
@@ -1480,26 +1496,37 @@ int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valTy
     } else {
         gatherTyped(std::true_type{});
     }
-#define OPSPARSE_BLOCK_REDUCE_LIVE(SHORT)                                                                           \
-    hipLaunchKernelGGL((SpmvBlockReduceKernel<true, SHORT>), dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads), 0,    \
-                       a.stream, static_cast<const float *>(nullptr), xg, rowLocal, ints(l.dstStartOff),               \
-                       ints(l.srcStartTOff), l.P, ints(l.orderOff), ints(l.blockRowOff), static_cast<float *>(a.y),     \
-                       static_cast<const float *>(a.yIn), a.alpha, a.beta, longRows ? ints(l.longFirstOff) : nullptr,   \
-                       ints(l.longRowsOff), longPartial, static_cast<const float *>(a.vals), ints(l.dstOfPosOff),       \
-                       ints(l.blockEntryOff), ints(l.longSpanOff))
+    auto reduceLive = [&](auto shortTag, auto valTag) {
+        constexpr bool kShort = decltype(shortTag)::value;
+        using ValT = decltype(valTag);
+        hipLaunchKernelGGL((SpmvBlockReduceKernel<true, kShort, ValT>), dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads),
+                           0, a.stream, static_cast<const float *>(nullptr), xg, rowLocal, ints(l.dstStartOff),
+                           ints(l.srcStartTOff), l.P, ints(l.orderOff), ints(l.blockRowOff), static_cast<float *>(a.y),
+                           static_cast<const float *>(a.yIn), a.alpha, a.beta, longRows ? ints(l.longFirstOff) : nullptr,
+                           ints(l.longRowsOff), longPartial, static_cast<const ValT *>(a.vals), ints(l.dstOfPosOff),
+                           ints(l.blockEntryOff), ints(l.longSpanOff));
+    };
+    auto reduceLiveTyped = [&](auto shortTag) {
+        if (valType == OPSPARSE_F16) {
+            reduceLive(shortTag, Half{});
+        } else if (valType == OPSPARSE_BF16) {
+            reduceLive(shortTag, Bf16{});
+        } else {
+            reduceLive(shortTag, float{});
+        }
+    };
     if (plan.liveValues == kLiveShortPositions) {
-        OPSPARSE_BLOCK_REDUCE_LIVE(true);
+        reduceLiveTyped(std::true_type{});
     } else if (plan.liveValues != 0) {
-        OPSPARSE_BLOCK_REDUCE_LIVE(false);
+        reduceLiveTyped(std::false_type{});
     } else {
-        hipLaunchKernelGGL((SpmvBlockReduceKernel<false, false>), dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads), 0,
+        hipLaunchKernelGGL((SpmvBlockReduceKernel<false, false, float>), dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads), 0,
                            a.stream, valD, xg, rowLocal, ints(l.dstStartOff), ints(l.srcStartTOff), l.P, ints(l.orderOff),
                            ints(l.blockRowOff), static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha,
                            a.beta, longRows ? ints(l.longFirstOff) : nullptr, ints(l.longRowsOff), longPartial,
                            static_cast<const float *>(nullptr), static_cast<const int32_t *>(nullptr),
                            static_cast<const int32_t *>(nullptr), static_cast<const int32_t *>(nullptr));
     }
-#undef OPSPARSE_BLOCK_REDUCE_LIVE
     if (longRows && plan.numDeferredLongRows > 0) {
         constexpr int kRowsPerBlock = kBlockThreads / kWave;
         hipLaunchKernelGGL(SpmvLongRowSumKernel, dim3((plan.numLongRows + kRowsPerBlock - 1) / kRowsPerBlock),
@@ -1540,9 +1567,6 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     const int32_t valueType = (flags & OPSPARSE_BLOCKED_VALUES_F16) != 0    ? OPSPARSE_F16
                               : (flags & OPSPARSE_BLOCKED_VALUES_BF16) != 0 ? OPSPARSE_BF16
                                                                             : OPSPARSE_F32;
-    if (valueType != OPSPARSE_F32 && live) {
-        return OPSPARSE_E_UNSUPPORTED;  // live values are read as fp32 by the launches
-    }
     const int64_t outputs = transposed ? cols : rows;
     const BlockedLayout l = transposed ? MakeBlockedLayout(cols, rows, nnz, true, live)
                                        : MakeBlockedLayout(rows, cols, nnz, false, live);

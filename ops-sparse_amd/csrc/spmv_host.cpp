@@ -130,8 +130,8 @@ Restored RestoredLayout(aclsparseHandle_t handle, aclsparseOperation_t opA, acls
                         aclsparseConstDnVecDescr_t vecX, aclsparseConstDnVecDescr_t vecY, aclDataType computeType,
                         aclsparseSpMVAlg_t alg)
 {
-    // fp32 throughout, or fp16 / bf16 values and x with an fp32 y (the frozen blocked-gather layout only: it keeps
-    // the values as fp32 and widens x as it loads it)
+    // fp32 throughout, or fp16 / bf16 values and x with an fp32 y (the blocked-gather layout only: it keeps frozen
+    // values as fp32 and widens live ones, and x, where it reads them)
     const int32_t valueType = RestoredValueType(matA, vecX);
     if (computeType != ACL_FLOAT || vecY->valueType != ACL_FLOAT || valueType < 0) {
         return {0, 0, false};
@@ -139,9 +139,6 @@ Restored RestoredLayout(aclsparseHandle_t handle, aclsparseOperation_t opA, acls
     const bool transpose = opA != ACL_SPARSE_OP_NON_TRANSPOSE;
     if (alg == ACL_SPARSE_SPMV_CSR_ALG2) {
         return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz, transpose, valueType);
-    }
-    if (valueType != OPSPARSE_F32) {
-        return {0, 0, false};
     }
     static const bool off = std::getenv("OPS_SPARSE_SPMV_NO_DEFAULT_BLOCKED") != nullptr ||
                             std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") != nullptr;

@@ -90,6 +90,45 @@ def _with_long_rows(rows, cols, seed):
     return rowptr, colind, val, rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("short_positions", [True, False])
+def test_default_plan_with_half_precision_values(osa, gpu_ctx, dtype, short_positions, monkeypatch):
+    """fp16 / bf16 values and x with an fp32 y get the same default plan: the live layout reads the caller's 2-byte
+    values at every call (the short entries into the LDS window of their row block, the long rows' straight into
+    the sums of their panel) and widens x as it loads a panel's slice.  Values changed in place are followed."""
+    if not short_positions:
+        monkeypatch.setenv("OPS_SPARSE_BLOCKED_NO_SHORT_POSITIONS", "1")
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = 300_000, 1_400_000
+    rowptr, colind, val, x, y0 = _with_long_rows(rows, cols, 13)
+    rnd = lambda a: torch.from_numpy(a).to(dtype).float().numpy()
+    val, x = rnd(val), rnd(x)
+    nnz = colind.size
+    want = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    d_rp, d_ci = to_dev(rowptr, dev), to_dev(colind, dev)
+    vbuf = torch.zeros(nnz + 1, dtype=dtype, device=dev)      # values at an address that is only 2-byte aligned
+    d_val = vbuf[1:]
+    d_val.copy_(torch.from_numpy(val).to(dtype))
+    assert d_val.data_ptr() % 4 == 2
+    d_x, d_y = to_dev(x, dev, dtype), to_dev(y0, dev)
+    A = osa.Csr(rows, cols, d_rp, d_ci, d_val)
+    op = osa.SpmvOp(handle, A, osa.DnVec(d_x), osa.DnVec(d_y))
+    assert op.buffer.numel() == want
+
+    def check(values, alpha, beta):
+        d_y.copy_(torch.from_numpy(y0))
+        op(alpha, beta)
+        stream.synchronize()
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, values, x, y0, alpha, beta)
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+    check(val, 1.0, 0.0)
+    val2 = rnd((val * np.float32(-0.5) + np.float32(0.25)).astype(np.float32))
+    d_val.copy_(torch.from_numpy(val2).to(dtype))
+    check(val2, 1.5, -0.5)
+
+
 def test_default_plan_sums_long_rows_from_the_callers_arrays(osa, gpu_ctx):
     """Rows of 64 entries per column panel and more (4096 at least) with ascending columns are kept out of the
     re-stored layout: the workgroup that has a panel's x in LDS sums their entries of that panel straight from
