@@ -218,6 +218,8 @@ __global__ __launch_bounds__(kBlockThreads) void GatherLocalityKernel(const int3
 
 // ------------------------------------------------------------- STREAM_ROWS
 
+constexpr int kStreamRowsMax = 767;  // rows of a stream-rows tile at most (their offsets pass through LDS)
+
 // Four consecutive matrix entries of one lane, still in storage type.
 template <typename ValT>
 struct Quad {
@@ -331,22 +333,37 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
     // `capacity` products fit the LDS of this launch (rowsPerBlock times the longest row the statistics saw).  A
     // tile with more entries — the row offsets changed since — stages nothing and sums straight from memory.
     bool staged = count <= capacity;
-    Quad<ValT> q[U];
-    IssueQuads<ValT, U>(colInd + first, vals + first, staged ? count : 0, q);
 
-    while (true) {
-        // Row bounds and old y for this lane's first row of the current tile.
-        int64_t r = r0 + group;
-        int32_t s = 0, e = 0;
-        AccT yOld = AccT(0);
-        if (r < r1) {
-            s = rowOffsets[r];
-            e = rowOffsets[r + 1];
-            if (!betaZero && lane == 0) {
-                yOld = ToAcc<AccT>(yIn[r]);
+    // The tile's row offsets and old y reach the lanes that sum the rows through LDS: they are asked for together
+    // with the tile's entries, a tile ahead, and the loop that sums the rows then holds no load from memory at
+    // all.  (Loads come back in the order they were issued: a row offset asked for inside that loop had to wait
+    // for the next tile's entries, asked for just before it, and the tile ahead was no longer ahead - a 27-point
+    // stencil on 128^3 points 163 us, 117 us with a workgroup a tile and nothing fetched ahead.)
+    __shared__ int32_t rowLds[kStreamRowsMax + 1];
+    __shared__ AccT yLds[kStreamRowsMax];
+    constexpr int kBoundRegs = (kStreamRowsMax + 1 + kBlockThreads - 1) / kBlockThreads;
+    int32_t bnd[kBoundRegs];
+    AccT yv[kBoundRegs];
+    auto issueBounds = [&](int64_t rFirst, int64_t rEnd) {
+#pragma unroll
+        for (int k = 0; k < kBoundRegs; ++k) {
+            const int64_t rr = rFirst + k * kBlockThreads + static_cast<int64_t>(threadIdx.x);
+            bnd[k] = 0;
+            yv[k] = AccT(0);
+            if (rr <= rEnd) {
+                bnd[k] = rowOffsets[rr];
+                if (!betaZero && rr < rEnd) {
+                    yv[k] = ToAcc<AccT>(yIn[rr]);
+                }
             }
         }
-        // Bounds of the next tile (scalar loads, needed after the barrier).
+    };
+    Quad<ValT> q[U];
+    IssueQuads<ValT, U>(colInd + first, vals + first, staged ? count : 0, q);
+    issueBounds(r0, r1);
+
+    while (true) {
+        // Bounds of the next tile (needed after the barrier to ask for its entries).
         const int64_t tNext = t + stride;
         const bool more = tNext < xcdTiles;
         int64_t r0Next = 0, r1Next = 0;
@@ -357,25 +374,27 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
             firstNext = rowOffsets[r0Next];
             countNext = rowOffsets[r1Next] - firstNext;
         }
-
+        const int32_t tileRows = static_cast<int32_t>(r1 - r0);
+#pragma unroll
+        for (int k = 0; k < kBoundRegs; ++k) {
+            const int32_t rr = k * kBlockThreads + static_cast<int32_t>(threadIdx.x);
+            if (rr <= tileRows) {
+                rowLds[rr] = bnd[k];
+                if (rr < tileRows) {
+                    yLds[rr] = yv[k];
+                }
+            }
+        }
         FinishQuads<ValT, AccT, U>(q, x, staged ? count : 0, prod);
         __syncthreads();
         const bool stagedNext = countNext <= capacity;
         if (more) {
             IssueQuads<ValT, U>(colInd + firstNext, vals + firstNext, stagedNext ? countNext : 0, q);
+            issueBounds(r0Next, r1Next);
         }
 
-        while (r < r1) {
-            const int64_t rNext = r + kGroups;
-            int32_t sNext = 0, eNext = 0;
-            AccT yNext = AccT(0);
-            if (rNext < r1) {
-                sNext = rowOffsets[rNext];
-                eNext = rowOffsets[rNext + 1];
-                if (!betaZero && lane == 0) {
-                    yNext = ToAcc<AccT>(yIn[rNext]);
-                }
-            }
+        for (int32_t rr = group; rr < tileRows; rr += kGroups) {
+            const int32_t s = rowLds[rr], e = rowLds[rr + 1];
             AccT sum = AccT(0);
             // skipLonger > 0: rows longer than that are SpmvLongRowsKernel's, which runs after this kernel
             const bool skip = skipLonger > 0 && e - s > skipLonger;
@@ -393,19 +412,15 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
             if (lane == 0 && !skip) {
                 AccT res = alpha * sum;
                 if (!betaZero) {
-                    res += beta * yOld;
+                    res += beta * yLds[rr];
                 }
-                y[r] = FromAcc<OutT>(res);
+                y[r0 + rr] = FromAcc<OutT>(res);
             }
-            r = rNext;
-            s = sNext;
-            e = eNext;
-            yOld = yNext;
         }
         if (!more) {
             break;
         }
-        __syncthreads();  // everyone is done reading prod before the next tile overwrites it
+        __syncthreads();  // everyone is done with prod and the row tables before the next tile overwrites them
         t = tNext;
         r0 = r0Next;
         r1 = r1Next;
@@ -1285,9 +1300,26 @@ MergeLayout MakeMergeLayout(int64_t rows, int64_t nnz)
 template <typename ValT, typename OutT, typename AccT, int G, int U>
 int LaunchStreamU(const SpmvArgs &a, int32_t rowsPerBlock, size_t lds, int32_t skipLonger)
 {
-    // Persistent launch: a few workgroups per CU walk over all tiles.
+    if (rowsPerBlock < 1 || rowsPerBlock > kStreamRowsMax) {
+        return OPSPARSE_E_INVALID;
+    }
+    // Persistent launch: the workgroups that fit a CU at once (eight at most) walk over all tiles.  One more than
+    // fit would start when the first is done and finish last (8 asked for where 7 fit: 163 us against 127 us).
     const uint32_t tiles = GridFor(a.rows, rowsPerBlock);
-    const uint32_t resident = static_cast<uint32_t>(ComputeUnits() * StreamBlocksPerCu());
+    // (asked of the runtime once per kernel and LDS size and thread)
+    thread_local size_t fitLds = ~static_cast<size_t>(0);
+    thread_local int fit = 1;
+    if (fitLds != lds) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&fit, SpmvStreamRowsKernel<ValT, OutT, AccT, G, U>,
+                                                         kBlockThreads, lds) != hipSuccess ||
+            fit < 1) {
+            (void)hipGetLastError();
+            fit = 1;
+        }
+        fitLds = lds;
+    }
+    const int perCu = StreamBlocksPerCu() < fit ? StreamBlocksPerCu() : fit;
+    const uint32_t resident = static_cast<uint32_t>(ComputeUnits() * perCu);
     const uint32_t grid = tiles < resident ? tiles : resident;
     hipLaunchKernelGGL((SpmvStreamRowsKernel<ValT, OutT, AccT, G, U>), dim3(grid), dim3(kBlockThreads), lds, a.stream,
                        a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
@@ -1839,7 +1871,7 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
             p.rowsPerBlock = rpb < 4 ? 4 : rpb;
             if (const char *env = std::getenv("OPS_SPARSE_STREAM_ROWS")) {
                 const int v = std::atoi(env);  // tuning override
-                if (v >= 1 && static_cast<int64_t>(v) * tileRow <= 3072) {
+                if (v >= 1 && v <= kStreamRowsMax && static_cast<int64_t>(v) * tileRow <= 3072) {
                     p.rowsPerBlock = v;
                 }
             }
