@@ -99,7 +99,7 @@ typedef struct OpsparseSpmvPlan {
     int32_t numDeferredLongRows; /* BLOCKED_GATHER: those of them that sit more than 64 to a row block: a third kernel,
                               a wavefront a row, adds their partial sums up instead of the block's workgroup */
     int32_t valueType;     /* BLOCKED_GATHER: the OPSPARSE_F32 / F16 / BF16 the layout was built from; launches must
-                              bring values and x of that type (and an fp32 y) */
+                              bring values and x of that type (y: fp32, or that type) */
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */
@@ -162,7 +162,7 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
                                      OpsparseSpmvPlan *plan, void *stream);
 
 /*
- * BLOCKED_GATHER analysis (fp32, or fp16 / bf16 values and x with an fp32 y): bytes of the workspace, or 0 when the family does
+ * BLOCKED_GATHER analysis (fp32, or fp16 / bf16 values and x with y fp32 or of the same type): bytes of the workspace, or 0 when the family does
  * not apply (x must have more than 2^20 and at most 2^25 elements, the matrix at least
  * two million entries, and a (panel, row block) chunk at least 32 entries on average).  transpose != 0 builds the layout of
  * y = alpha * A^T * x + beta * y instead: panels over the rows of A, blocks over its
@@ -181,7 +181,8 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
  * values change; rowOffsets / colInd must be the arrays of the analysis.
  * OPSPARSE_BLOCKED_VALUES_F16 / _BF16: csrValues (and, at the launches, x) are fp16 / bf16 instead of fp32; the
  * layout keeps frozen values as fp32, which holds them exactly, live ones are widened where the launches read
- * them, and the first kernel widens x while it loads a panel's slice.  y stays fp32.
+ * them, and the first kernel widens x while it loads a panel's slice.  At the launches y is fp32 or of the values'
+ * 16-bit type (one rounding of the fp64 sum).
  */
 #define OPSPARSE_BLOCKED_TRANSPOSE 1
 #define OPSPARSE_BLOCKED_LIVE_VALUES 2

@@ -1027,12 +1027,12 @@ constexpr int kRedThreads = kBlkThreads, kRedWaves = kRedThreads / kWave;
 // by window of kRefreshSpan positions (partDesc[partStart[block]] ..: entries, positions); the values of a window
 // are first collected in LDS from the caller's array, and the stream takes them from there.  Padding positions of
 // a window hold whatever LDS held: their products are formed and dropped.
-template <bool Live, bool Short, typename ValT>
+template <bool Live, bool Short, typename ValT, typename OutT>
 __global__ __launch_bounds__(kRedThreads) void SpmvBlockReduceKernel(
     const float *__restrict__ valD, const float *__restrict__ xg, const uint16_t *__restrict__ rowLocal,
     const int32_t *__restrict__ dstStart, const int32_t *__restrict__ srcStartT, int32_t P,
-    const int32_t *__restrict__ blockOrder, const int32_t *__restrict__ blockRow, float *__restrict__ y,
-    const float *__restrict__ yIn, OpsparseScalar alphaS, OpsparseScalar betaS, const int32_t *__restrict__ longFirst,
+    const int32_t *__restrict__ blockOrder, const int32_t *__restrict__ blockRow, OutT *__restrict__ y,
+    const OutT *__restrict__ yIn, OpsparseScalar alphaS, OpsparseScalar betaS, const int32_t *__restrict__ longFirst,
     const int32_t *__restrict__ longRows, const double *__restrict__ longPartial, const ValT *__restrict__ vals,
     const int32_t *__restrict__ dstOfPos, const int32_t *__restrict__ blockEntry, const int32_t *__restrict__ longSpan)
 {
@@ -1235,17 +1235,18 @@ __global__ __launch_bounds__(kRedThreads) void SpmvBlockReduceKernel(
         }
         double o = alpha * acc[i];
         if (beta != 0.0) {
-            o += beta * static_cast<double>(yIn[row]);
+            o += beta * ToAcc<double>(yIn[row]);
         }
-        y[row] = static_cast<float>(o);
+        y[row] = FromAcc<OutT>(o);
     }
 }
 
 // The long rows of the row blocks that hold more than kInBlockLongRows of them (longDeferred[l] != 0), a wavefront a
 // row: y[row] = alpha * (the row's partial sums, added up as phase 2 does) + beta * yIn[row].
+template <typename OutT>
 __global__ __launch_bounds__(kBlockThreads) void SpmvLongRowSumKernel(
     const int32_t *__restrict__ header, const int32_t *__restrict__ longRows, const int32_t *__restrict__ longDeferred,
-    const double *__restrict__ longPartial, int32_t P, float *__restrict__ y, const float *__restrict__ yIn,
+    const double *__restrict__ longPartial, int32_t P, OutT *__restrict__ y, const OutT *__restrict__ yIn,
     OpsparseScalar alphaS, OpsparseScalar betaS)
 {
     const int lane = threadIdx.x % kWave;
@@ -1276,9 +1277,9 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvLongRowSumKernel(
         const double alpha = ReadScalar<double>(alphaS), beta = ReadScalar<double>(betaS);
         double o = alpha * sum;
         if (beta != 0.0) {
-            o += beta * static_cast<double>(yIn[row]);
+            o += beta * ToAcc<double>(yIn[row]);
         }
-        y[row] = static_cast<float>(o);
+        y[row] = FromAcc<OutT>(o);
     }
 }
 
@@ -1441,10 +1442,13 @@ uint32_t GridOf(int64_t items, int64_t perBlock, int64_t cap)
 // valType: the type of the caller's values and of x (OPSPARSE_F32 / F16 / BF16); y is fp32.  Frozen fp16 and bf16
 // values sit in the layout as fp32, live ones are widened where they are read, and phase 1 widens x as it loads
 // the slice.
-int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valType)
+int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valType, int32_t outType)
 {
     if (plan.valueType != valType) {
         return OPSPARSE_E_INVALID;  // the plan was made for values of another type
+    }
+    if (outType != OPSPARSE_F32 && outType != valType) {
+        return OPSPARSE_E_UNSUPPORTED;  // y is fp32, or of the 16-bit type of the values
     }
     // a.rows outputs, a.cols inputs: the caller has exchanged them for op(A) = A^T
     const BlockedLayout l = MakeBlockedLayout(a.rows, a.cols, a.nnz, plan.transposed != 0, plan.liveValues != 0);
@@ -1496,42 +1500,56 @@ int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valTy
     } else {
         gatherTyped(std::true_type{});
     }
-    auto reduceLive = [&](auto shortTag, auto valTag) {
-        constexpr bool kShort = decltype(shortTag)::value;
+    // phase 2 (and the sums of deferred long rows) for the types of the values and of y
+    auto reduce = [&](auto valTag, auto outTag) {
         using ValT = decltype(valTag);
-        hipLaunchKernelGGL((SpmvBlockReduceKernel<true, kShort, ValT>), dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads),
-                           0, a.stream, static_cast<const float *>(nullptr), xg, rowLocal, ints(l.dstStartOff),
-                           ints(l.srcStartTOff), l.P, ints(l.orderOff), ints(l.blockRowOff), static_cast<float *>(a.y),
-                           static_cast<const float *>(a.yIn), a.alpha, a.beta, longRows ? ints(l.longFirstOff) : nullptr,
-                           ints(l.longRowsOff), longPartial, static_cast<const ValT *>(a.vals), ints(l.dstOfPosOff),
-                           ints(l.blockEntryOff), ints(l.longSpanOff));
-    };
-    auto reduceLiveTyped = [&](auto shortTag) {
-        if (valType == OPSPARSE_F16) {
-            reduceLive(shortTag, Half{});
-        } else if (valType == OPSPARSE_BF16) {
-            reduceLive(shortTag, Bf16{});
+        using OutT = decltype(outTag);
+        auto live = [&](auto shortTag) {
+            constexpr bool kShort = decltype(shortTag)::value;
+            hipLaunchKernelGGL((SpmvBlockReduceKernel<true, kShort, ValT, OutT>), dim3(static_cast<uint32_t>(l.B)),
+                               dim3(kRedThreads), 0, a.stream, static_cast<const float *>(nullptr), xg, rowLocal,
+                               ints(l.dstStartOff), ints(l.srcStartTOff), l.P, ints(l.orderOff), ints(l.blockRowOff),
+                               static_cast<OutT *>(a.y), static_cast<const OutT *>(a.yIn), a.alpha, a.beta,
+                               longRows ? ints(l.longFirstOff) : nullptr, ints(l.longRowsOff), longPartial,
+                               static_cast<const ValT *>(a.vals), ints(l.dstOfPosOff), ints(l.blockEntryOff),
+                               ints(l.longSpanOff));
+        };
+        if (plan.liveValues == kLiveShortPositions) {
+            live(std::true_type{});
+        } else if (plan.liveValues != 0) {
+            live(std::false_type{});
         } else {
-            reduceLive(shortTag, float{});
+            // (frozen values sit in the layout as fp32 whatever the caller's type)
+            hipLaunchKernelGGL((SpmvBlockReduceKernel<false, false, float, OutT>), dim3(static_cast<uint32_t>(l.B)),
+                               dim3(kRedThreads), 0, a.stream, valD, xg, rowLocal, ints(l.dstStartOff),
+                               ints(l.srcStartTOff), l.P, ints(l.orderOff), ints(l.blockRowOff), static_cast<OutT *>(a.y),
+                               static_cast<const OutT *>(a.yIn), a.alpha, a.beta,
+                               longRows ? ints(l.longFirstOff) : nullptr, ints(l.longRowsOff), longPartial,
+                               static_cast<const float *>(nullptr), static_cast<const int32_t *>(nullptr),
+                               static_cast<const int32_t *>(nullptr), static_cast<const int32_t *>(nullptr));
+        }
+        if (longRows && plan.numDeferredLongRows > 0) {
+            constexpr int kRowsPerBlock = kBlockThreads / kWave;
+            hipLaunchKernelGGL(SpmvLongRowSumKernel<OutT>, dim3((plan.numLongRows + kRowsPerBlock - 1) / kRowsPerBlock),
+                               dim3(kBlockThreads), 0, a.stream, header, ints(l.longRowsOff), ints(l.longDeferredOff),
+                               longPartial, l.P, static_cast<OutT *>(a.y), static_cast<const OutT *>(a.yIn), a.alpha,
+                               a.beta);
         }
     };
-    if (plan.liveValues == kLiveShortPositions) {
-        reduceLiveTyped(std::true_type{});
-    } else if (plan.liveValues != 0) {
-        reduceLiveTyped(std::false_type{});
+    if (valType == OPSPARSE_F16) {
+        if (outType == OPSPARSE_F16) {
+            reduce(Half{}, Half{});
+        } else {
+            reduce(Half{}, float{});
+        }
+    } else if (valType == OPSPARSE_BF16) {
+        if (outType == OPSPARSE_BF16) {
+            reduce(Bf16{}, Bf16{});
+        } else {
+            reduce(Bf16{}, float{});
+        }
     } else {
-        hipLaunchKernelGGL((SpmvBlockReduceKernel<false, false, float>), dim3(static_cast<uint32_t>(l.B)), dim3(kRedThreads), 0,
-                           a.stream, valD, xg, rowLocal, ints(l.dstStartOff), ints(l.srcStartTOff), l.P, ints(l.orderOff),
-                           ints(l.blockRowOff), static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha,
-                           a.beta, longRows ? ints(l.longFirstOff) : nullptr, ints(l.longRowsOff), longPartial,
-                           static_cast<const float *>(nullptr), static_cast<const int32_t *>(nullptr),
-                           static_cast<const int32_t *>(nullptr), static_cast<const int32_t *>(nullptr));
-    }
-    if (longRows && plan.numDeferredLongRows > 0) {
-        constexpr int kRowsPerBlock = kBlockThreads / kWave;
-        hipLaunchKernelGGL(SpmvLongRowSumKernel, dim3((plan.numLongRows + kRowsPerBlock - 1) / kRowsPerBlock),
-                           dim3(kBlockThreads), 0, a.stream, header, ints(l.longRowsOff), ints(l.longDeferredOff),
-                           longPartial, l.P, static_cast<float *>(a.y), static_cast<const float *>(a.yIn), a.alpha, a.beta);
+        reduce(float{}, float{});
     }
     return CheckLaunch();
 }

@@ -130,10 +130,11 @@ Restored RestoredLayout(aclsparseHandle_t handle, aclsparseOperation_t opA, acls
                         aclsparseConstDnVecDescr_t vecX, aclsparseConstDnVecDescr_t vecY, aclDataType computeType,
                         aclsparseSpMVAlg_t alg)
 {
-    // fp32 throughout, or fp16 / bf16 values and x with an fp32 y (the blocked-gather layout only: it keeps frozen
-    // values as fp32 and widens live ones, and x, where it reads them)
+    // fp32 throughout, or fp16 / bf16 values and x with y fp32 or of the same 16-bit type (the blocked-gather layout
+    // only: it keeps frozen values as fp32, widens live ones, and x, where it reads them, and rounds y once)
     const int32_t valueType = RestoredValueType(matA, vecX);
-    if (computeType != ACL_FLOAT || vecY->valueType != ACL_FLOAT || valueType < 0) {
+    if (computeType != ACL_FLOAT || valueType < 0 ||
+        (vecY->valueType != ACL_FLOAT && vecY->valueType != matA->valueType)) {
         return {0, 0, false};
     }
     const bool transpose = opA != ACL_SPARSE_OP_NON_TRANSPOSE;

@@ -30,6 +30,6 @@ inline int CheckLaunch()
 }
 
 // BLOCKED_GATHER launch, fp32 values / x / y (spmv_blocked.hip).
-int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valType);
+int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valType, int32_t outType);
 
 }  // namespace opsparse

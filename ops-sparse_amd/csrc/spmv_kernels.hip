@@ -1468,14 +1468,16 @@ int RunPlanned(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
                 return OPSPARSE_E_UNSUPPORTED;  // the panel copy holds fp32 values
             }
         case OPSPARSE_SPMV_BLOCKED_GATHER:
-            if constexpr (std::is_same<OutT, float>::value && std::is_same<AccT, double>::value &&
+            if constexpr (std::is_same<AccT, double>::value &&
                           (std::is_same<ValT, float>::value || std::is_same<ValT, Half>::value ||
-                           std::is_same<ValT, Bf16>::value)) {
-                return LaunchBlocked(a, plan, std::is_same<ValT, Half>::value   ? OPSPARSE_F16
-                                              : std::is_same<ValT, Bf16>::value ? OPSPARSE_BF16
-                                                                                : OPSPARSE_F32);
+                           std::is_same<ValT, Bf16>::value) &&
+                          (std::is_same<OutT, float>::value || std::is_same<OutT, ValT>::value)) {
+                constexpr int32_t kVal = std::is_same<ValT, Half>::value   ? OPSPARSE_F16
+                                         : std::is_same<ValT, Bf16>::value ? OPSPARSE_BF16
+                                                                           : OPSPARSE_F32;
+                return LaunchBlocked(a, plan, kVal, std::is_same<OutT, float>::value ? OPSPARSE_F32 : kVal);
             } else {
-                return OPSPARSE_E_UNSUPPORTED;  // the re-stored copy holds fp32 values, y is written as fp32
+                return OPSPARSE_E_UNSUPPORTED;  // fp32, fp16 or bf16 values; y fp32 or of the values' type
             }
         default:
             return OPSPARSE_E_INVALID;
@@ -2059,13 +2061,13 @@ int opsparse_spmv_csr_launch_zy(const OpsparseSpmvPlan *plan, int32_t transpose,
     }
     if (transpose && plan != nullptr && plan->kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {
         if (computeIsInt || (valType != OPSPARSE_F32 && valType != OPSPARSE_F16 && valType != OPSPARSE_BF16) ||
-            outType != OPSPARSE_F32) {
+            (outType != OPSPARSE_F32 && outType != valType)) {
             return OPSPARSE_E_UNSUPPORTED;
         }
         SpmvArgs t = a;  // the columns of A are the outputs, its rows the inputs
         t.rows = cols;
         t.cols = rows;
-        return LaunchBlocked(t, *plan, valType);
+        return LaunchBlocked(t, *plan, valType, outType);
     }
     if (transpose) {
         if (computeIsInt) {

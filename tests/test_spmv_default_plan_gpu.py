@@ -91,8 +91,8 @@ def _with_long_rows(rows, cols, seed):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("short_positions", [True, False])
-def test_default_plan_with_half_precision_values(osa, gpu_ctx, dtype, short_positions, monkeypatch):
+@pytest.mark.parametrize("short_positions,narrow_y", [(True, False), (False, False), (True, True)])
+def test_default_plan_with_half_precision_values(osa, gpu_ctx, dtype, short_positions, narrow_y, monkeypatch):
     """fp16 / bf16 values and x with an fp32 y get the same default plan: the live layout reads the caller's 2-byte
     values at every call (the short entries into the LDS window of their row block, the long rows' straight into
     the sums of their panel) and widens x as it loads a panel's slice.  Values changed in place are followed."""
@@ -111,17 +111,24 @@ def test_default_plan_with_half_precision_values(osa, gpu_ctx, dtype, short_posi
     d_val = vbuf[1:]
     d_val.copy_(torch.from_numpy(val).to(dtype))
     assert d_val.data_ptr() % 4 == 2
-    d_x, d_y = to_dev(x, dev, dtype), to_dev(y0, dev)
+    if narrow_y:                                              # y of the values' type: the fp64 sum rounded once
+        y0 = rnd(y0)
+    d_x, d_y = to_dev(x, dev, dtype), to_dev(y0, dev, dtype if narrow_y else None)
     A = osa.Csr(rows, cols, d_rp, d_ci, d_val)
     op = osa.SpmvOp(handle, A, osa.DnVec(d_x), osa.DnVec(d_y))
     assert op.buffer.numel() == want
+    half_ulp = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
 
     def check(values, alpha, beta):
-        d_y.copy_(torch.from_numpy(y0))
+        d_y.copy_(torch.from_numpy(y0).to(d_y.dtype))
         op(alpha, beta)
         stream.synchronize()
         gold = oracle.spmv_f64(rows, cols, rowptr, colind, values, x, y0, alpha, beta)
-        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+        got = d_y.float().cpu().numpy()
+        if narrow_y:
+            assert np.all(np.abs(got - gold) <= 1.001 * half_ulp * np.maximum(np.abs(gold), 2.0 ** -14))
+        else:
+            assert oracle.max_rel_err(got, gold) <= 1e-5
 
     check(val, 1.0, 0.0)
     val2 = rnd((val * np.float32(-0.5) + np.float32(0.25)).astype(np.float32))

@@ -375,8 +375,8 @@ def test_blocked_gather_transposed(osa, gpu_ctx, rows, cols):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("transpose", [False, True])
-def test_blocked_gather_csr_alg2_half_precision_values(osa, gpu_ctx, dtype, transpose):
+@pytest.mark.parametrize("transpose,narrow_y", [(False, False), (True, False), (False, True), (True, True)])
+def test_blocked_gather_csr_alg2_half_precision_values(osa, gpu_ctx, dtype, transpose, narrow_y):
     """fp16 / bf16 values and x with an fp32 y under ACL_SPARSE_SPMV_CSR_ALG2: the same re-stored layout (it keeps
     the values as fp32, which holds them exactly, and widens x as it loads a panel's slice), long rows included;
     against the fp64 oracle on the rounded inputs at the fp32 bar.  A launch with values of another type than the
@@ -400,18 +400,27 @@ def test_blocked_gather_csr_alg2_half_precision_values(osa, gpu_ctx, dtype, tran
     need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 1 if transpose else 0)
     assert need > 0
     d_rp, d_ci = to_dev(rowptr, dev), to_dev(colind, dev)
-    d_val, d_x, d_y = to_dev(val, dev, dtype), to_dev(x, dev, dtype), to_dev(y0, dev)
+    if narrow_y:                                             # y of the values' type: the fp64 sum rounded once
+        y0 = rnd(y0)
+    d_val, d_x, d_y = to_dev(val, dev, dtype), to_dev(x, dev, dtype), to_dev(y0, dev, dtype if narrow_y else None)
+    half_ulp = 2.0 ** -11 if dtype == torch.float16 else 2.0 ** -8
+
+    def close(gold):
+        got = d_y.float().cpu().numpy()
+        if narrow_y:
+            return bool(np.all(np.abs(got - gold) <= 1.001 * half_ulp * np.maximum(np.abs(gold), 2.0 ** -14)))
+        return oracle.max_rel_err(got, gold) <= 1e-5
+
     A = osa.Csr(rows, cols, d_rp, d_ci, d_val)
     op = osa.SpmvOp(handle, A, osa.DnVec(d_x), osa.DnVec(d_y), alg=osa.ACL_SPARSE_SPMV_CSR_ALG2,
                     op=osa.ACL_SPARSE_OP_TRANSPOSE if transpose else osa.ACL_SPARSE_OP_NON_TRANSPOSE)
     assert op.buffer.numel() >= need                         # the layout, not the ordinary plan's few hundred KB
     golden = oracle.spmv_trans_f64 if transpose else oracle.spmv_f64
     for alpha, beta in ((1.0, 0.0), (-2.0, 0.75)):
-        d_y.copy_(torch.from_numpy(y0))
+        d_y.copy_(torch.from_numpy(y0).to(d_y.dtype))
         op(alpha, beta)
         stream.synchronize()
-        gold = golden(rows, cols, rowptr, colind, val, x, y0, alpha, beta)
-        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+        assert close(golden(rows, cols, rowptr, colind, val, x, y0, alpha, beta))
     # raw layer: the plan remembers the type it was built from
     sp = ctypes.c_void_p(stream.cuda_stream)
     ws = torch.empty(need, dtype=torch.uint8, device=dev)
@@ -424,11 +433,12 @@ def test_blocked_gather_csr_alg2_half_precision_values(osa, gpu_ctx, dtype, tran
     one, zero = osa.OpsparseScalar(1.0, None, 0, 0), osa.OpsparseScalar(0.0, None, 0, 0)
     launch = lambda vt, v, xx: L.opsparse_spmv_csr_launch(ctypes.byref(plan), 1 if transpose else 0, d_rp.data_ptr(),
                                                           d_ci.data_ptr(), v.data_ptr(), xx.data_ptr(), d_y.data_ptr(), rows,
-                                                          cols, colind.size, one, zero, vt, osa.OPSPARSE_F32, 0,
+                                                          cols, colind.size, one, zero, vt,
+                                                          want if narrow_y else osa.OPSPARSE_F32, 0,
                                                           ws.data_ptr(), need, sp)
     assert launch(want, d_val, d_x) == 0
     stream.synchronize()
-    assert oracle.max_rel_err(d_y.cpu().numpy(), golden(rows, cols, rowptr, colind, val, x, y0, 1.0, 0.0)) <= 1e-5
+    assert close(golden(rows, cols, rowptr, colind, val, x, y0, 1.0, 0.0))
     f_val, f_x = to_dev(val, dev), to_dev(x, dev)
     assert launch(osa.OPSPARSE_F32, f_val, f_x) != 0         # fp32 operands with a plan built from 2-byte values
 
