@@ -163,7 +163,7 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
 
 /*
  * BLOCKED_GATHER analysis (fp32, or fp16 / bf16 values and x with y fp32 or of the same type): bytes of the workspace, or 0 when the family does
- * not apply (x must have more than 2^20 and at most 2^25 elements, the matrix at least
+ * not apply (x must have more than 2^18 and at most 2^25 elements, the matrix at least
  * two million entries, and a (panel, row block) chunk at least 32 entries on average).  transpose != 0 builds the layout of
  * y = alpha * A^T * x + beta * y instead: panels over the rows of A, blocks over its
  * columns, with no atomics on y; a plan serves the op(A) it was built for.  Like the panel

@@ -83,6 +83,12 @@ constexpr int32_t kRankedBlocks = 8192;           // up to here the block order 
 constexpr int64_t kMinEntryWindow = 16384;
 constexpr int64_t kMinEntryBlocks = 512;          // entry windows a matrix is cut into at least (if it has the entries)
 constexpr int64_t kMinEntries = 2000000;          // below this the ordinary kernels are as fast or faster
+// x of more than 2^18 elements.  An x of 1 - 4 MB fits an L2, but gathers scattered over it still cost the row-wise
+// kernels 5.5 us per million (the rate at which an L2 answers them) against 3.6 us per million entries for the
+// layout with frozen values: 1 M x 1 M with 32 random columns a row 189 -> 108 us (live values 143 us), over 2^19
+// columns 157 -> 106 us, a power-law matrix of 1 M rows 100 -> 46 us and its transpose 533 -> 48 us.  (The bound
+// used to be 2^20.)  Whether the gathers are scattered is for the sample of the column indices to say.
+constexpr int64_t kMinCols = int64_t{1} << 18;
 constexpr int64_t kMinChunkEntries = 32;          // below this mean chunk size the layout does not pay
 // Live values (the default plan, which competes with the merge path on the caller's arrays rather than with a
 // re-stored matrix): the window of values in LDS makes the row blocks short and the chunks with them; it pays down
@@ -1333,9 +1339,14 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     int64_t window = nnz / (fullBlocks > wantBlocks ? fullBlocks : wantBlocks);
     window = window < kMinEntryWindow ? kMinEntryWindow : window;
     const int64_t B = ((rows + (int64_t{1} << rowLog) - 1) >> rowLog) + nnz / window + 1;
-    // x must be larger than an L2 (2^20 columns) for the two passes to pay, and the chunks long enough to stream.
+    // x must be wide enough for scattered gathers to be what the row-wise kernels wait for, and the chunks long
+    // enough to stream.
     // Positions are 32-bit, and phase 2 looks two batches past a block's end before it clamps.
-    if (cols <= (int64_t{1} << 20) || nnz < kMinEntries || P > kMaxPanels ||
+    static const int64_t minCols = [] {  // tuning override
+        const char *env = std::getenv("OPS_SPARSE_BLOCKED_MIN_COLS");
+        return env != nullptr ? std::atoll(env) : kMinCols;
+    }();
+    if (cols <= minCols || nnz < kMinEntries || P > kMaxPanels ||
         P * B + 1 > INT32_MAX || nnz + kLaneEntries * P * B > INT32_MAX - 65536 ||
         nnz / (P * B) < (live ? kMinChunkEntriesLive : kMinChunkEntries)) {
         return l;

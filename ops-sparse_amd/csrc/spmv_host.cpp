@@ -257,10 +257,16 @@ int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *co
     // gathers far from the diagonal among them the row-wise kernels take about 1.2 us per million entries and 13 us
     // per million far gathers (4 M rows of a band and 1 .. 6 random columns each); the layouts take 3.6 us (values
     // frozen) and 5.2 us (live values) per million entries whatever the columns.
-    // op(A) = A^T keeps the layout either way: it replaces fp32 atomics on y, which it beats on the same Laplacian
-    // (86 us against 119 us) and whose result depends on the order of the updates.
+    // op(A) = A^T with a y beyond an L2 keeps the layout either way: it replaces fp32 atomics on y, which it beats
+    // on the same Laplacian (86 us against 119 us) and whose result depends on the order of the updates.  Where y
+    // fits an L2 the atomics of a mesh stay there and are as fast or faster (1000 x 1000 Laplacian: 38 us against
+    // 42 us; 700 x 700: 22 against 26), while scattered ones are not (500 000 x 500 000 with 16 random columns a
+    // row: 392 us against 42 us with the layout): the same question then.  (Not below 2^18 columns, where no column
+    // is far from any diagonal and many rows add to every element of y: 300 000 x 16 000 with 8 a row 111 us with
+    // atomics, 23 us with the layout.)
     int32_t scattered = 1000;
-    if (!transpose && !liveValues) {  // (a live-values request has asked already)
+    const bool ask = transpose ? cols > (int64_t{1} << 18) && cols <= (int64_t{1} << 20) : true;
+    if (!liveValues && ask) {  // (a live-values request has asked already)
         int rc = opsparse_spmv_csr_gathers_scattered(rowOffsets, colInd, rows, cols, nnz, buffer, bytes, &scattered,
                                                      stream);
         if (rc != OPSPARSE_OK) {

@@ -302,17 +302,17 @@ def test_raw_layer_argument_checks(osa, L):
 
 def test_restored_layout_applicability(osa, L, handle):
     """When ACL_SPARSE_SPMV_CSR_ALG2 gets a re-stored layout, decided on the host from the sizes alone: blocked
-    gather needs an x of more than 2^20 and at most 2^25 elements and 32 entries per (panel, row block) chunk;
+    gather needs an x of more than 2^18 and at most 2^25 elements and 32 entries per (panel, row block) chunk;
     (and two million entries in all); column panels (op(A) = A only) need 2 .. 16 panels of 2^20 columns.  GetBufferSize reports the larger of
     that layout and the ordinary buffer, and the ordinary one for anything else."""
     blocked, panels = L.opsparse_spmv_csr_blocked_workspace_bytes, L.opsparse_spmv_csr_panels_workspace_bytes
     m = 1 << 23
     assert blocked(m, m, 8 * m, 0) > 12 * 8 * m and blocked(m, m, 8 * m, 1) > 12 * 8 * m
-    assert blocked(m, 1 << 20, 8 * m, 0) == 0 and blocked(m, (1 << 20) + 1, 8 * m, 0) > 0     # x must exceed an L2
+    assert blocked(m, 1 << 18, 8 * m, 0) == 0 and blocked(m, (1 << 18) + 1, 8 * m, 0) > 0     # x must be wide enough
     assert blocked(m, (1 << 25) + 1, 64 * m, 0) == 0                                         # too many panels
     assert blocked(m, m, m // 64, 0) == 0                                                    # chunks too short
     assert blocked(50_000, m, 1_900_000, 0) == 0 and blocked(50_000, m, 2_100_000, 0) > 0     # too few entries
-    assert blocked(1 << 20, m, 8 * m, 1) == 0 and blocked(m, 1000, 8 * m, 1) > 0             # op(A) = A^T: x has m rows
+    assert blocked(1 << 18, m, 8 * m, 1) == 0 and blocked(m, 1000, 8 * m, 1) > 0             # op(A) = A^T: x has m rows
     assert blocked(0, m, 0, 0) == 0 and blocked(m, m, (1 << 31), 0) == 0
     assert panels(m, m, 8 * m) > 0 and panels(m, 1 << 20, 8 * m) == 0 and panels(m, (1 << 24) + 1, 8 * m) == 0
     n = ctypes.c_size_t(0)

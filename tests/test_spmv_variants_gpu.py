@@ -239,7 +239,7 @@ def test_column_panels_through_spmvop_alg2(osa, gpu_ctx, monkeypatch):
 
 
 @pytest.mark.parametrize("rows,cols,applies", [(60_000, 3_000_000, True), (60_000, 1_048_577, True),
-                                               (60_000, 9_000_000, True), (60_000, 1_000_000, False),
+                                               (60_000, 9_000_000, True), (60_000, 1_000_000, True), (60_000, 262_144, False),
                                                (20_000, 17_000_000, False),     # 519 panels: chunks of < 32 entries
                                                (300_000, 2_000_000, True)])
 def test_blocked_gather_csr_alg2(osa, gpu_ctx, rows, cols, applies):
@@ -332,7 +332,7 @@ def test_blocked_gather_giant_row_and_device_scalars(osa, gpu_ctx):
 
 @pytest.mark.parametrize("rows,cols", [(1_400_000, 50_000), (2_000_000, 2_000_000), (1_200_000, 900_000), (1_100_000, 300)])
 def test_blocked_gather_transposed(osa, gpu_ctx, rows, cols):
-    """ACL_SPARSE_SPMV_CSR_ALG2 with op(A) = A^T and more than 2^20 rows: the layout is built over the rows of A
+    """ACL_SPARSE_SPMV_CSR_ALG2 with op(A) = A^T and more than 2^18 rows: the layout is built over the rows of A
     (panels, x) and its columns (row blocks, y), and the product has no atomics on y: the 1e-5 bar of op(A) = A,
     not the reference's loose rule for its atomic transpose path.  A plan built for A^T does not serve A: the
     same descriptor and buffer then run op(A) = A through the ordinary kernels."""
@@ -526,6 +526,51 @@ def test_alg2_keeps_row_kernels_for_local_gathers(osa, workloads, gpu_ctx):
     gold = oracle.spmv_f64(rows, cols, A["rowptr"].cpu().numpy(), A["colind"].cpu().numpy(),
                            A["values"].cpu().numpy(), x, y0, 1.0, 0.5)
     assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+
+@pytest.mark.parametrize("shape", ["mesh 700^2", "random 500 000^2", "narrow y"])
+def test_alg2_transposed_below_2_20_outputs(osa, workloads, gpu_ctx, shape):
+    """op(A) = A^T under CSR_ALG2 where y fits an L2: a mesh keeps the ordinary (atomic) kernels, whose updates stay
+    in cache — the buffer then holds an ordinary plan and the values may change without a new Preprocess — while
+    scattered columns, and a y of so few elements that many rows add to each, get the re-stored layout.  Which one
+    ran shows in what a change of the values does: the layout holds a copy and does not follow it."""
+    dev, stream, handle = gpu_ctx
+    if shape.startswith("mesh"):
+        A = workloads.laplacian_2d(700, dev)
+        follows = True
+    elif shape.startswith("random"):
+        A = workloads.uniform_rows_csr(500_000, 500_000, 6, 3, dev)
+        follows = False
+    else:
+        A = workloads.uniform_rows_csr(300_000, 16_000, 8, 3, dev)
+        follows = False
+    rows, cols, nnz = A["rows"], A["cols"], int(A["colind"].numel())
+    assert osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, 1) > 0
+    rng = np.random.default_rng(4)
+    x, y0 = rng.uniform(-1, 1, rows).astype(np.float32), rng.uniform(-1, 1, cols).astype(np.float32)
+    d_x, d_y = to_dev(x, dev), to_dev(y0, dev)
+    vals = A["values"].clone()
+    op = osa.SpmvOp(handle, osa.Csr(rows, cols, A["rowptr"], A["colind"], vals), osa.DnVec(d_x), osa.DnVec(d_y),
+                    op=osa.ACL_SPARSE_OP_TRANSPOSE, alg=osa.ACL_SPARSE_SPMV_CSR_ALG2)
+    rp, ci = A["rowptr"].cpu().numpy(), A["colind"].cpu().numpy()
+
+    def close(want):
+        got = d_y.cpu().numpy()
+        if follows:                                           # fp32 atomics: the reference's rule for that path
+            return bool(np.all(np.abs(got - want) <= 2.0 ** -16 + 2.0 ** -10 * np.abs(want)))
+        return oracle.max_rel_err(got, want) <= 1e-5
+
+    op(1.0, 0.5)
+    stream.synchronize()
+    v0 = vals.cpu().numpy()
+    gold = oracle.spmv_trans_f64(rows, cols, rp, ci, v0, x, y0, 1.0, 0.5)
+    assert close(gold)
+    vals.mul_(2.0)
+    d_y.copy_(torch.from_numpy(y0))
+    op(1.0, 0.5)
+    stream.synchronize()
+    gold2 = oracle.spmv_trans_f64(rows, cols, rp, ci, 2.0 * v0, x, y0, 1.0, 0.5)
+    assert close(gold2 if follows else gold) and not close(gold if follows else gold2)
 
 
 def test_blocked_gather_through_spmvop_alg2(osa, gpu_ctx):
