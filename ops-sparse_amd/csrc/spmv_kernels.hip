@@ -120,11 +120,12 @@ __global__ __launch_bounds__(kBlockThreads) void ConvertFromFloatKernel(OutT *__
 
 // ------------------------------------------------------------- row statistics
 
-constexpr int kStreamMaxRow = 48;   // the stream-rows tiles are sized for rows up to this long
+constexpr int kStreamMaxRow = 512;  // the stream-rows tiles are sized for rows up to this long
+constexpr int kShortMaxRow = 48;    // "short rows with a few long ones among them": what counts as short
 constexpr int kBesideRow = 64;      // with SpmvLongRowsKernel beside them, the stream-rows kernels skip longer rows
 constexpr int kBesideMaxRow = 8192; // ... which one workgroup sums: beyond this length the merge path is the better answer
 
-// stats[0] = longest row, stats[1] = longest row of at most kStreamMaxRow entries, stats[2] = number of longer
+// stats[0] = longest row, stats[1] = longest row of at most kShortMaxRow entries, stats[2] = number of longer
 // rows, stats[3] = their entries.  stats must be zeroed before the launch.
 __global__ __launch_bounds__(kBlockThreads) void RowStatsKernel(const int32_t *__restrict__ rowOffsets, int64_t rows,
                                                                 int32_t *__restrict__ stats)
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(kBlockThreads) void RowStatsKernel(const int32_t *_
     for (int64_t r = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x; r < rows; r += stride) {
         const int32_t len = rowOffsets[r + 1] - rowOffsets[r];
         best = len > best ? len : best;
-        if (len <= kStreamMaxRow) {
+        if (len <= kShortMaxRow) {
             bestShort = len > bestShort ? len : bestShort;
         } else {
             ++numLong;
@@ -1445,6 +1446,9 @@ int RunPlanned(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
                 case 2: return LaunchStream<ValT, OutT, AccT, 2>(a, plan);
                 case 4: return LaunchStream<ValT, OutT, AccT, 4>(a, plan);
                 case 8: return LaunchStream<ValT, OutT, AccT, 8>(a, plan);
+                case 16: return LaunchStream<ValT, OutT, AccT, 16>(a, plan);
+                case 32: return LaunchStream<ValT, OutT, AccT, 32>(a, plan);
+                case 64: return LaunchStream<ValT, OutT, AccT, 64>(a, plan);
                 default: return OPSPARSE_E_INVALID;
             }
         case OPSPARSE_SPMV_VECTOR_ROWS:
@@ -1833,10 +1837,14 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
         // short (mean 16 - 48 even: 160 - 173 us against 195 - 200 us for the merge path; varied: 217 - 222 us
         // against 194 - 199 us); a lane group per row only pays for long rows of nearly equal length (mean 128 -
         // 256: 180 us against 195 us; varied rows 250 - 350 us against 189 us); the merge path does not care.
+        // Since the stream-rows tiles take rows of up to 512 entries (8 - 64 lanes a row), even rows of 49 - 512
+        // entries are theirs as well: 40 M entries in a band, 60 - 512 a row, 65 - 75 us against 64 - 116 us with a
+        // lane group a row or the merge path (100 a row: 117 -> 74 us), and random columns 167 - 186 us against
+        // 165 - 250 us.
         if (maxRow <= kStreamMaxRow && (maxRow <= 12 || static_cast<double>(maxRow) * static_cast<double>(rows) <=
                                                             1.25 * static_cast<double>(nnz))) {
             kernel = OPSPARSE_SPMV_STREAM_ROWS;
-        } else if (maxRow > kStreamMaxRow && maxRow <= kBesideMaxRow && maxShort >= 1 && numLong <= 4096 &&
+        } else if (maxRow > kShortMaxRow && maxRow <= kBesideMaxRow && maxShort >= 1 && numLong <= 4096 &&
                    static_cast<int64_t>(numLong) * 1024 <= rows &&
                    (maxShort <= 12 || static_cast<double>(maxShort) * static_cast<double>(rows) <=
                                           1.25 * static_cast<double>(nnzShort))) {
@@ -1862,7 +1870,7 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
                 return OPSPARSE_E_UNSUPPORTED;  // products of a row block would not fit LDS
             }
             p.tileRowNnz = tileRow;
-            const int32_t g = tileRow <= 12 ? 1 : (tileRow <= 24 ? 2 : 4);
+            const int32_t g = tileRow <= 12 ? 1 : (tileRow <= 24 ? 2 : (tileRow <= 48 ? 4 : (tileRow <= 96 ? 8 : (tileRow <= 192 ? 16 : (tileRow <= 384 ? 32 : 64)))));
             p.lanesPerRow = g;
             // As many rows as keep the tile's worst-case products within two full
             // rounds of the workgroup's loads (2 x 1024 entries, 16 KiB of LDS):
@@ -1871,6 +1879,15 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
             rpb = rpb > 512 ? 512 : rpb;
             rpb &= ~3;  // whole groups of four rows for the vectorised y path
             p.rowsPerBlock = rpb < 4 ? 4 : rpb;
+            if (tileRow > 48) {
+                // Few rows a tile: as many as the lane groups sum in whole turns (a band of 81 entries a row: 32
+                // rows 68.7 us, 25 rows 73.2 us, 37 rows 75.5 us); where not even one turn fits the 3072 slots, two
+                // rounds of loads or three, whichever the rows fill better.
+                const int32_t groups = kBlockThreads / g;
+                const int32_t r2 = 2048 / tileRow, r3 = 3072 / tileRow;
+                p.rowsPerBlock = r3 >= groups ? r3 / groups * groups
+                                              : (static_cast<int64_t>(r2) * 3 >= static_cast<int64_t>(r3) * 2 ? r2 : r3);
+            }
             if (const char *env = std::getenv("OPS_SPARSE_STREAM_ROWS")) {
                 const int v = std::atoi(env);  // tuning override
                 if (v >= 1 && v <= kStreamRowsMax && static_cast<int64_t>(v) * tileRow <= 3072) {
