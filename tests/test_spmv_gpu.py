@@ -130,7 +130,7 @@ def test_every_kernel_family(osa, gpu_ctx, family, case):
         rows, cols = 50000, 64
         lengths = np.zeros(rows, np.int64)
         lengths[::997] = 5
-    if family == "STREAM_ROWS" and lengths.max() > 48:
+    if family == "STREAM_ROWS" and lengths.max() > 512:
         pytest.skip("STREAM_ROWS only takes matrices whose longest row fits its LDS tile")
     rowptr, colind, val = csr_from_lengths(lengths, cols, seed=7)
     x = rng.uniform(-1, 1, cols).astype(np.float32)
@@ -138,3 +138,25 @@ def test_every_kernel_family(osa, gpu_ctx, family, case):
     fam = getattr(osa, "OPSPARSE_SPMV_" + family)
     y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 1.25, 0.75, force_kernel=fam)
     check_fp32(y, rows, cols, rowptr, colind, val, x, y0, 1.25, 0.75)
+
+
+@pytest.mark.parametrize("longest", [49, 60, 96, 97, 130, 192, 193, 300, 384, 385, 511, 512])
+@pytest.mark.parametrize("preprocess", [True, False])
+def test_even_rows_of_49_to_512_entries(osa, gpu_ctx, longest, preprocess):
+    """Rows of nearly equal length up to 512 entries go to the stream-rows tiles with 8 - 64 lanes a row; empty
+    rows, a first and a last row shorter than the rest, beta != 0."""
+    rng = np.random.default_rng(longest)
+    rows, cols = 2500, 9000
+    lengths = rng.integers(max(1, longest - longest // 6), longest + 1, rows)
+    lengths[[0, 17, rows - 1]] = [3, 0, 1]
+    lengths[5] = longest
+    rowptr, colind, val = csr_from_lengths(lengths, cols, seed=longest)
+    x = rng.uniform(-1, 1, cols).astype(np.float32)
+    y0 = rng.uniform(-1, 1, rows).astype(np.float32)
+    y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, -0.75, 1.5, preprocess=preprocess)
+    check_fp32(y, rows, cols, rowptr, colind, val, x, y0, -0.75, 1.5)
+    if preprocess and longest == 300:
+        # and through the raw layer, where the plan shows: the stream-rows family with 32 lanes a row
+        y = run_spmv(osa, gpu_ctx, rows, cols, rowptr, colind, val, x, y0, 2.0, 0.0,
+                     force_kernel=osa.OPSPARSE_SPMV_STREAM_ROWS)
+        check_fp32(y, rows, cols, rowptr, colind, val, x, y0, 2.0, 0.0)
