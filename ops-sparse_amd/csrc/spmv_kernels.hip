@@ -340,8 +340,9 @@ __global__ __launch_bounds__(kBlockThreads) void SpmvStreamRowsKernel(
     // all.  (Loads come back in the order they were issued: a row offset asked for inside that loop had to wait
     // for the next tile's entries, asked for just before it, and the tile ahead was no longer ahead - a 27-point
     // stencil on 128^3 points 163 us, 117 us with a workgroup a tile and nothing fetched ahead.)
-    __shared__ int32_t rowLds[kStreamRowsMax + 1];
-    __shared__ AccT yLds[kStreamRowsMax];
+    // (behind the products in the launch's LDS: rowsPerBlock old y, rowsPerBlock + 1 offsets)
+    AccT *const yLds = prod + capacity;
+    int32_t *const rowLds = reinterpret_cast<int32_t *>(yLds + rowsPerBlock);
     constexpr int kBoundRegs = (kStreamRowsMax + 1 + kBlockThreads - 1) / kBlockThreads;
     int32_t bnd[kBoundRegs];
     AccT yv[kBoundRegs];
@@ -1299,8 +1300,11 @@ MergeLayout MakeMergeLayout(int64_t rows, int64_t nnz)
 }
 
 template <typename ValT, typename OutT, typename AccT, int G, int U>
-int LaunchStreamU(const SpmvArgs &a, int32_t rowsPerBlock, size_t lds, int32_t skipLonger)
+int LaunchStreamU(const SpmvArgs &a, int32_t rowsPerBlock, size_t products, int32_t skipLonger)
 {
+    // the products of a tile, and behind them its old y and row offsets
+    const size_t lds = products * sizeof(AccT) + static_cast<size_t>(rowsPerBlock) * sizeof(AccT) +
+                       (static_cast<size_t>(rowsPerBlock) + 1) * sizeof(int32_t);
     if (rowsPerBlock < 1 || rowsPerBlock > kStreamRowsMax) {
         return OPSPARSE_E_INVALID;
     }
@@ -1325,7 +1329,7 @@ int LaunchStreamU(const SpmvArgs &a, int32_t rowsPerBlock, size_t lds, int32_t s
     hipLaunchKernelGGL((SpmvStreamRowsKernel<ValT, OutT, AccT, G, U>), dim3(grid), dim3(kBlockThreads), lds, a.stream,
                        a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x),
                        static_cast<OutT *>(a.y), static_cast<const OutT *>(a.yIn), a.rows, rowsPerBlock,
-                       static_cast<int32_t>(lds / sizeof(AccT)), skipLonger, a.alpha, a.beta);
+                       static_cast<int32_t>(products), skipLonger, a.alpha, a.beta);
     return CheckLaunch();
 }
 
@@ -1361,9 +1365,9 @@ int LaunchStreamTiles(const SpmvArgs &a, int32_t rowsPerBlock, int32_t tileRowNn
             return CheckLaunch();
         }
     }
-    if (products <= kBlockThreads * 4) return LaunchStreamU<ValT, OutT, AccT, G, 1>(a, rowsPerBlock, lds, skipLonger);
-    if (products <= kBlockThreads * 8) return LaunchStreamU<ValT, OutT, AccT, G, 2>(a, rowsPerBlock, lds, skipLonger);
-    return LaunchStreamU<ValT, OutT, AccT, G, 3>(a, rowsPerBlock, lds, skipLonger);
+    if (products <= kBlockThreads * 4) return LaunchStreamU<ValT, OutT, AccT, G, 1>(a, rowsPerBlock, products, skipLonger);
+    if (products <= kBlockThreads * 8) return LaunchStreamU<ValT, OutT, AccT, G, 2>(a, rowsPerBlock, products, skipLonger);
+    return LaunchStreamU<ValT, OutT, AccT, G, 3>(a, rowsPerBlock, products, skipLonger);
 }
 
 // The stream-rows family for a plan: the tiles, and the long rows beside them where the plan says so.
