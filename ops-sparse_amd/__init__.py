@@ -458,7 +458,7 @@ class SpmvOpPlan:
         check(lib().aclsparseSpMVOp_bufferSize(handle.h, *common, ctypes.byref(n)), "aclsparseSpMVOp_bufferSize")
         self.buffer_bytes = int(n.value)
         self.buffer = None
-        if alg == ACL_SPARSE_SPMVOP_ALG2:
+        if alg == ACL_SPARSE_SPMVOP_ALG2 or self.buffer_bytes > 0:
             self.buffer = torch.empty(max(self.buffer_bytes, 16), dtype=torch.uint8, device=z.t.device)
         check(lib().aclsparseSpMVOp_createDescr(handle.h, ctypes.byref(self.descr), *common,
                                                 _ptr(self.buffer) if self.buffer is not None else vp(None)),

@@ -139,7 +139,12 @@ struct RestoredChoice {
     size_t bytes;
     bool liveValues;  // BLOCKED_GATHER only: the layout holds no values, every call takes the caller's
 };
-// valueType: the OPSPARSE_* type of the values and of x (fp16 and bf16: BLOCKED_GATHER with frozen values only).
+// The layout a default-algorithm request for op(A) = A gets where it pays: BLOCKED_GATHER with live values (7 M
+// entries or more, an x the layout applies to, and a sample of the columns that says the gathers are scattered:
+// one short kernel and a synchronisation of the handle's stream), else none.
+RestoredChoice PickLiveLayout(aclsparseHandle_t handle, const int32_t *rowOffsets, const int32_t *colInd, int64_t rows,
+                              int64_t cols, int64_t nnz);
+// valueType: the OPSPARSE_* type of the values and of x.
 RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose, int32_t valueType);
 int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const void *values,
                     int32_t valueType, int64_t rows, int64_t cols, int64_t nnz, bool transpose, bool liveValues,

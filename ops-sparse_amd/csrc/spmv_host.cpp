@@ -141,41 +141,11 @@ Restored RestoredLayout(aclsparseHandle_t handle, aclsparseOperation_t opA, acls
     if (alg == ACL_SPARSE_SPMV_CSR_ALG2) {
         return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz, transpose, valueType);
     }
-    static const bool off = std::getenv("OPS_SPARSE_SPMV_NO_DEFAULT_BLOCKED") != nullptr ||
-                            std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") != nullptr;
-    if (off || transpose || matA->rowOffsets == nullptr || matA->colInd == nullptr) {
+    if (transpose) {
         return {0, 0, false};
     }
-    // Below 7 M entries the merge path on the caller's own arrays is as fast or faster (1 M rows x 4 entries: 30 us
-    // against 44 with the layout; 1.5 M x 4: 51 against 57; 2 M x 4: 87 against 71).  Tuning override, read at
-    // every call: OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ.
-    const char *minEnv = std::getenv("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ");
-    if (matA->nnz < (minEnv != nullptr ? std::atoll(minEnv) : 7000000LL)) {
-        return {0, 0, false};
-    }
-    const size_t bytes =
-        opsparse_spmv_csr_blocked_workspace_bytes(matA->rows, matA->cols, matA->nnz, OPSPARSE_BLOCKED_LIVE_VALUES);
-    if (bytes == 0) {
-        return {0, 0, false};
-    }
-    // scattered gathers?  Not under stream capture (nothing may synchronise there) and not without a workspace.
-    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-    if (hipStreamIsCapturing(handle->stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
-        (void)hipGetLastError();
-        return {0, 0, false};
-    }
-    if (opsparse::EnsureWorkspace(handle) != ACL_SPARSE_STATUS_SUCCESS) {
-        return {0, 0, false};
-    }
-    int32_t scattered = 0;
-    if (opsparse_spmv_csr_gathers_scattered(static_cast<const int32_t *>(matA->rowOffsets),
-                                            static_cast<const int32_t *>(matA->colInd), matA->rows, matA->cols,
-                                            matA->nnz, handle->workspace(), handle->workspaceBytes(), &scattered,
-                                            handle->stream) != OPSPARSE_OK ||
-        scattered < opsparse::kScatteredForLiveLayout) {
-        return {0, 0, false};
-    }
-    return {OPSPARSE_SPMV_BLOCKED_GATHER, bytes, true};
+    return opsparse::PickLiveLayout(handle, static_cast<const int32_t *>(matA->rowOffsets),
+                                    static_cast<const int32_t *>(matA->colInd), matA->rows, matA->cols, matA->nnz);
 }
 
 aclsparseStatus_t FromLaunch(int rc)
@@ -230,6 +200,43 @@ const OpsparseSpmvPlan *RowsSeen(aclsparseHandle_t handle, aclsparseConstSpMatDe
 }  // namespace
 
 namespace opsparse {
+
+RestoredChoice PickLiveLayout(aclsparseHandle_t handle, const int32_t *rowOffsets, const int32_t *colInd, int64_t rows,
+                              int64_t cols, int64_t nnz)
+{
+    static const bool off = std::getenv("OPS_SPARSE_SPMV_NO_DEFAULT_BLOCKED") != nullptr ||
+                            std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") != nullptr;
+    if (off || rowOffsets == nullptr || colInd == nullptr) {
+        return {0, 0, false};
+    }
+    // Below 7 M entries the merge path on the caller's own arrays is as fast or faster (1 M rows x 4 entries: 30 us
+    // against 44 with the layout; 1.5 M x 4: 51 against 57; 2 M x 4: 87 against 71).  Tuning override, read at
+    // every call: OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ.
+    const char *minEnv = std::getenv("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ");
+    if (nnz < (minEnv != nullptr ? std::atoll(minEnv) : 7000000LL)) {
+        return {0, 0, false};
+    }
+    const size_t bytes = opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, OPSPARSE_BLOCKED_LIVE_VALUES);
+    if (bytes == 0) {
+        return {0, 0, false};
+    }
+    // scattered gathers?  Not under stream capture (nothing may synchronise there) and not without a workspace.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(handle->stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return {0, 0, false};
+    }
+    if (EnsureWorkspace(handle) != ACL_SPARSE_STATUS_SUCCESS) {
+        return {0, 0, false};
+    }
+    int32_t scattered = 0;
+    if (opsparse_spmv_csr_gathers_scattered(rowOffsets, colInd, rows, cols, nnz, handle->workspace(),
+                                            handle->workspaceBytes(), &scattered, handle->stream) != OPSPARSE_OK ||
+        scattered < kScatteredForLiveLayout) {
+        return {0, 0, false};
+    }
+    return {OPSPARSE_SPMV_BLOCKED_GATHER, bytes, true};
+}
 
 RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose, int32_t valueType)
 {

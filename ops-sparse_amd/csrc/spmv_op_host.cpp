@@ -133,6 +133,19 @@ void LookAtRows(aclsparseHandle_t handle, aclsparseSpMVOpPlan *plan)
 // else column panels): the buffer then holds a copy of the matrix (indices and values), which is why csrValues
 // must not change under an ALG2 descriptor (reference include/cann_ops_sparse.h:64-69 says the same of its
 // own ALG2).
+// ALG1 / DEFAULT on a plain fp32 matrix whose gathers are scattered: the blocked-gather layout with live values,
+// as under aclsparseSpMVPreprocess with the default algorithm — if the caller brings the buffer that
+// aclsparseSpMVOp_bufferSize then asks for.  csrValues may change between executions, as ALG1 allows.
+opsparse::RestoredChoice LiveLayout(aclsparseHandle_t handle, aclsparseConstSpMatDescr_t matA)
+{
+    if (matA->rowOffsetsType != ACL_SPARSE_INDEX_32I || matA->idxBase != ACL_SPARSE_INDEX_BASE_ZERO ||
+        matA->valueType != ACL_FLOAT || matA->values == nullptr) {
+        return {0, 0, false};
+    }
+    return opsparse::PickLiveLayout(handle, static_cast<const int32_t *>(matA->rowOffsets),
+                                    static_cast<const int32_t *>(matA->colInd), matA->rows, matA->cols, matA->nnz);
+}
+
 opsparse::RestoredChoice RestoredLayout(aclsparseConstSpMatDescr_t matA)
 {
     if (matA->rowOffsetsType != ACL_SPARSE_INDEX_32I || matA->idxBase != ACL_SPARSE_INDEX_BASE_ZERO) {
@@ -180,12 +193,15 @@ aclsparseStatus_t aclsparseSpMVOp_bufferSize(aclsparseHandle_t handle, aclsparse
     if (matA->rows > INT32_MAX) {
         return ACL_SPARSE_STATUS_NOT_SUPPORTED;
     }
-    // ALG1 / DEFAULT need no buffer; ALG2 keeps its partition in one.
+    // ALG1 / DEFAULT need no buffer, but use one for a matrix with scattered gathers; ALG2 keeps its partition, or
+    // its copy of the matrix, in one.
     *bufferSize = 0;
     if (alg == ACL_SPARSE_SPMVOP_ALG2) {
         const size_t plain = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
         const size_t restored = RestoredLayout(matA).bytes;
         *bufferSize = restored > plain ? restored : plain;
+    } else {
+        *bufferSize = LiveLayout(handle, matA).bytes;
     }
     return ACL_SPARSE_STATUS_SUCCESS;
 }
@@ -268,6 +284,22 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
                 delete d;
                 return FromLaunch(rc);
             }
+            d->planned = true;
+        }
+    }
+    if (d->alg != ACL_SPARSE_SPMVOP_ALG2 && buffer != nullptr && Plain(d) && d->rows > 0 && d->nnz > 0) {
+        // the buffer aclsparseSpMVOp_bufferSize asked for (it asks the same question of the same arrays)
+        const opsparse::RestoredChoice live = LiveLayout(handle, matA);
+        if (live.kernel != 0) {
+            const int rc = opsparse::AnalyseRestored(live.kernel, static_cast<const int32_t *>(d->rowOffsets),
+                                                     static_cast<const int32_t *>(d->colInd), d->values, OPSPARSE_F32,
+                                                     d->rows, d->cols, d->nnz, false, true, buffer, live.bytes, &d->plan,
+                                                     handle->stream);
+            if (rc != OPSPARSE_OK) {
+                delete d;
+                return FromLaunch(rc);
+            }
+            d->userBuffer = buffer;
             d->planned = true;
         }
     }

@@ -69,6 +69,56 @@ def test_default_plan_is_the_live_blocked_layout_and_follows_the_values(osa, gpu
     assert 0 < resident < want
 
 
+@pytest.mark.parametrize("alias", [False, True])
+def test_spmvop_default_algorithm_takes_the_live_layout_when_given_the_buffer(osa, gpu_ctx, alias):
+    """aclsparseSpMVOp with the default algorithm on the same kind of matrix: bufferSize asks for the layout's
+    buffer, createDescr builds the layout in it, and the executions follow the values as they change in place (ALG1
+    promises nothing else).  Without the buffer the same call runs the ordinary kernels."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = 320_000, 1_500_000
+    rowptr, colind, val, x, y0 = _scattered(rows, cols, 6)
+    nnz = colind.size
+    want = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    A = osa.Csr(rows, cols, d[0], d[1], d[2])
+    d_y = to_dev(y0, dev)
+    d_z = d_y if alias else torch.zeros(rows, dtype=torch.float32, device=dev)
+    Y = osa.DnVec(d_y)
+    Z = Y if alias else osa.DnVec(d_z)
+    op = osa.SpmvOpPlan(handle, A, osa.DnVec(d[3]), Y, Z)    # ALG_DEFAULT
+    assert op.buffer_bytes == want > 0 and op.buffer is not None
+
+    def check(values, alpha, beta):
+        d_y.copy_(torch.from_numpy(y0))
+        op(alpha, beta)
+        stream.synchronize()
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, values, x, y0, alpha, beta)
+        assert oracle.max_rel_err(d_z.cpu().numpy(), gold) <= 1e-5
+        if not alias:
+            assert np.array_equal(d_y.cpu().numpy(), y0)
+
+    check(val, 1.0, 0.0)
+    val2 = (val * np.float32(0.5) - np.float32(0.125)).astype(np.float32)
+    d[2].copy_(torch.from_numpy(val2))
+    check(val2, -1.5, 0.75)
+    op.close()
+    # no buffer: the ordinary kernels, the same result
+    descr, plan = ctypes.c_void_p(), ctypes.c_void_p()
+    X = osa.DnVec(d[3])
+    common = (0, A.d, X.d, Y.d, Z.d, osa.ACL_FLOAT, osa.ACL_SPARSE_SPMVOP_ALG_DEFAULT)
+    assert L.aclsparseSpMVOp_createDescr(handle.h, ctypes.byref(descr), *common, None) == 0
+    assert L.aclsparseSpMVOp_createPlan(handle.h, descr, ctypes.byref(plan), None, 0) == 0
+    one, zero = ctypes.c_float(1.0), ctypes.c_float(0.0)
+    d_y.copy_(torch.from_numpy(y0))
+    assert L.aclsparseSpMVOp(handle.h, plan, ctypes.byref(one), ctypes.byref(zero), X.d, Y.d, Z.d) == 0
+    stream.synchronize()
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val2, x, y0, 1.0, 0.0)
+    assert oracle.max_rel_err(d_z.cpu().numpy(), gold) <= 1e-5
+    L.aclsparseSpMVOp_destroyPlan(plan)
+    L.aclsparseSpMVOp_destroyDescr(descr)
+
+
 def _with_long_rows(rows, cols, seed):
     """Short scattered rows and, among them, long ones: first row, last row, two neighbours, one with repeated
     columns (ascending all the same), one whose columns do not ascend, lengths either side of the threshold."""
