@@ -36,13 +36,16 @@ def _power_law(rows, cols, seed, longest, at_least=1):
     return csr_from_lengths(lengths, cols, seed + 1)
 
 
-@pytest.mark.parametrize("kind", ["stream_rows", "merge_path", "blocked_gather"])
+@pytest.mark.parametrize("kind", ["stream_rows", "stream_rows_lane_groups", "merge_path", "blocked_gather"])
 def test_spmv_replays(osa, gpu_ctx, kind):
     dev, stream, handle = gpu_ctx
     alg = osa.ACL_SPARSE_SPMV_ALG_DEFAULT
     if kind == "stream_rows":
         rows = cols = 40_000
         rowptr, colind, val = csr_from_lengths(np.full(rows, 5), cols, 1)
+    elif kind == "stream_rows_lane_groups":                 # rows of 100 entries: the persistent kernel, 16 lanes a row
+        rows = cols = 20_000
+        rowptr, colind, val = csr_from_lengths(np.random.default_rng(5).integers(90, 101, rows), cols, 1)
     elif kind == "merge_path":
         rows, cols = 30_000, 50_000
         rowptr, colind, val = _power_law(rows, cols, 2, 9_000)
