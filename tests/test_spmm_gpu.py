@@ -300,15 +300,17 @@ def test_row_length_mixes(osa, gpu_ctx, shape, n, beta):
     assert oracle.max_rel_err(got, gold) <= 1e-5
 
 
-def test_slab_table_cuts_by_work(osa, gpu_ctx):
+@pytest.mark.parametrize("longest,entries", [(256, 2048), (64, 1024)])
+def test_slab_table_cuts_by_work(osa, gpu_ctx, longest, entries):
     """The analysis leaves, for the slab kernel, the first row of every slab: slab s starts at the first row with
     s * share entries + rows in front of it, whatever the order of the rows (checked against numpy on rows sorted
-    by length, where slabs of equal numbers of rows would differ in work a hundredfold)."""
+    by length, where slabs of equal numbers of rows would differ in work a hundredfold).  About 2048 entries a
+    slab; 1024 where no row exceeds 64 entries and B has at most 128 columns."""
     import torch
     dev, stream, handle = gpu_ctx
     rng = np.random.default_rng(3)
     m = 300_000
-    lengths = np.sort(np.minimum((1.0 / rng.uniform(1e-4, 1.0, m)).astype(np.int64), 256))[::-1].copy()
+    lengths = np.sort(np.minimum((1.0 / rng.uniform(1e-4, 1.0, m)).astype(np.int64), longest))[::-1].copy()
     rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
     nnz = int(rowptr[-1])
     L = osa.lib()
@@ -324,12 +326,12 @@ def test_slab_table_cuts_by_work(osa, gpu_ctx):
     assert plan.numSlabs > 0 and plan.slabStartOff >= 256 and plan.bytes <= size.value
     table = ws[plan.slabStartOff: plan.slabStartOff + 4 * (plan.numSlabs + 1)].view(torch.int32).cpu().numpy()
     work = rowptr[:-1].astype(np.int64) + np.arange(m)            # entries + rows in front of row r
-    share = 2048 + min(max(2048 * m // nnz, 16), 4096)            # about 2048 entries and their rows a slab
+    share = entries + min(max(entries * m // nnz, 16), 4096)     # that many entries and their rows a slab
     assert plan.numSlabs == -(-(m + nnz) // share)
     want = np.concatenate([np.searchsorted(work, np.arange(plan.numSlabs) * share, side="left"), [m]])
     assert np.array_equal(table, want)
     per_slab = np.diff(np.concatenate([work, [m + nnz]])[table])
-    assert per_slab.max() <= share + 257                           # a slab overshoots its share by at most a row
+    assert per_slab.max() <= share + longest + 1                   # a slab overshoots its share by at most a row
 
 
 @pytest.mark.parametrize("lengths,binned", [("even 300", False), ("even 2048", False), ("even 2049", True),
