@@ -881,7 +881,9 @@ void LayoutPlan(OpsparseSpmmPlan *p)
     int64_t off = 256;
     p->numSlabs = SlabCount(p->rows, p->nnz, p->maxRowNnz, p->n);  // (maxRowNnz and n set by the caller)
     p->slabStartOff = off;
-    off = Align256(off + 4 * (p->numSlabs + 1));
+    // Room for the table of a narrow B whatever n is: a buffer sized for a wide B serves a narrower one as well.
+    const int64_t reserveSlabs = SlabCount(p->rows, p->nnz, p->maxRowNnz, 1);
+    off = Align256(off + 4 * ((reserveSlabs > p->numSlabs ? reserveSlabs : p->numSlabs) + 1));
     const int64_t slabEnd = off;
     p->longRowsOff = off;
     off = Align256(off + 4 * static_cast<int64_t>(p->numLongRows));

@@ -334,6 +334,35 @@ def test_slab_table_cuts_by_work(osa, gpu_ctx, longest, entries):
     assert per_slab.max() <= share + longest + 1                   # a slab overshoots its share by at most a row
 
 
+def test_buffer_sized_for_a_wide_b_serves_a_narrow_one(osa, gpu_ctx):
+    """GetBufferSize for n = 256, then the same buffer and matrix with n = 64 (rows of at most 64 entries, whose
+    slabs are shorter, and their table longer, for a narrow B): the size asked for the wide B covers it, and the
+    bytes behind the buffer stay as they were."""
+    import torch
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rng = np.random.default_rng(8)
+    m, k = 200_000, 5000
+    rowptr, colind, val = csr_from_lengths(rng.integers(20, 41, m), k, seed=4)
+    d_rp = to_dev(rowptr, dev)
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    wide, narrow = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    nnz = int(rowptr[-1])
+    assert L.opsparse_spmm_csr_workspace_bytes(d_rp.data_ptr(), m, nnz, 256, sp, ctypes.byref(wide)) == 0
+    assert L.opsparse_spmm_csr_workspace_bytes(d_rp.data_ptr(), m, nnz, 64, sp, ctypes.byref(narrow)) == 0
+    assert wide.value >= narrow.value > 0
+    guard = 4096
+    ws = torch.full((wide.value + guard,), 0x5A, dtype=torch.uint8, device=dev)
+    plan = osa.OpsparseSpmmPlan()
+    assert L.opsparse_spmm_csr_analyse(d_rp.data_ptr(), m, nnz, 64, ws.data_ptr(), wide.value, 0, ctypes.byref(plan),
+                                       sp) == 0
+    stream.synchronize()
+    assert plan.bytes <= wide.value and plan.slabStartOff + 4 * (plan.numSlabs + 1) <= wide.value
+    assert bool((ws[wide.value:] == 0x5A).all())
+    table = ws[plan.slabStartOff: plan.slabStartOff + 4 * (plan.numSlabs + 1)].view(torch.int32).cpu().numpy()
+    assert table[0] == 0 and table[-1] == m and np.all(np.diff(table) >= 0)
+
+
 @pytest.mark.parametrize("lengths,binned", [("even 300", False), ("even 2048", False), ("even 2049", True),
                                             ("300 among 10", False), ("2100 among 10", True)])
 def test_only_rows_beyond_2048_entries_are_cut_into_segments(osa, gpu_ctx, lengths, binned):
