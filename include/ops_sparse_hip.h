@@ -63,10 +63,19 @@ typedef enum OpsparseSpmvKernel {
     OPSPARSE_SPMV_COLUMN_PANELS = 5,/* x larger than an L2: the matrix re-stored as panels of 2^20 columns, each
                                       worked on one XCD so that its slice of x stays in that L2; fp32 only; holds a
                                       copy of the VALUES as they were at analysis time */
-    OPSPARSE_SPMV_BLOCKED_GATHER = 6 /* x larger than an L2: two passes.  Entries re-stored by panels of 2^15 columns,
-                                      x gathered from LDS into a linear stream; then row blocks of up to 2^14 rows
-                                      summed in LDS.  16 bytes of traffic per entry and no line-sized gathers;
-                                      fp32 only; holds a copy of the VALUES as they were at analysis time */
+    OPSPARSE_SPMV_BLOCKED_GATHER = 6,/* x larger than an L2: two passes.  The entries' columns re-stored by panels of
+                                      2^15 columns, x gathered from LDS into a linear stream; then row blocks whose
+                                      gathered x is put back into row order in LDS and summed against the values,
+                                      read in place, in an order that the layout fixes: the same bits at every
+                                      call.  16 bytes of traffic per entry and no line-sized gathers; fp32 / fp16 /
+                                      bf16 / int32, op(A) = A or (on a transposed copy) A^T */
+    OPSPARSE_SPMV_BLOCKED_LIVE = 7  /* the same two passes with the second one built for speed: it collects a row
+                                      block's values in LDS, streams the block's entries panel by panel against
+                                      them and adds into one fp64 accumulator a row with LDS atomics, in the order
+                                      the wavefronts get there: the last bit of a result may differ between two
+                                      calls.  The plan of aclsparseSpMVPreprocess under ACL_SPARSE_SPMV_ALG_DEFAULT,
+                                      whose results the reference lets vary; fp32 / fp16 / bf16, op(A) = A, values
+                                      read where the caller has them at every call */
 } OpsparseSpmvKernel;
 
 #define OPSPARSE_SPMV_MAX_PANELS 16
@@ -90,16 +99,17 @@ typedef struct OpsparseSpmvPlan {
     int32_t tileRowNnz;    /* STREAM_ROWS: the row length the tiles are sized for (0: maxRowNnz) */
     int32_t longRowsBeside;/* STREAM_ROWS: a few rows are longer than that: the tiles skip rows of more than 64
                               entries and a second kernel sums those, a workgroup per row */
-    int32_t liveValues;    /* BLOCKED_GATHER: the layout holds no values; every launch takes the caller's csrValues as
-                              they are then: nothing goes stale when values change in place or the values pointer
-                              is replaced (1: 32-bit positions of the entries, 2: 16-bit ones relative to their
-                              row block, which the analysis chooses where every block is shorter than 65535) */
+    int32_t liveValues;    /* BLOCKED_GATHER / BLOCKED_LIVE: the layout holds no values; every launch takes the caller's
+                              csrValues as they are then: nothing goes stale when values change in place or the
+                              values pointer is replaced (BLOCKED_LIVE: 1: 32-bit positions of the entries, 2: 16-bit
+                              ones relative to their row block, where every block is shorter than 65535) */
     int32_t numLongRows;   /* BLOCKED_GATHER: rows kept out of the re-stored layout: phase 1 sums them from the caller's
                               colInd / csrValues, panel by panel, with the panel's x in LDS */
     int32_t numDeferredLongRows; /* BLOCKED_GATHER: those of them that sit more than 64 to a row block: a third kernel,
                               a wavefront a row, adds their partial sums up instead of the block's workgroup */
-    int32_t valueType;     /* BLOCKED_GATHER: the OPSPARSE_F32 / F16 / BF16 the layout was built from; launches must
-                              bring values and x of that type (y: fp32, or that type) */
+    int32_t valueType;     /* BLOCKED_GATHER: the OPSPARSE_F32 / F16 / BF16 / I32 the layout was built from; launches
+                              must bring values and x of that type (y: fp32, or that type) */
+    int32_t numEmptyRows;  /* BLOCKED_GATHER: rows without entries; a small kernel of their own writes beta * y there */
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */
@@ -162,37 +172,57 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
                                      OpsparseSpmvPlan *plan, void *stream);
 
 /*
- * BLOCKED_GATHER analysis (fp32, or fp16 / bf16 values and x with y fp32 or of the same type): bytes of the workspace, or 0 when the family does
- * not apply (x must have more than 2^18 and at most 2^25 elements, the matrix at least
- * two million entries, and a (panel, row block) chunk at least 32 entries on average).  transpose != 0 builds the layout of
- * y = alpha * A^T * x + beta * y instead: panels over the rows of A, blocks over its
- * columns, with no atomics on y; a plan serves the op(A) it was built for.  Like the panel
- * analysis it re-stores indices AND values in the workspace; launches with the
- * resulting plan ignore the rowOffsets / colInd / csrValues arguments.  Returns
- * OPSPARSE_E_INVALID for a column index outside [0, cols).  Synchronises `stream` once.
- * Rows with many entries in every column panel and ascending columns ("long rows", plan->numLongRows of them)
- * are summed by the first kernel instead of going through the row-block order.
- * Launches touch only the first opsparse_spmv_csr_blocked_resident_bytes() of the workspace; the rest serves the
- * analysis and may be handed back afterwards (a launch accepts a workspace of at least the resident size).
- * `flags`: OPSPARSE_BLOCKED_TRANSPOSE (= 1, so that a plain 0 / 1 "transpose" still reads right) and / or
- * OPSPARSE_BLOCKED_LIVE_VALUES: the layout keeps the block-order position of every entry instead of the values
- * and every launch takes the values from the csrValues argument (8 more bytes of traffic per entry, all
- * streamed), and for the long rows the column indices from colInd as well: such a plan never goes stale when
- * values change; rowOffsets / colInd must be the arrays of the analysis.
- * OPSPARSE_BLOCKED_VALUES_F16 / _BF16: csrValues (and, at the launches, x) are fp16 / bf16 instead of fp32; the
- * layout keeps frozen values as fp32, which holds them exactly, live ones are widened where the launches read
- * them, and the first kernel widens x while it loads a panel's slice.  At the launches y is fp32 or of the values'
- * 16-bit type (one rounding of the fp64 sum).
+ * BLOCKED_GATHER analysis: bytes of the workspace, or 0 when the family does not apply (x must have more than 2^18
+ * and at most 2^25 elements, the matrix at least two million entries, and a (panel, row block) chunk at least 8
+ * entries on average).  Values and x are fp32, fp16, bf16 or int32 (`flags`); at the launches y is fp32 or of the
+ * values' own type, int32 under the integer compute type.
+ * The layout holds where the entries' columns sit in 2^15-column panels, the place of every entry in its row block,
+ * and small tables by which a block's kernel tells its rows apart.  Every row is summed in an order that the layout
+ * fixes (fp64 for floating-point data, rounded once; 32-bit wrap-around for the integer compute type): two launches
+ * on the same data give the same bits.
+ * `flags`:
+ *   OPSPARSE_BLOCKED_LIVE_VALUES  no value is kept: every launch reads csrValues (and, for long rows, colInd) where
+ *       the caller has them; rowOffsets / colInd must be the arrays of the analysis, the values may change.  Without
+ *       it (values frozen) the analysis keeps a copy of the values, launches ignore the rowOffsets / colInd /
+ *       csrValues arguments, and the analysis must be repeated after the values change; rows of 1024 entries and more
+ *       are then stored a second time panel by panel, which halves what they cost.
+ *   OPSPARSE_BLOCKED_TRANSPOSE (= 1, so that a plain 0 / 1 "transpose" still reads right)  the layout of
+ *       y = alpha * A^T * x + beta * y: the analysis transposes the matrix into the workspace (the CSC arrays of A
+ *       are the CSR arrays of A^T) and builds the layout of that copy; no atomics on y.  With live values it keeps
+ *       the entry of A behind every entry of the copy, and a launch first refreshes the copy's values from
+ *       csrValues.  A plan serves the op(A) it was built for.
+ *   OPSPARSE_BLOCKED_VALUES_F16 / _BF16 / _I32  the type of csrValues and x (default fp32).
+ * Rows with many entries in every column panel and ascending columns ("long rows", plan->numLongRows of them) are
+ * summed by the first kernel instead of going through the row blocks.  Returns OPSPARSE_E_INVALID for a column
+ * index outside [0, cols), OPSPARSE_E_UNSUPPORTED for a matrix with a row of more than about 50 000 entries that
+ * cannot go the long rows' way (its columns do not ascend).  Synchronises `stream` twice (three times for
+ * op(A) = A^T).  Launches touch only the first opsparse_spmv_csr_blocked_resident_bytes() of the workspace; the rest
+ * serves the analysis and may be handed back afterwards.
  */
 #define OPSPARSE_BLOCKED_TRANSPOSE 1
 #define OPSPARSE_BLOCKED_LIVE_VALUES 2
 #define OPSPARSE_BLOCKED_VALUES_F16 4
 #define OPSPARSE_BLOCKED_VALUES_BF16 8
+#define OPSPARSE_BLOCKED_VALUES_I32 16
 size_t opsparse_spmv_csr_blocked_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t flags);
 size_t opsparse_spmv_csr_blocked_resident_bytes(int64_t rows, int64_t cols, int64_t nnz, int32_t flags);
 int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
                                       int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
                                       size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream);
+
+/*
+ * BLOCKED_LIVE analysis (fp32, fp16 or bf16 values and x, op(A) = A, values read in place at every launch): the
+ * layout of the plan kernel OPSPARSE_SPMV_BLOCKED_LIVE, whose second kernel adds into LDS with atomics in the order
+ * the wavefronts get there — the fastest plan for a matrix with scattered columns whose values change between
+ * calls, for callers who do not need the last bit of a result to repeat.  Same applicability bounds as BLOCKED_GATHER
+ * except that a chunk needs 8 entries on average; `flags`: OPSPARSE_BLOCKED_VALUES_F16 / _BF16 only.  Synchronises
+ * `stream` twice.  No counterpart in the reference.
+ */
+size_t opsparse_spmv_csr_live_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz);
+size_t opsparse_spmv_csr_live_resident_bytes(int64_t rows, int64_t cols, int64_t nnz);
+int opsparse_spmv_csr_live_analyse(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
+                                   int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
+                                   size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream);
 
 /* Same as opsparse_spmv_csr_launch with separate input and output vectors:
  * z = alpha * op(A) * x + beta * yIn.  z may be yIn (in place); yIn is only read

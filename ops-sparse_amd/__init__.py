@@ -61,7 +61,9 @@ OPSPARSE_F32, OPSPARSE_F16, OPSPARSE_BF16, OPSPARSE_I32, OPSPARSE_I8 = range(5)
 OPSPARSE_OK, OPSPARSE_E_INVALID, OPSPARSE_E_UNSUPPORTED, OPSPARSE_E_WORKSPACE, OPSPARSE_E_LAUNCH = 0, -1, -2, -3, -4
 OPSPARSE_SPMV_COLUMN_PANELS = 5
 OPSPARSE_SPMV_BLOCKED_GATHER = 6
+OPSPARSE_SPMV_BLOCKED_LIVE = 7
 OPSPARSE_BLOCKED_TRANSPOSE, OPSPARSE_BLOCKED_LIVE_VALUES = 1, 2
+OPSPARSE_BLOCKED_VALUES_F16, OPSPARSE_BLOCKED_VALUES_BF16, OPSPARSE_BLOCKED_VALUES_I32 = 4, 8, 16
 OPSPARSE_SPMM_AUTO, OPSPARSE_SPMM_ROW_SPLIT, OPSPARSE_SPMM_BINNED = range(3)
 
 # Every symbol the two public headers declare; tests check that the library exports all of them.
@@ -96,6 +98,7 @@ OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_panels_workspace_bytes", "opsparse_spmv_csr_panels_analyse",
     "opsparse_spmv_csr_blocked_workspace_bytes", "opsparse_spmv_csr_blocked_resident_bytes",
     "opsparse_spmv_csr_blocked_analyse",
+    "opsparse_spmv_csr_live_workspace_bytes", "opsparse_spmv_csr_live_resident_bytes", "opsparse_spmv_csr_live_analyse",
     "opsparse_spmv_csr_gathers_scattered",
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
     "opsparse_dense_restage",
@@ -121,7 +124,7 @@ class OpsparseSpmvPlan(ctypes.Structure):
                 ("maxRowNnz", i32), ("partitionReady", i32), ("numPanels", i32),
                 ("panelShift", i32), ("numRowBlocks", i32), ("entryWindow", i32), ("transposed", i32),
                 ("guardTiles", i32), ("tileRowNnz", i32), ("longRowsBeside", i32), ("liveValues", i32),
-                ("numLongRows", i32), ("numDeferredLongRows", i32), ("valueType", i32), ("rows", i64), ("nnz", i64),
+                ("numLongRows", i32), ("numDeferredLongRows", i32), ("valueType", i32), ("numEmptyRows", i32), ("rows", i64), ("nnz", i64),
                 ("partOff", i64),
                 ("carryOff", i64), ("headOff", i64), ("bytes", i64), ("panelStart", i64 * 17)]
 
@@ -262,6 +265,13 @@ def lib():
     L.opsparse_spmv_csr_blocked_workspace_bytes.argtypes = [i64, i64, i64, i32]
     L.opsparse_spmv_csr_blocked_resident_bytes.restype = sz
     L.opsparse_spmv_csr_blocked_resident_bytes.argtypes = [i64, i64, i64, i32]
+    L.opsparse_spmv_csr_live_workspace_bytes.restype = sz
+    L.opsparse_spmv_csr_live_workspace_bytes.argtypes = [i64, i64, i64]
+    L.opsparse_spmv_csr_live_resident_bytes.restype = sz
+    L.opsparse_spmv_csr_live_resident_bytes.argtypes = [i64, i64, i64]
+    L.opsparse_spmv_csr_live_analyse.restype = ctypes.c_int
+    L.opsparse_spmv_csr_live_analyse.argtypes = [vp, vp, vp, i64, i64, i64, i32, vp, sz,
+                                                 ctypes.POINTER(OpsparseSpmvPlan), vp]
     L.opsparse_spmv_csr_blocked_analyse.restype = ctypes.c_int
     L.opsparse_spmv_csr_blocked_analyse.argtypes = [vp, vp, vp, i64, i64, i64, i32, vp, sz,
                                                     ctypes.POINTER(OpsparseSpmvPlan), vp]

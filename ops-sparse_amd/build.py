@@ -31,6 +31,7 @@ SOURCES = [
     "convert_host.cpp",
     "spmv_kernels.hip",
     "spmv_blocked.hip",
+    "spmv_blocked_live.hip",
     "spmm_kernels.hip",
     "convert_kernels.hip",
     "measure_kernels.hip",

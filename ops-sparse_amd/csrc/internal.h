@@ -50,6 +50,21 @@ struct OpsparseSpmvRowsSeen {
     OpsparseSpmvPlan plan{};
 };
 
+// What the last buffer-size query on a matrix answered (aclsparseSpMVGetBufferSize, aclsparseSpMVOp_bufferSize).
+// Preprocess / createDescr only know the caller's buffer by its address: they write a re-stored layout into it
+// only when this record says that a query on the same arrays asked for that many bytes; anything else (no query,
+// arrays replaced since, a query under stream capture that could not look at the columns) gets the plan that fits
+// the small size every query answers at least.
+struct OpsparseSpmvSized {
+    const void *rowOffsets = nullptr, *colInd = nullptr;
+    int64_t rows = -1, cols = -1, nnz = -1;
+    int32_t kernel = 0;      // OPSPARSE_SPMV_BLOCKED_GATHER / BLOCKED_LIVE / COLUMN_PANELS, 0: none
+    bool transpose = false;  // ... for this op(A)
+    bool liveValues = false;
+    int32_t valueType = -1;
+    size_t bytes = 0;        // of the layout
+};
+
 struct OpsparseSpmmBinding {
     const void *buffer = nullptr;
     OpsparseSpmmPlan plan{};
@@ -89,6 +104,7 @@ struct aclsparseSpMatDescr {
     // (sparse/spmm/arch35/spmm_host.cpp:360); `mutable` makes that explicit.
     mutable OpsparseSpmvBinding spmv;
     mutable OpsparseSpmvRowsSeen rowsSeen;
+    mutable OpsparseSpmvSized spmvSized;
     mutable OpsparseSpmmBinding spmm;
 };
 
@@ -137,13 +153,18 @@ constexpr int32_t kScatteredForLiveLayout = 310;
 struct RestoredChoice {
     int32_t kernel;
     size_t bytes;
-    bool liveValues;  // BLOCKED_GATHER only: the layout holds no values, every call takes the caller's
+    bool liveValues;  // BLOCKED_GATHER / BLOCKED_LIVE: the layout holds no values, every call takes the caller's
 };
-// The layout a default-algorithm request for op(A) = A gets where it pays: BLOCKED_GATHER with live values (7 M
+// The layout a default-algorithm request gets where it pays: blocked gather with live values (7 M
 // entries or more, an x the layout applies to, and a sample of the columns that says the gathers are scattered:
-// one short kernel and a synchronisation of the handle's stream), else none.
+// one short kernel and a synchronisation of the handle's stream), else none.  `repeatable`: the caller promises
+// the same bits from every execution (aclsparseSpMVOp): BLOCKED_GATHER; else BLOCKED_LIVE where it exists
+// (op(A) = A, floating-point values).
 RestoredChoice PickLiveLayout(aclsparseHandle_t handle, const int32_t *rowOffsets, const int32_t *colInd, int64_t rows,
-                              int64_t cols, int64_t nnz);
+                              int64_t cols, int64_t nnz, bool transpose, int32_t valueType, bool repeatable);
+// The size-query record of a matrix (OpsparseSpmvSized): written by the queries, asked by Preprocess / createDescr.
+void RememberSized(aclsparseConstSpMatDescr_t matA, const RestoredChoice &choice, bool transpose, int32_t valueType);
+bool SizedFor(aclsparseConstSpMatDescr_t matA, const RestoredChoice &choice, bool transpose, int32_t valueType);
 // valueType: the OPSPARSE_* type of the values and of x.
 RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose, int32_t valueType);
 int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const void *values,

@@ -102,10 +102,14 @@ aclsparseStatus_t ValidateData(SpmvCall *c, aclDataType computeType)
 // The re-stored layouts, where they apply (fp32, x larger than an L2).
 // CSR_ALG2 asks for one: the blocked-gather layout first, the column panels where that one does not fit the
 // matrix; both hold a copy of the values as they were at Preprocess.
-// ALG_DEFAULT / CSR_ALG1 with op(A) = A get the blocked-gather layout with LIVE values (every call re-reads the
-// caller's values, so nothing can go stale) when the gathers of x are scattered: 0.35 ms against 1.1 ms for the
-// merge path on an 8 M x 8 M power-law matrix.  GetBufferSize and Preprocess ask the same question of the same
-// arrays (a sample of the column indices, one short kernel and a synchronisation), so they agree on the size.
+// ALG_DEFAULT / CSR_ALG1 get a layout with LIVE values (every call re-reads the caller's values, so nothing can go
+// stale) when the gathers of x are scattered: 0.35 ms against 1.1 ms for the merge path on an 8 M x 8 M power-law
+// matrix.  For op(A) = A and floating-point values that is the layout whose row blocks add with LDS atomics: these
+// algorithm values promise no bit-wise repeatable result (reference include/cann_ops_sparse.h:57-60, only CSR_ALG2
+// is "deterministic").  OPS_SPARSE_SPMV_REPEATABLE in the environment (read at every size query / Preprocess) asks
+// for the ordered layout there too: same bits from every call, about 0.5 ms on that matrix.  op(A) = A^T and
+// int32 values always get the ordered one.  GetBufferSize and Preprocess ask the same question of the same arrays
+// (a sample of the column indices, one short kernel and a synchronisation), so they agree on the size.
 using Restored = opsparse::RestoredChoice;
 
 // The OPSPARSE_* type of values and x where a re-stored layout can hold them, else -1.
@@ -121,6 +125,8 @@ int32_t RestoredValueType(aclsparseConstSpMatDescr_t matA, aclsparseConstDnVecDe
             return OPSPARSE_F16;
         case ACL_BF16:
             return OPSPARSE_BF16;
+        case ACL_INT32:
+            return OPSPARSE_I32;
         default:
             return -1;
     }
@@ -130,22 +136,27 @@ Restored RestoredLayout(aclsparseHandle_t handle, aclsparseOperation_t opA, acls
                         aclsparseConstDnVecDescr_t vecX, aclsparseConstDnVecDescr_t vecY, aclDataType computeType,
                         aclsparseSpMVAlg_t alg)
 {
-    // fp32 throughout, or fp16 / bf16 values and x with y fp32 or of the same 16-bit type (the blocked-gather layout
-    // only: it keeps frozen values as fp32, widens live ones, and x, where it reads them, and rounds y once)
+    // fp32 throughout, fp16 / bf16 values and x with y fp32 or of the same 16-bit type, or int32 values and x with
+    // y int32 under the integer compute type and fp32 under the floating-point one (the blocked-gather layout
+    // only: it reads the values where they are, widens x where it loads it, and rounds y once)
     const int32_t valueType = RestoredValueType(matA, vecX);
-    if (computeType != ACL_FLOAT || valueType < 0 ||
-        (vecY->valueType != ACL_FLOAT && vecY->valueType != matA->valueType)) {
+    if (valueType < 0) {
+        return {0, 0, false};
+    }
+    if (valueType == OPSPARSE_I32) {
+        if (vecY->valueType != (computeType == ACL_INT32 ? ACL_INT32 : ACL_FLOAT)) {
+            return {0, 0, false};
+        }
+    } else if (computeType != ACL_FLOAT || (vecY->valueType != ACL_FLOAT && vecY->valueType != matA->valueType)) {
         return {0, 0, false};
     }
     const bool transpose = opA != ACL_SPARSE_OP_NON_TRANSPOSE;
     if (alg == ACL_SPARSE_SPMV_CSR_ALG2) {
         return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz, transpose, valueType);
     }
-    if (transpose) {
-        return {0, 0, false};
-    }
     return opsparse::PickLiveLayout(handle, static_cast<const int32_t *>(matA->rowOffsets),
-                                    static_cast<const int32_t *>(matA->colInd), matA->rows, matA->cols, matA->nnz);
+                                    static_cast<const int32_t *>(matA->colInd), matA->rows, matA->cols, matA->nnz,
+                                    transpose, valueType, std::getenv("OPS_SPARSE_SPMV_REPEATABLE") != nullptr);
 }
 
 aclsparseStatus_t FromLaunch(int rc)
@@ -201,8 +212,40 @@ const OpsparseSpmvPlan *RowsSeen(aclsparseHandle_t handle, aclsparseConstSpMatDe
 
 namespace opsparse {
 
+int32_t BlockedFlags(bool transpose, bool liveValues, int32_t valueType)
+{
+    return (transpose ? OPSPARSE_BLOCKED_TRANSPOSE : 0) | (liveValues ? OPSPARSE_BLOCKED_LIVE_VALUES : 0) |
+           (valueType == OPSPARSE_F16    ? OPSPARSE_BLOCKED_VALUES_F16
+            : valueType == OPSPARSE_BF16 ? OPSPARSE_BLOCKED_VALUES_BF16
+            : valueType == OPSPARSE_I32  ? OPSPARSE_BLOCKED_VALUES_I32
+                                         : 0);
+}
+
+void RememberSized(aclsparseConstSpMatDescr_t matA, const RestoredChoice &choice, bool transpose, int32_t valueType)
+{
+    OpsparseSpmvSized &z = matA->spmvSized;
+    z.rowOffsets = matA->rowOffsets;
+    z.colInd = matA->colInd;
+    z.rows = matA->rows;
+    z.cols = matA->cols;
+    z.nnz = matA->nnz;
+    z.kernel = choice.kernel;
+    z.transpose = transpose;
+    z.liveValues = choice.liveValues;
+    z.valueType = valueType;
+    z.bytes = choice.bytes;
+}
+
+bool SizedFor(aclsparseConstSpMatDescr_t matA, const RestoredChoice &choice, bool transpose, int32_t valueType)
+{
+    const OpsparseSpmvSized &z = matA->spmvSized;
+    return choice.kernel != 0 && z.kernel == choice.kernel && z.bytes >= choice.bytes && z.rowOffsets == matA->rowOffsets &&
+           z.colInd == matA->colInd && z.rows == matA->rows && z.cols == matA->cols && z.nnz == matA->nnz &&
+           z.transpose == transpose && z.liveValues == choice.liveValues && z.valueType == valueType;
+}
+
 RestoredChoice PickLiveLayout(aclsparseHandle_t handle, const int32_t *rowOffsets, const int32_t *colInd, int64_t rows,
-                              int64_t cols, int64_t nnz)
+                              int64_t cols, int64_t nnz, bool transpose, int32_t valueType, bool repeatable)
 {
     static const bool off = std::getenv("OPS_SPARSE_SPMV_NO_DEFAULT_BLOCKED") != nullptr ||
                             std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") != nullptr;
@@ -216,11 +259,16 @@ RestoredChoice PickLiveLayout(aclsparseHandle_t handle, const int32_t *rowOffset
     if (nnz < (minEnv != nullptr ? std::atoll(minEnv) : 7000000LL)) {
         return {0, 0, false};
     }
-    const size_t bytes = opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, OPSPARSE_BLOCKED_LIVE_VALUES);
+    // Results that may differ in the last bit between calls (the reference's ALG_DEFAULT / CSR_ALG1 of aclsparseSpMV)
+    // get the layout whose row blocks add with atomics, where there is one: op(A) = A, floating-point data.
+    const bool atomics = !repeatable && !transpose && valueType != OPSPARSE_I32;
+    const size_t bytes =
+        atomics ? opsparse_spmv_csr_live_workspace_bytes(rows, cols, nnz)
+                : opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, BlockedFlags(transpose, true, valueType));
     if (bytes == 0) {
         return {0, 0, false};
     }
-    // scattered gathers?  Not under stream capture (nothing may synchronise there) and not without a workspace.
+    // scattered gathers (op(A) = A^T: scattered updates of y)?  Not under stream capture (nothing may synchronise there) and not without a workspace.
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(handle->stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
         (void)hipGetLastError();
@@ -235,13 +283,14 @@ RestoredChoice PickLiveLayout(aclsparseHandle_t handle, const int32_t *rowOffset
         scattered < kScatteredForLiveLayout) {
         return {0, 0, false};
     }
-    return {OPSPARSE_SPMV_BLOCKED_GATHER, bytes, true};
+    return {atomics ? OPSPARSE_SPMV_BLOCKED_LIVE : OPSPARSE_SPMV_BLOCKED_GATHER, bytes, true};
 }
 
 RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose, int32_t valueType)
 {
     if (std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") == nullptr) {
-        const size_t blocked = opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, transpose ? 1 : 0);
+        const size_t blocked =
+            opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, BlockedFlags(transpose, false, valueType));
         if (blocked > 0) {
             return {OPSPARSE_SPMV_BLOCKED_GATHER, blocked, false};
         }
@@ -283,14 +332,19 @@ int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *co
     if (scattered < kScatteredForFrozenLayout) {
         return opsparse_spmv_csr_analyse(rowOffsets, rows, cols, nnz, buffer, bytes, OPSPARSE_SPMV_AUTO, plan, stream);
     }
+    if (kernel == OPSPARSE_SPMV_BLOCKED_LIVE) {
+        return opsparse_spmv_csr_live_analyse(rowOffsets, colInd, values, rows, cols, nnz,
+                                              BlockedFlags(false, true, valueType), buffer, bytes, plan, stream);
+    }
     if (kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {
-        return opsparse_spmv_csr_blocked_analyse(rowOffsets, colInd, values, rows, cols, nnz,
-                                                 (transpose ? OPSPARSE_BLOCKED_TRANSPOSE : 0) |
-                                                     (liveValues ? OPSPARSE_BLOCKED_LIVE_VALUES : 0) |
-                                                     (valueType == OPSPARSE_F16    ? OPSPARSE_BLOCKED_VALUES_F16
-                                                      : valueType == OPSPARSE_BF16 ? OPSPARSE_BLOCKED_VALUES_BF16
-                                                                                   : 0),
-                                                 buffer, bytes, plan, stream);
+        const int rc = opsparse_spmv_csr_blocked_analyse(rowOffsets, colInd, values, rows, cols, nnz,
+                                                         BlockedFlags(transpose, liveValues, valueType), buffer, bytes,
+                                                         plan, stream);
+        if (rc == OPSPARSE_E_UNSUPPORTED) {
+            // (a row too long for a row block that cannot go the long rows' way: the ordinary plan)
+            return opsparse_spmv_csr_analyse(rowOffsets, rows, cols, nnz, buffer, bytes, OPSPARSE_SPMV_AUTO, plan, stream);
+        }
+        return rc;
     }
     if (valueType != OPSPARSE_F32) {
         return OPSPARSE_E_UNSUPPORTED;
@@ -330,6 +384,7 @@ aclsparseStatus_t aclsparseSpMVGetBufferSize(aclsparseHandle_t handle, aclsparse
     }
     const size_t plain = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
     const Restored restored = RestoredLayout(handle, opA, matA, vecX, vecY, computeType, alg);
+    opsparse::RememberSized(matA, restored, c.transpose, RestoredValueType(matA, vecX));
     const size_t own = restored.bytes > plain ? restored.bytes : plain;
     *bufferSize = StagedTranspose(c) ? opsparse::AlignUp(own, 256) + StagingBytes(matA) : own;
     return ACL_SPARSE_STATUS_SUCCESS;
@@ -356,7 +411,12 @@ aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOpe
         return ACL_SPARSE_STATUS_INSUFFICIENT_RESOURCES;
     }
     OpsparseSpmvPlan plan{};
-    const Restored restored = RestoredLayout(handle, opA, matA, vecX, vecY, computeType, alg);
+    Restored restored = RestoredLayout(handle, opA, matA, vecX, vecY, computeType, alg);
+    if (!opsparse::SizedFor(matA, restored, c.transpose, RestoredValueType(matA, vecX))) {
+        // no size query on these arrays asked for the layout's bytes: the buffer may be as small as every query
+        // answers at least, and the ordinary plan fits that
+        restored = Restored{0, 0, false};
+    }
     int rc;
     if (restored.kernel != 0) {
         rc = opsparse::AnalyseRestored(restored.kernel, static_cast<const int32_t *>(matA->rowOffsets),
@@ -415,7 +475,8 @@ aclsparseStatus_t aclsparseSpMV(aclsparseHandle_t handle, aclsparseOperation_t o
     size_t wsBytes = 0;
     const bool bound = externalBuffer != nullptr && matA->spmv.buffer == externalBuffer &&
                        matA->spmv.plan.rows == matA->rows && matA->spmv.plan.nnz == matA->nnz;
-    const bool blockedPlan = bound && matA->spmv.plan.kernel == OPSPARSE_SPMV_BLOCKED_GATHER;
+    const bool blockedPlan = bound && (matA->spmv.plan.kernel == OPSPARSE_SPMV_BLOCKED_GATHER ||
+                                       matA->spmv.plan.kernel == OPSPARSE_SPMV_BLOCKED_LIVE);
     if (blockedPlan && (matA->spmv.plan.transposed != 0) != c.transpose) {
         // Preprocess built the re-stored layout for the other op(A): this call runs without it
         if (matA->nnz > 0 || (c.transpose && c.outType != OPSPARSE_F32)) {

@@ -29,7 +29,13 @@ inline int CheckLaunch()
     return hipGetLastError() == hipSuccess ? OPSPARSE_OK : OPSPARSE_E_LAUNCH;
 }
 
-// BLOCKED_GATHER launch, fp32 values / x / y (spmv_blocked.hip).
+// BLOCKED_GATHER launch (spmv_blocked.hip): values and x of valType, y of outType (fp32 or valType).
+int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valType, int32_t outType,
+                  int32_t computeIsInt);
+
+// BLOCKED_LIVE launch (spmv_blocked_live.hip): values and x of valType (fp32 / fp16 / bf16), y fp32 or of valType.
+namespace live_layout {
 int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valType, int32_t outType);
+}
 
 }  // namespace opsparse

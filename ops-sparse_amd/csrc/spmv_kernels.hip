@@ -1476,17 +1476,8 @@ int RunPlanned(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
                 return OPSPARSE_E_UNSUPPORTED;  // the panel copy holds fp32 values
             }
         case OPSPARSE_SPMV_BLOCKED_GATHER:
-            if constexpr (std::is_same<AccT, double>::value &&
-                          (std::is_same<ValT, float>::value || std::is_same<ValT, Half>::value ||
-                           std::is_same<ValT, Bf16>::value) &&
-                          (std::is_same<OutT, float>::value || std::is_same<OutT, ValT>::value)) {
-                constexpr int32_t kVal = std::is_same<ValT, Half>::value   ? OPSPARSE_F16
-                                         : std::is_same<ValT, Bf16>::value ? OPSPARSE_BF16
-                                                                           : OPSPARSE_F32;
-                return LaunchBlocked(a, plan, kVal, std::is_same<OutT, float>::value ? OPSPARSE_F32 : kVal);
-            } else {
-                return OPSPARSE_E_UNSUPPORTED;  // fp32, fp16 or bf16 values; y fp32 or of the values' type
-            }
+        case OPSPARSE_SPMV_BLOCKED_LIVE:
+            return OPSPARSE_E_INVALID;  // (launched before the types are dispatched: opsparse_spmv_csr_launch_zy)
         default:
             return OPSPARSE_E_INVALID;
     }
@@ -2080,15 +2071,19 @@ int opsparse_spmv_csr_launch_zy(const OpsparseSpmvPlan *plan, int32_t transpose,
     if (plan != nullptr && plan->kernel == OPSPARSE_SPMV_BLOCKED_GATHER && (plan->transposed != 0) != (transpose != 0)) {
         return OPSPARSE_E_INVALID;  // the re-stored layout serves the op(A) it was built for
     }
-    if (transpose && plan != nullptr && plan->kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {
-        if (computeIsInt || (valType != OPSPARSE_F32 && valType != OPSPARSE_F16 && valType != OPSPARSE_BF16) ||
-            (outType != OPSPARSE_F32 && outType != valType)) {
-            return OPSPARSE_E_UNSUPPORTED;
+    if (plan != nullptr && plan->kernel == OPSPARSE_SPMV_BLOCKED_LIVE && nnz > 0) {
+        if (transpose || computeIsInt) {
+            return OPSPARSE_E_INVALID;  // (built for op(A) = A and floating-point sums)
         }
-        SpmvArgs t = a;  // the columns of A are the outputs, its rows the inputs
-        t.rows = cols;
-        t.cols = rows;
-        return LaunchBlocked(t, *plan, valType, outType);
+        return live_layout::LaunchBlocked(a, *plan, valType, outType);
+    }
+    if (plan != nullptr && plan->kernel == OPSPARSE_SPMV_BLOCKED_GATHER && nnz > 0) {
+        SpmvArgs t = a;
+        if (transpose) {  // the columns of A are the outputs, its rows the inputs
+            t.rows = cols;
+            t.cols = rows;
+        }
+        return LaunchBlocked(t, *plan, valType, outType, computeIsInt);
     }
     if (transpose) {
         if (computeIsInt) {

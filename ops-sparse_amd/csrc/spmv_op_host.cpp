@@ -143,13 +143,14 @@ opsparse::RestoredChoice LiveLayout(aclsparseHandle_t handle, aclsparseConstSpMa
         return {0, 0, false};
     }
     return opsparse::PickLiveLayout(handle, static_cast<const int32_t *>(matA->rowOffsets),
-                                    static_cast<const int32_t *>(matA->colInd), matA->rows, matA->cols, matA->nnz);
+                                    static_cast<const int32_t *>(matA->colInd), matA->rows, matA->cols, matA->nnz,
+                                    false, OPSPARSE_F32, /*repeatable=*/true);
 }
 
 opsparse::RestoredChoice RestoredLayout(aclsparseConstSpMatDescr_t matA)
 {
     if (matA->rowOffsetsType != ACL_SPARSE_INDEX_32I || matA->idxBase != ACL_SPARSE_INDEX_BASE_ZERO) {
-        return {0, 0};
+        return {0, 0, false};
     }
     return opsparse::PickRestoredLayout(matA->rows, matA->cols, matA->nnz, false, OPSPARSE_F32);
 }
@@ -198,10 +199,13 @@ aclsparseStatus_t aclsparseSpMVOp_bufferSize(aclsparseHandle_t handle, aclsparse
     *bufferSize = 0;
     if (alg == ACL_SPARSE_SPMVOP_ALG2) {
         const size_t plain = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
-        const size_t restored = RestoredLayout(matA).bytes;
-        *bufferSize = restored > plain ? restored : plain;
+        const opsparse::RestoredChoice restored = RestoredLayout(matA);
+        opsparse::RememberSized(matA, restored, false, OPSPARSE_F32);
+        *bufferSize = restored.bytes > plain ? restored.bytes : plain;
     } else {
-        *bufferSize = LiveLayout(handle, matA).bytes;
+        const opsparse::RestoredChoice live = LiveLayout(handle, matA);
+        opsparse::RememberSized(matA, live, false, OPSPARSE_F32);
+        *bufferSize = live.bytes;
     }
     return ACL_SPARSE_STATUS_SUCCESS;
 }
@@ -269,7 +273,11 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
         d->userBuffer = buffer;
         // The nnz-balanced split of ALG2: analyse the rows into the caller's buffer.
         if ((Plain(d) || d->offsets32 != nullptr) && d->rows > 0 && d->nnz > 0 && d->rowOffsets != nullptr) {
-            const opsparse::RestoredChoice restored = RestoredLayout(matA);
+            // (a re-stored layout only into a buffer that a size query on these arrays sized for it)
+            opsparse::RestoredChoice restored = RestoredLayout(matA);
+            if (!opsparse::SizedFor(matA, restored, false, OPSPARSE_F32)) {
+                restored = opsparse::RestoredChoice{0, 0, false};
+            }
             const int rc =
                 restored.kernel != 0 && d->colInd != nullptr && d->values != nullptr
                     ? opsparse::AnalyseRestored(restored.kernel, static_cast<const int32_t *>(d->rowOffsets),
@@ -290,7 +298,7 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
     if (d->alg != ACL_SPARSE_SPMVOP_ALG2 && buffer != nullptr && Plain(d) && d->rows > 0 && d->nnz > 0) {
         // the buffer aclsparseSpMVOp_bufferSize asked for (it asks the same question of the same arrays)
         const opsparse::RestoredChoice live = LiveLayout(handle, matA);
-        if (live.kernel != 0) {
+        if (live.kernel != 0 && opsparse::SizedFor(matA, live, false, OPSPARSE_F32)) {
             const int rc = opsparse::AnalyseRestored(live.kernel, static_cast<const int32_t *>(d->rowOffsets),
                                                      static_cast<const int32_t *>(d->colInd), d->values, OPSPARSE_F32,
                                                      d->rows, d->cols, d->nnz, false, true, buffer, live.bytes, &d->plan,

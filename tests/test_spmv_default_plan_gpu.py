@@ -1,5 +1,8 @@
 """The plan aclsparseSpMVPreprocess picks for ACL_SPARSE_SPMV_ALG_DEFAULT on a large matrix with scattered
-columns: the blocked-gather layout with live values.  The contract under test: a caller that follows the
+columns: a blocked-gather layout with live values — the one whose row blocks add with atomics (plan kernel
+BLOCKED_LIVE) for op(A) = A and floating-point values, the ordered one (BLOCKED_GATHER, the same bits from every
+call) with OPS_SPARSE_SPMV_REPEATABLE in the environment, for op(A) = A^T, for int32 values and under
+aclsparseSpMVOp.  The contract under test: a caller that follows the
 reference's call pattern (GetBufferSize, Preprocess, SpMV with the default algorithm) may change the values in
 place, or hand the descriptor a new values array, between calls, and always gets the product of the values as
 they are at the call.  An explicit ACL_SPARSE_SPMV_CSR_ALG2 request holds a copy of the values: there
@@ -23,6 +26,23 @@ def _layout_for_small_matrices(monkeypatch):
     monkeypatch.setenv("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ", "0")
 
 
+def _default_bytes(osa, rows, cols, nnz, repeatable):
+    """What GetBufferSize answers for the default algorithm, op(A) = A, fp values, scattered columns."""
+    L = osa.lib()
+    if repeatable:
+        return L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    return L.opsparse_spmv_csr_live_workspace_bytes(rows, cols, nnz)
+
+
+@pytest.fixture(params=[False, True], ids=["atomics", "repeatable"])
+def repeatable(request, monkeypatch):
+    if request.param:
+        monkeypatch.setenv("OPS_SPARSE_SPMV_REPEATABLE", "1")
+    else:
+        monkeypatch.delenv("OPS_SPARSE_SPMV_REPEATABLE", raising=False)
+    return request.param
+
+
 def _scattered(rows, cols, seed, per_row=16):
     rng = np.random.default_rng(seed)
     lengths = rng.integers(0, per_row, rows)
@@ -33,13 +53,13 @@ def _scattered(rows, cols, seed, per_row=16):
     return rowptr, colind, val, rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
 
 
-def test_default_plan_is_the_live_blocked_layout_and_follows_the_values(osa, gpu_ctx):
+def test_default_plan_is_the_live_blocked_layout_and_follows_the_values(osa, gpu_ctx, repeatable):
     dev, stream, handle = gpu_ctx
     L = osa.lib()
     rows, cols = 320_000, 1_500_000
     rowptr, colind, val, x, y0 = _scattered(rows, cols, 5)
     nnz = colind.size
-    want = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    want = _default_bytes(osa, rows, cols, nnz, repeatable)
     assert want > L.opsparse_spmv_csr_workspace_bytes(rows, nnz) > 0
     d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
     A, X = osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3])
@@ -65,7 +85,8 @@ def test_default_plan_is_the_live_blocked_layout_and_follows_the_values(osa, gpu
     assert L.aclsparseSpMatSetValues(A.d, ctypes.c_void_p(d_val3.data_ptr())) == 0
     check(val3, -1.0, 0.0)
     # the layout only: a launch accepts a buffer cut down to the resident size
-    resident = L.opsparse_spmv_csr_blocked_resident_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    resident = (L.opsparse_spmv_csr_blocked_resident_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+                if repeatable else L.opsparse_spmv_csr_live_resident_bytes(rows, cols, nnz))
     assert 0 < resident < want
 
 
@@ -141,13 +162,12 @@ def _with_long_rows(rows, cols, seed):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("short_positions,narrow_y", [(True, False), (False, False), (True, True)])
-def test_default_plan_with_half_precision_values(osa, gpu_ctx, dtype, short_positions, narrow_y, monkeypatch):
+@pytest.mark.parametrize("narrow_y", [False, True])
+def test_default_plan_with_half_precision_values(osa, gpu_ctx, dtype, narrow_y, repeatable):
     """fp16 / bf16 values and x with an fp32 y get the same default plan: the live layout reads the caller's 2-byte
-    values at every call (the short entries into the LDS window of their row block, the long rows' straight into
-    the sums of their panel) and widens x as it loads a panel's slice.  Values changed in place are followed."""
-    if not short_positions:
-        monkeypatch.setenv("OPS_SPARSE_BLOCKED_NO_SHORT_POSITIONS", "1")
+    values at every call (a row block's linearly, beside the gathered x in the block's LDS window, the long rows'
+    straight into the sums of their panel) and widens x as it loads a panel's slice.  Values changed in place are
+    followed."""
     dev, stream, handle = gpu_ctx
     L = osa.lib()
     rows, cols = 300_000, 1_400_000
@@ -155,7 +175,10 @@ def test_default_plan_with_half_precision_values(osa, gpu_ctx, dtype, short_posi
     rnd = lambda a: torch.from_numpy(a).to(dtype).float().numpy()
     val, x = rnd(val), rnd(x)
     nnz = colind.size
-    want = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    want = (L.opsparse_spmv_csr_blocked_workspace_bytes(
+                rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES |
+                (osa.OPSPARSE_BLOCKED_VALUES_F16 if dtype == torch.float16 else osa.OPSPARSE_BLOCKED_VALUES_BF16))
+            if repeatable else L.opsparse_spmv_csr_live_workspace_bytes(rows, cols, nnz))
     d_rp, d_ci = to_dev(rowptr, dev), to_dev(colind, dev)
     vbuf = torch.zeros(nnz + 1, dtype=dtype, device=dev)      # values at an address that is only 2-byte aligned
     d_val = vbuf[1:]
@@ -186,7 +209,7 @@ def test_default_plan_with_half_precision_values(osa, gpu_ctx, dtype, short_posi
     check(val2, 1.5, -0.5)
 
 
-def test_default_plan_sums_long_rows_from_the_callers_arrays(osa, gpu_ctx):
+def test_default_plan_sums_long_rows_from_the_callers_arrays(osa, gpu_ctx, repeatable):
     """Rows of 64 entries per column panel and more (4096 at least) with ascending columns are kept out of the
     re-stored layout: the workgroup that has a panel's x in LDS sums their entries of that panel straight from
     colInd / csrValues.  The analysis must find exactly those rows; the product must follow values changed in
@@ -198,14 +221,16 @@ def test_default_plan_sums_long_rows_from_the_callers_arrays(osa, gpu_ctx):
     nnz = colind.size
     d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
     # the analysis through the raw layer: which rows it took
-    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    need = _default_bytes(osa, rows, cols, nnz, repeatable)
     ws = torch.empty(need, dtype=torch.uint8, device=dev)
     plan = osa.OpsparseSpmvPlan()
     pv = lambda t: ctypes.c_void_p(t.data_ptr())
-    assert L.opsparse_spmv_csr_blocked_analyse(pv(d[0]), pv(d[1]), pv(d[2]), rows, cols, nnz,
-                                               osa.OPSPARSE_BLOCKED_LIVE_VALUES, pv(ws), need, ctypes.byref(plan),
-                                               ctypes.c_void_p(stream.cuda_stream)) == 0
-    assert plan.liveValues == 2 and plan.numLongRows == 6     # 9000, 4096, 40 000, 20 000, 120 000, 5000; short positions
+    analyse = L.opsparse_spmv_csr_blocked_analyse if repeatable else L.opsparse_spmv_csr_live_analyse
+    assert analyse(pv(d[0]), pv(d[1]), pv(d[2]), rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES, pv(ws), need,
+                   ctypes.byref(plan), ctypes.c_void_p(stream.cuda_stream)) == 0
+    assert plan.kernel == (osa.OPSPARSE_SPMV_BLOCKED_GATHER if repeatable else osa.OPSPARSE_SPMV_BLOCKED_LIVE)
+    assert plan.liveValues == (1 if repeatable else 2)       # (atomics: 16-bit positions, every block is short)
+    assert plan.numLongRows == 6                              # 9000, 4096, 40 000, 20 000, 120 000, 5000
     del ws
     A, X = osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3])
     d_y = to_dev(y0, dev)
@@ -230,15 +255,17 @@ def test_default_plan_sums_long_rows_from_the_callers_arrays(osa, gpu_ctx):
 
 
 @pytest.mark.parametrize("live", [True, False])
-def test_many_long_rows_in_one_row_block_are_summed_by_their_own_kernel(osa, gpu_ctx, live):
+def test_many_long_rows_in_one_row_block_are_summed_by_their_own_kernel(osa, gpu_ctx, live, monkeypatch):
     """A row block's workgroup adds up the partial sums of at most 64 long rows; a block with more of them (here
     200 neighbouring rows of 4200 .. 5000 entries among short ones, and in a second matrix nothing but long rows)
-    marks them and leaves them to a kernel with a wavefront a row.  Default plan and ALG2; beta != 0 with y
-    read and written in place."""
+    leaves them to a kernel with a wavefront a row.  That is the layout with frozen values (ALG2); with live values
+    a long row ends its row block (the block's other entries are then one piece of the caller's arrays), so no block
+    holds more than one.  beta != 0 with y read and written in place."""
     dev, stream, handle = gpu_ctx
     L = osa.lib()
     pv = lambda t: ctypes.c_void_p(t.data_ptr())
     flags = osa.OPSPARSE_BLOCKED_LIVE_VALUES if live else 0
+    monkeypatch.setenv("OPS_SPARSE_SPMV_REPEATABLE", "1")   # the default algorithm on the ordered layout too
 
     def run(rows, cols, lengths, want_long, seed):
         rng = np.random.default_rng(seed)
@@ -256,7 +283,7 @@ def test_many_long_rows_in_one_row_block_are_summed_by_their_own_kernel(osa, gpu
         plan = osa.OpsparseSpmvPlan()
         assert L.opsparse_spmv_csr_blocked_analyse(pv(d[0]), pv(d[1]), pv(d[2]), rows, cols, nnz, flags, pv(ws), need,
                                                    ctypes.byref(plan), ctypes.c_void_p(stream.cuda_stream)) == 0
-        assert plan.numLongRows == want_long and plan.numDeferredLongRows == want_long
+        assert plan.numLongRows == want_long and plan.numDeferredLongRows == (0 if live else want_long)
         del ws
         d_y = to_dev(y0, dev)
         op = osa.SpmvOp(handle, osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3]), osa.DnVec(d_y),
@@ -276,40 +303,44 @@ def test_many_long_rows_in_one_row_block_are_summed_by_their_own_kernel(osa, gpu
     run(700, 1_300_000, np.full(700, 4500), 700, 43)         # long rows only: no entry in the row-block order
 
 
-def test_default_plan_keeps_32_bit_positions_for_a_block_of_70000_entries(osa, gpu_ctx):
-    """The positions of the entries in their row block are kept in 16 bits where every block is shorter than 65535
-    positions.  A row of 70 000 entries whose columns do not ascend cannot go the long rows' way, makes a block of
-    several windows, and the layout keeps its 32-bit positions (plan.liveValues == 1); same product either way."""
+def test_a_row_too_long_for_a_row_block_keeps_the_ordinary_plan(osa, gpu_ctx, monkeypatch):
+    """The place of an entry in its row block is kept in 16 bits.  A row of 70 000 entries whose columns do not
+    ascend cannot go the long rows' way and does not fit a block: the analysis says so (unsupported), and
+    Preprocess leaves the ordinary plan in the buffer instead; same product.  A row of 30 000 such entries fits
+    (a block worked in several windows)."""
     dev, stream, handle = gpu_ctx
     L = osa.lib()
+    monkeypatch.setenv("OPS_SPARSE_SPMV_REPEATABLE", "1")
     rows, cols = 300_000, 1_400_000
-    rng = np.random.default_rng(31)
-    lengths = rng.integers(0, 20, rows)
-    lengths[123_456] = 70_000
-    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
-    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)      # unsorted everywhere
-    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
-    x, y0 = rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
-    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
-    nnz = colind.size
-    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
-    ws = torch.empty(need, dtype=torch.uint8, device=dev)
-    plan = osa.OpsparseSpmvPlan()
-    pv = lambda t: ctypes.c_void_p(t.data_ptr())
-    assert L.opsparse_spmv_csr_blocked_analyse(pv(d[0]), pv(d[1]), pv(d[2]), rows, cols, nnz,
-                                               osa.OPSPARSE_BLOCKED_LIVE_VALUES, pv(ws), need, ctypes.byref(plan),
-                                               ctypes.c_void_p(stream.cuda_stream)) == 0
-    assert plan.liveValues == 1 and plan.numLongRows == 0
-    del ws
-    d_y = to_dev(y0, dev)
-    op = osa.SpmvOp(handle, osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3]), osa.DnVec(d_y))
-    for values, alpha, beta in ((val, 1.0, 0.0), ((val * np.float32(-2.0)).astype(np.float32), 0.5, 1.5)):
-        d[2].copy_(torch.from_numpy(values))
-        d_y.copy_(torch.from_numpy(y0))
-        op(alpha, beta)
-        stream.synchronize()
-        gold = oracle.spmv_f64(rows, cols, rowptr, colind, values, x, y0, alpha, beta)
-        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+    for longest, want_rc in ((70_000, osa.OPSPARSE_E_UNSUPPORTED), (30_000, 0)):
+        rng = np.random.default_rng(31)
+        lengths = rng.integers(0, 20, rows)
+        lengths[123_456] = longest
+        rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+        colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)      # unsorted everywhere
+        val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+        x, y0 = rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+        d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+        nnz = colind.size
+        need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+        ws = torch.empty(need, dtype=torch.uint8, device=dev)
+        plan = osa.OpsparseSpmvPlan()
+        pv = lambda t: ctypes.c_void_p(t.data_ptr())
+        assert L.opsparse_spmv_csr_blocked_analyse(pv(d[0]), pv(d[1]), pv(d[2]), rows, cols, nnz,
+                                                   osa.OPSPARSE_BLOCKED_LIVE_VALUES, pv(ws), need, ctypes.byref(plan),
+                                                   ctypes.c_void_p(stream.cuda_stream)) == want_rc
+        if want_rc == 0:
+            assert plan.liveValues == 1 and plan.numLongRows == 0
+        del ws
+        d_y = to_dev(y0, dev)
+        op = osa.SpmvOp(handle, osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3]), osa.DnVec(d_y))
+        for values, alpha, beta in ((val, 1.0, 0.0), ((val * np.float32(-2.0)).astype(np.float32), 0.5, 1.5)):
+            d[2].copy_(torch.from_numpy(values))
+            d_y.copy_(torch.from_numpy(y0))
+            op(alpha, beta)
+            stream.synchronize()
+            gold = oracle.spmv_f64(rows, cols, rowptr, colind, values, x, y0, alpha, beta)
+            assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
 
 
 def test_default_plan_leaves_small_matrices_to_the_merge_path(osa, gpu_ctx, monkeypatch):
@@ -323,7 +354,7 @@ def test_default_plan_leaves_small_matrices_to_the_merge_path(osa, gpu_ctx, monk
     assert 2_000_000 < nnz < 7_000_000
     d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
     A, X, Y = osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3]), osa.DnVec(to_dev(y0, dev))
-    layout = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    layout = L.opsparse_spmv_csr_live_workspace_bytes(rows, cols, nnz)
     assert layout > 0
     monkeypatch.delenv("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ")
     assert osa.SpmvOp(handle, A, X, Y).buffer.numel() == L.opsparse_spmv_csr_workspace_bytes(rows, nnz)
@@ -344,7 +375,7 @@ def test_default_plan_of_a_banded_matrix_stays_row_wise(osa, gpu_ctx, workloads)
     L = osa.lib()
     A = workloads.laplacian_2d(1200, dev)                   # 1.44 M columns, 7.2 M entries: the layout would apply
     rows, nnz = A["rows"], int(A["colind"].numel())
-    assert L.opsparse_spmv_csr_blocked_workspace_bytes(rows, rows, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES) > 0
+    assert L.opsparse_spmv_csr_live_workspace_bytes(rows, rows, nnz) > 0
     x = workloads.uniform(3, rows, -1.0, 1.0, dev)
     y = torch.zeros(rows, device=dev)
     op = osa.SpmvOp(handle, osa.Csr(rows, rows, A["rowptr"], A["colind"], A["values"]), osa.DnVec(x), osa.DnVec(y))
@@ -377,7 +408,7 @@ def test_a_band_with_some_random_columns_gets_the_layout_only_where_it_pays(osa,
     nnz = colind.size
     A, X = osa.Csr(rows, rows, d[0], d[1], d[2]), osa.DnVec(d[3])
     gold = oracle.spmv_f64(rows, rows, rowptr, colind, val, x, y0, 1.0, 0.5)
-    live_bytes = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, rows, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    live_bytes = L.opsparse_spmv_csr_live_workspace_bytes(rows, rows, nnz)
     assert live_bytes > 0
     for alg, want_layout in ((osa.ACL_SPARSE_SPMV_ALG_DEFAULT, layout_default), (osa.ACL_SPARSE_SPMV_CSR_ALG2, layout_alg2)):
         d_y = to_dev(y0, dev)
@@ -470,3 +501,62 @@ def test_alg2_layout_streams_long_rows_panel_by_panel(osa, gpu_ctx):
     val = rng.uniform(-1, 1, colind.size).astype(np.float32)
     run(rows, cols, rowptr, colind, val, rng.uniform(-1, 1, cols).astype(np.float32),
         rng.uniform(-1, 1, rows).astype(np.float32), want_long=3460)
+
+
+def test_a_layout_is_only_built_into_a_buffer_that_a_size_query_sized(osa, gpu_ctx):
+    """A caller may size the buffer from any earlier answer it trusts (the reference's SpMVOp answers 0 for ALG1,
+    spmv_op_host.cpp:152-160) or skip the query: Preprocess / createDescr then get a buffer with room for the
+    ordinary plan only.  The library builds a re-stored layout only where a size query ON THESE ARRAYS answered
+    that layout's bytes: without one, the ordinary plan goes into the buffer and nothing is written behind it."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = 320_000, 1_500_000
+    rowptr, colind, val, x, y0 = _scattered(rows, cols, 8)
+    nnz = colind.size
+    plain = L.opsparse_spmv_csr_workspace_bytes(rows, nnz)
+    assert 0 < plain < L.opsparse_spmv_csr_live_workspace_bytes(rows, cols, nnz)
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.0, 0.5)
+    guard = 1 << 16
+
+    def fresh():
+        d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]   # new arrays: no query has seen them
+        buf = torch.full((plain + guard,), 0xA5, dtype=torch.uint8, device=dev)
+        return d, osa.Csr(rows, cols, d[0], d[1], d[2]), buf
+
+    pv = lambda t: ctypes.c_void_p(t.data_ptr())
+    for alg in (osa.ACL_SPARSE_SPMV_ALG_DEFAULT, osa.ACL_SPARSE_SPMV_CSR_ALG2):
+        d, A, buf = fresh()
+        X, d_y = osa.DnVec(d[3]), to_dev(y0, dev)
+        Y = osa.DnVec(d_y)
+        assert L.aclsparseSpMVPreprocess(handle.h, 0, None, A.d, X.d, None, Y.d, osa.ACL_FLOAT, alg, pv(buf)) == 0
+        stream.synchronize()
+        assert bool((buf[plain:] == 0xA5).all())
+        one, half = ctypes.c_float(1.0), ctypes.c_float(0.5)
+        assert L.aclsparseSpMV(handle.h, 0, ctypes.byref(one), A.d, X.d, ctypes.byref(half), Y.d, osa.ACL_FLOAT, alg,
+                               pv(buf)) == 0
+        stream.synchronize()
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+        # a query for ANOTHER algorithm's layout does not count either: the default query, then an ALG2 Preprocess
+        if alg == osa.ACL_SPARSE_SPMV_CSR_ALG2:
+            n = ctypes.c_size_t(0)
+            assert L.aclsparseSpMVGetBufferSize(handle.h, 0, None, A.d, X.d, None, Y.d, osa.ACL_FLOAT,
+                                                osa.ACL_SPARSE_SPMV_ALG_DEFAULT, ctypes.byref(n)) == 0
+            assert n.value == L.opsparse_spmv_csr_live_workspace_bytes(rows, cols, nnz)
+            assert L.aclsparseSpMVPreprocess(handle.h, 0, None, A.d, X.d, None, Y.d, osa.ACL_FLOAT, alg, pv(buf)) == 0
+            stream.synchronize()
+            assert bool((buf[plain:] == 0xA5).all())
+    for alg in (osa.ACL_SPARSE_SPMVOP_ALG1, osa.ACL_SPARSE_SPMVOP_ALG2):
+        d, A, buf = fresh()
+        X, d_y = osa.DnVec(d[3]), to_dev(y0, dev)
+        Y = osa.DnVec(d_y)
+        descr, plan = ctypes.c_void_p(), ctypes.c_void_p()
+        assert L.aclsparseSpMVOp_createDescr(handle.h, ctypes.byref(descr), 0, A.d, X.d, Y.d, Y.d, osa.ACL_FLOAT, alg,
+                                             pv(buf)) == 0
+        assert L.aclsparseSpMVOp_createPlan(handle.h, descr, ctypes.byref(plan), None, 0) == 0
+        one, half = ctypes.c_float(1.0), ctypes.c_float(0.5)
+        assert L.aclsparseSpMVOp(handle.h, plan, ctypes.byref(one), ctypes.byref(half), X.d, Y.d, Y.d) == 0
+        stream.synchronize()
+        assert bool((buf[plain:] == 0xA5).all())
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+        L.aclsparseSpMVOp_destroyPlan(plan)
+        L.aclsparseSpMVOp_destroyDescr(descr)

@@ -240,7 +240,7 @@ def test_column_panels_through_spmvop_alg2(osa, gpu_ctx, monkeypatch):
 
 @pytest.mark.parametrize("rows,cols,applies", [(60_000, 3_000_000, True), (60_000, 1_048_577, True),
                                                (60_000, 9_000_000, True), (60_000, 1_000_000, True), (60_000, 262_144, False),
-                                               (20_000, 17_000_000, False),     # 519 panels: chunks of < 32 entries
+                                               (20_000, 17_000_000, True),      # 519 panels: chunks of 24 entries
                                                (300_000, 2_000_000, True)])
 def test_blocked_gather_csr_alg2(osa, gpu_ctx, rows, cols, applies):
     """ACL_SPARSE_SPMV_CSR_ALG2 on a matrix whose x is wider than an L2: Preprocess re-stores the entries by
@@ -378,7 +378,7 @@ def test_blocked_gather_transposed(osa, gpu_ctx, rows, cols):
 @pytest.mark.parametrize("transpose,narrow_y", [(False, False), (True, False), (False, True), (True, True)])
 def test_blocked_gather_csr_alg2_half_precision_values(osa, gpu_ctx, dtype, transpose, narrow_y):
     """fp16 / bf16 values and x with an fp32 y under ACL_SPARSE_SPMV_CSR_ALG2: the same re-stored layout (it keeps
-    the values as fp32, which holds them exactly, and widens x as it loads a panel's slice), long rows included;
+    the values in their own type and widens x as it loads a panel's slice), long rows included;
     against the fp64 oracle on the rounded inputs at the fp32 bar.  A launch with values of another type than the
     layout was built from is refused by the raw layer."""
     dev, stream, handle = gpu_ctx
@@ -397,7 +397,9 @@ def test_blocked_gather_csr_alg2_half_precision_values(osa, gpu_ctx, dtype, tran
     rnd = lambda a: torch.from_numpy(a).to(dtype).float().numpy()
     val, x = rnd(val), rnd(x)
     L = osa.lib()
-    need = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, colind.size, 1 if transpose else 0)
+    need = L.opsparse_spmv_csr_blocked_workspace_bytes(
+        rows, cols, colind.size, (osa.OPSPARSE_BLOCKED_TRANSPOSE if transpose else 0) |
+        (osa.OPSPARSE_BLOCKED_VALUES_F16 if dtype == torch.float16 else osa.OPSPARSE_BLOCKED_VALUES_BF16))
     assert need > 0
     d_rp, d_ci = to_dev(rowptr, dev), to_dev(colind, dev)
     if narrow_y:                                             # y of the values' type: the fp64 sum rounded once
@@ -615,6 +617,10 @@ def test_blocked_gather_rejects_column_out_of_range(osa, gpu_ctx):
     assert rc == osa.OPSPARSE_E_INVALID
     d_x, d_y = to_dev(x, dev), to_dev(y0, dev)
     A, X, Y = osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d_x), osa.DnVec(d_y)
+    asked = ctypes.c_size_t(0)
+    assert L.aclsparseSpMVGetBufferSize(handle.h, 0, None, A.d, X.d, None, Y.d, osa.ACL_FLOAT,
+                                        osa.ACL_SPARSE_SPMV_CSR_ALG2, ctypes.byref(asked)) == 0
+    assert asked.value == need
     st = L.aclsparseSpMVPreprocess(handle.h, 0, None, A.d, X.d, None, Y.d, osa.ACL_FLOAT,
                                    osa.ACL_SPARSE_SPMV_CSR_ALG2, p(ws))
     assert st == osa.ACL_SPARSE_STATUS_INVALID_VALUE
