@@ -140,7 +140,7 @@ def test_same_bits_from_every_run_and_every_plan(osa, gpu_ctx, case, monkeypatch
     assert torch.equal(with_beta[1], with_beta[0]) and torch.equal(with_beta[2], with_beta[0])
     if not transposed:
         # the order matters on this data: the rows stored backwards give other bits in many rows, within the bound
-        ci_b, va_b = _rows_stored_backwards(h_ci, h_va)
+        ci_b, va_b = _rows_stored_backwards(h_rp, h_ci, h_va)
         other = product(ci_b, va_b, 1.0, 0.0, 2)
         assert torch.equal(other[0], other[1])
         differing = int((other[0] != first[0]).sum())
