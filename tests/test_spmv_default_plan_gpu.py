@@ -560,3 +560,131 @@ def test_a_layout_is_only_built_into_a_buffer_that_a_size_query_sized(osa, gpu_c
         assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
         L.aclsparseSpMVOp_destroyPlan(plan)
         L.aclsparseSpMVOp_destroyDescr(descr)
+
+
+def _value_flag(osa, dtype):
+    return {torch.float32: 0, torch.float16: osa.OPSPARSE_BLOCKED_VALUES_F16,
+            torch.bfloat16: osa.OPSPARSE_BLOCKED_VALUES_BF16, torch.int32: osa.OPSPARSE_BLOCKED_VALUES_I32}[dtype]
+
+
+@pytest.mark.parametrize("dtype,narrow_y", [(torch.float32, False), (torch.float16, False), (torch.float16, True),
+                                            (torch.bfloat16, True)])
+def test_default_plan_for_the_transposed_product(osa, gpu_ctx, dtype, narrow_y):
+    """y = alpha * A^T x + beta * y with the default algorithm on a matrix whose updates of y are scattered:
+    Preprocess transposes A into the buffer, keeps for every entry of the copy where its value sits in csrValues,
+    and every call refreshes the copy's values from the caller's array before it runs the ordered kernels (no atomics
+    on y).  Values changed in place and a replaced values array are followed; the transposed plan does not serve
+    op(A) = A (that call runs without it, same buffer)."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = 1_400_000, 300_000                          # A^T: 300 000 rows, x of 1.4 M elements
+    rng = np.random.default_rng(17)
+    lengths = rng.integers(0, 5, rows)
+    lengths[[11, rows // 2]] = [30_000, 9_000]               # long rows of A: columns of A^T that hit many rows
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)
+    colind[:6000] = 77                                       # a column of A with 6000 entries: a long row of A^T
+    nnz = colind.size
+    rnd = lambda a: torch.from_numpy(a).to(dtype).float().numpy()
+    val, x = rnd(rng.uniform(-1, 1, nnz).astype(np.float32)), rnd(rng.uniform(-1, 1, rows).astype(np.float32))
+    y0 = rng.uniform(-1, 1, cols).astype(np.float32)
+    if narrow_y:
+        y0 = rnd(y0)
+    want = L.opsparse_spmv_csr_blocked_workspace_bytes(
+        rows, cols, nnz, osa.OPSPARSE_BLOCKED_TRANSPOSE | osa.OPSPARSE_BLOCKED_LIVE_VALUES | _value_flag(osa, dtype))
+    assert want > 0
+    d_rp, d_ci = to_dev(rowptr, dev), to_dev(colind, dev)
+    d_val, d_x = to_dev(val, dev, dtype), to_dev(x, dev, dtype)
+    d_y = to_dev(y0, dev, dtype if narrow_y else None)
+    A = osa.Csr(rows, cols, d_rp, d_ci, d_val)
+    op = osa.SpmvOp(handle, A, osa.DnVec(d_x), osa.DnVec(d_y), op=osa.ACL_SPARSE_OP_TRANSPOSE)
+    staging = 0 if not narrow_y else cols * 4                # (the fp32 staging vector of the atomics path, unused here)
+    assert want <= op.buffer.numel() <= want + 256 + staging
+    half_ulp = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}.get(dtype)
+
+    def check(values, alpha, beta):
+        d_y.copy_(torch.from_numpy(y0).to(d_y.dtype))
+        op(alpha, beta)
+        stream.synchronize()
+        gold = oracle.spmv_trans_f64(rows, cols, rowptr, colind, values, x, y0, alpha, beta)
+        got = d_y.float().cpu().numpy()
+        if narrow_y:
+            assert np.all(np.abs(got - gold) <= 1.001 * half_ulp * np.maximum(np.abs(gold), 2.0 ** -14))
+        else:
+            assert oracle.max_rel_err(got, gold) <= 1e-5     # fp64 sums rounded once: the bar of op(A) = A
+
+    check(val, 1.0, 0.0)
+    first = d_y.clone()
+    check(val, 1.0, 0.0)
+    assert torch.equal(first, d_y)
+    val2 = rnd((val * np.float32(-0.5) + np.float32(0.25)).astype(np.float32))
+    d_val.copy_(torch.from_numpy(val2).to(dtype))
+    check(val2, 1.5, -0.5)
+    val3 = rnd(np.random.default_rng(3).uniform(-3, 3, nnz).astype(np.float32))
+    d_val3 = to_dev(val3, dev, dtype)
+    assert L.aclsparseSpMatSetValues(A.d, ctypes.c_void_p(d_val3.data_ptr())) == 0
+    check(val3, -1.0, 0.0)
+    # the other op(A) on the same descriptor and buffer
+    d_xn, d_yn = to_dev(rnd(y0), dev, dtype), torch.zeros(rows, dtype=torch.float32, device=dev)
+    opn = osa.SpmvOp(handle, A, osa.DnVec(d_xn), osa.DnVec(d_yn), preprocess=False)
+    opn.buffer = op.buffer
+    opn(1.0, 0.0)
+    stream.synchronize()
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val3, rnd(y0), None, 1.0, 0.0)
+    assert oracle.max_rel_err(d_yn.cpu().numpy(), gold) <= 1e-5
+
+
+@pytest.mark.parametrize("transpose", [False, True])
+@pytest.mark.parametrize("int_compute", [True, False])
+def test_default_plan_with_int32_values(osa, gpu_ctx, transpose, int_compute):
+    """int32 values and x.  Under the integer compute type y is int32 and the sums wrap around (bit for bit the
+    oracle's, whatever the order); under ACL_FLOAT y is fp32 and the sums are fp64 of the exactly converted operands.
+    Both get the ordered layout with live values."""
+    import scipy.sparse as sp
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = (1_400_000, 300_000) if transpose else (300_000, 1_400_000)
+    rng = np.random.default_rng(23 + transpose)
+    lengths = rng.integers(0, 5 if transpose else 20, rows)
+    lengths[[5, rows // 3]] = [40_000, 5_000]
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)
+    for r in (5, rows // 3):
+        colind[rowptr[r]:rowptr[r + 1]].sort()
+    nnz = colind.size
+    big = 50_000 if int_compute else 2_000                   # products wrap in the integer sums
+    val = rng.integers(-big, big, nnz).astype(np.int32)
+    n_x, n_y = (rows, cols) if transpose else (cols, rows)
+    x = rng.integers(-big, big, n_x).astype(np.int32)
+    y0 = rng.integers(-1000, 1000, n_y).astype(np.int32) if int_compute else rng.uniform(-1, 1, n_y).astype(np.float32)
+    want = L.opsparse_spmv_csr_blocked_workspace_bytes(
+        rows, cols, nnz, (osa.OPSPARSE_BLOCKED_TRANSPOSE if transpose else 0) | osa.OPSPARSE_BLOCKED_LIVE_VALUES |
+        osa.OPSPARSE_BLOCKED_VALUES_I32)
+    assert want > 0
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    d_y = to_dev(y0, dev)
+    A = osa.Csr(rows, cols, d[0], d[1], d[2])
+    op = osa.SpmvOp(handle, A, osa.DnVec(d[3]), osa.DnVec(d_y),
+                    op=osa.ACL_SPARSE_OP_TRANSPOSE if transpose else osa.ACL_SPARSE_OP_NON_TRANSPOSE,
+                    compute_type=osa.ACL_INT32 if int_compute else osa.ACL_FLOAT)
+    assert op.buffer.numel() == want
+
+    def check(values, alpha, beta):
+        d_y.copy_(torch.from_numpy(y0))
+        op(alpha, beta)
+        stream.synchronize()
+        if transpose:                                        # the oracle's op(A) = A on the transposed arrays
+            t = sp.csr_matrix((values, colind, rowptr), shape=(rows, cols)).tocsc()
+            rp, ci, va = t.indptr.astype(np.int32), t.indices.astype(np.int32), t.data.astype(np.int32)
+        else:
+            rp, ci, va = rowptr, colind, values
+        if int_compute:
+            assert np.array_equal(d_y.cpu().numpy(), oracle.spmv_i32(n_y, rp, ci, va, x, y0, alpha, beta))
+        else:
+            gold = oracle.spmv_f64(n_y, n_x, rp, ci, va.astype(np.float32), x.astype(np.float32), y0, alpha, beta)
+            assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+    check(val, *((3, -2) if int_compute else (0.5, 1.0)))
+    val2 = rng.integers(-big, big, nnz).astype(np.int32)
+    d[2].copy_(torch.from_numpy(val2))                       # in place: followed
+    check(val2, *((-1, 0) if int_compute else (1.0, 0.0)))
