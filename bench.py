@@ -107,8 +107,9 @@ def load_traffic(name):
     return int(entry["fetch_kib"] * 1024 * table["fetch_scale"] + entry["write_kib"] * 1024 * table["write_scale"])
 
 
-def cpu_baseline_spmv(cfg, y_gpu, base=None, budget_s=15.0):
-    """The reference's SpmvCpu loop (oracle.spmv_f32), one thread, on the same matrix; the GPU result of one
+def cpu_baseline_spmv(cfg, y_gpu, base=None, budget_s=15.0, transpose=False):
+    """The reference's SpmvCpu loop (oracle.spmv_f32; op(A) = A^T: its SpmvTransCpu, oracle.spmv_trans_f32,
+    reference test/spmv/arch22/spmv_test.cpp:177-197), one thread, on the same matrix; the GPU result of one
     launch (y_gpu) is checked against the fp64-accumulated oracle on the way.  `base` is the result of an earlier
     call on the same matrix: the CPU timing is taken from it and only the check is repeated."""
     import oracle
@@ -116,33 +117,42 @@ def cpu_baseline_spmv(cfg, y_gpu, base=None, budget_s=15.0):
     rowptr, colind = A["rowptr"].cpu().numpy(), A["colind"].cpu().numpy()
     val = A["values"].cpu().float().numpy()
     x, y0 = cfg["x"].cpu().float().numpy(), cfg["y0"].cpu().float().numpy()
-    rows, nnz = A["rows"], int(colind.size)
-    gold = oracle.spmv_f64(rows, A["cols"], rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])
+    rows, cols, nnz = A["rows"], A["cols"], int(colind.size)
+    if transpose:
+        gold = oracle.spmv_trans_f64(rows, cols, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])
+        cpu = lambda: oracle.spmv_trans_f32(rows, cols, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])
+        name = "SpmvTransCpu"
+    else:
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])
+        cpu = lambda: oracle.spmv_f32(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])
+        name = "SpmvCpu"
     err = oracle.max_rel_err(y_gpu.cpu().numpy(), gold)
     if err > 1e-5:
         sys.exit("bench.py: the GPU result differs from the fp64 oracle (max relative error %.3g > 1e-5)" % err)
     if base is not None:
         return dict(base, gpu_vs_fp64_oracle_max_rel_err=err)
-    oracle.spmv_f32(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])  # warm
+    cpu()  # warm
     reps, t0 = 0, time.perf_counter()
     while reps < 10 and time.perf_counter() - t0 < budget_s:
-        oracle.spmv_f32(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"])
+        cpu()
         reps += 1
     dt = (time.perf_counter() - t0) / reps
-    # the same loop with its rows shared out among all host threads (second baseline, reported beside the first)
-    threads = oracle.host_threads()
-    oracle.spmv_f32_threads(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"], threads)
-    t0 = time.perf_counter()
-    for _ in range(5):
+    res = {"value": 2.0 * nnz / dt / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
+           "sample": "full matrix, %d repeats of the reference's %s loop restated in oracle/oracle.c "
+                     "(fp32 accumulate), %.1f ms each" % (reps, name, dt * 1e3),
+           "gpu_vs_fp64_oracle_max_rel_err": err}
+    if not transpose:
+        # the same loop with its rows shared out among all host threads (second baseline, reported beside the first)
+        threads = oracle.host_threads()
         oracle.spmv_f32_threads(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"], threads)
-    dt_all = (time.perf_counter() - t0) / 5
-    return {"value": 2.0 * nnz / dt / 1e9, "unit": "GFLOP/s", "cores": 1, "kind": "port",
-            "sample": "full matrix, %d repeats of the reference's SpmvCpu loop restated in oracle/oracle.c "
-                      "(fp32 accumulate), %.1f ms each" % (reps, dt * 1e3),
-            "all_cores": {"value": 2.0 * nnz / dt_all / 1e9, "unit": "GFLOP/s", "cores": threads,
-                          "sample": "the same loop, rows shared out among %d OpenMP threads, %.1f ms each"
-                                    % (threads, dt_all * 1e3)},
-            "gpu_vs_fp64_oracle_max_rel_err": err}
+        t0 = time.perf_counter()
+        for _ in range(5):
+            oracle.spmv_f32_threads(rows, rowptr, colind, val, x, y0, cfg["alpha"], cfg["beta"], threads)
+        dt_all = (time.perf_counter() - t0) / 5
+        res["all_cores"] = {"value": 2.0 * nnz / dt_all / 1e9, "unit": "GFLOP/s", "cores": threads,
+                            "sample": "the same loop, rows shared out among %d OpenMP threads, %.1f ms each"
+                                      % (threads, dt_all * 1e3)}
+    return res
 
 
 def cpu_baseline_spmm(cfg, c_gpu, base=None, rows_sample=262144):
@@ -268,16 +278,21 @@ def time_rounds(torch, stream, launch, steps, restore=None, min_gpu_ms=50.0, min
     """Rounds of `steps` back-to-back launches, each between two HIP events recorded on `stream` (the stream the
     kernels run on), repeated until `min_gpu_ms` of GPU time has been timed.  `launch(i)` gets the running launch
     number; `restore()` runs before every round, outside the timed region (y back to y0 when beta != 0).
-    Returns per-step milliseconds: (median round, fastest round, mean, number of rounds)."""
-    per_step, total, i = [], 0.0, 0
+    Returns per-step milliseconds (median round, fastest round, mean, number of rounds) and what a reader needs to
+    judge the spread: the slowest round, how many rounds took more than 1.5 x the median, and, for those, the time
+    the HOST spent inside the round's launch calls (a round that is slow because a launch call blocked the host shows
+    it there: the GPU then idles between the two events)."""
+    per_step, host_ms, total, i = [], [], 0.0, 0
     while (total < min_gpu_ms or len(per_step) < min_rounds) and len(per_step) < max_rounds:
         if restore is not None:
             restore()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(stream)
+        t0 = time.perf_counter()
         for _ in range(steps):
             launch(i)
             i += 1
+        host_ms.append((time.perf_counter() - t0) * 1e3)
         e1.record(stream)
         stream.synchronize()
         ms = e0.elapsed_time(e1)
@@ -285,19 +300,30 @@ def time_rounds(torch, stream, launch, steps, restore=None, min_gpu_ms=50.0, min
         total += ms
     if os.environ.get("BENCH_LOG_ROUNDS"):
         log("rounds (ms per step, in order): " + " ".join("%.4f" % v for v in per_step))
+        log("host ms inside the launch calls, per round: " + " ".join("%.2f" % v for v in host_ms))
     s = sorted(per_step)
-    return s[len(s) // 2], s[0], sum(s) / len(s), len(s)
+    median = s[len(s) // 2]
+    slow = [k for k, v in enumerate(per_step) if v > 1.5 * median]
+    spread = {"rounds": len(s), "slowest_round_ms_per_step": round(s[-1], 6),
+              "rounds_over_1p5x_median": len(slow),
+              "slow_rounds": [{"round": k, "ms_per_step": round(per_step[k], 6),
+                               "host_ms_in_launch_calls": round(host_ms[k], 3),
+                               "gpu_ms": round(per_step[k] * steps, 3)} for k in slow[:4]]}
+    return median, s[0], sum(s) / len(s), len(s), spread
 
 
 WORKLOADS = {
-    # key: (generator config, layout)
-    "c2": ("c2", "csr"),
-    "c3": ("c3", "csr"),
-    "c3_alg2": ("c3", "blocked_gather"),
-    "c3_panels": ("c3", "column_panels"),
-    "c4": ("c4", "csr"),
-    "c5": ("c5", "csr"),
+    # key: (generator config, layout asked for, op(A) = A^T, environment of the run)
+    "c2": ("c2", "csr", False, {}),
+    "c3": ("c3", "csr", False, {}),
+    "c3_repeatable": ("c3", "csr", False, {"OPS_SPARSE_SPMV_REPEATABLE": "1"}),
+    "c3_transposed": ("c3", "csr", True, {}),
+    "c3_alg2": ("c3", "blocked_gather", False, {}),
+    "c3_panels": ("c3", "column_panels", False, {"OPS_SPARSE_SPMV_NO_BLOCKED": "1"}),
+    "c4": ("c4", "csr", False, {}),
+    "c5": ("c5", "csr", False, {}),
 }
+BENCH_ENV = ("OPS_SPARSE_SPMV_NO_BLOCKED", "OPS_SPARSE_SPMV_REPEATABLE")
 _cfg_cache = {}
 
 
@@ -328,10 +354,10 @@ def make_config(wl, torch, dev, which, scale):
 
 def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
     """One workload: Preprocess once, then rounds of `--steps` calls; returns the fields of its JSON object."""
-    which, layout = WORKLOADS[key]
-    os.environ.pop("OPS_SPARSE_SPMV_NO_BLOCKED", None)
-    if layout == "column_panels":
-        os.environ["OPS_SPARSE_SPMV_NO_BLOCKED"] = "1"
+    which, layout, transpose, env = WORKLOADS[key]
+    for name in BENCH_ENV:
+        os.environ.pop(name, None)
+    os.environ.update(env)
     cfg = make_config(wl, torch, dev, which, args.scale)
     A = cfg["A"]
     rows, cols, nnz = A["rows"], A["cols"], int(A["colind"].numel())
@@ -357,10 +383,12 @@ def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
         stream.synchronize()
         t_pre = time.perf_counter()
         if not is_spmm:
+            # (op(A) = A^T: the configurations are square, x and y0 serve as they are)
             x = cfg["x"] if s <= 1 else cfg["x"].clone()
             y = cfg["y0"].clone()
             X, Y = osa.DnVec(x), osa.DnVec(y)
             op = osa.SpmvOp(handle, csr, X, Y, preprocess=not args.no_preprocess,
+                            op=osa.ACL_SPARSE_OP_TRANSPOSE if transpose else osa.ACL_SPARSE_OP_NON_TRANSPOSE,
                             alg=osa.ACL_SPARSE_SPMV_CSR_ALG2 if layout != "csr" else osa.ACL_SPARSE_SPMV_ALG_DEFAULT)
             out_t = y
         else:
@@ -378,12 +406,28 @@ def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
             preprocess_ms = dt      # GetBufferSize + buffer allocation + Preprocess: what a second matrix costs
         sets.append((op, out_t))
     if not is_spmm:
-        if layout == "blocked_gather" and not osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, 0):
-            layout = "column_panels" if osa.lib().opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz) else "csr"
-        live = osa.lib().opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
-        if layout == "csr" and live and sets[0][0].buffer is not None and sets[0][0].buffer.numel() == live:
-            # the default algorithm found the gathers scattered and took the re-stored layout with live values
+        # which plan Preprocess chose shows in the buffer it asked for
+        L = osa.lib()
+        got = sets[0][0].buffer.numel() if sets[0][0].buffer is not None else 0
+        tflag = osa.OPSPARSE_BLOCKED_TRANSPOSE if transpose else 0
+        frozen = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, tflag)
+        ordered_live = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz,
+                                                                   tflag | osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+        atomics_live = 0 if transpose else L.opsparse_spmv_csr_live_workspace_bytes(rows, cols, nnz)
+        if layout == "blocked_gather" and not (frozen and got == frozen):
+            layout = "column_panels" if L.opsparse_spmv_csr_panels_workspace_bytes(rows, cols, nnz) else "csr"
+        resident = None
+        if layout == "blocked_gather":
+            resident = L.opsparse_spmv_csr_blocked_resident_bytes(rows, cols, nnz, tflag)
+        elif layout == "csr" and atomics_live and got == atomics_live:
+            # the default algorithm found the gathers scattered: live values, row blocks summed with LDS atomics
+            layout = "blocked_live_atomics"
+            resident = L.opsparse_spmv_csr_live_resident_bytes(rows, cols, nnz)
+        elif layout == "csr" and ordered_live and got == ordered_live:
+            # ... or the same with every row summed in a fixed order (asked for, op(A) = A^T, int32)
             layout = "blocked_gather_live_values"
+            resident = L.opsparse_spmv_csr_blocked_resident_bytes(rows, cols, nnz,
+                                                                  tflag | osa.OPSPARSE_BLOCKED_LIVE_VALUES)
         ncols = 1
         bytes_alg = wl.spmv_bytes_alg(rows, cols, nnz, vb, 4, 4, beta != 0)
         bytes_gather = wl.spmv_bytes_gather(rows, cols, nnz, vb, 4, 4, beta != 0)
@@ -399,9 +443,8 @@ def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
     buf = getattr(sets[0][0], "buffer", None)
     buffer_mib = round(buf.numel() / 2.0 ** 20, 1) if buf is not None else 0.0
     resident_mib = buffer_mib
-    if layout.startswith("blocked_gather"):
-        flags = osa.OPSPARSE_BLOCKED_LIVE_VALUES if layout.endswith("live_values") else 0
-        resident_mib = round(osa.lib().opsparse_spmv_csr_blocked_resident_bytes(rows, cols, nnz, flags) / 2.0 ** 20, 1)
+    if not is_spmm and resident is not None:
+        resident_mib = round(resident / 2.0 ** 20, 1)
 
     def restore():
         if beta != 0:  # y back to y0 before every round, outside the timed region
@@ -415,11 +458,18 @@ def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
     for i in range(args.warmup):
         sets[i % len(sets)][0](alpha, beta)
     stream.synchronize()
-    ms, ms_min, ms_mean, nrounds = time_rounds(torch, stream, lambda i: sets[i % len(sets)][0](alpha, beta),
-                                               args.steps, restore, args.min_gpu_ms)
+    # Settling, untimed like the warm-up: the HIP runtime blocks the host for some 30 ms inside one launch call
+    # around a process's 330th kernel launch (and for 1 ms around the 170th) while it grows one of its pools, and
+    # the GPU's clocks take some 200 launches of this size to settle.  Both are one-off: left in the timed
+    # region they cost most of its 50 ms budget and put the median on the unsettled rounds.
+    for i in range(args.settle):
+        sets[i % len(sets)][0](alpha, beta)
+    stream.synchronize()
+    ms, ms_min, ms_mean, nrounds, spread = time_rounds(torch, stream, lambda i: sets[i % len(sets)][0](alpha, beta),
+                                                       args.steps, restore, args.min_gpu_ms)
     warm = None
     if len(sets) > 1:
-        w_ms, w_min, _, _ = time_rounds(torch, stream, lambda i: sets[0][0](alpha, beta), args.steps, restore,
+        w_ms, w_min, _, _, _ = time_rounds(torch, stream, lambda i: sets[0][0](alpha, beta), args.steps, restore,
                                         args.min_gpu_ms)
         warm = {"ms_per_step": round(w_ms, 6), "ms_per_step_min": round(w_min, 6),
                 "achieved": round(bytes_alg / (w_ms * 1e-3) / 1e9, 1),
@@ -434,18 +484,22 @@ def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
         % (key, ms * 1e3, nrounds, args.steps, ms_min * 1e3, ms_mean * 1e3, gflops, gbps, 100 * gbps / HBM_PEAK_GBPS,
            "; same operands every launch %.2f us = %.1f%%" % (warm["ms_per_step"] * 1e3, 100 * warm["frac"])
            if warm else ""))
-    traffic = load_traffic(cfg["name"] + ("+" + layout if layout != "csr" else "")) if args.scale == 1.0 else None
+    traffic = load_traffic(cfg["name"] + ("+" + layout if layout != "csr" else "") +
+                           ("+transposed" if transpose else "")) if args.scale == 1.0 else None
     out = {
         "value": round(gflops, 2), "unit": "GFLOP/s", "ms_per_step": round(ms, 6),
         "ms_per_step_min": round(ms_min, 6), "ms_per_step_mean": round(ms_mean, 6), "rounds": nrounds,
+        "round_spread": spread,
         "dtype": dtype,
         "config": {"workload": cfg["name"], "rows": rows, "cols": cols, "nnz": nnz, "ncols_dense": ncols,
                    "alpha": alpha, "beta": beta, "index": "int32", "preprocess_ms": round(preprocess_ms, 3),
                    "first_use_ms": round(first_use_ms, 3), "preprocessed": not args.no_preprocess, "layout": layout,
                    "operand_sets": len(sets), "buffer_mib": buffer_mib, "buffer_resident_mib": resident_mib,
+                   "op": "transpose" if transpose else "non_transpose",
                    "timing": "median over rounds of `steps` launches between HIP events on the handle's stream, "
-                             "rounds repeated until %.0f ms of GPU time%s" % (
-                                 args.min_gpu_ms, "; y restored to y0 before every round" if beta != 0 else "")},
+                             "rounds repeated until %.0f ms of GPU time, after `warmup` + %d untimed launches%s" % (
+                                 args.min_gpu_ms, args.settle,
+                                 "; y restored to y0 before every round" if beta != 0 else "")},
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
                      "traffic": traffic,
@@ -463,13 +517,164 @@ def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
         out["vendor_yardstick"] = vendor_yardstick(torch, cfg, is_spmm, flops, bytes_alg, max(5, args.steps // 4),
                                                    stream, sets[0][1].clone())
     if not args.no_cpu:
-        base = cpu_cache.get(which)
-        res = (cpu_baseline_spmm if is_spmm else cpu_baseline_spmv)(cfg, first_result, base)
-        cpu_cache[which] = res
+        ck = which + ("_t" if transpose else "")
+        base = cpu_cache.get(ck)
+        res = (cpu_baseline_spmm(cfg, first_result, base) if is_spmm else
+               cpu_baseline_spmv(cfg, first_result, base, transpose=transpose))
+        cpu_cache[ck] = res
         out["cpu_baseline"] = res
         out["gpu_vs_fp64_oracle_max_rel_err"] = res["gpu_vs_fp64_oracle_max_rel_err"]
     del sets
     return out
+
+
+def run_c1(args, osa, torch, dev, stream, handle):
+    """The reference's own CPU-runnable case: m = n = 4096, 16 entries a row from the reference's generator
+    (SparseFillGenerator, seed 42: reference test/frame/fill.h:71-111), values and x ~ U(-1, 1), alpha = 1,
+    beta = 0.  65 536 entries are 0.8 MB: a call is bound by launch latency, not bandwidth, so the entry gives
+    microseconds per call (with and without Preprocess) beside the time of the reference's SpmvCpu loop, and no
+    roofline.  The generator and the CPU loop are the oracle's: this entry is part of the CPU-baseline leg."""
+    import numpy as np
+    import oracle
+    rows = cols = 4096
+    rowptr, colind, val = oracle.fill_csr(42, rows, cols, rows * 16, -1.0, 1.0)
+    x = oracle.fill_dense(43, cols, -1.0, 1.0)
+    nnz = int(colind.size)
+    d = [torch.from_numpy(a).to(dev) for a in (rowptr, colind, val, x)]
+    csr = osa.Csr(rows, cols, d[0], d[1], d[2])
+    y = torch.zeros(rows, dtype=torch.float32, device=dev)
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, None, 1.0, 0.0)
+    out = {"config": {"workload": "c1_reference_generator_4096x4096_16_per_row", "rows": rows, "cols": cols,
+                      "nnz": nnz, "alpha": 1.0, "beta": 0.0, "seed": 42},
+           "unit": "us per call", "dtype": "f32",
+           "note": "latency-bound (0.8 MB of operands): no roofline figure is claimed for it"}
+    for name, pre in (("prepared", True), ("unprepared", False)):
+        op = osa.SpmvOp(handle, csr, osa.DnVec(d[3]), osa.DnVec(y), preprocess=pre)
+        y.fill_(float("nan"))
+        op(1.0, 0.0)
+        stream.synchronize()
+        err = oracle.max_rel_err(y.cpu().numpy(), gold)
+        if err > 1e-5:
+            sys.exit("bench.py: c1 (%s) differs from the fp64 oracle (%.3g)" % (name, err))
+        for _ in range(200):
+            op(1.0, 0.0)
+        stream.synchronize()
+        ms, ms_min, _, nrounds, spread = time_rounds(torch, stream, lambda i: op(1.0, 0.0), 100, None, 20.0)
+        # one call at a time: launch, then wait for it (what a caller that needs y at once sees)
+        t0 = time.perf_counter()
+        for _ in range(200):
+            op(1.0, 0.0)
+            stream.synchronize()
+        sync_us = (time.perf_counter() - t0) / 200 * 1e6
+        out[name] = {"us_per_call_back_to_back": round(ms * 1e3, 3), "us_per_call_fastest_round": round(ms_min * 1e3, 3),
+                     "us_per_call_with_synchronize": round(sync_us, 2), "rounds": nrounds,
+                     "gflops_back_to_back": round(2.0 * nnz / (ms * 1e-3) / 1e9, 2),
+                     "gpu_vs_fp64_oracle_max_rel_err": err}
+    oracle.spmv_f32(rows, rowptr, colind, val, x, np.zeros(rows, np.float32), 1.0, 0.0)
+    t0 = time.perf_counter()
+    reps = 2000
+    for _ in range(reps):
+        oracle.spmv_f32(rows, rowptr, colind, val, x, np.zeros(rows, np.float32), 1.0, 0.0)
+    dt = (time.perf_counter() - t0) / reps
+    out["cpu_baseline"] = {"value": round(dt * 1e6, 2), "unit": "us per call", "cores": 1, "kind": "port",
+                           "gflops": round(2.0 * nnz / dt / 1e9, 3),
+                           "sample": "%d repeats of the reference's SpmvCpu loop restated in oracle/oracle.c on the "
+                                     "whole matrix (through ctypes, a fresh y each)" % reps}
+    log("c1        prepared %.2f us, unprepared %.2f us per call back to back; SpmvCpu %.1f us"
+        % (out["prepared"]["us_per_call_back_to_back"], out["unprepared"]["us_per_call_back_to_back"], dt * 1e6))
+    return out
+
+
+def run_shapes(args, osa, wl, torch, dev, stream, handle):
+    """Time per call on the secondary shapes that the selection thresholds were set from: which plan a matrix gets
+    (the layouts from 7 M entries, 31 % / 19 % far gathers, 2^18 columns; the long-row cut-offs) is decided by these
+    grids.  Per shape: the default plan as selected, the default plan forced onto the caller's arrays (merge path /
+    row-wise kernels), the default plan with repeatable sums, and ACL_SPARSE_SPMV_CSR_ALG2.  --scale below 1 keeps
+    the first shapes of every group only."""
+    i64 = torch.int64
+
+    def rows_of(rows, per_row, cols, seed, sort):
+        """`per_row` random columns a row, unsorted (repeats possible) or sorted."""
+        idx = torch.arange(rows * per_row, dtype=i64, device=dev)
+        ci = (wl._lsr(wl.hash64(seed, idx), 11) % cols).view(rows, per_row)
+        if sort:
+            ci = ci.sort(dim=1).values
+        return {"rows": rows, "cols": cols, "rowptr": (torch.arange(rows + 1, dtype=i64, device=dev) * per_row).int(),
+                "colind": ci.reshape(-1).int(), "values": wl.uniform(seed + 1, rows * per_row, -1.0, 1.0, dev)}
+
+    def band(rows, near, far, seed):
+        idx = torch.arange(rows * (near + far), dtype=i64, device=dev)
+        h = wl._lsr(wl.hash64(seed, idx), 11).view(rows, near + far)
+        r = torch.arange(rows, dtype=i64, device=dev).view(rows, 1)
+        ci = torch.cat([(r + h[:, :near] % 81 - 40).clamp(0, rows - 1), h[:, near:] % rows], dim=1).sort(dim=1).values
+        return {"rows": rows, "cols": rows, "colind": ci.reshape(-1).int(),
+                "rowptr": (torch.arange(rows + 1, dtype=i64, device=dev) * (near + far)).int(),
+                "values": wl.uniform(seed + 1, rows * (near + far), -1.0, 1.0, dev)}
+
+    def power_law(m, alpha, lmax, mean):
+        A = wl.power_law_csr(m, m, alpha, 1, lmax, 2001, dev, target_mean=mean)
+        A["values"] = wl.uniform(2002, A["colind"].numel(), -1.0, 1.0, dev)
+        return A
+
+    M = 1 << 20
+    groups = {
+        "equal_rows_unsorted_columns": [("%g M x %d (%g M columns)" % (r / 1e6, k, c / 1e6),
+                                         lambda r=r, k=k, c=c: rows_of(r, k, c, 7, False))
+                                        for r, k, c in ((1000000, 4, 1100000), (1500000, 4, 1600000),
+                                                        (2000000, 4, 2200000), (1000000, 8, 2200000),
+                                                        (3000000, 3, 8000000), (2000000, 8, 2200000),
+                                                        (6000000, 2, 20000000), (2000000, 8, 33000000),
+                                                        (4000000, 4, 33000000), (1000000, 32, 16000000),
+                                                        (4000000, 8, 16000000), (2000000, 16, 30000000),
+                                                        (16000000, 2, 16000000), (8000000, 4, 33000000))],
+        "band_plus_random_4M_rows": [("%d + %d" % (n, f), lambda n=n, f=f: band(4000000, n, f, 11))
+                                     for n, f in ((5, 1), (15, 1), (14, 2), (12, 4), (4, 4), (30, 2), (30, 6), (60, 4))],
+        "equal_rows_sorted_columns": [("%d x %d (x of %g M)" % (r, k, c / 1e6),
+                                       lambda r=r, k=k, c=c: rows_of(r, k, c, 13, True))
+                                      for c in (3000000, 8000000, 300000, 600000, 1000000)
+                                      for r, k in ((20000, 2000), (50000, 1100), (4000, 8000), (2000, 20000),
+                                                   (200000, 300), (3000000, 12))
+                                      if (c == 8000000) == ((r, k) == (20000, 2000)) or c < 3000000],
+        "power_law": [("%g M rows, exponent %g, longest %d" % (m / M, a, lmax),
+                       lambda m=m, a=a, lmax=lmax, mean=mean: power_law(m, a, lmax, mean))
+                      for m, a, lmax, mean in ((1 * M, 2.0, 200000, None), (2 * M, 2.0, 200000, None),
+                                               (4 * M, 2.0, 200000, None), (8 * M, 2.5, 200000, 8.0),
+                                               (4 * M, 1.6, 100000, None))],
+    }
+    plans = (("default", {}, 0), ("default_on_callers_arrays", {"OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ": str(1 << 62)}, 0),
+             ("default_repeatable", {"OPS_SPARSE_SPMV_REPEATABLE": "1"}, 0),
+             ("alg2", {}, osa.ACL_SPARSE_SPMV_CSR_ALG2))
+    res = {}
+    for gname, shapes in groups.items():
+        res[gname] = {}
+        if args.scale < 1.0:
+            shapes = shapes[:2]
+        for sname, make in shapes:
+            torch.cuda.empty_cache()
+            A = make()
+            rows, cols, nnz = A["rows"], A["cols"], int(A["colind"].numel())
+            csr = osa.Csr(rows, cols, A["rowptr"], A["colind"], A["values"])
+            x = wl.uniform(5, cols, -1.0, 1.0, dev)
+            y = torch.zeros(rows, dtype=torch.float32, device=dev)
+            line = {"nnz": nnz}
+            for pname, env, alg in plans:
+                for name in BENCH_ENV + ("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ",):
+                    os.environ.pop(name, None)
+                os.environ.update(env)
+                op = osa.SpmvOp(handle, csr, osa.DnVec(x), osa.DnVec(y), alg=alg)
+                for _ in range(3):
+                    op(1.0, 0.0)
+                stream.synchronize()
+                ms, _, _, _, _ = time_rounds(torch, stream, lambda i: op(1.0, 0.0), 5, None, 15.0)
+                line[pname] = round(ms * 1e3, 1)
+                line[pname + "_buffer_mib"] = round(op.buffer.numel() / 2.0 ** 20, 1)
+                del op
+            for name in BENCH_ENV + ("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ",):
+                os.environ.pop(name, None)
+            res[gname][sname] = line
+            log("%-28s %-40s %s" % (gname, sname, json.dumps(line)))
+            del A, csr, x, y
+    return res
 
 
 def run_cache_probe(args, osa, wl, torch, dev, stream, handle):
@@ -531,7 +736,7 @@ def run_convert(args, osa, torch, dev, stream, handle):
         def timed(fn):
             fn()
             stream.synchronize()
-            ms, ms_min, _, _ = time_rounds(torch, stream, lambda i: fn(), 3, None, 20.0)
+            ms, ms_min, _, _, _ = time_rounds(torch, stream, lambda i: fn(), 3, None, 20.0)
             return ms
 
         t = timed(lambda: L.aclsparseXcsr2coo(handle.h, P(rowptr), nnz, m, P(rowsOut), 0))
@@ -597,11 +802,16 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all",
-                    choices=["all", "c2", "c3", "c4", "c5", "convert", "cache"],
-                    help="all: c2 as the headline plus c3 (default plan and ALG2), c4 and c5 in `workloads`")
+                    choices=["all", "c1", "c2", "c3", "c3_repeatable", "c3_transposed", "c4", "c5", "convert", "cache",
+                             "shapes"],
+                    help="all: c2 as the headline plus c1, c3 (default plan, repeatable default plan, ALG2, "
+                         "transposed), c4 and c5 in `workloads`; shapes: the grid of secondary shapes behind the "
+                         "selection thresholds")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
     ap.add_argument("--min-gpu-ms", type=float, default=50.0,
                     help="rounds of --steps launches are repeated until this much GPU time has been timed")
+    ap.add_argument("--settle", type=int, default=400,
+                    help="untimed launches after the warm-up, before the timed rounds (the runtime's one-off stalls)")
     ap.add_argument("--warm-only", action="store_true",
                     help="time every launch on one operand set also where that fits the Infinity Cache")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -633,6 +843,17 @@ def main():
                           "probe": run_cache_probe(args, osa, wl, torch, dev, stream, handle)}), flush=True)
         handle.close()
         return
+    if args.workload == "c1":
+        print(json.dumps({"metric": "CSR SpMV fp32, time per call on the reference's CPU-runnable case",
+                          "data": "synthetic", "c1": run_c1(args, osa, torch, dev, stream, handle)}), flush=True)
+        handle.close()
+        return
+    if args.workload == "shapes":
+        print(json.dumps({"metric": "CSR SpMV fp32, time per call by shape and plan", "unit": "us",
+                          "data": "synthetic", "shapes": run_shapes(args, osa, wl, torch, dev, stream, handle)}),
+              flush=True)
+        handle.close()
+        return
     if args.workload == "convert":
         print(json.dumps({"metric": "CSR producers, time per call", "unit": "ms", "data": "synthetic",
                           "operations": run_convert(args, osa, torch, dev, stream, handle)}), flush=True)
@@ -657,8 +878,11 @@ def main():
     out.update(head)
     if args.workload == "all":
         out["workloads"] = {}
-        for key in ("c4", "c5", "c3", "c3_alg2"):
+        for key in ("c4", "c5", "c3", "c3_repeatable", "c3_alg2", "c3_transposed"):
             out["workloads"][key] = run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache)
+        if not args.no_cpu:
+            _cfg_cache.clear()
+            out["workloads"]["c1"] = run_c1(args, osa, torch, dev, stream, handle)
     print(json.dumps(out), flush=True)
     handle.close()
 

@@ -1529,7 +1529,8 @@ int opsparse_spmv_csr_live_analyse(const int32_t *rowOffsets, const int32_t *col
         // Row blocks of fewer than 65535 positions, all of them (the rule unless a row that cannot go the long rows'
         // way is longer than that): 16-bit positions relative to the block, 2 bytes an entry less at every call.
         const int32_t longest = tail[0];
-        static const bool noShort = std::getenv("OPS_SPARSE_BLOCKED_NO_SHORT_POSITIONS") != nullptr;
+        // (tuning / test switch, read at every analysis)
+        const bool noShort = std::getenv("OPS_SPARSE_BLOCKED_NO_SHORT_POSITIONS") != nullptr;
         if (!noShort && longest < static_cast<int32_t>(kNoPosition16)) {
             hipLaunchKernelGGL(BlockedShortPositionsKernel, dim3(static_cast<uint32_t>(l.B)), dim3(kBlkThreads), 0, s,
                                ints(l.blockEntryOff), dstStart, l.P, ints(l.dstOfPosOff));

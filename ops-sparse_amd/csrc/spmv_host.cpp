@@ -247,8 +247,9 @@ bool SizedFor(aclsparseConstSpMatDescr_t matA, const RestoredChoice &choice, boo
 RestoredChoice PickLiveLayout(aclsparseHandle_t handle, const int32_t *rowOffsets, const int32_t *colInd, int64_t rows,
                               int64_t cols, int64_t nnz, bool transpose, int32_t valueType, bool repeatable)
 {
-    static const bool off = std::getenv("OPS_SPARSE_SPMV_NO_DEFAULT_BLOCKED") != nullptr ||
-                            std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") != nullptr;
+    // (read at every call, like the other switches of the selection: a process may set them between two matrices)
+    const bool off = std::getenv("OPS_SPARSE_SPMV_NO_DEFAULT_BLOCKED") != nullptr ||
+                     std::getenv("OPS_SPARSE_SPMV_NO_BLOCKED") != nullptr;
     if (off || rowOffsets == nullptr || colInd == nullptr) {
         return {0, 0, false};
     }

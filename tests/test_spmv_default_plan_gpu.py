@@ -688,3 +688,43 @@ def test_default_plan_with_int32_values(osa, gpu_ctx, transpose, int_compute):
     val2 = rng.integers(-big, big, nnz).astype(np.int32)
     d[2].copy_(torch.from_numpy(val2))                       # in place: followed
     check(val2, *((-1, 0) if int_compute else (1.0, 0.0)))
+
+
+@pytest.mark.parametrize("how", ["switch", "long_block"])
+def test_atomics_layout_with_32_bit_positions(osa, gpu_ctx, how, monkeypatch):
+    """The atomics layout keeps where every entry sits in its row block in 16 bits when every block is shorter than
+    65 535 positions, else in 32: asked for by the switch, and forced by a row of 70 000 entries whose columns do not
+    ascend (it cannot go the long rows' way and makes one block that long).  Same products either way."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = 300_000, 1_400_000
+    rng = np.random.default_rng(37)
+    lengths = rng.integers(0, 20, rows)
+    if how == "long_block":
+        lengths[123_456] = 70_000
+    else:
+        monkeypatch.setenv("OPS_SPARSE_BLOCKED_NO_SHORT_POSITIONS", "1")
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    x, y0 = rng.uniform(-1, 1, cols).astype(np.float32), rng.uniform(-1, 1, rows).astype(np.float32)
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    nnz = colind.size
+    need = L.opsparse_spmv_csr_live_workspace_bytes(rows, cols, nnz)
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    plan = osa.OpsparseSpmvPlan()
+    pv = lambda t: ctypes.c_void_p(t.data_ptr())
+    assert L.opsparse_spmv_csr_live_analyse(pv(d[0]), pv(d[1]), pv(d[2]), rows, cols, nnz, 0, pv(ws), need,
+                                            ctypes.byref(plan), ctypes.c_void_p(stream.cuda_stream)) == 0
+    assert plan.kernel == osa.OPSPARSE_SPMV_BLOCKED_LIVE and plan.liveValues == 1
+    del ws
+    d_y = to_dev(y0, dev)
+    op = osa.SpmvOp(handle, osa.Csr(rows, cols, d[0], d[1], d[2]), osa.DnVec(d[3]), osa.DnVec(d_y))
+    assert op.buffer.numel() == need
+    for values, alpha, beta in ((val, 1.0, 0.0), ((val * np.float32(-2.0)).astype(np.float32), 0.5, 1.5)):
+        d[2].copy_(torch.from_numpy(values))
+        d_y.copy_(torch.from_numpy(y0))
+        op(alpha, beta)
+        stream.synchronize()
+        gold = oracle.spmv_f64(rows, cols, rowptr, colind, values, x, y0, alpha, beta)
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
