@@ -287,7 +287,24 @@ aclsparseStatus_t aclsparseDnMatSetValues(aclsparseDnMatDescr_t dnMatDescr, void
  * Preprocess [ref: :490-514, declared by the reference without a definition]
  * analyse the row-length distribution once and store the kernel choice and the
  * merge-path partition in the caller's buffer; later aclsparseSpMV calls that
- * pass the same buffer skip that work.
+ * pass the same buffer skip that work.  For a large matrix with scattered
+ * columns the answer of GetBufferSize is larger and Preprocess re-stores the
+ * matrix in the buffer; it does so only where a GetBufferSize call on the same
+ * descriptor and arrays, with the same opA / types / alg, answered that size
+ * (a buffer sized any other way gets the ordinary plan, which fits every
+ * answer).
+ *
+ * Repeatability [ref: include/cann_ops_sparse.h:151-164]: ACL_SPARSE_SPMV_CSR_ALG2
+ * gives bit-wise the same y from every call on the same data, for either op(A)
+ * (the reference promises it for op(A) = A only).  So do ALG_DEFAULT / CSR_ALG1
+ * with op(A) = A wherever the plan is row-wise or merge-path (every unprepared
+ * call, every matrix under 7 M entries or with local columns) and for int32.
+ * The one plan that adds in the order its wavefronts arrive is the default
+ * algorithm's re-stored layout for op(A) = A on floating-point data, and
+ * op(A) = A^T without Preprocess (fp32 atomics on y): there the last bit of an
+ * element may differ between two calls, as the reference says of CSR_ALG1.
+ * OPS_SPARSE_SPMV_REPEATABLE=1 in the environment makes Preprocess choose
+ * the ordered layout there too.
  *
  * alpha / beta: typed by computeType; NULL means alpha = 1, beta = 0
  * [ref: spmv_host.cpp:183-199]; read according to the handle's pointer mode.
@@ -347,14 +364,23 @@ aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t o
  * Z = alpha * A * X + beta * Y with a descriptor / plan pair, fp32 only:
  * opA = NON_TRANSPOSE, computeType ACL_FLOAT, CSR with fp32 values, 32-bit
  * column indices, 32- or 64-bit row offsets, index base 0 or 1.  Z may be Y.
- * Results are deterministic (fixed summation order, fp64 accumulator) for every
- * algorithm value.
+ * Results are bit-wise repeatable for every algorithm value [ref:
+ * include/cann_ops_sparse.h:57-69]: every row is summed in fp64 in an order that
+ * depends on the matrix and the plan only, never on scheduling (no atomics on
+ * any path of this API), and rounded once.
  *
- *   bufferSize    0 for ALG_DEFAULT / ALG1; for ALG2 the bytes of the
- *                 nnz-balanced partition createDescr writes.
+ *   bufferSize    for ALG2 the bytes of what createDescr writes (the
+ *                 nnz-balanced partition, or a re-stored copy of the matrix
+ *                 where x does not fit a cache); for ALG_DEFAULT / ALG1 0,
+ *                 except for a large matrix with scattered columns (fp32,
+ *                 zero-based 32-bit offsets, 7 M entries or more), where it is
+ *                 the size of a re-stored index layout that createDescr builds
+ *                 IF it is given a buffer (NULL stays legal: the ordinary
+ *                 kernels then).  A layout is only built into a buffer when
+ *                 bufferSize was asked on the same descriptor and arrays.
  *   createDescr   snapshots matA's pointers and sizes (not its values: they may
- *                 change between executions); ALG2 needs `buffer`, which must
- *                 stay valid until destroyDescr.
+ *                 change between executions, except under ALG2); ALG2 needs
+ *                 `buffer`, which must stay valid until destroyDescr.
  *   createPlan    only the identity epilogue: a non-NULL LTO buffer or a
  *                 non-zero size gives NOT_SUPPORTED.
  *   destroy*      NULL is accepted and gives SUCCESS.
