@@ -110,6 +110,9 @@ typedef struct OpsparseSpmvPlan {
     int32_t valueType;     /* BLOCKED_GATHER: the OPSPARSE_F32 / F16 / BF16 / I32 the layout was built from; launches
                               must bring values and x of that type (y: fp32, or that type) */
     int32_t numEmptyRows;  /* BLOCKED_GATHER: rows without entries; a small kernel of their own writes beta * y there */
+    int32_t streamedBlocks;/* BLOCKED_GATHER: 1: the layout keeps the values, in (block, panel) order, and a wavefront
+                              streams a run of row blocks; 0: values read in row order through a window in LDS */
+    int32_t reserved0;
     int64_t rows;
     int64_t nnz;
     int64_t partOff;       /* byte offsets into the workspace */

@@ -124,7 +124,7 @@ class OpsparseSpmvPlan(ctypes.Structure):
                 ("maxRowNnz", i32), ("partitionReady", i32), ("numPanels", i32),
                 ("panelShift", i32), ("numRowBlocks", i32), ("entryWindow", i32), ("transposed", i32),
                 ("guardTiles", i32), ("tileRowNnz", i32), ("longRowsBeside", i32), ("liveValues", i32),
-                ("numLongRows", i32), ("numDeferredLongRows", i32), ("valueType", i32), ("numEmptyRows", i32), ("rows", i64), ("nnz", i64),
+                ("numLongRows", i32), ("numDeferredLongRows", i32), ("valueType", i32), ("numEmptyRows", i32), ("streamedBlocks", i32), ("reserved0", i32), ("rows", i64), ("nnz", i64),
                 ("partOff", i64),
                 ("carryOff", i64), ("headOff", i64), ("bytes", i64), ("panelStart", i64 * 17)]
 

@@ -77,6 +77,19 @@ constexpr int kMaxPanels = 1024;
 constexpr int kGatherBatch = 8;                   // groups of 4 entries in flight per lane, phase 1
 constexpr int kLaneEntries = 8;                   // in block order a chunk is padded to a multiple of this
 constexpr uint32_t kPadSlot = 0xffffu;            // slot of a padding position in block order
+// Streamed row blocks (values kept or refreshed in block order): a wavefront owns a block, its rows' sums in LDS.
+constexpr int kStreamRowLog = 10;                 // rows per block at most: 8 KiB of 64-bit sums a wavefront
+constexpr int kStreamRows = 1 << kStreamRowLog;
+constexpr int32_t kStreamWindow = 65536;          // a block is also cut wherever the entry count passes a multiple of this
+constexpr int32_t kStreamMinWindow = 4096;        // (of this, where the matrix has few rows: MakeBlockedLayout)
+constexpr int64_t kStreamBlocksWanted = 8192;
+constexpr int64_t kStreamMinChunkEntries = 16;
+constexpr int64_t kStreamMaxRowPanelEntries = 16;
+constexpr int kStreamThreads = 64;                // a wavefront a workgroup: nothing is shared, nothing waits
+constexpr int kTurnThreads = 256;
+constexpr uint32_t kStreamPadRow = 0x7ffu;        // row field of a padding position (rows take 10 of its 11 bits)
+constexpr int kStreamRoundShift = 11;             // above the row: the turn of the entry among those of its row that
+constexpr uint32_t kStreamMaxRound = 31;          // one LDS instruction would add together (31: "31st or later")
 constexpr int32_t kMaxBlockEntries = 65534;       // a block's slots are 16 bits
 // Phase 2 holds the gathered x of a row block in a window of LDS (kRowsWindow entries: two workgroups then share a
 // compute unit).  The blocks are cut at three quarters of that (plus the row in which the cut falls), so that
@@ -406,13 +419,13 @@ struct BlockMeta {
 __host__ __device__ __forceinline__ int32_t BlockBitsOff(int32_t short0, int32_t b) { return ((short0 >> 5) & ~3) + 8 * b; }
 __host__ __device__ __forceinline__ int32_t BlockOrdOff(int32_t row0, int32_t b) { return ((row0 + 7) & ~7) + 16 * b; }
 
-// Row block of a row: 2^12-row blocks, cut again wherever the row's first entry passes a multiple of the entry
+// Row block of a row: blocks of 2^rowLog rows, cut again wherever the row's first entry passes a multiple of the entry
 // window (`offsets`: the row offsets without the entries of long rows), and, with `longBefore` (the number of long
 // rows among rows 0 .. r), behind every long row.  Monotone in the row number.
 __device__ __forceinline__ int32_t RowBlockOf(const int32_t *__restrict__ offsets, int32_t row, int32_t window,
-                                              int32_t numBlocks, const int32_t *__restrict__ longBefore)
+                                              int32_t numBlocks, const int32_t *__restrict__ longBefore, int32_t rowLog)
 {
-    int32_t b = (row >> kRowBlockLog) + offsets[row] / window;
+    int32_t b = (row >> rowLog) + offsets[row] / window;
     if (longBefore != nullptr && row > 0) {
         b += longBefore[row - 1];
     }
@@ -455,7 +468,7 @@ __global__ __launch_bounds__(kBlockThreads) void IotaKernel(int32_t *__restrict_
 __global__ __launch_bounds__(kBlockThreads) void BlockedChunkKeysKernel(
     const int32_t *__restrict__ colSorted, const int32_t *__restrict__ pos, const int32_t *__restrict__ rowOfPos,
     const int32_t *__restrict__ offsets, int64_t nnz, int64_t cols, int32_t numBlocks, int32_t window,
-    const int32_t *__restrict__ longBefore, int32_t cutBehindLong, uint16_t *__restrict__ colLocal,
+    const int32_t *__restrict__ longBefore, int32_t cutBehindLong, int32_t rowLog, uint16_t *__restrict__ colLocal,
     int32_t *__restrict__ chunkKey, int32_t *__restrict__ rowOfSrc, int32_t *__restrict__ status)
 {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
@@ -471,7 +484,7 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedChunkKeysKernel(
             chunkKey[i] = -1;
         } else {
             chunkKey[i] = (col >> kPanelLog) * numBlocks +
-                          RowBlockOf(offsets, row, window, numBlocks, cutBehindLong != 0 ? longBefore : nullptr);
+                          RowBlockOf(offsets, row, window, numBlocks, cutBehindLong != 0 ? longBefore : nullptr, rowLog);
         }
     }
 }
@@ -685,15 +698,15 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedTablesKernel(const int32
 __global__ __launch_bounds__(kBlockThreads) void BlockedRowBlocksKernel(const int32_t *__restrict__ offsets,
                                                                         int32_t rows, int32_t window, int32_t B,
                                                                         const int32_t *__restrict__ longBefore,
-                                                                        int32_t *__restrict__ blockRow)
+                                                                        int32_t rowLog, int32_t *__restrict__ blockRow)
 {
     const int64_t r = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
     if (r >= rows) {
         return;
     }
     const int32_t row = static_cast<int32_t>(r);
-    const int32_t cur = RowBlockOf(offsets, row, window, B, longBefore);
-    const int32_t prev = row > 0 ? RowBlockOf(offsets, row - 1, window, B, longBefore) : -1;
+    const int32_t cur = RowBlockOf(offsets, row, window, B, longBefore, rowLog);
+    const int32_t prev = row > 0 ? RowBlockOf(offsets, row - 1, window, B, longBefore, rowLog) : -1;
     for (int32_t b = prev + 1; b <= cur; ++b) {
         blockRow[b] = row;
     }
@@ -712,10 +725,11 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedLongFirstKernel(const in
     }
 }
 
-// longDeferred[l] = 1 for the long rows of a row block that holds more than kInBlockLongRows of them, else 0;
+// longDeferred[l] = 1 for the long rows of a row block that holds more than kInBlockLongRows of them (`always`: of
+// every block: streamed blocks leave all long rows to SpmvLongRowSumKernel), else 0;
 // header[4] (zero before) = their number.
 __global__ __launch_bounds__(kBlockThreads) void BlockedLongDeferKernel(const int32_t *__restrict__ longFirst, int32_t B,
-                                                                        int32_t *__restrict__ longDeferred,
+                                                                        int32_t always, int32_t *__restrict__ longDeferred,
                                                                         int32_t *__restrict__ header)
 {
     const int32_t b = static_cast<int32_t>(blockIdx.x * blockDim.x + threadIdx.x);
@@ -723,7 +737,7 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedLongDeferKernel(const in
         return;
     }
     const int32_t l0 = longFirst[b], l1 = longFirst[b + 1];
-    const int32_t defer = l1 - l0 > kInBlockLongRows ? 1 : 0;
+    const int32_t defer = (always != 0 || l1 - l0 > kInBlockLongRows) ? 1 : 0;
     for (int32_t l = l0; l < l1; ++l) {
         longDeferred[l] = defer;
     }
@@ -953,6 +967,85 @@ __global__ __launch_bounds__(kBlockThreads) void BlockedScatterKernel(
         slot16[dst] = static_cast<uint16_t>(WindowPlace(static_cast<uint32_t>(slot)));
         if ((dst & (kLaneEntries - 1)) == 0) {
             src8[dst / kLaneEntries] = static_cast<int32_t>(i);  // where these eight positions sit in panel order
+        }
+    }
+}
+
+// Streamed row blocks: what the scatter above does for the windowed ones.  Per position of the (block, panel) order
+// the entry's row, counted from its block's first (the turn bits are added by StreamTurnsKernel), its value
+// (`valD`: values frozen) or where its value sits in the value array (`posD`: values read at every call), and per
+// eight positions where they sit in panel order.  Long entries as above.
+template <typename ValT>
+__global__ __launch_bounds__(kBlockThreads) void StreamScatterKernel(
+    const int32_t *__restrict__ pos, const int32_t *__restrict__ rowOfSrc, const int32_t *__restrict__ chunkKey,
+    const ValT *__restrict__ vals, const int32_t *__restrict__ srcStart, const int32_t *__restrict__ dstStart,
+    const int32_t *__restrict__ blockRow, int64_t nnz, int32_t P, int32_t B, uint16_t *__restrict__ field,
+    int32_t *__restrict__ src8, ValT *__restrict__ valD, int32_t *__restrict__ posD, uint32_t *__restrict__ longVals,
+    uint16_t *__restrict__ longRowOf, const int32_t *__restrict__ longBefore)
+{
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
+        const int32_t key = chunkKey[i];
+        if (key < 0) {
+            if (longVals != nullptr) {
+                longVals[i] = ToRaw(vals[pos[i]]);
+                longRowOf[i] = static_cast<uint16_t>(longBefore[rowOfSrc[i]] - 1);
+            }
+            continue;
+        }
+        const int32_t p = key / B, b = key % B;
+        const int64_t dst = i - srcStart[key] + dstStart[static_cast<int64_t>(b) * P + p];
+        int32_t local = rowOfSrc[i] - blockRow[b];
+        local = local < 0 ? 0 : (local < kStreamRows ? local : kStreamRows - 1);
+        field[dst] = static_cast<uint16_t>(local);
+        if (valD != nullptr) {
+            valD[dst] = vals[pos[i]];
+        }
+        if (posD != nullptr) {
+            posD[dst] = pos[i];
+        }
+        if ((dst & (kLaneEntries - 1)) == 0) {
+            src8[dst / kLaneEntries] = static_cast<int32_t>(i);
+        }
+    }
+}
+
+// The turns.  SpmvBlockStreamKernel's wavefront takes 256 positions of its block at a time, lane l the four
+// positions 4 l .. 4 l + 3 of them, and adds entry j of every lane to the rows' sums with one LDS instruction.  Two
+// lanes of such an instruction that hold the same row must not add at once (the order of the two additions would be
+// the hardware's choice): an entry's turn is the number of lower lanes of its instruction with the same row, and the
+// kernel adds turn by turn.  A workgroup a block, a wavefront 256 positions at a time; turns of 31 and more are
+// stored as 31 (the kernel takes those lanes one at a time, in lane order).
+__global__ __launch_bounds__(kTurnThreads) void StreamTurnsKernel(const BlockMeta *__restrict__ meta,
+                                                                    uint16_t *__restrict__ field)
+{
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    const BlockMeta m = meta[blockIdx.x];
+    constexpr int kStep = kWave * 4;
+    for (int32_t w = m.dBeg + wave * kStep; w < m.dEnd; w += (kTurnThreads / kWave) * kStep) {
+        const int32_t at = w + lane * 4;  // (dBeg and dEnd are multiples of 8: the four positions are inside or outside)
+        const bool inside = at < m.dEnd;
+        Uint2 f = Uint2{kStreamPadRow * 0x10001u, kStreamPadRow * 0x10001u};
+        if (inside) {
+            f = *reinterpret_cast<const Uint2 *>(field + at);
+        }
+        const uint32_t row[4] = {f.x & 0x7ffu, (f.x >> 16) & 0x7ffu, f.y & 0x7ffu, (f.y >> 16) & 0x7ffu};
+        uint32_t turn[4] = {0, 0, 0, 0};
+        for (int other = 0; other < kWave - 1; ++other) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t theirs = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(row[j]), other));
+                turn[j] += (other < lane && theirs == row[j]) ? 1u : 0u;
+            }
+        }
+        if (inside) {
+            uint32_t out[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t t = turn[j] < kStreamMaxRound ? turn[j] : kStreamMaxRound;
+                out[j] = row[j] == kStreamPadRow ? kStreamPadRow : (row[j] | (t << kStreamRoundShift));
+            }
+            *reinterpret_cast<Uint2 *>(field + at) = Uint2{out[0] | (out[1] << 16), out[2] | (out[3] << 16)};
         }
     }
 }
@@ -1653,6 +1746,209 @@ __global__ __launch_bounds__(kThreads, 2 * kThreads / kWave / 4) void SpmvBlockR
     }
 }
 
+// ---- phase 2, streamed --------------------------------------------------------------------------------------
+// A wavefront owns a row block of at most 2^10 rows: the rows' sums sit in its 8 KiB of LDS, and it streams the
+// block's positions of the (block, panel) order, 512 at a time with the next 1024 on their way: value, row field and
+// gathered x (eight positions of a chunk are eight neighbours in panel order, src8 says where).  Nothing is shared
+// between wavefronts and nothing waits for another wavefront: sixteen of them a compute unit hide each other's
+// loads, and the hardware deals the blocks out as wavefronts finish.  The order of the additions to a row's sum is
+// fixed by the layout: instruction by instruction in stream order, and inside an instruction turn by turn
+// (StreamTurnsKernel), so that no two lanes ever add to one sum at once.
+template <typename ValT, typename OutT>
+struct BlockStreamArgs {
+    const uint32_t *xg;
+    const uint16_t *field;
+    const int32_t *src8;
+    const BlockMeta *meta;
+    const ValT *valD;
+    OutT *y;
+    const OutT *yIn;
+    OpsparseScalar alpha, beta;
+    const int32_t *longRows;
+    int32_t B, xgEntries;
+};
+
+template <typename AccT>
+__device__ __forceinline__ void StreamAdd(uint64_t *acc, uint32_t row, AccT t)
+{
+    if constexpr (std::is_same<AccT, uint32_t>::value) {
+        atomicAdd(reinterpret_cast<uint32_t *>(acc + row), t);  // (the low word of the slot)
+    } else {
+        atomicAdd(reinterpret_cast<double *>(acc + row), t);
+    }
+}
+
+template <typename ValT, typename OutT, typename AccT>
+__global__ __launch_bounds__(kStreamThreads) void SpmvBlockStreamKernel(const BlockStreamArgs<ValT, OutT> a)
+{
+    constexpr bool kIntData = std::is_same<ValT, int32_t>::value;
+    constexpr int kSub = kWave * 4, kStep = 2 * kSub;
+    __shared__ __align__(16) uint64_t acc[kStreamRows + kWave];  // (behind the rows: a slot a lane, see below)
+    const int lane = threadIdx.x;
+    // neighbouring blocks read neighbouring pieces of every panel's xg: they go to one XCD, hence one L2
+    const int32_t b = static_cast<int32_t>(XcdContiguousTile(blockIdx.x, gridDim.x));
+    if (b >= a.B) {
+        return;  // (no barrier anywhere below)
+    }
+    const BlockMeta m = a.meta[b];
+    const int32_t nRows = m.nRows < 0 ? 0 : (m.nRows < kStreamRows ? m.nRows : kStreamRows);
+    if (nRows == 0) {
+        return;  // a block number that no row maps to
+    }
+    for (int i = lane; i < kStreamRows; i += kWave) {
+        acc[i] = 0;
+    }
+    for (int32_t l = m.l0 + lane; l < m.l1; l += kWave) {
+        const int32_t r = a.longRows[l] - m.row0;  // summed by phase 1 and SpmvLongRowSumKernel
+        if (r >= 0 && r < nRows) {
+            acc[r] = kJoinMark;
+        }
+    }
+    struct Piece {
+        Uint4 v[2], x[2];
+        Uint2 f[2];
+    };
+    struct Sources {
+        int32_t at[2];
+    };
+    const int32_t dBeg = m.dBeg, dEnd = m.dEnd;
+    // Where the lane's two runs of four positions of the 512 from `start` sit in panel order.  A wavefront issues
+    // its instructions in order: a load whose address waits for another load stalls everything behind it, so these
+    // are asked for well before the loads that need them.  Positions behind the block's last: its last four again.
+    auto sources = [&](int32_t start) {
+        Sources src;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            const int32_t mine = start + s * kSub + lane * 4;
+            const int32_t at = mine < dEnd ? mine : dEnd - 4;  // (a block in the loop has 8 positions at least)
+            // (nothing here or in `fetch` may look at what a load brings: that would wait for it, and for every load
+            // issued before it)
+            src.at[s] = __builtin_nontemporal_load(a.src8 + (at >> 3));
+        }
+        return src;
+    };
+    auto fetch = [&](int32_t start, const Sources &from) {
+        Piece piece;
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            const int32_t mine = start + s * kSub + lane * 4;
+            const int32_t at = mine < dEnd ? mine : dEnd - 4;
+            // (in range whatever the table holds; the four loaded may run past the last entry into the 256 bytes
+            // that xg has behind it: those are padding positions)
+            int32_t src = from.at[s] + (at & 4);
+            src = src < 0 ? 0 : (src < a.xgEntries ? src : a.xgEntries);
+            piece.v[s] = LoadFourRaw(a.valD + at);
+            piece.x[s] = __builtin_nontemporal_load(reinterpret_cast<const Uint4U *>(a.xg + src));
+            piece.f[s] = __builtin_nontemporal_load(reinterpret_cast<const Uint2 *>(a.field + at));
+        }
+        return piece;
+    };
+    auto process = [&](const Piece &cur, int32_t start) {
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+            const uint32_t vr[4] = {cur.v[s].x, cur.v[s].y, cur.v[s].z, cur.v[s].w};
+            const uint32_t xr[4] = {cur.x[s].x, cur.x[s].y, cur.x[s].z, cur.x[s].w};
+            // positions behind the block's last (a lane then holds the block's last four again): padding
+            const bool inside = start + s * kSub + lane * 4 < dEnd;
+            const Uint2 fs = inside ? cur.f[s] : Uint2{kStreamPadRow * 0x10001u, kStreamPadRow * 0x10001u};
+            const uint32_t fl[4] = {fs.x & 0xffffu, fs.x >> 16, fs.y & 0xffffu, fs.y >> 16};
+            uint32_t row[4];
+            AccT t[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                row[j] = fl[j] & 0x7ffu;
+                t[j] = RawToAcc<AccT, kIntData>(vr[j]) * RawToAcc<AccT, kIntData>(xr[j]);
+            }
+            const uint32_t first = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(row[0])));
+            const bool mineSame = row[0] == first && row[1] == first && row[2] == first && row[3] == first;
+            if (first != kStreamPadRow && __all(mineSame)) {
+                // one row fills the 256 positions: its sum across the lanes in a fixed shape, added once
+                AccT sum = (t[0] + t[1]) + (t[2] + t[3]);
+#pragma unroll
+                for (int off = kWave / 2; off > 0; off >>= 1) {
+                    sum += __shfl_xor(sum, off);
+                }
+                if (lane == 0) {
+                    StreamAdd<AccT>(acc, first, sum);
+                }
+                continue;
+            }
+            // The first turns: four instructions; then, where the 256 positions hold a row twice in one instruction
+            // (most do: a row with many entries has some in every chunk), the later turns, and the 31st and later
+            // of a row one lane at a time, in lane order.  A lane whose entry is not on adds to a slot of its own
+            // behind the rows' sums instead (nobody reads it): an address select costs less than switching lanes
+            // off and on again.
+            uint32_t turn[4], latest = 0;
+            const uint32_t idle = kStreamRows + lane;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool valid = row[j] != kStreamPadRow;
+                turn[j] = valid ? fl[j] >> kStreamRoundShift : 0xffffu;  // (padding: no turn)
+                latest = valid && turn[j] > latest ? turn[j] : latest;
+                StreamAdd<AccT>(acc, turn[j] == 0 ? row[j] : idle, t[j]);
+            }
+            if (__any(latest != 0)) {
+#pragma nounroll  // (the kernel's code has to stay inside the instruction cache)
+                for (uint32_t r = 1; r < kStreamMaxRound; ++r) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        StreamAdd<AccT>(acc, turn[j] == r ? row[j] : idle, t[j]);
+                    }
+                    if (!__any(latest > r)) {
+                        break;
+                    }
+                }
+                if (__any(latest == kStreamMaxRound)) {
+#pragma nounroll
+                    for (int j = 0; j < 4; ++j) {
+                        uint64_t late = __ballot(turn[j] == kStreamMaxRound);
+                        while (late != 0) {
+                            const int who = __builtin_ctzll(late);
+                            if (lane == who) {
+                                StreamAdd<AccT>(acc, row[j], t[j]);
+                            }
+                            late &= late - 1;
+                        }
+                    }
+                }
+            }
+        }
+    };
+    if (dBeg < dEnd) {
+        // A wavefront issues in order and its loads come back in order.  Piece n is asked for while piece n - 2 is
+        // added up, its sources while piece n - 4 is (before that slot's own piece, so that waiting for them does not
+        // wait for it): two pieces and two sets of sources are on their way at any time.  Four of each in turn, so
+        // that no register a load fills is ever copied (a copy would wait for the load).  Every load is issued
+        // whether or not its piece exists (past the end: on the block's last positions): with loads inside branches
+        // the compiler can no longer tell which of them a use has to wait for, and waits for all.
+        Sources src0 = sources(dBeg), src1 = sources(dBeg + kStep), src2 = sources(dBeg + 2 * kStep),
+                src3 = sources(dBeg + 3 * kStep);
+        Piece p0 = fetch(dBeg, src0), p1 = fetch(dBeg + kStep, src1), p2, p3;
+#define OPSPARSE_STREAM_SLOT(pNow, pAhead, srcAhead, srcFar)      \
+    srcFar = sources(start + 4 * kStep);                           \
+    pAhead = fetch(start + 2 * kStep, srcAhead);                   \
+    process(pNow, start);                                          \
+    start += kStep;                                                \
+    if (start >= dEnd) {                                           \
+        break;                                                     \
+    }
+        for (int32_t start = dBeg;;) {
+            OPSPARSE_STREAM_SLOT(p0, p2, src2, src0)
+            OPSPARSE_STREAM_SLOT(p1, p3, src3, src1)
+            OPSPARSE_STREAM_SLOT(p2, p0, src0, src2)
+            OPSPARSE_STREAM_SLOT(p3, p1, src1, src3)
+        }
+#undef OPSPARSE_STREAM_SLOT
+    }
+    const AccT alpha = ReadAcc<AccT>(a.alpha), beta = ReadAcc<AccT>(a.beta);
+    for (int32_t i = lane; i < nRows; i += kWave) {
+        const uint64_t slot = acc[i];
+        if (slot != kJoinMark) {
+            StoreOut<OutT, AccT>(a.y, a.yIn, static_cast<int64_t>(m.row0) + i, SlotToAcc<AccT>(slot), alpha, beta);
+        }
+    }
+}
+
 // The long rows of the row blocks that hold more than kInBlockLongRows of them (longDeferred[l] != 0), a wavefront a
 // row: y[row] = alpha * (the row's partial sums, added up as phase 2 does) + beta * yIn[row].
 template <typename OutT, typename AccT>
@@ -1680,6 +1976,9 @@ int32_t ValueBytes(int32_t valueType) { return valueType == OPSPARSE_F16 || valu
 
 struct BlockedLayout {
     int32_t P, B, window, passes;
+    bool streamed;      // row blocks of 2^10 rows that a wavefront streams (values kept in block order), not windowed
+    int32_t rowLog;     // rows of a block at most: 2^rowLog
+    int64_t valDOff;    // streamed: the values in block order
     int64_t padded;     // upper bound of the positions in block order
     // op(A) = A^T: the CSR arrays of A^T (= the CSC arrays of A), and with live values the entry of A behind each
     int64_t cscPtrOff, cscIndOff, cscValOff, permOff;
@@ -1722,6 +2021,30 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     }();
     int64_t window = cutEnv > 0 ? cutEnv : kRowsWindow * 7 / 8;
     window = window > kMaxBlockEntries / 2 ? kMaxBlockEntries / 2 : window;
+    // Values that the layout keeps (frozen values, either op(A)) are kept in block order and streamed by a wavefront
+    // a block; values read where the caller has them need the windowed blocks, which read them in row order.
+    static const bool noStream = std::getenv("OPS_SPARSE_BLOCKED_NO_STREAM") != nullptr;  // tuning switch
+    l.streamed = !live && !noStream;
+    if (l.streamed) {
+        // Streamed blocks are cut by their rows; the entry cut is there for matrices of few, long rows, which would
+        // otherwise make fewer blocks than the chip has wavefronts: about 8192 blocks of 4096 entries at least.
+        const int64_t byRows = rows >> kStreamRowLog;
+        int64_t cut = byRows >= kStreamBlocksWanted / 2 ? kStreamWindow : nnz / (kStreamBlocksWanted - byRows);
+        cut = cut < kStreamMinWindow ? kStreamMinWindow : (cut > kStreamWindow ? kStreamWindow : cut);
+        cut = cutEnv > 0 ? cutEnv : cut;
+        // They pay where a (panel, block) chunk has 16 entries on average (smaller ones are mostly padding, and a
+        // block of 2^10 rows has a quarter of the entries of a windowed one: many panels and few entries a row
+        // are the windowed blocks' case) and where a row does not put more than 16 entries into a panel on
+        // average (such rows meet themselves in every instruction of the stream: 200 000 rows of 300 entries over
+        // 10 panels 326 us streamed, 247 us windowed; over 19 panels 234 against 254).
+        const int64_t blocks = ((rows + kStreamRows - 1) >> kStreamRowLog) + nnz / cut + 1;
+        if (nnz / (P * blocks) < kStreamMinChunkEntries || nnz / rows / P > kStreamMaxRowPanelEntries) {
+            l.streamed = false;
+        } else {
+            window = cut;
+        }
+    }
+    l.rowLog = l.streamed ? kStreamRowLog : kRowBlockLog;
     // The values a launch reads: the caller's own (live values, op(A) = A), the transposed copy (op(A) = A^T), or,
     // for op(A) = A with frozen values, a compact copy without the long rows' values, whose entries are stored a
     // second time with their values.
@@ -1748,11 +2071,12 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
             l.frozenLong = frozenCopy;
         }
     }
-    // a block ends behind 2^12 rows, behind `window` entries and, where the values are read in place, behind a
-    // long row
-    const int64_t B = ((rows + kRowBlockRows - 1) >> kRowBlockLog) + nnz / window + 1 + (l.frozenLong ? 0 : l.maxLong);
+    // a block ends behind 2^rowLog rows, behind `window` entries and, where the values are read in place in row
+    // order, behind a long row
+    const bool cutBehindLong = !l.frozenLong && !l.streamed;
+    const int64_t B = ((rows + (int64_t{1} << l.rowLog) - 1) >> l.rowLog) + nnz / window + 1 + (cutBehindLong ? l.maxLong : 0);
     if (P * B + 1 > INT32_MAX || nnz + kLaneEntries * P * B > INT32_MAX - 65536 ||
-        nnz / (P * (B - (l.frozenLong ? 0 : l.maxLong))) < kMinChunkEntries) {
+        nnz / (P * (B - (cutBehindLong ? l.maxLong : 0))) < kMinChunkEntries) {
         return BlockedLayout{};
     }
     l.P = static_cast<int32_t>(P);
@@ -1781,12 +2105,15 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     l.src8Off = off; off += align(4 * (padded / kLaneEntries + 2));
     l.metaOff = off; off += align(static_cast<int64_t>(sizeof(BlockMeta)) * (B + 1));
     l.panelStartOff = off; off += align(4 * (P + 1));
-    l.rowBitsOff = off; off += align(4 * (nnz / 32 + 8 * B + 16));
-    l.bitPrefixOff = off; off += align(2 * (nnz / 32 + 8 * B + 16));
-    l.ordRowOff = off; off += align(2 * (rows + 16 * B + 32));
-    l.emptyRowsOff = off; off += align(4 * rows);
-    l.shortOffsetsOff = off; off += (l.maxLong > 0 || frozenCopy) ? align(4 * (rows + 1)) : 0;
-    l.valSOff = off; off += frozenCopy ? align(vb * nnz + 16) : 0;
+    // (streamed blocks need no row tables, write the rows without entries themselves and keep their values in
+    // block order)
+    l.rowBitsOff = off; off += l.streamed ? 0 : align(4 * (nnz / 32 + 8 * B + 16));
+    l.bitPrefixOff = off; off += l.streamed ? 0 : align(2 * (nnz / 32 + 8 * B + 16));
+    l.ordRowOff = off; off += l.streamed ? 0 : align(2 * (rows + 16 * B + 32));
+    l.emptyRowsOff = off; off += l.streamed ? 0 : align(4 * rows);
+    l.shortOffsetsOff = off; off += (l.maxLong > 0 || frozenCopy) && !l.streamed ? align(4 * (rows + 1)) : 0;
+    l.valSOff = off; off += frozenCopy && !l.streamed ? align(vb * nnz + 16) : 0;
+    l.valDOff = off; off += l.streamed ? align(vb * padded + 64) : 0;
     l.longRowsOff = off; off += align(4 * static_cast<int64_t>(l.maxLong));
     // in place: first entry of piece (p, l) in the CSR arrays at [p * maxLong + l], p = 0 .. P; stored again: in the
     // sorted order at [p * (maxLong + 1) + l], l = 0 .. L
@@ -1807,7 +2134,10 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     l.blockRowOff = off; off += align(4 * (B + 1));
     l.blockShortOff = off; off += align(4 * (B + 1));
     l.longFirstOff = off; off += l.maxLong > 0 ? align(4 * (B + 1)) : 0;
-    l.emptyFlagsOff = off; off += align(4 * rows);
+    l.emptyFlagsOff = off; off += l.streamed ? 0 : align(4 * rows);
+    if (l.streamed && l.maxLong > 0) {
+        l.shortOffsetsOff = off; off += align(4 * (rows + 1));  // (only the analysis reads them)
+    }
     l.tableOff = off; off += align(4 * RadixTableInts(nnz));
     int64_t scan = ScanScratchInts(RadixTableInts(nnz));
     scan = ScanScratchInts(P * B + 1) > scan ? ScanScratchInts(P * B + 1) : scan;
@@ -1881,6 +2211,9 @@ int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valTy
     if (plan.numEmptyRows < 0 || plan.numEmptyRows > a.rows || plan.numLongRows < 0 || plan.numLongRows > l.maxLong) {
         return OPSPARSE_E_INVALID;
     }
+    if ((plan.streamedBlocks != 0) != l.streamed) {
+        return OPSPARSE_E_INVALID;
+    }
     auto *base = static_cast<unsigned char *>(a.ws);
     auto ints = [&](int64_t off) { return reinterpret_cast<const int32_t *>(base + off); };
     const auto *colLocal = reinterpret_cast<const uint16_t *>(base + l.colLocalOff);
@@ -1895,7 +2228,8 @@ int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valTy
     }
     // the arrays the kernels read the matrix from
     const int32_t *colInd = transposed ? ints(l.cscIndOff) : a.colInd;
-    const void *vals = transposed ? base + l.cscValOff : (frozenCopy ? base + l.valSOff : a.vals);
+    const void *vals = transposed ? base + l.cscValOff : (frozenCopy ? base + l.valSOff : a.vals);  // (windowed blocks,
+                                                                                                    // in-place long rows)
     const bool longRows = plan.numLongRows > 0;
     if (longRows && !l.frozenLong && colInd == nullptr) {
         return OPSPARSE_E_INVALID;
@@ -1926,6 +2260,31 @@ int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valTy
                 gather(std::true_type{});
             } else {
                 gather(std::false_type{});  // (without long rows nothing of the matrix arrays is read)
+            }
+            if (l.streamed) {
+                BlockStreamArgs<ValT, OutT> args{};
+                args.xg = xg;
+                args.field = slot16;
+                args.src8 = ints(l.src8Off);
+                args.meta = reinterpret_cast<const BlockMeta *>(base + l.metaOff);
+                args.valD = reinterpret_cast<const ValT *>(base + l.valDOff);
+                args.y = static_cast<OutT *>(a.y);
+                args.yIn = static_cast<const OutT *>(a.yIn);
+                args.alpha = a.alpha;
+                args.beta = a.beta;
+                args.longRows = ints(l.longRowsOff);
+                args.B = l.B;
+                args.xgEntries = static_cast<int32_t>(a.nnz);
+                hipLaunchKernelGGL((SpmvBlockStreamKernel<ValT, OutT, AccT>), dim3(static_cast<uint32_t>(l.B)),
+                                   dim3(kStreamThreads), 0, a.stream, args);
+                if (longRows) {  // (every long row is left to this kernel)
+                    constexpr int kRowsPerBlock = kBlockThreads / kWave;
+                    hipLaunchKernelGGL((SpmvLongRowSumKernel<OutT, AccT>),
+                                       dim3((plan.numLongRows + kRowsPerBlock - 1) / kRowsPerBlock), dim3(kBlockThreads),
+                                       0, a.stream, header, ints(l.longRowsOff), ints(l.longDeferredOff), longPartial,
+                                       l.P, static_cast<OutT *>(a.y), static_cast<const OutT *>(a.yIn), a.alpha, a.beta);
+                }
+                return CheckLaunch();
             }
             BlockRowsArgs<ValT, OutT> args{};
             args.xg = xg;
@@ -2062,8 +2421,8 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     auto *slot16 = reinterpret_cast<uint16_t *>(base + l.slotOff);
 
     LaunchExpandRows(rowOffsets, outputs, nnz, 0, rowOfPos, s);
-    {
-        // the rows without entries, which the row blocks do not see
+    if (!l.streamed) {
+        // the rows without entries, which the windowed row blocks do not see
         int32_t *flags = ints(l.emptyFlagsOff);
         hipLaunchKernelGGL(EmptyRowFlagsKernel, dim3(GridOf(outputs, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
                            rowOffsets, outputs, flags);
@@ -2093,7 +2452,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
         hipLaunchKernelGGL(ShortOffsetsKernel, dim3(GridOf(outputs + 1, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
                            rowOffsets, outputs, shortOffsets);
         offsets = shortOffsets;  // the row blocks are cut by the entries that stay
-    } else if (frozenCopy) {
+    } else if (frozenCopy && !l.streamed) {
         // (a plan with frozen values reads nothing of the caller's arrays at the launches)
         if (hipMemcpyAsync(ints(l.shortOffsetsOff), rowOffsets, sizeof(int32_t) * static_cast<size_t>(outputs + 1),
                            hipMemcpyDeviceToDevice, s) != hipSuccess) {
@@ -2103,7 +2462,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
         offsets = ints(l.shortOffsetsOff);
     }
     // where the values are read in place a long row ends its block, so that a block's other entries are one piece
-    const int32_t *cutBehind = (longBefore != nullptr && !l.frozenLong) ? longBefore : nullptr;
+    const int32_t *cutBehind = (longBefore != nullptr && !l.frozenLong && !l.streamed) ? longBefore : nullptr;
     // Entries in (panel, original position) order: stable 4-bit radix passes over the panel number.
     const int32_t *firstKeys = colInd;
     if (longBefore != nullptr) {
@@ -2123,7 +2482,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     int32_t *chunkKey = keys[1 - cur], *rowOfSrc = poss[1 - cur];
     hipLaunchKernelGGL(BlockedChunkKeysKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
                        keys[cur], pos, rowOfPos, offsets, nnz, inputs, l.B, l.window, longBefore,
-                       cutBehind != nullptr ? 1 : 0, colLocal, chunkKey, rowOfSrc, status);
+                       cutBehind != nullptr ? 1 : 0, l.rowLog, colLocal, chunkKey, rowOfSrc, status);
     if (longBefore != nullptr && l.frozenLong) {
         hipLaunchKernelGGL(LongRowPanelsKernel, dim3(GridOf(l.P, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
                            keys[cur], nnz, l.P, l.maxLong, static_cast<int32_t>(l.P) << kPanelLog, ints(l.longChunkOff));
@@ -2145,28 +2504,44 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     hipLaunchKernelGGL(BlockedTablesKernel, dim3(GridOf(chunks, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
                        srcStart, l.P, l.B, dstStart);
     LaunchInclusiveScanI32(dstStart + 1, dstStart + 1, chunks, 0, scratch, s);
-    // padding positions: the slot kPadSlot
-    LaunchFillI32(reinterpret_cast<int32_t *>(slot16), (l.padded + 1) / 2, static_cast<int32_t>(kPadSlot * 0x10001u), s);
+    // padding positions: the slot kPadSlot, or the row field kStreamPadRow
+    LaunchFillI32(reinterpret_cast<int32_t *>(slot16), (l.padded + 1) / 2,
+                  static_cast<int32_t>((l.streamed ? kStreamPadRow : kPadSlot) * 0x10001u), s);
     LaunchFillI32(blockRow, l.B + 1, static_cast<int32_t>(outputs), s);
     hipLaunchKernelGGL(BlockedRowBlocksKernel, dim3(GridOf(outputs, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
-                       offsets, static_cast<int32_t>(outputs), l.window, l.B, cutBehind, blockRow);
+                       offsets, static_cast<int32_t>(outputs), l.window, l.B, cutBehind, l.rowLog, blockRow);
     if (longBefore != nullptr) {
         hipLaunchKernelGGL(BlockedLongFirstKernel, dim3(GridOf(l.B + 1, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
                            s, blockRow, longBefore, l.B, ints(l.longFirstOff));
         hipLaunchKernelGGL(BlockedLongDeferKernel, dim3(GridOf(l.B, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0, s,
-                           ints(l.longFirstOff), l.B, ints(l.longDeferredOff), status);
+                           ints(l.longFirstOff), l.B, l.streamed ? 1 : 0, ints(l.longDeferredOff), status);
     }
     const int64_t tableItems = (l.B > l.P ? l.B : l.P) + 1;
     hipLaunchKernelGGL(BlockedBlockTablesKernel, dim3(GridOf(tableItems, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
-                       s, offsets, frozenCopy ? offsets : rowOffsets, blockRow, dstStart, srcStart,
+                       s, offsets, frozenCopy || l.streamed ? offsets : rowOffsets, blockRow, dstStart, srcStart,
                        longBefore != nullptr ? ints(l.longFirstOff) : nullptr, l.P, l.B, ints(l.blockShortOff),
                        reinterpret_cast<BlockMeta *>(base + l.metaOff), ints(l.panelStartOff), status);
-    hipLaunchKernelGGL(BlockedRowTablesKernel, dim3(static_cast<uint32_t>(l.B)), dim3(kTableThreads), 0, s,
-                       reinterpret_cast<const BlockMeta *>(base + l.metaOff), offsets,
-                       reinterpret_cast<uint32_t *>(base + l.rowBitsOff), reinterpret_cast<uint16_t *>(base + l.bitPrefixOff),
-                       reinterpret_cast<uint16_t *>(base + l.ordRowOff));
+    if (!l.streamed) {
+        hipLaunchKernelGGL(BlockedRowTablesKernel, dim3(static_cast<uint32_t>(l.B)), dim3(kTableThreads), 0, s,
+                           reinterpret_cast<const BlockMeta *>(base + l.metaOff), offsets,
+                           reinterpret_cast<uint32_t *>(base + l.rowBitsOff),
+                           reinterpret_cast<uint16_t *>(base + l.bitPrefixOff),
+                           reinterpret_cast<uint16_t *>(base + l.ordRowOff));
+    }
     const int rcScatter = WithValueType(valueType, [&](auto tag) {
         using ValT = decltype(tag);
+        if (l.streamed) {
+            hipLaunchKernelGGL(StreamScatterKernel<ValT>, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0,
+                               s, pos, rowOfSrc, chunkKey, static_cast<const ValT *>(csrValues), srcStart, dstStart,
+                               blockRow, nnz, l.P, l.B, slot16, ints(l.src8Off),
+                               reinterpret_cast<ValT *>(base + l.valDOff), static_cast<int32_t *>(nullptr),
+                               longBefore != nullptr && l.frozenLong ? reinterpret_cast<uint32_t *>(base + l.xgOff)
+                                                                     : nullptr,
+                               slot16 + LongRowOfShift(l), longBefore);
+            hipLaunchKernelGGL(StreamTurnsKernel, dim3(static_cast<uint32_t>(l.B)), dim3(kTurnThreads), 0, s,
+                               reinterpret_cast<const BlockMeta *>(base + l.metaOff), slot16);
+            return OPSPARSE_OK;
+        }
         hipLaunchKernelGGL(BlockedScatterKernel<ValT>, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
                            pos, rowOfSrc, chunkKey, static_cast<const ValT *>(csrValues), rowOffsets, offsets, srcStart,
                            dstStart, ints(l.blockShortOff), nnz, l.P, l.B, slot16, ints(l.src8Off),
@@ -2187,7 +2562,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     if (CheckLaunch() != OPSPARSE_OK) {
         return OPSPARSE_E_LAUNCH;
     }
-    if (tail[0] > kMaxBlockEntries) {
+    if (!l.streamed && tail[0] > kMaxBlockEntries) {
         return OPSPARSE_E_UNSUPPORTED;  // a row too long for a block's 16-bit slots that cannot go the long rows' way
     }
     OpsparseSpmvPlan p{};
@@ -2201,6 +2576,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     p.valueType = valueType;
     p.numDeferredLongRows = tail[1];
     p.numEmptyRows = tail[2];
+    p.streamedBlocks = l.streamed ? 1 : 0;
     p.numLongRows = head[1];
     p.rows = rows;
     p.nnz = nnz;
