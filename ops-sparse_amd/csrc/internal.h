@@ -149,6 +149,8 @@ OpsparseScalar MakeScalar(const void *p, aclDataType computeType, aclsparsePoint
 // re-stored layout to pay: with the values frozen, and with live values.
 constexpr int32_t kScatteredForFrozenLayout = 190;
 constexpr int32_t kScatteredForLiveLayout = 310;
+// Columns from which the ordered layout with live values (repeatable sums) is taken for op(A) = A.
+constexpr int64_t kMinColsOrderedLive = int64_t{5} << 19;  // 2.6 M
 
 struct RestoredChoice {
     int32_t kernel;

@@ -269,6 +269,15 @@ RestoredChoice PickLiveLayout(aclsparseHandle_t handle, const int32_t *rowOffset
     if (bytes == 0) {
         return {0, 0, false};
     }
+    // The ordered layout reads the values through a window in LDS and is about half again as slow as the one with
+    // atomics: against the row-wise kernels on the caller's arrays it only wins where x is out of reach of the
+    // caches (x of 3 M elements: 363 us against 447 for 3 M rows of 12, 177 against 392 for 4000 rows of 8000; x of
+    // 2.2 M: 112 against 87 for 2 M rows of 4; x of 1 M and less: slower throughout).  (op(A) = A^T replaces atomics
+    // on y and keeps the bounds of AnalyseRestored.)
+    const char *minColsEnv = std::getenv("OPS_SPARSE_ORDERED_LIVE_MIN_COLS");  // tuning override, read at every call
+    if (!atomics && !transpose && cols < (minColsEnv != nullptr ? std::atoll(minColsEnv) : kMinColsOrderedLive)) {
+        return {0, 0, false};
+    }
     // scattered gathers (op(A) = A^T: scattered updates of y)?  Not under stream capture (nothing may synchronise there) and not without a workspace.
     hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(handle->stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {

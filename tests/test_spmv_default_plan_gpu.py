@@ -24,6 +24,7 @@ def _layout_for_small_matrices(monkeypatch):
     """The default plan takes the layout from 7 M entries on; the matrices here have 2.5 - 4 M so that the fp64
     oracle stays quick.  The override is read at every GetBufferSize / Preprocess."""
     monkeypatch.setenv("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ", "0")
+    monkeypatch.setenv("OPS_SPARSE_ORDERED_LIVE_MIN_COLS", "0")   # (the ordered live layout: from 2.6 M columns)
 
 
 def _default_bytes(osa, rows, cols, nnz, repeatable):
@@ -728,3 +729,29 @@ def test_atomics_layout_with_32_bit_positions(osa, gpu_ctx, how, monkeypatch):
         stream.synchronize()
         gold = oracle.spmv_f64(rows, cols, rowptr, colind, values, x, y0, alpha, beta)
         assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+
+def test_ordered_live_layout_only_where_x_is_out_of_reach_of_the_caches(osa, gpu_ctx, monkeypatch):
+    """The layout with live values and ordered sums (aclsparseSpMVOp DEFAULT / ALG1, and the default algorithm asked
+    for repeatable sums) is slower than the one with atomics; against the row-wise kernels it pays from 2.6 M
+    columns on.  Below that aclsparseSpMVOp_bufferSize answers 0 for these algorithms, as the reference does."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = 320_000, 1_500_000
+    rowptr, colind, val, x, y0 = _scattered(rows, cols, 5)
+    d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+    A = osa.Csr(rows, cols, d[0], d[1], d[2])
+    d_y = to_dev(y0, dev)
+    Y = osa.DnVec(d_y)
+    monkeypatch.delenv("OPS_SPARSE_ORDERED_LIVE_MIN_COLS")
+    op = osa.SpmvOpPlan(handle, A, osa.DnVec(d[3]), Y, Y)
+    assert op.buffer_bytes == 0
+    op(1.0, 0.5)
+    stream.synchronize()
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.0, 0.5)
+    assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+    monkeypatch.setenv("OPS_SPARSE_SPMV_REPEATABLE", "1")
+    plain = L.opsparse_spmv_csr_workspace_bytes(rows, colind.size)
+    assert osa.SpmvOp(handle, A, osa.DnVec(d[3]), Y).buffer.numel() == plain
+    monkeypatch.setenv("OPS_SPARSE_ORDERED_LIVE_MIN_COLS", str(cols))
+    assert osa.SpmvOp(handle, A, osa.DnVec(d[3]), Y).buffer.numel() > plain

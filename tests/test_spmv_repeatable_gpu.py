@@ -26,6 +26,7 @@ RUNS = 6
 @pytest.fixture(autouse=True)
 def _layout_for_small_matrices(monkeypatch):
     monkeypatch.setenv("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ", "0")
+    monkeypatch.setenv("OPS_SPARSE_ORDERED_LIVE_MIN_COLS", "0")   # (the ordered live layout: from 2.6 M columns)
 
 
 def _cancelling(seed):
