@@ -19,11 +19,22 @@
 #include <stddef.h>
 #include <stdint.h>
 
+/* The enums of this ABI are passed by value and checked by the callee: a caller may hand over any int.  C++ leaves a
+ * value outside an enum's enumerators undefined unless the enum has a fixed underlying type, so under C++ they get
+ * one (int, what they are in C anyway: neither size nor calling convention changes). */
+#ifndef OPSPARSE_ABI_ENUM
+#ifdef __cplusplus
+#define OPSPARSE_ABI_ENUM(name) enum name : int
+#else
+#define OPSPARSE_ABI_ENUM(name) enum name
+#endif
+#endif
+
 #ifdef __cplusplus
 extern "C" {
 #endif
 
-typedef enum {
+typedef OPSPARSE_ABI_ENUM(aclDataType) {
     ACL_DT_UNDEFINED = -1,
     ACL_FLOAT = 0,
     ACL_FLOAT16 = 1,

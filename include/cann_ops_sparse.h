@@ -32,20 +32,20 @@ extern "C" {
 /* ------------------------------------------------------------------ enums */
 
 /* [ref: include/cann_ops_sparse.h:24-28] operation applied to an operand. */
-typedef enum aclsparseOperation_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseOperation_t) {
     ACL_SPARSE_OP_NON_TRANSPOSE = 0,
     ACL_SPARSE_OP_TRANSPOSE,
     ACL_SPARSE_OP_CONJUGATE_TRANSPOSE
 } aclsparseOperation_t;
 
 /* [ref: :50-53] storage order of a dense matrix (B and C of SpMM). */
-typedef enum aclsparseOrder_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseOrder_t) {
     ACL_SPARSE_ORDER_ROW = 0,
     ACL_SPARSE_ORDER_COL = 1
 } aclsparseOrder_t;
 
 /* [ref: :56-70] algorithm selector of the SpMVOp API. */
-typedef enum aclsparseSpMVOpAlg_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseSpMVOpAlg_t) {
     ACL_SPARSE_SPMVOP_ALG_DEFAULT = 0,
     ACL_SPARSE_SPMVOP_ALG1,
     ACL_SPARSE_SPMVOP_ALG2
@@ -55,14 +55,14 @@ typedef enum aclsparseSpMVOpAlg_t {
  * kernels.  The reference's third value selects Kahan-compensated fp32
  * accumulation; here every floating-point SpMM kernel already accumulates in
  * fp64 and rounds once, so the three values give identical results. */
-typedef enum aclsparseSpMMAlg_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseSpMMAlg_t) {
     ACL_SPARSE_SPMM_ALG_DEFAULT = 0,
     ACL_SPARSE_SPMM_CSR_ALG1,
     ACL_SPARSE_SPMM_CSR_FP32_HIGH_PRECISION_ALG
 } aclsparseSpMMAlg_t;
 
 /* [ref: :98-148] status codes. */
-typedef enum aclsparseStatus_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseStatus_t) {
     ACL_SPARSE_STATUS_SUCCESS = 0,
     ACL_SPARSE_STATUS_NOT_INITIALIZED,
     ACL_SPARSE_STATUS_ALLOC_FAILED,
@@ -78,7 +78,7 @@ typedef enum aclsparseStatus_t {
 
 /* [ref: :150-168] SpMV algorithm selector; only ALG_DEFAULT is accepted by
  * aclsparseSpMV, as in the reference (sparse/spmv/arch22/spmv_host.cpp:144). */
-typedef enum aclsparseSpMVAlg_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseSpMVAlg_t) {
     ACL_SPARSE_SPMV_ALG_DEFAULT,
     ACL_SPARSE_SPMV_COO_ALG1,
     ACL_SPARSE_SPMV_COO_ALG2,
@@ -88,13 +88,13 @@ typedef enum aclsparseSpMVAlg_t {
 } aclsparseSpMVAlg_t;
 
 /* [ref: :213-222] width of row offsets / column indices. */
-typedef enum aclsparseIndexType_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseIndexType_t) {
     ACL_SPARSE_INDEX_32I = 0,
     ACL_SPARSE_INDEX_64I
 } aclsparseIndexType_t;
 
 /* [ref: :229-232] */
-typedef enum aclsparseIndexBase_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseIndexBase_t) {
     ACL_SPARSE_INDEX_BASE_ZERO = 0,
     ACL_SPARSE_INDEX_BASE_ONE
 } aclsparseIndexBase_t;
@@ -102,7 +102,7 @@ typedef enum aclsparseIndexBase_t {
 /* [ref: :235-248] sparse storage format tag; only CSR descriptors can be
  * created through this library, the other tags exist so that
  * aclsparseSpMatGetFormat has the reference's value space. */
-typedef enum aclsparseFormat_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseFormat_t) {
     ACL_SPARSE_FORMAT_COO = 0,
     ACL_SPARSE_FORMAT_CSR,
     ACL_SPARSE_FORMAT_CSC,
@@ -112,36 +112,36 @@ typedef enum aclsparseFormat_t {
 } aclsparseFormat_t;
 
 /* [ref: :898-901] where alpha / beta live. */
-typedef enum aclsparsePointerMode_t {
+typedef OPSPARSE_ABI_ENUM(aclsparsePointerMode_t) {
     ACL_SPARSE_POINTER_MODE_HOST = 0,
     ACL_SPARSE_POINTER_MODE_DEVICE = 1
 } aclsparsePointerMode_t;
 
 /* [ref: :192-210] attributes of the legacy matrix descriptor. */
-typedef enum aclsparseMatrixType_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseMatrixType_t) {
     ACL_SPARSE_MATRIX_TYPE_GENERAL = 0,
     ACL_SPARSE_MATRIX_TYPE_SYMMETRIC,
     ACL_SPARSE_MATRIX_TYPE_HERMITIAN,
     ACL_SPARSE_MATRIX_TYPE_TRIANGULAR
 } aclsparseMatrixType_t;
 
-typedef enum aclsparseDiagType_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseDiagType_t) {
     ACL_SPARSE_DIAG_TYPE_NON_UNIT = 0,
     ACL_SPARSE_DIAG_TYPE_UNIT
 } aclsparseDiagType_t;
 
-typedef enum aclsparseFillMode_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseFillMode_t) {
     ACL_SPARSE_FILL_MODE_LOWER = 0,
     ACL_SPARSE_FILL_MODE_UPPER
 } aclsparseFillMode_t;
 
 /* [ref: :1369-1379] CSR -> CSC: structure only, or structure and values; algorithm tag. */
-typedef enum aclsparseAction_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseAction_t) {
     ACL_SPARSE_ACTION_SYMBOLIC = 0,
     ACL_SPARSE_ACTION_NUMERIC
 } aclsparseAction_t;
 
-typedef enum aclsparseCsr2CscAlg_t {
+typedef OPSPARSE_ABI_ENUM(aclsparseCsr2CscAlg_t) {
     ACL_SPARSE_CSR2CSC_ALG_DEFAULT = 0,
     ACL_SPARSE_CSR2CSC_ALG1
 } aclsparseCsr2CscAlg_t;

@@ -22,6 +22,17 @@
 #include <stddef.h>
 #include <stdint.h>
 
+/* The enums of this ABI are passed by value and checked by the callee: a caller may hand over any int.  C++ leaves a
+ * value outside an enum's enumerators undefined unless the enum has a fixed underlying type, so under C++ they get
+ * one (int, what they are in C anyway: neither size nor calling convention changes). */
+#ifndef OPSPARSE_ABI_ENUM
+#ifdef __cplusplus
+#define OPSPARSE_ABI_ENUM(name) enum name : int
+#else
+#define OPSPARSE_ABI_ENUM(name) enum name
+#endif
+#endif
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -33,7 +44,7 @@ extern "C" {
 #define OPSPARSE_E_LAUNCH (-4)      /* the HIP runtime reported an error */
 
 /* Element types of device arrays. */
-typedef enum OpsparseDtype {
+typedef OPSPARSE_ABI_ENUM(OpsparseDtype) {
     OPSPARSE_F32 = 0,
     OPSPARSE_F16 = 1,
     OPSPARSE_BF16 = 2,
@@ -53,7 +64,7 @@ typedef struct OpsparseScalar {
 /* ------------------------------------------------------------------ SpMV */
 
 /* Kernel families of the row-length-binned SpMV dispatcher. */
-typedef enum OpsparseSpmvKernel {
+typedef OPSPARSE_ABI_ENUM(OpsparseSpmvKernel) {
     OPSPARSE_SPMV_AUTO = 0,        /* let the library pick from the statistics */
     OPSPARSE_SPMV_SCALE_ONLY = 1,  /* nnz == 0: y = beta * y */
     OPSPARSE_SPMV_STREAM_ROWS = 2, /* short rows: fixed row blocks, products staged in LDS,
@@ -273,7 +284,7 @@ int opsparse_spmv_csr_indexed_launch(const void *rowOffsets, int32_t rowOffsetsA
 
 /* ------------------------------------------------------------------ SpMM */
 
-typedef enum OpsparseSpmmKernel {
+typedef OPSPARSE_ABI_ENUM(OpsparseSpmmKernel) {
     OPSPARSE_SPMM_AUTO = 0,
     OPSPARSE_SPMM_ROW_SPLIT = 1, /* no row above the long-row threshold: every row whole by one lane group */
     OPSPARSE_SPMM_BINNED = 2     /* rows up to the long-row threshold as ROW_SPLIT, longer rows cut into

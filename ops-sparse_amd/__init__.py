@@ -144,10 +144,12 @@ def lib():
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(LIB_PATH):
+    # (OPS_SPARSE_LIBRARY: another build of the same library, e.g. the one `build.py --asan` makes)
+    path = os.environ.get("OPS_SPARSE_LIBRARY") or LIB_PATH
+    if not os.path.exists(path):
         raise RuntimeError(
-            "libops_sparse.so is not built (%s missing); run `python ops-sparse_amd/build.py`" % LIB_PATH)
-    L = ctypes.CDLL(LIB_PATH)
+            "libops_sparse.so is not built (%s missing); run `python ops-sparse_amd/build.py`" % path)
+    L = ctypes.CDLL(path)
     for name in ACLSPARSE_SYMBOLS:
         getattr(L, name).restype = None if name.startswith("aclsparseSetMat") else ctypes.c_int
     PV = ctypes.POINTER(vp)

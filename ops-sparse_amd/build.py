@@ -3,6 +3,7 @@
 hipcc cross-compiles without a GPU, so this runs anywhere ROCm is installed:
 
     python ops-sparse_amd/build.py
+    python ops-sparse_amd/build.py --asan     # host code under ASan / UBSan, then the CPU tests under it
 
 Every translation unit is compiled to an object under ops-sparse_amd/build/
 (in parallel) and linked into one shared library.  The library carries both
@@ -87,5 +88,92 @@ def build_library(verbose=True):
     return LIB_PATH
 
 
+# ---- host code under AddressSanitizer / UndefinedBehaviorSanitizer -------------------------------------------------
+# `python ops-sparse_amd/build.py --asan` builds a second copy of the library, of the CPU checker and of the C++
+# frame's self-test with the HOST code instrumented (device code is compiled as always: no sanitizer runs on the
+# GPU), and runs the tests that need no GPU under it: the status / argument tests of the C ABI, the checker's own
+# tests, the frame's self-test.  Python itself is not instrumented, so the sanitizer runtime is preloaded.
+ASAN_LIB_DIR = os.path.join(LIB_DIR, "asan")
+ASAN_HOST = ["-Xarch_host", "-fsanitize=address", "-Xarch_host", "-fsanitize=undefined", "-Xarch_host",
+             "-fno-omit-frame-pointer", "-g"]
+
+
+def _clang_dir():
+    out = subprocess.run([hipcc(), "-print-resource-dir"], capture_output=True, text=True).stdout.strip()
+    if not out:
+        out = subprocess.run([hipcc(), "--print-resource-dir"], capture_output=True, text=True).stdout.strip()
+    return out
+
+
+def asan_runtime():
+    path = os.path.join(_clang_dir(), "lib", "linux", "libclang_rt.asan-x86_64.so")
+    if not os.path.exists(path):
+        raise RuntimeError("the sanitizer runtime %s is missing" % path)
+    return path
+
+
+def build_asan(verbose=True):
+    obj_dir = OBJ_DIR + "_asan"
+    os.makedirs(obj_dir, exist_ok=True)
+    os.makedirs(ASAN_LIB_DIR, exist_ok=True)
+    flags = [f if f != "-O3" else "-O1" for f in COMMON_FLAGS] + ASAN_HOST
+
+    def compile_one(src):
+        obj = os.path.join(obj_dir, os.path.splitext(src)[0] + ".o")
+        proc = subprocess.run([hipcc(), "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj] + flags,
+                              capture_output=True, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError("hipcc failed for %s:\n%s" % (src, proc.stderr))
+        return obj
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+        objs = list(pool.map(compile_one, SOURCES))
+    lib = os.path.join(ASAN_LIB_DIR, "libops_sparse.so")
+    link = [hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-fsanitize=address", "-fsanitize=undefined",
+            "-shared-libsan", "-o", lib] + objs
+    proc = subprocess.run(link, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("link failed:\n" + proc.stderr)
+    clang = os.path.join(_clang_dir().rstrip("/").rsplit("/lib/clang", 1)[0], "bin", "clang")  # (the hipcc's own)
+    oracle_lib = os.path.join(ASAN_LIB_DIR, "liboracle.so")
+    proc = subprocess.run([clang, "-O1", "-g", "-std=c99", "-fPIC", "-shared", "-ffp-contract=off", "-fopenmp",
+                           "-fsanitize=address", "-fsanitize=undefined", "-fno-sanitize-recover=undefined",
+                           "-shared-libsan", "-fno-omit-frame-pointer", "-o", oracle_lib,
+                           os.path.join(ROOT, "oracle", "oracle.c"), "-lm"], capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("the checker failed to build under the sanitizers:\n" + proc.stderr)
+    selftest = os.path.join(ASAN_LIB_DIR, "frame_selftest")
+    proc = subprocess.run([hipcc(), "-std=c++17", "-O1", "-g", "-fsanitize=address", "-fsanitize=undefined",
+                           "-fno-sanitize-recover=undefined", "-shared-libsan", "-I" + os.path.join(ROOT, "include"),
+                           "-I" + os.path.join(ROOT, "tests", "cpp"),
+                           os.path.join(ROOT, "tests", "cpp", "frame_selftest.cpp"), "-o", selftest,
+                           "-L" + ASAN_LIB_DIR, "-lops_sparse", "-loracle", "-Wl,-rpath," + ASAN_LIB_DIR,
+                           "-Wl,-rpath," + os.path.dirname(asan_runtime())], capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("the frame's self-test failed to build under the sanitizers:\n" + proc.stderr)
+    if verbose:
+        print("built", lib, oracle_lib, selftest)
+    return lib, oracle_lib, selftest
+
+
+def run_asan():
+    """The CPU tests with the instrumented libraries in place of the ordinary ones; returns the exit status."""
+    lib, oracle_lib, selftest = build_asan()
+    env = dict(os.environ)
+    env["OPS_SPARSE_LIBRARY"] = lib
+    env["OPS_SPARSE_ORACLE_LIBRARY"] = oracle_lib
+    env["LD_PRELOAD"] = asan_runtime() + (":" + env["LD_PRELOAD"] if env.get("LD_PRELOAD") else "")
+    # (CPython and numpy keep their arenas until exit: no leak report; another preloaded library may come first)
+    env["ASAN_OPTIONS"] = "detect_leaks=0:verify_asan_link_order=0:abort_on_error=1"
+    env["UBSAN_OPTIONS"] = "print_stacktrace=0:halt_on_error=0"
+    tests = [os.path.join(ROOT, "tests", t) for t in ("test_abi_status.py", "test_oracle.py", "test_oracle_convert.py")]
+    rc = subprocess.run([sys.executable, "-m", "pytest", "-x", "-q", "-m", "not gpu"] + tests, env=env, cwd=ROOT).returncode
+    if rc == 0:
+        rc = subprocess.run([selftest, os.path.join(ROOT, "tests", "golden")], env=env).returncode
+    return rc
+
+
 if __name__ == "__main__":
+    if "--asan" in sys.argv[1:]:
+        sys.exit(run_asan())
     build_library()

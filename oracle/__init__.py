@@ -38,9 +38,12 @@ def build(force=False):
 def lib():
     global _lib
     if _lib is None:
-        if not os.path.exists(_LIB_PATH):
-            build()
-        _lib = ctypes.CDLL(_LIB_PATH)
+        path = os.environ.get("OPS_SPARSE_ORACLE_LIBRARY")  # (another build of the checker: build.py --asan)
+        if not path:
+            if not os.path.exists(_LIB_PATH):
+                build()
+            path = _LIB_PATH
+        _lib = ctypes.CDLL(path)
         _lib.oracle_fill_csr.restype = c_i64
         _lib.oracle_fnv1a.restype = ctypes.c_uint64
         _lib.oracle_f32_to_f16.restype = ctypes.c_uint16

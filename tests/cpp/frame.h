@@ -39,6 +39,7 @@ void oracle_csr2csc(int64_t m, int64_t n, int64_t nnz, int32_t base, const int32
 void oracle_csrsort(const int32_t *rowPtr, int64_t m, int32_t base, int32_t *colInd, int32_t *perm);
 void oracle_cscsort(const int32_t *colPtr, int64_t n, int32_t base, int32_t *rowInd, int32_t *perm);
 void oracle_coosort(int64_t nnz, int32_t byRow, int32_t *rows, int32_t *cols, int32_t *perm);
+uint64_t oracle_fnv1a(const void *data, int64_t bytes);
 }
 
 namespace frame {
@@ -272,49 +273,52 @@ struct CsrHost {
     int64_t nnz() const { return static_cast<int64_t>(colind.size()); }
 };
 
-// Seeded CSR: Binomial(cols, 1 - sparsity) entries per row (0 with probability emptyRowProb), distinct
-// sorted columns, values uniform in [lo, hi).  Same distribution as the reference generator, own stream.
-inline CsrHost RandomCsr(int64_t rows, int64_t cols, double sparsity, double emptyRowProb, uint32_t seed, float lo,
-                         float hi)
+// The reference's seeded matrices (SparseFillGenerator(seed) with setSparsity / setEmptyRowProb / setValueRange, then
+// generateCsr(rows, cols, nnzHint): reference test/frame/fill.h:55-111), bit for bit — the same engine, the same
+// distributions of the same standard library, drawn from in the same order: per row one uniform float against the
+// empty-row probability (only when that is above 0), the row length (Binomial(cols, 1 - sparsity), or nnzHint /
+// rows when a hint is given, capped at cols), then columns until that many distinct ones are found or four times
+// as many were drawn, and, after sorting, one value per entry.  frame_selftest holds it against fingerprints of
+// the reference's own output (tests/golden/fill_generator.json).
+inline CsrHost FillCsr(int64_t rows, int64_t cols, double sparsity, double emptyRowProb, uint32_t seed, float lo, float hi,
+                       int64_t nnzHint = -1)
 {
     CsrHost a;
     a.rows = rows;
     a.cols = cols;
-    a.rowptr.assign(static_cast<size_t>(rows) + 1, 0);
-    std::mt19937 rng(seed);
-    std::binomial_distribution<int64_t> len(cols, 1.0 - sparsity);
-    std::uniform_real_distribution<double> u01(0.0, 1.0);
-    std::uniform_real_distribution<float> uv(lo, hi);
-    std::vector<int32_t> stamp(static_cast<size_t>(cols), -1);
+    a.rowptr.assign(static_cast<size_t>(rows > 0 ? rows : 0) + 1, 0);
+    if (rows <= 0 || cols <= 0) {
+        return a;
+    }
+    std::mt19937 engine(seed);
+    std::uniform_real_distribution<float> chance(0.0f, 1.0f), value(lo, hi);
+    // (one object for all rows: it keeps a spare normal deviate between draws)
+    std::binomial_distribution<int> length(static_cast<int>(cols), 1.0 - std::min(std::max(sparsity, 0.0), 1.0));
+    const float skip = static_cast<float>(std::min(std::max(emptyRowProb, 0.0), 1.0));
+    std::vector<int> seenInRow(static_cast<size_t>(cols), -1);
+    std::vector<int32_t> picked;
     for (int64_t r = 0; r < rows; ++r) {
-        int64_t l = (cols > 0 && sparsity < 1.0) ? len(rng) : 0;
-        if (emptyRowProb > 0.0 && u01(rng) < emptyRowProb) {
-            l = 0;
+        a.rowptr[r] = static_cast<int32_t>(a.colind.size());
+        if (skip > 0.0f && chance(engine) < skip) {
+            continue;
         }
-        std::vector<int32_t> picked;
-        if (l * 2 > cols) {  // dense row: keep each column with probability l / cols, then trim / top up
-            for (int32_t c = 0; c < cols && static_cast<int64_t>(picked.size()) < l; ++c) {
-                if (cols - c <= l - static_cast<int64_t>(picked.size()) || u01(rng) * cols < l) {
-                    picked.push_back(c);
-                }
+        int want = nnzHint > 0 ? static_cast<int>(nnzHint / std::max<int64_t>(rows, 1)) : length(engine);
+        want = std::min(want, static_cast<int>(cols));
+        picked.clear();
+        for (int draws = 0; want > 0 && static_cast<int>(picked.size()) < want && draws < 4 * want; ++draws) {
+            const int32_t c = std::uniform_int_distribution<int32_t>(0, static_cast<int32_t>(cols) - 1)(engine);
+            if (seenInRow[c] != static_cast<int>(r)) {
+                seenInRow[c] = static_cast<int>(r);
+                picked.push_back(c);
             }
-        } else {
-            std::uniform_int_distribution<int32_t> uc(0, static_cast<int32_t>(cols) - 1);
-            while (static_cast<int64_t>(picked.size()) < l) {
-                const int32_t c = uc(rng);
-                if (stamp[c] != r) {
-                    stamp[c] = static_cast<int32_t>(r);
-                    picked.push_back(c);
-                }
-            }
-            std::sort(picked.begin(), picked.end());
         }
+        std::sort(picked.begin(), picked.end());
         for (int32_t c : picked) {
             a.colind.push_back(c);
-            a.val.push_back(uv(rng));
+            a.val.push_back(value(engine));
         }
-        a.rowptr[r + 1] = static_cast<int32_t>(a.colind.size());
     }
+    a.rowptr[rows] = static_cast<int32_t>(a.colind.size());
     return a;
 }
 
@@ -333,13 +337,14 @@ inline CsrHost DiagCsr(int64_t m)
     return a;
 }
 
-inline std::vector<float> RandomVector(int64_t n, float lo, float hi, uint32_t seed)
+// makeDenseFloat(n, lo, hi, seed) of the reference (test/frame/fill.h:199-203): n uniform floats from a fresh engine.
+inline std::vector<float> FillDense(int64_t n, float lo, float hi, uint32_t seed)
 {
-    std::mt19937 rng(seed);
-    std::uniform_real_distribution<float> u(lo, hi);
+    std::mt19937 engine(seed);
+    std::uniform_real_distribution<float> value(lo, hi);
     std::vector<float> v(static_cast<size_t>(n > 0 ? n : 0));
     for (auto &e : v) {
-        e = u(rng);
+        e = value(engine);
     }
     return v;
 }

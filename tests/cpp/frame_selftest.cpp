@@ -3,6 +3,8 @@
 //
 //   frame_selftest <directory with the csv case tables>
 #include <cstdio>
+#include <fstream>
+#include <sstream>
 
 #include "frame.h"
 
@@ -50,7 +52,7 @@ int main(int argc, char **argv)
     }
     // against the C checker on a seeded vector, including NaN / infinity on one and on both sides
     {
-        std::vector<float> gold = frame::RandomVector(5000, -4.0f, 4.0f, 7), out = gold;
+        std::vector<float> gold = frame::FillDense(5000, -4.0f, 4.0f, 7), out = gold;
         std::mt19937 rng(8);
         for (auto &v : out) {
             v *= 1.0f + 1e-4f * static_cast<float>(static_cast<int>(rng() % 2001) - 1000) / 1000.0f;
@@ -83,6 +85,61 @@ int main(int argc, char **argv)
     if (argc > 1) {
         const auto cases = frame::GetCasesFromCsv<SpmvOpParam>(std::string(argv[1]) + "/spmv_op_cases.csv");
         Expect(cases.size() == 70 && !cases[0].caseId().empty() && cases[0].m >= 0, "GetCasesFromCsv: 70 typed rows");
+    }
+    if (argc > 1) {
+        // The generator against fingerprints of the reference's own output (FNV-1a of the three arrays, written by
+        // tests/golden/make_fill_fixture.py): every object of the "csr" and "dense" lists of fill_generator.json.
+        std::ifstream in(std::string(argv[1]) + "/fill_generator.json");
+        std::stringstream all;
+        all << in.rdbuf();
+        const std::string text = all.str();
+        // (the file is flat enough for this: a field is "name": value up to the next comma, brace or bracket)
+        auto field = [&](size_t from, size_t to, const char *name) {
+            const std::string key = std::string("\"") + name + "\":";
+            const size_t at = text.find(key, from);
+            if (at == std::string::npos || at >= to) {
+                return std::string();
+            }
+            size_t b = at + key.size();
+            while (b < to && (text[b] == ' ' || text[b] == '"')) {
+                ++b;
+            }
+            size_t e = b;
+            while (e < to && text[e] != ',' && text[e] != '"' && text[e] != '}' && text[e] != '\n') {
+                ++e;
+            }
+            return text.substr(b, e - b);
+        };
+        auto hex = [](uint64_t v) {
+            char buf[17];
+            std::snprintf(buf, sizeof(buf), "%016llx", static_cast<unsigned long long>(v));
+            return std::string(buf);
+        };
+        const size_t csrAt = text.find("\"csr\":"), denseAt = text.find("\"dense\":");
+        int csrCases = 0, csrOk = 0, denseCases = 0, denseOk = 0;
+        for (size_t at = text.find('{', csrAt); at != std::string::npos && at < denseAt; at = text.find('{', at + 1)) {
+            const size_t end = text.find('}', at);
+            const frame::CsrHost a = frame::FillCsr(
+                std::stoll(field(at, end, "rows")), std::stoll(field(at, end, "cols")), std::stod(field(at, end, "sparsity")),
+                std::stod(field(at, end, "empty_row_prob")), static_cast<uint32_t>(std::stoul(field(at, end, "seed"))),
+                std::stof(field(at, end, "lo")), std::stof(field(at, end, "hi")), std::stoll(field(at, end, "nnz_hint")));
+            ++csrCases;
+            csrOk += (a.nnz() == std::stoll(field(at, end, "nnz")) &&
+                      hex(oracle_fnv1a(a.rowptr.data(), 4 * static_cast<int64_t>(a.rowptr.size()))) == field(at, end, "rowptr_fnv1a") &&
+                      hex(oracle_fnv1a(a.colind.data(), 4 * a.nnz())) == field(at, end, "colind_fnv1a") &&
+                      hex(oracle_fnv1a(a.val.data(), 4 * a.nnz())) == field(at, end, "values_fnv1a"))
+                         ? 1 : 0;
+        }
+        for (size_t at = text.find('{', denseAt); at != std::string::npos; at = text.find('{', at + 1)) {
+            const size_t end = text.find('}', at);
+            const std::vector<float> v = frame::FillDense(std::stoll(field(at, end, "n")), std::stof(field(at, end, "lo")),
+                                                          std::stof(field(at, end, "hi")),
+                                                          static_cast<uint32_t>(std::stoul(field(at, end, "seed"))));
+            ++denseCases;
+            denseOk += hex(oracle_fnv1a(v.data(), 4 * static_cast<int64_t>(v.size()))) == field(at, end, "fnv1a") ? 1 : 0;
+        }
+        Expect(csrCases >= 8 && csrOk == csrCases, "FillCsr: the reference generator's matrices, bit for bit (hint and binomial)");
+        Expect(denseCases >= 2 && denseOk == denseCases, "FillDense: the reference generator's vectors, bit for bit");
     }
     std::printf("%d failed\n", g_failed);
     return g_failed == 0 ? 0 : 1;

@@ -36,7 +36,7 @@ frame::CsrHost Matrix(const Row &r, const char *colsKey)
         a.rowptr.assign(static_cast<size_t>(m > 0 ? m : 0) + 1, 0);
         return a;
     }
-    return frame::RandomCsr(m, n, D(r, "sparsity"), D(r, "empty_row_prob"), static_cast<uint32_t>(I(r, "seed")), -5.0f,
+    return frame::FillCsr(m, n, D(r, "sparsity"), D(r, "empty_row_prob"), static_cast<uint32_t>(I(r, "seed")), -5.0f,
                             5.0f);
 }
 
@@ -55,8 +55,8 @@ bool SpmvOpCase(const frame::Stream &stream, const frame::Handle &handle, const 
             }
         }
     }
-    const std::vector<float> x = frame::RandomVector(k, -3.0f, 3.0f, seed + 1);
-    const std::vector<float> y = frame::RandomVector(m, -3.0f, 3.0f, seed + 2);
+    const std::vector<float> x = frame::FillDense(k, -3.0f, 3.0f, seed + 1);
+    const std::vector<float> y = frame::FillDense(m, -3.0f, 3.0f, seed + 2);
     const float alpha = static_cast<float>(D(r, "alpha")), beta = static_cast<float>(D(r, "beta"));
     std::vector<float> gold(static_cast<size_t>(m));
     oracle_spmv_f64(m, k, a.rowptr.data(), a.colind.data(), a.val.data(), x.data(), y.data(), alpha, beta, gold.data());

@@ -26,10 +26,15 @@ def main():
              (7, 100, 50, 1000, -3.0, 3.0, 0.3),
              (1234, 333, 777, 333 * 9, -2.0, 2.0, 0.0),
              (5, 1, 1000, 999, -3.0, 3.0, 0.0)]
-    for seed, rows, cols, hint, lo, hi, p in cases:
-        rowptr, colind, val = oracle.ref_fill_csr(seed, rows, cols, hint, empty_row_prob=p, lo=lo, hi=hi)
+    # (nnz_hint <= 0: binomial row lengths at density 1 - sparsity, the path the SpMVOp case table takes)
+    cases = [c + (0.9,) for c in cases] + [(42, 4, 4, -1, -5.0, 5.0, 0.0, 0.5), (61, 1024, 1024, -1, -5.0, 5.0, 0.0, 0.9),
+                                           (77, 300, 5000, -1, -5.0, 5.0, 0.25, 0.99), (9, 2000, 64, -1, -5.0, 5.0, 0.1, 0.3)]
+    for seed, rows, cols, hint, lo, hi, p, sparsity in cases:
+        rowptr, colind, val = oracle.ref_fill_csr(seed, rows, cols, hint, sparsity=sparsity, empty_row_prob=p, lo=lo,
+                                                  hi=hi)
         out["csr"].append({
-            "seed": seed, "rows": rows, "cols": cols, "nnz_hint": hint, "lo": lo, "hi": hi, "empty_row_prob": p,
+            "seed": seed, "rows": rows, "cols": cols, "nnz_hint": hint, "sparsity": sparsity, "lo": lo, "hi": hi,
+            "empty_row_prob": p,
             "nnz": int(colind.size), "rowptr_fnv1a": "%016x" % oracle.fnv1a(rowptr),
             "colind_fnv1a": "%016x" % oracle.fnv1a(colind), "values_fnv1a": "%016x" % oracle.fnv1a(val),
             "colind_head": colind[:4].tolist(), "values_head": [float(v) for v in val[:2]]})

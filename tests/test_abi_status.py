@@ -36,7 +36,7 @@ def test_every_declared_symbol_is_exported(osa, L):
 
 def test_enum_values_match_header(osa):
     text = open(os.path.join(ROOT, "include", "cann_ops_sparse.h")).read()
-    m = re.search(r"typedef enum aclsparseStatus_t \{(.*?)\}", text, re.S)
+    m = re.search(r"typedef OPSPARSE_ABI_ENUM\(aclsparseStatus_t\) \{(.*?)\}", text, re.S)
     names = re.findall(r"ACL_SPARSE_STATUS_(\w+)", m.group(1))
     assert names == osa.STATUS_NAMES
     assert osa.ACL_SPARSE_STATUS_HANDLE_IS_NULLPTR == 10 and osa.ACL_SPARSE_STATUS_NOT_SUPPORTED == 8

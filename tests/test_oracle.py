@@ -273,6 +273,8 @@ def test_fill_generator_matches_committed_fixture():
     """The restated generator reproduces the arrays the reference's own generator produced
     (fingerprints written by tests/golden/make_fill_fixture.py from oracle/_ref)."""
     for case in _fixture()["csr"]:
+        if case["nnz_hint"] <= 0:
+            continue  # binomial row lengths: restated in C++ (tests/cpp/frame.h), checked by frame_selftest
         rowptr, colind, val = oracle.fill_csr(case["seed"], case["rows"], case["cols"], case["nnz_hint"], case["lo"],
                                               case["hi"], case["empty_row_prob"])
         assert colind.size == case["nnz"]

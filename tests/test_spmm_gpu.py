@@ -514,3 +514,40 @@ def test_staging_needs_a_buffer_preprocessed_for_it(osa, gpu_ctx):
     gold = oracle.spmm_f64(m, n, rowptr, colind, val, B, k, C0, n, 1.0, 0.5, b_row_major=False, trans_b=False,
                            c_row_major=True)
     assert oracle.max_rel_err(d_C.cpu().numpy(), gold) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
+def test_b_of_4_gib_through_a_padded_leading_dimension(osa, gpu_ctx, dtype):
+    """B with 2^20 rows and a leading dimension of 4 KiB spans 4 GiB: a row's offset no longer fits 32 bits and the
+    slab kernel takes its instantiation with 64-bit gather addresses.  Only the 64 columns in use are ever touched
+    (the rest of the allocation stays as it was); the last row of B, at the highest offset, is gathered."""
+    dev, stream, handle = gpu_ctx
+    m, k, n = 20_000, 1 << 20, 64
+    ldb = 4096 // (4 if dtype == torch.float32 else 2)
+    rng = np.random.default_rng(77)
+    lengths = rng.integers(0, 33, m)
+    lengths[17] = 3000                                        # a row cut into segments, too
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, k, int(rowptr[-1])).astype(np.int32)
+    colind[:4] = [k - 1, 0, k - 2, k // 2]
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    Bc = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    if dtype == torch.float16:
+        val = torch.from_numpy(val).half().float().numpy()
+        Bc = torch.from_numpy(Bc).half().float().numpy()
+    C0 = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    d_B = torch.full((k * ldb,), 7.0, dtype=dtype, device=dev)   # 4 GiB
+    assert d_B.numel() * d_B.element_size() == 1 << 32
+    d_B.view(k, ldb)[:, :n] = torch.from_numpy(Bc).to(dev).to(dtype)
+    d = [to_dev(a, dev) for a in (rowptr, colind)]
+    d_val = to_dev(val, dev, dtype)
+    d_C = to_dev(C0.ravel(), dev)
+    A = osa.Csr(m, k, d[0], d[1], d_val)
+    op = osa.SpmmOp(handle, A, osa.DnMat(k, n, ldb, d_B), osa.DnMat(m, n, n, d_C))
+    op(1.5, -0.5)
+    stream.synchronize()
+    gold = oracle.spmm_f64_rowmajor(m, n, rowptr, colind, val, Bc, n, C0, n, 1.5, -0.5)
+    assert oracle.max_rel_err(d_C.cpu().numpy(), np.asarray(gold).ravel()) <= (1e-5 if dtype == torch.float32 else 1e-3)
+    assert bool((d_B.view(k, ldb)[:, n:] == 7.0).all())
+    del d_B
+    torch.cuda.empty_cache()
