@@ -292,7 +292,13 @@ aclsparseStatus_t aclsparseDnMatSetValues(aclsparseDnMatDescr_t dnMatDescr, void
  * matrix in the buffer; it does so only where a GetBufferSize call on the same
  * descriptor and arrays, with the same opA / types / alg, answered that size
  * (a buffer sized any other way gets the ordinary plan, which fits every
- * answer).
+ * answer).  For such a matrix (more than 2^18 columns, 7 M entries or more)
+ * GetBufferSize itself looks at the column indices: it launches one short
+ * kernel on the handle's stream, uses the handle's workspace (created on first
+ * use) and synchronises the stream once; inside a stream capture it does none of
+ * that and answers the ordinary plan's size.  Preprocess synchronises the stream
+ * (once for the ordinary plan, up to four times for a re-stored layout) and
+ * must not be captured; aclsparseSpMV itself only enqueues kernels.
  *
  * Repeatability [ref: include/cann_ops_sparse.h:151-164]: ACL_SPARSE_SPMV_CSR_ALG2
  * gives bit-wise the same y from every call on the same data, for either op(A)
@@ -377,7 +383,11 @@ aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t o
  *                 the size of a re-stored index layout that createDescr builds
  *                 IF it is given a buffer (NULL stays legal: the ordinary
  *                 kernels then).  A layout is only built into a buffer when
- *                 bufferSize was asked on the same descriptor and arrays.
+ *                 bufferSize was asked on the same descriptor and arrays.  For
+ *                 such a matrix bufferSize launches one short kernel on the
+ *                 handle's stream, uses the handle's workspace and synchronises
+ *                 once (not inside a stream capture, where it answers as for a
+ *                 small matrix).
  *   createDescr   snapshots matA's pointers and sizes (not its values: they may
  *                 change between executions, except under ALG2); ALG2 needs
  *                 `buffer`, which must stay valid until destroyDescr.

@@ -199,7 +199,11 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
  *       the caller has them; rowOffsets / colInd must be the arrays of the analysis, the values may change.  Without
  *       it (values frozen) the analysis keeps a copy of the values, launches ignore the rowOffsets / colInd /
  *       csrValues arguments, and the analysis must be repeated after the values change; rows of 1024 entries and more
- *       are then stored a second time panel by panel, which halves what they cost.
+ *       are then stored a second time panel by panel, which halves what they cost.  Frozen values are kept in the
+ *       order the second kernel streams them (plan->streamedBlocks = 1: row blocks of 2^10 rows, a wavefront
+ *       each) where a (panel, block) chunk then still holds 16 entries and a row at most 16 a panel on average;
+ *       else, like live values, they are read in row order through a window in LDS by a workgroup a block of 2^12
+ *       rows (which cannot hold a row of more than 65 534 entries: see OPSPARSE_E_UNSUPPORTED below).
  *   OPSPARSE_BLOCKED_TRANSPOSE (= 1, so that a plain 0 / 1 "transpose" still reads right)  the layout of
  *       y = alpha * A^T * x + beta * y: the analysis transposes the matrix into the workspace (the CSC arrays of A
  *       are the CSR arrays of A^T) and builds the layout of that copy; no atomics on y.  With live values it keeps
@@ -208,9 +212,9 @@ int opsparse_spmv_csr_panels_analyse(const int32_t *rowOffsets, const int32_t *c
  *   OPSPARSE_BLOCKED_VALUES_F16 / _BF16 / _I32  the type of csrValues and x (default fp32).
  * Rows with many entries in every column panel and ascending columns ("long rows", plan->numLongRows of them) are
  * summed by the first kernel instead of going through the row blocks.  Returns OPSPARSE_E_INVALID for a column
- * index outside [0, cols), OPSPARSE_E_UNSUPPORTED for a matrix with a row of more than about 50 000 entries that
- * cannot go the long rows' way (its columns do not ascend).  Synchronises `stream` twice (three times for
- * op(A) = A^T).  Launches touch only the first opsparse_spmv_csr_blocked_resident_bytes() of the workspace; the rest
+ * index outside [0, cols), OPSPARSE_E_UNSUPPORTED for a matrix with a row of more than 65 534 entries that cannot
+ * go the long rows' way (its columns do not ascend) where the blocks are the windowed ones.  Synchronises `stream`
+ * twice (three times for op(A) = A^T) and allocates nothing.  Launches touch only the first opsparse_spmv_csr_blocked_resident_bytes() of the workspace; the rest
  * serves the analysis and may be handed back afterwards.
  */
 #define OPSPARSE_BLOCKED_TRANSPOSE 1

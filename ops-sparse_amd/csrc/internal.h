@@ -69,6 +69,7 @@ struct OpsparseSpmmBinding {
     const void *buffer = nullptr;
     OpsparseSpmmPlan plan{};
     int64_t stagingBytes = 0;  // room behind the plan's tables for row-major copies of B / C (0: none)
+    int64_t widestN = 0;       // the widest C the buffer has been analysed for: its tables fit that width and less
 };
 
 // reference: sparse/common/aclsparse_handle_internal.h:56-72

@@ -169,6 +169,7 @@ aclsparseStatus_t BuildPlan(const aclsparseSpMatDescr *A, int64_t n, void *buffe
         opsparse::LogError("aclsparseSpMM: analysis failed (%d)", rc);
         return FromLaunch(rc);
     }
+    A->spmm.widestN = (A->spmm.buffer == buffer && A->spmm.widestN > n) ? A->spmm.widestN : n;
     A->spmm.buffer = buffer;
     A->spmm.plan = plan;
     A->spmm.stagingBytes = 0;
@@ -313,6 +314,10 @@ aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t o
         if (hipStreamIsCapturing(handle->stream, &capturing) != hipSuccess ||
             capturing != hipStreamCaptureStatusNone) {
             (void)hipGetLastError();
+            plan = nullptr;
+        } else if (bound && matC->cols > matA->spmm.widestN) {
+            // The bound buffer was sized for a narrower C: the tables of a wider one (8 bytes per long-row segment
+            // and column) need not fit it, and nothing says how large it is.  Without tables, then.
             plan = nullptr;
         } else {
             st = BuildPlan(matA, matC->cols, buffer, handle->stream);

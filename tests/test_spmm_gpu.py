@@ -551,3 +551,49 @@ def test_b_of_4_gib_through_a_padded_leading_dimension(osa, gpu_ctx, dtype):
     assert bool((d_B.view(k, ldb)[:, n:] == 7.0).all())
     del d_B
     torch.cuda.empty_cache()
+
+
+def test_buffer_preprocessed_for_a_narrow_c_is_not_re_analysed_for_a_wider_one(osa, gpu_ctx):
+    """Preprocess with n = 8 into a buffer of exactly the size GetBufferSize asked for, long rows in the matrix (their
+    segment table grows with n); then aclsparseSpMM on the same matrix and buffer with n = 256.  The library must
+    not lay a wider plan's tables into the buffer: the product runs without tables, the bytes behind the buffer
+    stay as they were, and the result is right.  The narrow product still works afterwards."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    m, k = 3000, 6000
+    rng = np.random.default_rng(21)
+    lengths = rng.integers(0, 30, m)
+    lengths[[3, 1500, 2999]] = [5000, 2500, 4000]
+    rowptr, colind, val = csr_from_lengths(lengths, k, seed=9)
+    d_rp, d_ci, d_val = to_dev(rowptr, dev), to_dev(colind, dev), to_dev(val, dev)
+    A = osa.Csr(m, k, d_rp, d_ci, d_val)
+
+    def operands(n):
+        B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+        C0 = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+        d_B, d_C = to_dev(B.ravel(), dev), to_dev(C0.ravel(), dev)
+        return B, C0, d_B, d_C, osa.DnMat(k, n, n, d_B), osa.DnMat(m, n, n, d_C)
+
+    B8, C8, dB8, dC8, mB8, mC8 = operands(8)
+    size = ctypes.c_size_t(0)
+    one, half = ctypes.c_float(1.0), ctypes.c_float(0.5)
+    args8 = (handle.h, 0, 0, ctypes.byref(one), A.d, mB8.d, ctypes.byref(half), mC8.d, osa.ACL_FLOAT, 0)
+    assert L.aclsparseSpMMGetBufferSize(*args8, ctypes.byref(size)) == 0
+    guard = 1 << 20
+    buf = torch.full((size.value + guard,), 0x3C, dtype=torch.uint8, device=dev)
+    pbuf = ctypes.c_void_p(buf.data_ptr())
+    assert L.aclsparseSpMMPreprocess(*args8, pbuf) == 0
+    B256, C256, dB256, dC256, mB256, mC256 = operands(256)
+    args256 = (handle.h, 0, 0, ctypes.byref(one), A.d, mB256.d, ctypes.byref(half), mC256.d, osa.ACL_FLOAT, 0)
+    wide = ctypes.c_size_t(0)
+    assert L.aclsparseSpMMGetBufferSize(*args256, ctypes.byref(wide)) == 0 and wide.value > size.value
+    assert L.aclsparseSpMM(*args256, pbuf) == 0
+    stream.synchronize()
+    assert bool((buf[size.value:] == 0x3C).all())
+    gold = oracle.spmm_f64_rowmajor(m, 256, rowptr, colind, val, B256, 256, C256, 256, 1.0, 0.5)
+    assert oracle.max_rel_err(dC256.cpu().numpy(), np.asarray(gold).ravel()) <= 1e-5
+    assert L.aclsparseSpMM(*args8, pbuf) == 0
+    stream.synchronize()
+    gold = oracle.spmm_f64_rowmajor(m, 8, rowptr, colind, val, B8, 8, C8, 8, 1.0, 0.5)
+    assert oracle.max_rel_err(dC8.cpu().numpy(), np.asarray(gold).ravel()) <= 1e-5
+    assert bool((buf[size.value:] == 0x3C).all())

@@ -45,6 +45,16 @@ def test_noalloc_matches_workspace_launch(osa, workloads, gpu_ctx):
         gold = oracle.spmv_f64(rows, cols, A["rowptr"].cpu().numpy(), A["colind"].cpu().numpy(),
                                A["values"].cpu().numpy(), x.cpu().numpy(), y0.cpu().numpy(), alpha, beta)
         assert oracle.max_rel_err(y_new.cpu().numpy(), gold) <= 1e-5
+        # and the device's free memory does not move over further calls (hipMemGetInfo: what any allocation, the
+        # library's or the runtime's on its behalf, would show in)
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info(dev)[0]
+        for _ in range(5):
+            assert L.opsparse_spmv_csr_launch_noalloc(P(A["rowptr"]), P(A["colind"]), P(A["values"]), P(x), P(y_new),
+                                                      rows, cols, nnz, S(alpha), S(beta), osa.OPSPARSE_F32,
+                                                      osa.OPSPARSE_F32, 0, sp) == osa.OPSPARSE_OK
+        stream.synchronize()
+        assert torch.cuda.mem_get_info(dev)[0] == free_before
 
 
 def test_noalloc_rejects_sizes_beyond_its_array(osa, gpu_ctx):
