@@ -227,6 +227,13 @@ size_t opsparse_spmv_csr_blocked_resident_bytes(int64_t rows, int64_t cols, int6
 int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
                                       int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
                                       size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream);
+/* The same with the two parts of the workspace apart: `workspace` (opsparse_spmv_csr_blocked_resident_bytes()) is
+ * what the launches keep, `scratchSpace` (the rest of opsparse_spmv_csr_blocked_workspace_bytes()) serves the analysis
+ * only and is free again when the call returns. */
+int opsparse_spmv_csr_blocked_analyse_split(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
+                                            int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
+                                            size_t workspaceBytes, void *scratchSpace, size_t scratchBytes,
+                                            OpsparseSpmvPlan *plan, void *stream);
 
 /*
  * BLOCKED_LIVE analysis (fp32, fp16 or bf16 values and x, op(A) = A, values read in place at every launch): the
@@ -241,6 +248,10 @@ size_t opsparse_spmv_csr_live_resident_bytes(int64_t rows, int64_t cols, int64_t
 int opsparse_spmv_csr_live_analyse(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
                                    int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
                                    size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream);
+int opsparse_spmv_csr_live_analyse_split(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
+                                         int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
+                                         size_t workspaceBytes, void *scratchSpace, size_t scratchBytes,
+                                         OpsparseSpmvPlan *plan, void *stream);
 
 /* Same as opsparse_spmv_csr_launch with separate input and output vectors:
  * z = alpha * op(A) * x + beta * yIn.  z may be yIn (in place); yIn is only read

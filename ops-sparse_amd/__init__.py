@@ -99,6 +99,7 @@ OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_blocked_workspace_bytes", "opsparse_spmv_csr_blocked_resident_bytes",
     "opsparse_spmv_csr_blocked_analyse",
     "opsparse_spmv_csr_live_workspace_bytes", "opsparse_spmv_csr_live_resident_bytes", "opsparse_spmv_csr_live_analyse",
+    "opsparse_spmv_csr_live_analyse_split", "opsparse_spmv_csr_blocked_analyse_split",
     "opsparse_spmv_csr_gathers_scattered",
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
     "opsparse_dense_restage",
@@ -274,6 +275,9 @@ def lib():
     L.opsparse_spmv_csr_live_analyse.restype = ctypes.c_int
     L.opsparse_spmv_csr_live_analyse.argtypes = [vp, vp, vp, i64, i64, i64, i32, vp, sz,
                                                  ctypes.POINTER(OpsparseSpmvPlan), vp]
+    for name in ("opsparse_spmv_csr_live_analyse_split", "opsparse_spmv_csr_blocked_analyse_split"):
+        getattr(L, name).restype = ctypes.c_int
+        getattr(L, name).argtypes = [vp, vp, vp, i64, i64, i64, i32, vp, sz, vp, sz, ctypes.POINTER(OpsparseSpmvPlan), vp]
     L.opsparse_spmv_csr_blocked_analyse.restype = ctypes.c_int
     L.opsparse_spmv_csr_blocked_analyse.argtypes = [vp, vp, vp, i64, i64, i64, i32, vp, sz,
                                                     ctypes.POINTER(OpsparseSpmvPlan), vp]

@@ -155,9 +155,16 @@ constexpr int64_t kMinColsOrderedLive = int64_t{5} << 19;  // 2.6 M
 
 struct RestoredChoice {
     int32_t kernel;
-    size_t bytes;
+    size_t bytes;     // of the whole layout, analysis scratch included
     bool liveValues;  // BLOCKED_GATHER / BLOCKED_LIVE: the layout holds no values, every call takes the caller's
+    size_t keep = 0;     // what the caller's buffer has to hold: `bytes`, or only what the launches keep ...
+    size_t scratch = 0;  // ... when the analysis takes this much from the handle's workspace (TrimToWorkspace)
 };
+// Where the handle has a workspace of the user's (aclsparseSetWorkspace) with room for the scratch of the layout's
+// analysis, the caller's buffer only needs what the launches keep (the 8 M-row power-law matrix: 0.79 GiB instead
+// of 2.09): sets keep / scratch accordingly, else keep = bytes.
+void TrimToWorkspace(aclsparseHandle_t handle, RestoredChoice *choice, int64_t rows, int64_t cols, int64_t nnz,
+                     bool transpose, int32_t valueType);
 // The layout a default-algorithm request gets where it pays: blocked gather with live values (7 M
 // entries or more, an x the layout applies to, and a sample of the columns that says the gathers are scattered:
 // one short kernel and a synchronisation of the handle's stream), else none.  `repeatable`: the caller promises
@@ -170,8 +177,11 @@ void RememberSized(aclsparseConstSpMatDescr_t matA, const RestoredChoice &choice
 bool SizedFor(aclsparseConstSpMatDescr_t matA, const RestoredChoice &choice, bool transpose, int32_t valueType);
 // valueType: the OPSPARSE_* type of the values and of x.
 RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose, int32_t valueType);
+// `scratch` / `scratchBytes`: where the analysis works when the buffer only has room for what the launches keep
+// (scratchBytes == 0: behind that, in the buffer itself).
 int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const void *values,
                     int32_t valueType, int64_t rows, int64_t cols, int64_t nnz, bool transpose, bool liveValues,
-                    void *buffer, size_t bytes, OpsparseSpmvPlan *plan, void *stream);
+                    void *buffer, size_t bytes, void *scratch, size_t scratchBytes, OpsparseSpmvPlan *plan,
+                    void *stream);
 
 }  // namespace opsparse

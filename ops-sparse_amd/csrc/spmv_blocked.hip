@@ -2353,9 +2353,10 @@ size_t opsparse_spmv_csr_blocked_resident_bytes(int64_t rows, int64_t cols, int6
                                   : MakeBlockedLayout(rows, cols, nnz, false, live, vt)).resident);
 }
 
-int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
+int opsparse_spmv_csr_blocked_analyse_split(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
                                       int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
-                                      size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream)
+                                      size_t workspaceBytes, void *scratchSpace, size_t scratchBytes,
+                                      OpsparseSpmvPlan *plan, void *stream)
 {
     if (plan == nullptr || rowOffsets == nullptr || colInd == nullptr || csrValues == nullptr) {
         return OPSPARSE_E_INVALID;
@@ -2367,12 +2368,17 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     if (l.P == 0) {
         return OPSPARSE_E_UNSUPPORTED;
     }
-    if (workspace == nullptr || static_cast<int64_t>(workspaceBytes) < l.bytes) {
+    // what the launches keep goes into `workspace`, what only the analysis needs into `scratchSpace`
+    if (workspace == nullptr || static_cast<int64_t>(workspaceBytes) < l.resident || scratchSpace == nullptr ||
+        static_cast<int64_t>(scratchBytes) < l.bytes - l.resident) {
         return OPSPARSE_E_WORKSPACE;
     }
     auto s = static_cast<hipStream_t>(stream);
-    auto *base = static_cast<unsigned char *>(workspace);
-    auto ints = [&](int64_t off) { return reinterpret_cast<int32_t *>(base + off); };
+    auto *residentBase = static_cast<unsigned char *>(workspace);
+    auto *scratchBase = static_cast<unsigned char *>(scratchSpace);
+    const int64_t residentEnd = l.resident;
+    auto at = [&](int64_t off) { return off < residentEnd ? residentBase + off : scratchBase + (off - residentEnd); };
+    auto ints = [&](int64_t off) { return reinterpret_cast<int32_t *>(at(off)); };
     int32_t *status = ints(0);
     // status, number of long rows, their entries, entries of the largest block, long rows summed on their own
     LaunchFillI32(status, 8, 0, s);
@@ -2390,7 +2396,7 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
             return OPSPARSE_E_INVALID;  // a column index outside [0, cols)
         }
         const void *srcVals = csrValues;
-        void *dstVals = base + l.cscValOff;
+        void *dstVals = at(l.cscValOff);
         int32_t vb = ValueBytes(valueType);
         if (live) {
             // what travels with an entry is its position in the caller's arrays; the values follow it at every call
@@ -2401,14 +2407,14 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
             vb = 4;
         }
         const int rc = opsparse_csr2csc_launch(rows, cols, nnz, srcVals, rowOffsets, colInd, dstVals, ints(l.cscPtrOff),
-                                               ints(l.cscIndOff), vb, 0, base + l.transposeWsOff,
+                                               ints(l.cscIndOff), vb, 0, at(l.transposeWsOff),
                                                static_cast<size_t>(l.transposeWsBytes), s);
         if (rc != OPSPARSE_OK) {
             return rc;
         }
         rowOffsets = ints(l.cscPtrOff);
         colInd = ints(l.cscIndOff);
-        csrValues = base + l.cscValOff;  // (live values: filled at every call; the analysis reads no value then)
+        csrValues = at(l.cscValOff);  // (live values: filled at every call; the analysis reads no value then)
     }
     // From here on: `outputs` rows, `inputs` columns, the arrays rowOffsets / colInd / csrValues.
     const bool frozenCopy = !live && !transposed;
@@ -2417,8 +2423,8 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     int32_t *rowOfPos = ints(l.rowOfPosOff), *table = ints(l.tableOff), *scratch = ints(l.scratchOff);
     int32_t *srcStart = ints(l.srcStartOff), *dstStart = ints(l.dstStartOff);
     int32_t *blockRow = ints(l.blockRowOff);
-    auto *colLocal = reinterpret_cast<uint16_t *>(base + l.colLocalOff);
-    auto *slot16 = reinterpret_cast<uint16_t *>(base + l.slotOff);
+    auto *colLocal = reinterpret_cast<uint16_t *>(at(l.colLocalOff));
+    auto *slot16 = reinterpret_cast<uint16_t *>(at(l.slotOff));
 
     LaunchExpandRows(rowOffsets, outputs, nnz, 0, rowOfPos, s);
     if (!l.streamed) {
@@ -2520,13 +2526,13 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     hipLaunchKernelGGL(BlockedBlockTablesKernel, dim3(GridOf(tableItems, kBlockThreads, INT32_MAX)), dim3(kBlockThreads), 0,
                        s, offsets, frozenCopy || l.streamed ? offsets : rowOffsets, blockRow, dstStart, srcStart,
                        longBefore != nullptr ? ints(l.longFirstOff) : nullptr, l.P, l.B, ints(l.blockShortOff),
-                       reinterpret_cast<BlockMeta *>(base + l.metaOff), ints(l.panelStartOff), status);
+                       reinterpret_cast<BlockMeta *>(at(l.metaOff)), ints(l.panelStartOff), status);
     if (!l.streamed) {
         hipLaunchKernelGGL(BlockedRowTablesKernel, dim3(static_cast<uint32_t>(l.B)), dim3(kTableThreads), 0, s,
-                           reinterpret_cast<const BlockMeta *>(base + l.metaOff), offsets,
-                           reinterpret_cast<uint32_t *>(base + l.rowBitsOff),
-                           reinterpret_cast<uint16_t *>(base + l.bitPrefixOff),
-                           reinterpret_cast<uint16_t *>(base + l.ordRowOff));
+                           reinterpret_cast<const BlockMeta *>(at(l.metaOff)), offsets,
+                           reinterpret_cast<uint32_t *>(at(l.rowBitsOff)),
+                           reinterpret_cast<uint16_t *>(at(l.bitPrefixOff)),
+                           reinterpret_cast<uint16_t *>(at(l.ordRowOff)));
     }
     const int rcScatter = WithValueType(valueType, [&](auto tag) {
         using ValT = decltype(tag);
@@ -2534,19 +2540,19 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
             hipLaunchKernelGGL(StreamScatterKernel<ValT>, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0,
                                s, pos, rowOfSrc, chunkKey, static_cast<const ValT *>(csrValues), srcStart, dstStart,
                                blockRow, nnz, l.P, l.B, slot16, ints(l.src8Off),
-                               reinterpret_cast<ValT *>(base + l.valDOff), static_cast<int32_t *>(nullptr),
-                               longBefore != nullptr && l.frozenLong ? reinterpret_cast<uint32_t *>(base + l.xgOff)
+                               reinterpret_cast<ValT *>(at(l.valDOff)), static_cast<int32_t *>(nullptr),
+                               longBefore != nullptr && l.frozenLong ? reinterpret_cast<uint32_t *>(at(l.xgOff))
                                                                      : nullptr,
                                slot16 + LongRowOfShift(l), longBefore);
             hipLaunchKernelGGL(StreamTurnsKernel, dim3(static_cast<uint32_t>(l.B)), dim3(kTurnThreads), 0, s,
-                               reinterpret_cast<const BlockMeta *>(base + l.metaOff), slot16);
+                               reinterpret_cast<const BlockMeta *>(at(l.metaOff)), slot16);
             return OPSPARSE_OK;
         }
         hipLaunchKernelGGL(BlockedScatterKernel<ValT>, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
                            pos, rowOfSrc, chunkKey, static_cast<const ValT *>(csrValues), rowOffsets, offsets, srcStart,
                            dstStart, ints(l.blockShortOff), nnz, l.P, l.B, slot16, ints(l.src8Off),
-                           frozenCopy ? reinterpret_cast<ValT *>(base + l.valSOff) : nullptr,
-                           longBefore != nullptr && l.frozenLong ? reinterpret_cast<uint32_t *>(base + l.xgOff) : nullptr,
+                           frozenCopy ? reinterpret_cast<ValT *>(at(l.valSOff)) : nullptr,
+                           longBefore != nullptr && l.frozenLong ? reinterpret_cast<uint32_t *>(at(l.xgOff)) : nullptr,
                            slot16 + LongRowOfShift(l), longBefore);
         return OPSPARSE_OK;
     });
@@ -2583,6 +2589,22 @@ int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *
     p.bytes = l.bytes;
     *plan = p;
     return OPSPARSE_OK;
+}
+
+int opsparse_spmv_csr_blocked_analyse(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
+                                      int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
+                                      size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream)
+{
+    // one piece: the analysis' scratch follows what the launches keep
+    const size_t resident = opsparse_spmv_csr_blocked_resident_bytes(rows, cols, nnz, flags);
+    if (resident == 0) {
+        return OPSPARSE_E_UNSUPPORTED;
+    }
+    if (workspace == nullptr || workspaceBytes < resident) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    return opsparse_spmv_csr_blocked_analyse_split(rowOffsets, colInd, csrValues, rows, cols, nnz, flags, workspace, resident,
+                                            static_cast<unsigned char *>(workspace) + resident, workspaceBytes - resident, plan, stream);
 }
 
 }  // extern "C"

@@ -1372,9 +1372,10 @@ size_t opsparse_spmv_csr_live_resident_bytes(int64_t rows, int64_t cols, int64_t
     return static_cast<size_t>(MakeBlockedLayout(rows, cols, nnz, false, true).resident);
 }
 
-int opsparse_spmv_csr_live_analyse(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
+int opsparse_spmv_csr_live_analyse_split(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
                                       int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
-                                      size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream)
+                                      size_t workspaceBytes, void *scratchSpace, size_t scratchBytes,
+                                      OpsparseSpmvPlan *plan, void *stream)
 {
     if (plan == nullptr || rowOffsets == nullptr || colInd == nullptr || csrValues == nullptr) {
         return OPSPARSE_E_INVALID;
@@ -1392,21 +1393,26 @@ int opsparse_spmv_csr_live_analyse(const int32_t *rowOffsets, const int32_t *col
     if (l.P == 0) {
         return OPSPARSE_E_UNSUPPORTED;
     }
-    if (workspace == nullptr || static_cast<int64_t>(workspaceBytes) < l.bytes) {
+    // what the launches keep goes into `workspace`, what only the analysis needs into `scratchSpace`
+    if (workspace == nullptr || static_cast<int64_t>(workspaceBytes) < l.resident || scratchSpace == nullptr ||
+        static_cast<int64_t>(scratchBytes) < l.bytes - l.resident) {
         return OPSPARSE_E_WORKSPACE;
     }
     auto s = static_cast<hipStream_t>(stream);
-    auto *base = static_cast<unsigned char *>(workspace);
-    auto ints = [&](int64_t off) { return reinterpret_cast<int32_t *>(base + off); };
+    auto *residentBase = static_cast<unsigned char *>(workspace);
+    auto *scratchBase = static_cast<unsigned char *>(scratchSpace);
+    const int64_t residentEnd = l.resident;
+    auto at = [&](int64_t off) { return off < residentEnd ? residentBase + off : scratchBase + (off - residentEnd); };
+    auto ints = [&](int64_t off) { return reinterpret_cast<int32_t *>(at(off)); };
     int32_t *status = ints(0);
     int32_t *keys[2] = {ints(l.keys0Off), ints(l.keys1Off)};
     int32_t *poss[2] = {ints(l.pos0Off), ints(l.pos1Off)};
     int32_t *rowOfPos = ints(l.rowOfPosOff), *table = ints(l.tableOff), *scratch = ints(l.scratchOff);
     int32_t *srcStart = ints(l.srcStartOff), *dstStart = ints(l.dstStartOff), *srcStartT = ints(l.srcStartTOff);
     int32_t *blockRow = ints(l.blockRowOff);
-    auto *colLocal = reinterpret_cast<uint16_t *>(base + l.colLocalOff);
-    auto *rowLocal = reinterpret_cast<uint16_t *>(base + l.rowLocalOff);
-    auto *valD = reinterpret_cast<float *>(base + l.valOff);
+    auto *colLocal = reinterpret_cast<uint16_t *>(at(l.colLocalOff));
+    auto *rowLocal = reinterpret_cast<uint16_t *>(at(l.rowLocalOff));
+    auto *valD = reinterpret_cast<float *>(at(l.valOff));
 
     // status, number of long rows, their entries, positions of the longest block, long rows summed on their own
     LaunchFillI32(status, 5, 0, s);
@@ -1495,7 +1501,7 @@ int opsparse_spmv_csr_live_analyse(const int32_t *rowOffsets, const int32_t *col
         hipLaunchKernelGGL(BlockedScatterKernel<ValT>, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s,
                            pos, rowOfSrc, chunkKey, static_cast<const ValT *>(csrValues), srcStart, dstStart, blockRow, nnz,
                            l.P, l.B, live ? nullptr : valD, rowLocal, live ? ints(l.dstOfPosOff) : nullptr,
-                           longBefore != nullptr && !live ? reinterpret_cast<float *>(base + l.xgOff) : nullptr,
+                           longBefore != nullptr && !live ? reinterpret_cast<float *>(at(l.xgOff)) : nullptr,
                            rowLocal + LongRowOfShift(l), longBefore);
     };
     if (valueType == OPSPARSE_F16) {
@@ -1556,6 +1562,22 @@ int opsparse_spmv_csr_live_analyse(const int32_t *rowOffsets, const int32_t *col
     p.bytes = l.bytes;
     *plan = p;
     return OPSPARSE_OK;
+}
+
+int opsparse_spmv_csr_live_analyse(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
+                                      int64_t rows, int64_t cols, int64_t nnz, int32_t flags, void *workspace,
+                                      size_t workspaceBytes, OpsparseSpmvPlan *plan, void *stream)
+{
+    // one piece: the analysis' scratch follows what the launches keep
+    const size_t resident = opsparse_spmv_csr_live_resident_bytes(rows, cols, nnz);
+    if (resident == 0) {
+        return OPSPARSE_E_UNSUPPORTED;
+    }
+    if (workspace == nullptr || workspaceBytes < resident) {
+        return OPSPARSE_E_WORKSPACE;
+    }
+    return opsparse_spmv_csr_live_analyse_split(rowOffsets, colInd, csrValues, rows, cols, nnz, flags, workspace, resident,
+                                         static_cast<unsigned char *>(workspace) + resident, workspaceBytes - resident, plan, stream);
 }
 
 }  // extern "C"

@@ -233,15 +233,35 @@ void RememberSized(aclsparseConstSpMatDescr_t matA, const RestoredChoice &choice
     z.transpose = transpose;
     z.liveValues = choice.liveValues;
     z.valueType = valueType;
-    z.bytes = choice.bytes;
+    z.bytes = choice.keep;
 }
 
 bool SizedFor(aclsparseConstSpMatDescr_t matA, const RestoredChoice &choice, bool transpose, int32_t valueType)
 {
     const OpsparseSpmvSized &z = matA->spmvSized;
-    return choice.kernel != 0 && z.kernel == choice.kernel && z.bytes >= choice.bytes && z.rowOffsets == matA->rowOffsets &&
+    return choice.kernel != 0 && z.kernel == choice.kernel && z.bytes >= choice.keep && z.rowOffsets == matA->rowOffsets &&
            z.colInd == matA->colInd && z.rows == matA->rows && z.cols == matA->cols && z.nnz == matA->nnz &&
            z.transpose == transpose && z.liveValues == choice.liveValues && z.valueType == valueType;
+}
+
+void TrimToWorkspace(aclsparseHandle_t handle, RestoredChoice *choice, int64_t rows, int64_t cols, int64_t nnz,
+                     bool transpose, int32_t valueType)
+{
+    choice->keep = choice->bytes;
+    choice->scratch = 0;
+    size_t resident = 0;
+    if (choice->kernel == OPSPARSE_SPMV_BLOCKED_LIVE) {
+        resident = opsparse_spmv_csr_live_resident_bytes(rows, cols, nnz);
+    } else if (choice->kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {
+        resident = opsparse_spmv_csr_blocked_resident_bytes(rows, cols, nnz,
+                                                            BlockedFlags(transpose, choice->liveValues, valueType));
+    }
+    if (resident == 0 || resident >= choice->bytes || handle == nullptr || !handle->useUserWorkspace ||
+        handle->userWorkspace == nullptr || handle->userWorkspaceBytes < choice->bytes - resident) {
+        return;
+    }
+    choice->keep = resident;
+    choice->scratch = choice->bytes - resident;
 }
 
 RestoredChoice PickLiveLayout(aclsparseHandle_t handle, const int32_t *rowOffsets, const int32_t *colInd, int64_t rows,
@@ -316,7 +336,8 @@ RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool 
 
 int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const void *values,
                     int32_t valueType, int64_t rows, int64_t cols, int64_t nnz, bool transpose, bool liveValues,
-                    void *buffer, size_t bytes, OpsparseSpmvPlan *plan, void *stream)
+                    void *buffer, size_t bytes, void *scratch, size_t scratchBytes, OpsparseSpmvPlan *plan,
+                    void *stream)
 {
     // A matrix whose gathers stay near the diagonal (a mesh, a band) keeps x in cache under the row-wise kernels:
     // those are then faster than any re-stored layout (the 2048 x 2048 Laplacian: 41 us against 91 us).  With some
@@ -343,13 +364,19 @@ int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *co
         return opsparse_spmv_csr_analyse(rowOffsets, rows, cols, nnz, buffer, bytes, OPSPARSE_SPMV_AUTO, plan, stream);
     }
     if (kernel == OPSPARSE_SPMV_BLOCKED_LIVE) {
-        return opsparse_spmv_csr_live_analyse(rowOffsets, colInd, values, rows, cols, nnz,
-                                              BlockedFlags(false, true, valueType), buffer, bytes, plan, stream);
+        const int32_t flags = BlockedFlags(false, true, valueType);
+        return scratchBytes > 0 ? opsparse_spmv_csr_live_analyse_split(rowOffsets, colInd, values, rows, cols, nnz, flags,
+                                                                       buffer, bytes, scratch, scratchBytes, plan, stream)
+                                : opsparse_spmv_csr_live_analyse(rowOffsets, colInd, values, rows, cols, nnz, flags, buffer,
+                                                                 bytes, plan, stream);
     }
     if (kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {
-        const int rc = opsparse_spmv_csr_blocked_analyse(rowOffsets, colInd, values, rows, cols, nnz,
-                                                         BlockedFlags(transpose, liveValues, valueType), buffer, bytes,
-                                                         plan, stream);
+        const int32_t flags = BlockedFlags(transpose, liveValues, valueType);
+        const int rc = scratchBytes > 0
+                           ? opsparse_spmv_csr_blocked_analyse_split(rowOffsets, colInd, values, rows, cols, nnz, flags,
+                                                                     buffer, bytes, scratch, scratchBytes, plan, stream)
+                           : opsparse_spmv_csr_blocked_analyse(rowOffsets, colInd, values, rows, cols, nnz, flags, buffer,
+                                                               bytes, plan, stream);
         if (rc == OPSPARSE_E_UNSUPPORTED) {
             // (a row too long for a row block that cannot go the long rows' way: the ordinary plan)
             return opsparse_spmv_csr_analyse(rowOffsets, rows, cols, nnz, buffer, bytes, OPSPARSE_SPMV_AUTO, plan, stream);
@@ -393,9 +420,11 @@ aclsparseStatus_t aclsparseSpMVGetBufferSize(aclsparseHandle_t handle, aclsparse
         return ACL_SPARSE_STATUS_INVALID_VALUE;
     }
     const size_t plain = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
-    const Restored restored = RestoredLayout(handle, opA, matA, vecX, vecY, computeType, alg);
+    Restored restored = RestoredLayout(handle, opA, matA, vecX, vecY, computeType, alg);
+    opsparse::TrimToWorkspace(handle, &restored, matA->rows, matA->cols, matA->nnz, c.transpose,
+                              RestoredValueType(matA, vecX));
     opsparse::RememberSized(matA, restored, c.transpose, RestoredValueType(matA, vecX));
-    const size_t own = restored.bytes > plain ? restored.bytes : plain;
+    const size_t own = restored.keep > plain ? restored.keep : plain;
     *bufferSize = StagedTranspose(c) ? opsparse::AlignUp(own, 256) + StagingBytes(matA) : own;
     return ACL_SPARSE_STATUS_SUCCESS;
 }
@@ -422,6 +451,8 @@ aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOpe
     }
     OpsparseSpmvPlan plan{};
     Restored restored = RestoredLayout(handle, opA, matA, vecX, vecY, computeType, alg);
+    opsparse::TrimToWorkspace(handle, &restored, matA->rows, matA->cols, matA->nnz, c.transpose,
+                              RestoredValueType(matA, vecX));
     if (!opsparse::SizedFor(matA, restored, c.transpose, RestoredValueType(matA, vecX))) {
         // no size query on these arrays asked for the layout's bytes: the buffer may be as small as every query
         // answers at least, and the ordinary plan fits that
@@ -433,7 +464,8 @@ aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOpe
                                        static_cast<const int32_t *>(matA->colInd), matA->values,
                                        RestoredValueType(matA, vecX), matA->rows, matA->cols, matA->nnz,
                                        opA != ACL_SPARSE_OP_NON_TRANSPOSE, restored.liveValues, externalBuffer,
-                                       restored.bytes, &plan, handle->stream);
+                                       restored.keep, restored.scratch > 0 ? handle->userWorkspace : nullptr,
+                                       restored.scratch > 0 ? handle->userWorkspaceBytes : 0, &plan, handle->stream);
     } else {
         const size_t bytes = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
         rc = opsparse_spmv_csr_analyse(static_cast<const int32_t *>(matA->rowOffsets), matA->rows, matA->cols,
@@ -450,7 +482,7 @@ aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOpe
     if (StagedTranspose(c)) {
         // behind everything GetBufferSize counted for the plan (the same sum as there)
         const size_t plain = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
-        const size_t own = restored.bytes > plain ? restored.bytes : plain;
+        const size_t own = restored.keep > plain ? restored.keep : plain;
         matA->spmv.stagingOffset = static_cast<int64_t>(opsparse::AlignUp(own, 256));
         matA->spmv.stagingBytes = static_cast<int64_t>(StagingBytes(matA));
     }

@@ -199,13 +199,15 @@ aclsparseStatus_t aclsparseSpMVOp_bufferSize(aclsparseHandle_t handle, aclsparse
     *bufferSize = 0;
     if (alg == ACL_SPARSE_SPMVOP_ALG2) {
         const size_t plain = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
-        const opsparse::RestoredChoice restored = RestoredLayout(matA);
+        opsparse::RestoredChoice restored = RestoredLayout(matA);
+        opsparse::TrimToWorkspace(handle, &restored, matA->rows, matA->cols, matA->nnz, false, OPSPARSE_F32);
         opsparse::RememberSized(matA, restored, false, OPSPARSE_F32);
-        *bufferSize = restored.bytes > plain ? restored.bytes : plain;
+        *bufferSize = restored.keep > plain ? restored.keep : plain;
     } else {
-        const opsparse::RestoredChoice live = LiveLayout(handle, matA);
+        opsparse::RestoredChoice live = LiveLayout(handle, matA);
+        opsparse::TrimToWorkspace(handle, &live, matA->rows, matA->cols, matA->nnz, false, OPSPARSE_F32);
         opsparse::RememberSized(matA, live, false, OPSPARSE_F32);
-        *bufferSize = live.bytes;
+        *bufferSize = live.keep;
     }
     return ACL_SPARSE_STATUS_SUCCESS;
 }
@@ -275,6 +277,7 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
         if ((Plain(d) || d->offsets32 != nullptr) && d->rows > 0 && d->nnz > 0 && d->rowOffsets != nullptr) {
             // (a re-stored layout only into a buffer that a size query on these arrays sized for it)
             opsparse::RestoredChoice restored = RestoredLayout(matA);
+            opsparse::TrimToWorkspace(handle, &restored, matA->rows, matA->cols, matA->nnz, false, OPSPARSE_F32);
             if (!opsparse::SizedFor(matA, restored, false, OPSPARSE_F32)) {
                 restored = opsparse::RestoredChoice{0, 0, false};
             }
@@ -282,8 +285,10 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
                 restored.kernel != 0 && d->colInd != nullptr && d->values != nullptr
                     ? opsparse::AnalyseRestored(restored.kernel, static_cast<const int32_t *>(d->rowOffsets),
                                                 static_cast<const int32_t *>(d->colInd), d->values, OPSPARSE_F32,
-                                                d->rows, d->cols, d->nnz, false, false, buffer, restored.bytes,
-                                                &d->plan, handle->stream)
+                                                d->rows, d->cols, d->nnz, false, false, buffer, restored.keep,
+                                                restored.scratch > 0 ? handle->userWorkspace : nullptr,
+                                                restored.scratch > 0 ? handle->userWorkspaceBytes : 0, &d->plan,
+                                                handle->stream)
                     : opsparse_spmv_csr_analyse(Offsets32(d), d->rows, d->cols, d->nnz, buffer,
                                                 opsparse_spmv_csr_workspace_bytes(d->rows, d->nnz), OPSPARSE_SPMV_AUTO,
                                                 &d->plan, handle->stream);
@@ -297,11 +302,14 @@ aclsparseStatus_t aclsparseSpMVOp_createDescr(aclsparseHandle_t handle, aclspars
     }
     if (d->alg != ACL_SPARSE_SPMVOP_ALG2 && buffer != nullptr && Plain(d) && d->rows > 0 && d->nnz > 0) {
         // the buffer aclsparseSpMVOp_bufferSize asked for (it asks the same question of the same arrays)
-        const opsparse::RestoredChoice live = LiveLayout(handle, matA);
+        opsparse::RestoredChoice live = LiveLayout(handle, matA);
+        opsparse::TrimToWorkspace(handle, &live, matA->rows, matA->cols, matA->nnz, false, OPSPARSE_F32);
         if (live.kernel != 0 && opsparse::SizedFor(matA, live, false, OPSPARSE_F32)) {
             const int rc = opsparse::AnalyseRestored(live.kernel, static_cast<const int32_t *>(d->rowOffsets),
                                                      static_cast<const int32_t *>(d->colInd), d->values, OPSPARSE_F32,
-                                                     d->rows, d->cols, d->nnz, false, true, buffer, live.bytes, &d->plan,
+                                                     d->rows, d->cols, d->nnz, false, true, buffer, live.keep,
+                                                     live.scratch > 0 ? handle->userWorkspace : nullptr,
+                                                     live.scratch > 0 ? handle->userWorkspaceBytes : 0, &d->plan,
                                                      handle->stream);
             if (rc != OPSPARSE_OK) {
                 delete d;

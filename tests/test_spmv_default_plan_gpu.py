@@ -755,3 +755,77 @@ def test_ordered_live_layout_only_where_x_is_out_of_reach_of_the_caches(osa, gpu
     assert osa.SpmvOp(handle, A, osa.DnVec(d[3]), Y).buffer.numel() == plain
     monkeypatch.setenv("OPS_SPARSE_ORDERED_LIVE_MIN_COLS", str(cols))
     assert osa.SpmvOp(handle, A, osa.DnVec(d[3]), Y).buffer.numel() > plain
+
+
+@pytest.mark.parametrize("alg_name", ["default", "alg2", "spmvop_default"])
+def test_buffer_holds_only_what_the_calls_keep_when_the_handle_lends_the_scratch(osa, gpu_ctx, alg_name):
+    """Two thirds of what a layout's analysis needs is scratch.  A handle that was given a workspace with room for it
+    (aclsparseSetWorkspace) lends it to Preprocess / createDescr, and the size query then only asks the caller for
+    what the later calls keep; without such a workspace the query asks for everything, as before.  Same products;
+    nothing is written behind the smaller buffer; a handle whose workspace went away between the query and
+    Preprocess gets the ordinary plan."""
+    dev, stream, handle = gpu_ctx
+    L = osa.lib()
+    rows, cols = 320_000, 1_500_000
+    rowptr, colind, val, x, y0 = _scattered(rows, cols, 15)
+    nnz = colind.size
+    gold = oracle.spmv_f64(rows, cols, rowptr, colind, val, x, y0, 1.5, -0.5)
+    if alg_name == "alg2":
+        whole = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, 0)
+        keep = L.opsparse_spmv_csr_blocked_resident_bytes(rows, cols, nnz, 0)
+    elif alg_name == "default":
+        whole = L.opsparse_spmv_csr_live_workspace_bytes(rows, cols, nnz)
+        keep = L.opsparse_spmv_csr_live_resident_bytes(rows, cols, nnz)
+    else:
+        whole = L.opsparse_spmv_csr_blocked_workspace_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+        keep = L.opsparse_spmv_csr_blocked_resident_bytes(rows, cols, nnz, osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+    assert 0 < keep < whole
+    lent = torch.empty(whole - keep, dtype=torch.uint8, device=dev)
+    guard = 1 << 16
+
+    def product(buffer_bytes, expect_layout):
+        d = [to_dev(a, dev) for a in (rowptr, colind, val, x)]
+        A = osa.Csr(rows, cols, d[0], d[1], d[2])
+        d_y = to_dev(y0, dev)
+        X, Y = osa.DnVec(d[3]), osa.DnVec(d_y)
+        one, half = ctypes.c_float(1.5), ctypes.c_float(-0.5)
+        n = ctypes.c_size_t(0)
+        if alg_name == "spmvop_default":
+            common = (0, A.d, X.d, Y.d, Y.d, osa.ACL_FLOAT, osa.ACL_SPARSE_SPMVOP_ALG_DEFAULT)
+            assert L.aclsparseSpMVOp_bufferSize(handle.h, *common, ctypes.byref(n)) == 0
+        else:
+            alg = osa.ACL_SPARSE_SPMV_CSR_ALG2 if alg_name == "alg2" else osa.ACL_SPARSE_SPMV_ALG_DEFAULT
+            common = (0, None, A.d, X.d, None, Y.d, osa.ACL_FLOAT, alg)
+            assert L.aclsparseSpMVGetBufferSize(handle.h, *common, ctypes.byref(n)) == 0
+        assert n.value == buffer_bytes
+        buf = torch.full((n.value + guard,), 0x77, dtype=torch.uint8, device=dev)
+        pbuf = ctypes.c_void_p(buf.data_ptr())
+        return d, A, X, Y, d_y, one, half, common, buf, pbuf, n.value
+
+    def run(state):
+        d, A, X, Y, d_y, one, half, common, buf, pbuf, size = state
+        if alg_name == "spmvop_default":
+            descr, plan = ctypes.c_void_p(), ctypes.c_void_p()
+            assert L.aclsparseSpMVOp_createDescr(handle.h, ctypes.byref(descr), *common, pbuf) == 0
+            assert L.aclsparseSpMVOp_createPlan(handle.h, descr, ctypes.byref(plan), None, 0) == 0
+            assert L.aclsparseSpMVOp(handle.h, plan, ctypes.byref(one), ctypes.byref(half), X.d, Y.d, Y.d) == 0
+            stream.synchronize()
+            L.aclsparseSpMVOp_destroyPlan(plan)
+            L.aclsparseSpMVOp_destroyDescr(descr)
+        else:
+            assert L.aclsparseSpMVPreprocess(handle.h, *common, pbuf) == 0
+            assert L.aclsparseSpMV(handle.h, 0, ctypes.byref(one), A.d, X.d, ctypes.byref(half), Y.d, osa.ACL_FLOAT,
+                                   common[-1], pbuf) == 0
+            stream.synchronize()
+        assert bool((buf[size:] == 0x77).all())
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5
+
+    try:
+        run(product(whole, True))                              # no workspace of the user's: everything in the buffer
+        assert L.aclsparseSetWorkspace(handle.h, ctypes.c_void_p(lent.data_ptr()), lent.numel()) == 0
+        run(product(keep, True))                               # the scratch is lent: the buffer keeps the layout only
+        state = product(keep, True)
+        assert L.aclsparseSetWorkspace(handle.h, None, 0) == 0  # ... and taken away again before Preprocess
+        run(state)                                             # the ordinary plan, inside the smaller buffer
+    finally:
+        L.aclsparseSetWorkspace(handle.h, None, 0)
