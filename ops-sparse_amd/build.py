@@ -4,6 +4,7 @@ hipcc cross-compiles without a GPU, so this runs anywhere ROCm is installed:
 
     python ops-sparse_amd/build.py
     python ops-sparse_amd/build.py --asan     # host code under ASan / UBSan, then the CPU tests under it
+    python ops-sparse_amd/build.py --coverage # a copy whose host code counts executed lines (see below)
 
 Every translation unit is compiled to an object under ops-sparse_amd/build/
 (in parallel) and linked into one shared library.  The library carries both
@@ -173,7 +174,97 @@ def run_asan():
     return rc
 
 
+# ---- which dispatch arms the tests reach ---------------------------------------------------------------------------
+# `python ops-sparse_amd/build.py --coverage` builds lib/cov/libops_sparse.so with the HOST code counting executed
+# lines (gcov format; device code as always).  Run any tests against it,
+#     OPS_SPARSE_LIBRARY=ops-sparse_amd/lib/cov/libops_sparse.so GCOV_PREFIX=<dir> python -m pytest tests -m gpu
+# (the counts are written at process exit below <dir>, or beside the objects without GCOV_PREFIX), then
+# `python ops-sparse_amd/build.py --coverage-report <dir> [<dir> ...]` lists, per source file, the host lines that
+# no run under any of the directories executed.
+COV_LIB_DIR = os.path.join(LIB_DIR, "cov")
+COV_OBJ_DIR = OBJ_DIR + "_cov"
+
+
+def build_coverage(verbose=True):
+    os.makedirs(COV_OBJ_DIR, exist_ok=True)
+    os.makedirs(COV_LIB_DIR, exist_ok=True)
+    flags = COMMON_FLAGS + ["-Xarch_host", "--coverage", "-Xarch_host", "-O0"]
+
+    def compile_one(src):
+        obj = os.path.join(COV_OBJ_DIR, os.path.splitext(src)[0] + ".o")
+        proc = subprocess.run([hipcc(), "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj] + flags,
+                              capture_output=True, text=True, cwd=ROOT)
+        if proc.returncode != 0:
+            raise RuntimeError("hipcc failed for %s:\n%s" % (src, proc.stderr))
+        return obj
+
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+        objs = list(pool.map(compile_one, SOURCES))
+    lib = os.path.join(COV_LIB_DIR, "libops_sparse.so")
+    runtime = os.path.join(_clang_dir(), "lib", "linux", "libclang_rt.profile-x86_64.a")
+    proc = subprocess.run([hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-o", lib] + objs + [runtime],
+                          capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("link failed:\n" + proc.stderr)
+    if verbose:
+        print("built", lib)
+    return lib
+
+
+def coverage_report(count_dirs):
+    """Sums the line counts of every run found below `count_dirs`; prints the host lines never executed."""
+    import collections
+    import glob
+    import tempfile
+    executed = collections.defaultdict(set)
+    known = collections.defaultdict(dict)
+    runs = []
+    for d in count_dirs:
+        for path in glob.glob(os.path.join(d, "**", "*.gcda"), recursive=True):
+            runs.append(path)
+    if not runs:
+        print("no counts found below", count_dirs)
+        return 1
+    for gcda in runs:
+        stem = os.path.splitext(os.path.basename(gcda))[0]
+        gcno = os.path.join(COV_OBJ_DIR, stem + ".gcno")
+        with tempfile.TemporaryDirectory() as tmp:
+            shutil.copy(gcda, tmp)
+            shutil.copy(gcno, tmp)
+            os.symlink(HERE, os.path.join(tmp, os.path.basename(HERE)))    # the notes name sources relative to ROOT
+            subprocess.run(["gcov", "-o", tmp, stem + ".o"], cwd=tmp, capture_output=True, text=True)
+            for out in glob.glob(os.path.join(tmp, "*.gcov")):
+                name = os.path.basename(out)[:-5]
+                if not os.path.exists(os.path.join(CSRC, name)):
+                    continue            # system and ROCm headers
+                for line in open(out, errors="replace"):
+                    parts = line.split(":", 2)
+                    if len(parts) < 3:
+                        continue
+                    count, number = parts[0].strip(), int(parts[1])
+                    if number == 0 or count == "-":
+                        continue
+                    known[name][number] = parts[2].rstrip("\n")
+                    if count not in ("#####", "====="):
+                        executed[name].add(number)
+    total = missed = 0
+    for name in sorted(known):
+        lines = sorted(n for n in known[name] if n not in executed[name])
+        total += len(known[name])
+        missed += len(lines)
+        print("%s: %d of %d host lines never executed" % (name, len(lines), len(known[name])))
+        for n in lines:
+            print("    %5d:%s" % (n, known[name][n]))
+    print("total: %d of %d host lines never executed" % (missed, total))
+    return 0
+
+
 if __name__ == "__main__":
     if "--asan" in sys.argv[1:]:
         sys.exit(run_asan())
+    if "--coverage" in sys.argv[1:]:
+        build_coverage()
+        sys.exit(0)
+    if "--coverage-report" in sys.argv[1:]:
+        sys.exit(coverage_report(sys.argv[sys.argv.index("--coverage-report") + 1:]))
     build_library()

@@ -985,7 +985,7 @@ int RowStats(const int32_t *rowOffsets, int64_t rows, int32_t *scratch, hipStrea
 // to the kernel with a lane group a row (for measurements).
 bool NoBinning()
 {
-    static const bool force = std::getenv("OPS_SPARSE_SPMM_NO_BINNING") != nullptr;
+    const bool force = std::getenv("OPS_SPARSE_SPMM_NO_BINNING") != nullptr;
     return force;
 }
 
@@ -1038,7 +1038,7 @@ void LaunchLongRows(const SpmmArgs &a)
 // exceeds its LDS) and one column tile per lane group.
 bool UseSlabKernel(const SpmmArgs &a, int64_t lanesNeeded)
 {
-    static const bool off = std::getenv("OPS_SPARSE_SPMM_NO_SLAB") != nullptr;
+    const bool off = std::getenv("OPS_SPARSE_SPMM_NO_SLAB") != nullptr;  // (read at every call: tests switch it)
     if (off || a.plan == nullptr || lanesNeeded > 64 * 65535) {
         return false;
     }
@@ -1054,12 +1054,12 @@ int LaunchSlab(const SpmmArgs &a)
 {
     const bool binned = a.plan->kernel == OPSPARSE_SPMM_BINNED && a.plan->numLongRows > 0;
     // Slabs of about kSlabTarget entries: of equal work from the plan's table, of equal numbers of rows without it.
-    static const int64_t target = std::getenv("OPS_SPARSE_SPMM_SLAB_ENTRIES") != nullptr
+    const int64_t target = std::getenv("OPS_SPARSE_SPMM_SLAB_ENTRIES") != nullptr
                                       ? std::atoll(std::getenv("OPS_SPARSE_SPMM_SLAB_ENTRIES"))
                                       : kSlabTarget;
     int64_t rps = a.nnz > 0 ? target * a.rows / a.nnz : 4096;
     rps = rps < 16 ? 16 : (rps > 4096 ? 4096 : rps);
-    static const bool noTable = std::getenv("OPS_SPARSE_SPMM_NO_SLAB_TABLE") != nullptr;
+    const bool noTable = std::getenv("OPS_SPARSE_SPMM_NO_SLAB_TABLE") != nullptr;
     const bool table = !noTable && a.plan->slabStartOff > 0 && a.plan->numSlabs > 0;
     const int32_t *slabStart =
         table ? reinterpret_cast<const int32_t *>(static_cast<unsigned char *>(a.ws) + a.plan->slabStartOff) : nullptr;
@@ -1132,8 +1132,9 @@ int RunGeneral(const SpmmArgs &a)
     return LaunchGeneral<ValT, CT, AccT, 64>(a);
 }
 
-// V elements of B per lane and gather.
-template <typename ValT, typename CT, typename AccT, int V>
+// V elements of B per lane and gather.  LMin .. LMax: the widths of lane group that the caller's range of n can ask
+// for (the others are not compiled).
+template <typename ValT, typename CT, typename AccT, int V, int LMin = 2, int LMax = 64>
 int RunTypedV(const SpmmArgs &a)
 {
     const bool fast = !a.bColMajor && !a.cColMajor && !a.transB && a.n % V == 0 && a.ldb % V == 0 &&
@@ -1143,20 +1144,21 @@ int RunTypedV(const SpmmArgs &a)
         return RunGeneral<ValT, CT, AccT>(a);
     }
     const int64_t lanesNeeded = a.n / V;
-    if (UseSlabKernel(a, lanesNeeded)) {
-        if (lanesNeeded <= 2) return LaunchSlab<ValT, CT, AccT, V, 2>(a);
-        if (lanesNeeded <= 4) return LaunchSlab<ValT, CT, AccT, V, 4>(a);
-        if (lanesNeeded <= 8) return LaunchSlab<ValT, CT, AccT, V, 8>(a);
-        if (lanesNeeded <= 16) return LaunchSlab<ValT, CT, AccT, V, 16>(a);
-        if (lanesNeeded <= 32) return LaunchSlab<ValT, CT, AccT, V, 32>(a);
-        return LaunchSlab<ValT, CT, AccT, V, 64>(a);
-    }
-    if (lanesNeeded <= 2) return LaunchRowSplit<ValT, CT, AccT, V, 2>(a);
-    if (lanesNeeded <= 4) return LaunchRowSplit<ValT, CT, AccT, V, 4>(a);
-    if (lanesNeeded <= 8) return LaunchRowSplit<ValT, CT, AccT, V, 8>(a);
-    if (lanesNeeded <= 16) return LaunchRowSplit<ValT, CT, AccT, V, 16>(a);
-    if (lanesNeeded <= 32) return LaunchRowSplit<ValT, CT, AccT, V, 32>(a);
-    return LaunchRowSplit<ValT, CT, AccT, V, 64>(a);
+    const bool slab = UseSlabKernel(a, lanesNeeded);
+    auto launch = [&](auto tag) {
+        constexpr int L = decltype(tag)::value;
+        if constexpr (L >= LMin && L <= LMax) {
+            return slab ? LaunchSlab<ValT, CT, AccT, V, L>(a) : LaunchRowSplit<ValT, CT, AccT, V, L>(a);
+        } else {
+            return static_cast<int>(OPSPARSE_E_INVALID);  // (n outside the range this V is called for)
+        }
+    };
+    if (lanesNeeded <= 2) return launch(std::integral_constant<int, 2>{});
+    if (lanesNeeded <= 4) return launch(std::integral_constant<int, 4>{});
+    if (lanesNeeded <= 8) return launch(std::integral_constant<int, 8>{});
+    if (lanesNeeded <= 16) return launch(std::integral_constant<int, 16>{});
+    if (lanesNeeded <= 32) return launch(std::integral_constant<int, 32>{});
+    return launch(std::integral_constant<int, 64>{});
 }
 
 template <typename ValT, typename CT, typename AccT>
@@ -1333,9 +1335,10 @@ int opsparse_spmm_csr_launch(const OpsparseSpmmPlan *plan, const int32_t *rowOff
         // per gather outweigh the gather itself (1 M rows of 32, n = 256: 6.1 ms with 16, 1.65 ms with 8, 2.7 ms
         // with 4; n = 16: 0.50 ms with 4, 0.54 ms with 8; the one-column-per-lane kernel 10.6 ms and 0.72 ms).
         if (a.n <= 32) {
-            return RunTypedV<int8_t, int32_t, int32_t, 4>(a);
+            return RunTypedV<int8_t, int32_t, int32_t, 4, 2, 8>(a);   // n / 4 <= 8 lanes
         }
-        return RunTypedV<int8_t, int32_t, int32_t, 8>(a);
+        return RunTypedV<int8_t, int32_t, int32_t, 8, 8, 64>(a);      // n / 8 >= 5 lanes
+
     }
     return OPSPARSE_E_UNSUPPORTED;
 }

@@ -2023,7 +2023,7 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     window = window > kMaxBlockEntries / 2 ? kMaxBlockEntries / 2 : window;
     // Values that the layout keeps (frozen values, either op(A)) are kept in block order and streamed by a wavefront
     // a block; values read where the caller has them need the windowed blocks, which read them in row order.
-    static const bool noStream = std::getenv("OPS_SPARSE_BLOCKED_NO_STREAM") != nullptr;  // tuning switch
+    const bool noStream = std::getenv("OPS_SPARSE_BLOCKED_NO_STREAM") != nullptr;  // tuning switch
     l.streamed = !live && !noStream;
     if (l.streamed) {
         // Streamed blocks are cut by their rows; the entry cut is there for matrices of few, long rows, which would
@@ -2049,7 +2049,7 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
     // for op(A) = A with frozen values, a compact copy without the long rows' values, whose entries are stored a
     // second time with their values.
     const bool frozenCopy = !live && !transposed;
-    static const bool noLong = std::getenv("OPS_SPARSE_BLOCKED_NO_LONG_ROWS") != nullptr;
+    const bool noLong = std::getenv("OPS_SPARSE_BLOCKED_NO_LONG_ROWS") != nullptr;
     if (!noLong) {
         static const int64_t chunkMean = [] {  // tuning override: entries a long row has per panel at least, on average
             const char *env = std::getenv("OPS_SPARSE_BLOCKED_LONG_MEAN");

@@ -1123,11 +1123,13 @@ struct BlockedLayout {
 
 // Layout for a product with `rows` outputs and `cols` inputs (op(A) = A^T: the columns of A are the outputs).
 // 0 panels: the layout does not apply.
-BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool transposed, bool live)
+BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz)
 {
+    // This file's layout is the one with live values for op(A) = A; the arms below that ask are those of the
+    // ordered layout it grew out of (spmv_blocked.hip), which the compiler drops here.
+    constexpr bool transposed = false, live = true;
     BlockedLayout l{};
-    if (rows <= 0 || cols <= 0 || nnz <= 0 || nnz > INT32_MAX || rows >= INT32_MAX || cols > INT32_MAX ||
-        (live && transposed)) {  // live values follow the caller's row order: op(A) = A only
+    if (rows <= 0 || cols <= 0 || nnz <= 0 || nnz > INT32_MAX || rows >= INT32_MAX || cols > INT32_MAX) {
         return l;
     }
     const int64_t P = (cols + kPanelCols - 1) >> kPanelLog;
@@ -1168,7 +1170,7 @@ BlockedLayout MakeBlockedLayout(int64_t rows, int64_t cols, int64_t nnz, bool tr
         ++bits;
     }
     l.passes = (bits + 3) / 4;
-    static const bool noLong = std::getenv("OPS_SPARSE_BLOCKED_NO_LONG_ROWS") != nullptr;
+    const bool noLong = std::getenv("OPS_SPARSE_BLOCKED_NO_LONG_ROWS") != nullptr;
     if (!transposed && !noLong) {
         static const int64_t chunkMean = [] {  // tuning override: entries a long row has per panel at least, on average
             const char *env = std::getenv("OPS_SPARSE_BLOCKED_LONG_MEAN");
@@ -1270,7 +1272,7 @@ int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valTy
         return OPSPARSE_E_UNSUPPORTED;  // y is fp32, or of the 16-bit type of the values
     }
     // a.rows outputs, a.cols inputs: the caller has exchanged them for op(A) = A^T
-    const BlockedLayout l = MakeBlockedLayout(a.rows, a.cols, a.nnz, plan.transposed != 0, plan.liveValues != 0);
+    const BlockedLayout l = MakeBlockedLayout(a.rows, a.cols, a.nnz);
     if (l.P == 0 || plan.numPanels != l.P || plan.numRowBlocks != l.B) {
         return OPSPARSE_E_INVALID;
     }
@@ -1364,12 +1366,12 @@ extern "C" {
 
 size_t opsparse_spmv_csr_live_workspace_bytes(int64_t rows, int64_t cols, int64_t nnz)
 {
-    return static_cast<size_t>(MakeBlockedLayout(rows, cols, nnz, false, true).bytes);
+    return static_cast<size_t>(MakeBlockedLayout(rows, cols, nnz).bytes);
 }
 
 size_t opsparse_spmv_csr_live_resident_bytes(int64_t rows, int64_t cols, int64_t nnz)
 {
-    return static_cast<size_t>(MakeBlockedLayout(rows, cols, nnz, false, true).resident);
+    return static_cast<size_t>(MakeBlockedLayout(rows, cols, nnz).resident);
 }
 
 int opsparse_spmv_csr_live_analyse_split(const int32_t *rowOffsets, const int32_t *colInd, const void *csrValues,
@@ -1388,8 +1390,7 @@ int opsparse_spmv_csr_live_analyse_split(const int32_t *rowOffsets, const int32_
                               : (flags & OPSPARSE_BLOCKED_VALUES_BF16) != 0 ? OPSPARSE_BF16
                                                                             : OPSPARSE_F32;
     const int64_t outputs = transposed ? cols : rows;
-    const BlockedLayout l = transposed ? MakeBlockedLayout(cols, rows, nnz, true, live)
-                                       : MakeBlockedLayout(rows, cols, nnz, false, live);
+    const BlockedLayout l = MakeBlockedLayout(rows, cols, nnz);
     if (l.P == 0) {
         return OPSPARSE_E_UNSUPPORTED;
     }

@@ -1341,7 +1341,7 @@ int LaunchStreamTiles(const SpmvArgs &a, int32_t rowsPerBlock, int32_t tileRowNn
     const size_t lds = products * sizeof(AccT);
     if constexpr (G == 1 && std::is_same<OutT, float>::value) {
         // Four rows per lane with vector row offsets / y where the shapes allow it.
-        static const bool quadOff = std::getenv("OPS_SPARSE_STREAM_NO_QUAD_ROWS") != nullptr;
+        const bool quadOff = std::getenv("OPS_SPARSE_STREAM_NO_QUAD_ROWS") != nullptr;
         if (!quadOff && rowsPerBlock % 4 == 0 && rowsPerBlock <= 4 * kBlockThreads &&
             reinterpret_cast<uintptr_t>(a.rowOffsets) % 16 == 0 && reinterpret_cast<uintptr_t>(a.y) % 16 == 0 &&
             reinterpret_cast<uintptr_t>(a.yIn) % 16 == 0) {
@@ -1824,7 +1824,6 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
     const int64_t nnzShort = nnz - static_cast<int64_t>(static_cast<uint32_t>(seen[3]));
     p.maxRowNnz = maxRow;
 
-    const double mean = static_cast<double>(nnz) / static_cast<double>(rows);
     int32_t kernel = forceKernel;
     if (kernel == OPSPARSE_SPMV_AUTO) {
         // Measured on 64 M entries, even rows and rows of 0.5 - 1.5 times the mean, banded and random columns:
@@ -1835,7 +1834,8 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
         // Since the stream-rows tiles take rows of up to 512 entries (8 - 64 lanes a row), even rows of 49 - 512
         // entries are theirs as well: 40 M entries in a band, 60 - 512 a row, 65 - 75 us against 64 - 116 us with a
         // lane group a row or the merge path (100 a row: 117 -> 74 us), and random columns 167 - 186 us against
-        // 165 - 250 us.
+        // 165 - 250 us.  That leaves nothing for the lane-group-a-row kernel to be chosen for here: it serves
+        // forced plans and calls that come without a workspace.
         if (maxRow <= kStreamMaxRow && (maxRow <= 12 || static_cast<double>(maxRow) * static_cast<double>(rows) <=
                                                             1.25 * static_cast<double>(nnz))) {
             kernel = OPSPARSE_SPMV_STREAM_ROWS;
@@ -1850,8 +1850,6 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
             kernel = OPSPARSE_SPMV_STREAM_ROWS;
             p.longRowsBeside = 1;
             p.tileRowNnz = maxShort;
-        } else if (mean >= 96.0 && mean <= 400.0 && static_cast<double>(maxRow) <= 1.125 * mean) {
-            kernel = OPSPARSE_SPMV_VECTOR_ROWS;
         } else {
             kernel = OPSPARSE_SPMV_MERGE_PATH;
         }
@@ -1876,12 +1874,10 @@ int opsparse_spmv_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t c
             p.rowsPerBlock = rpb < 4 ? 4 : rpb;
             if (tileRow > 48) {
                 // Few rows a tile: as many as the lane groups sum in whole turns (a band of 81 entries a row: 32
-                // rows 68.7 us, 25 rows 73.2 us, 37 rows 75.5 us); where not even one turn fits the 3072 slots, two
-                // rounds of loads or three, whichever the rows fill better.
+                // rows 68.7 us, 25 rows 73.2 us, 37 rows 75.5 us) within the 3072 slots.  (g lanes serve rows of up
+                // to 12 g entries, so at least one turn of the 256 / g groups always fits.)
                 const int32_t groups = kBlockThreads / g;
-                const int32_t r2 = 2048 / tileRow, r3 = 3072 / tileRow;
-                p.rowsPerBlock = r3 >= groups ? r3 / groups * groups
-                                              : (static_cast<int64_t>(r2) * 3 >= static_cast<int64_t>(r3) * 2 ? r2 : r3);
+                p.rowsPerBlock = 3072 / tileRow / groups * groups;
             }
             if (const char *env = std::getenv("OPS_SPARSE_STREAM_ROWS")) {
                 const int v = std::atoi(env);  // tuning override
