@@ -5,6 +5,7 @@ hipcc cross-compiles without a GPU, so this runs anywhere ROCm is installed:
     python ops-sparse_amd/build.py
     python ops-sparse_amd/build.py --asan     # host code under ASan / UBSan, then the CPU tests under it
     python ops-sparse_amd/build.py --coverage # a copy whose host code counts executed lines (see below)
+    python ops-sparse_amd/build.py --kernel-coverage <dirs>   # kernels that traced test runs never launched
 
 Every translation unit is compiled to an object under ops-sparse_amd/build/
 (in parallel) and linked into one shared library.  The library carries both
@@ -130,22 +131,23 @@ def build_asan(verbose=True):
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objs = list(pool.map(compile_one, SOURCES))
     lib = os.path.join(ASAN_LIB_DIR, "libops_sparse.so")
-    link = [hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-fsanitize=address", "-fsanitize=undefined",
-            "-shared-libsan", "-o", lib] + objs
+    link = [hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-fno-gpu-sanitize", "-fsanitize=address",
+            "-fsanitize=undefined", "-shared-libsan", "-o", lib] + objs
     proc = subprocess.run(link, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError("link failed:\n" + proc.stderr)
     clang = os.path.join(_clang_dir().rstrip("/").rsplit("/lib/clang", 1)[0], "bin", "clang")  # (the hipcc's own)
     oracle_lib = os.path.join(ASAN_LIB_DIR, "liboracle.so")
     proc = subprocess.run([clang, "-O1", "-g", "-std=c99", "-fPIC", "-shared", "-ffp-contract=off", "-fopenmp",
-                           "-fsanitize=address", "-fsanitize=undefined", "-fno-sanitize-recover=undefined",
+                           "-fno-gpu-sanitize", "-fsanitize=address", "-fsanitize=undefined", "-fno-sanitize-recover=undefined",
                            "-shared-libsan", "-fno-omit-frame-pointer", "-o", oracle_lib,
                            os.path.join(ROOT, "oracle", "oracle.c"), "-lm"], capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError("the checker failed to build under the sanitizers:\n" + proc.stderr)
     selftest = os.path.join(ASAN_LIB_DIR, "frame_selftest")
-    proc = subprocess.run([hipcc(), "-std=c++17", "-O1", "-g", "-fsanitize=address", "-fsanitize=undefined",
-                           "-fno-sanitize-recover=undefined", "-shared-libsan", "-I" + os.path.join(ROOT, "include"),
+    proc = subprocess.run([hipcc(), "-std=c++17", "-O1", "-g", "-fno-gpu-sanitize", "-fsanitize=address",
+                           "-fsanitize=undefined", "-fno-sanitize-recover=undefined", "-shared-libsan",
+                           "-I" + os.path.join(ROOT, "include"),
                            "-I" + os.path.join(ROOT, "tests", "cpp"),
                            os.path.join(ROOT, "tests", "cpp", "frame_selftest.cpp"), "-o", selftest,
                            "-L" + ASAN_LIB_DIR, "-lops_sparse", "-loracle", "-Wl,-rpath," + ASAN_LIB_DIR,
@@ -167,7 +169,8 @@ def run_asan():
     # (CPython and numpy keep their arenas until exit: no leak report; another preloaded library may come first)
     env["ASAN_OPTIONS"] = "detect_leaks=0:verify_asan_link_order=0:abort_on_error=1"
     env["UBSAN_OPTIONS"] = "print_stacktrace=0:halt_on_error=0"
-    tests = [os.path.join(ROOT, "tests", t) for t in ("test_abi_status.py", "test_oracle.py", "test_oracle_convert.py")]
+    names = ("test_abi_status.py", "test_launch_layer_status.py", "test_oracle.py", "test_oracle_convert.py")
+    tests = [os.path.join(ROOT, "tests", t) for t in names]
     rc = subprocess.run([sys.executable, "-m", "pytest", "-x", "-q", "-m", "not gpu"] + tests, env=env, cwd=ROOT).returncode
     if rc == 0:
         rc = subprocess.run([selftest, os.path.join(ROOT, "tests", "golden")], env=env).returncode
@@ -259,7 +262,37 @@ def coverage_report(count_dirs):
     return 0
 
 
+def kernel_coverage(trace_dirs):
+    """Which kernel instantiations of the built library no traced run launched.  `trace_dirs` hold the
+    `*kernel_stats.csv` files of `rocprofv3 --kernel-trace --stats -M --output-format csv -d <dir> -- python3 -m pytest
+    tests/<file> -m gpu` runs (-M: mangled names, which is what the library's symbol table has)."""
+    import csv
+    import glob
+    import re
+    out = subprocess.run(["nm", LIB_PATH], capture_output=True, text=True, check=True).stdout
+    compiled = set()
+    for line in out.splitlines():
+        m = re.search(r"\s(_Z\S*?)(\d+)__device_stub__(\S+)$", line)
+        if m:  # the host stub of a kernel: its name with "__device_stub__" in front of the last component
+            compiled.add(m.group(1) + str(int(m.group(2)) - len("__device_stub__")) + m.group(3))
+    launched = set()
+    for d in trace_dirs:
+        for path in glob.glob(os.path.join(d, "**", "*kernel_stats.csv"), recursive=True):
+            with open(path, newline="") as f:
+                for row in csv.DictReader(f):
+                    launched.add(row["Name"].replace(".kd", ""))
+    missing = sorted(compiled - launched)
+    print("%d kernel instantiations in %s, %d of them never launched by the traced runs" %
+          (len(compiled), os.path.relpath(LIB_PATH, ROOT), len(missing)))
+    if missing:
+        shown = subprocess.run(["c++filt"], input="\n".join(missing), capture_output=True, text=True).stdout
+        print(shown.rstrip())
+    return 1 if missing else 0
+
+
 if __name__ == "__main__":
+    if "--kernel-coverage" in sys.argv[1:]:
+        sys.exit(kernel_coverage(sys.argv[sys.argv.index("--kernel-coverage") + 1:]))
     if "--asan" in sys.argv[1:]:
         sys.exit(run_asan())
     if "--coverage" in sys.argv[1:]:
