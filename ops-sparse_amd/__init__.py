@@ -21,8 +21,7 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# OPS_SPARSE_LIB points at another build of the library (kernel tuning experiments).
-LIB_PATH = os.environ.get("OPS_SPARSE_LIB") or os.path.join(_HERE, "lib", "libops_sparse.so")
+LIB_PATH = os.path.join(_HERE, "lib", "libops_sparse.so")
 
 # ---- aclDataType (include/acl/acl_base_rt.h)
 ACL_FLOAT, ACL_FLOAT16, ACL_INT8, ACL_INT32 = 0, 1, 2, 3
@@ -145,7 +144,7 @@ def lib():
     global _lib
     if _lib is not None:
         return _lib
-    # (OPS_SPARSE_LIBRARY: another build of the same library, e.g. the one `build.py --asan` makes)
+    # (OPS_SPARSE_LIBRARY: another build of the same library, e.g. the ones `build.py --asan` / `--coverage` make)
     path = os.environ.get("OPS_SPARSE_LIBRARY") or LIB_PATH
     if not os.path.exists(path):
         raise RuntimeError(
