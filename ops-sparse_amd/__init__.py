@@ -61,6 +61,7 @@ OPSPARSE_OK, OPSPARSE_E_INVALID, OPSPARSE_E_UNSUPPORTED, OPSPARSE_E_WORKSPACE, O
 OPSPARSE_SPMV_COLUMN_PANELS = 5
 OPSPARSE_SPMV_BLOCKED_GATHER = 6
 OPSPARSE_SPMV_BLOCKED_LIVE = 7
+OPSPARSE_SPMV_SCATTER_LIVE = 8
 OPSPARSE_BLOCKED_TRANSPOSE, OPSPARSE_BLOCKED_LIVE_VALUES = 1, 2
 OPSPARSE_BLOCKED_VALUES_F16, OPSPARSE_BLOCKED_VALUES_BF16, OPSPARSE_BLOCKED_VALUES_I32 = 4, 8, 16
 OPSPARSE_SPMM_AUTO, OPSPARSE_SPMM_ROW_SPLIT, OPSPARSE_SPMM_BINNED = range(3)
@@ -99,6 +100,8 @@ OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_blocked_analyse",
     "opsparse_spmv_csr_live_workspace_bytes", "opsparse_spmv_csr_live_resident_bytes", "opsparse_spmv_csr_live_analyse",
     "opsparse_spmv_csr_live_analyse_split", "opsparse_spmv_csr_blocked_analyse_split",
+    "opsparse_spmv_csr_scatter_workspace_bytes", "opsparse_spmv_csr_scatter_resident_bytes",
+    "opsparse_spmv_csr_scatter_analyse", "opsparse_spmv_csr_scatter_analyse_split",
     "opsparse_spmv_csr_gathers_scattered",
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
     "opsparse_dense_restage",
@@ -271,6 +274,14 @@ def lib():
     L.opsparse_spmv_csr_live_workspace_bytes.argtypes = [i64, i64, i64]
     L.opsparse_spmv_csr_live_resident_bytes.restype = sz
     L.opsparse_spmv_csr_live_resident_bytes.argtypes = [i64, i64, i64]
+    for name in ("opsparse_spmv_csr_scatter_workspace_bytes", "opsparse_spmv_csr_scatter_resident_bytes"):
+        getattr(L, name).restype = sz
+        getattr(L, name).argtypes = [i64, i64, i64, i32]
+    L.opsparse_spmv_csr_scatter_analyse.restype = ctypes.c_int
+    L.opsparse_spmv_csr_scatter_analyse.argtypes = [vp, vp, i64, i64, i64, i32, vp, sz, ctypes.POINTER(OpsparseSpmvPlan), vp]
+    L.opsparse_spmv_csr_scatter_analyse_split.restype = ctypes.c_int
+    L.opsparse_spmv_csr_scatter_analyse_split.argtypes = [vp, vp, i64, i64, i64, i32, vp, sz, vp, sz,
+                                                          ctypes.POINTER(OpsparseSpmvPlan), vp]
     L.opsparse_spmv_csr_live_analyse.restype = ctypes.c_int
     L.opsparse_spmv_csr_live_analyse.argtypes = [vp, vp, vp, i64, i64, i64, i32, vp, sz,
                                                  ctypes.POINTER(OpsparseSpmvPlan), vp]

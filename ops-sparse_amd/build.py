@@ -35,6 +35,7 @@ SOURCES = [
     "spmv_kernels.hip",
     "spmv_blocked.hip",
     "spmv_blocked_live.hip",
+    "spmv_scatter.hip",
     "spmm_kernels.hip",
     "convert_kernels.hip",
     "measure_kernels.hip",

@@ -178,10 +178,12 @@ bool SizedFor(aclsparseConstSpMatDescr_t matA, const RestoredChoice &choice, boo
 // valueType: the OPSPARSE_* type of the values and of x.
 RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool transpose, int32_t valueType);
 // `scratch` / `scratchBytes`: where the analysis works when the buffer only has room for what the launches keep
-// (scratchBytes == 0: behind that, in the buffer itself).
+// (scratchBytes == 0: behind that, in the buffer itself).  `mayVary`: the caller's algorithm value lets the last bit
+// of a result differ between calls (aclsparseSpMV with ALG_DEFAULT / CSR_ALG1): op(A) = A^T may then take the
+// SCATTER_LIVE layout inside the same buffer.
 int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const void *values,
                     int32_t valueType, int64_t rows, int64_t cols, int64_t nnz, bool transpose, bool liveValues,
                     void *buffer, size_t bytes, void *scratch, size_t scratchBytes, OpsparseSpmvPlan *plan,
-                    void *stream);
+                    void *stream, bool mayVary = false);
 
 }  // namespace opsparse

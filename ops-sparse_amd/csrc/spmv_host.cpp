@@ -337,7 +337,7 @@ RestoredChoice PickRestoredLayout(int64_t rows, int64_t cols, int64_t nnz, bool 
 int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *colInd, const void *values,
                     int32_t valueType, int64_t rows, int64_t cols, int64_t nnz, bool transpose, bool liveValues,
                     void *buffer, size_t bytes, void *scratch, size_t scratchBytes, OpsparseSpmvPlan *plan,
-                    void *stream)
+                    void *stream, bool mayVary)
 {
     // A matrix whose gathers stay near the diagonal (a mesh, a band) keeps x in cache under the row-wise kernels:
     // those are then faster than any re-stored layout (the 2048 x 2048 Laplacian: 41 us against 91 us).  With some
@@ -369,6 +369,27 @@ int AnalyseRestored(int32_t kernel, const int32_t *rowOffsets, const int32_t *co
                                                                        buffer, bytes, scratch, scratchBytes, plan, stream)
                                 : opsparse_spmv_csr_live_analyse(rowOffsets, colInd, values, rows, cols, nnz, flags, buffer,
                                                                  bytes, plan, stream);
+    }
+    if (kernel == OPSPARSE_SPMV_BLOCKED_GATHER && transpose && liveValues && mayVary && valueType != OPSPARSE_I32 &&
+        std::getenv("OPS_SPARSE_SPMV_NO_SCATTER") == nullptr) {
+        // op(A) = A^T where the last bit may differ between calls, as it may under the reference's atomics on y:
+        // the layout that sorts the products by output panel through LDS and needs no transposed copy (the 8 M x 8 M
+        // power-law matrix: 0.3 ms a call against 1.4 ms), where the matrix is one for it.  Its buffer is smaller
+        // than the ordered layout's, which the size query answered with; where it does not apply (a column with
+        // thousands of entries, fewer than 2 M columns) the ordered layout over the transposed copy follows.
+        const int32_t flags = BlockedFlags(false, true, valueType);
+        const size_t need = opsparse_spmv_csr_scatter_workspace_bytes(rows, cols, nnz, flags);
+        const size_t keep = opsparse_spmv_csr_scatter_resident_bytes(rows, cols, nnz, flags);
+        int rc = OPSPARSE_E_UNSUPPORTED;
+        if (need > 0 && scratchBytes > 0 && keep <= bytes && need - keep <= scratchBytes) {
+            rc = opsparse_spmv_csr_scatter_analyse_split(rowOffsets, colInd, rows, cols, nnz, flags, buffer, bytes, scratch,
+                                                         scratchBytes, plan, stream);
+        } else if (need > 0 && scratchBytes == 0 && need <= bytes) {
+            rc = opsparse_spmv_csr_scatter_analyse(rowOffsets, colInd, rows, cols, nnz, flags, buffer, bytes, plan, stream);
+        }
+        if (rc != OPSPARSE_E_UNSUPPORTED && rc != OPSPARSE_E_WORKSPACE) {
+            return rc;
+        }
     }
     if (kernel == OPSPARSE_SPMV_BLOCKED_GATHER) {
         const int32_t flags = BlockedFlags(transpose, liveValues, valueType);
@@ -465,7 +486,9 @@ aclsparseStatus_t aclsparseSpMVPreprocess(aclsparseHandle_t handle, aclsparseOpe
                                        RestoredValueType(matA, vecX), matA->rows, matA->cols, matA->nnz,
                                        opA != ACL_SPARSE_OP_NON_TRANSPOSE, restored.liveValues, externalBuffer,
                                        restored.keep, restored.scratch > 0 ? handle->userWorkspace : nullptr,
-                                       restored.scratch > 0 ? handle->userWorkspaceBytes : 0, &plan, handle->stream);
+                                       restored.scratch > 0 ? handle->userWorkspaceBytes : 0, &plan, handle->stream,
+                                       alg != ACL_SPARSE_SPMV_CSR_ALG2 &&
+                                           std::getenv("OPS_SPARSE_SPMV_REPEATABLE") == nullptr);
     } else {
         const size_t bytes = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
         rc = opsparse_spmv_csr_analyse(static_cast<const int32_t *>(matA->rowOffsets), matA->rows, matA->cols,
@@ -518,7 +541,8 @@ aclsparseStatus_t aclsparseSpMV(aclsparseHandle_t handle, aclsparseOperation_t o
     const bool bound = externalBuffer != nullptr && matA->spmv.buffer == externalBuffer &&
                        matA->spmv.plan.rows == matA->rows && matA->spmv.plan.nnz == matA->nnz;
     const bool blockedPlan = bound && (matA->spmv.plan.kernel == OPSPARSE_SPMV_BLOCKED_GATHER ||
-                                       matA->spmv.plan.kernel == OPSPARSE_SPMV_BLOCKED_LIVE);
+                                       matA->spmv.plan.kernel == OPSPARSE_SPMV_BLOCKED_LIVE ||
+                                       matA->spmv.plan.kernel == OPSPARSE_SPMV_SCATTER_LIVE);
     if (blockedPlan && (matA->spmv.plan.transposed != 0) != c.transpose) {
         // Preprocess built the re-stored layout for the other op(A): this call runs without it
         if (matA->nnz > 0 || (c.transpose && c.outType != OPSPARSE_F32)) {

@@ -38,4 +38,9 @@ namespace live_layout {
 int LaunchBlocked(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valType, int32_t outType);
 }
 
+// SCATTER_LIVE launch (spmv_scatter.hip): op(A) = A^T; a.rows / a.cols are those of A.
+namespace scatter_layout {
+int Launch(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valType, int32_t outType);
+}
+
 }  // namespace opsparse

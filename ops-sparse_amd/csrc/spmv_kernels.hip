@@ -1477,6 +1477,7 @@ int RunPlanned(const SpmvArgs &a, const OpsparseSpmvPlan &plan)
             }
         case OPSPARSE_SPMV_BLOCKED_GATHER:
         case OPSPARSE_SPMV_BLOCKED_LIVE:
+        case OPSPARSE_SPMV_SCATTER_LIVE:
             return OPSPARSE_E_INVALID;  // (launched before the types are dispatched: opsparse_spmv_csr_launch_zy)
         default:
             return OPSPARSE_E_INVALID;
@@ -2066,6 +2067,12 @@ int opsparse_spmv_csr_launch_zy(const OpsparseSpmvPlan *plan, int32_t transpose,
 
     if (plan != nullptr && plan->kernel == OPSPARSE_SPMV_BLOCKED_GATHER && (plan->transposed != 0) != (transpose != 0)) {
         return OPSPARSE_E_INVALID;  // the re-stored layout serves the op(A) it was built for
+    }
+    if (plan != nullptr && plan->kernel == OPSPARSE_SPMV_SCATTER_LIVE && nnz > 0) {
+        if (!transpose || computeIsInt) {
+            return OPSPARSE_E_INVALID;  // (built for op(A) = A^T and floating-point sums)
+        }
+        return scatter_layout::Launch(a, *plan, valType, outType);
     }
     if (plan != nullptr && plan->kernel == OPSPARSE_SPMV_BLOCKED_LIVE && nnz > 0) {
         if (transpose || computeIsInt) {
