@@ -428,6 +428,12 @@ def run_workload(args, osa, wl, torch, dev, stream, handle, key, cpu_cache):
             layout = "blocked_gather_live_values"
             resident = L.opsparse_spmv_csr_blocked_resident_bytes(rows, cols, nnz,
                                                                   tflag | osa.OPSPARSE_BLOCKED_LIVE_VALUES)
+            scatter = L.opsparse_spmv_csr_scatter_resident_bytes(rows, cols, nnz, 0) if transpose else 0
+            if scatter and "OPS_SPARSE_SPMV_REPEATABLE" not in os.environ and "OPS_SPARSE_SPMV_NO_SCATTER" not in os.environ:
+                # op(A) = A^T where the last bit may vary: inside the same buffer Preprocess builds the layout that
+                # sorts the products by output panel (no column of the benchmark matrices is full enough to refuse it)
+                layout = "scatter_live"
+                resident = scatter
         ncols = 1
         bytes_alg = wl.spmv_bytes_alg(rows, cols, nnz, vb, 4, 4, beta != 0)
         bytes_gather = wl.spmv_bytes_gather(rows, cols, nnz, vb, 4, 4, beta != 0)

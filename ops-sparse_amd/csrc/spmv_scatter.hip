@@ -291,43 +291,40 @@ __device__ __forceinline__ float WidenOne(ValT v)
     return static_cast<float>(ToAcc<double, ValT>(v));
 }
 
-// Pass 1: the products of piece blockIdx.x, written to `inter` in panel order.
+// Pass 1: the products of the pieces blockIdx.x, blockIdx.x + gridDim.x, ... written to `inter` in panel order.  One
+// workgroup a compute unit (the staging area is most of its LDS), so nothing else would cover the time a piece's
+// loads are on their way: the workgroup asks for the next piece's values and slots before it writes the current one
+// out (one piece after the other: 309 us on the 8 M x 8 M power-law matrix).
 template <typename ValT, typename ProdT>
 __global__ __launch_bounds__(kThreads) void ScatterProductsKernel(const ValT *__restrict__ vals, const ValT *__restrict__ x,
                                                                   const uint32_t *__restrict__ meta,
                                                                   const int32_t *__restrict__ chunkDst,
                                                                   const int32_t *__restrict__ pieceBase,
                                                                   const int32_t *__restrict__ pieceRow, int64_t nnz, int32_t P,
-                                                                  ProdT *__restrict__ inter)
+                                                                  int32_t Q, ProdT *__restrict__ inter)
 {
     constexpr int kPiece = kStageBytes / static_cast<int>(sizeof(ProdT));
     constexpr int kRounds = kPiece / (kThreads * 4);  // a thread takes 4 consecutive entries a round
     __shared__ __align__(16) ProdT stage[kPiece];
     __shared__ int32_t base[kMaxPanels + 1];
     __shared__ int32_t dst[kMaxPanels];
-    const int32_t q = blockIdx.x;
     const int t = threadIdx.x;
-    const int64_t first = static_cast<int64_t>(q) * kPiece;
-    const int32_t count = nnz - first < kPiece ? static_cast<int32_t>(nnz - first) : kPiece;
-    for (int32_t p = t; p <= P; p += kThreads) {
-        base[p] = pieceBase[static_cast<int64_t>(q) * (P + 1) + p];
-    }
-    for (int32_t p = t; p < P; p += kThreads) {
-        dst[p] = chunkDst[static_cast<int64_t>(q) * P + p];
-    }
-    const ValT *xRow = x + pieceRow[q];
-    // four rounds of loads in flight at a time
-#pragma unroll 1
-    for (int half = 0; half < kRounds; half += 4) {
-        Uint4 m[4];
-        float v[4][4];
+    const int wave = t / kWave, lane = t % kWave;
+    Uint4 m[kRounds];
+    float v[kRounds][4];
+    // values and slots of piece q into registers: every load is issued whatever the piece's length (those past its end
+    // re-read its first entries and are not used), so that none waits for another
+    auto fetch = [&](int32_t q) {
+        const int64_t first = static_cast<int64_t>(q) * kPiece;
+        const int32_t count = nnz - first < kPiece ? static_cast<int32_t>(nnz - first) : kPiece;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int32_t k = ((half + r) * kThreads + t) * 4;
+        for (int r = 0; r < kRounds; ++r) {
+            const int32_t k = (r * kThreads + t) * 4;
             if (k + 4 <= count) {
                 m[r] = __builtin_nontemporal_load(reinterpret_cast<const Uint4 *>(meta + first + k));
                 LoadFour<ValT>(vals + first + k, v[r]);
             } else {
+#pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const bool in = k + j < count;
                     m[r][j] = in ? meta[first + k + j] : 0u;
@@ -335,18 +332,33 @@ __global__ __launch_bounds__(kThreads) void ScatterProductsKernel(const ValT *__
                 }
             }
         }
-        float xv[4][4];
+    };
+    int32_t q = blockIdx.x;
+    if (q < Q) {
+        fetch(q);
+    }
+    for (; q < Q; q += gridDim.x) {
+        const int64_t first = static_cast<int64_t>(q) * kPiece;
+        const int32_t count = nnz - first < kPiece ? static_cast<int32_t>(nnz - first) : kPiece;
+        for (int32_t p = t; p <= P; p += kThreads) {
+            base[p] = pieceBase[static_cast<int64_t>(q) * (P + 1) + p];
+        }
+        for (int32_t p = t; p < P; p += kThreads) {
+            dst[p] = chunkDst[static_cast<int64_t>(q) * P + p];
+        }
+        const ValT *xRow = x + pieceRow[q];
+        float xv[kRounds][4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int32_t k = ((half + r) * kThreads + t) * 4;
+        for (int r = 0; r < kRounds; ++r) {
+            const int32_t k = (r * kThreads + t) * 4;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 xv[r][j] = k + j < count ? WidenOne<ValT>(xRow[m[r][j] >> 16]) : 0.0f;
             }
         }
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int32_t k = ((half + r) * kThreads + t) * 4;
+        for (int r = 0; r < kRounds; ++r) {
+            const int32_t k = (r * kThreads + t) * 4;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 if (k + j < count) {
@@ -354,16 +366,22 @@ __global__ __launch_bounds__(kThreads) void ScatterProductsKernel(const ValT *__
                 }
             }
         }
-    }
-    __syncthreads();
-    // a wavefront a chunk: the piece's products of one panel, contiguous in the staging area and in memory
-    const int wave = t / kWave, lane = t % kWave;
-    for (int32_t p = wave; p < P; p += kThreads / kWave) {
-        const int32_t s0 = base[p], s1 = base[p + 1];
-        ProdT *out = inter + dst[p];
-        for (int32_t k = s0 + lane; k < s1; k += kWave) {
-            out[k - s0] = stage[k];
+        __syncthreads();
+        if (q + static_cast<int32_t>(gridDim.x) < Q) {
+            fetch(q + static_cast<int32_t>(gridDim.x));
         }
+        // a wavefront a chunk: the piece's products of one panel, contiguous in the staging area and in memory
+        // (four chunks at a time, their look-ups and LDS reads issued together, changed nothing: the kernel runs at
+        // the rate at which memory takes 256-byte pieces written to 512 places at once, 3.9 TB/s for reads and writes
+        // together, where the radix passes of the analysis, with 16 places, reach 2.6)
+        for (int32_t p = wave; p < P; p += kThreads / kWave) {
+            const int32_t s0 = base[p], s1 = base[p + 1];
+            ProdT *out = inter + dst[p];
+            for (int32_t k = s0 + lane; k < s1; k += kWave) {
+                out[k - s0] = stage[k];
+            }
+        }
+        __syncthreads();
     }
 }
 
@@ -422,6 +440,21 @@ __global__ __launch_bounds__(kThreads) void ScatterSumKernel(const ProdT *__rest
     }
 }
 
+// Compute units of the current device (256 on MI355X), asked once.
+int32_t ComputeUnits()
+{
+    static const int32_t cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            return 256;
+        }
+        return n;
+    }();
+    return cus;
+}
+
 // a.rows / a.cols: rows and columns of A; x has a.rows elements, y a.cols.
 int Launch(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valType, int32_t outType)
 {
@@ -449,9 +482,10 @@ int Launch(const SpmvArgs &a, const OpsparseSpmvPlan &plan, int32_t valType, int
     auto products = [&](auto valTag, auto prodTag) {
         using ValT = decltype(valTag);
         using ProdT = decltype(prodTag);
-        hipLaunchKernelGGL((ScatterProductsKernel<ValT, ProdT>), dim3(static_cast<uint32_t>(l.Q)), dim3(kThreads), 0, a.stream,
+        const int32_t grid = l.Q < ComputeUnits() ? l.Q : ComputeUnits();
+        hipLaunchKernelGGL((ScatterProductsKernel<ValT, ProdT>), dim3(static_cast<uint32_t>(grid)), dim3(kThreads), 0, a.stream,
                            static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.x), meta, ints(l.chunkDstOff),
-                           ints(l.pieceBaseOff), ints(l.pieceRowOff), a.nnz, l.P, static_cast<ProdT *>(inter));
+                           ints(l.pieceBaseOff), ints(l.pieceRowOff), a.nnz, l.P, l.Q, static_cast<ProdT *>(inter));
     };
     auto sums = [&](auto outTag, auto prodTag) {
         using OutT = decltype(outTag);
