@@ -305,12 +305,14 @@ aclsparseStatus_t aclsparseDnMatSetValues(aclsparseDnMatDescr_t dnMatDescr, void
  * (the reference promises it for op(A) = A only).  So do ALG_DEFAULT / CSR_ALG1
  * with op(A) = A wherever the plan is row-wise or merge-path (every unprepared
  * call, every matrix under 7 M entries or with local columns) and for int32.
- * The one plan that adds in the order its wavefronts arrive is the default
- * algorithm's re-stored layout for op(A) = A on floating-point data, and
- * op(A) = A^T without Preprocess (fp32 atomics on y): there the last bit of an
- * element may differ between two calls, as the reference says of CSR_ALG1.
+ * The plans that add in the order their wavefronts arrive are the default
+ * algorithm's re-stored layouts on floating-point data (op(A) = A: row blocks
+ * summed with LDS atomics; op(A) = A^T over more than 2 M columns: products
+ * sorted by output panel and summed with LDS atomics) and op(A) = A^T without
+ * Preprocess (fp32 atomics on y): there the last bit of an element may differ
+ * between two calls, as the reference says of CSR_ALG1.
  * OPS_SPARSE_SPMV_REPEATABLE=1 in the environment makes Preprocess choose
- * the ordered layout there too.
+ * the ordered layouts there too.
  *
  * alpha / beta: typed by computeType; NULL means alpha = 1, beta = 0
  * [ref: spmv_host.cpp:183-199]; read according to the handle's pointer mode.
