@@ -1548,8 +1548,8 @@ __global__ __launch_bounds__(kThreads, 2 * kThreads / kWave / 4) void SpmvBlockR
             for (int u = 0; u < kStagePasses; ++u) {
                 uint32_t at = static_cast<uint32_t>(src[u]);
                 at = at < static_cast<uint32_t>(a.xgEntries) ? at : 0u;  // (in range whatever the table holds)
-                const Uint4U v0 = __builtin_nontemporal_load(reinterpret_cast<const Uint4U *>(a.xg + at));
-                const Uint4U v1 = __builtin_nontemporal_load(reinterpret_cast<const Uint4U *>(a.xg + at + 4));
+                const Uint4U v0 = *reinterpret_cast<const Uint4U *>(a.xg + at);
+                const Uint4U v1 = *reinterpret_cast<const Uint4U *>(a.xg + at + 4);
                 xa[u] = Uint4{v0.x, v0.y, v0.z, v0.w};
                 xb[u] = Uint4{v1.x, v1.y, v1.z, v1.w};
             }
@@ -1838,7 +1838,7 @@ __global__ __launch_bounds__(kStreamThreads) void SpmvBlockStreamKernel(const Bl
             int32_t src = from.at[s] + (at & 4);
             src = src < 0 ? 0 : (src < a.xgEntries ? src : a.xgEntries);
             piece.v[s] = LoadFourRaw(a.valD + at);
-            piece.x[s] = __builtin_nontemporal_load(reinterpret_cast<const Uint4U *>(a.xg + src));
+            piece.x[s] = *reinterpret_cast<const Uint4U *>(a.xg + src);
             piece.f[s] = __builtin_nontemporal_load(reinterpret_cast<const Uint2 *>(a.field + at));
         }
         return piece;

@@ -979,7 +979,7 @@ __global__ __launch_bounds__(kRedThreads) void SpmvBlockReduceKernel(
                     piece.a[s] = __builtin_nontemporal_load(reinterpret_cast<const Float4U1 *>(valD + i0));
                 }
                 piece.rows[s] = __builtin_nontemporal_load(reinterpret_cast<const Uint2 *>(rowLocal + i0));
-                piece.x[s] = __builtin_nontemporal_load(reinterpret_cast<const Float4U1 *>(xg + (i0 + tabDelta[p])));
+                piece.x[s] = *reinterpret_cast<const Float4U1 *>(xg + (i0 + tabDelta[p]));
             }
             return piece;
         };
