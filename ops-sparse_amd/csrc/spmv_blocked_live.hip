@@ -1,60 +1,41 @@
-// BLOCKED_GATHER: CSR SpMV for a matrix whose x does not fit a cache, fp32.
+// BLOCKED_LIVE: CSR SpMV, op(A) = A, for a matrix whose x does not fit a cache, with the values read where the
+// caller has them at every call and the row sums formed with LDS atomics.
 //
-// Takes the place of the reference's aclsparseSpMVOp with ALG2 — a device-side
-// preprocessing pass that re-orders the rows into the caller's buffer, then a
-// thread-per-row kernel (sparse/spmv_op/arch35/spmv_op_host.cpp:543-573 and
-// :423-457, spmv_op_kernel.cpp:413-535) — and of aclsparseSpMV's kernel
-// (sparse/spmv/arch22/kernels/spmv_kernel.h:27-310) for that case.  A
-// row-wise kernel gathers x[col] straight from memory, and with random columns
-// every gather moves a
-// whole 128-byte line for 4 useful bytes: the gather rate, not the matrix
-// stream, sets the time.  Here x is gathered from LDS instead.
+// Takes the place of aclsparseSpMV's kernel (sparse/spmv/arch22/kernels/spmv_kernel.h:27-310) under
+// ACL_SPARSE_SPMV_ALG_DEFAULT / CSR_ALG1 for a matrix with scattered columns, after aclsparseSpMVPreprocess.  A
+// row-wise kernel gathers x[col] straight from memory, and with random columns every gather moves a whole 128-byte
+// line for 4 useful bytes: the gather rate, not the matrix stream, sets the time.  Here x is gathered from LDS.
+// This is the fast sibling of the ordered layout of spmv_blocked.hip, whose kernels sum every row in a fixed order:
+// the reference lets these two algorithm values differ in the last bit between runs
+// (include/cann_ops_sparse.h:57-60), and this file uses that.
 //
-//   phase 1  the entries are stored a second time sorted by column panel
-//            (2^15 columns = 128 KiB of x).  A workgroup copies its panel's
-//            slice of x into LDS and writes xg[i] = x[col[i]] for the panel's
-//            entries: 2 bytes of local column index read, 4 bytes written per
-//            entry, both as linear streams.
-//   phase 2  rows are grouped into row blocks (at most 2^14 rows, cut also
-//            wherever the entry count passes a multiple of the entry window,
-//            so that blocks of short rows hold similar numbers of entries).  A
-//            workgroup owns one block, keeps an fp64 accumulator per row in
-//            LDS and streams the block's entries in (block, panel) order:
-//            value and local row index linearly, the gathered xg in one
-//            contiguous piece per (panel, block) chunk.  Chunks are padded to
-//            multiples of 8 positions in that order, so that a lane's run of 4
-//            consecutive positions shares a chunk, the streams come as 16- and
-//            8-byte loads and the lanes of a wavefront read neighbouring
-//            pieces.  val * xg is exact in fp64; a row's result is
-//            rounded once when the block is written.  The blocks are started
-//            heaviest first.
+//   phase 1  the entries' local columns are stored a second time sorted by column panel (2^15 columns = 128 KiB
+//            of x).  A workgroup copies its panel's slice of x into LDS and writes xg[i] = x[col[i]] for the panel's
+//            entries: 2 bytes of local column index read, 4 bytes written per entry, both as linear streams.
+//   phase 2  rows are grouped into row blocks of at most 2^12 rows and about 20 000 entries.  A workgroup owns one
+//            block: it first collects the block's values, which are one piece of the caller's array, at their
+//            positions of the (block, panel) order in a 96 KiB window of LDS (the positions, 16 bits relative to
+//            the block where every block is shorter than 65 535, are part of the layout), then streams local row
+//            and gathered x in that order - a contiguous piece per (panel, block) chunk, chunks padded to
+//            multiples of 8 positions - against the window and adds val * xg (exact in fp64) to the row's fp64
+//            accumulator in LDS with an LDS atomic.  A row is rounded once when the block is written.  The blocks
+//            are started heaviest first.
 //
-// Every entry costs 16 bytes of HBM traffic (2 + 4 in phase 1, 4 + 2 + 4 in
-// phase 2, plus the padding) against 8 algorithmic bytes plus a 128-byte line
-// per gather in the row-wise kernels.  The order of the fp64 additions into a
-// row's accumulator depends on scheduling; the sum is rounded to fp32
-// afterwards.
+// The order of the fp64 additions into a row's accumulator depends on scheduling: two calls may differ in the last
+// bit of an element.  No value is kept: csrValues may change between calls, the structure may not.
 //
-// Preprocessing (once per matrix, all on the device): a stable radix sort of
-// the entries on the panel number keeps rows, hence row blocks, ascending inside
-// a panel, so it yields the (panel, block) order directly; the position of a
-// chunk in (block, panel) order follows from the chunk sizes by a prefix sum.
-// The VALUES are copied in (block, panel) order: the analysis must be repeated
-// after they change.  With "live values" none are copied: the phase-2 workgroup
-// of a row block reads the block's entries of the caller's array, linearly,
-// together with their positions in (block, panel) order, collects them in a
-// window of LDS and streams against that window.
+// Preprocessing (once per structure, all on the device): a stable radix sort of the entries on the panel number
+// keeps rows, hence row blocks, ascending inside a panel, so it yields the (panel, block) order directly; the
+// position of a chunk in (block, panel) order follows from the chunk sizes by a prefix sum.
 //
-// Long rows (op(A) = A only).  A row with many entries in every panel, whose columns ascend, is kept out of the
-// (block, panel) order: the phase-1 workgroup of a panel, which has the panel's x in LDS anyway, sums val * x over
-// the row's entries of that panel and leaves the fp64 sum in a small table; the phase-2 workgroup that owns the
-// row adds the row's sums up, in panel order, before it writes the row.  8 bytes an entry instead of 16.  With
-// frozen values (rows of 1024 entries and 4 per panel or more) the long entries are stored a second time, a
-// panel's in one piece in row order as (local column, value, number of the row), and stream into one fp64
-// accumulator a long row in LDS.  With live values (4096 entries and 64 per panel) a row's entries of a panel
-// are a contiguous piece of the caller's own arrays, found by a search in the sorted columns, and lane groups
-// take the pieces in turn: nothing is stored a second time, and the values read are the caller's as they are at
-// the call.
+// Long rows.  A row of 4096 entries and 64 per panel or more whose columns ascend is kept out of the (block, panel)
+// order: its entries of a panel are a contiguous piece of the caller's own arrays, found by a search in the sorted
+// columns, and the phase-1 workgroup of the panel, which has the panel's x in LDS anyway, sums val * x over the
+// piece with a lane group of 16 and leaves the fp64 sum in a small table; the phase-2 workgroup that owns the row
+// (or, where a block holds more than 64 such rows, a kernel with a wavefront a row) adds the row's sums up in
+// panel order.  8 bytes an entry instead of 18, and the values read are the caller's as they are at the call.
+// (The template and layout arms for frozen values and op(A) = A^T that this file grew out of are those of
+// spmv_blocked.hip; here they are compile-time constants and dropped by the compiler.)
 #include <climits>
 #include <cstdlib>
 
