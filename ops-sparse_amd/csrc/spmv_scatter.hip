@@ -65,7 +65,7 @@ struct ScatterLayout {
     int64_t panelStartOff; // [P + 1]
     int64_t resident;
     // the analysis only
-    int64_t keys0Off, keys1Off, pay0Off, pay1Off, rowIndOff, dstOfOff, countOff, inclOff, tableOff, scanOff, colCountOff;
+    int64_t keys0Off, keys1Off, pay0Off, pay1Off, rowIndOff, dstOfOff, countOff, inclOff, tableOff, scanOff;
     int64_t bytes;
 };
 
@@ -126,7 +126,6 @@ ScatterLayout MakeLayout(int64_t rows, int64_t cols, int64_t nnz, int32_t valueT
     l.tableOff = off; off += align(4 * RadixTableInts(nnz));
     const int64_t scanA = ScanScratchInts(RadixTableInts(nnz)), scanB = ScanScratchInts(P * Q + 1);
     l.scanOff = off; off += align(4 * (scanA > scanB ? scanA : scanB));
-    l.colCountOff = off; off += align(4 * cols);
     l.bytes = off;
     return l;
 }
@@ -140,56 +139,81 @@ inline uint32_t GridOf(int64_t items, int64_t perBlock, int64_t cap)
 
 // ---------------------------------------------------------------------------------------------- analysis kernels
 
-// status[0] |= 1 for a column index outside [0, cols); entries per column otherwise.
-__global__ __launch_bounds__(kBlockThreads) void ColumnCountKernel(const int32_t *__restrict__ colInd, int64_t nnz, int64_t cols,
-                                                                   int32_t *__restrict__ colCount, int32_t *__restrict__ status)
+// status[0] |= 1 for a column index outside [0, cols).
+__global__ __launch_bounds__(kBlockThreads) void ColumnRangeKernel(const int32_t *__restrict__ colInd, int64_t nnz, int64_t cols,
+                                                                   int32_t *__restrict__ status)
 {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     bool bad = false;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nnz; i += stride) {
         const int32_t c = colInd[i];
-        if (c < 0 || c >= cols) {
-            bad = true;
-        } else {
-            atomicAdd(colCount + c, 1);
-        }
+        bad = bad || c < 0 || c >= cols;
     }
     if (bad) {
         atomicOr(status, 1);
     }
 }
 
-// status[1] = entries of the fullest column.
-__global__ __launch_bounds__(kBlockThreads) void ColumnMaxKernel(const int32_t *__restrict__ colCount, int64_t cols,
-                                                                 int32_t *__restrict__ status)
+// A workgroup a panel: status[1] = entries of the fullest column, counted in LDS over the panel's sorted columns.
+__global__ __launch_bounds__(kThreads) void ColumnMaxKernel(const uint16_t *__restrict__ colLocal,
+                                                            const int32_t *__restrict__ panelStart,
+                                                            int32_t *__restrict__ status)
 {
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    __shared__ int32_t count[kOutCols];
+    const int t = threadIdx.x;
+    for (int32_t c = t; c < kOutCols; c += kThreads) {
+        count[c] = 0;
+    }
+    __syncthreads();
+    const int32_t s0 = panelStart[blockIdx.x], s1 = panelStart[blockIdx.x + 1];
+    for (int32_t s = s0 + t; s < s1; s += kThreads) {
+        atomicAdd(&count[colLocal[s]], 1);
+    }
+    __syncthreads();
     int32_t most = 0;
-    for (int64_t c = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; c < cols; c += stride) {
-        most = colCount[c] > most ? colCount[c] : most;
+    for (int32_t c = t; c < kOutCols; c += kThreads) {
+        most = count[c] > most ? count[c] : most;
     }
     for (int off = kWave / 2; off > 0; off >>= 1) {
         const int32_t other = __shfl_xor(most, off, kWave);
         most = other > most ? other : most;
     }
-    if ((threadIdx.x & (kWave - 1)) == 0 && most > 0) {
+    if (t % kWave == 0 && most > 0) {
         atomicMax(status + 1, most);
     }
 }
 
 // From the entries sorted by panel (key = column, payload = entry of the caller's arrays): the local column of every
-// product, where every entry's product goes, and the number of entries of every (panel, piece) chunk.
+// product, where every entry's product goes, and the number of entries of every (panel, piece) chunk.  A thread
+// takes eight consecutive sorted entries, which mostly share a chunk, and counts a run of them with one atomic.
 __global__ __launch_bounds__(kBlockThreads) void ChunkCountKernel(const int32_t *__restrict__ sortedCol,
                                                                   const int32_t *__restrict__ sortedEntry, int64_t nnz, int32_t Q,
                                                                   int32_t piece, uint16_t *__restrict__ colLocal,
                                                                   int32_t *__restrict__ dstOf, int32_t *__restrict__ count)
 {
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
-    for (int64_t s = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; s < nnz; s += stride) {
-        const int32_t c = sortedCol[s], i = sortedEntry[s];
-        colLocal[s] = static_cast<uint16_t>(c & (kOutCols - 1));
-        dstOf[i] = static_cast<int32_t>(s);
-        atomicAdd(count + static_cast<int64_t>(c >> kOutLog) * Q + i / piece, 1);
+    constexpr int kRun = 8;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x * kRun;
+    for (int64_t s0 = (static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x) * kRun; s0 < nnz; s0 += stride) {
+        int64_t chunk = -1;
+        int32_t run = 0;
+        for (int j = 0; j < kRun && s0 + j < nnz; ++j) {
+            const int64_t s = s0 + j;
+            const int32_t c = sortedCol[s], i = sortedEntry[s];
+            colLocal[s] = static_cast<uint16_t>(c & (kOutCols - 1));
+            dstOf[i] = static_cast<int32_t>(s);
+            const int64_t at = static_cast<int64_t>(c >> kOutLog) * Q + i / piece;
+            if (at != chunk) {
+                if (run > 0) {
+                    atomicAdd(count + chunk, run);
+                }
+                chunk = at;
+                run = 0;
+            }
+            ++run;
+        }
+        if (run > 0) {
+            atomicAdd(count + chunk, run);
+        }
     }
 }
 
@@ -560,15 +584,12 @@ int opsparse_spmv_csr_scatter_analyse_split(const int32_t *rowOffsets, const int
     int32_t *keys[2] = {ints(l.keys0Off), ints(l.keys1Off)};
     int32_t *pays[2] = {ints(l.pay0Off), ints(l.pay1Off)};
     int32_t *rowInd = ints(l.rowIndOff), *dstOf = ints(l.dstOfOff), *count = ints(l.countOff), *incl = ints(l.inclOff);
-    int32_t *table = ints(l.tableOff), *scan = ints(l.scanOff), *colCount = ints(l.colCountOff);
+    int32_t *table = ints(l.tableOff), *scan = ints(l.scanOff);
     const int64_t chunks = static_cast<int64_t>(l.P) * l.Q;
 
     LaunchFillI32(status, 4, 0, s);
-    LaunchFillI32(colCount, cols, 0, s);
     LaunchFillI32(count, chunks + 1, 0, s);
-    hipLaunchKernelGGL(ColumnCountKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s, colInd, nnz, cols,
-                       colCount, status);
-    hipLaunchKernelGGL(ColumnMaxKernel, dim3(GridOf(cols, kBlockThreads, 4096)), dim3(kBlockThreads), 0, s, colCount, cols,
+    hipLaunchKernelGGL(ColumnRangeKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s, colInd, nnz, cols,
                        status);
     int32_t seen[2] = {0, 0};
     if (hipMemcpyAsync(seen, status, sizeof(seen), hipMemcpyDeviceToHost, s) != hipSuccess ||
@@ -578,9 +599,6 @@ int opsparse_spmv_csr_scatter_analyse_split(const int32_t *rowOffsets, const int
     }
     if ((seen[0] & 1) != 0) {
         return OPSPARSE_E_INVALID;  // a column index outside [0, cols)
-    }
-    if (seen[1] > kMaxColumnEntries) {
-        return OPSPARSE_E_UNSUPPORTED;  // a column that would queue for one address of LDS
     }
     // Entries in (panel, caller's order) order: stable 4-bit radix passes over the panel number.
     int bits = 0;
@@ -595,19 +613,25 @@ int opsparse_spmv_csr_scatter_analyse_split(const int32_t *rowOffsets, const int
         payIn = pays[k & 1];
     }
     LaunchExpandRows(rowOffsets, rows, nnz, 0, rowInd, s);
-    hipLaunchKernelGGL(ChunkCountKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s, keysIn, payIn, nnz,
-                       l.Q, l.piece, reinterpret_cast<uint16_t *>(at(l.colLocalOff)), dstOf, count);
+    auto *colLocal = reinterpret_cast<uint16_t *>(at(l.colLocalOff));
+    hipLaunchKernelGGL(ChunkCountKernel, dim3(GridOf(nnz, kBlockThreads * 8, 16384)), dim3(kBlockThreads), 0, s, keysIn, payIn,
+                       nnz, l.Q, l.piece, colLocal, dstOf, count);
     LaunchInclusiveScanI32(count, incl, chunks, 0, scan, s);
     hipLaunchKernelGGL(PieceTablesKernel, dim3(static_cast<uint32_t>(l.Q)), dim3(kWave), 0, s, count, incl, rowInd, l.P, l.Q,
                        l.piece, nnz,
                        ints(l.chunkDstOff), ints(l.pieceBaseOff), ints(l.pieceRowOff), ints(l.panelStartOff));
+    hipLaunchKernelGGL(ColumnMaxKernel, dim3(static_cast<uint32_t>(l.P)), dim3(kThreads), 0, s, colLocal,
+                       ints(l.panelStartOff), status);
     hipLaunchKernelGGL(EntryMetaKernel, dim3(GridOf(nnz, kBlockThreads, 16384)), dim3(kBlockThreads), 0, s, colInd, rowInd, dstOf,
                        ints(l.chunkDstOff), ints(l.pieceBaseOff), ints(l.pieceRowOff), nnz, l.P, l.piece,
                        reinterpret_cast<uint32_t *>(at(l.metaOff)), status);
-    if (hipMemcpyAsync(seen, status, sizeof(int32_t), hipMemcpyDeviceToHost, s) != hipSuccess ||
+    if (hipMemcpyAsync(seen, status, sizeof(seen), hipMemcpyDeviceToHost, s) != hipSuccess ||
         hipStreamSynchronize(s) != hipSuccess || CheckLaunch() != OPSPARSE_OK) {
         (void)hipGetLastError();
         return OPSPARSE_E_LAUNCH;
+    }
+    if (seen[1] > kMaxColumnEntries) {
+        return OPSPARSE_E_UNSUPPORTED;  // a column that would queue for one address of LDS
     }
     if ((seen[0] & 2) != 0) {
         return OPSPARSE_E_UNSUPPORTED;  // a piece that spans more than 65 535 rows
