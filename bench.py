@@ -683,6 +683,63 @@ def run_shapes(args, osa, wl, torch, dev, stream, handle):
     return res
 
 
+def run_stencils(args, osa, wl, torch, dev, stream, handle):
+    """The headline kernel family on other meshes and bands than c2's: time of a call (default algorithm after
+    Preprocess, alpha = 1, beta = 0.5, every launch on the same operands) and the algorithmic bytes against 8 TB/s.
+    What separates these shapes is the number of gathers a row needs and how many of them a cache line serves."""
+    import itertools
+
+    def band(rows, width, seed):
+        """`width` distinct columns a row inside a window of 4 x width columns round the diagonal."""
+        idx = torch.arange(rows * width, dtype=torch.int64, device=dev).view(rows, width)
+        r = torch.arange(rows, dtype=torch.int64, device=dev).view(rows, 1)
+        step = (wl._lsr(wl.hash64(seed, idx.reshape(-1)), 11) % 4).view(rows, width)
+        ci = (r - 2 * width + 4 * torch.arange(width, dtype=torch.int64, device=dev).view(1, width) + step)
+        ci = ci.clamp(0, rows - 1)
+        return {"rows": rows, "cols": rows, "colind": ci.reshape(-1).int(),
+                "rowptr": (torch.arange(rows + 1, dtype=torch.int64, device=dev) * width).int(),
+                "values": wl.uniform(seed + 1, rows * width, -1.0, 1.0, dev)}
+
+    box3 = list(itertools.product((-1, 0, 1), repeat=3))
+    cross3 = [o for o in box3 if sum(abs(v) for v in o) <= 1]
+    box2 = list(itertools.product((-1, 0, 1), repeat=2))
+    cross2 = [o for o in box2 if sum(abs(v) for v in o) <= 1]
+    shapes = [
+        ("5-point, 2048^2 (c2)", lambda: wl.stencil_csr((2048, 2048), cross2, dev)),
+        ("9-point, 2048^2", lambda: wl.stencil_csr((2048, 2048), box2, dev)),
+        ("7-point, 160^3", lambda: wl.stencil_csr((160, 160, 160), cross3, dev)),
+        ("27-point, 128^3", lambda: wl.stencil_csr((128, 128, 128), box3, dev)),
+        ("band of 50, 1 M rows", lambda: band(1 << 20, 50, 21)),
+        ("band of 200, 256 K rows", lambda: band(1 << 18, 200, 22)),
+        ("band of 600, 64 K rows", lambda: band(1 << 16, 600, 23)),
+    ]
+    if args.scale < 1.0:
+        shapes = shapes[:2]
+    res = {}
+    for name, make in shapes:
+        torch.cuda.empty_cache()
+        A = make()
+        rows, nnz = A["rows"], int(A["colind"].numel())
+        csr = osa.Csr(rows, rows, A["rowptr"], A["colind"], A["values"])
+        x = wl.uniform(5, rows, -1.0, 1.0, dev)
+        y0 = wl.uniform(6, rows, -1.0, 1.0, dev)
+        y = y0.clone()
+        op = osa.SpmvOp(handle, csr, osa.DnVec(x), osa.DnVec(y))
+        for _ in range(5 + args.settle):   # (the clocks' ramp and the runtime's one-off stall: see run_workload)
+            op(1.0, 0.5)
+        stream.synchronize()
+        ms, ms_min, _, nrounds, _ = time_rounds(torch, stream, lambda i: op(1.0, 0.5), args.steps,
+                                                lambda: y.copy_(y0), args.min_gpu_ms)
+        bytes_alg = wl.spmv_bytes_alg(rows, rows, nnz, 4, 4, 4, True)
+        line = {"rows": rows, "nnz": nnz, "entries_per_row": round(nnz / rows, 1), "us_per_call": round(ms * 1e3, 2),
+                "us_fastest_round": round(ms_min * 1e3, 2), "rounds": nrounds, "bytes_alg": bytes_alg,
+                "frac_of_8TBs": round(bytes_alg / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+        res[name] = line
+        log("%-26s %s" % (name, json.dumps(line)))
+        del op, csr, A, x, y, y0
+    return res
+
+
 def run_cache_probe(args, osa, wl, torch, dev, stream, handle):
     """What the 256 MB Infinity Cache is worth on this path.  (1) The copy and read kernels on buffers from 8 MiB
     to 1 GiB, launched back to back on the same buffer.  (2) The c4 product (1 M rows of 32 entries, n = 64,
@@ -809,10 +866,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all",
                     choices=["all", "c1", "c2", "c3", "c3_repeatable", "c3_transposed", "c4", "c5", "convert", "cache",
-                             "shapes"],
+                             "shapes", "stencils"],
                     help="all: c2 as the headline plus c1, c3 (default plan, repeatable default plan, ALG2, "
                          "transposed), c4 and c5 in `workloads`; shapes: the grid of secondary shapes behind the "
-                         "selection thresholds")
+                         "selection thresholds; stencils: the headline kernels on other meshes and bands")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
     ap.add_argument("--min-gpu-ms", type=float, default=50.0,
                     help="rounds of --steps launches are repeated until this much GPU time has been timed")
@@ -858,6 +915,12 @@ def main():
         print(json.dumps({"metric": "CSR SpMV fp32, time per call by shape and plan", "unit": "us",
                           "data": "synthetic", "shapes": run_shapes(args, osa, wl, torch, dev, stream, handle)}),
               flush=True)
+        handle.close()
+        return
+    if args.workload == "stencils":
+        print(json.dumps({"metric": "CSR SpMV fp32 on meshes and bands, time per call and algorithmic bytes / 8 TB/s",
+                          "unit": "us", "data": "synthetic",
+                          "shapes": run_stencils(args, osa, wl, torch, dev, stream, handle)}), flush=True)
         handle.close()
         return
     if args.workload == "convert":

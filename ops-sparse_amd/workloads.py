@@ -83,6 +83,40 @@ def laplacian_2d(grid, device):
     }
 
 
+def stencil_csr(shape, offsets, device):
+    """A stencil on a mesh of `shape` points (2 or 3 extents, the last one fastest): row i couples the point i with
+    the points at `offsets` (tuples of as many signed steps) that exist - no wrap-around at the faces - columns
+    ascending; the centre carries the number of its neighbours in the stencil, every neighbour -1."""
+    dims = len(shape)
+    m = 1
+    for n in shape:
+        m *= n
+    i = torch.arange(m, dtype=torch.int64, device=device)
+    coords, rest = [], i
+    for n in reversed(shape):
+        coords.append(rest % n)
+        rest = rest // n
+    coords.reverse()
+    strides = [1] * dims
+    for d in range(dims - 2, -1, -1):
+        strides[d] = strides[d + 1] * shape[d + 1]
+    offsets = sorted(offsets, key=lambda o: sum(o[d] * strides[d] for d in range(dims)))
+    masks, cols, vals = [], [], []
+    for o in offsets:
+        ok = torch.ones(m, dtype=torch.bool, device=device)
+        for d in range(dims):
+            ok &= (coords[d] + o[d] >= 0) & (coords[d] + o[d] < shape[d])
+        masks.append(ok)
+        cols.append(i + sum(o[d] * strides[d] for d in range(dims)))
+        vals.append(float(len(offsets) - 1) if all(v == 0 for v in o) else -1.0)
+    mask = torch.stack(masks, dim=1)
+    rowptr = torch.zeros(m + 1, dtype=torch.int64, device=device)
+    rowptr[1:] = torch.cumsum(mask.sum(dim=1), dim=0)
+    values = torch.tensor(vals, dtype=torch.float32, device=device).expand(m, len(offsets))
+    return {"rows": m, "cols": m, "rowptr": rowptr.to(torch.int32),
+            "colind": torch.stack(cols, dim=1)[mask].to(torch.int32), "values": values[mask].contiguous()}
+
+
 def power_law_lengths(m, alpha, lmin, lmax, seed, device, target_mean=None, force_max_row=True):
     """Row lengths with P(l) ~ l^-alpha on [lmin, lmax] (inverse-CDF table lookup).
     target_mean rescales the draw (then clips again); force_max_row pins one row
