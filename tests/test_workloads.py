@@ -29,6 +29,27 @@ def test_laplacian_structure_and_closed_form(workloads):
     assert r + 1 not in colind[rowptr[r]:rowptr[r + 1]]
 
 
+def test_stencil_generator(workloads):
+    """The general mesh generator: its 5-point stencil in two dimensions is the Laplacian above array for array; a
+    27-point stencil has 27 entries inside and 8 in a corner, ascending columns, and A * 1 counts the neighbours that
+    a point at a face lacks."""
+    import itertools
+    cross = [o for o in itertools.product((-1, 0, 1), repeat=2) if sum(abs(v) for v in o) <= 1]
+    A, L = workloads.stencil_csr((7, 7), cross, "cpu"), workloads.laplacian_2d(7, "cpu")
+    assert all(torch.equal(A[k], L[k]) for k in ("rowptr", "colind", "values"))
+    shape = (4, 5, 6)
+    B = workloads.stencil_csr(shape, list(itertools.product((-1, 0, 1), repeat=3)), "cpu")
+    rowptr, colind, val = _np(B)
+    m = 4 * 5 * 6
+    lengths = np.diff(rowptr).reshape(shape)
+    assert B["rows"] == m and lengths[1, 2, 3] == 27 and lengths[0, 0, 0] == 8 and lengths[0, 2, 3] == 18
+    for r in range(m):
+        c = colind[rowptr[r]:rowptr[r + 1]]
+        assert np.all(np.diff(c) > 0) and r in c
+    y = oracle.spmv_f64(m, m, rowptr, colind, val, np.ones(m, np.float32), None, 1.0, 0.0).reshape(shape)
+    assert np.array_equal(y, 27 - lengths)
+
+
 def test_sorted_unique_uniform_columns(workloads):
     A = workloads.uniform_rows_csr(500, 300, 32, 3001, "cpu")
     rowptr, colind, val = _np(A)
