@@ -72,6 +72,40 @@ def test_spmv_replays(osa, gpu_ctx, kind):
         assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5, replay
 
 
+def test_transposed_scatter_layout_replays(osa, gpu_ctx, monkeypatch):
+    """op(A) = A^T under the default algorithm with the layout that sorts the products by output panel (its two
+    kernels and nothing else between capture and replay): new x and new values of A before every replay."""
+    dev, stream, handle = gpu_ctx
+    monkeypatch.setenv("OPS_SPARSE_SCATTER_MIN_PANELS", "8")
+    monkeypatch.setenv("OPS_SPARSE_DEFAULT_BLOCKED_MIN_NNZ", "0")
+    monkeypatch.delenv("OPS_SPARSE_SPMV_REPEATABLE", raising=False)
+    rows, cols = 1_200_000, 600_000
+    rng = np.random.default_rng(11)
+    lengths = rng.integers(0, 5, rows)
+    rowptr = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    colind = rng.integers(0, cols, int(rowptr[-1])).astype(np.int32)
+    nnz = colind.size
+    assert osa.lib().opsparse_spmv_csr_scatter_workspace_bytes(rows, cols, nnz, 0) > 0
+    y0 = rng.uniform(-1, 1, cols).astype(np.float32)
+    d_rp, d_ci = to_dev(rowptr, dev), to_dev(colind, dev)
+    d_val = torch.zeros(nnz, dtype=torch.float32, device=dev)
+    d_x = torch.zeros(rows, dtype=torch.float32, device=dev)
+    d_y = to_dev(y0, dev)
+    op = osa.SpmvOp(handle, osa.Csr(rows, cols, d_rp, d_ci, d_val), osa.DnVec(d_x), osa.DnVec(d_y),
+                    op=osa.ACL_SPARSE_OP_TRANSPOSE)
+    graph = _capture(stream, lambda: op(1.5, 0.5))
+    for replay in range(3):
+        x, val = rng.uniform(-1, 1, rows).astype(np.float32), rng.uniform(-1, 1, nnz).astype(np.float32)
+        d_x.copy_(torch.from_numpy(x))
+        d_val.copy_(torch.from_numpy(val))
+        d_y.copy_(torch.from_numpy(y0))
+        stream.synchronize()
+        graph.replay()
+        stream.synchronize()
+        gold = oracle.spmv_trans_f64(rows, cols, rowptr, colind, val, x, y0, 1.5, 0.5)
+        assert oracle.max_rel_err(d_y.cpu().numpy(), gold) <= 1e-5, replay
+
+
 def test_spmv_replays_read_device_scalars(osa, gpu_ctx):
     """Device pointer mode: the graph holds the addresses of alpha / beta, every replay reads their values."""
     dev, stream, handle = gpu_ctx
