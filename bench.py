@@ -323,7 +323,9 @@ WORKLOADS = {
     "c4": ("c4", "csr", False, {}),
     "c5": ("c5", "csr", False, {}),
 }
-BENCH_ENV = ("OPS_SPARSE_SPMV_NO_BLOCKED", "OPS_SPARSE_SPMV_REPEATABLE")
+BENCH_ENV = ("OPS_SPARSE_SPMV_NO_BLOCKED", "OPS_SPARSE_SPMV_REPEATABLE", "OPS_SPARSE_SPMV_NO_SCATTER",
+             "OPS_SPARSE_SCATTER_MIN_PANELS", "OPS_SPARSE_SPMV_NO_DEFAULT_BLOCKED", "OPS_SPARSE_ORDERED_LIVE_MIN_COLS",
+             "OPS_SPARSE_BLOCKED_NO_STREAM")
 _cfg_cache = {}
 
 

@@ -796,6 +796,327 @@ __global__ __launch_bounds__(kBlockThreads) void DenseRestageKernel(const T *__r
     }
 }
 
+// The same copy for a destination of at most 32 columns, where a 32 x 32 tile would be mostly padding (1 column:
+// 130 us for 4 M rows): a lane a row, the columns one after the other.  Whatever the two orders, the lanes of an
+// instruction touch consecutive rows of one column or the short rows of consecutive rows.
+// VecSrc / VecDst: that side is row-major with rows of whole, aligned groups of four elements, which then travel
+// as one load or store.
+template <typename T, bool VecSrc, bool VecDst>
+__global__ __launch_bounds__(kBlockThreads) void DenseRestageNarrowKernel(const T *__restrict__ src,
+                                                                          T *__restrict__ dst, int64_t rows,
+                                                                          int32_t cols, int32_t colsDst, int64_t ldSrc,
+                                                                          int32_t srcColMajor, int64_t ldDst,
+                                                                          int32_t dstColMajor)
+{
+    typedef T Vec4 __attribute__((ext_vector_type(4)));
+    const int64_t r = static_cast<int64_t>(blockIdx.x) * kBlockThreads + threadIdx.x;
+    if (r >= rows) {
+        return;
+    }
+    const T *from = src + (srcColMajor ? r : r * ldSrc);
+    T *to = dst + (dstColMajor ? r : r * ldDst);
+    const int64_t stepSrc = srcColMajor ? ldSrc : 1, stepDst = dstColMajor ? ldDst : 1;
+    for (int32_t c0 = 0; c0 < colsDst; c0 += 4) {
+        T v[4];
+        if (VecSrc && c0 + 4 <= cols) {
+            const Vec4 in = *reinterpret_cast<const Vec4 *>(from + c0);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[i] = in[i];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[i] = c0 + i < cols ? from[(c0 + i) * stepSrc] : T(0);
+            }
+        }
+        if (VecDst) {  // (colsDst is whole groups of four)
+            *reinterpret_cast<Vec4 *>(to + c0) = Vec4{v[0], v[1], v[2], v[3]};
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (c0 + i < colsDst) {
+                    to[(c0 + i) * stepDst] = v[i];
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------ narrow B
+// B of one or two 16-byte pieces a row (4 or 8 fp32 columns, 8 or 16 fp16 ones): a lane group spanning the columns
+// would be a lane or two wide, and the kernels above then spend their time on bookkeeping, not on the matrix.  Here
+// the product runs like an SpMV whose vector elements are short rows of B.  A persistent workgroup walks over tiles
+// of consecutive rows - the slabs of the plan's table, cut (MakeNarrowTiling) so that a tile holds at most
+// NarrowEntries(n) entries and its rows times pieces fill the workgroup's lanes a whole number of times.  Per
+// tile: every lane takes consecutive (column, value) pairs four at a time as 16-byte loads, gathers their rows of B
+// whole and drops them, with the values, into LDS; then one lane group per (row, piece of the row of C) adds up
+// its row's products from LDS, in fp64, a lane holding the piece's 4 (fp16: 8) sums.  Three tiles are under way at
+// once: while the sums of tile i are made from LDS, the rows of B of tile i + 1 and the entries of tile i + 2 are
+// in flight, and the tiles' bounds are read two turns further ahead still, so that no turn of the loop waits for a
+// load it has only just asked for.  In LDS the pieces lie so that the lanes of one store instruction - which hold
+// entries four apart - write consecutive slots: entry k of a tile is at slot (k mod 4) E / 4 + k / 4 (stored in
+// the order of the entries, a wavefront's 64 pieces fell on 8 of the 32 banks).  Lanes past the end of a tile load what the last lane inside it loads and store
+// to slots nobody reads: the loop holds no branch that depends on the lane.  Workgroups of one XCD share one
+// contiguous range of tiles.
+constexpr int kNarrowRows = 1023;    // rows of a tile at most (their offsets pass through LDS)
+constexpr int kNarrowMaxRow = 200;   // longest row of a matrix that takes this kernel
+
+// Entries a tile holds at most: a quad a lane.  (Two quads under a one-piece B - 44 KB of LDS, three workgroups a
+// compute unit instead of five - run no faster: what counts is the bytes in flight per compute unit.)
+constexpr int NarrowEntries(int64_t)
+{
+    return 1024;
+}
+
+template <typename ValT, typename CT, typename AccT, int W, int G>
+__global__ __launch_bounds__(kBlockThreads) void SpmmNarrowKernel(
+    const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
+    const ValT *__restrict__ B, CT *C, uint32_t ldb, uint32_t ldc, const int32_t *__restrict__ slabStart,
+    int64_t numSlabs, int64_t nnz, OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16)
+{
+    typedef int32_t Int4A __attribute__((ext_vector_type(4)));
+    constexpr int Q = W * static_cast<int>(sizeof(ValT)) / 16;  // 16-byte pieces of a row of B
+    constexpr int kPiece = 16 / static_cast<int>(sizeof(ValT));  // elements of a piece
+    constexpr int E = NarrowEntries(W);                          // entries of a tile at most
+    constexpr int U = E / (4 * kBlockThreads);                   // quads of entries a lane takes
+    static_assert(Q * kPiece == W && (Q == 1 || Q == 2), "one or two whole pieces");
+    static_assert(U * 4 * kBlockThreads == E && U >= 1, "whole quads");
+    __shared__ __align__(16) unsigned char bRaw[E * Q * 16];
+    __shared__ __align__(16) float valLds[E];
+    __shared__ int32_t rowLds[kNarrowRows + 1];
+    Int4A *const bPieces = reinterpret_cast<Int4A *>(bRaw);
+    typedef float Float4A __attribute__((ext_vector_type(4)));
+
+    const AccT alpha = ReadScalar<AccT>(alphaS);
+    const AccT beta = ReadScalar<AccT>(betaS);
+    const bool betaZero = (beta == AccT(0));
+    const int32_t tid = static_cast<int32_t>(threadIdx.x);
+
+    // This XCD's tiles, and this workgroup's stride through them.
+    const int64_t xcd = blockIdx.x % kNumXcd;
+    const int64_t perXcd = numSlabs / kNumXcd, rem = numSlabs % kNumXcd;
+    const int64_t xcdFirst = xcd * perXcd + (xcd < rem ? xcd : rem);
+    const int64_t xcdTiles = perXcd + (xcd < rem ? 1 : 0);
+    const int64_t stride = (gridDim.x - xcd + kNumXcd - 1) / kNumXcd;  // workgroups living on this XCD
+    const int64_t t0 = blockIdx.x / kNumXcd;
+    if (t0 >= xcdTiles) {
+        return;
+    }
+    const int64_t mine = (xcdTiles - t0 + stride - 1) / stride;  // tiles of this workgroup
+
+    struct Tile {
+        int32_t r0, r1, first, count;
+    };
+    auto loadRows = [&](int64_t i, Tile &m) {
+        const int64_t slab = xcdFirst + t0 + i * stride;
+        m.r0 = slabStart[slab];
+        m.r1 = slabStart[slab + 1];
+    };
+    auto loadEntries = [&](Tile &m) {
+        m.first = rowOffsets[m.r0];
+        m.count = rowOffsets[m.r1] - m.first;
+    };
+    // A tile that does not fit - the row offsets changed since the table was made - is summed straight from memory.
+    auto fits = [&](const Tile &m) {
+        return m.count >= 0 && m.count <= E && m.r1 - m.r0 <= kNarrowRows && m.first >= 0 &&
+               static_cast<int64_t>(m.first) + m.count <= nnz;
+    };
+
+    Int4U colN[U];
+    ValT valN[U][4];
+    Int4A piece[U][4][Q];
+    float valP[U][4];
+    constexpr int kBoundRegs = (kNarrowRows + 1) / kBlockThreads;
+    int32_t bnd[kBoundRegs];
+    // Requests this lane's entries of a tile that holds any; nothing is waited for.  A quad that would reach past
+    // the end of the arrays is read a few entries earlier (nnz >= 4), and issueGather moves its entries into place.
+    auto issueQuads = [&](const Tile &m) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if ((u * kBlockThreads + (tid & ~(kWave - 1))) * 4 >= m.count) {
+                continue;
+            }
+            int64_t at = static_cast<int64_t>(m.first) + (u * kBlockThreads + tid) * 4;
+            at = at + 4 <= nnz ? at : nnz - 4;
+            colN[u] = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(colInd + at));
+            if constexpr (sizeof(ValT) == 4) {
+                const Int4U v = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(vals + at));
+                __builtin_memcpy(valN[u], &v, 16);
+            } else {
+                const Short4U v = __builtin_nontemporal_load(reinterpret_cast<const Short4U *>(vals + at));
+                __builtin_memcpy(valN[u], &v, 8);
+            }
+        }
+    };
+    // Requests the rows of B of the entries issueQuads asked for (waiting for those), and the tile's row offsets.
+    // An entry past the tile's end takes the row of B of the tile's first entry.
+    auto issueGather = [&](const Tile &m) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t at = static_cast<int64_t>(m.first) + (u * kBlockThreads + tid) * 4;
+            int64_t late = at + 4 - nnz;  // entries by which the quad was read early
+            late = late > 3 ? 3 : late;
+            for (; late > 0; --late) {    // (the last lanes of the last tile)
+                colN[u] = Int4U{colN[u][1], colN[u][2], colN[u][3], colN[u][3]};
+                valN[u][0] = valN[u][1];
+                valN[u][1] = valN[u][2];
+                valN[u][2] = valN[u][3];
+            }
+        }
+        const int32_t colSafe = __shfl(colN[0][0], 0, kWave);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if ((u * kBlockThreads + (tid & ~(kWave - 1))) * 4 >= m.count) {
+                continue;  // a wavefront whose entries all lie past the tile's end
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int32_t k = (u * kBlockThreads + tid) * 4 + i;
+                const uint32_t col = static_cast<uint32_t>(k < m.count ? colN[u][i] : colSafe);
+                const ValT *bRow = B + static_cast<uint64_t>(col) * ldb;
+#pragma unroll
+                for (int q = 0; q < Q; ++q) {
+                    piece[u][i][q] = *reinterpret_cast<const Int4A *>(bRow + q * kPiece);
+                }
+                valP[u][i] = static_cast<float>(valN[u][i]);
+            }
+        }
+        const int32_t tileRows = m.r1 - m.r0;
+#pragma unroll
+        for (int b = 0; b < kBoundRegs; ++b) {
+            if (b * kBlockThreads <= tileRows) {
+                const int32_t rr = b * kBlockThreads + tid;
+                bnd[b] = rowOffsets[m.r0 + (rr < tileRows ? rr : tileRows)];
+            }
+        }
+    };
+
+    Tile m0{}, m1{}, m2{}, m3{};
+    loadRows(0, m0);
+    loadEntries(m0);
+    if (mine > 1) {
+        loadRows(1, m1);
+        loadEntries(m1);
+    }
+    if (mine > 2) {
+        loadRows(2, m2);
+        loadEntries(m2);
+    }
+    if (mine > 3) {
+        loadRows(3, m3);
+    }
+    if (fits(m0) && m0.count > 0) {
+        issueQuads(m0);
+        issueGather(m0);
+    }
+    if (mine > 1 && fits(m1) && m1.count > 0) {
+        issueQuads(m1);
+    }
+
+    constexpr int kGroups = kBlockThreads / G;
+    const int32_t lane = tid % G;
+    for (int64_t i = 0; i < mine; ++i) {
+        Tile m4{};
+        if (i + 4 < mine) {
+            loadRows(i + 4, m4);
+        }
+        if (i + 3 < mine) {
+            loadEntries(m3);
+        }
+        const bool staged = fits(m0);
+        const int32_t tileRows = m0.r1 - m0.r0;
+        if (staged && m0.count > 0) {
+#pragma unroll
+            for (int b = 0; b < kBoundRegs; ++b) {
+                if (b * kBlockThreads <= tileRows) {
+                    const int32_t rr = b * kBlockThreads + tid;
+                    rowLds[rr < tileRows ? rr : tileRows] = bnd[b];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int32_t k = (u * kBlockThreads + tid) * 4;
+                if ((u * kBlockThreads + (tid & ~(kWave - 1))) * 4 >= m0.count) {
+                    continue;
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+#pragma unroll
+                    for (int q = 0; q < Q; ++q) {
+                        bPieces[q * E + e * (E / 4) + (k >> 2)] = piece[u][e][q];
+                    }
+                }
+                *reinterpret_cast<Float4A *>(valLds + k) = Float4A{valP[u][0], valP[u][1], valP[u][2], valP[u][3]};
+            }
+        }
+        LdsBarrier();
+        if (i + 1 < mine && fits(m1) && m1.count > 0) {
+            issueGather(m1);
+        }
+        if (i + 2 < mine && fits(m2) && m2.count > 0) {
+            issueQuads(m2);
+        }
+
+        // one lane group per piece of the tile's rows of C
+        const int32_t items = tileRows * Q;
+        for (int32_t it = tid / G; it < items; it += kGroups) {
+            const int32_t rr = it / Q, q = it % Q;
+            AccT acc[kPiece];
+#pragma unroll
+            for (int c = 0; c < kPiece; ++c) {
+                acc[c] = AccT(0);
+            }
+            if (staged && m0.count > 0) {
+                int32_t s = rowLds[rr] - m0.first, e = rowLds[rr + 1] - m0.first;
+                s = s < 0 ? 0 : s;
+                e = e > m0.count ? m0.count : e;
+                for (int32_t k = s + lane; k < e; k += G) {
+                    const AccT v = static_cast<AccT>(valLds[k]);
+                    const Int4A p = bPieces[q * E + (k & 3) * (E / 4) + (k >> 2)];
+                    ValT b[kPiece];
+                    __builtin_memcpy(b, &p, 16);
+#pragma unroll
+                    for (int c = 0; c < kPiece; ++c) {
+                        acc[c] += v * ToAcc<AccT>(b[c]);
+                    }
+                }
+            } else {
+                const int64_t s = rowOffsets[m0.r0 + rr], e = rowOffsets[m0.r0 + rr + 1];
+                for (int64_t k = s + lane; k < e; k += G) {
+                    const AccT v = ToAcc<AccT>(vals[k]);
+                    const ValT *bRow = B + static_cast<uint64_t>(static_cast<uint32_t>(colInd[k])) * ldb + q * kPiece;
+#pragma unroll
+                    for (int c = 0; c < kPiece; ++c) {
+                        acc[c] += v * ToAcc<AccT>(bRow[c]);
+                    }
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < kPiece; ++c) {
+                acc[c] = GroupSum<G>(acc[c]);
+            }
+            if (lane == 0) {
+                CT *out = C + static_cast<uint64_t>(static_cast<uint32_t>(m0.r0 + rr)) * ldc + q * kPiece;
+                CT res[kPiece];
+#pragma unroll
+                for (int c = 0; c < kPiece; ++c) {
+                    res[c] = Epilogue<CT, AccT>::Apply(acc[c], alpha, beta, betaZero, out + c, clampF16 != 0);
+                }
+#pragma unroll
+                for (int c = 0; c < kPiece; ++c) {
+                    out[c] = res[c];
+                }
+            }
+        }
+        LdsBarrier();  // everyone is done with the tile before the next one overwrites it; its loads stay in flight
+        m0 = m1;
+        m1 = m2;
+        m2 = m3;
+        m3 = m4;
+    }
+}
+
 // Longest row, number of long rows and number of segments.  stats[0..2] zeroed
 // before the launch.
 __global__ __launch_bounds__(kBlockThreads) void SpmmRowStatsKernel(const int32_t *__restrict__ rowOffsets,
@@ -852,15 +1173,81 @@ inline int CheckLaunch()
 
 inline int64_t Align256(int64_t v) { return (v + 255) / 256 * 256; }
 
+// Number of compute units of the current device (256 on MI355X), read once.
+inline int ComputeUnits()
+{
+    static const int cus = [] {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess ||
+            prop.multiProcessorCount <= 0) {
+            (void)hipGetLastError();
+            return 256;
+        }
+        return prop.multiProcessorCount;
+    }();
+    return cus;
+}
+
 // Slabs of the slab kernel: about kSlabTarget entries each, cut where the running count of entries + rows passes
 // a multiple of `share` (a row costs its entries and one row of C), so that a matrix whose rows are sorted by
 // length is cut as evenly as one whose rows are mixed.  Half as long where no row exceeds 64 entries and B has at
 // most 128 columns: 1 M rows of 32, n = 64, 1.215 -> 1.187 ms; 2 M rows of 16 1.245 -> 1.213 ms (with longer rows
 // among them the shorter slabs lose: a power-law graph 1.38 -> 1.47 ms; with 256 columns 5.45 -> 5.52 ms).
+// The tiles of SpmmNarrowKernel for a B of at most 16 columns under rows of at most kNarrowMaxRow entries.  The
+// kernel gives a lane group to every 16-byte piece of a row of C: a tile of R rows and p pieces a row keeps the 256
+// lanes busy when R p times the lanes of a group is just below a multiple of 256.  R and the lanes of a group are
+// chosen here (for fp32 pieces; fp16 rows have half as many pieces and take twice the lanes), and the slab table
+// is cut with share = R (mean + 1): a slab's entries + rows stay below share + maxRow + 1 (SpmmSlabTableKernel),
+// so a tile holds about R rows and never more than NarrowEntries(n) entries.
+struct NarrowTiling {
+    bool ok;
+    int64_t share;
+    int32_t lanes;  // of a lane group, fp32
+};
+
+NarrowTiling MakeNarrowTiling(int64_t rows, int64_t nnz, int32_t maxRow, int64_t n)
+{
+    NarrowTiling t{};
+    if (n < 1 || n > 16 || maxRow < 1 || maxRow > kNarrowMaxRow || rows <= 0 || nnz <= 0) {
+        return t;
+    }
+    const double perRow = static_cast<double>(nnz) / static_cast<double>(rows) + 1.0;  // entries and the row itself
+    const double budget = static_cast<double>(NarrowEntries(n) - maxRow);
+    const int64_t pieces = (n + 3) / 4;
+    for (int32_t lanes = 1; lanes <= 32; lanes *= 2) {
+        const int64_t full = 250 / (lanes * pieces);  // rows that fill the lanes once (with a little room)
+        if (full < 1) {
+            break;
+        }
+        if (static_cast<double>(full) * perRow > budget) {
+            continue;
+        }
+        int64_t r = full;
+        if (lanes == 1) {
+            while (r + full <= 3 * full && static_cast<double>(r + full) * perRow <= budget) {
+                r += full;  // very short rows: two or three turns of the lanes a tile
+            }
+        }
+        t.ok = true;
+        t.share = static_cast<int64_t>(static_cast<double>(r) * perRow);
+        t.share = t.share < 1 ? 1 : t.share;
+        t.lanes = lanes;
+        return t;
+    }
+    return t;
+}
+
 int64_t SlabShare(int64_t rows, int64_t nnz, int32_t maxRow, int64_t n)
 {
     static const int64_t fixed =
         std::getenv("OPS_SPARSE_SPMM_SLAB_ENTRIES") != nullptr ? std::atoll(std::getenv("OPS_SPARSE_SPMM_SLAB_ENTRIES")) : 0;
+    if (fixed <= 0) {
+        const NarrowTiling narrow = MakeNarrowTiling(rows, nnz, maxRow, n);
+        if (narrow.ok) {
+            return narrow.share;
+        }
+    }
     const int64_t target = fixed > 0 ? fixed : (maxRow > 0 && maxRow <= 64 && n <= 128 ? kSlabTarget / 2 : kSlabTarget);
     const int64_t t = target < 64 ? 64 : target;
     int64_t rps = nnz > 0 ? t * rows / nnz : 4096;
@@ -881,8 +1268,13 @@ void LayoutPlan(OpsparseSpmmPlan *p)
     int64_t off = 256;
     p->numSlabs = SlabCount(p->rows, p->nnz, p->maxRowNnz, p->n);  // (maxRowNnz and n set by the caller)
     p->slabStartOff = off;
-    // Room for the table of a narrow B whatever n is: a buffer sized for a wide B serves a narrower one as well.
-    const int64_t reserveSlabs = SlabCount(p->rows, p->nnz, p->maxRowNnz, 1);
+    // Room for the table of any narrower B: a buffer sized for a wide B serves a narrower one as well.  (The share
+    // of a slab depends on the pieces of 16 bytes in a row of B up to four of them, and not on n beyond.)
+    int64_t reserveSlabs = 0;
+    for (int64_t width : {4, 8, 12, 16, 17}) {
+        const int64_t count = SlabCount(p->rows, p->nnz, p->maxRowNnz, width);
+        reserveSlabs = count > reserveSlabs ? count : reserveSlabs;
+    }
     off = Align256(off + 4 * ((reserveSlabs > p->numSlabs ? reserveSlabs : p->numSlabs) + 1));
     const int64_t slabEnd = off;
     p->longRowsOff = off;
@@ -1110,6 +1502,80 @@ int LaunchSlab(const SpmmArgs &a)
     return CheckLaunch();
 }
 
+// SpmmNarrowKernel for a plan whose slab table was cut for it; W = a.n columns.
+template <typename ValT, typename CT, typename AccT, int W>
+int LaunchNarrow(const SpmmArgs &a)
+{
+    const auto *slabStart =
+        reinterpret_cast<const int32_t *>(static_cast<unsigned char *>(a.ws) + a.plan->slabStartOff);
+    const NarrowTiling tiling = MakeNarrowTiling(a.plan->rows, a.plan->nnz, a.plan->maxRowNnz, a.plan->n);
+    // the tiling counted fp32 pieces: rows of fp16 have half as many, and twice the lanes each
+    const int lanes = tiling.lanes * (4 / static_cast<int>(sizeof(ValT)));
+    auto launch = [&](auto tag) {
+        constexpr int G = decltype(tag)::value;
+        static const int fit = [] {
+            int blocks = 1;
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, SpmmNarrowKernel<ValT, CT, AccT, W, G>,
+                                                             kBlockThreads, 0) != hipSuccess ||
+                blocks < 1) {
+                (void)hipGetLastError();
+                blocks = 1;
+            }
+            return blocks;
+        }();
+        // persistent: the workgroups that fit the device at once walk over all tiles
+        const int64_t resident = static_cast<int64_t>(ComputeUnits()) * fit;
+        const uint32_t grid = static_cast<uint32_t>(a.plan->numSlabs < resident ? a.plan->numSlabs : resident);
+        hipLaunchKernelGGL((SpmmNarrowKernel<ValT, CT, AccT, W, G>), dim3(grid), dim3(kBlockThreads), 0, a.stream,
+                           a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.B),
+                           static_cast<CT *>(a.C), static_cast<uint32_t>(a.ldb), static_cast<uint32_t>(a.ldc),
+                           slabStart, a.plan->numSlabs, a.nnz, a.alpha, a.beta, a.clampF16);
+        return CheckLaunch();
+    };
+    // fp32: 1 .. 32 lanes, fp16: 2 .. 64; with 16 columns (four fp32 pieces in the tiling's count) the tiling stops
+    // at 16, because three rows of at most kNarrowMaxRow entries always fit a tile
+    constexpr int kMin = 4 / static_cast<int>(sizeof(ValT));
+    constexpr int kMax = (W >= 16 ? 16 : 32) * kMin;
+    auto pick = [&](auto tag) {
+        constexpr int G = decltype(tag)::value;
+        if constexpr (G >= kMin && G <= kMax) {
+            return launch(tag);
+        } else {
+            return static_cast<int>(OPSPARSE_E_INVALID);
+        }
+    };
+    switch (lanes) {
+        case 1: return pick(std::integral_constant<int, 1>{});
+        case 2: return pick(std::integral_constant<int, 2>{});
+        case 4: return pick(std::integral_constant<int, 4>{});
+        case 8: return pick(std::integral_constant<int, 8>{});
+        case 16: return pick(std::integral_constant<int, 16>{});
+        case 32: return pick(std::integral_constant<int, 32>{});
+        case 64: return pick(std::integral_constant<int, 64>{});
+        default: return OPSPARSE_E_INVALID;
+    }
+}
+
+// Whether the product takes SpmmNarrowKernel: whole 16-byte rows of B of one or two pieces, an analysed matrix of
+// short rows whose slab table was cut for that kernel.
+template <typename ValT>
+bool UseNarrowKernel(const SpmmArgs &a)
+{
+    const bool off = std::getenv("OPS_SPARSE_SPMM_NO_NARROW") != nullptr;  // (read at every call: tests switch it)
+    const int64_t rowBytes = a.n * static_cast<int64_t>(sizeof(ValT));
+    if (off || sizeof(ValT) < 2 || (rowBytes != 16 && rowBytes != 32) || a.plan == nullptr || a.ws == nullptr ||
+        a.ldb > UINT32_MAX || a.ldc > UINT32_MAX || a.nnz < 4 || a.plan->n != a.n) {
+        return false;
+    }
+    const OpsparseSpmmPlan &p = *a.plan;
+    if (p.kernel == OPSPARSE_SPMM_BINNED || p.numLongRows != 0 || p.slabStartOff <= 0 || p.numSlabs <= 0 ||
+        std::getenv("OPS_SPARSE_SPMM_NO_SLAB_TABLE") != nullptr) {
+        return false;
+    }
+    const NarrowTiling tiling = MakeNarrowTiling(p.rows, p.nnz, p.maxRowNnz, p.n);
+    return tiling.ok && SlabShare(p.rows, p.nnz, p.maxRowNnz, p.n) == tiling.share;
+}
+
 template <typename ValT, typename CT, typename AccT, int L>
 int LaunchGeneral(const SpmmArgs &a)
 {
@@ -1144,6 +1610,11 @@ int RunTypedV(const SpmmArgs &a)
         return RunGeneral<ValT, CT, AccT>(a);
     }
     const int64_t lanesNeeded = a.n / V;
+    if constexpr (V * sizeof(ValT) == 16) {
+        if (UseNarrowKernel<ValT>(a)) {
+            return lanesNeeded == 1 ? LaunchNarrow<ValT, CT, AccT, V>(a) : LaunchNarrow<ValT, CT, AccT, 2 * V>(a);
+        }
+    }
     const bool slab = UseSlabKernel(a, lanesNeeded);
     auto launch = [&](auto tag) {
         constexpr int L = decltype(tag)::value;
@@ -1361,12 +1832,35 @@ int opsparse_dense_restage(const void *src, void *dst, int64_t rows, int64_t col
     if (src == nullptr || dst == nullptr) {
         return OPSPARSE_E_INVALID;
     }
+    auto s = static_cast<hipStream_t>(stream);
+    if (colsDst <= 32 && (rows + kBlockThreads - 1) / kBlockThreads <= INT32_MAX) {
+        const dim3 narrowGrid(static_cast<uint32_t>((rows + kBlockThreads - 1) / kBlockThreads));
+        const uintptr_t group = 4 * static_cast<uintptr_t>(elemBytes);
+        const bool vecSrc = !srcColMajor && ldSrc % 4 == 0 && reinterpret_cast<uintptr_t>(src) % group == 0;
+        const bool vecDst = !dstColMajor && ldDst % 4 == 0 && colsDst % 4 == 0 &&
+                            reinterpret_cast<uintptr_t>(dst) % group == 0;
+        auto launch = [&](auto zero) {
+            using T = decltype(zero);
+            auto kernel = vecSrc ? (vecDst ? DenseRestageNarrowKernel<T, true, true> : DenseRestageNarrowKernel<T, true, false>)
+                                 : (vecDst ? DenseRestageNarrowKernel<T, false, true> : DenseRestageNarrowKernel<T, false, false>);
+            hipLaunchKernelGGL(kernel, narrowGrid, dim3(kBlockThreads), 0, s, static_cast<const T *>(src),
+                               static_cast<T *>(dst), rows, static_cast<int32_t>(cols), static_cast<int32_t>(colsDst),
+                               ldSrc, srcColMajor, ldDst, dstColMajor);
+        };
+        if (elemBytes == 4) {
+            launch(uint32_t{});
+        } else if (elemBytes == 2) {
+            launch(uint16_t{});
+        } else {
+            launch(uint8_t{});
+        }
+        return CheckLaunch();
+    }
     const int64_t across = (colsDst + 31) / 32, down = (rows + 31) / 32;
     if (across * down > INT32_MAX) {
         return OPSPARSE_E_UNSUPPORTED;
     }
     const dim3 grid(static_cast<uint32_t>(across * down));
-    auto s = static_cast<hipStream_t>(stream);
     switch (elemBytes) {
         case 4:
             hipLaunchKernelGGL(DenseRestageKernel<uint32_t>, grid, dim3(kBlockThreads), 0, s,

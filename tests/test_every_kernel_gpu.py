@@ -479,6 +479,68 @@ def test_spmm_slab_kernel_with_64_bit_gather_addresses_every_width(osa, gpu_ctx,
         torch.cuda.empty_cache()
 
 
+NARROW_WIDTHS = {"f32": (4, 8), "f16_f16": (8, 16), "f16_f32": (8, 16)}      # one and two 16-byte pieces a row of B
+
+
+@pytest.mark.parametrize("types", list(NARROW_WIDTHS))
+@pytest.mark.parametrize("mean", [2, 6, 12, 25, 50, 100, 180])
+def test_spmm_narrow_kernel_every_width_and_lane_group(osa, gpu_ctx, types, mean, monkeypatch):
+    """SpmmNarrowKernel<ValT, CT, AccT, W, G> for a B of one or two 16-byte pieces a row under an analysed matrix of
+    short rows.  Rows of exactly `mean` entries select the lanes of a group: with one fp32 piece 1, 2, 4, 8, 16, 32
+    for means 2 .. 100; with two pieces the same from 6 .. 180; fp16 rows take twice the lanes, and 16 fp16
+    columns 2 .. 32.  The number of entries is odd, so the last lanes of the last tile read their entries a few
+    places early and move them; B and C have a padded leading dimension; beta is zero and not.  The same plan with
+    the kernel switched off must agree as well (SpmmSlabKernel)."""
+    m, k = 1201, 5000
+    for n in NARROW_WIDTHS[types]:
+        if n == 4 and mean == 180:
+            continue                                                     # (a 32-lane group is at mean 100 there)
+        lengths = np.full(m, mean)
+        lengths[::7] = mean - 1 if mean > 2 else 0                       # some variety; the longest row stays `mean`
+        if lengths.sum() % 4 == 0:
+            lengths[1] -= 1
+        p = RawSpmm(osa, gpu_ctx, types, m, k, n, lengths, seed=mean + n, ldb=n + 16)
+        assert p.nnz % 4 != 0
+        plan = p.analyse()
+        assert plan.kernel != osa.OPSPARSE_SPMM_BINNED and plan.maxRowNnz == mean and plan.slabStartOff > 0
+        p.launch_and_check(plan, 1.5, 0.0)
+        p.launch_and_check(plan, 0.75, -0.5)
+        monkeypatch.setenv("OPS_SPARSE_SPMM_NO_NARROW", "1")
+        p.launch_and_check(plan, 0.75, -0.5)
+        monkeypatch.delenv("OPS_SPARSE_SPMM_NO_NARROW")
+
+
+def test_spmm_narrow_kernel_rows_of_no_or_one_entry(osa, gpu_ctx):
+    """Rows of 0 or 1 entries: a tile holds two turns of the lanes (500 rows), and whole stretches of empty rows."""
+    m, k = 20000, 3000
+    rng = np.random.default_rng(5)
+    lengths = rng.integers(0, 2, m)
+    lengths[3000:6000] = 0
+    lengths[9000:9600] = 1
+    for types, n in (("f32", 4), ("f32", 8), ("f16_f32", 16)):
+        p = RawSpmm(osa, gpu_ctx, types, m, k, n, lengths, seed=n)
+        plan = p.analyse()
+        assert plan.maxRowNnz == 1 and plan.slabStartOff > 0
+        p.launch_and_check(plan, 2.0, 0.25)
+
+
+def test_spmm_narrow_kernel_on_row_offsets_that_changed_since_the_analysis(osa, gpu_ctx):
+    """The slab table is made for the row offsets Preprocess saw.  A caller of the launch layer who passes other
+    offsets of the same rows and entries with that plan still gets the product: a tile that no longer fits the
+    kernel's LDS is summed straight from memory."""
+    m, k, n = 4000, 6000, 4
+    even = np.full(m, 6)
+    p = RawSpmm(osa, gpu_ctx, "f32", m, k, n, even, seed=3)
+    plan = p.analyse()
+    skew = even.copy()
+    skew[:100] = 126                                                     # 100 x 120 more entries in front ...
+    skew[100:2100] = 0                                                   # ... taken from the 2000 rows behind
+    assert skew.sum() == even.sum()
+    q = RawSpmm(osa, gpu_ctx, "f32", m, k, n, skew, seed=4)
+    q.ws = p.ws
+    q.launch_and_check(plan, 1.0, 0.5)
+
+
 # ---------------------------------------------------------------------------------------------- blocked layouts
 
 def _wide_matrix(rows, cols, seed, long_rows=(), per_row=20):

@@ -482,6 +482,49 @@ def test_layouts_through_the_staging_area(osa, gpu_ctx, b_rm, c_rm, trans_b, n, 
         assert oracle.max_rel_err(got, gold) <= tol
 
 
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("b_rm,c_rm", [(True, True), (False, False), (True, False)])
+@pytest.mark.parametrize("half", [False, True])
+def test_few_columns_on_a_mesh(osa, gpu_ctx, n, b_rm, c_rm, half):
+    """One to eight columns of B under a 7-point mesh matrix (block Krylov methods, a few right-hand sides): the
+    widths are padded to whole 16-byte rows in the staging area where they are not, and the product of one or two
+    such pieces a row takes the kernel for narrow B.  Every layout, fp32 and fp16 values, beta zero (C holds NaN
+    and must not be read) and not."""
+    side = 24
+    m = k = side ** 3
+    r = np.arange(m)
+    z, y, x = r // (side * side), (r // side) % side, r % side
+    cols, keep = [], []
+    for d, coord in ((-side * side, z), (-side, y), (-1, x), (0, None), (1, x), (side, y), (side * side, z)):
+        ok = np.ones(m, bool) if coord is None else ((coord > 0) if d < 0 else (coord < side - 1))
+        cols.append(r + d)
+        keep.append(ok)
+    cols, keep = np.stack(cols, 1), np.stack(keep, 1)
+    rowptr = np.concatenate([[0], np.cumsum(keep.sum(1))]).astype(np.int32)
+    colind = cols[keep].astype(np.int32)
+    rng = np.random.default_rng(n + 10 * b_rm + 20 * c_rm)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    ldb = (n + 3) if b_rm else (k + 2)
+    ldc = (n + 1) if c_rm else (m + 6)
+    B = rng.uniform(-1, 1, (k if b_rm else n) * ldb).astype(np.float32)
+    vd, cd = (torch.float16, torch.float32) if half else (None, None)
+    if half:
+        val, B = (torch.from_numpy(a).to(torch.float16).float().numpy() for a in (val, B))
+    for alpha, beta in ((1.25, 0.0), (0.5, -1.5)):
+        C0 = rng.uniform(-1, 1, (m if c_rm else n) * ldc).astype(np.float32)
+        C_in = C0.copy()
+        if beta == 0.0:
+            idx = (np.arange(m)[:, None] * ldc + np.arange(n)[None, :]) if c_rm else \
+                  (np.arange(m)[:, None] + np.arange(n)[None, :] * ldc)
+            C_in[idx.ravel()] = np.nan
+        got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, ldb, C_in, ldc, alpha, beta,
+                       order_b=osa.ACL_SPARSE_ORDER_ROW if b_rm else osa.ACL_SPARSE_ORDER_COL,
+                       order_c=osa.ACL_SPARSE_ORDER_ROW if c_rm else osa.ACL_SPARSE_ORDER_COL, val_dtype=vd, c_dtype=cd)
+        gold = oracle.spmm_f64(m, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta, b_row_major=b_rm,
+                               trans_b=False, c_row_major=c_rm)
+        assert oracle.max_rel_err(got, gold) <= 1e-5
+
+
 def test_staging_needs_a_buffer_preprocessed_for_it(osa, gpu_ctx):
     """A buffer sized and preprocessed for row-major operands (256 bytes here) and then used with a column-major B:
     no staging area was promised, the product must run in place (slowly) and stay inside the buffer — the guard
