@@ -742,6 +742,73 @@ def run_stencils(args, osa, wl, torch, dev, stream, handle):
     return res
 
 
+def run_few_columns(args, osa, wl, torch, dev, stream, handle):
+    """SpMM with one to sixteen columns of B (a few right-hand sides, block Krylov methods) on meshes: time of a
+    call after Preprocess (alpha = 1, beta = 0), the algorithmic bytes against 8 TB/s, the same product as n
+    SpMV calls, and the call with the kernel for narrow B switched off (the lane-group kernels it replaced)."""
+    import itertools
+    box3 = list(itertools.product((-1, 0, 1), repeat=3))
+    cross3 = [o for o in box3 if sum(abs(v) for v in o) <= 1]
+    cross2 = [(-1, 0), (0, -1), (0, 0), (0, 1), (1, 0)]
+    shapes = [
+        ("5-point, 2048^2 (c2)", lambda: wl.stencil_csr((2048, 2048), cross2, dev)),
+        ("7-point, 160^3", lambda: wl.stencil_csr((160, 160, 160), cross3, dev)),
+        ("27-point, 128^3", lambda: wl.stencil_csr((128, 128, 128), box3, dev)),
+    ]
+    if args.scale < 1.0:
+        shapes = shapes[:1]
+    cases = [(torch.float32, n, order) for n in (1, 2, 4, 8) for order in ("row", "col")]
+    cases += [(torch.float16, 8, "row"), (torch.float16, 16, "row")]
+    res = {}
+    for name, make in shapes:
+        torch.cuda.empty_cache()
+        A = make()
+        rows, nnz = A["rows"], int(A["colind"].numel())
+        x = wl.uniform(5, rows, -1.0, 1.0, dev)
+        y = torch.zeros(rows, dtype=torch.float32, device=dev)
+        csr32 = osa.Csr(rows, rows, A["rowptr"], A["colind"], A["values"])
+        sv = osa.SpmvOp(handle, csr32, osa.DnVec(x), osa.DnVec(y))
+        for _ in range(5 + args.settle):   # (the clocks' ramp and the runtime's one-off stall: see run_workload)
+            sv(1.0, 0.0)
+        stream.synchronize()
+        spmv_us = time_rounds(torch, stream, lambda i: sv(1.0, 0.0), args.steps, None, args.min_gpu_ms)[0] * 1e3
+        res[name] = {"rows": rows, "nnz": nnz, "spmv_us": round(spmv_us, 2), "cases": {}}
+        log("%s: SpMV %.1f us" % (name, spmv_us))
+        for dtype, n, order in cases:
+            vb = 4 if dtype == torch.float32 else 2
+            vals = A["values"].to(dtype)
+            csr = osa.Csr(rows, rows, A["rowptr"], A["colind"], vals)
+            B = wl.uniform(7, rows * n, -1.0, 1.0, dev).to(dtype)
+            C = torch.zeros(rows * n, dtype=torch.float32, device=dev)
+            if order == "row":
+                dB, dC = osa.DnMat(rows, n, n, B), osa.DnMat(rows, n, n, C)
+            else:
+                dB = osa.DnMat(rows, n, rows, B, osa.ACL_SPARSE_ORDER_COL)
+                dC = osa.DnMat(rows, n, rows, C, osa.ACL_SPARSE_ORDER_COL)
+            op = osa.SpmmOp(handle, csr, dB, dC)
+            line = {}
+            for label, env in (("us_per_call", None), ("us_without_the_narrow_kernel", "OPS_SPARSE_SPMM_NO_NARROW")):
+                if env is not None:
+                    os.environ[env] = "1"
+                for _ in range(5):
+                    op(1.0, 0.0)
+                stream.synchronize()
+                ms = time_rounds(torch, stream, lambda i: op(1.0, 0.0), args.steps, None, args.min_gpu_ms)[0]
+                line[label] = round(ms * 1e3, 2)
+                if env is not None:
+                    del os.environ[env]
+            bytes_alg = wl.spmm_bytes_alg(rows, rows, n, nnz, vb, vb, 4, False)
+            line["bytes_alg"] = bytes_alg
+            line["frac_of_8TBs"] = round(bytes_alg / (line["us_per_call"] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)
+            line["n_spmv_calls_us"] = round(n * spmv_us, 2)
+            key = "%s n=%d %s-major" % ("fp32" if vb == 4 else "fp16->fp32", n, order)
+            res[name]["cases"][key] = line
+            log("  %-28s %s" % (key, json.dumps(line)))
+            del op, csr, B, C, dB, dC
+        del sv, csr32, A, x, y
+    return res
+
+
 def run_cache_probe(args, osa, wl, torch, dev, stream, handle):
     """What the 256 MB Infinity Cache is worth on this path.  (1) The copy and read kernels on buffers from 8 MiB
     to 1 GiB, launched back to back on the same buffer.  (2) The c4 product (1 M rows of 32 entries, n = 64,
@@ -868,10 +935,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all",
                     choices=["all", "c1", "c2", "c3", "c3_repeatable", "c3_transposed", "c4", "c5", "convert", "cache",
-                             "shapes", "stencils"],
+                             "shapes", "stencils", "few_columns"],
                     help="all: c2 as the headline plus c1, c3 (default plan, repeatable default plan, ALG2, "
                          "transposed), c4 and c5 in `workloads`; shapes: the grid of secondary shapes behind the "
-                         "selection thresholds; stencils: the headline kernels on other meshes and bands")
+                         "selection thresholds; stencils: the headline kernels on other meshes and bands; "
+                         "few_columns: SpMM with 1 - 16 columns of B on meshes")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
     ap.add_argument("--min-gpu-ms", type=float, default=50.0,
                     help="rounds of --steps launches are repeated until this much GPU time has been timed")
@@ -923,6 +991,12 @@ def main():
         print(json.dumps({"metric": "CSR SpMV fp32 on meshes and bands, time per call and algorithmic bytes / 8 TB/s",
                           "unit": "us", "data": "synthetic",
                           "shapes": run_stencils(args, osa, wl, torch, dev, stream, handle)}), flush=True)
+        handle.close()
+        return
+    if args.workload == "few_columns":
+        print(json.dumps({"metric": "CSR SpMM with few columns of B on meshes, time per call and algorithmic bytes / "
+                                    "8 TB/s", "unit": "us", "data": "synthetic",
+                          "shapes": run_few_columns(args, osa, wl, torch, dev, stream, handle)}), flush=True)
         handle.close()
         return
     if args.workload == "convert":

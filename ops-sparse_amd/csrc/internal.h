@@ -70,6 +70,11 @@ struct OpsparseSpmmBinding {
     OpsparseSpmmPlan plan{};
     int64_t stagingBytes = 0;  // room behind the plan's tables for row-major copies of B / C (0: none)
     int64_t widestN = 0;       // the widest C the buffer has been analysed for: its tables fit that width and less
+    // One or two columns of B and C that are vectors in memory run as SpMV calls: their plan, and where in the
+    // buffer its workspace lies (0: the buffer was not preprocessed for such operands).
+    OpsparseSpmvPlan vectorPlan{};
+    int64_t vectorOff = 0;
+    int64_t vectorBytes = 0;
 };
 
 // reference: sparse/common/aclsparse_handle_internal.h:56-72

@@ -149,6 +149,24 @@ int64_t PlanWidth(const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *B, co
     return g.bytes > 0 ? g.nPadded : C->cols;
 }
 
+// One or two columns that lie in memory as vectors (column-major operands; a single column with a leading dimension
+// of 1): the product is then n SpMV calls, which read the matrix n times and still beat the SpMM kernels, whose
+// rows of B would be padded to 16 bytes in the staging area (5-point mesh of 4 M rows, n = 1: 37 us against 98 us;
+// n = 2: 75 against 103; from n = 3 on the padded product wins).  fp32, and fp16 with fp32 C: the fp16 C of SpMM
+// is clamped to the finite range before rounding, which the SpMV kernels do not do.
+bool ColumnsAreVectors(const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *B, const aclsparseDnMatDescr *C,
+                       aclsparseOperation_t opB, const SpmmTypes &t)
+{
+    const int64_t n = C->cols;
+    if (n < 1 || n > 2 || opB != ACL_SPARSE_OP_NON_TRANSPOSE || A->rows <= 0 || A->cols <= 0 || A->nnz <= 0 ||
+        A->nnz > INT32_MAX || t.cType != OPSPARSE_F32 || (t.valType != OPSPARSE_F32 && t.valType != OPSPARSE_F16)) {
+        return false;
+    }
+    const bool bVectors = B->order == ACL_SPARSE_ORDER_COL ? B->ld >= A->cols : (n == 1 && B->ld == 1);
+    const bool cVectors = C->order == ACL_SPARSE_ORDER_COL ? C->ld >= A->rows : (n == 1 && C->ld == 1);
+    return bVectors && cVectors;
+}
+
 // Row statistics and long-row tables for width n into `buffer`; binds the buffer to A.
 aclsparseStatus_t BuildPlan(const aclsparseSpMatDescr *A, int64_t n, void *buffer, hipStream_t stream)
 {
@@ -173,7 +191,14 @@ aclsparseStatus_t BuildPlan(const aclsparseSpMatDescr *A, int64_t n, void *buffe
     A->spmm.buffer = buffer;
     A->spmm.plan = plan;
     A->spmm.stagingBytes = 0;
+    A->spmm.vectorOff = 0;
+    A->spmm.vectorBytes = 0;
     return ACL_SPARSE_STATUS_SUCCESS;
+}
+
+int64_t Align256(int64_t v)
+{
+    return (v + 255) / 256 * 256;
 }
 
 bool ScalarIsZero(const void *host, aclDataType computeType)
@@ -254,6 +279,11 @@ aclsparseStatus_t aclsparseSpMMGetBufferSize(aclsparseHandle_t handle, aclsparse
                                                      handle != nullptr ? handle->stream : nullptr, size);
     if (rc == OPSPARSE_OK) {
         *size += static_cast<size_t>(MakeStaging(matA, matB, matC, opB, t, static_cast<int64_t>(*size)).bytes);
+        if (ColumnsAreVectors(matA, matB, matC, opB, t)) {
+            // behind everything else: the workspace of the SpMV plan the columns run under
+            *size = static_cast<size_t>(Align256(static_cast<int64_t>(*size))) +
+                    opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
+        }
     }
     return FromLaunch(rc);
 }
@@ -278,6 +308,21 @@ aclsparseStatus_t aclsparseSpMMPreprocess(aclsparseHandle_t handle, aclsparseOpe
     if (built == ACL_SPARSE_STATUS_SUCCESS) {
         // the buffer was sized by GetBufferSize for these operands: their staging area exists
         matA->spmm.stagingBytes = MakeStaging(matA, matB, matC, opB, t, matA->spmm.plan.bytes).bytes;
+        if (ColumnsAreVectors(matA, matB, matC, opB, t)) {
+            // (GetBufferSize counted this region for these operands)
+            const int64_t off = Align256(matA->spmm.plan.bytes + matA->spmm.stagingBytes);
+            const size_t bytes = opsparse_spmv_csr_workspace_bytes(matA->rows, matA->nnz);
+            OpsparseSpmvPlan vectorPlan{};
+            const int rc = opsparse_spmv_csr_analyse(static_cast<const int32_t *>(matA->rowOffsets), matA->rows,
+                                                     matA->cols, matA->nnz, static_cast<unsigned char *>(buffer) + off,
+                                                     bytes, OPSPARSE_SPMV_AUTO, &vectorPlan,
+                                                     handle != nullptr ? handle->stream : nullptr);
+            if (rc == OPSPARSE_OK) {
+                matA->spmm.vectorPlan = vectorPlan;
+                matA->spmm.vectorOff = off;
+                matA->spmm.vectorBytes = static_cast<int64_t>(bytes);
+            }
+        }
     }
     return built;
 }
@@ -330,7 +375,22 @@ aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t o
     const OpsparseScalar a = opsparse::MakeScalar(alpha, computeType, handle->pointerMode, 0.0);
     const OpsparseScalar b = opsparse::MakeScalar(beta, computeType, handle->pointerMode, 0.0);
     int rc;
-    if (staged) {
+    const OpsparseSpmmBinding &bind = matA->spmm;
+    if (bound && bind.vectorOff > 0 && bind.vectorPlan.rows == matA->rows && bind.vectorPlan.nnz == matA->nnz &&
+        ColumnsAreVectors(matA, matB, matC, opB, t)) {
+        const int64_t bStep = matB->order == ACL_SPARSE_ORDER_COL ? matB->ld : 0;
+        const int64_t cStep = matC->order == ACL_SPARSE_ORDER_COL ? matC->ld : 0;
+        rc = OPSPARSE_OK;
+        for (int64_t j = 0; j < matC->cols && rc == OPSPARSE_OK; ++j) {
+            const auto *x = static_cast<const unsigned char *>(matB->values) + j * bStep * ElementBytes(t.valType);
+            auto *y = static_cast<unsigned char *>(matC->values) + j * cStep * ElementBytes(t.cType);
+            rc = opsparse_spmv_csr_launch_zy(&bind.vectorPlan, 0, static_cast<const int32_t *>(matA->rowOffsets),
+                                             static_cast<const int32_t *>(matA->colInd), matA->values, x, y, y,
+                                             matA->rows, matA->cols, matA->nnz, a, b, t.valType, t.cType, 0,
+                                             static_cast<unsigned char *>(buffer) + bind.vectorOff,
+                                             static_cast<size_t>(bind.vectorBytes), handle->stream);
+        }
+    } else if (staged) {
         rc = RunStaged(g, matA, matB, matC, opB, a, b, t, handle->pointerMode == ACL_SPARSE_POINTER_MODE_HOST &&
                                                               beta != nullptr && ScalarIsZero(beta, computeType),
                        buffer, handle->stream);

@@ -525,6 +525,34 @@ def test_few_columns_on_a_mesh(osa, gpu_ctx, n, b_rm, c_rm, half):
         assert oracle.max_rel_err(got, gold) <= 1e-5
 
 
+@pytest.mark.parametrize("half", [False, True])
+def test_one_column_with_unit_leading_dimensions_runs_as_a_vector(osa, gpu_ctx, half):
+    """n = 1, row-major B and C with a leading dimension of 1: the column is a vector in memory and the product
+    runs under an SpMV plan made at Preprocess, like one or two columns of column-major operands
+    (test_few_columns_on_a_mesh).  Called twice with other scalars: the plan is reused."""
+    m, k = 5000, 4000
+    rng = np.random.default_rng(11)
+    rowptr, colind, val = csr_from_lengths(rng.integers(0, 12, m), k, seed=2)
+    B = rng.uniform(-1, 1, k).astype(np.float32)
+    vd, cd = (torch.float16, torch.float32) if half else (None, None)
+    if half:
+        val, B = (torch.from_numpy(a).to(torch.float16).float().numpy() for a in (val, B))
+    dev, stream, handle = gpu_ctx
+    C0 = rng.uniform(-1, 1, m).astype(np.float32)
+    d = [to_dev(rowptr, dev), to_dev(colind, dev), to_dev(val, dev, vd), to_dev(B, dev, vd), to_dev(C0, dev, cd)]
+    A = osa.Csr(m, k, d[0], d[1], d[2])
+    op = osa.SpmmOp(handle, A, osa.DnMat(k, 1, 1, d[3]), osa.DnMat(m, 1, 1, d[4]))
+    op(1.5, 0.5)
+    stream.synchronize()
+    first = oracle.spmm_f64(m, 1, rowptr, colind, val, B, 1, C0, 1, 1.5, 0.5)
+    assert oracle.max_rel_err(d[4].cpu().numpy(), first) <= 1e-5
+    d[4].fill_(float("nan"))
+    op(-2.0, 0.0)
+    stream.synchronize()
+    again = oracle.spmm_f64(m, 1, rowptr, colind, val, B, 1, C0, 1, -2.0, 0.0)
+    assert oracle.max_rel_err(d[4].cpu().numpy(), again) <= 1e-5
+
+
 def test_staging_needs_a_buffer_preprocessed_for_it(osa, gpu_ctx):
     """A buffer sized and preprocessed for row-major operands (256 bytes here) and then used with a column-major B:
     no staging area was promised, the product must run in place (slowly) and stay inside the buffer — the guard
