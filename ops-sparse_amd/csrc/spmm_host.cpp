@@ -152,14 +152,18 @@ int64_t PlanWidth(const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *B, co
 // One or two columns that lie in memory as vectors (column-major operands; a single column with a leading dimension
 // of 1): the product is then n SpMV calls, which read the matrix n times and still beat the SpMM kernels, whose
 // rows of B would be padded to 16 bytes in the staging area (5-point mesh of 4 M rows, n = 1: 37 us against 98 us;
-// n = 2: 75 against 103; from n = 3 on the padded product wins).  fp32, and fp16 with fp32 C: the fp16 C of SpMM
-// is clamped to the finite range before rounding, which the SpMV kernels do not do.
+// n = 2: 75 against 103; from n = 3 on the padded product wins, and for n = 2 already under rows of 27 entries:
+// 244 us against 206, so two columns go this way up to 16 entries a row on average).  fp32, and fp16 with fp32 C:
+// the fp16 C of SpMM is clamped to the finite range before rounding, which the SpMV kernels do not do.
 bool ColumnsAreVectors(const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *B, const aclsparseDnMatDescr *C,
                        aclsparseOperation_t opB, const SpmmTypes &t)
 {
     const int64_t n = C->cols;
     if (n < 1 || n > 2 || opB != ACL_SPARSE_OP_NON_TRANSPOSE || A->rows <= 0 || A->cols <= 0 || A->nnz <= 0 ||
         A->nnz > INT32_MAX || t.cType != OPSPARSE_F32 || (t.valType != OPSPARSE_F32 && t.valType != OPSPARSE_F16)) {
+        return false;
+    }
+    if (n == 2 && A->nnz > 16 * A->rows) {
         return false;
     }
     const bool bVectors = B->order == ACL_SPARSE_ORDER_COL ? B->ld >= A->cols : (n == 1 && B->ld == 1);

@@ -656,6 +656,42 @@ def test_atomics_layout_with_many_long_rows_in_one_block(osa, gpu_ctx, dtype, na
     _check_spmv(d_y.cpu().float().numpy(), rows, cols, rowptr, colind, val, x, y0, -1.5, 0.75, out_dtype)
 
 
+@pytest.mark.parametrize("elem", [1, 2, 4])
+def test_dense_restage_of_narrow_matrices_every_form(osa, gpu_ctx, elem):
+    """opsparse_dense_restage to at most 32 columns: DenseRestageNarrowKernel<T, VecSrc, VecDst>, a lane a row.  A
+    row-major side whose rows are whole aligned groups of four elements travels as vectors; the other forms are a
+    column-major side, a leading dimension that is not a multiple of four, and a base that is not aligned.  Padding
+    columns of the destination come out zero, what lies between its rows or columns stays."""
+    dev, stream, _ = gpu_ctx
+    L = osa.lib()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+    np_t, t_t = {1: (np.uint8, torch.uint8), 2: (np.int16, torch.int16), 4: (np.int32, torch.int32)}[elem]
+    rng = np.random.default_rng(elem)
+    rows = 1000
+    # (cols, colsDst, source: column-major / ld / offset in elements, destination: the same)
+    forms = [(5, 8, (False, 8, 0), (False, 8, 0)),       # vectors on both sides
+             (5, 8, (False, 8, 0), (True, rows + 3, 0)),  # vectors in, columns out
+             (3, 4, (True, rows + 1, 0), (False, 4, 0)),  # columns in, vectors out
+             (6, 7, (False, 9, 0), (False, 7, 0)),        # leading dimensions that are not multiples of four
+             (4, 4, (False, 4, 1), (False, 4, 1)),        # bases one element off
+             (1, 4, (True, rows, 0), (True, rows, 0)),    # columns on both sides
+             (12, 12, (False, 12, 0), (True, rows, 0))]
+    for cols, cols_dst, (s_cm, s_ld, s_off), (d_cm, d_ld, d_off) in forms:
+        src = rng.integers(1, 100, s_off + (cols * s_ld if s_cm else rows * s_ld)).astype(np_t)
+        dst0 = rng.integers(100, 120, d_off + (cols_dst * d_ld if d_cm else rows * d_ld)).astype(np_t)
+        d_src, d_dst = to_dev(src, dev, t_t), to_dev(dst0, dev, t_t)
+        rc = L.opsparse_dense_restage(d_src.data_ptr() + s_off * elem, d_dst.data_ptr() + d_off * elem, rows, cols,
+                                      cols_dst, s_ld, int(s_cm), d_ld, int(d_cm), elem, sp)
+        assert rc == 0
+        stream.synchronize()
+        r, c = np.meshgrid(np.arange(rows), np.arange(cols_dst), indexing="ij")
+        logical = np.zeros((rows, cols_dst), np_t)
+        logical[:, :cols] = src[s_off + (c[:, :cols] * s_ld + r[:, :cols] if s_cm else r[:, :cols] * s_ld + c[:, :cols])]
+        want = dst0.copy()
+        want[d_off + (c * d_ld + r if d_cm else r * d_ld + c)] = logical
+        assert np.array_equal(d_dst.cpu().numpy(), want), (cols, cols_dst, s_cm, d_cm)
+
+
 # ---------------------------------------------------------------------------------------------- yard-stick kernels
 
 def test_measurement_kernels_copy_read_gather(osa, gpu_ctx):
