@@ -374,7 +374,10 @@ int opsparse_spmm_csr_analyse(const int32_t *rowOffsets, int64_t rows, int64_t n
  * clampF16: when cType is F16, clamp to +-65504 before rounding [ref: :229-237].
  * With a plan and row-major operands the rows are worked in slabs of consecutive
  * rows staged through LDS (short rows share gather batches); plan == NULL runs
- * one lane group per row without a workspace.
+ * one lane group per row without a workspace.  A plan made for n <= 16 of a matrix
+ * whose longest row has at most 200 entries cuts the slabs for the kernel that
+ * gathers whole rows of a B of 16 or 32 bytes a row (fp32 n = 4, 8; fp16 n = 8, 16;
+ * ldb and ldc below 2^32): pass the n the plan was analysed for.
  */
 int opsparse_spmm_csr_launch(const OpsparseSpmmPlan *plan, const int32_t *rowOffsets, const int32_t *colInd,
                              const void *csrValues, const void *B, void *C, int64_t rows, int64_t k, int64_t n,
