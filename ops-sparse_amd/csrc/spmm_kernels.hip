@@ -894,22 +894,23 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmNarrowKernel(
     const int32_t tid = static_cast<int32_t>(threadIdx.x);
 
     // This XCD's tiles, and this workgroup's stride through them.
-    const int64_t xcd = blockIdx.x % kNumXcd;
-    const int64_t perXcd = numSlabs / kNumXcd, rem = numSlabs % kNumXcd;
-    const int64_t xcdFirst = xcd * perXcd + (xcd < rem ? xcd : rem);
-    const int64_t xcdTiles = perXcd + (xcd < rem ? 1 : 0);
-    const int64_t stride = (gridDim.x - xcd + kNumXcd - 1) / kNumXcd;  // workgroups living on this XCD
-    const int64_t t0 = blockIdx.x / kNumXcd;
+    const int32_t slabs = static_cast<int32_t>(numSlabs);  // (below 2^31: the launcher checks)
+    const int32_t xcd = static_cast<int32_t>(blockIdx.x % kNumXcd);
+    const int32_t perXcd = slabs / kNumXcd, rem = slabs % kNumXcd;
+    const int32_t xcdFirst = xcd * perXcd + (xcd < rem ? xcd : rem);
+    const int32_t xcdTiles = perXcd + (xcd < rem ? 1 : 0);
+    const int32_t stride = (static_cast<int32_t>(gridDim.x) - xcd + kNumXcd - 1) / kNumXcd;  // workgroups on this XCD
+    const int32_t t0 = static_cast<int32_t>(blockIdx.x / kNumXcd);
     if (t0 >= xcdTiles) {
         return;
     }
-    const int64_t mine = (xcdTiles - t0 + stride - 1) / stride;  // tiles of this workgroup
+    const int32_t mine = (xcdTiles - t0 + stride - 1) / stride;  // tiles of this workgroup
 
     struct Tile {
         int32_t r0, r1, first, count;
     };
-    auto loadRows = [&](int64_t i, Tile &m) {
-        const int64_t slab = xcdFirst + t0 + i * stride;
+    auto loadRows = [&](int32_t i, Tile &m) {
+        const int32_t slab = xcdFirst + t0 + i * stride;
         m.r0 = slabStart[slab];
         m.r1 = slabStart[slab + 1];
     };
@@ -918,9 +919,10 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmNarrowKernel(
         m.count = rowOffsets[m.r1] - m.first;
     };
     // A tile that does not fit - the row offsets changed since the table was made - is summed straight from memory.
+    const int32_t nnz32 = static_cast<int32_t>(nnz);
     auto fits = [&](const Tile &m) {
         return m.count >= 0 && m.count <= E && m.r1 - m.r0 <= kNarrowRows && m.first >= 0 &&
-               static_cast<int64_t>(m.first) + m.count <= nnz;
+               m.first <= nnz32 - m.count;
     };
 
     Int4U colN[U];
@@ -937,8 +939,8 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmNarrowKernel(
             if ((u * kBlockThreads + (tid & ~(kWave - 1))) * 4 >= m.count) {
                 continue;
             }
-            int64_t at = static_cast<int64_t>(m.first) + (u * kBlockThreads + tid) * 4;
-            at = at + 4 <= nnz ? at : nnz - 4;
+            int32_t at = m.first + (u * kBlockThreads + tid) * 4;  // (first + count <= nnz <= INT32_MAX - 4 E)
+            at = at + 4 <= nnz32 ? at : nnz32 - 4;
             colN[u] = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(colInd + at));
             if constexpr (sizeof(ValT) == 4) {
                 const Int4U v = __builtin_nontemporal_load(reinterpret_cast<const Int4U *>(vals + at));
@@ -952,16 +954,17 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmNarrowKernel(
     // Requests the rows of B of the entries issueQuads asked for (waiting for those), and the tile's row offsets.
     // An entry past the tile's end takes the row of B of the tile's first entry.
     auto issueGather = [&](const Tile &m) {
+        if (m.first + E > nnz32) {  // the tile that may reach the end of the arrays
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int64_t at = static_cast<int64_t>(m.first) + (u * kBlockThreads + tid) * 4;
-            int64_t late = at + 4 - nnz;  // entries by which the quad was read early
-            late = late > 3 ? 3 : late;
-            for (; late > 0; --late) {    // (the last lanes of the last tile)
-                colN[u] = Int4U{colN[u][1], colN[u][2], colN[u][3], colN[u][3]};
-                valN[u][0] = valN[u][1];
-                valN[u][1] = valN[u][2];
-                valN[u][2] = valN[u][3];
+            for (int u = 0; u < U; ++u) {
+                int32_t late = m.first + (u * kBlockThreads + tid) * 4 + 4 - nnz32;  // entries the quad was read early
+                late = late > 3 ? 3 : late;
+                for (; late > 0; --late) {                                           // (the last lanes of that tile)
+                    colN[u] = Int4U{colN[u][1], colN[u][2], colN[u][3], colN[u][3]};
+                    valN[u][0] = valN[u][1];
+                    valN[u][1] = valN[u][2];
+                    valN[u][2] = valN[u][3];
+                }
             }
         }
         const int32_t colSafe = __shfl(colN[0][0], 0, kWave);
@@ -1016,7 +1019,7 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmNarrowKernel(
 
     constexpr int kGroups = kBlockThreads / G;
     const int32_t lane = tid % G;
-    for (int64_t i = 0; i < mine; ++i) {
+    for (int32_t i = 0; i < mine; ++i) {
         Tile m4{};
         if (i + 4 < mine) {
             loadRows(i + 4, m4);
@@ -1564,7 +1567,8 @@ bool UseNarrowKernel(const SpmmArgs &a)
     const bool off = std::getenv("OPS_SPARSE_SPMM_NO_NARROW") != nullptr;  // (read at every call: tests switch it)
     const int64_t rowBytes = a.n * static_cast<int64_t>(sizeof(ValT));
     if (off || sizeof(ValT) < 2 || (rowBytes != 16 && rowBytes != 32) || a.plan == nullptr || a.ws == nullptr ||
-        a.ldb > UINT32_MAX || a.ldc > UINT32_MAX || a.nnz < 4 || a.plan->n != a.n) {
+        a.ldb > UINT32_MAX || a.ldc > UINT32_MAX || a.nnz < 4 || a.nnz > INT32_MAX - 4 * NarrowEntries(a.n) ||
+        a.plan->numSlabs > INT32_MAX / 2 || a.plan->n != a.n) {
         return false;
     }
     const OpsparseSpmmPlan &p = *a.plan;
