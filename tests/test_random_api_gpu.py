@@ -117,6 +117,33 @@ def test_random_case(osa, gpu_ctx, seed):
             assert oracle.max_rel_err(got, gold) <= 1e-5
 
 
+@pytest.mark.parametrize("seed", range(60))
+def test_random_few_columns_case(osa, gpu_ctx, seed):
+    """SpMM with 1 - 16 columns of B on the same random matrices (those without a row beyond 200 entries take the
+    kernel for narrow B, one or two column-major columns the SpMV kernels; the others the lane-group kernels): any
+    storage order, padded leading dimensions, fp32 or fp16 values with fp32 C."""
+    rng = np.random.default_rng(77_000 + seed)
+    rows, cols, rowptr, colind, val = _matrix(rng)
+    alpha, beta = float(rng.choice([1.0, -0.5, 2.25])), float(rng.choice([0.0, 1.0, -1.5]))
+    n = int(rng.integers(1, 17))
+    half = bool(rng.integers(0, 3) == 0)
+    b_rm, c_rm = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    pad = int(rng.choice([0, 0, 1, 4]))
+    ldb = (n if b_rm else cols) + pad
+    ldc = (n if c_rm else rows) + pad
+    B = rng.uniform(-1, 1, (cols if b_rm else n) * ldb).astype(np.float32)
+    C0 = rng.uniform(-1, 1, (rows if c_rm else n) * ldc).astype(np.float32)
+    if half:
+        val, B = _half(val), _half(B)
+    got = run_spmm(osa, gpu_ctx, rows, cols, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta,
+                   order_b=osa.ACL_SPARSE_ORDER_ROW if b_rm else osa.ACL_SPARSE_ORDER_COL,
+                   order_c=osa.ACL_SPARSE_ORDER_ROW if c_rm else osa.ACL_SPARSE_ORDER_COL,
+                   val_dtype=torch.float16 if half else None, c_dtype=torch.float32 if half else None)
+    gold = oracle.spmm_f64(rows, n, rowptr, colind, val, B, ldb, C0, ldc, alpha, beta, b_row_major=b_rm,
+                           trans_b=False, c_row_major=c_rm)
+    assert oracle.max_rel_err(got, gold) <= 1e-5
+
+
 @pytest.mark.parametrize("seed", range(30))
 def test_random_conversion_case(osa, gpu_ctx, seed):
     """The CSR producers on the same random matrices (columns unsorted, with repeats): csrsort, the same arrays read
