@@ -386,6 +386,16 @@ int opsparse_spmm_csr_launch(const OpsparseSpmmPlan *plan, const int32_t *rowOff
                              int32_t cType, void *workspace, size_t workspaceBytes, void *stream);
 
 /*
+ * 1 when opsparse_spmm_csr_launch with this analysed plan and workspace takes row-major fp32 B and C of n <= 8
+ * columns at any leading dimension and 4-byte alignment where they are, with the kernel for a B of few columns; 0
+ * when operands that are not whole aligned 16-byte rows would run a lane a column in place and are better copied
+ * to padded rows first (opsparse_dense_restage).  The plan may have been analysed for n rounded up to a multiple of
+ * 4.  aclsparseSpMM asks before it uses its staging area.
+ */
+int opsparse_spmm_csr_narrow_rows(const OpsparseSpmmPlan *plan, const void *workspace, int64_t n, int64_t nnz,
+                                  int32_t valType, int32_t cType);
+
+/*
  * Dense rows x cols matrix copied from one storage order / leading dimension to another (elements of 1, 2 or
  * 4 bytes); columns cols .. colsDst-1 of the destination are written as zero.  aclsparseSpMM uses it to hand
  * column-major or transposed B / C to the row-major kernels through a staging area of the SpMM buffer: the

@@ -105,6 +105,7 @@ OPSPARSE_SYMBOLS = [
     "opsparse_spmv_csr_gathers_scattered",
     "opsparse_spmm_csr_workspace_bytes", "opsparse_spmm_csr_analyse", "opsparse_spmm_csr_launch",
     "opsparse_dense_restage",
+    "opsparse_spmm_csr_narrow_rows",
     "opsparse_scan_workspace_bytes", "opsparse_coo2csr_launch", "opsparse_csr2coo_launch",
     "opsparse_csrsort_workspace_bytes", "opsparse_csrsort_launch", "opsparse_coosort_workspace_bytes",
     "opsparse_coosort_launch", "opsparse_csr2csc_workspace_bytes",
@@ -307,6 +308,8 @@ def lib():
     L.opsparse_spmm_csr_launch.argtypes = [ctypes.POINTER(OpsparseSpmmPlan), vp, vp, vp, vp, vp, i64, i64, i64, i64,
                                            i64, i64, i32, i32, i32, OpsparseScalar, OpsparseScalar, i32, i32, vp, sz,
                                            vp]
+    L.opsparse_spmm_csr_narrow_rows.restype = ctypes.c_int
+    L.opsparse_spmm_csr_narrow_rows.argtypes = [ctypes.POINTER(OpsparseSpmmPlan), vp, i64, i64, i32, i32]
     L.opsparse_dense_restage.restype = ctypes.c_int
     L.opsparse_dense_restage.argtypes = [vp, vp, i64, i64, i64, i64, i32, i64, i32, i32, vp]
     L.opsparse_copy_launch.restype = ctypes.c_int

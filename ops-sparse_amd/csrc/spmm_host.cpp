@@ -356,7 +356,16 @@ aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t o
     bool staged = bound && g.bytes > 0 && g.bytes <= matA->spmm.stagingBytes && matA->spmm.plan.n == g.nPadded &&
                   matA->nnz > 0;
     const OpsparseSpmmPlan *plan = &matA->spmm.plan;
-    if (!staged && (!bound || matA->spmm.plan.n != matC->cols)) {
+    // A few row-major fp32 columns under a plan cut for the kernel for narrow B: that kernel reads and writes rows of
+    // any width up to 8, leading dimension and 4-byte alignment where they are, and the copies through the staging
+    // area are saved.
+    const bool direct = staged && opB == ACL_SPARSE_OP_NON_TRANSPOSE && matB->order == ACL_SPARSE_ORDER_ROW &&
+                        matC->order == ACL_SPARSE_ORDER_ROW &&
+                        opsparse_spmm_csr_narrow_rows(plan, buffer, matC->cols, matA->nnz, t.valType, t.cType) != 0;
+    if (direct) {
+        staged = false;
+    }
+    if (!direct && !staged && (!bound || matA->spmm.plan.n != matC->cols)) {
         // The analysis reads two numbers back and synchronises, which a stream under capture must not: such a call
         // runs without a plan (a lane group per row, no tables), like the raw launch layer with plan == NULL.
         hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;

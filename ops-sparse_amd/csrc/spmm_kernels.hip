@@ -869,12 +869,18 @@ constexpr int NarrowEntries(int64_t)
     return 1024;
 }
 
-template <typename ValT, typename CT, typename AccT, int W, int G>
+// Ragged: rows of B and C of nCols <= W fp32 elements at any leading dimension and 4-byte alignment (3 interleaved
+// components a point, say) are read and written where they are, the last piece of a row as 1 - 4 dwords, and sit
+// padded with zeros in LDS.  (Through the staging area such operands cost two copies on top: 4 M rows, n = 3,
+// 109 us against 71 for n = 4.)
+template <typename ValT, typename CT, typename AccT, int W, int G, bool Ragged = false>
 __global__ __launch_bounds__(kBlockThreads) void SpmmNarrowKernel(
     const int32_t *__restrict__ rowOffsets, const int32_t *__restrict__ colInd, const ValT *__restrict__ vals,
     const ValT *__restrict__ B, CT *C, uint32_t ldb, uint32_t ldc, const int32_t *__restrict__ slabStart,
-    int64_t numSlabs, int64_t nnz, OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16)
+    int64_t numSlabs, int64_t nnz, OpsparseScalar alphaS, OpsparseScalar betaS, int32_t clampF16, int32_t nCols)
 {
+    static_assert(!Ragged || (sizeof(ValT) == 4 && sizeof(CT) == 4), "ragged rows of 4-byte elements");
+    typedef int32_t Int2U __attribute__((ext_vector_type(2), aligned(4)));
     typedef int32_t Int4A __attribute__((ext_vector_type(4)));
     constexpr int Q = W * static_cast<int>(sizeof(ValT)) / 16;  // 16-byte pieces of a row of B
     constexpr int kPiece = 16 / static_cast<int>(sizeof(ValT));  // elements of a piece
@@ -980,7 +986,26 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmNarrowKernel(
                 const ValT *bRow = B + static_cast<uint64_t>(col) * ldb;
 #pragma unroll
                 for (int q = 0; q < Q; ++q) {
-                    piece[u][i][q] = *reinterpret_cast<const Int4A *>(bRow + q * kPiece);
+                    if constexpr (Ragged) {
+                        const int32_t have = nCols - q * kPiece;  // elements of this piece that exist (uniform)
+                        const int32_t *from = reinterpret_cast<const int32_t *>(bRow + q * kPiece);
+                        Int4A p = {0, 0, 0, 0};
+                        if (have >= 4) {
+                            const Int4U v = *reinterpret_cast<const Int4U *>(from);
+                            p = Int4A{v[0], v[1], v[2], v[3]};
+                        } else if (have == 3) {  // (two loads: a three-element vector type is loaded as four)
+                            const Int2U v = *reinterpret_cast<const Int2U *>(from);
+                            p = Int4A{v[0], v[1], from[2], 0};
+                        } else if (have == 2) {
+                            const Int2U v = *reinterpret_cast<const Int2U *>(from);
+                            p = Int4A{v[0], v[1], 0, 0};
+                        } else if (have == 1) {
+                            p = Int4A{from[0], 0, 0, 0};
+                        }
+                        piece[u][i][q] = p;
+                    } else {
+                        piece[u][i][q] = *reinterpret_cast<const Int4A *>(bRow + q * kPiece);
+                    }
                 }
                 valP[u][i] = static_cast<float>(valN[u][i]);
             }
@@ -1091,7 +1116,9 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmNarrowKernel(
                     const ValT *bRow = B + static_cast<uint64_t>(static_cast<uint32_t>(colInd[k])) * ldb + q * kPiece;
 #pragma unroll
                     for (int c = 0; c < kPiece; ++c) {
-                        acc[c] += v * ToAcc<AccT>(bRow[c]);
+                        if (!Ragged || q * kPiece + c < nCols) {
+                            acc[c] += v * ToAcc<AccT>(bRow[c]);
+                        }
                     }
                 }
             }
@@ -1101,14 +1128,33 @@ __global__ __launch_bounds__(kBlockThreads) void SpmmNarrowKernel(
             }
             if (lane == 0) {
                 CT *out = C + static_cast<uint64_t>(static_cast<uint32_t>(m0.r0 + rr)) * ldc + q * kPiece;
-                CT res[kPiece];
+                CT res[kPiece] = {};
+                const int32_t have = Ragged ? nCols - q * kPiece : kPiece;  // (uniform but for q)
 #pragma unroll
                 for (int c = 0; c < kPiece; ++c) {
-                    res[c] = Epilogue<CT, AccT>::Apply(acc[c], alpha, beta, betaZero, out + c, clampF16 != 0);
+                    if (c < have) {
+                        res[c] = Epilogue<CT, AccT>::Apply(acc[c], alpha, beta, betaZero, out + c, clampF16 != 0);
+                    }
                 }
+                if constexpr (Ragged) {
+                    int32_t bits[kPiece];
+                    __builtin_memcpy(bits, res, sizeof(bits));
+                    int32_t *to = reinterpret_cast<int32_t *>(out);
+                    if (have >= 4) {
+                        *reinterpret_cast<Int4U *>(to) = Int4U{bits[0], bits[1], bits[2], bits[3]};
+                    } else if (have == 3) {
+                        *reinterpret_cast<Int2U *>(to) = Int2U{bits[0], bits[1]};
+                        to[2] = bits[2];
+                    } else if (have == 2) {
+                        *reinterpret_cast<Int2U *>(to) = Int2U{bits[0], bits[1]};
+                    } else if (have == 1) {
+                        to[0] = bits[0];
+                    }
+                } else {
 #pragma unroll
-                for (int c = 0; c < kPiece; ++c) {
-                    out[c] = res[c];
+                    for (int c = 0; c < kPiece; ++c) {
+                        out[c] = res[c];
+                    }
                 }
             }
         }
@@ -1505,8 +1551,9 @@ int LaunchSlab(const SpmmArgs &a)
     return CheckLaunch();
 }
 
-// SpmmNarrowKernel for a plan whose slab table was cut for it; W = a.n columns.
-template <typename ValT, typename CT, typename AccT, int W>
+// SpmmNarrowKernel for a plan whose slab table was cut for it; W columns: a.n of them, or (Ragged) the a.n columns
+// rounded up to whole pieces.
+template <typename ValT, typename CT, typename AccT, int W, bool Ragged = false>
 int LaunchNarrow(const SpmmArgs &a)
 {
     const auto *slabStart =
@@ -1518,7 +1565,7 @@ int LaunchNarrow(const SpmmArgs &a)
         constexpr int G = decltype(tag)::value;
         static const int fit = [] {
             int blocks = 1;
-            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, SpmmNarrowKernel<ValT, CT, AccT, W, G>,
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, SpmmNarrowKernel<ValT, CT, AccT, W, G, Ragged>,
                                                              kBlockThreads, 0) != hipSuccess ||
                 blocks < 1) {
                 (void)hipGetLastError();
@@ -1529,10 +1576,11 @@ int LaunchNarrow(const SpmmArgs &a)
         // persistent: the workgroups that fit the device at once walk over all tiles
         const int64_t resident = static_cast<int64_t>(ComputeUnits()) * fit;
         const uint32_t grid = static_cast<uint32_t>(a.plan->numSlabs < resident ? a.plan->numSlabs : resident);
-        hipLaunchKernelGGL((SpmmNarrowKernel<ValT, CT, AccT, W, G>), dim3(grid), dim3(kBlockThreads), 0, a.stream,
-                           a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals), static_cast<const ValT *>(a.B),
-                           static_cast<CT *>(a.C), static_cast<uint32_t>(a.ldb), static_cast<uint32_t>(a.ldc),
-                           slabStart, a.plan->numSlabs, a.nnz, a.alpha, a.beta, a.clampF16);
+        hipLaunchKernelGGL((SpmmNarrowKernel<ValT, CT, AccT, W, G, Ragged>), dim3(grid), dim3(kBlockThreads), 0,
+                           a.stream, a.rowOffsets, a.colInd, static_cast<const ValT *>(a.vals),
+                           static_cast<const ValT *>(a.B), static_cast<CT *>(a.C), static_cast<uint32_t>(a.ldb),
+                           static_cast<uint32_t>(a.ldc), slabStart, a.plan->numSlabs, a.nnz, a.alpha, a.beta,
+                           a.clampF16, static_cast<int32_t>(a.n));
         return CheckLaunch();
     };
     // fp32: 1 .. 32 lanes, fp16: 2 .. 64; with 16 columns (four fp32 pieces in the tiling's count) the tiling stops
@@ -1559,25 +1607,44 @@ int LaunchNarrow(const SpmmArgs &a)
     }
 }
 
-// Whether the product takes SpmmNarrowKernel: whole 16-byte rows of B of one or two pieces, an analysed matrix of
-// short rows whose slab table was cut for that kernel.
-template <typename ValT>
-bool UseNarrowKernel(const SpmmArgs &a)
+// Whether a plan's slab table was cut for SpmmNarrowKernel and for as many columns as n rounded up to a multiple of
+// four: an analysed matrix of short rows.
+bool PlanTakesNarrow(const OpsparseSpmmPlan *plan, const void *workspace, int64_t n, int64_t nnz)
 {
     const bool off = std::getenv("OPS_SPARSE_SPMM_NO_NARROW") != nullptr;  // (read at every call: tests switch it)
-    const int64_t rowBytes = a.n * static_cast<int64_t>(sizeof(ValT));
-    if (off || sizeof(ValT) < 2 || (rowBytes != 16 && rowBytes != 32) || a.plan == nullptr || a.ws == nullptr ||
-        a.ldb > UINT32_MAX || a.ldc > UINT32_MAX || a.nnz < 4 || a.nnz > INT32_MAX - 4 * NarrowEntries(a.n) ||
-        a.plan->numSlabs > INT32_MAX / 2 || a.plan->n != a.n) {
+    if (off || plan == nullptr || workspace == nullptr || n < 1 || n > 16 || nnz < 4 ||
+        nnz > INT32_MAX - 4 * NarrowEntries(n) || plan->numSlabs > INT32_MAX / 2 ||
+        (plan->n + 3) / 4 != (n + 3) / 4) {
         return false;
     }
-    const OpsparseSpmmPlan &p = *a.plan;
+    const OpsparseSpmmPlan &p = *plan;
     if (p.kernel == OPSPARSE_SPMM_BINNED || p.numLongRows != 0 || p.slabStartOff <= 0 || p.numSlabs <= 0 ||
         std::getenv("OPS_SPARSE_SPMM_NO_SLAB_TABLE") != nullptr) {
         return false;
     }
     const NarrowTiling tiling = MakeNarrowTiling(p.rows, p.nnz, p.maxRowNnz, p.n);
     return tiling.ok && SlabShare(p.rows, p.nnz, p.maxRowNnz, p.n) == tiling.share;
+}
+
+// Whether the product takes SpmmNarrowKernel on whole 16-byte rows of B of one or two pieces.
+template <typename ValT>
+bool UseNarrowKernel(const SpmmArgs &a)
+{
+    const int64_t rowBytes = a.n * static_cast<int64_t>(sizeof(ValT));
+    if (sizeof(ValT) < 2 || (rowBytes != 16 && rowBytes != 32) || a.ldb > UINT32_MAX || a.ldc > UINT32_MAX ||
+        a.plan == nullptr || a.plan->n != a.n) {
+        return false;
+    }
+    return PlanTakesNarrow(a.plan, a.ws, a.n, a.nnz);
+}
+
+// ... and on row-major fp32 B and C of at most 8 columns that are not that: another width, leading dimension or
+// alignment.  The plan is one for the width rounded up to a multiple of four.
+bool UseNarrowRagged(const SpmmArgs &a)
+{
+    return !a.bColMajor && !a.cColMajor && !a.transB && a.n >= 1 && a.n <= 8 && a.ldb >= a.n && a.ldc >= a.n &&
+           a.ldb <= UINT32_MAX && a.ldc <= UINT32_MAX && reinterpret_cast<uintptr_t>(a.B) % 4 == 0 &&
+           reinterpret_cast<uintptr_t>(a.C) % 4 == 0 && PlanTakesNarrow(a.plan, a.ws, a.n, a.nnz);
 }
 
 template <typename ValT, typename CT, typename AccT, int L>
@@ -1610,6 +1677,11 @@ int RunTypedV(const SpmmArgs &a)
     const bool fast = !a.bColMajor && !a.cColMajor && !a.transB && a.n % V == 0 && a.ldb % V == 0 &&
                       a.ldc % V == 0 && reinterpret_cast<uintptr_t>(a.B) % 16 == 0 &&
                       reinterpret_cast<uintptr_t>(a.C) % 16 == 0;
+    if constexpr (std::is_same<ValT, float>::value && std::is_same<CT, float>::value) {
+        if (!fast && UseNarrowRagged(a)) {
+            return a.n <= 4 ? LaunchNarrow<ValT, CT, AccT, 4, true>(a) : LaunchNarrow<ValT, CT, AccT, 8, true>(a);
+        }
+    }
     if (!fast) {
         return RunGeneral<ValT, CT, AccT>(a);
     }
@@ -1816,6 +1888,13 @@ int opsparse_spmm_csr_launch(const OpsparseSpmmPlan *plan, const int32_t *rowOff
 
     }
     return OPSPARSE_E_UNSUPPORTED;
+}
+
+int opsparse_spmm_csr_narrow_rows(const OpsparseSpmmPlan *plan, const void *workspace, int64_t n, int64_t nnz,
+                                  int32_t valType, int32_t cType)
+{
+    return valType == OPSPARSE_F32 && cType == OPSPARSE_F32 && n <= 8 && PlanTakesNarrow(plan, workspace, n, nnz) ? 1
+                                                                                                                   : 0;
 }
 
 int opsparse_dense_restage(const void *src, void *dst, int64_t rows, int64_t cols, int64_t colsDst, int64_t ldSrc,
