@@ -8,6 +8,7 @@
 #include <climits>
 
 #include <cstdint>
+#include <cstdlib>
 
 #include "internal.h"
 
@@ -171,8 +172,52 @@ bool ColumnsAreVectors(const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *
     return bVectors && cVectors;
 }
 
+// Whether a matrix without long rows, under a B of n elements of elemBytes, is better served by the kernel that
+// gives every row whole to one lane group straight from memory than by the slabs staged through LDS.  Measured on
+// fp32 (us, slabs / rows; 1 - 2 M rows of meshes, bands, and uniformly random columns):
+//   n = 16: 5-point mesh 225 / 119, 27-point 440 / 283, band of 50 246 / 143, 32 random columns a row 494 / 419
+//   n = 32: 5-point 256 / 200, 27-point 555 / 308, band of 200 191 / 162, 8 random 191 / 183, 32 random 313 / 373
+//   n = 64: 5-point 394 / 515, 7-point 525 / 560, 27-point 778 / 582, band of 50 342 / 248, 32 random 591 / 618
+//   n = 128: 5-point 692 / 1027, 27-point 1139 / 1040, band of 200 459 / 384, 32 random 1194 / 1201
+// The slabs win where the gathers of B are what the product waits for (random columns, wide rows of B) and on
+// short rows under a wide B; rows of even length whose columns stay near the diagonal, and any narrow B, run
+// faster row by row.  Uneven rows stay with the slabs, which share them out by work.
+bool PrefersWholeRows(const aclsparseSpMatDescr *A, const OpsparseSpmmPlan &plan, int64_t n, int64_t elemBytes,
+                      void *buffer, hipStream_t stream)
+{
+    if (std::getenv("OPS_SPARSE_SPMM_NO_ROWS_RULE") != nullptr || stream == nullptr || elemBytes < 2 ||
+        plan.kernel == OPSPARSE_SPMM_BINNED || plan.numLongRows != 0 || plan.maxRowNnz <= 0 || A->rows <= 0 ||
+        A->colInd == nullptr) {
+        return false;
+    }
+    const int64_t rowBytes = n * elemBytes;
+    const double mean = static_cast<double>(A->nnz) / static_cast<double>(A->rows);
+    if ((rowBytes == 16 || rowBytes == 32) && plan.maxRowNnz <= 200) {
+        return false;  // the kernel for a B of one or two 16-byte pieces a row takes these
+    }
+    if (rowBytes > 512 || static_cast<double>(plan.maxRowNnz) > 4.0 * mean + 8.0) {
+        return false;
+    }
+    if (rowBytes <= 64 || (rowBytes <= 128 && mean < 24.0)) {
+        return true;
+    }
+    if (rowBytes > 128 && mean < 16.0) {
+        return false;
+    }
+    // what is left depends on whether the rows of B a row needs lie near each other: the sample of the SpMV plans
+    // (the first 256 bytes of the buffer are the analyses' scratch: no launch reads them)
+    int32_t scattered = 1000;
+    if (opsparse_spmv_csr_gathers_scattered(static_cast<const int32_t *>(A->rowOffsets),
+                                            static_cast<const int32_t *>(A->colInd), A->rows, A->cols, A->nnz, buffer,
+                                            256, &scattered, stream) != OPSPARSE_OK) {
+        return false;
+    }
+    return scattered < 250;
+}
+
 // Row statistics and long-row tables for width n into `buffer`; binds the buffer to A.
-aclsparseStatus_t BuildPlan(const aclsparseSpMatDescr *A, int64_t n, void *buffer, hipStream_t stream)
+aclsparseStatus_t BuildPlan(const aclsparseSpMatDescr *A, int64_t n, int64_t elemBytes, void *buffer,
+                            hipStream_t stream)
 {
     // An empty matrix has nothing to preprocess (spmm_csr_mat.cpp:148-150).
     if (A->rows <= 0) {
@@ -190,6 +235,14 @@ aclsparseStatus_t BuildPlan(const aclsparseSpMatDescr *A, int64_t n, void *buffe
     if (rc != OPSPARSE_OK) {
         opsparse::LogError("aclsparseSpMM: analysis failed (%d)", rc);
         return FromLaunch(rc);
+    }
+    if (PrefersWholeRows(A, plan, n, elemBytes, buffer, stream)) {
+        // a plan without tables: the launch layer then takes a lane group a row
+        const int again = opsparse_spmm_csr_analyse(static_cast<const int32_t *>(A->rowOffsets), A->rows, A->nnz, n,
+                                                    buffer, bytes, OPSPARSE_SPMM_ROW_SPLIT, &plan, stream);
+        if (again != OPSPARSE_OK) {
+            return FromLaunch(again);
+        }
     }
     A->spmm.widestN = (A->spmm.buffer == buffer && A->spmm.widestN > n) ? A->spmm.widestN : n;
     A->spmm.buffer = buffer;
@@ -307,8 +360,8 @@ aclsparseStatus_t aclsparseSpMMPreprocess(aclsparseHandle_t handle, aclsparseOpe
         return ACL_SPARSE_STATUS_INSUFFICIENT_RESOURCES;
     }
     // The reference ignores the handle here; its stream is used when there is one.
-    const aclsparseStatus_t built = BuildPlan(matA, PlanWidth(matA, matB, matC, opB, t), buffer,
-                                              handle != nullptr ? handle->stream : nullptr);
+    const aclsparseStatus_t built = BuildPlan(matA, PlanWidth(matA, matB, matC, opB, t), ElementBytes(t.valType),
+                                              buffer, handle != nullptr ? handle->stream : nullptr);
     if (built == ACL_SPARSE_STATUS_SUCCESS) {
         // the buffer was sized by GetBufferSize for these operands: their staging area exists
         matA->spmm.stagingBytes = MakeStaging(matA, matB, matC, opB, t, matA->spmm.plan.bytes).bytes;
@@ -378,7 +431,7 @@ aclsparseStatus_t aclsparseSpMM(aclsparseHandle_t handle, aclsparseOperation_t o
             // and column) need not fit it, and nothing says how large it is.  Without tables, then.
             plan = nullptr;
         } else {
-            st = BuildPlan(matA, matC->cols, buffer, handle->stream);
+            st = BuildPlan(matA, matC->cols, ElementBytes(t.valType), buffer, handle->stream);
             if (st != ACL_SPARSE_STATUS_SUCCESS) {
                 return st;
             }

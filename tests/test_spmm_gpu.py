@@ -482,16 +482,9 @@ def test_layouts_through_the_staging_area(osa, gpu_ctx, b_rm, c_rm, trans_b, n, 
         assert oracle.max_rel_err(got, gold) <= tol
 
 
-@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8])
-@pytest.mark.parametrize("b_rm,c_rm", [(True, True), (False, False), (True, False)])
-@pytest.mark.parametrize("half", [False, True])
-def test_few_columns_on_a_mesh(osa, gpu_ctx, n, b_rm, c_rm, half):
-    """One to eight columns of B under a 7-point mesh matrix (block Krylov methods, a few right-hand sides): the
-    widths are padded to whole 16-byte rows in the staging area where they are not, and the product of one or two
-    such pieces a row takes the kernel for narrow B.  Every layout, fp32 and fp16 values, beta zero (C holds NaN
-    and must not be read) and not."""
-    side = 24
-    m = k = side ** 3
+def _mesh7(side):
+    """The 7-point stencil on side^3 points, no wrap-around: rows, columns, row offsets, ascending column indices."""
+    m = side ** 3
     r = np.arange(m)
     z, y, x = r // (side * side), (r // side) % side, r % side
     cols, keep = [], []
@@ -501,7 +494,49 @@ def test_few_columns_on_a_mesh(osa, gpu_ctx, n, b_rm, c_rm, half):
         keep.append(ok)
     cols, keep = np.stack(cols, 1), np.stack(keep, 1)
     rowptr = np.concatenate([[0], np.cumsum(keep.sum(1))]).astype(np.int32)
-    colind = cols[keep].astype(np.int32)
+    return m, m, rowptr, cols[keep].astype(np.int32)
+
+
+@pytest.mark.parametrize("shape", ["mesh", "band", "random"])
+@pytest.mark.parametrize("n", [12, 16, 32, 64, 128])
+def test_kernel_choice_by_shape_and_width(osa, gpu_ctx, shape, n, monkeypatch):
+    """Preprocess picks, for a matrix without long rows, between the slabs staged through LDS and a lane group a row
+    straight from memory: by the width of B, the mean row length and - where those leave it open - by a sample of
+    how far the columns lie from the diagonal (a mesh of 7 entries a row, a band of 40, 40 random columns a row:
+    the rule's three kinds).  Either choice must give the product; so must the rule switched off."""
+    rng = np.random.default_rng(n)
+    if shape == "mesh":
+        m, k, rowptr, colind = _mesh7(20)
+    else:
+        m = 6000
+        k = 6000 if shape == "band" else 300_000      # (the sample counts columns further than 2^17 from the diagonal)
+        per = 40
+        rowptr = (np.arange(m + 1) * per).astype(np.int32)
+        if shape == "band":
+            base = np.clip(np.arange(m)[:, None] - per // 2 + np.arange(per)[None, :], 0, k - 1)
+            colind = base.ravel().astype(np.int32)
+        else:
+            colind = rng.integers(0, k, m * per).astype(np.int32)
+    val = rng.uniform(-1, 1, colind.size).astype(np.float32)
+    B = rng.uniform(-1, 1, k * n).astype(np.float32)
+    C0 = rng.uniform(-1, 1, m * n).astype(np.float32)
+    gold = oracle.spmm_f64(m, n, rowptr, colind, val, B, n, C0, n, 1.5, -0.5)
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, n, C0, n, 1.5, -0.5)
+    assert oracle.max_rel_err(got, gold) <= 1e-5
+    monkeypatch.setenv("OPS_SPARSE_SPMM_NO_ROWS_RULE", "1")
+    got = run_spmm(osa, gpu_ctx, m, k, n, rowptr, colind, val, B, n, C0, n, 1.5, -0.5)
+    assert oracle.max_rel_err(got, gold) <= 1e-5
+
+
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 8])
+@pytest.mark.parametrize("b_rm,c_rm", [(True, True), (False, False), (True, False)])
+@pytest.mark.parametrize("half", [False, True])
+def test_few_columns_on_a_mesh(osa, gpu_ctx, n, b_rm, c_rm, half):
+    """One to eight columns of B under a 7-point mesh matrix (block Krylov methods, a few right-hand sides): the
+    widths are padded to whole 16-byte rows in the staging area where they are not, and the product of one or two
+    such pieces a row takes the kernel for narrow B.  Every layout, fp32 and fp16 values, beta zero (C holds NaN
+    and must not be read) and not."""
+    m, k, rowptr, colind = _mesh7(24)
     rng = np.random.default_rng(n + 10 * b_rm + 20 * c_rm)
     val = rng.uniform(-1, 1, colind.size).astype(np.float32)
     ldb = (n + 3) if b_rm else (k + 2)
