@@ -742,6 +742,71 @@ def run_stencils(args, osa, wl, torch, dev, stream, handle):
     return res
 
 
+def run_spmm_shapes(args, osa, wl, torch, dev, stream, handle):
+    """SpMM fp32 with 16 - 128 columns of B on meshes, bands and uniformly random columns: the two kernels a matrix
+    without long rows can take - slabs staged through LDS (`OPS_SPARSE_SPMM_NO_ROWS_RULE=1` at Preprocess), a lane
+    group a row straight from memory (`OPS_SPARSE_SPMM_NO_SLAB=1` at the call) - and what Preprocess picks by
+    itself.  The grid behind that rule."""
+    import itertools
+
+    def band(rows, width, seed):
+        idx = torch.arange(rows * width, dtype=torch.int64, device=dev).view(rows, width)
+        r = torch.arange(rows, dtype=torch.int64, device=dev).view(rows, 1)
+        step = (wl._lsr(wl.hash64(seed, idx.reshape(-1)), 11) % 4).view(rows, width)
+        ci = (r - 2 * width + 4 * torch.arange(width, dtype=torch.int64, device=dev).view(1, width) + step)
+        return {"rows": rows, "cols": rows, "colind": ci.clamp(0, rows - 1).reshape(-1).int(),
+                "rowptr": (torch.arange(rows + 1, dtype=torch.int64, device=dev) * width).int(),
+                "values": wl.uniform(seed + 1, rows * width, -1.0, 1.0, dev)}
+
+    box3 = list(itertools.product((-1, 0, 1), repeat=3))
+    cross3 = [o for o in box3 if sum(abs(v) for v in o) <= 1]
+    shapes = [
+        ("5-point, 1448^2", lambda: wl.laplacian_2d(1448, dev)),
+        ("7-point, 128^3", lambda: wl.stencil_csr((128, 128, 128), cross3, dev)),
+        ("27-point, 100^3", lambda: wl.stencil_csr((100, 100, 100), box3, dev)),
+        ("band of 50, 256 K rows", lambda: band(1 << 18, 50, 21)),
+        ("band of 200, 64 K rows", lambda: band(1 << 16, 200, 22)),
+        ("8 random columns a row, 1 M rows", lambda: wl.uniform_rows_csr(1 << 20, 1 << 20, 8, 5, dev)),
+        ("32 random columns a row, 512 K rows", lambda: wl.uniform_rows_csr(1 << 19, 1 << 19, 32, 7, dev)),
+    ]
+    if args.scale < 1.0:
+        shapes = shapes[:1]
+    res = {}
+    for name, make in shapes:
+        torch.cuda.empty_cache()
+        A = make()
+        rows, nnz = A["rows"], int(A["colind"].numel())
+        csr = osa.Csr(rows, A["cols"], A["rowptr"], A["colind"], A["values"])
+        res[name] = {"rows": rows, "nnz": nnz, "widths": {}}
+        for n in (16, 32, 64, 128):
+            B = wl.uniform(7, A["cols"] * n, -1.0, 1.0, dev)
+            C = torch.zeros(rows * n, dtype=torch.float32, device=dev)
+            dB, dC = osa.DnMat(A["cols"], n, n, B), osa.DnMat(rows, n, n, C)
+
+            def timed(op):
+                for _ in range(10):
+                    op(1.0, 0.0)
+                stream.synchronize()
+                return round(time_rounds(torch, stream, lambda i: op(1.0, 0.0), args.steps, None,
+                                         min(args.min_gpu_ms, 20.0))[0] * 1e3, 1)
+
+            line = {"picked_us": timed(osa.SpmmOp(handle, csr, dB, dC))}
+            os.environ["OPS_SPARSE_SPMM_NO_ROWS_RULE"] = "1"
+            slabs = osa.SpmmOp(handle, csr, dB, dC)
+            del os.environ["OPS_SPARSE_SPMM_NO_ROWS_RULE"]
+            line["slabs_us"] = timed(slabs)
+            os.environ["OPS_SPARSE_SPMM_NO_SLAB"] = "1"
+            line["rows_us"] = timed(slabs)
+            del os.environ["OPS_SPARSE_SPMM_NO_SLAB"]
+            bytes_alg = wl.spmm_bytes_alg(rows, A["cols"], n, nnz, 4, 4, 4, False)
+            line["frac_of_8TBs"] = round(bytes_alg / (line["picked_us"] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)
+            res[name]["widths"]["n=%d" % n] = line
+            log("%-36s n=%-4d %s" % (name, n, json.dumps(line)))
+            del slabs, B, C, dB, dC
+        del csr, A
+    return res
+
+
 def run_few_columns(args, osa, wl, torch, dev, stream, handle):
     """SpMM with one to sixteen columns of B (a few right-hand sides, block Krylov methods) on meshes: time of a
     call after Preprocess (alpha = 1, beta = 0), the algorithmic bytes against 8 TB/s, the same product as n
@@ -935,11 +1000,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all",
                     choices=["all", "c1", "c2", "c3", "c3_repeatable", "c3_transposed", "c4", "c5", "convert", "cache",
-                             "shapes", "stencils", "few_columns"],
+                             "shapes", "stencils", "few_columns", "spmm_shapes"],
                     help="all: c2 as the headline plus c1, c3 (default plan, repeatable default plan, ALG2, "
                          "transposed), c4 and c5 in `workloads`; shapes: the grid of secondary shapes behind the "
                          "selection thresholds; stencils: the headline kernels on other meshes and bands; "
-                         "few_columns: SpMM with 1 - 16 columns of B on meshes")
+                         "few_columns: SpMM with 1 - 16 columns of B on meshes; spmm_shapes: SpMM with 16 - 128 columns on meshes, "
+                         "bands and random columns under either kernel")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
     ap.add_argument("--min-gpu-ms", type=float, default=50.0,
                     help="rounds of --steps launches are repeated until this much GPU time has been timed")
@@ -991,6 +1057,12 @@ def main():
         print(json.dumps({"metric": "CSR SpMV fp32 on meshes and bands, time per call and algorithmic bytes / 8 TB/s",
                           "unit": "us", "data": "synthetic",
                           "shapes": run_stencils(args, osa, wl, torch, dev, stream, handle)}), flush=True)
+        handle.close()
+        return
+    if args.workload == "spmm_shapes":
+        print(json.dumps({"metric": "CSR SpMM fp32 by matrix shape and width: the slab kernel, the row kernel and "
+                                    "what Preprocess picks", "unit": "us", "data": "synthetic",
+                          "shapes": run_spmm_shapes(args, osa, wl, torch, dev, stream, handle)}), flush=True)
         handle.close()
         return
     if args.workload == "few_columns":
