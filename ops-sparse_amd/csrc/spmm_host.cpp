@@ -175,10 +175,10 @@ bool ColumnsAreVectors(const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *
 // Whether a matrix without long rows, under a B of n elements of elemBytes, is better served by the kernel that
 // gives every row whole to one lane group straight from memory than by the slabs staged through LDS.  Measured on
 // fp32 (us, slabs / rows; 1 - 2 M rows of meshes, bands, and uniformly random columns):
-//   n = 16: 5-point mesh 225 / 119, 27-point 440 / 283, band of 50 246 / 143, 32 random columns a row 494 / 419
-//   n = 32: 5-point 256 / 200, 27-point 555 / 308, band of 200 191 / 162, 8 random 191 / 183, 32 random 313 / 373
-//   n = 64: 5-point 394 / 515, 7-point 525 / 560, 27-point 778 / 582, band of 50 342 / 248, 32 random 591 / 618
-//   n = 128: 5-point 692 / 1027, 27-point 1139 / 1040, band of 200 459 / 384, 32 random 1194 / 1201
+//   n = 16: 5-point mesh 223 / 106, 27-point 441 / 280, band of 50 246 / 153, 32 random columns a row 495 / 414
+//   n = 32: 5-point 255 / 182, 27-point 556 / 260, band of 200 191 / 104, 8 random 189 / 182, 32 random 316 / 374
+//   n = 64: 5-point 395 / 438, 7-point 523 / 484, 27-point 779 / 460, band of 50 343 / 195, 32 random 587 / 613
+//   n = 128: 5-point 693 / 869, 27-point 1137 / 824, band of 200 460 / 310, 32 random 1185 / 1199
 // The slabs win where the gathers of B are what the product waits for (random columns, wide rows of B) and on
 // short rows under a wide B; rows of even length whose columns stay near the diagonal, and any narrow B, run
 // faster row by row.  Uneven rows stay with the slabs, which share them out by work.

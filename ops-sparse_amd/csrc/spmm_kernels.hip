@@ -42,8 +42,10 @@ namespace opsparse {
 constexpr int32_t kLongRowNnz = 2048;  // rows longer than this are cut into segments
 constexpr int32_t kSegmentNnz = 256;  // entries per segment (128: c5 1.394 ms, 256: 1.378 ms, 512: 1.402 ms)
 // Rows a lane group of the row-split kernel takes one after the other, so that a
-// workgroup lives long enough to amortise its start-up.
-constexpr int kSpmmRowsPerGroup = 4;
+// workgroup lives long enough to amortise its start-up.  (Two: with four a 5-point mesh takes 120 / 200 / 510 us
+// under n = 16 / 32 / 64 instead of 107 / 181 / 431, a 27-point one 313 / 581 us under n = 32 / 64 instead of
+// 270 / 459; with one 107 / 212 / 508 and 274 / 492; random columns do not care.)
+constexpr int kSpmmRowsPerGroup = 2;
 
 // Index of element (r, c) of a dense matrix with leading dimension ld.
 __device__ __forceinline__ int64_t DenseIndex(int64_t r, int64_t c, int64_t ld, bool colMajor)
