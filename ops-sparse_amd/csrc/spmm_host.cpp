@@ -175,13 +175,13 @@ bool ColumnsAreVectors(const aclsparseSpMatDescr *A, const aclsparseDnMatDescr *
 // Whether a matrix without long rows, under a B of n elements of elemBytes, is better served by the kernel that
 // gives every row whole to one lane group straight from memory than by the slabs staged through LDS.  Measured on
 // fp32 (us, slabs / rows; 1 - 2 M rows of meshes, bands, and uniformly random columns):
-//   n = 16: 5-point mesh 223 / 106, 27-point 441 / 280, band of 50 246 / 153, 32 random columns a row 495 / 414
-//   n = 32: 5-point 255 / 182, 27-point 556 / 260, band of 200 191 / 104, 8 random 189 / 182, 32 random 316 / 374
-//   n = 64: 5-point 395 / 438, 7-point 523 / 484, 27-point 779 / 460, band of 50 343 / 195, 32 random 587 / 613
-//   n = 128: 5-point 693 / 869, 27-point 1137 / 824, band of 200 460 / 310, 32 random 1185 / 1199
+//   n = 16: 5-point mesh 224 / 104, 27-point 439 / 280, band of 50 245 / 153, 32 random columns a row 494 / 415
+//   n = 32: 5-point 255 / 182, 27-point 558 / 263, band of 200 190 / 103, 8 random 191 / 181, 32 random 315 / 375
+//   n = 64: 5-point 392 / 365, 7-point 521 / 425, 27-point 772 / 423, band of 50 340 / 193, 32 random 592 / 631
+//   n = 128: 5-point 694 / 730, 7-point 905 / 888, 27-point 1135 / 748, band of 200 458 / 299, 32 random 1198 / 1215
 // The slabs win where the gathers of B are what the product waits for (random columns, wide rows of B) and on
-// short rows under a wide B; rows of even length whose columns stay near the diagonal, and any narrow B, run
-// faster row by row.  Uneven rows stay with the slabs, which share them out by work.
+// the shortest rows under the widest B; rows of even length whose columns stay near the diagonal, and any narrow
+// B, run faster row by row.  Uneven rows stay with the slabs, which share them out by work.
 bool PrefersWholeRows(const aclsparseSpMatDescr *A, const OpsparseSpmmPlan &plan, int64_t n, int64_t elemBytes,
                       void *buffer, hipStream_t stream)
 {
@@ -201,7 +201,7 @@ bool PrefersWholeRows(const aclsparseSpMatDescr *A, const OpsparseSpmmPlan &plan
     if (rowBytes <= 64 || (rowBytes <= 128 && mean < 24.0)) {
         return true;
     }
-    if (rowBytes > 128 && mean < 16.0) {
+    if (rowBytes > 256 && mean < 6.0) {
         return false;
     }
     // what is left depends on whether the rows of B a row needs lie near each other: the sample of the SpMV plans

@@ -117,7 +117,9 @@ __device__ __forceinline__ void AccumulateEntries(const int32_t *__restrict__ co
     // Gathers issued back to back, U * 16 bytes in flight per lane.  Eight for the
     // 8-element (fp16) vectors: their fp64 conversion needs the registers, and more
     // resident wavefronts hide more latency than a deeper batch.
-    constexpr int UMAX = V >= 8 ? 8 : 16;
+    // (sixteen 16-byte gathers a lane cost the row kernel a third of its resident wavefronts: 5-point mesh, n = 64,
+    // 432 us with sixteen, 365 with eight; rows of 27 entries 458 and 423; four: rows of 27 under n = 32 314 for 272)
+    constexpr int UMAX = 8;
     constexpr int U = L < UMAX ? L : UMAX;
     constexpr int US = U < 8 ? U : 8;   // predicated batch size for the short tail of a row
     for (int32_t p0 = s; p0 < e; p0 += L) {
