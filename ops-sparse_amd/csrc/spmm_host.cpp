@@ -198,11 +198,20 @@ bool PrefersWholeRows(const aclsparseSpMatDescr *A, const OpsparseSpmmPlan &plan
     if (rowBytes > 512 || static_cast<double>(plan.maxRowNnz) > 4.0 * mean + 8.0) {
         return false;
     }
-    if (rowBytes <= 64 || (rowBytes <= 128 && mean < 24.0)) {
-        return true;
-    }
-    if (rowBytes > 256 && mean < 6.0) {
-        return false;
+    if (elemBytes == 2) {
+        // fp16, whose slab kernel is the one tuned on c5, keeps the slabs except under local rows of 16 entries or
+        // more (us, slabs / rows: 27-point mesh n = 32 361 / 245, n = 64 459 / 399, n = 256 1401 / 1207; but 5-point
+        // n = 64 267 / 305, n = 128 508 / 614, 32 random columns a row n = 32 292 / 412)
+        if (mean < 16.0) {
+            return false;
+        }
+    } else {
+        if (rowBytes <= 64 || (rowBytes <= 128 && mean < 24.0)) {
+            return true;
+        }
+        if (rowBytes > 256 && mean < 6.0) {
+            return false;
+        }
     }
     // what is left depends on whether the rows of B a row needs lie near each other: the sample of the SpMV plans
     // (the first 256 bytes of the buffer are the analyses' scratch: no launch reads them)
